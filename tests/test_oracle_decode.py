@@ -1,0 +1,189 @@
+"""Pins for the CPU oracle's viterbi tables, tree-to-sequence readout and best-tree trace.
+
+No golden vectors exist in the reference; the pins are brute-force enumeration over explicit derivations on tiny
+graphs and hand-derived outcomes for exact ties (the reference's 4-lane scan order, pcfg_best_tree.cu:123-174,
+pcfg_viterbi.cu:75-124).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import bruteforce as bf
+from oracle import oracle
+from pcfg_nat_amd import synth
+
+NINF = -math.inf
+
+
+def _masked_links(L, m, ml, seed):
+    out_len = torch.tensor([m])
+    gen = torch.Generator().manual_seed(seed)
+    return synth.make_links(1, L, out_len, ml, gen)[0].double().numpy()
+
+
+@pytest.mark.parametrize("ml,L,m", [(1, 24, 24), (1, 24, 20), (3, 34, 34), (3, 34, 30)])
+def test_viterbi_scores_and_yields_match_enumeration(ml, L, m):
+    rng = np.random.default_rng(L + m)
+    links = _masked_links(L, m, ml, seed=L * 7 + m)
+    ob = rng.normal(size=L) - 1.0
+    S, R, Lt, M = oracle.viterbi(ob[None], links[None], np.array([m]), dtype=np.float64)
+    max_len = m // 4 - 1
+    best = bf.viterbi_best(ob.tolist(), links.tolist(), m, ml, max_len)
+    assert len(best) >= 2
+    left_mask, _, _ = synth.support_masks(L, ml)
+    tokens = (np.arange(L) + 100)[None]
+    for ln in range(2, max_len + 1):
+        if ln not in best:
+            assert S[0, 1, ln] == NINF
+            continue
+        assert abs(S[0, 1, ln] - best[ln][0]) < 1e-10
+        got = oracle.viterbi_decoding(np.array([ln]), np.array([m]), Lt, R, M, tokens, left_mask.numpy(), 1)
+        assert [int(t) - 100 for t in got[0]] == list(best[ln][1])
+    # lengths the table does not cover stay -inf, length 1 is only reachable by the last node
+    assert S[0, 1, 0] == NINF and S[0, 1, 1] == NINF and S[0, m - 1, 1] == ob[m - 1]
+
+
+def test_readout_dedup_pad_and_ragged_batch():
+    ml, L = 1, 24
+    rng = np.random.default_rng(0)
+    m = np.array([24, 16])
+    links = np.stack([_masked_links(L, int(mm), ml, seed=int(mm)) for mm in m])
+    ob = rng.normal(size=(2, L)) - 1.0
+    S, R, Lt, M = oracle.viterbi(ob, links, m, dtype=np.float32)
+    left_mask, _, _ = synth.support_masks(L, ml)
+    pred = np.array([5, 3])
+    tokens = (np.arange(L) + 100)[None].repeat(2, 0)
+    ref = oracle.viterbi_decoding(pred, m, Lt, R, M, tokens, left_mask.numpy(), 1)
+    assert ref.dtype == np.float32 and ref.shape == (2, 5)
+    assert (ref[1, 3:] == 1).all() and (ref[1, :3] != 1).all()
+    # make the 2nd and 3rd emitted nodes of sentence 0 share a token, and the 4th a pad: 5 -> 3 tokens
+    y = [int(t) - 100 for t in ref[0]]
+    tok2 = tokens.copy()
+    tok2[0, y[2]] = tok2[0, y[1]]
+    tok2[0, y[3]] = 1
+    got = oracle.viterbi_decoding(pred, m, Lt, R, M, tok2, left_mask.numpy(), 1)
+    assert got.shape == (2, 3)
+    assert list(got[0]) == [tok2[0, y[0]], tok2[0, y[1]], tok2[0, y[4]]]
+
+
+def test_readout_stops_at_forbidden_left_child():
+    """A left pointer that the support tree forbids ends the descent without visiting it (pcfg_loss.cpp:39-42)."""
+    L, Lq = 8, 2
+    Lt = np.zeros((1, L, Lq), dtype=np.int64)
+    R = np.zeros_like(Lt)
+    M = np.zeros_like(Lt)
+    Lt[0, 1, 1] = 2  # node 1 points left to node 2, which its mask forbids
+    mask = np.ones((L, L), dtype=np.int64)
+    mask[1:, 0] = 0
+    tokens = (np.arange(L) + 100)[None]
+    got = oracle.viterbi_decoding(np.array([1]), np.array([8]), Lt, R, M, tokens, mask, 1)
+    assert list(got[0]) == [101]
+    mask[1, 2] = 0
+    got = oracle.viterbi_decoding(np.array([1]), np.array([8]), Lt, R, M, tokens, mask, 1)
+    assert list(got[0]) == [102, 101]
+
+
+def _suffix_ll(match, links, a, s, m, n, ml):
+    vals = []
+    for y, lp, _ in bf.main_derivations(a, m, ml, links, n - s, allow_composite_local=False):
+        if len(y) == n - s:
+            vals.append(lp + sum(match[node][s + i] for i, node in enumerate(y)))
+    return bf.lse(vals)
+
+
+@pytest.mark.parametrize("ml,L,m,n", [(1, 16, 16, 8), (1, 16, 12, 5), (3, 22, 22, 7)])
+def test_best_tree_matches_greedy_on_enumerated_tables(ml, L, m, n):
+    rng = np.random.default_rng(n * 31 + m)
+    links = _masked_links(L, m, ml, seed=m + n)
+    match = rng.normal(size=(L, n)) - 2.0
+    match[:, n - 1] = NINF
+    match[m - 1, n - 1] = -0.5
+    S, C = oracle.inside_fwd(match[None], links[None], np.array([m]), np.array([n]))
+    tree = oracle.best_tree(S, C, match[None], links[None], np.array([m]), np.array([n]))[0]
+    ml_, ll_ = match.tolist(), links.tolist()
+    want = [-1] * L
+    a, s = 1, 0
+    while True:
+        best = None
+        for c in range(a + ml + 1, m, ml + 1):
+            for k in range(ml + 1):
+                if k == 0:
+                    j, extra = 0, 0.0
+                else:
+                    b = a - k
+                    if b < 1 or (b - bf.group_lo(b, ml)) % 2 != 1:
+                        continue
+                    j, extra = 1, ml_[b][s]
+                if s + j + 1 > n - 1:
+                    continue
+                v = ll_[a][k][c] + _suffix_ll(ml_, ll_, c, s + j + 1, m, n, ml) + extra + ml_[a][s + j]
+                if v != NINF and (best is None or v > best[0]):
+                    best = (v, c, k, j)
+        if best is None:
+            want[a] = s
+            break
+        _, c, k, j = best
+        want[a] = s + j
+        if k:
+            want[a - k] = s
+        a, s = c, s + j + 1
+    assert list(tree) == want
+    used = [t for t in tree if t >= 0]
+    assert sorted(used) == list(range(n)) and tree[1] == 0 and tree[m - 1] == n - 1
+    assert used == sorted(used)
+
+
+def _uniform_case(L, m, n, dead_cids=()):
+    """ml=1 graph whose candidates all tie exactly: every allowed link is -1 (k=0 only), every emission -1."""
+    links = np.full((1, L, 2, L), NINF)
+    for a in range(1, m - 1, 2):
+        for c in range(a + 2, m, 2):
+            links[0, a, 0, c] = -1.0
+    match = np.full((1, L, n), -1.0)
+    for cid in dead_cids:
+        links[0, 1, 0, 2 * cid + 1] = NINF
+    return match, links
+
+
+def test_best_tree_tie_order_is_lane_structured():
+    """Root (a_id 0) scans c_id = 1+x, 5+x, ... in lane x; ties resolve by lane priority 0 > 2 > 1 > 3, then scan order.
+    n=3: the root must pick a child that can reach the last node in one hop, i.e. any c_id in 1..Mc-2, all tying."""
+    L = m = 14  # Mc = 7: c_id 1..6, last = 6
+    match, links = _uniform_case(L, m, 3)
+    S, C = oracle.inside_fwd(match, links, np.array([m]), np.array([3]))
+
+    def second_node(dead):
+        mt, lk = _uniform_case(L, m, 3, dead)
+        S, C = oracle.inside_fwd(mt, lk, np.array([m]), np.array([3]))
+        tree = oracle.best_tree(S, C, mt, lk, np.array([m]), np.array([3]))[0]
+        (pos,) = np.nonzero(tree == 1)
+        return int(pos[0] - 1) // 2
+
+    assert second_node(()) == 1          # lane 0, first scanned
+    assert second_node((1,)) == 5        # lane 0 still holds c_id 5
+    assert second_node((1, 5)) == 3      # lane 2 (c_id 3) beats lanes 1 (c_id 2) and 3 (c_id 4)
+    assert second_node((1, 5, 3)) == 2   # lane 1 beats lane 3
+    assert second_node((1, 5, 3, 2)) == 4
+
+
+def test_viterbi_tie_order_is_lane_structured():
+    """Viterbi scans c_id = a_id+x, a_id+4+x, ... (self child included, pcfg_viterbi.cu:75); same lane priority."""
+    L = m = 32  # Mc = 16, table lengths 2..7
+    _, links = _uniform_case(L, m, 3)
+    ob = np.full((1, L), -1.0)
+
+    def right_child_of_root(dead):
+        lk = links.copy()
+        for cid in dead:
+            lk[0, 1, 0, 2 * cid + 1] = NINF
+        S, R, Lt, M = oracle.viterbi(ob, lk, np.array([m]), dtype=np.float32)
+        assert np.isfinite(S[0, 1, 3])
+        return int(R[0, 1, 3] - 1) // 2
+
+    # length 3 from the root: child must have a finite length-2 entry: c_id 1..14 tie; lane of c_id is c_id % 4
+    assert right_child_of_root(()) == 4                      # lane 0: c_id 4 (c_id 0 is the dead self link)
+    assert right_child_of_root((4, 8, 12)) == 2              # lane 2 next
+    assert right_child_of_root((4, 8, 12, 2, 6, 10, 14)) == 1
+    assert right_child_of_root((4, 8, 12, 2, 6, 10, 14, 1, 5, 9, 13)) == 3
