@@ -1,0 +1,136 @@
+/*
+ * C-ABI of libpcfg_nat_hip.so: the MI355X (gfx950) implementation of PCFG-NAT's structured-loss hot path.
+ *
+ * Each entry point replaces one function of the reference's native module
+ * (fs_plugins/custom_ops/pcfg_loss.cpp:76-81, declarations :6-18) on raw device pointers: no torch types, no
+ * allocation of outputs (the caller owns every buffer), kernels are enqueued on the given HIP stream and the
+ * call returns without synchronising unless stated otherwise.
+ *
+ * Conventions
+ *   - `stream` is a hipStream_t passed as void* (NULL = the legacy default stream).
+ *   - every function returns PCFGNAT_OK (0) or an error code; pcfgnat_last_error() then holds a message
+ *     (thread-local).  Numerical failure (a sentence whose log-likelihood is -inf) is not an error.
+ *   - B = batch, L = graph size (decoder positions), T = padded target length, V = vocabulary,
+ *     ml = links.size(2) - 1 ("max_left"), Mc = (L-2)/(ml+1)+1 main-chain nodes, Lq = L/4.
+ *   - all PCFG tables are float32, lengths are int64, like every caller in the reference.
+ */
+#ifndef PCFG_NAT_HIP_H
+#define PCFG_NAT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PCFGNAT_OK 0
+#define PCFGNAT_EINVAL 1       /* argument out of contract */
+#define PCFGNAT_EUNSUPPORTED 2 /* valid in the reference but not built here */
+#define PCFGNAT_EHIP 3         /* a HIP runtime call failed */
+
+#define PCFGNAT_F16 0
+#define PCFGNAT_F32 1
+#define PCFGNAT_F64 2
+
+/* ABI version of this header (bumped on incompatible change). */
+int pcfgnat_abi_version(void);
+
+/* Message of the last error raised on the calling thread ("" if none). */
+const char *pcfgnat_last_error(void);
+
+/*
+ * Replaces logsoftmax_gather (logsoftmax_gather.cu:295-359).
+ *   word_ins_out [B,L,V] contiguous, dtype PCFGNAT_F16 / F32 / F64.
+ *   select_idx   int64, logical shape [B,L,T], element strides (sb, sl, st); the criterion passes a
+ *                stride-0 expanded view of the [B,T] targets (nat_pcfg_loss.py:109).
+ *   selected     [B,L,T] contiguous, float32 (float64 when dtype is F64):
+ *                selected[b,p,s] = word_ins_out[b,p,idx] - max_v - log sum_v exp(. - max_v).
+ *   require_grad != 0: word_ins_out is overwritten in place with softmax(word_ins_out) in its own dtype.
+ */
+int pcfgnat_logsoftmax_gather(void *word_ins_out, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl,
+                              int64_t st, void *selected, int require_grad, int64_t B, int64_t L, int64_t V,
+                              int64_t T, void *stream);
+
+/*
+ * Replaces the two torch calls of DagLogsoftmaxGatherFunc.backward (pcfg_loss.py:176-177) by one pass:
+ *   probs_inout[b,p,v] = probs[b,p,v] * cast(-sum_s g[b,p,s]);  probs_inout[b,p,idx[b,p,s]] += cast(g[b,p,s])
+ * with every operation rounded to the buffer's dtype as torch's mul_/scatter_add_ do (duplicates of an index are
+ * accumulated in ascending s).  grad_selected is float32 (float64 when dtype is F64), contiguous [B,L,T].
+ */
+int pcfgnat_logsoftmax_gather_backward(void *probs_inout, int dtype, const int64_t *select_idx, int64_t sb,
+                                       int64_t sl, int64_t st, const void *grad_selected, int64_t B, int64_t L,
+                                       int64_t V, int64_t T, void *stream);
+
+/* Number of floats of the auxiliary table the inside kernels exchange (takes the place of the reference's C
+ * table, pcfg_loss.cu:394, whose content for ml = 1 is a copy of match_all). */
+size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml);
+
+/*
+ * Replaces pcfg_loss (pcfg_loss.cu:379-401): the inside algorithm.
+ *   match_all [B,L,T], links [B,L,ml+1,L] contiguous float32 log-probabilities (-inf allowed).
+ *   output_length, target_length [B] int64 on the device.
+ *   S   [B,Mc,T+2] out: suffix table of main-chain nodes, -inf where undefined; log-likelihood = S[b,0,0].
+ *   aux [pcfgnat_pcfg_aux_floats] out: opaque, consumed by the backward and best-tree entry points.
+ * Precondition checked on the device per sentence (violations yield S[b,0,0] = NaN, never a fault):
+ *   4 <= m <= L, (m-2) % (ml+1) == 0, 2 <= n <= T.
+ */
+int pcfgnat_pcfg_loss(const float *match_all, const float *links, const int64_t *output_length,
+                      const int64_t *target_length, float *S, float *aux, int64_t B, int64_t L, int64_t T,
+                      int64_t ml, void *stream);
+
+/*
+ * Replaces pcfg_loss_backward (pcfg_loss_backward.cu:654-721): gradients of sum_b grad_output[b] * S[b,0,0].
+ *   grad_output [B] float32; S, aux as produced by pcfgnat_pcfg_loss on the same inputs.
+ *   match_all_grad [B,L,T], links_grad [B,L,ml+1,L] out (fully written, zeros outside the support).
+ * The result is the exact gradient of the forward recurrences; sentences with a non-finite log-likelihood get
+ * all-zero gradients.
+ */
+int pcfgnat_pcfg_loss_backward(const float *grad_output, const float *S, float *aux, const float *match_all,
+                               const float *links, const int64_t *output_length, const int64_t *target_length,
+                               float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T,
+                               int64_t ml, void *stream);
+
+/*
+ * Replaces pcfg_best_tree (pcfg_best_tree.cu:333-360): greedy top-down trace over the inside tables.
+ *   tree [B,L] int64 out: target position aligned to each node, -1 for nodes off the tree.
+ * Exact ties are resolved in the reference's scan order (lanes 0 > 2 > 1 > 3 of a 4-wide strided scan).
+ */
+int pcfgnat_pcfg_best_tree(const float *S, const float *aux, const float *match_all, const float *links,
+                           const int64_t *output_length, const int64_t *target_length, int64_t *tree, int64_t B,
+                           int64_t L, int64_t T, int64_t ml, void *stream);
+
+/*
+ * Replaces pcfg_viterbi (pcfg_viterbi.cu:272-301): max-product tables per output length.
+ *   ob_lprob [B,L] float32, links [B,L,ml+1,L] float32, output_length [B] int64.
+ *   S [B,L,Lq] float32 out (-inf where undefined; the Python wrapper returns row 1),
+ *   R, Lt, M [B,L,Lq] int64 out (right child, left child, left span; 0 where undefined).
+ * Values and arg-max decisions are bit-identical to a sequential fp32 evaluation in the reference's order.
+ */
+int pcfgnat_pcfg_viterbi(const float *ob_lprob, const float *links, const int64_t *output_length, float *S,
+                         int64_t *R, int64_t *Lt, int64_t *M, int64_t B, int64_t L, int64_t ml, void *stream);
+
+/*
+ * Replaces viterbi_decoding (pcfg_loss.cpp:12-73) for traces that live on the device: one walk per sentence.
+ *   pred_length, output_length [B] int64; Lt, R, M [B,L,Lq] int64; tokens [B,L] int64;
+ *   left_tree_mask [mask_dim,mask_dim] int64 (non-zero = forbidden).
+ *   out_tokens [B,L] int64 out: emitted tokens, right-padded with pad_index; out_count [B] int64 out: how many
+ *   (-1 for malformed traces); scratch [B,2L] int64: the explicit stacks of the walks.
+ */
+int pcfgnat_viterbi_decoding(const int64_t *pred_length, const int64_t *output_length, const int64_t *Lt,
+                             const int64_t *R, const int64_t *M, const int64_t *tokens,
+                             const int64_t *left_tree_mask, int64_t mask_dim, int64_t pad_index,
+                             int64_t *out_tokens, int64_t *out_count, int64_t *scratch, int64_t B, int64_t L,
+                             int64_t Lq, void *stream);
+
+/* The same walk on host memory (the reference's own call site hands over CPU tensors,
+ * glat_decomposed_with_link_two_hands_tri_pcfg.py:500-502).  Synchronous, touches no GPU. */
+int pcfgnat_viterbi_decoding_host(const int64_t *pred_length, const int64_t *output_length, const int64_t *Lt,
+                                  const int64_t *R, const int64_t *M, const int64_t *tokens,
+                                  const int64_t *left_tree_mask, int64_t mask_dim, int64_t pad_index,
+                                  int64_t *out_tokens, int64_t *out_count, int64_t B, int64_t L, int64_t Lq);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PCFG_NAT_HIP_H */

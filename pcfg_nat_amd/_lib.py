@@ -1,0 +1,73 @@
+"""ctypes binding of libpcfg_nat_hip.so (declared in include/pcfg_nat_hip.h).
+
+Takes the place of the reference's JIT loader ``get_pcfg_kernel`` (fs_plugins/custom_ops/pcfg_loss.py:18-47): the
+library is built ahead of time for gfx950 (``pcfg_nat_amd/csrc/Makefile``) and loaded once; a missing library or a
+missing GPU is an error, never a silent fallback.
+"""
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libpcfg_nat_hip.so")
+
+OK, EINVAL, EUNSUPPORTED, EHIP = 0, 1, 2, 3
+F16, F32, F64 = 0, 1, 2
+
+_lib = None
+
+_vp = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+
+# name -> (restype, argtypes); mirrors include/pcfg_nat_hip.h one to one
+SIGNATURES = {
+    "pcfgnat_abi_version": (_int, []),
+    "pcfgnat_last_error": (ctypes.c_char_p, []),
+    "pcfgnat_logsoftmax_gather": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _int, _i64, _i64, _i64, _i64, _vp]),
+    "pcfgnat_logsoftmax_gather_backward": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "pcfgnat_pcfg_aux_floats": (ctypes.c_size_t, [_i64, _i64, _i64, _i64]),
+    "pcfgnat_pcfg_loss": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "pcfgnat_pcfg_loss_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "pcfgnat_pcfg_best_tree": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "pcfgnat_pcfg_viterbi": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "pcfgnat_viterbi_decoding": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "pcfgnat_viterbi_decoding_host": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64]),
+}
+
+
+def build(verbose=False):
+    """Compile the library in-tree with hipcc for gfx950 (cross-compiles without a GPU)."""
+    cmd = ["make", "-C", os.path.join(_HERE, "csrc"), "-j4", "-B"]
+    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if verbose or out.returncode != 0:
+        print(out.stdout)
+    if out.returncode != 0:
+        raise RuntimeError("building libpcfg_nat_hip.so failed")
+    return LIB_PATH
+
+
+def load():
+    """Load the library (once) and attach the prototypes.  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "libpcfg_nat_hip.so is missing (%s): build it with `make -C pcfg_nat_amd/csrc` or "
+            "`python -c 'import __graft_entry__ as g; g.build()'`; there is no CPU fallback" % LIB_PATH)
+    import torch  # noqa: F401  (its HIP runtime must be the one this library binds to)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc, lib=None):
+    if rc != OK:
+        lib = lib or load()
+        msg = lib.pcfgnat_last_error().decode("utf-8", "replace")
+        raise RuntimeError(msg or ("libpcfg_nat_hip error code %d" % rc))

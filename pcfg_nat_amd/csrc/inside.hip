@@ -1,0 +1,538 @@
+// PCFG inside algorithm (loss forward), its exact backward, and the GLAT best-tree trace, for max_left = 1.
+//
+// Replaces the reference's pcfg_loss.cu (calculate_C_kernel :262-349, calculate_S_kernel :84-224),
+// pcfg_loss_backward.cu (seven kernels, :28-603) and pcfg_best_tree.cu (:64-301).
+//
+// With max_left = 1 (every shipped configuration) main-chain node a = 2*a_id+1 has one local leaf a-1 and the
+// recurrences collapse to
+//   S[a][s] = LSE( match[a][s]                 + F0[a][s+1],      F0[a][t] = LSE_{c>=a} links[a][0][c] + S[c][t]
+//                  match[a-1][s] + match[a][s+1] + F1[a][s+2] )     F1[a][t] = LSE_{c>=a} links[a][1][c] + S[c][t]
+// and, with the outside score beta[c][t] = log(dS[root][0]/dS[c][t]) - ... (posterior = exp(beta + S)),
+//   beta[c][t] = LSE_{a<=c}( links[a][0][c] + match[a][t-1] + beta[a][t-1],
+//                            links[a][1][c] + match[a-1][t-2] + match[a][t-1] + beta[a][t-2] ).
+//
+// Design (latency-bound, one workgroup of 1024 threads per sentence): the sentence's compact link matrices live in
+// registers for the whole sweep (one 16-lane DPP row per node, lanes strided over the other index), the current
+// column of S (or of the outside weights) is exchanged through LDS, one workgroup barrier per target position,
+// no global atomics or inter-workgroup spinning.  The forward leaves F0/F1 behind so that the backward needs a
+// single sweep: rule posteriors are accumulated in registers, emission posteriors come from an element-wise
+// epilogue.
+#include "common.hip.h"
+
+namespace pcfgnat {
+namespace {
+
+constexpr int NT = 1024;       // threads per sentence
+constexpr int GROUPS = NT / 16;  // 16-lane rows
+
+__device__ __forceinline__ float sanitize(float v) { return (v != v) ? NEG_INF_F : v; }
+
+__device__ __forceinline__ float lse2(float a, float b) {
+    float m = fmaxf(a, b);
+    if (m == NEG_INF_F) return NEG_INF_F;
+    return m + __logf(__expf(a - m) + __expf(b - m));
+}
+
+// Aux layout per sentence: F0, F1, BETA, each [Mc][T+2].
+struct AuxView {
+    float *F0, *F1, *BETA;
+    __device__ AuxView(float *aux, int b, int Mc, int T) {
+        size_t plane = (size_t)Mc * (T + 2);
+        float *base = aux + (size_t)b * 3 * plane;
+        F0 = base;
+        F1 = base + plane;
+        BETA = base + 2 * plane;
+    }
+};
+
+__device__ __forceinline__ bool lengths_ok(int m, int n, int L, int T) {
+    return m >= 4 && m <= L && (m % 2) == 0 && n >= 2 && n <= T;
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Forward.  R = ceil(Mc/64) nodes per 16-lane row, CN = 4R children per lane.
+// Dynamic LDS: col[2][64R] floats, then (if MATCH_LDS) match rows of main nodes [Mc][T] and of their leaves [Mc][T].
+// ------------------------------------------------------------------------------------------------------------
+template <int R, bool MATCH_LDS>
+__global__ __launch_bounds__(NT) void inside_fwd_ml1_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
+                                                           const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
+                                                           float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc) {
+    constexpr int CN = 4 * R;
+    constexpr int MP = 64 * R;
+    extern __shared__ float smem[];
+    float *col = smem;              // [2][MP]
+    float *sm_main = smem + 2 * MP;  // [Mc][T]
+    float *sm_leaf = sm_main + (MATCH_LDS ? Mc * T : 0);
+
+    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *mt = match_all + (size_t)b * L * T;
+    const float *lk = links + (size_t)b * L * 2 * L;
+    float *Sb = S + (size_t)b * Mc * (T + 2);
+    AuxView av(aux, b, Mc, T);
+
+    if (!lengths_ok(m, n, L, T)) {  // out of contract: poison the log-likelihood, touch nothing else
+        for (int i = tid; i < Mc * (T + 2); i += NT) Sb[i] = (i == 0) ? __builtin_nanf("") : NEG_INF_F;
+        return;
+    }
+    const int mc = m / 2;  // active main-chain nodes: a_id < mc
+
+    // link slabs -> registers
+    float A0[R][CN], A1[R][CN];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int a_id = gidx + 64 * r, a = 2 * a_id + 1;
+#pragma unroll
+        for (int q = 0; q < CN; q++) {
+            const int c_id = j + 16 * q, c = 2 * c_id + 1;
+            const bool ok = a_id < mc && c_id < mc && c_id >= a_id;
+            A0[r][q] = ok ? sanitize(lk[((size_t)a * 2 + 0) * L + c]) : NEG_INF_F;
+            A1[r][q] = (ok && a_id >= 1) ? sanitize(lk[((size_t)a * 2 + 1) * L + c]) : NEG_INF_F;
+        }
+    }
+    if (MATCH_LDS) {
+        for (int i = tid; i < Mc * T; i += NT) {
+            const int a_id = i / T, s = i - a_id * T;
+            const bool ok = a_id < mc && s < n;
+            sm_main[i] = ok ? sanitize(mt[(size_t)(2 * a_id + 1) * T + s]) : NEG_INF_F;
+            sm_leaf[i] = (ok && a_id >= 1) ? sanitize(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
+        }
+    }
+    // cells of S the sweep never writes: rows beyond the sentence, columns from n-1 on (except the base cell)
+    for (int i = tid; i < Mc * (T + 2); i += NT) {
+        const int a_id = i / (T + 2), s = i - a_id * (T + 2);
+        if (a_id >= mc || s >= n - 1) {
+            float v = NEG_INF_F;
+            if (a_id == mc - 1 && s == n - 1) v = sanitize(mt[(size_t)(m - 1) * T + (n - 1)]);
+            Sb[i] = v;
+        }
+    }
+    // column n-1: only the last node, emitting the last token (pcfg_loss.cu:142-147)
+    for (int i = tid; i < MP; i += NT) col[((n - 1) & 1) * MP + i] = (i == mc - 1) ? sanitize(mt[(size_t)(m - 1) * T + (n - 1)]) : NEG_INF_F;
+    float F1prev[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) F1prev[r] = NEG_INF_F;
+    __syncthreads();
+
+    for (int t = n - 1; t >= 1; t--) {
+        const float *cur = col + (t & 1) * MP;
+        float *nxt = col + ((t - 1) & 1) * MP;
+        float sc[CN];
+#pragma unroll
+        for (int q = 0; q < CN; q++) sc[q] = cur[j + 16 * q];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int a_id = gidx + 64 * r;
+            float v0[CN], v1[CN];
+            float m0 = NEG_INF_F, m1 = NEG_INF_F;
+#pragma unroll
+            for (int q = 0; q < CN; q++) {
+                v0[q] = A0[r][q] + sc[q];
+                v1[q] = A1[r][q] + sc[q];
+                m0 = fmaxf(m0, v0[q]);
+                m1 = fmaxf(m1, v1[q]);
+            }
+            m0 = row16_max(m0);
+            m1 = row16_max(m1);
+            const float m0s = (m0 == NEG_INF_F) ? 0.f : m0, m1s = (m1 == NEG_INF_F) ? 0.f : m1;
+            float e0 = 0.f, e1 = 0.f;
+#pragma unroll
+            for (int q = 0; q < CN; q++) {
+                e0 += __expf(v0[q] - m0s);
+                e1 += __expf(v1[q] - m1s);
+            }
+            e0 = row16_sum(e0);
+            e1 = row16_sum(e1);
+            const float F0 = (m0 == NEG_INF_F) ? NEG_INF_F : m0 + __logf(e0);
+            const float F1 = (m1 == NEG_INF_F) ? NEG_INF_F : m1 + __logf(e1);
+            float ma_p, ml_p, ma_t;  // match[a][t-1], match[a-1][t-1], match[a][t]
+            if (MATCH_LDS) {
+                const int ai = (a_id < Mc) ? a_id : 0;
+                ma_p = sm_main[ai * T + t - 1];
+                ml_p = sm_leaf[ai * T + t - 1];
+                ma_t = sm_main[ai * T + t];
+            } else {
+                const bool ok = a_id < mc;
+                const size_t ra = (size_t)(2 * a_id + 1) * T, rl = (size_t)(2 * a_id) * T;
+                ma_p = ok ? sanitize(mt[ra + t - 1]) : NEG_INF_F;
+                ml_p = (ok && a_id >= 1) ? sanitize(mt[rl + t - 1]) : NEG_INF_F;
+                ma_t = ok ? sanitize(mt[ra + t]) : NEG_INF_F;
+            }
+            float s_new = lse2(ma_p + F0, (ml_p + ma_t) + F1prev[r]);
+            if (a_id >= mc) s_new = NEG_INF_F;
+            F1prev[r] = F1;
+            if (j == 0) {
+                nxt[a_id] = s_new;
+                if (a_id < mc) {
+                    Sb[(size_t)a_id * (T + 2) + (t - 1)] = s_new;
+                    av.F0[(size_t)a_id * (T + 2) + t] = F0;
+                    av.F1[(size_t)a_id * (T + 2) + t] = F1;
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Backward: outside sweep t = 1 .. n-1 (one DPP row per child node c, lanes strided over parents a), rule
+// posteriors accumulated in registers, then the element-wise emission epilogue.
+// Dynamic LDS: w0[2][MP], w1[2][MP], then (if TAB_LDS) S table [Mc][T], match main [Mc][T], match leaf [Mc][T].
+// ------------------------------------------------------------------------------------------------------------
+template <int R, bool TAB_LDS>
+__global__ __launch_bounds__(NT) void inside_bwd_ml1_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
+                                                           float *__restrict__ aux, const float *__restrict__ match_all,
+                                                           const float *__restrict__ links, const int64_t *__restrict__ out_len,
+                                                           const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad,
+                                                           float *__restrict__ lgrad, int L, int T, int Mc) {
+    constexpr int CN = 4 * R;
+    constexpr int MP = 64 * R;
+    extern __shared__ float smem[];
+    float *w0 = smem;            // [2][MP]
+    float *w1 = smem + 2 * MP;    // [2][MP]
+    float *sm_S = smem + 4 * MP;  // [Mc][T]   (TAB_LDS)
+    float *sm_main = sm_S + (TAB_LDS ? Mc * T : 0);
+    float *sm_leaf = sm_main + (TAB_LDS ? Mc * T : 0);
+
+    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *mt = match_all + (size_t)b * L * T;
+    const float *lk = links + (size_t)b * L * 2 * L;
+    const float *Sb = S + (size_t)b * Mc * (T + 2);
+    float *mg = mgrad + (size_t)b * L * T;
+    float *lg = lgrad + (size_t)b * L * 2 * L;
+    AuxView av(aux, b, Mc, T);
+
+    const float ll = Sb[0];
+    const bool valid = lengths_ok(m, n, L, T) && (ll == ll) && (fabsf(ll) != __builtin_huge_valf());
+    if (!valid) {  // invalid sentence: all-zero gradients (nat_pcfg_loss.py:123-133 zeroes its loss as well)
+        for (int i = tid; i < L * T; i += NT) mg[i] = 0.f;
+        for (int i = tid; i < L * 2 * L; i += NT) lg[i] = 0.f;
+        return;
+    }
+    const int mc = m / 2;
+    const float g = grad_out[b];
+
+    // transposed link slabs: row = child c (this thread's DPP row), lanes over parents a <= c
+    float A0[R][CN], A1[R][CN], G0[R][CN], G1[R][CN];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int c_id = gidx + 64 * r, c = 2 * c_id + 1;
+#pragma unroll
+        for (int q = 0; q < CN; q++) {
+            const int a_id = j + 16 * q, a = 2 * a_id + 1;
+            const bool ok = a_id < mc && c_id < mc && a_id <= c_id;
+            A0[r][q] = ok ? sanitize(lk[((size_t)a * 2 + 0) * L + c]) : NEG_INF_F;
+            A1[r][q] = (ok && a_id >= 1) ? sanitize(lk[((size_t)a * 2 + 1) * L + c]) : NEG_INF_F;
+            G0[r][q] = 0.f;
+            G1[r][q] = 0.f;
+        }
+    }
+    if (TAB_LDS) {
+        for (int i = tid; i < Mc * T; i += NT) {
+            const int a_id = i / T, s = i - a_id * T;
+            const bool ok = a_id < mc && s < n;
+            sm_S[i] = ok ? Sb[(size_t)a_id * (T + 2) + s] : NEG_INF_F;
+            sm_main[i] = ok ? sanitize(mt[(size_t)(2 * a_id + 1) * T + s]) : NEG_INF_F;
+            sm_leaf[i] = (ok && a_id >= 1) ? sanitize(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
+        }
+    }
+    auto match_main = [&](int a_id, int s) -> float {
+        if (TAB_LDS) return sm_main[a_id * T + s];
+        return sanitize(mt[(size_t)(2 * a_id + 1) * T + s]);
+    };
+    auto match_leaf = [&](int a_id, int s) -> float {
+        if (TAB_LDS) return sm_leaf[a_id * T + s];
+        return a_id >= 1 ? sanitize(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
+    };
+    auto s_at = [&](int a_id, int s) -> float {
+        if (TAB_LDS) return sm_S[a_id * T + s];
+        return Sb[(size_t)a_id * (T + 2) + s];
+    };
+
+    const float beta00 = -ll;  // outside score of (root, 0) for a unit upstream gradient
+    for (int i = tid; i < MP; i += NT) {
+        w0[1 * MP + i] = NEG_INF_F;
+        w1[1 * MP + i] = NEG_INF_F;
+    }
+    // beta[.][0]
+    for (int i = tid; i < mc; i += NT) av.BETA[(size_t)i * (T + 2)] = (i == 0) ? beta00 : NEG_INF_F;
+    __syncthreads();
+    float bprev[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) bprev[r] = (gidx + 64 * r == 0) ? beta00 : NEG_INF_F;
+    if (tid == 0) w0[1 * MP + 0] = match_main(0, 0) + beta00;
+    __syncthreads();
+
+    for (int t = 1; t <= n - 1; t++) {
+        const float *c0 = w0 + (t & 1) * MP, *c1 = w1 + (t & 1) * MP;
+        float *n0 = w0 + ((t + 1) & 1) * MP, *n1 = w1 + ((t + 1) & 1) * MP;
+        float wa0[CN], wa1[CN];
+#pragma unroll
+        for (int q = 0; q < CN; q++) {
+            wa0[q] = c0[j + 16 * q];
+            wa1[q] = c1[j + 16 * q];
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int c_id = gidx + 64 * r;
+            const bool live = c_id < mc;
+            const int ci = live ? c_id : 0;
+            float v0[CN], v1[CN];
+            float mx = NEG_INF_F;
+#pragma unroll
+            for (int q = 0; q < CN; q++) {
+                v0[q] = A0[r][q] + wa0[q];
+                v1[q] = A1[r][q] + wa1[q];
+                mx = fmaxf(mx, fmaxf(v0[q], v1[q]));
+            }
+            mx = row16_max(mx);
+            const float mxs = (mx == NEG_INF_F) ? 0.f : mx;
+            float e0[CN], e1[CN], sum = 0.f;
+#pragma unroll
+            for (int q = 0; q < CN; q++) {
+                e0[q] = __expf(v0[q] - mxs);
+                e1[q] = __expf(v1[q] - mxs);
+                sum += e0[q] + e1[q];
+            }
+            sum = row16_sum(sum);
+            const float beta = (mx == NEG_INF_F || !live) ? NEG_INF_F : mx + __logf(sum);
+            const float sct = live ? s_at(ci, t) : NEG_INF_F;
+            const float scale = (mx == NEG_INF_F || sct == NEG_INF_F) ? 0.f : __expf(mxs + sct);
+#pragma unroll
+            for (int q = 0; q < CN; q++) {
+                G0[r][q] += e0[q] * scale;
+                G1[r][q] += e1[q] * scale;
+            }
+            // outside weights this node offers to its children at the next two positions
+            const float mc_t = live ? match_main(ci, t) : NEG_INF_F;
+            const float nw0 = mc_t + beta;
+            const float nw1 = (live ? (match_leaf(ci, t - 1) + mc_t) : NEG_INF_F) + bprev[r];
+            bprev[r] = beta;
+            if (j == 0) {
+                n0[c_id] = nw0;
+                n1[c_id] = nw1;
+                if (live) av.BETA[(size_t)c_id * (T + 2) + t] = beta;
+            }
+        }
+        __syncthreads();
+    }
+    __threadfence();
+    __syncthreads();
+
+    // rule posteriors -> links_grad (pcfg_loss_backward.cu:512-531); everything else in the slab is zero
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int c_id = gidx + 64 * r, c = 2 * c_id + 1;
+#pragma unroll
+        for (int q = 0; q < CN; q++) {
+            const int a_id = j + 16 * q, a = 2 * a_id + 1;
+            if (a_id < Mc && c_id < Mc && a_id <= c_id && c < L) {
+                lg[((size_t)a * 2 + 0) * L + c] = g * G0[r][q];
+                lg[((size_t)a * 2 + 1) * L + c] = g * G1[r][q];
+            }
+        }
+    }
+    for (int i = tid; i < L * 2 * L; i += NT) {
+        const int c = i % L, a = i / (2 * L);
+        const bool owned = (a & 1) && (c & 1) && (a >> 1) < Mc && (c >> 1) < Mc && (a >> 1) <= (c >> 1);
+        if (!owned) lg[i] = 0.f;
+    }
+
+    // emission posteriors -> match_all_grad (pcfg_loss_backward.cu:348-382, 429-433)
+    for (int i = tid; i < L * T; i += NT) {
+        const int x = i / T, s = i - x * T;
+        float out = 0.f;
+        if (x >= 1 && x < m && s < n) {
+            if (x & 1) {
+                const int a_id = x >> 1;
+                const size_t row = (size_t)a_id * (T + 2);
+                const float bs = av.BETA[row + s];
+                const float mas = match_main(a_id, s);
+                if (s + 1 <= n - 1) out += __expf(bs + mas + av.F0[row + s + 1]);  // a emits s with the null left child
+                if (s >= 1 && s + 1 <= n - 1 && a_id >= 1)                        // a emits s after its leaf emitted s-1
+                    out += __expf(av.BETA[row + s - 1] + match_leaf(a_id, s - 1) + mas + av.F1[row + s + 1]);
+                if (a_id == mc - 1 && s == n - 1) out += __expf(bs + mas);       // base cell
+            } else {
+                const int a_id = x >> 1;  // parent a = x+1
+                if (a_id >= 1 && a_id < mc && s + 2 <= n - 1) {
+                    const size_t row = (size_t)a_id * (T + 2);
+                    out += __expf(av.BETA[row + s] + match_leaf(a_id, s) + match_main(a_id, s + 1) + av.F1[row + s + 2]);
+                }
+            }
+            if (!(out == out)) out = 0.f;
+        }
+        mg[i] = g * out;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Best tree (pcfg_best_tree.cu:64-197, 239-301): a single top-down chain per sentence, one wave64 per sentence.
+// Candidate order for exact ties: lane = (c_id - a_id - 1) & 3 with priority 0 > 2 > 1 > 3, then c ascending, then
+// (j=0,k=0) before (j=1,k=1).
+// ------------------------------------------------------------------------------------------------------------
+__device__ __forceinline__ int tie_key(int rel_c, int j) {
+    const int lane = rel_c & 3;
+    const int rank = (lane == 0) ? 0 : (lane == 2) ? 1 : (lane == 1) ? 2 : 3;
+    return (rank << 24) | (rel_c << 1) | j;
+}
+
+__global__ __launch_bounds__(64) void best_tree_ml1_kernel(const float *__restrict__ S, const float *__restrict__ match_all,
+                                                          const float *__restrict__ links, const int64_t *__restrict__ out_len,
+                                                          const int64_t *__restrict__ tgt_len, int64_t *__restrict__ tree, int L,
+                                                          int T, int Mc) {
+    const int b = blockIdx.x, lane = threadIdx.x;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *mt = match_all + (size_t)b * L * T;
+    const float *lk = links + (size_t)b * L * 2 * L;
+    const float *Sb = S + (size_t)b * Mc * (T + 2);
+    int64_t *tr = tree + (size_t)b * L;
+    for (int i = lane; i < L; i += 64) tr[i] = -1;
+    if (!lengths_ok(m, n, L, T)) return;
+    const int mc = m / 2;
+    __threadfence_block();
+    int a_id = 0, s = 0;
+    // every marked cell (a, s) has s <= n by construction; the loop is bounded by the number of main-chain nodes
+    for (int hop = 0; hop < mc; hop++) {
+        const int a = 2 * a_id + 1;
+        float best = NEG_INF_F;
+        int best_key = 0x7fffffff, best_c = -1, best_j = 0;
+        const float ma_s = (s < n) ? mt[(size_t)a * T + s] : NEG_INF_F;
+        const bool j1 = (n - s > 1) && a_id >= 1;
+        const float ml_s = j1 ? mt[(size_t)(a - 1) * T + s] : NEG_INF_F;
+        const float ma_s1 = j1 ? mt[(size_t)a * T + s + 1] : NEG_INF_F;
+        for (int c_id = a_id + 1 + lane; c_id < mc; c_id += 64) {
+            const int c = 2 * c_id + 1;
+            if (s < n) {  // j = 0, null left child: ((links + S) + C[0][s][0]) + match, C = 0
+                float v = ((lk[((size_t)a * 2 + 0) * L + c] + Sb[(size_t)c_id * (T + 2) + s + 1]) + 0.f) + ma_s;
+                if (v != v) v = NEG_INF_F;
+                const int key = tie_key(c_id - a_id - 1, 0);
+                if (v > best || (v == best && v != NEG_INF_F && key < best_key)) { best = v; best_key = key; best_c = c_id; best_j = 0; }
+            }
+            if (j1) {  // j = 1, leaf a-1 emits s: ((links + S) + match[a-1][s]) + match[a][s+1]
+                float v = ((lk[((size_t)a * 2 + 1) * L + c] + Sb[(size_t)c_id * (T + 2) + s + 2]) + ml_s) + ma_s1;
+                if (v != v) v = NEG_INF_F;
+                const int key = tie_key(c_id - a_id - 1, 1);
+                if (v > best || (v == best && v != NEG_INF_F && key < best_key)) { best = v; best_key = key; best_c = c_id; best_j = 1; }
+            }
+        }
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(best, o);
+            const int ok = __shfl_xor(best_key, o), oc = __shfl_xor(best_c, o), oj = __shfl_xor(best_j, o);
+            if (ov > best || (ov == best && ov != NEG_INF_F && ok < best_key)) { best = ov; best_key = ok; best_c = oc; best_j = oj; }
+        }
+        if (lane == 0) {
+            tr[a] = s + best_j;                            // pcfg_best_tree.cu:182
+            if (best_c >= 0 && best_j == 1 && s < n - 2) tr[a - 1] = s;  // leaf cell (b, s, 1), :268-297 with i < n-gap-1
+        }
+        if (best_c < 0) break;
+        a_id = best_c;
+        s = s + best_j + 1;
+    }
+}
+
+template <int R>
+int launch_fwd(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B, int L,
+               int T, int Mc, hipStream_t stream) {
+    const size_t base = (size_t)2 * 64 * R * sizeof(float);
+    const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
+    if (with_match <= 96 * 1024) {
+        auto k = inside_fwd_ml1_kernel<R, true>;
+        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_match));
+        hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_match, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
+    } else {
+        hipLaunchKernelGGL((inside_fwd_ml1_kernel<R, false>), dim3(B), dim3(NT), base, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
+    }
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
+template <int R>
+int launch_bwd(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
+               const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, hipStream_t stream) {
+    const size_t base = (size_t)4 * 64 * R * sizeof(float);
+    const size_t with_tab = base + (size_t)3 * Mc * T * sizeof(float);
+    if (with_tab <= 96 * 1024) {
+        auto k = inside_bwd_ml1_kernel<R, true>;
+        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_tab));
+        hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_tab, stream, go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc);
+    } else {
+        hipLaunchKernelGGL((inside_bwd_ml1_kernel<R, false>), dim3(B), dim3(NT), base, stream, go, S, aux, match_all, links, ol, tl, mg,
+                           lg, L, T, Mc);
+    }
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
+int check_dims(const char *who, int64_t B, int64_t L, int64_t T, int64_t ml) {
+    PCFGNAT_REQUIRE(B >= 0 && L >= 4 && T >= 2, "%s: need B >= 0, L >= 4, T >= 2 (got B=%lld L=%lld T=%lld)", who, (long long)B,
+                    (long long)L, (long long)T);
+    PCFGNAT_REQUIRE(ml >= 0, "%s: links must have at least one left option", who);
+    PCFGNAT_REQUIRE(L <= 32768 && T <= 32768 && B <= (1 << 24), "%s: dimension too large", who);
+    if (ml != 1)
+        return fail(PCFGNAT_EUNSUPPORTED,
+                    "%s: max_left = %lld (links.size(2) = %lld); only max_left = 1 (--left-tree-layer 1, the setting of every shipped "
+                    "script) is built",
+                    who, (long long)ml, (long long)ml + 1);
+    return PCFGNAT_OK;
+}
+
+}  // namespace
+}  // namespace pcfgnat
+
+using namespace pcfgnat;
+
+extern "C" size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml) {
+    if (B <= 0 || L < 2 || T < 0 || ml < 0) return 0;
+    const int64_t Mc = (L - 2) / (ml + 1) + 1;
+    return (size_t)B * 3 * Mc * (T + 2);
+}
+
+extern "C" int pcfgnat_pcfg_loss(const float *match_all, const float *links, const int64_t *output_length,
+                                 const int64_t *target_length, float *S, float *aux, int64_t B, int64_t L, int64_t T, int64_t ml,
+                                 void *stream) {
+    int rc = check_dims("pcfg_loss", B, L, T, ml);
+    if (rc != PCFGNAT_OK) return rc;
+    if (B == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(match_all && links && output_length && target_length && S && aux, "pcfg_loss: null pointer");
+    const int Mc = (int)((L - 2) / 2 + 1);
+    hipStream_t s = (hipStream_t)stream;
+    if (Mc <= 64) return launch_fwd<1>(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s);
+    if (Mc <= 128) return launch_fwd<2>(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s);
+    return fail(PCFGNAT_EUNSUPPORTED, "pcfg_loss: graph size L=%lld exceeds the built limit of 256 nodes", (long long)L);
+}
+
+extern "C" int pcfgnat_pcfg_loss_backward(const float *grad_output, const float *S, float *aux, const float *match_all,
+                                          const float *links, const int64_t *output_length, const int64_t *target_length,
+                                          float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T, int64_t ml,
+                                          void *stream) {
+    int rc = check_dims("pcfg_loss_backward", B, L, T, ml);
+    if (rc != PCFGNAT_OK) return rc;
+    if (B == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(grad_output && S && aux && match_all && links && output_length && target_length && match_all_grad && links_grad,
+                    "pcfg_loss_backward: null pointer");
+    const int Mc = (int)((L - 2) / 2 + 1);
+    hipStream_t s = (hipStream_t)stream;
+    if (Mc <= 64)
+        return launch_bwd<1>(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
+                             (int)L, (int)T, Mc, s);
+    if (Mc <= 128)
+        return launch_bwd<2>(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
+                             (int)L, (int)T, Mc, s);
+    return fail(PCFGNAT_EUNSUPPORTED, "pcfg_loss_backward: graph size L=%lld exceeds the built limit of 256 nodes", (long long)L);
+}
+
+extern "C" int pcfgnat_pcfg_best_tree(const float *S, const float *aux, const float *match_all, const float *links,
+                                      const int64_t *output_length, const int64_t *target_length, int64_t *tree, int64_t B, int64_t L,
+                                      int64_t T, int64_t ml, void *stream) {
+    int rc = check_dims("pcfg_best_tree", B, L, T, ml);
+    if (rc != PCFGNAT_OK) return rc;
+    if (B == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(S && match_all && links && output_length && target_length && tree, "pcfg_best_tree: null pointer");
+    (void)aux;
+    const int Mc = (int)((L - 2) / 2 + 1);
+    hipLaunchKernelGGL(best_tree_ml1_kernel, dim3((unsigned)B), dim3(64), 0, (hipStream_t)stream, S, match_all, links, output_length,
+                       target_length, tree, (int)L, (int)T, Mc);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}

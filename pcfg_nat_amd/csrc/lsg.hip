@@ -1,0 +1,411 @@
+// Fused log-softmax + target gather over [B*L, V] logits, and its in-place backward.
+//
+// Replaces logsoftmax_gather_kernel (reference fs_plugins/custom_ops/logsoftmax_gather.cu:238-292), which reads
+// every row three times with scalar 2-byte loads, and the two generic torch passes of
+// DagLogsoftmaxGatherFunc.backward (fs_plugins/custom_ops/pcfg_loss.py:176-177).
+//
+// Design (HBM-bound, MI355X): one workgroup per row; the row is fetched once with 16-byte loads and kept in
+// registers (chunks beyond the register budget are re-streamed), so HBM sees one read and - when the gradient is
+// needed - one write per element.  Row max / sum use DPP wave reductions plus one LDS hop across waves.
+#include "common.hip.h"
+
+namespace pcfgnat {
+namespace {
+
+typedef unsigned int vec16 __attribute__((ext_vector_type(4)));  // one 16-byte global access
+
+template <typename T>
+struct Elem;
+template <>
+struct Elem<__half> {
+    using compute = float;
+    static constexpr int EPV = 8;
+    __device__ static __forceinline__ void unpack(const vec16 &v, float *o) {
+        const __half2 *h = reinterpret_cast<const __half2 *>(&v);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float2 f = __half22float2(h[i]);
+            o[2 * i] = f.x;
+            o[2 * i + 1] = f.y;
+        }
+    }
+    __device__ static __forceinline__ vec16 pack(const float *o) {
+        vec16 v;
+        __half2 *h = reinterpret_cast<__half2 *>(&v);
+#pragma unroll
+        for (int i = 0; i < 4; i++) h[i] = __floats2half2_rn(o[2 * i], o[2 * i + 1]);
+        return v;
+    }
+    __device__ static __forceinline__ float widen(__half x) { return __half2float(x); }
+    __device__ static __forceinline__ __half narrow(float x) { return __float2half_rn(x); }
+};
+template <>
+struct Elem<float> {
+    using compute = float;
+    static constexpr int EPV = 4;
+    __device__ static __forceinline__ void unpack(const vec16 &v, float *o) {
+        o[0] = __uint_as_float(v.x);
+        o[1] = __uint_as_float(v.y);
+        o[2] = __uint_as_float(v.z);
+        o[3] = __uint_as_float(v.w);
+    }
+    __device__ static __forceinline__ vec16 pack(const float *o) {
+        vec16 v = {__float_as_uint(o[0]), __float_as_uint(o[1]), __float_as_uint(o[2]), __float_as_uint(o[3])};
+        return v;
+    }
+    __device__ static __forceinline__ float widen(float x) { return x; }
+    __device__ static __forceinline__ float narrow(float x) { return x; }
+};
+template <>
+struct Elem<double> {
+    using compute = double;
+    static constexpr int EPV = 2;
+    __device__ static __forceinline__ void unpack(const vec16 &v, double *o) {
+        o[0] = __longlong_as_double(((long long)v.y << 32) | v.x);
+        o[1] = __longlong_as_double(((long long)v.w << 32) | v.z);
+    }
+    __device__ static __forceinline__ vec16 pack(const double *o) {
+        long long a = __double_as_longlong(o[0]), b = __double_as_longlong(o[1]);
+        vec16 v = {(unsigned)a, (unsigned)(a >> 32), (unsigned)b, (unsigned)(b >> 32)};
+        return v;
+    }
+    __device__ static __forceinline__ double widen(double x) { return x; }
+    __device__ static __forceinline__ double narrow(double x) { return x; }
+};
+
+__device__ __forceinline__ float fast_exp(float x) { return __expf(x); }
+__device__ __forceinline__ double fast_exp(double x) { return exp(x); }
+__device__ __forceinline__ float fast_log(float x) { return __logf(x); }
+__device__ __forceinline__ double fast_log(double x) { return log(x); }
+__device__ __forceinline__ float neg_inf(float) { return -__builtin_huge_valf(); }
+__device__ __forceinline__ double neg_inf(double) { return -__builtin_huge_val(); }
+__device__ __forceinline__ float vmax(float a, float b) { return fmaxf(a, b); }
+__device__ __forceinline__ double vmax(double a, double b) { return fmax(a, b); }
+
+__device__ __forceinline__ vec16 load16(const vec16 *p) { return __builtin_nontemporal_load(p); }
+// Makes the compiler forget what it knows about a register-resident chunk, so that each pass re-derives the widened
+// values from the packed registers instead of keeping both copies alive (which would halve the occupancy).
+__device__ __forceinline__ void opaque(vec16 &v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void store16(vec16 *p, const vec16 &v) { __builtin_nontemporal_store(v, p); }
+
+// Splits a row that starts at an arbitrary element address into [head scalars][16-byte chunks][tail scalars].
+template <typename T>
+struct RowSplit {
+    int head, nvec, tail;
+    __device__ RowSplit(const T *row, int V) {
+        constexpr int EPV = Elem<T>::EPV;
+        uintptr_t a = reinterpret_cast<uintptr_t>(row);
+        int h = (int)(((16 - (a & 15)) & 15) / sizeof(T));
+        head = h < V ? h : V;
+        nvec = (V - head) / EPV;
+        tail = V - head - nvec * EPV;
+    }
+    // element handled as a scalar by thread `tid` (at most one per thread), or -1
+    __device__ int edge_pos(int tid) const {
+        if (tid < head) return tid;
+        if (tid < head + tail) return head + nvec * Elem<T>::EPV + (tid - head);
+        return -1;
+    }
+};
+
+template <typename CT, int NW>
+__device__ __forceinline__ CT block_max(CT v, CT *slots, int wave, int lane) {
+    v = wave_max(v);
+    if (lane == 0) slots[wave] = v;
+    __syncthreads();
+    CT r = slots[0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) r = vmax(r, slots[w]);
+    return r;
+}
+template <typename CT, int NW>
+__device__ __forceinline__ CT block_sum(CT v, CT *slots, int wave, int lane) {
+    v = wave_sum(v);
+    if (lane == 0) slots[wave] = v;
+    __syncthreads();
+    CT r = slots[0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) r += slots[w];
+    return r;
+}
+
+// NT threads; up to MAXC 16-byte chunks per thread stay in registers, GMAX gathered targets per thread.
+template <typename T, int NT, int MAXC, int GMAX, bool GRAD>
+__global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const int64_t *__restrict__ idx, int64_t sb,
+                                                     int64_t sl, int64_t st,
+                                                     typename Elem<T>::compute *__restrict__ sel, int64_t rows, int L,
+                                                     int V, int Tn) {
+    using CT = typename Elem<T>::compute;
+    constexpr int EPV = Elem<T>::EPV;
+    constexpr int NW = NT / 64;
+    __shared__ CT s_max[NW];
+    __shared__ CT s_sum[NW];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        T *xr = x + row * (int64_t)V;
+        const RowSplit<T> sp(xr, V);
+        const vec16 *xv = reinterpret_cast<const vec16 *>(xr + sp.head);
+
+        // gathered logits first: they must be read before this workgroup overwrites the row
+        CT gv[GMAX];
+        {
+            const int64_t b = row / L, p = row % L;
+            const int64_t *ir = idx + b * sb + p * sl;
+#pragma unroll
+            for (int g = 0; g < GMAX; g++) {
+                int s = tid + g * NT;
+                gv[g] = 0;
+                if (s < Tn) {
+                    int64_t t = ir[(int64_t)s * st];
+                    gv[g] = ((uint64_t)t < (uint64_t)V) ? Elem<T>::widen(xr[t]) : (CT)NAN;
+                }
+            }
+        }
+        vec16 buf[MAXC];
+#pragma unroll
+        for (int i = 0; i < MAXC; i++) {
+            int c = tid + i * NT;
+            if (c < sp.nvec) buf[i] = load16(xv + c);
+        }
+        const int ep = sp.edge_pos(tid);
+        CT edge = neg_inf(CT());
+        if (ep >= 0) edge = Elem<T>::widen(xr[ep]);
+
+        // ---- max
+        CT mx = edge;
+#pragma unroll
+        for (int i = 0; i < MAXC; i++) {
+            if (tid + i * NT < sp.nvec) {
+                CT v[EPV];
+                Elem<T>::unpack(buf[i], v);
+#pragma unroll
+                for (int e = 0; e < EPV; e++) mx = vmax(mx, v[e]);
+            }
+        }
+        for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
+            CT v[EPV];
+            Elem<T>::unpack(load16(xv + c), v);
+#pragma unroll
+            for (int e = 0; e < EPV; e++) mx = vmax(mx, v[e]);
+        }
+        mx = block_max<CT, NW>(mx, s_max, wave, lane);
+#pragma unroll
+        for (int i = 0; i < MAXC; i++) opaque(buf[i]);
+
+        // ---- sum of exp
+        CT sum = (ep >= 0) ? fast_exp(edge - mx) : (CT)0;
+#pragma unroll
+        for (int i = 0; i < MAXC; i++) {
+            if (tid + i * NT < sp.nvec) {
+                CT v[EPV];
+                Elem<T>::unpack(buf[i], v);
+#pragma unroll
+                for (int e = 0; e < EPV; e++) sum += fast_exp(v[e] - mx);
+            }
+        }
+        for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
+            CT v[EPV];
+            Elem<T>::unpack(load16(xv + c), v);
+#pragma unroll
+            for (int e = 0; e < EPV; e++) sum += fast_exp(v[e] - mx);
+        }
+        sum = block_sum<CT, NW>(sum, s_sum, wave, lane);
+        const CT lg = fast_log(sum);
+#pragma unroll
+        for (int i = 0; i < MAXC; i++) opaque(buf[i]);
+
+#pragma unroll
+        for (int g = 0; g < GMAX; g++) {
+            int s = tid + g * NT;
+            if (s < Tn) sel[row * (int64_t)Tn + s] = (gv[g] - mx) - lg;
+        }
+
+        if (GRAD) {
+            const CT inv = (CT)1 / sum;
+            vec16 *xw = reinterpret_cast<vec16 *>(xr + sp.head);
+#pragma unroll
+            for (int i = 0; i < MAXC; i++) {
+                int c = tid + i * NT;
+                if (c < sp.nvec) {
+                    CT v[EPV];
+                    Elem<T>::unpack(buf[i], v);
+#pragma unroll
+                    for (int e = 0; e < EPV; e++) v[e] = fast_exp(v[e] - mx) * inv;
+                    store16(xw + c, Elem<T>::pack(v));
+                }
+            }
+            for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
+                CT v[EPV];
+                Elem<T>::unpack(load16(xv + c), v);
+#pragma unroll
+                for (int e = 0; e < EPV; e++) v[e] = fast_exp(v[e] - mx) * inv;
+                store16(xw + c, Elem<T>::pack(v));
+            }
+            if (ep >= 0) xr[ep] = Elem<T>::narrow(fast_exp(edge - mx) * inv);
+        }
+    }
+}
+
+// In-place backward.  TCAP = most targets per row handled through LDS.
+template <typename T, int NT, int TCAP>
+__global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const int64_t *__restrict__ idx, int64_t sb,
+                                                     int64_t sl, int64_t st,
+                                                     const typename Elem<T>::compute *__restrict__ gsel, int64_t rows,
+                                                     int L, int V, int Tn) {
+    using CT = typename Elem<T>::compute;
+    constexpr int EPV = Elem<T>::EPV;
+    __shared__ int s_idx[TCAP];
+    __shared__ CT s_g[TCAP];   // cast(g[s]) in the buffer's dtype, widened again
+    __shared__ CT s_p[TCAP];   // original probability at idx[s]
+    const int tid = threadIdx.x, lane = tid & 63;
+
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        T *pr = p + row * (int64_t)V;
+        const CT *gr = gsel + row * (int64_t)Tn;
+        const int64_t b = row / L, q = row % L;
+        const int64_t *ir = idx + b * sb + q * sl;
+
+        // -(sum_s g) rounded to the buffer dtype (pcfg_loss.py:176), computed redundantly by every wave
+        CT part = 0;
+        for (int s = lane; s < Tn; s += 64) part += gr[s];
+        const CT ns = Elem<T>::widen(Elem<T>::narrow(-wave_sum(part)));
+
+        for (int s = tid; s < Tn; s += NT) {
+            int64_t t = ir[(int64_t)s * st];
+            bool ok = (uint64_t)t < (uint64_t)V;
+            s_idx[s] = ok ? (int)t : -1;
+            s_g[s] = Elem<T>::widen(Elem<T>::narrow(gr[s]));
+            s_p[s] = ok ? Elem<T>::widen(pr[t]) : (CT)0;
+        }
+        __syncthreads();  // every original value at a target column is now in LDS
+
+        const RowSplit<T> sp(pr, V);
+        vec16 *pv = reinterpret_cast<vec16 *>(pr + sp.head);
+        for (int c = tid; c < sp.nvec; c += NT) {
+            CT v[EPV];
+            Elem<T>::unpack(load16(pv + c), v);
+#pragma unroll
+            for (int e = 0; e < EPV; e++) v[e] = v[e] * ns;
+            store16(pv + c, Elem<T>::pack(v));
+        }
+        const int ep = sp.edge_pos(tid);
+        if (ep >= 0) pr[ep] = Elem<T>::narrow(Elem<T>::widen(pr[ep]) * ns);
+
+        // scatter_add_ (pcfg_loss.py:177): the first occurrence of a column accumulates all its duplicates in order
+        CT fix[(TCAP + NT - 1) / NT];
+        bool lead[(TCAP + NT - 1) / NT];
+#pragma unroll
+        for (int r = 0; r < (TCAP + NT - 1) / NT; r++) {
+            int s = tid + r * NT;
+            lead[r] = false;
+            fix[r] = 0;
+            if (s < Tn && s_idx[s] >= 0) {
+                const int my = s_idx[s];
+                bool first = true;
+                for (int u = 0; u < s; u++) first = first && (s_idx[u] != my);
+                if (first) {
+                    CT v = Elem<T>::widen(Elem<T>::narrow(s_p[s] * ns));
+                    for (int u = s; u < Tn; u++)
+                        if (s_idx[u] == my) v = Elem<T>::widen(Elem<T>::narrow(v + s_g[u]));
+                    fix[r] = v;
+                    lead[r] = true;
+                }
+            }
+        }
+        __threadfence();
+        __syncthreads();  // the streamed row is complete before the target columns are patched
+#pragma unroll
+        for (int r = 0; r < (TCAP + NT - 1) / NT; r++) {
+            int s = tid + r * NT;
+            if (lead[r]) pr[s_idx[s]] = Elem<T>::narrow(fix[r]);
+        }
+        __syncthreads();  // LDS is reused by the next row
+    }
+}
+
+template <typename T>
+int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, void *sel, int grad, int64_t rows,
+               int L, int V, int Tn, hipStream_t stream) {
+    using CT = typename Elem<T>::compute;
+    constexpr int NT = 512;
+    // 10 chunks x 512 threads x 16 B = 80 KB of a row in registers: a 40k-entry fp16 row exactly, half of an fp32 one.
+    constexpr int MAXC = 10;
+    constexpr int GMAX = 2;
+    if (Tn > NT * GMAX) return fail(PCFGNAT_EUNSUPPORTED, "logsoftmax_gather: T=%d exceeds %d targets per row", Tn, NT * GMAX);
+    int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
+    if (grad)
+        hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, true>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)x, idx, sb,
+                           sl, st, (CT *)sel, rows, L, V, Tn);
+    else
+        hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, false>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)x, idx,
+                           sb, sl, st, (CT *)sel, rows, L, V, Tn);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
+template <typename T>
+int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, const void *g, int64_t rows, int L, int V,
+               int Tn, hipStream_t stream) {
+    using CT = typename Elem<T>::compute;
+    constexpr int NT = 512;
+    constexpr int TCAP = 1024;
+    if (Tn > TCAP) return fail(PCFGNAT_EUNSUPPORTED, "logsoftmax_gather_backward: T=%d exceeds %d targets per row", Tn, TCAP);
+    int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
+    hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, TCAP>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,
+                       (const CT *)g, rows, L, V, Tn);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
+int check_common(const void *x, const int64_t *idx, const void *o, int64_t B, int64_t L, int64_t V, int64_t T) {
+    PCFGNAT_REQUIRE(B >= 0 && L >= 0 && V >= 1 && T >= 0, "logsoftmax_gather: negative or empty dimension (B=%lld L=%lld V=%lld T=%lld)",
+                    (long long)B, (long long)L, (long long)V, (long long)T);
+    PCFGNAT_REQUIRE(V < (1LL << 31) && T < (1LL << 31) && L < (1LL << 31), "logsoftmax_gather: V, T, L must fit in int32");
+    if (B * L == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(x != nullptr && o != nullptr && (idx != nullptr || T == 0), "logsoftmax_gather: null pointer");
+    return PCFGNAT_OK;
+}
+
+}  // namespace
+}  // namespace pcfgnat
+
+using namespace pcfgnat;
+
+extern "C" int pcfgnat_logsoftmax_gather(void *word_ins_out, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl,
+                                         int64_t st, void *selected, int require_grad, int64_t B, int64_t L, int64_t V,
+                                         int64_t T, void *stream) {
+    int rc = check_common(word_ins_out, select_idx, selected, B, L, V, T);
+    if (rc != PCFGNAT_OK) return rc;
+    if (B * L == 0) return PCFGNAT_OK;
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case PCFGNAT_F16:
+            return launch_fwd<__half>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, s);
+        case PCFGNAT_F32:
+            return launch_fwd<float>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, s);
+        case PCFGNAT_F64:
+            return launch_fwd<double>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, s);
+        default:
+            return fail(PCFGNAT_EINVAL, "logsoftmax_gather: unknown dtype code %d (float16, float32, float64 are dispatched)", dtype);
+    }
+}
+
+extern "C" int pcfgnat_logsoftmax_gather_backward(void *probs_inout, int dtype, const int64_t *select_idx, int64_t sb,
+                                                  int64_t sl, int64_t st, const void *grad_selected, int64_t B, int64_t L,
+                                                  int64_t V, int64_t T, void *stream) {
+    int rc = check_common(probs_inout, select_idx, grad_selected, B, L, V, T);
+    if (rc != PCFGNAT_OK) return rc;
+    if (B * L == 0) return PCFGNAT_OK;
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case PCFGNAT_F16:
+            return launch_bwd<__half>(probs_inout, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, s);
+        case PCFGNAT_F32:
+            return launch_bwd<float>(probs_inout, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, s);
+        case PCFGNAT_F64:
+            return launch_bwd<double>(probs_inout, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, s);
+        default:
+            return fail(PCFGNAT_EINVAL, "logsoftmax_gather_backward: unknown dtype code %d", dtype);
+    }
+}

@@ -1,0 +1,249 @@
+// Viterbi (max-product) tables per output length with back-pointers, and the tree-to-sequence readout.
+//
+// Replaces the reference's pcfg_viterbi.cu (calculate_C_kernel :177-241, calculate_S_kernel :22-140) and the
+// host loop viterbi_decoding (pcfg_loss.cpp:12-73), for max_left = 1.
+//
+// S[a][len] = ob[a] + max over (c >= a, j in {0,1}) of links[a][j][c] + C[j] + S[c][len-j-1], with C[0] = 0 (null left
+// child) and C[1] = ob[a-1] (the local leaf).  Every candidate is evaluated as ((links + C) + S) + ob in fp32, the
+// reference's association order, so table values and arg-max decisions are reproducible bit for bit; exact ties
+// follow the reference's 4-lane strided scan (lane priority 0 > 2 > 1 > 3, then c ascending, then j ascending).
+//
+// Same sweep shape as the inside forward: one workgroup per sentence, one 16-lane DPP row per parent node, link
+// slabs in registers, one barrier per length.
+#include "common.hip.h"
+
+namespace pcfgnat {
+namespace {
+
+constexpr int NT = 1024;
+
+__device__ __forceinline__ int tie_key(int rel_c, int j) {
+    const int lane = rel_c & 3;
+    const int rank = (lane == 0) ? 0 : (lane == 2) ? 1 : (lane == 1) ? 2 : 3;
+    return (rank << 24) | (rel_c << 1) | j;
+}
+
+__device__ __forceinline__ void take_better(float &best, int &key, float ov, int ok) {
+    if (ov > best || (ov == best && ok < key)) {
+        best = ov;
+        key = ok;
+    }
+}
+
+template <int CTRL>
+__device__ __forceinline__ void row16_argmax_step(float &best, int &key) {
+    const float ov = dpp_f<CTRL>(best);
+    const int ok = dpp_i<CTRL>(key);
+    take_better(best, key, ov, ok);
+}
+
+__device__ __forceinline__ float nan_to_ninf(float v) { return (v != v) ? NEG_INF_F : v; }
+
+template <int R>
+__global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict__ ob_lprob, const float *__restrict__ links,
+                                                        const int64_t *__restrict__ out_len, float *__restrict__ S,
+                                                        int64_t *__restrict__ Rt, int64_t *__restrict__ Lt, int64_t *__restrict__ Mt,
+                                                        int L, int Lq) {
+    constexpr int CN = 4 * R;
+    constexpr int MP = 64 * R;
+    __shared__ float col[2 * MP];
+    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j16 = tid & 15;
+    const int m = (int)out_len[b];
+    const float *ob = ob_lprob + (size_t)b * L;
+    const float *lk = links + (size_t)b * L * 2 * L;
+    const size_t tab = (size_t)b * L * Lq;
+    float *Sb = S + tab;
+    int64_t *Rb = Rt + tab, *Lb = Lt + tab, *Mb = Mt + tab;
+
+    // tables start as -inf / 0 (pcfg_viterbi.cu:159, 287-289)
+    for (size_t i = tid; i < (size_t)L * Lq; i += NT) {
+        Sb[i] = NEG_INF_F;
+        Rb[i] = 0;
+        Lb[i] = 0;
+        Mb[i] = 0;
+    }
+    if (m < 2 || m > L || (m % 2) != 0) return;  // out of contract: leave the empty tables
+    const int mc = m / 2;
+
+    float A0[R][CN], A1[R][CN], ob_a[R], ob_leaf[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int a_id = gidx + 64 * r, a = 2 * a_id + 1;
+        ob_a[r] = (a_id < mc) ? ob[a] : NEG_INF_F;
+        ob_leaf[r] = (a_id < mc && a_id >= 1) ? ob[a - 1] : NEG_INF_F;
+#pragma unroll
+        for (int q = 0; q < CN; q++) {
+            const int c_id = j16 + 16 * q, c = 2 * c_id + 1;
+            const bool ok = a_id < mc && c_id < mc && c_id >= a_id;
+            A0[r][q] = ok ? lk[((size_t)a * 2 + 0) * L + c] : NEG_INF_F;
+            A1[r][q] = (ok && a_id >= 1) ? lk[((size_t)a * 2 + 1) * L + c] : NEG_INF_F;
+        }
+    }
+    // length 1: only the last node (pcfg_viterbi.cu:57-59)
+    for (int i = tid; i < MP; i += NT) col[1 * MP + i] = (i == mc - 1) ? ob[m - 1] : NEG_INF_F;
+    float sc2[CN];
+#pragma unroll
+    for (int q = 0; q < CN; q++) sc2[q] = NEG_INF_F;  // S[c][0] = -inf
+    __threadfence();
+    __syncthreads();
+    if (tid == 0 && Lq > 1) Sb[(size_t)(m - 1) * Lq + 1] = ob[m - 1];
+
+    const int len_end = m / 4;  // pcfg_viterbi.cu:67
+    for (int len = 2; len < len_end; len++) {
+        const float *cur = col + ((len - 1) & 1) * MP;
+        float *nxt = col + (len & 1) * MP;
+        float sc1[CN];
+#pragma unroll
+        for (int q = 0; q < CN; q++) sc1[q] = cur[j16 + 16 * q];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int a_id = gidx + 64 * r;
+            float best = NEG_INF_F;
+            int key = 0x7fffffff;
+#pragma unroll
+            for (int q = 0; q < CN; q++) {
+                const int rel = j16 + 16 * q - a_id;
+                const float c0 = nan_to_ninf(((A0[r][q] + 0.f) + sc1[q]) + ob_a[r]);
+                const float c1 = nan_to_ninf(((A1[r][q] + ob_leaf[r]) + sc2[q]) + ob_a[r]);
+                if (c0 != NEG_INF_F) take_better(best, key, c0, tie_key(rel, 0));
+                if (c1 != NEG_INF_F) take_better(best, key, c1, tie_key(rel, 1));
+            }
+            row16_argmax_step<DPP_QUAD_XOR1>(best, key);
+            row16_argmax_step<DPP_QUAD_XOR2>(best, key);
+            row16_argmax_step<DPP_ROW_HALF_MIRROR>(best, key);
+            row16_argmax_step<DPP_ROW_MIRROR>(best, key);
+            if (j16 == 0) {
+                nxt[a_id] = best;
+                if (best != NEG_INF_F && a_id < mc) {  // pcfg_viterbi.cu:125-131
+                    const int a = 2 * a_id + 1;
+                    const int jj = key & 1, rel = (key >> 1) & 0x7fffff;
+                    const size_t o = (size_t)a * Lq + len;
+                    Sb[o] = best;
+                    Lb[o] = jj ? (a - 1) : 0;
+                    Rb[o] = 2 * (a_id + rel) + 1;
+                    Mb[o] = jj;
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < CN; q++) sc2[q] = sc1[q];
+        __syncthreads();
+    }
+}
+
+// One walk per sentence (pcfg_loss.cpp:22-59).  Shared by the device kernel and the host entry point.
+__host__ __device__ inline int64_t readout_one(int64_t pred_len, int64_t max_h, const int64_t *Li, const int64_t *Ri,
+                                               const int64_t *Mi, const int64_t *tok, const int64_t *mask, int64_t mask_dim,
+                                               int64_t pad, int64_t *out, int64_t *stack_node, int64_t *stack_len, int L, int Lq) {
+    const int cap = L;
+    int sp = 0;
+    int64_t cnt = 0, node = 1, len = pred_len, last = -1;
+    if (len < 0 || len >= Lq) return -1;
+    int64_t budget = (int64_t)L * Lq + L;  // well-formed traces visit each (node, len) cell at most once
+    while ((node < max_h && node != 0) || sp > 0) {
+        if (--budget < 0) return -1;
+        while (node < max_h && node != 0) {
+            if (sp >= cap || node < 0 || node >= L || len < 0 || len >= Lq) return -1;
+            stack_node[sp] = node;
+            stack_len[sp] = len;
+            sp++;
+            int64_t l = Li[node * Lq + len];
+            l = (l == node) ? 0 : l;
+            if (l < 0 || l >= mask_dim || node >= mask_dim) return -1;
+            if (mask[node * mask_dim + l]) break;
+            const int64_t nl = Mi[node * Lq + len];
+            node = l;
+            len = nl;
+        }
+        sp--;
+        node = stack_node[sp];
+        len = stack_len[sp];
+        const int64_t t = tok[node];
+        if (t != pad && t != last) {
+            last = t;
+            if (cnt >= cap) return -1;
+            out[cnt++] = t;
+        }
+        const int64_t r = Ri[node * Lq + len];
+        const int64_t nl = len - Mi[node * Lq + len] - 1;
+        node = r;
+        len = nl;
+    }
+    return cnt;
+}
+
+__global__ void readout_kernel(const int64_t *pred_length, const int64_t *output_length, const int64_t *Lt, const int64_t *Rt,
+                               const int64_t *Mt, const int64_t *tokens, const int64_t *mask, int64_t mask_dim, int64_t pad,
+                               int64_t *out_tokens, int64_t *out_count, int64_t *scratch, int B, int L, int Lq) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= B) return;
+    int64_t *out = out_tokens + (size_t)i * L;
+    for (int k = 0; k < L; k++) out[k] = pad;
+    const size_t tab = (size_t)i * L * Lq;
+    int64_t *stack_node = scratch + (size_t)i * 2 * L, *stack_len = stack_node + L;
+    out_count[i] = readout_one(pred_length[i], output_length[i], Lt + tab, Rt + tab, Mt + tab, tokens + (size_t)i * L, mask, mask_dim,
+                               pad, out, stack_node, stack_len, L, Lq);
+}
+
+}  // namespace
+}  // namespace pcfgnat
+
+using namespace pcfgnat;
+
+extern "C" int pcfgnat_pcfg_viterbi(const float *ob_lprob, const float *links, const int64_t *output_length, float *S, int64_t *R,
+                                    int64_t *Lt, int64_t *M, int64_t B, int64_t L, int64_t ml, void *stream) {
+    PCFGNAT_REQUIRE(B >= 0 && L >= 4, "pcfg_viterbi: need B >= 0 and L >= 4 (got B=%lld L=%lld)", (long long)B, (long long)L);
+    if (ml != 1)
+        return fail(PCFGNAT_EUNSUPPORTED, "pcfg_viterbi: max_left = %lld; only max_left = 1 (--left-tree-layer 1) is built", (long long)ml);
+    PCFGNAT_REQUIRE(L / 4 > ml, "pcfg_viterbi: L/4 must exceed max_left");
+    if (B == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(ob_lprob && links && output_length && S && R && Lt && M, "pcfg_viterbi: null pointer");
+    const int Mc = (int)((L - 2) / 2 + 1);
+    const int Lq = (int)(L / 4);
+    hipStream_t s = (hipStream_t)stream;
+    if (Mc <= 64)
+        hipLaunchKernelGGL((viterbi_ml1_kernel<1>), dim3((unsigned)B), dim3(NT), 0, s, ob_lprob, links, output_length, S, R, Lt, M, (int)L, Lq);
+    else if (Mc <= 128)
+        hipLaunchKernelGGL((viterbi_ml1_kernel<2>), dim3((unsigned)B), dim3(NT), 0, s, ob_lprob, links, output_length, S, R, Lt, M, (int)L, Lq);
+    else
+        return fail(PCFGNAT_EUNSUPPORTED, "pcfg_viterbi: graph size L=%lld exceeds the built limit of 256 nodes", (long long)L);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
+extern "C" int pcfgnat_viterbi_decoding(const int64_t *pred_length, const int64_t *output_length, const int64_t *Lt, const int64_t *R,
+                                        const int64_t *M, const int64_t *tokens, const int64_t *left_tree_mask, int64_t mask_dim,
+                                        int64_t pad_index, int64_t *out_tokens, int64_t *out_count, int64_t *scratch, int64_t B,
+                                        int64_t L, int64_t Lq, void *stream) {
+    PCFGNAT_REQUIRE(B >= 0 && L >= 1 && Lq >= 1 && mask_dim >= 1, "viterbi_decoding: bad dimensions");
+    if (B == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(pred_length && output_length && Lt && R && M && tokens && left_tree_mask && out_tokens && out_count && scratch,
+                    "viterbi_decoding: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    const int threads = 64;
+    hipLaunchKernelGGL(readout_kernel, dim3((unsigned)((B + threads - 1) / threads)), dim3(threads), 0, s, pred_length, output_length, Lt,
+                       R, M, tokens, left_tree_mask, mask_dim, pad_index, out_tokens, out_count, scratch, (int)B, (int)L, (int)Lq);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
+extern "C" int pcfgnat_viterbi_decoding_host(const int64_t *pred_length, const int64_t *output_length, const int64_t *Lt,
+                                             const int64_t *R, const int64_t *M, const int64_t *tokens, const int64_t *left_tree_mask,
+                                             int64_t mask_dim, int64_t pad_index, int64_t *out_tokens, int64_t *out_count, int64_t B,
+                                             int64_t L, int64_t Lq) {
+    PCFGNAT_REQUIRE(B >= 0 && L >= 1 && Lq >= 1 && mask_dim >= 1, "viterbi_decoding: bad dimensions");
+    if (B == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(pred_length && output_length && Lt && R && M && tokens && left_tree_mask && out_tokens && out_count,
+                    "viterbi_decoding: null pointer");
+    int64_t *stack = (int64_t *)malloc(sizeof(int64_t) * 2 * (size_t)L);
+    if (!stack) return fail(PCFGNAT_EINVAL, "viterbi_decoding: out of host memory");
+    for (int64_t i = 0; i < B; i++) {
+        int64_t *out = out_tokens + (size_t)i * L;
+        for (int64_t k = 0; k < L; k++) out[k] = pad_index;
+        const size_t tab = (size_t)i * L * Lq;
+        out_count[i] = readout_one(pred_length[i], output_length[i], Lt + tab, R + tab, M + tab, tokens + (size_t)i * L, left_tree_mask,
+                                   mask_dim, pad_index, out, stack, stack + L, (int)L, (int)Lq);
+    }
+    free(stack);
+    return PCFGNAT_OK;
+}

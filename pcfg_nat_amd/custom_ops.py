@@ -1,0 +1,343 @@
+"""Operator API of the structured-loss path, signature-compatible with the reference's
+``fs_plugins/custom_ops/pcfg_loss.py`` (exports of ``fs_plugins/custom_ops/__init__.py:1``):
+
+    cuda_pcfg_loss, cuda_pcfg_best_tree, cuda_pcfg_viterbi, dag_logsoftmax_gather_inplace, viterbi_decoding
+
+The autograd Functions keep the reference's names, argument order, class attributes, return order and in-place
+contract; the arithmetic runs in hand-written HIP kernels for gfx950 reached through the C-ABI of
+``libpcfg_nat_hip.so`` on the current HIP stream.  There is no CPU path: calling with CPU tensors (other than
+``viterbi_decoding``, whose reference version is itself a host loop) raises.
+"""
+import torch
+from torch.autograd import Function
+
+from . import _lib
+
+_DTYPE_CODE = {torch.float16: _lib.F16, torch.float32: _lib.F32, torch.float64: _lib.F64}
+
+
+def get_pcfg_kernel():
+    """Loader with the reference's name (pcfg_loss.py:18-47).  Returns the ctypes library handle."""
+    if not torch.cuda.is_available():
+        raise RuntimeError("You need GPU to use the custom cuda operations")
+    return _lib.load()
+
+
+def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _need_cuda(name, *tensors):
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("%s: expected tensors on the GPU, got a %s tensor" % (name, t.device.type))
+    dev = tensors[0].device
+    for t in tensors[1:]:
+        if t.device != dev:
+            raise RuntimeError("%s: tensors are on different devices (%s vs %s)" % (name, dev, t.device))
+
+
+def _lengths(name, t, batch):
+    if t.dim() != 1 or t.size(0) != batch:
+        raise RuntimeError("%s: length tensor must have shape [%d], got %s" % (name, batch, tuple(t.shape)))
+    if t.dtype != torch.int64:
+        raise RuntimeError("%s: lengths should be long" % name)
+    return t.contiguous()
+
+
+def _check_pcfg_inputs(name, match_all, links, output_length, target_length):
+    _need_cuda(name, match_all, links, output_length, target_length)
+    if match_all.dim() != 3:
+        raise RuntimeError("%s: match_all dim != 3" % name)
+    if links.dim() != 4:
+        raise RuntimeError("%s: links dim != 4" % name)
+    B, L, T = match_all.shape
+    if links.size(0) != B or links.size(1) != L or links.size(3) != L:
+        raise RuntimeError("%s: links must be [bsz, prelen, max_left+1, prelen] = [%d, %d, *, %d], got %s"
+                           % (name, B, L, L, tuple(links.shape)))
+    if match_all.dtype != torch.float32 or links.dtype != torch.float32:
+        raise RuntimeError("%s: match_all and links must be float32 (got %s, %s)" % (name, match_all.dtype, links.dtype))
+    return B, L, T, links.size(2) - 1
+
+
+def _pcfg_loss_tables(match_all, links, output_length, target_length, config, name):
+    """pcfg_loss (pcfg_loss.cu:379-401): returns (S [B,Mc,T+2], aux)."""
+    if not (1 <= config <= 4):
+        raise RuntimeError("config should be 1~4")
+    lib = get_pcfg_kernel()
+    B, L, T, ml = _check_pcfg_inputs(name, match_all, links, output_length, target_length)
+    output_length = _lengths(name, output_length, B)
+    target_length = _lengths(name, target_length, B)
+    Mc = (L - 2) // (ml + 1) + 1
+    with torch.cuda.device(match_all.device):
+        S = torch.empty((B, Mc, T + 2), dtype=torch.float32, device=match_all.device)
+        aux = torch.empty((max(1, lib.pcfgnat_pcfg_aux_floats(B, L, T, ml)),), dtype=torch.float32, device=match_all.device)
+        _lib.check(lib.pcfgnat_pcfg_loss(match_all.data_ptr(), links.data_ptr(), output_length.data_ptr(),
+                                         target_length.data_ptr(), S.data_ptr(), aux.data_ptr(), B, L, T, ml,
+                                         _stream(match_all)), lib)
+    return S, aux, output_length, target_length
+
+
+def _pcfg_loss_backward(grad_output, S, aux, match_all, links, output_length, target_length, config):
+    """pcfg_loss_backward (pcfg_loss_backward.cu:654-721)."""
+    if not (1 <= config <= 4):
+        raise RuntimeError("config should be 1~4")
+    lib = get_pcfg_kernel()
+    B, L, T = match_all.shape
+    ml = links.size(2) - 1
+    with torch.cuda.device(match_all.device):
+        match_all_grad = torch.empty_like(match_all)
+        links_grad = torch.empty_like(links)
+        _lib.check(lib.pcfgnat_pcfg_loss_backward(grad_output.data_ptr(), S.data_ptr(), aux.data_ptr(),
+                                                  match_all.data_ptr(), links.data_ptr(), output_length.data_ptr(),
+                                                  target_length.data_ptr(), match_all_grad.data_ptr(),
+                                                  links_grad.data_ptr(), B, L, T, ml, _stream(match_all)), lib)
+    return match_all_grad, links_grad
+
+
+class CUDAPCFGLossFunc(Function):
+    """Inside-algorithm log-likelihood (reference: pcfg_loss.py:49-85)."""
+    config = 1
+    config1 = 1
+    config2 = 1
+
+    @staticmethod
+    def forward(
+        ctx,
+        match_all,      # bsz * prelen * tarlen
+        links,          # bsz * prelen * (max_left+1) * prelen
+        output_length,  # bsz
+        target_length,  # bsz
+    ):
+        batch_size = match_all.shape[0]
+        require_gradient = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        match_all = match_all.contiguous()
+        links = links.contiguous()
+        S, aux, ol, tl = _pcfg_loss_tables(match_all, links, output_length, target_length, CUDAPCFGLossFunc.config,
+                                           "cuda_pcfg_loss")
+        if require_gradient:
+            # like the reference (pcfg_loss.py:71-73) the backward sweep runs eagerly with a unit upstream gradient
+            ones = torch.ones((batch_size,), dtype=S.dtype, device=S.device)
+            match_all_grad, links_grad = _pcfg_loss_backward(ones, S, aux, match_all, links, ol, tl,
+                                                             CUDAPCFGLossFunc.config)
+            ctx.save_for_backward(match_all_grad, links_grad)
+        return S[:, 0, 0].clone()
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+            match_all_grad, links_grad = ctx.saved_tensors
+            batch_size = match_all_grad.shape[0]
+            return (match_all_grad * grad_output.view(batch_size, 1, 1),
+                    links_grad * grad_output.view(batch_size, 1, 1, 1), None, None)
+        return None, None, None, None
+
+
+cuda_pcfg_loss = CUDAPCFGLossFunc.apply
+
+
+class CUDAPCFGBestTreeFunc(Function):
+    """GLAT alignment: greedy top-down trace over the inside tables (reference: pcfg_loss.py:89-117)."""
+    config = 1
+
+    @staticmethod
+    def forward(
+        ctx,
+        match_all,      # bsz * prelen * tarlen
+        links,          # bsz * prelen * (max_left+1) * prelen
+        output_length,  # bsz
+        target_length,  # bsz
+    ):
+        match_all = match_all.contiguous()
+        links = links.contiguous()
+        S, aux, ol, tl = _pcfg_loss_tables(match_all, links, output_length, target_length,
+                                           CUDAPCFGBestTreeFunc.config, "cuda_pcfg_best_tree")
+        lib = get_pcfg_kernel()
+        B, L, T = match_all.shape
+        ml = links.size(2) - 1
+        with torch.cuda.device(match_all.device):
+            tree = torch.empty((B, L), dtype=torch.int64, device=match_all.device)
+            _lib.check(lib.pcfgnat_pcfg_best_tree(S.data_ptr(), aux.data_ptr(), match_all.data_ptr(), links.data_ptr(),
+                                                  ol.data_ptr(), tl.data_ptr(), tree.data_ptr(), B, L, T, ml,
+                                                  _stream(match_all)), lib)
+        ctx.mark_non_differentiable(tree)
+        return tree, S[:, 0, 0].clone()
+
+    @staticmethod
+    def backward(ctx, grad_tree, grad_output):
+        return None, None, None, None
+
+
+cuda_pcfg_best_tree = CUDAPCFGBestTreeFunc.apply
+
+
+class CUDAPCFGViterbiFunc(Function):
+    """Max-product tables per output length (reference: pcfg_loss.py:119-142).  Returns (scores, R, L, M)."""
+    config = 1
+
+    @staticmethod
+    def forward(
+        ctx,
+        ob_lprob,       # bsz * prelen
+        links,          # bsz * prelen * (max_left+1) * prelen
+        output_length,  # bsz
+    ):
+        # the reference reads CUDAPCFGBestTreeFunc.config here (pcfg_loss.py:133); kept
+        if not (1 <= CUDAPCFGBestTreeFunc.config <= 4):
+            raise RuntimeError("config should be 1~4")
+        lib = get_pcfg_kernel()
+        _need_cuda("cuda_pcfg_viterbi", ob_lprob, links, output_length)
+        if ob_lprob.dim() != 2 or links.dim() != 4:
+            raise RuntimeError("cuda_pcfg_viterbi: ob_lprob must be [bsz, prelen] and links [bsz, prelen, max_left+1, prelen]")
+        if ob_lprob.dtype != torch.float32 or links.dtype != torch.float32:
+            raise RuntimeError("cuda_pcfg_viterbi: ob_lprob and links must be float32 (got %s, %s)"
+                               % (ob_lprob.dtype, links.dtype))
+        B, L = ob_lprob.shape
+        if links.size(0) != B or links.size(1) != L or links.size(3) != L:
+            raise RuntimeError("cuda_pcfg_viterbi: links shape %s does not match ob_lprob %s"
+                               % (tuple(links.shape), tuple(ob_lprob.shape)))
+        ml = links.size(2) - 1
+        ob_lprob = ob_lprob.contiguous()
+        links = links.contiguous()
+        output_length = _lengths("cuda_pcfg_viterbi", output_length, B)
+        Lq = L // 4
+        with torch.cuda.device(ob_lprob.device):
+            S = torch.empty((B, L, Lq), dtype=torch.float32, device=ob_lprob.device)
+            R = torch.empty((B, L, Lq), dtype=torch.int64, device=ob_lprob.device)
+            Lt = torch.empty_like(R)
+            M = torch.empty_like(R)
+            _lib.check(lib.pcfgnat_pcfg_viterbi(ob_lprob.data_ptr(), links.data_ptr(), output_length.data_ptr(),
+                                                S.data_ptr(), R.data_ptr(), Lt.data_ptr(), M.data_ptr(), B, L, ml,
+                                                _stream(ob_lprob)), lib)
+        ctx.mark_non_differentiable(R, Lt, M)
+        return S[:, 1, :].clone(), R, Lt, M
+
+    @staticmethod
+    def backward(ctx, *grads):
+        return None, None, None
+
+
+cuda_pcfg_viterbi = CUDAPCFGViterbiFunc.apply
+
+
+class DagLogsoftmaxGatherFunc(Function):
+    """Fused log-softmax + gather with the reference's in-place contract (pcfg_loss.py:144-181): the logits buffer is
+    returned dirty (it holds softmax probabilities when a gradient is required) and becomes the gradient buffer in
+    backward, which may run once."""
+
+    @staticmethod
+    def forward(
+        ctx,
+        word_ins_out,  # bsz * prelen * vocabsize
+        select_idx,    # bsz * prelen * slen
+    ):
+        require_gradient = ctx.needs_input_grad[0]
+        selected_result = _logsoftmax_gather(word_ins_out, select_idx, require_gradient)
+        # Note: the kernel modifies word_ins_out and the backward reuses it
+        ctx.mark_dirty(word_ins_out)
+        ctx.set_materialize_grads(False)
+
+        if require_gradient:
+            ctx.save_for_backward(word_ins_out, select_idx)
+            ctx.has_backward = False
+        return word_ins_out, selected_result  # bsz * prelen * slen
+
+    @staticmethod
+    def backward(ctx, grad_word_ins_out, grad_output):
+        if not ctx.needs_input_grad[0]:
+            return None, None
+        assert grad_word_ins_out is None, "Cannot reuse word_ins_out after logsoftmax_gather"
+        if grad_output is None:
+            return None, None
+
+        assert not ctx.has_backward, "Cannot backward twice in logsoftmax_gather"
+        ctx.has_backward = True
+
+        grad_input, selected_idx = ctx.saved_tensors
+        _logsoftmax_gather_backward(grad_input, selected_idx, grad_output)
+        return grad_input, None
+
+
+dag_logsoftmax_gather_inplace = DagLogsoftmaxGatherFunc.apply
+
+
+def _logsoftmax_gather(word_ins_out, select_idx, require_gradient):
+    """logsoftmax_gather (logsoftmax_gather.cu:295-359), argument checks included (:297-309)."""
+    lib = get_pcfg_kernel()
+    _need_cuda("logsoftmax_gather", word_ins_out, select_idx)
+    if word_ins_out.dim() != 3:
+        raise RuntimeError("word_ins_out dim != 3")
+    if select_idx.dim() != 3:
+        raise RuntimeError("select_idx dim != 3")
+    B, L, V = word_ins_out.shape
+    T = select_idx.size(2)
+    if select_idx.size(0) != B:
+        raise RuntimeError("batch size not match")
+    if select_idx.size(1) != L:
+        raise RuntimeError("prelen size not match")
+    if select_idx.dtype != torch.int64:
+        raise RuntimeError("select_idx should be long")
+    if not word_ins_out.is_contiguous():
+        raise RuntimeError("word_ins_out is not contiguous")
+    code = _DTYPE_CODE.get(word_ins_out.dtype)
+    if code is None:
+        raise RuntimeError("logsoftmax_gather: unsupported dtype %s (float16, float32, float64 are dispatched)"
+                           % word_ins_out.dtype)
+    out_dtype = torch.float64 if word_ins_out.dtype == torch.float64 else torch.float32
+    with torch.cuda.device(word_ins_out.device):
+        selected = torch.empty((B, L, T), dtype=out_dtype, device=word_ins_out.device)
+        sb, sl, st = select_idx.stride()
+        _lib.check(lib.pcfgnat_logsoftmax_gather(word_ins_out.data_ptr(), code, select_idx.data_ptr(), sb, sl, st,
+                                                 selected.data_ptr(), int(bool(require_gradient)), B, L, V, T,
+                                                 _stream(word_ins_out)), lib)
+    return selected
+
+
+def _logsoftmax_gather_backward(buf, select_idx, grad_output):
+    """One fused pass for ``buf.mul_(-(sum g).to(dtype)); buf.scatter_add_(-1, idx, g.to(dtype))`` (pcfg_loss.py:176-177)."""
+    lib = get_pcfg_kernel()
+    B, L, V = buf.shape
+    T = select_idx.size(2)
+    want = torch.float64 if buf.dtype == torch.float64 else torch.float32
+    g = grad_output.to(want).contiguous()
+    with torch.cuda.device(buf.device):
+        sb, sl, st = select_idx.stride()
+        _lib.check(lib.pcfgnat_logsoftmax_gather_backward(buf.data_ptr(), _DTYPE_CODE[buf.dtype], select_idx.data_ptr(),
+                                                          sb, sl, st, g.data_ptr(), B, L, V, T, _stream(buf)), lib)
+    return buf
+
+
+def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unreduced_tokens, left_tree_mask, pad_index):
+    """Tree-to-sequence readout (reference: pcfg_loss.py:183-184 -> pcfg_loss.cpp:12-73).
+
+    Walks the (L, R, M) back-pointers from (node 1, pred_length) in order, emitting ``unreduced_tokens[node]`` unless
+    it is the pad symbol or repeats the previous emission.  Returns float32 ``[B, maxlen]`` right-padded with
+    ``pad_index`` (the reference's dtype, :65; it can only assemble rows of equal length, ragged batches get the
+    evidently intended padding).  Traces on the GPU are walked on the GPU (one thread per sentence); CPU tensors, which
+    is what the reference's caller passes, are walked by the library's host routine.
+    """
+    lib = _lib.load()
+    B, L, Lq = L_trace.shape
+    tensors = [pred_length, output_length, L_trace, R_trace, M_trace, unreduced_tokens, left_tree_mask]
+    dev = L_trace.device
+    args = [t.to(device=dev, dtype=torch.int64).contiguous() for t in tensors]
+    pl, ol, Lt, Rt, Mt, tok, mask = args
+    if mask.dim() != 2 or mask.size(0) != mask.size(1):
+        raise RuntimeError("viterbi_decoding: left_tree_mask must be square")
+    out = torch.empty((B, L), dtype=torch.int64, device=dev)
+    cnt = torch.empty((B,), dtype=torch.int64, device=dev)
+    if dev.type == "cuda":
+        with torch.cuda.device(dev):
+            scratch = torch.empty((B, 2 * L), dtype=torch.int64, device=dev)
+            _lib.check(lib.pcfgnat_viterbi_decoding(pl.data_ptr(), ol.data_ptr(), Lt.data_ptr(), Rt.data_ptr(), Mt.data_ptr(),
+                                                    tok.data_ptr(), mask.data_ptr(), mask.size(0), int(pad_index),
+                                                    out.data_ptr(), cnt.data_ptr(), scratch.data_ptr(), B, L, Lq,
+                                                    _stream(out)), lib)
+    else:
+        _lib.check(lib.pcfgnat_viterbi_decoding_host(pl.data_ptr(), ol.data_ptr(), Lt.data_ptr(), Rt.data_ptr(),
+                                                     Mt.data_ptr(), tok.data_ptr(), mask.data_ptr(), mask.size(0),
+                                                     int(pad_index), out.data_ptr(), cnt.data_ptr(), B, L, Lq), lib)
+    if B and int(cnt.min()) < 0:
+        raise RuntimeError("viterbi_decoding: malformed traces")
+    maxlen = int(cnt.max()) if B else 0
+    return out[:, :maxlen].to(torch.float32)

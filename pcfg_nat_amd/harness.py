@@ -1,0 +1,96 @@
+"""The glue the reference wraps around the ops, restated without fairseq so that the path can be driven end to end:
+
+* ``compute_pcfg_loss``   <- ``NATPCFGoss._compute_pfcg_loss``   (fs_plugins/criterions/nat_pcfg_loss.py:98-145)
+* ``glat_alignment``      <- ``glat_function``                    (fs_plugins/criterions/nat_pcfg_loss.py:193-269)
+* ``viterbi_decode``      <- the ``viterbi`` branch of ``forward_decoder``
+                             (fs_plugins/models/glat_decomposed_with_link_two_hands_tri_pcfg.py:414-416, 483-502)
+
+Each function takes the ops as a namespace argument (``ops``), by default this package's HIP-backed ones, so that tests
+can run the very same glue over the CPU oracle.
+"""
+import torch
+
+from . import custom_ops as _default_ops
+from .synth import PAD
+
+
+def eos_masked(match_all, output_length, target_length):
+    """Only the last graph node may emit the last target token (nat_pcfg_loss.py:111-115)."""
+    batch_size = match_all.shape[0]
+    eos_mask = torch.zeros_like(match_all, dtype=torch.bool)
+    rows = torch.arange(batch_size, device=match_all.device)
+    eos_mask[rows, :, target_length - 1] = True
+    eos_mask[rows, output_length - 1, target_length - 1] = False
+    return match_all.masked_fill(eos_mask, float("-inf"))
+
+
+def compute_pcfg_loss(outputs, output_masks, targets, target_masks, links, ops=_default_ops):
+    """loss = -(log-likelihood / target_length).mean() with invalid sentences zeroed (nat_pcfg_loss.py:98-145).
+    ``outputs`` [B,L,V] is consumed in place (it holds softmax probabilities afterwards and the gradient after
+    backward).  Returns a dict with ``loss``, ``ll`` (per sentence), ``invalid_nsentences``."""
+    prelen = outputs.shape[1]
+    output_length = output_masks.sum(dim=-1)
+    target_length = target_masks.sum(dim=-1)
+    outputs, match_all = ops.dag_logsoftmax_gather_inplace(outputs, targets.unsqueeze(1).expand(-1, prelen, -1))
+    match_all_eos_masked = eos_masked(match_all, output_length, target_length)
+    loss_result = ops.cuda_pcfg_loss(match_all_eos_masked, links, output_length, target_length)
+    invalid_masks = loss_result.isinf().logical_or(loss_result.isnan())
+    loss_result = loss_result.masked_fill(invalid_masks, 0)
+    loss = -(loss_result / target_length).mean()
+    return {"loss": loss, "ll": loss_result, "invalid_nsentences": invalid_masks.sum().detach(),
+            "match_all": match_all_eos_masked}
+
+
+def glat_alignment(word_ins_out, tgt_tokens, prev_output_tokens, links, context_p, pad=PAD, ops=_default_ops,
+                   generator=None):
+    """GLAT glancing with the ``number-random`` strategy (nat_pcfg_loss.py:193-269): best-tree alignment of target
+    tokens to graph nodes, then a random subset of the aligned nodes is revealed.  RNG order: ``randn`` then ``rand``."""
+    batch_size, prelen = links.shape[0], links.shape[1]
+    tarlen = tgt_tokens.shape[1]
+    target_length = (~tgt_tokens.eq(pad)).sum(1)
+    output_length = prev_output_tokens.ne(pad).sum(1)
+    pred_tokens = word_ins_out.argmax(-1)
+    word_ins_out, match = ops.dag_logsoftmax_gather_inplace(word_ins_out, tgt_tokens.unsqueeze(1).expand(-1, prelen, -1))
+    match_all_eos_masked = eos_masked(match, output_length, target_length)
+    path, max_tree_lprob = ops.cuda_pcfg_best_tree(match_all_eos_masked, links, output_length, target_length)
+    invalid_masks = max_tree_lprob.isinf().logical_or(max_tree_lprob.isnan())
+    max_tree_lprob = max_tree_lprob.masked_fill(invalid_masks, 0)
+    path = path.clone()
+    predict_align_mask = path >= 0
+    path[path + 1 >= (tarlen + 1)] = -1
+    path[path + 1 < 0] = -1
+    matchmask = torch.zeros(batch_size, tarlen + 1, prelen, device=match.device, dtype=torch.bool).scatter_(
+        1, path.unsqueeze(1) + 1, 1)[:, 1:]
+    oracle = tgt_tokens.gather(-1, path.clip(min=0))
+    same_num = ((pred_tokens == oracle) & predict_align_mask).sum(1)
+    dev = tgt_tokens.device
+    prob = torch.randn(oracle.shape, device=dev, dtype=torch.float, generator=generator)
+    prob.masked_fill_(~predict_align_mask, -100)
+    glance_nums = ((target_length - same_num) * context_p + 0.5).to(torch.long)
+    prob_thresh = prob.sort(descending=True)[0].gather(-1, (glance_nums - 1).clip(min=0).unsqueeze(-1)).squeeze(-1)
+    prob_thresh.masked_fill_(glance_nums == 0, 100)
+    keep_prob = (prob >= prob_thresh.unsqueeze(-1)).to(prob.dtype)
+    keep_word_mask = (torch.rand(prev_output_tokens.shape, device=dev, generator=generator) < keep_prob).bool()
+    glat_prev_output_tokens = prev_output_tokens.masked_fill(keep_word_mask, 0) + oracle.masked_fill(~keep_word_mask, 0)
+    return {"path": path, "matchmask": matchmask, "keep_word_mask": keep_word_mask,
+            "glat_prev_output_tokens": glat_prev_output_tokens, "same_num": same_num, "glance_nums": glance_nums,
+            "max_tree_lprob": -(max_tree_lprob / target_length).mean()}
+
+
+def viterbi_decode(unreduced_logits, unreduced_tokens, links, output_length, left_tree_mask, pad=PAD, beta=1.0,
+                   ops=_default_ops, traces_on_host=False):
+    """Viterbi decoding glue (glat_decomposed_with_link_two_hands_tri_pcfg.py:483-502): tables, length selection with the
+    ``decode_viterbibeta`` penalty, readout.  Returns (tokens float32 [B,maxlen], pred_length [B])."""
+    prelen = unreduced_logits.shape[1]
+    scores, R_trace, L_trace, M_trace = ops.cuda_pcfg_viterbi(unreduced_logits, links, output_length.long())
+    lengths = torch.arange(prelen // 4, device=scores.device).unsqueeze(0)
+    length_penalty = lengths ** beta
+    scores = scores / length_penalty
+    scores = scores.masked_fill(scores.isnan(), float("-inf"))
+    _, pred_length = torch.max(scores[:, 1:], dim=-1)
+    pred_length = pred_length + 1
+    if traces_on_host:  # what the reference does (:500)
+        R_trace, L_trace, M_trace = R_trace.cpu(), L_trace.cpu(), M_trace.cpu()
+    tokens = ops.viterbi_decoding(pred_length.long(), output_length.long(), L_trace.long(), R_trace.long(),
+                                  M_trace.long(), unreduced_tokens.long(), left_tree_mask.long(), pad)
+    return tokens.to(device=pred_length.device), pred_length

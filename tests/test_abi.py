@@ -1,0 +1,69 @@
+"""CPU-side checks of the boundary: the C-ABI library loads without a GPU, exports exactly what include/pcfg_nat_hip.h
+declares, and its host-only entry point (the tree-to-sequence readout, a CPU function in the reference as well,
+pcfg_loss.cpp:12-73) agrees with the oracle.  No GPU compute is called here."""
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle
+from pcfg_nat_amd import _lib, custom_ops, synth
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "pcfg_nat_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pcfgnat_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared()
+    assert len(names) >= 10
+    for name in names:
+        assert hasattr(lib, name), name
+        assert name in _lib.SIGNATURES, "binding table lacks %s" % name
+    assert sorted(_lib.SIGNATURES) == names
+    assert lib.pcfgnat_abi_version() == 1
+    assert lib.pcfgnat_pcfg_aux_floats(40, 128, 32, 1) == 40 * 3 * 64 * 34
+
+
+def test_argument_errors_without_gpu():
+    lib = _lib.load()
+    rc = lib.pcfgnat_pcfg_loss(None, None, None, None, None, None, 2, 16, 4, 3, None)
+    assert rc == _lib.EUNSUPPORTED and b"max_left" in lib.pcfgnat_last_error()
+    rc = lib.pcfgnat_logsoftmax_gather(None, 7, None, 0, 0, 0, None, 0, 1, 1, 8, 1, None)
+    assert rc == _lib.EINVAL
+    with pytest.raises(RuntimeError):
+        _lib.check(rc)
+
+
+def test_ops_refuse_to_run_without_gpu():
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    with pytest.raises(RuntimeError, match="GPU"):
+        custom_ops.cuda_pcfg_loss(torch.zeros(1, 8, 4), torch.zeros(1, 8, 2, 8), torch.tensor([8]), torch.tensor([4]))
+    with pytest.raises(RuntimeError, match="GPU"):
+        custom_ops.dag_logsoftmax_gather_inplace(torch.zeros(1, 8, 4), torch.zeros(1, 8, 2, dtype=torch.int64))
+
+
+def test_host_readout_matches_oracle():
+    ml, L = 1, 48
+    m = torch.tensor([48, 32, 20, 8])
+    gen = torch.Generator().manual_seed(21)
+    links = synth.make_links(4, L, m, ml, gen)
+    ob = torch.randn(4, L, generator=gen) - 1.0
+    tokens = torch.randint(0, 6, (4, L), generator=gen)  # tiny vocabulary: repeats and pads (1) occur
+    S, R, Lt, M = oracle.viterbi(ob.numpy(), links.numpy(), m.numpy(), dtype=np.float32)
+    left_mask, _, _ = synth.support_masks(L, ml)
+    for pred in ([5, 4, 3, 1], [11, 7, 2, 1], [2, 2, 2, 1]):
+        pred_t = torch.tensor(pred)
+        want = oracle.viterbi_decoding(pred_t.numpy(), m.numpy(), Lt, R, M, tokens.numpy(), left_mask.numpy(), 1)
+        got = custom_ops.viterbi_decoding(pred_t, m, torch.from_numpy(Lt), torch.from_numpy(R), torch.from_numpy(M),
+                                          tokens, left_mask, 1)
+        assert got.dtype == torch.float32
+        assert np.array_equal(got.numpy(), want)

@@ -1,0 +1,327 @@
+"""GPU parity tests: the HIP path (through the operator API, which calls the C-ABI) against the CPU oracle and torch's
+library routines on identical seeded inputs.
+
+Bars: integer outputs (trees, traces, decoded tokens) bit-exact; viterbi scores bit-exact (same fp32 association
+order); fp32 log-likelihoods within 1e-5 relative, gradients within 1e-4 of the gradient scale; fp16 buffers within
+one fp16 rounding step.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle
+from pcfg_nat_amd import custom_ops as ops
+from pcfg_nat_amd import harness, synth
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _gather_ref(x, idx):
+    return torch.log_softmax(x.float() if x.dtype != torch.float64 else x, -1).gather(-1, idx)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.float64])
+@pytest.mark.parametrize("V", [7, 512, 1001, 40000, 50257])
+def test_lsg_forward_and_inplace_softmax(dtype, V):
+    g = torch.Generator().manual_seed(V)
+    B, L, T = 3, 5, 9
+    x = (torch.randn(B, L, V, generator=g) * 2).to(dtype)
+    tgt = torch.randint(0, V, (B, T), generator=g)
+    idx = tgt.unsqueeze(1).expand(-1, L, -1)
+    xd = x.to(DEV)
+    keep = xd.clone()
+    # no gradient: logits untouched
+    sel = ops._logsoftmax_gather(xd, idx.to(DEV), False)
+    assert torch.equal(xd, keep)
+    want = _gather_ref(x, idx)
+    tol = 1e-12 if dtype == torch.float64 else 2e-5
+    assert sel.dtype == (torch.float64 if dtype == torch.float64 else torch.float32)
+    assert torch.allclose(sel.cpu(), want, rtol=tol, atol=tol)
+    # oracle agrees too (rows enumerated by the C loops)
+    osel, oprobs = oracle.lsg_fwd(x.numpy(), idx.numpy(), want_probs=True)
+    assert np.allclose(sel.cpu().numpy(), osel, rtol=tol, atol=tol)
+    # with gradient: same gathered values, logits replaced by softmax in their own dtype
+    sel2 = ops._logsoftmax_gather(xd, idx.to(DEV), True)
+    assert torch.allclose(sel2, sel, rtol=tol, atol=tol)
+    probs = torch.from_numpy(oprobs)
+    got = xd.cpu().double()
+    if dtype == torch.float16:
+        assert (got - probs).abs().max() <= (probs.abs() * 2 ** -10 + 2 ** -24).max()
+        assert torch.allclose(got, probs, rtol=2 ** -10, atol=2 ** -24)
+    elif dtype == torch.float32:
+        assert torch.allclose(got, probs, rtol=1e-5, atol=1e-10)
+    else:
+        assert torch.allclose(got, probs, rtol=1e-12, atol=1e-300)
+
+
+def test_lsg_misaligned_rows_and_strided_indices():
+    """V odd => rows start at every 2-byte alignment; index tensor genuinely 3-d and non-contiguous."""
+    g = torch.Generator().manual_seed(5)
+    B, L, V, T = 2, 9, 333, 6
+    x = (torch.randn(B, L, V, generator=g) * 3).half()
+    idx = torch.randint(0, V, (B, T, L), generator=g).transpose(1, 2)
+    xd = x.to(DEV)
+    sel = ops._logsoftmax_gather(xd, idx.to(DEV), True)
+    assert torch.allclose(sel.cpu(), _gather_ref(x, idx), rtol=2e-5, atol=2e-5)
+    want_p = torch.softmax(x.float(), -1)
+    assert torch.allclose(xd.cpu().float(), want_p, rtol=2 ** -10, atol=2 ** -24)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_lsg_backward_matches_torch_ops(dtype):
+    """The fused backward against the reference's own two torch calls (pcfg_loss.py:176-177) on the same buffer."""
+    g = torch.Generator().manual_seed(9)
+    B, L, V, T = 4, 6, 2048, 12
+    probs = torch.softmax(torch.randn(B, L, V, generator=g) * 2, -1).to(dtype).to(DEV)
+    tgt = torch.randint(0, V, (B, T), generator=g)
+    tgt[:, 3] = tgt[:, 1]  # duplicate columns
+    tgt[:, 7:] = 1         # pads
+    idx = tgt.unsqueeze(1).expand(-1, L, -1).to(DEV)
+    gout = torch.randn(B, L, T, generator=g).to(DEV)
+    gout[:, :, 7:] = 0
+    ref = probs.clone()
+    ref.mul_(gout.sum(-1, keepdim=True).neg_().to(ref.dtype))
+    ref.scatter_add_(-1, idx, gout.to(ref.dtype))
+    got = probs.clone()
+    ops._logsoftmax_gather_backward(got, idx, gout)
+    if dtype == torch.float16:
+        # the row factor -(sum g) is rounded to fp16 from differently ordered fp32 sums: allow one rounding step
+        assert torch.allclose(got.float(), ref.float(), rtol=2 ** -9, atol=2 ** -20)
+        same = (got == ref).float().mean().item()
+        assert same > 0.99
+    else:
+        assert torch.allclose(got, ref, rtol=1e-5, atol=1e-9)
+
+
+def test_lsg_autograd_contract():
+    g = torch.Generator().manual_seed(2)
+    B, L, V, T = 2, 4, 640, 5
+    leaf = (torch.randn(B, L, V, generator=g)).to(DEV).requires_grad_(True)
+    x = leaf * 1.0  # non-leaf, as in the model
+    tgt = torch.randint(0, V, (B, T), generator=g).to(DEV)
+    idx = tgt.unsqueeze(1).expand(-1, L, -1)
+    out, sel = ops.dag_logsoftmax_gather_inplace(x, idx)
+    assert out.data_ptr() == x.data_ptr()
+    w = torch.randn(B, L, T, generator=g).to(DEV)
+    (sel * w).sum().backward()
+    ref_leaf = leaf.detach().clone().requires_grad_(True)
+    (torch.log_softmax(ref_leaf, -1).gather(-1, idx) * w).sum().backward()
+    assert torch.allclose(leaf.grad, ref_leaf.grad, rtol=1e-4, atol=1e-6)
+    # no gradient requested: buffer untouched, no graph
+    y = torch.randn(B, L, V, generator=g).to(DEV)
+    keep = y.clone()
+    out, sel = ops.dag_logsoftmax_gather_inplace(y, idx)
+    assert torch.equal(y, keep) and not sel.requires_grad
+
+
+def _oracle_inside(batch, match):
+    links = batch["links"].numpy()
+    ol, tl = batch["output_length"].numpy(), batch["target_length"].numpy()
+    S, C = oracle.inside_fwd(match, links, ol, tl, dtype=np.float64)
+    mg, lg = oracle.inside_bwd(np.ones(len(ol)), S, C, match, links, ol, tl, dtype=np.float64)
+    return S, C, mg, lg
+
+
+def _train_case(name):
+    if name == "cfg1":
+        return synth.config1()
+    if name == "wmt_small":  # config-2 shaped, smaller vocabulary and batch
+        return synth.config2(B=6, V=1000, seed=1, logit_dtype=torch.float32)
+    if name == "ragged_short":
+        return synth.training_batch(5, 64, 12, 300, [64, 40, 22, 8, 4], [12, 9, 7, 3, 2], seed=8)
+    if name == "L256":
+        return synth.training_batch(3, 256, 40, 200, [256, 200, 130], [40, 33, 38], seed=12)
+    raise KeyError(name)
+
+
+def _match_for(batch):
+    sel = torch.log_softmax(batch["logits"].double(), -1).gather(
+        -1, batch["targets"].unsqueeze(1).expand(-1, batch["logits"].shape[1], -1))
+    return harness.eos_masked(sel.float(), batch["output_length"], batch["target_length"])
+
+
+@pytest.mark.parametrize("case", ["cfg1", "wmt_small", "ragged_short", "L256"])
+def test_inside_forward_backward_vs_oracle(case):
+    batch = _train_case(case)
+    match = _match_for(batch)
+    S64, C64, mg64, lg64 = _oracle_inside(batch, match.numpy())
+    md = match.to(DEV).requires_grad_(True)
+    ld = batch["links"].to(DEV).requires_grad_(True)
+    ll = ops.cuda_pcfg_loss(md, ld, batch["output_length"].to(DEV), batch["target_length"].to(DEV))
+    want_ll = S64[:, 0, 0]
+    got_ll = ll.detach().cpu().double().numpy()
+    fin = np.isfinite(want_ll)
+    assert fin.any()
+    assert np.array_equal(np.isfinite(got_ll), fin)
+    assert np.allclose(got_ll[fin], want_ll[fin], rtol=1e-5)
+    w = torch.linspace(0.5, 1.5, ll.numel(), device=DEV)
+    (ll.masked_fill(~torch.isfinite(ll), 0) * w).sum().backward()
+    wn = w.cpu().double().numpy()
+    mg_want = mg64 * wn[:, None, None]
+    lg_want = lg64 * wn[:, None, None, None]
+    mg_got, lg_got = md.grad.cpu().double().numpy(), ld.grad.cpu().double().numpy()
+    assert np.isfinite(mg_got).all() and np.isfinite(lg_got).all()
+    for bi in range(len(wn)):
+        scale = max(np.abs(mg_want[bi]).max(), 1e-30)
+        assert np.abs(mg_got[bi] - mg_want[bi]).max() <= 1e-4 * scale, (case, bi)
+        scale = max(np.abs(lg_want[bi]).max(), 1e-30)
+        assert np.abs(lg_got[bi] - lg_want[bi]).max() <= 1e-4 * scale, (case, bi)
+        if not fin[bi]:
+            assert not mg_got[bi].any() and not lg_got[bi].any()
+
+
+def test_inside_tables_match_oracle_layout():
+    batch = _train_case("ragged_short")
+    match = _match_for(batch)
+    S64, _, _, _ = _oracle_inside(batch, match.numpy())
+    S, aux, _, _ = ops._pcfg_loss_tables(match.to(DEV), batch["links"].to(DEV), batch["output_length"].to(DEV),
+                                         batch["target_length"].to(DEV), 1, "test")
+    S = S.cpu().double().numpy()
+    assert S.shape == S64.shape
+    assert np.array_equal(np.isneginf(S), np.isneginf(S64))
+    fin = np.isfinite(S64)
+    assert np.allclose(S[fin], S64[fin], rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("case", ["cfg1", "wmt_small", "ragged_short", "L256"])
+def test_best_tree_bit_exact(case):
+    batch = _train_case(case)
+    match = _match_for(batch)
+    links = batch["links"]
+    ol, tl = batch["output_length"], batch["target_length"]
+    tree, ll = ops.cuda_pcfg_best_tree(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV))
+    assert tree.dtype == torch.int64 and not tree.requires_grad
+    S_gpu, _, _, _ = ops._pcfg_loss_tables(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV), 1, "test")
+    S64, C64 = oracle.inside_fwd(match.numpy(), links.numpy(), ol.numpy(), tl.numpy(), dtype=np.float32)
+    # the trace of the oracle fed with the very tables the GPU trace saw: must agree bit for bit
+    want = oracle.best_tree(S_gpu.cpu().numpy(), C64, match.numpy(), links.numpy(), ol.numpy(), tl.numpy(), dtype=np.float32)
+    assert np.array_equal(tree.cpu().numpy(), want)
+    # and the trace over the oracle's own float64 tables is the same alignment on these inputs
+    S64d, C64d = oracle.inside_fwd(match.numpy(), links.numpy(), ol.numpy(), tl.numpy(), dtype=np.float64)
+    want64 = oracle.best_tree(S64d, C64d, match.numpy(), links.numpy(), ol.numpy(), tl.numpy(), dtype=np.float64)
+    assert np.array_equal(tree.cpu().numpy(), want64)
+    for bi in range(tree.shape[0]):
+        if math.isfinite(float(ll[bi])):
+            used = tree[bi][tree[bi] >= 0].cpu().tolist()
+            assert used == list(range(int(tl[bi])))
+
+
+def test_best_tree_exact_ties_follow_reference_order():
+    L = m = 14
+    n = 3
+    links = torch.full((1, L, 2, L), -math.inf)
+    for a in range(1, m - 1, 2):
+        links[0, a, 0, a + 2:m:2] = -1.0
+    match = torch.full((1, L, n), -1.0)
+    ol, tl = torch.tensor([m]), torch.tensor([n])
+
+    def second(dead):
+        lk = links.clone()
+        for cid in dead:
+            lk[0, 1, 0, 2 * cid + 1] = -math.inf
+        tree, _ = ops.cuda_pcfg_best_tree(match.to(DEV), lk.to(DEV), ol.to(DEV), tl.to(DEV))
+        pos = (tree[0] == 1).nonzero().item()
+        return (pos - 1) // 2
+
+    assert second(()) == 1
+    assert second((1,)) == 5
+    assert second((1, 5)) == 3
+    assert second((1, 5, 3)) == 2
+    assert second((1, 5, 3, 2)) == 4
+
+
+def _decode_case(name):
+    if name == "short":
+        return synth.decode_batch([5, 9, 16, 3, 12], seed=3, V=500)
+    if name == "L256":
+        return synth.decode_batch([64, 40, 33], seed=4, V=300)
+    raise KeyError(name)
+
+
+@pytest.mark.parametrize("case", ["short", "L256"])
+def test_viterbi_tables_bit_exact_and_decode(case):
+    batch = _decode_case(case)
+    ob, tok = synth.ob_and_tokens(batch["logits"])
+    links, ol = batch["links"], batch["output_length"]
+    L = links.shape[1]
+    scores, R, Lt, M = ops.cuda_pcfg_viterbi(ob.to(DEV), links.to(DEV), ol.to(DEV))
+    S_o, R_o, L_o, M_o = oracle.viterbi(ob.numpy(), links.numpy(), ol.numpy(), dtype=np.float32)
+    assert scores.shape == (links.shape[0], L // 4)
+    assert np.array_equal(scores.cpu().numpy(), S_o[:, 1, :])  # bit-exact, -inf included
+    assert np.array_equal(R.cpu().numpy(), R_o)
+    assert np.array_equal(Lt.cpu().numpy(), L_o)
+    assert np.array_equal(M.cpu().numpy(), M_o)
+    left_mask, _, _ = synth.support_masks(L, 1)
+    # glue + readout, traces on the device and on the host, against the same glue over the oracle
+    import oracle_ops
+    want_tok, want_len = harness.viterbi_decode(ob, tok, links, ol, left_mask, ops=oracle_ops)
+    for on_host in (False, True):
+        got_tok, got_len = harness.viterbi_decode(ob.to(DEV), tok.to(DEV), links.to(DEV), ol.to(DEV), left_mask.to(DEV),
+                                                  traces_on_host=on_host)
+        assert torch.equal(got_len.cpu(), want_len)
+        assert got_tok.dtype == torch.float32 and torch.equal(got_tok.cpu(), want_tok)
+
+
+def test_viterbi_exact_ties_follow_reference_order():
+    L = m = 32
+    links = torch.full((1, L, 2, L), -math.inf)
+    for a in range(1, m - 1, 2):
+        links[0, a, 0, a + 2:m:2] = -1.0
+    ob = torch.full((1, L), -1.0)
+    ol = torch.tensor([m])
+
+    def right_child(dead):
+        lk = links.clone()
+        for cid in dead:
+            lk[0, 1, 0, 2 * cid + 1] = -math.inf
+        _, R, _, _ = ops.cuda_pcfg_viterbi(ob.to(DEV), lk.to(DEV), ol.to(DEV))
+        return (int(R[0, 1, 3]) - 1) // 2
+
+    assert right_child(()) == 4
+    assert right_child((4, 8, 12)) == 2
+    assert right_child((4, 8, 12, 2, 6, 10, 14)) == 1
+    assert right_child((4, 8, 12, 2, 6, 10, 14, 1, 5, 9, 13)) == 3
+
+
+def test_criterion_glue_end_to_end_cfg1():
+    """logsoftmax_gather -> eos mask -> inside loss -> backward through both ops, against the same glue over the oracle."""
+    import oracle_ops
+    batch = synth.config1()
+    B, L, V = batch["logits"].shape
+    out_mask = torch.arange(L).view(1, L) < batch["output_length"].view(B, 1)
+    tgt_mask = batch["targets"].ne(synth.PAD)
+
+    def run(dev, opsmod):
+        leaf = batch["logits"].clone().to(dev).requires_grad_(True)
+        links = batch["links"].clone().to(dev).requires_grad_(True)
+        res = harness.compute_pcfg_loss(leaf * 1.0, out_mask.to(dev), batch["targets"].to(dev), tgt_mask.to(dev), links,
+                                        ops=opsmod)
+        res["loss"].backward()
+        return res["loss"].detach().cpu(), leaf.grad.cpu(), links.grad.cpu()
+
+    loss_g, gl_g, gk_g = run(DEV, ops)
+    loss_o, gl_o, gk_o = run("cpu", oracle_ops)
+    assert torch.allclose(loss_g, loss_o, rtol=1e-5)
+    assert (gl_g - gl_o).abs().max() <= 1e-4 * gl_o.abs().max()
+    assert (gk_g - gk_o).abs().max() <= 1e-4 * gk_o.abs().max()
+
+
+def test_errors_are_loud():
+    x = torch.randn(2, 3, 16, device=DEV)
+    with pytest.raises(RuntimeError, match="select_idx should be long"):
+        ops._logsoftmax_gather(x, torch.zeros(2, 3, 4, dtype=torch.int32, device=DEV), False)
+    with pytest.raises(RuntimeError, match="not contiguous"):
+        ops._logsoftmax_gather(x.transpose(0, 1), torch.zeros(3, 2, 4, dtype=torch.int64, device=DEV), False)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ops.cuda_pcfg_loss(torch.zeros(1, 8, 4), torch.zeros(1, 8, 2, 8), torch.tensor([8]), torch.tensor([4]))
+    # out-of-contract lengths poison the log-likelihood instead of faulting
+    match = torch.zeros(1, 8, 4, device=DEV)
+    links = torch.zeros(1, 8, 2, 8, device=DEV)
+    ll = ops.cuda_pcfg_loss(match, links, torch.tensor([7], device=DEV), torch.tensor([4], device=DEV))
+    assert torch.isnan(ll).all()
+    with pytest.raises(RuntimeError, match="max_left"):
+        ops.cuda_pcfg_loss(match, torch.zeros(1, 8, 4, 8, device=DEV), torch.tensor([8], device=DEV),
+                           torch.tensor([4], device=DEV))

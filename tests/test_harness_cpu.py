@@ -1,0 +1,98 @@
+"""The criterion / decoder glue (pcfg_nat_amd/harness.py) run over the CPU oracle: checks the glue itself (eos masking,
+loss reduction, GLAT sampling, length selection) on the tiny plumbing configuration."""
+import numpy as np
+import torch
+
+import oracle_ops
+from pcfg_nat_amd import harness, synth
+
+
+def _masks(batch):
+    B, L, _ = batch["logits"].shape
+    out_mask = torch.arange(L).view(1, L) < batch["output_length"].view(B, 1)
+    return out_mask, batch["targets"].ne(synth.PAD)
+
+
+def test_eos_mask_semantics():
+    match = torch.zeros(2, 6, 4)
+    out = harness.eos_masked(match, torch.tensor([6, 4]), torch.tensor([4, 3]))
+    assert torch.isinf(out[0, :5, 3]).all() and out[0, 5, 3] == 0
+    assert torch.isinf(out[1, [0, 1, 2, 4, 5], 2]).all() and out[1, 3, 2] == 0
+    assert (out[1, :, 3] == 0).all() and (out[:, :, :2] == 0).all()
+
+
+def test_loss_and_gradients_config1():
+    batch = synth.config1()
+    out_mask, tgt_mask = _masks(batch)
+    leaf = batch["logits"].clone().requires_grad_(True)
+    links = batch["links"].clone().requires_grad_(True)
+    res = harness.compute_pcfg_loss(leaf * 1.0, out_mask, batch["targets"], tgt_mask, links, ops=oracle_ops)
+    assert torch.isfinite(res["loss"]) and int(res["invalid_nsentences"]) == 0
+    res["loss"].backward()
+    # d loss / d logits sums to zero over the vocabulary (softmax gradient), rows of pads get nothing
+    assert leaf.grad.sum(-1).abs().max() < 1e-5
+    assert torch.isfinite(links.grad).all()
+    # the loss is -(ll / n).mean(): every sentence's emission posterior mass is n, so the logits gradient w.r.t. the
+    # gathered columns carries total mass -1/B per sentence
+    B = leaf.shape[0]
+    tgt = batch["targets"]
+    # finite-difference spot check through the whole glue
+    eps = 1e-3
+    b, p, v = 0, 5, int(tgt[0, 3])
+    xp, xm = batch["logits"].clone().double(), batch["logits"].clone().double()
+    xp[b, p, v] += eps
+    xm[b, p, v] -= eps
+    lp = harness.compute_pcfg_loss(xp, out_mask, tgt, tgt_mask, batch["links"].double(), ops=oracle_ops)["loss"]
+    lm = harness.compute_pcfg_loss(xm, out_mask, tgt, tgt_mask, batch["links"].double(), ops=oracle_ops)["loss"]
+    fd = float(lp - lm) / (2 * eps)
+    assert abs(fd - float(leaf.grad[b, p, v])) < 1e-4 * max(1.0, abs(fd)) + 1e-6
+
+
+def test_glat_alignment_is_deterministic_and_consistent():
+    batch = synth.config1()
+    B, L, V = batch["logits"].shape
+    prev = torch.full((B, L), 3, dtype=torch.int64)  # unk everywhere, no pads: output_length = L
+    outs = []
+    for _ in range(2):
+        gen = torch.Generator().manual_seed(7)
+        outs.append(harness.glat_alignment(batch["logits"].clone(), batch["targets"], prev, batch["links"], 0.5,
+                                           ops=oracle_ops, generator=gen))
+    a, b = outs
+    assert torch.equal(a["keep_word_mask"], b["keep_word_mask"])
+    assert torch.equal(a["glat_prev_output_tokens"], b["glat_prev_output_tokens"])
+    path = a["path"]
+    n = batch["target_length"]
+    for i in range(B):
+        used = path[i][path[i] >= 0]
+        assert used.tolist() == list(range(int(n[i])))
+    # revealed nodes carry exactly their aligned target token, the others keep the previous token (times zero trick of
+    # the reference: masked_fill(keep, 0) + oracle.masked_fill(~keep, 0))
+    keep = a["keep_word_mask"]
+    oracle_tok = batch["targets"].gather(-1, path.clip(min=0))
+    assert torch.equal(a["glat_prev_output_tokens"][keep], oracle_tok[keep])
+    assert (a["glat_prev_output_tokens"][~keep] == 3).all()
+    assert (keep.sum(1) <= a["glance_nums"]).all()
+    assert a["matchmask"].shape == (B, batch["targets"].shape[1], L)
+    assert torch.equal(a["matchmask"].sum(-1).sum(-1), n)
+
+
+def test_viterbi_decode_glue():
+    batch = synth.decode_batch([6, 10, 4], seed=5, V=64, logit_dtype=torch.float32)
+    ob, tok = synth.ob_and_tokens(batch["logits"])
+    L = batch["links"].shape[1]
+    left_mask, _, _ = synth.support_masks(L, 1)
+    tokens, pred_len = harness.viterbi_decode(ob, tok, batch["links"], batch["output_length"], left_mask, ops=oracle_ops)
+    assert tokens.dtype == torch.float32 and tokens.shape[0] == 3
+    assert (pred_len >= 1).all() and (pred_len < batch["output_length"] // 4).all()
+    # the number of emitted tokens never exceeds the predicted length (dedup and pad-skip only remove)
+    assert ((tokens != synth.PAD).sum(1) <= pred_len).all()
+
+
+def test_support_masks_closed_form():
+    left, right, main = synth.support_masks(10, 1)
+    assert main.tolist() == [False, True, False, True, False, True, False, True, False, True]
+    assert left[3, 2] == 0 and left[3, 0] == 0 and left[3, 1] == 1 and left[1, 0] == 0 and left[0, 0] == 1
+    assert right[1, 2:].eq(0).all() and right[2].eq(1).all()
+    left3, right3, main3 = synth.support_masks(14, 3)
+    assert main3.nonzero().flatten().tolist() == [1, 5, 9, 13]
+    assert left3[5, 2:5].eq(0).all() and left3[3, 2] == 0 and right3[3, 4] == 0 and left3[3, 4] == 1
