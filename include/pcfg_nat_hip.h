@@ -53,6 +53,16 @@ int pcfgnat_logsoftmax_gather(void *word_ins_out, int dtype, const int64_t *sele
                               int64_t T, void *stream);
 
 /*
+ * logsoftmax_gather with the criterion's eos mask folded into the gather (nat_pcfg_loss.py:111-115, 201-207):
+ * selected[b, p, target_length[b]-1] = -inf for every node p != output_length[b]-1.  Same as calling
+ * pcfgnat_logsoftmax_gather and then masked_fill, without the extra passes over [B,L,T].
+ */
+int pcfgnat_logsoftmax_gather_eos(void *word_ins_out, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl,
+                                  int64_t st, void *selected, int require_grad, const int64_t *output_length,
+                                  const int64_t *target_length, int64_t B, int64_t L, int64_t V, int64_t T,
+                                  void *stream);
+
+/*
  * Replaces the two torch calls of DagLogsoftmaxGatherFunc.backward (pcfg_loss.py:176-177) by one pass:
  *   probs_inout[b,p,v] = probs[b,p,v] * cast(-sum_s g[b,p,s]);  probs_inout[b,p,idx[b,p,s]] += cast(g[b,p,s])
  * with every operation rounded to the buffer's dtype as torch's mul_/scatter_add_ do (duplicates of an index are
@@ -81,7 +91,8 @@ int pcfgnat_pcfg_loss(const float *match_all, const float *links, const int64_t 
 
 /*
  * Replaces pcfg_loss_backward (pcfg_loss_backward.cu:654-721): gradients of sum_b grad_output[b] * S[b,0,0].
- *   grad_output [B] float32; S, aux as produced by pcfgnat_pcfg_loss on the same inputs.
+ *   grad_output [B] float32, or NULL for the criterion's own weights -1/(target_length[b]*B), i.e. the gradient of
+ *   loss = -(ll/target_length).mean() (nat_pcfg_loss.py:135); S, aux as produced by pcfgnat_pcfg_loss on the same inputs.
  *   match_all_grad [B,L,T], links_grad [B,L,ml+1,L] out (fully written, zeros outside the support).
  * The result is the exact gradient of the forward recurrences; sentences with a non-finite log-likelihood get
  * all-zero gradients.

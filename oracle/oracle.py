@@ -92,6 +92,23 @@ def lsg_fwd(x, idx, want_probs=False, dtype=np.float64):
     return sel.reshape(B, L, T), (probs.reshape(B, L, V) if want_probs else None)
 
 
+def lsg_bwd(probs, idx, grad_sel, dtype=np.float64):
+    """Backward of logsoftmax_gather as DagLogsoftmaxGatherFunc.backward performs it (pcfg_loss.py:176-177), without the
+    rounding to the buffer dtype.  Returns the gradient w.r.t. the logits [B,L,V] in ``dtype``."""
+    sfx, _ = _sfx(dtype)
+    B, L, V = probs.shape
+    T = idx.shape[2]
+    buf = np.array(probs.reshape(B * L, V), dtype=dtype, order="C", copy=True)
+    g = _c(grad_sel.reshape(B * L, T), dtype)
+    item = idx.itemsize
+    s0, s1, s2 = (s // item for s in idx.strides)
+    base = np.ascontiguousarray(
+        (np.arange(B, dtype=np.int64)[:, None] * s0 + np.arange(L, dtype=np.int64)[None, :] * s1).reshape(-1))
+    getattr(_lib(), "oracle_lsg_bwd" + sfx)(_p(buf), ctypes.c_void_p(idx.ctypes.data), _p(base), ctypes.c_int64(s2), _p(g),
+                                             ctypes.c_int64(B * L), ctypes.c_int64(V), ctypes.c_int64(T))
+    return buf.reshape(B, L, V)
+
+
 def inside_fwd(match, links, out_len, tgt_len, dtype=np.float64):
     """pcfg_loss (pcfg_loss.cu:379-401).  Returns (S [B,Mc,T+2], C [B,Lc,T+2,ml+2]); ll = S[:,0,0]."""
     sfx, _ = _sfx(dtype)

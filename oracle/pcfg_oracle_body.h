@@ -67,6 +67,24 @@ void FN(oracle_lsg_fwd)(const REAL *x, const int64_t *idx, const int64_t *idx_ba
 }
 
 /* ---------------------------------------------------------------------------------------------
+ * Backward of logsoftmax_gather as the autograd wrapper performs it (pcfg_loss.py:176-177), in REAL
+ * arithmetic: buf = probs * -(sum_s g[s]); buf[idx[s]] += g[s] for s ascending.  In place on `buf`.
+ * ------------------------------------------------------------------------------------------- */
+void FN(oracle_lsg_bwd)(REAL *buf, const int64_t *idx, const int64_t *idx_base, int64_t idx_col_stride, const REAL *g,
+                        int64_t rows, int64_t V, int64_t T)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; r++) {
+        REAL *br = buf + r * V;
+        REAL sum = 0;
+        for (int64_t s = 0; s < T; s++) sum += g[r * T + s];
+        REAL ns = -sum;
+        for (int64_t v = 0; v < V; v++) br[v] *= ns;
+        for (int64_t s = 0; s < T; s++) br[idx[idx_base[r] + s * idx_col_stride]] += g[r * T + s];
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------
  * Inside forward for one sentence.  calculate_C_kernel (pcfg_loss.cu:262-349) then
  * calculate_S_kernel (pcfg_loss.cu:84-224).  Tables are filled with -inf first (:246, :365).
  * ------------------------------------------------------------------------------------------- */

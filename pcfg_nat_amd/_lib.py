@@ -25,6 +25,7 @@ SIGNATURES = {
     "pcfgnat_abi_version": (_int, []),
     "pcfgnat_last_error": (ctypes.c_char_p, []),
     "pcfgnat_logsoftmax_gather": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _int, _i64, _i64, _i64, _i64, _vp]),
+    "pcfgnat_logsoftmax_gather_eos": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_logsoftmax_gather_backward": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_pcfg_aux_floats": (ctypes.c_size_t, [_i64, _i64, _i64, _i64]),
     "pcfgnat_pcfg_loss": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),

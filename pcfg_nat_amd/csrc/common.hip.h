@@ -94,4 +94,11 @@ __device__ __forceinline__ double wave_sum(double v) {
 
 constexpr float NEG_INF_F = -__builtin_huge_valf();
 
+// Workgroup barrier that orders LDS traffic only: outstanding global stores keep draining in the background instead
+// of being waited for (what __syncthreads() does), which matters in sweeps that write a few table cells per step.
+// Global data written before it must not be read by other waves after it.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 }  // namespace pcfgnat

@@ -23,7 +23,6 @@ namespace pcfgnat {
 namespace {
 
 constexpr int NT = 1024;       // threads per sentence
-constexpr int GROUPS = NT / 16;  // 16-lane rows
 
 __device__ __forceinline__ float sanitize(float v) { return (v != v) ? NEG_INF_F : v; }
 
@@ -170,7 +169,7 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_kernel(const float *__restr
                 }
             }
         }
-        __syncthreads();
+        lds_barrier();
     }
 }
 
@@ -211,7 +210,8 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_kernel(const float *__restr
         return;
     }
     const int mc = m / 2;
-    const float g = grad_out[b];
+    // a null grad_output selects the criterion's own weights: d(-(ll/n).mean())/d ll_b = -1/(n_b * B)
+    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)gridDim.x);
 
     // transposed link slabs: row = child c (this thread's DPP row), lanes over parents a <= c
     float A0[R][CN], A1[R][CN], G0[R][CN], G1[R][CN];
@@ -315,9 +315,8 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_kernel(const float *__restr
                 if (live) av.BETA[(size_t)c_id * (T + 2) + t] = beta;
             }
         }
-        __syncthreads();
+        lds_barrier();
     }
-    __threadfence();
     __syncthreads();
 
     // rule posteriors -> links_grad (pcfg_loss_backward.cu:512-531); everything else in the slab is zero
@@ -390,7 +389,6 @@ __global__ __launch_bounds__(64) void best_tree_ml1_kernel(const float *__restri
     for (int i = lane; i < L; i += 64) tr[i] = -1;
     if (!lengths_ok(m, n, L, T)) return;
     const int mc = m / 2;
-    __threadfence_block();
     int a_id = 0, s = 0;
     // every marked cell (a, s) has s <= n by construction; the loop is bounded by the number of main-chain nodes
     for (int hop = 0; hop < mc; hop++) {
@@ -509,7 +507,7 @@ extern "C" int pcfgnat_pcfg_loss_backward(const float *grad_output, const float 
     int rc = check_dims("pcfg_loss_backward", B, L, T, ml);
     if (rc != PCFGNAT_OK) return rc;
     if (B == 0) return PCFGNAT_OK;
-    PCFGNAT_REQUIRE(grad_output && S && aux && match_all && links && output_length && target_length && match_all_grad && links_grad,
+    PCFGNAT_REQUIRE(S && aux && match_all && links && output_length && target_length && match_all_grad && links_grad,
                     "pcfg_loss_backward: null pointer");
     const int Mc = (int)((L - 2) / 2 + 1);
     hipStream_t s = (hipStream_t)stream;

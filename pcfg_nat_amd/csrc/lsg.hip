@@ -134,7 +134,8 @@ template <typename T, int NT, int MAXC, int GMAX, bool GRAD>
 __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const int64_t *__restrict__ idx, int64_t sb,
                                                      int64_t sl, int64_t st,
                                                      typename Elem<T>::compute *__restrict__ sel, int64_t rows, int L,
-                                                     int V, int Tn) {
+                                                     int V, int Tn, const int64_t *__restrict__ eos_out_len,
+                                                     const int64_t *__restrict__ eos_tgt_len) {
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
     constexpr int NW = NT / 64;
@@ -215,10 +216,16 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
 #pragma unroll
         for (int i = 0; i < MAXC; i++) opaque(buf[i]);
 
+        // optional fused eos mask (nat_pcfg_loss.py:111-115): only the last graph node may emit the last target token
+        int eos_col = -1;
+        if (eos_out_len != nullptr) {
+            const int64_t b = row / L, pnode = row % L;
+            if (pnode != eos_out_len[b] - 1) eos_col = (int)(eos_tgt_len[b] - 1);
+        }
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
             int s = tid + g * NT;
-            if (s < Tn) sel[row * (int64_t)Tn + s] = (gv[g] - mx) - lg;
+            if (s < Tn) sel[row * (int64_t)Tn + s] = (s == eos_col) ? neg_inf(CT()) : (gv[g] - mx) - lg;
         }
 
         if (GRAD) {
@@ -247,14 +254,15 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
     }
 }
 
-// In-place backward.  TCAP = most targets per row handled through LDS.
-template <typename T, int NT, int TCAP>
+// In-place backward.  TCAP = most targets per row handled through LDS; up to MAXC chunks per thread are in flight.
+template <typename T, int NT, int MAXC, int TCAP>
 __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const int64_t *__restrict__ idx, int64_t sb,
                                                      int64_t sl, int64_t st,
                                                      const typename Elem<T>::compute *__restrict__ gsel, int64_t rows,
                                                      int L, int V, int Tn) {
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
+    constexpr int FIX = (TCAP + NT - 1) / NT;
     __shared__ int s_idx[TCAP];
     __shared__ CT s_g[TCAP];   // cast(g[s]) in the buffer's dtype, widened again
     __shared__ CT s_p[TCAP];   // original probability at idx[s]
@@ -265,6 +273,19 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
         const CT *gr = gsel + row * (int64_t)Tn;
         const int64_t b = row / L, q = row % L;
         const int64_t *ir = idx + b * sb + q * sl;
+        const RowSplit<T> sp(pr, V);
+        vec16 *pv = reinterpret_cast<vec16 *>(pr + sp.head);
+
+        // the row's chunks are requested first so that they travel while the small per-row work is done
+        vec16 buf[MAXC];
+#pragma unroll
+        for (int i = 0; i < MAXC; i++) {
+            int c = tid + i * NT;
+            if (c < sp.nvec) buf[i] = load16(pv + c);
+        }
+        const int ep = sp.edge_pos(tid);
+        CT edge = 0;
+        if (ep >= 0) edge = Elem<T>::widen(pr[ep]);
 
         // -(sum_s g) rounded to the buffer dtype (pcfg_loss.py:176), computed redundantly by every wave
         CT part = 0;
@@ -278,25 +299,33 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
             s_g[s] = Elem<T>::widen(Elem<T>::narrow(gr[s]));
             s_p[s] = ok ? Elem<T>::widen(pr[t]) : (CT)0;
         }
-        __syncthreads();  // every original value at a target column is now in LDS
+        __syncthreads();  // every original value at a target column is in LDS before any store to the row
 
-        const RowSplit<T> sp(pr, V);
-        vec16 *pv = reinterpret_cast<vec16 *>(pr + sp.head);
-        for (int c = tid; c < sp.nvec; c += NT) {
+#pragma unroll
+        for (int i = 0; i < MAXC; i++) {
+            int c = tid + i * NT;
+            if (c < sp.nvec) {
+                CT v[EPV];
+                Elem<T>::unpack(buf[i], v);
+#pragma unroll
+                for (int e = 0; e < EPV; e++) v[e] = v[e] * ns;
+                store16(pv + c, Elem<T>::pack(v));
+            }
+        }
+        for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
             CT v[EPV];
             Elem<T>::unpack(load16(pv + c), v);
 #pragma unroll
             for (int e = 0; e < EPV; e++) v[e] = v[e] * ns;
             store16(pv + c, Elem<T>::pack(v));
         }
-        const int ep = sp.edge_pos(tid);
-        if (ep >= 0) pr[ep] = Elem<T>::narrow(Elem<T>::widen(pr[ep]) * ns);
+        if (ep >= 0) pr[ep] = Elem<T>::narrow(edge * ns);
 
         // scatter_add_ (pcfg_loss.py:177): the first occurrence of a column accumulates all its duplicates in order
-        CT fix[(TCAP + NT - 1) / NT];
-        bool lead[(TCAP + NT - 1) / NT];
+        CT fix[FIX];
+        bool lead[FIX];
 #pragma unroll
-        for (int r = 0; r < (TCAP + NT - 1) / NT; r++) {
+        for (int r = 0; r < FIX; r++) {
             int s = tid + r * NT;
             lead[r] = false;
             fix[r] = 0;
@@ -313,10 +342,11 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
                 }
             }
         }
-        __threadfence();
-        __syncthreads();  // the streamed row is complete before the target columns are patched
+        // workgroup barrier (release/acquire at workgroup scope): the streamed stores of this row are ordered before the
+        // patches of its target columns, which hit addresses other threads of the workgroup have just written
+        __syncthreads();
 #pragma unroll
-        for (int r = 0; r < (TCAP + NT - 1) / NT; r++) {
+        for (int r = 0; r < FIX; r++) {
             int s = tid + r * NT;
             if (lead[r]) pr[s_idx[s]] = Elem<T>::narrow(fix[r]);
         }
@@ -326,7 +356,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
 
 template <typename T>
 int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, void *sel, int grad, int64_t rows,
-               int L, int V, int Tn, hipStream_t stream) {
+               int L, int V, int Tn, const int64_t *eos_ol, const int64_t *eos_tl, hipStream_t stream) {
     using CT = typename Elem<T>::compute;
     constexpr int NT = 512;
     // 10 chunks x 512 threads x 16 B = 80 KB of a row in registers: a 40k-entry fp16 row exactly, half of an fp32 one.
@@ -336,10 +366,10 @@ int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
     int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
     if (grad)
         hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, true>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)x, idx, sb,
-                           sl, st, (CT *)sel, rows, L, V, Tn);
+                           sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl);
     else
         hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, false>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)x, idx,
-                           sb, sl, st, (CT *)sel, rows, L, V, Tn);
+                           sb, sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -349,10 +379,11 @@ int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
                int Tn, hipStream_t stream) {
     using CT = typename Elem<T>::compute;
     constexpr int NT = 512;
+    constexpr int MAXC = 10;
     constexpr int TCAP = 1024;
     if (Tn > TCAP) return fail(PCFGNAT_EUNSUPPORTED, "logsoftmax_gather_backward: T=%d exceeds %d targets per row", Tn, TCAP);
     int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
-    hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, TCAP>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,
+    hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,
                        (const CT *)g, rows, L, V, Tn);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
@@ -372,23 +403,39 @@ int check_common(const void *x, const int64_t *idx, const void *o, int64_t B, in
 
 using namespace pcfgnat;
 
-extern "C" int pcfgnat_logsoftmax_gather(void *word_ins_out, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl,
-                                         int64_t st, void *selected, int require_grad, int64_t B, int64_t L, int64_t V,
-                                         int64_t T, void *stream) {
+static int lsg_forward_dispatch(void *word_ins_out, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
+                                void *selected, int require_grad, int64_t B, int64_t L, int64_t V, int64_t T,
+                                const int64_t *eos_ol, const int64_t *eos_tl, void *stream) {
     int rc = check_common(word_ins_out, select_idx, selected, B, L, V, T);
     if (rc != PCFGNAT_OK) return rc;
     if (B * L == 0) return PCFGNAT_OK;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case PCFGNAT_F16:
-            return launch_fwd<__half>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, s);
+            return launch_fwd<__half>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, s);
         case PCFGNAT_F32:
-            return launch_fwd<float>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, s);
+            return launch_fwd<float>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, s);
         case PCFGNAT_F64:
-            return launch_fwd<double>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, s);
+            return launch_fwd<double>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, s);
         default:
             return fail(PCFGNAT_EINVAL, "logsoftmax_gather: unknown dtype code %d (float16, float32, float64 are dispatched)", dtype);
     }
+}
+
+extern "C" int pcfgnat_logsoftmax_gather(void *word_ins_out, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl,
+                                         int64_t st, void *selected, int require_grad, int64_t B, int64_t L, int64_t V,
+                                         int64_t T, void *stream) {
+    return lsg_forward_dispatch(word_ins_out, dtype, select_idx, sb, sl, st, selected, require_grad, B, L, V, T, nullptr, nullptr,
+                                stream);
+}
+
+extern "C" int pcfgnat_logsoftmax_gather_eos(void *word_ins_out, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl,
+                                             int64_t st, void *selected, int require_grad, const int64_t *output_length,
+                                             const int64_t *target_length, int64_t B, int64_t L, int64_t V, int64_t T,
+                                             void *stream) {
+    PCFGNAT_REQUIRE(B == 0 || (output_length && target_length), "logsoftmax_gather_eos: null length pointer");
+    return lsg_forward_dispatch(word_ins_out, dtype, select_idx, sb, sl, st, selected, require_grad, B, L, V, T, output_length,
+                                target_length, stream);
 }
 
 extern "C" int pcfgnat_logsoftmax_gather_backward(void *probs_inout, int dtype, const int64_t *select_idx, int64_t sb,

@@ -84,7 +84,6 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
     float sc2[CN];
 #pragma unroll
     for (int q = 0; q < CN; q++) sc2[q] = NEG_INF_F;  // S[c][0] = -inf
-    __threadfence();
     __syncthreads();
     if (tid == 0 && Lq > 1) Sb[(size_t)(m - 1) * Lq + 1] = ob[m - 1];
 
@@ -127,7 +126,7 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
         }
 #pragma unroll
         for (int q = 0; q < CN; q++) sc2[q] = sc1[q];
-        __syncthreads();
+        lds_barrier();
     }
 }
 

@@ -79,7 +79,8 @@ def _pcfg_loss_tables(match_all, links, output_length, target_length, config, na
 
 
 def _pcfg_loss_backward(grad_output, S, aux, match_all, links, output_length, target_length, config):
-    """pcfg_loss_backward (pcfg_loss_backward.cu:654-721)."""
+    """pcfg_loss_backward (pcfg_loss_backward.cu:654-721).  ``grad_output=None`` selects the criterion's own weights
+    -1/(target_length*B), the gradient of ``-(ll/target_length).mean()`` (nat_pcfg_loss.py:135)."""
     if not (1 <= config <= 4):
         raise RuntimeError("config should be 1~4")
     lib = get_pcfg_kernel()
@@ -88,7 +89,7 @@ def _pcfg_loss_backward(grad_output, S, aux, match_all, links, output_length, ta
     with torch.cuda.device(match_all.device):
         match_all_grad = torch.empty_like(match_all)
         links_grad = torch.empty_like(links)
-        _lib.check(lib.pcfgnat_pcfg_loss_backward(grad_output.data_ptr(), S.data_ptr(), aux.data_ptr(),
+        _lib.check(lib.pcfgnat_pcfg_loss_backward(grad_output.data_ptr() if grad_output is not None else None, S.data_ptr(), aux.data_ptr(),
                                                   match_all.data_ptr(), links.data_ptr(), output_length.data_ptr(),
                                                   target_length.data_ptr(), match_all_grad.data_ptr(),
                                                   links_grad.data_ptr(), B, L, T, ml, _stream(match_all)), lib)
@@ -261,8 +262,9 @@ class DagLogsoftmaxGatherFunc(Function):
 dag_logsoftmax_gather_inplace = DagLogsoftmaxGatherFunc.apply
 
 
-def _logsoftmax_gather(word_ins_out, select_idx, require_gradient):
-    """logsoftmax_gather (logsoftmax_gather.cu:295-359), argument checks included (:297-309)."""
+def _logsoftmax_gather(word_ins_out, select_idx, require_gradient, eos_lengths=None):
+    """logsoftmax_gather (logsoftmax_gather.cu:295-359), argument checks included (:297-309).  ``eos_lengths`` =
+    (output_length, target_length) folds the criterion's eos mask (nat_pcfg_loss.py:111-115) into the gather."""
     lib = get_pcfg_kernel()
     _need_cuda("logsoftmax_gather", word_ins_out, select_idx)
     if word_ins_out.dim() != 3:
@@ -287,9 +289,17 @@ def _logsoftmax_gather(word_ins_out, select_idx, require_gradient):
     with torch.cuda.device(word_ins_out.device):
         selected = torch.empty((B, L, T), dtype=out_dtype, device=word_ins_out.device)
         sb, sl, st = select_idx.stride()
-        _lib.check(lib.pcfgnat_logsoftmax_gather(word_ins_out.data_ptr(), code, select_idx.data_ptr(), sb, sl, st,
-                                                 selected.data_ptr(), int(bool(require_gradient)), B, L, V, T,
-                                                 _stream(word_ins_out)), lib)
+        if eos_lengths is None:
+            _lib.check(lib.pcfgnat_logsoftmax_gather(word_ins_out.data_ptr(), code, select_idx.data_ptr(), sb, sl, st,
+                                                     selected.data_ptr(), int(bool(require_gradient)), B, L, V, T,
+                                                     _stream(word_ins_out)), lib)
+        else:
+            ol = _lengths("logsoftmax_gather", eos_lengths[0], B)
+            tl = _lengths("logsoftmax_gather", eos_lengths[1], B)
+            _need_cuda("logsoftmax_gather", word_ins_out, ol, tl)
+            _lib.check(lib.pcfgnat_logsoftmax_gather_eos(word_ins_out.data_ptr(), code, select_idx.data_ptr(), sb, sl, st,
+                                                         selected.data_ptr(), int(bool(require_gradient)), ol.data_ptr(),
+                                                         tl.data_ptr(), B, L, V, T, _stream(word_ins_out)), lib)
     return selected
 
 

@@ -94,3 +94,62 @@ def viterbi_decode(unreduced_logits, unreduced_tokens, links, output_length, lef
     tokens = ops.viterbi_decoding(pred_length.long(), output_length.long(), L_trace.long(), R_trace.long(),
                                   M_trace.long(), unreduced_tokens.long(), left_tree_mask.long(), pad)
     return tokens.to(device=pred_length.device), pred_length
+
+
+def train_step_direct(logits, targets, links, output_length, target_length, ops=_default_ops, mark=None):
+    """One training pass of the structured loss issued as the bare sequence of native calls that autograd performs for
+    ``compute_pcfg_loss(...)['loss'].backward()`` (nat_pcfg_loss.py:98-145 and pcfg_loss.py:55-83, 147-179), without
+    autograd bookkeeping: logsoftmax_gather (in place) -> eos mask -> inside forward + eager backward -> loss ->
+    gradient scaling -> logsoftmax_gather backward (in place).  ``logits`` [B,L,V] holds d loss / d logits afterwards.
+    ``mark(name, phase)`` is called before (0) and after (1) each native call so that a caller can bracket them with
+    events.  Returns (loss, links_grad, ll)."""
+    mark = mark or (lambda name, phase: None)
+    B, L, _ = logits.shape
+    idx = targets.unsqueeze(1).expand(-1, L, -1)
+    mark("lsg_fwd", 0)
+    match = ops._logsoftmax_gather(logits, idx, True)
+    mark("lsg_fwd", 1)
+    match_m = eos_masked(match, output_length, target_length)
+    mark("inside_fwd", 0)
+    S, aux, ol, tl = ops._pcfg_loss_tables(match_m, links, output_length, target_length, 1, "cuda_pcfg_loss")
+    mark("inside_fwd", 1)
+    ones = torch.ones((B,), dtype=S.dtype, device=S.device)
+    mark("inside_bwd", 0)
+    mg, lg = ops._pcfg_loss_backward(ones, S, aux, match_m, links, ol, tl, 1)
+    mark("inside_bwd", 1)
+    ll = S[:, 0, 0]
+    invalid = ll.isinf().logical_or(ll.isnan())
+    loss = -(ll.masked_fill(invalid, 0) / target_length).mean()
+    coef = (-1.0 / (target_length * B)).to(mg.dtype).masked_fill(invalid, 0)
+    gmatch = mg * coef.view(B, 1, 1)
+    glinks = lg * coef.view(B, 1, 1, 1)
+    mark("lsg_bwd", 0)
+    ops._logsoftmax_gather_backward(logits, idx, gmatch)
+    mark("lsg_bwd", 1)
+    return loss, glinks, ll
+
+
+def train_step_fused(logits, targets, links, output_length, target_length, ops=_default_ops, mark=None):
+    """The same training pass as ``train_step_direct`` with the criterion's glue folded into the kernels: the eos mask is
+    applied inside the gather (no [B,L,T] mask tensors), and the inside backward is seeded with the criterion's own
+    weights -1/(n_b*B) instead of ones followed by two scaling passes; sentences with a non-finite log-likelihood get
+    zero gradients from the kernel itself.  Four kernel launches.  Returns (loss, links_grad, ll)."""
+    mark = mark or (lambda name, phase: None)
+    L = logits.shape[1]
+    idx = targets.unsqueeze(1).expand(-1, L, -1)
+    mark("lsg_fwd", 0)
+    match_m = ops._logsoftmax_gather(logits, idx, True, eos_lengths=(output_length, target_length))
+    mark("lsg_fwd", 1)
+    mark("inside_fwd", 0)
+    S, aux, ol, tl = ops._pcfg_loss_tables(match_m, links, output_length, target_length, 1, "cuda_pcfg_loss")
+    mark("inside_fwd", 1)
+    mark("inside_bwd", 0)
+    gmatch, glinks = ops._pcfg_loss_backward(None, S, aux, match_m, links, ol, tl, 1)
+    mark("inside_bwd", 1)
+    mark("lsg_bwd", 0)
+    ops._logsoftmax_gather_backward(logits, idx, gmatch)
+    mark("lsg_bwd", 1)
+    ll = S[:, 0, 0]
+    invalid = ll.isinf().logical_or(ll.isnan())
+    loss = -(ll.masked_fill(invalid, 0) / target_length).mean()
+    return loss, glinks, ll

@@ -325,3 +325,27 @@ def test_errors_are_loud():
     with pytest.raises(RuntimeError, match="max_left"):
         ops.cuda_pcfg_loss(match, torch.zeros(1, 8, 4, 8, device=DEV), torch.tensor([8], device=DEV),
                            torch.tensor([4], device=DEV))
+
+
+def test_fused_step_equals_autograd_step():
+    """train_step_fused / train_step_direct leave the same loss, logits gradient and links gradient as autograd through
+    the operator API (one invalid sentence included: its gradients must vanish)."""
+    batch = synth.training_batch(4, 64, 12, 700, [64, 40, 22, 8], [12, 9, 12, 12], seed=31, logit_scale=2.0,
+                                 logit_dtype=torch.float16)
+    B, L, V = batch["logits"].shape
+    out_mask = (torch.arange(L).view(1, L) < batch["output_length"].view(B, 1)).to(DEV)
+    tgt = batch["targets"].to(DEV)
+    tgt_mask = tgt.ne(synth.PAD)
+    ol, tl = batch["output_length"].to(DEV), batch["target_length"].to(DEV)
+    leaf = batch["logits"].to(DEV).float().requires_grad_(True)
+    links = batch["links"].to(DEV).requires_grad_(True)
+    res = harness.compute_pcfg_loss(leaf.half(), out_mask, tgt, tgt_mask, links)
+    assert int(res["invalid_nsentences"]) == 1
+    res["loss"].backward()
+    for step in (harness.train_step_direct, harness.train_step_fused):
+        buf = batch["logits"].to(DEV).clone()
+        loss, glinks, ll = step(buf, tgt, batch["links"].to(DEV), ol, tl)
+        assert torch.allclose(loss, res["loss"].detach(), rtol=1e-6)
+        assert torch.allclose(glinks, links.grad, rtol=1e-5, atol=1e-9)
+        assert torch.allclose(buf.float(), leaf.grad, rtol=2 ** -9, atol=2 ** -22)
+        assert not glinks[3].any() and not buf[3].any()

@@ -31,3 +31,18 @@ def test_lsg_f32_and_half_inputs():
     sel, _ = oracle.lsg_fwd(x.numpy(), idx.numpy(), dtype=np.float32)
     want = torch.log_softmax(x.float(), -1).gather(-1, idx)
     assert np.allclose(sel, want.numpy(), rtol=1e-5, atol=1e-5)
+
+
+def test_lsg_bwd_is_the_gradient():
+    """Autograd of the library expression pins the backward restatement."""
+    g = torch.Generator().manual_seed(4)
+    B, L, V, T = 2, 3, 50, 6
+    x = torch.randn(B, L, V, generator=g, dtype=torch.float64, requires_grad=True)
+    tgt = torch.randint(0, V, (B, T), generator=g)
+    tgt[:, 4] = tgt[:, 2]
+    idx = tgt.unsqueeze(1).expand(-1, L, -1)
+    w = torch.randn(B, L, T, generator=g, dtype=torch.float64)
+    (torch.log_softmax(x, -1).gather(-1, idx) * w).sum().backward()
+    _, probs = oracle.lsg_fwd(x.detach().numpy(), idx.numpy(), want_probs=True)
+    got = oracle.lsg_bwd(probs, idx.numpy(), w.numpy())
+    assert np.allclose(got, x.grad.numpy(), rtol=1e-12, atol=1e-14)
