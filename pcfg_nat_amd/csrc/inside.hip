@@ -429,6 +429,429 @@ __global__ __launch_bounds__(64) void best_tree_ml1_kernel(const float *__restri
     }
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// Streaming variants for graphs whose link slabs do not fit in registers (Mc > 128): same sweeps, but the link
+// values are fetched from L2 every step (forward: straight from `links`; backward: from a compact transposed copy
+// so that lanes read consecutive parents), rows are processed in tiles of 64, and the row reductions are online
+// log-sum-exps over chunks of children.  Rule posteriors are produced by a separate, fully parallel kernel from the
+// outside weights the sweep leaves behind.
+// Aux layout per sentence (Mc > 128): F0, F1, BETA, W0, W1 [Mc][T+2] each, then At [2][Mc][Mc].
+// ------------------------------------------------------------------------------------------------------------
+struct AuxViewStream {
+    float *F0, *F1, *BETA, *W0, *W1, *At;
+    __device__ AuxViewStream(float *aux, int b, int Mc, int T) {
+        const size_t plane = (size_t)Mc * (T + 2);
+        float *base = aux + (size_t)b * (5 * plane + (size_t)2 * Mc * Mc);
+        F0 = base;
+        F1 = base + plane;
+        BETA = base + 2 * plane;
+        W0 = base + 3 * plane;
+        W1 = base + 4 * plane;
+        At = base + 5 * plane;
+    }
+};
+
+struct OnlineLse {
+    float m, s;
+    __device__ OnlineLse() : m(NEG_INF_F), s(0.f) {}
+    // fold four terms in
+    __device__ __forceinline__ void add4(const float *v) {
+        const float cm = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
+        if (cm > m) {
+            s *= __expf(m - cm);  // m = -inf gives 0 * 0
+            m = cm;
+        }
+        if (m != NEG_INF_F) s += (__expf(v[0] - m) + __expf(v[1] - m)) + (__expf(v[2] - m) + __expf(v[3] - m));
+    }
+    // combine the 16 lanes of a DPP row; every lane gets log-sum-exp of all folded terms
+    __device__ __forceinline__ float finish16() const {
+        const float M = row16_max(m);
+        const float part = (m == NEG_INF_F) ? 0.f : s * __expf(m - M);
+        const float tot = row16_sum(part);
+        return (M == NEG_INF_F) ? NEG_INF_F : M + __logf(tot);
+    }
+};
+
+// Dynamic LDS: col[2][MP], f1prev[MP], then (if MATCH_LDS) match main [Mc][T], match leaf [Mc][T].
+template <bool MATCH_LDS>
+__global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
+                                                                  const int64_t *__restrict__ out_len,
+                                                                  const int64_t *__restrict__ tgt_len, float *__restrict__ S,
+                                                                  float *__restrict__ aux, int L, int T, int Mc, int MP) {
+    extern __shared__ float smem[];
+    float *col = smem;               // [2][MP]
+    float *f1prev = smem + 2 * MP;    // [MP]
+    float *sm_main = smem + 3 * MP;   // [Mc][T]
+    float *sm_leaf = sm_main + (MATCH_LDS ? Mc * T : 0);
+
+    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *mt = match_all + (size_t)b * L * T;
+    const float *lk = links + (size_t)b * L * 2 * L;
+    float *Sb = S + (size_t)b * Mc * (T + 2);
+    AuxViewStream av(aux, b, Mc, T);
+
+    if (!lengths_ok(m, n, L, T)) {
+        for (int i = tid; i < Mc * (T + 2); i += NT) Sb[i] = (i == 0) ? __builtin_nanf("") : NEG_INF_F;
+        return;
+    }
+    const int mc = m / 2;
+    if (MATCH_LDS) {
+        for (int i = tid; i < Mc * T; i += NT) {
+            const int a_id = i / T, s = i - a_id * T;
+            const bool ok = a_id < mc && s < n;
+            sm_main[i] = ok ? sanitize(mt[(size_t)(2 * a_id + 1) * T + s]) : NEG_INF_F;
+            sm_leaf[i] = (ok && a_id >= 1) ? sanitize(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
+        }
+    }
+    for (int i = tid; i < Mc * (T + 2); i += NT) {
+        const int a_id = i / (T + 2), s = i - a_id * (T + 2);
+        if (a_id >= mc || s >= n - 1) {
+            float v = NEG_INF_F;
+            if (a_id == mc - 1 && s == n - 1) v = sanitize(mt[(size_t)(m - 1) * T + (n - 1)]);
+            Sb[i] = v;
+        }
+    }
+    for (int i = tid; i < MP; i += NT) {
+        col[((n - 1) & 1) * MP + i] = (i == mc - 1) ? sanitize(mt[(size_t)(m - 1) * T + (n - 1)]) : NEG_INF_F;
+        col[((n - 2) & 1) * MP + i] = NEG_INF_F;
+        f1prev[i] = NEG_INF_F;
+    }
+    __syncthreads();
+
+    const int ntiles = (mc + 63) / 64;
+    const int nq = (mc + 15) / 16;
+    for (int t = n - 1; t >= 1; t--) {
+        const float *cur = col + (t & 1) * MP;
+        float *nxt = col + ((t - 1) & 1) * MP;
+        for (int tile = 0; tile < ntiles; tile++) {
+            const int a_id = tile * 64 + gidx, a = 2 * a_id + 1;
+            const bool row_ok = a_id < mc;
+            const float *l0 = lk + ((size_t)a * 2 + 0) * L, *l1 = lk + ((size_t)a * 2 + 1) * L;
+            // emissions of this row first: their latency overlaps the child loop
+            float ma_p, ml_p, ma_t;
+            if (MATCH_LDS) {
+                const int ai = row_ok ? a_id : 0;
+                ma_p = sm_main[ai * T + t - 1];
+                ml_p = sm_leaf[ai * T + t - 1];
+                ma_t = sm_main[ai * T + t];
+            } else {
+                const size_t ra = (size_t)a * T, rl = (size_t)(a - 1) * T;
+                ma_p = row_ok ? sanitize(mt[ra + t - 1]) : NEG_INF_F;
+                ml_p = (row_ok && a_id >= 1) ? sanitize(mt[rl + t - 1]) : NEG_INF_F;
+                ma_t = row_ok ? sanitize(mt[ra + t]) : NEG_INF_F;
+            }
+            OnlineLse acc0, acc1;
+            for (int qb = 4 * tile; qb < nq; qb += 4) {
+                float v0[4], v1[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int c_id = j + 16 * (qb + u);
+                    const bool ok = row_ok && c_id < mc && c_id >= a_id;
+                    const float sc = (c_id < MP) ? cur[c_id] : NEG_INF_F;
+                    const float x0 = ok ? sanitize(l0[2 * c_id + 1]) : NEG_INF_F;
+                    const float x1 = (ok && a_id >= 1) ? sanitize(l1[2 * c_id + 1]) : NEG_INF_F;
+                    v0[u] = x0 + sc;
+                    v1[u] = x1 + sc;
+                }
+                acc0.add4(v0);
+                acc1.add4(v1);
+            }
+            const float F0 = acc0.finish16();
+            const float F1 = acc1.finish16();
+            const int ai = (a_id < MP) ? a_id : 0;
+            const float f1p = f1prev[ai];
+            float s_new = lse2(ma_p + F0, (ml_p + ma_t) + f1p);
+            if (!row_ok) s_new = NEG_INF_F;
+            if (j == 0 && a_id < MP) {
+                nxt[a_id] = s_new;
+                f1prev[a_id] = F1;
+                if (row_ok) {
+                    Sb[(size_t)a_id * (T + 2) + (t - 1)] = s_new;
+                    av.F0[(size_t)a_id * (T + 2) + t] = F0;
+                    av.F1[(size_t)a_id * (T + 2) + t] = F1;
+                }
+            }
+        }
+        lds_barrier();
+    }
+}
+
+// At[k][c_id][a_id] = links[2*a_id+1][k][2*c_id+1] (compact, transposed), -inf outside a_id <= c_id < mc.
+__global__ __launch_bounds__(256) void transpose_links_ml1_kernel(const float *__restrict__ links, const int64_t *__restrict__ out_len,
+                                                                 float *__restrict__ aux, int L, int T, int Mc) {
+    __shared__ float tile[2][32][33];
+    const int b = blockIdx.z;
+    const int m = (int)out_len[b];
+    const int mc = (m >= 2 && m <= L) ? m / 2 : 0;
+    AuxViewStream av(aux, b, Mc, T);
+    const float *lk = links + (size_t)b * L * 2 * L;
+    const int a0 = blockIdx.y * 32, c0 = blockIdx.x * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    for (int r = ty; r < 32; r += 8) {
+        const int a_id = a0 + r, c_id = c0 + tx;
+        const bool ok = a_id < mc && c_id < mc && a_id <= c_id;
+        const size_t row = (size_t)(2 * a_id + 1) * 2;
+        tile[0][r][tx] = ok ? sanitize(lk[(row + 0) * L + 2 * c_id + 1]) : NEG_INF_F;
+        tile[1][r][tx] = (ok && a_id >= 1) ? sanitize(lk[(row + 1) * L + 2 * c_id + 1]) : NEG_INF_F;
+    }
+    __syncthreads();
+    for (int r = ty; r < 32; r += 8) {
+        const int c_id = c0 + r, a_id = a0 + tx;
+        if (c_id < Mc && a_id < Mc) {
+            av.At[((size_t)0 * Mc + c_id) * Mc + a_id] = tile[0][tx][r];
+            av.At[((size_t)1 * Mc + c_id) * Mc + a_id] = tile[1][tx][r];
+        }
+    }
+}
+
+// Outside sweep.  Dynamic LDS: w0[2][MP], w1[2][MP], bprev[MP], then (if MATCH_LDS) match main/leaf [Mc][T] each.
+template <bool MATCH_LDS>
+__global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *__restrict__ S, float *__restrict__ aux,
+                                                                  const float *__restrict__ match_all,
+                                                                  const int64_t *__restrict__ out_len,
+                                                                  const int64_t *__restrict__ tgt_len, int L, int T, int Mc, int MP) {
+    extern __shared__ float smem[];
+    float *w0 = smem;             // [2][MP]
+    float *w1 = smem + 2 * MP;     // [2][MP]
+    float *bprev = smem + 4 * MP;  // [MP]
+    float *sm_main = smem + 5 * MP;
+    float *sm_leaf = sm_main + (MATCH_LDS ? Mc * T : 0);
+
+    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *mt = match_all + (size_t)b * L * T;
+    const float *Sb = S + (size_t)b * Mc * (T + 2);
+    AuxViewStream av(aux, b, Mc, T);
+    const float ll = Sb[0];
+    const bool valid = lengths_ok(m, n, L, T) && (ll == ll) && (fabsf(ll) != __builtin_huge_valf());
+    if (!valid) return;  // the posterior kernels write zeros for such sentences
+    const int mc = m / 2;
+    if (MATCH_LDS) {
+        for (int i = tid; i < Mc * T; i += NT) {
+            const int a_id = i / T, s = i - a_id * T;
+            const bool ok = a_id < mc && s < n;
+            sm_main[i] = ok ? sanitize(mt[(size_t)(2 * a_id + 1) * T + s]) : NEG_INF_F;
+            sm_leaf[i] = (ok && a_id >= 1) ? sanitize(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
+        }
+        __syncthreads();
+    }
+    auto match_main = [&](int a_id, int s) -> float {
+        if (MATCH_LDS) return sm_main[a_id * T + s];
+        return sanitize(mt[(size_t)(2 * a_id + 1) * T + s]);
+    };
+    auto match_leaf = [&](int a_id, int s) -> float {
+        if (MATCH_LDS) return sm_leaf[a_id * T + s];
+        return a_id >= 1 ? sanitize(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
+    };
+    const float beta00 = -ll;
+    const float w00 = match_main(0, 0) + beta00;
+    for (int i = tid; i < MP; i += NT) {
+        w0[1 * MP + i] = (i == 0) ? w00 : NEG_INF_F;
+        w1[1 * MP + i] = NEG_INF_F;
+        w0[0 * MP + i] = NEG_INF_F;
+        w1[0 * MP + i] = NEG_INF_F;
+        bprev[i] = (i == 0) ? beta00 : NEG_INF_F;
+    }
+    for (int i = tid; i < mc; i += NT) {
+        av.BETA[(size_t)i * (T + 2)] = (i == 0) ? beta00 : NEG_INF_F;
+        av.W0[(size_t)i * (T + 2) + 1] = (i == 0) ? w00 : NEG_INF_F;
+        av.W1[(size_t)i * (T + 2) + 1] = NEG_INF_F;
+    }
+    __syncthreads();
+
+    const int ntiles = (mc + 63) / 64;
+    for (int t = 1; t <= n - 1; t++) {
+        const float *c0 = w0 + (t & 1) * MP, *c1 = w1 + (t & 1) * MP;
+        float *n0 = w0 + ((t + 1) & 1) * MP, *n1 = w1 + ((t + 1) & 1) * MP;
+        for (int tile = 0; tile < ntiles; tile++) {
+            const int c_id = tile * 64 + gidx;
+            const bool live = c_id < mc;
+            const int ci = live ? c_id : 0;
+            const float mc_t = live ? match_main(ci, t) : NEG_INF_F;
+            const float ml_p = live ? match_leaf(ci, t - 1) : NEG_INF_F;
+            const float *at0 = av.At + ((size_t)0 * Mc + ci) * Mc, *at1 = av.At + ((size_t)1 * Mc + ci) * Mc;
+            OnlineLse acc;
+            const int q_end = min((mc + 15) / 16, 4 * tile + 4);
+            for (int qb = 0; qb < q_end; qb += 4) {
+                float v0[4], v1[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int a_id = j + 16 * (qb + u);
+                    const bool ok = live && a_id < mc && a_id <= c_id;
+                    const float x0 = ok ? at0[a_id] : NEG_INF_F;
+                    const float x1 = ok ? at1[a_id] : NEG_INF_F;
+                    const float u0 = (a_id < MP) ? c0[a_id] : NEG_INF_F;
+                    const float u1 = (a_id < MP) ? c1[a_id] : NEG_INF_F;
+                    v0[u] = x0 + u0;
+                    v1[u] = x1 + u1;
+                }
+                acc.add4(v0);
+                acc.add4(v1);
+            }
+            float beta = acc.finish16();
+            if (!live) beta = NEG_INF_F;
+            const int cs = (c_id < MP) ? c_id : 0;
+            const float bp = bprev[cs];
+            const float nw0 = mc_t + beta;
+            const float nw1 = (ml_p + mc_t) + bp;
+            if (j == 0 && c_id < MP) {
+                n0[c_id] = nw0;
+                n1[c_id] = nw1;
+                bprev[c_id] = beta;
+                if (live) {
+                    av.BETA[(size_t)c_id * (T + 2) + t] = beta;
+                    av.W0[(size_t)c_id * (T + 2) + t + 1] = nw0;
+                    av.W1[(size_t)c_id * (T + 2) + t + 1] = nw1;
+                }
+            }
+        }
+        lds_barrier();
+    }
+}
+
+// Rule posteriors from the outside weights: lg[a][k][c] = g * sum_{t=1}^{n-1} exp(links[a][k][c] + Wk[a][t] + S[c][t]).
+// One block per 32x32 tile of (parent, child) pairs; the slab has been zero-filled beforehand.
+__global__ __launch_bounds__(1024) void links_grad_ml1_stream_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
+                                                                    const float *__restrict__ aux_c, const float *__restrict__ links,
+                                                                    const int64_t *__restrict__ out_len,
+                                                                    const int64_t *__restrict__ tgt_len, float *__restrict__ lgrad,
+                                                                    int L, int T, int Mc, int B) {
+    __shared__ float sw0[32][33], sw1[32][33], ss[32][33];
+    const int b = blockIdx.z, at = blockIdx.y, ct = blockIdx.x;
+    if (ct < at) return;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *Sb = S + (size_t)b * Mc * (T + 2);
+    const float ll = Sb[0];
+    if (!(lengths_ok(m, n, L, T) && (ll == ll) && (fabsf(ll) != __builtin_huge_valf()))) return;
+    const int mc = m / 2;
+    if (at * 32 >= mc || ct * 32 >= mc) return;
+    AuxViewStream av(const_cast<float *>(aux_c), b, Mc, T);
+    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)B);
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const int a_id = at * 32 + ty, c_id = ct * 32 + tx;
+    const int a = 2 * a_id + 1, c = 2 * c_id + 1;
+    const bool ok = a_id < mc && c_id < mc && a_id <= c_id;
+    const float *lk = links + (size_t)b * L * 2 * L;
+    const float A0 = ok ? sanitize(lk[((size_t)a * 2 + 0) * L + c]) : NEG_INF_F;
+    const float A1 = (ok && a_id >= 1) ? sanitize(lk[((size_t)a * 2 + 1) * L + c]) : NEG_INF_F;
+    float acc0 = 0.f, acc1 = 0.f;
+    for (int t0 = 1; t0 <= n - 1; t0 += 32) {
+        // rows = nodes of the tile, columns = 32 consecutive target positions
+        const int tt = t0 + tx;
+        const int ra = at * 32 + ty, rc = ct * 32 + ty;
+        const bool tin = tt <= n - 1;
+        sw0[ty][tx] = (tin && ra < mc) ? av.W0[(size_t)ra * (T + 2) + tt] : NEG_INF_F;
+        sw1[ty][tx] = (tin && ra < mc) ? av.W1[(size_t)ra * (T + 2) + tt] : NEG_INF_F;
+        ss[ty][tx] = (tin && rc < mc) ? Sb[(size_t)rc * (T + 2) + tt] : NEG_INF_F;
+        __syncthreads();
+#pragma unroll 8
+        for (int u = 0; u < 32; u++) {
+            const float sc = ss[tx][u];
+            acc0 += __expf((A0 + sw0[ty][u]) + sc);
+            acc1 += __expf((A1 + sw1[ty][u]) + sc);
+        }
+        __syncthreads();
+    }
+    if (ok) {
+        float *lg = lgrad + (size_t)b * L * 2 * L;
+        lg[((size_t)a * 2 + 0) * L + c] = (acc0 == acc0) ? g * acc0 : 0.f;
+        lg[((size_t)a * 2 + 1) * L + c] = (acc1 == acc1) ? g * acc1 : 0.f;
+    }
+}
+
+// Emission posteriors (element-wise) from BETA, F0, F1: the epilogue of the register-resident backward as a kernel.
+__global__ __launch_bounds__(256) void match_grad_ml1_stream_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
+                                                                   const float *__restrict__ aux_c, const float *__restrict__ match_all,
+                                                                   const int64_t *__restrict__ out_len,
+                                                                   const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad, int L,
+                                                                   int T, int Mc, int B) {
+    const int b = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= L * T) return;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *Sb = S + (size_t)b * Mc * (T + 2);
+    const float *mt = match_all + (size_t)b * L * T;
+    float *mg = mgrad + (size_t)b * L * T;
+    const float ll = Sb[0];
+    if (!(lengths_ok(m, n, L, T) && (ll == ll) && (fabsf(ll) != __builtin_huge_valf()))) {
+        mg[i] = 0.f;
+        return;
+    }
+    const int mc = m / 2;
+    AuxViewStream av(const_cast<float *>(aux_c), b, Mc, T);
+    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)B);
+    const int x = i / T, s = i - x * T;
+    float out = 0.f;
+    if (x >= 1 && x < m && s < n) {
+        const int a_id = x >> 1;
+        const size_t row = (size_t)a_id * (T + 2);
+        if (x & 1) {
+            const float bs = av.BETA[row + s];
+            const float mas = sanitize(mt[(size_t)x * T + s]);
+            if (s + 1 <= n - 1) out += __expf(bs + mas + av.F0[row + s + 1]);
+            if (s >= 1 && s + 1 <= n - 1 && a_id >= 1)
+                out += __expf(av.BETA[row + s - 1] + sanitize(mt[(size_t)(x - 1) * T + s - 1]) + mas + av.F1[row + s + 1]);
+            if (a_id == mc - 1 && s == n - 1) out += __expf(bs + mas);
+        } else if (a_id >= 1 && a_id < mc && s + 2 <= n - 1) {
+            out += __expf(av.BETA[row + s] + sanitize(mt[(size_t)x * T + s]) + sanitize(mt[(size_t)(x + 1) * T + s + 1]) +
+                          av.F1[row + s + 2]);
+        }
+        if (!(out == out)) out = 0.f;
+    }
+    mg[i] = g * out;
+}
+
+__global__ void fill_zero_kernel(float *p, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0.f;
+}
+
+constexpr size_t LDS_BUDGET = 128 * 1024;  // of the 160 KB a gfx950 workgroup may use
+
+int launch_fwd_stream(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B,
+                      int L, int T, int Mc, hipStream_t stream) {
+    const int MP = ((Mc + 63) / 64) * 64;
+    const size_t base = (size_t)3 * MP * sizeof(float);
+    const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
+    if (with_match <= LDS_BUDGET) {
+        auto k = inside_fwd_ml1_stream_kernel<true>;
+        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_match));
+        hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_match, stream, match_all, links, ol, tl, S, aux, L, T, Mc, MP);
+    } else {
+        hipLaunchKernelGGL((inside_fwd_ml1_stream_kernel<false>), dim3(B), dim3(NT), base, stream, match_all, links, ol, tl, S, aux, L, T,
+                           Mc, MP);
+    }
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
+int launch_bwd_stream(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
+                      const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, hipStream_t stream) {
+    const int MP = ((Mc + 63) / 64) * 64;
+    const int tiles = (Mc + 31) / 32;
+    hipLaunchKernelGGL(transpose_links_ml1_kernel, dim3(tiles, tiles, B), dim3(256), 0, stream, links, ol, aux, L, T, Mc);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    const size_t base = (size_t)5 * MP * sizeof(float);
+    const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
+    if (with_match <= LDS_BUDGET) {
+        auto k = inside_bwd_ml1_stream_kernel<true>;
+        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_match));
+        hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_match, stream, S, aux, match_all, ol, tl, L, T, Mc, MP);
+    } else {
+        hipLaunchKernelGGL((inside_bwd_ml1_stream_kernel<false>), dim3(B), dim3(NT), base, stream, S, aux, match_all, ol, tl, L, T, Mc, MP);
+    }
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    const size_t nlg = (size_t)B * L * 2 * L;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, stream, lg, nlg);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(links_grad_ml1_stream_kernel, dim3(tiles, tiles, B), dim3(1024), 0, stream, go, S, aux, links, ol, tl, lg, L, T, Mc, B);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(match_grad_ml1_stream_kernel, dim3((L * T + 255) / 256, B), dim3(256), 0, stream, go, S, aux, match_all, ol, tl, mg, L,
+                       T, Mc, B);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
 template <int R>
 int launch_fwd(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B, int L,
                int T, int Mc, hipStream_t stream) {
@@ -466,7 +889,7 @@ int check_dims(const char *who, int64_t B, int64_t L, int64_t T, int64_t ml) {
     PCFGNAT_REQUIRE(B >= 0 && L >= 4 && T >= 2, "%s: need B >= 0, L >= 4, T >= 2 (got B=%lld L=%lld T=%lld)", who, (long long)B,
                     (long long)L, (long long)T);
     PCFGNAT_REQUIRE(ml >= 0, "%s: links must have at least one left option", who);
-    PCFGNAT_REQUIRE(L <= 32768 && T <= 32768 && B <= (1 << 24), "%s: dimension too large", who);
+    PCFGNAT_REQUIRE(L <= 4096 && T <= 4096 && B <= 65535, "%s: dimension too large (L, T <= 4096, B <= 65535)", who);
     if (ml != 1)
         return fail(PCFGNAT_EUNSUPPORTED,
                     "%s: max_left = %lld (links.size(2) = %lld); only max_left = 1 (--left-tree-layer 1, the setting of every shipped "
@@ -483,7 +906,8 @@ using namespace pcfgnat;
 extern "C" size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml) {
     if (B <= 0 || L < 2 || T < 0 || ml < 0) return 0;
     const int64_t Mc = (L - 2) / (ml + 1) + 1;
-    return (size_t)B * 3 * Mc * (T + 2);
+    if (Mc <= 128) return (size_t)B * 3 * Mc * (T + 2);
+    return (size_t)B * ((size_t)5 * Mc * (T + 2) + (size_t)2 * Mc * Mc);
 }
 
 extern "C" int pcfgnat_pcfg_loss(const float *match_all, const float *links, const int64_t *output_length,
@@ -497,7 +921,7 @@ extern "C" int pcfgnat_pcfg_loss(const float *match_all, const float *links, con
     hipStream_t s = (hipStream_t)stream;
     if (Mc <= 64) return launch_fwd<1>(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s);
     if (Mc <= 128) return launch_fwd<2>(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s);
-    return fail(PCFGNAT_EUNSUPPORTED, "pcfg_loss: graph size L=%lld exceeds the built limit of 256 nodes", (long long)L);
+    return launch_fwd_stream(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s);
 }
 
 extern "C" int pcfgnat_pcfg_loss_backward(const float *grad_output, const float *S, float *aux, const float *match_all,
@@ -517,7 +941,8 @@ extern "C" int pcfgnat_pcfg_loss_backward(const float *grad_output, const float 
     if (Mc <= 128)
         return launch_bwd<2>(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
                              (int)L, (int)T, Mc, s);
-    return fail(PCFGNAT_EUNSUPPORTED, "pcfg_loss_backward: graph size L=%lld exceeds the built limit of 256 nodes", (long long)L);
+    return launch_bwd_stream(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
+                             (int)L, (int)T, Mc, s);
 }
 
 extern "C" int pcfgnat_pcfg_best_tree(const float *S, const float *aux, const float *match_all, const float *links,

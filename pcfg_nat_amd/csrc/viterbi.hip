@@ -130,6 +130,83 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
     }
 }
 
+// Streaming variant for graphs whose link slabs do not fit in registers (Mc > 128): rows in tiles of 64, link values
+// fetched from L2 every step.  LDS: three rotating columns (lengths len, len-1, len-2).
+__global__ __launch_bounds__(NT) void viterbi_ml1_stream_kernel(const float *__restrict__ ob_lprob, const float *__restrict__ links,
+                                                               const int64_t *__restrict__ out_len, float *__restrict__ S,
+                                                               int64_t *__restrict__ Rt, int64_t *__restrict__ Lt,
+                                                               int64_t *__restrict__ Mt, int L, int Lq, int MP) {
+    extern __shared__ float col[];  // [3][MP]
+    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j16 = tid & 15;
+    const int m = (int)out_len[b];
+    const float *ob = ob_lprob + (size_t)b * L;
+    const float *lk = links + (size_t)b * L * 2 * L;
+    const size_t tab = (size_t)b * L * Lq;
+    float *Sb = S + tab;
+    int64_t *Rb = Rt + tab, *Lb = Lt + tab, *Mb = Mt + tab;
+    for (size_t i = tid; i < (size_t)L * Lq; i += NT) {
+        Sb[i] = NEG_INF_F;
+        Rb[i] = 0;
+        Lb[i] = 0;
+        Mb[i] = 0;
+    }
+    if (m < 2 || m > L || (m % 2) != 0) return;
+    const int mc = m / 2;
+    for (int i = tid; i < 3 * MP; i += NT) col[i] = NEG_INF_F;
+    __syncthreads();
+    if (tid == 0) {
+        col[1 * MP + mc - 1] = ob[m - 1];
+        if (Lq > 1) Sb[(size_t)(m - 1) * Lq + 1] = ob[m - 1];
+    }
+    __syncthreads();
+
+    const int ntiles = (mc + 63) / 64;
+    const int nq = (mc + 15) / 16;
+    const int len_end = m / 4;
+    for (int len = 2; len < len_end; len++) {
+        const float *cur1 = col + ((len - 1) % 3) * MP, *cur2 = col + ((len - 2) % 3) * MP;
+        float *nxt = col + (len % 3) * MP;
+        for (int tile = 0; tile < ntiles; tile++) {
+            const int a_id = tile * 64 + gidx, a = 2 * a_id + 1;
+            const bool row_ok = a_id < mc;
+            const float ob_a = row_ok ? ob[a] : NEG_INF_F;
+            const float ob_leaf = (row_ok && a_id >= 1) ? ob[a - 1] : NEG_INF_F;
+            const float *l0 = lk + ((size_t)a * 2 + 0) * L, *l1 = lk + ((size_t)a * 2 + 1) * L;
+            float best = NEG_INF_F;
+            int key = 0x7fffffff;
+            for (int q = 4 * tile; q < nq; q++) {
+                const int c_id = j16 + 16 * q;
+                const bool ok = row_ok && c_id < mc && c_id >= a_id;
+                const float x0 = ok ? l0[2 * c_id + 1] : NEG_INF_F;
+                const float x1 = (ok && a_id >= 1) ? l1[2 * c_id + 1] : NEG_INF_F;
+                const float s1 = (c_id < MP) ? cur1[c_id] : NEG_INF_F;
+                const float s2 = (c_id < MP) ? cur2[c_id] : NEG_INF_F;
+                const float c0 = nan_to_ninf(((x0 + 0.f) + s1) + ob_a);
+                const float c1 = nan_to_ninf(((x1 + ob_leaf) + s2) + ob_a);
+                const int rel = c_id - a_id;
+                if (c0 != NEG_INF_F) take_better(best, key, c0, tie_key(rel, 0));
+                if (c1 != NEG_INF_F) take_better(best, key, c1, tie_key(rel, 1));
+            }
+            row16_argmax_step<DPP_QUAD_XOR1>(best, key);
+            row16_argmax_step<DPP_QUAD_XOR2>(best, key);
+            row16_argmax_step<DPP_ROW_HALF_MIRROR>(best, key);
+            row16_argmax_step<DPP_ROW_MIRROR>(best, key);
+            if (j16 == 0 && a_id < MP) {
+                nxt[a_id] = best;
+                if (best != NEG_INF_F && row_ok) {
+                    const int jj = key & 1, rel = (key >> 1) & 0x7fffff;
+                    const size_t o = (size_t)a * Lq + len;
+                    Sb[o] = best;
+                    Lb[o] = jj ? (a - 1) : 0;
+                    Rb[o] = 2 * (a_id + rel) + 1;
+                    Mb[o] = jj;
+                }
+            }
+        }
+        lds_barrier();
+    }
+}
+
 // One walk per sentence (pcfg_loss.cpp:22-59).  Shared by the device kernel and the host entry point.
 __host__ __device__ inline int64_t readout_one(int64_t pred_len, int64_t max_h, const int64_t *Li, const int64_t *Ri,
                                                const int64_t *Mi, const int64_t *tok, const int64_t *mask, int64_t mask_dim,
@@ -204,8 +281,12 @@ extern "C" int pcfgnat_pcfg_viterbi(const float *ob_lprob, const float *links, c
         hipLaunchKernelGGL((viterbi_ml1_kernel<1>), dim3((unsigned)B), dim3(NT), 0, s, ob_lprob, links, output_length, S, R, Lt, M, (int)L, Lq);
     else if (Mc <= 128)
         hipLaunchKernelGGL((viterbi_ml1_kernel<2>), dim3((unsigned)B), dim3(NT), 0, s, ob_lprob, links, output_length, S, R, Lt, M, (int)L, Lq);
-    else
-        return fail(PCFGNAT_EUNSUPPORTED, "pcfg_viterbi: graph size L=%lld exceeds the built limit of 256 nodes", (long long)L);
+    else {
+        PCFGNAT_REQUIRE(L <= 4096, "pcfg_viterbi: graph size L=%lld exceeds 4096 nodes", (long long)L);
+        const int MP = ((Mc + 63) / 64) * 64;
+        hipLaunchKernelGGL(viterbi_ml1_stream_kernel, dim3((unsigned)B), dim3(NT), (size_t)3 * MP * sizeof(float), s, ob_lprob, links,
+                           output_length, S, R, Lt, M, (int)L, Lq, MP);
+    }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }

@@ -134,6 +134,12 @@ def _train_case(name):
         return synth.training_batch(5, 64, 12, 300, [64, 40, 22, 8, 4], [12, 9, 7, 3, 2], seed=8)
     if name == "L256":
         return synth.training_batch(3, 256, 40, 200, [256, 200, 130], [40, 33, 38], seed=12)
+    if name == "L512":  # streaming kernels, emissions staged in LDS
+        return synth.training_batch(3, 512, 30, 100, [512, 300, 258], [30, 25, 30], seed=13)
+    if name == "L512_long":  # config-3 shaped: streaming kernels, emissions read from global memory
+        return synth.training_batch(2, 512, 140, 100, [512, 444], [140, 120], seed=14)
+    if name == "L1026":
+        return synth.training_batch(2, 1026, 20, 50, [1026, 600], [20, 17], seed=15)
     raise KeyError(name)
 
 
@@ -143,7 +149,7 @@ def _match_for(batch):
     return harness.eos_masked(sel.float(), batch["output_length"], batch["target_length"])
 
 
-@pytest.mark.parametrize("case", ["cfg1", "wmt_small", "ragged_short", "L256"])
+@pytest.mark.parametrize("case", ["cfg1", "wmt_small", "ragged_short", "L256", "L512", "L512_long", "L1026"])
 def test_inside_forward_backward_vs_oracle(case):
     batch = _train_case(case)
     match = _match_for(batch)
@@ -186,7 +192,7 @@ def test_inside_tables_match_oracle_layout():
     assert np.allclose(S[fin], S64[fin], rtol=1e-5, atol=1e-5)
 
 
-@pytest.mark.parametrize("case", ["cfg1", "wmt_small", "ragged_short", "L256"])
+@pytest.mark.parametrize("case", ["cfg1", "wmt_small", "ragged_short", "L256", "L512", "L512_long"])
 def test_best_tree_bit_exact(case):
     batch = _train_case(case)
     match = _match_for(batch)
@@ -238,10 +244,12 @@ def _decode_case(name):
         return synth.decode_batch([5, 9, 16, 3, 12], seed=3, V=500)
     if name == "L256":
         return synth.decode_batch([64, 40, 33], seed=4, V=300)
+    if name == "L400":  # longest graph of the inference configuration: streaming kernel
+        return synth.decode_batch([100, 71, 5], seed=6, V=100)
     raise KeyError(name)
 
 
-@pytest.mark.parametrize("case", ["short", "L256"])
+@pytest.mark.parametrize("case", ["short", "L256", "L400"])
 def test_viterbi_tables_bit_exact_and_decode(case):
     batch = _decode_case(case)
     ob, tok = synth.ob_and_tokens(batch["logits"])
