@@ -20,6 +20,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+# HBM bytes per launch of lsg_fwd_kernel<half, grad> at this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled against
+# a plain device copy of known size (FETCH x1.99989, WRITE x1.0); summary in profiles/lsg_cfg2_hbm_traffic_pmc.md
+LSG_FWD_MEASURED_TRAFFIC_BYTES = 820.75e6
 
 
 def parse():
@@ -30,6 +33,9 @@ def parse():
     ap.add_argument("--cpu-sentences", type=int, default=40, help="sentences of the batch timed on the CPU oracle")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the viterbi decode timing")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain device copy of a logits-sized fp16 buffer (409.6 MB read, 409.6 MB written): "
+                         "the reference point for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--unfused", action="store_true",
                     help="issue the criterion's glue (eos mask, gradient scaling) as separate torch ops, like the reference")
     return ap.parse_args()
@@ -141,6 +147,11 @@ def main():
     sample_logits = bufs[args.warmup][:args.cpu_sentences].cpu() if not args.no_cpu_baseline else None
     torch.cuda.synchronize()
 
+    if args.calibrate_copy:
+        dst = torch.empty_like(bufs[0])
+        dst.copy_(bufs[0])
+        torch.cuda.synchronize()
+        del dst
     pairs = {}
 
     def mark(name, phase):
@@ -189,7 +200,7 @@ def main():
                                + ("as separate torch ops" if args.unfused else "folded into the kernels"),
                    "global_batch": B, "graph_nodes": L, "target_len": T, "vocab": V},
         "roofline": {"bound": "hbm", "kernel": "lsg_fwd_kernel<half, grad>", "achieved": achieved, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": LSG_FWD_MEASURED_TRAFFIC_BYTES,
                      "algorithmic_bytes": fwd_bytes, "avg_ms": kern_ms["lsg_fwd"]},
         "kernels_ms": kern_ms,
         "lsg_bwd_gbs": bwd_achieved,
