@@ -103,6 +103,27 @@ int pcfgnat_pcfg_loss_backward(const float *grad_output, const float *S, float *
                                int64_t ml, void *stream);
 
 /*
+ * The criterion's reduction (nat_pcfg_loss.py:123-135) on the device: out[0] = -(1/B) sum_b ll_b/target_length[b] over
+ * sentences with a finite ll_b = S[b,0,0]; out[1] = number of sentences with a non-finite ll_b.  Deterministic.
+ */
+int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *out, int64_t B, int64_t L, int64_t T,
+                           int64_t ml, void *stream);
+
+/*
+ * One call for the criterion's whole training pass (nat_pcfg_loss.py:98-145 plus the backward autograd derives from it):
+ * logsoftmax_gather with eos mask -> inside forward -> inside backward with weights -1/(target_length*B) ->
+ * logsoftmax_gather backward -> loss.  targets is the contiguous [B,T] int64 target matrix (the gather index of every
+ * graph node).  On return (stream order) logits holds d loss / d logits, links_grad d loss / d links, loss_out[0] the
+ * loss, loss_out[1] the number of invalid sentences; match_all, S, aux, match_all_grad are caller workspaces of the
+ * shapes documented at the individual entry points.  events: NULL, or eight hipEvent_t (entries may be NULL) recorded on the
+ * stream before/after the gather forward, the inside forward, the inside backward and the gather backward (for timing).
+ */
+int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, const float *links,
+                           const int64_t *output_length, const int64_t *target_length, float *match_all, float *S,
+                           float *aux, float *match_all_grad, float *links_grad, float *loss_out, int64_t B, int64_t L,
+                           int64_t V, int64_t T, int64_t ml, void *stream, void *const *events);
+
+/*
  * Replaces pcfg_best_tree (pcfg_best_tree.cu:333-360): greedy top-down trace over the inside tables.
  *   tree [B,L] int64 out: target position aligned to each node, -1 for nodes off the tree.
  * Exact ties are resolved in the reference's scan order (lanes 0 > 2 > 1 > 3 of a 4-wide strided scan).

@@ -11,3 +11,38 @@ char *error_buffer() {
 extern "C" int pcfgnat_abi_version(void) { return 1; }
 
 extern "C" const char *pcfgnat_last_error(void) { return pcfgnat::error_buffer(); }
+
+// One call for the whole training pass of the criterion (fs_plugins/criterions/nat_pcfg_loss.py:98-145 and the backward
+// autograd derives from it): gather with eos mask -> inside forward -> inside backward seeded with -1/(n_b*B) ->
+// in-place gather backward -> loss.  Five kernels enqueued back to back; nothing is allocated.
+extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, const float *links,
+                                      const int64_t *output_length, const int64_t *target_length, float *match_all, float *S,
+                                      float *aux, float *match_all_grad, float *links_grad, float *loss_out, int64_t B, int64_t L,
+                                      int64_t V, int64_t T, int64_t ml, void *stream, void *const *events) {
+    if (dtype == PCFGNAT_F64)
+        return pcfgnat::fail(PCFGNAT_EUNSUPPORTED, "criterion_step: float64 logits gather to float64, the PCFG kernels are float32");
+    hipStream_t s = (hipStream_t)stream;
+#define PCFGNAT_MARK(i)                                                        \
+    do {                                                                       \
+        if (events && events[i]) PCFGNAT_HIP_CHECK(hipEventRecord((hipEvent_t)events[i], s)); \
+    } while (0)
+    PCFGNAT_MARK(0);
+    int rc = pcfgnat_logsoftmax_gather_eos(logits, dtype, targets, T, 0, 1, match_all, 1, output_length, target_length, B, L, V, T, stream);
+    if (rc != PCFGNAT_OK) return rc;
+    PCFGNAT_MARK(1);
+    PCFGNAT_MARK(2);
+    rc = pcfgnat_pcfg_loss(match_all, links, output_length, target_length, S, aux, B, L, T, ml, stream);
+    if (rc != PCFGNAT_OK) return rc;
+    PCFGNAT_MARK(3);
+    PCFGNAT_MARK(4);
+    rc = pcfgnat_pcfg_loss_backward(nullptr, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, B, L, T,
+                                    ml, stream);
+    if (rc != PCFGNAT_OK) return rc;
+    PCFGNAT_MARK(5);
+    PCFGNAT_MARK(6);
+    rc = pcfgnat_logsoftmax_gather_backward(logits, dtype, targets, T, 0, 1, match_all_grad, B, L, V, T, stream);
+    if (rc != PCFGNAT_OK) return rc;
+    PCFGNAT_MARK(7);
+#undef PCFGNAT_MARK
+    return pcfgnat_criterion_loss(S, target_length, loss_out, B, L, T, ml, stream);
+}

@@ -808,6 +808,35 @@ __global__ void fill_zero_kernel(float *p, size_t n) {
 
 constexpr size_t LDS_BUDGET = 128 * 1024;  // of the 160 KB a gfx950 workgroup may use
 
+// loss = -(1/B) * sum_b [ll_b finite] ll_b / n_b and the number of invalid sentences (nat_pcfg_loss.py:123-135), reduced
+// in a fixed order by one workgroup.  out[0] = loss, out[1] = invalid count.
+__global__ __launch_bounds__(256) void criterion_loss_kernel(const float *__restrict__ S, const int64_t *__restrict__ tgt_len,
+                                                            float *__restrict__ out, int B, int Mc, int T) {
+    __shared__ float s_sum[256];
+    __shared__ float s_bad[256];
+    float acc = 0.f, bad = 0.f;
+    for (int b = threadIdx.x; b < B; b += 256) {
+        const float ll = S[(size_t)b * Mc * (T + 2)];
+        const bool ok = (ll == ll) && (fabsf(ll) != __builtin_huge_valf());
+        if (ok) acc += ll / (float)tgt_len[b];
+        else bad += 1.f;
+    }
+    s_sum[threadIdx.x] = acc;
+    s_bad[threadIdx.x] = bad;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if ((int)threadIdx.x < o) {
+            s_sum[threadIdx.x] += s_sum[threadIdx.x + o];
+            s_bad[threadIdx.x] += s_bad[threadIdx.x + o];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        out[0] = -s_sum[0] / (float)B;
+        out[1] = s_bad[0];
+    }
+}
+
 int launch_fwd_stream(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B,
                       int L, int T, int Mc, hipStream_t stream) {
     const int MP = ((Mc + 63) / 64) * 64;
@@ -943,6 +972,17 @@ extern "C" int pcfgnat_pcfg_loss_backward(const float *grad_output, const float 
                              (int)L, (int)T, Mc, s);
     return launch_bwd_stream(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
                              (int)L, (int)T, Mc, s);
+}
+
+extern "C" int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *out, int64_t B, int64_t L, int64_t T,
+                                      int64_t ml, void *stream) {
+    int rc = check_dims("criterion_loss", B, L, T, ml);
+    if (rc != PCFGNAT_OK) return rc;
+    PCFGNAT_REQUIRE(B >= 1 && S && target_length && out, "criterion_loss: null pointer or empty batch");
+    const int Mc = (int)((L - 2) / 2 + 1);
+    hipLaunchKernelGGL(criterion_loss_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, S, target_length, out, (int)B, Mc, (int)T);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
 }
 
 extern "C" int pcfgnat_pcfg_best_tree(const float *S, const float *aux, const float *match_all, const float *links,

@@ -82,11 +82,22 @@ __device__ __forceinline__ double neg_inf(double) { return -__builtin_huge_val()
 __device__ __forceinline__ float vmax(float a, float b) { return fmaxf(a, b); }
 __device__ __forceinline__ double vmax(double a, double b) { return fmax(a, b); }
 
+#ifndef LSG_LOAD
+#define LSG_LOAD 1
+#endif
+#if LSG_LOAD == 1
 __device__ __forceinline__ vec16 load16(const vec16 *p) { return __builtin_nontemporal_load(p); }
+#else
+__device__ __forceinline__ vec16 load16(const vec16 *p) { return *p; }
+#endif
 // Makes the compiler forget what it knows about a register-resident chunk, so that each pass re-derives the widened
 // values from the packed registers instead of keeping both copies alive (which would halve the occupancy).
 __device__ __forceinline__ void opaque(vec16 &v) { asm volatile("" : "+v"(v)); }
+#if !defined(LSG_STORE) || LSG_STORE == 1
 __device__ __forceinline__ void store16(vec16 *p, const vec16 &v) { __builtin_nontemporal_store(v, p); }
+#else
+__device__ __forceinline__ void store16(vec16 *p, const vec16 &v) { *p = v; }
+#endif
 
 // Splits a row that starts at an arbitrary element address into [head scalars][16-byte chunks][tail scalars].
 template <typename T>

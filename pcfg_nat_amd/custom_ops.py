@@ -351,3 +351,47 @@ def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unre
         raise RuntimeError("viterbi_decoding: malformed traces")
     maxlen = int(cnt.max()) if B else 0
     return out[:, :maxlen].to(torch.float32)
+
+
+def pcfg_criterion_step(logits, targets, links, output_length, target_length, events=None):
+    """The criterion's whole training pass in one native call (``pcfgnat_criterion_step``): ``logits`` [B,L,V] (fp16 or
+    fp32, contiguous) is consumed in place and holds d loss / d logits afterwards.  ``events``: optional list of eight
+    ``torch.cuda.Event(enable_timing=True)`` (each recorded at least once before; entries may be None) that the library records before/after
+    the gather forward, inside forward, inside backward and gather backward.  Returns
+    (loss_and_invalid [2] float32, links_grad, ll [B], match_all_eos_masked)."""
+    lib = get_pcfg_kernel()
+    _need_cuda("pcfg_criterion_step", logits, targets, links, output_length, target_length)
+    if logits.dim() != 3 or not logits.is_contiguous():
+        raise RuntimeError("pcfg_criterion_step: logits must be a contiguous [bsz, prelen, vocab] tensor")
+    B, L, V = logits.shape
+    if targets.dim() != 2 or targets.size(0) != B or targets.dtype != torch.int64:
+        raise RuntimeError("pcfg_criterion_step: targets must be an int64 [bsz, tarlen] tensor")
+    T = targets.size(1)
+    code = _DTYPE_CODE.get(logits.dtype)
+    if code is None or code == _lib.F64:
+        raise RuntimeError("pcfg_criterion_step: logits must be float16 or float32")
+    if links.dim() != 4 or links.size(0) != B or links.size(1) != L or links.size(3) != L or links.dtype != torch.float32:
+        raise RuntimeError("pcfg_criterion_step: links must be float32 [bsz, prelen, max_left+1, prelen]")
+    ml = links.size(2) - 1
+    targets, links = targets.contiguous(), links.contiguous()
+    ol = _lengths("pcfg_criterion_step", output_length, B)
+    tl = _lengths("pcfg_criterion_step", target_length, B)
+    Mc = (L - 2) // (ml + 1) + 1
+    dev = logits.device
+    ev_arr = None
+    if events is not None:
+        import ctypes
+        if len(events) != 8:
+            raise RuntimeError("pcfg_criterion_step: events must hold eight torch.cuda.Event objects")
+        ev_arr = (ctypes.c_void_p * 8)(*[(e.cuda_event if e is not None else None) for e in events])
+    with torch.cuda.device(dev):
+        match = torch.empty((B, L, T), dtype=torch.float32, device=dev)
+        S = torch.empty((B, Mc, T + 2), dtype=torch.float32, device=dev)
+        aux = torch.empty((max(1, lib.pcfgnat_pcfg_aux_floats(B, L, T, ml)),), dtype=torch.float32, device=dev)
+        mg = torch.empty_like(match)
+        lg = torch.empty_like(links)
+        out = torch.empty((2,), dtype=torch.float32, device=dev)
+        _lib.check(lib.pcfgnat_criterion_step(logits.data_ptr(), code, targets.data_ptr(), links.data_ptr(), ol.data_ptr(),
+                                              tl.data_ptr(), match.data_ptr(), S.data_ptr(), aux.data_ptr(), mg.data_ptr(),
+                                              lg.data_ptr(), out.data_ptr(), B, L, V, T, ml, _stream(logits), ev_arr), lib)
+    return out, lg, S[:, 0, 0], match
