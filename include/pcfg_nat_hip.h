@@ -103,6 +103,16 @@ int pcfgnat_pcfg_loss_backward(const float *grad_output, const float *S, float *
                                int64_t ml, void *stream);
 
 /*
+ * pcfgnat_pcfg_loss followed by pcfgnat_pcfg_loss_backward (same arguments and results: S, match_all_grad, links_grad)
+ * as one launch when every per-sentence table fits in LDS (it does for all shipped training shapes), otherwise as the
+ * two calls.  aux is only touched by the two-call path.
+ */
+int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *match_all, const float *links,
+                                       const int64_t *output_length, const int64_t *target_length, float *S, float *aux,
+                                       float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T, int64_t ml,
+                                       void *stream);
+
+/*
  * The criterion's reduction (nat_pcfg_loss.py:123-135) on the device: out[0] = -(1/B) sum_b ll_b/target_length[b] over
  * sentences with a finite ll_b = S[b,0,0]; out[1] = number of sentences with a non-finite ll_b.  Deterministic.
  */

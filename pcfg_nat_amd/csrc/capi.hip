@@ -31,12 +31,10 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
     if (rc != PCFGNAT_OK) return rc;
     PCFGNAT_MARK(1);
     PCFGNAT_MARK(2);
-    rc = pcfgnat_pcfg_loss(match_all, links, output_length, target_length, S, aux, B, L, T, ml, stream);
-    if (rc != PCFGNAT_OK) return rc;
-    PCFGNAT_MARK(3);
+    PCFGNAT_MARK(3);  // forward and backward run as one launch where the tables fit in LDS: bracketed together by 4..5
     PCFGNAT_MARK(4);
-    rc = pcfgnat_pcfg_loss_backward(nullptr, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, B, L, T,
-                                    ml, stream);
+    rc = pcfgnat_pcfg_loss_forward_backward(nullptr, match_all, links, output_length, target_length, S, aux, match_all_grad,
+                                            links_grad, B, L, T, ml, stream);
     if (rc != PCFGNAT_OK) return rc;
     PCFGNAT_MARK(5);
     PCFGNAT_MARK(6);

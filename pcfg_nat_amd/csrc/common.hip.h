@@ -101,4 +101,18 @@ __device__ __forceinline__ void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+
+// Phase timestamps for tuning builds only (-DPCFGNAT_PHASE_TIMING): thread 0 of workgroup 0 stores the 100 MHz wall clock.
+#ifdef PCFGNAT_PHASE_TIMING
+__device__ unsigned long long pcfgnat_phase_ts[32];
+#define PCFGNAT_PHASE(i)                                                                     \
+    do {                                                                                     \
+        if (blockIdx.x == 0 && threadIdx.x == 0) pcfgnat::pcfgnat_phase_ts[i] = wall_clock64(); \
+    } while (0)
+#else
+#define PCFGNAT_PHASE(i) \
+    do {                 \
+    } while (0)
+#endif
+
 }  // namespace pcfgnat

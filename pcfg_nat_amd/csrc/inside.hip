@@ -32,7 +32,7 @@ __device__ __forceinline__ float lse2(float a, float b) {
     return m + __logf(__expf(a - m) + __expf(b - m));
 }
 
-// Aux layout per sentence: F0, F1, BETA, each [Mc][T+2].
+// Aux layout per sentence (Mc <= 128): F0, F1, BETA, each [Mc][T+2], log-domain values in base 2.
 struct AuxView {
     float *F0, *F1, *BETA;
     __device__ AuxView(float *aux, int b, int Mc, int T) {
@@ -49,123 +49,130 @@ __device__ __forceinline__ bool lengths_ok(int m, int n, int L, int T) {
 }
 
 // ------------------------------------------------------------------------------------------------------------
-// Forward.  R = ceil(Mc/64) nodes per 16-lane row, CN = 4R children per lane.
-// Dynamic LDS: col[2][64R] floats, then (if MATCH_LDS) match rows of main nodes [Mc][T] and of their leaves [Mc][T].
+// Register-resident sweeps (Mc <= 128).  512 threads = 8 waves; a node is owned by an 8-lane group (two groups per DPP
+// row), the 8 lanes stride over the other index in chunks of 8.  Link slabs are triangular (children c >= a), so wave w
+// takes node block perm(w) = {0,1,2,3,7,6,5,4}[w] of every 64-node tile: the two waves that share a SIMD (w, w+4) then
+// own blocks p and 7-p and together always process 9 of the 16 chunks, whole chunks below the diagonal being skipped
+// with wave-uniform branches.  All log-domain quantities are held in base 2 (pre-multiplied by log2 e) so that the
+// hardware exp2/log2 are used without extra multiplies; tables that leave the kernel in the reference's layout (S) are
+// converted back on store, the private auxiliary tables (F0, F1, BETA) stay in base 2.
 // ------------------------------------------------------------------------------------------------------------
-template <int R, bool MATCH_LDS>
-__global__ __launch_bounds__(NT) void inside_fwd_ml1_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
-                                                           const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
-                                                           float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc) {
-    constexpr int CN = 4 * R;
+constexpr int NTR = 512;
+constexpr size_t LDS_BUDGET = 128 * 1024;  // of the 160 KB a gfx950 workgroup may use
+constexpr float LOG2E_F = 1.4426950408889634f;
+constexpr float LN2_F = 0.6931471805599453f;
+
+__device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float lg2(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float to_b2(float natural) { return sanitize(natural) * LOG2E_F; }
+
+__device__ __forceinline__ float row8_max(float v) {
+    v = fmaxf(v, dpp_f<DPP_QUAD_XOR1>(v));
+    v = fmaxf(v, dpp_f<DPP_QUAD_XOR2>(v));
+    v = fmaxf(v, dpp_f<DPP_ROW_HALF_MIRROR>(v));
+    return v;
+}
+__device__ __forceinline__ float row8_sum(float v) {
+    v += dpp_f<DPP_QUAD_XOR1>(v);
+    v += dpp_f<DPP_QUAD_XOR2>(v);
+    v += dpp_f<DPP_ROW_HALF_MIRROR>(v);
+    return v;
+}
+__device__ __forceinline__ float lse2_b2(float a, float b) {
+    const float m = fmaxf(a, b);
+    if (m == NEG_INF_F) return NEG_INF_F;
+    return m + lg2(ex2(a - m) + ex2(b - m));
+}
+// node block of wave w inside a 64-node tile (wave-uniform scalar)
+__device__ __forceinline__ int wave_block(int wave) { return __builtin_amdgcn_readfirstlane(wave < 4 ? wave : 11 - wave); }
+
+// Keeps a value (and the load that produced it) out of the conditionally executed blocks that consume it, so that all
+// LDS reads of a step are issued back to back instead of one per branch, each followed by its own wait.
+__device__ __forceinline__ void pin(float &v) { asm volatile("" : "+v"(v)); }
+
+struct FwdSweepArgs {
+    float *col, *sm_main, *sm_leaf, *sm_S, *sm_F0, *sm_F1;
+    const float *mt;
+    float *Sb, *gF0, *gF1;
+    int n, mc, Mc, T, j, g8;
+};
+
+// The forward sweep of one wave, specialised on its node block P so that the chunks below the diagonal (q < 8r + P)
+// vanish at compile time.  Executes n-1 workgroup barriers regardless of P.
+template <int R, bool TAB_LDS, int P>
+__device__ __forceinline__ void fwd_sweep(const float (&A0)[R][8 * R], const float (&A1)[R][8 * R], const FwdSweepArgs &x) {
+    constexpr int NQ = 8 * R;
     constexpr int MP = 64 * R;
-    extern __shared__ float smem[];
-    float *col = smem;              // [2][MP]
-    float *sm_main = smem + 2 * MP;  // [Mc][T]
-    float *sm_leaf = sm_main + (MATCH_LDS ? Mc * T : 0);
-
-    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
-    const int m = (int)out_len[b], n = (int)tgt_len[b];
-    const float *mt = match_all + (size_t)b * L * T;
-    const float *lk = links + (size_t)b * L * 2 * L;
-    float *Sb = S + (size_t)b * Mc * (T + 2);
-    AuxView av(aux, b, Mc, T);
-
-    if (!lengths_ok(m, n, L, T)) {  // out of contract: poison the log-likelihood, touch nothing else
-        for (int i = tid; i < Mc * (T + 2); i += NT) Sb[i] = (i == 0) ? __builtin_nanf("") : NEG_INF_F;
-        return;
-    }
-    const int mc = m / 2;  // active main-chain nodes: a_id < mc
-
-    // link slabs -> registers
-    float A0[R][CN], A1[R][CN];
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-        const int a_id = gidx + 64 * r, a = 2 * a_id + 1;
-#pragma unroll
-        for (int q = 0; q < CN; q++) {
-            const int c_id = j + 16 * q, c = 2 * c_id + 1;
-            const bool ok = a_id < mc && c_id < mc && c_id >= a_id;
-            A0[r][q] = ok ? sanitize(lk[((size_t)a * 2 + 0) * L + c]) : NEG_INF_F;
-            A1[r][q] = (ok && a_id >= 1) ? sanitize(lk[((size_t)a * 2 + 1) * L + c]) : NEG_INF_F;
-        }
-    }
-    if (MATCH_LDS) {
-        for (int i = tid; i < Mc * T; i += NT) {
-            const int a_id = i / T, s = i - a_id * T;
-            const bool ok = a_id < mc && s < n;
-            sm_main[i] = ok ? sanitize(mt[(size_t)(2 * a_id + 1) * T + s]) : NEG_INF_F;
-            sm_leaf[i] = (ok && a_id >= 1) ? sanitize(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
-        }
-    }
-    // cells of S the sweep never writes: rows beyond the sentence, columns from n-1 on (except the base cell)
-    for (int i = tid; i < Mc * (T + 2); i += NT) {
-        const int a_id = i / (T + 2), s = i - a_id * (T + 2);
-        if (a_id >= mc || s >= n - 1) {
-            float v = NEG_INF_F;
-            if (a_id == mc - 1 && s == n - 1) v = sanitize(mt[(size_t)(m - 1) * T + (n - 1)]);
-            Sb[i] = v;
-        }
-    }
-    // column n-1: only the last node, emitting the last token (pcfg_loss.cu:142-147)
-    for (int i = tid; i < MP; i += NT) col[((n - 1) & 1) * MP + i] = (i == mc - 1) ? sanitize(mt[(size_t)(m - 1) * T + (n - 1)]) : NEG_INF_F;
+    const int T = x.T, TS = x.T + 2, j = x.j;
     float F1prev[R];
 #pragma unroll
     for (int r = 0; r < R; r++) F1prev[r] = NEG_INF_F;
-    __syncthreads();
-
-    for (int t = n - 1; t >= 1; t--) {
-        const float *cur = col + (t & 1) * MP;
-        float *nxt = col + ((t - 1) & 1) * MP;
-        float sc[CN];
-#pragma unroll
-        for (int q = 0; q < CN; q++) sc[q] = cur[j + 16 * q];
+    for (int t = x.n - 1; t >= 1; t--) {
+        const float *cur = x.col + (t & 1) * MP;
+        float *nxt = x.col + ((t - 1) & 1) * MP;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const int a_id = gidx + 64 * r;
-            float v0[CN], v1[CN];
+            const int a_id = 64 * r + 8 * P + x.g8;
+            const int q0 = 8 * r + P;  // chunks below hold only children c < a
+            const int ai = (a_id < x.Mc) ? a_id : 0;
+            float sc[NQ];
+#pragma unroll
+            for (int q = 0; q < NQ; q++)
+                if (q >= q0) sc[q] = cur[j + 8 * q];
+            float ma_p, ml_p, ma_t;  // match[a][t-1], match[a-1][t-1], match[a][t]
+            if (TAB_LDS) {
+                ma_p = x.sm_main[ai * T + t - 1];
+                ml_p = x.sm_leaf[ai * T + t - 1];
+                ma_t = x.sm_main[ai * T + t];
+            } else {
+                const size_t ra = (size_t)(2 * ai + 1) * T, rl = (size_t)(2 * ai) * T;
+                const float x0 = x.mt[ra + t - 1], x1 = x.mt[rl + t - 1], x2 = x.mt[ra + t];
+                const bool ok = a_id < x.mc;
+                ma_p = ok ? to_b2(x0) : NEG_INF_F;
+                ml_p = (ok && a_id >= 1) ? to_b2(x1) : NEG_INF_F;
+                ma_t = ok ? to_b2(x2) : NEG_INF_F;
+            }
+            float v0[NQ], v1[NQ];
             float m0 = NEG_INF_F, m1 = NEG_INF_F;
 #pragma unroll
-            for (int q = 0; q < CN; q++) {
-                v0[q] = A0[r][q] + sc[q];
-                v1[q] = A1[r][q] + sc[q];
-                m0 = fmaxf(m0, v0[q]);
-                m1 = fmaxf(m1, v1[q]);
+            for (int q = 0; q < NQ; q++) {
+                if (q >= q0) {
+                    v0[q] = A0[r][q] + sc[q];
+                    v1[q] = A1[r][q] + sc[q];
+                    m0 = fmaxf(m0, v0[q]);
+                    m1 = fmaxf(m1, v1[q]);
+                }
             }
-            m0 = row16_max(m0);
-            m1 = row16_max(m1);
+            m0 = row8_max(m0);
+            m1 = row8_max(m1);
             const float m0s = (m0 == NEG_INF_F) ? 0.f : m0, m1s = (m1 == NEG_INF_F) ? 0.f : m1;
             float e0 = 0.f, e1 = 0.f;
 #pragma unroll
-            for (int q = 0; q < CN; q++) {
-                e0 += __expf(v0[q] - m0s);
-                e1 += __expf(v1[q] - m1s);
+            for (int q = 0; q < NQ; q++) {
+                if (q >= q0) {
+                    e0 += ex2(v0[q] - m0s);
+                    e1 += ex2(v1[q] - m1s);
+                }
             }
-            e0 = row16_sum(e0);
-            e1 = row16_sum(e1);
-            const float F0 = (m0 == NEG_INF_F) ? NEG_INF_F : m0 + __logf(e0);
-            const float F1 = (m1 == NEG_INF_F) ? NEG_INF_F : m1 + __logf(e1);
-            float ma_p, ml_p, ma_t;  // match[a][t-1], match[a-1][t-1], match[a][t]
-            if (MATCH_LDS) {
-                const int ai = (a_id < Mc) ? a_id : 0;
-                ma_p = sm_main[ai * T + t - 1];
-                ml_p = sm_leaf[ai * T + t - 1];
-                ma_t = sm_main[ai * T + t];
-            } else {
-                const bool ok = a_id < mc;
-                const size_t ra = (size_t)(2 * a_id + 1) * T, rl = (size_t)(2 * a_id) * T;
-                ma_p = ok ? sanitize(mt[ra + t - 1]) : NEG_INF_F;
-                ml_p = (ok && a_id >= 1) ? sanitize(mt[rl + t - 1]) : NEG_INF_F;
-                ma_t = ok ? sanitize(mt[ra + t]) : NEG_INF_F;
-            }
-            float s_new = lse2(ma_p + F0, (ml_p + ma_t) + F1prev[r]);
-            if (a_id >= mc) s_new = NEG_INF_F;
+            e0 = row8_sum(e0);
+            e1 = row8_sum(e1);
+            const float F0 = (m0 == NEG_INF_F) ? NEG_INF_F : m0 + lg2(e0);
+            const float F1 = (m1 == NEG_INF_F) ? NEG_INF_F : m1 + lg2(e1);
+            float s_new = lse2_b2(ma_p + F0, (ml_p + ma_t) + F1prev[r]);
+            if (a_id >= x.mc) s_new = NEG_INF_F;
             F1prev[r] = F1;
             if (j == 0) {
                 nxt[a_id] = s_new;
-                if (a_id < mc) {
-                    Sb[(size_t)a_id * (T + 2) + (t - 1)] = s_new;
-                    av.F0[(size_t)a_id * (T + 2) + t] = F0;
-                    av.F1[(size_t)a_id * (T + 2) + t] = F1;
+                if (a_id < x.mc) {
+                    if (TAB_LDS) {
+                        x.sm_S[a_id * TS + (t - 1)] = s_new;
+                        x.sm_F0[a_id * TS + t] = F0;
+                        x.sm_F1[a_id * TS + t] = F1;
+                    } else {
+                        x.Sb[(size_t)a_id * TS + (t - 1)] = s_new * LN2_F;
+                        x.gF0[(size_t)a_id * TS + t] = F0;
+                        x.gF1[(size_t)a_id * TS + t] = F1;
+                    }
                 }
             }
         }
@@ -173,31 +180,231 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_kernel(const float *__restr
     }
 }
 
-// ------------------------------------------------------------------------------------------------------------
-// Backward: outside sweep t = 1 .. n-1 (one DPP row per child node c, lanes strided over parents a), rule
-// posteriors accumulated in registers, then the element-wise emission epilogue.
-// Dynamic LDS: w0[2][MP], w1[2][MP], then (if TAB_LDS) S table [Mc][T], match main [Mc][T], match leaf [Mc][T].
-// ------------------------------------------------------------------------------------------------------------
+// Forward.  Dynamic LDS: col[2][64R]; with TAB_LDS also the emissions of main nodes and of their leaves [Mc][T] and the
+// S, F0, F1 tables [Mc][T+2] (all base 2), which are copied out in bulk when the sweep is over - the sweep itself then
+// touches no global memory.
 template <int R, bool TAB_LDS>
-__global__ __launch_bounds__(NT) void inside_bwd_ml1_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
-                                                           float *__restrict__ aux, const float *__restrict__ match_all,
-                                                           const float *__restrict__ links, const int64_t *__restrict__ out_len,
-                                                           const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad,
-                                                           float *__restrict__ lgrad, int L, int T, int Mc) {
-    constexpr int CN = 4 * R;
+__global__ __launch_bounds__(NTR) void inside_fwd_ml1_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
+                                                            const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
+                                                            float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc) {
+    constexpr int NQ = 8 * R;
     constexpr int MP = 64 * R;
+    const int TS = T + 2;
     extern __shared__ float smem[];
-    float *w0 = smem;            // [2][MP]
-    float *w1 = smem + 2 * MP;    // [2][MP]
-    float *sm_S = smem + 4 * MP;  // [Mc][T]   (TAB_LDS)
-    float *sm_main = sm_S + (TAB_LDS ? Mc * T : 0);
+    float *col = smem;               // [2][MP]
+    float *sm_main = smem + 2 * MP;  // [Mc][T]
     float *sm_leaf = sm_main + (TAB_LDS ? Mc * T : 0);
+    float *sm_S = sm_leaf + (TAB_LDS ? Mc * T : 0);  // [Mc][TS]
+    float *sm_F0 = sm_S + (TAB_LDS ? Mc * TS : 0);
+    float *sm_F1 = sm_F0 + (TAB_LDS ? Mc * TS : 0);
 
-    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
+    const int b = blockIdx.x, tid = threadIdx.x, j = tid & 7, g8 = (tid >> 3) & 7;
+    const int p = wave_block(tid >> 6);
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const float *mt = match_all + (size_t)b * L * T;
     const float *lk = links + (size_t)b * L * 2 * L;
-    const float *Sb = S + (size_t)b * Mc * (T + 2);
+    float *Sb = S + (size_t)b * Mc * TS;
+    AuxView av(aux, b, Mc, T);
+
+    if (!lengths_ok(m, n, L, T)) {  // out of contract: poison the log-likelihood, touch nothing else
+        for (int i = tid; i < Mc * TS; i += NTR) Sb[i] = (i == 0) ? __builtin_nanf("") : NEG_INF_F;
+        return;
+    }
+    const int mc = m / 2;  // active main-chain nodes: a_id < mc
+    PCFGNAT_PHASE(0);
+
+    // link slabs -> registers; the loads are unconditional (clamped addresses) so that they are all in flight together
+    float A0[R][NQ], A1[R][NQ];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int a_id = 64 * r + 8 * p + g8;
+        const size_t row = (size_t)(2 * min(a_id, Mc - 1) + 1) * 2;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            const int c = 2 * min(j + 8 * q, Mc - 1) + 1;
+            A0[r][q] = lk[(row + 0) * L + c];
+            A1[r][q] = lk[(row + 1) * L + c];
+        }
+    }
+    const float base_cell = sanitize(mt[(size_t)(m - 1) * T + (n - 1)]);  // pcfg_loss.cu:142-147
+    if (TAB_LDS) {
+        for (int i = tid; i < Mc * T; i += NTR) {
+            const int a_id = i / T, s = i - a_id * T;
+            const float vm = mt[(size_t)(2 * a_id + 1) * T + s], vl = mt[(size_t)(2 * a_id) * T + s];
+            const bool ok = a_id < mc && s < n;
+            sm_main[i] = ok ? to_b2(vm) : NEG_INF_F;
+            sm_leaf[i] = (ok && a_id >= 1) ? to_b2(vl) : NEG_INF_F;
+        }
+        for (int i = tid; i < Mc * TS; i += NTR) {
+            sm_S[i] = (i == (mc - 1) * TS + (n - 1)) ? base_cell * LOG2E_F : NEG_INF_F;
+            sm_F0[i] = NEG_INF_F;
+            sm_F1[i] = NEG_INF_F;
+        }
+    } else {
+        // cells of S the sweep never writes: rows beyond the sentence, columns from n-1 on (except the base cell)
+        for (int i = tid; i < Mc * TS; i += NTR) {
+            const int a_id = i / TS, s = i - a_id * TS;
+            if (a_id >= mc || s >= n - 1) Sb[i] = (a_id == mc - 1 && s == n - 1) ? base_cell : NEG_INF_F;
+        }
+    }
+    for (int i = tid; i < MP; i += NTR) col[((n - 1) & 1) * MP + i] = (i == mc - 1) ? base_cell * LOG2E_F : NEG_INF_F;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int a_id = 64 * r + 8 * p + g8;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            const int c_id = j + 8 * q;
+            const bool ok = a_id < mc && c_id < mc && c_id >= a_id;
+            A0[r][q] = ok ? to_b2(A0[r][q]) : NEG_INF_F;
+            A1[r][q] = (ok && a_id >= 1) ? to_b2(A1[r][q]) : NEG_INF_F;
+        }
+    }
+    __syncthreads();
+    PCFGNAT_PHASE(1);
+    FwdSweepArgs sa{col, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, av.F0, av.F1, n, mc, Mc, T, j, g8};
+    switch (p) {  // wave-uniform: every wave runs the sweep specialised for its node block
+        case 0: fwd_sweep<R, TAB_LDS, 0>(A0, A1, sa); break;
+        case 1: fwd_sweep<R, TAB_LDS, 1>(A0, A1, sa); break;
+        case 2: fwd_sweep<R, TAB_LDS, 2>(A0, A1, sa); break;
+        case 3: fwd_sweep<R, TAB_LDS, 3>(A0, A1, sa); break;
+        case 4: fwd_sweep<R, TAB_LDS, 4>(A0, A1, sa); break;
+        case 5: fwd_sweep<R, TAB_LDS, 5>(A0, A1, sa); break;
+        case 6: fwd_sweep<R, TAB_LDS, 6>(A0, A1, sa); break;
+        default: fwd_sweep<R, TAB_LDS, 7>(A0, A1, sa); break;
+    }
+    PCFGNAT_PHASE(2);
+    if (TAB_LDS) {
+        for (int i = tid; i < Mc * TS; i += NTR) {
+            Sb[i] = sm_S[i] * LN2_F;
+            av.F0[i] = sm_F0[i];
+            av.F1[i] = sm_F1[i];
+        }
+    }
+    PCFGNAT_PHASE(3);
+}
+
+struct BwdSweepArgs {
+    float *w0, *w1, *sm_S, *sm_B, *sm_main, *sm_leaf;
+    const float *mt, *Sb;
+    float *gBETA;
+    float beta00;
+    int n, mc, Mc, T, j, g8;
+};
+
+// The outside sweep of one wave, specialised on its node block P: only the chunks q <= 8r + P can hold parents a <= c.
+template <int R, bool TAB_LDS, int P>
+__device__ __forceinline__ void bwd_sweep(const float (&A0)[R][8 * R], const float (&A1)[R][8 * R], float (&G0)[R][8 * R],
+                                          float (&G1)[R][8 * R], const BwdSweepArgs &x) {
+    constexpr int NQ = 8 * R;
+    constexpr int MP = 64 * R;
+    const int T = x.T, TS = x.T + 2, j = x.j;
+    float bprev[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) bprev[r] = (64 * r + 8 * P + x.g8 == 0) ? x.beta00 : NEG_INF_F;
+    for (int t = 1; t <= x.n - 1; t++) {
+        const float *c0 = x.w0 + (t & 1) * MP, *c1 = x.w1 + (t & 1) * MP;
+        float *n0 = x.w0 + ((t + 1) & 1) * MP, *n1 = x.w1 + ((t + 1) & 1) * MP;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int c_id = 64 * r + 8 * P + x.g8;
+            const int q_end = 8 * r + P + 1;  // chunks beyond hold only parents a > c
+            const bool live = c_id < x.mc;
+            const int ci = live ? c_id : 0;
+            float u0[NQ], u1[NQ];
+#pragma unroll
+            for (int q = 0; q < NQ; q++) {
+                if (q < q_end) {
+                    u0[q] = c0[j + 8 * q];
+                    u1[q] = c1[j + 8 * q];
+                }
+            }
+            float sct, mc_t, ml_p;
+            if (TAB_LDS) {
+                sct = x.sm_S[ci * TS + t];
+                mc_t = x.sm_main[ci * T + t];
+                ml_p = x.sm_leaf[ci * T + t - 1];
+            } else {
+                sct = x.Sb[(size_t)ci * TS + t] * LOG2E_F;
+                mc_t = to_b2(x.mt[(size_t)(2 * ci + 1) * T + t]);
+                const float xl = x.mt[(size_t)(2 * ci) * T + t - 1];
+                ml_p = ci >= 1 ? to_b2(xl) : NEG_INF_F;
+            }
+            if (!live) {
+                sct = NEG_INF_F;
+                mc_t = NEG_INF_F;
+                ml_p = NEG_INF_F;
+            }
+            float v0[NQ], v1[NQ];
+            float mx = NEG_INF_F;
+#pragma unroll
+            for (int q = 0; q < NQ; q++) {
+                if (q < q_end) {
+                    v0[q] = A0[r][q] + u0[q];
+                    v1[q] = A1[r][q] + u1[q];
+                    mx = fmaxf(mx, fmaxf(v0[q], v1[q]));
+                }
+            }
+            mx = row8_max(mx);
+            const float mxs = (mx == NEG_INF_F) ? 0.f : mx;
+            const float scale = (mx == NEG_INF_F || sct == NEG_INF_F) ? 0.f : ex2(mxs + sct);
+            float sum = 0.f;
+#pragma unroll
+            for (int q = 0; q < NQ; q++) {
+                if (q < q_end) {
+                    const float e0 = ex2(v0[q] - mxs), e1 = ex2(v1[q] - mxs);
+                    sum += e0 + e1;
+                    G0[r][q] += e0 * scale;
+                    G1[r][q] += e1 * scale;
+                }
+            }
+            sum = row8_sum(sum);
+            const float beta = (mx == NEG_INF_F || !live) ? NEG_INF_F : mx + lg2(sum);
+            // outside weights this node offers to its children at the next two positions
+            const float nw0 = mc_t + beta;
+            const float nw1 = (ml_p + mc_t) + bprev[r];
+            bprev[r] = beta;
+            if (j == 0) {
+                n0[c_id] = nw0;
+                n1[c_id] = nw1;
+                if (live) {
+                    if (TAB_LDS) x.sm_B[c_id * TS + t] = beta;
+                    else x.gBETA[(size_t)c_id * TS + t] = beta;
+                }
+            }
+        }
+        lds_barrier();
+    }
+}
+
+// Backward: outside sweep t = 1 .. n-1 (one 8-lane group per child node c, lanes strided over parents a <= c), rule
+// posteriors accumulated in registers, then the element-wise emission epilogue.
+// Dynamic LDS: w0[2][MP], w1[2][MP]; with TAB_LDS also S, F0, F1, BETA [Mc][T+2] and the emissions of main nodes and
+// leaves [Mc][T], all base 2: sweep and epilogue then read no global memory.
+template <int R, bool TAB_LDS>
+__global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
+                                                            float *__restrict__ aux, const float *__restrict__ match_all,
+                                                            const float *__restrict__ links, const int64_t *__restrict__ out_len,
+                                                            const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad,
+                                                            float *__restrict__ lgrad, int L, int T, int Mc) {
+    constexpr int NQ = 8 * R;
+    constexpr int MP = 64 * R;
+    const int TS = T + 2;
+    extern __shared__ float smem[];
+    float *w0 = smem;            // [2][MP]
+    float *w1 = smem + 2 * MP;    // [2][MP]
+    float *sm_S = smem + 4 * MP;  // [Mc][TS]   (TAB_LDS)
+    float *sm_F0 = sm_S + (TAB_LDS ? Mc * TS : 0);
+    float *sm_F1 = sm_F0 + (TAB_LDS ? Mc * TS : 0);
+    float *sm_B = sm_F1 + (TAB_LDS ? Mc * TS : 0);
+    float *sm_main = sm_B + (TAB_LDS ? Mc * TS : 0);  // [Mc][T]
+    float *sm_leaf = sm_main + (TAB_LDS ? Mc * T : 0);
+
+    const int b = blockIdx.x, tid = threadIdx.x, j = tid & 7, g8 = (tid >> 3) & 7;
+    const int p = wave_block(tid >> 6);
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *mt = match_all + (size_t)b * L * T;
+    const float *lk = links + (size_t)b * L * 2 * L;
+    const float *Sb = S + (size_t)b * Mc * TS;
     float *mg = mgrad + (size_t)b * L * T;
     float *lg = lgrad + (size_t)b * L * 2 * L;
     AuxView av(aux, b, Mc, T);
@@ -205,159 +412,325 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_kernel(const float *__restr
     const float ll = Sb[0];
     const bool valid = lengths_ok(m, n, L, T) && (ll == ll) && (fabsf(ll) != __builtin_huge_valf());
     if (!valid) {  // invalid sentence: all-zero gradients (nat_pcfg_loss.py:123-133 zeroes its loss as well)
-        for (int i = tid; i < L * T; i += NT) mg[i] = 0.f;
-        for (int i = tid; i < L * 2 * L; i += NT) lg[i] = 0.f;
+        for (int i = tid; i < L * T; i += NTR) mg[i] = 0.f;
+        for (int i = tid; i < L * 2 * L; i += NTR) lg[i] = 0.f;
         return;
     }
     const int mc = m / 2;
     // a null grad_output selects the criterion's own weights: d(-(ll/n).mean())/d ll_b = -1/(n_b * B)
     const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)gridDim.x);
 
-    // transposed link slabs: row = child c (this thread's DPP row), lanes over parents a <= c
-    float A0[R][CN], A1[R][CN], G0[R][CN], G1[R][CN];
+    PCFGNAT_PHASE(8);
+    // links_grad is zero outside the cells the register accumulators own (written at the very end, after the barriers of
+    // the sweep have ordered them behind this fill): clear the whole slab now, while the loads below are in flight
+    {
+        const int total = L * 2 * L;
+        if ((total & 3) == 0 && (reinterpret_cast<uintptr_t>(lg) & 15) == 0) {
+            float4 *lg4 = reinterpret_cast<float4 *>(lg);
+            for (int i = tid; i < total / 4; i += NTR) lg4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        } else {
+            for (int i = tid; i < total; i += NTR) lg[i] = 0.f;
+        }
+    }
+    // transposed link slabs: this thread's group owns child c, its lanes the parents a <= c; unconditional loads
+    float A0[R][NQ], A1[R][NQ], G0[R][NQ], G1[R][NQ];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        const int c_id = gidx + 64 * r, c = 2 * c_id + 1;
+        const int c = 2 * min(64 * r + 8 * p + g8, Mc - 1) + 1;
 #pragma unroll
-        for (int q = 0; q < CN; q++) {
-            const int a_id = j + 16 * q, a = 2 * a_id + 1;
-            const bool ok = a_id < mc && c_id < mc && a_id <= c_id;
-            A0[r][q] = ok ? sanitize(lk[((size_t)a * 2 + 0) * L + c]) : NEG_INF_F;
-            A1[r][q] = (ok && a_id >= 1) ? sanitize(lk[((size_t)a * 2 + 1) * L + c]) : NEG_INF_F;
+        for (int q = 0; q < NQ; q++) {
+            const size_t row = (size_t)(2 * min(j + 8 * q, Mc - 1) + 1) * 2;
+            A0[r][q] = lk[(row + 0) * L + c];
+            A1[r][q] = lk[(row + 1) * L + c];
             G0[r][q] = 0.f;
             G1[r][q] = 0.f;
         }
     }
     if (TAB_LDS) {
-        for (int i = tid; i < Mc * T; i += NT) {
+        for (int i = tid; i < Mc * T; i += NTR) {
             const int a_id = i / T, s = i - a_id * T;
+            const float vm = mt[(size_t)(2 * a_id + 1) * T + s], vl = mt[(size_t)(2 * a_id) * T + s];
             const bool ok = a_id < mc && s < n;
-            sm_S[i] = ok ? Sb[(size_t)a_id * (T + 2) + s] : NEG_INF_F;
-            sm_main[i] = ok ? sanitize(mt[(size_t)(2 * a_id + 1) * T + s]) : NEG_INF_F;
-            sm_leaf[i] = (ok && a_id >= 1) ? sanitize(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
+            sm_main[i] = ok ? to_b2(vm) : NEG_INF_F;
+            sm_leaf[i] = (ok && a_id >= 1) ? to_b2(vl) : NEG_INF_F;
+        }
+        for (int i = tid; i < Mc * TS; i += NTR) {
+            sm_S[i] = Sb[i] * LOG2E_F;
+            sm_F0[i] = av.F0[i];
+            sm_F1[i] = av.F1[i];
+            sm_B[i] = NEG_INF_F;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int c_id = 64 * r + 8 * p + g8;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            const int a_id = j + 8 * q;
+            const bool ok = a_id < mc && c_id < mc && a_id <= c_id;
+            A0[r][q] = ok ? to_b2(A0[r][q]) : NEG_INF_F;
+            A1[r][q] = (ok && a_id >= 1) ? to_b2(A1[r][q]) : NEG_INF_F;
         }
     }
     auto match_main = [&](int a_id, int s) -> float {
         if (TAB_LDS) return sm_main[a_id * T + s];
-        return sanitize(mt[(size_t)(2 * a_id + 1) * T + s]);
+        return to_b2(mt[(size_t)(2 * a_id + 1) * T + s]);
     };
     auto match_leaf = [&](int a_id, int s) -> float {
         if (TAB_LDS) return sm_leaf[a_id * T + s];
-        return a_id >= 1 ? sanitize(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
+        const float x = mt[(size_t)(2 * a_id) * T + s];
+        return a_id >= 1 ? to_b2(x) : NEG_INF_F;
     };
-    auto s_at = [&](int a_id, int s) -> float {
-        if (TAB_LDS) return sm_S[a_id * T + s];
-        return Sb[(size_t)a_id * (T + 2) + s];
-    };
+    auto f0_at = [&](int a_id, int s) -> float { return TAB_LDS ? sm_F0[a_id * TS + s] : av.F0[(size_t)a_id * TS + s]; };
+    auto f1_at = [&](int a_id, int s) -> float { return TAB_LDS ? sm_F1[a_id * TS + s] : av.F1[(size_t)a_id * TS + s]; };
+    auto beta_at = [&](int a_id, int s) -> float { return TAB_LDS ? sm_B[a_id * TS + s] : av.BETA[(size_t)a_id * TS + s]; };
 
-    const float beta00 = -ll;  // outside score of (root, 0) for a unit upstream gradient
-    for (int i = tid; i < MP; i += NT) {
+    const float beta00 = -ll * LOG2E_F;  // outside score of (root, 0) for a unit upstream gradient
+    for (int i = tid; i < MP; i += NTR) {
         w0[1 * MP + i] = NEG_INF_F;
         w1[1 * MP + i] = NEG_INF_F;
     }
-    // beta[.][0]
-    for (int i = tid; i < mc; i += NT) av.BETA[(size_t)i * (T + 2)] = (i == 0) ? beta00 : NEG_INF_F;
+    if (!TAB_LDS)
+        for (int i = tid; i < mc; i += NTR) av.BETA[(size_t)i * TS] = (i == 0) ? beta00 : NEG_INF_F;
     __syncthreads();
-    float bprev[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) bprev[r] = (gidx + 64 * r == 0) ? beta00 : NEG_INF_F;
-    if (tid == 0) w0[1 * MP + 0] = match_main(0, 0) + beta00;
-    __syncthreads();
-
-    for (int t = 1; t <= n - 1; t++) {
-        const float *c0 = w0 + (t & 1) * MP, *c1 = w1 + (t & 1) * MP;
-        float *n0 = w0 + ((t + 1) & 1) * MP, *n1 = w1 + ((t + 1) & 1) * MP;
-        float wa0[CN], wa1[CN];
-#pragma unroll
-        for (int q = 0; q < CN; q++) {
-            wa0[q] = c0[j + 16 * q];
-            wa1[q] = c1[j + 16 * q];
-        }
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            const int c_id = gidx + 64 * r;
-            const bool live = c_id < mc;
-            const int ci = live ? c_id : 0;
-            float v0[CN], v1[CN];
-            float mx = NEG_INF_F;
-#pragma unroll
-            for (int q = 0; q < CN; q++) {
-                v0[q] = A0[r][q] + wa0[q];
-                v1[q] = A1[r][q] + wa1[q];
-                mx = fmaxf(mx, fmaxf(v0[q], v1[q]));
-            }
-            mx = row16_max(mx);
-            const float mxs = (mx == NEG_INF_F) ? 0.f : mx;
-            float e0[CN], e1[CN], sum = 0.f;
-#pragma unroll
-            for (int q = 0; q < CN; q++) {
-                e0[q] = __expf(v0[q] - mxs);
-                e1[q] = __expf(v1[q] - mxs);
-                sum += e0[q] + e1[q];
-            }
-            sum = row16_sum(sum);
-            const float beta = (mx == NEG_INF_F || !live) ? NEG_INF_F : mx + __logf(sum);
-            const float sct = live ? s_at(ci, t) : NEG_INF_F;
-            const float scale = (mx == NEG_INF_F || sct == NEG_INF_F) ? 0.f : __expf(mxs + sct);
-#pragma unroll
-            for (int q = 0; q < CN; q++) {
-                G0[r][q] += e0[q] * scale;
-                G1[r][q] += e1[q] * scale;
-            }
-            // outside weights this node offers to its children at the next two positions
-            const float mc_t = live ? match_main(ci, t) : NEG_INF_F;
-            const float nw0 = mc_t + beta;
-            const float nw1 = (live ? (match_leaf(ci, t - 1) + mc_t) : NEG_INF_F) + bprev[r];
-            bprev[r] = beta;
-            if (j == 0) {
-                n0[c_id] = nw0;
-                n1[c_id] = nw1;
-                if (live) av.BETA[(size_t)c_id * (T + 2) + t] = beta;
-            }
-        }
-        lds_barrier();
+    if (tid == 0) {
+        w0[1 * MP + 0] = match_main(0, 0) + beta00;
+        if (TAB_LDS) sm_B[0] = beta00;
     }
     __syncthreads();
+    PCFGNAT_PHASE(9);
+    BwdSweepArgs sa{w0, w1, sm_S, sm_B, sm_main, sm_leaf, mt, Sb, av.BETA, beta00, n, mc, Mc, T, j, g8};
+    switch (p) {  // wave-uniform
+        case 0: bwd_sweep<R, TAB_LDS, 0>(A0, A1, G0, G1, sa); break;
+        case 1: bwd_sweep<R, TAB_LDS, 1>(A0, A1, G0, G1, sa); break;
+        case 2: bwd_sweep<R, TAB_LDS, 2>(A0, A1, G0, G1, sa); break;
+        case 3: bwd_sweep<R, TAB_LDS, 3>(A0, A1, G0, G1, sa); break;
+        case 4: bwd_sweep<R, TAB_LDS, 4>(A0, A1, G0, G1, sa); break;
+        case 5: bwd_sweep<R, TAB_LDS, 5>(A0, A1, G0, G1, sa); break;
+        case 6: bwd_sweep<R, TAB_LDS, 6>(A0, A1, G0, G1, sa); break;
+        default: bwd_sweep<R, TAB_LDS, 7>(A0, A1, G0, G1, sa); break;
+    }
+    __syncthreads();  // BETA written by the group leaders is read by every thread below
+    PCFGNAT_PHASE(10);
 
     // rule posteriors -> links_grad (pcfg_loss_backward.cu:512-531); everything else in the slab is zero
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        const int c_id = gidx + 64 * r, c = 2 * c_id + 1;
+        const int c_id = 64 * r + 8 * p + g8, c = 2 * c_id + 1;
 #pragma unroll
-        for (int q = 0; q < CN; q++) {
-            const int a_id = j + 16 * q, a = 2 * a_id + 1;
-            if (a_id < Mc && c_id < Mc && a_id <= c_id && c < L) {
+        for (int q = 0; q < NQ; q++) {
+            const int a_id = j + 8 * q, a = 2 * a_id + 1;
+            if (a_id < Mc && c_id < Mc && a_id <= c_id) {
                 lg[((size_t)a * 2 + 0) * L + c] = g * G0[r][q];
                 lg[((size_t)a * 2 + 1) * L + c] = g * G1[r][q];
             }
         }
     }
-    for (int i = tid; i < L * 2 * L; i += NT) {
-        const int c = i % L, a = i / (2 * L);
-        const bool owned = (a & 1) && (c & 1) && (a >> 1) < Mc && (c >> 1) < Mc && (a >> 1) <= (c >> 1);
-        if (!owned) lg[i] = 0.f;
-    }
-
+    PCFGNAT_PHASE(11);
+    PCFGNAT_PHASE(12);
     // emission posteriors -> match_all_grad (pcfg_loss_backward.cu:348-382, 429-433)
-    for (int i = tid; i < L * T; i += NT) {
+    for (int i = tid; i < L * T; i += NTR) {
         const int x = i / T, s = i - x * T;
         float out = 0.f;
         if (x >= 1 && x < m && s < n) {
+            const int a_id = x >> 1;
             if (x & 1) {
-                const int a_id = x >> 1;
-                const size_t row = (size_t)a_id * (T + 2);
-                const float bs = av.BETA[row + s];
+                const float bs = beta_at(a_id, s);
                 const float mas = match_main(a_id, s);
-                if (s + 1 <= n - 1) out += __expf(bs + mas + av.F0[row + s + 1]);  // a emits s with the null left child
-                if (s >= 1 && s + 1 <= n - 1 && a_id >= 1)                        // a emits s after its leaf emitted s-1
-                    out += __expf(av.BETA[row + s - 1] + match_leaf(a_id, s - 1) + mas + av.F1[row + s + 1]);
-                if (a_id == mc - 1 && s == n - 1) out += __expf(bs + mas);       // base cell
-            } else {
-                const int a_id = x >> 1;  // parent a = x+1
-                if (a_id >= 1 && a_id < mc && s + 2 <= n - 1) {
-                    const size_t row = (size_t)a_id * (T + 2);
-                    out += __expf(av.BETA[row + s] + match_leaf(a_id, s) + match_main(a_id, s + 1) + av.F1[row + s + 2]);
-                }
+                if (s + 1 <= n - 1) out += ex2(bs + mas + f0_at(a_id, s + 1));  // a emits s with the null left child
+                if (s >= 1 && s + 1 <= n - 1 && a_id >= 1)                      // a emits s after its leaf emitted s-1
+                    out += ex2(beta_at(a_id, s - 1) + match_leaf(a_id, s - 1) + mas + f1_at(a_id, s + 1));
+                if (a_id == mc - 1 && s == n - 1) out += ex2(bs + mas);        // base cell
+            } else if (a_id >= 1 && a_id < mc && s + 2 <= n - 1) {             // leaf of parent a = x+1
+                out += ex2(beta_at(a_id, s) + match_leaf(a_id, s) + match_main(a_id, s + 1) + f1_at(a_id, s + 2));
+            }
+            if (!(out == out)) out = 0.f;
+        }
+        mg[i] = g * out;
+    }
+    PCFGNAT_PHASE(13);
+}
+
+// Forward and backward in one launch (used by the single-call criterion step when every table fits in LDS): the
+// tables the backward needs (S, F0, F1, emissions) never leave LDS, only S is also written to global memory in the
+// reference's layout.  Dynamic LDS: w0[2][MP] (doubles as the forward's S columns), w1[2][MP], S/F0/F1/BETA [Mc][T+2],
+// emissions of main nodes and leaves [Mc][T].
+template <int R>
+__global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__restrict__ grad_out, const float *__restrict__ match_all,
+                                                              const float *__restrict__ links, const int64_t *__restrict__ out_len,
+                                                              const int64_t *__restrict__ tgt_len, float *__restrict__ S,
+                                                              float *__restrict__ mgrad, float *__restrict__ lgrad, int L, int T,
+                                                              int Mc) {
+    constexpr int NQ = 8 * R;
+    constexpr int MP = 64 * R;
+    const int TS = T + 2;
+    extern __shared__ float smem[];
+    float *w0 = smem;            // [2][MP]
+    float *w1 = smem + 2 * MP;    // [2][MP]
+    float *sm_S = smem + 4 * MP;  // [Mc][TS]
+    float *sm_F0 = sm_S + Mc * TS;
+    float *sm_F1 = sm_F0 + Mc * TS;
+    float *sm_B = sm_F1 + Mc * TS;
+    float *sm_main = sm_B + Mc * TS;  // [Mc][T]
+    float *sm_leaf = sm_main + Mc * T;
+
+    const int b = blockIdx.x, tid = threadIdx.x, j = tid & 7, g8 = (tid >> 3) & 7;
+    const int p = wave_block(tid >> 6);
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *mt = match_all + (size_t)b * L * T;
+    const float *lk = links + (size_t)b * L * 2 * L;
+    float *Sb = S + (size_t)b * Mc * TS;
+    float *mg = mgrad + (size_t)b * L * T;
+    float *lg = lgrad + (size_t)b * L * 2 * L;
+
+    {   // links_grad: everything outside the accumulator-owned cells is zero (see inside_bwd_ml1_kernel)
+        const int total = L * 2 * L;
+        if ((total & 3) == 0 && (reinterpret_cast<uintptr_t>(lg) & 15) == 0) {
+            float4 *lg4 = reinterpret_cast<float4 *>(lg);
+            for (int i = tid; i < total / 4; i += NTR) lg4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        } else {
+            for (int i = tid; i < total; i += NTR) lg[i] = 0.f;
+        }
+    }
+    if (!lengths_ok(m, n, L, T)) {  // out of contract: poisoned log-likelihood, zero gradients
+        for (int i = tid; i < Mc * TS; i += NTR) Sb[i] = (i == 0) ? __builtin_nanf("") : NEG_INF_F;
+        for (int i = tid; i < L * T; i += NTR) mg[i] = 0.f;
+        return;
+    }
+    const int mc = m / 2;
+    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)gridDim.x);
+
+    // ---- forward
+    float A0[R][NQ], A1[R][NQ];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const size_t row = (size_t)(2 * min(64 * r + 8 * p + g8, Mc - 1) + 1) * 2;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            const int c = 2 * min(j + 8 * q, Mc - 1) + 1;
+            A0[r][q] = lk[(row + 0) * L + c];
+            A1[r][q] = lk[(row + 1) * L + c];
+        }
+    }
+    const float base_cell = sanitize(mt[(size_t)(m - 1) * T + (n - 1)]);
+    for (int i = tid; i < Mc * T; i += NTR) {
+        const int a_id = i / T, s = i - a_id * T;
+        const float vm = mt[(size_t)(2 * a_id + 1) * T + s], vl = mt[(size_t)(2 * a_id) * T + s];
+        const bool ok = a_id < mc && s < n;
+        sm_main[i] = ok ? to_b2(vm) : NEG_INF_F;
+        sm_leaf[i] = (ok && a_id >= 1) ? to_b2(vl) : NEG_INF_F;
+    }
+    for (int i = tid; i < Mc * TS; i += NTR) {
+        sm_S[i] = (i == (mc - 1) * TS + (n - 1)) ? base_cell * LOG2E_F : NEG_INF_F;
+        sm_F0[i] = NEG_INF_F;
+        sm_F1[i] = NEG_INF_F;
+        sm_B[i] = NEG_INF_F;
+    }
+    for (int i = tid; i < MP; i += NTR) w0[((n - 1) & 1) * MP + i] = (i == mc - 1) ? base_cell * LOG2E_F : NEG_INF_F;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int a_id = 64 * r + 8 * p + g8;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            const int c_id = j + 8 * q;
+            const bool ok = a_id < mc && c_id < mc && c_id >= a_id;
+            A0[r][q] = ok ? to_b2(A0[r][q]) : NEG_INF_F;
+            A1[r][q] = (ok && a_id >= 1) ? to_b2(A1[r][q]) : NEG_INF_F;
+        }
+    }
+    __syncthreads();
+    {
+        FwdSweepArgs sa{w0, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, nullptr, nullptr, n, mc, Mc, T, j, g8};
+        switch (p) {
+            case 0: fwd_sweep<R, true, 0>(A0, A1, sa); break;
+            case 1: fwd_sweep<R, true, 1>(A0, A1, sa); break;
+            case 2: fwd_sweep<R, true, 2>(A0, A1, sa); break;
+            case 3: fwd_sweep<R, true, 3>(A0, A1, sa); break;
+            case 4: fwd_sweep<R, true, 4>(A0, A1, sa); break;
+            case 5: fwd_sweep<R, true, 5>(A0, A1, sa); break;
+            case 6: fwd_sweep<R, true, 6>(A0, A1, sa); break;
+            default: fwd_sweep<R, true, 7>(A0, A1, sa); break;
+        }
+    }
+    // ---- backward: transposed slabs are requested first, S goes out to global memory while they travel
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int c = 2 * min(64 * r + 8 * p + g8, Mc - 1) + 1;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            const size_t row = (size_t)(2 * min(j + 8 * q, Mc - 1) + 1) * 2;
+            A0[r][q] = lk[(row + 0) * L + c];
+            A1[r][q] = lk[(row + 1) * L + c];
+        }
+    }
+    for (int i = tid; i < Mc * TS; i += NTR) Sb[i] = sm_S[i] * LN2_F;
+    const float ll2 = sm_S[0];  // base 2
+    const bool valid = (ll2 == ll2) && (fabsf(ll2) != __builtin_huge_valf());
+    if (!valid) {  // workgroup-uniform
+        for (int i = tid; i < L * T; i += NTR) mg[i] = 0.f;
+        return;
+    }
+    float G0[R][NQ], G1[R][NQ];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int c_id = 64 * r + 8 * p + g8;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            const int a_id = j + 8 * q;
+            const bool ok = a_id < mc && c_id < mc && a_id <= c_id;
+            A0[r][q] = ok ? to_b2(A0[r][q]) : NEG_INF_F;
+            A1[r][q] = (ok && a_id >= 1) ? to_b2(A1[r][q]) : NEG_INF_F;
+            G0[r][q] = 0.f;
+            G1[r][q] = 0.f;
+        }
+    }
+    const float beta00 = -ll2;
+    for (int i = tid; i < MP; i += NTR) {
+        w0[1 * MP + i] = (i == 0) ? sm_main[0] + beta00 : NEG_INF_F;
+        w1[1 * MP + i] = NEG_INF_F;
+    }
+    if (tid == 0) sm_B[0] = beta00;
+    __syncthreads();
+    {
+        BwdSweepArgs sa{w0, w1, sm_S, sm_B, sm_main, sm_leaf, mt, Sb, nullptr, beta00, n, mc, Mc, T, j, g8};
+        switch (p) {
+            case 0: bwd_sweep<R, true, 0>(A0, A1, G0, G1, sa); break;
+            case 1: bwd_sweep<R, true, 1>(A0, A1, G0, G1, sa); break;
+            case 2: bwd_sweep<R, true, 2>(A0, A1, G0, G1, sa); break;
+            case 3: bwd_sweep<R, true, 3>(A0, A1, G0, G1, sa); break;
+            case 4: bwd_sweep<R, true, 4>(A0, A1, G0, G1, sa); break;
+            case 5: bwd_sweep<R, true, 5>(A0, A1, G0, G1, sa); break;
+            case 6: bwd_sweep<R, true, 6>(A0, A1, G0, G1, sa); break;
+            default: bwd_sweep<R, true, 7>(A0, A1, G0, G1, sa); break;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int c_id = 64 * r + 8 * p + g8, c = 2 * c_id + 1;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            const int a_id = j + 8 * q, a = 2 * a_id + 1;
+            if (a_id < Mc && c_id < Mc && a_id <= c_id) {
+                lg[((size_t)a * 2 + 0) * L + c] = g * G0[r][q];
+                lg[((size_t)a * 2 + 1) * L + c] = g * G1[r][q];
+            }
+        }
+    }
+    for (int i = tid; i < L * T; i += NTR) {
+        const int x = i / T, s = i - x * T;
+        float out = 0.f;
+        if (x >= 1 && x < m && s < n) {
+            const int a_id = x >> 1;
+            if (x & 1) {
+                const float bs = sm_B[a_id * TS + s];
+                const float mas = sm_main[a_id * T + s];
+                if (s + 1 <= n - 1) out += ex2(bs + mas + sm_F0[a_id * TS + s + 1]);
+                if (s >= 1 && s + 1 <= n - 1 && a_id >= 1)
+                    out += ex2(sm_B[a_id * TS + s - 1] + sm_leaf[a_id * T + s - 1] + mas + sm_F1[a_id * TS + s + 1]);
+                if (a_id == mc - 1 && s == n - 1) out += ex2(bs + mas);
+            } else if (a_id >= 1 && a_id < mc && s + 2 <= n - 1) {
+                out += ex2(sm_B[a_id * TS + s] + sm_leaf[a_id * T + s] + sm_main[a_id * T + s + 1] + sm_F1[a_id * TS + s + 2]);
             }
             if (!(out == out)) out = 0.f;
         }
@@ -806,7 +1179,6 @@ __global__ void fill_zero_kernel(float *p, size_t n) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0.f;
 }
 
-constexpr size_t LDS_BUDGET = 128 * 1024;  // of the 160 KB a gfx950 workgroup may use
 
 // loss = -(1/B) * sum_b [ll_b finite] ll_b / n_b and the number of invalid sentences (nat_pcfg_loss.py:123-135), reduced
 // in a fixed order by one workgroup.  out[0] = loss, out[1] = invalid count.
@@ -885,13 +1257,13 @@ template <int R>
 int launch_fwd(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B, int L,
                int T, int Mc, hipStream_t stream) {
     const size_t base = (size_t)2 * 64 * R * sizeof(float);
-    const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
-    if (with_match <= 96 * 1024) {
+    const size_t with_tab = base + ((size_t)2 * Mc * T + (size_t)3 * Mc * (T + 2)) * sizeof(float);
+    if (with_tab <= LDS_BUDGET) {
         auto k = inside_fwd_ml1_kernel<R, true>;
-        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_match));
-        hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_match, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
+        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_tab));
+        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), with_tab, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
     } else {
-        hipLaunchKernelGGL((inside_fwd_ml1_kernel<R, false>), dim3(B), dim3(NT), base, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
+        hipLaunchKernelGGL((inside_fwd_ml1_kernel<R, false>), dim3(B), dim3(NTR), base, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
@@ -901,16 +1273,31 @@ template <int R>
 int launch_bwd(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
                const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, hipStream_t stream) {
     const size_t base = (size_t)4 * 64 * R * sizeof(float);
-    const size_t with_tab = base + (size_t)3 * Mc * T * sizeof(float);
-    if (with_tab <= 96 * 1024) {
+    const size_t with_tab = base + ((size_t)2 * Mc * T + (size_t)4 * Mc * (T + 2)) * sizeof(float);
+    if (with_tab <= LDS_BUDGET) {
         auto k = inside_bwd_ml1_kernel<R, true>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_tab));
-        hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_tab, stream, go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc);
+        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), with_tab, stream, go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc);
     } else {
-        hipLaunchKernelGGL((inside_bwd_ml1_kernel<R, false>), dim3(B), dim3(NT), base, stream, go, S, aux, match_all, links, ol, tl, mg,
+        hipLaunchKernelGGL((inside_bwd_ml1_kernel<R, false>), dim3(B), dim3(NTR), base, stream, go, S, aux, match_all, links, ol, tl, mg,
                            lg, L, T, Mc);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
+// Returns PCFGNAT_EUNSUPPORTED (without a message being an error for the caller) when the fused kernel does not apply.
+template <int R>
+int launch_fused(const float *go, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *mg,
+                 float *lg, int B, int L, int T, int Mc, hipStream_t stream, bool *done) {
+    const size_t need = ((size_t)4 * 64 * R + (size_t)4 * Mc * (T + 2) + (size_t)2 * Mc * T) * sizeof(float);
+    *done = false;
+    if (need > LDS_BUDGET) return PCFGNAT_OK;
+    auto k = inside_fused_ml1_kernel<R>;
+    PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)need));
+    hipLaunchKernelGGL(k, dim3(B), dim3(NTR), need, stream, go, match_all, links, ol, tl, S, mg, lg, L, T, Mc);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    *done = true;
     return PCFGNAT_OK;
 }
 
@@ -972,6 +1359,31 @@ extern "C" int pcfgnat_pcfg_loss_backward(const float *grad_output, const float 
                              (int)L, (int)T, Mc, s);
     return launch_bwd_stream(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
                              (int)L, (int)T, Mc, s);
+}
+
+extern "C" int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *match_all, const float *links,
+                                                 const int64_t *output_length, const int64_t *target_length, float *S, float *aux,
+                                                 float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T,
+                                                 int64_t ml, void *stream) {
+    int rc = check_dims("pcfg_loss_forward_backward", B, L, T, ml);
+    if (rc != PCFGNAT_OK) return rc;
+    if (B == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(match_all && links && output_length && target_length && S && aux && match_all_grad && links_grad,
+                    "pcfg_loss_forward_backward: null pointer");
+    const int Mc = (int)((L - 2) / 2 + 1);
+    hipStream_t s = (hipStream_t)stream;
+    bool done = false;
+    if (Mc <= 64)
+        rc = launch_fused<1>(grad_output, match_all, links, output_length, target_length, S, match_all_grad, links_grad, (int)B, (int)L,
+                             (int)T, Mc, s, &done);
+    else if (Mc <= 128)
+        rc = launch_fused<2>(grad_output, match_all, links, output_length, target_length, S, match_all_grad, links_grad, (int)B, (int)L,
+                             (int)T, Mc, s, &done);
+    if (rc != PCFGNAT_OK || done) return rc;
+    rc = pcfgnat_pcfg_loss(match_all, links, output_length, target_length, S, aux, B, L, T, ml, stream);
+    if (rc != PCFGNAT_OK) return rc;
+    return pcfgnat_pcfg_loss_backward(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, B,
+                                      L, T, ml, stream);
 }
 
 extern "C" int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *out, int64_t B, int64_t L, int64_t T,
