@@ -125,13 +125,18 @@ int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *
  * logsoftmax_gather backward -> loss.  targets is the contiguous [B,T] int64 target matrix (the gather index of every
  * graph node).  On return (stream order) logits holds d loss / d logits, links_grad d loss / d links, loss_out[0] the
  * loss, loss_out[1] the number of invalid sentences; match_all, S, aux, match_all_grad are caller workspaces of the
- * shapes documented at the individual entry points.  events: NULL, or eight hipEvent_t (entries may be NULL) recorded on the
- * stream before/after the gather forward, the inside forward, the inside backward and the gather backward (for timing).
+ * shapes documented at the individual entry points.
+ * slices: 1 = the whole batch at once; k > 1 = the batch is processed as k slices (sentences [i*B/k, (i+1)*B/k)) that
+ * alternate between `stream` and one helper stream the library keeps per device (created on first use, default
+ * priority), so that the latency-bound inside kernels of one slice run beside the bandwidth-bound gather kernels of the
+ * next; the helper stream forks from and joins back into `stream`, so the call stays ordered on `stream`.
+ * events: NULL, or eight hipEvent_t (entries may be NULL) recorded before/after the gather forward, (unused pair), the
+ * inside forward+backward and the gather backward of slice 0 (for timing).
  */
 int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, const float *links,
                            const int64_t *output_length, const int64_t *target_length, float *match_all, float *S,
                            float *aux, float *match_all_grad, float *links_grad, float *loss_out, int64_t B, int64_t L,
-                           int64_t V, int64_t T, int64_t ml, void *stream, void *const *events);
+                           int64_t V, int64_t T, int64_t ml, int64_t slices, void *stream, void *const *events);
 
 /*
  * Replaces pcfg_best_tree (pcfg_best_tree.cu:333-360): greedy top-down trace over the inside tables.

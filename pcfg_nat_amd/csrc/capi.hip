@@ -1,6 +1,8 @@
 // Library-wide pieces of the C-ABI: version and the thread-local error message.
 #include "common.hip.h"
 
+#include <mutex>
+
 namespace pcfgnat {
 char *error_buffer() {
     static thread_local char buf[512] = {0};
@@ -12,35 +14,105 @@ extern "C" int pcfgnat_abi_version(void) { return 1; }
 
 extern "C" const char *pcfgnat_last_error(void) { return pcfgnat::error_buffer(); }
 
+// ---------------------------------------------------------------------------------------------------------------
 // One call for the whole training pass of the criterion (fs_plugins/criterions/nat_pcfg_loss.py:98-145 and the backward
-// autograd derives from it): gather with eos mask -> inside forward -> inside backward seeded with -1/(n_b*B) ->
-// in-place gather backward -> loss.  Five kernels enqueued back to back; nothing is allocated.
+// autograd derives from it): gather with eos mask -> inside forward+backward seeded with -1/(n_b*B) -> in-place gather
+// backward -> loss.  Nothing is allocated.
+//
+// With slices > 1 the batch is cut into slices that alternate between the caller's stream and one helper stream per
+// device: the inside kernels of a slice are latency-bound on a few dozen CUs, the gather kernels of its neighbour are
+// HBM-bound on all of them, so running them side by side hides the former.  The helper stream forks from and joins
+// back into the caller's stream through events, i.e. for the caller everything is ordered on `stream` as usual.
+// ---------------------------------------------------------------------------------------------------------------
+namespace {
+struct DeviceHelper {
+    hipStream_t stream = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr, gathered[2] = {nullptr, nullptr};
+    bool ready = false;
+};
+constexpr int MAX_DEVICES = 64;
+DeviceHelper g_helpers[MAX_DEVICES];
+std::mutex g_helpers_mutex;
+
+int get_helper(DeviceHelper **out) {
+    int dev = 0;
+    PCFGNAT_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return pcfgnat::fail(PCFGNAT_EINVAL, "criterion_step: device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_helpers_mutex);
+    DeviceHelper &h = g_helpers[dev];
+    if (!h.ready) {
+        PCFGNAT_HIP_CHECK(hipStreamCreateWithFlags(&h.stream, hipStreamNonBlocking));  // default priority
+        PCFGNAT_HIP_CHECK(hipEventCreateWithFlags(&h.fork, hipEventDisableTiming));
+        PCFGNAT_HIP_CHECK(hipEventCreateWithFlags(&h.join, hipEventDisableTiming));
+        PCFGNAT_HIP_CHECK(hipEventCreateWithFlags(&h.gathered[0], hipEventDisableTiming));
+        PCFGNAT_HIP_CHECK(hipEventCreateWithFlags(&h.gathered[1], hipEventDisableTiming));
+        h.ready = true;
+    }
+    *out = &h;
+    return PCFGNAT_OK;
+}
+}  // namespace
+
 extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, const float *links,
                                       const int64_t *output_length, const int64_t *target_length, float *match_all, float *S,
                                       float *aux, float *match_all_grad, float *links_grad, float *loss_out, int64_t B, int64_t L,
-                                      int64_t V, int64_t T, int64_t ml, void *stream, void *const *events) {
-    if (dtype == PCFGNAT_F64)
-        return pcfgnat::fail(PCFGNAT_EUNSUPPORTED, "criterion_step: float64 logits gather to float64, the PCFG kernels are float32");
-    hipStream_t s = (hipStream_t)stream;
-#define PCFGNAT_MARK(i)                                                        \
-    do {                                                                       \
-        if (events && events[i]) PCFGNAT_HIP_CHECK(hipEventRecord((hipEvent_t)events[i], s)); \
+                                      int64_t V, int64_t T, int64_t ml, int64_t slices, void *stream, void *const *events) {
+    if (dtype != PCFGNAT_F16 && dtype != PCFGNAT_F32)
+        return pcfgnat::fail(PCFGNAT_EUNSUPPORTED, "criterion_step: logits must be float16 or float32 (the PCFG kernels are float32)");
+    PCFGNAT_REQUIRE(B >= 1 && L >= 4 && T >= 2 && V >= 1 && ml >= 0, "criterion_step: bad dimensions");
+    PCFGNAT_REQUIRE(logits && targets && links && output_length && target_length && match_all && S && aux && match_all_grad &&
+                        links_grad && loss_out,
+                    "criterion_step: null pointer");
+    if (slices < 1) slices = 1;
+    if (slices > B) slices = B;
+    hipStream_t main_stream = (hipStream_t)stream;
+    DeviceHelper *h = nullptr;
+    if (slices > 1) {
+        int rc = get_helper(&h);
+        if (rc != PCFGNAT_OK) return rc;
+        PCFGNAT_HIP_CHECK(hipEventRecord(h->fork, main_stream));
+        PCFGNAT_HIP_CHECK(hipStreamWaitEvent(h->stream, h->fork, 0));
+    }
+    const size_t esz = (dtype == PCFGNAT_F16) ? 2 : 4;
+    const int64_t Mc = (L - 2) / (ml + 1) + 1;
+    const size_t aux_per_sentence = pcfgnat_pcfg_aux_floats(1, L, T, ml);
+    for (int64_t i = 0; i < slices; i++) {
+        const int64_t b0 = i * B / slices, b1 = (i + 1) * B / slices, nb = b1 - b0;
+        if (nb == 0) continue;
+        hipStream_t s = (i & 1) ? h->stream : main_stream;
+        char *lg_i = (char *)logits + (size_t)b0 * L * V * esz;
+        const int64_t *tg_i = targets + (size_t)b0 * T, *ol_i = output_length + b0, *tl_i = target_length + b0;
+        const float *lk_i = links + (size_t)b0 * L * (ml + 1) * L;
+        float *ma_i = match_all + (size_t)b0 * L * T, *S_i = S + (size_t)b0 * Mc * (T + 2), *aux_i = aux + (size_t)b0 * aux_per_sentence;
+        float *mg_i = match_all_grad + (size_t)b0 * L * T, *lkg_i = links_grad + (size_t)b0 * L * (ml + 1) * L;
+        const bool mark = events && i == 0;  // timing events bracket the kernels of slice 0
+#define PCFGNAT_MARK(k)                                                                   \
+    do {                                                                                  \
+        if (mark && events[k]) PCFGNAT_HIP_CHECK(hipEventRecord((hipEvent_t)events[k], s)); \
     } while (0)
-    PCFGNAT_MARK(0);
-    int rc = pcfgnat_logsoftmax_gather_eos(logits, dtype, targets, T, 0, 1, match_all, 1, output_length, target_length, B, L, V, T, stream);
-    if (rc != PCFGNAT_OK) return rc;
-    PCFGNAT_MARK(1);
-    PCFGNAT_MARK(2);
-    PCFGNAT_MARK(3);  // forward and backward run as one launch where the tables fit in LDS: bracketed together by 4..5
-    PCFGNAT_MARK(4);
-    rc = pcfgnat_pcfg_loss_forward_backward(nullptr, match_all, links, output_length, target_length, S, aux, match_all_grad,
-                                            links_grad, B, L, T, ml, stream);
-    if (rc != PCFGNAT_OK) return rc;
-    PCFGNAT_MARK(5);
-    PCFGNAT_MARK(6);
-    rc = pcfgnat_logsoftmax_gather_backward(logits, dtype, targets, T, 0, 1, match_all_grad, B, L, V, T, stream);
-    if (rc != PCFGNAT_OK) return rc;
-    PCFGNAT_MARK(7);
+        // stagger: the gather of slice i starts when the gather of slice i-1 is done, so that it runs beside the inside
+        // kernels of slice i-1 rather than beside its gather
+        if (i > 0) PCFGNAT_HIP_CHECK(hipStreamWaitEvent(s, h->gathered[(i - 1) & 1], 0));
+        PCFGNAT_MARK(0);
+        int rc = pcfgnat_logsoftmax_gather_eos(lg_i, dtype, tg_i, T, 0, 1, ma_i, 1, ol_i, tl_i, nb, L, V, T, s);
+        if (rc != PCFGNAT_OK) return rc;
+        PCFGNAT_MARK(1);
+        if (slices > 1) PCFGNAT_HIP_CHECK(hipEventRecord(h->gathered[i & 1], s));
+        PCFGNAT_MARK(2);
+        PCFGNAT_MARK(3);  // forward and backward run as one launch where the tables fit in LDS: bracketed together by 4..5
+        PCFGNAT_MARK(4);
+        rc = pcfgnat::inside_forward_backward_impl(nullptr, ma_i, lk_i, ol_i, tl_i, S_i, aux_i, mg_i, lkg_i, nb, L, T, ml, B, s);
+        if (rc != PCFGNAT_OK) return rc;
+        PCFGNAT_MARK(5);
+        PCFGNAT_MARK(6);
+        rc = pcfgnat_logsoftmax_gather_backward(lg_i, dtype, tg_i, T, 0, 1, mg_i, nb, L, V, T, s);
+        if (rc != PCFGNAT_OK) return rc;
+        PCFGNAT_MARK(7);
 #undef PCFGNAT_MARK
+    }
+    if (slices > 1) {
+        PCFGNAT_HIP_CHECK(hipEventRecord(h->join, h->stream));
+        PCFGNAT_HIP_CHECK(hipStreamWaitEvent(main_stream, h->join, 0));
+    }
     return pcfgnat_criterion_loss(S, target_length, loss_out, B, L, T, ml, stream);
 }

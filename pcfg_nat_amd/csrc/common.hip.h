@@ -33,6 +33,16 @@ inline int fail(int code, const char *fmt, ...) {
         if (!(cond)) return ::pcfgnat::fail(PCFGNAT_EINVAL, __VA_ARGS__); \
     } while (0)
 
+// ---- internal entry points shared between translation units ---------------------------------------------------
+// Like the public functions of the same name, with the batch size that normalises the criterion's weights
+// (-1/(n_b * norm_B) when grad_output is null) passed separately, so that a batch can be processed in slices.
+int inside_backward_impl(const float *grad_output, const float *S, float *aux, const float *match_all, const float *links,
+                         const int64_t *output_length, const int64_t *target_length, float *match_all_grad, float *links_grad, int64_t B,
+                         int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream);
+int inside_forward_backward_impl(const float *grad_output, const float *match_all, const float *links, const int64_t *output_length,
+                                 const int64_t *target_length, float *S, float *aux, float *match_all_grad, float *links_grad,
+                                 int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream);
+
 // ---- DPP helpers: reductions inside a row of 16 lanes and across a wave64 -------------------------------------
 // dpp_ctrl encodings (GFX9): quad_perm = perm bits, row_half_mirror = 0x141, row_mirror = 0x140.
 template <int CTRL>

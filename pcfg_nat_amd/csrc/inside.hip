@@ -385,7 +385,7 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
                                                             float *__restrict__ aux, const float *__restrict__ match_all,
                                                             const float *__restrict__ links, const int64_t *__restrict__ out_len,
                                                             const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad,
-                                                            float *__restrict__ lgrad, int L, int T, int Mc) {
+                                                            float *__restrict__ lgrad, int L, int T, int Mc, int norm_B) {
     constexpr int NQ = 8 * R;
     constexpr int MP = 64 * R;
     const int TS = T + 2;
@@ -417,8 +417,8 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
         return;
     }
     const int mc = m / 2;
-    // a null grad_output selects the criterion's own weights: d(-(ll/n).mean())/d ll_b = -1/(n_b * B)
-    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)gridDim.x);
+    // a null grad_output selects the criterion's own weights: d(-(ll/n).mean())/d ll_b = -1/(n_b * norm_B)
+    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)norm_B);
 
     PCFGNAT_PHASE(8);
     // links_grad is zero outside the cells the register accumulators own (written at the very end, after the barriers of
@@ -560,7 +560,7 @@ __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__re
                                                               const float *__restrict__ links, const int64_t *__restrict__ out_len,
                                                               const int64_t *__restrict__ tgt_len, float *__restrict__ S,
                                                               float *__restrict__ mgrad, float *__restrict__ lgrad, int L, int T,
-                                                              int Mc) {
+                                                              int Mc, int norm_B) {
     constexpr int NQ = 8 * R;
     constexpr int MP = 64 * R;
     const int TS = T + 2;
@@ -598,7 +598,7 @@ __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__re
         return;
     }
     const int mc = m / 2;
-    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)gridDim.x);
+    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)norm_B);
 
     // ---- forward
     float A0[R][NQ], A1[R][NQ];
@@ -1227,7 +1227,7 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
 }
 
 int launch_bwd_stream(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
-                      const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, hipStream_t stream) {
+                      const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream) {
     const int MP = ((Mc + 63) / 64) * 64;
     const int tiles = (Mc + 31) / 32;
     hipLaunchKernelGGL(transpose_links_ml1_kernel, dim3(tiles, tiles, B), dim3(256), 0, stream, links, ol, aux, L, T, Mc);
@@ -1245,10 +1245,10 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
     const size_t nlg = (size_t)B * L * 2 * L;
     hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, stream, lg, nlg);
     PCFGNAT_HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL(links_grad_ml1_stream_kernel, dim3(tiles, tiles, B), dim3(1024), 0, stream, go, S, aux, links, ol, tl, lg, L, T, Mc, B);
+    hipLaunchKernelGGL(links_grad_ml1_stream_kernel, dim3(tiles, tiles, B), dim3(1024), 0, stream, go, S, aux, links, ol, tl, lg, L, T, Mc, norm_B);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL(match_grad_ml1_stream_kernel, dim3((L * T + 255) / 256, B), dim3(256), 0, stream, go, S, aux, match_all, ol, tl, mg, L,
-                       T, Mc, B);
+                       T, Mc, norm_B);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -1271,16 +1271,16 @@ int launch_fwd(const float *match_all, const float *links, const int64_t *ol, co
 
 template <int R>
 int launch_bwd(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
-               const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, hipStream_t stream) {
+               const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream) {
     const size_t base = (size_t)4 * 64 * R * sizeof(float);
     const size_t with_tab = base + ((size_t)2 * Mc * T + (size_t)4 * Mc * (T + 2)) * sizeof(float);
     if (with_tab <= LDS_BUDGET) {
         auto k = inside_bwd_ml1_kernel<R, true>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_tab));
-        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), with_tab, stream, go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc);
+        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), with_tab, stream, go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc, norm_B);
     } else {
         hipLaunchKernelGGL((inside_bwd_ml1_kernel<R, false>), dim3(B), dim3(NTR), base, stream, go, S, aux, match_all, links, ol, tl, mg,
-                           lg, L, T, Mc);
+                           lg, L, T, Mc, norm_B);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
@@ -1289,13 +1289,13 @@ int launch_bwd(const float *go, const float *S, float *aux, const float *match_a
 // Returns PCFGNAT_EUNSUPPORTED (without a message being an error for the caller) when the fused kernel does not apply.
 template <int R>
 int launch_fused(const float *go, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *mg,
-                 float *lg, int B, int L, int T, int Mc, hipStream_t stream, bool *done) {
+                 float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream, bool *done) {
     const size_t need = ((size_t)4 * 64 * R + (size_t)4 * Mc * (T + 2) + (size_t)2 * Mc * T) * sizeof(float);
     *done = false;
     if (need > LDS_BUDGET) return PCFGNAT_OK;
     auto k = inside_fused_ml1_kernel<R>;
     PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)need));
-    hipLaunchKernelGGL(k, dim3(B), dim3(NTR), need, stream, go, match_all, links, ol, tl, S, mg, lg, L, T, Mc);
+    hipLaunchKernelGGL(k, dim3(B), dim3(NTR), need, stream, go, match_all, links, ol, tl, S, mg, lg, L, T, Mc, norm_B);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     *done = true;
     return PCFGNAT_OK;
@@ -1340,10 +1340,9 @@ extern "C" int pcfgnat_pcfg_loss(const float *match_all, const float *links, con
     return launch_fwd_stream(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s);
 }
 
-extern "C" int pcfgnat_pcfg_loss_backward(const float *grad_output, const float *S, float *aux, const float *match_all,
-                                          const float *links, const int64_t *output_length, const int64_t *target_length,
-                                          float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T, int64_t ml,
-                                          void *stream) {
+int pcfgnat::inside_backward_impl(const float *grad_output, const float *S, float *aux, const float *match_all, const float *links,
+                                  const int64_t *output_length, const int64_t *target_length, float *match_all_grad, float *links_grad,
+                                  int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream) {
     int rc = check_dims("pcfg_loss_backward", B, L, T, ml);
     if (rc != PCFGNAT_OK) return rc;
     if (B == 0) return PCFGNAT_OK;
@@ -1353,18 +1352,26 @@ extern "C" int pcfgnat_pcfg_loss_backward(const float *grad_output, const float 
     hipStream_t s = (hipStream_t)stream;
     if (Mc <= 64)
         return launch_bwd<1>(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
-                             (int)L, (int)T, Mc, s);
+                             (int)L, (int)T, Mc, (int)norm_B, s);
     if (Mc <= 128)
         return launch_bwd<2>(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
-                             (int)L, (int)T, Mc, s);
+                             (int)L, (int)T, Mc, (int)norm_B, s);
     return launch_bwd_stream(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
-                             (int)L, (int)T, Mc, s);
+                             (int)L, (int)T, Mc, (int)norm_B, s);
 }
 
-extern "C" int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *match_all, const float *links,
-                                                 const int64_t *output_length, const int64_t *target_length, float *S, float *aux,
-                                                 float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T,
-                                                 int64_t ml, void *stream) {
+extern "C" int pcfgnat_pcfg_loss_backward(const float *grad_output, const float *S, float *aux, const float *match_all,
+                                          const float *links, const int64_t *output_length, const int64_t *target_length,
+                                          float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T, int64_t ml,
+                                          void *stream) {
+    return inside_backward_impl(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, B, L, T,
+                                ml, B, stream);
+}
+
+int pcfgnat::inside_forward_backward_impl(const float *grad_output, const float *match_all, const float *links,
+                                          const int64_t *output_length, const int64_t *target_length, float *S, float *aux,
+                                          float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T, int64_t ml,
+                                          int64_t norm_B, void *stream) {
     int rc = check_dims("pcfg_loss_forward_backward", B, L, T, ml);
     if (rc != PCFGNAT_OK) return rc;
     if (B == 0) return PCFGNAT_OK;
@@ -1375,15 +1382,23 @@ extern "C" int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, cons
     bool done = false;
     if (Mc <= 64)
         rc = launch_fused<1>(grad_output, match_all, links, output_length, target_length, S, match_all_grad, links_grad, (int)B, (int)L,
-                             (int)T, Mc, s, &done);
+                             (int)T, Mc, (int)norm_B, s, &done);
     else if (Mc <= 128)
         rc = launch_fused<2>(grad_output, match_all, links, output_length, target_length, S, match_all_grad, links_grad, (int)B, (int)L,
-                             (int)T, Mc, s, &done);
+                             (int)T, Mc, (int)norm_B, s, &done);
     if (rc != PCFGNAT_OK || done) return rc;
     rc = pcfgnat_pcfg_loss(match_all, links, output_length, target_length, S, aux, B, L, T, ml, stream);
     if (rc != PCFGNAT_OK) return rc;
-    return pcfgnat_pcfg_loss_backward(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, B,
-                                      L, T, ml, stream);
+    return inside_backward_impl(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, B, L, T,
+                                ml, norm_B, stream);
+}
+
+extern "C" int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *match_all, const float *links,
+                                                 const int64_t *output_length, const int64_t *target_length, float *S, float *aux,
+                                                 float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T,
+                                                 int64_t ml, void *stream) {
+    return inside_forward_backward_impl(grad_output, match_all, links, output_length, target_length, S, aux, match_all_grad, links_grad,
+                                        B, L, T, ml, B, stream);
 }
 
 extern "C" int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *out, int64_t B, int64_t L, int64_t T,

@@ -353,11 +353,13 @@ def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unre
     return out[:, :maxlen].to(torch.float32)
 
 
-def pcfg_criterion_step(logits, targets, links, output_length, target_length, events=None):
+def pcfg_criterion_step(logits, targets, links, output_length, target_length, events=None, slices=None):
     """The criterion's whole training pass in one native call (``pcfgnat_criterion_step``): ``logits`` [B,L,V] (fp16 or
     fp32, contiguous) is consumed in place and holds d loss / d logits afterwards.  ``events``: optional list of eight
     ``torch.cuda.Event(enable_timing=True)`` (each recorded at least once before; entries may be None) that the library records before/after
-    the gather forward, inside forward, inside backward and gather backward.  Returns
+    the gather forward, inside forward, inside backward and gather backward of the first slice.  ``slices``: how many
+    batch slices alternate between the current stream and the library's helper stream (default 1: measured on MI355X the
+    bandwidth-bound gather kernels leave no room for a second kernel on the CUs, so slicing does not pay).  Returns
     (loss_and_invalid [2] float32, links_grad, ll [B], match_all_eos_masked)."""
     lib = get_pcfg_kernel()
     _need_cuda("pcfg_criterion_step", logits, targets, links, output_length, target_length)
@@ -378,6 +380,8 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
     tl = _lengths("pcfg_criterion_step", target_length, B)
     Mc = (L - 2) // (ml + 1) + 1
     dev = logits.device
+    if slices is None:
+        slices = 1
     ev_arr = None
     if events is not None:
         import ctypes
@@ -393,5 +397,5 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
         out = torch.empty((2,), dtype=torch.float32, device=dev)
         _lib.check(lib.pcfgnat_criterion_step(logits.data_ptr(), code, targets.data_ptr(), links.data_ptr(), ol.data_ptr(),
                                               tl.data_ptr(), match.data_ptr(), S.data_ptr(), aux.data_ptr(), mg.data_ptr(),
-                                              lg.data_ptr(), out.data_ptr(), B, L, V, T, ml, _stream(logits), ev_arr), lib)
+                                              lg.data_ptr(), out.data_ptr(), B, L, V, T, ml, slices, _stream(logits), ev_arr), lib)
     return out, lg, S[:, 0, 0], match

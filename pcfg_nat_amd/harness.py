@@ -155,11 +155,12 @@ def train_step_fused(logits, targets, links, output_length, target_length, ops=_
     return loss, glinks, ll
 
 
-def train_step_single_call(logits, targets, links, output_length, target_length, ops=_default_ops, mark=None):
+def train_step_single_call(logits, targets, links, output_length, target_length, ops=_default_ops, mark=None, slices=None):
     """``train_step_fused`` issued as one native call (``pcfgnat_criterion_step``): the five kernels are enqueued back to
     back by the library and the scalar loss is reduced on the device.  Returns (loss, links_grad, ll)."""
     events = None
     if mark is not None:
         events = mark("events", 8)  # the caller hands out eight timing events for this step
-    out, glinks, ll, _ = ops.pcfg_criterion_step(logits, targets, links, output_length, target_length, events=events)
+    out, glinks, ll, _ = ops.pcfg_criterion_step(logits, targets, links, output_length, target_length, events=events,
+                                                 slices=slices)
     return out[0], glinks, ll

@@ -350,7 +350,10 @@ def test_fused_step_equals_autograd_step():
     res = harness.compute_pcfg_loss(leaf.half(), out_mask, tgt, tgt_mask, links)
     assert int(res["invalid_nsentences"]) == 1
     res["loss"].backward()
-    for step in (harness.train_step_direct, harness.train_step_fused, harness.train_step_single_call):
+    def sliced(k):
+        return lambda *a: harness.train_step_single_call(*a, slices=k)
+
+    for step in (harness.train_step_direct, harness.train_step_fused, sliced(1), sliced(2), sliced(3)):
         buf = batch["logits"].to(DEV).clone()
         loss, glinks, ll = step(buf, tgt, batch["links"].to(DEV), ol, tl)
         assert torch.allclose(loss, res["loss"].detach(), rtol=1e-6)
