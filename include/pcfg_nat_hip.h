@@ -142,8 +142,9 @@ int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, cons
  * Replaces pcfg_best_tree (pcfg_best_tree.cu:333-360): greedy top-down trace over the inside tables.
  *   tree [B,L] int64 out: target position aligned to each node, -1 for nodes off the tree.
  * Exact ties are resolved in the reference's scan order (lanes 0 > 2 > 1 > 3 of a 4-wide strided scan).
+ * aux: the table left by pcfgnat_pcfg_loss on the same inputs (read, and for max_left != 1 partly reused as mark space).
  */
-int pcfgnat_pcfg_best_tree(const float *S, const float *aux, const float *match_all, const float *links,
+int pcfgnat_pcfg_best_tree(const float *S, float *aux, const float *match_all, const float *links,
                            const int64_t *output_length, const int64_t *target_length, int64_t *tree, int64_t B,
                            int64_t L, int64_t T, int64_t ml, void *stream);
 

@@ -43,6 +43,17 @@ int inside_forward_backward_impl(const float *grad_output, const float *match_al
                                  const int64_t *target_length, float *S, float *aux, float *match_all_grad, float *links_grad,
                                  int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream);
 
+// General max_left (generic_ml.hip)
+size_t generic_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml);
+int generic_forward(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int64_t B,
+                    int64_t L, int64_t T, int64_t ml, void *stream);
+int generic_backward(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
+                     const int64_t *tl, float *mg, float *lg, int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream);
+int generic_best_tree(const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl,
+                      int64_t *tree, int64_t B, int64_t L, int64_t T, int64_t ml, void *stream);
+int generic_viterbi(const float *ob, const float *links, const int64_t *ol, float *S, int64_t *R, int64_t *Lt, int64_t *M, int64_t B,
+                    int64_t L, int64_t ml, void *stream);
+
 // ---- DPP helpers: reductions inside a row of 16 lanes and across a wave64 -------------------------------------
 // dpp_ctrl encodings (GFX9): quad_perm = perm bits, row_half_mirror = 0x141, row_mirror = 0x140.
 template <int CTRL>

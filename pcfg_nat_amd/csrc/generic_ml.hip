@@ -1,0 +1,441 @@
+// General max_left ("ml" = links.size(2) - 1 = 2^left_tree_layer - 1): the inside loss, its exact backward, the best-tree
+// trace and the viterbi tables for any ml other than 1 (ml = 1, the setting of every shipped script, has its own tuned
+// kernels in inside.hip / viterbi.hip).
+//
+// Replaces the general-ml paths of the reference's pcfg_loss.cu (:84-349), pcfg_loss_backward.cu (:28-603),
+// pcfg_best_tree.cu (:64-301) and pcfg_viterbi.cu (:22-241).
+//
+// Correct-but-plain design: one workgroup per sentence, the loops of the reference kept as they are with the outermost
+// row loop spread over the threads and a workgroup barrier wherever the reference has a dependency between steps.
+// Tables live in global memory (L2-resident).  Scatter-adds of the backward use float atomics.
+#include "common.hip.h"
+
+namespace pcfgnat {
+namespace {
+
+constexpr int NTG = 256;
+
+struct Dims {
+    int L, T, ml, Mc, Lc, TS, G;  // TS = T+2, G = ml+2
+    __host__ __device__ Dims(int L_, int T_, int ml_) : L(L_), T(T_), ml(ml_) {
+        Mc = (L - 2) / (ml + 1) + 1;
+        Lc = L - Mc;
+        TS = T + 2;
+        G = ml + 2;
+    }
+    __device__ int mc_i2e(int x) const { return x * (ml + 1) + 1; }
+    __device__ int mc_e2i(int x) const { return (x - 1) / (ml + 1); }
+    __device__ int lt_i2e(int x) const { return x == 0 ? 0 : x + (x - 1) / (ml > 0 ? ml : 1) + 1; }
+    __device__ int lt_e2i(int x) const { return x == 0 ? 0 : x - (x - 1) / (ml + 1) - 1; }
+    __device__ int lo(int a) const { return ((a - 1) / (ml + 1)) * (ml + 1) + 1; }
+    __device__ int hi(int a) const { return ((a - 1) / (ml + 1) + 1) * (ml + 1) + 1; }
+    __device__ size_t s_at(int a_id, int s) const { return (size_t)a_id * TS + s; }
+    __device__ size_t c_at(int b_id, int i, int g) const { return ((size_t)b_id * TS + i) * G + g; }
+    __device__ size_t lk(int a, int k, int c) const { return ((size_t)a * (ml + 1) + k) * L + c; }
+    __host__ __device__ size_t s_size() const { return (size_t)Mc * TS; }
+    __host__ __device__ size_t c_size() const { return (size_t)Lc * TS * G; }
+    // aux per sentence: C | Cg | Ct (c_size each) | Sg | St (s_size each); Ct/St are the best-tree marks
+    __host__ __device__ size_t aux_floats() const { return 3 * c_size() + 2 * s_size(); }
+};
+
+__device__ __forceinline__ bool bad(float v) { return v != v; }
+// Cells that other threads update with (L2) atomics must not be read through a possibly stale L1 line.
+__device__ __forceinline__ float coherent_load(const float *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ bool len_ok(const Dims &d, int m, int n) {
+    return m >= d.ml + 3 && m <= d.L && ((m - 2) % (d.ml + 1)) == 0 && n >= 2 && n <= d.T;
+}
+
+// ---- inside forward (pcfg_loss.cu:262-349 then :84-224) -----------------------------------------------------
+__global__ __launch_bounds__(NTG) void generic_fwd_kernel(const float *__restrict__ match_all, const float *__restrict__ links_all,
+                                                         const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
+                                                         float *__restrict__ S_all, float *__restrict__ aux_all, int L, int T, int ml) {
+    const Dims d(L, T, ml);
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *match = match_all + (size_t)b * L * T;
+    const float *links = links_all + (size_t)b * L * (ml + 1) * L;
+    float *S = S_all + (size_t)b * d.s_size();
+    float *C = aux_all + (size_t)b * d.aux_floats();
+    for (size_t i = tid; i < d.s_size(); i += NTG) S[i] = NEG_INF_F;
+    if (!len_ok(d, m, n)) {
+        __syncthreads();
+        if (tid == 0) S[0] = __builtin_nanf("");
+        return;
+    }
+    for (size_t i = tid; i < d.c_size(); i += NTG) C[i] = NEG_INF_F;
+    __syncthreads();
+    // :288-300
+    for (int i = tid; i <= n; i += NTG) C[d.c_at(0, i, 0)] = 0.f;
+    for (int w = tid; w < d.Lc * n; w += NTG) {
+        const int a_id = w / n, i = w - a_id * n;
+        const int a = d.lt_i2e(a_id);
+        if (a > 0 && a < m && ((a - d.lo(a)) % 2 == 1)) C[d.c_at(a_id, i, 1)] = match[(size_t)a * T + i];
+    }
+    __syncthreads();
+    // :301-348
+    for (int gap = 2; gap < ml + 2; gap++) {
+        const int ni = n - gap - 1;
+        for (int w = tid; ni > 0 && w < d.Lc * ni; w += NTG) {
+            const int a_id = w / ni, i = w - a_id * ni;
+            const int a = d.lt_i2e(a_id);
+            if (!(a > 0 && a < m)) continue;
+            const int hi = d.hi(a), b_start = a - ml < 1 ? 1 : a - ml;
+            float maxval = NEG_INF_F;
+            for (int pass = 0; pass < 2; pass++) {
+                float sum = 0.f;
+                for (int j = 0; j < gap; j++)
+                    for (int bb = b_start; bb < a + 1; bb++) {
+                        const int b_id = d.lt_e2i(bb == a ? 0 : bb);
+                        for (int c = a + 1; c < hi && c < m; c++) {
+                            float t = links[d.lk(a, a - bb, c)] + C[d.c_at(b_id, i, j)] + C[d.c_at(d.lt_e2i(c), i + j + 1, gap - j - 1)] +
+                                      match[(size_t)a * T + i + j];
+                            if (bad(t)) t = NEG_INF_F;
+                            if (pass == 0) maxval = fmaxf(maxval, t);
+                            else sum += expf(t - maxval);
+                        }
+                    }
+                if (pass == 0 && maxval == NEG_INF_F) break;
+                if (pass == 1) C[d.c_at(a_id, i, gap)] = logf(sum) + maxval;
+            }
+        }
+        __syncthreads();
+    }
+    // :142-147
+    if (tid == 0) S[d.s_at(d.mc_e2i(m - 1), n - 1)] = match[(size_t)(m - 1) * T + (n - 1)];
+    __syncthreads();
+    // :148-214
+    for (int start = n - 2; start >= 0; start--) {
+        for (int a_id = tid; a_id < d.Mc; a_id += NTG) {
+            const int a = d.mc_i2e(a_id);
+            if (!(a > 0 && a < m)) continue;
+            const int b_start = a - ml < 1 ? 1 : a - ml;
+            float maxval = NEG_INF_F;
+            for (int pass = 0; pass < 2; pass++) {
+                float sum = 0.f;
+                for (int c_id = a_id; d.mc_i2e(c_id) < m; c_id++) {
+                    const int c = d.mc_i2e(c_id);
+                    for (int j = 0; j < n - start && j < ml + 1; j++)
+                        for (int bb = b_start; bb < a + 1; bb++) {
+                            const int b_id = d.lt_e2i(bb == a ? 0 : bb);
+                            float t = links[d.lk(a, a - bb, c)] + S[d.s_at(c_id, start + j + 1)] + C[d.c_at(b_id, start, j)] +
+                                      match[(size_t)a * T + start + j];
+                            if (bad(t)) t = NEG_INF_F;
+                            if (pass == 0) maxval = fmaxf(maxval, t);
+                            else sum += expf(t - maxval);
+                        }
+                }
+                if (pass == 0 && maxval == NEG_INF_F) break;
+                if (pass == 1) S[d.s_at(a_id, start)] = logf(sum) + maxval;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// ---- backward: exact gradient of the recurrences above (organised like pcfg_loss_backward.cu:28-603) ------------
+__global__ __launch_bounds__(NTG) void generic_bwd_kernel(const float *__restrict__ grad_out, const float *__restrict__ S_all,
+                                                         float *__restrict__ aux_all, const float *__restrict__ match_all,
+                                                         const float *__restrict__ links_all, const int64_t *__restrict__ out_len,
+                                                         const int64_t *__restrict__ tgt_len, float *__restrict__ mg_all,
+                                                         float *__restrict__ lg_all, int L, int T, int ml, int norm_B) {
+    const Dims d(L, T, ml);
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *match = match_all + (size_t)b * L * T;
+    const float *links = links_all + (size_t)b * L * (ml + 1) * L;
+    const float *S = S_all + (size_t)b * d.s_size();
+    float *aux = aux_all + (size_t)b * d.aux_floats();
+    const float *C = aux;
+    float *Cg = aux + d.c_size();
+    float *Sg = aux + 3 * d.c_size();
+    float *mg = mg_all + (size_t)b * L * T;
+    float *lg = lg_all + (size_t)b * L * (ml + 1) * L;
+    for (size_t i = tid; i < (size_t)L * T; i += NTG) mg[i] = 0.f;
+    for (size_t i = tid; i < (size_t)L * (ml + 1) * L; i += NTG) lg[i] = 0.f;
+    const float ll = S[0];
+    if (!len_ok(d, m, n) || ll != ll || fabsf(ll) == __builtin_huge_valf()) return;  // invalid sentence: zero gradients
+    for (size_t i = tid; i < d.s_size(); i += NTG) Sg[i] = 0.f;
+    for (size_t i = tid; i < d.c_size(); i += NTG) Cg[i] = 0.f;
+    __syncthreads();
+    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)norm_B);
+    if (tid == 0) Sg[0] = g;  // :76-80
+    __syncthreads();
+    // main chain, start ascending (:83-112, 175-205, 348-376, 512-531)
+    for (int s = 0; s < n; s++) {
+        for (int a_id = tid; a_id < d.Mc; a_id += NTG) {
+            const int a = d.mc_i2e(a_id);
+            if (!(a > 0 && a < m)) continue;
+            const float sg = coherent_load(&Sg[d.s_at(a_id, s)]), sa = S[d.s_at(a_id, s)];
+            if (sg == 0.f || sa != sa || fabsf(sa) == __builtin_huge_valf()) continue;
+            const int b_start = a - ml < 1 ? 1 : a - ml;
+            for (int c_id = a_id; d.mc_i2e(c_id) < m; c_id++) {
+                const int c = d.mc_i2e(c_id);
+                for (int j = 0; j < n - s && j < ml + 1; j++) {
+                    const float sc = S[d.s_at(c_id, s + j + 1)];
+                    if (sc != sc || fabsf(sc) == __builtin_huge_valf()) continue;
+                    for (int bb = b_start; bb < a + 1; bb++) {
+                        const int b_id = d.lt_e2i(bb == a ? 0 : bb);
+                        const float t = links[d.lk(a, a - bb, c)] + sc + C[d.c_at(b_id, s, j)] + match[(size_t)a * T + s + j] - sa;
+                        if (bad(t) || t == NEG_INF_F) continue;
+                        const float p = sg * expf(t);
+                        atomicAdd(&Sg[d.s_at(c_id, s + j + 1)], p);
+                        if (b_id != 0) atomicAdd(&Cg[d.c_at(b_id, s, j)], p);
+                        atomicAdd(&mg[(size_t)a * T + s + j], p);
+                        atomicAdd(&lg[d.lk(a, a - bb, c)], p);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (tid == 0) atomicAdd(&mg[(size_t)(m - 1) * T + (n - 1)], coherent_load(&Sg[d.s_at(d.mc_e2i(m - 1), n - 1)]));  // :379-382
+    __syncthreads();
+    // local trees, gap descending (:236-276, 407-428, 556-599; every gap >= 2, the forward's own ranges)
+    for (int gap = ml + 1; gap >= 2; gap--) {
+        const int ni = n - gap - 1;
+        for (int w = tid; ni > 0 && w < d.Lc * ni; w += NTG) {
+            const int a_id = w / ni, i = w - a_id * ni;
+            const int a = d.lt_i2e(a_id);
+            if (!(a > 0 && a < m)) continue;
+            const float cg = coherent_load(&Cg[d.c_at(a_id, i, gap)]), ca = C[d.c_at(a_id, i, gap)];
+            if (cg == 0.f || ca != ca || fabsf(ca) == __builtin_huge_valf()) continue;
+            const int hi = d.hi(a), b_start = a - ml < 1 ? 1 : a - ml;
+            for (int j = 0; j < gap; j++)
+                for (int bb = b_start; bb < a + 1; bb++) {
+                    const int b_id = d.lt_e2i(bb == a ? 0 : bb);
+                    for (int c = a + 1; c < hi && c < m; c++) {
+                        const int c_id = d.lt_e2i(c);
+                        const float t = links[d.lk(a, a - bb, c)] + C[d.c_at(b_id, i, j)] + C[d.c_at(c_id, i + j + 1, gap - j - 1)] +
+                                        match[(size_t)a * T + i + j] - ca;
+                        if (bad(t) || t == NEG_INF_F) continue;
+                        const float p = cg * expf(t);
+                        if (b_id != 0) atomicAdd(&Cg[d.c_at(b_id, i, j)], p);
+                        atomicAdd(&Cg[d.c_at(c_id, i + j + 1, gap - j - 1)], p);
+                        atomicAdd(&mg[(size_t)a * T + i + j], p);
+                        atomicAdd(&lg[d.lk(a, a - bb, c)], p);
+                    }
+                }
+        }
+        __syncthreads();
+    }
+    // leaves (:429-433)
+    for (int w = tid; w < d.Lc * n; w += NTG) {
+        const int a_id = w / n, i = w - a_id * n;
+        const int a = d.lt_i2e(a_id);
+        if (a > 0 && a < m && ((a - d.lo(a)) % 2 == 1)) atomicAdd(&mg[(size_t)a * T + i], coherent_load(&Cg[d.c_at(a_id, i, 1)]));
+    }
+}
+
+// ---- best tree (pcfg_best_tree.cu:64-197, 239-301); the 4-lane scan order is emulated per node -----------------
+__global__ __launch_bounds__(NTG) void generic_best_tree_kernel(const float *__restrict__ S_all, float *__restrict__ aux_all,
+                                                               const float *__restrict__ match_all, const float *__restrict__ links_all,
+                                                               const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
+                                                               int64_t *__restrict__ tree_all, int L, int T, int ml) {
+    const Dims d(L, T, ml);
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *match = match_all + (size_t)b * L * T;
+    const float *links = links_all + (size_t)b * L * (ml + 1) * L;
+    const float *S = S_all + (size_t)b * d.s_size();
+    float *aux = aux_all + (size_t)b * d.aux_floats();
+    const float *C = aux;
+    float *St = aux + 3 * d.c_size() + d.s_size();  // marks (0 / 1)
+    float *Ct = aux + 2 * d.c_size();
+    int64_t *tree = tree_all + (size_t)b * L;
+    for (int i = tid; i < L; i += NTG) tree[i] = -1;
+    if (!len_ok(d, m, n)) return;
+    for (size_t i = tid; i < d.s_size(); i += NTG) St[i] = 0.f;
+    for (size_t i = tid; i < d.c_size(); i += NTG) Ct[i] = 0.f;
+    __syncthreads();
+    if (tid == 0) St[0] = 1.f;
+    __syncthreads();
+    for (int s = 0; s <= n; s++) {
+        for (int a_id = tid; a_id < d.Mc; a_id += NTG) {
+            const int a = d.mc_i2e(a_id);
+            if (!(a > 0 && a < m && St[d.s_at(a_id, s)] != 0.f)) continue;
+            const int b_start = a - ml < 1 ? 1 : a - ml;
+            float lane_val[4];
+            int lane_c[4], lane_j[4], lane_b[4];
+            for (int x = 0; x < 4; x++) {
+                float maxval = NEG_INF_F;
+                int max_c = -1, max_j = 0, max_b = -1;
+                for (int c_id = a_id + x + 1; d.mc_i2e(c_id) < m; c_id += 4) {
+                    const int c = d.mc_i2e(c_id);
+                    for (int j = 0; j < n - s && j < ml + 1; j++)
+                        for (int bb = b_start; bb < a + 1; bb++) {
+                            const int b_id = d.lt_e2i(bb == a ? 0 : bb);
+                            float t = links[d.lk(a, a - bb, c)] + S[d.s_at(c_id, s + j + 1)] + C[d.c_at(b_id, s, j)] +
+                                      match[(size_t)a * T + s + j];
+                            if (bad(t)) t = NEG_INF_F;
+                            if (t > maxval) { maxval = t; max_c = c_id; max_j = j; max_b = b_id; }
+                        }
+                }
+                lane_val[x] = maxval; lane_c[x] = max_c; lane_j[x] = max_j; lane_b[x] = max_b;
+            }
+            for (int x = 0; x < 2; x++)
+                if (lane_val[x + 2] > lane_val[x]) { lane_val[x] = lane_val[x + 2]; lane_c[x] = lane_c[x + 2]; lane_j[x] = lane_j[x + 2]; lane_b[x] = lane_b[x + 2]; }
+            if (lane_val[1] > lane_val[0]) { lane_val[0] = lane_val[1]; lane_c[0] = lane_c[1]; lane_j[0] = lane_j[1]; lane_b[0] = lane_b[1]; }
+            if (lane_c[0] != -1 && lane_b[0] != -1) {
+                St[d.s_at(lane_c[0], s + lane_j[0] + 1)] = 1.f;
+                Ct[d.c_at(lane_b[0], s, lane_j[0])] = 1.f;
+            }
+            tree[a] = s + lane_j[0];
+        }
+        __syncthreads();
+    }
+    if (ml == 0) return;
+    for (int gap = ml + 1; gap >= 1; gap--) {
+        const int ni = n - gap - 1;
+        for (int w = tid; ni > 0 && w < (d.Lc - 1) * ni; w += NTG) {
+            const int a_id = 1 + w / ni, i = w % ni;
+            const int a = d.lt_i2e(a_id);
+            if (!(a > 0 && a < m) || Ct[d.c_at(a_id, i, gap)] == 0.f) continue;
+            const int hi = d.hi(a), b_start = a - ml < 1 ? 1 : a - ml;
+            int max_j = 0, max_b = -1, max_c = -1;
+            float maxval = NEG_INF_F;
+            for (int j = 0; j < gap; j++)
+                for (int bb = b_start; bb < a + 1; bb++) {
+                    const int b_id = d.lt_e2i(bb == a ? 0 : bb);
+                    for (int c = a + 1; c < hi && c < m; c++) {
+                        const int c_id = d.lt_e2i(c);
+                        float t = links[d.lk(a, a - bb, c)] + C[d.c_at(b_id, i, j)] + C[d.c_at(c_id, i + j + 1, gap - j - 1)] +
+                                  match[(size_t)a * T + i + j];
+                        if (bad(t)) t = NEG_INF_F;
+                        if (t > maxval) { maxval = t; max_j = j; max_b = b_id; max_c = c_id; }
+                    }
+                }
+            if (max_b != -1 && max_c != -1) {
+                Ct[d.c_at(max_b, i, max_j)] = 1.f;
+                Ct[d.c_at(max_c, i + max_j + 1, gap - max_j - 1)] = 1.f;
+            }
+            tree[a] = i + max_j;
+        }
+        __syncthreads();
+    }
+}
+
+// ---- viterbi (pcfg_viterbi.cu:177-241 then :22-140); tables [L][Lq] by external node id --------------------------
+__global__ __launch_bounds__(NTG) void generic_viterbi_kernel(const float *__restrict__ ob_all, const float *__restrict__ links_all,
+                                                             const int64_t *__restrict__ out_len, float *__restrict__ S_all,
+                                                             int64_t *__restrict__ R_all,
+                                                             int64_t *__restrict__ Lt_all, int64_t *__restrict__ M_all, int L, int ml) {
+    const int Lq = L / 4;
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const int m = (int)out_len[b];
+    const float *ob = ob_all + (size_t)b * L;
+    const float *links = links_all + (size_t)b * L * (ml + 1) * L;
+    const size_t tab = (size_t)b * L * Lq;
+    // the local-tree table lives in the rows of S that belong to local nodes and node 0 (the S sweep only touches
+    // main-chain rows); those cells are put back to -inf at the end, as the reference returns them
+    float *S = S_all + tab, *Cv = S;
+    int64_t *R = R_all + tab, *Lt = Lt_all + tab, *M = M_all + tab;
+    auto at = [&](int a, int l) -> size_t { return (size_t)a * Lq + l; };
+    auto lk = [&](int a, int k, int c) -> size_t { return ((size_t)a * (ml + 1) + k) * L + c; };
+    for (size_t i = tid; i < (size_t)L * Lq; i += NTG) { S[i] = NEG_INF_F; R[i] = 0; Lt[i] = 0; M[i] = 0; }
+    if (m < 2 || m > L || ((m - 2) % (ml + 1)) != 0) return;
+    __syncthreads();
+    for (int a = 1 + tid; a < L; a += NTG) {
+        const int lo = ((a - 1) / (ml + 1)) * (ml + 1) + 1;
+        if (a < m && ((a - lo) % 2 == 1) && Lq > 1) Cv[at(a, 1)] = ob[a];
+    }
+    if (tid == 0) Cv[at(0, 0)] = 0.f;
+    __syncthreads();
+    for (int gap = 2; gap < ml + 1 && gap < Lq; gap++) {
+        for (int a = 1 + tid; a < L; a += NTG) {
+            if (!(a < m && (a % (ml + 1) != 1))) continue;
+            const int hi = ((a - 1) / (ml + 1) + 1) * (ml + 1) + 1, b_start = a - ml < 1 ? 1 : a - ml;
+            float maxval = NEG_INF_F;
+            int max_b = 0, max_c = 0, max_j = 0;
+            for (int j = 0; j < gap; j++)
+                for (int bb = b_start; bb < a + 1; bb++) {
+                    const int _b = bb == a ? 0 : bb;
+                    for (int c = a + 1; c < hi && c < m; c++) {
+                        float t = ((links[lk(a, a - bb, c)] + Cv[at(_b, j)]) + Cv[at(c, gap - j - 1)]) + ob[a];
+                        if (bad(t)) t = NEG_INF_F;
+                        if (t > maxval) { maxval = t; max_b = _b; max_c = c; max_j = j; }
+                    }
+                }
+            if (maxval != NEG_INF_F) { Cv[at(a, gap)] = maxval; R[at(a, gap)] = max_c; Lt[at(a, gap)] = max_b; M[at(a, gap)] = max_j; }
+        }
+        __syncthreads();
+    }
+    if (tid == 0 && Lq > 1) S[at(m - 1, 1)] = ob[m - 1];
+    __syncthreads();
+    for (int len = 2; len < m / 4; len++) {
+        for (int id = tid; id * (ml + 1) + 1 < m; id += NTG) {
+            const int a = id * (ml + 1) + 1, b_start = a - ml < 1 ? 1 : a - ml;
+            float lane_val[4];
+            int lane_c[4], lane_j[4], lane_b[4];
+            for (int x = 0; x < 4; x++) {
+                float maxval = NEG_INF_F;
+                int max_b = 0, max_c = 0, max_j = 0;
+                for (int c_id = id + x; c_id * (ml + 1) + 1 < m; c_id += 4) {
+                    const int c = c_id * (ml + 1) + 1;
+                    for (int j = 0; j < ml + 1; j++)
+                        for (int bb = b_start; bb < a + 1; bb++) {
+                            const int _b = bb == a ? 0 : bb;
+                            const float sc = (len - j - 1 >= 0) ? S[at(c, len - j - 1)] : NEG_INF_F;
+                            const float cj = (j < Lq) ? Cv[at(_b, j)] : NEG_INF_F;
+                            float t = ((links[lk(a, a - bb, c)] + cj) + sc) + ob[a];
+                            if (bad(t)) t = NEG_INF_F;
+                            if (t > maxval) { maxval = t; max_b = _b; max_c = c; max_j = j; }
+                        }
+                }
+                lane_val[x] = maxval; lane_c[x] = max_c; lane_j[x] = max_j; lane_b[x] = max_b;
+            }
+            for (int x = 0; x < 2; x++)
+                if (lane_val[x + 2] > lane_val[x]) { lane_val[x] = lane_val[x + 2]; lane_c[x] = lane_c[x + 2]; lane_j[x] = lane_j[x + 2]; lane_b[x] = lane_b[x + 2]; }
+            if (lane_val[1] > lane_val[0]) { lane_val[0] = lane_val[1]; lane_c[0] = lane_c[1]; lane_j[0] = lane_j[1]; lane_b[0] = lane_b[1]; }
+            if (lane_val[0] != NEG_INF_F) {
+                S[at(a, len)] = lane_val[0]; Lt[at(a, len)] = lane_b[0]; R[at(a, len)] = lane_c[0]; M[at(a, len)] = lane_j[0];
+            }
+        }
+        __syncthreads();
+    }
+    for (int w = tid; w < L * Lq; w += NTG) {
+        const int a = w / Lq;
+        if (a == 0 || (a % (ml + 1)) != 1 || ml == 0) {
+            if (a == 0 || ml > 0) S[w] = NEG_INF_F;
+        }
+    }
+}
+
+}  // namespace
+
+size_t generic_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml) { return (size_t)B * Dims((int)L, (int)T, (int)ml).aux_floats(); }
+
+int generic_forward(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int64_t B,
+                    int64_t L, int64_t T, int64_t ml, void *stream) {
+    hipLaunchKernelGGL(generic_fwd_kernel, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, match_all, links, ol, tl, S, aux, (int)L,
+                       (int)T, (int)ml);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
+int generic_backward(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
+                     const int64_t *tl, float *mg, float *lg, int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream) {
+    hipLaunchKernelGGL(generic_bwd_kernel, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, go, S, aux, match_all, links, ol, tl, mg, lg,
+                       (int)L, (int)T, (int)ml, (int)norm_B);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
+int generic_best_tree(const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl,
+                      int64_t *tree, int64_t B, int64_t L, int64_t T, int64_t ml, void *stream) {
+    hipLaunchKernelGGL(generic_best_tree_kernel, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, S, aux, match_all, links, ol, tl, tree,
+                       (int)L, (int)T, (int)ml);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
+int generic_viterbi(const float *ob, const float *links, const int64_t *ol, float *S, int64_t *R, int64_t *Lt, int64_t *M, int64_t B,
+                    int64_t L, int64_t ml, void *stream) {
+    hipLaunchKernelGGL(generic_viterbi_kernel, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, ob, links, ol, S, R, Lt, M, (int)L,
+                       (int)ml);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
+}  // namespace pcfgnat

@@ -1306,11 +1306,8 @@ int check_dims(const char *who, int64_t B, int64_t L, int64_t T, int64_t ml) {
                     (long long)L, (long long)T);
     PCFGNAT_REQUIRE(ml >= 0, "%s: links must have at least one left option", who);
     PCFGNAT_REQUIRE(L <= 4096 && T <= 4096 && B <= 65535, "%s: dimension too large (L, T <= 4096, B <= 65535)", who);
-    if (ml != 1)
-        return fail(PCFGNAT_EUNSUPPORTED,
-                    "%s: max_left = %lld (links.size(2) = %lld); only max_left = 1 (--left-tree-layer 1, the setting of every shipped "
-                    "script) is built",
-                    who, (long long)ml, (long long)ml + 1);
+    PCFGNAT_REQUIRE(ml <= 63 && L >= ml + 3, "%s: max_left = %lld needs a graph of at least max_left + 3 nodes (and max_left <= 63)", who,
+                    (long long)ml);
     return PCFGNAT_OK;
 }
 
@@ -1321,6 +1318,7 @@ using namespace pcfgnat;
 
 extern "C" size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml) {
     if (B <= 0 || L < 2 || T < 0 || ml < 0) return 0;
+    if (ml != 1) return generic_aux_floats(B, L, T, ml);
     const int64_t Mc = (L - 2) / (ml + 1) + 1;
     if (Mc <= 128) return (size_t)B * 3 * Mc * (T + 2);
     return (size_t)B * ((size_t)5 * Mc * (T + 2) + (size_t)2 * Mc * Mc);
@@ -1333,6 +1331,7 @@ extern "C" int pcfgnat_pcfg_loss(const float *match_all, const float *links, con
     if (rc != PCFGNAT_OK) return rc;
     if (B == 0) return PCFGNAT_OK;
     PCFGNAT_REQUIRE(match_all && links && output_length && target_length && S && aux, "pcfg_loss: null pointer");
+    if (ml != 1) return generic_forward(match_all, links, output_length, target_length, S, aux, B, L, T, ml, stream);
     const int Mc = (int)((L - 2) / 2 + 1);
     hipStream_t s = (hipStream_t)stream;
     if (Mc <= 64) return launch_fwd<1>(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s);
@@ -1348,6 +1347,9 @@ int pcfgnat::inside_backward_impl(const float *grad_output, const float *S, floa
     if (B == 0) return PCFGNAT_OK;
     PCFGNAT_REQUIRE(S && aux && match_all && links && output_length && target_length && match_all_grad && links_grad,
                     "pcfg_loss_backward: null pointer");
+    if (ml != 1)
+        return generic_backward(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, B, L, T,
+                                ml, norm_B, stream);
     const int Mc = (int)((L - 2) / 2 + 1);
     hipStream_t s = (hipStream_t)stream;
     if (Mc <= 64)
@@ -1380,7 +1382,9 @@ int pcfgnat::inside_forward_backward_impl(const float *grad_output, const float 
     const int Mc = (int)((L - 2) / 2 + 1);
     hipStream_t s = (hipStream_t)stream;
     bool done = false;
-    if (Mc <= 64)
+    if (ml != 1) {
+        // general max_left: the two plain kernels
+    } else if (Mc <= 64)
         rc = launch_fused<1>(grad_output, match_all, links, output_length, target_length, S, match_all_grad, links_grad, (int)B, (int)L,
                              (int)T, Mc, (int)norm_B, s, &done);
     else if (Mc <= 128)
@@ -1406,20 +1410,23 @@ extern "C" int pcfgnat_criterion_loss(const float *S, const int64_t *target_leng
     int rc = check_dims("criterion_loss", B, L, T, ml);
     if (rc != PCFGNAT_OK) return rc;
     PCFGNAT_REQUIRE(B >= 1 && S && target_length && out, "criterion_loss: null pointer or empty batch");
-    const int Mc = (int)((L - 2) / 2 + 1);
+    const int Mc = (int)((L - 2) / (ml + 1) + 1);
     hipLaunchKernelGGL(criterion_loss_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, S, target_length, out, (int)B, Mc, (int)T);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
 
-extern "C" int pcfgnat_pcfg_best_tree(const float *S, const float *aux, const float *match_all, const float *links,
+extern "C" int pcfgnat_pcfg_best_tree(const float *S, float *aux, const float *match_all, const float *links,
                                       const int64_t *output_length, const int64_t *target_length, int64_t *tree, int64_t B, int64_t L,
                                       int64_t T, int64_t ml, void *stream) {
     int rc = check_dims("pcfg_best_tree", B, L, T, ml);
     if (rc != PCFGNAT_OK) return rc;
     if (B == 0) return PCFGNAT_OK;
     PCFGNAT_REQUIRE(S && match_all && links && output_length && target_length && tree, "pcfg_best_tree: null pointer");
-    (void)aux;
+    if (ml != 1) {
+        PCFGNAT_REQUIRE(aux != nullptr, "pcfg_best_tree: the auxiliary table of pcfg_loss is required for max_left != 1");
+        return generic_best_tree(S, aux, match_all, links, output_length, target_length, tree, B, L, T, ml, stream);
+    }
     const int Mc = (int)((L - 2) / 2 + 1);
     hipLaunchKernelGGL(best_tree_ml1_kernel, dim3((unsigned)B), dim3(64), 0, (hipStream_t)stream, S, match_all, links, output_length,
                        target_length, tree, (int)L, (int)T, Mc);

@@ -269,11 +269,11 @@ using namespace pcfgnat;
 extern "C" int pcfgnat_pcfg_viterbi(const float *ob_lprob, const float *links, const int64_t *output_length, float *S, int64_t *R,
                                     int64_t *Lt, int64_t *M, int64_t B, int64_t L, int64_t ml, void *stream) {
     PCFGNAT_REQUIRE(B >= 0 && L >= 4, "pcfg_viterbi: need B >= 0 and L >= 4 (got B=%lld L=%lld)", (long long)B, (long long)L);
-    if (ml != 1)
-        return fail(PCFGNAT_EUNSUPPORTED, "pcfg_viterbi: max_left = %lld; only max_left = 1 (--left-tree-layer 1) is built", (long long)ml);
+    PCFGNAT_REQUIRE(ml >= 0 && ml <= 63, "pcfg_viterbi: max_left out of range");
     PCFGNAT_REQUIRE(L / 4 > ml, "pcfg_viterbi: L/4 must exceed max_left");
     if (B == 0) return PCFGNAT_OK;
     PCFGNAT_REQUIRE(ob_lprob && links && output_length && S && R && Lt && M, "pcfg_viterbi: null pointer");
+    if (ml != 1) return generic_viterbi(ob_lprob, links, output_length, S, R, Lt, M, B, L, ml, stream);
     const int Mc = (int)((L - 2) / 2 + 1);
     const int Lq = (int)(L / 4);
     hipStream_t s = (hipStream_t)stream;

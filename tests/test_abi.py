@@ -34,8 +34,8 @@ def test_library_exports_every_declared_symbol():
 
 def test_argument_errors_without_gpu():
     lib = _lib.load()
-    rc = lib.pcfgnat_pcfg_loss(None, None, None, None, None, None, 2, 16, 4, 3, None)
-    assert rc == _lib.EUNSUPPORTED and b"max_left" in lib.pcfgnat_last_error()
+    rc = lib.pcfgnat_pcfg_loss(None, None, None, None, None, None, 2, 16, 4, 30, None)
+    assert rc == _lib.EINVAL and b"max_left" in lib.pcfgnat_last_error()
     rc = lib.pcfgnat_logsoftmax_gather(None, 7, None, 0, 0, 0, None, 0, 1, 1, 8, 1, None)
     assert rc == _lib.EINVAL
     with pytest.raises(RuntimeError):

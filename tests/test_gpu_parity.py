@@ -330,8 +330,8 @@ def test_errors_are_loud():
     links = torch.zeros(1, 8, 2, 8, device=DEV)
     ll = ops.cuda_pcfg_loss(match, links, torch.tensor([7], device=DEV), torch.tensor([4], device=DEV))
     assert torch.isnan(ll).all()
-    with pytest.raises(RuntimeError, match="max_left"):
-        ops.cuda_pcfg_loss(match, torch.zeros(1, 8, 4, 8, device=DEV), torch.tensor([8], device=DEV),
+    with pytest.raises(RuntimeError, match="max_left"):  # a graph of 8 nodes cannot hold max_left = 7
+        ops.cuda_pcfg_loss(match, torch.zeros(1, 8, 8, 8, device=DEV), torch.tensor([8], device=DEV),
                            torch.tensor([4], device=DEV))
 
 
@@ -360,3 +360,62 @@ def test_fused_step_equals_autograd_step():
         assert torch.allclose(glinks, links.grad, rtol=1e-5, atol=1e-9)
         assert torch.allclose(buf.float(), leaf.grad, rtol=2 ** -9, atol=2 ** -22)
         assert not glinks[3].any() and not buf[3].any()
+
+
+def _generic_batch(ml, L, ms, ns, seed, generic_local):
+    """Batch for a general max_left: links with the grammar's structural support (optionally with composite local trees),
+    random emissions with the eos column masked."""
+    from test_oracle_inside import random_links
+    rng = np.random.default_rng(seed)
+    B, T = len(ms), max(ns)
+    links = np.stack([random_links(rng, L, m, ml, p_drop=0.1, generic_local=generic_local) for m in ms]).astype(np.float32)
+    match = (rng.normal(size=(B, L, T)) - 2.0).astype(np.float32)
+    ol, tl = torch.tensor(ms), torch.tensor(ns)
+    match = harness.eos_masked(torch.from_numpy(match), ol, tl)
+    return match, torch.from_numpy(links), ol, tl
+
+
+@pytest.mark.parametrize("ml,L,ms,ns,generic_local", [
+    (3, 30, [30, 22, 14], [9, 8, 5], True),
+    (3, 66, [66, 50], [14, 20], False),
+    (7, 42, [42, 26], [8, 6], True),
+    (0, 12, [12, 9, 5], [7, 9, 3], False),
+    (2, 32, [32, 20], [9, 7], True),
+])
+def test_general_max_left_vs_oracle(ml, L, ms, ns, generic_local):
+    match, links, ol, tl = _generic_batch(ml, L, ms, ns, seed=ml * 100 + L, generic_local=generic_local)
+    S64, C64 = oracle.inside_fwd(match.numpy(), links.numpy(), ol.numpy(), tl.numpy(), dtype=np.float64)
+    mg64, lg64 = oracle.inside_bwd(np.ones(len(ms)), S64, C64, match.numpy(), links.numpy(), ol.numpy(), tl.numpy())
+    md = match.to(DEV).requires_grad_(True)
+    ld = links.to(DEV).requires_grad_(True)
+    ll = ops.cuda_pcfg_loss(md, ld, ol.to(DEV), tl.to(DEV))
+    want = S64[:, 0, 0]
+    got = ll.detach().cpu().double().numpy()
+    fin = np.isfinite(want)
+    assert fin.any() and np.array_equal(np.isfinite(got), fin)
+    assert np.allclose(got[fin], want[fin], rtol=1e-5)
+    ll.masked_fill(~torch.isfinite(ll), 0).sum().backward()
+    for bi in range(len(ms)):
+        for g_got, g_want in ((md.grad[bi], mg64[bi]), (ld.grad[bi], lg64[bi])):
+            g_got = g_got.cpu().double().numpy()
+            assert np.isfinite(g_got).all()
+            assert np.abs(g_got - g_want).max() <= 1e-4 * max(np.abs(g_want).max(), 1e-30)
+    # best tree: same alignment as the oracle on these seeds, and a valid alignment
+    tree, ll2 = ops.cuda_pcfg_best_tree(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV))
+    want_tree = oracle.best_tree(S64, C64, match.numpy(), links.numpy(), ol.numpy(), tl.numpy())
+    assert np.array_equal(tree.cpu().numpy(), want_tree)
+    assert torch.allclose(ll2, ll.detach(), rtol=1e-6, equal_nan=True)
+
+
+@pytest.mark.parametrize("ml,L,ms", [(3, 66, [66, 50, 34]), (7, 74, [74, 42]), (0, 24, [24, 13]), (2, 50, [50, 32])])
+def test_general_max_left_viterbi_bit_exact(ml, L, ms):
+    from test_oracle_inside import random_links
+    rng = np.random.default_rng(ml + L)
+    links = np.stack([random_links(rng, L, m, ml, p_drop=0.1, generic_local=True) for m in ms]).astype(np.float32)
+    ob = (rng.normal(size=(len(ms), L)) - 1.0).astype(np.float32)
+    ol = torch.tensor(ms)
+    scores, R, Lt, M = ops.cuda_pcfg_viterbi(torch.from_numpy(ob).to(DEV), torch.from_numpy(links).to(DEV), ol.to(DEV))
+    S_o, R_o, L_o, M_o = oracle.viterbi(ob, links, ol.numpy(), dtype=np.float32)
+    assert np.isfinite(S_o[:, 1, :]).any()
+    assert np.array_equal(scores.cpu().numpy(), S_o[:, 1, :])
+    assert np.array_equal(R.cpu().numpy(), R_o) and np.array_equal(Lt.cpu().numpy(), L_o) and np.array_equal(M.cpu().numpy(), M_o)
