@@ -360,7 +360,7 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
     the gather forward, inside forward, inside backward and gather backward of the first slice.  ``slices``: how many
     batch slices alternate between the current stream and the library's helper stream (default 1: measured on MI355X the
     bandwidth-bound gather kernels leave no room for a second kernel on the CUs, so slicing does not pay).  Returns
-    (loss_and_invalid [2] float32, links_grad, ll [B], match_all_eos_masked)."""
+    (loss_and_invalid [2] float32, links_grad, ll [B], match_all_eos_masked, match_all_grad)."""
     lib = get_pcfg_kernel()
     _need_cuda("pcfg_criterion_step", logits, targets, links, output_length, target_length)
     if logits.dim() != 3 or not logits.is_contiguous():
@@ -398,4 +398,4 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
         _lib.check(lib.pcfgnat_criterion_step(logits.data_ptr(), code, targets.data_ptr(), links.data_ptr(), ol.data_ptr(),
                                               tl.data_ptr(), match.data_ptr(), S.data_ptr(), aux.data_ptr(), mg.data_ptr(),
                                               lg.data_ptr(), out.data_ptr(), B, L, V, T, ml, slices, _stream(logits), ev_arr), lib)
-    return out, lg, S[:, 0, 0], match
+    return out, lg, S[:, 0, 0], match, mg

@@ -42,9 +42,11 @@ def compute_pcfg_loss(outputs, output_masks, targets, target_masks, links, ops=_
 
 
 def glat_alignment(word_ins_out, tgt_tokens, prev_output_tokens, links, context_p, pad=PAD, ops=_default_ops,
-                   generator=None):
+                   generator=None, noise_device=None):
     """GLAT glancing with the ``number-random`` strategy (nat_pcfg_loss.py:193-269): best-tree alignment of target
-    tokens to graph nodes, then a random subset of the aligned nodes is revealed.  RNG order: ``randn`` then ``rand``."""
+    tokens to graph nodes, then a random subset of the aligned nodes is revealed.  RNG order: ``randn`` then ``rand``.
+    The reference draws both on the tokens' device; ``noise_device`` (e.g. "cpu") draws them elsewhere and moves them,
+    which makes a run reproducible across devices."""
     batch_size, prelen = links.shape[0], links.shape[1]
     tarlen = tgt_tokens.shape[1]
     target_length = (~tgt_tokens.eq(pad)).sum(1)
@@ -64,13 +66,14 @@ def glat_alignment(word_ins_out, tgt_tokens, prev_output_tokens, links, context_
     oracle = tgt_tokens.gather(-1, path.clip(min=0))
     same_num = ((pred_tokens == oracle) & predict_align_mask).sum(1)
     dev = tgt_tokens.device
-    prob = torch.randn(oracle.shape, device=dev, dtype=torch.float, generator=generator)
+    ndev = dev if noise_device is None else torch.device(noise_device)
+    prob = torch.randn(oracle.shape, device=ndev, dtype=torch.float, generator=generator).to(dev)
     prob.masked_fill_(~predict_align_mask, -100)
     glance_nums = ((target_length - same_num) * context_p + 0.5).to(torch.long)
     prob_thresh = prob.sort(descending=True)[0].gather(-1, (glance_nums - 1).clip(min=0).unsqueeze(-1)).squeeze(-1)
     prob_thresh.masked_fill_(glance_nums == 0, 100)
     keep_prob = (prob >= prob_thresh.unsqueeze(-1)).to(prob.dtype)
-    keep_word_mask = (torch.rand(prev_output_tokens.shape, device=dev, generator=generator) < keep_prob).bool()
+    keep_word_mask = (torch.rand(prev_output_tokens.shape, device=ndev, generator=generator).to(dev) < keep_prob).bool()
     glat_prev_output_tokens = prev_output_tokens.masked_fill(keep_word_mask, 0) + oracle.masked_fill(~keep_word_mask, 0)
     return {"path": path, "matchmask": matchmask, "keep_word_mask": keep_word_mask,
             "glat_prev_output_tokens": glat_prev_output_tokens, "same_num": same_num, "glance_nums": glance_nums,
@@ -161,6 +164,6 @@ def train_step_single_call(logits, targets, links, output_length, target_length,
     events = None
     if mark is not None:
         events = mark("events", 8)  # the caller hands out eight timing events for this step
-    out, glinks, ll, _ = ops.pcfg_criterion_step(logits, targets, links, output_length, target_length, events=events,
+    out, glinks, ll, _, _ = ops.pcfg_criterion_step(logits, targets, links, output_length, target_length, events=events,
                                                  slices=slices)
     return out[0], glinks, ll

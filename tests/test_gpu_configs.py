@@ -1,0 +1,142 @@
+"""The BASELINE configurations at their full sizes on the GPU: checked against torch's library routines on the device,
+against the CPU oracle on a bounded sample of sentences, and through size-independent properties (posterior mass per
+target token, rule mass = emission mass, softmax rows summing to one, gradients of the gathered logits summing to zero).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle_ops
+from oracle import oracle
+from pcfg_nat_amd import custom_ops as ops
+from pcfg_nat_amd import harness, synth
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _check_training_batch(batch, sample, grad_tol=1e-4):
+    B, L, V = batch["logits"].shape
+    T = batch["targets"].shape[1]
+    ol, tl = batch["output_length"], batch["target_length"]
+    logits = batch["logits"].to(DEV)
+    targets, links = batch["targets"].to(DEV), batch["links"].to(DEV)
+    idx = targets.unsqueeze(1).expand(-1, L, -1)
+    want_sel = torch.log_softmax(logits.float(), -1).gather(-1, idx)
+    want_sel = harness.eos_masked(want_sel, ol.to(DEV), tl.to(DEV))
+    buf = logits.clone()
+    out, glinks, ll, match, mgrad = ops.pcfg_criterion_step(buf, targets, links, ol.to(DEV), tl.to(DEV))
+    fin = torch.isfinite(want_sel)
+    assert torch.equal(torch.isfinite(match), fin)
+    assert torch.allclose(match[fin], want_sel[fin], rtol=2e-5, atol=2e-5)
+    assert torch.isfinite(ll).all() and float(out[1]) == 0
+    assert torch.allclose(out[0], -(ll / tl.to(DEV)).mean(), rtol=1e-6)
+    # gradient of the loss w.r.t. the logits: every row sums to ~0 (softmax), fp16 storage
+    g = buf.float()
+    assert torch.isfinite(g).all()
+    # (each of the V entries is rounded to fp16, most of them in the subnormal range whose spacing is 2^-24)
+    row_sums = g.sum(-1).abs().max().item()
+    assert row_sums < V * 2.0 ** -25 + 1e-6
+    # every target token is emitted by exactly one node: posterior mass per position = d loss / d ll_b
+    coef = (-1.0 / (tl.double() * B))
+    mgd = mgrad.double().cpu()
+    lg = glinks.double().cpu()
+    assert torch.isfinite(lg).all() and torch.isfinite(mgd).all()
+    pos = torch.arange(T).view(1, T)
+    want_mass = torch.where(pos < tl.view(B, 1), coef.view(B, 1).expand(B, T), torch.zeros(B, T, dtype=torch.float64))
+    assert torch.allclose(mgd.sum(1), want_mass, rtol=2 * grad_tol, atol=1e-12)
+    # the rule mass of each main-chain parent equals its emission mass (the last node emits once without a rule)
+    rule_mass = lg.sum(dim=(2, 3))                       # [B, L]
+    emit_mass = mgd.sum(2)                               # [B, L]
+    last = (ol - 1).view(B, 1)
+    emit_mass = emit_mass - torch.zeros(B, L, dtype=torch.float64).scatter_(1, last, coef.view(B, 1))
+    main_rows = (torch.arange(L) % 2 == 1).view(1, L)
+    assert (rule_mass - emit_mass)[main_rows.expand(B, L)].abs().max() <= 2 * grad_tol * coef.abs().max()
+    assert not rule_mass[~main_rows.expand(B, L)].any()
+    # oracle on a few sentences, end to end through the same glue
+    sub = {k: (v[sample] if torch.is_tensor(v) else v) for k, v in batch.items()}
+    leaf = sub["logits"].float().clone().requires_grad_(True)
+    lk = sub["links"].clone().requires_grad_(True)
+    n_s = len(sample)
+    out_mask = torch.arange(L).view(1, L) < sub["output_length"].view(n_s, 1)
+    res = harness.compute_pcfg_loss(leaf * 1.0, out_mask, sub["targets"], sub["targets"].ne(synth.PAD), lk, ops=oracle_ops)
+    ll_o = res["ll"].detach()
+    assert torch.allclose(ll[sample].cpu(), ll_o, rtol=2e-5)
+    (res["ll"] * coef[sample].float()).sum().backward()
+    lg_o = lk.grad.double()
+    for i, b in enumerate(sample):
+        err = ((lg[b] - lg_o[i]).abs().max() / lg_o[i].abs().max()).item()
+        print("links_grad normwise error, sentence %d: %.2e" % (b, err))
+        assert err <= grad_tol
+        want_g = leaf.grad[i]
+        got_g = g[b].cpu()
+        # fp16 buffer: each element within fp16 rounding of the fp32 gradient (plus the rounding of the row factor)
+        assert (got_g - want_g).abs().max() <= 2 ** -9 * want_g.abs().max() + 1e-9
+
+
+def test_config2_full_size():
+    _check_training_batch(synth.config2(), sample=[0, 7, 39])
+
+
+def test_config3_full_size():
+    # 139 sequential steps on table entries of magnitude ~1.8e3, where fp32 spacing is 1.2e-4: a sequential fp32 evaluation
+    # (the oracle's float instantiation, which follows the reference) is itself 1.3e-4 .. 1.5e-4 away from float64 here
+    _check_training_batch(synth.config3(), sample=[3], grad_tol=5e-4)
+
+
+def test_config5_glat_alignment():
+    batch = synth.config2()
+    B, L, V = batch["logits"].shape
+    prev = torch.full((B, L), 3, dtype=torch.int64)
+    prev = prev.masked_fill(torch.arange(L).view(1, L) >= batch["output_length"].view(B, 1), synth.PAD)
+    logits = batch["logits"].to(DEV)
+    g1 = torch.Generator().manual_seed(7)
+    got = harness.glat_alignment(logits, batch["targets"].to(DEV), prev.to(DEV), batch["links"].to(DEV), 0.5, generator=g1,
+                                 noise_device="cpu")
+    assert torch.equal(logits, batch["logits"].to(DEV))  # no gradient requested: logits untouched
+    # oracle trace on the GPU's own inside table: bit-exact
+    idx = batch["targets"].unsqueeze(1).expand(-1, L, -1)
+    sel = ops._logsoftmax_gather(logits, idx.to(DEV), False)
+    match = harness.eos_masked(sel, batch["output_length"].to(DEV), batch["target_length"].to(DEV))
+    S_gpu, _, _, _ = ops._pcfg_loss_tables(match, batch["links"].to(DEV), batch["output_length"].to(DEV),
+                                           batch["target_length"].to(DEV), 1, "test")
+    m_np, l_np = match.cpu().numpy(), batch["links"].numpy()
+    ol, tl = batch["output_length"].numpy(), batch["target_length"].numpy()
+    _, C32 = oracle.inside_fwd(m_np, l_np, ol, tl, dtype=np.float32)
+    want_tree = oracle.best_tree(S_gpu.cpu().numpy(), C32, m_np, l_np, ol, tl, dtype=np.float32)
+    tree = torch.from_numpy(want_tree)
+    path = tree.clone()
+    path[path + 1 >= batch["targets"].shape[1] + 1] = -1
+    assert torch.equal(got["path"].cpu(), path)
+    # the same glue over the oracle (CPU) with the same noise: identical glancing decisions
+    g2 = torch.Generator().manual_seed(7)
+    want = harness.glat_alignment(batch["logits"].float(), batch["targets"], prev, batch["links"], 0.5, ops=oracle_ops,
+                                  generator=g2)
+    assert torch.equal(got["path"].cpu(), want["path"])
+    assert torch.equal(got["keep_word_mask"].cpu(), want["keep_word_mask"])
+    assert torch.equal(got["glat_prev_output_tokens"].cpu(), want["glat_prev_output_tokens"])
+    assert torch.equal(got["matchmask"].cpu(), want["matchmask"])
+
+
+def test_config4_viterbi_decode():
+    lens = synth.config4_lengths()
+    srt = torch.sort(lens)[0]
+    gen = torch.Generator(device=DEV).manual_seed(3)
+
+    def case(src):
+        m = 4 * src
+        Lx = int(m.max())
+        g = torch.Generator().manual_seed(int(src.sum()))
+        links = synth.make_links(len(src), Lx, m, 1, g)
+        logits = (torch.randn(len(src), Lx, 40000, device=DEV, generator=gen) * 3).half()
+        ob, tok = synth.ob_and_tokens(logits)  # computed once, fed to both paths
+        del logits
+        return ob, tok, links, m, synth.support_masks(Lx, 1)[0]
+
+    chunks = [srt[0:64], srt[480:544], srt[936:1000]] + [lens[i:i + 1] for i in range(12)]
+    for src in chunks:
+        ob, tok, links, m, mask = case(src)
+        got_tok, got_len = harness.viterbi_decode(ob, tok, links.to(DEV), m.to(DEV), mask.to(DEV))
+        want_tok, want_len = harness.viterbi_decode(ob.cpu(), tok.cpu(), links, m, mask, ops=oracle_ops)
+        assert torch.equal(got_len.cpu(), want_len)
+        assert torch.equal(got_tok.cpu(), want_tok)
