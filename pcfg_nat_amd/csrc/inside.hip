@@ -32,15 +32,47 @@ __device__ __forceinline__ float lse2(float a, float b) {
     return m + __logf(__expf(a - m) + __expf(b - m));
 }
 
-// Aux layout per sentence (Mc <= 128): F0, F1, BETA, each [Mc][T+2], log-domain values in base 2.
+// Column offsets.  Entries of S grow like (tokens left) x (log-probability per token), thousands for long sentences,
+// where fp32 resolves only ~1e-4 - and posteriors are exponentials of sums of such entries.  Every sweep therefore
+// keeps column t of the inside table relative to a per-column offset O_t (S[a][t] = R_t[a] + O_t), chosen on the fly as
+// O_{t-1} = O_t + D_t with D_t following the column maximum (max_a R_t[a] in the streaming kernels, max_a R_{t+1}[a] in
+// the register-resident ones, whose reduction thus stays off the critical path; any D_t is exact, the choice only bounds
+// magnitudes), so that all stored and exchanged numbers stay within a few tens of units and only the offsets
+// (accumulated in double) are large.  The tables the backward consumes are kept in this
+// relative form:  F0h_t[a] = LSE_c(links[a][0][c] + R_t[c]) - D_t  (= F0[a][t] - O_{t-1}),  same for F1h, and the
+// outside sweep produces Bh_t[c] = beta[c][t] + O_t, so that log-posteriors are sums of small numbers:
+//   emission  (a,s), null left child:  Bh_s[a] + match[a][s] + F0h_{s+1}[a]
+//   emission  (a,s), leaf emitted s:   Bh_s[a] + match[a-1][s] + match[a][s+1] + F1h_{s+2}[a] - D_{s+1}
+//   rule      a -> c at column t:      links[a][k][c] + Wk_t[a] + R_t[c],   W0_t[a] = match[a][t-1] + Bh_{t-1}[a] - D_t,
+//                                      W1_t[a] = match[a-1][t-2] + match[a][t-1] + Bh_{t-2}[a] - D_t - D_{t-1}.
+//
+// Aux layout per sentence (Mc <= 128): F0h, F1h, Bh, R, each [Mc][T+2], then D [T+4]; log-domain values in base 2.
+__host__ __device__ inline size_t aux_stride_reg(int Mc, int T) { return (size_t)4 * Mc * (T + 2) + (size_t)(T + 4); }
 struct AuxView {
-    float *F0, *F1, *BETA;
+    float *F0, *F1, *BETA, *SR, *D;
     __device__ AuxView(float *aux, int b, int Mc, int T) {
         size_t plane = (size_t)Mc * (T + 2);
-        float *base = aux + (size_t)b * 3 * plane;
+        float *base = aux + (size_t)b * aux_stride_reg(Mc, T);
         F0 = base;
         F1 = base + plane;
         BETA = base + 2 * plane;
+        SR = base + 3 * plane;
+        D = base + 4 * plane;
+    }
+};
+
+// Head of the dynamic LDS of the register-resident kernels: per-wave column maxima slots[2][8] (16-byte aligned), the
+// column offsets O [T+2] (double) and the shifts D [T+4].
+__host__ __device__ inline int head_floats(int T) { return 16 + 2 * (T + 2) + (T + 4); }
+struct LdsHead {
+    float *slots, *D;
+    double *O;
+    float *rest;
+    __device__ LdsHead(float *smem, int T) {
+        slots = smem;
+        O = reinterpret_cast<double *>(smem + 16);
+        D = smem + 16 + 2 * (T + 2);
+        rest = smem + head_floats(T);
     }
 };
 
@@ -60,16 +92,33 @@ __device__ __forceinline__ bool lengths_ok(int m, int n, int L, int T) {
 constexpr int NTR = 512;
 constexpr size_t LDS_BUDGET = 128 * 1024;  // of the 160 KB a gfx950 workgroup may use
 constexpr float LOG2E_F = 1.4426950408889634f;
-constexpr float LN2_F = 0.6931471805599453f;
+constexpr double LN2_D = 0.6931471805599453094;
 
 __device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float lg2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float to_b2(float natural) { return sanitize(natural) * LOG2E_F; }
 
+// max(v, v of the partner lane) as one DPP instruction.  Written in assembly because fmaxf() on a value that comes out
+// of a DPP move (or an LDS load) is compiled to move + canonicalise + max, four instructions in loops that are bound by
+// instruction issue; the hardware max already quiets NaNs in the IEEE mode kernels run in.  The leading s_nop covers
+// the two wait states a DPP read needs after a VALU write of the same register, which the compiler does not track
+// through inline assembly; inputs must not come straight from a transcendental instruction (v_exp/v_log), same reason.
+#define PCFGNAT_DPP_MAX(name, ctrl)                                                                          \
+    __device__ __forceinline__ float name(float v) {                                                          \
+        float r;                                                                                              \
+        asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v)); \
+        return r;                                                                                             \
+    }
+PCFGNAT_DPP_MAX(dpp_max_xor1, "quad_perm:[1,0,3,2]")
+PCFGNAT_DPP_MAX(dpp_max_xor2, "quad_perm:[2,3,0,1]")
+PCFGNAT_DPP_MAX(dpp_max_half_mirror, "row_half_mirror")
+PCFGNAT_DPP_MAX(dpp_max_mirror, "row_mirror")
+#undef PCFGNAT_DPP_MAX
+
 __device__ __forceinline__ float row8_max(float v) {
-    v = fmaxf(v, dpp_f<DPP_QUAD_XOR1>(v));
-    v = fmaxf(v, dpp_f<DPP_QUAD_XOR2>(v));
-    v = fmaxf(v, dpp_f<DPP_ROW_HALF_MIRROR>(v));
+    v = dpp_max_xor1(v);
+    v = dpp_max_xor2(v);
+    v = dpp_max_half_mirror(v);
     return v;
 }
 __device__ __forceinline__ float row8_sum(float v) {
@@ -93,9 +142,33 @@ __device__ __forceinline__ void pin(float &v) { asm volatile("" : "+v"(v)); }
 struct FwdSweepArgs {
     float *col, *sm_main, *sm_leaf, *sm_S, *sm_F0, *sm_F1;
     const float *mt;
-    float *Sb, *gF0, *gF1;
+    float *Sb, *gF0, *gF1, *gSR;
+    float *slots, *sm_D;
+    double *sm_O;
+    float base_b2;  // the base cell S[last][n-1], base 2
     int n, mc, Mc, T, j, g8;
 };
+
+// max of three values that need no canonicalisation (loaded from tables this kernel wrote)
+__device__ __forceinline__ float max3_raw(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+// maximum of eight floats stored at a 16-byte aligned LDS address (two broadcast reads)
+__device__ __forceinline__ float max8(const float *p) {
+    const float4 a = *reinterpret_cast<const float4 *>(p), b = *reinterpret_cast<const float4 *>(p + 4);
+    return max3_raw(max3_raw(a.x, a.y, a.z), max3_raw(a.w, b.x, b.y), max3_raw(b.z, b.w, b.w));
+}
+// maximum over the wave of a value that is uniform inside each 8-lane group
+__device__ __forceinline__ float wave_max_of_groups(float v) {
+    v = dpp_max_mirror(v);
+    const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
 
 // The forward sweep of one wave, specialised on its node block P so that the chunks below the diagonal (q < 8r + P)
 // vanish at compile time.  Executes n-1 workgroup barriers regardless of P.
@@ -107,9 +180,15 @@ __device__ __forceinline__ void fwd_sweep(const float (&A0)[R][8 * R], const flo
     float F1prev[R];
 #pragma unroll
     for (int r = 0; r < R; r++) F1prev[r] = NEG_INF_F;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    double O = 0.0;           // offset of the column being read
+    float wprev = x.base_b2;  // this wave's maximum of the column written by the previous step
     for (int t = x.n - 1; t >= 1; t--) {
         const float *cur = x.col + (t & 1) * MP;
         float *nxt = x.col + ((t - 1) & 1) * MP;
+        float wmax = NEG_INF_F;
+        float Ds = 0.f;
+        double O_new = 0.0;
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const int a_id = 64 * r + 8 * P + x.g8;
@@ -119,6 +198,20 @@ __device__ __forceinline__ void fwd_sweep(const float (&A0)[R][8 * R], const flo
 #pragma unroll
             for (int q = 0; q < NQ; q++)
                 if (q >= q0) sc[q] = cur[j + 8 * q];
+            if (r == 0) {
+                // Bookkeeping in the shadow of the column loads (issued after them on purpose).  Shift of this step: the
+                // maximum of column t+1, whose per-wave parts were published one step ago.  (LDS float-max atomics on
+                // one cell would give the maximum of column t itself without the reduction below, but 64 of them per
+                // step on one address cost ten times more than this.)
+                const float D = max8(x.slots + ((t + 1) & 1) * 8);
+                x.slots[(t & 1) * 8 + wave] = wave_max_of_groups(wprev);  // maximum of column t, read by step t-1
+                Ds = (D == NEG_INF_F) ? 0.f : D;
+                if (!TAB_LDS || wave == 0) O_new = O + (double)Ds;  // offset of column t-1
+                if (wave == 0) {
+                    x.sm_D[t] = Ds;
+                    x.sm_O[t - 1] = O_new;
+                }
+            }
             float ma_p, ml_p, ma_t;  // match[a][t-1], match[a-1][t-1], match[a][t]
             if (TAB_LDS) {
                 ma_p = x.sm_main[ai * T + t - 1];
@@ -156,11 +249,12 @@ __device__ __forceinline__ void fwd_sweep(const float (&A0)[R][8 * R], const flo
             }
             e0 = row8_sum(e0);
             e1 = row8_sum(e1);
-            const float F0 = (m0 == NEG_INF_F) ? NEG_INF_F : m0 + lg2(e0);
-            const float F1 = (m1 == NEG_INF_F) ? NEG_INF_F : m1 + lg2(e1);
-            float s_new = lse2_b2(ma_p + F0, (ml_p + ma_t) + F1prev[r]);
+            const float F0 = (m0 == NEG_INF_F) ? NEG_INF_F : (m0 - Ds) + lg2(e0);
+            const float F1 = (m1 == NEG_INF_F) ? NEG_INF_F : (m1 - Ds) + lg2(e1);
+            float s_new = lse2_b2(ma_p + F0, (ml_p + ma_t) + (F1prev[r] - Ds));
             if (a_id >= x.mc) s_new = NEG_INF_F;
             F1prev[r] = F1;
+            wmax = fmaxf(wmax, s_new);
             if (j == 0) {
                 nxt[a_id] = s_new;
                 if (a_id < x.mc) {
@@ -169,20 +263,23 @@ __device__ __forceinline__ void fwd_sweep(const float (&A0)[R][8 * R], const flo
                         x.sm_F0[a_id * TS + t] = F0;
                         x.sm_F1[a_id * TS + t] = F1;
                     } else {
-                        x.Sb[(size_t)a_id * TS + (t - 1)] = s_new * LN2_F;
+                        x.Sb[(size_t)a_id * TS + (t - 1)] = (float)(((double)s_new + O_new) * LN2_D);
+                        x.gSR[(size_t)a_id * TS + (t - 1)] = s_new;
                         x.gF0[(size_t)a_id * TS + t] = F0;
                         x.gF1[(size_t)a_id * TS + t] = F1;
                     }
                 }
             }
         }
+        wprev = wmax;
+        O = O_new;
         lds_barrier();
     }
 }
 
-// Forward.  Dynamic LDS: col[2][64R]; with TAB_LDS also the emissions of main nodes and of their leaves [Mc][T] and the
-// S, F0, F1 tables [Mc][T+2] (all base 2), which are copied out in bulk when the sweep is over - the sweep itself then
-// touches no global memory.
+// Forward.  Dynamic LDS: head (see LdsHead), col[2][64R]; with TAB_LDS also the emissions of main nodes and of their
+// leaves [Mc][T] and the R, F0h, F1h tables [Mc][T+2] (all base 2), which are copied out in bulk when the sweep is over -
+// the sweep itself then touches no global memory.
 template <int R, bool TAB_LDS>
 __global__ __launch_bounds__(NTR) void inside_fwd_ml1_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
                                                             const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
@@ -191,8 +288,9 @@ __global__ __launch_bounds__(NTR) void inside_fwd_ml1_kernel(const float *__rest
     constexpr int MP = 64 * R;
     const int TS = T + 2;
     extern __shared__ float smem[];
-    float *col = smem;               // [2][MP]
-    float *sm_main = smem + 2 * MP;  // [Mc][T]
+    LdsHead hd(smem, T);
+    float *col = hd.rest;            // [2][MP]
+    float *sm_main = col + 2 * MP;   // [Mc][T]
     float *sm_leaf = sm_main + (TAB_LDS ? Mc * T : 0);
     float *sm_S = sm_leaf + (TAB_LDS ? Mc * T : 0);  // [Mc][TS]
     float *sm_F0 = sm_S + (TAB_LDS ? Mc * TS : 0);
@@ -241,13 +339,22 @@ __global__ __launch_bounds__(NTR) void inside_fwd_ml1_kernel(const float *__rest
             sm_F1[i] = NEG_INF_F;
         }
     } else {
-        // cells of S the sweep never writes: rows beyond the sentence, columns from n-1 on (except the base cell)
+        // cells of S and R the sweep never writes: rows beyond the sentence, columns from n-1 on (except the base cell)
         for (int i = tid; i < Mc * TS; i += NTR) {
             const int a_id = i / TS, s = i - a_id * TS;
-            if (a_id >= mc || s >= n - 1) Sb[i] = (a_id == mc - 1 && s == n - 1) ? base_cell : NEG_INF_F;
+            if (a_id >= mc || s >= n - 1) {
+                const bool is_base = (a_id == mc - 1 && s == n - 1);
+                Sb[i] = is_base ? base_cell : NEG_INF_F;
+                av.SR[i] = is_base ? base_cell * LOG2E_F : NEG_INF_F;
+            }
         }
     }
     for (int i = tid; i < MP; i += NTR) col[((n - 1) & 1) * MP + i] = (i == mc - 1) ? base_cell * LOG2E_F : NEG_INF_F;
+    for (int i = tid; i < TS + 2; i += NTR) {
+        hd.D[i] = 0.f;
+        if (i < TS) hd.O[i] = 0.0;
+    }
+    if (tid < 16) hd.slots[tid] = base_cell * LOG2E_F;  // maximum of column n-1
 #pragma unroll
     for (int r = 0; r < R; r++) {
         const int a_id = 64 * r + 8 * p + g8;
@@ -261,7 +368,7 @@ __global__ __launch_bounds__(NTR) void inside_fwd_ml1_kernel(const float *__rest
     }
     __syncthreads();
     PCFGNAT_PHASE(1);
-    FwdSweepArgs sa{col, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, av.F0, av.F1, n, mc, Mc, T, j, g8};
+    FwdSweepArgs sa{col, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, av.F0, av.F1, av.SR, hd.slots, hd.D, hd.O, base_cell * LOG2E_F, n, mc, Mc, T, j, g8};
     switch (p) {  // wave-uniform: every wave runs the sweep specialised for its node block
         case 0: fwd_sweep<R, TAB_LDS, 0>(A0, A1, sa); break;
         case 1: fwd_sweep<R, TAB_LDS, 1>(A0, A1, sa); break;
@@ -275,18 +382,23 @@ __global__ __launch_bounds__(NTR) void inside_fwd_ml1_kernel(const float *__rest
     PCFGNAT_PHASE(2);
     if (TAB_LDS) {
         for (int i = tid; i < Mc * TS; i += NTR) {
-            Sb[i] = sm_S[i] * LN2_F;
+            const int t = i - (i / TS) * TS;
+            const float r2 = sm_S[i];
+            Sb[i] = (float)(((double)r2 + hd.O[t]) * LN2_D);
+            av.SR[i] = r2;
             av.F0[i] = sm_F0[i];
             av.F1[i] = sm_F1[i];
         }
     }
+    for (int i = tid; i < TS + 2; i += NTR) av.D[i] = hd.D[i];
     PCFGNAT_PHASE(3);
 }
 
 struct BwdSweepArgs {
     float *w0, *w1, *sm_S, *sm_B, *sm_main, *sm_leaf;
-    const float *mt, *Sb;
+    const float *mt, *gSR;
     float *gBETA;
+    const float *sm_D;
     float beta00;
     int n, mc, Mc, T, j, g8;
 };
@@ -304,6 +416,7 @@ __device__ __forceinline__ void bwd_sweep(const float (&A0)[R][8 * R], const flo
     for (int t = 1; t <= x.n - 1; t++) {
         const float *c0 = x.w0 + (t & 1) * MP, *c1 = x.w1 + (t & 1) * MP;
         float *n0 = x.w0 + ((t + 1) & 1) * MP, *n1 = x.w1 + ((t + 1) & 1) * MP;
+        const float d_next = x.sm_D[t + 1], d_both = d_next + x.sm_D[t];
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const int c_id = 64 * r + 8 * P + x.g8;
@@ -324,7 +437,7 @@ __device__ __forceinline__ void bwd_sweep(const float (&A0)[R][8 * R], const flo
                 mc_t = x.sm_main[ci * T + t];
                 ml_p = x.sm_leaf[ci * T + t - 1];
             } else {
-                sct = x.Sb[(size_t)ci * TS + t] * LOG2E_F;
+                sct = x.gSR[(size_t)ci * TS + t];
                 mc_t = to_b2(x.mt[(size_t)(2 * ci + 1) * T + t]);
                 const float xl = x.mt[(size_t)(2 * ci) * T + t - 1];
                 ml_p = ci >= 1 ? to_b2(xl) : NEG_INF_F;
@@ -360,8 +473,8 @@ __device__ __forceinline__ void bwd_sweep(const float (&A0)[R][8 * R], const flo
             sum = row8_sum(sum);
             const float beta = (mx == NEG_INF_F || !live) ? NEG_INF_F : mx + lg2(sum);
             // outside weights this node offers to its children at the next two positions
-            const float nw0 = mc_t + beta;
-            const float nw1 = (ml_p + mc_t) + bprev[r];
+            const float nw0 = (mc_t + beta) - d_next;
+            const float nw1 = ((ml_p + mc_t) + bprev[r]) - d_both;
             bprev[r] = beta;
             if (j == 0) {
                 n0[c_id] = nw0;
@@ -378,8 +491,8 @@ __device__ __forceinline__ void bwd_sweep(const float (&A0)[R][8 * R], const flo
 
 // Backward: outside sweep t = 1 .. n-1 (one 8-lane group per child node c, lanes strided over parents a <= c), rule
 // posteriors accumulated in registers, then the element-wise emission epilogue.
-// Dynamic LDS: w0[2][MP], w1[2][MP]; with TAB_LDS also S, F0, F1, BETA [Mc][T+2] and the emissions of main nodes and
-// leaves [Mc][T], all base 2: sweep and epilogue then read no global memory.
+// Dynamic LDS: head (see LdsHead), w0[2][MP], w1[2][MP]; with TAB_LDS also R, F0h, F1h, Bh [Mc][T+2] and the emissions of
+// main nodes and leaves [Mc][T], all base 2: sweep and epilogue then read no global memory.
 template <int R, bool TAB_LDS>
 __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
                                                             float *__restrict__ aux, const float *__restrict__ match_all,
@@ -390,9 +503,10 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
     constexpr int MP = 64 * R;
     const int TS = T + 2;
     extern __shared__ float smem[];
-    float *w0 = smem;            // [2][MP]
-    float *w1 = smem + 2 * MP;    // [2][MP]
-    float *sm_S = smem + 4 * MP;  // [Mc][TS]   (TAB_LDS)
+    LdsHead hd(smem, T);
+    float *w0 = hd.rest;         // [2][MP]
+    float *w1 = w0 + 2 * MP;      // [2][MP]
+    float *sm_S = w0 + 4 * MP;    // [Mc][TS]   (TAB_LDS)
     float *sm_F0 = sm_S + (TAB_LDS ? Mc * TS : 0);
     float *sm_F1 = sm_F0 + (TAB_LDS ? Mc * TS : 0);
     float *sm_B = sm_F1 + (TAB_LDS ? Mc * TS : 0);
@@ -455,12 +569,13 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
             sm_leaf[i] = (ok && a_id >= 1) ? to_b2(vl) : NEG_INF_F;
         }
         for (int i = tid; i < Mc * TS; i += NTR) {
-            sm_S[i] = Sb[i] * LOG2E_F;
+            sm_S[i] = av.SR[i];
             sm_F0[i] = av.F0[i];
             sm_F1[i] = av.F1[i];
             sm_B[i] = NEG_INF_F;
         }
     }
+    for (int i = tid; i < TS + 2; i += NTR) hd.D[i] = av.D[i];
 #pragma unroll
     for (int r = 0; r < R; r++) {
         const int c_id = 64 * r + 8 * p + g8;
@@ -485,7 +600,7 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
     auto f1_at = [&](int a_id, int s) -> float { return TAB_LDS ? sm_F1[a_id * TS + s] : av.F1[(size_t)a_id * TS + s]; };
     auto beta_at = [&](int a_id, int s) -> float { return TAB_LDS ? sm_B[a_id * TS + s] : av.BETA[(size_t)a_id * TS + s]; };
 
-    const float beta00 = -ll * LOG2E_F;  // outside score of (root, 0) for a unit upstream gradient
+    const float beta00 = -av.SR[0];  // outside score of (root, 0), relative to the offset of column 0
     for (int i = tid; i < MP; i += NTR) {
         w0[1 * MP + i] = NEG_INF_F;
         w1[1 * MP + i] = NEG_INF_F;
@@ -494,12 +609,12 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
         for (int i = tid; i < mc; i += NTR) av.BETA[(size_t)i * TS] = (i == 0) ? beta00 : NEG_INF_F;
     __syncthreads();
     if (tid == 0) {
-        w0[1 * MP + 0] = match_main(0, 0) + beta00;
+        w0[1 * MP + 0] = (match_main(0, 0) + beta00) - hd.D[1];
         if (TAB_LDS) sm_B[0] = beta00;
     }
     __syncthreads();
     PCFGNAT_PHASE(9);
-    BwdSweepArgs sa{w0, w1, sm_S, sm_B, sm_main, sm_leaf, mt, Sb, av.BETA, beta00, n, mc, Mc, T, j, g8};
+    BwdSweepArgs sa{w0, w1, sm_S, sm_B, sm_main, sm_leaf, mt, av.SR, av.BETA, hd.D, beta00, n, mc, Mc, T, j, g8};
     switch (p) {  // wave-uniform
         case 0: bwd_sweep<R, TAB_LDS, 0>(A0, A1, G0, G1, sa); break;
         case 1: bwd_sweep<R, TAB_LDS, 1>(A0, A1, G0, G1, sa); break;
@@ -539,10 +654,10 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
                 const float mas = match_main(a_id, s);
                 if (s + 1 <= n - 1) out += ex2(bs + mas + f0_at(a_id, s + 1));  // a emits s with the null left child
                 if (s >= 1 && s + 1 <= n - 1 && a_id >= 1)                      // a emits s after its leaf emitted s-1
-                    out += ex2(beta_at(a_id, s - 1) + match_leaf(a_id, s - 1) + mas + f1_at(a_id, s + 1));
+                    out += ex2(beta_at(a_id, s - 1) + match_leaf(a_id, s - 1) + mas + (f1_at(a_id, s + 1) - hd.D[s]));
                 if (a_id == mc - 1 && s == n - 1) out += ex2(bs + mas);        // base cell
             } else if (a_id >= 1 && a_id < mc && s + 2 <= n - 1) {             // leaf of parent a = x+1
-                out += ex2(beta_at(a_id, s) + match_leaf(a_id, s) + match_main(a_id, s + 1) + f1_at(a_id, s + 2));
+                out += ex2(beta_at(a_id, s) + match_leaf(a_id, s) + match_main(a_id, s + 1) + (f1_at(a_id, s + 2) - hd.D[s + 1]));
             }
             if (!(out == out)) out = 0.f;
         }
@@ -553,8 +668,8 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
 
 // Forward and backward in one launch (used by the single-call criterion step when every table fits in LDS): the
 // tables the backward needs (S, F0, F1, emissions) never leave LDS, only S is also written to global memory in the
-// reference's layout.  Dynamic LDS: w0[2][MP] (doubles as the forward's S columns), w1[2][MP], S/F0/F1/BETA [Mc][T+2],
-// emissions of main nodes and leaves [Mc][T].
+// reference's layout.  Dynamic LDS: head (see LdsHead), w0[2][MP] (doubles as the forward's columns), w1[2][MP],
+// R/F0h/F1h/Bh [Mc][T+2], emissions of main nodes and leaves [Mc][T].
 template <int R>
 __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__restrict__ grad_out, const float *__restrict__ match_all,
                                                               const float *__restrict__ links, const int64_t *__restrict__ out_len,
@@ -565,9 +680,10 @@ __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__re
     constexpr int MP = 64 * R;
     const int TS = T + 2;
     extern __shared__ float smem[];
-    float *w0 = smem;            // [2][MP]
-    float *w1 = smem + 2 * MP;    // [2][MP]
-    float *sm_S = smem + 4 * MP;  // [Mc][TS]
+    LdsHead hd(smem, T);
+    float *w0 = hd.rest;         // [2][MP]
+    float *w1 = w0 + 2 * MP;      // [2][MP]
+    float *sm_S = w0 + 4 * MP;    // [Mc][TS]
     float *sm_F0 = sm_S + Mc * TS;
     float *sm_F1 = sm_F0 + Mc * TS;
     float *sm_B = sm_F1 + Mc * TS;
@@ -627,6 +743,11 @@ __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__re
         sm_B[i] = NEG_INF_F;
     }
     for (int i = tid; i < MP; i += NTR) w0[((n - 1) & 1) * MP + i] = (i == mc - 1) ? base_cell * LOG2E_F : NEG_INF_F;
+    for (int i = tid; i < TS + 2; i += NTR) {
+        hd.D[i] = 0.f;
+        if (i < TS) hd.O[i] = 0.0;
+    }
+    if (tid < 16) hd.slots[tid] = base_cell * LOG2E_F;
 #pragma unroll
     for (int r = 0; r < R; r++) {
         const int a_id = 64 * r + 8 * p + g8;
@@ -640,7 +761,7 @@ __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__re
     }
     __syncthreads();
     {
-        FwdSweepArgs sa{w0, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, nullptr, nullptr, n, mc, Mc, T, j, g8};
+        FwdSweepArgs sa{w0, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, nullptr, nullptr, nullptr, hd.slots, hd.D, hd.O, base_cell * LOG2E_F, n, mc, Mc, T, j, g8};
         switch (p) {
             case 0: fwd_sweep<R, true, 0>(A0, A1, sa); break;
             case 1: fwd_sweep<R, true, 1>(A0, A1, sa); break;
@@ -663,8 +784,11 @@ __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__re
             A1[r][q] = lk[(row + 1) * L + c];
         }
     }
-    for (int i = tid; i < Mc * TS; i += NTR) Sb[i] = sm_S[i] * LN2_F;
-    const float ll2 = sm_S[0];  // base 2
+    for (int i = tid; i < Mc * TS; i += NTR) {
+        const int t = i - (i / TS) * TS;
+        Sb[i] = (float)(((double)sm_S[i] + hd.O[t]) * LN2_D);
+    }
+    const float ll2 = sm_S[0];  // base 2, relative to the offset of column 0
     const bool valid = (ll2 == ll2) && (fabsf(ll2) != __builtin_huge_valf());
     if (!valid) {  // workgroup-uniform
         for (int i = tid; i < L * T; i += NTR) mg[i] = 0.f;
@@ -686,13 +810,13 @@ __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__re
     }
     const float beta00 = -ll2;
     for (int i = tid; i < MP; i += NTR) {
-        w0[1 * MP + i] = (i == 0) ? sm_main[0] + beta00 : NEG_INF_F;
+        w0[1 * MP + i] = (i == 0) ? (sm_main[0] + beta00) - hd.D[1] : NEG_INF_F;
         w1[1 * MP + i] = NEG_INF_F;
     }
     if (tid == 0) sm_B[0] = beta00;
     __syncthreads();
     {
-        BwdSweepArgs sa{w0, w1, sm_S, sm_B, sm_main, sm_leaf, mt, Sb, nullptr, beta00, n, mc, Mc, T, j, g8};
+        BwdSweepArgs sa{w0, w1, sm_S, sm_B, sm_main, sm_leaf, mt, nullptr, nullptr, hd.D, beta00, n, mc, Mc, T, j, g8};
         switch (p) {
             case 0: bwd_sweep<R, true, 0>(A0, A1, G0, G1, sa); break;
             case 1: bwd_sweep<R, true, 1>(A0, A1, G0, G1, sa); break;
@@ -727,10 +851,11 @@ __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__re
                 const float mas = sm_main[a_id * T + s];
                 if (s + 1 <= n - 1) out += ex2(bs + mas + sm_F0[a_id * TS + s + 1]);
                 if (s >= 1 && s + 1 <= n - 1 && a_id >= 1)
-                    out += ex2(sm_B[a_id * TS + s - 1] + sm_leaf[a_id * T + s - 1] + mas + sm_F1[a_id * TS + s + 1]);
+                    out += ex2(sm_B[a_id * TS + s - 1] + sm_leaf[a_id * T + s - 1] + mas + (sm_F1[a_id * TS + s + 1] - hd.D[s]));
                 if (a_id == mc - 1 && s == n - 1) out += ex2(bs + mas);
             } else if (a_id >= 1 && a_id < mc && s + 2 <= n - 1) {
-                out += ex2(sm_B[a_id * TS + s] + sm_leaf[a_id * T + s] + sm_main[a_id * T + s + 1] + sm_F1[a_id * TS + s + 2]);
+                out += ex2(sm_B[a_id * TS + s] + sm_leaf[a_id * T + s] + sm_main[a_id * T + s + 1] +
+                           (sm_F1[a_id * TS + s + 2] - hd.D[s + 1]));
             }
             if (!(out == out)) out = 0.f;
         }
@@ -808,19 +933,25 @@ __global__ __launch_bounds__(64) void best_tree_ml1_kernel(const float *__restri
 // so that lanes read consecutive parents), rows are processed in tiles of 64, and the row reductions are online
 // log-sum-exps over chunks of children.  Rule posteriors are produced by a separate, fully parallel kernel from the
 // outside weights the sweep leaves behind.
-// Aux layout per sentence (Mc > 128): F0, F1, BETA, W0, W1 [Mc][T+2] each, then At [2][Mc][Mc].
+// All tables are relative to the column offsets described at the top of this file (natural logarithms here).
+// Aux layout per sentence (Mc > 128): F0h, F1h, Bh, W0, W1, R [Mc][T+2] each, D [T+4], then At [2][Mc][Mc].
 // ------------------------------------------------------------------------------------------------------------
+__host__ __device__ inline size_t aux_stride_stream(int Mc, int T) {
+    return (size_t)6 * Mc * (T + 2) + (size_t)(T + 4) + (size_t)2 * Mc * Mc;
+}
 struct AuxViewStream {
-    float *F0, *F1, *BETA, *W0, *W1, *At;
+    float *F0, *F1, *BETA, *W0, *W1, *SR, *D, *At;
     __device__ AuxViewStream(float *aux, int b, int Mc, int T) {
         const size_t plane = (size_t)Mc * (T + 2);
-        float *base = aux + (size_t)b * (5 * plane + (size_t)2 * Mc * Mc);
+        float *base = aux + (size_t)b * aux_stride_stream(Mc, T);
         F0 = base;
         F1 = base + plane;
         BETA = base + 2 * plane;
         W0 = base + 3 * plane;
         W1 = base + 4 * plane;
-        At = base + 5 * plane;
+        SR = base + 5 * plane;
+        D = base + 6 * plane;
+        At = D + (T + 4);
     }
 };
 
@@ -845,7 +976,8 @@ struct OnlineLse {
     }
 };
 
-// Dynamic LDS: col[2][MP], f1prev[MP], then (if MATCH_LDS) match main [Mc][T], match leaf [Mc][T].
+// Dynamic LDS: col[2][MP], f1prev[MP], per-wave column maxima slots[2][16], then (if MATCH_LDS) match main [Mc][T],
+// match leaf [Mc][T].
 template <bool MATCH_LDS>
 __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
                                                                   const int64_t *__restrict__ out_len,
@@ -854,7 +986,8 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
     extern __shared__ float smem[];
     float *col = smem;               // [2][MP]
     float *f1prev = smem + 2 * MP;    // [MP]
-    float *sm_main = smem + 3 * MP;   // [Mc][T]
+    float *slots = smem + 3 * MP;     // [2][16]
+    float *sm_main = slots + 32;      // [Mc][T]
     float *sm_leaf = sm_main + (MATCH_LDS ? Mc * T : 0);
 
     const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
@@ -883,20 +1016,29 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
             float v = NEG_INF_F;
             if (a_id == mc - 1 && s == n - 1) v = sanitize(mt[(size_t)(m - 1) * T + (n - 1)]);
             Sb[i] = v;
+            av.SR[i] = v;
         }
     }
+    const float base_cell = sanitize(mt[(size_t)(m - 1) * T + (n - 1)]);
     for (int i = tid; i < MP; i += NT) {
-        col[((n - 1) & 1) * MP + i] = (i == mc - 1) ? sanitize(mt[(size_t)(m - 1) * T + (n - 1)]) : NEG_INF_F;
+        col[((n - 1) & 1) * MP + i] = (i == mc - 1) ? base_cell : NEG_INF_F;
         col[((n - 2) & 1) * MP + i] = NEG_INF_F;
         f1prev[i] = NEG_INF_F;
     }
+    if (tid < 32) slots[tid] = base_cell;  // maximum of column n-1
+    for (int i = tid; i < T + 4; i += NT) av.D[i] = 0.f;
     __syncthreads();
 
     const int ntiles = (mc + 63) / 64;
     const int nq = (mc + 15) / 16;
+    double O = 0.0;  // offset of the column being read
     for (int t = n - 1; t >= 1; t--) {
         const float *cur = col + (t & 1) * MP;
         float *nxt = col + ((t - 1) & 1) * MP;
+        const float D = fmaxf(max8(slots + (t & 1) * 16), max8(slots + (t & 1) * 16 + 8));
+        const float Ds = (D == NEG_INF_F) ? 0.f : D;
+        const double O_new = O + (double)Ds;
+        float wmax = NEG_INF_F;
         for (int tile = 0; tile < ntiles; tile++) {
             const int a_id = tile * 64 + gidx, a = 2 * a_id + 1;
             const bool row_ok = a_id < mc;
@@ -930,22 +1072,33 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
                 acc0.add4(v0);
                 acc1.add4(v1);
             }
-            const float F0 = acc0.finish16();
-            const float F1 = acc1.finish16();
+            const float F0 = acc0.finish16() - Ds;
+            const float F1 = acc1.finish16() - Ds;
             const int ai = (a_id < MP) ? a_id : 0;
             const float f1p = f1prev[ai];
-            float s_new = lse2(ma_p + F0, (ml_p + ma_t) + f1p);
+            float s_new = lse2(ma_p + F0, (ml_p + ma_t) + (f1p - Ds));
             if (!row_ok) s_new = NEG_INF_F;
+            wmax = fmaxf(wmax, s_new);
             if (j == 0 && a_id < MP) {
                 nxt[a_id] = s_new;
                 f1prev[a_id] = F1;
                 if (row_ok) {
-                    Sb[(size_t)a_id * (T + 2) + (t - 1)] = s_new;
+                    Sb[(size_t)a_id * (T + 2) + (t - 1)] = (float)((double)s_new + O_new);
+                    av.SR[(size_t)a_id * (T + 2) + (t - 1)] = s_new;
                     av.F0[(size_t)a_id * (T + 2) + t] = F0;
                     av.F1[(size_t)a_id * (T + 2) + t] = F1;
                 }
             }
         }
+        {   // s_new is uniform inside each 16-lane row: combine the four rows of the wave
+            const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wmax), 0));
+            const float bq = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wmax), 16));
+            const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wmax), 32));
+            const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wmax), 48));
+            if ((tid & 63) == 0) slots[((t - 1) & 1) * 16 + (tid >> 6)] = fmaxf(fmaxf(a, bq), fmaxf(c, d));
+        }
+        if (tid == 0) av.D[t] = Ds;
+        O = O_new;
         lds_barrier();
     }
 }
@@ -978,7 +1131,7 @@ __global__ __launch_bounds__(256) void transpose_links_ml1_kernel(const float *_
     }
 }
 
-// Outside sweep.  Dynamic LDS: w0[2][MP], w1[2][MP], bprev[MP], then (if MATCH_LDS) match main/leaf [Mc][T] each.
+// Outside sweep.  Dynamic LDS: w0[2][MP], w1[2][MP], bprev[MP], D[T+4], then (if MATCH_LDS) match main/leaf [Mc][T] each.
 template <bool MATCH_LDS>
 __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *__restrict__ S, float *__restrict__ aux,
                                                                   const float *__restrict__ match_all,
@@ -988,7 +1141,8 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
     float *w0 = smem;             // [2][MP]
     float *w1 = smem + 2 * MP;     // [2][MP]
     float *bprev = smem + 4 * MP;  // [MP]
-    float *sm_main = smem + 5 * MP;
+    float *sm_D = smem + 5 * MP;   // [T+4]
+    float *sm_main = sm_D + (T + 4);
     float *sm_leaf = sm_main + (MATCH_LDS ? Mc * T : 0);
 
     const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
@@ -1007,8 +1161,9 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
             sm_main[i] = ok ? sanitize(mt[(size_t)(2 * a_id + 1) * T + s]) : NEG_INF_F;
             sm_leaf[i] = (ok && a_id >= 1) ? sanitize(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
         }
-        __syncthreads();
     }
+    for (int i = tid; i < T + 4; i += NT) sm_D[i] = av.D[i];
+    __syncthreads();
     auto match_main = [&](int a_id, int s) -> float {
         if (MATCH_LDS) return sm_main[a_id * T + s];
         return sanitize(mt[(size_t)(2 * a_id + 1) * T + s]);
@@ -1017,8 +1172,8 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
         if (MATCH_LDS) return sm_leaf[a_id * T + s];
         return a_id >= 1 ? sanitize(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
     };
-    const float beta00 = -ll;
-    const float w00 = match_main(0, 0) + beta00;
+    const float beta00 = -av.SR[0];  // relative to the offset of column 0
+    const float w00 = (match_main(0, 0) + beta00) - sm_D[1];
     for (int i = tid; i < MP; i += NT) {
         w0[1 * MP + i] = (i == 0) ? w00 : NEG_INF_F;
         w1[1 * MP + i] = NEG_INF_F;
@@ -1037,6 +1192,7 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
     for (int t = 1; t <= n - 1; t++) {
         const float *c0 = w0 + (t & 1) * MP, *c1 = w1 + (t & 1) * MP;
         float *n0 = w0 + ((t + 1) & 1) * MP, *n1 = w1 + ((t + 1) & 1) * MP;
+        const float d_next = sm_D[t + 1], d_both = d_next + sm_D[t];
         for (int tile = 0; tile < ntiles; tile++) {
             const int c_id = tile * 64 + gidx;
             const bool live = c_id < mc;
@@ -1066,8 +1222,8 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
             if (!live) beta = NEG_INF_F;
             const int cs = (c_id < MP) ? c_id : 0;
             const float bp = bprev[cs];
-            const float nw0 = mc_t + beta;
-            const float nw1 = (ml_p + mc_t) + bp;
+            const float nw0 = (mc_t + beta) - d_next;
+            const float nw1 = ((ml_p + mc_t) + bp) - d_both;
             if (j == 0 && c_id < MP) {
                 n0[c_id] = nw0;
                 n1[c_id] = nw1;
@@ -1083,7 +1239,7 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
     }
 }
 
-// Rule posteriors from the outside weights: lg[a][k][c] = g * sum_{t=1}^{n-1} exp(links[a][k][c] + Wk[a][t] + S[c][t]).
+// Rule posteriors from the outside weights: lg[a][k][c] = g * sum_{t=1}^{n-1} exp(links[a][k][c] + Wk[a][t] + R[c][t]).
 // One block per 32x32 tile of (parent, child) pairs; the slab has been zero-filled beforehand.
 __global__ __launch_bounds__(1024) void links_grad_ml1_stream_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
                                                                     const float *__restrict__ aux_c, const float *__restrict__ links,
@@ -1116,7 +1272,7 @@ __global__ __launch_bounds__(1024) void links_grad_ml1_stream_kernel(const float
         const bool tin = tt <= n - 1;
         sw0[ty][tx] = (tin && ra < mc) ? av.W0[(size_t)ra * (T + 2) + tt] : NEG_INF_F;
         sw1[ty][tx] = (tin && ra < mc) ? av.W1[(size_t)ra * (T + 2) + tt] : NEG_INF_F;
-        ss[ty][tx] = (tin && rc < mc) ? Sb[(size_t)rc * (T + 2) + tt] : NEG_INF_F;
+        ss[ty][tx] = (tin && rc < mc) ? av.SR[(size_t)rc * (T + 2) + tt] : NEG_INF_F;
         __syncthreads();
 #pragma unroll 8
         for (int u = 0; u < 32; u++) {
@@ -1164,11 +1320,11 @@ __global__ __launch_bounds__(256) void match_grad_ml1_stream_kernel(const float 
             const float mas = sanitize(mt[(size_t)x * T + s]);
             if (s + 1 <= n - 1) out += __expf(bs + mas + av.F0[row + s + 1]);
             if (s >= 1 && s + 1 <= n - 1 && a_id >= 1)
-                out += __expf(av.BETA[row + s - 1] + sanitize(mt[(size_t)(x - 1) * T + s - 1]) + mas + av.F1[row + s + 1]);
+                out += __expf(av.BETA[row + s - 1] + sanitize(mt[(size_t)(x - 1) * T + s - 1]) + mas + (av.F1[row + s + 1] - av.D[s]));
             if (a_id == mc - 1 && s == n - 1) out += __expf(bs + mas);
         } else if (a_id >= 1 && a_id < mc && s + 2 <= n - 1) {
             out += __expf(av.BETA[row + s] + sanitize(mt[(size_t)x * T + s]) + sanitize(mt[(size_t)(x + 1) * T + s + 1]) +
-                          av.F1[row + s + 2]);
+                          (av.F1[row + s + 2] - av.D[s + 1]));
         }
         if (!(out == out)) out = 0.f;
     }
@@ -1212,7 +1368,7 @@ __global__ __launch_bounds__(256) void criterion_loss_kernel(const float *__rest
 int launch_fwd_stream(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B,
                       int L, int T, int Mc, hipStream_t stream) {
     const int MP = ((Mc + 63) / 64) * 64;
-    const size_t base = (size_t)3 * MP * sizeof(float);
+    const size_t base = ((size_t)3 * MP + 32) * sizeof(float);
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
     if (with_match <= LDS_BUDGET) {
         auto k = inside_fwd_ml1_stream_kernel<true>;
@@ -1232,7 +1388,7 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
     const int tiles = (Mc + 31) / 32;
     hipLaunchKernelGGL(transpose_links_ml1_kernel, dim3(tiles, tiles, B), dim3(256), 0, stream, links, ol, aux, L, T, Mc);
     PCFGNAT_HIP_CHECK(hipGetLastError());
-    const size_t base = (size_t)5 * MP * sizeof(float);
+    const size_t base = ((size_t)5 * MP + T + 4) * sizeof(float);
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
     if (with_match <= LDS_BUDGET) {
         auto k = inside_bwd_ml1_stream_kernel<true>;
@@ -1256,14 +1412,17 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
 template <int R>
 int launch_fwd(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B, int L,
                int T, int Mc, hipStream_t stream) {
-    const size_t base = (size_t)2 * 64 * R * sizeof(float);
+    const size_t base = ((size_t)head_floats(T) + 2 * 64 * R) * sizeof(float);
     const size_t with_tab = base + ((size_t)2 * Mc * T + (size_t)3 * Mc * (T + 2)) * sizeof(float);
     if (with_tab <= LDS_BUDGET) {
         auto k = inside_fwd_ml1_kernel<R, true>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_tab));
         hipLaunchKernelGGL(k, dim3(B), dim3(NTR), with_tab, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
     } else {
-        hipLaunchKernelGGL((inside_fwd_ml1_kernel<R, false>), dim3(B), dim3(NTR), base, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
+        auto k = inside_fwd_ml1_kernel<R, false>;
+        PCFGNAT_REQUIRE(base <= LDS_BUDGET, "pcfg_loss: target length %d too large for the column offsets in LDS", T);
+        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)base));
+        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), base, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
@@ -1272,15 +1431,17 @@ int launch_fwd(const float *match_all, const float *links, const int64_t *ol, co
 template <int R>
 int launch_bwd(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
                const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream) {
-    const size_t base = (size_t)4 * 64 * R * sizeof(float);
+    const size_t base = ((size_t)head_floats(T) + 4 * 64 * R) * sizeof(float);
     const size_t with_tab = base + ((size_t)2 * Mc * T + (size_t)4 * Mc * (T + 2)) * sizeof(float);
     if (with_tab <= LDS_BUDGET) {
         auto k = inside_bwd_ml1_kernel<R, true>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_tab));
         hipLaunchKernelGGL(k, dim3(B), dim3(NTR), with_tab, stream, go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc, norm_B);
     } else {
-        hipLaunchKernelGGL((inside_bwd_ml1_kernel<R, false>), dim3(B), dim3(NTR), base, stream, go, S, aux, match_all, links, ol, tl, mg,
-                           lg, L, T, Mc, norm_B);
+        auto k = inside_bwd_ml1_kernel<R, false>;
+        PCFGNAT_REQUIRE(base <= LDS_BUDGET, "pcfg_loss_backward: target length %d too large for the column offsets in LDS", T);
+        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)base));
+        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), base, stream, go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc, norm_B);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
@@ -1290,7 +1451,7 @@ int launch_bwd(const float *go, const float *S, float *aux, const float *match_a
 template <int R>
 int launch_fused(const float *go, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *mg,
                  float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream, bool *done) {
-    const size_t need = ((size_t)4 * 64 * R + (size_t)4 * Mc * (T + 2) + (size_t)2 * Mc * T) * sizeof(float);
+    const size_t need = ((size_t)head_floats(T) + 4 * 64 * R + (size_t)4 * Mc * (T + 2) + (size_t)2 * Mc * T) * sizeof(float);
     *done = false;
     if (need > LDS_BUDGET) return PCFGNAT_OK;
     auto k = inside_fused_ml1_kernel<R>;
@@ -1320,8 +1481,8 @@ extern "C" size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64
     if (B <= 0 || L < 2 || T < 0 || ml < 0) return 0;
     if (ml != 1) return generic_aux_floats(B, L, T, ml);
     const int64_t Mc = (L - 2) / (ml + 1) + 1;
-    if (Mc <= 128) return (size_t)B * 3 * Mc * (T + 2);
-    return (size_t)B * ((size_t)5 * Mc * (T + 2) + (size_t)2 * Mc * Mc);
+    if (Mc <= 128) return (size_t)B * aux_stride_reg((int)Mc, (int)T);
+    return (size_t)B * aux_stride_stream((int)Mc, (int)T);
 }
 
 extern "C" int pcfgnat_pcfg_loss(const float *match_all, const float *links, const int64_t *output_length,

@@ -79,9 +79,10 @@ def test_config2_full_size():
 
 
 def test_config3_full_size():
-    # 139 sequential steps on table entries of magnitude ~1.8e3, where fp32 spacing is 1.2e-4: a sequential fp32 evaluation
-    # (the oracle's float instantiation, which follows the reference) is itself 1.3e-4 .. 1.5e-4 away from float64 here
-    _check_training_batch(synth.config3(), sample=[3], grad_tol=5e-4)
+    # table entries reach ~1.8e3 here, where fp32 spacing is 1.2e-4: a plain sequential fp32 evaluation (the oracle's float
+    # instantiation, which follows the reference) is 1.3e-4 .. 1.5e-4 away from float64; the kernels keep the tables
+    # relative to per-column offsets and stay within the same 1e-4 as at the short lengths
+    _check_training_batch(synth.config3(), sample=[3])
 
 
 def test_config5_glat_alignment():
