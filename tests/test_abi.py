@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
         assert name in _lib.SIGNATURES, "binding table lacks %s" % name
     assert sorted(_lib.SIGNATURES) == names
     assert lib.pcfgnat_abi_version() == 1
-    assert lib.pcfgnat_pcfg_aux_floats(40, 128, 32, 1) == 40 * 3 * 64 * 34
+    assert lib.pcfgnat_pcfg_aux_floats(40, 128, 32, 1) == 40 * (4 * 64 * 34 + 36)
 
 
 def test_argument_errors_without_gpu():
