@@ -1,13 +1,13 @@
 """Benchmark of the structured-loss hot path on one MI355X.
 
 A step is one training pass over one WMT14 En-De shaped batch (B=40, L=128, T=32, V=40000, fp16 logits):
-logsoftmax_gather (writes softmax in place) -> eos mask -> inside forward + backward -> loss -> logsoftmax_gather
-backward (in place), exactly the native calls autograd issues for the criterion.  Inputs are resident in HBM before the
-timed region; each step consumes a fresh logits buffer because the path overwrites it.
+logsoftmax_gather -> eos mask -> inside forward + backward -> loss -> logsoftmax_gather backward (in place), the work
+autograd performs for the criterion.  Inputs are resident in HBM before the timed region; each step consumes a fresh
+logits buffer because the path overwrites it with the gradient.
 
-Prints one JSON line: whole-job throughput in sentences/s, the HBM roofline of the dominant kernel
-(logsoftmax_gather forward) from HIP events recorded around it inside the timed region, and the CPU oracle timed on the
-host cores over a bounded sample of the same batch.
+Prints one JSON line: whole-job throughput in sentences/s, the HBM roofline of the dominant kernel (the in-place
+logsoftmax_gather backward: logits read, gradient written) from HIP events recorded around it inside the timed region,
+and the CPU oracle timed on the host cores over a bounded sample of the same batch.
 """
 import argparse
 import json
@@ -20,9 +20,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
-# HBM bytes per launch of lsg_fwd_kernel<half, grad> at this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled against
-# a plain device copy of known size (FETCH x1.99989, WRITE x1.0); summary in profiles/lsg_cfg2_hbm_traffic_pmc.md
-LSG_FWD_MEASURED_TRAFFIC_BYTES = 820.75e6
+# HBM bytes per launch of the roofline kernel at this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled against a
+# plain device copy of known size; summary in profiles/lsg_cfg2_hbm_traffic_pmc.md.  None = not measured for this build.
+ROOFLINE_KERNEL = {"single": "lsg_bwd", "fused": "lsg_bwd", "unfused": "lsg_fwd"}
+ROOFLINE_KERNEL_NAME = {"lsg_bwd": "lsg_bwd_kernel<half, from logits>", "lsg_fwd": "lsg_fwd_kernel<half, grad>"}
+MEASURED_TRAFFIC_BYTES = {"lsg_bwd": None, "lsg_fwd": 820.75e6}
 
 
 def parse():
@@ -159,13 +161,15 @@ def main():
     pairs = {}
 
     detail = {"on": False}  # timed region: events around the roofline kernel only; afterwards: around all four
+    mode = "unfused" if args.unfused else args.step
+    roof = ROOFLINE_KERNEL[mode]
 
     def mark(name, phase):
         if name == "events":  # single-call step: the library records the events we hand out around its kernels
             evs = []
             for kernel in ("lsg_fwd", "inside_fwd", "inside_bwd", "lsg_bwd"):
                 for _ in range(2):
-                    if kernel != "lsg_fwd" and not detail["on"]:
+                    if kernel != roof and not detail["on"]:
                         evs.append(None)
                         continue
                     ev = torch.cuda.Event(enable_timing=True)
@@ -173,13 +177,12 @@ def main():
                     pairs.setdefault(kernel, []).append(ev)
                     evs.append(ev)
             return evs
-        if name != "lsg_fwd" and not detail["on"]:
+        if name != roof and not detail["on"]:
             return
         ev = torch.cuda.Event(enable_timing=True)
         ev.record()
         pairs.setdefault(name, []).append(ev)
 
-    mode = "unfused" if args.unfused else args.step
     if mode == "single":
         def step_fn(*a, **kw):
             return harness.train_step_single_call(*a, slices=args.slices, **kw)
@@ -207,19 +210,25 @@ def main():
             out[name] = sum(d) / len(d)
         return out
 
-    kern_ms = averages()  # lsg_fwd only: measured inside the timed region
-    # per-kernel detail from a separate instrumented pass over buffers that have already been consumed (same work)
-    lsg_in_region = kern_ms["lsg_fwd"]
+    kern_ms = averages()  # the roofline kernel only: measured inside the timed region
+    # per-kernel detail from a separate instrumented pass over buffers that have already been consumed (same work:
+    # every value is finite, the kernels do not branch on data)
+    roof_in_region = kern_ms[roof]
     pairs.clear()
     detail["on"] = True
     for i in range(min(5, total)):
         step_fn(bufs[i], targets, links, ol, tl, mark=mark)
     torch.cuda.synchronize()
     kern_ms = averages()
-    kern_ms["lsg_fwd"] = lsg_in_region
-    fwd_bytes = synth.lsg_fwd_bytes(B_timed, L, V, T, 2, True)
-    achieved = fwd_bytes / (kern_ms["lsg_fwd"] * 1e-3) / 1e9
-    bwd_achieved = synth.lsg_bwd_bytes(B_timed, L, V, T, 2) / (kern_ms["lsg_bwd"] * 1e-3) / 1e9
+    kern_ms[roof] = roof_in_region
+    if mode == "single":  # the library runs the inside forward and backward as one launch, bracketed by the third pair
+        kern_ms.pop("inside_fwd", None)
+        kern_ms["inside_fwd_bwd"] = kern_ms.pop("inside_bwd")
+    fwd_bytes = synth.lsg_fwd_bytes(B_timed, L, V, T, 2, require_grad=(mode == "unfused"))
+    bwd_bytes = synth.lsg_bwd_bytes(B_timed, L, V, T, 2)
+    roof_bytes = bwd_bytes if roof == "lsg_bwd" else fwd_bytes
+    achieved = roof_bytes / (kern_ms[roof] * 1e-3) / 1e9
+    traffic = MEASURED_TRAFFIC_BYTES[roof]
 
     result = {
         "metric": "inside fwd+bwd sentences/s at B=40,L=128,T=32,V=40k; Viterbi ms/sentence",
@@ -236,17 +245,21 @@ def main():
         "data": "synthetic",
         "config": {"workload": "WMT14 En-De shaped training batch (BASELINE config 2): B=40, L=128, T=32, V=40000, "
                                "fp16 logits ~N(0,2), src ~U[10,32] x4, max_left=1; logsoftmax_gather fwd -> eos mask -> "
-                               "inside fwd+bwd -> loss -> logsoftmax_gather bwd; criterion glue "
+                               "inside fwd+bwd -> loss -> logsoftmax_gather bwd (%s); criterion glue "
+                               % ("forward overwrites the logits with softmax, four passes over the logits" if mode == "unfused"
+                                  else "forward read-only, backward recomputes softmax from row log-sum-exps, three passes "
+                                       "over the logits")
                                + ("as separate torch ops" if args.unfused else "folded into the kernels, %s" %
                                   ("one native call per step, %d batch slice(s) on two streams" % args.slices if args.step == "single"
                                    else "four native calls per step")),
                    "global_batch": B, "graph_nodes": L, "target_len": T, "vocab": V},
-        "roofline": {"bound": "hbm", "kernel": "lsg_fwd_kernel<half, grad>", "achieved": achieved, "peak": HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": ROOFLINE_KERNEL_NAME[roof], "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": LSG_FWD_MEASURED_TRAFFIC_BYTES * B_timed / B,
-                     "algorithmic_bytes": fwd_bytes, "avg_ms": kern_ms["lsg_fwd"], "sentences_per_launch": B_timed},
+                     "traffic": (traffic * B_timed / B) if traffic else None,
+                     "algorithmic_bytes": roof_bytes, "avg_ms": kern_ms[roof], "sentences_per_launch": B_timed},
         "kernels_ms": kern_ms,
-        "lsg_bwd_gbs": bwd_achieved,
+        "lsg_fwd_gbs": fwd_bytes / (kern_ms["lsg_fwd"] * 1e-3) / 1e9,
+        "lsg_bwd_gbs": bwd_bytes / (kern_ms["lsg_bwd"] * 1e-3) / 1e9,
     }
     if not args.no_decode:
         result["viterbi"] = decode_timing(dev)

@@ -72,6 +72,22 @@ int pcfgnat_logsoftmax_gather_backward(void *probs_inout, int dtype, const int64
                                        int64_t sl, int64_t st, const void *grad_selected, int64_t B, int64_t L,
                                        int64_t V, int64_t T, void *stream);
 
+/*
+ * The same pair with the work split differently (no counterpart in the reference, whose forward always overwrites the
+ * logits, logsoftmax_gather.cu:238-292): the forward only reads word_ins_out and also returns the log-sum-exp of every
+ * row, lse [B,L] (float32; float64 when dtype is F64); the backward turns the untouched logits into the gradient in place,
+ *   logits_inout[b,p,v] = -exp(logits[b,p,v] - lse[b,p]) * sum_s g[b,p,s];  logits_inout[b,p,idx[b,p,s]] += g[b,p,s],
+ * computed in float32 (float64) and rounded to the buffer's dtype once.  Three passes over the logits per training step
+ * instead of four.  output_length/target_length: both NULL, or the lengths for the eos mask of
+ * pcfgnat_logsoftmax_gather_eos.
+ */
+int pcfgnat_logsoftmax_gather_lse(const void *word_ins_out, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl,
+                                  int64_t st, void *selected, void *lse, const int64_t *output_length,
+                                  const int64_t *target_length, int64_t B, int64_t L, int64_t V, int64_t T, void *stream);
+int pcfgnat_logsoftmax_gather_backward_lse(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb,
+                                           int64_t sl, int64_t st, const void *grad_selected, const void *lse, int64_t B,
+                                           int64_t L, int64_t V, int64_t T, void *stream);
+
 /* Number of floats of the auxiliary table the inside kernels exchange (takes the place of the reference's C
  * table, pcfg_loss.cu:394, whose content for ml = 1 is a copy of match_all). */
 size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml);
@@ -121,11 +137,11 @@ int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *
 
 /*
  * One call for the criterion's whole training pass (nat_pcfg_loss.py:98-145 plus the backward autograd derives from it):
- * logsoftmax_gather with eos mask -> inside forward -> inside backward with weights -1/(target_length*B) ->
- * logsoftmax_gather backward -> loss.  targets is the contiguous [B,T] int64 target matrix (the gather index of every
+ * logsoftmax_gather with eos mask (log-sum-exp split, see pcfgnat_logsoftmax_gather_lse) -> inside forward -> inside
+ * backward with weights -1/(target_length*B) -> logsoftmax_gather backward -> loss.  targets is the contiguous [B,T] int64 target matrix (the gather index of every
  * graph node).  On return (stream order) logits holds d loss / d logits, links_grad d loss / d links, loss_out[0] the
- * loss, loss_out[1] the number of invalid sentences; match_all, S, aux, match_all_grad are caller workspaces of the
- * shapes documented at the individual entry points.
+ * loss, loss_out[1] the number of invalid sentences; match_all, S, aux, match_all_grad and row_lse ([B,L] float32) are
+ * caller workspaces of the shapes documented at the individual entry points.
  * slices: 1 = the whole batch at once; k > 1 = the batch is processed as k slices (sentences [i*B/k, (i+1)*B/k)) that
  * alternate between `stream` and one helper stream the library keeps per device (created on first use, default
  * priority), so that the latency-bound inside kernels of one slice run beside the bandwidth-bound gather kernels of the
@@ -135,8 +151,8 @@ int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *
  */
 int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, const float *links,
                            const int64_t *output_length, const int64_t *target_length, float *match_all, float *S,
-                           float *aux, float *match_all_grad, float *links_grad, float *loss_out, int64_t B, int64_t L,
-                           int64_t V, int64_t T, int64_t ml, int64_t slices, void *stream, void *const *events);
+                           float *aux, float *match_all_grad, float *links_grad, float *row_lse, float *loss_out, int64_t B,
+                           int64_t L, int64_t V, int64_t T, int64_t ml, int64_t slices, void *stream, void *const *events);
 
 /*
  * Replaces pcfg_best_tree (pcfg_best_tree.cu:333-360): greedy top-down trace over the inside tables.

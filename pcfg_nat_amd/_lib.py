@@ -27,13 +27,15 @@ SIGNATURES = {
     "pcfgnat_logsoftmax_gather": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _int, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_logsoftmax_gather_eos": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_logsoftmax_gather_backward": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "pcfgnat_logsoftmax_gather_lse": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "pcfgnat_logsoftmax_gather_backward_lse": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_pcfg_aux_floats": (ctypes.c_size_t, [_i64, _i64, _i64, _i64]),
     "pcfgnat_pcfg_loss": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_pcfg_loss_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_pcfg_loss_forward_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_criterion_loss": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
-    "pcfgnat_criterion_step": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
-                                      _vp, _vp]),
+    "pcfgnat_criterion_step": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
+                                      _i64, _vp, _vp]),
     "pcfgnat_pcfg_best_tree": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_pcfg_viterbi": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "pcfgnat_viterbi_decoding": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),

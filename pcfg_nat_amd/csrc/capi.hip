@@ -55,13 +55,14 @@ int get_helper(DeviceHelper **out) {
 
 extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, const float *links,
                                       const int64_t *output_length, const int64_t *target_length, float *match_all, float *S,
-                                      float *aux, float *match_all_grad, float *links_grad, float *loss_out, int64_t B, int64_t L,
-                                      int64_t V, int64_t T, int64_t ml, int64_t slices, void *stream, void *const *events) {
+                                      float *aux, float *match_all_grad, float *links_grad, float *row_lse, float *loss_out, int64_t B,
+                                      int64_t L, int64_t V, int64_t T, int64_t ml, int64_t slices, void *stream,
+                                      void *const *events) {
     if (dtype != PCFGNAT_F16 && dtype != PCFGNAT_F32)
         return pcfgnat::fail(PCFGNAT_EUNSUPPORTED, "criterion_step: logits must be float16 or float32 (the PCFG kernels are float32)");
     PCFGNAT_REQUIRE(B >= 1 && L >= 4 && T >= 2 && V >= 1 && ml >= 0, "criterion_step: bad dimensions");
     PCFGNAT_REQUIRE(logits && targets && links && output_length && target_length && match_all && S && aux && match_all_grad &&
-                        links_grad && loss_out,
+                        links_grad && row_lse && loss_out,
                     "criterion_step: null pointer");
     if (slices < 1) slices = 1;
     if (slices > B) slices = B;
@@ -85,6 +86,7 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
         const float *lk_i = links + (size_t)b0 * L * (ml + 1) * L;
         float *ma_i = match_all + (size_t)b0 * L * T, *S_i = S + (size_t)b0 * Mc * (T + 2), *aux_i = aux + (size_t)b0 * aux_per_sentence;
         float *mg_i = match_all_grad + (size_t)b0 * L * T, *lkg_i = links_grad + (size_t)b0 * L * (ml + 1) * L;
+        float *lse_i = row_lse + (size_t)b0 * L;
         const bool mark = events && i == 0;  // timing events bracket the kernels of slice 0
 #define PCFGNAT_MARK(k)                                                                   \
     do {                                                                                  \
@@ -94,7 +96,7 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
         // kernels of slice i-1 rather than beside its gather
         if (i > 0) PCFGNAT_HIP_CHECK(hipStreamWaitEvent(s, h->gathered[(i - 1) & 1], 0));
         PCFGNAT_MARK(0);
-        int rc = pcfgnat_logsoftmax_gather_eos(lg_i, dtype, tg_i, T, 0, 1, ma_i, 1, ol_i, tl_i, nb, L, V, T, s);
+        int rc = pcfgnat_logsoftmax_gather_lse(lg_i, dtype, tg_i, T, 0, 1, ma_i, lse_i, ol_i, tl_i, nb, L, V, T, s);
         if (rc != PCFGNAT_OK) return rc;
         PCFGNAT_MARK(1);
         if (slices > 1) PCFGNAT_HIP_CHECK(hipEventRecord(h->gathered[i & 1], s));
@@ -105,7 +107,7 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
         if (rc != PCFGNAT_OK) return rc;
         PCFGNAT_MARK(5);
         PCFGNAT_MARK(6);
-        rc = pcfgnat_logsoftmax_gather_backward(lg_i, dtype, tg_i, T, 0, 1, mg_i, nb, L, V, T, s);
+        rc = pcfgnat_logsoftmax_gather_backward_lse(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, s);
         if (rc != PCFGNAT_OK) return rc;
         PCFGNAT_MARK(7);
 #undef PCFGNAT_MARK

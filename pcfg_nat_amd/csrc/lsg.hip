@@ -7,6 +7,13 @@
 // Design (HBM-bound, MI355X): one workgroup per row; the row is fetched once with 16-byte loads and kept in
 // registers (chunks beyond the register budget are re-streamed), so HBM sees one read and - when the gradient is
 // needed - one write per element.  Row max / sum use DPP wave reductions plus one LDS hop across waves.
+//
+// Two ways to split the work between forward and backward:
+//   * reference split: the forward overwrites the logits with softmax probabilities (read + write), the backward
+//     scales them and scatters the target gradients (read + write): four passes over the logits per training step;
+//   * log-sum-exp split: the forward only reads (and keeps one log-sum-exp per row), the backward recomputes
+//     exp(x - lse) while it writes the gradient (read + write): three passes, and the fp16 gradient is rounded once
+//     instead of twice.  The logits must stay untouched between the two calls.
 #include "common.hip.h"
 
 namespace pcfgnat {
@@ -146,7 +153,8 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
                                                      int64_t sl, int64_t st,
                                                      typename Elem<T>::compute *__restrict__ sel, int64_t rows, int L,
                                                      int V, int Tn, const int64_t *__restrict__ eos_out_len,
-                                                     const int64_t *__restrict__ eos_tgt_len) {
+                                                     const int64_t *__restrict__ eos_tgt_len,
+                                                     typename Elem<T>::compute *__restrict__ lse_out) {
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
     constexpr int NW = NT / 64;
@@ -224,6 +232,7 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
         }
         sum = block_sum<CT, NW>(sum, s_sum, wave, lane);
         const CT lg = fast_log(sum);
+        if (lse_out != nullptr && tid == 0) lse_out[row] = mx + lg;
 #pragma unroll
         for (int i = 0; i < MAXC; i++) opaque(buf[i]);
 
@@ -266,11 +275,14 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
 }
 
 // In-place backward.  TCAP = most targets per row handled through LDS; up to MAXC chunks per thread are in flight.
-template <typename T, int NT, int MAXC, int TCAP>
+// FROM_LOGITS = false: the buffer holds the probabilities the forward left (reference split, with the reference's
+// roundings to the buffer dtype); true: it holds the untouched logits and `lse` the row log-sum-exps.
+template <typename T, int NT, int MAXC, int TCAP, bool FROM_LOGITS>
 __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const int64_t *__restrict__ idx, int64_t sb,
                                                      int64_t sl, int64_t st,
                                                      const typename Elem<T>::compute *__restrict__ gsel, int64_t rows,
-                                                     int L, int V, int Tn) {
+                                                     int L, int V, int Tn,
+                                                     const typename Elem<T>::compute *__restrict__ lse) {
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
     constexpr int FIX = (TCAP + NT - 1) / NT;
@@ -298,17 +310,23 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
         CT edge = 0;
         if (ep >= 0) edge = Elem<T>::widen(pr[ep]);
 
-        // -(sum_s g) rounded to the buffer dtype (pcfg_loss.py:176), computed redundantly by every wave
+        // -(sum_s g), computed redundantly by every wave; rounded to the buffer dtype in the reference split (pcfg_loss.py:176)
         CT part = 0;
         for (int s = lane; s < Tn; s += 64) part += gr[s];
-        const CT ns = Elem<T>::widen(Elem<T>::narrow(-wave_sum(part)));
+        const CT ns = FROM_LOGITS ? -wave_sum(part) : Elem<T>::widen(Elem<T>::narrow(-wave_sum(part)));
+        const CT row_lse = FROM_LOGITS ? lse[row] : (CT)0;
 
         for (int s = tid; s < Tn; s += NT) {
             int64_t t = ir[(int64_t)s * st];
             bool ok = (uint64_t)t < (uint64_t)V;
             s_idx[s] = ok ? (int)t : -1;
-            s_g[s] = Elem<T>::widen(Elem<T>::narrow(gr[s]));
-            s_p[s] = ok ? Elem<T>::widen(pr[t]) : (CT)0;
+            if (FROM_LOGITS) {
+                s_g[s] = gr[s];
+                s_p[s] = ok ? fast_exp(Elem<T>::widen(pr[t]) - row_lse) : (CT)0;
+            } else {
+                s_g[s] = Elem<T>::widen(Elem<T>::narrow(gr[s]));
+                s_p[s] = ok ? Elem<T>::widen(pr[t]) : (CT)0;
+            }
         }
         __syncthreads();  // every original value at a target column is in LDS before any store to the row
 
@@ -319,7 +337,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
                 CT v[EPV];
                 Elem<T>::unpack(buf[i], v);
 #pragma unroll
-                for (int e = 0; e < EPV; e++) v[e] = v[e] * ns;
+                for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? fast_exp(v[e] - row_lse) : v[e]) * ns;
                 store16(pv + c, Elem<T>::pack(v));
             }
         }
@@ -327,10 +345,10 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
             CT v[EPV];
             Elem<T>::unpack(load16(pv + c), v);
 #pragma unroll
-            for (int e = 0; e < EPV; e++) v[e] = v[e] * ns;
+            for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? fast_exp(v[e] - row_lse) : v[e]) * ns;
             store16(pv + c, Elem<T>::pack(v));
         }
-        if (ep >= 0) pr[ep] = Elem<T>::narrow(edge * ns);
+        if (ep >= 0) pr[ep] = Elem<T>::narrow((FROM_LOGITS ? fast_exp(edge - row_lse) : edge) * ns);
 
         // scatter_add_ (pcfg_loss.py:177): the first occurrence of a column accumulates all its duplicates in order
         CT fix[FIX];
@@ -345,9 +363,10 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
                 bool first = true;
                 for (int u = 0; u < s; u++) first = first && (s_idx[u] != my);
                 if (first) {
-                    CT v = Elem<T>::widen(Elem<T>::narrow(s_p[s] * ns));
+                    CT v = s_p[s] * ns;
+                    if (!FROM_LOGITS) v = Elem<T>::widen(Elem<T>::narrow(v));
                     for (int u = s; u < Tn; u++)
-                        if (s_idx[u] == my) v = Elem<T>::widen(Elem<T>::narrow(v + s_g[u]));
+                        if (s_idx[u] == my) v = FROM_LOGITS ? v + s_g[u] : Elem<T>::widen(Elem<T>::narrow(v + s_g[u]));
                     fix[r] = v;
                     lead[r] = true;
                 }
@@ -367,7 +386,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
 
 template <typename T>
 int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, void *sel, int grad, int64_t rows,
-               int L, int V, int Tn, const int64_t *eos_ol, const int64_t *eos_tl, hipStream_t stream) {
+               int L, int V, int Tn, const int64_t *eos_ol, const int64_t *eos_tl, void *lse, hipStream_t stream) {
     using CT = typename Elem<T>::compute;
     constexpr int NT = 512;
     // 10 chunks x 512 threads x 16 B = 80 KB of a row in registers: a 40k-entry fp16 row exactly, half of an fp32 one.
@@ -377,25 +396,29 @@ int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
     int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
     if (grad)
         hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, true>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)x, idx, sb,
-                           sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl);
+                           sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse);
     else
         hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, false>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)x, idx,
-                           sb, sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl);
+                           sb, sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
 
 template <typename T>
 int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, const void *g, int64_t rows, int L, int V,
-               int Tn, hipStream_t stream) {
+               int Tn, const void *lse, hipStream_t stream) {
     using CT = typename Elem<T>::compute;
     constexpr int NT = 512;
     constexpr int MAXC = 10;
     constexpr int TCAP = 1024;
     if (Tn > TCAP) return fail(PCFGNAT_EUNSUPPORTED, "logsoftmax_gather_backward: T=%d exceeds %d targets per row", Tn, TCAP);
     int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
-    hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,
-                       (const CT *)g, rows, L, V, Tn);
+    if (lse != nullptr)
+        hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, true>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,
+                           (const CT *)g, rows, L, V, Tn, (const CT *)lse);
+    else
+        hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, false>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl,
+                           st, (const CT *)g, rows, L, V, Tn, (const CT *)nullptr);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -416,18 +439,18 @@ using namespace pcfgnat;
 
 static int lsg_forward_dispatch(void *word_ins_out, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                 void *selected, int require_grad, int64_t B, int64_t L, int64_t V, int64_t T,
-                                const int64_t *eos_ol, const int64_t *eos_tl, void *stream) {
+                                const int64_t *eos_ol, const int64_t *eos_tl, void *lse, void *stream) {
     int rc = check_common(word_ins_out, select_idx, selected, B, L, V, T);
     if (rc != PCFGNAT_OK) return rc;
     if (B * L == 0) return PCFGNAT_OK;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case PCFGNAT_F16:
-            return launch_fwd<__half>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, s);
+            return launch_fwd<__half>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, s);
         case PCFGNAT_F32:
-            return launch_fwd<float>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, s);
+            return launch_fwd<float>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, s);
         case PCFGNAT_F64:
-            return launch_fwd<double>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, s);
+            return launch_fwd<double>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, s);
         default:
             return fail(PCFGNAT_EINVAL, "logsoftmax_gather: unknown dtype code %d (float16, float32, float64 are dispatched)", dtype);
     }
@@ -437,7 +460,7 @@ extern "C" int pcfgnat_logsoftmax_gather(void *word_ins_out, int dtype, const in
                                          int64_t st, void *selected, int require_grad, int64_t B, int64_t L, int64_t V,
                                          int64_t T, void *stream) {
     return lsg_forward_dispatch(word_ins_out, dtype, select_idx, sb, sl, st, selected, require_grad, B, L, V, T, nullptr, nullptr,
-                                stream);
+                                nullptr, stream);
 }
 
 extern "C" int pcfgnat_logsoftmax_gather_eos(void *word_ins_out, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl,
@@ -446,24 +469,47 @@ extern "C" int pcfgnat_logsoftmax_gather_eos(void *word_ins_out, int dtype, cons
                                              void *stream) {
     PCFGNAT_REQUIRE(B == 0 || (output_length && target_length), "logsoftmax_gather_eos: null length pointer");
     return lsg_forward_dispatch(word_ins_out, dtype, select_idx, sb, sl, st, selected, require_grad, B, L, V, T, output_length,
-                                target_length, stream);
+                                target_length, nullptr, stream);
 }
 
-extern "C" int pcfgnat_logsoftmax_gather_backward(void *probs_inout, int dtype, const int64_t *select_idx, int64_t sb,
-                                                  int64_t sl, int64_t st, const void *grad_selected, int64_t B, int64_t L,
-                                                  int64_t V, int64_t T, void *stream) {
-    int rc = check_common(probs_inout, select_idx, grad_selected, B, L, V, T);
+extern "C" int pcfgnat_logsoftmax_gather_lse(const void *word_ins_out, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl,
+                                             int64_t st, void *selected, void *lse, const int64_t *output_length,
+                                             const int64_t *target_length, int64_t B, int64_t L, int64_t V, int64_t T,
+                                             void *stream) {
+    PCFGNAT_REQUIRE(B * L == 0 || lse != nullptr, "logsoftmax_gather_lse: null lse pointer");
+    PCFGNAT_REQUIRE((output_length == nullptr) == (target_length == nullptr),
+                    "logsoftmax_gather_lse: output_length and target_length must be given together");
+    return lsg_forward_dispatch(const_cast<void *>(word_ins_out), dtype, select_idx, sb, sl, st, selected, 0, B, L, V, T, output_length,
+                                target_length, lse, stream);
+}
+
+static int lsg_backward_dispatch(void *buf, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
+                                 const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T, void *stream) {
+    int rc = check_common(buf, select_idx, grad_selected, B, L, V, T);
     if (rc != PCFGNAT_OK) return rc;
     if (B * L == 0) return PCFGNAT_OK;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case PCFGNAT_F16:
-            return launch_bwd<__half>(probs_inout, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, s);
+            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, s);
         case PCFGNAT_F32:
-            return launch_bwd<float>(probs_inout, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, s);
+            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, s);
         case PCFGNAT_F64:
-            return launch_bwd<double>(probs_inout, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, s);
+            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, s);
         default:
             return fail(PCFGNAT_EINVAL, "logsoftmax_gather_backward: unknown dtype code %d", dtype);
     }
+}
+
+extern "C" int pcfgnat_logsoftmax_gather_backward(void *probs_inout, int dtype, const int64_t *select_idx, int64_t sb,
+                                                  int64_t sl, int64_t st, const void *grad_selected, int64_t B, int64_t L,
+                                                  int64_t V, int64_t T, void *stream) {
+    return lsg_backward_dispatch(probs_inout, dtype, select_idx, sb, sl, st, grad_selected, nullptr, B, L, V, T, stream);
+}
+
+extern "C" int pcfgnat_logsoftmax_gather_backward_lse(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb,
+                                                      int64_t sl, int64_t st, const void *grad_selected, const void *lse, int64_t B,
+                                                      int64_t L, int64_t V, int64_t T, void *stream) {
+    PCFGNAT_REQUIRE(B * L == 0 || lse != nullptr, "logsoftmax_gather_backward_lse: null lse pointer");
+    return lsg_backward_dispatch(logits_inout, dtype, select_idx, sb, sl, st, grad_selected, lse, B, L, V, T, stream);
 }

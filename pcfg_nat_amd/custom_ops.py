@@ -223,8 +223,10 @@ cuda_pcfg_viterbi = CUDAPCFGViterbiFunc.apply
 
 class DagLogsoftmaxGatherFunc(Function):
     """Fused log-softmax + gather with the reference's in-place contract (pcfg_loss.py:144-181): the logits buffer is
-    returned dirty (it holds softmax probabilities when a gradient is required) and becomes the gradient buffer in
-    backward, which may run once."""
+    handed back marked dirty, must not be used by the caller any more, and becomes the gradient buffer in backward,
+    which may run once.  Unlike the reference, whose forward already overwrites the buffer with softmax probabilities,
+    the forward here only reads it and keeps one log-sum-exp per row; the backward recomputes the probabilities while
+    it writes the gradient (three passes over the logits per step instead of four)."""
 
     @staticmethod
     def forward(
@@ -233,13 +235,16 @@ class DagLogsoftmaxGatherFunc(Function):
         select_idx,    # bsz * prelen * slen
     ):
         require_gradient = ctx.needs_input_grad[0]
-        selected_result = _logsoftmax_gather(word_ins_out, select_idx, require_gradient)
-        # Note: the kernel modifies word_ins_out and the backward reuses it
+        if require_gradient:
+            selected_result, row_lse = _logsoftmax_gather_lse(word_ins_out, select_idx)
+        else:
+            selected_result = _logsoftmax_gather(word_ins_out, select_idx, False)
+        # Note: the backward reuses word_ins_out as the gradient buffer
         ctx.mark_dirty(word_ins_out)
         ctx.set_materialize_grads(False)
 
         if require_gradient:
-            ctx.save_for_backward(word_ins_out, select_idx)
+            ctx.save_for_backward(word_ins_out, select_idx, row_lse)
             ctx.has_backward = False
         return word_ins_out, selected_result  # bsz * prelen * slen
 
@@ -254,8 +259,8 @@ class DagLogsoftmaxGatherFunc(Function):
         assert not ctx.has_backward, "Cannot backward twice in logsoftmax_gather"
         ctx.has_backward = True
 
-        grad_input, selected_idx = ctx.saved_tensors
-        _logsoftmax_gather_backward(grad_input, selected_idx, grad_output)
+        grad_input, selected_idx, row_lse = ctx.saved_tensors
+        _logsoftmax_gather_backward_lse(grad_input, selected_idx, grad_output, row_lse)
         return grad_input, None
 
 
@@ -301,6 +306,64 @@ def _logsoftmax_gather(word_ins_out, select_idx, require_gradient, eos_lengths=N
                                                          selected.data_ptr(), int(bool(require_gradient)), ol.data_ptr(),
                                                          tl.data_ptr(), B, L, V, T, _stream(word_ins_out)), lib)
     return selected
+
+
+def _logsoftmax_gather_lse(word_ins_out, select_idx, eos_lengths=None):
+    """Read-only forward of the log-sum-exp split: returns (selected [B,L,T], row log-sum-exp [B,L]); same checks as
+    ``_logsoftmax_gather``.  ``word_ins_out`` must stay untouched until ``_logsoftmax_gather_backward_lse`` consumes it."""
+    lib = get_pcfg_kernel()
+    _need_cuda("logsoftmax_gather", word_ins_out, select_idx)
+    if word_ins_out.dim() != 3:
+        raise RuntimeError("word_ins_out dim != 3")
+    if select_idx.dim() != 3:
+        raise RuntimeError("select_idx dim != 3")
+    B, L, V = word_ins_out.shape
+    T = select_idx.size(2)
+    if select_idx.size(0) != B:
+        raise RuntimeError("batch size not match")
+    if select_idx.size(1) != L:
+        raise RuntimeError("prelen size not match")
+    if select_idx.dtype != torch.int64:
+        raise RuntimeError("select_idx should be long")
+    if not word_ins_out.is_contiguous():
+        raise RuntimeError("word_ins_out is not contiguous")
+    code = _DTYPE_CODE.get(word_ins_out.dtype)
+    if code is None:
+        raise RuntimeError("logsoftmax_gather: unsupported dtype %s (float16, float32, float64 are dispatched)"
+                           % word_ins_out.dtype)
+    out_dtype = torch.float64 if word_ins_out.dtype == torch.float64 else torch.float32
+    with torch.cuda.device(word_ins_out.device):
+        selected = torch.empty((B, L, T), dtype=out_dtype, device=word_ins_out.device)
+        row_lse = torch.empty((B, L), dtype=out_dtype, device=word_ins_out.device)
+        sb, sl, st = select_idx.stride()
+        ol_ptr = tl_ptr = None
+        if eos_lengths is not None:
+            ol = _lengths("logsoftmax_gather", eos_lengths[0], B)
+            tl = _lengths("logsoftmax_gather", eos_lengths[1], B)
+            _need_cuda("logsoftmax_gather", word_ins_out, ol, tl)
+            ol_ptr, tl_ptr = ol.data_ptr(), tl.data_ptr()
+        _lib.check(lib.pcfgnat_logsoftmax_gather_lse(word_ins_out.data_ptr(), code, select_idx.data_ptr(), sb, sl, st,
+                                                     selected.data_ptr(), row_lse.data_ptr(), ol_ptr, tl_ptr, B, L, V, T,
+                                                     _stream(word_ins_out)), lib)
+    return selected, row_lse
+
+
+def _logsoftmax_gather_backward_lse(buf, select_idx, grad_output, row_lse):
+    """In place: ``buf`` (the untouched logits) becomes d/d logits of sum(grad_output * selected): one pass that
+    recomputes exp(x - lse), scales by -(sum g) and adds g at the gathered columns, rounded to buf's dtype once."""
+    lib = get_pcfg_kernel()
+    B, L, V = buf.shape
+    T = select_idx.size(2)
+    want = torch.float64 if buf.dtype == torch.float64 else torch.float32
+    g = grad_output.to(want).contiguous()
+    if row_lse.dtype != want or row_lse.shape != (B, L) or not row_lse.is_contiguous():
+        raise RuntimeError("logsoftmax_gather_backward: row_lse must be a contiguous [bsz, prelen] tensor of %s" % want)
+    with torch.cuda.device(buf.device):
+        sb, sl, st = select_idx.stride()
+        _lib.check(lib.pcfgnat_logsoftmax_gather_backward_lse(buf.data_ptr(), _DTYPE_CODE[buf.dtype], select_idx.data_ptr(),
+                                                              sb, sl, st, g.data_ptr(), row_lse.data_ptr(), B, L, V, T,
+                                                              _stream(buf)), lib)
+    return buf
 
 
 def _logsoftmax_gather_backward(buf, select_idx, grad_output):
@@ -394,8 +457,10 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
         aux = torch.empty((max(1, lib.pcfgnat_pcfg_aux_floats(B, L, T, ml)),), dtype=torch.float32, device=dev)
         mg = torch.empty_like(match)
         lg = torch.empty_like(links)
+        row_lse = torch.empty((B, L), dtype=torch.float32, device=dev)
         out = torch.empty((2,), dtype=torch.float32, device=dev)
         _lib.check(lib.pcfgnat_criterion_step(logits.data_ptr(), code, targets.data_ptr(), links.data_ptr(), ol.data_ptr(),
                                               tl.data_ptr(), match.data_ptr(), S.data_ptr(), aux.data_ptr(), mg.data_ptr(),
-                                              lg.data_ptr(), out.data_ptr(), B, L, V, T, ml, slices, _stream(logits), ev_arr), lib)
+                                              lg.data_ptr(), row_lse.data_ptr(), out.data_ptr(), B, L, V, T, ml, slices,
+                                              _stream(logits), ev_arr), lib)
     return out, lg, S[:, 0, 0], match, mg

@@ -136,12 +136,14 @@ def train_step_fused(logits, targets, links, output_length, target_length, ops=_
     """The same training pass as ``train_step_direct`` with the criterion's glue folded into the kernels: the eos mask is
     applied inside the gather (no [B,L,T] mask tensors), and the inside backward is seeded with the criterion's own
     weights -1/(n_b*B) instead of ones followed by two scaling passes; sentences with a non-finite log-likelihood get
-    zero gradients from the kernel itself.  Four kernel launches.  Returns (loss, links_grad, ll)."""
+    zero gradients from the kernel itself; the gather forward only reads the logits and the gather backward recomputes
+    the softmax from the row log-sum-exps (three passes over the logits instead of four).  Four kernel launches.
+    Returns (loss, links_grad, ll)."""
     mark = mark or (lambda name, phase: None)
     L = logits.shape[1]
     idx = targets.unsqueeze(1).expand(-1, L, -1)
     mark("lsg_fwd", 0)
-    match_m = ops._logsoftmax_gather(logits, idx, True, eos_lengths=(output_length, target_length))
+    match_m, row_lse = ops._logsoftmax_gather_lse(logits, idx, eos_lengths=(output_length, target_length))
     mark("lsg_fwd", 1)
     mark("inside_fwd", 0)
     S, aux, ol, tl = ops._pcfg_loss_tables(match_m, links, output_length, target_length, 1, "cuda_pcfg_loss")
@@ -150,7 +152,7 @@ def train_step_fused(logits, targets, links, output_length, target_length, ops=_
     gmatch, glinks = ops._pcfg_loss_backward(None, S, aux, match_m, links, ol, tl, 1)
     mark("inside_bwd", 1)
     mark("lsg_bwd", 0)
-    ops._logsoftmax_gather_backward(logits, idx, gmatch)
+    ops._logsoftmax_gather_backward_lse(logits, idx, gmatch, row_lse)
     mark("lsg_bwd", 1)
     ll = S[:, 0, 0]
     invalid = ll.isinf().logical_or(ll.isnan())

@@ -168,13 +168,13 @@ def links_bytes(B, L, ml):
 
 
 def lsg_fwd_bytes(B, L, V, T, itemsize, require_grad=True):
-    """Algorithmic HBM bytes of one logsoftmax_gather forward: logits read once, softmax written once when the
-    gradient is needed, gathered fp32 written, un-expanded int64 targets read."""
-    return (2 if require_grad else 1) * B * L * V * itemsize + B * L * T * 4 + B * T * 8
+    """Algorithmic HBM bytes of one logsoftmax_gather forward: logits read once, gathered fp32 written, un-expanded int64
+    targets read; plus the softmax written in place (reference split, ``require_grad``) or one fp32 log-sum-exp per row."""
+    return (2 if require_grad else 1) * B * L * V * itemsize + B * L * T * 4 + B * T * 8 + (0 if require_grad else B * L * 4)
 
 
 def lsg_bwd_bytes(B, L, V, T, itemsize):
-    """Algorithmic HBM bytes of the in-place backward: probabilities read, gradients written, grad_output read."""
+    """Algorithmic HBM bytes of the in-place backward: probabilities (or logits) read, gradients written, grad_output read."""
     return 2 * B * L * V * itemsize + B * L * T * 4
 
 

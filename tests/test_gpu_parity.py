@@ -96,6 +96,45 @@ def test_lsg_backward_matches_torch_ops(dtype):
         assert torch.allclose(got, ref, rtol=1e-5, atol=1e-9)
 
 
+@pytest.mark.parametrize("dtype,V", [(torch.float16, 2048), (torch.float16, 333), (torch.float32, 1001), (torch.float64, 257)])
+def test_lsg_lse_split_matches_autograd(dtype, V):
+    """Read-only forward + recomputing backward against torch's own log_softmax/gather gradient in float64."""
+    g = torch.Generator().manual_seed(11)
+    B, L, T = 3, 7, 12
+    x = (torch.randn(B, L, V, generator=g) * 3).to(dtype)
+    tgt = torch.randint(0, V, (B, T), generator=g)
+    tgt[:, 3] = tgt[:, 1]  # duplicate columns
+    tgt[:, 9:] = 1         # pads
+    idx = tgt.unsqueeze(1).expand(-1, L, -1)
+    gout = torch.randn(B, L, T, generator=g)
+    gout[:, :, 9:] = 0
+    ol = torch.tensor([7, 5, 6])
+    tl = torch.tensor([9, 4, 6])
+    xd = x.to(DEV)
+    sel, lse = ops._logsoftmax_gather_lse(xd, idx.to(DEV), eos_lengths=(ol.to(DEV), tl.to(DEV)))
+    assert torch.equal(xd.cpu(), x)  # forward leaves the logits alone
+    leaf = x.double().requires_grad_(True)
+    ref_sel = torch.log_softmax(leaf, -1).gather(-1, idx)
+    ref_lse = torch.logsumexp(leaf.detach(), -1)
+    want = harness.eos_masked(ref_sel.detach(), ol, tl)
+    fin = torch.isfinite(want)
+    tol = 1e-12 if dtype == torch.float64 else 2e-5
+    assert torch.equal(torch.isfinite(sel.cpu()), fin)
+    assert torch.allclose(sel.cpu().double()[fin], want[fin], rtol=tol, atol=tol)
+    assert torch.allclose(lse.cpu().double(), ref_lse, rtol=tol, atol=tol)
+    gdev = gout.to(DEV).to(sel.dtype)
+    ops._logsoftmax_gather_backward_lse(xd, idx.to(DEV), gdev, lse)
+    (ref_sel * gout.double()).sum().backward()
+    got = xd.cpu().double()
+    if dtype == torch.float16:
+        # one rounding to fp16 of the float32 result
+        assert torch.allclose(got, leaf.grad, rtol=2 ** -10, atol=2 ** -24)
+    elif dtype == torch.float32:
+        assert torch.allclose(got, leaf.grad, rtol=1e-5, atol=1e-7)
+    else:
+        assert torch.allclose(got, leaf.grad, rtol=1e-12, atol=1e-14)
+
+
 def test_lsg_autograd_contract():
     g = torch.Generator().manual_seed(2)
     B, L, V, T = 2, 4, 640, 5
