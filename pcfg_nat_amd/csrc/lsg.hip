@@ -80,10 +80,65 @@ struct Elem<double> {
     __device__ static __forceinline__ double narrow(double x) { return x; }
 };
 
-__device__ __forceinline__ float fast_exp(float x) { return __expf(x); }
-__device__ __forceinline__ double fast_exp(double x) { return exp(x); }
-__device__ __forceinline__ float fast_log(float x) { return __logf(x); }
-__device__ __forceinline__ double fast_log(double x) { return log(x); }
+// Row normalisation: e(v) = exp(v - max) and the row log-sum-exp from sum_v e(v).  In float the subtraction, the change
+// of base and the widening of an fp16 input are folded into one fused multiply-add in front of the hardware exp2
+// (e(v) = 2^(v*log2e + nb), nb = -max*log2e rounded once; the log-sum-exp undoes exactly that nb, so the rounding of nb
+// does not bias the result), which takes the loops below from five VALU instructions per element to two plus the exp2.
+template <typename CT>
+struct RowNorm;
+template <>
+struct RowNorm<float> {
+    float nb;
+    __device__ __forceinline__ explicit RowNorm(float mx) : nb(-mx * 1.4426950408889634f) {}
+    __device__ __forceinline__ float e(float v) const { return __builtin_amdgcn_exp2f(__builtin_fmaf(v, 1.4426950408889634f, nb)); }
+    __device__ __forceinline__ float lse(float sum) const { return (__builtin_amdgcn_logf(sum) - nb) * 0.6931471805599453f; }
+    // exp(v - l) for a given log-sum-exp l
+    __device__ static __forceinline__ RowNorm from_lse(float l) { return RowNorm(l); }
+};
+template <>
+struct RowNorm<double> {
+    double mx;
+    __device__ __forceinline__ explicit RowNorm(double m) : mx(m) {}
+    __device__ __forceinline__ double e(double v) const { return exp(v - mx); }
+    __device__ __forceinline__ double lse(double sum) const { return mx + log(sum); }
+    __device__ static __forceinline__ RowNorm from_lse(double l) { return RowNorm(l); }
+};
+
+// Running maximum of a row: packed fp16 maxima for half inputs (two elements per instruction, no widening), plain
+// compute-type maxima otherwise.
+template <typename T>
+struct RowMax {
+    typename Elem<T>::compute m;
+    __device__ __forceinline__ RowMax() : m(-__builtin_huge_val()) {}
+    __device__ __forceinline__ void chunk(const vec16 &v) {
+        typename Elem<T>::compute o[Elem<T>::EPV];
+        Elem<T>::unpack(v, o);
+#pragma unroll
+        for (int e = 0; e < Elem<T>::EPV; e++) m = (m > o[e] || !(o[e] == o[e])) ? m : o[e];
+    }
+    __device__ __forceinline__ void scalar(T x) {
+        const typename Elem<T>::compute o = Elem<T>::widen(x);
+        m = (m > o || !(o == o)) ? m : o;
+    }
+    __device__ __forceinline__ typename Elem<T>::compute value() const { return m; }
+};
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+template <>
+struct RowMax<__half> {
+    f16x2 m;
+    __device__ __forceinline__ RowMax() : m{(_Float16)-__builtin_huge_valf(), (_Float16)-__builtin_huge_valf()} {}
+    __device__ __forceinline__ void chunk(const vec16 &v) {
+        const f16x2 *h = reinterpret_cast<const f16x2 *>(&v);
+#pragma unroll
+        for (int i = 0; i < 4; i++) m = __builtin_elementwise_max(m, h[i]);
+    }
+    __device__ __forceinline__ void scalar(__half x) {
+        const _Float16 f = *reinterpret_cast<const _Float16 *>(&x);
+        m = __builtin_elementwise_max(m, f16x2{f, f});
+    }
+    __device__ __forceinline__ float value() const { return fmaxf((float)m.x, (float)m.y); }
+};
+
 __device__ __forceinline__ float neg_inf(float) { return -__builtin_huge_valf(); }
 __device__ __forceinline__ double neg_inf(double) { return -__builtin_huge_val(); }
 __device__ __forceinline__ float vmax(float a, float b) { return fmaxf(a, b); }
@@ -193,46 +248,37 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
         if (ep >= 0) edge = Elem<T>::widen(xr[ep]);
 
         // ---- max
-        CT mx = edge;
+        RowMax<T> rmax;
+        if (ep >= 0) rmax.scalar(xr[ep]);
 #pragma unroll
-        for (int i = 0; i < MAXC; i++) {
-            if (tid + i * NT < sp.nvec) {
-                CT v[EPV];
-                Elem<T>::unpack(buf[i], v);
-#pragma unroll
-                for (int e = 0; e < EPV; e++) mx = vmax(mx, v[e]);
-            }
-        }
-        for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
-            CT v[EPV];
-            Elem<T>::unpack(load16(xv + c), v);
-#pragma unroll
-            for (int e = 0; e < EPV; e++) mx = vmax(mx, v[e]);
-        }
-        mx = block_max<CT, NW>(mx, s_max, wave, lane);
+        for (int i = 0; i < MAXC; i++)
+            if (tid + i * NT < sp.nvec) rmax.chunk(buf[i]);
+        for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) rmax.chunk(load16(xv + c));
+        const CT mx = block_max<CT, NW>(rmax.value(), s_max, wave, lane);
+        const RowNorm<CT> rn(mx);
 #pragma unroll
         for (int i = 0; i < MAXC; i++) opaque(buf[i]);
 
         // ---- sum of exp
-        CT sum = (ep >= 0) ? fast_exp(edge - mx) : (CT)0;
+        CT sum = (ep >= 0) ? rn.e(edge) : (CT)0;
 #pragma unroll
         for (int i = 0; i < MAXC; i++) {
             if (tid + i * NT < sp.nvec) {
                 CT v[EPV];
                 Elem<T>::unpack(buf[i], v);
 #pragma unroll
-                for (int e = 0; e < EPV; e++) sum += fast_exp(v[e] - mx);
+                for (int e = 0; e < EPV; e++) sum += rn.e(v[e]);
             }
         }
         for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
             CT v[EPV];
             Elem<T>::unpack(load16(xv + c), v);
 #pragma unroll
-            for (int e = 0; e < EPV; e++) sum += fast_exp(v[e] - mx);
+            for (int e = 0; e < EPV; e++) sum += rn.e(v[e]);
         }
         sum = block_sum<CT, NW>(sum, s_sum, wave, lane);
-        const CT lg = fast_log(sum);
-        if (lse_out != nullptr && tid == 0) lse_out[row] = mx + lg;
+        const CT row_lse = rn.lse(sum);
+        if (lse_out != nullptr && tid == 0) lse_out[row] = row_lse;
 #pragma unroll
         for (int i = 0; i < MAXC; i++) opaque(buf[i]);
 
@@ -245,7 +291,7 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
             int s = tid + g * NT;
-            if (s < Tn) sel[row * (int64_t)Tn + s] = (s == eos_col) ? neg_inf(CT()) : (gv[g] - mx) - lg;
+            if (s < Tn) sel[row * (int64_t)Tn + s] = (s == eos_col) ? neg_inf(CT()) : gv[g] - row_lse;
         }
 
         if (GRAD) {
@@ -258,7 +304,7 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
                     CT v[EPV];
                     Elem<T>::unpack(buf[i], v);
 #pragma unroll
-                    for (int e = 0; e < EPV; e++) v[e] = fast_exp(v[e] - mx) * inv;
+                    for (int e = 0; e < EPV; e++) v[e] = rn.e(v[e]) * inv;
                     store16(xw + c, Elem<T>::pack(v));
                 }
             }
@@ -266,10 +312,10 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
                 CT v[EPV];
                 Elem<T>::unpack(load16(xv + c), v);
 #pragma unroll
-                for (int e = 0; e < EPV; e++) v[e] = fast_exp(v[e] - mx) * inv;
+                for (int e = 0; e < EPV; e++) v[e] = rn.e(v[e]) * inv;
                 store16(xw + c, Elem<T>::pack(v));
             }
-            if (ep >= 0) xr[ep] = Elem<T>::narrow(fast_exp(edge - mx) * inv);
+            if (ep >= 0) xr[ep] = Elem<T>::narrow(rn.e(edge) * inv);
         }
     }
 }
@@ -314,7 +360,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
         CT part = 0;
         for (int s = lane; s < Tn; s += 64) part += gr[s];
         const CT ns = FROM_LOGITS ? -wave_sum(part) : Elem<T>::widen(Elem<T>::narrow(-wave_sum(part)));
-        const CT row_lse = FROM_LOGITS ? lse[row] : (CT)0;
+        const RowNorm<CT> rn = RowNorm<CT>::from_lse(FROM_LOGITS ? lse[row] : (CT)0);
 
         for (int s = tid; s < Tn; s += NT) {
             int64_t t = ir[(int64_t)s * st];
@@ -322,7 +368,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
             s_idx[s] = ok ? (int)t : -1;
             if (FROM_LOGITS) {
                 s_g[s] = gr[s];
-                s_p[s] = ok ? fast_exp(Elem<T>::widen(pr[t]) - row_lse) : (CT)0;
+                s_p[s] = ok ? rn.e(Elem<T>::widen(pr[t])) : (CT)0;
             } else {
                 s_g[s] = Elem<T>::widen(Elem<T>::narrow(gr[s]));
                 s_p[s] = ok ? Elem<T>::widen(pr[t]) : (CT)0;
@@ -337,7 +383,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
                 CT v[EPV];
                 Elem<T>::unpack(buf[i], v);
 #pragma unroll
-                for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? fast_exp(v[e] - row_lse) : v[e]) * ns;
+                for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
                 store16(pv + c, Elem<T>::pack(v));
             }
         }
@@ -345,10 +391,10 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
             CT v[EPV];
             Elem<T>::unpack(load16(pv + c), v);
 #pragma unroll
-            for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? fast_exp(v[e] - row_lse) : v[e]) * ns;
+            for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
             store16(pv + c, Elem<T>::pack(v));
         }
-        if (ep >= 0) pr[ep] = Elem<T>::narrow((FROM_LOGITS ? fast_exp(edge - row_lse) : edge) * ns);
+        if (ep >= 0) pr[ep] = Elem<T>::narrow((FROM_LOGITS ? rn.e(edge) : edge) * ns);
 
         // scatter_add_ (pcfg_loss.py:177): the first occurrence of a column accumulates all its duplicates in order
         CT fix[FIX];
@@ -388,10 +434,13 @@ template <typename T>
 int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, void *sel, int grad, int64_t rows,
                int L, int V, int Tn, const int64_t *eos_ol, const int64_t *eos_tl, void *lse, hipStream_t stream) {
     using CT = typename Elem<T>::compute;
-    constexpr int NT = 512;
+#ifndef LSG_FWD_NT
+#define LSG_FWD_NT 512
+#endif
+    constexpr int NT = LSG_FWD_NT;
     // 10 chunks x 512 threads x 16 B = 80 KB of a row in registers: a 40k-entry fp16 row exactly, half of an fp32 one.
-    constexpr int MAXC = 10;
-    constexpr int GMAX = 2;
+    constexpr int MAXC = 5120 / NT;
+    constexpr int GMAX = 1024 / NT;
     if (Tn > NT * GMAX) return fail(PCFGNAT_EUNSUPPORTED, "logsoftmax_gather: T=%d exceeds %d targets per row", Tn, NT * GMAX);
     int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
     if (grad)

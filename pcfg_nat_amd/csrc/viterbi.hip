@@ -9,7 +9,7 @@
 // follow the reference's 4-lane strided scan (lane priority 0 > 2 > 1 > 3, then c ascending, then j ascending).
 //
 // Same sweep shape as the inside forward: one workgroup per sentence, one 16-lane DPP row per parent node, link
-// slabs in registers, one barrier per length.
+// slabs in registers (graphs of up to 514 nodes), one barrier per length.
 #include "common.hip.h"
 
 namespace pcfgnat {
@@ -39,14 +39,40 @@ __device__ __forceinline__ void row16_argmax_step(float &best, int &key) {
 
 __device__ __forceinline__ float nan_to_ninf(float v) { return (v != v) ? NEG_INF_F : v; }
 
-template <int R>
+// Row maximum with one DPP instruction per step (fmaxf() on a DPP result costs move + canonicalise + max).  The leading
+// s_nop covers the wait states a DPP read needs after a VALU write of its source, which the compiler does not track
+// through inline assembly.  Inputs are never NaN here.
+#define PCFGNAT_DPP_MAX(name, ctrl)                                                                          \
+    __device__ __forceinline__ float name(float v) {                                                          \
+        float r;                                                                                              \
+        asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v)); \
+        return r;                                                                                             \
+    }
+PCFGNAT_DPP_MAX(vit_max_xor1, "quad_perm:[1,0,3,2]")
+PCFGNAT_DPP_MAX(vit_max_xor2, "quad_perm:[2,3,0,1]")
+PCFGNAT_DPP_MAX(vit_max_half_mirror, "row_half_mirror")
+PCFGNAT_DPP_MAX(vit_max_mirror, "row_mirror")
+#undef PCFGNAT_DPP_MAX
+__device__ __forceinline__ float row16_max_raw(float v) {
+    return vit_max_mirror(vit_max_half_mirror(vit_max_xor2(vit_max_xor1(v))));
+}
+
+// NQ = number of 16-node chunks of the main chain (mc <= 16*NQ <= 256).  Row pass r handles parents 64r .. 64r+63, one
+// 16-lane row per parent; its lanes stride over the children, of which only chunks q >= 4r can hold c >= a, so the
+// triangular slabs cost NQ + (NQ-4) + (NQ-8) + ... chunk pairs of registers per thread.  Everything that does not
+// change from length to length is folded into the slabs once (links + 0 and links + ob[leaf], in the reference's
+// association order), which leaves two adds, one compare and two selects per candidate and length.  Inside a thread the
+// candidates are visited in ascending (child, j) order and only a strictly larger value replaces the running best,
+// which is the reference's tie order for one lane of its strided scan; the full tie key is built once per row and used
+// in the cross-lane reduction.  LDS: three rotating columns (lengths len, len-1, len-2).
+template <int NQ>
 __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict__ ob_lprob, const float *__restrict__ links,
                                                         const int64_t *__restrict__ out_len, float *__restrict__ S,
                                                         int64_t *__restrict__ Rt, int64_t *__restrict__ Lt, int64_t *__restrict__ Mt,
                                                         int L, int Lq) {
-    constexpr int CN = 4 * R;
+    constexpr int R = (NQ + 3) / 4;
     constexpr int MP = 64 * R;
-    __shared__ float col[2 * MP];
+    __shared__ float col[3 * MP];
     const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j16 = tid & 15;
     const int m = (int)out_len[b];
     const float *ob = ob_lprob + (size_t)b * L;
@@ -65,58 +91,101 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
     if (m < 2 || m > L || (m % 2) != 0) return;  // out of contract: leave the empty tables
     const int mc = m / 2;
 
-    float A0[R][CN], A1[R][CN], ob_a[R], ob_leaf[R];
+    // slabs: unconditional loads from clamped addresses (all in flight together), masked afterwards
+    float A0[R][NQ], A1[R][NQ], ob_a[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        const int a_id = gidx + 64 * r, a = 2 * a_id + 1;
-        ob_a[r] = (a_id < mc) ? ob[a] : NEG_INF_F;
-        ob_leaf[r] = (a_id < mc && a_id >= 1) ? ob[a - 1] : NEG_INF_F;
+        const int a_id = gidx + 64 * r, a = 2 * min(a_id, mc - 1) + 1;
 #pragma unroll
-        for (int q = 0; q < CN; q++) {
-            const int c_id = j16 + 16 * q, c = 2 * c_id + 1;
-            const bool ok = a_id < mc && c_id < mc && c_id >= a_id;
-            A0[r][q] = ok ? lk[((size_t)a * 2 + 0) * L + c] : NEG_INF_F;
-            A1[r][q] = (ok && a_id >= 1) ? lk[((size_t)a * 2 + 1) * L + c] : NEG_INF_F;
+        for (int q = 0; q < NQ; q++) {
+            if (q >= 4 * r) {
+                const int c = 2 * min(j16 + 16 * q, mc - 1) + 1;
+                A0[r][q] = lk[((size_t)a * 2 + 0) * L + c];
+                A1[r][q] = lk[((size_t)a * 2 + 1) * L + c];
+            }
         }
     }
-    // length 1: only the last node (pcfg_viterbi.cu:57-59)
-    for (int i = tid; i < MP; i += NT) col[1 * MP + i] = (i == mc - 1) ? ob[m - 1] : NEG_INF_F;
-    float sc2[CN];
 #pragma unroll
-    for (int q = 0; q < CN; q++) sc2[q] = NEG_INF_F;  // S[c][0] = -inf
+    for (int r = 0; r < R; r++) {
+        const int a_id = gidx + 64 * r, a = 2 * min(a_id, mc - 1) + 1;
+        const float oa = ob[a], ol = ob[a - 1];
+        ob_a[r] = (a_id < mc) ? oa : NEG_INF_F;
+        const float ob_leaf = (a_id < mc && a_id >= 1) ? ol : NEG_INF_F;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            if (q >= 4 * r) {
+                const int c_id = j16 + 16 * q;
+                const bool ok = a_id < mc && c_id < mc && c_id >= a_id;
+                A0[r][q] = ok ? A0[r][q] + 0.f : NEG_INF_F;
+                A1[r][q] = (ok && a_id >= 1) ? A1[r][q] + ob_leaf : NEG_INF_F;
+            }
+        }
+    }
+    // length 0: nothing; length 1: only the last node (pcfg_viterbi.cu:57-59)
+    for (int i = tid; i < 3 * MP; i += NT) col[i] = (i == 1 * MP + mc - 1) ? ob[m - 1] : NEG_INF_F;
     __syncthreads();
     if (tid == 0 && Lq > 1) Sb[(size_t)(m - 1) * Lq + 1] = ob[m - 1];
 
     const int len_end = m / 4;  // pcfg_viterbi.cu:67
+    int i1 = 1, i2 = 0, i0 = 2;  // column slots of len-1, len-2, len
     for (int len = 2; len < len_end; len++) {
-        const float *cur = col + ((len - 1) & 1) * MP;
-        float *nxt = col + (len & 1) * MP;
-        float sc1[CN];
+        const float *cur1 = col + i1 * MP, *cur2 = col + i2 * MP;
+        float *nxt = col + i0 * MP;
+        // the two columns stay in registers across the row passes, except for the widest slabs, which re-read them from
+        // LDS in every pass to stay inside the register budget of a 1024-thread workgroup
+        constexpr bool RELOAD = NQ > 12;
+        float sc1[NQ], sc2[NQ];
+        if (!RELOAD) {
 #pragma unroll
-        for (int q = 0; q < CN; q++) sc1[q] = cur[j16 + 16 * q];
+            for (int q = 0; q < NQ; q++) {
+                sc1[q] = cur1[j16 + 16 * q];
+                sc2[q] = cur2[j16 + 16 * q];
+            }
+        }
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const int a_id = gidx + 64 * r;
             float best = NEG_INF_F;
-            int key = 0x7fffffff;
+            int sel = -1;
+            if (RELOAD) {
+                asm volatile("" ::: "memory");  // keeps the compiler from merging the passes' loads back into one set
 #pragma unroll
-            for (int q = 0; q < CN; q++) {
-                const int rel = j16 + 16 * q - a_id;
-                const float c0 = nan_to_ninf(((A0[r][q] + 0.f) + sc1[q]) + ob_a[r]);
-                const float c1 = nan_to_ninf(((A1[r][q] + ob_leaf[r]) + sc2[q]) + ob_a[r]);
-                if (c0 != NEG_INF_F) take_better(best, key, c0, tie_key(rel, 0));
-                if (c1 != NEG_INF_F) take_better(best, key, c1, tie_key(rel, 1));
+                for (int q = 0; q < NQ; q++) {
+                    if (q >= 4 * r) {
+                        sc1[q] = cur1[j16 + 16 * q];
+                        sc2[q] = cur2[j16 + 16 * q];
+                    }
+                }
             }
-            row16_argmax_step<DPP_QUAD_XOR1>(best, key);
-            row16_argmax_step<DPP_QUAD_XOR2>(best, key);
-            row16_argmax_step<DPP_ROW_HALF_MIRROR>(best, key);
-            row16_argmax_step<DPP_ROW_MIRROR>(best, key);
+#pragma unroll
+            for (int q = 0; q < NQ; q++) {
+                if (q >= 4 * r) {
+                    const float c0 = (A0[r][q] + sc1[q]) + ob_a[r];
+                    const float c1 = (A1[r][q] + sc2[q]) + ob_a[r];
+                    if (c0 > best) {  // false for NaN and for -inf against the initial -inf
+                        best = c0;
+                        sel = 2 * q;
+                    }
+                    if (c1 > best) {
+                        best = c1;
+                        sel = 2 * q + 1;
+                    }
+                }
+            }
+            // row maximum first, then the smallest tie key among the lanes that hold it
+            const float mine = best;
+            best = row16_max_raw(best);
+            int key = (sel < 0 || mine != best) ? 0x7fffffff : tie_key(j16 + 16 * (sel >> 1) - a_id, sel & 1);
+            key = min(key, dpp_i<DPP_QUAD_XOR1>(key));
+            key = min(key, dpp_i<DPP_QUAD_XOR2>(key));
+            key = min(key, dpp_i<DPP_ROW_HALF_MIRROR>(key));
+            key = min(key, dpp_i<DPP_ROW_MIRROR>(key));
             if (j16 == 0) {
                 nxt[a_id] = best;
                 if (best != NEG_INF_F && a_id < mc) {  // pcfg_viterbi.cu:125-131
                     const int a = 2 * a_id + 1;
                     const int jj = key & 1, rel = (key >> 1) & 0x7fffff;
-                    const size_t o = (size_t)a * Lq + len;
+                    const unsigned o = (unsigned)(a * Lq + len);  // 32-bit offset from the uniform table bases
                     Sb[o] = best;
                     Lb[o] = jj ? (a - 1) : 0;
                     Rb[o] = 2 * (a_id + rel) + 1;
@@ -124,13 +193,15 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
                 }
             }
         }
-#pragma unroll
-        for (int q = 0; q < CN; q++) sc2[q] = sc1[q];
+        const int t = i2;
+        i2 = i1;
+        i1 = i0;
+        i0 = t;
         lds_barrier();
     }
 }
 
-// Streaming variant for graphs whose link slabs do not fit in registers (Mc > 128): rows in tiles of 64, link values
+// Streaming variant for graphs whose link slabs do not fit in registers (Mc > 256): rows in tiles of 64, link values
 // fetched from L2 every step.  LDS: three rotating columns (lengths len, len-1, len-2).
 __global__ __launch_bounds__(NT) void viterbi_ml1_stream_kernel(const float *__restrict__ ob_lprob, const float *__restrict__ links,
                                                                const int64_t *__restrict__ out_len, float *__restrict__ S,
@@ -277,10 +348,21 @@ extern "C" int pcfgnat_pcfg_viterbi(const float *ob_lprob, const float *links, c
     const int Mc = (int)((L - 2) / 2 + 1);
     const int Lq = (int)(L / 4);
     hipStream_t s = (hipStream_t)stream;
-    if (Mc <= 64)
-        hipLaunchKernelGGL((viterbi_ml1_kernel<1>), dim3((unsigned)B), dim3(NT), 0, s, ob_lprob, links, output_length, S, R, Lt, M, (int)L, Lq);
-    else if (Mc <= 128)
-        hipLaunchKernelGGL((viterbi_ml1_kernel<2>), dim3((unsigned)B), dim3(NT), 0, s, ob_lprob, links, output_length, S, R, Lt, M, (int)L, Lq);
+#define PCFGNAT_VITERBI_CASE(nq)                                                                                              \
+    else if (Mc <= 16 * (nq))                                                                                                \
+        hipLaunchKernelGGL((viterbi_ml1_kernel<nq>), dim3((unsigned)B), dim3(NT), 0, s, ob_lprob, links, output_length, S, R, Lt, M, \
+                           (int)L, Lq)
+    if (false) {
+    }
+    PCFGNAT_VITERBI_CASE(2);
+    PCFGNAT_VITERBI_CASE(4);
+    PCFGNAT_VITERBI_CASE(6);
+    PCFGNAT_VITERBI_CASE(8);
+    PCFGNAT_VITERBI_CASE(10);
+    PCFGNAT_VITERBI_CASE(12);
+    PCFGNAT_VITERBI_CASE(14);
+    PCFGNAT_VITERBI_CASE(16);
+#undef PCFGNAT_VITERBI_CASE
     else {
         PCFGNAT_REQUIRE(L <= 4096, "pcfg_viterbi: graph size L=%lld exceeds 4096 nodes", (long long)L);
         const int MP = ((Mc + 63) / 64) * 64;

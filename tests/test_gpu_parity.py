@@ -283,12 +283,19 @@ def _decode_case(name):
         return synth.decode_batch([5, 9, 16, 3, 12], seed=3, V=500)
     if name == "L256":
         return synth.decode_batch([64, 40, 33], seed=4, V=300)
-    if name == "L400":  # longest graph of the inference configuration: streaming kernel
+    if name == "L400":  # longest graph of the inference configuration: widest register-resident slabs but one
         return synth.decode_batch([100, 71, 5], seed=6, V=100)
+    if name == "L512":  # widest register-resident slabs
+        return synth.decode_batch([128, 117, 20], seed=7, V=64)
+    if name == "L600":  # beyond the register-resident kernels: streaming kernel
+        return synth.decode_batch([150, 90], seed=8, V=64)
+    if name in ("L96", "L160", "L224", "L288", "L352"):  # one case per slab width in between
+        n = int(name[1:]) // 4
+        return synth.decode_batch([n, n - 3, 7], seed=n, V=64)
     raise KeyError(name)
 
 
-@pytest.mark.parametrize("case", ["short", "L256", "L400"])
+@pytest.mark.parametrize("case", ["short", "L96", "L160", "L224", "L256", "L288", "L352", "L400", "L512", "L600"])
 def test_viterbi_tables_bit_exact_and_decode(case):
     batch = _decode_case(case)
     ob, tok = synth.ob_and_tokens(batch["logits"])
