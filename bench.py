@@ -80,8 +80,9 @@ def cpu_baseline(batch_cpu, logits_sample, n_sent, repeats=9):
 
 def decode_timing(dev):
     """Viterbi decode of the inference configuration (src ~U[5,100], L = 4*src, V=40000): tables + length selection +
-    readout.  Batch 1 latency over a sample of sentences and batch 64 throughput.  ob/tokens precomputed, as in the
-    parity tests; the log-softmax/max pass over the logits is not part of these numbers."""
+    readout as one native call, result on the host side (token counts are read back).  Batch 1 latency over a sample of
+    sentences and batch 64 throughput.  ob/tokens precomputed, as in the parity tests; the log-softmax/max pass over the
+    logits is not part of these numbers."""
     import torch
     from pcfg_nat_amd import harness, synth
 
@@ -103,21 +104,21 @@ def decode_timing(dev):
         sample = lens[:32]
         cases = [make(sample[i:i + 1]) for i in range(len(sample))]
         for c in cases[:4]:
-            harness.viterbi_decode(*c)
+            harness.viterbi_decode(*c, single_call=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for c in cases:
-            harness.viterbi_decode(*c)
+            harness.viterbi_decode(*c, single_call=True)
         torch.cuda.synchronize()
         out["b1_ms_per_sentence"] = (time.perf_counter() - t0) * 1e3 / len(cases)
         # batch 64: sorted by length
         srt = torch.sort(lens)[0]
         chunks = [make(srt[i:i + 64]) for i in range(0, 640, 64)]
-        harness.viterbi_decode(*chunks[0])
+        harness.viterbi_decode(*chunks[0], single_call=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for c in chunks:
-            harness.viterbi_decode(*c)
+            harness.viterbi_decode(*c, single_call=True)
         torch.cuda.synchronize()
         out["b64_sentences_per_s"] = 640 / (time.perf_counter() - t0)
     except RuntimeError as e:  # a shape the library does not build yet

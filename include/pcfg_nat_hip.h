@@ -187,6 +187,21 @@ int pcfgnat_viterbi_decoding(const int64_t *pred_length, const int64_t *output_l
                              int64_t *out_tokens, int64_t *out_count, int64_t *scratch, int64_t B, int64_t L,
                              int64_t Lq, void *stream);
 
+/*
+ * The whole Viterbi decode of glat_decomposed_with_link_two_hands_tri_pcfg.py:483-502 in one call: tables
+ * (pcfg_viterbi.cu:272-301), length selection pred_length = 1 + argmax_{len >= 1} S[b,1,len] / length_penalty[len] with NaN
+ * read as -inf and the first maximum winning (:489-497), and the walk (pcfg_loss.cpp:12-73).  length_penalty [L/4] float32
+ * is the caller's arange(L/4) ** decode_viterbibeta.  For max_left = 1 and graphs of up to 514 nodes this is a single
+ * launch whose traces are one int32 per cell in `workspace`; otherwise the three steps run back to back on full
+ * tables in `workspace`.  workspace: pcfgnat_viterbi_decode_workspace_bytes(B, L, max_left) bytes, 8-byte aligned.
+ *   out_tokens [B,L] int64, out_count [B] int64 (as pcfgnat_viterbi_decoding), pred_length [B] int64.
+ */
+size_t pcfgnat_viterbi_decode_workspace_bytes(int64_t B, int64_t L, int64_t ml);
+int pcfgnat_viterbi_decode(const float *ob_lprob, const float *links, const int64_t *output_length, const int64_t *tokens,
+                           const int64_t *left_tree_mask, int64_t mask_dim, int64_t pad_index, const float *length_penalty,
+                           void *workspace, int64_t *out_tokens, int64_t *out_count, int64_t *pred_length, int64_t B,
+                           int64_t L, int64_t ml, void *stream);
+
 /* The same walk on host memory (the reference's own call site hands over CPU tensors,
  * glat_decomposed_with_link_two_hands_tri_pcfg.py:500-502).  Synchronous, touches no GPU. */
 int pcfgnat_viterbi_decoding_host(const int64_t *pred_length, const int64_t *output_length, const int64_t *Lt,

@@ -57,6 +57,99 @@ __device__ __forceinline__ float row16_max_raw(float v) {
     return vit_max_mirror(vit_max_half_mirror(vit_max_xor2(vit_max_xor1(v))));
 }
 
+// Back-pointer accessors of the readout walk.  FullTraces: the reference's three int64 tables [L][Lq].
+struct FullTraces {
+    const int64_t *Li, *Ri, *Mi;
+    int Lq;
+    __host__ __device__ int64_t left(int64_t node, int64_t len) const { return Li[node * Lq + len]; }
+    __host__ __device__ int64_t right(int64_t node, int64_t len) const { return Ri[node * Lq + len]; }
+    __host__ __device__ int64_t mid(int64_t node, int64_t len) const { return Mi[node * Lq + len]; }
+};
+// CompactTraces: one int32 per (main-chain node, length), 0 = empty cell, else 1 + ((c_id - a_id) << 1 | j); the rows of
+// the local leaves are never written by the sweep and read as zeros, as they do in the full tables.
+struct CompactTraces {
+    const int *W;
+    int Lq, rows;
+    __device__ int rec(int64_t node, int64_t len) const {
+        const int64_t a_id = node >> 1;
+        return ((node & 1) && a_id < rows) ? W[a_id * Lq + len] : 0;
+    }
+    __device__ int64_t left(int64_t node, int64_t len) const {
+        const int r = rec(node, len);
+        return (r != 0 && ((r - 1) & 1)) ? node - 1 : 0;
+    }
+    __device__ int64_t right(int64_t node, int64_t len) const {
+        const int r = rec(node, len);
+        return r == 0 ? 0 : 2 * ((node >> 1) + ((r - 1) >> 1)) + 1;
+    }
+    __device__ int64_t mid(int64_t node, int64_t len) const {
+        const int r = rec(node, len);
+        return r == 0 ? 0 : ((r - 1) & 1);
+    }
+};
+
+// One walk per sentence (pcfg_loss.cpp:22-59).  Shared by the device kernels and the host entry point.  SI = integer
+// type of the explicit stacks.
+template <typename Traces, typename SI>
+__host__ __device__ inline int64_t readout_one(int64_t pred_len, int64_t max_h, const Traces &tr, const int64_t *tok,
+                                               const int64_t *mask, int64_t mask_dim, int64_t pad, int64_t *out, SI *stack_node,
+                                               SI *stack_len, int L, int Lq) {
+    const int cap = L;
+    int sp = 0;
+    int64_t cnt = 0, node = 1, len = pred_len, last = -1;
+    if (len < 0 || len >= Lq) return -1;
+    int64_t budget = (int64_t)L * Lq + L;  // well-formed traces visit each (node, len) cell at most once
+    while ((node < max_h && node != 0) || sp > 0) {
+        if (--budget < 0) return -1;
+        while (node < max_h && node != 0) {
+            if (sp >= cap || node < 0 || node >= L || len < 0 || len >= Lq) return -1;
+            stack_node[sp] = (SI)node;
+            stack_len[sp] = (SI)len;
+            sp++;
+            int64_t l = tr.left(node, len);
+            l = (l == node) ? 0 : l;
+            if (l < 0 || l >= mask_dim || node >= mask_dim) return -1;
+            if (mask[node * mask_dim + l]) break;
+            const int64_t nl = tr.mid(node, len);
+            node = l;
+            len = nl;
+        }
+        sp--;
+        node = stack_node[sp];
+        len = stack_len[sp];
+        const int64_t t = tok[node];
+        if (t != pad && t != last) {
+            last = t;
+            if (cnt >= cap) return -1;
+            out[cnt++] = t;
+        }
+        const int64_t r = tr.right(node, len);
+        const int64_t nl = len - tr.mid(node, len) - 1;
+        node = r;
+        len = nl;
+    }
+    return cnt;
+}
+
+// Length selection (glat_decomposed_with_link_two_hands_tri_pcfg.py:489-497) by one wave: arg max over len >= 1 of
+// scores[len] / penalty[len] with NaN read as -inf, first maximum wins; every lane returns the result.
+__device__ __forceinline__ int select_length(const float *scores, const float *penalty, int Lq, int lane) {
+    float best = NEG_INF_F;
+    int idx = 0x7fffffff;
+    for (int len = 1 + lane; len < Lq; len += 64) {
+        float v = scores[len] / penalty[len];
+        v = (v != v) ? NEG_INF_F : v;
+        if (v > best) {
+            best = v;
+            idx = len;
+        }
+    }
+    const float top = wave_max(best);
+    int cand = (best == top && idx != 0x7fffffff) ? idx : 0x7fffffff;
+    for (int o = 32; o > 0; o >>= 1) cand = min(cand, __shfl_xor(cand, o));
+    return cand == 0x7fffffff ? 1 : cand;  // nothing above -inf: torch.max returns the first index
+}
+
 // NQ = number of 16-node chunks of the main chain (mc <= 16*NQ <= 256).  Row pass r handles parents 64r .. 64r+63, one
 // 16-lane row per parent; its lanes stride over the children, of which only chunks q >= 4r can hold c >= a, so the
 // triangular slabs cost NQ + (NQ-4) + (NQ-8) + ... chunk pairs of registers per thread.  Everything that does not
@@ -65,14 +158,28 @@ __device__ __forceinline__ float row16_max_raw(float v) {
 // candidates are visited in ascending (child, j) order and only a strictly larger value replaces the running best,
 // which is the reference's tie order for one lane of its strided scan; the full tie key is built once per row and used
 // in the cross-lane reduction.  LDS: three rotating columns (lengths len, len-1, len-2).
-template <int NQ>
+//
+// COMPACT = false: the reference's outputs, S and the three int64 trace tables.  COMPACT = true (whole decode in one
+// launch): the sweep only leaves one int32 per (main node, length) in a workspace and the root's scores in LDS; the
+// same workgroup then selects the output length and walks the tree.
+struct DecodeArgs {
+    const int64_t *tokens, *mask;  // [B][L], [mask_dim][mask_dim]
+    const float *penalty;          // [Lq]
+    int *W;                        // [B][L/2][Lq] workspace
+    int64_t *out_tokens, *out_count, *pred_length;
+    int64_t mask_dim, pad;
+};
+
+template <int NQ, bool COMPACT>
 __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict__ ob_lprob, const float *__restrict__ links,
                                                         const int64_t *__restrict__ out_len, float *__restrict__ S,
                                                         int64_t *__restrict__ Rt, int64_t *__restrict__ Lt, int64_t *__restrict__ Mt,
-                                                        int L, int Lq) {
+                                                        int L, int Lq, DecodeArgs dec) {
     constexpr int R = (NQ + 3) / 4;
     constexpr int MP = 64 * R;
     __shared__ float col[3 * MP];
+    extern __shared__ int dyn[];  // COMPACT: scores [Lq] (float), stacks [2][L] (int)
+    float *sm_scores = reinterpret_cast<float *>(dyn);
     const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j16 = tid & 15;
     const int m = (int)out_len[b];
     const float *ob = ob_lprob + (size_t)b * L;
@@ -80,15 +187,25 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
     const size_t tab = (size_t)b * L * Lq;
     float *Sb = S + tab;
     int64_t *Rb = Rt + tab, *Lb = Lt + tab, *Mb = Mt + tab;
+    const int rowsW = L / 2;
+    int *Wb = COMPACT ? dec.W + (size_t)b * rowsW * Lq : nullptr;
+    const bool in_contract = !(m < 2 || m > L || (m % 2) != 0);
 
-    // tables start as -inf / 0 (pcfg_viterbi.cu:159, 287-289)
-    for (size_t i = tid; i < (size_t)L * Lq; i += NT) {
-        Sb[i] = NEG_INF_F;
-        Rb[i] = 0;
-        Lb[i] = 0;
-        Mb[i] = 0;
+    if (COMPACT) {
+        for (int i = tid; i < rowsW * Lq; i += NT) Wb[i] = 0;
+        for (int i = tid; i < Lq; i += NT) sm_scores[i] = NEG_INF_F;
+        for (int i = tid; i < L; i += NT) dec.out_tokens[(size_t)b * L + i] = dec.pad;
+    } else {
+        // tables start as -inf / 0 (pcfg_viterbi.cu:159, 287-289)
+        for (size_t i = tid; i < (size_t)L * Lq; i += NT) {
+            Sb[i] = NEG_INF_F;
+            Rb[i] = 0;
+            Lb[i] = 0;
+            Mb[i] = 0;
+        }
+        if (!in_contract) return;  // out of contract: leave the empty tables
     }
-    if (m < 2 || m > L || (m % 2) != 0) return;  // out of contract: leave the empty tables
+    if (in_contract) {
     const int mc = m / 2;
 
     // slabs: unconditional loads from clamped addresses (all in flight together), masked afterwards
@@ -124,7 +241,13 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
     // length 0: nothing; length 1: only the last node (pcfg_viterbi.cu:57-59)
     for (int i = tid; i < 3 * MP; i += NT) col[i] = (i == 1 * MP + mc - 1) ? ob[m - 1] : NEG_INF_F;
     __syncthreads();
-    if (tid == 0 && Lq > 1) Sb[(size_t)(m - 1) * Lq + 1] = ob[m - 1];
+    if (tid == 0 && Lq > 1) {
+        if (COMPACT) {
+            if (m - 1 == 1) sm_scores[1] = ob[m - 1];
+        } else {
+            Sb[(size_t)(m - 1) * Lq + 1] = ob[m - 1];
+        }
+    }
 
     const int len_end = m / 4;  // pcfg_viterbi.cu:67
     int i1 = 1, i2 = 0, i0 = 2;  // column slots of len-1, len-2, len
@@ -185,11 +308,16 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
                 if (best != NEG_INF_F && a_id < mc) {  // pcfg_viterbi.cu:125-131
                     const int a = 2 * a_id + 1;
                     const int jj = key & 1, rel = (key >> 1) & 0x7fffff;
-                    const unsigned o = (unsigned)(a * Lq + len);  // 32-bit offset from the uniform table bases
-                    Sb[o] = best;
-                    Lb[o] = jj ? (a - 1) : 0;
-                    Rb[o] = 2 * (a_id + rel) + 1;
-                    Mb[o] = jj;
+                    if (COMPACT) {
+                        Wb[(unsigned)(a_id * Lq + len)] = 1 + ((rel << 1) | jj);
+                        if (a_id == 0) sm_scores[len] = best;
+                    } else {
+                        const unsigned o = (unsigned)(a * Lq + len);  // 32-bit offset from the uniform table bases
+                        Sb[o] = best;
+                        Lb[o] = jj ? (a - 1) : 0;
+                        Rb[o] = 2 * (a_id + rel) + 1;
+                        Mb[o] = jj;
+                    }
                 }
             }
         }
@@ -198,6 +326,20 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
         i1 = i0;
         i0 = t;
         lds_barrier();
+    }
+    }  // in_contract
+    if (COMPACT) {
+        __syncthreads();  // the workspace records and the padded output row are visible to the walking thread
+        if (tid < 64) {
+            const int pl = select_length(sm_scores, dec.penalty, Lq, tid);
+            if (tid == 0) {
+                int *stack_node = dyn + Lq, *stack_len = stack_node + L;
+                const CompactTraces tr{Wb, Lq, rowsW};
+                dec.pred_length[b] = pl;
+                dec.out_count[b] = readout_one(pl, out_len[b], tr, dec.tokens + (size_t)b * L, dec.mask, dec.mask_dim, dec.pad,
+                                               dec.out_tokens + (size_t)b * L, stack_node, stack_len, L, Lq);
+            }
+        }
     }
 }
 
@@ -278,47 +420,6 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_stream_kernel(const float *__r
     }
 }
 
-// One walk per sentence (pcfg_loss.cpp:22-59).  Shared by the device kernel and the host entry point.
-__host__ __device__ inline int64_t readout_one(int64_t pred_len, int64_t max_h, const int64_t *Li, const int64_t *Ri,
-                                               const int64_t *Mi, const int64_t *tok, const int64_t *mask, int64_t mask_dim,
-                                               int64_t pad, int64_t *out, int64_t *stack_node, int64_t *stack_len, int L, int Lq) {
-    const int cap = L;
-    int sp = 0;
-    int64_t cnt = 0, node = 1, len = pred_len, last = -1;
-    if (len < 0 || len >= Lq) return -1;
-    int64_t budget = (int64_t)L * Lq + L;  // well-formed traces visit each (node, len) cell at most once
-    while ((node < max_h && node != 0) || sp > 0) {
-        if (--budget < 0) return -1;
-        while (node < max_h && node != 0) {
-            if (sp >= cap || node < 0 || node >= L || len < 0 || len >= Lq) return -1;
-            stack_node[sp] = node;
-            stack_len[sp] = len;
-            sp++;
-            int64_t l = Li[node * Lq + len];
-            l = (l == node) ? 0 : l;
-            if (l < 0 || l >= mask_dim || node >= mask_dim) return -1;
-            if (mask[node * mask_dim + l]) break;
-            const int64_t nl = Mi[node * Lq + len];
-            node = l;
-            len = nl;
-        }
-        sp--;
-        node = stack_node[sp];
-        len = stack_len[sp];
-        const int64_t t = tok[node];
-        if (t != pad && t != last) {
-            last = t;
-            if (cnt >= cap) return -1;
-            out[cnt++] = t;
-        }
-        const int64_t r = Ri[node * Lq + len];
-        const int64_t nl = len - Mi[node * Lq + len] - 1;
-        node = r;
-        len = nl;
-    }
-    return cnt;
-}
-
 __global__ void readout_kernel(const int64_t *pred_length, const int64_t *output_length, const int64_t *Lt, const int64_t *Rt,
                                const int64_t *Mt, const int64_t *tokens, const int64_t *mask, int64_t mask_dim, int64_t pad,
                                int64_t *out_tokens, int64_t *out_count, int64_t *scratch, int B, int L, int Lq) {
@@ -328,8 +429,17 @@ __global__ void readout_kernel(const int64_t *pred_length, const int64_t *output
     for (int k = 0; k < L; k++) out[k] = pad;
     const size_t tab = (size_t)i * L * Lq;
     int64_t *stack_node = scratch + (size_t)i * 2 * L, *stack_len = stack_node + L;
-    out_count[i] = readout_one(pred_length[i], output_length[i], Lt + tab, Rt + tab, Mt + tab, tokens + (size_t)i * L, mask, mask_dim,
-                               pad, out, stack_node, stack_len, L, Lq);
+    const FullTraces tr{Lt + tab, Rt + tab, Mt + tab, Lq};
+    out_count[i] = readout_one(pred_length[i], output_length[i], tr, tokens + (size_t)i * L, mask, mask_dim, pad, out, stack_node,
+                               stack_len, L, Lq);
+}
+
+// Length selection on full tables (one wave per sentence): scores[len] = S[b][1][len].
+__global__ __launch_bounds__(64) void select_length_kernel(const float *__restrict__ S, const float *__restrict__ penalty,
+                                                          int64_t *__restrict__ pred_length, int L, int Lq) {
+    const int b = blockIdx.x;
+    const int pl = select_length(S + ((size_t)b * L + 1) * Lq, penalty, Lq, threadIdx.x);
+    if (threadIdx.x == 0) pred_length[b] = pl;
 }
 
 }  // namespace
@@ -350,8 +460,8 @@ extern "C" int pcfgnat_pcfg_viterbi(const float *ob_lprob, const float *links, c
     hipStream_t s = (hipStream_t)stream;
 #define PCFGNAT_VITERBI_CASE(nq)                                                                                              \
     else if (Mc <= 16 * (nq))                                                                                                \
-        hipLaunchKernelGGL((viterbi_ml1_kernel<nq>), dim3((unsigned)B), dim3(NT), 0, s, ob_lprob, links, output_length, S, R, Lt, M, \
-                           (int)L, Lq)
+        hipLaunchKernelGGL((viterbi_ml1_kernel<nq, false>), dim3((unsigned)B), dim3(NT), 0, s, ob_lprob, links, output_length, S, R, Lt, \
+                           M, (int)L, Lq, DecodeArgs{})
     if (false) {
     }
     PCFGNAT_VITERBI_CASE(2);
@@ -371,6 +481,67 @@ extern "C" int pcfgnat_pcfg_viterbi(const float *ob_lprob, const float *links, c
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
+}
+
+namespace {
+// the single-launch decode applies to max_left = 1 graphs whose slabs fit in registers
+bool decode_is_fused(int64_t L, int64_t ml) { return ml == 1 && (L - 2) / 2 + 1 <= 256; }
+}  // namespace
+
+extern "C" size_t pcfgnat_viterbi_decode_workspace_bytes(int64_t B, int64_t L, int64_t ml) {
+    if (B <= 0 || L < 4) return 0;
+    const size_t Lq = (size_t)(L / 4);
+    if (decode_is_fused(L, ml)) return (size_t)B * (size_t)(L / 2) * Lq * sizeof(int);
+    // full tables S (float) + R, L, M (int64), then the walk stacks [B][2L] int64
+    return (size_t)B * L * Lq * (sizeof(float) + 3 * sizeof(int64_t)) + (size_t)B * 2 * L * sizeof(int64_t);
+}
+
+extern "C" int pcfgnat_viterbi_decode(const float *ob_lprob, const float *links, const int64_t *output_length, const int64_t *tokens,
+                                      const int64_t *left_tree_mask, int64_t mask_dim, int64_t pad_index, const float *length_penalty,
+                                      void *workspace, int64_t *out_tokens, int64_t *out_count, int64_t *pred_length, int64_t B,
+                                      int64_t L, int64_t ml, void *stream) {
+    PCFGNAT_REQUIRE(B >= 0 && L >= 4, "viterbi_decode: need B >= 0 and L >= 4 (got B=%lld L=%lld)", (long long)B, (long long)L);
+    PCFGNAT_REQUIRE(ml >= 0 && ml <= 63 && L / 4 > ml, "viterbi_decode: max_left out of range for this graph size");
+    PCFGNAT_REQUIRE(mask_dim >= 1, "viterbi_decode: bad mask dimension");
+    if (B == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(ob_lprob && links && output_length && tokens && left_tree_mask && length_penalty && workspace && out_tokens &&
+                        out_count && pred_length,
+                    "viterbi_decode: null pointer");
+    PCFGNAT_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 7) == 0, "viterbi_decode: workspace must be 8-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    const int Lq = (int)(L / 4);
+    if (decode_is_fused(L, ml)) {
+        const int Mc = (int)((L - 2) / 2 + 1);
+        DecodeArgs dec{tokens, left_tree_mask, length_penalty, (int *)workspace, out_tokens, out_count, pred_length, mask_dim, pad_index};
+        const size_t dyn = ((size_t)Lq + 2 * (size_t)L) * sizeof(int);
+#define PCFGNAT_DECODE_CASE(nq)                                                                                                 \
+    else if (Mc <= 16 * (nq))                                                                                                   \
+        hipLaunchKernelGGL((viterbi_ml1_kernel<nq, true>), dim3((unsigned)B), dim3(NT), dyn, s, ob_lprob, links, output_length, nullptr, \
+                           nullptr, nullptr, nullptr, (int)L, Lq, dec)
+        if (false) {
+        }
+        PCFGNAT_DECODE_CASE(2);
+        PCFGNAT_DECODE_CASE(4);
+        PCFGNAT_DECODE_CASE(6);
+        PCFGNAT_DECODE_CASE(8);
+        PCFGNAT_DECODE_CASE(10);
+        PCFGNAT_DECODE_CASE(12);
+        PCFGNAT_DECODE_CASE(14);
+        PCFGNAT_DECODE_CASE(16);
+#undef PCFGNAT_DECODE_CASE
+        PCFGNAT_HIP_CHECK(hipGetLastError());
+        return PCFGNAT_OK;
+    }
+    // general path: full tables in the workspace, then selection and walk as separate launches
+    const size_t cells = (size_t)B * L * Lq;
+    int64_t *Rw = (int64_t *)workspace, *Lw = Rw + cells, *Mw = Lw + cells, *stacks = Mw + cells;
+    float *Sw = (float *)(stacks + (size_t)B * 2 * L);
+    int rc = pcfgnat_pcfg_viterbi(ob_lprob, links, output_length, Sw, Rw, Lw, Mw, B, L, ml, stream);
+    if (rc != PCFGNAT_OK) return rc;
+    hipLaunchKernelGGL(select_length_kernel, dim3((unsigned)B), dim3(64), 0, s, Sw, length_penalty, pred_length, (int)L, Lq);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return pcfgnat_viterbi_decoding(pred_length, output_length, Lw, Rw, Mw, tokens, left_tree_mask, mask_dim, pad_index, out_tokens,
+                                    out_count, stacks, B, L, Lq, stream);
 }
 
 extern "C" int pcfgnat_viterbi_decoding(const int64_t *pred_length, const int64_t *output_length, const int64_t *Lt, const int64_t *R,
@@ -403,8 +574,9 @@ extern "C" int pcfgnat_viterbi_decoding_host(const int64_t *pred_length, const i
         int64_t *out = out_tokens + (size_t)i * L;
         for (int64_t k = 0; k < L; k++) out[k] = pad_index;
         const size_t tab = (size_t)i * L * Lq;
-        out_count[i] = readout_one(pred_length[i], output_length[i], Lt + tab, R + tab, M + tab, tokens + (size_t)i * L, left_tree_mask,
-                                   mask_dim, pad_index, out, stack, stack + L, (int)L, (int)Lq);
+        const FullTraces tr{Lt + tab, R + tab, M + tab, (int)Lq};
+        out_count[i] = readout_one(pred_length[i], output_length[i], tr, tokens + (size_t)i * L, left_tree_mask, mask_dim, pad_index, out,
+                                   stack, stack + L, (int)L, (int)Lq);
     }
     free(stack);
     return PCFGNAT_OK;

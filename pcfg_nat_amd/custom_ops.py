@@ -416,6 +416,59 @@ def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unre
     return out[:, :maxlen].to(torch.float32)
 
 
+_PENALTY_CACHE = {}
+
+
+def _length_penalty(Lq, beta, device):
+    """``arange(Lq) ** beta`` as the reference computes it (glat_decomposed_with_link_two_hands_tri_pcfg.py:489-492),
+    cached per (Lq, beta, device)."""
+    key = (int(Lq), float(beta), str(device))
+    pen = _PENALTY_CACHE.get(key)
+    if pen is None:
+        pen = (torch.arange(Lq).unsqueeze(0) ** beta).to(device=device, dtype=torch.float32).contiguous().view(-1)
+        _PENALTY_CACHE[key] = pen
+    return pen
+
+
+def pcfg_viterbi_decode(unreduced_logits, links, output_length, unreduced_tokens, left_tree_mask, pad_index, beta=1.0):
+    """The model's whole Viterbi decode (glat_decomposed_with_link_two_hands_tri_pcfg.py:483-502) in one native call:
+    ``cuda_pcfg_viterbi`` -> length penalty ``arange ** beta`` -> NaN masking -> arg max over lengths >= 1 ->
+    ``viterbi_decoding``.  Returns (tokens float32 [B, maxlen] right-padded with ``pad_index``, pred_length int64 [B]),
+    the values the separate calls give."""
+    lib = get_pcfg_kernel()
+    _need_cuda("pcfg_viterbi_decode", unreduced_logits, links, output_length, unreduced_tokens, left_tree_mask)
+    if unreduced_logits.dim() != 2 or links.dim() != 4:
+        raise RuntimeError("pcfg_viterbi_decode: unreduced_logits must be [bsz, prelen] and links [bsz, prelen, max_left+1, prelen]")
+    if unreduced_logits.dtype != torch.float32 or links.dtype != torch.float32:
+        raise RuntimeError("pcfg_viterbi_decode: unreduced_logits and links must be float32")
+    B, L = unreduced_logits.shape
+    if links.size(0) != B or links.size(1) != L or links.size(3) != L:
+        raise RuntimeError("pcfg_viterbi_decode: links shape %s does not match unreduced_logits %s"
+                           % (tuple(links.shape), tuple(unreduced_logits.shape)))
+    if left_tree_mask.dim() != 2 or left_tree_mask.size(0) != left_tree_mask.size(1):
+        raise RuntimeError("pcfg_viterbi_decode: left_tree_mask must be square")
+    ml = links.size(2) - 1
+    dev = unreduced_logits.device
+    ob, links = unreduced_logits.contiguous(), links.contiguous()
+    ol = _lengths("pcfg_viterbi_decode", output_length, B)
+    tok = unreduced_tokens.to(dtype=torch.int64).contiguous()
+    mask = left_tree_mask.to(dtype=torch.int64).contiguous()
+    pen = _length_penalty(L // 4, beta, dev)
+    with torch.cuda.device(dev):
+        nbytes = lib.pcfgnat_viterbi_decode_workspace_bytes(B, L, ml)
+        work = torch.empty(((nbytes + 7) // 8,), dtype=torch.int64, device=dev)
+        out = torch.empty((B, L), dtype=torch.int64, device=dev)
+        meta = torch.empty((2, B), dtype=torch.int64, device=dev)  # row 0: emitted counts, row 1: predicted lengths
+        _lib.check(lib.pcfgnat_viterbi_decode(ob.data_ptr(), links.data_ptr(), ol.data_ptr(), tok.data_ptr(), mask.data_ptr(),
+                                              mask.size(0), int(pad_index), pen.data_ptr(), work.data_ptr(), out.data_ptr(),
+                                              meta[0].data_ptr(), meta[1].data_ptr(), B, L, ml, _stream(ob)), lib)
+    host = meta.cpu()  # one synchronising copy: counts for the trimming below, lengths for the caller
+    if B and int(host[0].min()) < 0:
+        raise RuntimeError("viterbi_decoding: malformed traces")
+    maxlen = int(host[0].max()) if B else 0
+    return out[:, :maxlen].to(torch.float32), meta[1]
+
+
 def pcfg_criterion_step(logits, targets, links, output_length, target_length, events=None, slices=None):
     """The criterion's whole training pass in one native call (``pcfgnat_criterion_step``): ``logits`` [B,L,V] (fp16 or
     fp32, contiguous) is consumed in place and holds d loss / d logits afterwards.  ``events``: optional list of eight

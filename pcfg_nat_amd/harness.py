@@ -81,9 +81,12 @@ def glat_alignment(word_ins_out, tgt_tokens, prev_output_tokens, links, context_
 
 
 def viterbi_decode(unreduced_logits, unreduced_tokens, links, output_length, left_tree_mask, pad=PAD, beta=1.0,
-                   ops=_default_ops, traces_on_host=False):
+                   ops=_default_ops, traces_on_host=False, single_call=False):
     """Viterbi decoding glue (glat_decomposed_with_link_two_hands_tri_pcfg.py:483-502): tables, length selection with the
-    ``decode_viterbibeta`` penalty, readout.  Returns (tokens float32 [B,maxlen], pred_length [B])."""
+    ``decode_viterbibeta`` penalty, readout.  ``single_call``: the same three steps as one native call
+    (``ops.pcfg_viterbi_decode``).  Returns (tokens float32 [B,maxlen], pred_length [B])."""
+    if single_call:
+        return ops.pcfg_viterbi_decode(unreduced_logits, links, output_length.long(), unreduced_tokens, left_tree_mask, pad, beta)
     prelen = unreduced_logits.shape[1]
     scores, R_trace, L_trace, M_trace = ops.cuda_pcfg_viterbi(unreduced_logits, links, output_length.long())
     lengths = torch.arange(prelen // 4, device=scores.device).unsqueeze(0)

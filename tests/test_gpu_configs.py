@@ -137,7 +137,8 @@ def test_config4_viterbi_decode():
     chunks = [srt[0:64], srt[480:544], srt[936:1000]] + [lens[i:i + 1] for i in range(12)]
     for src in chunks:
         ob, tok, links, m, mask = case(src)
-        got_tok, got_len = harness.viterbi_decode(ob, tok, links.to(DEV), m.to(DEV), mask.to(DEV))
         want_tok, want_len = harness.viterbi_decode(ob.cpu(), tok.cpu(), links, m, mask, ops=oracle_ops)
-        assert torch.equal(got_len.cpu(), want_len)
-        assert torch.equal(got_tok.cpu(), want_tok)
+        for single_call in (False, True):
+            got_tok, got_len = harness.viterbi_decode(ob, tok, links.to(DEV), m.to(DEV), mask.to(DEV), single_call=single_call)
+            assert torch.equal(got_len.cpu(), want_len)
+            assert torch.equal(got_tok.cpu(), want_tok)

@@ -317,6 +317,13 @@ def test_viterbi_tables_bit_exact_and_decode(case):
                                                   traces_on_host=on_host)
         assert torch.equal(got_len.cpu(), want_len)
         assert got_tok.dtype == torch.float32 and torch.equal(got_tok.cpu(), want_tok)
+    # the whole decode as one native call, with and without a length penalty exponent
+    for beta in (1.0, 0.7):
+        want_tok, want_len = harness.viterbi_decode(ob, tok, links, ol, left_mask, ops=oracle_ops, beta=beta)
+        got_tok, got_len = harness.viterbi_decode(ob.to(DEV), tok.to(DEV), links.to(DEV), ol.to(DEV), left_mask.to(DEV),
+                                                  beta=beta, single_call=True)
+        assert got_len.dtype == torch.int64 and torch.equal(got_len.cpu(), want_len)
+        assert got_tok.dtype == torch.float32 and torch.equal(got_tok.cpu(), want_tok)
 
 
 def test_viterbi_exact_ties_follow_reference_order():
