@@ -88,6 +88,14 @@ int pcfgnat_logsoftmax_gather_backward_lse(void *logits_inout, int dtype, const 
                                            int64_t sl, int64_t st, const void *grad_selected, const void *lse, int64_t B,
                                            int64_t L, int64_t V, int64_t T, void *stream);
 
+/*
+ * Decode front-end (glat_decomposed_with_link_two_hands_tri_pcfg.py:414-415: log_softmax followed by max over the
+ * vocabulary) in one read of the logits: best_lprob[b,p] = max_v logits[b,p,v] - log sum_v exp(logits[b,p,v]) (float32;
+ * float64 when dtype is F64), best_idx[b,p] = the first v that attains it (int64).  logits [B,L,V] contiguous.
+ */
+int pcfgnat_logsoftmax_max(const void *logits, int dtype, void *best_lprob, int64_t *best_idx, int64_t B, int64_t L,
+                           int64_t V, void *stream);
+
 /* Number of floats of the auxiliary table the inside kernels exchange (takes the place of the reference's C
  * table, pcfg_loss.cu:394, whose content for ml = 1 is a copy of match_all). */
 size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml);

@@ -27,6 +27,7 @@ SIGNATURES = {
     "pcfgnat_logsoftmax_gather": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _int, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_logsoftmax_gather_eos": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_logsoftmax_gather_backward": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "pcfgnat_logsoftmax_max": (_int, [_vp, _int, _vp, _vp, _i64, _i64, _i64, _vp]),
     "pcfgnat_logsoftmax_gather_lse": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_logsoftmax_gather_backward_lse": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_pcfg_aux_floats": (ctypes.c_size_t, [_i64, _i64, _i64, _i64]),

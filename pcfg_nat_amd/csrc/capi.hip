@@ -107,7 +107,11 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
         if (rc != PCFGNAT_OK) return rc;
         PCFGNAT_MARK(5);
         PCFGNAT_MARK(6);
-        rc = pcfgnat_logsoftmax_gather_backward_lse(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, s);
+        if (slices == 1)  // the loss is reduced by the first workgroup of the same launch (S is complete by now)
+            rc = pcfgnat::lsg_backward_lse_with_loss(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, S, Mc * (T + 2), target_length,
+                                                     loss_out, s);
+        else
+            rc = pcfgnat_logsoftmax_gather_backward_lse(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, s);
         if (rc != PCFGNAT_OK) return rc;
         PCFGNAT_MARK(7);
 #undef PCFGNAT_MARK
@@ -116,5 +120,6 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
         PCFGNAT_HIP_CHECK(hipEventRecord(h->join, h->stream));
         PCFGNAT_HIP_CHECK(hipStreamWaitEvent(main_stream, h->join, 0));
     }
+    if (slices == 1) return PCFGNAT_OK;
     return pcfgnat_criterion_loss(S, target_length, loss_out, B, L, T, ml, stream);
 }

@@ -43,6 +43,11 @@ int inside_forward_backward_impl(const float *grad_output, const float *match_al
                                  const int64_t *target_length, float *S, float *aux, float *match_all_grad, float *links_grad,
                                  int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream);
 
+// pcfgnat_logsoftmax_gather_backward_lse whose first workgroup also reduces the criterion's loss (lsg.hip)
+int lsg_backward_lse_with_loss(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
+                               const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T,
+                               const float *S, int64_t ll_stride, const int64_t *target_length, float *loss_out, void *stream);
+
 // General max_left (generic_ml.hip)
 size_t generic_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml);
 int generic_forward(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int64_t B,
@@ -114,6 +119,43 @@ __device__ __forceinline__ double wave_sum(double v) {
 }
 
 constexpr float NEG_INF_F = -__builtin_huge_valf();
+
+// The criterion's reduction (nat_pcfg_loss.py:123-135) by one workgroup of NT threads, in a fixed order:
+// out[0] = -(1/B) * sum_b [ll_b finite] ll_b / n_b, out[1] = number of sentences with a non-finite ll_b, where
+// ll_b = S[b * stride].  Every thread of the workgroup must call it.
+struct LossTask {
+    const float *S;
+    const int64_t *tgt_len;
+    float *out;  // null: nothing to do
+    int B;
+    int64_t stride;
+};
+template <int NT>
+__device__ __forceinline__ void criterion_loss_block(const LossTask &t) {
+    __shared__ float s_sum[NT];
+    __shared__ float s_bad[NT];
+    float acc = 0.f, bad = 0.f;
+    for (int b = threadIdx.x; b < t.B; b += NT) {
+        const float ll = t.S[(size_t)b * t.stride];
+        const bool ok = (ll == ll) && (fabsf(ll) != __builtin_huge_valf());
+        if (ok) acc += ll / (float)t.tgt_len[b];
+        else bad += 1.f;
+    }
+    s_sum[threadIdx.x] = acc;
+    s_bad[threadIdx.x] = bad;
+    __syncthreads();
+    for (int o = NT / 2; o > 0; o >>= 1) {
+        if ((int)threadIdx.x < o) {
+            s_sum[threadIdx.x] += s_sum[threadIdx.x + o];
+            s_bad[threadIdx.x] += s_bad[threadIdx.x + o];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        t.out[0] = -s_sum[0] / (float)t.B;
+        t.out[1] = s_bad[0];
+    }
+}
 
 // Workgroup barrier that orders LDS traffic only: outstanding global stores keep draining in the background instead
 // of being waited for (what __syncthreads() does), which matters in sweeps that write a few table cells per step.

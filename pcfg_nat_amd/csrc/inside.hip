@@ -1340,29 +1340,7 @@ __global__ void fill_zero_kernel(float *p, size_t n) {
 // in a fixed order by one workgroup.  out[0] = loss, out[1] = invalid count.
 __global__ __launch_bounds__(256) void criterion_loss_kernel(const float *__restrict__ S, const int64_t *__restrict__ tgt_len,
                                                             float *__restrict__ out, int B, int Mc, int T) {
-    __shared__ float s_sum[256];
-    __shared__ float s_bad[256];
-    float acc = 0.f, bad = 0.f;
-    for (int b = threadIdx.x; b < B; b += 256) {
-        const float ll = S[(size_t)b * Mc * (T + 2)];
-        const bool ok = (ll == ll) && (fabsf(ll) != __builtin_huge_valf());
-        if (ok) acc += ll / (float)tgt_len[b];
-        else bad += 1.f;
-    }
-    s_sum[threadIdx.x] = acc;
-    s_bad[threadIdx.x] = bad;
-    __syncthreads();
-    for (int o = 128; o > 0; o >>= 1) {
-        if ((int)threadIdx.x < o) {
-            s_sum[threadIdx.x] += s_sum[threadIdx.x + o];
-            s_bad[threadIdx.x] += s_bad[threadIdx.x + o];
-        }
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) {
-        out[0] = -s_sum[0] / (float)B;
-        out[1] = s_bad[0];
-    }
+    criterion_loss_block<256>(LossTask{S, tgt_len, out, B, (int64_t)Mc * (T + 2)});
 }
 
 int launch_fwd_stream(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B,

@@ -92,6 +92,10 @@ struct RowNorm<float> {
     __device__ __forceinline__ explicit RowNorm(float mx) : nb(-mx * 1.4426950408889634f) {}
     __device__ __forceinline__ float e(float v) const { return __builtin_amdgcn_exp2f(__builtin_fmaf(v, 1.4426950408889634f, nb)); }
     __device__ __forceinline__ float lse(float sum) const { return (__builtin_amdgcn_logf(sum) - nb) * 0.6931471805599453f; }
+    // v - lse(sum) without the cancellation of two large numbers
+    __device__ __forceinline__ float logprob(float v, float sum) const {
+        return (__builtin_fmaf(v, 1.4426950408889634f, nb) - __builtin_amdgcn_logf(sum)) * 0.6931471805599453f;
+    }
     // exp(v - l) for a given log-sum-exp l
     __device__ static __forceinline__ RowNorm from_lse(float l) { return RowNorm(l); }
 };
@@ -101,6 +105,7 @@ struct RowNorm<double> {
     __device__ __forceinline__ explicit RowNorm(double m) : mx(m) {}
     __device__ __forceinline__ double e(double v) const { return exp(v - mx); }
     __device__ __forceinline__ double lse(double sum) const { return mx + log(sum); }
+    __device__ __forceinline__ double logprob(double v, double sum) const { return (v - mx) - log(sum); }
     __device__ static __forceinline__ RowNorm from_lse(double l) { return RowNorm(l); }
 };
 
@@ -222,19 +227,17 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
         const RowSplit<T> sp(xr, V);
         const vec16 *xv = reinterpret_cast<const vec16 *>(xr + sp.head);
 
-        // gathered logits first: they must be read before this workgroup overwrites the row
-        CT gv[GMAX];
+        // Load order: target indices, then the whole row, then the gathered logits.  The gathers depend on the indices;
+        // issued before the row they would hold its loads back by one memory round trip per row.  They still complete
+        // before anything is stored to the row (the stores come after two workgroup reductions over the loaded data).
+        int64_t tg[GMAX];
         {
             const int64_t b = row / L, p = row % L;
             const int64_t *ir = idx + b * sb + p * sl;
 #pragma unroll
             for (int g = 0; g < GMAX; g++) {
-                int s = tid + g * NT;
-                gv[g] = 0;
-                if (s < Tn) {
-                    int64_t t = ir[(int64_t)s * st];
-                    gv[g] = ((uint64_t)t < (uint64_t)V) ? Elem<T>::widen(xr[t]) : (CT)NAN;
-                }
+                const int s = tid + g * NT;
+                tg[g] = (s < Tn) ? ir[(int64_t)s * st] : 0;
             }
         }
         vec16 buf[MAXC];
@@ -246,6 +249,13 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
         const int ep = sp.edge_pos(tid);
         CT edge = neg_inf(CT());
         if (ep >= 0) edge = Elem<T>::widen(xr[ep]);
+        CT gv[GMAX];
+#pragma unroll
+        for (int g = 0; g < GMAX; g++) {
+            const int s = tid + g * NT;
+            gv[g] = 0;
+            if (s < Tn) gv[g] = ((uint64_t)tg[g] < (uint64_t)V) ? Elem<T>::widen(xr[tg[g]]) : (CT)NAN;
+        }
 
         // ---- max
         RowMax<T> rmax;
@@ -291,7 +301,7 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
             int s = tid + g * NT;
-            if (s < Tn) sel[row * (int64_t)Tn + s] = (s == eos_col) ? neg_inf(CT()) : gv[g] - row_lse;
+            if (s < Tn) sel[row * (int64_t)Tn + s] = (s == eos_col) ? neg_inf(CT()) : rn.logprob(gv[g], sum);
         }
 
         if (GRAD) {
@@ -320,6 +330,98 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
     }
 }
 
+// Decode front-end: best token of every row and its log-probability, max_v log_softmax(x)[v] and the first arg max
+// (glat_decomposed_with_link_two_hands_tri_pcfg.py:414-415), in one read of the logits instead of materialising the
+// log-softmax.  Same row-in-registers structure as the gather forward; the position of the maximum is recovered by
+// the (usually single) thread whose own maximum equals the row's.
+template <typename T, int NT, int MAXC>
+__global__ __launch_bounds__(NT) void ls_max_kernel(const T *__restrict__ x, typename Elem<T>::compute *__restrict__ best_lprob,
+                                                    int64_t *__restrict__ best_idx, int64_t rows, int V) {
+    using CT = typename Elem<T>::compute;
+    constexpr int EPV = Elem<T>::EPV;
+    constexpr int NW = NT / 64;
+    __shared__ CT s_max[NW];
+    __shared__ CT s_sum[NW];
+    __shared__ int s_arg;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const T *xr = x + row * (int64_t)V;
+        const RowSplit<T> sp(xr, V);
+        const vec16 *xv = reinterpret_cast<const vec16 *>(xr + sp.head);
+        vec16 buf[MAXC];
+#pragma unroll
+        for (int i = 0; i < MAXC; i++) {
+            int c = tid + i * NT;
+            if (c < sp.nvec) buf[i] = load16(xv + c);
+        }
+        const int ep = sp.edge_pos(tid);
+        CT edge = neg_inf(CT());
+        if (ep >= 0) edge = Elem<T>::widen(xr[ep]);
+        if (tid == 0) s_arg = 0x7fffffff;
+
+        RowMax<T> rmax;
+        if (ep >= 0) rmax.scalar(xr[ep]);
+#pragma unroll
+        for (int i = 0; i < MAXC; i++)
+            if (tid + i * NT < sp.nvec) rmax.chunk(buf[i]);
+        for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) rmax.chunk(load16(xv + c));
+        const CT mine = rmax.value();
+        const CT mx = block_max<CT, NW>(mine, s_max, wave, lane);  // barrier inside: s_arg is initialised
+        const RowNorm<CT> rn(mx);
+#pragma unroll
+        for (int i = 0; i < MAXC; i++) opaque(buf[i]);
+
+        if (mine == mx) {  // first position of the maximum among this thread's elements
+            int first = 0x7fffffff;
+            if (ep >= 0 && edge == mx) first = ep;
+#pragma unroll
+            for (int i = 0; i < MAXC; i++) {
+                const int c = tid + i * NT;
+                if (c < sp.nvec) {
+                    CT v[EPV];
+                    Elem<T>::unpack(buf[i], v);
+#pragma unroll
+                    for (int e = EPV - 1; e >= 0; e--)
+                        if (v[e] == mx) first = min(first, sp.head + c * EPV + e);
+                }
+            }
+            for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
+                CT v[EPV];
+                Elem<T>::unpack(load16(xv + c), v);
+#pragma unroll
+                for (int e = EPV - 1; e >= 0; e--)
+                    if (v[e] == mx) first = min(first, sp.head + c * EPV + e);
+            }
+            atomicMin(&s_arg, first);
+        }
+
+        CT sum = (ep >= 0) ? rn.e(edge) : (CT)0;
+#pragma unroll
+        for (int i = 0; i < MAXC; i++) {
+            if (tid + i * NT < sp.nvec) {
+                CT v[EPV];
+                Elem<T>::unpack(buf[i], v);
+#pragma unroll
+                for (int e = 0; e < EPV; e++) sum += rn.e(v[e]);
+            }
+        }
+        for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
+            CT v[EPV];
+            Elem<T>::unpack(load16(xv + c), v);
+#pragma unroll
+            for (int e = 0; e < EPV; e++) sum += rn.e(v[e]);
+        }
+        sum = block_sum<CT, NW>(sum, s_sum, wave, lane);  // barrier inside: s_arg is final
+        if (tid == 0) {
+            best_lprob[row] = rn.logprob(mx, sum);
+            // a row whose maximum is NaN-free but never found (all NaN) keeps index 0, like an all-equal row
+            best_idx[row] = (s_arg == 0x7fffffff) ? 0 : s_arg;
+        }
+        __syncthreads();  // s_arg and the reduction slots are reused by the next row
+    }
+}
+
 // In-place backward.  TCAP = most targets per row handled through LDS; up to MAXC chunks per thread are in flight.
 // FROM_LOGITS = false: the buffer holds the probabilities the forward left (reference split, with the reference's
 // roundings to the buffer dtype); true: it holds the untouched logits and `lse` the row log-sum-exps.
@@ -328,10 +430,11 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
                                                      int64_t sl, int64_t st,
                                                      const typename Elem<T>::compute *__restrict__ gsel, int64_t rows,
                                                      int L, int V, int Tn,
-                                                     const typename Elem<T>::compute *__restrict__ lse) {
+                                                     const typename Elem<T>::compute *__restrict__ lse, LossTask loss) {
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
     constexpr int FIX = (TCAP + NT - 1) / NT;
+    if (loss.out != nullptr && blockIdx.x == 0) criterion_loss_block<NT>(loss);  // workgroup-uniform
     __shared__ int s_idx[TCAP];
     __shared__ CT s_g[TCAP];   // cast(g[s]) in the buffer's dtype, widened again
     __shared__ CT s_p[TCAP];   // original probability at idx[s]
@@ -455,7 +558,7 @@ int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
 
 template <typename T>
 int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, const void *g, int64_t rows, int L, int V,
-               int Tn, const void *lse, hipStream_t stream) {
+               int Tn, const void *lse, const LossTask &loss, hipStream_t stream) {
     using CT = typename Elem<T>::compute;
     constexpr int NT = 512;
     constexpr int MAXC = 10;
@@ -464,10 +567,22 @@ int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
     int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
     if (lse != nullptr)
         hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, true>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,
-                           (const CT *)g, rows, L, V, Tn, (const CT *)lse);
+                           (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss);
     else
         hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, false>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl,
-                           st, (const CT *)g, rows, L, V, Tn, (const CT *)nullptr);
+                           st, (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
+template <typename T>
+int launch_ls_max(const void *x, void *best_lprob, int64_t *best_idx, int64_t rows, int V, hipStream_t stream) {
+    using CT = typename Elem<T>::compute;
+    constexpr int NT = 512;
+    constexpr int MAXC = 10;
+    int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
+    hipLaunchKernelGGL((ls_max_kernel<T, NT, MAXC>), dim3((unsigned)grid), dim3(NT), 0, stream, (const T *)x, (CT *)best_lprob, best_idx,
+                       rows, V);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -532,19 +647,35 @@ extern "C" int pcfgnat_logsoftmax_gather_lse(const void *word_ins_out, int dtype
                                 target_length, lse, stream);
 }
 
+extern "C" int pcfgnat_logsoftmax_max(const void *logits, int dtype, void *best_lprob, int64_t *best_idx, int64_t B, int64_t L,
+                                      int64_t V, void *stream) {
+    PCFGNAT_REQUIRE(B >= 0 && L >= 0 && V >= 1 && V < (1LL << 31), "logsoftmax_max: bad dimensions (B=%lld L=%lld V=%lld)", (long long)B,
+                    (long long)L, (long long)V);
+    if (B * L == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(logits && best_lprob && best_idx, "logsoftmax_max: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case PCFGNAT_F16: return launch_ls_max<__half>(logits, best_lprob, best_idx, B * L, (int)V, s);
+        case PCFGNAT_F32: return launch_ls_max<float>(logits, best_lprob, best_idx, B * L, (int)V, s);
+        case PCFGNAT_F64: return launch_ls_max<double>(logits, best_lprob, best_idx, B * L, (int)V, s);
+        default: return fail(PCFGNAT_EINVAL, "logsoftmax_max: unknown dtype code %d", dtype);
+    }
+}
+
 static int lsg_backward_dispatch(void *buf, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
-                                 const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T, void *stream) {
+                                 const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T, void *stream,
+                                 const LossTask &loss = LossTask{nullptr, nullptr, nullptr, 0, 0}) {
     int rc = check_common(buf, select_idx, grad_selected, B, L, V, T);
     if (rc != PCFGNAT_OK) return rc;
     if (B * L == 0) return PCFGNAT_OK;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case PCFGNAT_F16:
-            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, s);
+            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s);
         case PCFGNAT_F32:
-            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, s);
+            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s);
         case PCFGNAT_F64:
-            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, s);
+            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s);
         default:
             return fail(PCFGNAT_EINVAL, "logsoftmax_gather_backward: unknown dtype code %d", dtype);
     }
@@ -554,6 +685,15 @@ extern "C" int pcfgnat_logsoftmax_gather_backward(void *probs_inout, int dtype, 
                                                   int64_t sl, int64_t st, const void *grad_selected, int64_t B, int64_t L,
                                                   int64_t V, int64_t T, void *stream) {
     return lsg_backward_dispatch(probs_inout, dtype, select_idx, sb, sl, st, grad_selected, nullptr, B, L, V, T, stream);
+}
+
+int pcfgnat::lsg_backward_lse_with_loss(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
+                                        const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T,
+                                        const float *S, int64_t ll_stride, const int64_t *target_length, float *loss_out,
+                                        void *stream) {
+    PCFGNAT_REQUIRE(B >= 1 && L >= 1 && lse && S && target_length && loss_out, "logsoftmax_gather_backward: null pointer or empty batch");
+    return lsg_backward_dispatch(logits_inout, dtype, select_idx, sb, sl, st, grad_selected, lse, B, L, V, T, stream,
+                                 LossTask{S, target_length, loss_out, (int)B, ll_stride});
 }
 
 extern "C" int pcfgnat_logsoftmax_gather_backward_lse(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb,

@@ -308,6 +308,26 @@ def _logsoftmax_gather(word_ins_out, select_idx, require_gradient, eos_lengths=N
     return selected
 
 
+def logsoftmax_max(logits):
+    """``logits.log_softmax(-1).max(-1)`` (glat_decomposed_with_link_two_hands_tri_pcfg.py:414-415) in one read of the
+    logits: returns (best log-probability [B,L] float32 - float64 for float64 logits -, first arg max [B,L] int64)."""
+    lib = get_pcfg_kernel()
+    _need_cuda("logsoftmax_max", logits)
+    if logits.dim() != 3 or not logits.is_contiguous():
+        raise RuntimeError("logsoftmax_max: logits must be a contiguous [bsz, prelen, vocab] tensor")
+    code = _DTYPE_CODE.get(logits.dtype)
+    if code is None:
+        raise RuntimeError("logsoftmax_max: unsupported dtype %s (float16, float32, float64 are dispatched)" % logits.dtype)
+    B, L, V = logits.shape
+    out_dtype = torch.float64 if logits.dtype == torch.float64 else torch.float32
+    with torch.cuda.device(logits.device):
+        best = torch.empty((B, L), dtype=out_dtype, device=logits.device)
+        idx = torch.empty((B, L), dtype=torch.int64, device=logits.device)
+        _lib.check(lib.pcfgnat_logsoftmax_max(logits.data_ptr(), code, best.data_ptr(), idx.data_ptr(), B, L, V,
+                                              _stream(logits)), lib)
+    return best, idx
+
+
 def _logsoftmax_gather_lse(word_ins_out, select_idx, eos_lengths=None):
     """Read-only forward of the log-sum-exp split: returns (selected [B,L,T], row log-sum-exp [B,L]); same checks as
     ``_logsoftmax_gather``.  ``word_ins_out`` must stay untouched until ``_logsoftmax_gather_backward_lse`` consumes it."""

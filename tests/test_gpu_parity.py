@@ -135,6 +135,25 @@ def test_lsg_lse_split_matches_autograd(dtype, V):
         assert torch.allclose(got, leaf.grad, rtol=1e-12, atol=1e-14)
 
 
+@pytest.mark.parametrize("dtype,V", [(torch.float16, 40000), (torch.float16, 333), (torch.float32, 1001), (torch.float64, 257),
+                                     (torch.float16, 48000)])
+def test_logsoftmax_max_matches_torch(dtype, V):
+    g = torch.Generator().manual_seed(V)
+    B, L = 2, 5
+    x = (torch.randn(B, L, V, generator=g) * 3).to(dtype)
+    x[0, 1, 7] = x[0, 1].max()   # exact ties: the first position wins
+    x[0, 1, V - 3] = x[0, 1, 7]
+    x[1, 2, :] = 0.5             # a constant row
+    x[1, 3, 5:9] = -math.inf
+    best, idx = ops.logsoftmax_max(x.to(DEV))
+    want_best, want_idx = torch.log_softmax(x.double(), -1).max(-1)
+    first = (x == x.max(-1, keepdim=True)[0]).int().argmax(-1)   # first maximum
+    assert torch.equal(idx.cpu(), first)
+    assert torch.equal(x.gather(-1, idx.cpu().unsqueeze(-1)), x.gather(-1, want_idx.unsqueeze(-1)))
+    tol = 1e-12 if dtype == torch.float64 else 2e-6
+    assert torch.allclose(best.cpu().double(), want_best, rtol=tol, atol=tol)
+
+
 def test_lsg_autograd_contract():
     g = torch.Generator().manual_seed(2)
     B, L, V, T = 2, 4, 640, 5
