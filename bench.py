@@ -24,7 +24,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # plain device copy of known size; summary in profiles/lsg_cfg2_hbm_traffic_pmc.md.  None = not measured for this build.
 ROOFLINE_KERNEL = {"single": "lsg_bwd", "fused": "lsg_bwd", "unfused": "lsg_fwd"}
 ROOFLINE_KERNEL_NAME = {"lsg_bwd": "lsg_bwd_kernel<half, from logits>", "lsg_fwd": "lsg_fwd_kernel<half, grad>"}
-MEASURED_TRAFFIC_BYTES = {"lsg_bwd": None, "lsg_fwd": 820.75e6}
+MEASURED_TRAFFIC_BYTES = {"lsg_bwd": 831.36e6, "lsg_fwd": None}
 
 
 def parse():

@@ -466,8 +466,8 @@ __device__ __forceinline__ void bwd_sweep(const float (&A0)[R][8 * R], const flo
                 if (q < q_end) {
                     const float e0 = ex2(v0[q] - mxs), e1 = ex2(v1[q] - mxs);
                     sum += e0 + e1;
-                    G0[r][q] += e0 * scale;
-                    G1[r][q] += e1 * scale;
+                    G0[r][q] = __builtin_fmaf(e0, scale, G0[r][q]);
+                    G1[r][q] = __builtin_fmaf(e1, scale, G1[r][q]);
                 }
             }
             sum = row8_sum(sum);
