@@ -163,6 +163,26 @@ int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, cons
                            int64_t L, int64_t V, int64_t T, int64_t ml, int64_t slices, void *stream, void *const *events);
 
 /*
+ * GLAT glancing with the `number-random` strategy (nat_pcfg_loss.py:193-269) in one call: lengths from the pad counts
+ * (:195-196), arg max of the logits (:199), logsoftmax_gather without gradient + eos mask (:200-207), best-tree alignment
+ * (:210), and everything the criterion derives from the alignment (:212-255).
+ *   logits [B,L,V] (F16/F32/F64, read only); targets [B,T], prev_output_tokens [B,L] int64; links [B,L,ml+1,L] float32;
+ *   noise [B,L] float32: the caller's randn draw of :235 (the uniform draw of :253 cannot change the result, because
+ *   keep_prob is 0 or 1; the caller still makes it to keep its random stream in step); context_p: glancing ratio.
+ * Workspaces: match_all [B,L,T], S [B,Mc,T+2], aux [pcfgnat_pcfg_aux_floats] float32; pred_tokens [B,L], lengths [2,B] int64.
+ * Outputs: path [B,L] int64 (target position of every node, -1 off the tree); matchmask [B,T,L], keep_word_mask [B,L]
+ * (one byte per flag, 0/1); glat_prev_output_tokens [B,L], same_num [B], glance_nums [B] int64; loss_out[0] =
+ * -(ll/target_length).mean() over sentences with a finite best-tree likelihood ll = S[b,0,0], loss_out[1] = number of
+ * the others.  On return lengths[0,:] = output_length and lengths[1,:] = target_length.
+ */
+int pcfgnat_glat_step(const void *logits, int dtype, const int64_t *targets, const int64_t *prev_output_tokens,
+                      const float *links, const float *noise, float context_p, int64_t pad_index, float *match_all, float *S,
+                      float *aux, int64_t *pred_tokens, int64_t *lengths, int64_t *path, unsigned char *matchmask,
+                      unsigned char *keep_word_mask, int64_t *glat_prev_output_tokens, int64_t *same_num,
+                      int64_t *glance_nums, float *loss_out, int64_t B, int64_t L, int64_t V, int64_t T, int64_t ml,
+                      void *stream);
+
+/*
  * Replaces pcfg_best_tree (pcfg_best_tree.cu:333-360): greedy top-down trace over the inside tables.
  *   tree [B,L] int64 out: target position aligned to each node, -1 for nodes off the tree.
  * Exact ties are resolved in the reference's scan order (lanes 0 > 2 > 1 > 3 of a 4-wide strided scan).

@@ -864,7 +864,7 @@ __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__re
 }
 
 // ------------------------------------------------------------------------------------------------------------
-// Best tree (pcfg_best_tree.cu:64-197, 239-301): a single top-down chain per sentence, one wave64 per sentence.
+// Best tree (pcfg_best_tree.cu:64-197, 239-301): a single top-down chain per sentence, walked by one wave64.
 // Candidate order for exact ties: lane = (c_id - a_id - 1) & 3 with priority 0 > 2 > 1 > 3, then c ascending, then
 // (j=0,k=0) before (j=1,k=1).
 // ------------------------------------------------------------------------------------------------------------
@@ -874,49 +874,87 @@ __device__ __forceinline__ int tie_key(int rel_c, int j) {
     return (rank << 24) | (rel_c << 1) | j;
 }
 
-__global__ __launch_bounds__(64) void best_tree_ml1_kernel(const float *__restrict__ S, const float *__restrict__ match_all,
-                                                          const float *__restrict__ links, const int64_t *__restrict__ out_len,
-                                                          const int64_t *__restrict__ tgt_len, int64_t *__restrict__ tree, int L,
-                                                          int T, int Mc) {
-    const int b = blockIdx.x, lane = threadIdx.x;
+// 256 threads stage the sentence's inside table and its emissions (MODE >= 1) and its compact link matrices (MODE 2) in
+// LDS; the first wave then walks the chain without touching global memory.  MODE 0 reads everything from global memory
+// (tables too large for LDS).  Dynamic LDS: S [Mc][T+2], main/leaf emissions [Mc][T] each, matrices [2][Mc][Mc].
+constexpr int BT_NT = 256;
+template <int MODE>
+__global__ __launch_bounds__(BT_NT) void best_tree_ml1_kernel(const float *__restrict__ S, const float *__restrict__ match_all,
+                                                             const float *__restrict__ links, const int64_t *__restrict__ out_len,
+                                                             const int64_t *__restrict__ tgt_len, int64_t *__restrict__ tree, int L,
+                                                             int T, int Mc) {
+    constexpr bool TAB_LDS = MODE >= 1, LINKS_LDS = MODE == 2;
+    extern __shared__ float smem[];
+    const int TS = T + 2;
+    float *sS = smem;                  // [Mc][TS]
+    float *sMain = sS + Mc * TS;       // [Mc][T]
+    float *sLeaf = sMain + Mc * T;     // [Mc][T]
+    float *sA0 = sLeaf + Mc * T;       // [Mc][Mc]  (LINKS_LDS)
+    float *sA1 = sA0 + (LINKS_LDS ? Mc * Mc : 0);
+    const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const float *mt = match_all + (size_t)b * L * T;
     const float *lk = links + (size_t)b * L * 2 * L;
-    const float *Sb = S + (size_t)b * Mc * (T + 2);
+    const float *Sb = S + (size_t)b * Mc * TS;
     int64_t *tr = tree + (size_t)b * L;
-    for (int i = lane; i < L; i += 64) tr[i] = -1;
+    for (int i = tid; i < L; i += BT_NT) tr[i] = -1;
     if (!lengths_ok(m, n, L, T)) return;
     const int mc = m / 2;
+    if (TAB_LDS) {
+        for (int i = tid; i < mc * TS; i += BT_NT) sS[i] = Sb[i];
+        for (int i = tid; i < mc * T; i += BT_NT) {
+            const int a_id = i / T, t = i - a_id * T;
+            sMain[i] = mt[(size_t)(2 * a_id + 1) * T + t];
+            sLeaf[i] = mt[(size_t)(2 * a_id) * T + t];
+        }
+    }
+    auto s_at = [&](int c_id, int t) -> float { return TAB_LDS ? sS[c_id * TS + t] : Sb[(size_t)c_id * TS + t]; };
+    auto main_at = [&](int x_id, int t) -> float { return TAB_LDS ? sMain[x_id * T + t] : mt[(size_t)(2 * x_id + 1) * T + t]; };
+    auto leaf_at = [&](int x_id, int t) -> float { return TAB_LDS ? sLeaf[x_id * T + t] : mt[(size_t)(2 * x_id) * T + t]; };
+    if (LINKS_LDS) {
+        for (int i = tid; i < mc * mc; i += BT_NT) {
+            const int a_id = i / mc, c_id = i - a_id * mc;
+            const size_t row = (size_t)(2 * a_id + 1) * 2;
+            sA0[a_id * Mc + c_id] = lk[(row + 0) * L + 2 * c_id + 1];
+            sA1[a_id * Mc + c_id] = lk[(row + 1) * L + 2 * c_id + 1];
+        }
+    }
+    __syncthreads();  // orders the -1 fill of `tree` before the chain's stores as well
+    if (tid >= 64) return;
     int a_id = 0, s = 0;
     // every marked cell (a, s) has s <= n by construction; the loop is bounded by the number of main-chain nodes
     for (int hop = 0; hop < mc; hop++) {
         const int a = 2 * a_id + 1;
         float best = NEG_INF_F;
-        int best_key = 0x7fffffff, best_c = -1, best_j = 0;
-        const float ma_s = (s < n) ? mt[(size_t)a * T + s] : NEG_INF_F;
+        int best_key = 0x7fffffff;
+        const float ma_s = (s < n) ? main_at(a_id, s) : NEG_INF_F;
         const bool j1 = (n - s > 1) && a_id >= 1;
-        const float ml_s = j1 ? mt[(size_t)(a - 1) * T + s] : NEG_INF_F;
-        const float ma_s1 = j1 ? mt[(size_t)a * T + s + 1] : NEG_INF_F;
+        const float ml_s = j1 ? leaf_at(a_id, s) : NEG_INF_F;
+        const float ma_s1 = j1 ? main_at(a_id, s + 1) : NEG_INF_F;
         for (int c_id = a_id + 1 + lane; c_id < mc; c_id += 64) {
             const int c = 2 * c_id + 1;
             if (s < n) {  // j = 0, null left child: ((links + S) + C[0][s][0]) + match, C = 0
-                float v = ((lk[((size_t)a * 2 + 0) * L + c] + Sb[(size_t)c_id * (T + 2) + s + 1]) + 0.f) + ma_s;
+                const float l0 = LINKS_LDS ? sA0[a_id * Mc + c_id] : lk[((size_t)a * 2 + 0) * L + c];
+                float v = ((l0 + s_at(c_id, s + 1)) + 0.f) + ma_s;
                 if (v != v) v = NEG_INF_F;
                 const int key = tie_key(c_id - a_id - 1, 0);
-                if (v > best || (v == best && v != NEG_INF_F && key < best_key)) { best = v; best_key = key; best_c = c_id; best_j = 0; }
+                if (v > best || (v == best && v != NEG_INF_F && key < best_key)) { best = v; best_key = key; }
             }
             if (j1) {  // j = 1, leaf a-1 emits s: ((links + S) + match[a-1][s]) + match[a][s+1]
-                float v = ((lk[((size_t)a * 2 + 1) * L + c] + Sb[(size_t)c_id * (T + 2) + s + 2]) + ml_s) + ma_s1;
+                const float l1 = LINKS_LDS ? sA1[a_id * Mc + c_id] : lk[((size_t)a * 2 + 1) * L + c];
+                float v = ((l1 + s_at(c_id, s + 2)) + ml_s) + ma_s1;
                 if (v != v) v = NEG_INF_F;
                 const int key = tie_key(c_id - a_id - 1, 1);
-                if (v > best || (v == best && v != NEG_INF_F && key < best_key)) { best = v; best_key = key; best_c = c_id; best_j = 1; }
+                if (v > best || (v == best && v != NEG_INF_F && key < best_key)) { best = v; best_key = key; }
             }
         }
-        for (int o = 32; o > 0; o >>= 1) {
-            const float ov = __shfl_xor(best, o);
-            const int ok = __shfl_xor(best_key, o), oc = __shfl_xor(best_c, o), oj = __shfl_xor(best_j, o);
-            if (ov > best || (ov == best && ov != NEG_INF_F && ok < best_key)) { best = ov; best_key = ok; best_c = oc; best_j = oj; }
-        }
+        // wave arg max: the maximum first, then the smallest tie key among the lanes that hold it
+        const float top = wave_max(best);
+        int key = (best == top && best != NEG_INF_F) ? best_key : 0x7fffffff;
+        for (int o = 32; o > 0; o >>= 1) key = min(key, __shfl_xor(key, o));
+        const bool found = key != 0x7fffffff;
+        const int best_j = found ? (key & 1) : 0;
+        const int best_c = found ? a_id + 1 + ((key >> 1) & 0x7fffff) : -1;
         if (lane == 0) {
             tr[a] = s + best_j;                            // pcfg_best_tree.cu:182
             if (best_c >= 0 && best_j == 1 && s < n - 2) tr[a - 1] = s;  // leaf cell (b, s, 1), :268-297 with i < n-gap-1
@@ -1567,8 +1605,22 @@ extern "C" int pcfgnat_pcfg_best_tree(const float *S, float *aux, const float *m
         return generic_best_tree(S, aux, match_all, links, output_length, target_length, tree, B, L, T, ml, stream);
     }
     const int Mc = (int)((L - 2) / 2 + 1);
-    hipLaunchKernelGGL(best_tree_ml1_kernel, dim3((unsigned)B), dim3(64), 0, (hipStream_t)stream, S, match_all, links, output_length,
-                       target_length, tree, (int)L, (int)T, Mc);
+    const size_t tables = ((size_t)Mc * (T + 2) + (size_t)2 * Mc * T) * sizeof(float);
+    const size_t with_links = tables + (size_t)2 * Mc * Mc * sizeof(float);
+    if (with_links <= LDS_BUDGET) {
+        auto k = best_tree_ml1_kernel<2>;
+        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_links));
+        hipLaunchKernelGGL(k, dim3((unsigned)B), dim3(BT_NT), with_links, (hipStream_t)stream, S, match_all, links, output_length,
+                           target_length, tree, (int)L, (int)T, Mc);
+    } else if (tables <= LDS_BUDGET) {
+        auto k = best_tree_ml1_kernel<1>;
+        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)tables));
+        hipLaunchKernelGGL(k, dim3((unsigned)B), dim3(BT_NT), tables, (hipStream_t)stream, S, match_all, links, output_length,
+                           target_length, tree, (int)L, (int)T, Mc);
+    } else {
+        hipLaunchKernelGGL(best_tree_ml1_kernel<0>, dim3((unsigned)B), dim3(BT_NT), 0, (hipStream_t)stream, S, match_all, links,
+                           output_length, target_length, tree, (int)L, (int)T, Mc);
+    }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }

@@ -207,6 +207,35 @@ __device__ __forceinline__ CT block_sum(CT v, CT *slots, int wave, int lane) {
     return r;
 }
 
+// First position, among the elements this thread holds, whose value equals the row maximum (0x7fffffff if none).
+template <typename T, int NT, int MAXC>
+__device__ __forceinline__ int first_pos_of_max(const vec16 (&buf)[MAXC], const RowSplit<T> &sp, const vec16 *xv, int tid, int ep,
+                                                typename Elem<T>::compute edge, typename Elem<T>::compute mx) {
+    using CT = typename Elem<T>::compute;
+    constexpr int EPV = Elem<T>::EPV;
+    int first = 0x7fffffff;
+    if (ep >= 0 && edge == mx) first = ep;
+#pragma unroll
+    for (int i = 0; i < MAXC; i++) {
+        const int c = tid + i * NT;
+        if (c < sp.nvec) {
+            CT v[EPV];
+            Elem<T>::unpack(buf[i], v);
+#pragma unroll
+            for (int e = EPV - 1; e >= 0; e--)
+                if (v[e] == mx) first = min(first, sp.head + c * EPV + e);
+        }
+    }
+    for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
+        CT v[EPV];
+        Elem<T>::unpack(load16(xv + c), v);
+#pragma unroll
+        for (int e = EPV - 1; e >= 0; e--)
+            if (v[e] == mx) first = min(first, sp.head + c * EPV + e);
+    }
+    return first;
+}
+
 // NT threads; up to MAXC 16-byte chunks per thread stay in registers, GMAX gathered targets per thread.
 template <typename T, int NT, int MAXC, int GMAX, bool GRAD>
 __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const int64_t *__restrict__ idx, int64_t sb,
@@ -214,12 +243,14 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
                                                      typename Elem<T>::compute *__restrict__ sel, int64_t rows, int L,
                                                      int V, int Tn, const int64_t *__restrict__ eos_out_len,
                                                      const int64_t *__restrict__ eos_tgt_len,
-                                                     typename Elem<T>::compute *__restrict__ lse_out) {
+                                                     typename Elem<T>::compute *__restrict__ lse_out,
+                                                     int64_t *__restrict__ argmax_out) {
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
     constexpr int NW = NT / 64;
     __shared__ CT s_max[NW];
     __shared__ CT s_sum[NW];
+    __shared__ int s_arg;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
@@ -264,10 +295,14 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
         for (int i = 0; i < MAXC; i++)
             if (tid + i * NT < sp.nvec) rmax.chunk(buf[i]);
         for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) rmax.chunk(load16(xv + c));
-        const CT mx = block_max<CT, NW>(rmax.value(), s_max, wave, lane);
+        if (argmax_out != nullptr && tid == 0) s_arg = 0x7fffffff;
+        const CT mine = rmax.value();
+        const CT mx = block_max<CT, NW>(mine, s_max, wave, lane);  // barrier inside
         const RowNorm<CT> rn(mx);
 #pragma unroll
         for (int i = 0; i < MAXC; i++) opaque(buf[i]);
+        // optional arg max of the row (first maximum): found by the threads whose own maximum is the row's
+        if (argmax_out != nullptr && mine == mx) atomicMin(&s_arg, first_pos_of_max<T, NT, MAXC>(buf, sp, xv, tid, ep, edge, mx));
 
         // ---- sum of exp
         CT sum = (ep >= 0) ? rn.e(edge) : (CT)0;
@@ -287,8 +322,9 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
             for (int e = 0; e < EPV; e++) sum += rn.e(v[e]);
         }
         sum = block_sum<CT, NW>(sum, s_sum, wave, lane);
-        const CT row_lse = rn.lse(sum);
+        const CT row_lse = rn.lse(sum);  // (the reduction's barrier also completes s_arg)
         if (lse_out != nullptr && tid == 0) lse_out[row] = row_lse;
+        if (argmax_out != nullptr && tid == 0) argmax_out[row] = (s_arg == 0x7fffffff) ? 0 : s_arg;
 #pragma unroll
         for (int i = 0; i < MAXC; i++) opaque(buf[i]);
 
@@ -372,29 +408,7 @@ __global__ __launch_bounds__(NT) void ls_max_kernel(const T *__restrict__ x, typ
 #pragma unroll
         for (int i = 0; i < MAXC; i++) opaque(buf[i]);
 
-        if (mine == mx) {  // first position of the maximum among this thread's elements
-            int first = 0x7fffffff;
-            if (ep >= 0 && edge == mx) first = ep;
-#pragma unroll
-            for (int i = 0; i < MAXC; i++) {
-                const int c = tid + i * NT;
-                if (c < sp.nvec) {
-                    CT v[EPV];
-                    Elem<T>::unpack(buf[i], v);
-#pragma unroll
-                    for (int e = EPV - 1; e >= 0; e--)
-                        if (v[e] == mx) first = min(first, sp.head + c * EPV + e);
-                }
-            }
-            for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
-                CT v[EPV];
-                Elem<T>::unpack(load16(xv + c), v);
-#pragma unroll
-                for (int e = EPV - 1; e >= 0; e--)
-                    if (v[e] == mx) first = min(first, sp.head + c * EPV + e);
-            }
-            atomicMin(&s_arg, first);
-        }
+        if (mine == mx) atomicMin(&s_arg, first_pos_of_max<T, NT, MAXC>(buf, sp, xv, tid, ep, edge, mx));
 
         CT sum = (ep >= 0) ? rn.e(edge) : (CT)0;
 #pragma unroll
@@ -535,7 +549,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
 
 template <typename T>
 int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, void *sel, int grad, int64_t rows,
-               int L, int V, int Tn, const int64_t *eos_ol, const int64_t *eos_tl, void *lse, hipStream_t stream) {
+               int L, int V, int Tn, const int64_t *eos_ol, const int64_t *eos_tl, void *lse, int64_t *argmax, hipStream_t stream) {
     using CT = typename Elem<T>::compute;
 #ifndef LSG_FWD_NT
 #define LSG_FWD_NT 512
@@ -548,10 +562,10 @@ int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
     int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
     if (grad)
         hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, true>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)x, idx, sb,
-                           sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse);
+                           sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax);
     else
         hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, false>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)x, idx,
-                           sb, sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse);
+                           sb, sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -603,18 +617,18 @@ using namespace pcfgnat;
 
 static int lsg_forward_dispatch(void *word_ins_out, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                 void *selected, int require_grad, int64_t B, int64_t L, int64_t V, int64_t T,
-                                const int64_t *eos_ol, const int64_t *eos_tl, void *lse, void *stream) {
+                                const int64_t *eos_ol, const int64_t *eos_tl, void *lse, void *stream, int64_t *argmax = nullptr) {
     int rc = check_common(word_ins_out, select_idx, selected, B, L, V, T);
     if (rc != PCFGNAT_OK) return rc;
     if (B * L == 0) return PCFGNAT_OK;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case PCFGNAT_F16:
-            return launch_fwd<__half>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, s);
+            return launch_fwd<__half>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s);
         case PCFGNAT_F32:
-            return launch_fwd<float>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, s);
+            return launch_fwd<float>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s);
         case PCFGNAT_F64:
-            return launch_fwd<double>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, s);
+            return launch_fwd<double>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s);
         default:
             return fail(PCFGNAT_EINVAL, "logsoftmax_gather: unknown dtype code %d (float16, float32, float64 are dispatched)", dtype);
     }
@@ -685,6 +699,13 @@ extern "C" int pcfgnat_logsoftmax_gather_backward(void *probs_inout, int dtype, 
                                                   int64_t sl, int64_t st, const void *grad_selected, int64_t B, int64_t L,
                                                   int64_t V, int64_t T, void *stream) {
     return lsg_backward_dispatch(probs_inout, dtype, select_idx, sb, sl, st, grad_selected, nullptr, B, L, V, T, stream);
+}
+
+int pcfgnat::lsg_forward_eos_argmax(const void *logits, int dtype, const int64_t *targets, void *selected, int64_t *argmax,
+                                    const int64_t *output_length, const int64_t *target_length, int64_t B, int64_t L, int64_t V,
+                                    int64_t T, void *stream) {
+    return lsg_forward_dispatch(const_cast<void *>(logits), dtype, targets, T, 0, 1, selected, 0, B, L, V, T, output_length, target_length,
+                                nullptr, stream, argmax);
 }
 
 int pcfgnat::lsg_backward_lse_with_loss(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,

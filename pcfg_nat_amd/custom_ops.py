@@ -436,6 +436,54 @@ def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unre
     return out[:, :maxlen].to(torch.float32)
 
 
+def pcfg_glat_step(word_ins_out, tgt_tokens, prev_output_tokens, links, context_p, pad_index, generator=None,
+                   noise_device=None):
+    """GLAT glancing, ``number-random`` strategy (nat_pcfg_loss.py:193-269), as one native call.  Same results as the
+    torch glue over the separate ops; ``word_ins_out`` is only read.  The two random draws of the reference (``randn``
+    for the glance scores, then ``rand``) are made here, in that order, on the tokens' device or on ``noise_device``.
+    Returns the dict of ``harness.glat_alignment``."""
+    lib = get_pcfg_kernel()
+    _need_cuda("pcfg_glat_step", word_ins_out, tgt_tokens, prev_output_tokens, links)
+    if word_ins_out.dim() != 3 or not word_ins_out.is_contiguous():
+        raise RuntimeError("pcfg_glat_step: word_ins_out must be a contiguous [bsz, prelen, vocab] tensor")
+    B, L, V = word_ins_out.shape
+    code = _DTYPE_CODE.get(word_ins_out.dtype)
+    if code is None:
+        raise RuntimeError("pcfg_glat_step: unsupported dtype %s" % word_ins_out.dtype)
+    if tgt_tokens.dim() != 2 or tgt_tokens.size(0) != B or tgt_tokens.dtype != torch.int64:
+        raise RuntimeError("pcfg_glat_step: tgt_tokens must be an int64 [bsz, tarlen] tensor")
+    if prev_output_tokens.shape != (B, L) or prev_output_tokens.dtype != torch.int64:
+        raise RuntimeError("pcfg_glat_step: prev_output_tokens must be an int64 [bsz, prelen] tensor")
+    if links.dim() != 4 or links.size(0) != B or links.size(1) != L or links.size(3) != L or links.dtype != torch.float32:
+        raise RuntimeError("pcfg_glat_step: links must be float32 [bsz, prelen, max_left+1, prelen]")
+    T = tgt_tokens.size(1)
+    ml = links.size(2) - 1
+    Mc = (L - 2) // (ml + 1) + 1
+    dev = word_ins_out.device
+    tgt, prev, links = tgt_tokens.contiguous(), prev_output_tokens.contiguous(), links.contiguous()
+    ndev = dev if noise_device is None else torch.device(noise_device)
+    noise = torch.randn((B, L), device=ndev, dtype=torch.float, generator=generator).to(dev)
+    torch.rand((B, L), device=ndev, generator=generator)  # the reference's second draw: cannot change the result
+    with torch.cuda.device(dev):
+        f32 = dict(dtype=torch.float32, device=dev)
+        i64 = dict(dtype=torch.int64, device=dev)
+        match = torch.empty((B, L, T), **f32)
+        S = torch.empty((B, Mc, T + 2), **f32)
+        aux = torch.empty((max(1, lib.pcfgnat_pcfg_aux_floats(B, L, T, ml)),), **f32)
+        ints = torch.empty((4, B, L), **i64)       # pred_tokens, path, glat tokens, (unused)
+        small = torch.empty((4, B), **i64)         # output_length, target_length, same_num, glance_nums
+        matchmask = torch.empty((B, T, L), dtype=torch.bool, device=dev)
+        keep = torch.empty((B, L), dtype=torch.bool, device=dev)
+        out = torch.empty((2,), **f32)
+        _lib.check(lib.pcfgnat_glat_step(word_ins_out.data_ptr(), code, tgt.data_ptr(), prev.data_ptr(), links.data_ptr(),
+                                         noise.data_ptr(), float(context_p), int(pad_index), match.data_ptr(), S.data_ptr(),
+                                         aux.data_ptr(), ints[0].data_ptr(), small[0].data_ptr(), ints[1].data_ptr(),
+                                         matchmask.data_ptr(), keep.data_ptr(), ints[2].data_ptr(), small[2].data_ptr(),
+                                         small[3].data_ptr(), out.data_ptr(), B, L, V, T, ml, _stream(word_ins_out)), lib)
+    return {"path": ints[1], "matchmask": matchmask, "keep_word_mask": keep, "glat_prev_output_tokens": ints[2],
+            "same_num": small[2], "glance_nums": small[3], "max_tree_lprob": out[0]}
+
+
 _PENALTY_CACHE = {}
 
 

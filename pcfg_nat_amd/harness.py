@@ -42,11 +42,15 @@ def compute_pcfg_loss(outputs, output_masks, targets, target_masks, links, ops=_
 
 
 def glat_alignment(word_ins_out, tgt_tokens, prev_output_tokens, links, context_p, pad=PAD, ops=_default_ops,
-                   generator=None, noise_device=None):
+                   generator=None, noise_device=None, single_call=False):
     """GLAT glancing with the ``number-random`` strategy (nat_pcfg_loss.py:193-269): best-tree alignment of target
     tokens to graph nodes, then a random subset of the aligned nodes is revealed.  RNG order: ``randn`` then ``rand``.
     The reference draws both on the tokens' device; ``noise_device`` (e.g. "cpu") draws them elsewhere and moves them,
-    which makes a run reproducible across devices."""
+    which makes a run reproducible across devices.  ``single_call``: the same pass as one native call
+    (``ops.pcfg_glat_step``)."""
+    if single_call:
+        return ops.pcfg_glat_step(word_ins_out, tgt_tokens, prev_output_tokens, links, context_p, pad, generator=generator,
+                                  noise_device=noise_device)
     batch_size, prelen = links.shape[0], links.shape[1]
     tarlen = tgt_tokens.shape[1]
     target_length = (~tgt_tokens.eq(pad)).sum(1)

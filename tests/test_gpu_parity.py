@@ -297,6 +297,35 @@ def test_best_tree_exact_ties_follow_reference_order():
     assert second((1, 5, 3, 2)) == 4
 
 
+@pytest.mark.parametrize("ml", [1, 3])
+def test_glat_single_call_small_ragged(ml):
+    """Ragged small batch (one sentence whose target cannot be derived) through the one-call GLAT pass against the torch
+    glue over the oracle ops, for the tuned (max_left 1) and the general kernels."""
+    import oracle_ops
+    g = torch.Generator().manual_seed(40 + ml)
+    L, T, V = 8 * (ml + 1) + 2, 9, 97
+    ms = [L, L - 2 * (ml + 1), (ml + 1) * 2 + 2, L]
+    ns = [9, 6, 9, 7]  # sentence 2: nine tokens from three main-chain nodes, impossible
+    B = len(ms)
+    m = torch.tensor(ms)
+    links = synth.make_links(B, L, m, ml, g)
+    tgt = torch.full((B, T), synth.PAD, dtype=torch.int64)
+    for b, n in enumerate(ns):
+        tgt[b, :n] = torch.randint(4, V, (n,), generator=g)
+    prev = torch.full((B, L), 3, dtype=torch.int64).masked_fill(torch.arange(L).view(1, L) >= m.view(B, 1), synth.PAD)
+    logits = torch.randn(B, L, V, generator=g)
+    for b in range(B):  # let some predictions agree with the targets
+        logits[b, 1, tgt[b, 0]] += 20.0
+    g1, g2 = torch.Generator().manual_seed(5), torch.Generator().manual_seed(5)
+    want = harness.glat_alignment(logits.clone(), tgt, prev, links, 0.5, ops=oracle_ops, generator=g1)
+    got = harness.glat_alignment(logits.to(DEV), tgt.to(DEV), prev.to(DEV), links.to(DEV), 0.5, generator=g2, noise_device="cpu",
+                                 single_call=True)
+    for key in ("path", "keep_word_mask", "glat_prev_output_tokens", "matchmask", "same_num", "glance_nums"):
+        assert got[key].dtype == want[key].dtype and torch.equal(got[key].cpu(), want[key]), key
+    assert int(want["same_num"].sum()) >= 1
+    assert torch.allclose(got["max_tree_lprob"].cpu(), want["max_tree_lprob"], rtol=2e-5)
+
+
 def _decode_case(name):
     if name == "short":
         return synth.decode_batch([5, 9, 16, 3, 12], seed=3, V=500)
