@@ -114,6 +114,17 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (a + b) + (c + d);
 }
 
+// Wave64 minimum of an int: DPP inside the rows, the four row results through scalar registers.
+__device__ __forceinline__ int wave_min(int v) {
+    v = min(v, dpp_i<DPP_QUAD_XOR1>(v));
+    v = min(v, dpp_i<DPP_QUAD_XOR2>(v));
+    v = min(v, dpp_i<DPP_ROW_HALF_MIRROR>(v));
+    v = min(v, dpp_i<DPP_ROW_MIRROR>(v));
+    const int a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+    const int c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+    return min(min(a, b), min(c, d));
+}
+
 __device__ __forceinline__ double wave_max(double v) {
     for (int o = 32; o > 0; o >>= 1) v = fmax(v, __shfl_xor(v, o));
     return v;

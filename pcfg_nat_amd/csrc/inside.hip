@@ -874,10 +874,10 @@ __device__ __forceinline__ int tie_key(int rel_c, int j) {
     return (rank << 24) | (rel_c << 1) | j;
 }
 
-// 256 threads stage the sentence's inside table and its emissions (MODE >= 1) and its compact link matrices (MODE 2) in
+// 1024 threads stage the sentence's inside table and its emissions (MODE >= 1) and its compact link matrices (MODE 2) in
 // LDS; the first wave then walks the chain without touching global memory.  MODE 0 reads everything from global memory
 // (tables too large for LDS).  Dynamic LDS: S [Mc][T+2], main/leaf emissions [Mc][T] each, matrices [2][Mc][Mc].
-constexpr int BT_NT = 256;
+constexpr int BT_NT = 1024;
 template <int MODE>
 __global__ __launch_bounds__(BT_NT) void best_tree_ml1_kernel(const float *__restrict__ S, const float *__restrict__ match_all,
                                                              const float *__restrict__ links, const int64_t *__restrict__ out_len,
@@ -900,8 +900,10 @@ __global__ __launch_bounds__(BT_NT) void best_tree_ml1_kernel(const float *__res
     for (int i = tid; i < L; i += BT_NT) tr[i] = -1;
     if (!lengths_ok(m, n, L, T)) return;
     const int mc = m / 2;
-    if (TAB_LDS) {
+    if (TAB_LDS) {  // (loops unrolled so that several loads are in flight per thread)
+#pragma unroll 4
         for (int i = tid; i < mc * TS; i += BT_NT) sS[i] = Sb[i];
+#pragma unroll 4
         for (int i = tid; i < mc * T; i += BT_NT) {
             const int a_id = i / T, t = i - a_id * T;
             sMain[i] = mt[(size_t)(2 * a_id + 1) * T + t];
@@ -912,6 +914,7 @@ __global__ __launch_bounds__(BT_NT) void best_tree_ml1_kernel(const float *__res
     auto main_at = [&](int x_id, int t) -> float { return TAB_LDS ? sMain[x_id * T + t] : mt[(size_t)(2 * x_id + 1) * T + t]; };
     auto leaf_at = [&](int x_id, int t) -> float { return TAB_LDS ? sLeaf[x_id * T + t] : mt[(size_t)(2 * x_id) * T + t]; };
     if (LINKS_LDS) {
+#pragma unroll 4
         for (int i = tid; i < mc * mc; i += BT_NT) {
             const int a_id = i / mc, c_id = i - a_id * mc;
             const size_t row = (size_t)(2 * a_id + 1) * 2;
@@ -950,8 +953,7 @@ __global__ __launch_bounds__(BT_NT) void best_tree_ml1_kernel(const float *__res
         }
         // wave arg max: the maximum first, then the smallest tie key among the lanes that hold it
         const float top = wave_max(best);
-        int key = (best == top && best != NEG_INF_F) ? best_key : 0x7fffffff;
-        for (int o = 32; o > 0; o >>= 1) key = min(key, __shfl_xor(key, o));
+        const int key = wave_min((best == top && best != NEG_INF_F) ? best_key : 0x7fffffff);
         const bool found = key != 0x7fffffff;
         const int best_j = found ? (key & 1) : 0;
         const int best_c = found ? a_id + 1 + ((key >> 1) & 0x7fffff) : -1;

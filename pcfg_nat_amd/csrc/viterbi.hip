@@ -145,8 +145,7 @@ __device__ __forceinline__ int select_length(const float *scores, const float *p
         }
     }
     const float top = wave_max(best);
-    int cand = (best == top && idx != 0x7fffffff) ? idx : 0x7fffffff;
-    for (int o = 32; o > 0; o >>= 1) cand = min(cand, __shfl_xor(cand, o));
+    const int cand = wave_min((best == top && idx != 0x7fffffff) ? idx : 0x7fffffff);
     return cand == 0x7fffffff ? 1 : cand;  // nothing above -inf: torch.max returns the first index
 }
 
