@@ -126,6 +126,28 @@ def decode_timing(dev):
     return out
 
 
+def glat_timing(logits, targets, links, out_len):
+    """The GLAT alignment pass that precedes the loss in every training step (nat_pcfg_loss.py:193-269) on the same
+    batch, as one native call: gather + eos mask + arg max, inside forward, best tree, glancing glue."""
+    import torch
+    from pcfg_nat_amd import harness, synth
+
+    B, L, _ = logits.shape
+    prev = torch.full((B, L), 3, dtype=torch.int64, device=logits.device)
+    prev = prev.masked_fill(torch.arange(L, device=logits.device).view(1, L) >= out_len.view(B, 1), synth.PAD)
+    for _ in range(3):
+        harness.glat_alignment(logits, targets, prev, links, 0.5, single_call=True)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    reps = 20
+    for _ in range(reps):
+        harness.glat_alignment(logits, targets, prev, links, 0.5, single_call=True)
+    end.record()
+    torch.cuda.synchronize()
+    return {"ms_per_call": start.elapsed_time(end) / reps}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -264,6 +286,7 @@ def main():
     }
     if not args.no_decode:
         result["viterbi"] = decode_timing(dev)
+        result["glat_alignment"] = glat_timing(torch.randn(B, L, V, device=dev, generator=ggen).mul_(2).half(), targets, links, ol)
     if not args.no_cpu_baseline:
         batch_cpu = {"output_length": m, "target_length": n, "links": links_cpu, "targets": targets_cpu}
         result["cpu_baseline"] = cpu_baseline(batch_cpu, sample_logits, args.cpu_sentences)
