@@ -96,6 +96,29 @@ def _pcfg_loss_backward(grad_output, S, aux, match_all, links, output_length, ta
     return match_all_grad, links_grad
 
 
+def _pcfg_loss_forward_backward(grad_output, match_all, links, output_length, target_length, config, name):
+    """pcfg_loss followed by pcfg_loss_backward (the eager pair of pcfg_loss.py:67-73) as one native call, a single launch
+    when the sentence's tables fit in LDS.  Returns (S, match_all_grad, links_grad)."""
+    if not (1 <= config <= 4):
+        raise RuntimeError("config should be 1~4")
+    lib = get_pcfg_kernel()
+    B, L, T, ml = _check_pcfg_inputs(name, match_all, links, output_length, target_length)
+    output_length = _lengths(name, output_length, B)
+    target_length = _lengths(name, target_length, B)
+    Mc = (L - 2) // (ml + 1) + 1
+    with torch.cuda.device(match_all.device):
+        S = torch.empty((B, Mc, T + 2), dtype=torch.float32, device=match_all.device)
+        aux = torch.empty((max(1, lib.pcfgnat_pcfg_aux_floats(B, L, T, ml)),), dtype=torch.float32, device=match_all.device)
+        match_all_grad = torch.empty_like(match_all)
+        links_grad = torch.empty_like(links)
+        _lib.check(lib.pcfgnat_pcfg_loss_forward_backward(grad_output.data_ptr() if grad_output is not None else None,
+                                                          match_all.data_ptr(), links.data_ptr(), output_length.data_ptr(),
+                                                          target_length.data_ptr(), S.data_ptr(), aux.data_ptr(),
+                                                          match_all_grad.data_ptr(), links_grad.data_ptr(), B, L, T, ml,
+                                                          _stream(match_all)), lib)
+    return S, match_all_grad, links_grad
+
+
 class CUDAPCFGLossFunc(Function):
     """Inside-algorithm log-likelihood (reference: pcfg_loss.py:49-85)."""
     config = 1
@@ -114,14 +137,15 @@ class CUDAPCFGLossFunc(Function):
         require_gradient = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
         match_all = match_all.contiguous()
         links = links.contiguous()
-        S, aux, ol, tl = _pcfg_loss_tables(match_all, links, output_length, target_length, CUDAPCFGLossFunc.config,
-                                           "cuda_pcfg_loss")
         if require_gradient:
             # like the reference (pcfg_loss.py:71-73) the backward sweep runs eagerly with a unit upstream gradient
-            ones = torch.ones((batch_size,), dtype=S.dtype, device=S.device)
-            match_all_grad, links_grad = _pcfg_loss_backward(ones, S, aux, match_all, links, ol, tl,
-                                                             CUDAPCFGLossFunc.config)
+            ones = torch.ones((batch_size,), dtype=torch.float32, device=match_all.device)
+            S, match_all_grad, links_grad = _pcfg_loss_forward_backward(ones, match_all, links, output_length, target_length,
+                                                                        CUDAPCFGLossFunc.config, "cuda_pcfg_loss")
             ctx.save_for_backward(match_all_grad, links_grad)
+        else:
+            S, _, _, _ = _pcfg_loss_tables(match_all, links, output_length, target_length, CUDAPCFGLossFunc.config,
+                                           "cuda_pcfg_loss")
         return S[:, 0, 0].clone()
 
     @staticmethod
