@@ -230,6 +230,20 @@ int pcfgnat_viterbi_decode(const float *ob_lprob, const float *links, const int6
                            void *workspace, int64_t *out_tokens, int64_t *out_count, int64_t *pred_length, int64_t B,
                            int64_t L, int64_t ml, void *stream);
 
+/*
+ * The `lookahead` and `greedy` decode strategies of glat_decomposed_with_link_two_hands_tri_pcfg.py:419-481 in one launch:
+ * per node the first arg max over (k, c) of (links[b,a,k,c] + ob[b,c]*beta) + ob[b,left(a,k)]*beta (lookahead; ob_lprob
+ * NULL selects greedy: links alone), then the in-order walk from node 1 over these pointers.  The reference builds the
+ * left term from sentence 0's logits for every sentence of a batch (:424, a batch-1 routine); the per-sentence term is
+ * used here.  Tokens are not de-duplicated (unlike pcfgnat_viterbi_decoding).
+ *   links_idx [B,L] int64 out (may be NULL): k*L + c per node; out_tokens [B,L] int64, right-padded with pad_index;
+ *   out_count [B] int64 (-1 if a walk does not terminate).
+ */
+int pcfgnat_lookahead_decode(const float *links, const float *ob_lprob, float beta, const int64_t *output_length,
+                             const int64_t *tokens, const int64_t *left_tree_mask, int64_t mask_dim, int64_t pad_index,
+                             int64_t *links_idx, int64_t *out_tokens, int64_t *out_count, int64_t B, int64_t L, int64_t ml,
+                             void *stream);
+
 /* The same walk on host memory (the reference's own call site hands over CPU tensors,
  * glat_decomposed_with_link_two_hands_tri_pcfg.py:500-502).  Synchronous, touches no GPU. */
 int pcfgnat_viterbi_decoding_host(const int64_t *pred_length, const int64_t *output_length, const int64_t *Lt,

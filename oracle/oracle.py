@@ -189,3 +189,24 @@ def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unre
         raise RuntimeError("viterbi_decoding: malformed traces")
     maxlen = int(out_len.max()) if B else 0
     return out[:, :maxlen].astype(np.float32)
+
+
+def lookahead_decode(links, unreduced_logits, output_length, unreduced_tokens, left_tree_mask, pad_index, beta=1.0):
+    """`lookahead` decode (glat_decomposed_with_link_two_hands_tri_pcfg.py:419-481); ``unreduced_logits=None`` gives the
+    `greedy` strategy (:432-434).  Returns (tokens int64 [B, maxlen] right-padded with pad_index, links_idx [B, L])."""
+    links = _c(links, np.float32)
+    B, L, K, _ = links.shape
+    ob = None if unreduced_logits is None else _c(unreduced_logits, np.float32)
+    output_length = _c(output_length, np.int64)
+    tokens, mask = _c(unreduced_tokens, np.int64), _c(left_tree_mask, np.int64)
+    cap = L
+    idx = np.zeros((B, L), dtype=np.int64)
+    out = np.full((B, cap), pad_index, dtype=np.int64)
+    out_len = np.zeros(B, dtype=np.int64)
+    _lib().oracle_lookahead_decode(_p(links), _p(ob) if ob is not None else None, ctypes.c_float(beta), _p(output_length),
+                                   _p(tokens), _p(mask), ctypes.c_int64(mask.shape[0]), ctypes.c_int64(pad_index), _p(idx),
+                                   _p(out), _p(out_len), B, L, K - 1, cap)
+    if (out_len < 0).any():
+        raise RuntimeError("lookahead_decode: the walk does not terminate")
+    maxlen = int(out_len.max()) if B else 0
+    return out[:, :maxlen], idx

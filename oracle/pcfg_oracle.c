@@ -98,3 +98,72 @@ void oracle_viterbi_decoding(const int64_t *pred_len, const int64_t *out_length,
         free(stack_len);
     }
 }
+
+
+/*
+ * `lookahead` / `greedy` decode (glat_decomposed_with_link_two_hands_tri_pcfg.py:419-481).
+ *
+ * Pointers (:420-431): links_idx[b][a] = first arg max over the flattened (k, c) of
+ *   lookahead: (links[b][a][k][c] + ob[b][c] * beta) + ob[b][left(a,k)] * beta,  left(a,0) = 0, left(a,k) = max(a-k, 0)
+ *              (the `_max_left_index` table, :214-218), each product and sum rounded to fp32 in this order;
+ *   greedy (ob == NULL): links[b][a][k][c].
+ * The reference builds the left term from `unreduced_logits.unsqueeze(1).repeat(bsz, prelen, 1)` gathered with a
+ * batch-1 index (:424), which for bsz > 1 takes sentence 0's logits for every sentence; like its viterbi_decoding it is
+ * effectively a batch-1 routine, and the evidently intended per-sentence term is used here.
+ * Walk (:434-476): in-order traversal from node 1: descend to the left child (0 if k = 0, else a - k) unless
+ * left_mask[a][left] is set, emit tokens[a] unless it is the pad symbol, continue with the right child c; stop when the
+ * stack is empty and the current node is 0 or >= output_length.  No de-duplication (unlike viterbi_decoding).
+ * out [B][cap], out_len [B] (-1 if the walk does not terminate within the cell budget).
+ */
+void oracle_lookahead_decode(const float *links, const float *ob, float beta, const int64_t *out_length, const int64_t *tokens,
+                             const int64_t *left_mask, int64_t mask_dim, int64_t pad_index, int64_t *links_idx, int64_t *out,
+                             int64_t *out_len, int B, int L, int ml, int cap)
+{
+    const int K = ml + 1;
+    for (int b = 0; b < B; b++) {
+        const float *lk = links + (size_t)b * L * K * L;
+        for (int a = 0; a < L; a++) {
+            float best = 0.f;
+            int best_i = -1;
+            for (int k = 0; k < K; k++) {
+                const int left = (k == 0) ? 0 : (a - k < 0 ? 0 : a - k);
+                for (int c = 0; c < L; c++) {
+                    float v = lk[((size_t)a * K + k) * L + c];
+                    if (ob) {
+                        const float r = ob[(size_t)b * L + c] * beta;
+                        const float l = ob[(size_t)b * L + left] * beta;
+                        v = (v + r) + l;
+                    }
+                    if (best_i < 0 || v > best) { best = v; best_i = k * L + c; }
+                }
+            }
+            links_idx[(size_t)b * L + a] = best_i;
+        }
+        int64_t *stack = (int64_t *)malloc(sizeof(int64_t) * (size_t)(L + 4));
+        int sp = 0, cnt = 0, bad = 0;
+        int64_t now = 1, length = out_length[b];
+        int64_t budget = 4 * (int64_t)L + 8;
+        while ((now < length && now != 0) || sp > 0) {
+            if (--budget < 0) { bad = 1; break; }
+            while (now < length && now != 0) {
+                if (sp >= L + 4 || now < 0 || now >= L) { bad = 1; break; }
+                stack[sp++] = now;
+                const int64_t k = links_idx[(size_t)b * L + now] / L;
+                const int64_t left = (k == 0) ? 0 : now - k;
+                if (left < 0 || left >= mask_dim || now >= mask_dim) { bad = 1; break; }
+                if (left_mask[(size_t)now * mask_dim + left]) break;
+                now = left;
+            }
+            if (bad) break;
+            now = stack[--sp];
+            const int64_t tok = tokens[(size_t)b * L + now];
+            if (tok != pad_index) {
+                if (cnt < cap) out[(size_t)b * cap + cnt] = tok; else bad = 1;
+                cnt++;
+            }
+            now = links_idx[(size_t)b * L + now] % L;
+        }
+        out_len[b] = bad ? -1 : cnt;
+        free(stack);
+    }
+}

@@ -441,10 +441,103 @@ __global__ __launch_bounds__(64) void select_length_kernel(const float *__restri
     if (threadIdx.x == 0) pred_length[b] = pl;
 }
 
+// `lookahead` / `greedy` decode (glat_decomposed_with_link_two_hands_tri_pcfg.py:419-481), one workgroup per sentence:
+// every wave takes rows of the sentence's link tensor and finds the first arg max over the flattened (k, c) of
+//   (links[a][k][c] + ob[c] * beta) + ob[left(a,k)] * beta     (lookahead, :421-427; left(a,0) = 0, left(a,k) = max(a-k, 0))
+//   links[a][k][c]                                              (greedy, ob == null, :432-434)
+// in fp32 in this association order; the pointers go to LDS (and to `links_idx`), then one thread walks the tree in
+// order (:434-476): left child unless left_tree_mask forbids it, emit the node's token unless it is the pad symbol,
+// right child.  Dynamic LDS: pointers [L], stack [L + 4].
+__global__ __launch_bounds__(NT) void lookahead_decode_kernel(const float *__restrict__ links, const float *__restrict__ ob_lprob,
+                                                             float beta, const int64_t *__restrict__ out_len,
+                                                             const int64_t *__restrict__ tokens, const int64_t *__restrict__ mask,
+                                                             int64_t mask_dim, int64_t pad, int64_t *__restrict__ links_idx,
+                                                             int64_t *__restrict__ out_tokens, int64_t *__restrict__ out_count, int L,
+                                                             int K) {
+    extern __shared__ int dyn[];
+    int *s_idx = dyn;        // [L]
+    int *s_stack = dyn + L;  // [L + 4]
+    const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float *lk = links + (size_t)b * L * K * L;
+    const float *ob = ob_lprob ? ob_lprob + (size_t)b * L : nullptr;
+    const int row_len = K * L;
+    for (int i = tid; i < L; i += NT) out_tokens[(size_t)b * L + i] = pad;
+    for (int a = wave; a < L; a += NT / 64) {
+        const float *row = lk + (size_t)a * row_len;
+        float best = NEG_INF_F;
+        int arg = 0x7fffffff;
+        for (int i = lane; i < row_len; i += 64) {
+            float v = row[i];
+            if (ob) {
+                const int k = i / L, c = i - k * L;
+                const int left = (k == 0) ? 0 : (a - k < 0 ? 0 : a - k);
+                const float r = ob[c] * beta, l = ob[left] * beta;
+                v = (v + r) + l;
+            }
+            if (v > best) {  // ascending scan, strict: the first maximum of this lane
+                best = v;
+                arg = i;
+            }
+        }
+        const float top = wave_max(best);
+        const int first = wave_min((best == top && arg != 0x7fffffff) ? arg : 0x7fffffff);
+        if (lane == 0) {
+            const int r = (first == 0x7fffffff) ? 0 : first;  // a row of -inf: index 0, like torch.max
+            s_idx[a] = r;
+            if (links_idx) links_idx[(size_t)b * L + a] = r;
+        }
+    }
+    __syncthreads();
+    if (tid != 0) return;
+    const int64_t length = out_len[b];
+    int sp = 0;
+    int64_t cnt = 0, now = 1;
+    int64_t budget = 4 * (int64_t)L + 8;
+    bool bad = false;
+    while ((now < length && now != 0) || sp > 0) {
+        if (--budget < 0) { bad = true; break; }
+        while (now < length && now != 0) {
+            if (sp >= L + 4 || now < 0 || now >= L) { bad = true; break; }
+            s_stack[sp++] = (int)now;
+            const int64_t k = s_idx[now] / L;
+            const int64_t left = (k == 0) ? 0 : now - k;
+            if (left < 0 || left >= mask_dim || now >= mask_dim) { bad = true; break; }
+            if (mask[now * mask_dim + left]) break;
+            now = left;
+        }
+        if (bad) break;
+        now = s_stack[--sp];
+        const int64_t t = tokens[(size_t)b * L + now];
+        if (t != pad) {
+            if (cnt < L) out_tokens[(size_t)b * L + cnt] = t;
+            else bad = true;
+            cnt++;
+        }
+        now = s_idx[now] % L;
+    }
+    out_count[b] = bad ? -1 : cnt;
+}
+
 }  // namespace
 }  // namespace pcfgnat
 
 using namespace pcfgnat;
+
+extern "C" int pcfgnat_lookahead_decode(const float *links, const float *ob_lprob, float beta, const int64_t *output_length,
+                                        const int64_t *tokens, const int64_t *left_tree_mask, int64_t mask_dim, int64_t pad_index,
+                                        int64_t *links_idx, int64_t *out_tokens, int64_t *out_count, int64_t B, int64_t L,
+                                        int64_t ml, void *stream) {
+    PCFGNAT_REQUIRE(B >= 0 && L >= 2 && ml >= 0 && mask_dim >= 1, "lookahead_decode: bad dimensions");
+    PCFGNAT_REQUIRE(L <= 8192 && (ml + 1) * L < (1LL << 30), "lookahead_decode: graph too large");
+    if (B == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(links && output_length && tokens && left_tree_mask && out_tokens && out_count, "lookahead_decode: null pointer");
+    const size_t dyn = ((size_t)2 * L + 4) * sizeof(int);
+    hipLaunchKernelGGL(lookahead_decode_kernel, dim3((unsigned)B), dim3(NT), dyn, (hipStream_t)stream, links, ob_lprob, beta,
+                       output_length, tokens, left_tree_mask, mask_dim, pad_index, links_idx, out_tokens, out_count, (int)L,
+                       (int)(ml + 1));
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
 
 extern "C" int pcfgnat_pcfg_viterbi(const float *ob_lprob, const float *links, const int64_t *output_length, float *S, int64_t *R,
                                     int64_t *Lt, int64_t *M, int64_t B, int64_t L, int64_t ml, void *stream) {

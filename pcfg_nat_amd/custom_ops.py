@@ -561,6 +561,47 @@ def pcfg_viterbi_decode(unreduced_logits, links, output_length, unreduced_tokens
     return out[:, :maxlen].to(torch.float32), meta[1]
 
 
+def pcfg_lookahead_decode(links, unreduced_logits, unreduced_tokens, output_length, left_tree_mask, pad_index, beta=1.0,
+                          strategy="lookahead", return_pointers=False):
+    """The `lookahead` / `greedy` decode strategies (glat_decomposed_with_link_two_hands_tri_pcfg.py:419-481) in one
+    launch: arg max pointers per node and the in-order walk.  Returns int64 tokens [B, maxlen] right-padded with
+    ``pad_index`` (and the pointers ``k * prelen + c`` [B, prelen] if asked)."""
+    if strategy not in ("lookahead", "greedy"):
+        raise RuntimeError("pcfg_lookahead_decode: strategy must be 'lookahead' or 'greedy'")
+    lib = get_pcfg_kernel()
+    _need_cuda("pcfg_lookahead_decode", links, unreduced_tokens, output_length, left_tree_mask)
+    if links.dim() != 4 or links.dtype != torch.float32 or links.size(1) != links.size(3):
+        raise RuntimeError("pcfg_lookahead_decode: links must be float32 [bsz, prelen, max_left+1, prelen]")
+    B, L, K, _ = links.shape
+    dev = links.device
+    links = links.contiguous()
+    ob_ptr = None
+    if strategy == "lookahead":
+        _need_cuda("pcfg_lookahead_decode", unreduced_logits)
+        if unreduced_logits.shape != (B, L) or unreduced_logits.dtype != torch.float32:
+            raise RuntimeError("pcfg_lookahead_decode: unreduced_logits must be float32 [bsz, prelen]")
+        ob = unreduced_logits.contiguous()
+        ob_ptr = ob.data_ptr()
+    if left_tree_mask.dim() != 2 or left_tree_mask.size(0) != left_tree_mask.size(1):
+        raise RuntimeError("pcfg_lookahead_decode: left_tree_mask must be square")
+    ol = _lengths("pcfg_lookahead_decode", output_length, B)
+    tok = unreduced_tokens.to(dtype=torch.int64).contiguous()
+    mask = left_tree_mask.to(dtype=torch.int64).contiguous()
+    with torch.cuda.device(dev):
+        idx = torch.empty((B, L), dtype=torch.int64, device=dev)
+        out = torch.empty((B, L), dtype=torch.int64, device=dev)
+        cnt = torch.empty((B,), dtype=torch.int64, device=dev)
+        _lib.check(lib.pcfgnat_lookahead_decode(links.data_ptr(), ob_ptr, float(beta), ol.data_ptr(), tok.data_ptr(), mask.data_ptr(),
+                                                mask.size(0), int(pad_index), idx.data_ptr(), out.data_ptr(), cnt.data_ptr(), B, L,
+                                                K - 1, _stream(links)), lib)
+    host = cnt.cpu()
+    if B and int(host.min()) < 0:
+        raise RuntimeError("pcfg_lookahead_decode: the walk does not terminate")
+    maxlen = int(host.max()) if B else 0
+    tokens = out[:, :maxlen]
+    return (tokens, idx) if return_pointers else tokens
+
+
 def pcfg_criterion_step(logits, targets, links, output_length, target_length, events=None, slices=None):
     """The criterion's whole training pass in one native call (``pcfgnat_criterion_step``): ``logits`` [B,L,V] (fp16 or
     fp32, contiguous) is consumed in place and holds d loss / d logits afterwards.  ``events``: optional list of eight

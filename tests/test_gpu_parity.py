@@ -374,6 +374,25 @@ def test_viterbi_tables_bit_exact_and_decode(case):
         assert got_tok.dtype == torch.float32 and torch.equal(got_tok.cpu(), want_tok)
 
 
+@pytest.mark.parametrize("ml,L,ms", [(1, 32, [32, 20, 8]), (3, 34, [34, 26]), (1, 400, [400, 284, 20, 400]), (1, 18, [18])])
+@pytest.mark.parametrize("strategy", ["lookahead", "greedy"])
+def test_lookahead_decode_bit_exact(ml, L, ms, strategy):
+    B = len(ms)
+    gen = torch.Generator().manual_seed(L + ml)
+    links = synth.make_links(B, L, torch.tensor(ms), ml, gen)
+    ob = torch.randn(B, L, generator=gen) - 2.0
+    tok = torch.randint(4, 60, (B, L), generator=gen)
+    tok[:, 5] = synth.PAD
+    left_mask, _, _ = synth.support_masks(L, ml)
+    beta = 0.9
+    want, want_idx = oracle.lookahead_decode(links.numpy(), None if strategy == "greedy" else ob.numpy(), np.array(ms), tok.numpy(),
+                                             left_mask.numpy(), synth.PAD, beta)
+    got, idx = ops.pcfg_lookahead_decode(links.to(DEV), ob.to(DEV), tok.to(DEV), torch.tensor(ms).to(DEV), left_mask.to(DEV), synth.PAD,
+                                         beta=beta, strategy=strategy, return_pointers=True)
+    assert idx.dtype == torch.int64 and np.array_equal(idx.cpu().numpy(), want_idx)
+    assert got.dtype == torch.int64 and np.array_equal(got.cpu().numpy(), want)
+
+
 def test_viterbi_exact_ties_follow_reference_order():
     L = m = 32
     links = torch.full((1, L, 2, L), -math.inf)

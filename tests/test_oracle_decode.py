@@ -187,3 +187,93 @@ def test_viterbi_tie_order_is_lane_structured():
     assert right_child_of_root((4, 8, 12)) == 2              # lane 2 next
     assert right_child_of_root((4, 8, 12, 2, 6, 10, 14)) == 1
     assert right_child_of_root((4, 8, 12, 2, 6, 10, 14, 1, 5, 9, 13)) == 3
+
+
+# ---- lookahead / greedy decode (glat_decomposed_with_link_two_hands_tri_pcfg.py:419-481) -------------------------------
+
+def _inorder(node, length, idx, L, mask, tokens, pad, out):
+    """Textbook recursive in-order traversal of the pointer tree: left subtree, node, right subtree."""
+    if not (node < length and node != 0):
+        return
+    k, c = divmod(int(idx[node]), L)
+    left = 0 if k == 0 else node - k
+    if not mask[node][left]:
+        _inorder(left, length, idx, L, mask, tokens, pad, out)
+    if tokens[node] != pad:
+        out.append(int(tokens[node]))
+    _inorder(c, length, idx, L, mask, tokens, pad, out)
+
+
+@pytest.mark.parametrize("ml,L,ms", [(1, 32, [32, 20, 8]), (3, 34, [34, 26]), (1, 16, [16])])
+@pytest.mark.parametrize("greedy", [False, True])
+def test_lookahead_decode_is_inorder_traversal_of_argmax_pointers(ml, L, ms, greedy):
+    B = len(ms)
+    gen = torch.Generator().manual_seed(L + ml + int(greedy))
+    links = synth.make_links(B, L, torch.tensor(ms), ml, gen).numpy()
+    rng = np.random.default_rng(L * 3 + ml)
+    ob = (rng.normal(size=(B, L)) - 2.0).astype(np.float32)
+    tokens = rng.integers(4, 50, size=(B, L)).astype(np.int64)
+    tokens[:, 5] = synth.PAD  # a pad prediction in the middle is skipped
+    beta = 0.7
+    left_mask, _, _ = synth.support_masks(L, ml)
+    got, idx = oracle.lookahead_decode(links, None if greedy else ob, np.array(ms), tokens, left_mask.numpy(), synth.PAD, beta)
+    # pointers: independent numpy evaluation of :420-431 in the same fp32 association order
+    K = ml + 1
+    for b in range(B):
+        if greedy:
+            score = links[b]
+        else:
+            left_idx = np.zeros((L, K), dtype=np.int64)
+            for k in range(1, K):
+                left_idx[:, k] = np.maximum(np.arange(L) - k, 0)
+            right = links[b] + (ob[b] * np.float32(beta))[None, None, :]
+            score = right + (ob[b][left_idx] * np.float32(beta))[:, :, None]
+        want_idx = score.reshape(L, K * L).argmax(-1)  # numpy: first maximum
+        assert np.array_equal(idx[b], want_idx)
+        want = []
+        _inorder(1, ms[b], want_idx, L, left_mask.numpy(), tokens[b], synth.PAD, want)
+        n = len(want)
+        assert n >= 2
+        assert got[b, :n].tolist() == want
+        assert (got[b, n:] == synth.PAD).all()
+
+
+def test_lookahead_decode_batch1_matches_the_reference_expression():
+    """For one sentence the reference's tensor expression (:421-427) is well defined; restated with the same torch calls."""
+    L, ml, m = 24, 1, 24
+    gen = torch.Generator().manual_seed(3)
+    links = synth.make_links(1, L, torch.tensor([m]), ml, gen)
+    ob = torch.randn(1, L, generator=gen) - 2.0
+    beta = 1.3
+    max_left_index = torch.arange(0, L).unsqueeze(0).unsqueeze(-1) + torch.zeros(1, L, ml + 1, dtype=torch.int64)
+    max_left_index[:, :, 0] = 0
+    for i in range(1, ml + 1):
+        max_left_index[:, :, i] = torch.where((max_left_index[:, :, i] - i) < 0, 0, max_left_index[:, :, i] - i)
+    right = links + ob.unsqueeze(1).unsqueeze(1) * beta
+    left = torch.gather(ob.unsqueeze(1).repeat(1, L, 1), dim=2, index=max_left_index[:, :L]) * beta
+    want_idx = (right + left.unsqueeze(-1)).view(1, L, (ml + 1) * L).max(dim=-1)[1]
+    tokens = torch.arange(L).view(1, L) + 10
+    left_mask, _, _ = synth.support_masks(L, ml)
+    _, idx = oracle.lookahead_decode(links.numpy(), ob.numpy(), np.array([m]), tokens.numpy(), left_mask.numpy(), synth.PAD, beta)
+    assert np.array_equal(idx, want_idx.numpy())
+
+
+def test_lookahead_decode_hand_case():
+    """Six nodes, main chain 1 -> 3 -> 5; node 3 takes its leaf 2 as left child: yield = tok[1], tok[2], tok[3], tok[5]."""
+    L, m = 6, 6
+    links = np.full((1, L, 2, L), NINF, dtype=np.float32)
+    links[0, 1, 0, 3] = -0.1   # root: null left child, right child 3
+    links[0, 1, 0, 5] = -3.0
+    links[0, 3, 1, 5] = -0.2   # node 3: left child 2 (k = 1), right child 5
+    links[0, 3, 0, 5] = -2.0
+    tokens = np.array([[90, 11, 12, 13, 14, 15]], dtype=np.int64)
+    left_mask, _, _ = synth.support_masks(L, 1)
+    got, idx = oracle.lookahead_decode(links, None, np.array([m]), tokens, left_mask.numpy(), synth.PAD)
+    assert idx[0, 1] == 0 * L + 3 and idx[0, 3] == 1 * L + 5
+    assert got.tolist() == [[11, 12, 13, 15]]
+    # a strong lookahead score on the direct jump 1 -> 5 changes the root's choice
+    ob = np.zeros((1, L), dtype=np.float32)
+    ob[0, 3] = -10.0
+    got, idx = oracle.lookahead_decode(links, ob, np.array([m]), tokens, left_mask.numpy(), synth.PAD, 1.0)
+    assert idx[0, 1] == 0 * L + 5
+    assert got.tolist() == [[11, 15]]
