@@ -326,6 +326,35 @@ def test_glat_single_call_small_ragged(ml):
     assert torch.allclose(got["max_tree_lprob"].cpu(), want["max_tree_lprob"], rtol=2e-5)
 
 
+@pytest.mark.parametrize("B,L,H,F,dtype", [(3, 18, 2, 4, torch.float32), (2, 34, 8, 16, torch.float32), (4, 128, 8, 64, torch.float16),
+                                            (2, 514, 4, 8, torch.float32), (2, 22, 16, 8, torch.float32), (2, 12, 1, 8, torch.float32)])
+def test_extract_links_forward_backward_vs_torch_restatement(B, L, H, F, dtype):
+    from oracle import extract_links_ref as ref
+    g = torch.Generator().manual_seed(L + H)
+    q, kl, kr = ((torch.randn(B, L, H, F, generator=g) * 0.7).to(dtype) for _ in range(3))
+    gate = torch.randn(B, L, H, generator=g).to(dtype)
+    ms = [L, max(4, (L // 2) // 2 * 2), 4, L][:B]
+    m = torch.tensor(ms)
+    prev = torch.full((B, L), 3).masked_fill(torch.arange(L).view(1, L) >= m.view(B, 1), synth.PAD)
+    lm, rm, mc = synth.support_masks(L, 1)
+    leaves = [t.double().requires_grad_(True) for t in (q, kl, kr, gate)]
+    want = ref.extract_links(*leaves, prev, synth.PAD, lm, rm, mc).double()
+    fin = torch.isfinite(want)
+    G = torch.randn(want.shape, generator=g, dtype=torch.float64).masked_fill(~fin, 0)
+    want.masked_fill(~fin, 0).mul(G).sum().backward()
+    dleaves = [t.to(DEV).requires_grad_(True) for t in (q, kl, kr, gate)]
+    got = ops.pcfg_extract_links(*dleaves, prev.to(DEV), synth.PAD, lm.to(DEV), rm.to(DEV), mc.to(DEV))
+    assert got.dtype == torch.float32 and torch.equal(torch.isfinite(got).cpu(), fin)
+    assert torch.allclose(got.cpu().double()[fin], want.detach()[fin], rtol=2e-5, atol=2e-5)
+    got.masked_fill(~fin.to(DEV), 0).mul(G.float().to(DEV)).sum().backward()
+    for name, mine, theirs in zip(("q", "kl", "kr", "gate"), dleaves, leaves):
+        assert mine.grad.dtype == dtype
+        scale = theirs.grad.abs().max().item()
+        err = (mine.grad.cpu().double() - theirs.grad).abs().max().item()
+        tol = 2e-3 if dtype == torch.float16 else 1e-4
+        assert err <= tol * scale, (name, err, scale)
+
+
 def _decode_case(name):
     if name == "short":
         return synth.decode_batch([5, 9, 16, 3, 12], seed=3, V=500)
