@@ -164,30 +164,35 @@ int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, cons
 
 /*
  * The link scorer of the model (glat_decomposed_with_link_two_hands_tri_pcfg.py:140-201, `extract_links`) after its four
- * projections and its batched products, for max_left = 1:
+ * projections, for max_left = 1:
  *   links[b,a,k,c] = logsumexp_h( log_softmax_h(gate_logits[b,a,:])[h] + log_softmax_{(k,c)}( z[b,a,:,:,h] )[k,c] ),
- *   z[b,a,k,c,h] = ( q[b,h,a].kl[b,h,left(a,k)] + Zbc[b,h,src(a,k),c] + Zac[b,h,a,c] ) / sqrt(F),
+ *   z[b,a,k,c,h] = ( q[b,a,h].kl[b,left(a,k),h] + kl[b,src(a,k),h].kr[b,c,h] + q[b,a,h].kr[b,c,h] ) / sqrt(F),
  * left(a,0) = src(a,0) = 0, left(a,1) = max(a-1,0), src(a,1) = a-1 cyclically; masked entries (:171-184) and rows
- * without an allowed left option or right child (:176-181, 199) are -inf.
- *   q, kl [B,H,L,F] float32 (head-major copies of the query / left-key chunks); Zac = q.kr^T, Zbc = kl.kr^T [B,H,L,L]
- *   float32, computed by the caller's GEMM library; gate_logits [B,L,H] float32; prev_output_tokens [B,L] int64;
- *   left_tree_mask, right_tree_mask [L,L], main_chain [L]: one byte per flag (masks: non-zero = forbidden).
- *   links [B,L,2,L] float32 out; head_lse [B,L,H] float32 out (softmax normalisers, consumed by the backward).
- * Backward: from grad_links it writes dZac, dZbc1 (the k = 1 part, complete), dZ0 (the k = 0 part per parent; its sum over
- * the parent axis belongs to row 0 of the gradient of Zbc) [B,H,L,L], dsab [B,H,L,2] (gradient of the two q.kl dot products
- * of every parent) and dgate [B,L,H]; the gradients of q, kl, kr follow by the transposed products.
+ * without an allowed left option or right child (:176-181, 199) are -inf.  The batched products go through the
+ * caller's GEMM library; the five calls are, in order:
+ *   pack:     query/left-key/right-key chunks [B,L,H,F] (F16/F32/F64) -> A [B,H,2L,F] (query rows, then left-key rows) and
+ *             Kr [B,H,L,F], float32.                      Caller: Z = A . Kr^T  [B,H,2L,L].
+ *   forward:  Z, A, gate_logits [B,L,H] float32, prev_output_tokens [B,L] int64, left_tree_mask / right_tree_mask [L,L]
+ *             and main_chain [L] (one byte per flag; masks: non-zero = forbidden) -> links [B,L,2,L], head_lse [B,L,H].
+ *   backward: grad_links, links, head_lse, Z, A, ... -> dZ [B,H,2L,L] (gradient of Z, complete), dZ0 [B,H,L,L] (scratch),
+ *             dsab [B,H,L,2] (gradient of the two q.kl dot products of every parent), dgate [B,L,H] (gradient of the
+ *             gate logits).                               Caller: dA = dZ . Kr, dKr = dZ^T . A.
+ *   unpack:   dA, dKr, dsab, A -> gradients of the three chunk tensors [B,L,H,F] in `dtype`.
  * Nothing of size [B,L,2L,H] is materialised in either direction.
  */
-int pcfgnat_extract_links_forward(const float *Zac, const float *Zbc, const float *q, const float *kl, const float *gate_logits,
-                                  const int64_t *prev_output_tokens, int64_t pad_index, const unsigned char *left_tree_mask,
-                                  const unsigned char *right_tree_mask, const unsigned char *main_chain, float *links,
-                                  float *head_lse, int64_t B, int64_t L, int64_t H, int64_t F, void *stream);
-int pcfgnat_extract_links_backward(const float *grad_links, const float *links, const float *head_lse, const float *Zac,
-                                   const float *Zbc, const float *q, const float *kl, const float *gate_logits,
-                                   const int64_t *prev_output_tokens, int64_t pad_index, const unsigned char *left_tree_mask,
-                                   const unsigned char *right_tree_mask, const unsigned char *main_chain, float *dZac,
-                                   float *dZbc1, float *dZ0, float *dsab, float *dgate, int64_t B, int64_t L, int64_t H,
-                                   int64_t F, void *stream);
+int pcfgnat_extract_links_pack(const void *query_chunks, const void *key_chunks_left, const void *key_chunks_right, int dtype,
+                               float *A, float *Kr, int64_t B, int64_t L, int64_t H, int64_t F, void *stream);
+int pcfgnat_extract_links_forward(const float *Z, const float *A, const float *gate_logits, const int64_t *prev_output_tokens,
+                                  int64_t pad_index, const unsigned char *left_tree_mask, const unsigned char *right_tree_mask,
+                                  const unsigned char *main_chain, float *links, float *head_lse, int64_t B, int64_t L,
+                                  int64_t H, int64_t F, void *stream);
+int pcfgnat_extract_links_backward(const float *grad_links, const float *links, const float *head_lse, const float *Z,
+                                   const float *A, const float *gate_logits, const int64_t *prev_output_tokens,
+                                   int64_t pad_index, const unsigned char *left_tree_mask,
+                                   const unsigned char *right_tree_mask, const unsigned char *main_chain, float *dZ, float *dZ0,
+                                   float *dsab, float *dgate, int64_t B, int64_t L, int64_t H, int64_t F, void *stream);
+int pcfgnat_extract_links_unpack(const float *dA, const float *dKr, const float *dsab, const float *A, int dtype, void *dq,
+                                 void *dkl, void *dkr, int64_t B, int64_t L, int64_t H, int64_t F, void *stream);
 
 /*
  * GLAT glancing with the `number-random` strategy (nat_pcfg_loss.py:193-269) in one call: lengths from the pad counts

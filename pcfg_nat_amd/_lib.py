@@ -37,9 +37,11 @@ SIGNATURES = {
     "pcfgnat_criterion_loss": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_criterion_step": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                                       _i64, _vp, _vp]),
-    "pcfgnat_extract_links_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
-    "pcfgnat_extract_links_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
-                                              _i64, _i64, _i64, _i64, _vp]),
+    "pcfgnat_extract_links_pack": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "pcfgnat_extract_links_forward": (_int, [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "pcfgnat_extract_links_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
+                                              _i64, _i64, _vp]),
+    "pcfgnat_extract_links_unpack": (_int, [_vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_glat_step": (_int, [_vp, _int, _vp, _vp, _vp, _vp, ctypes.c_float, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                  _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_pcfg_best_tree": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),

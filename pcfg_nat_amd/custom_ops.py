@@ -462,9 +462,9 @@ def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unre
 
 class PCFGExtractLinksFunc(Function):
     """The model's link scorer after its projections (glat_decomposed_with_link_two_hands_tri_pcfg.py:153-199): the
-    three batched products go through torch's GEMM library, everything else (masking, the gather of the left terms, the
-    joint log-softmax over (left option, right child) per head, the gate mixture and the whole backward of these) runs
-    in two kernels that never materialise a [B,L,2L,H] tensor."""
+    batched products go through torch's GEMM library (one product forward, two backward), everything else (packing,
+    masking, the gather of the left terms, the joint log-softmax over (left option, right child) per head, the gate
+    mixture and the whole backward of these) runs in five small kernels that never materialise a [B,L,2L,H] tensor."""
 
     @staticmethod
     def forward(ctx, query_chunks, key_chunks_left, key_chunks_right, gate_logits, prev_output_tokens, pad_index,
@@ -474,61 +474,64 @@ class PCFGExtractLinksFunc(Function):
                    left_tree_mask, right_tree_mask, main_chain)
         if query_chunks.dim() != 4 or key_chunks_left.shape != query_chunks.shape or key_chunks_right.shape != query_chunks.shape:
             raise RuntimeError("pcfg_extract_links: query and key chunks must share the shape [bsz, prelen, heads, head_dim]")
+        if not (query_chunks.dtype == key_chunks_left.dtype == key_chunks_right.dtype) or query_chunks.dtype not in _DTYPE_CODE:
+            raise RuntimeError("pcfg_extract_links: query and key chunks must share one of float16, float32, float64")
         B, L, H, F = query_chunks.shape
         if gate_logits.shape != (B, L, H) or prev_output_tokens.shape != (B, L):
             raise RuntimeError("pcfg_extract_links: gate_logits must be [bsz, prelen, heads] and prev_output_tokens [bsz, prelen]")
         if left_tree_mask.shape != (L, L) or right_tree_mask.shape != (L, L) or main_chain.shape != (L,):
             raise RuntimeError("pcfg_extract_links: tree masks must be [prelen, prelen] and main_chain [prelen]")
         dev = query_chunks.device
+        code = _DTYPE_CODE[query_chunks.dtype]
         with torch.cuda.device(dev):
-            qf = query_chunks.float().permute(0, 2, 1, 3).contiguous()
-            klf = key_chunks_left.float().permute(0, 2, 1, 3).contiguous()
-            krf = key_chunks_right.float().permute(0, 2, 1, 3).contiguous()
-            Zac = torch.matmul(qf, krf.transpose(-1, -2))
-            Zbc = torch.matmul(klf, krf.transpose(-1, -2))
+            st = _stream(query_chunks)
+            q, kl, kr = query_chunks.contiguous(), key_chunks_left.contiguous(), key_chunks_right.contiguous()
+            A = torch.empty((B, H, 2 * L, F), dtype=torch.float32, device=dev)
+            Kr = torch.empty((B, H, L, F), dtype=torch.float32, device=dev)
+            _lib.check(lib.pcfgnat_extract_links_pack(q.data_ptr(), kl.data_ptr(), kr.data_ptr(), code, A.data_ptr(), Kr.data_ptr(),
+                                                      B, L, H, F, st), lib)
+            Z = torch.matmul(A, Kr.transpose(-1, -2))
             gate = gate_logits.float().contiguous()
             prev = prev_output_tokens.to(torch.int64).contiguous()
-            ltm = left_tree_mask.ne(0).to(torch.uint8).contiguous()
-            rtm = right_tree_mask.ne(0).to(torch.uint8).contiguous()
-            mc = main_chain.ne(0).to(torch.uint8).contiguous()
+            masks = []
+            for t in (left_tree_mask, right_tree_mask, main_chain):
+                masks.append(t.contiguous() if t.dtype in (torch.bool, torch.uint8) else t.ne(0).contiguous())
             links = torch.empty((B, L, 2, L), dtype=torch.float32, device=dev)
             lse = torch.empty((B, L, H), dtype=torch.float32, device=dev)
-            _lib.check(lib.pcfgnat_extract_links_forward(Zac.data_ptr(), Zbc.data_ptr(), qf.data_ptr(), klf.data_ptr(), gate.data_ptr(),
-                                                         prev.data_ptr(), int(pad_index), ltm.data_ptr(), rtm.data_ptr(), mc.data_ptr(),
-                                                         links.data_ptr(), lse.data_ptr(), B, L, H, F, _stream(qf)), lib)
-        ctx.save_for_backward(links, lse, Zac, Zbc, qf, klf, krf, gate, prev, ltm, rtm, mc)
+            _lib.check(lib.pcfgnat_extract_links_forward(Z.data_ptr(), A.data_ptr(), gate.data_ptr(), prev.data_ptr(), int(pad_index),
+                                                         masks[0].data_ptr(), masks[1].data_ptr(), masks[2].data_ptr(),
+                                                         links.data_ptr(), lse.data_ptr(), B, L, H, F, st), lib)
+        ctx.save_for_backward(links, lse, Z, A, Kr, gate, prev, *masks)
         ctx.pad_index = int(pad_index)
-        ctx.in_dtypes = (query_chunks.dtype, key_chunks_left.dtype, key_chunks_right.dtype, gate_logits.dtype)
+        ctx.chunk_dtype, ctx.gate_dtype = query_chunks.dtype, gate_logits.dtype
         return links
 
     @staticmethod
     def backward(ctx, grad_links):
         lib = get_pcfg_kernel()
-        links, lse, Zac, Zbc, qf, klf, krf, gate, prev, ltm, rtm, mc = ctx.saved_tensors
-        B, H, L, F = qf.shape
-        with torch.cuda.device(qf.device):
+        links, lse, Z, A, Kr, gate, prev, ltm, rtm, mc = ctx.saved_tensors
+        B, H, L2, F = A.shape
+        L = L2 // 2
+        dev = A.device
+        with torch.cuda.device(dev):
+            st = _stream(A)
             G = grad_links.float().contiguous()
-            dZac, dZbc, dZ0 = torch.empty_like(Zac), torch.empty_like(Zac), torch.empty_like(Zac)
-            dsab = torch.empty((B, H, L, 2), dtype=torch.float32, device=qf.device)
-            dgate = torch.empty((B, L, H), dtype=torch.float32, device=qf.device)
-            _lib.check(lib.pcfgnat_extract_links_backward(G.data_ptr(), links.data_ptr(), lse.data_ptr(), Zac.data_ptr(), Zbc.data_ptr(),
-                                                          qf.data_ptr(), klf.data_ptr(), gate.data_ptr(), prev.data_ptr(), ctx.pad_index,
-                                                          ltm.data_ptr(), rtm.data_ptr(), mc.data_ptr(), dZac.data_ptr(), dZbc.data_ptr(),
-                                                          dZ0.data_ptr(), dsab.data_ptr(), dgate.data_ptr(), B, L, H, F, _stream(qf)), lib)
-            dZbc[:, :, 0, :] += dZ0.sum(dim=2)  # every parent's null left child is node 0
-            dq = torch.matmul(dZac, krf)
-            dkr = torch.matmul(dZac.transpose(-1, -2), qf) + torch.matmul(dZbc.transpose(-1, -2), klf)
-            dkl = torch.matmul(dZbc, krf)
-            # the two q.kl dot products of every parent a: with kl[0] and with kl[max(a-1, 0)]
-            d0, d1 = dsab[..., 0:1], dsab[..., 1:2]
-            kl_prev = torch.cat((klf[:, :, :1], klf[:, :, :-1]), dim=2)
-            dq += d0 * klf[:, :, 0:1, :] + d1 * kl_prev
-            t = d1 * qf
-            dkl[:, :, 0, :] += (d0 * qf).sum(dim=2) + t[:, :, 0, :]
-            dkl[:, :, :-1, :] += t[:, :, 1:, :]
-        dt = ctx.in_dtypes
-        return (dq.permute(0, 2, 1, 3).to(dt[0]), dkl.permute(0, 2, 1, 3).to(dt[1]), dkr.permute(0, 2, 1, 3).to(dt[2]),
-                dgate.to(dt[3]), None, None, None, None, None)
+            dZ = torch.empty_like(Z)
+            dZ0 = torch.empty((B, H, L, L), dtype=torch.float32, device=dev)
+            dsab = torch.empty((B, H, L, 2), dtype=torch.float32, device=dev)
+            dgate = torch.empty((B, L, H), dtype=torch.float32, device=dev)
+            _lib.check(lib.pcfgnat_extract_links_backward(G.data_ptr(), links.data_ptr(), lse.data_ptr(), Z.data_ptr(), A.data_ptr(),
+                                                          gate.data_ptr(), prev.data_ptr(), ctx.pad_index, ltm.data_ptr(), rtm.data_ptr(),
+                                                          mc.data_ptr(), dZ.data_ptr(), dZ0.data_ptr(), dsab.data_ptr(), dgate.data_ptr(),
+                                                          B, L, H, F, st), lib)
+            dA = torch.matmul(dZ, Kr)
+            dKr = torch.matmul(dZ.transpose(-1, -2), A)
+            dq = torch.empty((B, L, H, F), dtype=ctx.chunk_dtype, device=dev)
+            dkl, dkr = torch.empty_like(dq), torch.empty_like(dq)
+            _lib.check(lib.pcfgnat_extract_links_unpack(dA.data_ptr(), dKr.data_ptr(), dsab.data_ptr(), A.data_ptr(),
+                                                        _DTYPE_CODE[ctx.chunk_dtype], dq.data_ptr(), dkl.data_ptr(), dkr.data_ptr(),
+                                                        B, L, H, F, st), lib)
+        return dq, dkl, dkr, dgate.to(ctx.gate_dtype), None, None, None, None, None
 
 
 def pcfg_extract_links(query_chunks, key_chunks_left, key_chunks_right, gate_logits, prev_output_tokens, pad_index, left_tree_mask,
