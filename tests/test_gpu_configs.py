@@ -155,3 +155,51 @@ def test_config4_viterbi_decode():
             got_tok, got_len = harness.viterbi_decode(ob, tok, links.to(DEV), m.to(DEV), mask.to(DEV), single_call=single_call)
             assert torch.equal(got_len.cpu(), want_len)
             assert torch.equal(got_tok.cpu(), want_tok)
+
+
+def test_config2_link_scorer_full_size():
+    """The link scorer at the training shape (B=40, L=128, 8 heads of 64): forward and all four gradients against the torch
+    restatement evaluated in float64 on the device; prints the time of both (the restatement in fp32, as the model runs it)."""
+    import time
+    from oracle import extract_links_ref as ref
+    B, L, H, F = 40, 128, 8, 64
+    g = torch.Generator().manual_seed(0)
+    q, kl, kr = ((torch.randn(B, L, H, F, generator=g) * 0.5).half().to(DEV) for _ in range(3))
+    gate = torch.randn(B, L, H, generator=g).half().to(DEV)
+    m, _ = synth._wmt_lengths(B, torch.Generator().manual_seed(1001), 10, L // 4, 32)
+    prev = torch.full((B, L), 3).masked_fill(torch.arange(L).view(1, L) >= m.view(B, 1), synth.PAD).to(DEV)
+    lm, rm, mc = (x.to(DEV) for x in synth.support_masks(L, 1))
+    leaves = [t.double().requires_grad_(True) for t in (q, kl, kr, gate)]
+    want = ref.extract_links(*leaves, prev, synth.PAD, lm, rm, mc).double()
+    fin = torch.isfinite(want)
+    G = torch.randn(want.shape, generator=g, dtype=torch.float64).to(DEV).masked_fill(~fin, 0)
+    want.masked_fill(~fin, 0).mul(G).sum().backward()
+    mine = [t.clone().requires_grad_(True) for t in (q, kl, kr, gate)]
+    got = ops.pcfg_extract_links(*mine, prev, synth.PAD, lm, rm, mc)
+    assert torch.equal(torch.isfinite(got), fin)
+    assert torch.allclose(got.double()[fin], want.detach()[fin], rtol=2e-5, atol=2e-5)
+    rows = torch.logsumexp(got.view(B, L, -1), -1)
+    usable = torch.isfinite(rows)
+    assert torch.allclose(rows[usable], torch.zeros_like(rows[usable]), atol=2e-5)  # every usable row is a distribution
+    got.backward(G.float())
+    for name, a, b in zip(("q", "kl", "kr", "gate"), mine, leaves):
+        err = ((a.grad.double() - b.grad).abs().max() / b.grad.abs().max()).item()
+        print("link scorer gradient %s: normwise error %.2e" % (name, err))
+        assert err <= 2e-3  # gradients are returned in the inputs' fp16
+
+    def timed(fn, reps=10):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps * 1e6
+
+    def run(fn_links):
+        ts = [t.detach().clone().requires_grad_(True) for t in (q, kl, kr, gate)]
+        fn_links(*ts).backward(G.float())
+    t_ours = timed(lambda: run(lambda *t: ops.pcfg_extract_links(*t, prev, synth.PAD, lm, rm, mc)))
+    t_ref = timed(lambda: run(lambda *t: ref.extract_links(*t, prev, synth.PAD, lm, rm, mc).masked_fill(~fin, 0)))
+    print("link scorer forward+backward: %.0f us here, %.0f us for the torch restatement" % (t_ours, t_ref))
