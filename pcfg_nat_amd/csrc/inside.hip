@@ -974,13 +974,16 @@ __global__ __launch_bounds__(BT_NT) void best_tree_ml1_kernel(const float *__res
 // log-sum-exps over chunks of children.  Rule posteriors are produced by a separate, fully parallel kernel from the
 // outside weights the sweep leaves behind.
 // All tables are relative to the column offsets described at the top of this file (natural logarithms here).
-// Aux layout per sentence (Mc > 128): F0h, F1h, Bh, W0, W1, R [Mc][T+2] each, D [T+4], then At [2][Mc][Mc].
+// Aux layout per sentence (Mc > 128): F0h, F1h, Bh, W0, W1, R [Mc][T+2] each, D [T+4], padding to a 16-byte boundary,
+// then the compact link matrices with masked entries already -inf and rows padded to MP = 64*ceil(Mc/64) floats:
+// Ac [2][Mc][MP] by parent (Ac[k][a][c]) for the forward sweep and At [2][Mc][MP] by child (At[k][c][a]) for the
+// outside sweep, so that the sweeps stream them with unconditional 16-byte loads.
 // ------------------------------------------------------------------------------------------------------------
-__host__ __device__ inline size_t aux_stride_stream(int Mc, int T) {
-    return (size_t)6 * Mc * (T + 2) + (size_t)(T + 4) + (size_t)2 * Mc * Mc;
-}
+__host__ __device__ inline int stream_mp(int Mc) { return ((Mc + 63) / 64) * 64; }
+__host__ __device__ inline size_t stream_planes(int Mc, int T) { return (((size_t)6 * Mc * (T + 2) + (size_t)(T + 4)) + 3) & ~(size_t)3; }
+__host__ __device__ inline size_t aux_stride_stream(int Mc, int T) { return stream_planes(Mc, T) + (size_t)4 * Mc * stream_mp(Mc); }
 struct AuxViewStream {
-    float *F0, *F1, *BETA, *W0, *W1, *SR, *D, *At;
+    float *F0, *F1, *BETA, *W0, *W1, *SR, *D, *Ac, *At;
     __device__ AuxViewStream(float *aux, int b, int Mc, int T) {
         const size_t plane = (size_t)Mc * (T + 2);
         float *base = aux + (size_t)b * aux_stride_stream(Mc, T);
@@ -991,7 +994,8 @@ struct AuxViewStream {
         W1 = base + 4 * plane;
         SR = base + 5 * plane;
         D = base + 6 * plane;
-        At = D + (T + 4);
+        Ac = base + stream_planes(Mc, T);
+        At = Ac + (size_t)2 * Mc * stream_mp(Mc);
     }
 };
 
@@ -1006,6 +1010,10 @@ struct OnlineLse {
             m = cm;
         }
         if (m != NEG_INF_F) s += (__expf(v[0] - m) + __expf(v[1] - m)) + (__expf(v[2] - m) + __expf(v[3] - m));
+    }
+    __device__ __forceinline__ void add4(const float4 &a, const float4 &b) {  // folds a + b
+        const float v[4] = {a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w};
+        add4(v);
     }
     // combine the 16 lanes of a DPP row; every lane gets log-sum-exp of all folded terms
     __device__ __forceinline__ float finish16() const {
@@ -1033,7 +1041,6 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
     const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const float *mt = match_all + (size_t)b * L * T;
-    const float *lk = links + (size_t)b * L * 2 * L;
     float *Sb = S + (size_t)b * Mc * (T + 2);
     AuxViewStream av(aux, b, Mc, T);
 
@@ -1070,7 +1077,7 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
     __syncthreads();
 
     const int ntiles = (mc + 63) / 64;
-    const int nq = (mc + 15) / 16;
+    const int nq64 = (mc + 63) / 64;
     double O = 0.0;  // offset of the column being read
     for (int t = n - 1; t >= 1; t--) {
         const float *cur = col + (t & 1) * MP;
@@ -1082,7 +1089,6 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
         for (int tile = 0; tile < ntiles; tile++) {
             const int a_id = tile * 64 + gidx, a = 2 * a_id + 1;
             const bool row_ok = a_id < mc;
-            const float *l0 = lk + ((size_t)a * 2 + 0) * L, *l1 = lk + ((size_t)a * 2 + 1) * L;
             // emissions of this row first: their latency overlaps the child loop
             float ma_p, ml_p, ma_t;
             if (MATCH_LDS) {
@@ -1096,21 +1102,22 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
                 ml_p = (row_ok && a_id >= 1) ? sanitize(mt[rl + t - 1]) : NEG_INF_F;
                 ma_t = row_ok ? sanitize(mt[ra + t]) : NEG_INF_F;
             }
+            // children in chunks of 64 (16 lanes x 4), the next chunk's link values requested before this one is folded
             OnlineLse acc0, acc1;
-            for (int qb = 4 * tile; qb < nq; qb += 4) {
-                float v0[4], v1[4];
-#pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    const int c_id = j + 16 * (qb + u);
-                    const bool ok = row_ok && c_id < mc && c_id >= a_id;
-                    const float sc = (c_id < MP) ? cur[c_id] : NEG_INF_F;
-                    const float x0 = ok ? sanitize(l0[2 * c_id + 1]) : NEG_INF_F;
-                    const float x1 = (ok && a_id >= 1) ? sanitize(l1[2 * c_id + 1]) : NEG_INF_F;
-                    v0[u] = x0 + sc;
-                    v1[u] = x1 + sc;
+            const int ar = row_ok ? a_id : Mc - 1;  // rows beyond the sentence: any valid address, the result is discarded
+            const float4 *r0 = reinterpret_cast<const float4 *>(av.Ac + ((size_t)0 * Mc + ar) * MP) + j;
+            const float4 *r1 = reinterpret_cast<const float4 *>(av.Ac + ((size_t)1 * Mc + ar) * MP) + j;
+            const float4 *cv = reinterpret_cast<const float4 *>(cur) + j;
+            float4 x0 = r0[16 * tile], x1 = r1[16 * tile];
+            for (int q = tile; q < nq64; q++) {
+                const float4 y0 = x0, y1 = x1;
+                if (q + 1 < nq64) {
+                    x0 = r0[16 * (q + 1)];
+                    x1 = r1[16 * (q + 1)];
                 }
-                acc0.add4(v0);
-                acc1.add4(v1);
+                const float4 sc = cv[16 * q];
+                acc0.add4(y0, sc);
+                acc1.add4(y1, sc);
             }
             const float F0 = acc0.finish16() - Ds;
             const float F1 = acc1.finish16() - Ds;
@@ -1143,9 +1150,11 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
     }
 }
 
-// At[k][c_id][a_id] = links[2*a_id+1][k][2*c_id+1] (compact, transposed), -inf outside a_id <= c_id < mc.
-__global__ __launch_bounds__(256) void transpose_links_ml1_kernel(const float *__restrict__ links, const int64_t *__restrict__ out_len,
-                                                                 float *__restrict__ aux, int L, int T, int Mc) {
+// Compact copies of the main-chain links for the streaming sweeps: Ac[k][a_id][c_id] = At[k][c_id][a_id] =
+// links[2*a_id+1][k][2*c_id+1] where a_id <= c_id < mc (k = 1 needs a_id >= 1), -inf everywhere else including the
+// padding columns up to MP.  One block per 32 x 32 tile of (parent, child) pairs, grid (MP/32, MP/32, B).
+__global__ __launch_bounds__(256) void compact_links_ml1_kernel(const float *__restrict__ links, const int64_t *__restrict__ out_len,
+                                                               float *__restrict__ aux, int L, int T, int Mc, int MP) {
     __shared__ float tile[2][32][33];
     const int b = blockIdx.z;
     const int m = (int)out_len[b];
@@ -1158,15 +1167,21 @@ __global__ __launch_bounds__(256) void transpose_links_ml1_kernel(const float *_
         const int a_id = a0 + r, c_id = c0 + tx;
         const bool ok = a_id < mc && c_id < mc && a_id <= c_id;
         const size_t row = (size_t)(2 * a_id + 1) * 2;
-        tile[0][r][tx] = ok ? sanitize(lk[(row + 0) * L + 2 * c_id + 1]) : NEG_INF_F;
-        tile[1][r][tx] = (ok && a_id >= 1) ? sanitize(lk[(row + 1) * L + 2 * c_id + 1]) : NEG_INF_F;
+        const float x0 = ok ? sanitize(lk[(row + 0) * L + 2 * c_id + 1]) : NEG_INF_F;
+        const float x1 = (ok && a_id >= 1) ? sanitize(lk[(row + 1) * L + 2 * c_id + 1]) : NEG_INF_F;
+        tile[0][r][tx] = x0;
+        tile[1][r][tx] = x1;
+        if (a_id < Mc) {
+            av.Ac[((size_t)0 * Mc + a_id) * MP + c_id] = x0;
+            av.Ac[((size_t)1 * Mc + a_id) * MP + c_id] = x1;
+        }
     }
     __syncthreads();
     for (int r = ty; r < 32; r += 8) {
         const int c_id = c0 + r, a_id = a0 + tx;
-        if (c_id < Mc && a_id < Mc) {
-            av.At[((size_t)0 * Mc + c_id) * Mc + a_id] = tile[0][tx][r];
-            av.At[((size_t)1 * Mc + c_id) * Mc + a_id] = tile[1][tx][r];
+        if (c_id < Mc) {
+            av.At[((size_t)0 * Mc + c_id) * MP + a_id] = tile[0][tx][r];
+            av.At[((size_t)1 * Mc + c_id) * MP + a_id] = tile[1][tx][r];
         }
     }
 }
@@ -1239,24 +1254,20 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
             const int ci = live ? c_id : 0;
             const float mc_t = live ? match_main(ci, t) : NEG_INF_F;
             const float ml_p = live ? match_leaf(ci, t - 1) : NEG_INF_F;
-            const float *at0 = av.At + ((size_t)0 * Mc + ci) * Mc, *at1 = av.At + ((size_t)1 * Mc + ci) * Mc;
+            // parents in chunks of 64 (16 lanes x 4) up to the child's own chunk, the next chunk requested ahead
+            const float4 *r0 = reinterpret_cast<const float4 *>(av.At + ((size_t)0 * Mc + ci) * MP) + j;
+            const float4 *r1 = reinterpret_cast<const float4 *>(av.At + ((size_t)1 * Mc + ci) * MP) + j;
+            const float4 *u0 = reinterpret_cast<const float4 *>(c0) + j, *u1 = reinterpret_cast<const float4 *>(c1) + j;
             OnlineLse acc;
-            const int q_end = min((mc + 15) / 16, 4 * tile + 4);
-            for (int qb = 0; qb < q_end; qb += 4) {
-                float v0[4], v1[4];
-#pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    const int a_id = j + 16 * (qb + u);
-                    const bool ok = live && a_id < mc && a_id <= c_id;
-                    const float x0 = ok ? at0[a_id] : NEG_INF_F;
-                    const float x1 = ok ? at1[a_id] : NEG_INF_F;
-                    const float u0 = (a_id < MP) ? c0[a_id] : NEG_INF_F;
-                    const float u1 = (a_id < MP) ? c1[a_id] : NEG_INF_F;
-                    v0[u] = x0 + u0;
-                    v1[u] = x1 + u1;
+            float4 x0 = r0[0], x1 = r1[0];
+            for (int q = 0; q <= tile; q++) {
+                const float4 y0 = x0, y1 = x1;
+                if (q < tile) {
+                    x0 = r0[16 * (q + 1)];
+                    x1 = r1[16 * (q + 1)];
                 }
-                acc.add4(v0);
-                acc.add4(v1);
+                acc.add4(y0, u0[16 * q]);
+                acc.add4(y1, u1[16 * q]);
             }
             float beta = acc.finish16();
             if (!live) beta = NEG_INF_F;
@@ -1385,7 +1396,10 @@ __global__ __launch_bounds__(256) void criterion_loss_kernel(const float *__rest
 
 int launch_fwd_stream(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B,
                       int L, int T, int Mc, hipStream_t stream) {
-    const int MP = ((Mc + 63) / 64) * 64;
+    const int MP = stream_mp(Mc);
+    PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss: aux must be 16-byte aligned");
+    hipLaunchKernelGGL(compact_links_ml1_kernel, dim3(MP / 32, MP / 32, B), dim3(256), 0, stream, links, ol, aux, L, T, Mc, MP);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
     const size_t base = ((size_t)3 * MP + 32) * sizeof(float);
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
     if (with_match <= LDS_BUDGET) {
@@ -1402,10 +1416,9 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
 
 int launch_bwd_stream(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
                       const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream) {
-    const int MP = ((Mc + 63) / 64) * 64;
+    const int MP = stream_mp(Mc);
     const int tiles = (Mc + 31) / 32;
-    hipLaunchKernelGGL(transpose_links_ml1_kernel, dim3(tiles, tiles, B), dim3(256), 0, stream, links, ol, aux, L, T, Mc);
-    PCFGNAT_HIP_CHECK(hipGetLastError());
+    PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss_backward: aux must be 16-byte aligned");
     const size_t base = ((size_t)5 * MP + T + 4) * sizeof(float);
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
     if (with_match <= LDS_BUDGET) {
