@@ -974,8 +974,9 @@ __global__ __launch_bounds__(BT_NT) void best_tree_ml1_kernel(const float *__res
 // log-sum-exps over chunks of children.  Rule posteriors are produced by a separate, fully parallel kernel from the
 // outside weights the sweep leaves behind.
 // All tables are relative to the column offsets described at the top of this file (natural logarithms here).
-// Aux layout per sentence (Mc > 128): F0h, F1h, Bh, W0, W1, R [Mc][T+2] each, D [T+4], padding to a 16-byte boundary,
-// then the compact link matrices with masked entries already -inf and rows padded to MP = 64*ceil(Mc/64) floats:
+// Aux layout per sentence (Mc > 128), log-domain values in base 2 like everything inside these kernels: F0h, F1h, Bh,
+// W0, W1, R [Mc][T+2] each, D [T+4], padding to a 16-byte boundary, then the compact link matrices (times log2 e) with
+// masked entries already -inf and rows padded to MP = 64*ceil(Mc/64) floats:
 // Ac [2][Mc][MP] by parent (Ac[k][a][c]) for the forward sweep and At [2][Mc][MP] by child (At[k][c][a]) for the
 // outside sweep, so that the sweeps stream them with unconditional 16-byte loads.
 // ------------------------------------------------------------------------------------------------------------
@@ -999,34 +1000,117 @@ struct AuxViewStream {
     }
 };
 
-struct OnlineLse {
+// The streaming sweeps give a node SL lanes (4, 8 or 16), each of which takes four consecutive entries of every chunk of
+// 4*SL, and handle NT/SL nodes per pass.  Fewer lanes per node mean fewer passes and reductions per column, more lanes
+// mean longer contiguous reads per node.
+template <int SL>
+__device__ __forceinline__ float node_max(float v) {
+    if (SL == 4) return dpp_max_xor2(dpp_max_xor1(v));
+    return SL == 8 ? row8_max(v) : row16_max(v);
+}
+template <int SL>
+__device__ __forceinline__ float node_sum(float v) {
+    if (SL == 4) {
+        v += dpp_f<DPP_QUAD_XOR1>(v);
+        v += dpp_f<DPP_QUAD_XOR2>(v);
+        return v;
+    }
+    return SL == 8 ? row8_sum(v) : row16_sum(v);
+}
+
+// log2-sum-exp2 with a running maximum, four terms at a time; SL lanes share a row
+template <int SL>
+struct RunningLse {
     float m, s;
-    __device__ OnlineLse() : m(NEG_INF_F), s(0.f) {}
-    // fold four terms in
-    __device__ __forceinline__ void add4(const float *v) {
-        const float cm = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
+    __device__ RunningLse() : m(NEG_INF_F), s(0.f) {}
+    __device__ __forceinline__ void add4(const float4 &a, const float4 &b) {  // folds a + b
+        const float v0 = a.x + b.x, v1 = a.y + b.y, v2 = a.z + b.z, v3 = a.w + b.w;
+        const float cm = fmaxf(fmaxf(v0, v1), fmaxf(v2, v3));
         if (cm > m) {
-            s *= __expf(m - cm);  // m = -inf gives 0 * 0
+            s *= ex2(m - cm);  // m = -inf gives 0 * 0
             m = cm;
         }
-        if (m != NEG_INF_F) s += (__expf(v[0] - m) + __expf(v[1] - m)) + (__expf(v[2] - m) + __expf(v[3] - m));
+        if (m != NEG_INF_F) s += (ex2(v0 - m) + ex2(v1 - m)) + (ex2(v2 - m) + ex2(v3 - m));
     }
-    __device__ __forceinline__ void add4(const float4 &a, const float4 &b) {  // folds a + b
-        const float v[4] = {a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w};
-        add4(v);
+    __device__ __forceinline__ void merge(const RunningLse<SL> &o) {
+        const float M = fmaxf(m, o.m);
+        if (M == NEG_INF_F) return;
+        s = s * ex2(m - M) + o.s * ex2(o.m - M);
+        m = M;
     }
-    // combine the 16 lanes of a DPP row; every lane gets log-sum-exp of all folded terms
-    __device__ __forceinline__ float finish16() const {
-        const float M = row16_max(m);
-        const float part = (m == NEG_INF_F) ? 0.f : s * __expf(m - M);
-        const float tot = row16_sum(part);
-        return (M == NEG_INF_F) ? NEG_INF_F : M + __logf(tot);
+    // combine the lanes of a node; every lane gets the log2-sum-exp2 of all folded terms
+    __device__ __forceinline__ float finish() const {
+        const float M = node_max<SL>(m + 0.f);  // the add keeps the reduction's input from being a raw exp/log result
+        const float part = (m == NEG_INF_F) ? 0.f : s * ex2(m - M);
+        const float tot = node_sum<SL>(part);
+        return (M == NEG_INF_F) ? NEG_INF_F : M + lg2(tot);
     }
 };
 
-// Dynamic LDS: col[2][MP], f1prev[MP], per-wave column maxima slots[2][16], then (if MATCH_LDS) match main [Mc][T],
-// match leaf [Mc][T].
-template <bool MATCH_LDS>
+__device__ __forceinline__ float sum4_ex2(const float4 &a, const float4 &b, float g) {
+    return (ex2((a.x + b.x) - g) + ex2((a.y + b.y) - g)) + (ex2((a.z + b.z) - g) + ex2((a.w + b.w) - g));
+}
+__device__ __forceinline__ bool is_finite(float v) { return fabsf(v) < __builtin_huge_valf(); }  // false for NaN too
+
+// Base-2 log-sum-exp of one node's two link rows r0, r1 (SL lanes per node, each lane four consecutive entries of every
+// chunk q in [q0, q1)) against LDS columns: out0 = LSE_i(r0[i] + u0[i]), out1 = LSE_i(r1[i] + u1[i]), or with
+// JOINT the one value LSE over both in out0; has1 = false says that r1 is known to be all -inf.  The terms are first summed relative to a guess of the result (the same
+// node's value one column earlier, which differs by about one token's log-probability).  The sum is accepted when it
+// lies in [2^-90, 2^100]: then no term overflowed and the terms flushed to zero are below 2^-126 each, i.e. far below
+// rounding.  Otherwise (no derivation at all, first columns, a guess that is far off) the rows are read again and
+// folded with a running maximum, which is exact for any input.  Link values are requested one chunk ahead: x0, x1 hold
+// the row's first chunk on entry and, on exit, the chunk at n0, n1 (the first chunk of the row this lane handles next).
+template <bool JOINT, int SL>
+__device__ __forceinline__ void stream_row_lse(const float4 *__restrict__ r0, const float4 *__restrict__ r1, const float4 *u0,
+                                               const float4 *u1, int q0, int q1, bool live, bool has1, float g0, float g1,
+                                               float4 &x0, float4 &x1, const float4 *__restrict__ n0,
+                                               const float4 *__restrict__ n1, float &out0, float &out1) {
+    g0 = is_finite(g0) ? g0 : 0.f;
+    g1 = JOINT ? g0 : (is_finite(g1) ? g1 : 0.f);
+    float s0 = 0.f, s1 = 0.f;
+    for (int q = q0; q < q1; q++) {
+        const float4 y0 = x0, y1 = x1;
+        const bool last = q + 1 == q1;
+        x0 = *(last ? n0 : r0 + SL * (q + 1));
+        x1 = *(last ? n1 : r1 + SL * (q + 1));
+        const float4 c0 = u0[SL * q];
+        const float4 c1 = JOINT ? u1[SL * q] : c0;
+        s0 += sum4_ex2(y0, c0, g0);
+        s1 += sum4_ex2(y1, c1, g1);
+    }
+    bool ok;
+    if (JOINT) {
+        const float tot = node_sum<SL>(s0 + s1);
+        ok = tot >= 0x1p-90f && tot <= 0x1p100f;
+        out0 = g0 + lg2(tot);
+        out1 = out0;
+    } else {
+        const float t0 = node_sum<SL>(s0), t1 = node_sum<SL>(s1);
+        ok = t0 >= 0x1p-90f && t0 <= 0x1p100f && ((t1 >= 0x1p-90f && t1 <= 0x1p100f) || !has1);
+        out0 = g0 + lg2(t0);
+        out1 = has1 ? g1 + lg2(t1) : NEG_INF_F;
+    }
+    if (live && !ok) {  // uniform over the lanes of the node
+        RunningLse<SL> a0, a1;
+        for (int q = q0; q < q1; q++) {
+            const float4 c0 = u0[SL * q];
+            const float4 c1 = JOINT ? u1[SL * q] : c0;
+            a0.add4(r0[SL * q], c0);
+            a1.add4(r1[SL * q], c1);
+        }
+        if (JOINT) {
+            a0.merge(a1);
+            out0 = out1 = a0.finish();
+        } else {
+            out0 = a0.finish();
+            out1 = a1.finish();
+        }
+    }
+}
+
+// Dynamic LDS: col[2][MP], f1prev[MP], f0prev[MP], per-wave column maxima slots[2][16], then (if MATCH_LDS) match main
+// [Mc][T], match leaf [Mc][T].
+template <bool MATCH_LDS, int SL>
 __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
                                                                   const int64_t *__restrict__ out_len,
                                                                   const int64_t *__restrict__ tgt_len, float *__restrict__ S,
@@ -1034,11 +1118,13 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
     extern __shared__ float smem[];
     float *col = smem;               // [2][MP]
     float *f1prev = smem + 2 * MP;    // [MP]
-    float *slots = smem + 3 * MP;     // [2][16]
+    float *f0prev = smem + 3 * MP;    // [MP]  (only a guess for the next column)
+    float *slots = smem + 4 * MP;     // [2][16]
     float *sm_main = slots + 32;      // [Mc][T]
     float *sm_leaf = sm_main + (MATCH_LDS ? Mc * T : 0);
 
-    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
+    constexpr int SCH = 4 * SL, SROWS = NT / SL;
+    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid / SL, j = tid % SL;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const float *mt = match_all + (size_t)b * L * T;
     float *Sb = S + (size_t)b * Mc * (T + 2);
@@ -1053,8 +1139,8 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
         for (int i = tid; i < Mc * T; i += NT) {
             const int a_id = i / T, s = i - a_id * T;
             const bool ok = a_id < mc && s < n;
-            sm_main[i] = ok ? sanitize(mt[(size_t)(2 * a_id + 1) * T + s]) : NEG_INF_F;
-            sm_leaf[i] = (ok && a_id >= 1) ? sanitize(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
+            sm_main[i] = ok ? to_b2(mt[(size_t)(2 * a_id + 1) * T + s]) : NEG_INF_F;
+            sm_leaf[i] = (ok && a_id >= 1) ? to_b2(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
         }
     }
     for (int i = tid; i < Mc * (T + 2); i += NT) {
@@ -1063,21 +1149,50 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
             float v = NEG_INF_F;
             if (a_id == mc - 1 && s == n - 1) v = sanitize(mt[(size_t)(m - 1) * T + (n - 1)]);
             Sb[i] = v;
-            av.SR[i] = v;
+            av.SR[i] = v * LOG2E_F;
         }
     }
-    const float base_cell = sanitize(mt[(size_t)(m - 1) * T + (n - 1)]);
+    const float base_cell = to_b2(mt[(size_t)(m - 1) * T + (n - 1)]);
     for (int i = tid; i < MP; i += NT) {
         col[((n - 1) & 1) * MP + i] = (i == mc - 1) ? base_cell : NEG_INF_F;
         col[((n - 2) & 1) * MP + i] = NEG_INF_F;
         f1prev[i] = NEG_INF_F;
+        f0prev[i] = NEG_INF_F;
     }
     if (tid < 32) slots[tid] = base_cell;  // maximum of column n-1
     for (int i = tid; i < T + 4; i += NT) av.D[i] = 0.f;
     __syncthreads();
 
-    const int ntiles = (mc + 63) / 64;
-    const int nq64 = (mc + 63) / 64;
+    const int ntiles = (mc + SROWS - 1) / SROWS, nq = (mc + SCH - 1) / SCH;
+    // What a lane needs from memory for node tile*SROWS+gidx at step t, requested one node ahead (across the step's
+    // barrier too: none of it depends on the column being computed).  q0 = the chunk that holds the node's diagonal, the
+    // same for all nodes of a wave.
+    struct Ahead {
+        const float4 *r0, *r1;
+        float ma_p, ml_p, ma_t;
+        int q0;
+    };
+    auto look_ahead = [&](int tile, int t) -> Ahead {
+        const int a_id = tile * SROWS + gidx;
+        const int ar = a_id < mc ? a_id : Mc - 1;  // rows beyond the sentence: any valid address, the result is discarded
+        Ahead h;
+        h.q0 = min(__builtin_amdgcn_readfirstlane(a_id / SCH), nq - 1);
+        h.r0 = reinterpret_cast<const float4 *>(av.Ac + ((size_t)0 * Mc + ar) * MP) + j;
+        h.r1 = reinterpret_cast<const float4 *>(av.Ac + ((size_t)1 * Mc + ar) * MP) + j;
+        if (MATCH_LDS) {
+            h.ma_p = sm_main[ar * T + t - 1];
+            h.ml_p = sm_leaf[ar * T + t - 1];
+            h.ma_t = sm_main[ar * T + t];
+        } else {
+            const float *ra = mt + (size_t)(2 * ar + 1) * T, *rl = mt + (size_t)(2 * ar) * T;
+            h.ma_p = to_b2(ra[t - 1]);
+            h.ml_p = ar >= 1 ? to_b2(rl[t - 1]) : NEG_INF_F;
+            h.ma_t = to_b2(ra[t]);
+        }
+        return h;
+    };
+    Ahead nx = look_ahead(0, n - 1);
+    float4 x0 = nx.r0[SL * nx.q0], x1 = nx.r1[SL * nx.q0];
     double O = 0.0;  // offset of the column being read
     for (int t = n - 1; t >= 1; t--) {
         const float *cur = col + (t & 1) * MP;
@@ -1087,62 +1202,38 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
         const double O_new = O + (double)Ds;
         float wmax = NEG_INF_F;
         for (int tile = 0; tile < ntiles; tile++) {
-            const int a_id = tile * 64 + gidx, a = 2 * a_id + 1;
+            const int a_id = tile * SROWS + gidx;
             const bool row_ok = a_id < mc;
-            // emissions of this row first: their latency overlaps the child loop
-            float ma_p, ml_p, ma_t;
-            if (MATCH_LDS) {
-                const int ai = row_ok ? a_id : 0;
-                ma_p = sm_main[ai * T + t - 1];
-                ml_p = sm_leaf[ai * T + t - 1];
-                ma_t = sm_main[ai * T + t];
-            } else {
-                const size_t ra = (size_t)a * T, rl = (size_t)(a - 1) * T;
-                ma_p = row_ok ? sanitize(mt[ra + t - 1]) : NEG_INF_F;
-                ml_p = (row_ok && a_id >= 1) ? sanitize(mt[rl + t - 1]) : NEG_INF_F;
-                ma_t = row_ok ? sanitize(mt[ra + t]) : NEG_INF_F;
-            }
-            // children in chunks of 64 (16 lanes x 4), the next chunk's link values requested before this one is folded
-            OnlineLse acc0, acc1;
-            const int ar = row_ok ? a_id : Mc - 1;  // rows beyond the sentence: any valid address, the result is discarded
-            const float4 *r0 = reinterpret_cast<const float4 *>(av.Ac + ((size_t)0 * Mc + ar) * MP) + j;
-            const float4 *r1 = reinterpret_cast<const float4 *>(av.Ac + ((size_t)1 * Mc + ar) * MP) + j;
+            const Ahead me = nx;
+            const bool last_tile = tile + 1 == ntiles;
+            nx = look_ahead(last_tile ? 0 : tile + 1, (last_tile && t > 1) ? t - 1 : t);
+            // children c >= a, from the chunk that holds the diagonal
             const float4 *cv = reinterpret_cast<const float4 *>(cur) + j;
-            float4 x0 = r0[16 * tile], x1 = r1[16 * tile];
-            for (int q = tile; q < nq64; q++) {
-                const float4 y0 = x0, y1 = x1;
-                if (q + 1 < nq64) {
-                    x0 = r0[16 * (q + 1)];
-                    x1 = r1[16 * (q + 1)];
-                }
-                const float4 sc = cv[16 * q];
-                acc0.add4(y0, sc);
-                acc1.add4(y1, sc);
-            }
-            const float F0 = acc0.finish16() - Ds;
-            const float F1 = acc1.finish16() - Ds;
-            const int ai = (a_id < MP) ? a_id : 0;
+            const int ai = min(a_id, MP - 1);  // the last tile may reach beyond the padded node count
             const float f1p = f1prev[ai];
-            float s_new = lse2(ma_p + F0, (ml_p + ma_t) + (f1p - Ds));
+            float F0, F1;
+            stream_row_lse<false, SL>(me.r0, me.r1, cv, cv, me.q0, nq, row_ok, a_id >= 1, f0prev[ai], f1p, x0, x1, nx.r0 + SL * nx.q0,
+                                  nx.r1 + SL * nx.q0, F0, F1);
+            F0 -= Ds;
+            F1 -= Ds;
+            float s_new = lse2_b2(me.ma_p + F0, (me.ml_p + me.ma_t) + (f1p - Ds));
             if (!row_ok) s_new = NEG_INF_F;
             wmax = fmaxf(wmax, s_new);
             if (j == 0 && a_id < MP) {
                 nxt[a_id] = s_new;
                 f1prev[a_id] = F1;
+                f0prev[a_id] = F0;
                 if (row_ok) {
-                    Sb[(size_t)a_id * (T + 2) + (t - 1)] = (float)((double)s_new + O_new);
+                    Sb[(size_t)a_id * (T + 2) + (t - 1)] = (float)(((double)s_new + O_new) * LN2_D);
                     av.SR[(size_t)a_id * (T + 2) + (t - 1)] = s_new;
                     av.F0[(size_t)a_id * (T + 2) + t] = F0;
                     av.F1[(size_t)a_id * (T + 2) + t] = F1;
                 }
             }
         }
-        {   // s_new is uniform inside each 16-lane row: combine the four rows of the wave
-            const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wmax), 0));
-            const float bq = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wmax), 16));
-            const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wmax), 32));
-            const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wmax), 48));
-            if ((tid & 63) == 0) slots[((t - 1) & 1) * 16 + (tid >> 6)] = fmaxf(fmaxf(a, bq), fmaxf(c, d));
+        {
+            const float wm = wave_max(wmax);
+            if ((tid & 63) == 0) slots[((t - 1) & 1) * 16 + (tid >> 6)] = wm;
         }
         if (tid == 0) av.D[t] = Ds;
         O = O_new;
@@ -1151,7 +1242,7 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
 }
 
 // Compact copies of the main-chain links for the streaming sweeps: Ac[k][a_id][c_id] = At[k][c_id][a_id] =
-// links[2*a_id+1][k][2*c_id+1] where a_id <= c_id < mc (k = 1 needs a_id >= 1), -inf everywhere else including the
+// log2(e) * links[2*a_id+1][k][2*c_id+1] where a_id <= c_id < mc (k = 1 needs a_id >= 1), -inf everywhere else including the
 // padding columns up to MP.  One block per 32 x 32 tile of (parent, child) pairs, grid (MP/32, MP/32, B).
 __global__ __launch_bounds__(256) void compact_links_ml1_kernel(const float *__restrict__ links, const int64_t *__restrict__ out_len,
                                                                float *__restrict__ aux, int L, int T, int Mc, int MP) {
@@ -1167,8 +1258,8 @@ __global__ __launch_bounds__(256) void compact_links_ml1_kernel(const float *__r
         const int a_id = a0 + r, c_id = c0 + tx;
         const bool ok = a_id < mc && c_id < mc && a_id <= c_id;
         const size_t row = (size_t)(2 * a_id + 1) * 2;
-        const float x0 = ok ? sanitize(lk[(row + 0) * L + 2 * c_id + 1]) : NEG_INF_F;
-        const float x1 = (ok && a_id >= 1) ? sanitize(lk[(row + 1) * L + 2 * c_id + 1]) : NEG_INF_F;
+        const float x0 = ok ? to_b2(lk[(row + 0) * L + 2 * c_id + 1]) : NEG_INF_F;
+        const float x1 = (ok && a_id >= 1) ? to_b2(lk[(row + 1) * L + 2 * c_id + 1]) : NEG_INF_F;
         tile[0][r][tx] = x0;
         tile[1][r][tx] = x1;
         if (a_id < Mc) {
@@ -1187,7 +1278,7 @@ __global__ __launch_bounds__(256) void compact_links_ml1_kernel(const float *__r
 }
 
 // Outside sweep.  Dynamic LDS: w0[2][MP], w1[2][MP], bprev[MP], D[T+4], then (if MATCH_LDS) match main/leaf [Mc][T] each.
-template <bool MATCH_LDS>
+template <bool MATCH_LDS, int SL>
 __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *__restrict__ S, float *__restrict__ aux,
                                                                   const float *__restrict__ match_all,
                                                                   const int64_t *__restrict__ out_len,
@@ -1200,7 +1291,8 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
     float *sm_main = sm_D + (T + 4);
     float *sm_leaf = sm_main + (MATCH_LDS ? Mc * T : 0);
 
-    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
+    constexpr int SCH = 4 * SL, SROWS = NT / SL;
+    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid / SL, j = tid % SL;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const float *mt = match_all + (size_t)b * L * T;
     const float *Sb = S + (size_t)b * Mc * (T + 2);
@@ -1213,19 +1305,19 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
         for (int i = tid; i < Mc * T; i += NT) {
             const int a_id = i / T, s = i - a_id * T;
             const bool ok = a_id < mc && s < n;
-            sm_main[i] = ok ? sanitize(mt[(size_t)(2 * a_id + 1) * T + s]) : NEG_INF_F;
-            sm_leaf[i] = (ok && a_id >= 1) ? sanitize(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
+            sm_main[i] = ok ? to_b2(mt[(size_t)(2 * a_id + 1) * T + s]) : NEG_INF_F;
+            sm_leaf[i] = (ok && a_id >= 1) ? to_b2(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
         }
     }
     for (int i = tid; i < T + 4; i += NT) sm_D[i] = av.D[i];
     __syncthreads();
     auto match_main = [&](int a_id, int s) -> float {
         if (MATCH_LDS) return sm_main[a_id * T + s];
-        return sanitize(mt[(size_t)(2 * a_id + 1) * T + s]);
+        return to_b2(mt[(size_t)(2 * a_id + 1) * T + s]);
     };
     auto match_leaf = [&](int a_id, int s) -> float {
         if (MATCH_LDS) return sm_leaf[a_id * T + s];
-        return a_id >= 1 ? sanitize(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
+        return a_id >= 1 ? to_b2(mt[(size_t)(2 * a_id) * T + s]) : NEG_INF_F;
     };
     const float beta00 = -av.SR[0];  // relative to the offset of column 0
     const float w00 = (match_main(0, 0) + beta00) - sm_D[1];
@@ -1243,36 +1335,45 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
     }
     __syncthreads();
 
-    const int ntiles = (mc + 63) / 64;
+    const int ntiles = (mc + SROWS - 1) / SROWS, nq = (mc + SCH - 1) / SCH;
+    // what a lane needs from memory for node tile*SROWS+gidx at step t, requested one node ahead; q1 = one past the chunk
+    // that holds the node's diagonal, the same for all nodes of a wave
+    struct Ahead {
+        const float4 *r0, *r1;
+        float mc_t, ml_p;
+        int q1;
+    };
+    auto look_ahead = [&](int tile, int t) -> Ahead {
+        const int c_id = tile * SROWS + gidx;
+        const bool live = c_id < mc;
+        const int ci = live ? c_id : 0;
+        Ahead h;
+        h.q1 = min(__builtin_amdgcn_readfirstlane(c_id / SCH), nq - 1) + 1;
+        h.r0 = reinterpret_cast<const float4 *>(av.At + ((size_t)0 * Mc + ci) * MP) + j;
+        h.r1 = reinterpret_cast<const float4 *>(av.At + ((size_t)1 * Mc + ci) * MP) + j;
+        h.mc_t = live ? match_main(ci, t) : NEG_INF_F;
+        h.ml_p = live ? match_leaf(ci, t - 1) : NEG_INF_F;
+        return h;
+    };
+    Ahead nx = look_ahead(0, 1);
+    float4 x0 = nx.r0[0], x1 = nx.r1[0];
     for (int t = 1; t <= n - 1; t++) {
         const float *c0 = w0 + (t & 1) * MP, *c1 = w1 + (t & 1) * MP;
         float *n0 = w0 + ((t + 1) & 1) * MP, *n1 = w1 + ((t + 1) & 1) * MP;
         const float d_next = sm_D[t + 1], d_both = d_next + sm_D[t];
         for (int tile = 0; tile < ntiles; tile++) {
-            const int c_id = tile * 64 + gidx;
+            const int c_id = tile * SROWS + gidx;
             const bool live = c_id < mc;
-            const int ci = live ? c_id : 0;
-            const float mc_t = live ? match_main(ci, t) : NEG_INF_F;
-            const float ml_p = live ? match_leaf(ci, t - 1) : NEG_INF_F;
-            // parents in chunks of 64 (16 lanes x 4) up to the child's own chunk, the next chunk requested ahead
-            const float4 *r0 = reinterpret_cast<const float4 *>(av.At + ((size_t)0 * Mc + ci) * MP) + j;
-            const float4 *r1 = reinterpret_cast<const float4 *>(av.At + ((size_t)1 * Mc + ci) * MP) + j;
+            const Ahead me = nx;
+            const bool last_tile = tile + 1 == ntiles;
+            nx = look_ahead(last_tile ? 0 : tile + 1, (last_tile && t < n - 1) ? t + 1 : t);
+            const float mc_t = me.mc_t, ml_p = me.ml_p;
+            // parents a <= c, up to the chunk that holds the diagonal
             const float4 *u0 = reinterpret_cast<const float4 *>(c0) + j, *u1 = reinterpret_cast<const float4 *>(c1) + j;
-            OnlineLse acc;
-            float4 x0 = r0[0], x1 = r1[0];
-            for (int q = 0; q <= tile; q++) {
-                const float4 y0 = x0, y1 = x1;
-                if (q < tile) {
-                    x0 = r0[16 * (q + 1)];
-                    x1 = r1[16 * (q + 1)];
-                }
-                acc.add4(y0, u0[16 * q]);
-                acc.add4(y1, u1[16 * q]);
-            }
-            float beta = acc.finish16();
+            const float bp = bprev[min(c_id, MP - 1)];  // the last tile may reach beyond the padded node count
+            float beta, unused;
+            stream_row_lse<true, SL>(me.r0, me.r1, u0, u1, 0, me.q1, live, true, bp, bp, x0, x1, nx.r0, nx.r1, beta, unused);
             if (!live) beta = NEG_INF_F;
-            const int cs = (c_id < MP) ? c_id : 0;
-            const float bp = bprev[cs];
             const float nw0 = (mc_t + beta) - d_next;
             const float nw1 = ((ml_p + mc_t) + bp) - d_both;
             if (j == 0 && c_id < MP) {
@@ -1313,8 +1414,8 @@ __global__ __launch_bounds__(1024) void links_grad_ml1_stream_kernel(const float
     const int a = 2 * a_id + 1, c = 2 * c_id + 1;
     const bool ok = a_id < mc && c_id < mc && a_id <= c_id;
     const float *lk = links + (size_t)b * L * 2 * L;
-    const float A0 = ok ? sanitize(lk[((size_t)a * 2 + 0) * L + c]) : NEG_INF_F;
-    const float A1 = (ok && a_id >= 1) ? sanitize(lk[((size_t)a * 2 + 1) * L + c]) : NEG_INF_F;
+    const float A0 = ok ? to_b2(lk[((size_t)a * 2 + 0) * L + c]) : NEG_INF_F;
+    const float A1 = (ok && a_id >= 1) ? to_b2(lk[((size_t)a * 2 + 1) * L + c]) : NEG_INF_F;
     float acc0 = 0.f, acc1 = 0.f;
     for (int t0 = 1; t0 <= n - 1; t0 += 32) {
         // rows = nodes of the tile, columns = 32 consecutive target positions
@@ -1328,8 +1429,8 @@ __global__ __launch_bounds__(1024) void links_grad_ml1_stream_kernel(const float
 #pragma unroll 8
         for (int u = 0; u < 32; u++) {
             const float sc = ss[tx][u];
-            acc0 += __expf((A0 + sw0[ty][u]) + sc);
-            acc1 += __expf((A1 + sw1[ty][u]) + sc);
+            acc0 += ex2((A0 + sw0[ty][u]) + sc);
+            acc1 += ex2((A1 + sw1[ty][u]) + sc);
         }
         __syncthreads();
     }
@@ -1368,14 +1469,14 @@ __global__ __launch_bounds__(256) void match_grad_ml1_stream_kernel(const float 
         const size_t row = (size_t)a_id * (T + 2);
         if (x & 1) {
             const float bs = av.BETA[row + s];
-            const float mas = sanitize(mt[(size_t)x * T + s]);
-            if (s + 1 <= n - 1) out += __expf(bs + mas + av.F0[row + s + 1]);
+            const float mas = to_b2(mt[(size_t)x * T + s]);
+            if (s + 1 <= n - 1) out += ex2(bs + mas + av.F0[row + s + 1]);
             if (s >= 1 && s + 1 <= n - 1 && a_id >= 1)
-                out += __expf(av.BETA[row + s - 1] + sanitize(mt[(size_t)(x - 1) * T + s - 1]) + mas + (av.F1[row + s + 1] - av.D[s]));
-            if (a_id == mc - 1 && s == n - 1) out += __expf(bs + mas);
+                out += ex2(av.BETA[row + s - 1] + to_b2(mt[(size_t)(x - 1) * T + s - 1]) + mas + (av.F1[row + s + 1] - av.D[s]));
+            if (a_id == mc - 1 && s == n - 1) out += ex2(bs + mas);
         } else if (a_id >= 1 && a_id < mc && s + 2 <= n - 1) {
-            out += __expf(av.BETA[row + s] + sanitize(mt[(size_t)x * T + s]) + sanitize(mt[(size_t)(x + 1) * T + s + 1]) +
-                          (av.F1[row + s + 2] - av.D[s + 1]));
+            out += ex2(av.BETA[row + s] + to_b2(mt[(size_t)x * T + s]) + to_b2(mt[(size_t)(x + 1) * T + s + 1]) +
+                       (av.F1[row + s + 2] - av.D[s + 1]));
         }
         if (!(out == out)) out = 0.f;
     }
@@ -1400,15 +1501,15 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
     PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss: aux must be 16-byte aligned");
     hipLaunchKernelGGL(compact_links_ml1_kernel, dim3(MP / 32, MP / 32, B), dim3(256), 0, stream, links, ol, aux, L, T, Mc, MP);
     PCFGNAT_HIP_CHECK(hipGetLastError());
-    const size_t base = ((size_t)3 * MP + 32) * sizeof(float);
+    const size_t base = ((size_t)4 * MP + 32) * sizeof(float);
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
     if (with_match <= LDS_BUDGET) {
-        auto k = inside_fwd_ml1_stream_kernel<true>;
+        auto k = inside_fwd_ml1_stream_kernel<true, 4>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_match));
         hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_match, stream, match_all, links, ol, tl, S, aux, L, T, Mc, MP);
     } else {
-        hipLaunchKernelGGL((inside_fwd_ml1_stream_kernel<false>), dim3(B), dim3(NT), base, stream, match_all, links, ol, tl, S, aux, L, T,
-                           Mc, MP);
+        hipLaunchKernelGGL((inside_fwd_ml1_stream_kernel<false, 4>), dim3(B), dim3(NT), base, stream, match_all, links, ol, tl, S, aux, L,
+                           T, Mc, MP);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
@@ -1421,12 +1522,14 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
     PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss_backward: aux must be 16-byte aligned");
     const size_t base = ((size_t)5 * MP + T + 4) * sizeof(float);
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
+    // lanes per node: four while one pass covers all nodes; beyond that the outside sweep measured faster with eight
     if (with_match <= LDS_BUDGET) {
-        auto k = inside_bwd_ml1_stream_kernel<true>;
+        auto k = Mc <= NT / 4 ? inside_bwd_ml1_stream_kernel<true, 4> : inside_bwd_ml1_stream_kernel<true, 8>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_match));
         hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_match, stream, S, aux, match_all, ol, tl, L, T, Mc, MP);
     } else {
-        hipLaunchKernelGGL((inside_bwd_ml1_stream_kernel<false>), dim3(B), dim3(NT), base, stream, S, aux, match_all, ol, tl, L, T, Mc, MP);
+        auto k = Mc <= NT / 4 ? inside_bwd_ml1_stream_kernel<false, 4> : inside_bwd_ml1_stream_kernel<false, 8>;
+        hipLaunchKernelGGL(k, dim3(B), dim3(NT), base, stream, S, aux, match_all, ol, tl, L, T, Mc, MP);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     const size_t nlg = (size_t)B * L * 2 * L;
