@@ -237,6 +237,44 @@ def test_inside_forward_backward_vs_oracle(case):
             assert not mg_got[bi].any() and not lg_got[bi].any()
 
 
+@pytest.mark.parametrize("L,T,ms,ns", [(128, 30, [128, 90], [30, 22]), (320, 40, [320, 262], [40, 31]), (600, 24, [600, 520], [24, 24])])
+def test_inside_spiky_inputs_vs_oracle(L, T, ms, ns):
+    """Emissions and links with jumps of hundreds of units and scattered -inf entries: neighbouring columns of the tables
+    then differ by far more than one token's log-probability, which is what the streaming sweeps' guessed shifts (and
+    the column offsets of all sweeps) must survive.  Whole S table (including its -inf pattern) and both gradients
+    against the float64 oracle."""
+    batch = synth.training_batch(len(ms), L, T, 60, ms, ns, seed=L + T)
+    g = torch.Generator().manual_seed(5 * L + 1)
+    match = _match_for(batch)
+    u = torch.rand(match.shape, generator=g)
+    match = match - 300.0 * (u < 0.3) - 700.0 * (u > 0.93)
+    match = match.masked_fill(torch.rand(match.shape, generator=g) < 0.03, float("-inf"))
+    links = batch["links"].clone()
+    v = torch.rand(links.shape, generator=g)
+    links = links - 250.0 * (v < 0.2)
+    links = links.masked_fill(torch.rand(links.shape, generator=g) < 0.05, float("-inf"))
+    batch = dict(batch, links=links)
+    S64, C64, mg64, lg64 = _oracle_inside(batch, match.numpy())
+    ol, tl = batch["output_length"].to(DEV), batch["target_length"].to(DEV)
+    S, _, _, _ = ops._pcfg_loss_tables(match.to(DEV), links.to(DEV), ol, tl, 1, "test")
+    S = S.cpu().double().numpy()
+    assert np.array_equal(np.isneginf(S), np.isneginf(S64))
+    fin = np.isfinite(S64)
+    assert np.isfinite(S64[:, 0, 0]).any()
+    assert np.allclose(S[fin], S64[fin], rtol=2e-6, atol=1e-4)
+    md, ld = match.to(DEV).requires_grad_(True), links.to(DEV).requires_grad_(True)
+    ll = ops.cuda_pcfg_loss(md, ld, ol, tl)
+    ll.masked_fill(~torch.isfinite(ll), 0).sum().backward()
+    mg_got, lg_got = md.grad.cpu().double().numpy(), ld.grad.cpu().double().numpy()
+    assert np.isfinite(mg_got).all() and np.isfinite(lg_got).all()
+    for bi in range(len(ms)):
+        if not np.isfinite(S64[bi, 0, 0]):
+            assert not mg_got[bi].any() and not lg_got[bi].any()
+            continue
+        assert np.abs(mg_got[bi] - mg64[bi]).max() <= 1e-4 * np.abs(mg64[bi]).max(), bi
+        assert np.abs(lg_got[bi] - lg64[bi]).max() <= 1e-4 * np.abs(lg64[bi]).max(), bi
+
+
 def test_inside_tables_match_oracle_layout():
     batch = _train_case("ragged_short")
     match = _match_for(batch)
