@@ -148,6 +148,35 @@ def glat_timing(logits, targets, links, out_len):
     return {"ms_per_call": start.elapsed_time(end) / reps}
 
 
+def long_sentence_timing(dev):
+    """The single-call training pass at the long-sentence configuration (BASELINE config 3: B=8, L=512, T=140, V=40000,
+    every sentence at full length), where the inside sweeps run their streaming kernels (256 main-chain nodes per
+    sentence, link rows re-read from L2 every target position, one CU per sentence)."""
+    import torch
+    from pcfg_nat_amd import harness, synth
+
+    B, L, T, V = 8, 512, 140, 40000
+    gen = torch.Generator().manual_seed(2)
+    m, n = torch.full((B,), L, dtype=torch.int64), torch.full((B,), T, dtype=torch.int64)
+    links = synth.make_links(B, L, m, 1, gen).to(dev)
+    targets = synth.make_targets(B, T, n, V, gen).to(dev)
+    ol, tl = m.to(dev), n.to(dev)
+    ggen = torch.Generator(device=dev).manual_seed(12)
+    warm, reps = 2, 6
+    bufs = [(torch.randn(B, L, V, device=dev, dtype=torch.float32, generator=ggen) * 2).half() for _ in range(warm + reps)]
+    for i in range(warm):
+        harness.train_step_single_call(bufs[i], targets, links, ol, tl)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for i in range(warm, warm + reps):
+        out = harness.train_step_single_call(bufs[i], targets, links, ol, tl)
+    end.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(end) / reps
+    return {"ms_per_step": ms, "sentences_per_s": B / (ms * 1e-3), "workload": "B=8, L=512, T=140, V=40000, fp16 logits"}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -287,6 +316,7 @@ def main():
     if not args.no_decode:
         result["viterbi"] = decode_timing(dev)
         result["glat_alignment"] = glat_timing(torch.randn(B, L, V, device=dev, generator=ggen).mul_(2).half(), targets, links, ol)
+        result["long_sentences"] = long_sentence_timing(dev)
     if not args.no_cpu_baseline:
         batch_cpu = {"output_length": m, "target_length": n, "links": links_cpu, "targets": targets_cpu}
         result["cpu_baseline"] = cpu_baseline(batch_cpu, sample_logits, args.cpu_sentences)

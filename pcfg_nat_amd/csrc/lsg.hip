@@ -449,7 +449,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
     constexpr int EPV = Elem<T>::EPV;
     constexpr int FIX = (TCAP + NT - 1) / NT;
     if (loss.out != nullptr && blockIdx.x == 0) criterion_loss_block<NT>(loss);  // workgroup-uniform
-    __shared__ int s_idx[TCAP];
+    __shared__ __attribute__((aligned(16))) int s_idx[TCAP + 4];  // padded to a multiple of four with -2 (matches nothing)
     __shared__ CT s_g[TCAP];   // cast(g[s]) in the buffer's dtype, widened again
     __shared__ CT s_p[TCAP];   // original probability at idx[s]
     const int tid = threadIdx.x, lane = tid & 63;
@@ -479,7 +479,11 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
         const CT ns = FROM_LOGITS ? -wave_sum(part) : Elem<T>::widen(Elem<T>::narrow(-wave_sum(part)));
         const RowNorm<CT> rn = RowNorm<CT>::from_lse(FROM_LOGITS ? lse[row] : (CT)0);
 
-        for (int s = tid; s < Tn; s += NT) {
+        for (int s = tid; s < ((Tn + 3) & ~3); s += NT) {
+            if (s >= Tn) {
+                s_idx[s] = -2;
+                continue;
+            }
             int64_t t = ir[(int64_t)s * st];
             bool ok = (uint64_t)t < (uint64_t)V;
             s_idx[s] = ok ? (int)t : -1;
@@ -523,12 +527,19 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
             fix[r] = 0;
             if (s < Tn && s_idx[s] >= 0) {
                 const int my = s_idx[s];
-                bool first = true;
-                for (int u = 0; u < s; u++) first = first && (s_idx[u] != my);
-                if (first) {
+                // occurrences of the same column before and after s, four entries per LDS read
+                const int4 *si4 = reinterpret_cast<const int4 *>(s_idx);
+                int before = 0, after = 0;
+                for (int w = 0; w < (Tn + 3) >> 2; w++) {
+                    const int4 q = si4[w];
+                    const int u = 4 * w;
+                    before += (q.x == my && u < s) + (q.y == my && u + 1 < s) + (q.z == my && u + 2 < s) + (q.w == my && u + 3 < s);
+                    after += (q.x == my && u > s) + (q.y == my && u + 1 > s) + (q.z == my && u + 2 > s) + (q.w == my && u + 3 > s);
+                }
+                if (before == 0) {
                     CT v = s_p[s] * ns;
                     if (!FROM_LOGITS) v = Elem<T>::widen(Elem<T>::narrow(v));
-                    for (int u = s; u < Tn; u++)
+                    for (int u = s; u < (after ? Tn : s + 1); u++)
                         if (s_idx[u] == my) v = FROM_LOGITS ? v + s_g[u] : Elem<T>::widen(Elem<T>::narrow(v + s_g[u]));
                     fix[r] = v;
                     lead[r] = true;
