@@ -1047,48 +1047,57 @@ struct RunningLse {
     }
 };
 
-__device__ __forceinline__ float sum4_ex2(const float4 &a, const float4 &b, float g) {
-    return (ex2((a.x + b.x) - g) + ex2((a.y + b.y) - g)) + (ex2((a.z + b.z) - g) + ex2((a.w + b.w) - g));
+__device__ __forceinline__ float sum4_ex2(const float4 &a, const float4 &b) {
+    return (ex2(a.x + b.x) + ex2(a.y + b.y)) + (ex2(a.z + b.z) + ex2(a.w + b.w));
 }
+__device__ __forceinline__ float4 minus(const float4 &a, float g) { return make_float4(a.x - g, a.y - g, a.z - g, a.w - g); }
 __device__ __forceinline__ bool is_finite(float v) { return fabsf(v) < __builtin_huge_valf(); }  // false for NaN too
 
 // Base-2 log-sum-exp of one node's two link rows r0, r1 (SL lanes per node, each lane four consecutive entries of every
 // chunk q in [q0, q1)) against LDS columns: out0 = LSE_i(r0[i] + u0[i]), out1 = LSE_i(r1[i] + u1[i]), or with
-// JOINT the one value LSE over both in out0; has1 = false says that r1 is known to be all -inf.  The terms are first summed relative to a guess of the result (the same
-// node's value one column earlier, which differs by about one token's log-probability).  The sum is accepted when it
+// JOINT the one value LSE over both in out0; has1 = false says that r1 is known to be all -inf.  The terms are first
+// summed relative to a guess g of the results (the node's out0 one column earlier, which differs from the new one by about
+// one token's log-probability and from out1 by about one link's).  A sum is accepted when it
 // lies in [2^-90, 2^100]: then no term overflowed and the terms flushed to zero are below 2^-126 each, i.e. far below
 // rounding.  Otherwise (no derivation at all, first columns, a guess that is far off) the rows are read again and
 // folded with a running maximum, which is exact for any input.  Link values are requested one chunk ahead: x0, x1 hold
 // the row's first chunk on entry and, on exit, the chunk at n0, n1 (the first chunk of the row this lane handles next).
 template <bool JOINT, int SL>
 __device__ __forceinline__ void stream_row_lse(const float4 *__restrict__ r0, const float4 *__restrict__ r1, const float4 *u0,
-                                               const float4 *u1, int q0, int q1, bool live, bool has1, float g0, float g1,
-                                               float4 &x0, float4 &x1, const float4 *__restrict__ n0,
+                                               const float4 *u1, int q0, int q1, bool live, bool has1, float g, float4 &x0, float4 &x1, const float4 *__restrict__ n0,
                                                const float4 *__restrict__ n1, float &out0, float &out1) {
-    g0 = is_finite(g0) ? g0 : 0.f;
-    g1 = JOINT ? g0 : (is_finite(g1) ? g1 : 0.f);
+    g = is_finite(g) ? g : 0.f;
     float s0 = 0.f, s1 = 0.f;
-    for (int q = q0; q < q1; q++) {
+#pragma unroll 2
+    for (int q = q0; q + 1 < q1; q++) {
         const float4 y0 = x0, y1 = x1;
-        const bool last = q + 1 == q1;
-        x0 = *(last ? n0 : r0 + SL * (q + 1));
-        x1 = *(last ? n1 : r1 + SL * (q + 1));
-        const float4 c0 = u0[SL * q];
-        const float4 c1 = JOINT ? u1[SL * q] : c0;
-        s0 += sum4_ex2(y0, c0, g0);
-        s1 += sum4_ex2(y1, c1, g1);
+        x0 = r0[SL * (q + 1)];
+        x1 = r1[SL * (q + 1)];
+        const float4 c0 = minus(u0[SL * q], g);
+        const float4 c1 = JOINT ? minus(u1[SL * q], g) : c0;
+        s0 += sum4_ex2(y0, c0);
+        s1 += sum4_ex2(y1, c1);
+    }
+    {   // last chunk of this node, first chunk of the next one requested
+        const float4 y0 = x0, y1 = x1;
+        x0 = *n0;
+        x1 = *n1;
+        const float4 c0 = minus(u0[SL * (q1 - 1)], g);
+        const float4 c1 = JOINT ? minus(u1[SL * (q1 - 1)], g) : c0;
+        s0 += sum4_ex2(y0, c0);
+        s1 += sum4_ex2(y1, c1);
     }
     bool ok;
     if (JOINT) {
         const float tot = node_sum<SL>(s0 + s1);
         ok = tot >= 0x1p-90f && tot <= 0x1p100f;
-        out0 = g0 + lg2(tot);
+        out0 = g + lg2(tot);
         out1 = out0;
     } else {
         const float t0 = node_sum<SL>(s0), t1 = node_sum<SL>(s1);
         ok = t0 >= 0x1p-90f && t0 <= 0x1p100f && ((t1 >= 0x1p-90f && t1 <= 0x1p100f) || !has1);
-        out0 = g0 + lg2(t0);
-        out1 = has1 ? g1 + lg2(t1) : NEG_INF_F;
+        out0 = g + lg2(t0);
+        out1 = has1 ? g + lg2(t1) : NEG_INF_F;
     }
     if (live && !ok) {  // uniform over the lanes of the node
         RunningLse<SL> a0, a1;
@@ -1212,7 +1221,7 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
             const int ai = min(a_id, MP - 1);  // the last tile may reach beyond the padded node count
             const float f1p = f1prev[ai];
             float F0, F1;
-            stream_row_lse<false, SL>(me.r0, me.r1, cv, cv, me.q0, nq, row_ok, a_id >= 1, f0prev[ai], f1p, x0, x1, nx.r0 + SL * nx.q0,
+            stream_row_lse<false, SL>(me.r0, me.r1, cv, cv, me.q0, nq, row_ok, a_id >= 1, f0prev[ai], x0, x1, nx.r0 + SL * nx.q0,
                                   nx.r1 + SL * nx.q0, F0, F1);
             F0 -= Ds;
             F1 -= Ds;
@@ -1372,7 +1381,7 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
             const float4 *u0 = reinterpret_cast<const float4 *>(c0) + j, *u1 = reinterpret_cast<const float4 *>(c1) + j;
             const float bp = bprev[min(c_id, MP - 1)];  // the last tile may reach beyond the padded node count
             float beta, unused;
-            stream_row_lse<true, SL>(me.r0, me.r1, u0, u1, 0, me.q1, live, true, bp, bp, x0, x1, nx.r0, nx.r1, beta, unused);
+            stream_row_lse<true, SL>(me.r0, me.r1, u0, u1, 0, me.q1, live, true, bp, x0, x1, nx.r0, nx.r1, beta, unused);
             if (!live) beta = NEG_INF_F;
             const float nw0 = (mc_t + beta) - d_next;
             const float nw1 = ((ml_p + mc_t) + bp) - d_both;
