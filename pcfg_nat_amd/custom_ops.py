@@ -604,6 +604,19 @@ def _length_penalty(Lq, beta, device):
     return pen
 
 
+_PINNED_COUNTS = {}
+
+
+def _pinned_counts(device, n):
+    """A pinned int64 host buffer of n entries per device, reused between calls (grown when a larger batch comes)."""
+    key = str(device)
+    buf = _PINNED_COUNTS.get(key)
+    if buf is None or buf.numel() < n:
+        buf = torch.empty((max(n, 64),), dtype=torch.int64, pin_memory=True)
+        _PINNED_COUNTS[key] = buf
+    return buf[:n]
+
+
 def pcfg_viterbi_decode(unreduced_logits, links, output_length, unreduced_tokens, left_tree_mask, pad_index, beta=1.0):
     """The model's whole Viterbi decode (glat_decomposed_with_link_two_hands_tri_pcfg.py:483-502) in one native call:
     ``cuda_pcfg_viterbi`` -> length penalty ``arange ** beta`` -> NaN masking -> arg max over lengths >= 1 ->
@@ -629,17 +642,25 @@ def pcfg_viterbi_decode(unreduced_logits, links, output_length, unreduced_tokens
     mask = left_tree_mask.to(dtype=torch.int64).contiguous()
     pen = _length_penalty(L // 4, beta, dev)
     with torch.cuda.device(dev):
-        nbytes = lib.pcfgnat_viterbi_decode_workspace_bytes(B, L, ml)
-        work = torch.empty(((nbytes + 7) // 8,), dtype=torch.int64, device=dev)
-        out = torch.empty((B, L), dtype=torch.int64, device=dev)
-        meta = torch.empty((2, B), dtype=torch.int64, device=dev)  # row 0: emitted counts, row 1: predicted lengths
+        nwork = (lib.pcfgnat_viterbi_decode_workspace_bytes(B, L, ml) + 7) // 8
+        # one allocation: workspace | tokens [B,L] | emitted counts [B] | predicted lengths [B]
+        block = torch.empty((nwork + B * L + 2 * B,), dtype=torch.int64, device=dev)
+        out = block[nwork:nwork + B * L].view(B, L)
+        meta = block[nwork + B * L:].view(2, B)
+        base = block.data_ptr()
         _lib.check(lib.pcfgnat_viterbi_decode(ob.data_ptr(), links.data_ptr(), ol.data_ptr(), tok.data_ptr(), mask.data_ptr(),
-                                              mask.size(0), int(pad_index), pen.data_ptr(), work.data_ptr(), out.data_ptr(),
-                                              meta[0].data_ptr(), meta[1].data_ptr(), B, L, ml, _stream(ob)), lib)
-    host = meta.cpu()  # one synchronising copy: counts for the trimming below, lengths for the caller
-    if B and int(host[0].min()) < 0:
+                                              mask.size(0), int(pad_index), pen.data_ptr(), base, base + 8 * nwork,
+                                              base + 8 * (nwork + B * L), base + 8 * (nwork + B * L + B), B, L, ml,
+                                              _stream(ob)), lib)
+        # the one synchronisation of the decode: counts for the trimming below (through a pinned buffer: one asynchronous
+        # copy and a stream wait instead of a staged blocking copy)
+        host = _pinned_counts(dev, B)
+        host.copy_(meta[0], non_blocking=True)
+        torch.cuda.current_stream(dev).synchronize()
+    counts = host.tolist()
+    if B and min(counts) < 0:
         raise RuntimeError("viterbi_decoding: malformed traces")
-    maxlen = int(host[0].max()) if B else 0
+    maxlen = max(counts) if B else 0
     return out[:, :maxlen].to(torch.float32), meta[1]
 
 
