@@ -137,6 +137,27 @@ int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *ma
                                        void *stream);
 
 /*
+ * The float64 instantiation the reference also dispatches (AT_DISPATCH_FLOATING_TYPES in pcfg_loss.cu:395,
+ * pcfg_loss_backward.cu:693, pcfg_best_tree.cu:349, pcfg_viterbi.cu:291; no shipped script uses it).  Same arguments,
+ * layouts and results as the float32 entry points above and below with double tables; every max_left, 1 included,
+ * runs the plain one-workgroup-per-sentence kernels, so these are for checking, not for speed.  grad_output is required
+ * (no NULL shorthand).  aux holds pcfgnat_pcfg_aux_elems_f64 doubles.
+ */
+size_t pcfgnat_pcfg_aux_elems_f64(int64_t B, int64_t L, int64_t T, int64_t ml);
+int pcfgnat_pcfg_loss_f64(const double *match_all, const double *links, const int64_t *output_length,
+                          const int64_t *target_length, double *S, double *aux, int64_t B, int64_t L, int64_t T, int64_t ml,
+                          void *stream);
+int pcfgnat_pcfg_loss_backward_f64(const double *grad_output, const double *S, double *aux, const double *match_all,
+                                   const double *links, const int64_t *output_length, const int64_t *target_length,
+                                   double *match_all_grad, double *links_grad, int64_t B, int64_t L, int64_t T, int64_t ml,
+                                   void *stream);
+int pcfgnat_pcfg_best_tree_f64(const double *S, double *aux, const double *match_all, const double *links,
+                               const int64_t *output_length, const int64_t *target_length, int64_t *tree, int64_t B, int64_t L,
+                               int64_t T, int64_t ml, void *stream);
+int pcfgnat_pcfg_viterbi_f64(const double *ob_lprob, const double *links, const int64_t *output_length, double *S, int64_t *R,
+                             int64_t *Lt, int64_t *M, int64_t B, int64_t L, int64_t ml, void *stream);
+
+/*
  * The criterion's reduction (nat_pcfg_loss.py:123-135) on the device: out[0] = -(1/B) sum_b ll_b/target_length[b] over
  * sentences with a finite ll_b = S[b,0,0]; out[1] = number of sentences with a non-finite ll_b.  Deterministic.
  */

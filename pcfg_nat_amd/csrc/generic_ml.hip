@@ -38,9 +38,26 @@ struct Dims {
     __host__ __device__ size_t aux_floats() const { return 3 * c_size() + 2 * s_size(); }
 };
 
-__device__ __forceinline__ bool bad(float v) { return v != v; }
+// The kernels are templates over the table type RT (float, or double: the reference dispatches both, pcfg_loss.cu:395).
+template <typename RT>
+__device__ __forceinline__ RT neg_inf();
+template <>
+__device__ __forceinline__ float neg_inf<float>() { return NEG_INF_F; }
+template <>
+__device__ __forceinline__ double neg_inf<double>() { return -__builtin_huge_val(); }
+__device__ __forceinline__ float rexp(float x) { return expf(x); }
+__device__ __forceinline__ double rexp(double x) { return exp(x); }
+__device__ __forceinline__ float rlog(float x) { return logf(x); }
+__device__ __forceinline__ double rlog(double x) { return log(x); }
+__device__ __forceinline__ float rmax(float a, float b) { return fmaxf(a, b); }
+__device__ __forceinline__ double rmax(double a, double b) { return fmax(a, b); }
+__device__ __forceinline__ bool is_inf(float x) { return fabsf(x) == __builtin_huge_valf(); }
+__device__ __forceinline__ bool is_inf(double x) { return fabs(x) == __builtin_huge_val(); }
+template <typename RT>
+__device__ __forceinline__ bool bad(RT v) { return v != v; }
 // Cells that other threads update with (L2) atomics must not be read through a possibly stale L1 line.
-__device__ __forceinline__ float coherent_load(const float *p) {
+template <typename RT>
+__device__ __forceinline__ RT coherent_load(const RT *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ bool len_ok(const Dims &d, int m, int n) {
@@ -48,23 +65,24 @@ __device__ __forceinline__ bool len_ok(const Dims &d, int m, int n) {
 }
 
 // ---- inside forward (pcfg_loss.cu:262-349 then :84-224) -----------------------------------------------------
-__global__ __launch_bounds__(NTG) void generic_fwd_kernel(const float *__restrict__ match_all, const float *__restrict__ links_all,
+template <typename RT>
+__global__ __launch_bounds__(NTG) void generic_fwd_kernel(const RT *__restrict__ match_all, const RT *__restrict__ links_all,
                                                          const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
-                                                         float *__restrict__ S_all, float *__restrict__ aux_all, int L, int T, int ml) {
+                                                         RT *__restrict__ S_all, RT *__restrict__ aux_all, int L, int T, int ml) {
     const Dims d(L, T, ml);
     const int b = blockIdx.x, tid = threadIdx.x;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
-    const float *match = match_all + (size_t)b * L * T;
-    const float *links = links_all + (size_t)b * L * (ml + 1) * L;
-    float *S = S_all + (size_t)b * d.s_size();
-    float *C = aux_all + (size_t)b * d.aux_floats();
-    for (size_t i = tid; i < d.s_size(); i += NTG) S[i] = NEG_INF_F;
+    const RT *match = match_all + (size_t)b * L * T;
+    const RT *links = links_all + (size_t)b * L * (ml + 1) * L;
+    RT *S = S_all + (size_t)b * d.s_size();
+    RT *C = aux_all + (size_t)b * d.aux_floats();
+    for (size_t i = tid; i < d.s_size(); i += NTG) S[i] = neg_inf<RT>();
     if (!len_ok(d, m, n)) {
         __syncthreads();
-        if (tid == 0) S[0] = __builtin_nanf("");
+        if (tid == 0) S[0] = (RT)__builtin_nanf("");
         return;
     }
-    for (size_t i = tid; i < d.c_size(); i += NTG) C[i] = NEG_INF_F;
+    for (size_t i = tid; i < d.c_size(); i += NTG) C[i] = neg_inf<RT>();
     __syncthreads();
     // :288-300
     for (int i = tid; i <= n; i += NTG) C[d.c_at(0, i, 0)] = 0.f;
@@ -82,22 +100,22 @@ __global__ __launch_bounds__(NTG) void generic_fwd_kernel(const float *__restric
             const int a = d.lt_i2e(a_id);
             if (!(a > 0 && a < m)) continue;
             const int hi = d.hi(a), b_start = a - ml < 1 ? 1 : a - ml;
-            float maxval = NEG_INF_F;
+            RT maxval = neg_inf<RT>();
             for (int pass = 0; pass < 2; pass++) {
-                float sum = 0.f;
+                RT sum = 0.f;
                 for (int j = 0; j < gap; j++)
                     for (int bb = b_start; bb < a + 1; bb++) {
                         const int b_id = d.lt_e2i(bb == a ? 0 : bb);
                         for (int c = a + 1; c < hi && c < m; c++) {
-                            float t = links[d.lk(a, a - bb, c)] + C[d.c_at(b_id, i, j)] + C[d.c_at(d.lt_e2i(c), i + j + 1, gap - j - 1)] +
+                            RT t = links[d.lk(a, a - bb, c)] + C[d.c_at(b_id, i, j)] + C[d.c_at(d.lt_e2i(c), i + j + 1, gap - j - 1)] +
                                       match[(size_t)a * T + i + j];
-                            if (bad(t)) t = NEG_INF_F;
-                            if (pass == 0) maxval = fmaxf(maxval, t);
-                            else sum += expf(t - maxval);
+                            if (bad(t)) t = neg_inf<RT>();
+                            if (pass == 0) maxval = rmax(maxval, t);
+                            else sum += rexp(t - maxval);
                         }
                     }
-                if (pass == 0 && maxval == NEG_INF_F) break;
-                if (pass == 1) C[d.c_at(a_id, i, gap)] = logf(sum) + maxval;
+                if (pass == 0 && maxval == neg_inf<RT>()) break;
+                if (pass == 1) C[d.c_at(a_id, i, gap)] = rlog(sum) + maxval;
             }
         }
         __syncthreads();
@@ -111,23 +129,23 @@ __global__ __launch_bounds__(NTG) void generic_fwd_kernel(const float *__restric
             const int a = d.mc_i2e(a_id);
             if (!(a > 0 && a < m)) continue;
             const int b_start = a - ml < 1 ? 1 : a - ml;
-            float maxval = NEG_INF_F;
+            RT maxval = neg_inf<RT>();
             for (int pass = 0; pass < 2; pass++) {
-                float sum = 0.f;
+                RT sum = 0.f;
                 for (int c_id = a_id; d.mc_i2e(c_id) < m; c_id++) {
                     const int c = d.mc_i2e(c_id);
                     for (int j = 0; j < n - start && j < ml + 1; j++)
                         for (int bb = b_start; bb < a + 1; bb++) {
                             const int b_id = d.lt_e2i(bb == a ? 0 : bb);
-                            float t = links[d.lk(a, a - bb, c)] + S[d.s_at(c_id, start + j + 1)] + C[d.c_at(b_id, start, j)] +
+                            RT t = links[d.lk(a, a - bb, c)] + S[d.s_at(c_id, start + j + 1)] + C[d.c_at(b_id, start, j)] +
                                       match[(size_t)a * T + start + j];
-                            if (bad(t)) t = NEG_INF_F;
-                            if (pass == 0) maxval = fmaxf(maxval, t);
-                            else sum += expf(t - maxval);
+                            if (bad(t)) t = neg_inf<RT>();
+                            if (pass == 0) maxval = rmax(maxval, t);
+                            else sum += rexp(t - maxval);
                         }
                 }
-                if (pass == 0 && maxval == NEG_INF_F) break;
-                if (pass == 1) S[d.s_at(a_id, start)] = logf(sum) + maxval;
+                if (pass == 0 && maxval == neg_inf<RT>()) break;
+                if (pass == 1) S[d.s_at(a_id, start)] = rlog(sum) + maxval;
             }
         }
         __syncthreads();
@@ -135,31 +153,32 @@ __global__ __launch_bounds__(NTG) void generic_fwd_kernel(const float *__restric
 }
 
 // ---- backward: exact gradient of the recurrences above (organised like pcfg_loss_backward.cu:28-603) ------------
-__global__ __launch_bounds__(NTG) void generic_bwd_kernel(const float *__restrict__ grad_out, const float *__restrict__ S_all,
-                                                         float *__restrict__ aux_all, const float *__restrict__ match_all,
-                                                         const float *__restrict__ links_all, const int64_t *__restrict__ out_len,
-                                                         const int64_t *__restrict__ tgt_len, float *__restrict__ mg_all,
-                                                         float *__restrict__ lg_all, int L, int T, int ml, int norm_B) {
+template <typename RT>
+__global__ __launch_bounds__(NTG) void generic_bwd_kernel(const RT *__restrict__ grad_out, const RT *__restrict__ S_all,
+                                                         RT *__restrict__ aux_all, const RT *__restrict__ match_all,
+                                                         const RT *__restrict__ links_all, const int64_t *__restrict__ out_len,
+                                                         const int64_t *__restrict__ tgt_len, RT *__restrict__ mg_all,
+                                                         RT *__restrict__ lg_all, int L, int T, int ml, int norm_B) {
     const Dims d(L, T, ml);
     const int b = blockIdx.x, tid = threadIdx.x;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
-    const float *match = match_all + (size_t)b * L * T;
-    const float *links = links_all + (size_t)b * L * (ml + 1) * L;
-    const float *S = S_all + (size_t)b * d.s_size();
-    float *aux = aux_all + (size_t)b * d.aux_floats();
-    const float *C = aux;
-    float *Cg = aux + d.c_size();
-    float *Sg = aux + 3 * d.c_size();
-    float *mg = mg_all + (size_t)b * L * T;
-    float *lg = lg_all + (size_t)b * L * (ml + 1) * L;
+    const RT *match = match_all + (size_t)b * L * T;
+    const RT *links = links_all + (size_t)b * L * (ml + 1) * L;
+    const RT *S = S_all + (size_t)b * d.s_size();
+    RT *aux = aux_all + (size_t)b * d.aux_floats();
+    const RT *C = aux;
+    RT *Cg = aux + d.c_size();
+    RT *Sg = aux + 3 * d.c_size();
+    RT *mg = mg_all + (size_t)b * L * T;
+    RT *lg = lg_all + (size_t)b * L * (ml + 1) * L;
     for (size_t i = tid; i < (size_t)L * T; i += NTG) mg[i] = 0.f;
     for (size_t i = tid; i < (size_t)L * (ml + 1) * L; i += NTG) lg[i] = 0.f;
-    const float ll = S[0];
-    if (!len_ok(d, m, n) || ll != ll || fabsf(ll) == __builtin_huge_valf()) return;  // invalid sentence: zero gradients
+    const RT ll = S[0];
+    if (!len_ok(d, m, n) || ll != ll || is_inf(ll)) return;  // invalid sentence: zero gradients
     for (size_t i = tid; i < d.s_size(); i += NTG) Sg[i] = 0.f;
     for (size_t i = tid; i < d.c_size(); i += NTG) Cg[i] = 0.f;
     __syncthreads();
-    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)norm_B);
+    const RT g = grad_out ? grad_out[b] : -1.0f / ((RT)n * (RT)norm_B);
     if (tid == 0) Sg[0] = g;  // :76-80
     __syncthreads();
     // main chain, start ascending (:83-112, 175-205, 348-376, 512-531)
@@ -167,19 +186,19 @@ __global__ __launch_bounds__(NTG) void generic_bwd_kernel(const float *__restric
         for (int a_id = tid; a_id < d.Mc; a_id += NTG) {
             const int a = d.mc_i2e(a_id);
             if (!(a > 0 && a < m)) continue;
-            const float sg = coherent_load(&Sg[d.s_at(a_id, s)]), sa = S[d.s_at(a_id, s)];
-            if (sg == 0.f || sa != sa || fabsf(sa) == __builtin_huge_valf()) continue;
+            const RT sg = coherent_load(&Sg[d.s_at(a_id, s)]), sa = S[d.s_at(a_id, s)];
+            if (sg == 0.f || sa != sa || is_inf(sa)) continue;
             const int b_start = a - ml < 1 ? 1 : a - ml;
             for (int c_id = a_id; d.mc_i2e(c_id) < m; c_id++) {
                 const int c = d.mc_i2e(c_id);
                 for (int j = 0; j < n - s && j < ml + 1; j++) {
-                    const float sc = S[d.s_at(c_id, s + j + 1)];
-                    if (sc != sc || fabsf(sc) == __builtin_huge_valf()) continue;
+                    const RT sc = S[d.s_at(c_id, s + j + 1)];
+                    if (sc != sc || is_inf(sc)) continue;
                     for (int bb = b_start; bb < a + 1; bb++) {
                         const int b_id = d.lt_e2i(bb == a ? 0 : bb);
-                        const float t = links[d.lk(a, a - bb, c)] + sc + C[d.c_at(b_id, s, j)] + match[(size_t)a * T + s + j] - sa;
-                        if (bad(t) || t == NEG_INF_F) continue;
-                        const float p = sg * expf(t);
+                        const RT t = links[d.lk(a, a - bb, c)] + sc + C[d.c_at(b_id, s, j)] + match[(size_t)a * T + s + j] - sa;
+                        if (bad(t) || t == neg_inf<RT>()) continue;
+                        const RT p = sg * rexp(t);
                         atomicAdd(&Sg[d.s_at(c_id, s + j + 1)], p);
                         if (b_id != 0) atomicAdd(&Cg[d.c_at(b_id, s, j)], p);
                         atomicAdd(&mg[(size_t)a * T + s + j], p);
@@ -199,18 +218,18 @@ __global__ __launch_bounds__(NTG) void generic_bwd_kernel(const float *__restric
             const int a_id = w / ni, i = w - a_id * ni;
             const int a = d.lt_i2e(a_id);
             if (!(a > 0 && a < m)) continue;
-            const float cg = coherent_load(&Cg[d.c_at(a_id, i, gap)]), ca = C[d.c_at(a_id, i, gap)];
-            if (cg == 0.f || ca != ca || fabsf(ca) == __builtin_huge_valf()) continue;
+            const RT cg = coherent_load(&Cg[d.c_at(a_id, i, gap)]), ca = C[d.c_at(a_id, i, gap)];
+            if (cg == 0.f || ca != ca || is_inf(ca)) continue;
             const int hi = d.hi(a), b_start = a - ml < 1 ? 1 : a - ml;
             for (int j = 0; j < gap; j++)
                 for (int bb = b_start; bb < a + 1; bb++) {
                     const int b_id = d.lt_e2i(bb == a ? 0 : bb);
                     for (int c = a + 1; c < hi && c < m; c++) {
                         const int c_id = d.lt_e2i(c);
-                        const float t = links[d.lk(a, a - bb, c)] + C[d.c_at(b_id, i, j)] + C[d.c_at(c_id, i + j + 1, gap - j - 1)] +
+                        const RT t = links[d.lk(a, a - bb, c)] + C[d.c_at(b_id, i, j)] + C[d.c_at(c_id, i + j + 1, gap - j - 1)] +
                                         match[(size_t)a * T + i + j] - ca;
-                        if (bad(t) || t == NEG_INF_F) continue;
-                        const float p = cg * expf(t);
+                        if (bad(t) || t == neg_inf<RT>()) continue;
+                        const RT p = cg * rexp(t);
                         if (b_id != 0) atomicAdd(&Cg[d.c_at(b_id, i, j)], p);
                         atomicAdd(&Cg[d.c_at(c_id, i + j + 1, gap - j - 1)], p);
                         atomicAdd(&mg[(size_t)a * T + i + j], p);
@@ -229,20 +248,21 @@ __global__ __launch_bounds__(NTG) void generic_bwd_kernel(const float *__restric
 }
 
 // ---- best tree (pcfg_best_tree.cu:64-197, 239-301); the 4-lane scan order is emulated per node -----------------
-__global__ __launch_bounds__(NTG) void generic_best_tree_kernel(const float *__restrict__ S_all, float *__restrict__ aux_all,
-                                                               const float *__restrict__ match_all, const float *__restrict__ links_all,
+template <typename RT>
+__global__ __launch_bounds__(NTG) void generic_best_tree_kernel(const RT *__restrict__ S_all, RT *__restrict__ aux_all,
+                                                               const RT *__restrict__ match_all, const RT *__restrict__ links_all,
                                                                const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
                                                                int64_t *__restrict__ tree_all, int L, int T, int ml) {
     const Dims d(L, T, ml);
     const int b = blockIdx.x, tid = threadIdx.x;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
-    const float *match = match_all + (size_t)b * L * T;
-    const float *links = links_all + (size_t)b * L * (ml + 1) * L;
-    const float *S = S_all + (size_t)b * d.s_size();
-    float *aux = aux_all + (size_t)b * d.aux_floats();
-    const float *C = aux;
-    float *St = aux + 3 * d.c_size() + d.s_size();  // marks (0 / 1)
-    float *Ct = aux + 2 * d.c_size();
+    const RT *match = match_all + (size_t)b * L * T;
+    const RT *links = links_all + (size_t)b * L * (ml + 1) * L;
+    const RT *S = S_all + (size_t)b * d.s_size();
+    RT *aux = aux_all + (size_t)b * d.aux_floats();
+    const RT *C = aux;
+    RT *St = aux + 3 * d.c_size() + d.s_size();  // marks (0 / 1)
+    RT *Ct = aux + 2 * d.c_size();
     int64_t *tree = tree_all + (size_t)b * L;
     for (int i = tid; i < L; i += NTG) tree[i] = -1;
     if (!len_ok(d, m, n)) return;
@@ -256,19 +276,19 @@ __global__ __launch_bounds__(NTG) void generic_best_tree_kernel(const float *__r
             const int a = d.mc_i2e(a_id);
             if (!(a > 0 && a < m && St[d.s_at(a_id, s)] != 0.f)) continue;
             const int b_start = a - ml < 1 ? 1 : a - ml;
-            float lane_val[4];
+            RT lane_val[4];
             int lane_c[4], lane_j[4], lane_b[4];
             for (int x = 0; x < 4; x++) {
-                float maxval = NEG_INF_F;
+                RT maxval = neg_inf<RT>();
                 int max_c = -1, max_j = 0, max_b = -1;
                 for (int c_id = a_id + x + 1; d.mc_i2e(c_id) < m; c_id += 4) {
                     const int c = d.mc_i2e(c_id);
                     for (int j = 0; j < n - s && j < ml + 1; j++)
                         for (int bb = b_start; bb < a + 1; bb++) {
                             const int b_id = d.lt_e2i(bb == a ? 0 : bb);
-                            float t = links[d.lk(a, a - bb, c)] + S[d.s_at(c_id, s + j + 1)] + C[d.c_at(b_id, s, j)] +
+                            RT t = links[d.lk(a, a - bb, c)] + S[d.s_at(c_id, s + j + 1)] + C[d.c_at(b_id, s, j)] +
                                       match[(size_t)a * T + s + j];
-                            if (bad(t)) t = NEG_INF_F;
+                            if (bad(t)) t = neg_inf<RT>();
                             if (t > maxval) { maxval = t; max_c = c_id; max_j = j; max_b = b_id; }
                         }
                 }
@@ -294,15 +314,15 @@ __global__ __launch_bounds__(NTG) void generic_best_tree_kernel(const float *__r
             if (!(a > 0 && a < m) || Ct[d.c_at(a_id, i, gap)] == 0.f) continue;
             const int hi = d.hi(a), b_start = a - ml < 1 ? 1 : a - ml;
             int max_j = 0, max_b = -1, max_c = -1;
-            float maxval = NEG_INF_F;
+            RT maxval = neg_inf<RT>();
             for (int j = 0; j < gap; j++)
                 for (int bb = b_start; bb < a + 1; bb++) {
                     const int b_id = d.lt_e2i(bb == a ? 0 : bb);
                     for (int c = a + 1; c < hi && c < m; c++) {
                         const int c_id = d.lt_e2i(c);
-                        float t = links[d.lk(a, a - bb, c)] + C[d.c_at(b_id, i, j)] + C[d.c_at(c_id, i + j + 1, gap - j - 1)] +
+                        RT t = links[d.lk(a, a - bb, c)] + C[d.c_at(b_id, i, j)] + C[d.c_at(c_id, i + j + 1, gap - j - 1)] +
                                   match[(size_t)a * T + i + j];
-                        if (bad(t)) t = NEG_INF_F;
+                        if (bad(t)) t = neg_inf<RT>();
                         if (t > maxval) { maxval = t; max_j = j; max_b = b_id; max_c = c_id; }
                     }
                 }
@@ -317,23 +337,24 @@ __global__ __launch_bounds__(NTG) void generic_best_tree_kernel(const float *__r
 }
 
 // ---- viterbi (pcfg_viterbi.cu:177-241 then :22-140); tables [L][Lq] by external node id --------------------------
-__global__ __launch_bounds__(NTG) void generic_viterbi_kernel(const float *__restrict__ ob_all, const float *__restrict__ links_all,
-                                                             const int64_t *__restrict__ out_len, float *__restrict__ S_all,
+template <typename RT>
+__global__ __launch_bounds__(NTG) void generic_viterbi_kernel(const RT *__restrict__ ob_all, const RT *__restrict__ links_all,
+                                                             const int64_t *__restrict__ out_len, RT *__restrict__ S_all,
                                                              int64_t *__restrict__ R_all,
                                                              int64_t *__restrict__ Lt_all, int64_t *__restrict__ M_all, int L, int ml) {
     const int Lq = L / 4;
     const int b = blockIdx.x, tid = threadIdx.x;
     const int m = (int)out_len[b];
-    const float *ob = ob_all + (size_t)b * L;
-    const float *links = links_all + (size_t)b * L * (ml + 1) * L;
+    const RT *ob = ob_all + (size_t)b * L;
+    const RT *links = links_all + (size_t)b * L * (ml + 1) * L;
     const size_t tab = (size_t)b * L * Lq;
     // the local-tree table lives in the rows of S that belong to local nodes and node 0 (the S sweep only touches
     // main-chain rows); those cells are put back to -inf at the end, as the reference returns them
-    float *S = S_all + tab, *Cv = S;
+    RT *S = S_all + tab, *Cv = S;
     int64_t *R = R_all + tab, *Lt = Lt_all + tab, *M = M_all + tab;
     auto at = [&](int a, int l) -> size_t { return (size_t)a * Lq + l; };
     auto lk = [&](int a, int k, int c) -> size_t { return ((size_t)a * (ml + 1) + k) * L + c; };
-    for (size_t i = tid; i < (size_t)L * Lq; i += NTG) { S[i] = NEG_INF_F; R[i] = 0; Lt[i] = 0; M[i] = 0; }
+    for (size_t i = tid; i < (size_t)L * Lq; i += NTG) { S[i] = neg_inf<RT>(); R[i] = 0; Lt[i] = 0; M[i] = 0; }
     if (m < 2 || m > L || ((m - 2) % (ml + 1)) != 0) return;
     __syncthreads();
     for (int a = 1 + tid; a < L; a += NTG) {
@@ -346,18 +367,18 @@ __global__ __launch_bounds__(NTG) void generic_viterbi_kernel(const float *__res
         for (int a = 1 + tid; a < L; a += NTG) {
             if (!(a < m && (a % (ml + 1) != 1))) continue;
             const int hi = ((a - 1) / (ml + 1) + 1) * (ml + 1) + 1, b_start = a - ml < 1 ? 1 : a - ml;
-            float maxval = NEG_INF_F;
+            RT maxval = neg_inf<RT>();
             int max_b = 0, max_c = 0, max_j = 0;
             for (int j = 0; j < gap; j++)
                 for (int bb = b_start; bb < a + 1; bb++) {
                     const int _b = bb == a ? 0 : bb;
                     for (int c = a + 1; c < hi && c < m; c++) {
-                        float t = ((links[lk(a, a - bb, c)] + Cv[at(_b, j)]) + Cv[at(c, gap - j - 1)]) + ob[a];
-                        if (bad(t)) t = NEG_INF_F;
+                        RT t = ((links[lk(a, a - bb, c)] + Cv[at(_b, j)]) + Cv[at(c, gap - j - 1)]) + ob[a];
+                        if (bad(t)) t = neg_inf<RT>();
                         if (t > maxval) { maxval = t; max_b = _b; max_c = c; max_j = j; }
                     }
                 }
-            if (maxval != NEG_INF_F) { Cv[at(a, gap)] = maxval; R[at(a, gap)] = max_c; Lt[at(a, gap)] = max_b; M[at(a, gap)] = max_j; }
+            if (maxval != neg_inf<RT>()) { Cv[at(a, gap)] = maxval; R[at(a, gap)] = max_c; Lt[at(a, gap)] = max_b; M[at(a, gap)] = max_j; }
         }
         __syncthreads();
     }
@@ -366,20 +387,20 @@ __global__ __launch_bounds__(NTG) void generic_viterbi_kernel(const float *__res
     for (int len = 2; len < m / 4; len++) {
         for (int id = tid; id * (ml + 1) + 1 < m; id += NTG) {
             const int a = id * (ml + 1) + 1, b_start = a - ml < 1 ? 1 : a - ml;
-            float lane_val[4];
+            RT lane_val[4];
             int lane_c[4], lane_j[4], lane_b[4];
             for (int x = 0; x < 4; x++) {
-                float maxval = NEG_INF_F;
+                RT maxval = neg_inf<RT>();
                 int max_b = 0, max_c = 0, max_j = 0;
                 for (int c_id = id + x; c_id * (ml + 1) + 1 < m; c_id += 4) {
                     const int c = c_id * (ml + 1) + 1;
                     for (int j = 0; j < ml + 1; j++)
                         for (int bb = b_start; bb < a + 1; bb++) {
                             const int _b = bb == a ? 0 : bb;
-                            const float sc = (len - j - 1 >= 0) ? S[at(c, len - j - 1)] : NEG_INF_F;
-                            const float cj = (j < Lq) ? Cv[at(_b, j)] : NEG_INF_F;
-                            float t = ((links[lk(a, a - bb, c)] + cj) + sc) + ob[a];
-                            if (bad(t)) t = NEG_INF_F;
+                            const RT sc = (len - j - 1 >= 0) ? S[at(c, len - j - 1)] : neg_inf<RT>();
+                            const RT cj = (j < Lq) ? Cv[at(_b, j)] : neg_inf<RT>();
+                            RT t = ((links[lk(a, a - bb, c)] + cj) + sc) + ob[a];
+                            if (bad(t)) t = neg_inf<RT>();
                             if (t > maxval) { maxval = t; max_b = _b; max_c = c; max_j = j; }
                         }
                 }
@@ -388,7 +409,7 @@ __global__ __launch_bounds__(NTG) void generic_viterbi_kernel(const float *__res
             for (int x = 0; x < 2; x++)
                 if (lane_val[x + 2] > lane_val[x]) { lane_val[x] = lane_val[x + 2]; lane_c[x] = lane_c[x + 2]; lane_j[x] = lane_j[x + 2]; lane_b[x] = lane_b[x + 2]; }
             if (lane_val[1] > lane_val[0]) { lane_val[0] = lane_val[1]; lane_c[0] = lane_c[1]; lane_j[0] = lane_j[1]; lane_b[0] = lane_b[1]; }
-            if (lane_val[0] != NEG_INF_F) {
+            if (lane_val[0] != neg_inf<RT>()) {
                 S[at(a, len)] = lane_val[0]; Lt[at(a, len)] = lane_b[0]; R[at(a, len)] = lane_c[0]; M[at(a, len)] = lane_j[0];
             }
         }
@@ -397,7 +418,7 @@ __global__ __launch_bounds__(NTG) void generic_viterbi_kernel(const float *__res
     for (int w = tid; w < L * Lq; w += NTG) {
         const int a = w / Lq;
         if (a == 0 || (a % (ml + 1)) != 1 || ml == 0) {
-            if (a == 0 || ml > 0) S[w] = NEG_INF_F;
+            if (a == 0 || ml > 0) S[w] = neg_inf<RT>();
         }
     }
 }
@@ -406,36 +427,119 @@ __global__ __launch_bounds__(NTG) void generic_viterbi_kernel(const float *__res
 
 size_t generic_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml) { return (size_t)B * Dims((int)L, (int)T, (int)ml).aux_floats(); }
 
-int generic_forward(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int64_t B,
-                    int64_t L, int64_t T, int64_t ml, void *stream) {
-    hipLaunchKernelGGL(generic_fwd_kernel, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, match_all, links, ol, tl, S, aux, (int)L,
+namespace {
+template <typename RT>
+int forward_t(const RT *match_all, const RT *links, const int64_t *ol, const int64_t *tl, RT *S, RT *aux, int64_t B, int64_t L, int64_t T,
+              int64_t ml, void *stream) {
+    hipLaunchKernelGGL(generic_fwd_kernel<RT>, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, match_all, links, ol, tl, S, aux, (int)L,
                        (int)T, (int)ml);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
-
-int generic_backward(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
-                     const int64_t *tl, float *mg, float *lg, int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream) {
-    hipLaunchKernelGGL(generic_bwd_kernel, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, go, S, aux, match_all, links, ol, tl, mg, lg,
-                       (int)L, (int)T, (int)ml, (int)norm_B);
+template <typename RT>
+int backward_t(const RT *go, const RT *S, RT *aux, const RT *match_all, const RT *links, const int64_t *ol, const int64_t *tl, RT *mg, RT *lg,
+               int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream) {
+    hipLaunchKernelGGL(generic_bwd_kernel<RT>, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, go, S, aux, match_all, links, ol, tl, mg,
+                       lg, (int)L, (int)T, (int)ml, (int)norm_B);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
-
-int generic_best_tree(const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl,
-                      int64_t *tree, int64_t B, int64_t L, int64_t T, int64_t ml, void *stream) {
-    hipLaunchKernelGGL(generic_best_tree_kernel, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, S, aux, match_all, links, ol, tl, tree,
-                       (int)L, (int)T, (int)ml);
+template <typename RT>
+int best_tree_t(const RT *S, RT *aux, const RT *match_all, const RT *links, const int64_t *ol, const int64_t *tl, int64_t *tree, int64_t B,
+                int64_t L, int64_t T, int64_t ml, void *stream) {
+    hipLaunchKernelGGL(generic_best_tree_kernel<RT>, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, S, aux, match_all, links, ol, tl,
+                       tree, (int)L, (int)T, (int)ml);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
-
-int generic_viterbi(const float *ob, const float *links, const int64_t *ol, float *S, int64_t *R, int64_t *Lt, int64_t *M, int64_t B,
-                    int64_t L, int64_t ml, void *stream) {
-    hipLaunchKernelGGL(generic_viterbi_kernel, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, ob, links, ol, S, R, Lt, M, (int)L,
+template <typename RT>
+int viterbi_t(const RT *ob, const RT *links, const int64_t *ol, RT *S, int64_t *R, int64_t *Lt, int64_t *M, int64_t B, int64_t L, int64_t ml,
+              void *stream) {
+    hipLaunchKernelGGL(generic_viterbi_kernel<RT>, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, ob, links, ol, S, R, Lt, M, (int)L,
                        (int)ml);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
 
+int check_f64(const char *who, int64_t B, int64_t L, int64_t T, int64_t ml) {
+    PCFGNAT_REQUIRE(B >= 0 && L >= 4 && T >= 2, "%s: need B >= 0, L >= 4, T >= 2 (got B=%lld L=%lld T=%lld)", who, (long long)B,
+                    (long long)L, (long long)T);
+    PCFGNAT_REQUIRE(L <= 4096 && T <= 4096 && B <= 65535, "%s: dimension too large (L, T <= 4096, B <= 65535)", who);
+    PCFGNAT_REQUIRE(ml >= 0 && ml <= 63 && L >= ml + 3, "%s: max_left = %lld needs a graph of at least max_left + 3 nodes (and max_left <= 63)",
+                    who, (long long)ml);
+    return PCFGNAT_OK;
+}
+}  // namespace
+
+int generic_forward(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int64_t B,
+                    int64_t L, int64_t T, int64_t ml, void *stream) {
+    return forward_t<float>(match_all, links, ol, tl, S, aux, B, L, T, ml, stream);
+}
+
+int generic_backward(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
+                     const int64_t *tl, float *mg, float *lg, int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream) {
+    return backward_t<float>(go, S, aux, match_all, links, ol, tl, mg, lg, B, L, T, ml, norm_B, stream);
+}
+
+int generic_best_tree(const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl,
+                      int64_t *tree, int64_t B, int64_t L, int64_t T, int64_t ml, void *stream) {
+    return best_tree_t<float>(S, aux, match_all, links, ol, tl, tree, B, L, T, ml, stream);
+}
+
+int generic_viterbi(const float *ob, const float *links, const int64_t *ol, float *S, int64_t *R, int64_t *Lt, int64_t *M, int64_t B,
+                    int64_t L, int64_t ml, void *stream) {
+    return viterbi_t<float>(ob, links, ol, S, R, Lt, M, B, L, ml, stream);
+}
+
 }  // namespace pcfgnat
+
+using namespace pcfgnat;
+
+// ---- float64 entry points: every max_left (1 included) runs the plain kernels above ---------------------------------
+extern "C" size_t pcfgnat_pcfg_aux_elems_f64(int64_t B, int64_t L, int64_t T, int64_t ml) {
+    if (B <= 0 || L < 4 || T < 2 || ml < 0 || L < ml + 3) return 0;
+    return generic_aux_floats(B, L, T, ml);
+}
+
+extern "C" int pcfgnat_pcfg_loss_f64(const double *match_all, const double *links, const int64_t *output_length,
+                                     const int64_t *target_length, double *S, double *aux, int64_t B, int64_t L, int64_t T, int64_t ml,
+                                     void *stream) {
+    int rc = check_f64("pcfg_loss_f64", B, L, T, ml);
+    if (rc != PCFGNAT_OK) return rc;
+    if (B == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(match_all && links && output_length && target_length && S && aux, "pcfg_loss_f64: null pointer");
+    return forward_t<double>(match_all, links, output_length, target_length, S, aux, B, L, T, ml, stream);
+}
+
+extern "C" int pcfgnat_pcfg_loss_backward_f64(const double *grad_output, const double *S, double *aux, const double *match_all,
+                                              const double *links, const int64_t *output_length, const int64_t *target_length,
+                                              double *match_all_grad, double *links_grad, int64_t B, int64_t L, int64_t T, int64_t ml,
+                                              void *stream) {
+    int rc = check_f64("pcfg_loss_backward_f64", B, L, T, ml);
+    if (rc != PCFGNAT_OK) return rc;
+    if (B == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(grad_output && S && aux && match_all && links && output_length && target_length && match_all_grad && links_grad,
+                    "pcfg_loss_backward_f64: null pointer");
+    return backward_t<double>(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, B, L, T, ml,
+                              B, stream);
+}
+
+extern "C" int pcfgnat_pcfg_best_tree_f64(const double *S, double *aux, const double *match_all, const double *links,
+                                          const int64_t *output_length, const int64_t *target_length, int64_t *tree, int64_t B, int64_t L,
+                                          int64_t T, int64_t ml, void *stream) {
+    int rc = check_f64("pcfg_best_tree_f64", B, L, T, ml);
+    if (rc != PCFGNAT_OK) return rc;
+    if (B == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(S && aux && match_all && links && output_length && target_length && tree, "pcfg_best_tree_f64: null pointer");
+    return best_tree_t<double>(S, aux, match_all, links, output_length, target_length, tree, B, L, T, ml, stream);
+}
+
+extern "C" int pcfgnat_pcfg_viterbi_f64(const double *ob_lprob, const double *links, const int64_t *output_length, double *S, int64_t *R,
+                                        int64_t *Lt, int64_t *M, int64_t B, int64_t L, int64_t ml, void *stream) {
+    PCFGNAT_REQUIRE(B >= 0 && L >= 4 && L <= 4096, "pcfg_viterbi_f64: need B >= 0 and 4 <= L <= 4096 (got B=%lld L=%lld)", (long long)B,
+                    (long long)L);
+    PCFGNAT_REQUIRE(ml >= 0 && ml <= 63 && L / 4 > ml, "pcfg_viterbi_f64: max_left out of range for this graph size");
+    if (B == 0) return PCFGNAT_OK;
+    PCFGNAT_REQUIRE(ob_lprob && links && output_length && S && R && Lt && M, "pcfg_viterbi_f64: null pointer");
+    return viterbi_t<double>(ob_lprob, links, output_length, S, R, Lt, M, B, L, ml, stream);
+}

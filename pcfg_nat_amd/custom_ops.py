@@ -55,9 +55,15 @@ def _check_pcfg_inputs(name, match_all, links, output_length, target_length):
     if links.size(0) != B or links.size(1) != L or links.size(3) != L:
         raise RuntimeError("%s: links must be [bsz, prelen, max_left+1, prelen] = [%d, %d, *, %d], got %s"
                            % (name, B, L, L, tuple(links.shape)))
-    if match_all.dtype != torch.float32 or links.dtype != torch.float32:
-        raise RuntimeError("%s: match_all and links must be float32 (got %s, %s)" % (name, match_all.dtype, links.dtype))
+    if match_all.dtype != links.dtype or match_all.dtype not in (torch.float32, torch.float64):
+        raise RuntimeError("%s: match_all and links must both be float32 or both float64 (got %s, %s)"
+                           % (name, match_all.dtype, links.dtype))
     return B, L, T, links.size(2) - 1
+
+
+def _is_f64(t):
+    """float64 tables (which the reference also dispatches, pcfg_loss.cu:395) go to the plain float64 entry points."""
+    return t.dtype == torch.float64
 
 
 def _pcfg_loss_tables(match_all, links, output_length, target_length, config, name):
@@ -70,11 +76,15 @@ def _pcfg_loss_tables(match_all, links, output_length, target_length, config, na
     target_length = _lengths(name, target_length, B)
     Mc = (L - 2) // (ml + 1) + 1
     with torch.cuda.device(match_all.device):
-        S = torch.empty((B, Mc, T + 2), dtype=torch.float32, device=match_all.device)
-        aux = torch.empty((max(1, lib.pcfgnat_pcfg_aux_floats(B, L, T, ml)),), dtype=torch.float32, device=match_all.device)
-        _lib.check(lib.pcfgnat_pcfg_loss(match_all.data_ptr(), links.data_ptr(), output_length.data_ptr(),
-                                         target_length.data_ptr(), S.data_ptr(), aux.data_ptr(), B, L, T, ml,
-                                         _stream(match_all)), lib)
+        S = torch.empty((B, Mc, T + 2), dtype=match_all.dtype, device=match_all.device)
+        if _is_f64(match_all):
+            aux = torch.empty((max(1, lib.pcfgnat_pcfg_aux_elems_f64(B, L, T, ml)),), dtype=torch.float64, device=match_all.device)
+            fn = lib.pcfgnat_pcfg_loss_f64
+        else:
+            aux = torch.empty((max(1, lib.pcfgnat_pcfg_aux_floats(B, L, T, ml)),), dtype=torch.float32, device=match_all.device)
+            fn = lib.pcfgnat_pcfg_loss
+        _lib.check(fn(match_all.data_ptr(), links.data_ptr(), output_length.data_ptr(), target_length.data_ptr(), S.data_ptr(),
+                      aux.data_ptr(), B, L, T, ml, _stream(match_all)), lib)
     return S, aux, output_length, target_length
 
 
@@ -89,10 +99,16 @@ def _pcfg_loss_backward(grad_output, S, aux, match_all, links, output_length, ta
     with torch.cuda.device(match_all.device):
         match_all_grad = torch.empty_like(match_all)
         links_grad = torch.empty_like(links)
-        _lib.check(lib.pcfgnat_pcfg_loss_backward(grad_output.data_ptr() if grad_output is not None else None, S.data_ptr(), aux.data_ptr(),
-                                                  match_all.data_ptr(), links.data_ptr(), output_length.data_ptr(),
-                                                  target_length.data_ptr(), match_all_grad.data_ptr(),
-                                                  links_grad.data_ptr(), B, L, T, ml, _stream(match_all)), lib)
+        if _is_f64(match_all):
+            if grad_output is None:
+                raise RuntimeError("pcfg_loss_backward: the float64 path needs an explicit grad_output")
+            fn = lib.pcfgnat_pcfg_loss_backward_f64
+            grad_output = grad_output.to(torch.float64).contiguous()
+        else:
+            fn = lib.pcfgnat_pcfg_loss_backward
+        _lib.check(fn(grad_output.data_ptr() if grad_output is not None else None, S.data_ptr(), aux.data_ptr(),
+                      match_all.data_ptr(), links.data_ptr(), output_length.data_ptr(), target_length.data_ptr(),
+                      match_all_grad.data_ptr(), links_grad.data_ptr(), B, L, T, ml, _stream(match_all)), lib)
     return match_all_grad, links_grad
 
 
@@ -105,6 +121,10 @@ def _pcfg_loss_forward_backward(grad_output, match_all, links, output_length, ta
     B, L, T, ml = _check_pcfg_inputs(name, match_all, links, output_length, target_length)
     output_length = _lengths(name, output_length, B)
     target_length = _lengths(name, target_length, B)
+    if _is_f64(match_all):  # two plain calls
+        S, aux, output_length, target_length = _pcfg_loss_tables(match_all, links, output_length, target_length, config, name)
+        mg, lg = _pcfg_loss_backward(grad_output, S, aux, match_all, links, output_length, target_length, config)
+        return S, mg, lg
     Mc = (L - 2) // (ml + 1) + 1
     with torch.cuda.device(match_all.device):
         S = torch.empty((B, Mc, T + 2), dtype=torch.float32, device=match_all.device)
@@ -139,7 +159,7 @@ class CUDAPCFGLossFunc(Function):
         links = links.contiguous()
         if require_gradient:
             # like the reference (pcfg_loss.py:71-73) the backward sweep runs eagerly with a unit upstream gradient
-            ones = torch.ones((batch_size,), dtype=torch.float32, device=match_all.device)
+            ones = torch.ones((batch_size,), dtype=match_all.dtype, device=match_all.device)
             S, match_all_grad, links_grad = _pcfg_loss_forward_backward(ones, match_all, links, output_length, target_length,
                                                                         CUDAPCFGLossFunc.config, "cuda_pcfg_loss")
             ctx.save_for_backward(match_all_grad, links_grad)
@@ -182,9 +202,9 @@ class CUDAPCFGBestTreeFunc(Function):
         ml = links.size(2) - 1
         with torch.cuda.device(match_all.device):
             tree = torch.empty((B, L), dtype=torch.int64, device=match_all.device)
-            _lib.check(lib.pcfgnat_pcfg_best_tree(S.data_ptr(), aux.data_ptr(), match_all.data_ptr(), links.data_ptr(),
-                                                  ol.data_ptr(), tl.data_ptr(), tree.data_ptr(), B, L, T, ml,
-                                                  _stream(match_all)), lib)
+            fn = lib.pcfgnat_pcfg_best_tree_f64 if _is_f64(match_all) else lib.pcfgnat_pcfg_best_tree
+            _lib.check(fn(S.data_ptr(), aux.data_ptr(), match_all.data_ptr(), links.data_ptr(), ol.data_ptr(), tl.data_ptr(),
+                          tree.data_ptr(), B, L, T, ml, _stream(match_all)), lib)
         ctx.mark_non_differentiable(tree)
         return tree, S[:, 0, 0].clone()
 
@@ -214,8 +234,8 @@ class CUDAPCFGViterbiFunc(Function):
         _need_cuda("cuda_pcfg_viterbi", ob_lprob, links, output_length)
         if ob_lprob.dim() != 2 or links.dim() != 4:
             raise RuntimeError("cuda_pcfg_viterbi: ob_lprob must be [bsz, prelen] and links [bsz, prelen, max_left+1, prelen]")
-        if ob_lprob.dtype != torch.float32 or links.dtype != torch.float32:
-            raise RuntimeError("cuda_pcfg_viterbi: ob_lprob and links must be float32 (got %s, %s)"
+        if ob_lprob.dtype != links.dtype or ob_lprob.dtype not in (torch.float32, torch.float64):
+            raise RuntimeError("cuda_pcfg_viterbi: ob_lprob and links must both be float32 or both float64 (got %s, %s)"
                                % (ob_lprob.dtype, links.dtype))
         B, L = ob_lprob.shape
         if links.size(0) != B or links.size(1) != L or links.size(3) != L:
@@ -227,13 +247,13 @@ class CUDAPCFGViterbiFunc(Function):
         output_length = _lengths("cuda_pcfg_viterbi", output_length, B)
         Lq = L // 4
         with torch.cuda.device(ob_lprob.device):
-            S = torch.empty((B, L, Lq), dtype=torch.float32, device=ob_lprob.device)
+            S = torch.empty((B, L, Lq), dtype=ob_lprob.dtype, device=ob_lprob.device)
             R = torch.empty((B, L, Lq), dtype=torch.int64, device=ob_lprob.device)
             Lt = torch.empty_like(R)
             M = torch.empty_like(R)
-            _lib.check(lib.pcfgnat_pcfg_viterbi(ob_lprob.data_ptr(), links.data_ptr(), output_length.data_ptr(),
-                                                S.data_ptr(), R.data_ptr(), Lt.data_ptr(), M.data_ptr(), B, L, ml,
-                                                _stream(ob_lprob)), lib)
+            fn = lib.pcfgnat_pcfg_viterbi_f64 if _is_f64(ob_lprob) else lib.pcfgnat_pcfg_viterbi
+            _lib.check(fn(ob_lprob.data_ptr(), links.data_ptr(), output_length.data_ptr(), S.data_ptr(), R.data_ptr(),
+                          Lt.data_ptr(), M.data_ptr(), B, L, ml, _stream(ob_lprob)), lib)
         ctx.mark_non_differentiable(R, Lt, M)
         return S[:, 1, :].clone(), R, Lt, M
 

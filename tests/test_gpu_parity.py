@@ -606,3 +606,53 @@ def test_general_max_left_viterbi_bit_exact(ml, L, ms):
     assert np.isfinite(S_o[:, 1, :]).any()
     assert np.array_equal(scores.cpu().numpy(), S_o[:, 1, :])
     assert np.array_equal(R.cpu().numpy(), R_o) and np.array_equal(Lt.cpu().numpy(), L_o) and np.array_equal(M.cpu().numpy(), M_o)
+
+
+@pytest.mark.parametrize("ml,L,ms,ns,generic_local", [
+    (1, 32, [32, 20, 8], [10, 8, 3], False),
+    (1, 130, [130, 96], [22, 30], False),
+    (3, 30, [30, 22, 14], [9, 8, 5], True),
+])
+def test_float64_tables_vs_oracle(ml, L, ms, ns, generic_local):
+    """The float64 instantiation the reference also dispatches (pcfg_loss.cu:395): log-likelihood, both gradients (scaled
+    by a non-trivial upstream gradient through autograd) and the best-tree alignment against the float64 oracle."""
+    match, links, ol, tl = _generic_batch(ml, L, ms, ns, seed=7 * ml + L, generic_local=generic_local)
+    match, links = match.double(), links.double()
+    S64, C64 = oracle.inside_fwd(match.numpy(), links.numpy(), ol.numpy(), tl.numpy(), dtype=np.float64)
+    mg64, lg64 = oracle.inside_bwd(np.ones(len(ms)), S64, C64, match.numpy(), links.numpy(), ol.numpy(), tl.numpy())
+    md = match.to(DEV).requires_grad_(True)
+    ld = links.to(DEV).requires_grad_(True)
+    ll = ops.cuda_pcfg_loss(md, ld, ol.to(DEV), tl.to(DEV))
+    assert ll.dtype == torch.float64
+    want = S64[:, 0, 0]
+    got = ll.detach().cpu().numpy()
+    fin = np.isfinite(want)
+    assert fin.any() and np.array_equal(np.isfinite(got), fin)
+    assert np.allclose(got[fin], want[fin], rtol=1e-12)
+    w = torch.linspace(0.5, 1.5, ll.numel(), device=DEV, dtype=torch.float64)
+    (ll.masked_fill(~torch.isfinite(ll), 0) * w).sum().backward()
+    wn = w.cpu().numpy()
+    for bi in range(len(ms)):
+        for g_got, g_want in ((md.grad[bi], mg64[bi] * wn[bi]), (ld.grad[bi], lg64[bi] * wn[bi])):
+            g_got = g_got.cpu().numpy()
+            assert np.isfinite(g_got).all()
+            assert np.abs(g_got - g_want).max() <= 1e-10 * max(np.abs(g_want).max(), 1e-30)
+    tree, ll2 = ops.cuda_pcfg_best_tree(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV))
+    want_tree = oracle.best_tree(S64, C64, match.numpy(), links.numpy(), ol.numpy(), tl.numpy(), dtype=np.float64)
+    assert np.array_equal(tree.cpu().numpy(), want_tree)
+    assert torch.allclose(ll2, ll.detach(), rtol=1e-12, equal_nan=True)
+
+
+@pytest.mark.parametrize("ml,L,ms", [(1, 64, [64, 40, 12]), (3, 66, [66, 50])])
+def test_float64_viterbi_bit_exact(ml, L, ms):
+    from test_oracle_inside import random_links
+    rng = np.random.default_rng(11 * ml + L)
+    links = np.stack([random_links(rng, L, m, ml, p_drop=0.1, generic_local=ml != 1) for m in ms])
+    ob = rng.normal(size=(len(ms), L)) - 1.0
+    ol = torch.tensor(ms)
+    scores, R, Lt, M = ops.cuda_pcfg_viterbi(torch.from_numpy(ob).to(DEV), torch.from_numpy(links).to(DEV), ol.to(DEV))
+    assert scores.dtype == torch.float64
+    S_o, R_o, L_o, M_o = oracle.viterbi(ob, links, ol.numpy(), dtype=np.float64)
+    assert np.isfinite(S_o[:, 1, :]).any()
+    assert np.array_equal(scores.cpu().numpy(), S_o[:, 1, :])
+    assert np.array_equal(R.cpu().numpy(), R_o) and np.array_equal(Lt.cpu().numpy(), L_o) and np.array_equal(M.cpu().numpy(), M_o)
