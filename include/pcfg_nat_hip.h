@@ -171,6 +171,10 @@ int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *
  * graph node).  On return (stream order) logits holds d loss / d logits, links_grad d loss / d links, loss_out[0] the
  * loss, loss_out[1] the number of invalid sentences; match_all, S, aux, match_all_grad and row_lse ([B,L] float32) are
  * caller workspaces of the shapes documented at the individual entry points.
+ * matchmask [B,T,L] / keep_word_mask [B,L] (bytes, 0 = false; both NULL = off): the criterion's force-emit masking
+ * (nat_pcfg_loss.py:116-121) with the outputs of the glancing step - a graph node whose input was revealed
+ * (keep_word_mask) may only emit the target position it is aligned to (matchmask), through a detached value, i.e. the
+ * logits row of such a node gets a zero gradient.
  * slices: 1 = the whole batch at once; k > 1 = the batch is processed as k slices (sentences [i*B/k, (i+1)*B/k)) that
  * alternate between `stream` and one helper stream the library keeps per device (created on first use, default
  * priority), so that the latency-bound inside kernels of one slice run beside the bandwidth-bound gather kernels of the
@@ -179,7 +183,8 @@ int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *
  * inside forward+backward and the gather backward of slice 0 (for timing).
  */
 int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, const float *links,
-                           const int64_t *output_length, const int64_t *target_length, float *match_all, float *S,
+                           const int64_t *output_length, const int64_t *target_length, const unsigned char *matchmask,
+                           const unsigned char *keep_word_mask, float *match_all, float *S,
                            float *aux, float *match_all_grad, float *links_grad, float *row_lse, float *loss_out, int64_t B,
                            int64_t L, int64_t V, int64_t T, int64_t ml, int64_t slices, void *stream, void *const *events);
 

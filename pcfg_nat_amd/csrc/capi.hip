@@ -54,7 +54,8 @@ int get_helper(DeviceHelper **out) {
 }  // namespace
 
 extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, const float *links,
-                                      const int64_t *output_length, const int64_t *target_length, float *match_all, float *S,
+                                      const int64_t *output_length, const int64_t *target_length, const unsigned char *matchmask,
+                                      const unsigned char *keep_word_mask, float *match_all, float *S,
                                       float *aux, float *match_all_grad, float *links_grad, float *row_lse, float *loss_out, int64_t B,
                                       int64_t L, int64_t V, int64_t T, int64_t ml, int64_t slices, void *stream,
                                       void *const *events) {
@@ -64,6 +65,8 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
     PCFGNAT_REQUIRE(logits && targets && links && output_length && target_length && match_all && S && aux && match_all_grad &&
                         links_grad && row_lse && loss_out,
                     "criterion_step: null pointer");
+    PCFGNAT_REQUIRE((matchmask == nullptr) == (keep_word_mask == nullptr),
+                    "criterion_step: matchmask and keep_word_mask must be given together (or both be null)");
     if (slices < 1) slices = 1;
     if (slices > B) slices = B;
     hipStream_t main_stream = (hipStream_t)stream;
@@ -87,6 +90,8 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
         float *ma_i = match_all + (size_t)b0 * L * T, *S_i = S + (size_t)b0 * Mc * (T + 2), *aux_i = aux + (size_t)b0 * aux_per_sentence;
         float *mg_i = match_all_grad + (size_t)b0 * L * T, *lkg_i = links_grad + (size_t)b0 * L * (ml + 1) * L;
         float *lse_i = row_lse + (size_t)b0 * L;
+        const unsigned char *mm_i = matchmask ? matchmask + (size_t)b0 * T * L : nullptr;
+        const unsigned char *keep_i = keep_word_mask ? keep_word_mask + (size_t)b0 * L : nullptr;
         const bool mark = events && i == 0;  // timing events bracket the kernels of slice 0
 #define PCFGNAT_MARK(k)                                                                   \
     do {                                                                                  \
@@ -96,7 +101,7 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
         // kernels of slice i-1 rather than beside its gather
         if (i > 0) PCFGNAT_HIP_CHECK(hipStreamWaitEvent(s, h->gathered[(i - 1) & 1], 0));
         PCFGNAT_MARK(0);
-        int rc = pcfgnat_logsoftmax_gather_lse(lg_i, dtype, tg_i, T, 0, 1, ma_i, lse_i, ol_i, tl_i, nb, L, V, T, s);
+        int rc = pcfgnat::lsg_forward_lse_force(lg_i, dtype, tg_i, ma_i, lse_i, ol_i, tl_i, mm_i, keep_i, nb, L, V, T, s);
         if (rc != PCFGNAT_OK) return rc;
         PCFGNAT_MARK(1);
         if (slices > 1) PCFGNAT_HIP_CHECK(hipEventRecord(h->gathered[i & 1], s));
@@ -109,9 +114,10 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
         PCFGNAT_MARK(6);
         if (slices == 1)  // the loss is reduced by the first workgroup of the same launch (S is complete by now)
             rc = pcfgnat::lsg_backward_lse_with_loss(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, S, Mc * (T + 2), target_length,
-                                                     loss_out, s);
+                                                     loss_out, keep_i, s);
         else
-            rc = pcfgnat_logsoftmax_gather_backward_lse(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, s);
+            rc = pcfgnat::lsg_backward_lse_with_loss(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, nullptr, 0, nullptr, nullptr,
+                                                     keep_i, s);
         if (rc != PCFGNAT_OK) return rc;
         PCFGNAT_MARK(7);
 #undef PCFGNAT_MARK

@@ -48,10 +48,16 @@ int lsg_forward_eos_argmax(const void *logits, int dtype, const int64_t *targets
                            const int64_t *output_length, const int64_t *target_length, int64_t B, int64_t L, int64_t V, int64_t T,
                            void *stream);
 
-// pcfgnat_logsoftmax_gather_backward_lse whose first workgroup also reduces the criterion's loss (lsg.hip)
+// pcfgnat_logsoftmax_gather_backward_lse whose first workgroup also reduces the criterion's loss when loss_out is given
+// (lsg.hip); rows with keep[row] != 0 get a zero gradient
 int lsg_backward_lse_with_loss(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T,
-                               const float *S, int64_t ll_stride, const int64_t *target_length, float *loss_out, void *stream);
+                               const float *S, int64_t ll_stride, const int64_t *target_length, float *loss_out,
+                               const unsigned char *keep, void *stream);
+// pcfgnat_logsoftmax_gather_lse over the [B,T] targets with the eos mask and the force-emit masks
+int lsg_forward_lse_force(const void *logits, int dtype, const int64_t *targets, void *selected, void *lse,
+                          const int64_t *output_length, const int64_t *target_length, const unsigned char *matchmask,
+                          const unsigned char *keep, int64_t B, int64_t L, int64_t V, int64_t T, void *stream);
 
 // General max_left (generic_ml.hip)
 size_t generic_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml);
@@ -139,6 +145,14 @@ constexpr float NEG_INF_F = -__builtin_huge_valf();
 // The criterion's reduction (nat_pcfg_loss.py:123-135) by one workgroup of NT threads, in a fixed order:
 // out[0] = -(1/B) * sum_b [ll_b finite] ll_b / n_b, out[1] = number of sentences with a non-finite ll_b, where
 // ll_b = S[b * stride].  Every thread of the workgroup must call it.
+// The criterion's force-emit masking (nat_pcfg_loss.py:116-121) folded into the gather: graph nodes whose input token was
+// revealed by glancing (keep[b,p] != 0) may only emit the target position they are aligned to (matchmask[b,s,p] != 0,
+// every other position becomes -inf) and pass no gradient to their logits.  keep = null: off.
+struct ForceEmit {
+    const unsigned char *matchmask;  // [B,T,L]
+    const unsigned char *keep;       // [B,L]
+};
+
 struct LossTask {
     const float *S;
     const int64_t *tgt_len;

@@ -244,7 +244,7 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
                                                      int V, int Tn, const int64_t *__restrict__ eos_out_len,
                                                      const int64_t *__restrict__ eos_tgt_len,
                                                      typename Elem<T>::compute *__restrict__ lse_out,
-                                                     int64_t *__restrict__ argmax_out) {
+                                                     int64_t *__restrict__ argmax_out, ForceEmit fe) {
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
     constexpr int NW = NT / 64;
@@ -334,10 +334,15 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
             const int64_t b = row / L, pnode = row % L;
             if (pnode != eos_out_len[b] - 1) eos_col = (int)(eos_tgt_len[b] - 1);
         }
+        const bool forced = fe.keep != nullptr && fe.keep[row] != 0;  // (nat_pcfg_loss.py:116-121)
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
             int s = tid + g * NT;
-            if (s < Tn) sel[row * (int64_t)Tn + s] = (s == eos_col) ? neg_inf(CT()) : rn.logprob(gv[g], sum);
+            if (s < Tn) {
+                CT val = (s == eos_col) ? neg_inf(CT()) : rn.logprob(gv[g], sum);
+                if (forced && fe.matchmask[((row / L) * (int64_t)Tn + s) * L + row % L] == 0) val = neg_inf(CT());
+                sel[row * (int64_t)Tn + s] = val;
+            }
         }
 
         if (GRAD) {
@@ -444,7 +449,8 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
                                                      int64_t sl, int64_t st,
                                                      const typename Elem<T>::compute *__restrict__ gsel, int64_t rows,
                                                      int L, int V, int Tn,
-                                                     const typename Elem<T>::compute *__restrict__ lse, LossTask loss) {
+                                                     const typename Elem<T>::compute *__restrict__ lse, LossTask loss,
+                                                     const unsigned char *__restrict__ detach_rows) {
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
     constexpr int FIX = (TCAP + NT - 1) / NT;
@@ -474,8 +480,10 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
         if (ep >= 0) edge = Elem<T>::widen(pr[ep]);
 
         // -(sum_s g), computed redundantly by every wave; rounded to the buffer dtype in the reference split (pcfg_loss.py:176)
+        // a row whose gathered values were detached (force-emit, nat_pcfg_loss.py:121) gets no gradient at all
+        const bool live = detach_rows == nullptr || detach_rows[row] == 0;
         CT part = 0;
-        for (int s = lane; s < Tn; s += 64) part += gr[s];
+        for (int s = lane; s < Tn && live; s += 64) part += gr[s];
         const CT ns = FROM_LOGITS ? -wave_sum(part) : Elem<T>::widen(Elem<T>::narrow(-wave_sum(part)));
         const RowNorm<CT> rn = RowNorm<CT>::from_lse(FROM_LOGITS ? lse[row] : (CT)0);
 
@@ -488,10 +496,10 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
             bool ok = (uint64_t)t < (uint64_t)V;
             s_idx[s] = ok ? (int)t : -1;
             if (FROM_LOGITS) {
-                s_g[s] = gr[s];
+                s_g[s] = live ? gr[s] : (CT)0;
                 s_p[s] = ok ? rn.e(Elem<T>::widen(pr[t])) : (CT)0;
             } else {
-                s_g[s] = Elem<T>::widen(Elem<T>::narrow(gr[s]));
+                s_g[s] = live ? Elem<T>::widen(Elem<T>::narrow(gr[s])) : (CT)0;
                 s_p[s] = ok ? Elem<T>::widen(pr[t]) : (CT)0;
             }
         }
@@ -560,7 +568,8 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
 
 template <typename T>
 int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, void *sel, int grad, int64_t rows,
-               int L, int V, int Tn, const int64_t *eos_ol, const int64_t *eos_tl, void *lse, int64_t *argmax, hipStream_t stream) {
+               int L, int V, int Tn, const int64_t *eos_ol, const int64_t *eos_tl, void *lse, int64_t *argmax, hipStream_t stream,
+               ForceEmit fe = ForceEmit{nullptr, nullptr}) {
     using CT = typename Elem<T>::compute;
 #ifndef LSG_FWD_NT
 #define LSG_FWD_NT 512
@@ -573,17 +582,17 @@ int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
     int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
     if (grad)
         hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, true>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)x, idx, sb,
-                           sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax);
+                           sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax, fe);
     else
         hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, false>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)x, idx,
-                           sb, sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax);
+                           sb, sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax, fe);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
 
 template <typename T>
 int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, const void *g, int64_t rows, int L, int V,
-               int Tn, const void *lse, const LossTask &loss, hipStream_t stream) {
+               int Tn, const void *lse, const LossTask &loss, hipStream_t stream, const unsigned char *detach_rows = nullptr) {
     using CT = typename Elem<T>::compute;
     constexpr int NT = 512;
     constexpr int MAXC = 10;
@@ -592,10 +601,10 @@ int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
     int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
     if (lse != nullptr)
         hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, true>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,
-                           (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss);
+                           (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss, detach_rows);
     else
         hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, false>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl,
-                           st, (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss);
+                           st, (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss, detach_rows);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -628,18 +637,19 @@ using namespace pcfgnat;
 
 static int lsg_forward_dispatch(void *word_ins_out, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                 void *selected, int require_grad, int64_t B, int64_t L, int64_t V, int64_t T,
-                                const int64_t *eos_ol, const int64_t *eos_tl, void *lse, void *stream, int64_t *argmax = nullptr) {
+                                const int64_t *eos_ol, const int64_t *eos_tl, void *lse, void *stream, int64_t *argmax = nullptr,
+                                ForceEmit fe = ForceEmit{nullptr, nullptr}) {
     int rc = check_common(word_ins_out, select_idx, selected, B, L, V, T);
     if (rc != PCFGNAT_OK) return rc;
     if (B * L == 0) return PCFGNAT_OK;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case PCFGNAT_F16:
-            return launch_fwd<__half>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s);
+            return launch_fwd<__half>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe);
         case PCFGNAT_F32:
-            return launch_fwd<float>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s);
+            return launch_fwd<float>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe);
         case PCFGNAT_F64:
-            return launch_fwd<double>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s);
+            return launch_fwd<double>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe);
         default:
             return fail(PCFGNAT_EINVAL, "logsoftmax_gather: unknown dtype code %d (float16, float32, float64 are dispatched)", dtype);
     }
@@ -689,18 +699,19 @@ extern "C" int pcfgnat_logsoftmax_max(const void *logits, int dtype, void *best_
 
 static int lsg_backward_dispatch(void *buf, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                  const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T, void *stream,
-                                 const LossTask &loss = LossTask{nullptr, nullptr, nullptr, 0, 0}) {
+                                 const LossTask &loss = LossTask{nullptr, nullptr, nullptr, 0, 0},
+                                 const unsigned char *detach_rows = nullptr) {
     int rc = check_common(buf, select_idx, grad_selected, B, L, V, T);
     if (rc != PCFGNAT_OK) return rc;
     if (B * L == 0) return PCFGNAT_OK;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case PCFGNAT_F16:
-            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s);
+            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows);
         case PCFGNAT_F32:
-            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s);
+            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows);
         case PCFGNAT_F64:
-            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s);
+            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows);
         default:
             return fail(PCFGNAT_EINVAL, "logsoftmax_gather_backward: unknown dtype code %d", dtype);
     }
@@ -722,10 +733,20 @@ int pcfgnat::lsg_forward_eos_argmax(const void *logits, int dtype, const int64_t
 int pcfgnat::lsg_backward_lse_with_loss(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                         const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T,
                                         const float *S, int64_t ll_stride, const int64_t *target_length, float *loss_out,
-                                        void *stream) {
-    PCFGNAT_REQUIRE(B >= 1 && L >= 1 && lse && S && target_length && loss_out, "logsoftmax_gather_backward: null pointer or empty batch");
+                                        const unsigned char *keep, void *stream) {
+    PCFGNAT_REQUIRE(B >= 1 && L >= 1 && lse && (loss_out == nullptr || (S && target_length)),
+                    "logsoftmax_gather_backward: null pointer or empty batch");
     return lsg_backward_dispatch(logits_inout, dtype, select_idx, sb, sl, st, grad_selected, lse, B, L, V, T, stream,
-                                 LossTask{S, target_length, loss_out, (int)B, ll_stride});
+                                 LossTask{S, target_length, loss_out, (int)B, ll_stride}, keep);
+}
+
+int pcfgnat::lsg_forward_lse_force(const void *logits, int dtype, const int64_t *targets, void *selected, void *lse,
+                                   const int64_t *output_length, const int64_t *target_length, const unsigned char *matchmask,
+                                   const unsigned char *keep, int64_t B, int64_t L, int64_t V, int64_t T, void *stream) {
+    PCFGNAT_REQUIRE(B * L == 0 || (lse && output_length && target_length), "logsoftmax_gather_lse: null pointer");
+    PCFGNAT_REQUIRE((matchmask == nullptr) == (keep == nullptr), "criterion_step: matchmask and keep_word_mask must be given together");
+    return lsg_forward_dispatch(const_cast<void *>(logits), dtype, targets, T, 0, 1, selected, 0, B, L, V, T, output_length, target_length,
+                                lse, stream, nullptr, ForceEmit{matchmask, keep});
 }
 
 extern "C" int pcfgnat_logsoftmax_gather_backward_lse(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb,

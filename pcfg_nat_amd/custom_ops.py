@@ -725,13 +725,16 @@ def pcfg_lookahead_decode(links, unreduced_logits, unreduced_tokens, output_leng
     return (tokens, idx) if return_pointers else tokens
 
 
-def pcfg_criterion_step(logits, targets, links, output_length, target_length, events=None, slices=None):
+def pcfg_criterion_step(logits, targets, links, output_length, target_length, events=None, slices=None, matchmask=None,
+                        keep_word_mask=None):
     """The criterion's whole training pass in one native call (``pcfgnat_criterion_step``): ``logits`` [B,L,V] (fp16 or
     fp32, contiguous) is consumed in place and holds d loss / d logits afterwards.  ``events``: optional list of eight
     ``torch.cuda.Event(enable_timing=True)`` (each recorded at least once before; entries may be None) that the library records before/after
     the gather forward, inside forward, inside backward and gather backward of the first slice.  ``slices``: how many
     batch slices alternate between the current stream and the library's helper stream (default 1: measured on MI355X the
-    bandwidth-bound gather kernels leave no room for a second kernel on the CUs, so slicing does not pay).  Returns
+    bandwidth-bound gather kernels leave no room for a second kernel on the CUs, so slicing does not pay).
+    ``matchmask`` [B,T,L] / ``keep_word_mask`` [B,L] (bool, as the glancing step returns them): the criterion's
+    force-emit masking (nat_pcfg_loss.py:116-121); both None = off (``--no-force-emit``).  Returns
     (loss_and_invalid [2] float32, links_grad, ll [B], match_all_eos_masked, match_all_grad)."""
     lib = get_pcfg_kernel()
     _need_cuda("pcfg_criterion_step", logits, targets, links, output_length, target_length)
@@ -754,6 +757,16 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
     dev = logits.device
     if slices is None:
         slices = 1
+    if (matchmask is None) != (keep_word_mask is None):
+        raise RuntimeError("pcfg_criterion_step: matchmask and keep_word_mask go together")
+    mm_ptr = keep_ptr = None
+    if matchmask is not None:
+        _need_cuda("pcfg_criterion_step", logits, matchmask, keep_word_mask)
+        if tuple(matchmask.shape) != (B, T, L) or tuple(keep_word_mask.shape) != (B, L):
+            raise RuntimeError("pcfg_criterion_step: matchmask must be [bsz, tarlen, prelen] and keep_word_mask [bsz, prelen]")
+        mm8 = matchmask.to(torch.uint8).contiguous()
+        keep8 = keep_word_mask.to(torch.uint8).contiguous()
+        mm_ptr, keep_ptr = mm8.data_ptr(), keep8.data_ptr()
     ev_arr = None
     if events is not None:
         import ctypes
@@ -769,7 +782,7 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
         row_lse = torch.empty((B, L), dtype=torch.float32, device=dev)
         out = torch.empty((2,), dtype=torch.float32, device=dev)
         _lib.check(lib.pcfgnat_criterion_step(logits.data_ptr(), code, targets.data_ptr(), links.data_ptr(), ol.data_ptr(),
-                                              tl.data_ptr(), match.data_ptr(), S.data_ptr(), aux.data_ptr(), mg.data_ptr(),
+                                              tl.data_ptr(), mm_ptr, keep_ptr, match.data_ptr(), S.data_ptr(), aux.data_ptr(), mg.data_ptr(),
                                               lg.data_ptr(), row_lse.data_ptr(), out.data_ptr(), B, L, V, T, ml, slices,
                                               _stream(logits), ev_arr), lib)
     return out, lg, S[:, 0, 0], match, mg

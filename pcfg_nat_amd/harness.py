@@ -24,15 +24,23 @@ def eos_masked(match_all, output_length, target_length):
     return match_all.masked_fill(eos_mask, float("-inf"))
 
 
-def compute_pcfg_loss(outputs, output_masks, targets, target_masks, links, ops=_default_ops):
+def compute_pcfg_loss(outputs, output_masks, targets, target_masks, links, ops=_default_ops, matchmask=None, keep_word_mask=None,
+                      no_force_emit=False):
     """loss = -(log-likelihood / target_length).mean() with invalid sentences zeroed (nat_pcfg_loss.py:98-145).
     ``outputs`` [B,L,V] is consumed in place (it holds softmax probabilities afterwards and the gradient after
-    backward).  Returns a dict with ``loss``, ``ll`` (per sentence), ``invalid_nsentences``."""
+    backward).  ``matchmask`` [B,T,L] / ``keep_word_mask`` [B,L] (from the glancing step): unless ``no_force_emit``, a
+    revealed graph node may only emit the target position it is aligned to, through a detached value (:116-121).
+    Returns a dict with ``loss``, ``ll`` (per sentence), ``invalid_nsentences``."""
     prelen = outputs.shape[1]
     output_length = output_masks.sum(dim=-1)
     target_length = target_masks.sum(dim=-1)
     outputs, match_all = ops.dag_logsoftmax_gather_inplace(outputs, targets.unsqueeze(1).expand(-1, prelen, -1))
     match_all_eos_masked = eos_masked(match_all, output_length, target_length)
+    if matchmask is not None and not no_force_emit:
+        glat_prev_mask = keep_word_mask.unsqueeze(-1)
+        mm = matchmask.transpose(1, 2)
+        match_all_eos_masked = (match_all_eos_masked.masked_fill(glat_prev_mask, 0) +
+                                match_all_eos_masked.masked_fill(~mm, float("-inf")).masked_fill(~glat_prev_mask, 0).detach())
     loss_result = ops.cuda_pcfg_loss(match_all_eos_masked, links, output_length, target_length)
     invalid_masks = loss_result.isinf().logical_or(loss_result.isnan())
     loss_result = loss_result.masked_fill(invalid_masks, 0)
@@ -167,12 +175,13 @@ def train_step_fused(logits, targets, links, output_length, target_length, ops=_
     return loss, glinks, ll
 
 
-def train_step_single_call(logits, targets, links, output_length, target_length, ops=_default_ops, mark=None, slices=None):
+def train_step_single_call(logits, targets, links, output_length, target_length, ops=_default_ops, mark=None, slices=None,
+                           matchmask=None, keep_word_mask=None):
     """``train_step_fused`` issued as one native call (``pcfgnat_criterion_step``): the five kernels are enqueued back to
     back by the library and the scalar loss is reduced on the device.  Returns (loss, links_grad, ll)."""
     events = None
     if mark is not None:
         events = mark("events", 8)  # the caller hands out eight timing events for this step
     out, glinks, ll, _, _ = ops.pcfg_criterion_step(logits, targets, links, output_length, target_length, events=events,
-                                                 slices=slices)
+                                                 slices=slices, matchmask=matchmask, keep_word_mask=keep_word_mask)
     return out[0], glinks, ll

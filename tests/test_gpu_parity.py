@@ -549,6 +549,40 @@ def test_fused_step_equals_autograd_step():
         assert not glinks[3].any() and not buf[3].any()
 
 
+def test_force_emit_step_equals_autograd_step():
+    """The criterion with force-emit masking (nat_pcfg_loss.py:116-121; on in the scripts without --no-force-emit): the
+    masks come from a glancing pass over the same batch; autograd through the torch restatement of those lines against
+    the single-call step that folds them into the gather kernels.  Revealed nodes must end up with a zero logits
+    gradient, and the loss must differ from the unmasked one (the masks do something)."""
+    batch = synth.training_batch(4, 64, 12, 700, [64, 40, 22, 8], [12, 9, 7, 3], seed=33, logit_scale=2.0,
+                                 logit_dtype=torch.float16)
+    B, L, V = batch["logits"].shape
+    out_mask = (torch.arange(L).view(1, L) < batch["output_length"].view(B, 1)).to(DEV)
+    tgt = batch["targets"].to(DEV)
+    tgt_mask = tgt.ne(synth.PAD)
+    ol, tl = batch["output_length"].to(DEV), batch["target_length"].to(DEV)
+    prev = torch.full((B, L), 3, dtype=torch.int64, device=DEV).masked_fill(~out_mask, synth.PAD)
+    gen = torch.Generator().manual_seed(5)
+    glat = harness.glat_alignment(batch["logits"].to(DEV).clone(), tgt, prev, batch["links"].to(DEV), 0.5, generator=gen,
+                                  noise_device="cpu")
+    mm, keep = glat["matchmask"], glat["keep_word_mask"]
+    assert keep.any() and not keep.all()
+    leaf = batch["logits"].to(DEV).float().requires_grad_(True)
+    links = batch["links"].to(DEV).requires_grad_(True)
+    res = harness.compute_pcfg_loss(leaf.half(), out_mask, tgt, tgt_mask, links, matchmask=mm, keep_word_mask=keep)
+    res["loss"].backward()
+    plain = harness.compute_pcfg_loss(batch["logits"].to(DEV).clone(), out_mask, tgt, tgt_mask, batch["links"].to(DEV))
+    assert abs(float(plain["loss"].detach()) - float(res["loss"].detach())) > 1e-3
+    for k in (1, 2):
+        buf = batch["logits"].to(DEV).clone()
+        loss, glinks, ll = harness.train_step_single_call(buf, tgt, batch["links"].to(DEV), ol, tl, slices=k, matchmask=mm,
+                                                          keep_word_mask=keep)
+        assert torch.allclose(loss, res["loss"].detach(), rtol=1e-6)
+        assert torch.allclose(glinks, links.grad, rtol=1e-5, atol=1e-9)
+        assert torch.allclose(buf.float(), leaf.grad, rtol=2 ** -9, atol=2 ** -22)
+        assert not buf[keep].any()
+
+
 def _generic_batch(ml, L, ms, ns, seed, generic_local):
     """Batch for a general max_left: links with the grammar's structural support (optionally with composite local trees),
     random emissions with the eos column masked."""

@@ -76,6 +76,46 @@ def test_glat_alignment_is_deterministic_and_consistent():
     assert torch.equal(a["matchmask"].sum(-1).sum(-1), n)
 
 
+def test_force_emit_semantics():
+    """Force-emit (nat_pcfg_loss.py:116-121) over the oracle ops: revealed nodes keep only their aligned target position
+    and pass no gradient; with every node marked as revealed the loss is that of the single derivation the alignment
+    spells (its emissions + its links), which is computed here by hand from the path."""
+    batch = synth.config1()
+    out_mask, tgt_mask = _masks(batch)
+    B, L, V = batch["logits"].shape
+    prev = torch.full((B, L), 3, dtype=torch.int64)
+    gen = torch.Generator().manual_seed(3)
+    glat = harness.glat_alignment(batch["logits"].clone(), batch["targets"], prev, batch["links"], 0.5, ops=oracle_ops,
+                                  generator=gen)
+    mm, keep = glat["matchmask"], glat["keep_word_mask"]
+    assert keep.any()
+    leaf = batch["logits"].clone().requires_grad_(True)
+    res = harness.compute_pcfg_loss(leaf * 1.0, out_mask, batch["targets"], tgt_mask, batch["links"], ops=oracle_ops,
+                                    matchmask=mm, keep_word_mask=keep)
+    res["loss"].backward()
+    assert torch.isfinite(res["loss"])
+    assert not leaf.grad[keep].any() and leaf.grad[~keep].any()
+    off = harness.compute_pcfg_loss(batch["logits"].clone(), out_mask, batch["targets"], tgt_mask, batch["links"],
+                                    ops=oracle_ops, matchmask=mm, keep_word_mask=keep, no_force_emit=True)
+    plain = harness.compute_pcfg_loss(batch["logits"].clone(), out_mask, batch["targets"], tgt_mask, batch["links"],
+                                      ops=oracle_ops)
+    assert torch.equal(off["loss"], plain["loss"]) and float(res["loss"].detach()) > float(plain["loss"])
+    # every node marked as revealed (nodes off the alignment then can emit nothing): only the aligned derivation survives
+    path = glat["path"]
+    all_keep = torch.ones_like(path, dtype=torch.bool)
+    one = harness.compute_pcfg_loss(batch["logits"].clone(), out_mask, batch["targets"], tgt_mask, batch["links"],
+                                    ops=oracle_ops, matchmask=mm, keep_word_mask=all_keep)
+    logp = torch.log_softmax(batch["logits"].double(), -1)
+    for b in range(B):
+        nodes = [a for a in range(L) if path[b, a] >= 0]
+        total = sum(float(logp[b, a, batch["targets"][b, path[b, a]]]) for a in nodes)
+        mains = [a for a in nodes if a % 2 == 1]
+        for a, c in zip(mains[:-1], mains[1:]):
+            k = 1 if (a - 1) in nodes and a - 1 >= 1 else 0  # the leaf in front of a is on the tree: left option 1
+            total += float(batch["links"][b, a, k, c])
+        assert abs(float(one["ll"][b]) - total) < 1e-4 * abs(total), (b, float(one["ll"][b]), total)
+
+
 def test_viterbi_decode_glue():
     batch = synth.decode_batch([6, 10, 4], seed=5, V=64, logit_dtype=torch.float32)
     ob, tok = synth.ob_and_tokens(batch["logits"])
