@@ -177,6 +177,69 @@ def long_sentence_timing(dev):
     return {"ms_per_step": ms, "sentences_per_s": B / (ms * 1e-3), "workload": "B=8, L=512, T=140, V=40000, fp16 logits"}
 
 
+def link_scorer_timing(dev):
+    """The model's link scorer after its projections at the training shape (B=40, L=128, 8 heads of 64, fp16 chunks):
+    forward alone (what the glancing pass and inference run) and forward + backward."""
+    import torch
+    from pcfg_nat_amd import custom_ops as ops, synth
+
+    B, L, H, F = 40, 128, 8, 64
+    g = torch.Generator().manual_seed(0)
+    q, kl, kr = ((torch.randn(B, L, H, F, generator=g) * 0.5).half().to(dev) for _ in range(3))
+    gate = torch.randn(B, L, H, generator=g).half().to(dev)
+    m, _ = synth._wmt_lengths(B, torch.Generator().manual_seed(1001), 10, L // 4, 32)
+    prev = torch.full((B, L), 3).masked_fill(torch.arange(L).view(1, L) >= m.view(B, 1), synth.PAD).to(dev)
+    lm, rm, mc = (x.to(dev) for x in synth.support_masks(L, 1))
+    G = torch.randn(B, L, 2, L, generator=g).to(dev)
+
+    def fwd():
+        with torch.no_grad():
+            return ops.pcfg_extract_links(q, kl, kr, gate, prev, synth.PAD, lm, rm, mc)
+
+    G = G.masked_fill(~torch.isfinite(fwd()), 0)  # the upstream gradient of masked links is zero
+
+    def fwd_bwd():
+        ts = [t.detach().requires_grad_(True) for t in (q, kl, kr, gate)]
+        ops.pcfg_extract_links(*ts, prev, synth.PAD, lm, rm, mc).backward(G)
+
+    res = {}
+    for name, fn in (("forward_ms", fwd), ("forward_backward_ms", fwd_bwd)):
+        for _ in range(3):
+            fn()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(20):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        res[name] = start.elapsed_time(end) / 20
+    return res
+
+
+def decode_front_end_timing(dev):
+    """max_v log_softmax and arg max over the vocabulary in one read of the logits (the model's decode front-end) at
+    B=64, L=400, V=40000 fp16 (2.05 GB)."""
+    import torch
+    from pcfg_nat_amd import custom_ops as ops
+
+    B, L, V = 64, 400, 40000
+    ggen = torch.Generator(device=dev).manual_seed(13)
+    x = (torch.randn(B, L, V, device=dev, dtype=torch.float32, generator=ggen) * 3).half()
+    for _ in range(2):
+        ops.logsoftmax_max(x)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(5):
+        ops.logsoftmax_max(x)
+    end.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(end) / 5
+    nbytes = B * L * V * 2 + B * L * 12
+    return {"ms_per_call": ms, "gb_per_s": nbytes / (ms * 1e-3) / 1e9, "workload": "B=64, L=400, V=40000, fp16 logits"}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -317,6 +380,8 @@ def main():
         result["viterbi"] = decode_timing(dev)
         result["glat_alignment"] = glat_timing(torch.randn(B, L, V, device=dev, generator=ggen).mul_(2).half(), targets, links, ol)
         result["long_sentences"] = long_sentence_timing(dev)
+        result["link_scorer"] = link_scorer_timing(dev)
+        result["decode_front_end"] = decode_front_end_timing(dev)
     if not args.no_cpu_baseline:
         batch_cpu = {"output_length": m, "target_length": n, "links": links_cpu, "targets": targets_cpu}
         result["cpu_baseline"] = cpu_baseline(batch_cpu, sample_logits, args.cpu_sentences)
