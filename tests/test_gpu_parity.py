@@ -365,7 +365,8 @@ def test_glat_single_call_small_ragged(ml):
 
 
 @pytest.mark.parametrize("B,L,H,F,dtype", [(3, 18, 2, 4, torch.float32), (2, 34, 8, 16, torch.float32), (4, 128, 8, 64, torch.float16),
-                                            (2, 514, 4, 8, torch.float32), (2, 22, 16, 8, torch.float32), (2, 12, 1, 8, torch.float32)])
+                                            (2, 514, 4, 8, torch.float32), (2, 22, 16, 8, torch.float32), (2, 12, 1, 8, torch.float32),
+                                            (2, 200, 4, 16, torch.float16), (2, 256, 2, 24, torch.float32)])
 def test_extract_links_forward_backward_vs_torch_restatement(B, L, H, F, dtype):
     from oracle import extract_links_ref as ref
     g = torch.Generator().manual_seed(L + H)
