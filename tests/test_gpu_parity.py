@@ -691,3 +691,43 @@ def test_float64_viterbi_bit_exact(ml, L, ms):
     assert np.isfinite(S_o[:, 1, :]).any()
     assert np.array_equal(scores.cpu().numpy(), S_o[:, 1, :])
     assert np.array_equal(R.cpu().numpy(), R_o) and np.array_equal(Lt.cpu().numpy(), L_o) and np.array_equal(M.cpu().numpy(), M_o)
+
+
+def test_smallest_shapes_through_every_entry_point():
+    """The smallest shapes the grammar allows (a graph of 4 nodes, i.e. two main-chain nodes; 2 target tokens; one
+    sentence) and an empty batch, through loss + gradients, best tree, the single-call step, viterbi and the decodes."""
+    batch = synth.training_batch(1, 4, 2, 9, [4], [2], seed=2)
+    match = _match_for(batch)
+    S64, C64, mg64, lg64 = _oracle_inside(batch, match.numpy())
+    assert np.isfinite(S64[0, 0, 0])
+    ol, tl = batch["output_length"].to(DEV), batch["target_length"].to(DEV)
+    md, ld = match.to(DEV).requires_grad_(True), batch["links"].to(DEV).requires_grad_(True)
+    ll = ops.cuda_pcfg_loss(md, ld, ol, tl)
+    assert np.allclose(ll.detach().cpu().numpy(), S64[:, 0, 0], rtol=1e-5)
+    ll.sum().backward()
+    assert np.allclose(md.grad.cpu().numpy(), mg64, atol=1e-5) and np.allclose(ld.grad.cpu().numpy(), lg64, atol=1e-5)
+    tree, _ = ops.cuda_pcfg_best_tree(match.to(DEV), batch["links"].to(DEV), ol, tl)
+    want_tree = oracle.best_tree(*oracle.inside_fwd(match.numpy(), batch["links"].numpy(), ol.cpu().numpy(), tl.cpu().numpy(),
+                                                    dtype=np.float32),
+                                 match.numpy(), batch["links"].numpy(), ol.cpu().numpy(), tl.cpu().numpy(), dtype=np.float32)
+    assert np.array_equal(tree.cpu().numpy(), want_tree)
+    buf = batch["logits"].to(DEV).half()
+    loss, glinks, ll2 = harness.train_step_single_call(buf, batch["targets"].to(DEV), batch["links"].to(DEV), ol, tl)
+    assert torch.isfinite(loss) and torch.isfinite(buf.float()).all()
+    # decode: 8 nodes is the smallest graph with a non-trivial length table (L/4 = 2)
+    dec = synth.decode_batch([2], seed=4, V=16, logit_dtype=torch.float32)
+    ob, tok = synth.ob_and_tokens(dec["logits"])
+    L = dec["links"].shape[1]
+    lmask = synth.support_masks(L, 1)[0]
+    want_tok, want_len = harness.viterbi_decode(ob, tok, dec["links"], dec["output_length"], lmask, ops=__import__("oracle_ops"))
+    for single in (False, True):
+        got_tok, got_len = harness.viterbi_decode(ob.to(DEV), tok.to(DEV), dec["links"].to(DEV), dec["output_length"].to(DEV),
+                                                  lmask.to(DEV), single_call=single)
+        assert torch.equal(got_len.cpu(), want_len) and torch.equal(got_tok.cpu(), want_tok)
+    # empty batch: nothing to do, nothing to fault on
+    e = torch.empty
+    ll0 = ops.cuda_pcfg_loss(e(0, 8, 4, device=DEV), e(0, 8, 2, 8, device=DEV), e(0, dtype=torch.int64, device=DEV),
+                             e(0, dtype=torch.int64, device=DEV))
+    assert ll0.shape == (0,)
+    sc, R, Lt, M = ops.cuda_pcfg_viterbi(e(0, 8, device=DEV), e(0, 8, 2, 8, device=DEV), e(0, dtype=torch.int64, device=DEV))
+    assert sc.shape == (0, 2) and R.shape == (0, 8, 2)
