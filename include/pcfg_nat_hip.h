@@ -137,6 +137,16 @@ int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *ma
                                        void *stream);
 
 /*
+ * No counterpart in the reference: tuning of the long-graph path (max_left = 1, 258 <= L <= 1026).  There a sentence is
+ * swept by a cluster of L/128 (rounded up) cooperating workgroups as long as all clusters of the batch fit on the device
+ * at once, B * cluster size <= max_workgroups (default 512), and by one workgroup otherwise.  A workgroup that waits for its
+ * peers for more than spin_limit polls (default 2^20, about a second) gives the sentence up, and the one-workgroup sweep
+ * redoes it in the same call; results are the same either way up to fp32 rounding.  max_workgroups = 0 switches the
+ * clusters off; a negative argument leaves that setting unchanged.  Process-wide, takes effect with the next call.
+ */
+void pcfgnat_cluster_config(int max_workgroups, int spin_limit);
+
+/*
  * The float64 instantiation the reference also dispatches (AT_DISPATCH_FLOATING_TYPES in pcfg_loss.cu:395,
  * pcfg_loss_backward.cu:693, pcfg_best_tree.cu:349, pcfg_viterbi.cu:291; no shipped script uses it).  Same arguments,
  * layouts and results as the float32 entry points above and below with double tables; every max_left, 1 included,

@@ -19,6 +19,8 @@
 // epilogue.
 #include "common.hip.h"
 
+#include <atomic>
+
 namespace pcfgnat {
 namespace {
 
@@ -978,11 +980,16 @@ __global__ __launch_bounds__(BT_NT) void best_tree_ml1_kernel(const float *__res
 // W0, W1, R [Mc][T+2] each, D [T+4], padding to a 16-byte boundary, then the compact link matrices (times log2 e) with
 // masked entries already -inf and rows padded to MP = 64*ceil(Mc/64) floats:
 // Ac [2][Mc][MP] by parent (Ac[k][a][c]) for the forward sweep and At [2][Mc][MP] by child (At[k][c][a]) for the
-// outside sweep, so that the sweeps stream them with unconditional 16-byte loads.
+// outside sweep, so that the sweeps stream them with unconditional 16-byte loads.  Last comes the exchange area of the
+// cluster sweeps (below): tagged 16-byte slots, forward column [2][MP] and outside weights [2][MP], and four ints
+// (forward gave up, outside sweep gave up, two unused).
 // ------------------------------------------------------------------------------------------------------------
 __host__ __device__ inline int stream_mp(int Mc) { return ((Mc + 63) / 64) * 64; }
 __host__ __device__ inline size_t stream_planes(int Mc, int T) { return (((size_t)6 * Mc * (T + 2) + (size_t)(T + 4)) + 3) & ~(size_t)3; }
-__host__ __device__ inline size_t aux_stride_stream(int Mc, int T) { return stream_planes(Mc, T) + (size_t)4 * Mc * stream_mp(Mc); }
+__host__ __device__ inline size_t exchange_floats(int Mc) { return (size_t)16 * stream_mp(Mc) + 4; }
+__host__ __device__ inline size_t aux_stride_stream(int Mc, int T) {
+    return stream_planes(Mc, T) + (size_t)4 * Mc * stream_mp(Mc) + exchange_floats(Mc);
+}
 struct AuxViewStream {
     float *F0, *F1, *BETA, *W0, *W1, *SR, *D, *Ac, *At;
     __device__ AuxViewStream(float *aux, int b, int Mc, int T) {
@@ -999,6 +1006,19 @@ struct AuxViewStream {
         At = Ac + (size_t)2 * Mc * stream_mp(Mc);
     }
 };
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+struct ExchangeView {
+    u32x4 *fcol, *bw;
+    int *flags;
+    __device__ ExchangeView(float *aux, int b, int Mc, int T) {
+        const int MP = stream_mp(Mc);
+        float *base = aux + (size_t)b * aux_stride_stream(Mc, T) + stream_planes(Mc, T) + (size_t)4 * Mc * MP;
+        fcol = reinterpret_cast<u32x4 *>(base);
+        bw = fcol + 2 * MP;
+        flags = reinterpret_cast<int *>(bw + 2 * MP);
+    }
+};
+constexpr int FLAG_FWD = 0, FLAG_BWD = 1;
 
 // The streaming sweeps give a node SL lanes (4, 8 or 16), each of which takes four consecutive entries of every chunk of
 // 4*SL, and handle NT/SL nodes per pass.  Fewer lanes per node mean fewer passes and reductions per column, more lanes
@@ -1123,7 +1143,10 @@ template <bool MATCH_LDS, int SL>
 __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
                                                                   const int64_t *__restrict__ out_len,
                                                                   const int64_t *__restrict__ tgt_len, float *__restrict__ S,
-                                                                  float *__restrict__ aux, int L, int T, int Mc, int MP) {
+                                                                  float *__restrict__ aux, int L, int T, int Mc, int MP,
+                                                                  int only_flagged) {
+    // only_flagged: run only for sentences whose cluster sweep gave up (the flag was written by an earlier launch)
+    if (only_flagged && ExchangeView(aux, blockIdx.x, Mc, T).flags[FLAG_FWD] == 0) return;
     extern __shared__ float smem[];
     float *col = smem;               // [2][MP]
     float *f1prev = smem + 2 * MP;    // [MP]
@@ -1252,7 +1275,8 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
 
 // Compact copies of the main-chain links for the streaming sweeps: Ac[k][a_id][c_id] = At[k][c_id][a_id] =
 // log2(e) * links[2*a_id+1][k][2*c_id+1] where a_id <= c_id < mc (k = 1 needs a_id >= 1), -inf everywhere else including the
-// padding columns up to MP.  One block per 32 x 32 tile of (parent, child) pairs, grid (MP/32, MP/32, B).
+// padding columns up to MP.  One block per 32 x 32 tile of (parent, child) pairs, grid (MP/32, MP/32, B).  The first block
+// of a sentence also zeroes its exchange area.
 __global__ __launch_bounds__(256) void compact_links_ml1_kernel(const float *__restrict__ links, const int64_t *__restrict__ out_len,
                                                                float *__restrict__ aux, int L, int T, int Mc, int MP) {
     __shared__ float tile[2][32][33];
@@ -1263,6 +1287,10 @@ __global__ __launch_bounds__(256) void compact_links_ml1_kernel(const float *__r
     const float *lk = links + (size_t)b * L * 2 * L;
     const int a0 = blockIdx.y * 32, c0 = blockIdx.x * 32;
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    if (blockIdx.x == 0 && blockIdx.y == 0) {  // empty exchange slots and lowered flags for the cluster sweeps
+        int *x = reinterpret_cast<int *>(ExchangeView(aux, b, Mc, T).fcol);
+        for (int i = threadIdx.x; i < (int)exchange_floats(Mc); i += 256) x[i] = 0;
+    }
     for (int r = ty; r < 32; r += 8) {
         const int a_id = a0 + r, c_id = c0 + tx;
         const bool ok = a_id < mc && c_id < mc && a_id <= c_id;
@@ -1291,7 +1319,9 @@ template <bool MATCH_LDS, int SL>
 __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *__restrict__ S, float *__restrict__ aux,
                                                                   const float *__restrict__ match_all,
                                                                   const int64_t *__restrict__ out_len,
-                                                                  const int64_t *__restrict__ tgt_len, int L, int T, int Mc, int MP) {
+                                                                  const int64_t *__restrict__ tgt_len, int L, int T, int Mc, int MP,
+                                                                  int only_flagged) {
+    if (only_flagged && ExchangeView(aux, blockIdx.x, Mc, T).flags[FLAG_BWD] == 0) return;
     extern __shared__ float smem[];
     float *w0 = smem;             // [2][MP]
     float *w1 = smem + 2 * MP;     // [2][MP]
@@ -1400,6 +1430,369 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
     }
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// Cluster sweeps (128 < Mc <= 512, batches of few sentences): CL = MP/NL workgroups of 16*NL threads share a sentence
+// (NL = 32 nodes each up to 256 nodes, 64 beyond).  Workgroup w owns the nodes a_id = CL*i + w (interleaved, so that the
+// triangular link rows are spread evenly), 16 lanes per node, and keeps their link rows in registers for the whole
+// sweep, NQ = MP/64 chunks of 64 entries, 4 per lane and chunk.  One
+// workgroup per sentence is bound by the instruction issue of one compute unit and by fetching the link rows from L2
+// for every column; a cluster divides both by CL and pays one exchange of the column through memory per target
+// position instead.
+//
+// Exchange: a node's entry travels as one 16-byte slot (tag, value, value, tag) - (tag, w0, w1, tag) in the outside
+// sweep - written and read with single device-scope 16-byte accesses, tag = (launch nonce << 12) | column, so that a
+// reader can tell a fresh entry from whatever the slot held before without any ordering between different slots; the
+// tag at both ends covers an access that the memory system splits into 8-byte halves.  Slots are laid out by workgroup,
+// [w][i] for node CL*i + w, so that the four nodes of a wave fill one 64-byte line with one store: entries of different
+// workgroups interleaved in a line make every store a partial write of a line that the others are polling.  The slots
+// alternate between two buffers; a workgroup can only publish column t-2 after it has seen all of column t-1, which
+// the others publish after reading column t, so two are enough.  Slots start out zero (compact_links_ml1_kernel) and
+// the nonce changes with every launch, so that neither an earlier call nor an earlier outside sweep over the same
+// tables can be mistaken for this one.
+//
+// The wait for a slot is bounded: after spin_limit polls (or when another workgroup of the sentence has given up) the
+// workgroup raises the sentence's flag and leaves; the one-workgroup streaming sweep, launched right behind with
+// only_flagged set, then redoes that sentence from scratch.  Workgroups are dispatched in index order and a cluster's
+// workgroups are adjacent, so this only happens when the device is shared with work that keeps them apart for long.
+// ------------------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void slot_store(u32x4 *p, unsigned tag, float a, float b) {
+    const u32x4 v = {tag, __float_as_uint(a), __float_as_uint(b), tag};
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ u32x4 slot_load(const u32x4 *p) {
+    u32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+// Waits for the entry tagged `tag`; false when the wait was given up.
+__device__ __forceinline__ bool poll_slot(const u32x4 *slot, unsigned tag, const int *flag, int spin_limit, u32x4 &x) {
+    for (int spins = 0;; spins++) {
+        x = slot_load(slot);
+        if (x.x == tag && x.w == tag) return true;
+        if (spins >= spin_limit || ((spins & 255) == 255 && __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0))
+            return false;
+    }
+}
+
+// stream_row_lse on link rows held in registers: chunks q in [qa, qb) of the NQ the lane holds (both wave-uniform).
+template <int NQ, bool JOINT>
+__device__ __forceinline__ void slab_row_lse(const float4 (&A0)[NQ], const float4 (&A1)[NQ], const float4 *u0, const float4 *u1, int qa,
+                                             int qb, bool live, bool has1, float g, float &out0, float &out1) {
+    g = is_finite(g) ? g : 0.f;
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+        if (q >= qa && q < qb) {
+            const float4 c0 = minus(u0[16 * q], g);
+            const float4 c1 = JOINT ? minus(u1[16 * q], g) : c0;
+            s0 += sum4_ex2(A0[q], c0);
+            s1 += sum4_ex2(A1[q], c1);
+        }
+    }
+    bool ok;
+    if (JOINT) {
+        const float tot = node_sum<16>(s0 + s1);
+        ok = tot >= 0x1p-90f && tot <= 0x1p100f;
+        out0 = g + lg2(tot);
+        out1 = out0;
+    } else {
+        const float t0 = node_sum<16>(s0), t1 = node_sum<16>(s1);
+        ok = t0 >= 0x1p-90f && t0 <= 0x1p100f && ((t1 >= 0x1p-90f && t1 <= 0x1p100f) || !has1);
+        out0 = g + lg2(t0);
+        out1 = has1 ? g + lg2(t1) : NEG_INF_F;
+    }
+    if (live && !ok) {  // uniform over the lanes of the node
+        RunningLse<16> a0, a1;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            if (q >= qa && q < qb) {
+                const float4 c0 = u0[16 * q];
+                const float4 c1 = JOINT ? u1[16 * q] : c0;
+                a0.add4(A0[q], c0);
+                a1.add4(A1[q], c1);
+            }
+        }
+        if (JOINT) {
+            a0.merge(a1);
+            out0 = out1 = a0.finish();
+        } else {
+            out0 = a0.finish();
+            out1 = a1.finish();
+        }
+    }
+}
+
+// Forward sweep of one cluster member.  Same tables as inside_fwd_ml1_stream_kernel.  Dynamic LDS (MATCH_LDS): the
+// emissions of the workgroup's 64 nodes, main [64][T] and leaf [64][T], so that the sweep itself waits for nothing
+// from memory but the exchange; without it they are requested one column ahead.
+template <int NQ, int NL, bool MATCH_LDS>
+__global__ __launch_bounds__(16 * NL) void inside_fwd_ml1_cluster_kernel(const float *__restrict__ match_all,
+                                                                   const int64_t *__restrict__ out_len,
+                                                                   const int64_t *__restrict__ tgt_len, float *__restrict__ S,
+                                                                   float *__restrict__ aux, int L, int T, int Mc, unsigned nonce,
+                                                                   int spin_limit) {
+    constexpr int MP = 64 * NQ, CL = MP / NL, NTC = 16 * NL;  // row length, workgroups per sentence, threads
+    __shared__ __attribute__((aligned(16))) float col[2][MP];
+    __shared__ __attribute__((aligned(16))) float slots[2][8];  // maxima of the column's 64-entry blocks
+    __shared__ int sm_dead;
+    extern __shared__ float sm_match[];
+    float *sm_main = sm_match, *sm_leaf = sm_match + NL * T;
+    const int b = blockIdx.x / CL, w = blockIdx.x % CL, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
+    // The column is collected by the last waves: they own the shortest link rows, are through with a column first and
+    // then sit waiting for the entries while the others still compute.
+    const int pidx = NTC - 1 - tid;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *mt = match_all + (size_t)b * L * T;
+    float *Sb = S + (size_t)b * Mc * (T + 2);
+    AuxViewStream av(aux, b, Mc, T);
+    ExchangeView xv(aux, b, Mc, T);
+    const int part = w * NTC + tid, nparts = CL * NTC;  // the sentence's element-wise work is split over the cluster
+
+    if (!lengths_ok(m, n, L, T)) {
+        for (int i = part; i < Mc * (T + 2); i += nparts) Sb[i] = (i == 0) ? __builtin_nanf("") : NEG_INF_F;
+        return;
+    }
+    const int mc = m / 2;
+    for (int i = part; i < Mc * (T + 2); i += nparts) {
+        const int a_id = i / (T + 2), s = i - a_id * (T + 2);
+        if (a_id >= mc || s >= n - 1) {
+            float v = NEG_INF_F;
+            if (a_id == mc - 1 && s == n - 1) v = sanitize(mt[(size_t)(m - 1) * T + (n - 1)]);
+            Sb[i] = v;
+            av.SR[i] = v * LOG2E_F;
+        }
+    }
+    const float base_cell = to_b2(mt[(size_t)(m - 1) * T + (n - 1)]);
+    if (tid < MP) {
+        col[(n - 1) & 1][tid] = (tid == mc - 1) ? base_cell : NEG_INF_F;
+        col[(n - 2) & 1][tid] = NEG_INF_F;
+    }
+    if (w == 0)
+        for (int i = tid; i < T + 4; i += NTC) av.D[i] = 0.f;
+    if (tid == 0) sm_dead = 0;
+    if (tid < 16) slots[tid >> 3][tid & 7] = (tid == 8 * ((n - 1) & 1)) ? base_cell : NEG_INF_F;
+
+    // this lane's node and its link rows (rows beyond the sentence: any valid row, the result is discarded)
+    const int a_id = CL * gidx + w;
+    const bool row_ok = a_id < mc;
+    const int ar = row_ok ? a_id : 0;
+    const int q0 = __builtin_amdgcn_readfirstlane((CL * 4 * (tid >> 6) + w) / 64);  // chunk of the wave's first node's diagonal
+    float4 A0[NQ], A1[NQ];
+    {
+        const float4 *r0 = reinterpret_cast<const float4 *>(av.Ac + ((size_t)0 * Mc + ar) * MP) + j;
+        const float4 *r1 = reinterpret_cast<const float4 *>(av.Ac + ((size_t)1 * Mc + ar) * MP) + j;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            A0[q] = r0[16 * q];
+            A1[q] = r1[16 * q];
+        }
+    }
+    const float *ra = mt + (size_t)(2 * ar + 1) * T, *rl = mt + (size_t)(2 * ar) * T;
+    if (MATCH_LDS) {
+        for (int i = tid; i < NL * T; i += NTC) {
+            const int g = i / T, s = i - g * T, node = CL * g + w;
+            const bool ok = node < mc && s < n;
+            sm_main[i] = ok ? to_b2(mt[(size_t)(2 * node + 1) * T + s]) : NEG_INF_F;
+            sm_leaf[i] = (ok && node >= 1) ? to_b2(mt[(size_t)(2 * node) * T + s]) : NEG_INF_F;
+        }
+        __syncthreads();
+    }
+    float ma_t = MATCH_LDS ? sm_main[gidx * T + n - 1] : to_b2(ra[n - 1]);                        // main[a][t]
+    float ma_p = MATCH_LDS ? sm_main[gidx * T + n - 2] : to_b2(ra[n - 2]);                        // main[a][t-1]
+    float ml_p = MATCH_LDS ? sm_leaf[gidx * T + n - 2] : (ar >= 1 ? to_b2(rl[n - 2]) : NEG_INF_F);  // leaf[a][t-1]
+    float f0g = NEG_INF_F, f1p = NEG_INF_F;                  // the node's F0, F1 one column earlier
+    // The link rows must have arrived before the sweep starts: a wait for them inside the loop would, from the second
+    // column on, be a wait for the stores of the column before.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+
+    double O = 0.0;  // offset of the column being read
+    for (int t = n - 1; t >= 1; t--) {
+        const float *cur = col[t & 1];
+        float *nxt = col[(t - 1) & 1];
+        const float D = max8(slots[t & 1]);
+        const float Ds = (D == NEG_INF_F) ? 0.f : D;
+        const double O_new = O + (double)Ds;
+        // the next column's emissions: from LDS, or requested now so that they travel during the column's work
+        float ma_raw = 0.f, ml_raw = 0.f;
+        if (t > 1) {
+            ma_raw = MATCH_LDS ? sm_main[gidx * T + t - 2] : ra[t - 2];
+            ml_raw = MATCH_LDS ? sm_leaf[gidx * T + t - 2] : rl[t - 2];
+        }
+        const float4 *cv = reinterpret_cast<const float4 *>(cur) + j;
+        float F0, F1;
+        slab_row_lse<NQ, false>(A0, A1, cv, cv, q0, NQ, row_ok, a_id >= 1, f0g, F0, F1);
+        F0 -= Ds;
+        F1 -= Ds;
+        float s_new = lse2_b2(ma_p + F0, (ml_p + ma_t) + (f1p - Ds));
+        if (!row_ok) s_new = NEG_INF_F;
+        f1p = F1;
+        f0g = F0;
+        const unsigned tag = (nonce << 12) | (unsigned)t;
+        if (j == 0 && row_ok && t > 1) slot_store(xv.fcol + ((t - 1) & 1) * MP + w * NL + gidx, tag, s_new, s_new);
+        if (t > 1 && pidx < MP) {  // whole waves; slot pidx belongs to node CL * (pidx % NL) + pidx / NL
+            const int node = CL * (pidx % NL) + pidx / NL;
+            float v = NEG_INF_F;
+            if (node < mc) {
+                u32x4 x;
+                if (poll_slot(xv.fcol + ((t - 1) & 1) * MP + pidx, tag, xv.flags + FLAG_FWD, spin_limit, x)) v = __uint_as_float(x.y);
+                else sm_dead = 1;
+            }
+            nxt[node] = v;
+            const float wm = wave_max(v + 0.f);
+            if ((tid & 63) == 0) slots[(t - 1) & 1][pidx >> 6] = wm;
+        }
+        // the table cells go out after the exchange, so that the wait for the entries is not also a wait for these stores
+        if (j == 0 && row_ok) {
+            Sb[(size_t)a_id * (T + 2) + (t - 1)] = (float)(((double)s_new + O_new) * LN2_D);
+            av.SR[(size_t)a_id * (T + 2) + (t - 1)] = s_new;
+            av.F0[(size_t)a_id * (T + 2) + t] = F0;
+            av.F1[(size_t)a_id * (T + 2) + t] = F1;
+        }
+        if (w == 0 && tid == 0) av.D[t] = Ds;
+        ma_t = ma_p;
+        ma_p = MATCH_LDS ? ma_raw : to_b2(ma_raw);
+        ml_p = MATCH_LDS ? ml_raw : (ar >= 1 ? to_b2(ml_raw) : NEG_INF_F);
+        O = O_new;
+        lds_barrier();
+        if (sm_dead) {  // uniform: written before the barrier
+            if (tid == 0) __hip_atomic_store(xv.flags + FLAG_FWD, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+    }
+}
+
+// Outside sweep of one cluster member.  Same tables as inside_bwd_ml1_stream_kernel.  Dynamic LDS: D [T+4], then
+// (MATCH_LDS) the emissions of the workgroup's NL nodes, main [NL][T] and leaf [NL][T].
+template <int NQ, int NL, bool MATCH_LDS>
+__global__ __launch_bounds__(16 * NL) void inside_bwd_ml1_cluster_kernel(const float *__restrict__ S, float *__restrict__ aux,
+                                                                   const float *__restrict__ match_all,
+                                                                   const int64_t *__restrict__ out_len,
+                                                                   const int64_t *__restrict__ tgt_len, int L, int T, int Mc,
+                                                                   unsigned nonce, int spin_limit) {
+    constexpr int MP = 64 * NQ, CL = MP / NL, NTC = 16 * NL;  // row length, workgroups per sentence, threads
+    __shared__ __attribute__((aligned(16))) float w0[2][MP];
+    __shared__ __attribute__((aligned(16))) float w1[2][MP];
+    __shared__ int sm_dead;
+    extern __shared__ float sm_D[];  // [T+4]
+    float *sm_main = sm_D + (T + 4), *sm_leaf = sm_main + NL * T;
+    const int b = blockIdx.x / CL, w = blockIdx.x % CL, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *mt = match_all + (size_t)b * L * T;
+    const float *Sb = S + (size_t)b * Mc * (T + 2);
+    AuxViewStream av(aux, b, Mc, T);
+    ExchangeView xv(aux, b, Mc, T);
+    const float ll = Sb[0];
+    const bool valid = lengths_ok(m, n, L, T) && (ll == ll) && (fabsf(ll) != __builtin_huge_valf());
+    if (!valid) return;  // the posterior kernels write zeros for such sentences
+    const int mc = m / 2;
+    for (int i = tid; i < T + 4; i += NTC) sm_D[i] = av.D[i];
+    if (tid == 0) sm_dead = 0;
+    if (MATCH_LDS) {
+        for (int i = tid; i < NL * T; i += NTC) {
+            const int g = i / T, s = i - g * T, node = CL * g + w;
+            const bool ok = node < mc && s < n;
+            sm_main[i] = ok ? to_b2(mt[(size_t)(2 * node + 1) * T + s]) : NEG_INF_F;
+            sm_leaf[i] = (ok && node >= 1) ? to_b2(mt[(size_t)(2 * node) * T + s]) : NEG_INF_F;
+        }
+    }
+
+    // this lane's node and its transposed link rows: parents a <= c, chunks [0, q1)
+    const int c_id = CL * gidx + w;
+    const bool live = c_id < mc;
+    const int ci = live ? c_id : 0;
+    const int q1 = min(__builtin_amdgcn_readfirstlane((CL * (4 * (tid >> 6) + 3) + w) / 64), NQ - 1) + 1;  // the wave's last node
+    float4 A0[NQ], A1[NQ];
+    {
+        const float4 *r0 = reinterpret_cast<const float4 *>(av.At + ((size_t)0 * Mc + ci) * MP) + j;
+        const float4 *r1 = reinterpret_cast<const float4 *>(av.At + ((size_t)1 * Mc + ci) * MP) + j;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            A0[q] = r0[16 * q];
+            A1[q] = r1[16 * q];
+        }
+    }
+    const float *ra = mt + (size_t)(2 * ci + 1) * T, *rl = mt + (size_t)(2 * ci) * T;
+    __syncthreads();  // sm_D
+    const float beta00 = -av.SR[0];  // relative to the offset of column 0
+    const float w00 = (to_b2(mt[(size_t)1 * T]) + beta00) - sm_D[1];
+    if (tid < MP) {
+        w0[1][tid] = (tid == 0) ? w00 : NEG_INF_F;
+        w1[1][tid] = NEG_INF_F;
+        w0[0][tid] = NEG_INF_F;
+        w1[0][tid] = NEG_INF_F;
+    }
+    float bp = (c_id == 0) ? beta00 : NEG_INF_F;  // the node's outside score one column earlier
+    if (j == 0 && live) {
+        av.BETA[(size_t)c_id * (T + 2)] = bp;
+        av.W0[(size_t)c_id * (T + 2) + 1] = (c_id == 0) ? w00 : NEG_INF_F;
+        av.W1[(size_t)c_id * (T + 2) + 1] = NEG_INF_F;
+    }
+    float mc_t, ml_p;  // main[c][t], leaf[c][t-1]
+    if (MATCH_LDS) {
+        mc_t = sm_main[gidx * T + 1];
+        ml_p = sm_leaf[gidx * T];
+    } else {
+        mc_t = live ? to_b2(ra[1]) : NEG_INF_F;
+        ml_p = (live && ci >= 1) ? to_b2(rl[0]) : NEG_INF_F;
+    }
+    // The link rows must have arrived before the sweep starts: a wait for them inside the loop would, from the second
+    // column on, be a wait for the stores of the column before.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+
+    for (int t = 1; t <= n - 1; t++) {
+        const float *c0 = w0[t & 1], *c1 = w1[t & 1];
+        float *n0 = w0[(t + 1) & 1], *n1 = w1[(t + 1) & 1];
+        const float d_next = sm_D[t + 1], d_both = d_next + sm_D[t];
+        const bool more = t < n - 1;
+        float mc_raw = 0.f, ml_raw = 0.f;
+        if (more) {
+            mc_raw = MATCH_LDS ? sm_main[gidx * T + t + 1] : ra[t + 1];
+            ml_raw = MATCH_LDS ? sm_leaf[gidx * T + t] : rl[t];
+        }
+        const float4 *u0 = reinterpret_cast<const float4 *>(c0) + j, *u1 = reinterpret_cast<const float4 *>(c1) + j;
+        float beta, unused;
+        slab_row_lse<NQ, true>(A0, A1, u0, u1, 0, q1, live, true, bp, beta, unused);
+        if (!live) beta = NEG_INF_F;
+        const float nw0 = (mc_t + beta) - d_next;
+        const float nw1 = ((ml_p + mc_t) + bp) - d_both;
+        const unsigned tag = (nonce << 12) | (unsigned)(t + 1);
+        if (j == 0 && live && more) slot_store(xv.bw + ((t + 1) & 1) * MP + w * NL + gidx, tag, nw0, nw1);
+        // collected by the first waves, whose nodes have the fewest parents
+        if (more) {
+            for (int i = tid; i < MP; i += NTC) {  // slot i belongs to node CL * (i % NL) + i / NL
+                const int node = CL * (i % NL) + i / NL;
+                float v0 = NEG_INF_F, v1 = NEG_INF_F;
+                if (node < mc) {
+                    u32x4 x;
+                    if (poll_slot(xv.bw + ((t + 1) & 1) * MP + i, tag, xv.flags + FLAG_BWD, spin_limit, x)) {
+                        v0 = __uint_as_float(x.y);
+                        v1 = __uint_as_float(x.z);
+                    } else {
+                        sm_dead = 1;
+                    }
+                }
+                n0[node] = v0;
+                n1[node] = v1;
+            }
+        }
+        if (j == 0 && live) {  // after the exchange, so that the wait for the entries is not also a wait for these stores
+            av.BETA[(size_t)c_id * (T + 2) + t] = beta;
+            av.W0[(size_t)c_id * (T + 2) + t + 1] = nw0;
+            av.W1[(size_t)c_id * (T + 2) + t + 1] = nw1;
+        }
+        bp = beta;
+        mc_t = MATCH_LDS ? mc_raw : (live ? to_b2(mc_raw) : NEG_INF_F);
+        ml_p = MATCH_LDS ? ml_raw : ((live && ci >= 1) ? to_b2(ml_raw) : NEG_INF_F);
+        lds_barrier();
+        if (sm_dead) {  // uniform: written before the barrier
+            if (tid == 0) __hip_atomic_store(xv.flags + FLAG_BWD, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+    }
+}
+
 // Rule posteriors from the outside weights: lg[a][k][c] = g * sum_{t=1}^{n-1} exp(links[a][k][c] + Wk[a][t] + R[c][t]).
 // One block per 32x32 tile of (parent, child) pairs; the slab has been zero-filled beforehand.
 __global__ __launch_bounds__(1024) void links_grad_ml1_stream_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
@@ -1504,21 +1897,84 @@ __global__ __launch_bounds__(256) void criterion_loss_kernel(const float *__rest
     criterion_loss_block<256>(LossTask{S, tgt_len, out, B, (int64_t)Mc * (T + 2)});
 }
 
+// Cluster sweeps are used when all their workgroups fit on the device together (two per compute unit).  Both numbers can
+// be changed through pcfgnat_cluster_config.
+std::atomic<int> g_cluster_max_wg{512}, g_cluster_spin_limit{1 << 20};
+std::atomic<unsigned> g_cluster_nonce{0};
+unsigned next_nonce() { return g_cluster_nonce.fetch_add(1) % 0xFFFFFu + 1u; }  // 1 .. 2^20 - 1: tags are never zero
+struct ClusterShape {
+    int NQ, NL, CL;  // chunks of 64 per link row, nodes per workgroup, workgroups per sentence; CL = 0: not applicable
+};
+ClusterShape cluster_shape(int B, int T, int Mc) {
+    const int NQ = stream_mp(Mc) / 64, NL = NQ <= 4 ? 32 : 64, CL = 64 * NQ / NL;
+    const bool ok = NQ >= 3 && NQ <= 8 && T + 2 < 4096 && (int64_t)B * CL <= g_cluster_max_wg.load();
+    return ClusterShape{NQ, NL, ok ? CL : 0};
+}
+
+template <int NQ, int NL>
+int launch_fwd_cluster(const float *match_all, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B, int L, int T, int Mc,
+                       hipStream_t stream) {
+    constexpr int CL = 64 * NQ / NL, NTC = 16 * NL;
+    const size_t match_bytes = (size_t)2 * NL * T * sizeof(float);
+    if (match_bytes <= LDS_BUDGET - 8192) {
+        auto k = inside_fwd_ml1_cluster_kernel<NQ, NL, true>;
+        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)match_bytes));
+        hipLaunchKernelGGL(k, dim3(B * CL), dim3(NTC), match_bytes, stream, match_all, ol, tl, S, aux, L, T, Mc, next_nonce(),
+                           g_cluster_spin_limit.load());
+    } else {
+        hipLaunchKernelGGL((inside_fwd_ml1_cluster_kernel<NQ, NL, false>), dim3(B * CL), dim3(NTC), 0, stream, match_all, ol, tl, S, aux,
+                           L, T, Mc, next_nonce(), g_cluster_spin_limit.load());
+    }
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+template <int NQ, int NL>
+int launch_bwd_cluster(const float *S, float *aux, const float *match_all, const int64_t *ol, const int64_t *tl, int B, int L, int T,
+                       int Mc, hipStream_t stream) {
+    constexpr int CL = 64 * NQ / NL, NTC = 16 * NL;
+    const size_t base = (size_t)(T + 4) * sizeof(float), with_match = base + (size_t)2 * NL * T * sizeof(float);
+    if (with_match <= LDS_BUDGET - 8192) {
+        auto k = inside_bwd_ml1_cluster_kernel<NQ, NL, true>;
+        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_match));
+        hipLaunchKernelGGL(k, dim3(B * CL), dim3(NTC), with_match, stream, S, aux, match_all, ol, tl, L, T, Mc, next_nonce(),
+                           g_cluster_spin_limit.load());
+    } else {
+        hipLaunchKernelGGL((inside_bwd_ml1_cluster_kernel<NQ, NL, false>), dim3(B * CL), dim3(NTC), base, stream, S, aux, match_all, ol,
+                           tl, L, T, Mc, next_nonce(), g_cluster_spin_limit.load());
+    }
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
+
 int launch_fwd_stream(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B,
                       int L, int T, int Mc, hipStream_t stream) {
     const int MP = stream_mp(Mc);
     PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss: aux must be 16-byte aligned");
     hipLaunchKernelGGL(compact_links_ml1_kernel, dim3(MP / 32, MP / 32, B), dim3(256), 0, stream, links, ol, aux, L, T, Mc, MP);
     PCFGNAT_HIP_CHECK(hipGetLastError());
+    // cluster sweep first where it applies; the one-workgroup sweep then only redoes sentences whose cluster gave up
+    const ClusterShape cs = cluster_shape(B, T, Mc);
+    int rc = PCFGNAT_OK;
+    switch (cs.CL ? cs.NQ : 0) {
+        case 3: rc = launch_fwd_cluster<3, 32>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
+        case 4: rc = launch_fwd_cluster<4, 32>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
+        case 5: rc = launch_fwd_cluster<5, 64>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
+        case 6: rc = launch_fwd_cluster<6, 64>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
+        case 7: rc = launch_fwd_cluster<7, 64>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
+        case 8: rc = launch_fwd_cluster<8, 64>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
+        default: break;
+    }
+    if (rc != PCFGNAT_OK) return rc;
+    const int only_flagged = cs.CL != 0;
     const size_t base = ((size_t)4 * MP + 32) * sizeof(float);
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
     if (with_match <= LDS_BUDGET) {
         auto k = inside_fwd_ml1_stream_kernel<true, 4>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_match));
-        hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_match, stream, match_all, links, ol, tl, S, aux, L, T, Mc, MP);
+        hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_match, stream, match_all, links, ol, tl, S, aux, L, T, Mc, MP, only_flagged);
     } else {
         hipLaunchKernelGGL((inside_fwd_ml1_stream_kernel<false, 4>), dim3(B), dim3(NT), base, stream, match_all, links, ol, tl, S, aux, L,
-                           T, Mc, MP);
+                           T, Mc, MP, only_flagged);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
@@ -1531,14 +1987,27 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
     PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss_backward: aux must be 16-byte aligned");
     const size_t base = ((size_t)5 * MP + T + 4) * sizeof(float);
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
+    const ClusterShape cs = cluster_shape(B, T, Mc);
+    int rc = PCFGNAT_OK;
+    switch (cs.CL ? cs.NQ : 0) {
+        case 3: rc = launch_bwd_cluster<3, 32>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
+        case 4: rc = launch_bwd_cluster<4, 32>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
+        case 5: rc = launch_bwd_cluster<5, 64>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
+        case 6: rc = launch_bwd_cluster<6, 64>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
+        case 7: rc = launch_bwd_cluster<7, 64>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
+        case 8: rc = launch_bwd_cluster<8, 64>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
+        default: break;
+    }
+    if (rc != PCFGNAT_OK) return rc;
+    const int only_flagged = cs.CL != 0;
     // lanes per node: four while one pass covers all nodes; beyond that the outside sweep measured faster with eight
     if (with_match <= LDS_BUDGET) {
         auto k = Mc <= NT / 4 ? inside_bwd_ml1_stream_kernel<true, 4> : inside_bwd_ml1_stream_kernel<true, 8>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_match));
-        hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_match, stream, S, aux, match_all, ol, tl, L, T, Mc, MP);
+        hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_match, stream, S, aux, match_all, ol, tl, L, T, Mc, MP, only_flagged);
     } else {
         auto k = Mc <= NT / 4 ? inside_bwd_ml1_stream_kernel<false, 4> : inside_bwd_ml1_stream_kernel<false, 8>;
-        hipLaunchKernelGGL(k, dim3(B), dim3(NT), base, stream, S, aux, match_all, ol, tl, L, T, Mc, MP);
+        hipLaunchKernelGGL(k, dim3(B), dim3(NT), base, stream, S, aux, match_all, ol, tl, L, T, Mc, MP, only_flagged);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     const size_t nlg = (size_t)B * L * 2 * L;
@@ -1619,6 +2088,11 @@ int check_dims(const char *who, int64_t B, int64_t L, int64_t T, int64_t ml) {
 }  // namespace pcfgnat
 
 using namespace pcfgnat;
+
+extern "C" void pcfgnat_cluster_config(int max_workgroups, int spin_limit) {
+    if (max_workgroups >= 0) g_cluster_max_wg.store(max_workgroups);
+    if (spin_limit >= 0) g_cluster_spin_limit.store(spin_limit);
+}
 
 extern "C" size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml) {
     if (B <= 0 || L < 2 || T < 0 || ml < 0) return 0;

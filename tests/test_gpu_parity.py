@@ -237,6 +237,41 @@ def test_inside_forward_backward_vs_oracle(case):
             assert not mg_got[bi].any() and not lg_got[bi].any()
 
 
+def _inside_all(batch, match):
+    md = match.to(DEV).requires_grad_(True)
+    ld = batch["links"].to(DEV).requires_grad_(True)
+    ll = ops.cuda_pcfg_loss(md, ld, batch["output_length"].to(DEV), batch["target_length"].to(DEV))
+    w = torch.linspace(0.5, 1.5, ll.numel(), device=DEV)
+    (ll.masked_fill(~torch.isfinite(ll), 0) * w).sum().backward()
+    return ll.detach().cpu(), md.grad.cpu(), ld.grad.cpu()
+
+
+@pytest.mark.parametrize("mode", ["one_workgroup", "clusters_give_up"])
+@pytest.mark.parametrize("L,T,ms,ns", [(320, 40, [320, 262, 4], [40, 31, 2]), (512, 140, [512, 444], [140, 120]),
+                                       (600, 24, [600, 520], [24, 24]), (1024, 30, [1024, 770, 900], [30, 22, 30])])
+def test_long_graph_sweeps_agree(mode, L, T, ms, ns):
+    """Graphs of 258..1026 nodes: the cluster sweeps (default for small batches), the one-workgroup streaming sweeps
+    (clusters switched off) and the redo path (clusters that give up at once: spin limit 0) compute the same tables; the
+    default path is compared with the oracle in test_inside_forward_backward_vs_oracle."""
+    batch = synth.training_batch(len(ms), L, T, 60, ms, ns, seed=L + T)
+    match = _match_for(batch)
+    ll0, mg0, lg0 = _inside_all(batch, match)
+    try:
+        if mode == "one_workgroup":
+            ops.cluster_config(max_workgroups=0)
+        else:
+            ops.cluster_config(spin_limit=0)
+        ll1, mg1, lg1 = _inside_all(batch, match)
+    finally:
+        ops.cluster_config(max_workgroups=512, spin_limit=1 << 20)
+    fin = torch.isfinite(ll0)
+    assert fin.any() and torch.equal(fin, torch.isfinite(ll1))
+    assert torch.allclose(ll0[fin], ll1[fin], rtol=1e-5)
+    for b in range(len(ms)):
+        for g0, g1 in ((mg0[b], mg1[b]), (lg0[b], lg1[b])):
+            assert (g0 - g1).abs().max() <= 1e-4 * max(g0.abs().max().item(), 1e-30)
+
+
 @pytest.mark.parametrize("L,T,ms,ns", [(128, 30, [128, 90], [30, 22]), (320, 40, [320, 262], [40, 31]), (600, 24, [600, 520], [24, 24])])
 def test_inside_spiky_inputs_vs_oracle(L, T, ms, ns):
     """Emissions and links with jumps of hundreds of units and scattered -inf entries: neighbouring columns of the tables
