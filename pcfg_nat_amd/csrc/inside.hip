@@ -13,10 +13,10 @@
 //
 // Design (latency-bound, one workgroup of 1024 threads per sentence): the sentence's compact link matrices live in
 // registers for the whole sweep (one 16-lane DPP row per node, lanes strided over the other index), the current
-// column of S (or of the outside weights) is exchanged through LDS, one workgroup barrier per target position,
-// no global atomics or inter-workgroup spinning.  The forward leaves F0/F1 behind so that the backward needs a
-// single sweep: rule posteriors are accumulated in registers, emission posteriors come from an element-wise
-// epilogue.
+// column of S (or of the outside weights) is exchanged through LDS, one workgroup barrier per target position.
+// The forward leaves F0/F1 behind so that the backward needs a single sweep: rule posteriors are accumulated in
+// registers, emission posteriors come from an element-wise epilogue.  Graphs of more than 256 nodes use the streaming
+// or the pipelined sweeps further down (link rows from L2, or spread over several workgroups per sentence).
 #include "common.hip.h"
 
 #include <atomic>
@@ -981,14 +981,16 @@ __global__ __launch_bounds__(BT_NT) void best_tree_ml1_kernel(const float *__res
 // masked entries already -inf and rows padded to MP = 64*ceil(Mc/64) floats:
 // Ac [2][Mc][MP] by parent (Ac[k][a][c]) for the forward sweep and At [2][Mc][MP] by child (At[k][c][a]) for the
 // outside sweep, so that the sweeps stream them with unconditional 16-byte loads.  Last comes the exchange area of the
-// cluster sweeps (below): tagged 16-byte slots, forward column [2][MP] and outside weights [2][MP], and four ints
-// (forward gave up, outside sweep gave up, two unused).
+// pipelined sweeps (below): the forward columns as doubles [T+2][MP], the outside weights [T+2][2][MP], the shifts every
+// block of 16 nodes chose [MP/16][T+4], and four ints (forward gave up, outside sweep gave up, two unused).
 // ------------------------------------------------------------------------------------------------------------
 __host__ __device__ inline int stream_mp(int Mc) { return ((Mc + 63) / 64) * 64; }
 __host__ __device__ inline size_t stream_planes(int Mc, int T) { return (((size_t)6 * Mc * (T + 2) + (size_t)(T + 4)) + 3) & ~(size_t)3; }
-__host__ __device__ inline size_t exchange_floats(int Mc) { return (size_t)16 * stream_mp(Mc) + 4; }
+__host__ __device__ inline size_t exchange_floats(int Mc, int T) {
+    return (size_t)4 * stream_mp(Mc) * (T + 2) + (size_t)(stream_mp(Mc) / 16) * (T + 4) + 4;
+}
 __host__ __device__ inline size_t aux_stride_stream(int Mc, int T) {
-    return stream_planes(Mc, T) + (size_t)4 * Mc * stream_mp(Mc) + exchange_floats(Mc);
+    return stream_planes(Mc, T) + (size_t)4 * Mc * stream_mp(Mc) + exchange_floats(Mc, T);
 }
 struct AuxViewStream {
     float *F0, *F1, *BETA, *W0, *W1, *SR, *D, *Ac, *At;
@@ -1006,16 +1008,18 @@ struct AuxViewStream {
         At = Ac + (size_t)2 * Mc * stream_mp(Mc);
     }
 };
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 struct ExchangeView {
-    u32x4 *fcol, *bw;
+    unsigned long long *fcol;  // [T+2][MP]
+    unsigned *bw;              // [T+2][2][MP]
+    float *shifts;             // [MP/16][T+4]
     int *flags;
     __device__ ExchangeView(float *aux, int b, int Mc, int T) {
         const int MP = stream_mp(Mc);
         float *base = aux + (size_t)b * aux_stride_stream(Mc, T) + stream_planes(Mc, T) + (size_t)4 * Mc * MP;
-        fcol = reinterpret_cast<u32x4 *>(base);
-        bw = fcol + 2 * MP;
-        flags = reinterpret_cast<int *>(bw + 2 * MP);
+        fcol = reinterpret_cast<unsigned long long *>(base);
+        bw = reinterpret_cast<unsigned *>(base + (size_t)2 * MP * (T + 2));
+        shifts = base + (size_t)4 * MP * (T + 2);
+        flags = reinterpret_cast<int *>(shifts + (size_t)(MP / 16) * (T + 4));
     }
 };
 constexpr int FLAG_FWD = 0, FLAG_BWD = 1;
@@ -1145,7 +1149,7 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
                                                                   const int64_t *__restrict__ tgt_len, float *__restrict__ S,
                                                                   float *__restrict__ aux, int L, int T, int Mc, int MP,
                                                                   int only_flagged) {
-    // only_flagged: run only for sentences whose cluster sweep gave up (the flag was written by an earlier launch)
+    // only_flagged: run only for sentences whose pipelined sweep gave up (the flag was written by an earlier launch)
     if (only_flagged && ExchangeView(aux, blockIdx.x, Mc, T).flags[FLAG_FWD] == 0) return;
     extern __shared__ float smem[];
     float *col = smem;               // [2][MP]
@@ -1275,8 +1279,8 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
 
 // Compact copies of the main-chain links for the streaming sweeps: Ac[k][a_id][c_id] = At[k][c_id][a_id] =
 // log2(e) * links[2*a_id+1][k][2*c_id+1] where a_id <= c_id < mc (k = 1 needs a_id >= 1), -inf everywhere else including the
-// padding columns up to MP.  One block per 32 x 32 tile of (parent, child) pairs, grid (MP/32, MP/32, B).  The first block
-// of a sentence also zeroes its exchange area.
+// padding columns up to MP.  One block per 32 x 32 tile of (parent, child) pairs, grid (MP/32, MP/32, B).  The blocks of a
+// sentence also share the filling of its exchange tables.
 __global__ __launch_bounds__(256) void compact_links_ml1_kernel(const float *__restrict__ links, const int64_t *__restrict__ out_len,
                                                                float *__restrict__ aux, int L, int T, int Mc, int MP) {
     __shared__ float tile[2][32][33];
@@ -1287,9 +1291,13 @@ __global__ __launch_bounds__(256) void compact_links_ml1_kernel(const float *__r
     const float *lk = links + (size_t)b * L * 2 * L;
     const int a0 = blockIdx.y * 32, c0 = blockIdx.x * 32;
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
-    if (blockIdx.x == 0 && blockIdx.y == 0) {  // empty exchange slots and lowered flags for the cluster sweeps
-        int *x = reinterpret_cast<int *>(ExchangeView(aux, b, Mc, T).fcol);
-        for (int i = threadIdx.x; i < (int)exchange_floats(Mc); i += 256) x[i] = 0;
+    {   // the exchange tables of the pipelined sweeps start out empty (all ones), their flags lowered
+        ExchangeView xv(aux, b, Mc, T);
+        unsigned *x = reinterpret_cast<unsigned *>(xv.fcol);
+        const size_t words = (size_t)4 * MP * (T + 2);
+        const size_t nthreads = (size_t)gridDim.x * gridDim.y * 256, me = ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
+        for (size_t i = me; i < words; i += nthreads) x[i] = 0xFFFFFFFFu;
+        if (me < 4) xv.flags[me] = 0;
     }
     for (int r = ty; r < 32; r += 8) {
         const int a_id = a0 + r, c_id = c0 + tx;
@@ -1431,48 +1439,52 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
 }
 
 // ------------------------------------------------------------------------------------------------------------
-// Cluster sweeps (128 < Mc <= 512, batches of few sentences): CL = MP/NL workgroups of 16*NL threads share a sentence
-// (NL = 32 nodes each up to 256 nodes, 64 beyond).  Workgroup w owns the nodes a_id = CL*i + w (interleaved, so that the
-// triangular link rows are spread evenly), 16 lanes per node, and keeps their link rows in registers for the whole
-// sweep, NQ = MP/64 chunks of 64 entries, 4 per lane and chunk.  One
-// workgroup per sentence is bound by the instruction issue of one compute unit and by fetching the link rows from L2
-// for every column; a cluster divides both by CL and pays one exchange of the column through memory per target
-// position instead.
+// Pipelined sweeps (128 < Mc <= 512, batches of few sentences): a sentence's nodes are cut into blocks of 16, one
+// workgroup per block: four compute waves (16 lanes per node, the node's two link rows in registers for the whole sweep,
+// NQ = MP/64 float4 per lane and plane) and one collector wave.  One workgroup per sentence is bound by the instruction
+// issue of one compute unit and by fetching the link rows from L2 for every column; here every block has a compute
+// unit of its own.
 //
-// Exchange: a node's entry travels as one 16-byte slot (tag, value, value, tag) - (tag, w0, w1, tag) in the outside
-// sweep - written and read with single device-scope 16-byte accesses, tag = (launch nonce << 12) | column, so that a
-// reader can tell a fresh entry from whatever the slot held before without any ordering between different slots; the
-// tag at both ends covers an access that the memory system splits into 8-byte halves.  Slots are laid out by workgroup,
-// [w][i] for node CL*i + w, so that the four nodes of a wave fill one 64-byte line with one store: entries of different
-// workgroups interleaved in a line make every store a partial write of a line that the others are polling.  The slots
-// alternate between two buffers; a workgroup can only publish column t-2 after it has seen all of column t-1, which
-// the others publish after reading column t, so two are enough.  Slots start out zero (compact_links_ml1_kernel) and
-// the nonce changes with every launch, so that neither an earlier call nor an earlier outside sweep over the same
-// tables can be mistaken for this one.
+// The link matrices are triangular - a node combines children c >= a only - so block k of the forward sweep needs
+// the column entries of the blocks above it and nothing from below: the top block runs free, and every other block
+// follows the one above at the distance of one exchange through memory.  That latency (about a microsecond) is paid
+// once per block as a skew of the pipeline, not once per column as it would be if all blocks advanced in lock step.
+// The outside sweep (parents a <= c) runs the same way with the lowest block leading.
 //
-// The wait for a slot is bounded: after spin_limit polls (or when another workgroup of the sentence has given up) the
-// workgroup raises the sentence's flag and leaves; the one-workgroup streaming sweep, launched right behind with
-// only_flagged set, then redoes that sentence from scratch.  Workgroups are dispatched in index order and a cluster's
-// workgroups are adjacent, so this only happens when the device is shared with work that keeps them apart for long.
+// Exchange: one table entry per (column, node), written once per launch with a device-scope store by the owner and read
+// with device-scope loads by the collector waves of the blocks that follow; compact_links_ml1_kernel fills the tables
+// with an impossible bit pattern (all ones) first, which marks an entry that has not arrived.  The collector works one
+// column ahead of the compute waves (the two meet at the one LDS barrier per column), so an entry that is already
+// there costs the compute waves nothing.
+//
+// Column offsets: a block sees only its own and the leading blocks' part of a column, so every block chooses its own
+// shifts (maximum of what it saw of the previous column) and keeps its own offsets; what it publishes in the forward
+// sweep are absolute values (offset added, as doubles), which the readers bring to their own offsets.  The tables a
+// block leaves behind (R, F0h, F1h) are relative to its own offsets; pipeline_rebase_kernel then moves them to the
+// offsets of block 0, which saw every column whole and whose shifts are the ones stored in D.  The outside sweep works
+// on those common offsets throughout.
+//
+// The wait for an entry is bounded: after spin_limit rounds of polling (or when another block of the sentence has
+// given up) the block raises the sentence's flag and leaves; the one-workgroup streaming sweep, launched right behind
+// with only_flagged set, then redoes that sentence from scratch.  Leading blocks have the lower workgroup indices, so
+// that with in-order dispatch a block never waits for one that has not been started.
 // ------------------------------------------------------------------------------------------------------------
-__device__ __forceinline__ void slot_store(u32x4 *p, unsigned tag, float a, float b) {
-    const u32x4 v = {tag, __float_as_uint(a), __float_as_uint(b), tag};
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+constexpr int NLP = 16;             // nodes per block
+constexpr int NTP = 16 * NLP + 64;  // four compute waves and the collector wave
+constexpr unsigned EMPTY32 = 0xFFFFFFFFu;
+constexpr unsigned long long EMPTY64 = ~0ull;
+
+__device__ __forceinline__ unsigned long long entry_load(const unsigned long long *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ u32x4 slot_load(const u32x4 *p) {
-    u32x4 v;
-    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
-    return v;
+__device__ __forceinline__ unsigned entry_load(const unsigned *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void entry_store(unsigned long long *p, double v) {
+    __hip_atomic_store(p, (unsigned long long)__double_as_longlong(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// Waits for the entry tagged `tag`; false when the wait was given up.
-__device__ __forceinline__ bool poll_slot(const u32x4 *slot, unsigned tag, const int *flag, int spin_limit, u32x4 &x) {
-    for (int spins = 0;; spins++) {
-        x = slot_load(slot);
-        if (x.x == tag && x.w == tag) return true;
-        if (spins >= spin_limit || ((spins & 255) == 255 && __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0))
-            return false;
-    }
+__device__ __forceinline__ void entry_store(unsigned *p, float v) {
+    __hip_atomic_store(p, __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ bool gave_up(const int *flag) { return __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0; }
 
 // stream_row_lse on link rows held in registers: chunks q in [qa, qb) of the NQ the lane holds (both wave-uniform).
 template <int NQ, bool JOINT>
@@ -1522,31 +1534,29 @@ __device__ __forceinline__ void slab_row_lse(const float4 (&A0)[NQ], const float
     }
 }
 
-// Forward sweep of one cluster member.  Same tables as inside_fwd_ml1_stream_kernel.  Dynamic LDS (MATCH_LDS): the
-// emissions of the workgroup's 64 nodes, main [64][T] and leaf [64][T], so that the sweep itself waits for nothing
-// from memory but the exchange; without it they are requested one column ahead.
-template <int NQ, int NL, bool MATCH_LDS>
-__global__ __launch_bounds__(16 * NL) void inside_fwd_ml1_cluster_kernel(const float *__restrict__ match_all,
-                                                                   const int64_t *__restrict__ out_len,
-                                                                   const int64_t *__restrict__ tgt_len, float *__restrict__ S,
-                                                                   float *__restrict__ aux, int L, int T, int Mc, unsigned nonce,
-                                                                   int spin_limit) {
-    constexpr int MP = 64 * NQ, CL = MP / NL, NTC = 16 * NL;  // row length, workgroups per sentence, threads
+// Forward sweep of one block.  Same tables as inside_fwd_ml1_stream_kernel, relative to the block's own offsets (see
+// above).  Dynamic LDS (MATCH_LDS): the emissions of the block's nodes, main [NLP][T] and leaf [NLP][T]; without it they
+// are requested one column ahead.
+template <int NQ, bool MATCH_LDS>
+__global__ __launch_bounds__(NTP) void inside_fwd_ml1_pipe_kernel(const float *__restrict__ match_all,
+                                                                 const int64_t *__restrict__ out_len,
+                                                                 const int64_t *__restrict__ tgt_len, float *__restrict__ S,
+                                                                 float *__restrict__ aux, int L, int T, int Mc, int spin_limit) {
+    constexpr int MP = 64 * NQ, CL = MP / NLP;
     __shared__ __attribute__((aligned(16))) float col[2][MP];
-    __shared__ __attribute__((aligned(16))) float slots[2][8];  // maxima of the column's 64-entry blocks
+    __shared__ float sm_Dv[2];  // shift of the step that reads column t: maximum of the visible part of column t+1
     __shared__ int sm_dead;
     extern __shared__ float sm_match[];
-    float *sm_main = sm_match, *sm_leaf = sm_match + NL * T;
-    const int b = blockIdx.x / CL, w = blockIdx.x % CL, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
-    // The column is collected by the last waves: they own the shortest link rows, are through with a column first and
-    // then sit waiting for the entries while the others still compute.
-    const int pidx = NTC - 1 - tid;
+    float *sm_main = sm_match, *sm_leaf = sm_match + NLP * T;
+    const int b = blockIdx.x / CL, k = CL - 1 - blockIdx.x % CL;  // the leading (highest) block first
+    const int tid = threadIdx.x, gidx = (tid >> 4) & (NLP - 1), j = tid & 15, lane = tid & 63;
+    const bool collector = tid >= 16 * NLP;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const float *mt = match_all + (size_t)b * L * T;
     float *Sb = S + (size_t)b * Mc * (T + 2);
     AuxViewStream av(aux, b, Mc, T);
     ExchangeView xv(aux, b, Mc, T);
-    const int part = w * NTC + tid, nparts = CL * NTC;  // the sentence's element-wise work is split over the cluster
+    const int part = (blockIdx.x % CL) * NTP + tid, nparts = CL * NTP;  // the sentence's element-wise work is split over the blocks
 
     if (!lengths_ok(m, n, L, T)) {
         for (int i = part; i < Mc * (T + 2); i += nparts) Sb[i] = (i == 0) ? __builtin_nanf("") : NEG_INF_F;
@@ -1562,23 +1572,26 @@ __global__ __launch_bounds__(16 * NL) void inside_fwd_ml1_cluster_kernel(const f
             av.SR[i] = v * LOG2E_F;
         }
     }
+    if (k == 0)
+        for (int i = tid; i < T + 4; i += NTP) av.D[i] = 0.f;
+    if (NLP * k >= mc) return;  // no node of the sentence in this block: nobody waits for it
     const float base_cell = to_b2(mt[(size_t)(m - 1) * T + (n - 1)]);
-    if (tid < MP) {
-        col[(n - 1) & 1][tid] = (tid == mc - 1) ? base_cell : NEG_INF_F;
-        col[(n - 2) & 1][tid] = NEG_INF_F;
+    for (int i = tid; i < 2 * MP; i += NTP) (&col[0][0])[i] = NEG_INF_F;
+    __syncthreads();
+    if (tid == 0) {
+        col[(n - 1) & 1][mc - 1] = base_cell;
+        sm_Dv[0] = 0.f;
+        sm_Dv[1] = 0.f;
+        sm_dead = 0;
     }
-    if (w == 0)
-        for (int i = tid; i < T + 4; i += NTC) av.D[i] = 0.f;
-    if (tid == 0) sm_dead = 0;
-    if (tid < 16) slots[tid >> 3][tid & 7] = (tid == 8 * ((n - 1) & 1)) ? base_cell : NEG_INF_F;
 
     // this lane's node and its link rows (rows beyond the sentence: any valid row, the result is discarded)
-    const int a_id = CL * gidx + w;
+    const int a_id = NLP * k + gidx;
     const bool row_ok = a_id < mc;
-    const int ar = row_ok ? a_id : 0;
-    const int q0 = __builtin_amdgcn_readfirstlane((CL * 4 * (tid >> 6) + w) / 64);  // chunk of the wave's first node's diagonal
+    const int ar = row_ok ? a_id : NLP * k;
+    const int q0 = (NLP * k) / 64;  // the chunk that holds the block's diagonal
     float4 A0[NQ], A1[NQ];
-    {
+    if (!collector) {
         const float4 *r0 = reinterpret_cast<const float4 *>(av.Ac + ((size_t)0 * Mc + ar) * MP) + j;
         const float4 *r1 = reinterpret_cast<const float4 *>(av.Ac + ((size_t)1 * Mc + ar) * MP) + j;
 #pragma unroll
@@ -1589,8 +1602,8 @@ __global__ __launch_bounds__(16 * NL) void inside_fwd_ml1_cluster_kernel(const f
     }
     const float *ra = mt + (size_t)(2 * ar + 1) * T, *rl = mt + (size_t)(2 * ar) * T;
     if (MATCH_LDS) {
-        for (int i = tid; i < NL * T; i += NTC) {
-            const int g = i / T, s = i - g * T, node = CL * g + w;
+        for (int i = tid; i < NLP * T; i += NTP) {
+            const int g = i / T, s = i - g * T, node = NLP * k + g;
             const bool ok = node < mc && s < n;
             sm_main[i] = ok ? to_b2(mt[(size_t)(2 * node + 1) * T + s]) : NEG_INF_F;
             sm_leaf[i] = (ok && node >= 1) ? to_b2(mt[(size_t)(2 * node) * T + s]) : NEG_INF_F;
@@ -1606,53 +1619,87 @@ __global__ __launch_bounds__(16 * NL) void inside_fwd_ml1_cluster_kernel(const f
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
 
+    unsigned long long *Xf = xv.fcol;
+    float *Dk = xv.shifts + (size_t)k * (T + 4);
     double O = 0.0;  // offset of the column being read
     for (int t = n - 1; t >= 1; t--) {
         const float *cur = col[t & 1];
         float *nxt = col[(t - 1) & 1];
-        const float D = max8(slots[t & 1]);
+        const float D = sm_Dv[t & 1];
         const float Ds = (D == NEG_INF_F) ? 0.f : D;
-        const double O_new = O + (double)Ds;
-        // the next column's emissions: from LDS, or requested now so that they travel during the column's work
-        float ma_raw = 0.f, ml_raw = 0.f;
-        if (t > 1) {
-            ma_raw = MATCH_LDS ? sm_main[gidx * T + t - 2] : ra[t - 2];
-            ml_raw = MATCH_LDS ? sm_leaf[gidx * T + t - 2] : rl[t - 2];
-        }
-        const float4 *cv = reinterpret_cast<const float4 *>(cur) + j;
-        float F0, F1;
-        slab_row_lse<NQ, false>(A0, A1, cv, cv, q0, NQ, row_ok, a_id >= 1, f0g, F0, F1);
-        F0 -= Ds;
-        F1 -= Ds;
-        float s_new = lse2_b2(ma_p + F0, (ml_p + ma_t) + (f1p - Ds));
-        if (!row_ok) s_new = NEG_INF_F;
-        f1p = F1;
-        f0g = F0;
-        const unsigned tag = (nonce << 12) | (unsigned)t;
-        if (j == 0 && row_ok && t > 1) slot_store(xv.fcol + ((t - 1) & 1) * MP + w * NL + gidx, tag, s_new, s_new);
-        if (t > 1 && pidx < MP) {  // whole waves; slot pidx belongs to node CL * (pidx % NL) + pidx / NL
-            const int node = CL * (pidx % NL) + pidx / NL;
-            float v = NEG_INF_F;
-            if (node < mc) {
-                u32x4 x;
-                if (poll_slot(xv.fcol + ((t - 1) & 1) * MP + pidx, tag, xv.flags + FLAG_FWD, spin_limit, x)) v = __uint_as_float(x.y);
-                else sm_dead = 1;
+        const double O_new = O + (double)Ds;  // offset of column t-1
+        if (collector) {
+            // the shift of the next step from the visible part of column t, which is complete
+            float vm = NEG_INF_F;
+#pragma unroll
+            for (int r = 0; r < NQ; r++) {
+                const int i = NLP * k + 64 * r + lane;
+                if (i < MP) vm = fmaxf(vm, cur[i]);
             }
-            nxt[node] = v;
-            const float wm = wave_max(v + 0.f);
-            if ((tid & 63) == 0) slots[(t - 1) & 1][pidx >> 6] = wm;
+            vm = wave_max(vm);
+            if (lane == 0) sm_Dv[(t - 1) & 1] = vm;
+            if (t > 1) {  // column t-1 of the blocks above
+                const unsigned long long *src = Xf + (size_t)(t - 1) * MP + NLP * (k + 1) + lane;
+                unsigned long long x[NQ];
+#pragma unroll
+                for (int r = 0; r < NQ; r++) {
+                    const int i = NLP * (k + 1) + 64 * r + lane;
+                    x[r] = (i < mc) ? entry_load(src + 64 * r) : (unsigned long long)__double_as_longlong(-__builtin_huge_val());
+                }
+                for (int spins = 0;; spins++) {
+                    bool pending = false;
+#pragma unroll
+                    for (int r = 0; r < NQ; r++) pending |= (x[r] == EMPTY64);
+                    if (!__any(pending)) break;
+                    if (spins >= spin_limit || ((spins & 63) == 63 && gave_up(xv.flags + FLAG_FWD))) {
+                        sm_dead = 1;
+                        break;
+                    }
+#pragma unroll
+                    for (int r = 0; r < NQ; r++)
+                        if (x[r] == EMPTY64) x[r] = entry_load(src + 64 * r);
+                }
+#pragma unroll
+                for (int r = 0; r < NQ; r++) {
+                    const int i = NLP * (k + 1) + 64 * r + lane;
+                    if (i < MP) nxt[i] = (x[r] == EMPTY64) ? NEG_INF_F : (float)(__longlong_as_double((long long)x[r]) - O_new);
+                }
+            }
+        } else {
+            // the next column's emissions: from LDS, or requested now so that they travel during the column's work
+            float ma_raw = 0.f, ml_raw = 0.f;
+            if (t > 1) {
+                ma_raw = MATCH_LDS ? sm_main[gidx * T + t - 2] : ra[t - 2];
+                ml_raw = MATCH_LDS ? sm_leaf[gidx * T + t - 2] : rl[t - 2];
+            }
+            const float4 *cv = reinterpret_cast<const float4 *>(cur) + j;
+            float F0, F1;
+            slab_row_lse<NQ, false>(A0, A1, cv, cv, q0, NQ, row_ok, a_id >= 1, f0g, F0, F1);
+            F0 -= Ds;
+            F1 -= Ds;
+            float s_new = lse2_b2(ma_p + F0, (ml_p + ma_t) + (f1p - Ds));
+            if (!row_ok) s_new = NEG_INF_F;
+            f1p = F1;
+            f0g = F0;
+            if (j == 0) {
+                nxt[a_id] = s_new;
+                if (row_ok) {
+                    const double s_abs = (double)s_new + O_new;
+                    if (t > 1) entry_store(Xf + (size_t)(t - 1) * MP + a_id, s_abs);
+                    Sb[(size_t)a_id * (T + 2) + (t - 1)] = (float)(s_abs * LN2_D);
+                    av.SR[(size_t)a_id * (T + 2) + (t - 1)] = s_new;
+                    av.F0[(size_t)a_id * (T + 2) + t] = F0;
+                    av.F1[(size_t)a_id * (T + 2) + t] = F1;
+                }
+            }
+            if (tid == 0) {
+                Dk[t] = Ds;
+                if (k == 0) av.D[t] = Ds;
+            }
+            ma_t = ma_p;
+            ma_p = MATCH_LDS ? ma_raw : to_b2(ma_raw);
+            ml_p = MATCH_LDS ? ml_raw : (ar >= 1 ? to_b2(ml_raw) : NEG_INF_F);
         }
-        // the table cells go out after the exchange, so that the wait for the entries is not also a wait for these stores
-        if (j == 0 && row_ok) {
-            Sb[(size_t)a_id * (T + 2) + (t - 1)] = (float)(((double)s_new + O_new) * LN2_D);
-            av.SR[(size_t)a_id * (T + 2) + (t - 1)] = s_new;
-            av.F0[(size_t)a_id * (T + 2) + t] = F0;
-            av.F1[(size_t)a_id * (T + 2) + t] = F1;
-        }
-        if (w == 0 && tid == 0) av.D[t] = Ds;
-        ma_t = ma_p;
-        ma_p = MATCH_LDS ? ma_raw : to_b2(ma_raw);
-        ml_p = MATCH_LDS ? ml_raw : (ar >= 1 ? to_b2(ml_raw) : NEG_INF_F);
         O = O_new;
         lds_barrier();
         if (sm_dead) {  // uniform: written before the barrier
@@ -1662,21 +1709,56 @@ __global__ __launch_bounds__(16 * NL) void inside_fwd_ml1_cluster_kernel(const f
     }
 }
 
-// Outside sweep of one cluster member.  Same tables as inside_bwd_ml1_stream_kernel.  Dynamic LDS: D [T+4], then
-// (MATCH_LDS) the emissions of the workgroup's NL nodes, main [NL][T] and leaf [NL][T].
-template <int NQ, int NL, bool MATCH_LDS>
-__global__ __launch_bounds__(16 * NL) void inside_bwd_ml1_cluster_kernel(const float *__restrict__ S, float *__restrict__ aux,
-                                                                   const float *__restrict__ match_all,
-                                                                   const int64_t *__restrict__ out_len,
-                                                                   const int64_t *__restrict__ tgt_len, int L, int T, int Mc,
-                                                                   unsigned nonce, int spin_limit) {
-    constexpr int MP = 64 * NQ, CL = MP / NL, NTC = 16 * NL;  // row length, workgroups per sentence, threads
+// Moves the tables of blocks 1 .. CL-1 from their own column offsets to those of block 0 (see above): with
+// O_s = sum_{t > s} D_t, R[a][s] is relative to O_s and F0h[a][t], F1h[a][t] to O_{t-1}.  Grid (CL-1, B).
+__global__ __launch_bounds__(256) void pipeline_rebase_kernel(float *__restrict__ aux, const int64_t *__restrict__ out_len,
+                                                             const int64_t *__restrict__ tgt_len, int L, int T, int Mc) {
+    extern __shared__ double sm_delta[];  // [T+2]: own offset minus block 0's, per column
+    const int k = blockIdx.x + 1, b = blockIdx.y, tid = threadIdx.x;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    if (!lengths_ok(m, n, L, T)) return;
+    const int mc = m / 2;
+    if (NLP * k >= mc) return;
+    AuxViewStream av(aux, b, Mc, T);
+    ExchangeView xv(aux, b, Mc, T);
+    if (xv.flags[FLAG_FWD] != 0) return;  // the sentence is redone from scratch
+    const float *Dk = xv.shifts + (size_t)k * (T + 4), *D0 = xv.shifts;
+    for (int s = tid; s <= n - 1; s += 256) {
+        double acc = 0.0;
+        for (int t = s + 1; t <= n - 1; t++) acc += (double)Dk[t] - (double)D0[t];
+        sm_delta[s] = acc;
+    }
+    __syncthreads();
+    const int TS = T + 2;
+    for (int i = tid; i < NLP * TS; i += 256) {
+        const int g = i / TS, s = i - g * TS, a_id = NLP * k + g;
+        if (a_id >= mc) continue;
+        const size_t o = (size_t)a_id * TS + s;
+        if (s <= n - 2) av.SR[o] = (float)((double)av.SR[o] + sm_delta[s]);
+        if (s >= 1 && s <= n - 1) {
+            av.F0[o] = (float)((double)av.F0[o] + sm_delta[s - 1]);
+            av.F1[o] = (float)((double)av.F1[o] + sm_delta[s - 1]);
+        }
+    }
+}
+
+// Outside sweep of one block.  Same tables as inside_bwd_ml1_stream_kernel.  Dynamic LDS: D [T+4], then (MATCH_LDS) the
+// emissions of the block's nodes, main [NLP][T] and leaf [NLP][T].
+template <int NQ, bool MATCH_LDS>
+__global__ __launch_bounds__(NTP) void inside_bwd_ml1_pipe_kernel(const float *__restrict__ S, float *__restrict__ aux,
+                                                                 const float *__restrict__ match_all,
+                                                                 const int64_t *__restrict__ out_len,
+                                                                 const int64_t *__restrict__ tgt_len, int L, int T, int Mc,
+                                                                 int spin_limit) {
+    constexpr int MP = 64 * NQ, CL = MP / NLP;
     __shared__ __attribute__((aligned(16))) float w0[2][MP];
     __shared__ __attribute__((aligned(16))) float w1[2][MP];
     __shared__ int sm_dead;
     extern __shared__ float sm_D[];  // [T+4]
-    float *sm_main = sm_D + (T + 4), *sm_leaf = sm_main + NL * T;
-    const int b = blockIdx.x / CL, w = blockIdx.x % CL, tid = threadIdx.x, gidx = tid >> 4, j = tid & 15;
+    float *sm_main = sm_D + (T + 4), *sm_leaf = sm_main + NLP * T;
+    const int b = blockIdx.x / CL, k = blockIdx.x % CL;  // the leading (lowest) block first
+    const int tid = threadIdx.x, gidx = (tid >> 4) & (NLP - 1), j = tid & 15, lane = tid & 63;
+    const bool collector = tid >= 16 * NLP;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const float *mt = match_all + (size_t)b * L * T;
     const float *Sb = S + (size_t)b * Mc * (T + 2);
@@ -1686,11 +1768,16 @@ __global__ __launch_bounds__(16 * NL) void inside_bwd_ml1_cluster_kernel(const f
     const bool valid = lengths_ok(m, n, L, T) && (ll == ll) && (fabsf(ll) != __builtin_huge_valf());
     if (!valid) return;  // the posterior kernels write zeros for such sentences
     const int mc = m / 2;
-    for (int i = tid; i < T + 4; i += NTC) sm_D[i] = av.D[i];
+    if (NLP * k >= mc) return;  // no node of the sentence in this block: nobody waits for it
+    for (int i = tid; i < T + 4; i += NTP) sm_D[i] = av.D[i];
+    for (int i = tid; i < 2 * MP; i += NTP) {
+        (&w0[0][0])[i] = NEG_INF_F;
+        (&w1[0][0])[i] = NEG_INF_F;
+    }
     if (tid == 0) sm_dead = 0;
     if (MATCH_LDS) {
-        for (int i = tid; i < NL * T; i += NTC) {
-            const int g = i / T, s = i - g * T, node = CL * g + w;
+        for (int i = tid; i < NLP * T; i += NTP) {
+            const int g = i / T, s = i - g * T, node = NLP * k + g;
             const bool ok = node < mc && s < n;
             sm_main[i] = ok ? to_b2(mt[(size_t)(2 * node + 1) * T + s]) : NEG_INF_F;
             sm_leaf[i] = (ok && node >= 1) ? to_b2(mt[(size_t)(2 * node) * T + s]) : NEG_INF_F;
@@ -1698,12 +1785,12 @@ __global__ __launch_bounds__(16 * NL) void inside_bwd_ml1_cluster_kernel(const f
     }
 
     // this lane's node and its transposed link rows: parents a <= c, chunks [0, q1)
-    const int c_id = CL * gidx + w;
+    const int c_id = NLP * k + gidx;
     const bool live = c_id < mc;
-    const int ci = live ? c_id : 0;
-    const int q1 = min(__builtin_amdgcn_readfirstlane((CL * (4 * (tid >> 6) + 3) + w) / 64), NQ - 1) + 1;  // the wave's last node
+    const int ci = live ? c_id : NLP * k;
+    const int q1 = (NLP * k + NLP - 1) / 64 + 1;
     float4 A0[NQ], A1[NQ];
-    {
+    if (!collector) {
         const float4 *r0 = reinterpret_cast<const float4 *>(av.At + ((size_t)0 * Mc + ci) * MP) + j;
         const float4 *r1 = reinterpret_cast<const float4 *>(av.At + ((size_t)1 * Mc + ci) * MP) + j;
 #pragma unroll
@@ -1713,17 +1800,12 @@ __global__ __launch_bounds__(16 * NL) void inside_bwd_ml1_cluster_kernel(const f
         }
     }
     const float *ra = mt + (size_t)(2 * ci + 1) * T, *rl = mt + (size_t)(2 * ci) * T;
-    __syncthreads();  // sm_D
+    __syncthreads();  // sm_D, the cleared columns
     const float beta00 = -av.SR[0];  // relative to the offset of column 0
     const float w00 = (to_b2(mt[(size_t)1 * T]) + beta00) - sm_D[1];
-    if (tid < MP) {
-        w0[1][tid] = (tid == 0) ? w00 : NEG_INF_F;
-        w1[1][tid] = NEG_INF_F;
-        w0[0][tid] = NEG_INF_F;
-        w1[0][tid] = NEG_INF_F;
-    }
+    if (tid == 0) w0[1][0] = w00;
     float bp = (c_id == 0) ? beta00 : NEG_INF_F;  // the node's outside score one column earlier
-    if (j == 0 && live) {
+    if (!collector && j == 0 && live) {
         av.BETA[(size_t)c_id * (T + 2)] = bp;
         av.W0[(size_t)c_id * (T + 2) + 1] = (c_id == 0) ? w00 : NEG_INF_F;
         av.W1[(size_t)c_id * (T + 2) + 1] = NEG_INF_F;
@@ -1741,50 +1823,76 @@ __global__ __launch_bounds__(16 * NL) void inside_bwd_ml1_cluster_kernel(const f
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
 
+    unsigned *Xb = xv.bw;
     for (int t = 1; t <= n - 1; t++) {
         const float *c0 = w0[t & 1], *c1 = w1[t & 1];
         float *n0 = w0[(t + 1) & 1], *n1 = w1[(t + 1) & 1];
-        const float d_next = sm_D[t + 1], d_both = d_next + sm_D[t];
         const bool more = t < n - 1;
-        float mc_raw = 0.f, ml_raw = 0.f;
-        if (more) {
-            mc_raw = MATCH_LDS ? sm_main[gidx * T + t + 1] : ra[t + 1];
-            ml_raw = MATCH_LDS ? sm_leaf[gidx * T + t] : rl[t];
-        }
-        const float4 *u0 = reinterpret_cast<const float4 *>(c0) + j, *u1 = reinterpret_cast<const float4 *>(c1) + j;
-        float beta, unused;
-        slab_row_lse<NQ, true>(A0, A1, u0, u1, 0, q1, live, true, bp, beta, unused);
-        if (!live) beta = NEG_INF_F;
-        const float nw0 = (mc_t + beta) - d_next;
-        const float nw1 = ((ml_p + mc_t) + bp) - d_both;
-        const unsigned tag = (nonce << 12) | (unsigned)(t + 1);
-        if (j == 0 && live && more) slot_store(xv.bw + ((t + 1) & 1) * MP + w * NL + gidx, tag, nw0, nw1);
-        // collected by the first waves, whose nodes have the fewest parents
-        if (more) {
-            for (int i = tid; i < MP; i += NTC) {  // slot i belongs to node CL * (i % NL) + i / NL
-                const int node = CL * (i % NL) + i / NL;
-                float v0 = NEG_INF_F, v1 = NEG_INF_F;
-                if (node < mc) {
-                    u32x4 x;
-                    if (poll_slot(xv.bw + ((t + 1) & 1) * MP + i, tag, xv.flags + FLAG_BWD, spin_limit, x)) {
-                        v0 = __uint_as_float(x.y);
-                        v1 = __uint_as_float(x.z);
-                    } else {
+        if (collector) {
+            if (more && k > 0) {  // the weights of the blocks below for column t+1
+                const unsigned *src = Xb + (size_t)(t + 1) * 2 * MP + lane;
+                unsigned x0[NQ], x1[NQ];
+                const int end = min(NLP * k, mc);
+#pragma unroll
+                for (int r = 0; r < NQ; r++) {
+                    const bool need = 64 * r + lane < end;
+                    x0[r] = need ? entry_load(src + 64 * r) : __float_as_uint(NEG_INF_F);
+                    x1[r] = need ? entry_load(src + MP + 64 * r) : __float_as_uint(NEG_INF_F);
+                }
+                for (int spins = 0;; spins++) {
+                    bool pending = false;
+#pragma unroll
+                    for (int r = 0; r < NQ; r++) pending |= (x0[r] == EMPTY32) | (x1[r] == EMPTY32);
+                    if (!__any(pending)) break;
+                    if (spins >= spin_limit || ((spins & 63) == 63 && gave_up(xv.flags + FLAG_BWD))) {
                         sm_dead = 1;
+                        break;
+                    }
+#pragma unroll
+                    for (int r = 0; r < NQ; r++) {
+                        if (x0[r] == EMPTY32) x0[r] = entry_load(src + 64 * r);
+                        if (x1[r] == EMPTY32) x1[r] = entry_load(src + MP + 64 * r);
                     }
                 }
-                n0[node] = v0;
-                n1[node] = v1;
+#pragma unroll
+                for (int r = 0; r < NQ; r++) {
+                    const int i = 64 * r + lane;
+                    if (i < NLP * k) {
+                        n0[i] = (x0[r] == EMPTY32) ? NEG_INF_F : __uint_as_float(x0[r]);
+                        n1[i] = (x1[r] == EMPTY32) ? NEG_INF_F : __uint_as_float(x1[r]);
+                    }
+                }
             }
+        } else {
+            const float d_next = sm_D[t + 1], d_both = d_next + sm_D[t];
+            float mc_raw = 0.f, ml_raw = 0.f;
+            if (more) {
+                mc_raw = MATCH_LDS ? sm_main[gidx * T + t + 1] : ra[t + 1];
+                ml_raw = MATCH_LDS ? sm_leaf[gidx * T + t] : rl[t];
+            }
+            const float4 *u0 = reinterpret_cast<const float4 *>(c0) + j, *u1 = reinterpret_cast<const float4 *>(c1) + j;
+            float beta, unused;
+            slab_row_lse<NQ, true>(A0, A1, u0, u1, 0, q1, live, true, bp, beta, unused);
+            if (!live) beta = NEG_INF_F;
+            const float nw0 = (mc_t + beta) - d_next;
+            const float nw1 = ((ml_p + mc_t) + bp) - d_both;
+            if (j == 0) {
+                n0[c_id] = nw0;
+                n1[c_id] = nw1;
+                if (live) {
+                    if (more) {
+                        entry_store(Xb + (size_t)(t + 1) * 2 * MP + c_id, nw0);
+                        entry_store(Xb + (size_t)(t + 1) * 2 * MP + MP + c_id, nw1);
+                    }
+                    av.BETA[(size_t)c_id * (T + 2) + t] = beta;
+                    av.W0[(size_t)c_id * (T + 2) + t + 1] = nw0;
+                    av.W1[(size_t)c_id * (T + 2) + t + 1] = nw1;
+                }
+            }
+            bp = beta;
+            mc_t = MATCH_LDS ? mc_raw : (live ? to_b2(mc_raw) : NEG_INF_F);
+            ml_p = MATCH_LDS ? ml_raw : ((live && ci >= 1) ? to_b2(ml_raw) : NEG_INF_F);
         }
-        if (j == 0 && live) {  // after the exchange, so that the wait for the entries is not also a wait for these stores
-            av.BETA[(size_t)c_id * (T + 2) + t] = beta;
-            av.W0[(size_t)c_id * (T + 2) + t + 1] = nw0;
-            av.W1[(size_t)c_id * (T + 2) + t + 1] = nw1;
-        }
-        bp = beta;
-        mc_t = MATCH_LDS ? mc_raw : (live ? to_b2(mc_raw) : NEG_INF_F);
-        ml_p = MATCH_LDS ? ml_raw : ((live && ci >= 1) ? to_b2(ml_raw) : NEG_INF_F);
         lds_barrier();
         if (sm_dead) {  // uniform: written before the barrier
             if (tid == 0) __hip_atomic_store(xv.flags + FLAG_BWD, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1897,50 +2005,47 @@ __global__ __launch_bounds__(256) void criterion_loss_kernel(const float *__rest
     criterion_loss_block<256>(LossTask{S, tgt_len, out, B, (int64_t)Mc * (T + 2)});
 }
 
-// Cluster sweeps are used when all their workgroups fit on the device together (two per compute unit).  Both numbers can
-// be changed through pcfgnat_cluster_config.
-std::atomic<int> g_cluster_max_wg{512}, g_cluster_spin_limit{1 << 20};
-std::atomic<unsigned> g_cluster_nonce{0};
-unsigned next_nonce() { return g_cluster_nonce.fetch_add(1) % 0xFFFFFu + 1u; }  // 1 .. 2^20 - 1: tags are never zero
-struct ClusterShape {
-    int NQ, NL, CL;  // chunks of 64 per link row, nodes per workgroup, workgroups per sentence; CL = 0: not applicable
-};
-ClusterShape cluster_shape(int B, int T, int Mc) {
-    const int NQ = stream_mp(Mc) / 64, NL = NQ <= 4 ? 32 : 64, CL = 64 * NQ / NL;
-    const bool ok = NQ >= 3 && NQ <= 8 && T + 2 < 4096 && (int64_t)B * CL <= g_cluster_max_wg.load();
-    return ClusterShape{NQ, NL, ok ? CL : 0};
+// The pipelined sweeps are used while a batch needs no more than g_cluster_max_wg workgroups (a few per compute unit).
+// Both numbers can be changed through pcfgnat_cluster_config.
+std::atomic<int> g_cluster_max_wg{1024}, g_cluster_spin_limit{1 << 20};
+int pipeline_chunks(int B, int T, int Mc) {  // NQ, or 0 where the pipelined sweeps do not apply
+    const int NQ = stream_mp(Mc) / 64, CL = 64 * NQ / NLP;
+    return (NQ >= 3 && NQ <= 8 && T + 2 < 4096 && (int64_t)B * CL <= g_cluster_max_wg.load()) ? NQ : 0;
 }
 
-template <int NQ, int NL>
-int launch_fwd_cluster(const float *match_all, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B, int L, int T, int Mc,
-                       hipStream_t stream) {
-    constexpr int CL = 64 * NQ / NL, NTC = 16 * NL;
-    const size_t match_bytes = (size_t)2 * NL * T * sizeof(float);
+template <int NQ>
+int launch_fwd_pipe(const float *match_all, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B, int L, int T, int Mc,
+                    hipStream_t stream) {
+    constexpr int CL = 64 * NQ / NLP;
+    const size_t match_bytes = (size_t)2 * NLP * T * sizeof(float);
     if (match_bytes <= LDS_BUDGET - 8192) {
-        auto k = inside_fwd_ml1_cluster_kernel<NQ, NL, true>;
+        auto k = inside_fwd_ml1_pipe_kernel<NQ, true>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)match_bytes));
-        hipLaunchKernelGGL(k, dim3(B * CL), dim3(NTC), match_bytes, stream, match_all, ol, tl, S, aux, L, T, Mc, next_nonce(),
+        hipLaunchKernelGGL(k, dim3(B * CL), dim3(NTP), match_bytes, stream, match_all, ol, tl, S, aux, L, T, Mc,
                            g_cluster_spin_limit.load());
     } else {
-        hipLaunchKernelGGL((inside_fwd_ml1_cluster_kernel<NQ, NL, false>), dim3(B * CL), dim3(NTC), 0, stream, match_all, ol, tl, S, aux,
-                           L, T, Mc, next_nonce(), g_cluster_spin_limit.load());
+        hipLaunchKernelGGL((inside_fwd_ml1_pipe_kernel<NQ, false>), dim3(B * CL), dim3(NTP), 0, stream, match_all, ol, tl, S, aux, L, T,
+                           Mc, g_cluster_spin_limit.load());
     }
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(pipeline_rebase_kernel, dim3(CL - 1, B), dim3(256), (size_t)(T + 2) * sizeof(double), stream, aux, ol, tl, L, T,
+                       Mc);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
-template <int NQ, int NL>
-int launch_bwd_cluster(const float *S, float *aux, const float *match_all, const int64_t *ol, const int64_t *tl, int B, int L, int T,
-                       int Mc, hipStream_t stream) {
-    constexpr int CL = 64 * NQ / NL, NTC = 16 * NL;
-    const size_t base = (size_t)(T + 4) * sizeof(float), with_match = base + (size_t)2 * NL * T * sizeof(float);
+template <int NQ>
+int launch_bwd_pipe(const float *S, float *aux, const float *match_all, const int64_t *ol, const int64_t *tl, int B, int L, int T,
+                    int Mc, hipStream_t stream) {
+    constexpr int CL = 64 * NQ / NLP;
+    const size_t base = (size_t)(T + 4) * sizeof(float), with_match = base + (size_t)2 * NLP * T * sizeof(float);
     if (with_match <= LDS_BUDGET - 8192) {
-        auto k = inside_bwd_ml1_cluster_kernel<NQ, NL, true>;
+        auto k = inside_bwd_ml1_pipe_kernel<NQ, true>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_match));
-        hipLaunchKernelGGL(k, dim3(B * CL), dim3(NTC), with_match, stream, S, aux, match_all, ol, tl, L, T, Mc, next_nonce(),
+        hipLaunchKernelGGL(k, dim3(B * CL), dim3(NTP), with_match, stream, S, aux, match_all, ol, tl, L, T, Mc,
                            g_cluster_spin_limit.load());
     } else {
-        hipLaunchKernelGGL((inside_bwd_ml1_cluster_kernel<NQ, NL, false>), dim3(B * CL), dim3(NTC), base, stream, S, aux, match_all, ol,
-                           tl, L, T, Mc, next_nonce(), g_cluster_spin_limit.load());
+        hipLaunchKernelGGL((inside_bwd_ml1_pipe_kernel<NQ, false>), dim3(B * CL), dim3(NTP), base, stream, S, aux, match_all, ol, tl, L,
+                           T, Mc, g_cluster_spin_limit.load());
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
@@ -1952,20 +2057,20 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
     PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss: aux must be 16-byte aligned");
     hipLaunchKernelGGL(compact_links_ml1_kernel, dim3(MP / 32, MP / 32, B), dim3(256), 0, stream, links, ol, aux, L, T, Mc, MP);
     PCFGNAT_HIP_CHECK(hipGetLastError());
-    // cluster sweep first where it applies; the one-workgroup sweep then only redoes sentences whose cluster gave up
-    const ClusterShape cs = cluster_shape(B, T, Mc);
+    // pipelined sweep first where it applies; the one-workgroup sweep then only redoes sentences whose blocks gave up
+    const int NQ = pipeline_chunks(B, T, Mc);
     int rc = PCFGNAT_OK;
-    switch (cs.CL ? cs.NQ : 0) {
-        case 3: rc = launch_fwd_cluster<3, 32>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
-        case 4: rc = launch_fwd_cluster<4, 32>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
-        case 5: rc = launch_fwd_cluster<5, 64>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
-        case 6: rc = launch_fwd_cluster<6, 64>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
-        case 7: rc = launch_fwd_cluster<7, 64>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
-        case 8: rc = launch_fwd_cluster<8, 64>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
+    switch (NQ) {
+        case 3: rc = launch_fwd_pipe<3>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
+        case 4: rc = launch_fwd_pipe<4>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
+        case 5: rc = launch_fwd_pipe<5>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
+        case 6: rc = launch_fwd_pipe<6>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
+        case 7: rc = launch_fwd_pipe<7>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
+        case 8: rc = launch_fwd_pipe<8>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
         default: break;
     }
     if (rc != PCFGNAT_OK) return rc;
-    const int only_flagged = cs.CL != 0;
+    const int only_flagged = NQ != 0;
     const size_t base = ((size_t)4 * MP + 32) * sizeof(float);
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
     if (with_match <= LDS_BUDGET) {
@@ -1987,19 +2092,19 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
     PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss_backward: aux must be 16-byte aligned");
     const size_t base = ((size_t)5 * MP + T + 4) * sizeof(float);
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
-    const ClusterShape cs = cluster_shape(B, T, Mc);
+    const int NQ = pipeline_chunks(B, T, Mc);
     int rc = PCFGNAT_OK;
-    switch (cs.CL ? cs.NQ : 0) {
-        case 3: rc = launch_bwd_cluster<3, 32>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
-        case 4: rc = launch_bwd_cluster<4, 32>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
-        case 5: rc = launch_bwd_cluster<5, 64>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
-        case 6: rc = launch_bwd_cluster<6, 64>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
-        case 7: rc = launch_bwd_cluster<7, 64>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
-        case 8: rc = launch_bwd_cluster<8, 64>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
+    switch (NQ) {
+        case 3: rc = launch_bwd_pipe<3>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
+        case 4: rc = launch_bwd_pipe<4>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
+        case 5: rc = launch_bwd_pipe<5>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
+        case 6: rc = launch_bwd_pipe<6>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
+        case 7: rc = launch_bwd_pipe<7>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
+        case 8: rc = launch_bwd_pipe<8>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
         default: break;
     }
     if (rc != PCFGNAT_OK) return rc;
-    const int only_flagged = cs.CL != 0;
+    const int only_flagged = NQ != 0;
     // lanes per node: four while one pass covers all nodes; beyond that the outside sweep measured faster with eight
     if (with_match <= LDS_BUDGET) {
         auto k = Mc <= NT / 4 ? inside_bwd_ml1_stream_kernel<true, 4> : inside_bwd_ml1_stream_kernel<true, 8>;

@@ -246,12 +246,12 @@ def _inside_all(batch, match):
     return ll.detach().cpu(), md.grad.cpu(), ld.grad.cpu()
 
 
-@pytest.mark.parametrize("mode", ["one_workgroup", "clusters_give_up"])
+@pytest.mark.parametrize("mode", ["one_workgroup", "blocks_give_up"])
 @pytest.mark.parametrize("L,T,ms,ns", [(320, 40, [320, 262, 4], [40, 31, 2]), (512, 140, [512, 444], [140, 120]),
                                        (600, 24, [600, 520], [24, 24]), (1024, 30, [1024, 770, 900], [30, 22, 30])])
 def test_long_graph_sweeps_agree(mode, L, T, ms, ns):
-    """Graphs of 258..1026 nodes: the cluster sweeps (default for small batches), the one-workgroup streaming sweeps
-    (clusters switched off) and the redo path (clusters that give up at once: spin limit 0) compute the same tables; the
+    """Graphs of 258..1026 nodes: the pipelined sweeps (default for small batches), the one-workgroup streaming sweeps
+    (pipeline switched off) and the redo path (blocks that give up at once: spin limit 0) compute the same tables; the
     default path is compared with the oracle in test_inside_forward_backward_vs_oracle."""
     batch = synth.training_batch(len(ms), L, T, 60, ms, ns, seed=L + T)
     match = _match_for(batch)
@@ -263,7 +263,7 @@ def test_long_graph_sweeps_agree(mode, L, T, ms, ns):
             ops.cluster_config(spin_limit=0)
         ll1, mg1, lg1 = _inside_all(batch, match)
     finally:
-        ops.cluster_config(max_workgroups=512, spin_limit=1 << 20)
+        ops.cluster_config(max_workgroups=1024, spin_limit=1 << 20)
     fin = torch.isfinite(ll0)
     assert fin.any() and torch.equal(fin, torch.isfinite(ll1))
     assert torch.allclose(ll0[fin], ll1[fin], rtol=1e-5)
