@@ -1655,6 +1655,7 @@ __global__ __launch_bounds__(NTP) void inside_fwd_ml1_pipe_kernel(const float *_
                         sm_dead = 1;
                         break;
                     }
+                    __builtin_amdgcn_s_sleep(2);  // leave the issue slots of this SIMD to its compute wave
 #pragma unroll
                     for (int r = 0; r < NQ; r++)
                         if (x[r] == EMPTY64) x[r] = entry_load(src + 64 * r);
@@ -1714,6 +1715,7 @@ __global__ __launch_bounds__(NTP) void inside_fwd_ml1_pipe_kernel(const float *_
 __global__ __launch_bounds__(256) void pipeline_rebase_kernel(float *__restrict__ aux, const int64_t *__restrict__ out_len,
                                                              const int64_t *__restrict__ tgt_len, int L, int T, int Mc) {
     extern __shared__ double sm_delta[];  // [T+2]: own offset minus block 0's, per column
+    __shared__ double sm_part[4];
     const int k = blockIdx.x + 1, b = blockIdx.y, tid = threadIdx.x;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     if (!lengths_ok(m, n, L, T)) return;
@@ -1723,21 +1725,53 @@ __global__ __launch_bounds__(256) void pipeline_rebase_kernel(float *__restrict_
     ExchangeView xv(aux, b, Mc, T);
     if (xv.flags[FLAG_FWD] != 0) return;  // the sentence is redone from scratch
     const float *Dk = xv.shifts + (size_t)k * (T + 4), *D0 = xv.shifts;
-    for (int s = tid; s <= n - 1; s += 256) {
-        double acc = 0.0;
-        for (int t = s + 1; t <= n - 1; t++) acc += (double)Dk[t] - (double)D0[t];
-        sm_delta[s] = acc;
+    // delta[s] = sum_{t = s+1}^{n-1} (Dk[t] - D0[t]): every thread sums a run of columns, the runs are then chained
+    const int run = (n + 255) / 256;  // columns per thread
+    const int hi = n - 1 - tid * run;  // this thread's columns: hi, hi-1, ..., hi-run+1 (those >= 1)
+    double acc = 0.0;
+    for (int i = 0; i < run; i++) {
+        const int t = hi - i;
+        if (t >= 1) acc += (double)Dk[t] - (double)D0[t];
+    }
+    double incl = acc;  // inclusive prefix over the threads: inside the wave by shuffles, across the four waves through LDS
+    for (int o = 1; o < 64; o <<= 1) {
+        const double y = __shfl_up(incl, o);
+        if ((tid & 63) >= o) incl += y;
+    }
+    if ((tid & 63) == 63) sm_part[tid >> 6] = incl;
+    __syncthreads();
+    double before = incl - acc;  // the sum over the runs of the threads below, i.e. over the columns above hi
+    for (int w = 0; w < (tid >> 6); w++) before += sm_part[w];
+    acc = before;
+    for (int i = 0; i < run; i++) {
+        const int t = hi - i;  // delta[t] excludes column t itself
+        if (t >= 0 && t <= n - 1) sm_delta[t] = acc;
+        if (t >= 1) acc += (double)Dk[t] - (double)D0[t];
     }
     __syncthreads();
-    const int TS = T + 2;
-    for (int i = tid; i < NLP * TS; i += 256) {
-        const int g = i / TS, s = i - g * TS, a_id = NLP * k + g;
-        if (a_id >= mc) continue;
-        const size_t o = (size_t)a_id * TS + s;
-        if (s <= n - 2) av.SR[o] = (float)((double)av.SR[o] + sm_delta[s]);
-        if (s >= 1 && s <= n - 1) {
-            av.F0[o] = (float)((double)av.F0[o] + sm_delta[s - 1]);
-            av.F1[o] = (float)((double)av.F1[o] + sm_delta[s - 1]);
+    const int TS = T + 2, cells = NLP * TS;
+    for (int base = tid; base < cells; base += 4 * 256) {
+        float r[4], f0[4], f1[4];
+        size_t o[4];
+        int sc[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int i = base + u * 256, g = i / TS, s = i - g * TS, a_id = NLP * k + g;
+            const bool ok = i < cells && a_id < mc && s <= n - 1;
+            sc[u] = ok ? s : -1;
+            o[u] = (size_t)(ok ? a_id : NLP * k) * TS + (ok ? s : 0);
+            r[u] = av.SR[o[u]];
+            f0[u] = av.F0[o[u]];
+            f1[u] = av.F1[o[u]];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int s = sc[u];
+            if (s >= 0 && s <= n - 2) av.SR[o[u]] = (float)((double)r[u] + sm_delta[s]);
+            if (s >= 1) {
+                av.F0[o[u]] = (float)((double)f0[u] + sm_delta[s - 1]);
+                av.F1[o[u]] = (float)((double)f1[u] + sm_delta[s - 1]);
+            }
         }
     }
 }
@@ -1848,6 +1882,7 @@ __global__ __launch_bounds__(NTP) void inside_bwd_ml1_pipe_kernel(const float *_
                         sm_dead = 1;
                         break;
                     }
+                    __builtin_amdgcn_s_sleep(2);  // leave the issue slots of this SIMD to its compute wave
 #pragma unroll
                     for (int r = 0; r < NQ; r++) {
                         if (x0[r] == EMPTY32) x0[r] = entry_load(src + 64 * r);
