@@ -1621,6 +1621,13 @@ __global__ __launch_bounds__(NTP) void inside_fwd_ml1_pipe_kernel(const float *_
 
     unsigned long long *Xf = xv.fcol;
     float *Dk = xv.shifts + (size_t)k * (T + 4);
+    const unsigned long long MINUS_INF64 = (unsigned long long)__double_as_longlong(-__builtin_huge_val());
+    unsigned long long x[NQ];  // collector: the entries of the blocks above, requested one step before they are handed on
+#pragma unroll
+    for (int r = 0; r < NQ; r++) {
+        const int i = NLP * (k + 1) + 64 * r + lane;
+        x[r] = (collector && n >= 3) ? entry_load(Xf + (size_t)(n - 2) * MP + i) : MINUS_INF64;
+    }
     double O = 0.0;  // offset of the column being read
     for (int t = n - 1; t >= 1; t--) {
         const float *cur = col[t & 1];
@@ -1629,23 +1636,13 @@ __global__ __launch_bounds__(NTP) void inside_fwd_ml1_pipe_kernel(const float *_
         const float Ds = (D == NEG_INF_F) ? 0.f : D;
         const double O_new = O + (double)Ds;  // offset of column t-1
         if (collector) {
-            // the shift of the next step from the visible part of column t, which is complete
-            float vm = NEG_INF_F;
-#pragma unroll
-            for (int r = 0; r < NQ; r++) {
-                const int i = NLP * k + 64 * r + lane;
-                if (i < MP) vm = fmaxf(vm, cur[i]);
-            }
-            vm = wave_max(vm);
-            if (lane == 0) sm_Dv[(t - 1) & 1] = vm;
-            if (t > 1) {  // column t-1 of the blocks above
+            if (t > 1) {  // column t-1 of the blocks above, requested one iteration ago
                 const unsigned long long *src = Xf + (size_t)(t - 1) * MP + NLP * (k + 1) + lane;
-                unsigned long long x[NQ];
+                // the requests went out for every lane (a branch around a load ends in a wait for it); entries beyond the
+                // sentence are never written and read as -inf
 #pragma unroll
-                for (int r = 0; r < NQ; r++) {
-                    const int i = NLP * (k + 1) + 64 * r + lane;
-                    x[r] = (i < mc) ? entry_load(src + 64 * r) : (unsigned long long)__double_as_longlong(-__builtin_huge_val());
-                }
+                for (int r = 0; r < NQ; r++)
+                    if (NLP * (k + 1) + 64 * r + lane >= mc) x[r] = MINUS_INF64;
                 for (int spins = 0;; spins++) {
                     bool pending = false;
 #pragma unroll
@@ -1666,6 +1663,19 @@ __global__ __launch_bounds__(NTP) void inside_fwd_ml1_pipe_kernel(const float *_
                     if (i < MP) nxt[i] = (x[r] == EMPTY64) ? NEG_INF_F : (float)(__longlong_as_double((long long)x[r]) - O_new);
                 }
             }
+            if (t > 2) {  // request column t-2 now: it has the whole next step to arrive
+#pragma unroll
+                for (int r = 0; r < NQ; r++) x[r] = entry_load(Xf + (size_t)(t - 2) * MP + NLP * (k + 1) + 64 * r + lane);
+            }
+            // the shift of the next step from the visible part of column t, which is complete
+            float vm = NEG_INF_F;
+#pragma unroll
+            for (int r = 0; r < NQ; r++) {
+                const int i = NLP * k + 64 * r + lane;
+                if (i < MP) vm = fmaxf(vm, cur[i]);
+            }
+            vm = wave_max(vm);
+            if (lane == 0) sm_Dv[(t - 1) & 1] = vm;
         } else {
             // the next column's emissions: from LDS, or requested now so that they travel during the column's work
             float ma_raw = 0.f, ml_raw = 0.f;
@@ -1858,20 +1868,28 @@ __global__ __launch_bounds__(NTP) void inside_bwd_ml1_pipe_kernel(const float *_
     __syncthreads();
 
     unsigned *Xb = xv.bw;
+    unsigned x0[NQ], x1[NQ];  // collector: the entries of the blocks below, requested one step before they are handed on
+#pragma unroll
+    for (int r = 0; r < NQ; r++) {
+        const bool need = collector && k > 0 && n >= 3;
+        x0[r] = need ? entry_load(Xb + (size_t)2 * 2 * MP + 64 * r + lane) : __float_as_uint(NEG_INF_F);
+        x1[r] = need ? entry_load(Xb + (size_t)2 * 2 * MP + MP + 64 * r + lane) : __float_as_uint(NEG_INF_F);
+    }
     for (int t = 1; t <= n - 1; t++) {
         const float *c0 = w0[t & 1], *c1 = w1[t & 1];
         float *n0 = w0[(t + 1) & 1], *n1 = w1[(t + 1) & 1];
         const bool more = t < n - 1;
         if (collector) {
-            if (more && k > 0) {  // the weights of the blocks below for column t+1
+            if (more && k > 0) {  // the weights of the blocks below for column t+1, requested one iteration ago
                 const unsigned *src = Xb + (size_t)(t + 1) * 2 * MP + lane;
-                unsigned x0[NQ], x1[NQ];
-                const int end = min(NLP * k, mc);
+                // the requests went out for every lane (a branch around a load ends in a wait for it); entries of other
+                // blocks' nodes beyond the sentence are never written and read as -inf
 #pragma unroll
                 for (int r = 0; r < NQ; r++) {
-                    const bool need = 64 * r + lane < end;
-                    x0[r] = need ? entry_load(src + 64 * r) : __float_as_uint(NEG_INF_F);
-                    x1[r] = need ? entry_load(src + MP + 64 * r) : __float_as_uint(NEG_INF_F);
+                    if (64 * r + lane >= min(NLP * k, mc)) {
+                        x0[r] = __float_as_uint(NEG_INF_F);
+                        x1[r] = __float_as_uint(NEG_INF_F);
+                    }
                 }
                 for (int spins = 0;; spins++) {
                     bool pending = false;
@@ -1896,6 +1914,14 @@ __global__ __launch_bounds__(NTP) void inside_bwd_ml1_pipe_kernel(const float *_
                         n0[i] = (x0[r] == EMPTY32) ? NEG_INF_F : __uint_as_float(x0[r]);
                         n1[i] = (x1[r] == EMPTY32) ? NEG_INF_F : __uint_as_float(x1[r]);
                     }
+                }
+            }
+            if (t + 2 <= n - 1 && k > 0) {  // request column t+2 now: it has the whole next step to arrive
+                const unsigned *src = Xb + (size_t)(t + 2) * 2 * MP + lane;
+#pragma unroll
+                for (int r = 0; r < NQ; r++) {
+                    x0[r] = entry_load(src + 64 * r);
+                    x1[r] = entry_load(src + MP + 64 * r);
                 }
             }
         } else {
