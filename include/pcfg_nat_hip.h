@@ -137,7 +137,8 @@ int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *ma
                                        void *stream);
 
 /*
- * No counterpart in the reference: tuning of the long-graph path (max_left = 1, 258 <= L <= 1026).  There a sentence is
+ * No counterpart in the reference: tuning of the long-graph paths (max_left = 1; inside sweeps for 258 <= L <= 1026, the
+ * Viterbi sweep of pcfgnat_viterbi_decode for 194 <= L <= 514).  There a sentence is
  * swept by one workgroup per block of 16 main-chain nodes, the blocks following each other as a pipeline, as long as the
  * batch needs no more than max_workgroups of them (B * 4 * ceil((L/2)/64) <= max_workgroups, default 1024), and by one
  * workgroup per sentence otherwise.  A block that waits for the one ahead of it for more than spin_limit rounds of polling
@@ -288,9 +289,11 @@ int pcfgnat_viterbi_decoding(const int64_t *pred_length, const int64_t *output_l
  * The whole Viterbi decode of glat_decomposed_with_link_two_hands_tri_pcfg.py:483-502 in one call: tables
  * (pcfg_viterbi.cu:272-301), length selection pred_length = 1 + argmax_{len >= 1} S[b,1,len] / length_penalty[len] with NaN
  * read as -inf and the first maximum winning (:489-497), and the walk (pcfg_loss.cpp:12-73).  length_penalty [L/4] float32
- * is the caller's arange(L/4) ** decode_viterbibeta.  For max_left = 1 and graphs of up to 514 nodes this is a single
- * launch whose traces are one int32 per cell in `workspace`; otherwise the three steps run back to back on full
- * tables in `workspace`.  workspace: pcfgnat_viterbi_decode_workspace_bytes(B, L, max_left) bytes, 8-byte aligned.
+ * is the caller's arange(L/4) ** decode_viterbibeta.  For max_left = 1 and graphs of up to 514 nodes the traces are one
+ * int32 per cell in `workspace` and the call is a single launch, or - from about 200 nodes on, see pcfgnat_cluster_config -
+ * a sweep by a pipeline of workgroups per sentence followed by the selection and the walk; otherwise the three steps run
+ * back to back on full tables in `workspace`.  workspace: pcfgnat_viterbi_decode_workspace_bytes(B, L, max_left) bytes,
+ * 8-byte aligned.
  *   out_tokens [B,L] int64, out_count [B] int64 (as pcfgnat_viterbi_decoding), pred_length [B] int64.
  */
 size_t pcfgnat_viterbi_decode_workspace_bytes(int64_t B, int64_t L, int64_t ml);

@@ -59,6 +59,11 @@ int lsg_forward_lse_force(const void *logits, int dtype, const int64_t *targets,
                           const int64_t *output_length, const int64_t *target_length, const unsigned char *matchmask,
                           const unsigned char *keep, int64_t B, int64_t L, int64_t V, int64_t T, void *stream);
 
+// Settings of pcfgnat_cluster_config (inside.hip): the most workgroups a pipelined sweep may use (0 = pipelines off) and the
+// bound on a block's wait for the one ahead of it, in rounds of polling
+int pipeline_max_workgroups();
+int pipeline_spin_limit();
+
 // General max_left (generic_ml.hip)
 size_t generic_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml);
 int generic_forward(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int64_t B,
@@ -194,6 +199,24 @@ __device__ __forceinline__ void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+
+// Exchange between the workgroups of one launch (pipelined sweeps): table entries are written once with a device-scope
+// store by their owner and polled with device-scope loads by the readers; an all-ones bit pattern, with which the tables
+// are filled by an earlier launch, marks an entry that has not arrived.
+constexpr unsigned EMPTY32 = 0xFFFFFFFFu;
+constexpr unsigned long long EMPTY64 = ~0ull;
+
+__device__ __forceinline__ unsigned long long entry_load(const unsigned long long *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned entry_load(const unsigned *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void entry_store(unsigned long long *p, double v) {
+    __hip_atomic_store(p, (unsigned long long)__double_as_longlong(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void entry_store(unsigned *p, float v) {
+    __hip_atomic_store(p, __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ bool gave_up(const int *flag) { return __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0; }
 
 // Phase timestamps for tuning builds only (-DPCFGNAT_PHASE_TIMING): thread 0 of workgroup 0 stores the 100 MHz wall clock.
 #ifdef PCFGNAT_PHASE_TIMING

@@ -1471,21 +1471,6 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
 // ------------------------------------------------------------------------------------------------------------
 constexpr int NLP = 16;             // nodes per block
 constexpr int NTP = 16 * NLP + 64;  // four compute waves and the collector wave
-constexpr unsigned EMPTY32 = 0xFFFFFFFFu;
-constexpr unsigned long long EMPTY64 = ~0ull;
-
-__device__ __forceinline__ unsigned long long entry_load(const unsigned long long *p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ unsigned entry_load(const unsigned *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ void entry_store(unsigned long long *p, double v) {
-    __hip_atomic_store(p, (unsigned long long)__double_as_longlong(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void entry_store(unsigned *p, float v) {
-    __hip_atomic_store(p, __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ bool gave_up(const int *flag) { return __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0; }
-
 // stream_row_lse on link rows held in registers: chunks q in [qa, qb) of the NQ the lane holds (both wave-uniform).
 template <int NQ, bool JOINT>
 __device__ __forceinline__ void slab_row_lse(const float4 (&A0)[NQ], const float4 (&A1)[NQ], const float4 *u0, const float4 *u1, int qa,
@@ -2254,6 +2239,9 @@ int check_dims(const char *who, int64_t B, int64_t L, int64_t T, int64_t ml) {
 }  // namespace pcfgnat
 
 using namespace pcfgnat;
+
+int pcfgnat::pipeline_max_workgroups() { return g_cluster_max_wg.load(); }
+int pcfgnat::pipeline_spin_limit() { return g_cluster_spin_limit.load(); }
 
 extern "C" void pcfgnat_cluster_config(int max_workgroups, int spin_limit) {
     if (max_workgroups >= 0) g_cluster_max_wg.store(max_workgroups);

@@ -167,6 +167,10 @@ struct DecodeArgs {
     int *W;                        // [B][L/2][Lq] workspace
     int64_t *out_tokens, *out_count, *pred_length;
     int64_t mask_dim, pad;
+    // set when the pipelined sweep has run before this kernel: sentences whose flag is down only need the length
+    // selection (root scores [B][Lq]) and the walk, the others are redone from scratch
+    const int *pipe_flags;
+    const float *pipe_scores;
 };
 
 template <int NQ, bool COMPACT>
@@ -189,10 +193,12 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
     const int rowsW = L / 2;
     int *Wb = COMPACT ? dec.W + (size_t)b * rowsW * Lq : nullptr;
     const bool in_contract = !(m < 2 || m > L || (m % 2) != 0);
+    const bool from_pipe = COMPACT && dec.pipe_flags != nullptr && dec.pipe_flags[b] == 0;  // workgroup-uniform
 
     if (COMPACT) {
-        for (int i = tid; i < rowsW * Lq; i += NT) Wb[i] = 0;
-        for (int i = tid; i < Lq; i += NT) sm_scores[i] = NEG_INF_F;
+        if (!from_pipe)
+            for (int i = tid; i < rowsW * Lq; i += NT) Wb[i] = 0;
+        for (int i = tid; i < Lq; i += NT) sm_scores[i] = from_pipe ? dec.pipe_scores[(size_t)b * Lq + i] : NEG_INF_F;
         for (int i = tid; i < L; i += NT) dec.out_tokens[(size_t)b * L + i] = dec.pad;
     } else {
         // tables start as -inf / 0 (pcfg_viterbi.cu:159, 287-289)
@@ -204,7 +210,7 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
         }
         if (!in_contract) return;  // out of contract: leave the empty tables
     }
-    if (in_contract) {
+    if (in_contract && !from_pipe) {
     const int mc = m / 2;
 
     // slabs: unconditional loads from clamped addresses (all in flight together), masked afterwards
@@ -338,6 +344,163 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
                 dec.out_count[b] = readout_one(pl, out_len[b], tr, dec.tokens + (size_t)b * L, dec.mask, dec.mask_dim, dec.pad,
                                                dec.out_tokens + (size_t)b * L, stack_node, stack_len, L, Lq);
             }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Pipelined sweep for the single-call decode of long graphs (same idea as the pipelined inside sweeps): the main chain is
+// cut into blocks of 16 parents, one workgroup per block - four compute waves (one 16-lane row per parent, its
+// triangular link slabs in registers) and one collector wave.  A parent combines children c >= a only, so the top
+// block runs free and every other block follows the one above at the distance of one exchange through memory; the
+// score table travels through X [B][Lq][16*NQ] (one entry per length and node, written once by its owner, all ones =
+// not arrived, filled by viterbi_pipe_fill_kernel).  The sweep leaves the back-pointer records W and the root's scores;
+// viterbi_ml1_kernel<NQ, true> then selects the length and walks the tree (and redoes a sentence whose blocks gave up).
+// Values and arg-max decisions are those of viterbi_ml1_kernel: same candidate order inside a lane, same tie key.
+// ------------------------------------------------------------------------------------------------------------
+constexpr int VP_NT = 16 * 16 + 64;
+
+__global__ __launch_bounds__(256) void viterbi_pipe_fill_kernel(unsigned *X, size_t nx, int *W, size_t nw, float *scores, size_t ns,
+                                                               int *flags, int B) {
+    const size_t me = (size_t)blockIdx.x * 256 + threadIdx.x, all = (size_t)gridDim.x * 256;
+    for (size_t i = me; i < nx; i += all) X[i] = EMPTY32;
+    for (size_t i = me; i < nw; i += all) W[i] = 0;
+    for (size_t i = me; i < ns; i += all) scores[i] = NEG_INF_F;
+    if (me < (size_t)B) flags[me] = 0;
+}
+
+template <int NQ>
+__global__ __launch_bounds__(VP_NT) void viterbi_ml1_pipe_kernel(const float *__restrict__ ob_lprob, const float *__restrict__ links,
+                                                                const int64_t *__restrict__ out_len, int L, int Lq,
+                                                                unsigned *__restrict__ X, float *__restrict__ scores,
+                                                                int *__restrict__ W, int *__restrict__ flags, int spin_limit) {
+    constexpr int MP = 16 * NQ, RQ = (NQ + 3) / 4;  // RQ loads of 64 entries cover a column
+    __shared__ float col[3 * MP];
+    __shared__ int sm_dead;
+    const int b = blockIdx.x / NQ, k = NQ - 1 - blockIdx.x % NQ;  // the leading (highest) block first
+    const int tid = threadIdx.x, gidx = (tid >> 4) & 15, j16 = tid & 15, lane = tid & 63;
+    const bool collector = tid >= 256;
+    const int m = (int)out_len[b];
+    if (m < 2 || m > L || (m % 2) != 0) return;  // out of contract: the empty tables stay
+    const int mc = m / 2;
+    if (16 * k >= mc) return;  // no node of the sentence in this block: nobody waits for it
+    const float *ob = ob_lprob + (size_t)b * L;
+    const float *lk = links + (size_t)b * L * 2 * L;
+    unsigned *Xb = X + (size_t)b * Lq * MP;
+    int *Wb = W + (size_t)b * (L / 2) * Lq;
+
+    // slabs: unconditional loads from clamped addresses (all in flight together), masked afterwards
+    const int a_id = 16 * k + gidx, a = 2 * min(a_id, mc - 1) + 1;
+    float A0[NQ], A1[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+        if (q >= k) {
+            const int c = 2 * min(j16 + 16 * q, mc - 1) + 1;
+            A0[q] = lk[((size_t)a * 2 + 0) * L + c];
+            A1[q] = lk[((size_t)a * 2 + 1) * L + c];
+        }
+    }
+    const float oa = ob[a], ol = ob[a - 1];
+    const float ob_a = (a_id < mc) ? oa : NEG_INF_F;
+    const float ob_leaf = (a_id < mc && a_id >= 1) ? ol : NEG_INF_F;
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+        if (q >= k) {
+            const int c_id = j16 + 16 * q;
+            const bool ok = a_id < mc && c_id < mc && c_id >= a_id;
+            A0[q] = ok ? A0[q] + 0.f : NEG_INF_F;
+            A1[q] = (ok && a_id >= 1) ? A1[q] + ob_leaf : NEG_INF_F;
+        }
+    }
+    // length 0: nothing; length 1: only the last node (pcfg_viterbi.cu:57-59)
+    for (int i = tid; i < 3 * MP; i += VP_NT) col[i] = (i == 1 * MP + mc - 1) ? ob[m - 1] : NEG_INF_F;
+    if (tid == 0) {
+        sm_dead = 0;
+        if (k == 0 && Lq > 1 && m - 1 == 1) scores[(size_t)b * Lq + 1] = ob[m - 1];
+    }
+    const int len_end = m / 4;  // pcfg_viterbi.cu:67
+    // collector: the entries of the blocks above are requested one step before they are handed on
+    unsigned x[RQ];
+#pragma unroll
+    for (int r = 0; r < RQ; r++)
+        x[r] = (collector && len_end > 2) ? entry_load(Xb + (size_t)2 * MP + 16 * (k + 1) + 64 * r + lane) : __float_as_uint(NEG_INF_F);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the slabs have arrived before the sweep starts
+    __syncthreads();
+
+    for (int len = 2; len < len_end; len++) {
+        const float *cur1 = col + ((len - 1) % 3) * MP, *cur2 = col + ((len - 2) % 3) * MP;
+        float *nxt = col + (len % 3) * MP;
+        if (collector) {
+            // length len of the blocks above; the requests went out for every lane, entries beyond the sentence or the
+            // padded row are never written and read as -inf
+#pragma unroll
+            for (int r = 0; r < RQ; r++)
+                if (16 * (k + 1) + 64 * r + lane >= mc) x[r] = __float_as_uint(NEG_INF_F);
+            for (int spins = 0;; spins++) {
+                bool pending = false;
+#pragma unroll
+                for (int r = 0; r < RQ; r++) pending |= (x[r] == EMPTY32);
+                if (!__any(pending)) break;
+                if (spins >= spin_limit || ((spins & 63) == 63 && gave_up(flags + b))) {
+                    sm_dead = 1;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
+#pragma unroll
+                for (int r = 0; r < RQ; r++)
+                    if (x[r] == EMPTY32) x[r] = entry_load(Xb + (size_t)len * MP + 16 * (k + 1) + 64 * r + lane);
+            }
+#pragma unroll
+            for (int r = 0; r < RQ; r++) {
+                const int i = 16 * (k + 1) + 64 * r + lane;
+                if (i < MP) nxt[i] = (x[r] == EMPTY32) ? NEG_INF_F : __uint_as_float(x[r]);
+            }
+            if (len + 1 < len_end) {
+#pragma unroll
+                for (int r = 0; r < RQ; r++) x[r] = entry_load(Xb + (size_t)(len + 1) * MP + 16 * (k + 1) + 64 * r + lane);
+            }
+        } else {
+            float best = NEG_INF_F;
+            int sel = -1;
+#pragma unroll
+            for (int q = 0; q < NQ; q++) {
+                if (q >= k) {
+                    const float c0 = (A0[q] + cur1[j16 + 16 * q]) + ob_a;
+                    const float c1 = (A1[q] + cur2[j16 + 16 * q]) + ob_a;
+                    if (c0 > best) {  // false for NaN and for -inf against the initial -inf
+                        best = c0;
+                        sel = 2 * q;
+                    }
+                    if (c1 > best) {
+                        best = c1;
+                        sel = 2 * q + 1;
+                    }
+                }
+            }
+            // row maximum first, then the smallest tie key among the lanes that hold it
+            const float mine = best;
+            best = row16_max_raw(best);
+            int key = (sel < 0 || mine != best) ? 0x7fffffff : tie_key(j16 + 16 * (sel >> 1) - a_id, sel & 1);
+            key = min(key, dpp_i<DPP_QUAD_XOR1>(key));
+            key = min(key, dpp_i<DPP_QUAD_XOR2>(key));
+            key = min(key, dpp_i<DPP_ROW_HALF_MIRROR>(key));
+            key = min(key, dpp_i<DPP_ROW_MIRROR>(key));
+            if (j16 == 0) {
+                nxt[a_id] = best;
+                if (a_id < mc) {
+                    entry_store(Xb + (size_t)len * MP + a_id, best);
+                    if (best != NEG_INF_F) {  // pcfg_viterbi.cu:125-131
+                        const int jj = key & 1, rel = (key >> 1) & 0x7fffff;
+                        Wb[(unsigned)(a_id * Lq + len)] = 1 + ((rel << 1) | jj);
+                        if (a_id == 0) scores[(size_t)b * Lq + len] = best;
+                    }
+                }
+            }
+        }
+        lds_barrier();
+        if (sm_dead) {  // uniform: written before the barrier
+            if (tid == 0) __hip_atomic_store(flags + b, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
         }
     }
 }
@@ -578,12 +741,51 @@ extern "C" int pcfgnat_pcfg_viterbi(const float *ob_lprob, const float *links, c
 namespace {
 // the single-launch decode applies to max_left = 1 graphs whose slabs fit in registers
 bool decode_is_fused(int64_t L, int64_t ml) { return ml == 1 && (L - 2) / 2 + 1 <= 256; }
+// 16-node chunks of the main chain, rounded to the kernels that exist (2, 4, .., 16)
+int decode_chunks(int64_t L) { return 2 * (int)(((L - 2) / 2 + 1 + 31) / 32); }
+// The pipelined sweep pays from about 200 graph nodes on while every block gets a compute unit of its own, from about
+// 260 nodes otherwise (measured: batch 1, 240 nodes 132 -> 123 us per call, 400 nodes 322 -> 192 us; batch 64, 200 nodes
+// 125 -> 134 us, 400 nodes 338 -> 231 us); below that one workgroup is through before a pipeline has filled.
+bool decode_pipelined(int NQ, int64_t B) {
+    if (B * NQ > pipeline_max_workgroups()) return false;
+    return NQ >= 10 || (NQ >= 8 && B * NQ <= 256);
+}
+
+template <int NQ>
+int launch_decode(const float *ob_lprob, const float *links, const int64_t *output_length, DecodeArgs dec, void *workspace, int64_t B,
+                  int64_t L, hipStream_t s) {
+    const int Lq = (int)(L / 4);
+    const size_t dyn = ((size_t)Lq + 2 * (size_t)L) * sizeof(int);
+    const size_t nw = (size_t)B * (size_t)(L / 2) * Lq, nx = (size_t)B * Lq * 16 * NQ, ns = (size_t)B * Lq;
+    if (decode_pipelined(NQ, B)) {
+        int *W = (int *)workspace;
+        unsigned *X = (unsigned *)(W + nw);
+        float *scores = (float *)(X + nx);
+        int *flags = (int *)(scores + ns);
+        const size_t total = nw + nx + ns;
+        const unsigned fill_blocks = (unsigned)((total / 4 + 255) / 256 < 1024 ? (total / 4 + 255) / 256 : 1024);
+        hipLaunchKernelGGL(viterbi_pipe_fill_kernel, dim3(fill_blocks ? fill_blocks : 1), dim3(256), 0, s, X, nx, W, nw, scores, ns, flags,
+                           (int)B);
+        PCFGNAT_HIP_CHECK(hipGetLastError());
+        hipLaunchKernelGGL(viterbi_ml1_pipe_kernel<NQ>, dim3((unsigned)(B * NQ)), dim3(VP_NT), 0, s, ob_lprob, links, output_length, (int)L,
+                           Lq, X, scores, W, flags, pipeline_spin_limit());
+        PCFGNAT_HIP_CHECK(hipGetLastError());
+        dec.pipe_flags = flags;
+        dec.pipe_scores = scores;
+    }
+    hipLaunchKernelGGL((viterbi_ml1_kernel<NQ, true>), dim3((unsigned)B), dim3(NT), dyn, s, ob_lprob, links, output_length, nullptr, nullptr,
+                       nullptr, nullptr, (int)L, Lq, dec);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
+}
 }  // namespace
 
 extern "C" size_t pcfgnat_viterbi_decode_workspace_bytes(int64_t B, int64_t L, int64_t ml) {
     if (B <= 0 || L < 4) return 0;
     const size_t Lq = (size_t)(L / 4);
-    if (decode_is_fused(L, ml)) return (size_t)B * (size_t)(L / 2) * Lq * sizeof(int);
+    // back-pointer records [B][L/2][Lq], then (pipelined sweep) the score exchange [B][Lq][16*chunks], root scores [B][Lq], flags [B]
+    if (decode_is_fused(L, ml))
+        return ((size_t)B * (size_t)(L / 2) * Lq + (size_t)B * Lq * 16 * decode_chunks(L) + (size_t)B * Lq + (size_t)B) * sizeof(int);
     // full tables S (float) + R, L, M (int64), then the walk stacks [B][2L] int64
     return (size_t)B * L * Lq * (sizeof(float) + 3 * sizeof(int64_t)) + (size_t)B * 2 * L * sizeof(int64_t);
 }
@@ -603,26 +805,18 @@ extern "C" int pcfgnat_viterbi_decode(const float *ob_lprob, const float *links,
     hipStream_t s = (hipStream_t)stream;
     const int Lq = (int)(L / 4);
     if (decode_is_fused(L, ml)) {
-        const int Mc = (int)((L - 2) / 2 + 1);
-        DecodeArgs dec{tokens, left_tree_mask, length_penalty, (int *)workspace, out_tokens, out_count, pred_length, mask_dim, pad_index};
-        const size_t dyn = ((size_t)Lq + 2 * (size_t)L) * sizeof(int);
-#define PCFGNAT_DECODE_CASE(nq)                                                                                                 \
-    else if (Mc <= 16 * (nq))                                                                                                   \
-        hipLaunchKernelGGL((viterbi_ml1_kernel<nq, true>), dim3((unsigned)B), dim3(NT), dyn, s, ob_lprob, links, output_length, nullptr, \
-                           nullptr, nullptr, nullptr, (int)L, Lq, dec)
-        if (false) {
+        DecodeArgs dec{tokens,     left_tree_mask, length_penalty, (int *)workspace, out_tokens, out_count,
+                       pred_length, mask_dim,       pad_index,      nullptr,          nullptr};
+        switch (decode_chunks(L)) {
+            case 2: return launch_decode<2>(ob_lprob, links, output_length, dec, workspace, B, L, s);
+            case 4: return launch_decode<4>(ob_lprob, links, output_length, dec, workspace, B, L, s);
+            case 6: return launch_decode<6>(ob_lprob, links, output_length, dec, workspace, B, L, s);
+            case 8: return launch_decode<8>(ob_lprob, links, output_length, dec, workspace, B, L, s);
+            case 10: return launch_decode<10>(ob_lprob, links, output_length, dec, workspace, B, L, s);
+            case 12: return launch_decode<12>(ob_lprob, links, output_length, dec, workspace, B, L, s);
+            case 14: return launch_decode<14>(ob_lprob, links, output_length, dec, workspace, B, L, s);
+            default: return launch_decode<16>(ob_lprob, links, output_length, dec, workspace, B, L, s);
         }
-        PCFGNAT_DECODE_CASE(2);
-        PCFGNAT_DECODE_CASE(4);
-        PCFGNAT_DECODE_CASE(6);
-        PCFGNAT_DECODE_CASE(8);
-        PCFGNAT_DECODE_CASE(10);
-        PCFGNAT_DECODE_CASE(12);
-        PCFGNAT_DECODE_CASE(14);
-        PCFGNAT_DECODE_CASE(16);
-#undef PCFGNAT_DECODE_CASE
-        PCFGNAT_HIP_CHECK(hipGetLastError());
-        return PCFGNAT_OK;
     }
     // general path: full tables in the workspace, then selection and walk as separate launches
     const size_t cells = (size_t)B * L * Lq;

@@ -477,6 +477,29 @@ def test_viterbi_tables_bit_exact_and_decode(case):
         assert got_tok.dtype == torch.float32 and torch.equal(got_tok.cpu(), want_tok)
 
 
+@pytest.mark.parametrize("mode", ["one_workgroup", "blocks_give_up"])
+@pytest.mark.parametrize("case", ["L224", "L288", "L400", "L512"])
+def test_single_call_decode_sweeps_agree(mode, case):
+    """Graphs of 194..514 nodes: the pipelined Viterbi sweep (default), the one-workgroup sweep (pipeline switched off) and
+    the redo path (blocks that give up at once: spin limit 0) return the same tokens and lengths as the oracle."""
+    import oracle_ops
+    batch = _decode_case(case)
+    ob, tok = synth.ob_and_tokens(batch["logits"])
+    links, ol = batch["links"], batch["output_length"]
+    left_mask, _, _ = synth.support_masks(links.shape[1], 1)
+    want_tok, want_len = harness.viterbi_decode(ob, tok, links, ol, left_mask, ops=oracle_ops)
+    try:
+        if mode == "one_workgroup":
+            ops.cluster_config(max_workgroups=0)
+        else:
+            ops.cluster_config(spin_limit=0)
+        got_tok, got_len = harness.viterbi_decode(ob.to(DEV), tok.to(DEV), links.to(DEV), ol.to(DEV), left_mask.to(DEV),
+                                                  single_call=True)
+    finally:
+        ops.cluster_config(max_workgroups=1024, spin_limit=1 << 20)
+    assert torch.equal(got_len.cpu(), want_len) and torch.equal(got_tok.cpu(), want_tok)
+
+
 @pytest.mark.parametrize("ml,L,ms", [(1, 32, [32, 20, 8]), (3, 34, [34, 26]), (1, 400, [400, 284, 20, 400]), (1, 18, [18])])
 @pytest.mark.parametrize("strategy", ["lookahead", "greedy"])
 def test_lookahead_decode_bit_exact(ml, L, ms, strategy):
