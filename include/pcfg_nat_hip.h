@@ -146,7 +146,7 @@ int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *ma
  * are the same either way up to fp32 rounding.  max_workgroups = 0 switches the pipeline off; a negative argument leaves
  * that setting unchanged.  Process-wide, takes effect with the next call.
  */
-void pcfgnat_cluster_config(int max_workgroups, int spin_limit);
+void pcfgnat_pipeline_config(int max_workgroups, int spin_limit);
 
 /*
  * The float64 instantiation the reference also dispatches (AT_DISPATCH_FLOATING_TYPES in pcfg_loss.cu:395,
@@ -290,7 +290,7 @@ int pcfgnat_viterbi_decoding(const int64_t *pred_length, const int64_t *output_l
  * (pcfg_viterbi.cu:272-301), length selection pred_length = 1 + argmax_{len >= 1} S[b,1,len] / length_penalty[len] with NaN
  * read as -inf and the first maximum winning (:489-497), and the walk (pcfg_loss.cpp:12-73).  length_penalty [L/4] float32
  * is the caller's arange(L/4) ** decode_viterbibeta.  For max_left = 1 and graphs of up to 514 nodes the traces are one
- * int32 per cell in `workspace` and the call is a single launch, or - from about 200 nodes on, see pcfgnat_cluster_config -
+ * int32 per cell in `workspace` and the call is a single launch, or - from about 200 nodes on, see pcfgnat_pipeline_config -
  * a sweep by a pipeline of workgroups per sentence followed by the selection and the walk; otherwise the three steps run
  * back to back on full tables in `workspace`.  workspace: pcfgnat_viterbi_decode_workspace_bytes(B, L, max_left) bytes,
  * 8-byte aligned.

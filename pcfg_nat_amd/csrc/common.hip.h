@@ -59,7 +59,7 @@ int lsg_forward_lse_force(const void *logits, int dtype, const int64_t *targets,
                           const int64_t *output_length, const int64_t *target_length, const unsigned char *matchmask,
                           const unsigned char *keep, int64_t B, int64_t L, int64_t V, int64_t T, void *stream);
 
-// Settings of pcfgnat_cluster_config (inside.hip): the most workgroups a pipelined sweep may use (0 = pipelines off) and the
+// Settings of pcfgnat_pipeline_config (inside.hip): the most workgroups a pipelined sweep may use (0 = pipelines off) and the
 // bound on a block's wait for the one ahead of it, in rounds of polling
 int pipeline_max_workgroups();
 int pipeline_spin_limit();

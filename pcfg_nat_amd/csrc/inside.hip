@@ -2051,15 +2051,15 @@ __global__ __launch_bounds__(256) void criterion_loss_kernel(const float *__rest
     criterion_loss_block<256>(LossTask{S, tgt_len, out, B, (int64_t)Mc * (T + 2)});
 }
 
-// The pipelined sweeps are used while a batch needs no more than g_cluster_max_wg workgroups.  The default is no limit in
+// The pipelined sweeps are used while a batch needs no more than g_pipeline_max_wg workgroups.  The default is no limit in
 // practice: measured at 512 graph nodes and 140 target tokens they beat one workgroup per sentence 3.5x at 16 sentences
 // and still 1.8x at 512 sentences (8192 workgroups: the blocks of a sentence are adjacent in dispatch order, leading
 // block first, so a block never waits for one that has not been started).  Both numbers can be changed through
-// pcfgnat_cluster_config.
-std::atomic<int> g_cluster_max_wg{1 << 20}, g_cluster_spin_limit{1 << 20};
+// pcfgnat_pipeline_config.
+std::atomic<int> g_pipeline_max_wg{1 << 20}, g_pipeline_spin_limit{1 << 20};
 int pipeline_chunks(int B, int T, int Mc) {  // NQ, or 0 where the pipelined sweeps do not apply
     const int NQ = stream_mp(Mc) / 64, CL = 64 * NQ / NLP;
-    return (NQ >= 3 && NQ <= 8 && T + 2 < 4096 && (int64_t)B * CL <= g_cluster_max_wg.load()) ? NQ : 0;
+    return (NQ >= 3 && NQ <= 8 && T + 2 < 4096 && (int64_t)B * CL <= g_pipeline_max_wg.load()) ? NQ : 0;
 }
 
 template <int NQ>
@@ -2071,10 +2071,10 @@ int launch_fwd_pipe(const float *match_all, const int64_t *ol, const int64_t *tl
         auto k = inside_fwd_ml1_pipe_kernel<NQ, true>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)match_bytes));
         hipLaunchKernelGGL(k, dim3(B * CL), dim3(NTP), match_bytes, stream, match_all, ol, tl, S, aux, L, T, Mc,
-                           g_cluster_spin_limit.load());
+                           g_pipeline_spin_limit.load());
     } else {
         hipLaunchKernelGGL((inside_fwd_ml1_pipe_kernel<NQ, false>), dim3(B * CL), dim3(NTP), 0, stream, match_all, ol, tl, S, aux, L, T,
-                           Mc, g_cluster_spin_limit.load());
+                           Mc, g_pipeline_spin_limit.load());
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL(pipeline_rebase_kernel, dim3(CL - 1, B), dim3(256), (size_t)(T + 2) * sizeof(double), stream, aux, ol, tl, L, T,
@@ -2091,10 +2091,10 @@ int launch_bwd_pipe(const float *S, float *aux, const float *match_all, const in
         auto k = inside_bwd_ml1_pipe_kernel<NQ, true>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_match));
         hipLaunchKernelGGL(k, dim3(B * CL), dim3(NTP), with_match, stream, S, aux, match_all, ol, tl, L, T, Mc,
-                           g_cluster_spin_limit.load());
+                           g_pipeline_spin_limit.load());
     } else {
         hipLaunchKernelGGL((inside_bwd_ml1_pipe_kernel<NQ, false>), dim3(B * CL), dim3(NTP), base, stream, S, aux, match_all, ol, tl, L,
-                           T, Mc, g_cluster_spin_limit.load());
+                           T, Mc, g_pipeline_spin_limit.load());
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
@@ -2243,12 +2243,12 @@ int check_dims(const char *who, int64_t B, int64_t L, int64_t T, int64_t ml) {
 
 using namespace pcfgnat;
 
-int pcfgnat::pipeline_max_workgroups() { return g_cluster_max_wg.load(); }
-int pcfgnat::pipeline_spin_limit() { return g_cluster_spin_limit.load(); }
+int pcfgnat::pipeline_max_workgroups() { return g_pipeline_max_wg.load(); }
+int pcfgnat::pipeline_spin_limit() { return g_pipeline_spin_limit.load(); }
 
-extern "C" void pcfgnat_cluster_config(int max_workgroups, int spin_limit) {
-    if (max_workgroups >= 0) g_cluster_max_wg.store(max_workgroups);
-    if (spin_limit >= 0) g_cluster_spin_limit.store(spin_limit);
+extern "C" void pcfgnat_pipeline_config(int max_workgroups, int spin_limit) {
+    if (max_workgroups >= 0) g_pipeline_max_wg.store(max_workgroups);
+    if (spin_limit >= 0) g_pipeline_spin_limit.store(spin_limit);
 }
 
 extern "C" size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml) {

@@ -258,12 +258,12 @@ def test_long_graph_sweeps_agree(mode, L, T, ms, ns):
     ll0, mg0, lg0 = _inside_all(batch, match)
     try:
         if mode == "one_workgroup":
-            ops.cluster_config(max_workgroups=0)
+            ops.pipeline_config(max_workgroups=0)
         else:
-            ops.cluster_config(spin_limit=0)
+            ops.pipeline_config(spin_limit=0)
         ll1, mg1, lg1 = _inside_all(batch, match)
     finally:
-        ops.cluster_config(max_workgroups=1 << 20, spin_limit=1 << 20)
+        ops.pipeline_config(max_workgroups=1 << 20, spin_limit=1 << 20)
     fin = torch.isfinite(ll0)
     assert fin.any() and torch.equal(fin, torch.isfinite(ll1))
     assert torch.allclose(ll0[fin], ll1[fin], rtol=1e-5)
@@ -490,13 +490,13 @@ def test_single_call_decode_sweeps_agree(mode, case):
     want_tok, want_len = harness.viterbi_decode(ob, tok, links, ol, left_mask, ops=oracle_ops)
     try:
         if mode == "one_workgroup":
-            ops.cluster_config(max_workgroups=0)
+            ops.pipeline_config(max_workgroups=0)
         else:
-            ops.cluster_config(spin_limit=0)
+            ops.pipeline_config(spin_limit=0)
         got_tok, got_len = harness.viterbi_decode(ob.to(DEV), tok.to(DEV), links.to(DEV), ol.to(DEV), left_mask.to(DEV),
                                                   single_call=True)
     finally:
-        ops.cluster_config(max_workgroups=1 << 20, spin_limit=1 << 20)
+        ops.pipeline_config(max_workgroups=1 << 20, spin_limit=1 << 20)
     assert torch.equal(got_len.cpu(), want_len) and torch.equal(got_tok.cpu(), want_tok)
 
 
