@@ -505,27 +505,8 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
         }
         __syncthreads();  // every original value at a target column is in LDS before any store to the row
 
-#pragma unroll
-        for (int i = 0; i < MAXC; i++) {
-            int c = tid + i * NT;
-            if (c < sp.nvec) {
-                CT v[EPV];
-                Elem<T>::unpack(buf[i], v);
-#pragma unroll
-                for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
-                store16(pv + c, Elem<T>::pack(v));
-            }
-        }
-        for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
-            CT v[EPV];
-            Elem<T>::unpack(load16(pv + c), v);
-#pragma unroll
-            for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
-            store16(pv + c, Elem<T>::pack(v));
-        }
-        if (ep >= 0) pr[ep] = Elem<T>::narrow((FROM_LOGITS ? rn.e(edge) : edge) * ns);
-
-        // scatter_add_ (pcfg_loss.py:177): the first occurrence of a column accumulates all its duplicates in order
+        // scatter_add_ (pcfg_loss.py:177): the first occurrence of a column accumulates all its duplicates in order.  Worked
+        // out here, from LDS only, while the row's chunks are still on their way.
         CT fix[FIX];
         bool lead[FIX];
 #pragma unroll
@@ -554,6 +535,27 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
                 }
             }
         }
+
+#pragma unroll
+        for (int i = 0; i < MAXC; i++) {
+            int c = tid + i * NT;
+            if (c < sp.nvec) {
+                CT v[EPV];
+                Elem<T>::unpack(buf[i], v);
+#pragma unroll
+                for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
+                store16(pv + c, Elem<T>::pack(v));
+            }
+        }
+        for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
+            CT v[EPV];
+            Elem<T>::unpack(load16(pv + c), v);
+#pragma unroll
+            for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
+            store16(pv + c, Elem<T>::pack(v));
+        }
+        if (ep >= 0) pr[ep] = Elem<T>::narrow((FROM_LOGITS ? rn.e(edge) : edge) * ns);
+
         // workgroup barrier (release/acquire at workgroup scope): the streamed stores of this row are ordered before the
         // patches of its target columns, which hit addresses other threads of the workgroup have just written
         __syncthreads();
