@@ -137,7 +137,7 @@ int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *ma
                                        void *stream);
 
 /*
- * No counterpart in the reference: tuning of the long-graph paths (max_left = 1; inside sweeps for 258 <= L <= 1026, the
+ * No counterpart in the reference: tuning of the long-graph paths (max_left = 1; inside sweeps for 130 <= L <= 1026, the
  * Viterbi sweep of pcfgnat_viterbi_decode for 194 <= L <= 514).  There a sentence is
  * swept by one workgroup per block of 16 main-chain nodes, the blocks following each other as a pipeline, as long as the
  * batch needs no more than max_workgroups of them (B * 4 * ceil((L/2)/64) <= max_workgroups, default 2^20), and by one

@@ -15,7 +15,7 @@
 // registers for the whole sweep (one 16-lane DPP row per node, lanes strided over the other index), the current
 // column of S (or of the outside weights) is exchanged through LDS, one workgroup barrier per target position.
 // The forward leaves F0/F1 behind so that the backward needs a single sweep: rule posteriors are accumulated in
-// registers, emission posteriors come from an element-wise epilogue.  Graphs of more than 256 nodes use the streaming
+// registers, emission posteriors come from an element-wise epilogue.  Graphs of more than 130 nodes use the streaming
 // or the pipelined sweeps further down (link rows from L2, or spread over several workgroups per sentence).
 #include "common.hip.h"
 
@@ -48,7 +48,7 @@ __device__ __forceinline__ float lse2(float a, float b) {
 //   rule      a -> c at column t:      links[a][k][c] + Wk_t[a] + R_t[c],   W0_t[a] = match[a][t-1] + Bh_{t-1}[a] - D_t,
 //                                      W1_t[a] = match[a-1][t-2] + match[a][t-1] + Bh_{t-2}[a] - D_t - D_{t-1}.
 //
-// Aux layout per sentence (Mc <= 128): F0h, F1h, Bh, R, each [Mc][T+2], then D [T+4]; log-domain values in base 2.
+// Aux layout per sentence (Mc <= 64): F0h, F1h, Bh, R, each [Mc][T+2], then D [T+4]; log-domain values in base 2.
 __host__ __device__ inline size_t aux_stride_reg(int Mc, int T) { return (size_t)4 * Mc * (T + 2) + (size_t)(T + 4); }
 struct AuxView {
     float *F0, *F1, *BETA, *SR, *D;
@@ -83,7 +83,7 @@ __device__ __forceinline__ bool lengths_ok(int m, int n, int L, int T) {
 }
 
 // ------------------------------------------------------------------------------------------------------------
-// Register-resident sweeps (Mc <= 128).  512 threads = 8 waves; a node is owned by an 8-lane group (two groups per DPP
+// Register-resident sweeps (Mc <= 64 in use; the kernels take up to 128 nodes with R = 2).  512 threads = 8 waves; a node is owned by an 8-lane group (two groups per DPP
 // row), the 8 lanes stride over the other index in chunks of 8.  Link slabs are triangular (children c >= a), so wave w
 // takes node block perm(w) = {0,1,2,3,7,6,5,4}[w] of every 64-node tile: the two waves that share a SIMD (w, w+4) then
 // own blocks p and 7-p and together always process 9 of the 16 chunks, whole chunks below the diagonal being skipped
@@ -970,13 +970,14 @@ __global__ __launch_bounds__(BT_NT) void best_tree_ml1_kernel(const float *__res
 }
 
 // ------------------------------------------------------------------------------------------------------------
-// Streaming variants for graphs whose link slabs do not fit in registers (Mc > 128): same sweeps, but the link
+// Streaming variants for longer graphs (Mc > 64; the redo path of the pipelined sweeps up to 512 nodes and the only path
+// beyond): same sweeps, but the link
 // values are fetched from L2 every step (forward: straight from `links`; backward: from a compact transposed copy
 // so that lanes read consecutive parents), rows are processed in tiles of 64, and the row reductions are online
 // log-sum-exps over chunks of children.  Rule posteriors are produced by a separate, fully parallel kernel from the
 // outside weights the sweep leaves behind.
 // All tables are relative to the column offsets described at the top of this file (natural logarithms here).
-// Aux layout per sentence (Mc > 128), log-domain values in base 2 like everything inside these kernels: F0h, F1h, Bh,
+// Aux layout per sentence (Mc > 64), log-domain values in base 2 like everything inside these kernels: F0h, F1h, Bh,
 // W0, W1, R [Mc][T+2] each, D [T+4], padding to a 16-byte boundary, then the compact link matrices (times log2 e) with
 // masked entries already -inf and rows padded to MP = 64*ceil(Mc/64) floats:
 // Ac [2][Mc][MP] by parent (Ac[k][a][c]) for the forward sweep and At [2][Mc][MP] by child (At[k][c][a]) for the
@@ -1439,7 +1440,7 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
 }
 
 // ------------------------------------------------------------------------------------------------------------
-// Pipelined sweeps (128 < Mc <= 512, batches of few sentences): a sentence's nodes are cut into blocks of 16, one
+// Pipelined sweeps (64 < Mc <= 512): a sentence's nodes are cut into blocks of 16, one
 // workgroup per block: four compute waves (16 lanes per node, the node's two link rows in registers for the whole sweep,
 // NQ = MP/64 float4 per lane and plane) and one collector wave.  One workgroup per sentence is bound by the instruction
 // issue of one compute unit and by fetching the link rows from L2 for every column; here every block has a compute
@@ -2059,7 +2060,7 @@ __global__ __launch_bounds__(256) void criterion_loss_kernel(const float *__rest
 std::atomic<int> g_pipeline_max_wg{1 << 20}, g_pipeline_spin_limit{1 << 20};
 int pipeline_chunks(int B, int T, int Mc) {  // NQ, or 0 where the pipelined sweeps do not apply
     const int NQ = stream_mp(Mc) / 64, CL = 64 * NQ / NLP;
-    return (NQ >= 3 && NQ <= 8 && T + 2 < 4096 && (int64_t)B * CL <= g_pipeline_max_wg.load()) ? NQ : 0;
+    return (NQ >= 2 && NQ <= 8 && T + 2 < 4096 && (int64_t)B * CL <= g_pipeline_max_wg.load()) ? NQ : 0;
 }
 
 template <int NQ>
@@ -2110,6 +2111,7 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
     const int NQ = pipeline_chunks(B, T, Mc);
     int rc = PCFGNAT_OK;
     switch (NQ) {
+        case 2: rc = launch_fwd_pipe<2>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
         case 3: rc = launch_fwd_pipe<3>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
         case 4: rc = launch_fwd_pipe<4>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
         case 5: rc = launch_fwd_pipe<5>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
@@ -2144,6 +2146,7 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
     const int NQ = pipeline_chunks(B, T, Mc);
     int rc = PCFGNAT_OK;
     switch (NQ) {
+        case 2: rc = launch_bwd_pipe<2>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
         case 3: rc = launch_bwd_pipe<3>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
         case 4: rc = launch_bwd_pipe<4>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
         case 5: rc = launch_bwd_pipe<5>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
@@ -2255,7 +2258,7 @@ extern "C" size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64
     if (B <= 0 || L < 2 || T < 0 || ml < 0) return 0;
     if (ml != 1) return generic_aux_floats(B, L, T, ml);
     const int64_t Mc = (L - 2) / (ml + 1) + 1;
-    if (Mc <= 128) return (size_t)B * aux_stride_reg((int)Mc, (int)T);
+    if (Mc <= 64) return (size_t)B * aux_stride_reg((int)Mc, (int)T);
     return (size_t)B * aux_stride_stream((int)Mc, (int)T);
 }
 
@@ -2270,7 +2273,6 @@ extern "C" int pcfgnat_pcfg_loss(const float *match_all, const float *links, con
     const int Mc = (int)((L - 2) / 2 + 1);
     hipStream_t s = (hipStream_t)stream;
     if (Mc <= 64) return launch_fwd<1>(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s);
-    if (Mc <= 128) return launch_fwd<2>(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s);
     return launch_fwd_stream(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s);
 }
 
@@ -2289,9 +2291,6 @@ int pcfgnat::inside_backward_impl(const float *grad_output, const float *S, floa
     hipStream_t s = (hipStream_t)stream;
     if (Mc <= 64)
         return launch_bwd<1>(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
-                             (int)L, (int)T, Mc, (int)norm_B, s);
-    if (Mc <= 128)
-        return launch_bwd<2>(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
                              (int)L, (int)T, Mc, (int)norm_B, s);
     return launch_bwd_stream(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
                              (int)L, (int)T, Mc, (int)norm_B, s);
@@ -2321,9 +2320,6 @@ int pcfgnat::inside_forward_backward_impl(const float *grad_output, const float 
         // general max_left: the two plain kernels
     } else if (Mc <= 64)
         rc = launch_fused<1>(grad_output, match_all, links, output_length, target_length, S, match_all_grad, links_grad, (int)B, (int)L,
-                             (int)T, Mc, (int)norm_B, s, &done);
-    else if (Mc <= 128)
-        rc = launch_fused<2>(grad_output, match_all, links, output_length, target_length, S, match_all_grad, links_grad, (int)B, (int)L,
                              (int)T, Mc, (int)norm_B, s, &done);
     if (rc != PCFGNAT_OK || done) return rc;
     rc = pcfgnat_pcfg_loss(match_all, links, output_length, target_length, S, aux, B, L, T, ml, stream);

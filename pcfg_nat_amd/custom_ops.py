@@ -24,7 +24,7 @@ def get_pcfg_kernel():
 
 
 def pipeline_config(max_workgroups=None, spin_limit=None):
-    """Tuning of the long-graph inside sweeps (no counterpart in the reference): graphs of 258..1026 nodes are swept by
+    """Tuning of the long-graph inside sweeps (no counterpart in the reference): graphs of 130..1026 nodes are swept by
     one workgroup per block of 16 main-chain nodes, pipelined, while the batch needs no more than ``max_workgroups`` of
     them (default 2**20; 0 = always one workgroup per sentence).  ``spin_limit`` bounds the wait of a block for the one
     ahead of it (default 2**20 rounds of polling); a sentence whose blocks give up is redone by the one-workgroup sweep

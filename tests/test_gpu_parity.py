@@ -247,10 +247,11 @@ def _inside_all(batch, match):
 
 
 @pytest.mark.parametrize("mode", ["one_workgroup", "blocks_give_up"])
-@pytest.mark.parametrize("L,T,ms,ns", [(320, 40, [320, 262, 4], [40, 31, 2]), (512, 140, [512, 444], [140, 120]),
+@pytest.mark.parametrize("L,T,ms,ns", [(200, 50, [200, 132, 164], [50, 30, 44]), (320, 40, [320, 262, 4], [40, 31, 2]),
+                                       (512, 140, [512, 444], [140, 120]),
                                        (600, 24, [600, 520], [24, 24]), (1024, 30, [1024, 770, 900], [30, 22, 30])])
 def test_long_graph_sweeps_agree(mode, L, T, ms, ns):
-    """Graphs of 258..1026 nodes: the pipelined sweeps (default for small batches), the one-workgroup streaming sweeps
+    """Graphs of 130..1026 nodes: the pipelined sweeps (default), the one-workgroup streaming sweeps
     (pipeline switched off) and the redo path (blocks that give up at once: spin limit 0) compute the same tables; the
     default path is compared with the oracle in test_inside_forward_backward_vs_oracle."""
     batch = synth.training_batch(len(ms), L, T, 60, ms, ns, seed=L + T)
