@@ -196,6 +196,8 @@ def _train_case(name):
         return synth.training_batch(3, 512, 30, 100, [512, 300, 258], [30, 25, 30], seed=13)
     if name == "L512_long":  # config-3 shaped: streaming kernels, emissions read from global memory
         return synth.training_batch(2, 512, 140, 100, [512, 444], [140, 120], seed=14)
+    if name == "L320_mixed":  # pipelined sweeps: a full sentence, a target too long for its graph (-inf), a minimal one
+        return synth.training_batch(3, 320, 40, 100, [320, 20, 4], [40, 30, 2], seed=16)
     if name == "L1026":
         return synth.training_batch(2, 1026, 20, 50, [1026, 600], [20, 17], seed=15)
     raise KeyError(name)
@@ -207,7 +209,7 @@ def _match_for(batch):
     return harness.eos_masked(sel.float(), batch["output_length"], batch["target_length"])
 
 
-@pytest.mark.parametrize("case", ["cfg1", "wmt_small", "ragged_short", "L256", "L512", "L512_long", "L1026"])
+@pytest.mark.parametrize("case", ["cfg1", "wmt_small", "ragged_short", "L256", "L320_mixed", "L512", "L512_long", "L1026"])
 def test_inside_forward_backward_vs_oracle(case):
     batch = _train_case(case)
     match = _match_for(batch)
