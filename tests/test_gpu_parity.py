@@ -198,6 +198,8 @@ def _train_case(name):
         return synth.training_batch(2, 512, 140, 100, [512, 444], [140, 120], seed=14)
     if name == "L320_mixed":  # pipelined sweeps: a full sentence, a target too long for its graph (-inf), a minimal one
         return synth.training_batch(3, 320, 40, 100, [320, 20, 4], [40, 30, 2], seed=16)
+    if name == "L2050":  # beyond the pipelined sweeps: one workgroup per sentence streams the link rows
+        return synth.training_batch(2, 2050, 6, 50, [2050, 1400], [6, 5], seed=17)
     if name == "L1026":
         return synth.training_batch(2, 1026, 20, 50, [1026, 600], [20, 17], seed=15)
     raise KeyError(name)
@@ -209,7 +211,7 @@ def _match_for(batch):
     return harness.eos_masked(sel.float(), batch["output_length"], batch["target_length"])
 
 
-@pytest.mark.parametrize("case", ["cfg1", "wmt_small", "ragged_short", "L256", "L320_mixed", "L512", "L512_long", "L1026"])
+@pytest.mark.parametrize("case", ["cfg1", "wmt_small", "ragged_short", "L256", "L320_mixed", "L512", "L512_long", "L1026", "L2050"])
 def test_inside_forward_backward_vs_oracle(case):
     batch = _train_case(case)
     match = _match_for(batch)
