@@ -128,8 +128,11 @@ int pcfgnat_pcfg_loss_backward(const float *grad_output, const float *S, float *
 
 /*
  * pcfgnat_pcfg_loss followed by pcfgnat_pcfg_loss_backward (same arguments and results: S, match_all_grad, links_grad)
- * as one launch when every per-sentence table fits in LDS (it does for all shipped training shapes), otherwise as the
- * two calls.  aux is only touched by the two-call path.
+ * in one call.  For max_left = 1 and graphs of up to 128 nodes whose tables fit in LDS (every shipped training shape) the
+ * inside and the outside sweep of a sentence run side by side as two workgroups of one launch - the outside recurrence
+ * depends on links, emissions and its own earlier columns only, not on the inside table - and a second launch multiplies
+ * their tables into the gradients; otherwise the sweeps follow each other as in the two calls.  aux (8-byte aligned,
+ * pcfgnat_pcfg_aux_floats floats) carries the tables between the launches.
  */
 int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *match_all, const float *links,
                                        const int64_t *output_length, const int64_t *target_length, float *S, float *aux,

@@ -48,18 +48,27 @@ __device__ __forceinline__ float lse2(float a, float b) {
 //   rule      a -> c at column t:      links[a][k][c] + Wk_t[a] + R_t[c],   W0_t[a] = match[a][t-1] + Bh_{t-1}[a] - D_t,
 //                                      W1_t[a] = match[a-1][t-2] + match[a][t-1] + Bh_{t-2}[a] - D_t - D_{t-1}.
 //
-// Aux layout per sentence (Mc <= 64): F0h, F1h, Bh, R, each [Mc][T+2], then D [T+4]; log-domain values in base 2.
-__host__ __device__ inline size_t aux_stride_reg(int Mc, int T) { return (size_t)4 * Mc * (T + 2) + (size_t)(T + 4); }
+// Aux layout per sentence (Mc <= 64): the column offsets of the forward sweep O [T+4] and of an outside sweep that ran beside
+// it P [T+4] (doubles), then F0h, F1h, Bh, R, each [Mc][T+2], the forward's shifts D [T+4], the outside weights W0h, W1h
+// [Mc][T+2] and the outside sweep's shifts E [T+4]; log-domain values in base 2.  The buffer must be 8-byte aligned.
+__host__ __device__ inline size_t aux_stride_reg(int Mc, int T) { return (size_t)6 * Mc * (T + 2) + (size_t)6 * (T + 4); }
 struct AuxView {
-    float *F0, *F1, *BETA, *SR, *D;
+    double *O, *P;
+    float *F0, *F1, *BETA, *SR, *D, *W0, *W1, *E;
     __device__ AuxView(float *aux, int b, int Mc, int T) {
         size_t plane = (size_t)Mc * (T + 2);
         float *base = aux + (size_t)b * aux_stride_reg(Mc, T);
+        O = reinterpret_cast<double *>(base);
+        P = O + (T + 4);
+        base += 4 * (T + 4);
         F0 = base;
         F1 = base + plane;
         BETA = base + 2 * plane;
         SR = base + 3 * plane;
         D = base + 4 * plane;
+        W0 = D + (T + 4);
+        W1 = W0 + plane;
+        E = W1 + plane;
     }
 };
 
@@ -283,9 +292,9 @@ __device__ __forceinline__ void fwd_sweep(const float (&A0)[R][8 * R], const flo
 // leaves [Mc][T] and the R, F0h, F1h tables [Mc][T+2] (all base 2), which are copied out in bulk when the sweep is over -
 // the sweep itself then touches no global memory.
 template <int R, bool TAB_LDS>
-__global__ __launch_bounds__(NTR) void inside_fwd_ml1_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
-                                                            const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
-                                                            float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc) {
+__device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__restrict__ match_all, const float *__restrict__ links,
+                                                   const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
+                                                   float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc) {
     constexpr int NQ = 8 * R;
     constexpr int MP = 64 * R;
     const int TS = T + 2;
@@ -298,7 +307,7 @@ __global__ __launch_bounds__(NTR) void inside_fwd_ml1_kernel(const float *__rest
     float *sm_F0 = sm_S + (TAB_LDS ? Mc * TS : 0);
     float *sm_F1 = sm_F0 + (TAB_LDS ? Mc * TS : 0);
 
-    const int b = blockIdx.x, tid = threadIdx.x, j = tid & 7, g8 = (tid >> 3) & 7;
+    const int tid = threadIdx.x, j = tid & 7, g8 = (tid >> 3) & 7;
     const int p = wave_block(tid >> 6);
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const float *mt = match_all + (size_t)b * L * T;
@@ -392,8 +401,18 @@ __global__ __launch_bounds__(NTR) void inside_fwd_ml1_kernel(const float *__rest
             av.F1[i] = sm_F1[i];
         }
     }
-    for (int i = tid; i < TS + 2; i += NTR) av.D[i] = hd.D[i];
+    for (int i = tid; i < TS + 2; i += NTR) {
+        av.D[i] = hd.D[i];
+        if (i < TS) av.O[i] = hd.O[i];
+    }
     PCFGNAT_PHASE(3);
+}
+
+template <int R, bool TAB_LDS>
+__global__ __launch_bounds__(NTR) void inside_fwd_ml1_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
+                                                            const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
+                                                            float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc) {
+    inside_fwd_ml1_body<R, TAB_LDS>(blockIdx.x, match_all, links, out_len, tgt_len, S, aux, L, T, Mc);
 }
 
 struct BwdSweepArgs {
@@ -862,6 +881,315 @@ __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__re
             if (!(out == out)) out = 0.f;
         }
         mg[i] = g * out;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Forward and outside sweep side by side (graphs of up to 130 nodes).  The outside recurrence (see the top of this file)
+// only needs the links, the emissions and its own earlier columns - the inside table enters the posteriors, not the sweep
+// - so the two sweeps of a sentence are independent chains.  One workgroup already saturates the instruction issue of
+// its compute unit with one sweep, so they run as two workgroups: inside_pair_ml1_kernel launches 2B of them, the even
+// ones do what inside_fwd_ml1_kernel does, the odd ones the outside sweep, which halves the sequential part of the pass;
+// inside_combine_ml1_kernel then turns the tables into posteriors, in parallel over the cells.
+//
+// The outside sweep cannot use the forward's column offsets (they are being produced at the other end of the sentence),
+// so it keeps offsets of its own: beta[root][0] = 0, W_t columns relative to P_t = E_1 + .. + E_t with the shift E_{t+1}
+// chosen as the maximum of the relative beta column t-1.  Posteriors then take one correction per column,
+//   corr_t  = P_t     + O_t - ll      (rule a -> c at column t; emission with the null left child; base cell)
+//   corr1_t = P_{t-1} + O_t - ll      (emissions that go through the local leaf),
+// computed in double from the two offset sequences.
+// ------------------------------------------------------------------------------------------------------------
+struct OutsideFreeArgs {
+    float *w0, *w1;                // rotating columns [2][64]
+    float *sm_B, *sm_W0, *sm_W1;   // tables [Mc][T+2]
+    const float *sm_main, *sm_leaf;
+    float *slots;                  // [2][8] per-wave maxima of the relative beta columns
+    float *sm_E;                   // [T+4] shifts
+    double *sm_P;                  // [T+4] offsets
+    int n, mc, T, j, g8, wave;
+};
+
+template <int P>
+__device__ __forceinline__ void outside_sweep_free(const float (&A0)[1][8], const float (&A1)[1][8], const OutsideFreeArgs &x) {
+    constexpr int NQ = 8, MP = 64;
+    const int T = x.T, TS = x.T + 2, j = x.j;
+    const int c_id = 8 * P + x.g8;
+    const int q_end = P + 1;  // chunks beyond hold only parents a > c
+    const bool live = c_id < x.mc;
+    const int ci = live ? c_id : 0;
+    float bprev = (c_id == 0) ? 0.f : NEG_INF_F;  // relative beta of column t-1 (beta[root][0] = 0)
+    float e_cur = 0.f;                             // E_t
+    double Pt = 0.0;                               // P_t
+    for (int t = 1; t <= x.n - 1; t++) {
+        const float *c0 = x.w0 + (t & 1) * MP, *c1 = x.w1 + (t & 1) * MP;
+        float *n0 = x.w0 + ((t + 1) & 1) * MP, *n1 = x.w1 + ((t + 1) & 1) * MP;
+        float u0[NQ], u1[NQ];
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            if (q < q_end) {
+                u0[q] = c0[j + 8 * q];
+                u1[q] = c1[j + 8 * q];
+            }
+        }
+        // shift of the next column: the maximum of the relative beta column t-1, published one step ago
+        const float Dm = max8(x.slots + ((t - 1) & 1) * 8);
+        const float e_next = (Dm == NEG_INF_F) ? 0.f : Dm;
+        const double P_next = Pt + (double)e_next;
+        if (x.wave == 0 && j == 0 && x.g8 == 0) {
+            x.sm_E[t + 1] = e_next;
+            x.sm_P[t + 1] = P_next;
+        }
+        float mc_t = x.sm_main[ci * T + t], ml_p = x.sm_leaf[ci * T + t - 1];
+        if (!live) {
+            mc_t = NEG_INF_F;
+            ml_p = NEG_INF_F;
+        }
+        float v0[NQ], v1[NQ];
+        float mx = NEG_INF_F;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            if (q < q_end) {
+                v0[q] = A0[0][q] + u0[q];
+                v1[q] = A1[0][q] + u1[q];
+                mx = fmaxf(mx, fmaxf(v0[q], v1[q]));
+            }
+        }
+        mx = row8_max(mx);
+        const float mxs = (mx == NEG_INF_F) ? 0.f : mx;
+        float sum = 0.f;
+#pragma unroll
+        for (int q = 0; q < NQ; q++)
+            if (q < q_end) sum += ex2(v0[q] - mxs) + ex2(v1[q] - mxs);
+        sum = row8_sum(sum);
+        const float beta = (mx == NEG_INF_F || !live) ? NEG_INF_F : mx + lg2(sum);
+        // outside weights this node offers to its children at the next two positions
+        const float nw0 = (mc_t + beta) - e_next;
+        const float nw1 = ((ml_p + mc_t) + bprev) - (e_next + e_cur);
+        bprev = beta;
+        const float wm = wave_max_of_groups(beta + 0.f);
+        if ((threadIdx.x & 63) == 0) x.slots[(t & 1) * 8 + x.wave] = wm;
+        if (j == 0) {
+            n0[c_id] = nw0;
+            n1[c_id] = nw1;
+            if (live) {
+                x.sm_B[c_id * TS + t] = beta;
+                x.sm_W0[c_id * TS + t + 1] = nw0;
+                x.sm_W1[c_id * TS + t + 1] = nw1;
+            }
+        }
+        e_cur = e_next;
+        Pt = P_next;
+        lds_barrier();
+    }
+}
+
+// Dynamic LDS of the outside role: P [T+4] (double), slots [16], E [T+4], w0 [2][64], w1 [2][64], Bh, W0h, W1h [Mc][T+2],
+// emissions of main nodes and leaves [Mc][T].
+__host__ __device__ inline size_t outside_role_bytes(int Mc, int T) {
+    return (size_t)(T + 4) * sizeof(double) + ((size_t)16 + (T + 4) + 4 * 64 + (size_t)3 * Mc * (T + 2) + (size_t)2 * Mc * T) * sizeof(float);
+}
+
+__device__ __forceinline__ void inside_outside_ml1_body(const int b, const float *__restrict__ match_all,
+                                                       const float *__restrict__ links, const int64_t *__restrict__ out_len,
+                                                       const int64_t *__restrict__ tgt_len, float *__restrict__ aux, int L, int T,
+                                                       int Mc) {
+    constexpr int NQ = 8, MP = 64;
+    const int TS = T + 2, TP = T + 4;
+    extern __shared__ double smem_d[];
+    double *sm_P = smem_d;                                    // [TP]
+    float *slots = reinterpret_cast<float *>(sm_P + TP);     // [16]
+    float *sm_E = slots + 16;                                 // [TP]
+    float *w0 = sm_E + TP;                                    // [2][MP]
+    float *w1 = w0 + 2 * MP;                                  // [2][MP]
+    float *sm_B = w1 + 2 * MP;                                // [Mc][TS] each
+    float *sm_W0 = sm_B + Mc * TS;
+    float *sm_W1 = sm_W0 + Mc * TS;
+    float *sm_main = sm_W1 + Mc * TS;                         // [Mc][T]
+    float *sm_leaf = sm_main + Mc * T;
+
+    const int tid = threadIdx.x, j = tid & 7, g8 = (tid >> 3) & 7;
+    const int p = wave_block(tid >> 6);
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    if (!lengths_ok(m, n, L, T)) return;  // the forward role poisons the log-likelihood, the combine kernel writes zeros
+    const int mc = m / 2;
+    const float *mt = match_all + (size_t)b * L * T;
+    const float *lk = links + (size_t)b * L * 2 * L;
+    AuxView av(aux, b, Mc, T);
+
+    // transposed link slabs: this thread's group owns child c, its lanes the parents a <= c; unconditional loads
+    const int own = 8 * p + g8;
+    float A0[1][NQ], A1[1][NQ];
+    {
+        const int c = 2 * min(own, Mc - 1) + 1;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            const size_t row = (size_t)(2 * min(j + 8 * q, Mc - 1) + 1) * 2;
+            A0[0][q] = lk[(row + 0) * L + c];
+            A1[0][q] = lk[(row + 1) * L + c];
+        }
+    }
+    for (int i = tid; i < Mc * T; i += NTR) {
+        const int a_id = i / T, s = i - a_id * T;
+        const float vm = mt[(size_t)(2 * a_id + 1) * T + s], vl = mt[(size_t)(2 * a_id) * T + s];
+        const bool ok = a_id < mc && s < n;
+        sm_main[i] = ok ? to_b2(vm) : NEG_INF_F;
+        sm_leaf[i] = (ok && a_id >= 1) ? to_b2(vl) : NEG_INF_F;
+    }
+    for (int i = tid; i < Mc * TS; i += NTR) {
+        sm_B[i] = (i == 0) ? 0.f : NEG_INF_F;  // beta[root][0] = 0
+        sm_W0[i] = NEG_INF_F;
+        sm_W1[i] = NEG_INF_F;
+    }
+    for (int i = tid; i < 2 * MP; i += NTR) {
+        w0[i] = NEG_INF_F;
+        w1[i] = NEG_INF_F;
+    }
+    for (int i = tid; i < TP; i += NTR) {
+        sm_E[i] = 0.f;
+        sm_P[i] = 0.0;
+    }
+    if (tid < 16) slots[tid] = (tid < 8) ? 0.f : NEG_INF_F;  // maximum of the relative beta column 0
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+        const int a_id = j + 8 * q;
+        const bool ok = a_id < mc && own < mc && a_id <= own;
+        A0[0][q] = ok ? to_b2(A0[0][q]) : NEG_INF_F;
+        A1[0][q] = (ok && a_id >= 1) ? to_b2(A1[0][q]) : NEG_INF_F;
+    }
+    __syncthreads();
+    if (tid == 0) {  // W_1 columns: the root offers match[root][0] to its null-left children
+        const float w00 = sm_main[0];
+        w0[1 * MP + 0] = w00;
+        sm_W0[0 * TS + 1] = w00;
+    }
+    __syncthreads();
+    {
+        OutsideFreeArgs sa{w0, w1, sm_B, sm_W0, sm_W1, sm_main, sm_leaf, slots, sm_E, sm_P, n, mc, T, j, g8, (tid >> 6)};
+        switch (p) {  // wave-uniform
+            case 0: outside_sweep_free<0>(A0, A1, sa); break;
+            case 1: outside_sweep_free<1>(A0, A1, sa); break;
+            case 2: outside_sweep_free<2>(A0, A1, sa); break;
+            case 3: outside_sweep_free<3>(A0, A1, sa); break;
+            case 4: outside_sweep_free<4>(A0, A1, sa); break;
+            case 5: outside_sweep_free<5>(A0, A1, sa); break;
+            case 6: outside_sweep_free<6>(A0, A1, sa); break;
+            default: outside_sweep_free<7>(A0, A1, sa); break;
+        }
+    }
+    __syncthreads();
+    for (int i = tid; i < Mc * TS; i += NTR) {
+        av.BETA[i] = sm_B[i];
+        av.W0[i] = sm_W0[i];
+        av.W1[i] = sm_W1[i];
+    }
+    for (int i = tid; i < TP; i += NTR) {
+        av.E[i] = sm_E[i];
+        av.P[i] = sm_P[i];
+    }
+}
+
+// 2B workgroups: 2b runs the forward sweep of sentence b, 2b+1 its outside sweep.
+__global__ __launch_bounds__(NTR) void inside_pair_ml1_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
+                                                             const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
+                                                             float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc) {
+    const int b = blockIdx.x >> 1;
+    if ((blockIdx.x & 1) == 0) inside_fwd_ml1_body<1, true>(b, match_all, links, out_len, tgt_len, S, aux, L, T, Mc);
+    else inside_outside_ml1_body(b, match_all, links, out_len, tgt_len, aux, L, T, Mc);
+}
+
+// Posteriors from the tables of the two sweeps: grid (16, B), 256 threads.  Workgroup (q, b) owns the parents 4q .. 4q+3 of
+// sentence b: it writes the rows 8q .. 8q+7 of the links_grad slab (zeros included) and a sixteenth of the match_all_grad
+// cells.  One thread per (parent, child) pair sums both planes over the columns.
+// Dynamic LDS: corr [T+4], R [Mc][T+2], W0h, W1h of the workgroup's parents [4][T+2].
+__global__ __launch_bounds__(256) void inside_combine_ml1_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
+                                                                float *__restrict__ aux, const float *__restrict__ match_all,
+                                                                const float *__restrict__ links, const int64_t *__restrict__ out_len,
+                                                                const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad,
+                                                                float *__restrict__ lgrad, int L, int T, int Mc, int norm_B) {
+    const int TS = T + 2, TP = T + 4;
+    extern __shared__ float smem[];
+    float *corr = smem;               // [TP]
+    float *sm_R = corr + TP;          // [Mc][TS]
+    float *sm_W0 = sm_R + Mc * TS;    // [4][TS]
+    float *sm_W1 = sm_W0 + 4 * TS;    // [4][TS]
+    const int part = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *mt = match_all + (size_t)b * L * T;
+    const float *lk = links + (size_t)b * L * 2 * L;
+    float *mg = mgrad + (size_t)b * L * T;
+    float *lg = lgrad + (size_t)b * L * 2 * L;
+    AuxView av(aux, b, Mc, T);
+    const int cells = L * T, cell0 = (int)((int64_t)cells * part / 16), cell1 = (int)((int64_t)cells * (part + 1) / 16);
+    const int row0 = min(8 * part, L), row1 = min(8 * part + 8, L);
+    for (int i = row0 * 2 * L + tid; i < row1 * 2 * L; i += 256) lg[i] = 0.f;
+    const float ll = S[(size_t)b * Mc * TS];
+    const bool valid = lengths_ok(m, n, L, T) && (ll == ll) && (fabsf(ll) != __builtin_huge_valf());
+    if (!valid) {  // invalid sentence: all-zero gradients (nat_pcfg_loss.py:123-133 zeroes its loss as well)
+        for (int i = cell0 + tid; i < cell1; i += 256) mg[i] = 0.f;
+        return;
+    }
+    const int mc = m / 2;
+    // a null grad_output selects the criterion's own weights: d(-(ll/n).mean())/d ll_b = -1/(n_b * norm_B)
+    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)norm_B);
+    // this thread's pair: parent 4*part + tid/64, child tid%64; its two link values travel during the staging
+    const int a_id = 4 * part + (tid >> 6), c_id = tid & 63;
+    const bool pair_ok = a_id < mc && c_id < mc && a_id <= c_id;
+    const size_t cell = ((size_t)(2 * min(a_id, Mc - 1) + 1) * 2) * L + 2 * min(c_id, Mc - 1) + 1;
+    const float l0 = lk[cell], l1 = lk[cell + L];
+    const double ll_abs = (double)av.SR[0] + av.O[0];
+    for (int t = tid; t <= n - 1; t += 256) corr[t] = (float)(av.P[t] + av.O[t] - ll_abs);
+    for (int i0 = 0; i0 < Mc * TS; i0 += 8 * 256) {  // eight loads in flight per thread
+        float v[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) v[k] = av.SR[min(i0 + k * 256 + tid, Mc * TS - 1)];
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+            if (i0 + k * 256 + tid < Mc * TS) sm_R[i0 + k * 256 + tid] = v[k];
+    }
+    for (int i = tid; i < 4 * TS; i += 256) {
+        const bool in = 4 * part + i / TS < Mc;
+        sm_W0[i] = in ? av.W0[(size_t)4 * part * TS + i] : NEG_INF_F;
+        sm_W1[i] = in ? av.W1[(size_t)4 * part * TS + i] : NEG_INF_F;
+    }
+    // emission posteriors -> match_all_grad (pcfg_loss_backward.cu:348-382, 429-433)
+    // every operand is loaded whatever the cell's case (clamped addresses), so the loads travel together; the case picks the terms
+    for (int i = cell0 + tid; i < cell1; i += 256) {
+        const int x = i / T, s = i - x * T, e_id = x >> 1;
+        const size_t o = (size_t)e_id * TS + s;
+        const double ps = av.P[s], os = av.O[s], ps1 = av.P[max(s, 1) - 1], os1 = av.O[s + 1];
+        const float bs = av.BETA[o], bs1 = av.BETA[max(o, (size_t)1) - 1];
+        const float f0n = av.F0[o + 1], f1n = av.F1[o + 1], f1nn = av.F1[o + 2];
+        const float mas = to_b2(mt[i]);
+        const float mprev = to_b2(mt[max(i - T - 1, 0)]);            // (x-1, s-1): the leaf's emission before parent x
+        const float mnext = to_b2(mt[min(i + T + 1, L * T - 1)]);    // (x+1, s+1): the parent's emission after leaf x
+        const float cs = (float)(ps + os - ll_abs), cs1 = (float)(ps1 + os - ll_abs), cs2 = (float)(ps + os1 - ll_abs);
+        const bool in = x >= 1 && x < m && s < n, odd = x & 1;
+        float out = 0.f;
+        // a emits s with the null left child
+        out += (in && odd && s + 1 <= n - 1) ? ex2((bs + mas + f0n) + cs) : 0.f;
+        // a emits s after its leaf emitted s-1
+        out += (in && odd && s >= 1 && s + 1 <= n - 1 && e_id >= 1) ? ex2((bs1 + mprev + mas + f1n) + cs1) : 0.f;
+        // base cell
+        out += (in && odd && e_id == mc - 1 && s == n - 1) ? ex2((bs + mas) + cs) : 0.f;
+        // leaf of parent a = x+1
+        out += (in && !odd && e_id >= 1 && e_id < mc && s + 2 <= n - 1) ? ex2((bs + mas + mnext + f1nn) + cs2) : 0.f;
+        if (!(out == out)) out = 0.f;
+        mg[i] = g * out;
+    }
+    __syncthreads();  // also orders the zero fill of the slab rows before the posteriors written below
+
+    // rule posteriors -> links_grad (pcfg_loss_backward.cu:512-531): lg[a][k][c] = g * sum_t 2^(links + Wkh_t[a] + R_t[c] + corr_t)
+    if (pair_ok) {
+        const float A0 = to_b2(l0), A1 = (a_id >= 1) ? to_b2(l1) : NEG_INF_F;
+        const float *w0r = sm_W0 + (tid >> 6) * TS, *w1r = sm_W1 + (tid >> 6) * TS, *rr = sm_R + c_id * TS;
+        float acc0 = 0.f, acc1 = 0.f;
+        for (int t = 1; t <= n - 1; t++) {
+            const float rc = rr[t] + corr[t];
+            acc0 += ex2((A0 + w0r[t]) + rc);
+            acc1 += ex2((A1 + w1r[t]) + rc);
+        }
+        lg[cell] = g * ((acc0 == acc0) ? acc0 : 0.f);
+        lg[cell + L] = g * ((acc1 == acc1) ? acc1 : 0.f);
     }
 }
 
@@ -2218,10 +2546,28 @@ int launch_bwd(const float *go, const float *S, float *aux, const float *match_a
 
 // Returns PCFGNAT_EUNSUPPORTED (without a message being an error for the caller) when the fused kernel does not apply.
 template <int R>
-int launch_fused(const float *go, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *mg,
-                 float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream, bool *done) {
+int launch_fused(const float *go, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux,
+                 float *mg, float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream, bool *done) {
     const size_t need = ((size_t)head_floats(T) + 4 * 64 * R + (size_t)4 * Mc * (T + 2) + (size_t)2 * Mc * T) * sizeof(float);
     *done = false;
+    if (R == 1) {  // the two sweeps side by side as two workgroups per sentence, then the posteriors
+        const size_t fwd_bytes = ((size_t)head_floats(T) + 2 * 64 + (size_t)2 * Mc * T + (size_t)3 * Mc * (T + 2)) * sizeof(float);
+        const size_t pair_bytes = fwd_bytes > outside_role_bytes(Mc, T) ? fwd_bytes : outside_role_bytes(Mc, T);
+        const size_t comb_bytes = ((size_t)(T + 4) + (size_t)Mc * (T + 2) + (size_t)8 * (T + 2)) * sizeof(float);
+        if (pair_bytes <= LDS_BUDGET && comb_bytes <= 64 * 1024 && L <= 128) {
+            PCFGNAT_REQUIRE(((uintptr_t)aux & 7) == 0, "pcfg_loss_forward_backward: aux must be 8-byte aligned");
+            PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)inside_pair_ml1_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                  (int)pair_bytes));
+            hipLaunchKernelGGL(inside_pair_ml1_kernel, dim3(2 * B), dim3(NTR), pair_bytes, stream, match_all, links, ol, tl, S, aux, L, T,
+                               Mc);
+            PCFGNAT_HIP_CHECK(hipGetLastError());
+            hipLaunchKernelGGL(inside_combine_ml1_kernel, dim3(16, B), dim3(256), comb_bytes, stream, go, S, aux, match_all, links, ol, tl,
+                               mg, lg, L, T, Mc, norm_B);
+            PCFGNAT_HIP_CHECK(hipGetLastError());
+            *done = true;
+            return PCFGNAT_OK;
+        }
+    }
     if (need > LDS_BUDGET) return PCFGNAT_OK;
     auto k = inside_fused_ml1_kernel<R>;
     PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)need));
@@ -2319,7 +2665,7 @@ int pcfgnat::inside_forward_backward_impl(const float *grad_output, const float 
     if (ml != 1) {
         // general max_left: the two plain kernels
     } else if (Mc <= 64)
-        rc = launch_fused<1>(grad_output, match_all, links, output_length, target_length, S, match_all_grad, links_grad, (int)B, (int)L,
+        rc = launch_fused<1>(grad_output, match_all, links, output_length, target_length, S, aux, match_all_grad, links_grad, (int)B, (int)L,
                              (int)T, Mc, (int)norm_B, s, &done);
     if (rc != PCFGNAT_OK || done) return rc;
     rc = pcfgnat_pcfg_loss(match_all, links, output_length, target_length, S, aux, B, L, T, ml, stream);

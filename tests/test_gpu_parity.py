@@ -190,6 +190,12 @@ def _train_case(name):
         return synth.config2(B=6, V=1000, seed=1, logit_dtype=torch.float32)
     if name == "ragged_short":
         return synth.training_batch(5, 64, 12, 300, [64, 40, 22, 8, 4], [12, 9, 7, 3, 2], seed=8)
+    if name == "L128_T100":  # the longest targets the paired sweeps hold in LDS; one target too long for its graph
+        return synth.training_batch(4, 128, 100, 60, [128, 100, 20, 6], [100, 64, 60, 3], seed=18)
+    if name == "L126_T96":  # an odd number of main-chain nodes
+        return synth.training_batch(3, 126, 96, 60, [126, 126, 70], [96, 2, 51], seed=19)
+    if name == "L128_T104":  # just beyond: forward and outside sweeps as separate launches
+        return synth.training_batch(2, 128, 104, 60, [128, 96], [104, 80], seed=20)
     if name == "L256":
         return synth.training_batch(3, 256, 40, 200, [256, 200, 130], [40, 33, 38], seed=12)
     if name == "L512":  # streaming kernels, emissions staged in LDS
@@ -211,7 +217,7 @@ def _match_for(batch):
     return harness.eos_masked(sel.float(), batch["output_length"], batch["target_length"])
 
 
-@pytest.mark.parametrize("case", ["cfg1", "wmt_small", "ragged_short", "L256", "L320_mixed", "L512", "L512_long", "L1026", "L2050"])
+@pytest.mark.parametrize("case", ["cfg1", "wmt_small", "ragged_short", "L128_T100", "L126_T96", "L128_T104", "L256", "L320_mixed", "L512", "L512_long", "L1026", "L2050"])
 def test_inside_forward_backward_vs_oracle(case):
     batch = _train_case(case)
     match = _match_for(batch)
