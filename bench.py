@@ -22,9 +22,10 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the roofline kernel at this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled against a
 # plain device copy of known size; summary in profiles/lsg_cfg2_hbm_traffic_pmc.md.  None = not measured for this build.
+# (lsg_bwd: the single-call step at this batch's lengths - 3408 of 5120 rows read, all written.)
 ROOFLINE_KERNEL = {"single": "lsg_bwd", "fused": "lsg_bwd", "unfused": "lsg_fwd"}
 ROOFLINE_KERNEL_NAME = {"lsg_bwd": "lsg_bwd_kernel<half, from logits>", "lsg_fwd": "lsg_fwd_kernel<half, grad>"}
-MEASURED_TRAFFIC_BYTES = {"lsg_bwd": 831.36e6, "lsg_fwd": None}
+MEASURED_TRAFFIC_BYTES = {"lsg_bwd": 691.06e6, "lsg_fwd": None}
 
 
 def parse():
@@ -340,8 +341,11 @@ def main():
     if mode == "single":  # the library runs the inside forward and backward as one launch, bracketed by the third pair
         kern_ms.pop("inside_fwd", None)
         kern_ms["inside_fwd_bwd"] = kern_ms.pop("inside_bwd")
-    fwd_bytes = synth.lsg_fwd_bytes(B_timed, L, V, T, 2, require_grad=(mode == "unfused"))
-    bwd_bytes = synth.lsg_bwd_bytes(B_timed, L, V, T, 2)
+    # the single-call step neither reads the logits of the pad nodes behind a sentence's graph nor re-reads them in the
+    # backward (their gradient rows are written as zeros); the other modes go through the operator API, which cannot know
+    live_rows = int(m[:B_timed].sum()) if mode == "single" else None
+    fwd_bytes = synth.lsg_fwd_bytes(B_timed, L, V, T, 2, require_grad=(mode == "unfused"), live_rows=live_rows)
+    bwd_bytes = synth.lsg_bwd_bytes(B_timed, L, V, T, 2, live_rows=live_rows)
     roof_bytes = bwd_bytes if roof == "lsg_bwd" else fwd_bytes
     achieved = roof_bytes / (kern_ms[roof] * 1e-3) / 1e9
     traffic = MEASURED_TRAFFIC_BYTES[roof]
@@ -372,7 +376,8 @@ def main():
         "roofline": {"bound": "hbm", "kernel": ROOFLINE_KERNEL_NAME[roof], "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": (traffic * B_timed / B) if traffic else None,
-                     "algorithmic_bytes": roof_bytes, "avg_ms": kern_ms[roof], "sentences_per_launch": B_timed},
+                     "algorithmic_bytes": roof_bytes, "avg_ms": kern_ms[roof], "sentences_per_launch": B_timed,
+                     "rows_per_launch": B_timed * L, "rows_read": live_rows if live_rows is not None else B_timed * L},
         "kernels_ms": kern_ms,
         "lsg_fwd_gbs": fwd_bytes / (kern_ms["lsg_fwd"] * 1e-3) / 1e9,
         "lsg_bwd_gbs": bwd_bytes / (kern_ms["lsg_bwd"] * 1e-3) / 1e9,

@@ -186,6 +186,10 @@ int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *
  * graph node).  On return (stream order) logits holds d loss / d logits, links_grad d loss / d links, loss_out[0] the
  * loss, loss_out[1] the number of invalid sentences; match_all, S, aux, match_all_grad and row_lse ([B,L] float32) are
  * caller workspaces of the shapes documented at the individual entry points.
+ * The rows of the pad nodes at or beyond a sentence's output_length feed nothing in this pass (no sweep reads their
+ * gathered values, their gradient is zero): their logits are never read - the gather leaves zeros in match_all and
+ * row_lse for them, and the backward writes their gradient rows as zeros - so a step moves the bytes of the live rows
+ * three times and those of the pad rows once.
  * matchmask [B,T,L] / keep_word_mask [B,L] (bytes, 0 = false; both NULL = off): the criterion's force-emit masking
  * (nat_pcfg_loss.py:116-121) with the outputs of the glancing step - a graph node whose input was revealed
  * (keep_word_mask) may only emit the target position it is aligned to (matchmask), through a detached value, i.e. the
@@ -242,7 +246,8 @@ int pcfgnat_extract_links_unpack(const float *dA, const float *dKr, const float 
  *   logits [B,L,V] (F16/F32/F64, read only); targets [B,T], prev_output_tokens [B,L] int64; links [B,L,ml+1,L] float32;
  *   noise [B,L] float32: the caller's randn draw of :235 (the uniform draw of :253 cannot change the result, because
  *   keep_prob is 0 or 1; the caller still makes it to keep its random stream in step); context_p: glancing ratio.
- * Workspaces: match_all [B,L,T], S [B,Mc,T+2], aux [pcfgnat_pcfg_aux_floats] float32; pred_tokens [B,L], lengths [2,B] int64.
+ * Workspaces: match_all [B,L,T], S [B,Mc,T+2], aux [pcfgnat_pcfg_aux_floats] float32; pred_tokens [B,L], lengths [2,B] int64
+ * (the logits of pad nodes at or beyond a sentence's output length are not read: zeros in match_all and pred_tokens).
  * Outputs: path [B,L] int64 (target position of every node, -1 off the tree); matchmask [B,T,L], keep_word_mask [B,L]
  * (one byte per flag, 0/1); glat_prev_output_tokens [B,L], same_num [B], glance_nums [B] int64; loss_out[0] =
  * -(ll/target_length).mean() over sentences with a finite best-tree likelihood ll = S[b,0,0], loss_out[1] = number of

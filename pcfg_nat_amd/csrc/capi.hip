@@ -114,10 +114,10 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
         PCFGNAT_MARK(6);
         if (slices == 1)  // the loss is reduced by the first workgroup of the same launch (S is complete by now)
             rc = pcfgnat::lsg_backward_lse_with_loss(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, S, Mc * (T + 2), target_length,
-                                                     loss_out, keep_i, s);
+                                                     loss_out, keep_i, ol_i, s);
         else
             rc = pcfgnat::lsg_backward_lse_with_loss(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, nullptr, 0, nullptr, nullptr,
-                                                     keep_i, s);
+                                                     keep_i, ol_i, s);
         if (rc != PCFGNAT_OK) return rc;
         PCFGNAT_MARK(7);
 #undef PCFGNAT_MARK

@@ -43,18 +43,21 @@ int inside_forward_backward_impl(const float *grad_output, const float *match_al
                                  const int64_t *target_length, float *S, float *aux, float *match_all_grad, float *links_grad,
                                  int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream);
 
-// Read-only logsoftmax_gather over the [B,T] targets with the eos mask, which also returns the first arg max of every row
+// Read-only logsoftmax_gather over the [B,T] targets with the eos mask, which also returns the first arg max of every row;
+// the rows of nodes at or beyond a sentence's output length are left unread (zeros in selected and argmax)
 int lsg_forward_eos_argmax(const void *logits, int dtype, const int64_t *targets, void *selected, int64_t *argmax,
                            const int64_t *output_length, const int64_t *target_length, int64_t B, int64_t L, int64_t V, int64_t T,
                            void *stream);
 
 // pcfgnat_logsoftmax_gather_backward_lse whose first workgroup also reduces the criterion's loss when loss_out is given
-// (lsg.hip); rows with keep[row] != 0 get a zero gradient
+// (lsg.hip); rows with keep[row] != 0 get a zero gradient; with pad_output_length, the rows of nodes at or beyond a
+// sentence's output length (whose grad_selected rows the caller guarantees to be all zero) are zeroed without being read
 int lsg_backward_lse_with_loss(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T,
                                const float *S, int64_t ll_stride, const int64_t *target_length, float *loss_out,
-                               const unsigned char *keep, void *stream);
-// pcfgnat_logsoftmax_gather_lse over the [B,T] targets with the eos mask and the force-emit masks
+                               const unsigned char *keep, const int64_t *pad_output_length, void *stream);
+// pcfgnat_logsoftmax_gather_lse over the [B,T] targets with the eos mask and the force-emit masks; the rows of nodes at
+// or beyond a sentence's output length are left unread (zeros in selected and lse)
 int lsg_forward_lse_force(const void *logits, int dtype, const int64_t *targets, void *selected, void *lse,
                           const int64_t *output_length, const int64_t *target_length, const unsigned char *matchmask,
                           const unsigned char *keep, int64_t B, int64_t L, int64_t V, int64_t T, void *stream);

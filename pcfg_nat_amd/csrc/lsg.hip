@@ -244,7 +244,7 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
                                                      int V, int Tn, const int64_t *__restrict__ eos_out_len,
                                                      const int64_t *__restrict__ eos_tgt_len,
                                                      typename Elem<T>::compute *__restrict__ lse_out,
-                                                     int64_t *__restrict__ argmax_out, ForceEmit fe) {
+                                                     int64_t *__restrict__ argmax_out, ForceEmit fe, int skip_pad_rows) {
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
     constexpr int NW = NT / 64;
@@ -255,6 +255,16 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
 
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
         T *xr = x + row * (int64_t)V;
+        // Rows of nodes beyond the sentence's graph (pads) feed nothing downstream of the criterion: neither sweep reads
+        // them and their gradient is zero.  When asked to, leave them unread and define their outputs as zeros.
+        if (skip_pad_rows && row % L >= eos_out_len[row / L]) {  // workgroup-uniform
+            for (int s2 = tid; s2 < Tn; s2 += NT) sel[row * (int64_t)Tn + s2] = (CT)0;
+            if (tid == 0) {
+                if (lse_out != nullptr) lse_out[row] = (CT)0;
+                if (argmax_out != nullptr) argmax_out[row] = 0;
+            }
+            continue;
+        }
         const RowSplit<T> sp(xr, V);
         const vec16 *xv = reinterpret_cast<const vec16 *>(xr + sp.head);
 
@@ -450,7 +460,8 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
                                                      const typename Elem<T>::compute *__restrict__ gsel, int64_t rows,
                                                      int L, int V, int Tn,
                                                      const typename Elem<T>::compute *__restrict__ lse, LossTask loss,
-                                                     const unsigned char *__restrict__ detach_rows) {
+                                                     const unsigned char *__restrict__ detach_rows,
+                                                     const int64_t *__restrict__ pad_out_len) {
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
     constexpr int FIX = (TCAP + NT - 1) / NT;
@@ -468,6 +479,18 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
         const RowSplit<T> sp(pr, V);
         vec16 *pv = reinterpret_cast<vec16 *>(pr + sp.head);
 
+        const int ep = sp.edge_pos(tid);
+        // Rows of nodes beyond the sentence's graph (pads) get no gradient from the criterion, whose backward sweep leaves
+        // their upstream gradient all zero: p * 0 plus zeros is zero whatever the row holds, so such a row is written
+        // without being read.  The lengths come through the scalar cache, so live rows do not wait on them.
+        if (pad_out_len != nullptr && q >= pad_out_len[b]) {  // workgroup-uniform
+            vec16 z;
+            z.x = z.y = z.z = z.w = 0;
+            for (int c = tid; c < sp.nvec; c += NT) store16(pv + c, z);
+            if (ep >= 0) pr[ep] = Elem<T>::narrow((CT)0);
+            continue;
+        }
+
         // the row's chunks are requested first so that they travel while the small per-row work is done
         vec16 buf[MAXC];
 #pragma unroll
@@ -475,7 +498,6 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
             int c = tid + i * NT;
             if (c < sp.nvec) buf[i] = load16(pv + c);
         }
-        const int ep = sp.edge_pos(tid);
         CT edge = 0;
         if (ep >= 0) edge = Elem<T>::widen(pr[ep]);
 
@@ -571,7 +593,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
 template <typename T>
 int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, void *sel, int grad, int64_t rows,
                int L, int V, int Tn, const int64_t *eos_ol, const int64_t *eos_tl, void *lse, int64_t *argmax, hipStream_t stream,
-               ForceEmit fe = ForceEmit{nullptr, nullptr}) {
+               ForceEmit fe = ForceEmit{nullptr, nullptr}, int skip_pad_rows = 0) {
     using CT = typename Elem<T>::compute;
 #ifndef LSG_FWD_NT
 #define LSG_FWD_NT 512
@@ -584,17 +606,18 @@ int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
     int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
     if (grad)
         hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, true>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)x, idx, sb,
-                           sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax, fe);
+                           sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax, fe, skip_pad_rows);
     else
         hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, false>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)x, idx,
-                           sb, sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax, fe);
+                           sb, sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax, fe, skip_pad_rows);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
 
 template <typename T>
 int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, const void *g, int64_t rows, int L, int V,
-               int Tn, const void *lse, const LossTask &loss, hipStream_t stream, const unsigned char *detach_rows = nullptr) {
+               int Tn, const void *lse, const LossTask &loss, hipStream_t stream, const unsigned char *detach_rows = nullptr,
+               const int64_t *pad_out_len = nullptr) {
     using CT = typename Elem<T>::compute;
     constexpr int NT = 512;
     constexpr int MAXC = 10;
@@ -603,10 +626,10 @@ int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
     int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
     if (lse != nullptr)
         hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, true>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,
-                           (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss, detach_rows);
+                           (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss, detach_rows, pad_out_len);
     else
         hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, false>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl,
-                           st, (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss, detach_rows);
+                           st, (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss, detach_rows, pad_out_len);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -640,18 +663,18 @@ using namespace pcfgnat;
 static int lsg_forward_dispatch(void *word_ins_out, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                 void *selected, int require_grad, int64_t B, int64_t L, int64_t V, int64_t T,
                                 const int64_t *eos_ol, const int64_t *eos_tl, void *lse, void *stream, int64_t *argmax = nullptr,
-                                ForceEmit fe = ForceEmit{nullptr, nullptr}) {
+                                ForceEmit fe = ForceEmit{nullptr, nullptr}, int skip_pad_rows = 0) {
     int rc = check_common(word_ins_out, select_idx, selected, B, L, V, T);
     if (rc != PCFGNAT_OK) return rc;
     if (B * L == 0) return PCFGNAT_OK;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case PCFGNAT_F16:
-            return launch_fwd<__half>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe);
+            return launch_fwd<__half>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe, skip_pad_rows);
         case PCFGNAT_F32:
-            return launch_fwd<float>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe);
+            return launch_fwd<float>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe, skip_pad_rows);
         case PCFGNAT_F64:
-            return launch_fwd<double>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe);
+            return launch_fwd<double>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe, skip_pad_rows);
         default:
             return fail(PCFGNAT_EINVAL, "logsoftmax_gather: unknown dtype code %d (float16, float32, float64 are dispatched)", dtype);
     }
@@ -702,18 +725,18 @@ extern "C" int pcfgnat_logsoftmax_max(const void *logits, int dtype, void *best_
 static int lsg_backward_dispatch(void *buf, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                  const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T, void *stream,
                                  const LossTask &loss = LossTask{nullptr, nullptr, nullptr, 0, 0},
-                                 const unsigned char *detach_rows = nullptr) {
+                                 const unsigned char *detach_rows = nullptr, const int64_t *pad_out_len = nullptr) {
     int rc = check_common(buf, select_idx, grad_selected, B, L, V, T);
     if (rc != PCFGNAT_OK) return rc;
     if (B * L == 0) return PCFGNAT_OK;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case PCFGNAT_F16:
-            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows);
+            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len);
         case PCFGNAT_F32:
-            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows);
+            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len);
         case PCFGNAT_F64:
-            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows);
+            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len);
         default:
             return fail(PCFGNAT_EINVAL, "logsoftmax_gather_backward: unknown dtype code %d", dtype);
     }
@@ -729,17 +752,17 @@ int pcfgnat::lsg_forward_eos_argmax(const void *logits, int dtype, const int64_t
                                     const int64_t *output_length, const int64_t *target_length, int64_t B, int64_t L, int64_t V,
                                     int64_t T, void *stream) {
     return lsg_forward_dispatch(const_cast<void *>(logits), dtype, targets, T, 0, 1, selected, 0, B, L, V, T, output_length, target_length,
-                                nullptr, stream, argmax);
+                                nullptr, stream, argmax, ForceEmit{nullptr, nullptr}, 1);
 }
 
 int pcfgnat::lsg_backward_lse_with_loss(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                         const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T,
                                         const float *S, int64_t ll_stride, const int64_t *target_length, float *loss_out,
-                                        const unsigned char *keep, void *stream) {
+                                        const unsigned char *keep, const int64_t *pad_output_length, void *stream) {
     PCFGNAT_REQUIRE(B >= 1 && L >= 1 && lse && (loss_out == nullptr || (S && target_length)),
                     "logsoftmax_gather_backward: null pointer or empty batch");
     return lsg_backward_dispatch(logits_inout, dtype, select_idx, sb, sl, st, grad_selected, lse, B, L, V, T, stream,
-                                 LossTask{S, target_length, loss_out, (int)B, ll_stride}, keep);
+                                 LossTask{S, target_length, loss_out, (int)B, ll_stride}, keep, pad_output_length);
 }
 
 int pcfgnat::lsg_forward_lse_force(const void *logits, int dtype, const int64_t *targets, void *selected, void *lse,
@@ -748,7 +771,7 @@ int pcfgnat::lsg_forward_lse_force(const void *logits, int dtype, const int64_t 
     PCFGNAT_REQUIRE(B * L == 0 || (lse && output_length && target_length), "logsoftmax_gather_lse: null pointer");
     PCFGNAT_REQUIRE((matchmask == nullptr) == (keep == nullptr), "criterion_step: matchmask and keep_word_mask must be given together");
     return lsg_forward_dispatch(const_cast<void *>(logits), dtype, targets, T, 0, 1, selected, 0, B, L, V, T, output_length, target_length,
-                                lse, stream, nullptr, ForceEmit{matchmask, keep});
+                                lse, stream, nullptr, ForceEmit{matchmask, keep}, 1);
 }
 
 extern "C" int pcfgnat_logsoftmax_gather_backward_lse(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb,

@@ -744,7 +744,9 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
     batch slices alternate between the current stream and the library's helper stream (default 1: measured on MI355X the
     bandwidth-bound gather kernels leave no room for a second kernel on the CUs, so slicing does not pay).
     ``matchmask`` [B,T,L] / ``keep_word_mask`` [B,L] (bool, as the glancing step returns them): the criterion's
-    force-emit masking (nat_pcfg_loss.py:116-121); both None = off (``--no-force-emit``).  Returns
+    force-emit masking (nat_pcfg_loss.py:116-121); both None = off (``--no-force-emit``).  The rows of the pad nodes at
+    or beyond a sentence's ``output_length`` feed nothing (neither sweep reads them, their gradient is zero): the gather
+    forward leaves them unread (zeros in the returned ``match_all``) and the backward zeroes them without reading.  Returns
     (loss_and_invalid [2] float32, links_grad, ll [B], match_all_eos_masked, match_all_grad)."""
     lib = get_pcfg_kernel()
     _need_cuda("pcfg_criterion_step", logits, targets, links, output_length, target_length)

@@ -167,15 +167,19 @@ def links_bytes(B, L, ml):
     return B * L * (ml + 1) * L * 4
 
 
-def lsg_fwd_bytes(B, L, V, T, itemsize, require_grad=True):
+def lsg_fwd_bytes(B, L, V, T, itemsize, require_grad=True, live_rows=None):
     """Algorithmic HBM bytes of one logsoftmax_gather forward: logits read once, gathered fp32 written, un-expanded int64
-    targets read; plus the softmax written in place (reference split, ``require_grad``) or one fp32 log-sum-exp per row."""
-    return (2 if require_grad else 1) * B * L * V * itemsize + B * L * T * 4 + B * T * 8 + (0 if require_grad else B * L * 4)
+    targets read; plus the softmax written in place (reference split, ``require_grad``) or one fp32 log-sum-exp per row.
+    ``live_rows``: rows whose logits are read at all (the criterion step skips the pad nodes behind each graph)."""
+    rows = B * L if live_rows is None else live_rows
+    return (2 if require_grad else 1) * rows * V * itemsize + B * L * T * 4 + B * T * 8 + (0 if require_grad else B * L * 4)
 
 
-def lsg_bwd_bytes(B, L, V, T, itemsize):
-    """Algorithmic HBM bytes of the in-place backward: probabilities (or logits) read, gradients written, grad_output read."""
-    return 2 * B * L * V * itemsize + B * L * T * 4
+def lsg_bwd_bytes(B, L, V, T, itemsize, live_rows=None):
+    """Algorithmic HBM bytes of the in-place backward: probabilities (or logits) read, gradients written, grad_output read.
+    ``live_rows``: rows that are read; the others (pad nodes in the criterion step) are only written."""
+    rows = B * L if live_rows is None else live_rows
+    return (rows + B * L) * V * itemsize + rows * T * 4
 
 
 def _selfcheck():  # pragma: no cover

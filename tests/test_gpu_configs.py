@@ -26,9 +26,12 @@ def _check_training_batch(batch, sample, grad_tol=1e-4):
     want_sel = harness.eos_masked(want_sel, ol.to(DEV), tl.to(DEV))
     buf = logits.clone()
     out, glinks, ll, match, mgrad = ops.pcfg_criterion_step(buf, targets, links, ol.to(DEV), tl.to(DEV))
-    fin = torch.isfinite(want_sel)
-    assert torch.equal(torch.isfinite(match), fin)
+    # the step leaves the rows of the pad nodes behind each sentence's graph unread: zeros in `match`, zero gradients
+    live = (torch.arange(L).view(1, L) < ol.view(B, 1)).to(DEV)
+    fin = torch.isfinite(want_sel) & live.unsqueeze(-1)
+    assert torch.equal(torch.isfinite(match) & live.unsqueeze(-1), fin)
     assert torch.allclose(match[fin], want_sel[fin], rtol=2e-5, atol=2e-5)
+    assert not match[~live].any() and not buf[~live].any()
     assert torch.isfinite(ll).all() and float(out[1]) == 0
     assert torch.allclose(out[0], -(ll / tl.to(DEV)).mean(), rtol=1e-6)
     # gradient of the loss w.r.t. the logits: every row sums to ~0 (softmax), fp16 storage

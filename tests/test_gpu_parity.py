@@ -592,11 +592,24 @@ def test_errors_are_loud():
                            torch.tensor([4], device=DEV))
 
 
-def test_fused_step_equals_autograd_step():
+@pytest.mark.parametrize("shape", ["L64", "L320", "L1100", "ml3"])
+def test_fused_step_equals_autograd_step(shape):
     """train_step_fused / train_step_direct leave the same loss, logits gradient and links gradient as autograd through
-    the operator API (one invalid sentence included: its gradients must vanish)."""
-    batch = synth.training_batch(4, 64, 12, 700, [64, 40, 22, 8], [12, 9, 12, 12], seed=31, logit_scale=2.0,
-                                 logit_dtype=torch.float16)
+    the operator API (one invalid sentence included: its gradients must vanish).  Every shape has sentences shorter than
+    the padded graph: the single-call step leaves the rows of those pad nodes unread and must still zero their gradients
+    (register-resident, pipelined, streaming and general max_left sweeps)."""
+    if shape == "L64":
+        batch = synth.training_batch(4, 64, 12, 700, [64, 40, 22, 8], [12, 9, 12, 12], seed=31, logit_scale=2.0,
+                                     logit_dtype=torch.float16)
+    elif shape == "L320":
+        batch = synth.training_batch(4, 320, 24, 300, [320, 200, 64, 8], [24, 20, 9, 12], seed=32, logit_scale=2.0,
+                                     logit_dtype=torch.float16)
+    elif shape == "L1100":
+        batch = synth.training_batch(4, 1100, 12, 120, [1100, 800, 64, 8], [12, 8, 9, 12], seed=34, logit_scale=2.0,
+                                     logit_dtype=torch.float16)
+    else:
+        batch = synth.training_batch(4, 66, 12, 300, [66, 50, 22, 10], [12, 9, 7, 12], seed=35, ml=3, logit_scale=2.0,
+                                     logit_dtype=torch.float16)
     B, L, V = batch["logits"].shape
     out_mask = (torch.arange(L).view(1, L) < batch["output_length"].view(B, 1)).to(DEV)
     tgt = batch["targets"].to(DEV)
@@ -617,6 +630,7 @@ def test_fused_step_equals_autograd_step():
         assert torch.allclose(glinks, links.grad, rtol=1e-5, atol=1e-9)
         assert torch.allclose(buf.float(), leaf.grad, rtol=2 ** -9, atol=2 ** -22)
         assert not glinks[3].any() and not buf[3].any()
+        assert not buf[~out_mask].any()
 
 
 def test_force_emit_step_equals_autograd_step():
