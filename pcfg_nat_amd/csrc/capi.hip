@@ -108,16 +108,19 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
         PCFGNAT_MARK(2);
         PCFGNAT_MARK(3);  // forward and backward run as one launch where the tables fit in LDS: bracketed together by 4..5
         PCFGNAT_MARK(4);
-        rc = pcfgnat::inside_forward_backward_impl(nullptr, ma_i, lk_i, ol_i, tl_i, S_i, aux_i, mg_i, lkg_i, nb, L, T, ml, B, s);
+        // the rows of pad nodes of the logits gradient are zeroed beside the sweeps where the inside launch can host that
+        bool pad_done = false;
+        rc = pcfgnat::inside_forward_backward_impl(nullptr, ma_i, lk_i, ol_i, tl_i, S_i, aux_i, mg_i, lkg_i, nb, L, T, ml, B, s,
+                                                   pcfgnat::PadFill{(unsigned char *)lg_i, (int64_t)V * (int64_t)esz}, &pad_done);
         if (rc != PCFGNAT_OK) return rc;
         PCFGNAT_MARK(5);
         PCFGNAT_MARK(6);
         if (slices == 1)  // the loss is reduced by the first workgroup of the same launch (S is complete by now)
             rc = pcfgnat::lsg_backward_lse_with_loss(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, S, Mc * (T + 2), target_length,
-                                                     loss_out, keep_i, ol_i, s);
+                                                     loss_out, keep_i, ol_i, pad_done ? 1 : 0, s);
         else
             rc = pcfgnat::lsg_backward_lse_with_loss(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, nullptr, 0, nullptr, nullptr,
-                                                     keep_i, ol_i, s);
+                                                     keep_i, ol_i, pad_done ? 1 : 0, s);
         if (rc != PCFGNAT_OK) return rc;
         PCFGNAT_MARK(7);
 #undef PCFGNAT_MARK

@@ -39,9 +39,18 @@ inline int fail(int code, const char *fmt, ...) {
 int inside_backward_impl(const float *grad_output, const float *S, float *aux, const float *match_all, const float *links,
                          const int64_t *output_length, const int64_t *target_length, float *match_all_grad, float *links_grad, int64_t B,
                          int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream);
+// A side task for the launch that holds the sweeps of short graphs, which leaves most of the chip and all of the memory
+// bandwidth idle: zero the rows of the pad nodes (at or beyond a sentence's output length) of a [B,L,row_bytes] buffer -
+// the criterion step's logits, whose gradient rows they are.  base null: nothing to do.  *pad_done (if given) tells
+// whether the path taken carried the task out.
+struct PadFill {
+    unsigned char *base;
+    int64_t row_bytes;
+};
 int inside_forward_backward_impl(const float *grad_output, const float *match_all, const float *links, const int64_t *output_length,
                                  const int64_t *target_length, float *S, float *aux, float *match_all_grad, float *links_grad,
-                                 int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream);
+                                 int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream,
+                                 PadFill pad = PadFill{nullptr, 0}, bool *pad_done = nullptr);
 
 // Read-only logsoftmax_gather over the [B,T] targets with the eos mask, which also returns the first arg max of every row;
 // the rows of nodes at or beyond a sentence's output length are left unread (zeros in selected and argmax)
@@ -51,11 +60,12 @@ int lsg_forward_eos_argmax(const void *logits, int dtype, const int64_t *targets
 
 // pcfgnat_logsoftmax_gather_backward_lse whose first workgroup also reduces the criterion's loss when loss_out is given
 // (lsg.hip); rows with keep[row] != 0 get a zero gradient; with pad_output_length, the rows of nodes at or beyond a
-// sentence's output length (whose grad_selected rows the caller guarantees to be all zero) are zeroed without being read
+// sentence's output length (whose grad_selected rows the caller guarantees to be all zero) are zeroed without being read,
+// or left alone when the caller has zeroed them already (pad_rows_zeroed)
 int lsg_backward_lse_with_loss(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T,
                                const float *S, int64_t ll_stride, const int64_t *target_length, float *loss_out,
-                               const unsigned char *keep, const int64_t *pad_output_length, void *stream);
+                               const unsigned char *keep, const int64_t *pad_output_length, int pad_rows_zeroed, void *stream);
 // pcfgnat_logsoftmax_gather_lse over the [B,T] targets with the eos mask and the force-emit masks; the rows of nodes at
 // or beyond a sentence's output length are left unread (zeros in selected and lse)
 int lsg_forward_lse_force(const void *logits, int dtype, const int64_t *targets, void *selected, void *lse,

@@ -1088,10 +1088,49 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
     }
 }
 
-// 2B workgroups: 2b runs the forward sweep of sentence b, 2b+1 its outside sweep.
+// Workgroups per sentence that zero the rows of its pad nodes beside the sweeps (see PadFill).
+constexpr int PAD_WGS = 32;
+constexpr size_t PAD_EXCLUSIVE_LDS = 84 * 1024;  // more than half of the 160 KB of a gfx950 compute unit
+
+// Zeroes the bytes of rows [m_b, L) of sentence b - one contiguous span - as one of PAD_WGS workgroups: 16-byte
+// streaming stores over the aligned body, byte stores over what is left at either end.
+__device__ __forceinline__ void pad_fill_block(const PadFill pad, const int64_t *__restrict__ out_len, int z, int L) {
+    const int b = z / PAD_WGS, part = z % PAD_WGS, tid = threadIdx.x;
+    int64_t m = out_len[b];
+    m = m < 0 ? 0 : (m > L ? L : m);
+    unsigned char *begin = pad.base + ((int64_t)b * L + m) * pad.row_bytes;
+    unsigned char *end = pad.base + ((int64_t)b + 1) * L * pad.row_bytes;
+    if (begin >= end) return;
+    unsigned char *body = reinterpret_cast<unsigned char *>((reinterpret_cast<uintptr_t>(begin) + 15) & ~(uintptr_t)15);
+    unsigned char *body_end = reinterpret_cast<unsigned char *>(reinterpret_cast<uintptr_t>(end) & ~(uintptr_t)15);
+    if (body >= body_end) {  // shorter than one aligned chunk
+        if (part == 0)
+            for (unsigned char *q = begin + tid; q < end; q += NTR) *q = 0;
+        return;
+    }
+    if (part == 0) {
+        if (begin + tid < body) begin[tid] = 0;
+        if (body_end + tid < end) body_end[tid] = 0;
+    }
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 *v = reinterpret_cast<u32x4 *>(body);
+    const int64_t nv = (body_end - body) >> 4, per = (nv + PAD_WGS - 1) / PAD_WGS;
+    const int64_t lo = per * part, hi = (lo + per < nv) ? lo + per : nv;
+    u32x4 zero;
+    zero.x = zero.y = zero.z = zero.w = 0;
+    for (int64_t i = lo + tid; i < hi; i += NTR) __builtin_nontemporal_store(zero, v + i);
+}
+
+// 2*nsent workgroups: 2b runs the forward sweep of sentence b, 2b+1 its outside sweep; PAD_WGS*nsent more when there is
+// a pad-fill task, which land on the compute units the sweeps leave free.
 __global__ __launch_bounds__(NTR) void inside_pair_ml1_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
                                                              const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
-                                                             float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc) {
+                                                             float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc,
+                                                             int nsent, PadFill pad) {
+    if ((int)blockIdx.x >= 2 * nsent) {  // workgroup-uniform
+        pad_fill_block(pad, out_len, (int)blockIdx.x - 2 * nsent, L);
+        return;
+    }
     const int b = blockIdx.x >> 1;
     if ((blockIdx.x & 1) == 0) inside_fwd_ml1_body<1, true>(b, match_all, links, out_len, tgt_len, S, aux, L, T, Mc);
     else inside_outside_ml1_body(b, match_all, links, out_len, tgt_len, aux, L, T, Mc);
@@ -2547,7 +2586,8 @@ int launch_bwd(const float *go, const float *S, float *aux, const float *match_a
 // Returns PCFGNAT_EUNSUPPORTED (without a message being an error for the caller) when the fused kernel does not apply.
 template <int R>
 int launch_fused(const float *go, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux,
-                 float *mg, float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream, bool *done) {
+                 float *mg, float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream, bool *done,
+                 PadFill pad = PadFill{nullptr, 0}, bool *pad_done = nullptr) {
     const size_t need = ((size_t)head_floats(T) + 4 * 64 * R + (size_t)4 * Mc * (T + 2) + (size_t)2 * Mc * T) * sizeof(float);
     *done = false;
     if (R == 1) {  // the two sweeps side by side as two workgroups per sentence, then the posteriors
@@ -2558,9 +2598,17 @@ int launch_fused(const float *go, const float *match_all, const float *links, co
             PCFGNAT_REQUIRE(((uintptr_t)aux & 7) == 0, "pcfg_loss_forward_backward: aux must be 8-byte aligned");
             PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)inside_pair_ml1_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                                   (int)pair_bytes));
-            hipLaunchKernelGGL(inside_pair_ml1_kernel, dim3(2 * B), dim3(NTR), pair_bytes, stream, match_all, links, ol, tl, S, aux, L, T,
-                               Mc);
+            const bool fill = pad.base != nullptr && pad.row_bytes > 0;
+            // With the fill, every workgroup of the launch claims more than half of a compute unit's LDS, so that no fill
+            // workgroup shares a compute unit (and its instruction issue) with a sweep.
+            const size_t launch_bytes = (fill && pair_bytes < PAD_EXCLUSIVE_LDS) ? PAD_EXCLUSIVE_LDS : pair_bytes;
+            if (launch_bytes != pair_bytes)
+                PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)inside_pair_ml1_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                      (int)launch_bytes));
+            hipLaunchKernelGGL(inside_pair_ml1_kernel, dim3((2 + (fill ? PAD_WGS : 0)) * B), dim3(NTR), launch_bytes, stream, match_all,
+                               links, ol, tl, S, aux, L, T, Mc, B, pad);
             PCFGNAT_HIP_CHECK(hipGetLastError());
+            if (fill && pad_done) *pad_done = true;
             hipLaunchKernelGGL(inside_combine_ml1_kernel, dim3(16, B), dim3(256), comb_bytes, stream, go, S, aux, match_all, links, ol, tl,
                                mg, lg, L, T, Mc, norm_B);
             PCFGNAT_HIP_CHECK(hipGetLastError());
@@ -2653,7 +2701,8 @@ extern "C" int pcfgnat_pcfg_loss_backward(const float *grad_output, const float 
 int pcfgnat::inside_forward_backward_impl(const float *grad_output, const float *match_all, const float *links,
                                           const int64_t *output_length, const int64_t *target_length, float *S, float *aux,
                                           float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T, int64_t ml,
-                                          int64_t norm_B, void *stream) {
+                                          int64_t norm_B, void *stream, PadFill pad, bool *pad_done) {
+    if (pad_done) *pad_done = false;
     int rc = check_dims("pcfg_loss_forward_backward", B, L, T, ml);
     if (rc != PCFGNAT_OK) return rc;
     if (B == 0) return PCFGNAT_OK;
@@ -2666,7 +2715,7 @@ int pcfgnat::inside_forward_backward_impl(const float *grad_output, const float 
         // general max_left: the two plain kernels
     } else if (Mc <= 64)
         rc = launch_fused<1>(grad_output, match_all, links, output_length, target_length, S, aux, match_all_grad, links_grad, (int)B, (int)L,
-                             (int)T, Mc, (int)norm_B, s, &done);
+                             (int)T, Mc, (int)norm_B, s, &done, pad, pad_done);
     if (rc != PCFGNAT_OK || done) return rc;
     rc = pcfgnat_pcfg_loss(match_all, links, output_length, target_length, S, aux, B, L, T, ml, stream);
     if (rc != PCFGNAT_OK) return rc;

@@ -461,7 +461,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
                                                      int L, int V, int Tn,
                                                      const typename Elem<T>::compute *__restrict__ lse, LossTask loss,
                                                      const unsigned char *__restrict__ detach_rows,
-                                                     const int64_t *__restrict__ pad_out_len) {
+                                                     const int64_t *__restrict__ pad_out_len, int pad_rows_zeroed) {
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
     constexpr int FIX = (TCAP + NT - 1) / NT;
@@ -484,6 +484,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
         // their upstream gradient all zero: p * 0 plus zeros is zero whatever the row holds, so such a row is written
         // without being read.  The lengths come through the scalar cache, so live rows do not wait on them.
         if (pad_out_len != nullptr && q >= pad_out_len[b]) {  // workgroup-uniform
+            if (pad_rows_zeroed) continue;  // an earlier launch of the caller has written the zeros
             vec16 z;
             z.x = z.y = z.z = z.w = 0;
             for (int c = tid; c < sp.nvec; c += NT) store16(pv + c, z);
@@ -617,7 +618,7 @@ int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
 template <typename T>
 int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, const void *g, int64_t rows, int L, int V,
                int Tn, const void *lse, const LossTask &loss, hipStream_t stream, const unsigned char *detach_rows = nullptr,
-               const int64_t *pad_out_len = nullptr) {
+               const int64_t *pad_out_len = nullptr, int pad_rows_zeroed = 0) {
     using CT = typename Elem<T>::compute;
     constexpr int NT = 512;
     constexpr int MAXC = 10;
@@ -626,10 +627,10 @@ int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
     int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
     if (lse != nullptr)
         hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, true>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,
-                           (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss, detach_rows, pad_out_len);
+                           (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss, detach_rows, pad_out_len, pad_rows_zeroed);
     else
         hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, false>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl,
-                           st, (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss, detach_rows, pad_out_len);
+                           st, (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss, detach_rows, pad_out_len, pad_rows_zeroed);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -725,18 +726,19 @@ extern "C" int pcfgnat_logsoftmax_max(const void *logits, int dtype, void *best_
 static int lsg_backward_dispatch(void *buf, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                  const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T, void *stream,
                                  const LossTask &loss = LossTask{nullptr, nullptr, nullptr, 0, 0},
-                                 const unsigned char *detach_rows = nullptr, const int64_t *pad_out_len = nullptr) {
+                                 const unsigned char *detach_rows = nullptr, const int64_t *pad_out_len = nullptr,
+                                 int pad_rows_zeroed = 0) {
     int rc = check_common(buf, select_idx, grad_selected, B, L, V, T);
     if (rc != PCFGNAT_OK) return rc;
     if (B * L == 0) return PCFGNAT_OK;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case PCFGNAT_F16:
-            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len);
+            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed);
         case PCFGNAT_F32:
-            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len);
+            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed);
         case PCFGNAT_F64:
-            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len);
+            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed);
         default:
             return fail(PCFGNAT_EINVAL, "logsoftmax_gather_backward: unknown dtype code %d", dtype);
     }
@@ -758,11 +760,12 @@ int pcfgnat::lsg_forward_eos_argmax(const void *logits, int dtype, const int64_t
 int pcfgnat::lsg_backward_lse_with_loss(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                         const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T,
                                         const float *S, int64_t ll_stride, const int64_t *target_length, float *loss_out,
-                                        const unsigned char *keep, const int64_t *pad_output_length, void *stream) {
+                                        const unsigned char *keep, const int64_t *pad_output_length, int pad_rows_zeroed,
+                                        void *stream) {
     PCFGNAT_REQUIRE(B >= 1 && L >= 1 && lse && (loss_out == nullptr || (S && target_length)),
                     "logsoftmax_gather_backward: null pointer or empty batch");
     return lsg_backward_dispatch(logits_inout, dtype, select_idx, sb, sl, st, grad_selected, lse, B, L, V, T, stream,
-                                 LossTask{S, target_length, loss_out, (int)B, ll_stride}, keep, pad_output_length);
+                                 LossTask{S, target_length, loss_out, (int)B, ll_stride}, keep, pad_output_length, pad_rows_zeroed);
 }
 
 int pcfgnat::lsg_forward_lse_force(const void *logits, int dtype, const int64_t *targets, void *selected, void *lse,

@@ -175,11 +175,14 @@ def lsg_fwd_bytes(B, L, V, T, itemsize, require_grad=True, live_rows=None):
     return (2 if require_grad else 1) * rows * V * itemsize + B * L * T * 4 + B * T * 8 + (0 if require_grad else B * L * 4)
 
 
-def lsg_bwd_bytes(B, L, V, T, itemsize, live_rows=None):
+def lsg_bwd_bytes(B, L, V, T, itemsize, live_rows=None, pads_zeroed_elsewhere=False):
     """Algorithmic HBM bytes of the in-place backward: probabilities (or logits) read, gradients written, grad_output read.
-    ``live_rows``: rows that are read; the others (pad nodes in the criterion step) are only written."""
+    ``live_rows``: rows that are read; the others (pad nodes in the criterion step) are only written - or not touched at
+    all when another launch has zeroed them (``pads_zeroed_elsewhere``: graphs of up to 128 nodes, where the launch that
+    holds the inside and outside sweeps does it beside them)."""
     rows = B * L if live_rows is None else live_rows
-    return (rows + B * L) * V * itemsize + rows * T * 4
+    written = rows if pads_zeroed_elsewhere else B * L
+    return (rows + written) * V * itemsize + rows * T * 4
 
 
 def _selfcheck():  # pragma: no cover
