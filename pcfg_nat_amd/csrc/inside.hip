@@ -1090,6 +1090,7 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
 
 // Workgroups per sentence that zero the rows of its pad nodes beside the sweeps (see PadFill).
 constexpr int PAD_WGS = 32;
+constexpr int PAD_MAX_SWEEP_WGS = 192;  // of the 256 compute units
 constexpr size_t PAD_EXCLUSIVE_LDS = 84 * 1024;  // more than half of the 160 KB of a gfx950 compute unit
 
 // Zeroes the bytes of rows [m_b, L) of sentence b - one contiguous span - as one of PAD_WGS workgroups: 16-byte
@@ -2598,7 +2599,9 @@ int launch_fused(const float *go, const float *match_all, const float *links, co
             PCFGNAT_REQUIRE(((uintptr_t)aux & 7) == 0, "pcfg_loss_forward_backward: aux must be 8-byte aligned");
             PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)inside_pair_ml1_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                                   (int)pair_bytes));
-            const bool fill = pad.base != nullptr && pad.row_bytes > 0;
+            // the fill rides along only while the sweeps leave compute units free for it (the gather backward writes the
+            // zeros itself otherwise)
+            const bool fill = pad.base != nullptr && pad.row_bytes > 0 && 2 * B <= PAD_MAX_SWEEP_WGS;
             // With the fill, every workgroup of the launch claims more than half of a compute unit's LDS, so that no fill
             // workgroup shares a compute unit (and its instruction issue) with a sweep.
             const size_t launch_bytes = (fill && pair_bytes < PAD_EXCLUSIVE_LDS) ? PAD_EXCLUSIVE_LDS : pair_bytes;

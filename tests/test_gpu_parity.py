@@ -643,6 +643,31 @@ def test_fused_step_equals_autograd_step(shape):
         assert not buf[~out_mask].any()
 
 
+def test_single_call_step_large_batch_of_short_graphs():
+    """100 sentences of at most 16 nodes: more sweeps than the launch that holds them can spare compute units for the zeros
+    of the pad rows, which the gather backward then writes itself.  Against the four-call step over the same kernels."""
+    B, L, T, V = 100, 16, 6, 50
+    gen = torch.Generator().manual_seed(41)
+    ms = (2 * torch.randint(2, L // 2 + 1, (B,), generator=gen)).tolist()
+    ns = torch.randint(2, T + 1, (B,), generator=gen).tolist()
+    ms[0], ns[0] = L, T
+    batch = synth.training_batch(B, L, T, V, ms, ns, seed=42, logit_scale=2.0, logit_dtype=torch.float16)
+    tgt, links = batch["targets"].to(DEV), batch["links"].to(DEV)
+    ol, tl = batch["output_length"].to(DEV), batch["target_length"].to(DEV)
+    want_buf = batch["logits"].to(DEV).clone()
+    want_loss, want_glinks, want_ll = harness.train_step_fused(want_buf, tgt, links, ol, tl)
+    buf = batch["logits"].to(DEV).clone()
+    loss, glinks, ll = harness.train_step_single_call(buf, tgt, links, ol, tl)
+    fin = torch.isfinite(want_ll)
+    assert fin.any() and torch.equal(fin, torch.isfinite(ll))
+    assert torch.allclose(ll[fin], want_ll[fin], rtol=1e-6)
+    assert torch.allclose(loss, want_loss, rtol=1e-6)
+    assert torch.allclose(glinks, want_glinks, rtol=1e-5, atol=1e-9)
+    assert torch.allclose(buf.float(), want_buf.float(), rtol=2 ** -9, atol=2 ** -22)
+    out_mask = torch.arange(L, device=DEV).view(1, L) < ol.view(B, 1)
+    assert not buf[~out_mask].any()
+
+
 def test_force_emit_step_equals_autograd_step():
     """The criterion with force-emit masking (nat_pcfg_loss.py:116-121; on in the scripts without --no-force-emit): the
     masks come from a glancing pass over the same batch; autograd through the torch restatement of those lines against
