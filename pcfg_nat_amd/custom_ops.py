@@ -798,3 +798,50 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
                                               lg.data_ptr(), row_lse.data_ptr(), out.data_ptr(), B, L, V, T, ml, slices,
                                               _stream(logits), ev_arr), lib)
     return out, lg, S[:, 0, 0], match, mg
+
+
+class PCFGCriterionFunc(Function):
+    """The criterion's loss (nat_pcfg_loss.py:98-145) as one differentiable op over ``pcfg_criterion_step``.  Like the
+    reference's own ops (pcfg_loss.py:67-73 runs the inside backward eagerly inside the forward; :144-181 hands the logits
+    buffer back as the gradient) the forward already leaves d loss / d logits in the logits buffer - which is returned
+    marked dirty and must not be used any more - and keeps d loss / d links; the backward hands both out, scaled by the
+    upstream gradient of the loss (no pass over the logits when that is exactly 1; one in-place multiply otherwise, e.g.
+    under fp16 loss scaling).  May run backward once."""
+
+    @staticmethod
+    def forward(ctx, outputs, links, targets, output_length, target_length, matchmask, keep_word_mask):
+        need = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        out, links_grad, ll, _, _ = pcfg_criterion_step(outputs, targets, links, output_length, target_length,
+                                                       matchmask=matchmask, keep_word_mask=keep_word_mask)
+        ctx.mark_dirty(outputs)
+        ctx.set_materialize_grads(False)
+        if need:
+            ctx.save_for_backward(outputs, links_grad)
+            ctx.has_backward = False
+        invalid = ll.isinf().logical_or(ll.isnan())
+        return outputs, out[0], ll.masked_fill(invalid, 0), out[1]
+
+    @staticmethod
+    def backward(ctx, grad_outputs, grad_loss, grad_ll, grad_invalid):
+        assert grad_outputs is None, "Cannot reuse the logits after pcfg_criterion"
+        assert grad_ll is None, "pcfg_criterion: only the loss is differentiable (use cuda_pcfg_loss for per-sentence gradients)"
+        if grad_loss is None:
+            return (None,) * 7
+        assert not ctx.has_backward, "Cannot backward twice in pcfg_criterion"
+        ctx.has_backward = True
+        buf, links_grad = ctx.saved_tensors
+        if not bool((grad_loss == 1).all()):  # the one host read of the backward; exact 1 is autograd's seed for loss.backward()
+            buf.mul_(grad_loss.to(buf.dtype))
+            links_grad = links_grad * grad_loss.to(links_grad.dtype)
+        return (buf if ctx.needs_input_grad[0] else None, links_grad if ctx.needs_input_grad[1] else None, None, None, None, None,
+                None)
+
+
+def pcfg_criterion(outputs, targets, links, output_length, target_length, matchmask=None, keep_word_mask=None):
+    """loss = -(log-likelihood / target_length).mean() over the sentences with a finite log-likelihood, differentiable in
+    ``outputs`` [B,L,V] (fp16/fp32 logits, consumed in place) and ``links``; one native call in the forward.  Returns
+    (loss, ll [B] with invalid sentences zeroed, number of invalid sentences) - the dict entries of
+    ``harness.compute_pcfg_loss``."""
+    _, loss, ll, invalid = PCFGCriterionFunc.apply(outputs, links, targets, output_length, target_length, matchmask, keep_word_mask)
+    return loss, ll, invalid
+

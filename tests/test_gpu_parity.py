@@ -643,6 +643,31 @@ def test_fused_step_equals_autograd_step(shape):
         assert not buf[~out_mask].any()
 
 
+@pytest.mark.parametrize("scale", [1.0, 128.0])
+def test_criterion_op_under_autograd(scale):
+    """pcfg_criterion (one native call in the forward, gradients handed out by backward) against autograd through the
+    separate ops, with and without an upstream factor on the loss (fp16 loss scaling)."""
+    batch = synth.training_batch(4, 64, 12, 700, [64, 40, 22, 8], [12, 9, 12, 12], seed=43, logit_scale=2.0,
+                                 logit_dtype=torch.float16)
+    B, L, V = batch["logits"].shape
+    out_mask = (torch.arange(L).view(1, L) < batch["output_length"].view(B, 1)).to(DEV)
+    tgt = batch["targets"].to(DEV)
+    ol, tl = batch["output_length"].to(DEV), batch["target_length"].to(DEV)
+    leaf = batch["logits"].to(DEV).float().requires_grad_(True)
+    links = batch["links"].to(DEV).requires_grad_(True)
+    res = harness.compute_pcfg_loss(leaf.half(), out_mask, tgt, tgt.ne(synth.PAD), links)
+    (res["loss"] * scale).backward()
+    leaf2 = batch["logits"].to(DEV).float().requires_grad_(True)
+    links2 = batch["links"].to(DEV).requires_grad_(True)
+    loss, ll, invalid = ops.pcfg_criterion(leaf2.half(), tgt, links2, ol, tl)
+    assert torch.allclose(loss, res["loss"].detach(), rtol=1e-6) and int(invalid) == 1
+    assert torch.allclose(ll, res["ll"].detach(), rtol=1e-6)
+    (loss * scale).backward()
+    assert torch.allclose(links2.grad, links.grad, rtol=1e-5, atol=1e-9 * scale)
+    assert torch.allclose(leaf2.grad, leaf.grad, rtol=2 ** -8, atol=2 ** -22 * scale)
+    assert not leaf2.grad[~out_mask].any() and not leaf2.grad[3].any()
+
+
 def test_single_call_step_large_batch_of_short_graphs():
     """100 sentences of at most 16 nodes: more sweeps than the launch that holds them can spare compute units for the zeros
     of the pad rows, which the gather backward then writes itself.  Against the four-call step over the same kernels."""
