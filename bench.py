@@ -338,7 +338,7 @@ def main():
     torch.cuda.synchronize()
     kern_ms = averages()
     kern_ms[roof] = roof_in_region
-    if mode == "single":  # the library runs the inside forward and backward as one launch, bracketed by the third pair
+    if mode == "single":  # the library issues the inside forward and backward together, bracketed by the third pair
         kern_ms.pop("inside_fwd", None)
         kern_ms["inside_fwd_bwd"] = kern_ms.pop("inside_bwd")
     # the single-call step neither reads the logits of the pad nodes behind a sentence's graph nor re-reads them in the

@@ -106,7 +106,7 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
         PCFGNAT_MARK(1);
         if (slices > 1) PCFGNAT_HIP_CHECK(hipEventRecord(h->gathered[i & 1], s));
         PCFGNAT_MARK(2);
-        PCFGNAT_MARK(3);  // forward and backward run as one launch where the tables fit in LDS: bracketed together by 4..5
+        PCFGNAT_MARK(3);  // forward and backward are issued by one internal call: bracketed together by 4..5
         PCFGNAT_MARK(4);
         // the rows of pad nodes of the logits gradient are zeroed beside the sweeps where the inside launch can host that
         bool pad_done = false;

@@ -11,12 +11,15 @@
 //   beta[c][t] = LSE_{a<=c}( links[a][0][c] + match[a][t-1] + beta[a][t-1],
 //                            links[a][1][c] + match[a-1][t-2] + match[a][t-1] + beta[a][t-2] ).
 //
-// Design (latency-bound, one workgroup of 1024 threads per sentence): the sentence's compact link matrices live in
-// registers for the whole sweep (one 16-lane DPP row per node, lanes strided over the other index), the current
-// column of S (or of the outside weights) is exchanged through LDS, one workgroup barrier per target position.
-// The forward leaves F0/F1 behind so that the backward needs a single sweep: rule posteriors are accumulated in
-// registers, emission posteriors come from an element-wise epilogue.  Graphs of more than 130 nodes use the streaming
-// or the pipelined sweeps further down (link rows from L2, or spread over several workgroups per sentence).
+// Design (latency-bound sweeps over the target positions, one workgroup of 512 threads per sentence and sweep): the
+// sentence's compact link matrices live in registers for the whole sweep (one 8-lane group per node, lanes strided over
+// the other index), the current column of S (or of the outside weights) is exchanged through LDS, one workgroup barrier
+// per target position.  The forward leaves F0/F1 behind so that the backward needs a single outside sweep; that sweep
+// reads links, emissions and its own earlier columns only, so in the single call the two run side by side as two
+// workgroups (inside_pair_ml1_kernel) and a parallel kernel multiplies their tables into the posteriors
+// (inside_combine_ml1_kernel); in the two-call API the outside sweep accumulates rule posteriors in registers and
+// emission posteriors come from an element-wise epilogue.  Graphs of more than 130 nodes use the streaming or the
+// pipelined sweeps further down (link rows from L2, or spread over several workgroups per sentence).
 #include "common.hip.h"
 
 #include <atomic>
@@ -687,7 +690,8 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
     PCFGNAT_PHASE(13);
 }
 
-// Forward and backward in one launch (used by the single-call criterion step when every table fits in LDS): the
+// Forward and backward in one launch, one workgroup per sentence (the single call's path where the paired sweeps further
+// down do not apply: more than 128 nodes, or tables beyond their LDS budget but within this kernel's): the
 // tables the backward needs (S, F0, F1, emissions) never leave LDS, only S is also written to global memory in the
 // reference's layout.  Dynamic LDS: head (see LdsHead), w0[2][MP] (doubles as the forward's columns), w1[2][MP],
 // R/F0h/F1h/Bh [Mc][T+2], emissions of main nodes and leaves [Mc][T].

@@ -177,7 +177,7 @@ def train_step_fused(logits, targets, links, output_length, target_length, ops=_
 
 def train_step_single_call(logits, targets, links, output_length, target_length, ops=_default_ops, mark=None, slices=None,
                            matchmask=None, keep_word_mask=None):
-    """``train_step_fused`` issued as one native call (``pcfgnat_criterion_step``): the five kernels are enqueued back to
+    """``train_step_fused`` issued as one native call (``pcfgnat_criterion_step``): the kernels are enqueued back to
     back by the library and the scalar loss is reduced on the device.  Returns (loss, links_grad, ll)."""
     events = None
     if mark is not None:
