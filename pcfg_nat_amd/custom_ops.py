@@ -472,21 +472,24 @@ def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unre
     if mask.dim() != 2 or mask.size(0) != mask.size(1):
         raise RuntimeError("viterbi_decoding: left_tree_mask must be square")
     out = torch.empty((B, L), dtype=torch.int64, device=dev)
-    cnt = torch.empty((B,), dtype=torch.int64, device=dev)
     if dev.type == "cuda":
         with torch.cuda.device(dev):
             scratch = torch.empty((B, 2 * L), dtype=torch.int64, device=dev)
+            cnt = _pinned_counts(dev, B)  # written by the kernel, read after the one stream wait
             _lib.check(lib.pcfgnat_viterbi_decoding(pl.data_ptr(), ol.data_ptr(), Lt.data_ptr(), Rt.data_ptr(), Mt.data_ptr(),
                                                     tok.data_ptr(), mask.data_ptr(), mask.size(0), int(pad_index),
                                                     out.data_ptr(), cnt.data_ptr(), scratch.data_ptr(), B, L, Lq,
                                                     _stream(out)), lib)
+            torch.cuda.current_stream(dev).synchronize()
     else:
+        cnt = torch.empty((B,), dtype=torch.int64)
         _lib.check(lib.pcfgnat_viterbi_decoding_host(pl.data_ptr(), ol.data_ptr(), Lt.data_ptr(), Rt.data_ptr(),
                                                      Mt.data_ptr(), tok.data_ptr(), mask.data_ptr(), mask.size(0),
                                                      int(pad_index), out.data_ptr(), cnt.data_ptr(), B, L, Lq), lib)
-    if B and int(cnt.min()) < 0:
+    counts = cnt.tolist()
+    if B and min(counts) < 0:
         raise RuntimeError("viterbi_decoding: malformed traces")
-    maxlen = int(cnt.max()) if B else 0
+    maxlen = max(counts) if B else 0
     return out[:, :maxlen].to(torch.float32)
 
 
@@ -638,7 +641,9 @@ _PINNED_COUNTS = {}
 
 
 def _pinned_counts(device, n):
-    """A pinned int64 host buffer of n entries per device, reused between calls (grown when a larger batch comes)."""
+    """A pinned int64 host buffer of n entries per device, reused between calls (grown when a larger batch comes).  Pinned
+    host memory is addressable from the device, so the decode kernels write their per-sentence token counts straight
+    into it; the caller reads them after waiting for the stream (calls that overlap on one device would share it)."""
     key = str(device)
     buf = _PINNED_COUNTS.get(key)
     if buf is None or buf.numel() < n:
@@ -674,24 +679,22 @@ def pcfg_viterbi_decode(unreduced_logits, links, output_length, unreduced_tokens
     with torch.cuda.device(dev):
         nwork = (lib.pcfgnat_viterbi_decode_workspace_bytes(B, L, ml) + 7) // 8
         # one allocation: workspace | tokens [B,L] | emitted counts [B] | predicted lengths [B]
-        block = torch.empty((nwork + B * L + 2 * B,), dtype=torch.int64, device=dev)
+        block = torch.empty((nwork + B * L + B,), dtype=torch.int64, device=dev)
         out = block[nwork:nwork + B * L].view(B, L)
-        meta = block[nwork + B * L:].view(2, B)
+        pred = block[nwork + B * L:]
         base = block.data_ptr()
+        # the emitted counts go straight into pinned host memory, which the device addresses like its own: the one
+        # synchronisation of the decode is a stream wait, with no copy in front of it
+        host = _pinned_counts(dev, B)
         _lib.check(lib.pcfgnat_viterbi_decode(ob.data_ptr(), links.data_ptr(), ol.data_ptr(), tok.data_ptr(), mask.data_ptr(),
                                               mask.size(0), int(pad_index), pen.data_ptr(), base, base + 8 * nwork,
-                                              base + 8 * (nwork + B * L), base + 8 * (nwork + B * L + B), B, L, ml,
-                                              _stream(ob)), lib)
-        # the one synchronisation of the decode: counts for the trimming below (through a pinned buffer: one asynchronous
-        # copy and a stream wait instead of a staged blocking copy)
-        host = _pinned_counts(dev, B)
-        host.copy_(meta[0], non_blocking=True)
+                                              host.data_ptr(), base + 8 * (nwork + B * L), B, L, ml, _stream(ob)), lib)
         torch.cuda.current_stream(dev).synchronize()
     counts = host.tolist()
     if B and min(counts) < 0:
         raise RuntimeError("viterbi_decoding: malformed traces")
     maxlen = max(counts) if B else 0
-    return out[:, :maxlen].to(torch.float32), meta[1]
+    return out[:, :maxlen].to(torch.float32), pred
 
 
 def pcfg_lookahead_decode(links, unreduced_logits, unreduced_tokens, output_length, left_tree_mask, pad_index, beta=1.0,
@@ -723,14 +726,15 @@ def pcfg_lookahead_decode(links, unreduced_logits, unreduced_tokens, output_leng
     with torch.cuda.device(dev):
         idx = torch.empty((B, L), dtype=torch.int64, device=dev)
         out = torch.empty((B, L), dtype=torch.int64, device=dev)
-        cnt = torch.empty((B,), dtype=torch.int64, device=dev)
+        cnt = _pinned_counts(dev, B)  # written by the kernel, read after the one stream wait
         _lib.check(lib.pcfgnat_lookahead_decode(links.data_ptr(), ob_ptr, float(beta), ol.data_ptr(), tok.data_ptr(), mask.data_ptr(),
                                                 mask.size(0), int(pad_index), idx.data_ptr(), out.data_ptr(), cnt.data_ptr(), B, L,
                                                 K - 1, _stream(links)), lib)
-    host = cnt.cpu()
-    if B and int(host.min()) < 0:
+        torch.cuda.current_stream(dev).synchronize()
+    counts = cnt.tolist()
+    if B and min(counts) < 0:
         raise RuntimeError("pcfg_lookahead_decode: the walk does not terminate")
-    maxlen = int(host.max()) if B else 0
+    maxlen = max(counts) if B else 0
     tokens = out[:, :maxlen]
     return (tokens, idx) if return_pointers else tokens
 
