@@ -97,7 +97,8 @@ int pcfgnat_logsoftmax_max(const void *logits, int dtype, void *best_lprob, int6
                            int64_t V, void *stream);
 
 /* Number of floats of the auxiliary table the inside kernels exchange (takes the place of the reference's C
- * table, pcfg_loss.cu:394, whose content for ml = 1 is a copy of match_all). */
+ * table, pcfg_loss.cu:394, whose content for ml = 1 is a copy of match_all).  The buffer must be aligned to 16 bytes
+ * (the entry points check it where they rely on it). */
 size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml);
 
 /*
