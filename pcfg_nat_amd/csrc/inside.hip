@@ -1359,8 +1359,12 @@ __global__ __launch_bounds__(BT_NT) void best_tree_ml1_kernel(const float *__res
 // ------------------------------------------------------------------------------------------------------------
 __host__ __device__ inline int stream_mp(int Mc) { return ((Mc + 63) / 64) * 64; }
 __host__ __device__ inline size_t stream_planes(int Mc, int T) { return (((size_t)6 * Mc * (T + 2) + (size_t)(T + 4)) + 3) & ~(size_t)3; }
+__host__ __device__ inline int corr_len(int T) { return (T + 5) & ~1; }
 __host__ __device__ inline size_t exchange_floats(int Mc, int T) {
-    return (size_t)4 * stream_mp(Mc) * (T + 2) + (size_t)(stream_mp(Mc) / 16) * (T + 4) + 4;
+    const size_t MP = stream_mp(Mc);
+    // forward columns + outside weights, block shifts, flags; then, for the sweeps that run side by side: the outside
+    // weights as absolute doubles, the outside sweep's block shifts, the two correction rows of the posteriors
+    return 4 * MP * (T + 2) + (MP / 16) * (T + 4) + 4 + 4 * MP * (T + 2) + (MP / 16) * (T + 4) + 2 * (size_t)corr_len(T);
 }
 __host__ __device__ inline size_t aux_stride_stream(int Mc, int T) {
     return stream_planes(Mc, T) + (size_t)4 * Mc * stream_mp(Mc) + exchange_floats(Mc, T);
@@ -1386,6 +1390,9 @@ struct ExchangeView {
     unsigned *bw;              // [T+2][2][MP]
     float *shifts;             // [MP/16][T+4]
     int *flags;
+    unsigned long long *obw;   // [T+2][2][MP]: outside weights as absolute doubles (sweeps side by side)
+    float *shiftsE;            // [MP/16][T+4]: shifts of the outside sweep's blocks (sweeps side by side)
+    float *corr;               // [2][corr_len(T)]: corrections of the posteriors, corr_t and corr1_t
     __device__ ExchangeView(float *aux, int b, int Mc, int T) {
         const int MP = stream_mp(Mc);
         float *base = aux + (size_t)b * aux_stride_stream(Mc, T) + stream_planes(Mc, T) + (size_t)4 * Mc * MP;
@@ -1393,6 +1400,10 @@ struct ExchangeView {
         bw = reinterpret_cast<unsigned *>(base + (size_t)2 * MP * (T + 2));
         shifts = base + (size_t)4 * MP * (T + 2);
         flags = reinterpret_cast<int *>(shifts + (size_t)(MP / 16) * (T + 4));
+        float *more = shifts + (size_t)(MP / 16) * (T + 4) + 4;
+        obw = reinterpret_cast<unsigned long long *>(more);
+        shiftsE = more + (size_t)4 * MP * (T + 2);
+        corr = shiftsE + (size_t)(MP / 16) * (T + 4);
     }
 };
 constexpr int FLAG_FWD = 0, FLAG_BWD = 1;
@@ -1669,7 +1680,11 @@ __global__ __launch_bounds__(256) void compact_links_ml1_kernel(const float *__r
         unsigned *x = reinterpret_cast<unsigned *>(xv.fcol);
         const size_t words = (size_t)4 * MP * (T + 2);
         const size_t nthreads = (size_t)gridDim.x * gridDim.y * 256, me = ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
-        for (size_t i = me; i < words; i += nthreads) x[i] = 0xFFFFFFFFu;
+        unsigned *y = reinterpret_cast<unsigned *>(xv.obw);
+        for (size_t i = me; i < words; i += nthreads) {
+            x[i] = 0xFFFFFFFFu;
+            y[i] = 0xFFFFFFFFu;
+        }
         if (me < 4) xv.flags[me] = 0;
     }
     for (int r = ty; r < 32; r += 8) {
@@ -1896,17 +1911,17 @@ __device__ __forceinline__ void slab_row_lse(const float4 (&A0)[NQ], const float
 // above).  Dynamic LDS (MATCH_LDS): the emissions of the block's nodes, main [NLP][T] and leaf [NLP][T]; without it they
 // are requested one column ahead.
 template <int NQ, bool MATCH_LDS>
-__global__ __launch_bounds__(NTP) void inside_fwd_ml1_pipe_kernel(const float *__restrict__ match_all,
-                                                                 const int64_t *__restrict__ out_len,
-                                                                 const int64_t *__restrict__ tgt_len, float *__restrict__ S,
-                                                                 float *__restrict__ aux, int L, int T, int Mc, int spin_limit) {
+__device__ __forceinline__ void inside_fwd_ml1_pipe_body(const int bid, const float *__restrict__ match_all,
+                                                        const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
+                                                        float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc,
+                                                        int spin_limit) {
     constexpr int MP = 64 * NQ, CL = MP / NLP;
     __shared__ __attribute__((aligned(16))) float col[2][MP];
     __shared__ float sm_Dv[2];  // shift of the step that reads column t: maximum of the visible part of column t+1
     __shared__ int sm_dead;
     extern __shared__ float sm_match[];
     float *sm_main = sm_match, *sm_leaf = sm_match + NLP * T;
-    const int b = blockIdx.x / CL, k = CL - 1 - blockIdx.x % CL;  // the leading (highest) block first
+    const int b = bid / CL, k = CL - 1 - bid % CL;  // the leading (highest) block first
     const int tid = threadIdx.x, gidx = (tid >> 4) & (NLP - 1), j = tid & 15, lane = tid & 63;
     const bool collector = tid >= 16 * NLP;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
@@ -1914,7 +1929,7 @@ __global__ __launch_bounds__(NTP) void inside_fwd_ml1_pipe_kernel(const float *_
     float *Sb = S + (size_t)b * Mc * (T + 2);
     AuxViewStream av(aux, b, Mc, T);
     ExchangeView xv(aux, b, Mc, T);
-    const int part = (blockIdx.x % CL) * NTP + tid, nparts = CL * NTP;  // the sentence's element-wise work is split over the blocks
+    const int part = (bid % CL) * NTP + tid, nparts = CL * NTP;  // the sentence's element-wise work is split over the blocks
 
     if (!lengths_ok(m, n, L, T)) {
         for (int i = part; i < Mc * (T + 2); i += nparts) Sb[i] = (i == 0) ? __builtin_nanf("") : NEG_INF_F;
@@ -2074,6 +2089,317 @@ __global__ __launch_bounds__(NTP) void inside_fwd_ml1_pipe_kernel(const float *_
         if (sm_dead) {  // uniform: written before the barrier
             if (tid == 0) __hip_atomic_store(xv.flags + FLAG_FWD, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             return;
+        }
+    }
+}
+
+template <int NQ, bool MATCH_LDS>
+__global__ __launch_bounds__(NTP) void inside_fwd_ml1_pipe_kernel(const float *__restrict__ match_all,
+                                                                 const int64_t *__restrict__ out_len,
+                                                                 const int64_t *__restrict__ tgt_len, float *__restrict__ S,
+                                                                 float *__restrict__ aux, int L, int T, int Mc, int spin_limit) {
+    inside_fwd_ml1_pipe_body<NQ, MATCH_LDS>((int)blockIdx.x, match_all, out_len, tgt_len, S, aux, L, T, Mc, spin_limit);
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// The two pipelined sweeps side by side (single call, graphs of 130..1026 nodes).  Like the paired sweeps of short graphs:
+// the outside recurrence needs links, emissions and its own earlier columns, not the inside table, so the outside pipeline
+// need not follow the forward one - provided it stops borrowing the forward's column shifts.  Here every block of the
+// outside sweep chooses its own shifts (e_{t+1} = maximum of the part of the weight columns W0_{t-1}, W1_{t-1} it saw) and
+// keeps offsets P_t = e_1 + .. + e_t of its own (true value = relative value + P_t); what it publishes are absolute
+// weights (as doubles) which the readers bring to their own offsets, exactly as the forward sweep does with its
+// columns.  pipeline_finish_outside_kernel then moves the blocks' tables (Bh, W0, W1) to the offsets of the last block
+// that holds nodes of the sentence - it saw every column whole - and writes one correction per column for the
+// posterior kernels,
+//   corr_t  = P_t     + O_t - ll      (rule a -> c at column t; emission with the null left child; base cell)
+//   corr1_t = P_{t-1} + O_t - ll      (emissions that go through the local leaf),
+// with O_t the forward's offsets; for a sentence whose outside sweep was redone on the forward's offsets by the
+// one-workgroup kernel they are 0 and -D_t.
+// ------------------------------------------------------------------------------------------------------------
+template <int NQ, bool MATCH_LDS>
+__device__ __forceinline__ void outside_free_ml1_pipe_body(const int bid, const float *__restrict__ match_all,
+                                                          const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
+                                                          float *__restrict__ aux, int L, int T, int Mc, int spin_limit) {
+    constexpr int MP = 64 * NQ, CL = MP / NLP;
+    __shared__ __attribute__((aligned(16))) float w0[2][MP];
+    __shared__ __attribute__((aligned(16))) float w1[2][MP];
+    __shared__ float sm_Ev[2];  // shift chosen at the step that reads the columns t: maximum of the visible part of the columns t-1
+    __shared__ int sm_dead;
+    extern __shared__ float sm_em[];
+    float *sm_main = sm_em, *sm_leaf = sm_em + NLP * T;
+    const int b = bid / CL, k = bid % CL;  // the leading (lowest) block first
+    const int tid = threadIdx.x, gidx = (tid >> 4) & (NLP - 1), j = tid & 15, lane = tid & 63;
+    const bool collector = tid >= 16 * NLP;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *mt = match_all + (size_t)b * L * T;
+    AuxViewStream av(aux, b, Mc, T);
+    ExchangeView xv(aux, b, Mc, T);
+    if (!lengths_ok(m, n, L, T)) return;  // the posterior kernels write zeros for such sentences
+    const int mc = m / 2;
+    if (NLP * k >= mc) return;  // no node of the sentence in this block: nobody waits for it
+    for (int i = tid; i < 2 * MP; i += NTP) {
+        (&w0[0][0])[i] = NEG_INF_F;
+        (&w1[0][0])[i] = NEG_INF_F;
+    }
+    if (tid == 0) {
+        sm_dead = 0;
+        sm_Ev[0] = 0.f;
+        sm_Ev[1] = 0.f;
+    }
+    if (MATCH_LDS) {
+        for (int i = tid; i < NLP * T; i += NTP) {
+            const int g = i / T, s = i - g * T, node = NLP * k + g;
+            const bool ok = node < mc && s < n;
+            sm_main[i] = ok ? to_b2(mt[(size_t)(2 * node + 1) * T + s]) : NEG_INF_F;
+            sm_leaf[i] = (ok && node >= 1) ? to_b2(mt[(size_t)(2 * node) * T + s]) : NEG_INF_F;
+        }
+    }
+
+    // this lane's node and its transposed link rows: parents a <= c, chunks [0, q1)
+    const int c_id = NLP * k + gidx;
+    const bool live = c_id < mc;
+    const int ci = live ? c_id : NLP * k;
+    const int q1 = (NLP * k + NLP - 1) / 64 + 1;
+    float4 A0[NQ], A1[NQ];
+    if (!collector) {
+        const float4 *r0 = reinterpret_cast<const float4 *>(av.At + ((size_t)0 * Mc + ci) * MP) + j;
+        const float4 *r1 = reinterpret_cast<const float4 *>(av.At + ((size_t)1 * Mc + ci) * MP) + j;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            A0[q] = r0[16 * q];
+            A1[q] = r1[16 * q];
+        }
+    }
+    const float *ra = mt + (size_t)(2 * ci + 1) * T, *rl = mt + (size_t)(2 * ci) * T;
+    __syncthreads();  // the cleared columns
+    // beta[root][0] = 0 with P_0 = P_1 = 0: the only weight of column 1 is the root's, match[root][0]
+    const float w00 = to_b2(mt[(size_t)1 * T]);
+    if (tid == 0) w0[1][0] = w00;
+    float bp = (c_id == 0) ? 0.f : NEG_INF_F;  // the node's relative outside score one column earlier
+    if (!collector && j == 0 && live) {
+        av.BETA[(size_t)c_id * (T + 2)] = bp;
+        av.W0[(size_t)c_id * (T + 2) + 1] = (c_id == 0) ? w00 : NEG_INF_F;
+        av.W1[(size_t)c_id * (T + 2) + 1] = NEG_INF_F;
+    }
+    float mc_t, ml_p;  // main[c][t], leaf[c][t-1]
+    if (MATCH_LDS) {
+        mc_t = sm_main[gidx * T + 1];
+        ml_p = sm_leaf[gidx * T];
+    } else {
+        mc_t = live ? to_b2(ra[1]) : NEG_INF_F;
+        ml_p = (live && ci >= 1) ? to_b2(rl[0]) : NEG_INF_F;
+    }
+    // The link rows must have arrived before the sweep starts: a wait for them inside the loop would, from the second
+    // column on, be a wait for the stores of the column before.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+
+    unsigned long long *Xo = xv.obw;
+    float *Ek = xv.shiftsE + (size_t)k * (T + 4);
+    if (tid == 0) {
+        Ek[0] = 0.f;
+        Ek[1] = 0.f;
+    }
+    const unsigned long long MINUS_INF64 = (unsigned long long)__double_as_longlong(-__builtin_huge_val());
+    unsigned long long x0[NQ], x1[NQ];  // collector: the entries of the blocks below, requested one step before they are handed on
+#pragma unroll
+    for (int r = 0; r < NQ; r++) {
+        const bool need = collector && k > 0 && n >= 3;
+        x0[r] = need ? entry_load(Xo + (size_t)2 * 2 * MP + 64 * r + lane) : MINUS_INF64;
+        x1[r] = need ? entry_load(Xo + (size_t)2 * 2 * MP + MP + 64 * r + lane) : MINUS_INF64;
+    }
+    double P = 0.0;      // P_t, the offset of the columns being read
+    float e_cur = 0.f;   // e_t
+    for (int t = 1; t <= n - 1; t++) {
+        const float *c0 = w0[t & 1], *c1 = w1[t & 1];
+        float *n0 = w0[(t + 1) & 1], *n1 = w1[(t + 1) & 1];
+        const bool more = t < n - 1;
+        const float E = sm_Ev[t & 1];
+        const float e_next = is_finite(E) ? E : 0.f;  // e_{t+1}
+        const double P_next = P + (double)e_next;     // P_{t+1}
+        if (collector) {
+            if (more && k > 0) {  // the weights of the blocks below for column t+1, requested one iteration ago
+                const unsigned long long *src = Xo + (size_t)(t + 1) * 2 * MP + lane;
+                // the requests went out for every lane (a branch around a load ends in a wait for it); entries of other
+                // blocks' nodes beyond the sentence are never written and read as -inf
+#pragma unroll
+                for (int r = 0; r < NQ; r++) {
+                    if (64 * r + lane >= min(NLP * k, mc)) {
+                        x0[r] = MINUS_INF64;
+                        x1[r] = MINUS_INF64;
+                    }
+                }
+                for (int spins = 0;; spins++) {
+                    bool pending = false;
+#pragma unroll
+                    for (int r = 0; r < NQ; r++) pending |= (x0[r] == EMPTY64) | (x1[r] == EMPTY64);
+                    if (!__any(pending)) break;
+                    if (spins >= spin_limit || ((spins & 63) == 63 && gave_up(xv.flags + FLAG_BWD))) {
+                        sm_dead = 1;
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(2);  // leave the issue slots of this SIMD to its compute wave
+#pragma unroll
+                    for (int r = 0; r < NQ; r++) {
+                        if (x0[r] == EMPTY64) x0[r] = entry_load(src + 64 * r);
+                        if (x1[r] == EMPTY64) x1[r] = entry_load(src + MP + 64 * r);
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < NQ; r++) {
+                    const int i = 64 * r + lane;
+                    if (i < NLP * k) {
+                        n0[i] = (x0[r] == EMPTY64) ? NEG_INF_F : (float)(__longlong_as_double((long long)x0[r]) - P_next);
+                        n1[i] = (x1[r] == EMPTY64) ? NEG_INF_F : (float)(__longlong_as_double((long long)x1[r]) - P_next);
+                    }
+                }
+            }
+            if (t + 2 <= n - 1 && k > 0) {  // request column t+2 now: it has the whole next step to arrive
+                const unsigned long long *src = Xo + (size_t)(t + 2) * 2 * MP + lane;
+#pragma unroll
+                for (int r = 0; r < NQ; r++) {
+                    x0[r] = entry_load(src + 64 * r);
+                    x1[r] = entry_load(src + MP + 64 * r);
+                }
+            }
+            // the shift of the next step from the visible part of the columns t, which is complete
+            float vm = NEG_INF_F;
+#pragma unroll
+            for (int r = 0; r < NQ; r++) {
+                const int i = 64 * r + lane;
+                if (i < NLP * (k + 1)) vm = fmaxf(vm, fmaxf(c0[i], c1[i]));
+            }
+            vm = wave_max(vm);
+            if (lane == 0) sm_Ev[(t + 1) & 1] = vm;
+        } else {
+            float mc_raw = 0.f, ml_raw = 0.f;
+            if (more) {
+                mc_raw = MATCH_LDS ? sm_main[gidx * T + t + 1] : ra[t + 1];
+                ml_raw = MATCH_LDS ? sm_leaf[gidx * T + t] : rl[t];
+            }
+            const float4 *u0 = reinterpret_cast<const float4 *>(c0) + j, *u1 = reinterpret_cast<const float4 *>(c1) + j;
+            float beta, unused;
+            slab_row_lse<NQ, true>(A0, A1, u0, u1, 0, q1, live, true, bp, beta, unused);
+            if (!live) beta = NEG_INF_F;
+            const float nw0 = (mc_t + beta) - e_next;
+            const float nw1 = ((ml_p + mc_t) + bp) - (e_next + e_cur);
+            if (j == 0) {
+                n0[c_id] = nw0;
+                n1[c_id] = nw1;
+                if (live) {
+                    if (more) {
+                        entry_store(Xo + (size_t)(t + 1) * 2 * MP + c_id, (double)nw0 + P_next);
+                        entry_store(Xo + (size_t)(t + 1) * 2 * MP + MP + c_id, (double)nw1 + P_next);
+                    }
+                    av.BETA[(size_t)c_id * (T + 2) + t] = beta;
+                    av.W0[(size_t)c_id * (T + 2) + t + 1] = nw0;
+                    av.W1[(size_t)c_id * (T + 2) + t + 1] = nw1;
+                }
+            }
+            if (tid == 0) Ek[t + 1] = e_next;
+            bp = beta;
+            mc_t = MATCH_LDS ? mc_raw : (live ? to_b2(mc_raw) : NEG_INF_F);
+            ml_p = MATCH_LDS ? ml_raw : ((live && ci >= 1) ? to_b2(ml_raw) : NEG_INF_F);
+        }
+        e_cur = e_next;
+        P = P_next;
+        lds_barrier();
+        if (sm_dead) {  // uniform: written before the barrier
+            if (tid == 0) __hip_atomic_store(xv.flags + FLAG_BWD, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+    }
+}
+
+// Both sweeps in one launch: the first `fwd_blocks` workgroups are the forward pipeline's, the others the outside one's
+// (leading blocks first within either).
+template <int NQ, bool MATCH_LDS>
+__global__ __launch_bounds__(NTP) void inside_both_ml1_pipe_kernel(const float *__restrict__ match_all,
+                                                                  const int64_t *__restrict__ out_len,
+                                                                  const int64_t *__restrict__ tgt_len, float *__restrict__ S,
+                                                                  float *__restrict__ aux, int L, int T, int Mc, int spin_limit,
+                                                                  int fwd_blocks) {
+    if ((int)blockIdx.x < fwd_blocks)  // workgroup-uniform
+        inside_fwd_ml1_pipe_body<NQ, MATCH_LDS>((int)blockIdx.x, match_all, out_len, tgt_len, S, aux, L, T, Mc, spin_limit);
+    else
+        outside_free_ml1_pipe_body<NQ, MATCH_LDS>((int)blockIdx.x - fwd_blocks, match_all, out_len, tgt_len, aux, L, T, Mc, spin_limit);
+}
+
+// After the sweeps side by side (and the forward's redo, if any): grid (CL, B), 256 threads.  Block k < K (K = the last
+// block with nodes of the sentence) moves its outside tables to block K's offsets, delta_t = P^k_t - P^K_t:
+// Bh[c][t], W0[c][t], W1[c][t] += delta_t.  Block K writes the corrections corr_t, corr1_t (see above).  A sentence
+// whose outside sweep gave up is redone afterwards on the forward's offsets: corr = 0, corr1_t = -D_t.
+// Dynamic LDS: two rows of T+4 doubles.
+__global__ __launch_bounds__(256) void pipeline_finish_outside_kernel(float *__restrict__ aux, const int64_t *__restrict__ out_len,
+                                                                     const int64_t *__restrict__ tgt_len, int L, int T, int Mc) {
+    extern __shared__ double sm_row[];  // [2][T+4]
+    double *sm_a = sm_row, *sm_b = sm_row + (T + 4);
+    const int k = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    if (!lengths_ok(m, n, L, T)) return;
+    const int mc = m / 2, K = (mc - 1) / NLP, CLEN = corr_len(T);
+    if (k > K) return;
+    AuxViewStream av(aux, b, Mc, T);
+    ExchangeView xv(aux, b, Mc, T);
+    const bool redo = xv.flags[FLAG_BWD] != 0;
+    const float *EK = xv.shiftsE + (size_t)K * (T + 4);
+    if (k == K) {
+        if (redo) {
+            for (int t = tid; t < T + 4 && t < CLEN; t += 256) {
+                xv.corr[t] = 0.f;
+                xv.corr[CLEN + t] = -av.D[t];
+            }
+            return;
+        }
+        // P_t = e_1 + .. + e_t (sm_a), O_t = D_{t+1} + .. + D_{n-1} (sm_b); short serial scans by one thread
+        for (int t = tid; t < T + 4; t += 256) {
+            sm_a[t] = (t >= 1 && t <= n - 1) ? (double)EK[t] : 0.0;
+            sm_b[t] = (t >= 1 && t <= n - 1) ? (double)av.D[t] : 0.0;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            double acc = 0.0;
+            for (int t = 0; t <= n - 1; t++) {
+                acc += sm_a[t];
+                sm_a[t] = acc;
+            }
+            acc = 0.0;
+            for (int t = n - 1; t >= 0; t--) {
+                const double d = sm_b[t];
+                sm_b[t] = acc;
+                acc += d;
+            }
+        }
+        __syncthreads();
+        const double ll_abs = (double)av.SR[0] + sm_b[0];
+        for (int t = tid; t < CLEN; t += 256) {
+            const bool in = t <= n - 1;
+            xv.corr[t] = in ? (float)(sm_a[t] + sm_b[t] - ll_abs) : 0.f;
+            xv.corr[CLEN + t] = (in && t >= 1) ? (float)(sm_a[t - 1] + sm_b[t] - ll_abs) : 0.f;
+        }
+        return;
+    }
+    if (redo) return;
+    const float *Ek = xv.shiftsE + (size_t)k * (T + 4);
+    for (int t = tid; t < T + 4; t += 256) sm_a[t] = (t >= 1 && t <= n - 1) ? (double)Ek[t] - (double)EK[t] : 0.0;
+    __syncthreads();
+    if (tid == 0) {
+        double acc = 0.0;
+        for (int t = 0; t <= n - 1; t++) {
+            acc += sm_a[t];
+            sm_a[t] = acc;  // delta_t
+        }
+    }
+    __syncthreads();
+    const int TS = T + 2, cells = NLP * TS;
+    for (int i = tid; i < cells; i += 256) {
+        const int g = i / TS, t = i - g * TS, c_id = NLP * k + g;
+        if (c_id >= mc || t > n - 1) continue;
+        const size_t o = (size_t)c_id * TS + t;
+        av.BETA[o] = (float)((double)av.BETA[o] + sm_a[t]);
+        if (t >= 1) {
+            av.W0[o] = (float)((double)av.W0[o] + sm_a[t]);
+            av.W1[o] = (float)((double)av.W1[o] + sm_a[t]);
         }
     }
 }
@@ -2321,12 +2647,13 @@ __global__ __launch_bounds__(NTP) void inside_bwd_ml1_pipe_kernel(const float *_
 }
 
 // Rule posteriors from the outside weights: lg[a][k][c] = g * sum_{t=1}^{n-1} exp(links[a][k][c] + Wk[a][t] + R[c][t]).
-// One block per 32x32 tile of (parent, child) pairs; the slab has been zero-filled beforehand.
+// One block per 32x32 tile of (parent, child) pairs; the slab has been zero-filled beforehand.  use_corr: the outside
+// tables are relative to offsets of their own (sweeps side by side) and every column takes its correction corr_t.
 __global__ __launch_bounds__(1024) void links_grad_ml1_stream_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
                                                                     const float *__restrict__ aux_c, const float *__restrict__ links,
                                                                     const int64_t *__restrict__ out_len,
                                                                     const int64_t *__restrict__ tgt_len, float *__restrict__ lgrad,
-                                                                    int L, int T, int Mc, int B) {
+                                                                    int L, int T, int Mc, int B, int use_corr) {
     __shared__ float sw0[32][33], sw1[32][33], ss[32][33];
     const int b = blockIdx.z, at = blockIdx.y, ct = blockIdx.x;
     if (ct < at) return;
@@ -2337,6 +2664,7 @@ __global__ __launch_bounds__(1024) void links_grad_ml1_stream_kernel(const float
     const int mc = m / 2;
     if (at * 32 >= mc || ct * 32 >= mc) return;
     AuxViewStream av(const_cast<float *>(aux_c), b, Mc, T);
+    const float *corr = ExchangeView(const_cast<float *>(aux_c), b, Mc, T).corr;  // per column, when the sweeps ran side by side
     const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)B);
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     const int a_id = at * 32 + ty, c_id = ct * 32 + tx;
@@ -2353,7 +2681,7 @@ __global__ __launch_bounds__(1024) void links_grad_ml1_stream_kernel(const float
         const bool tin = tt <= n - 1;
         sw0[ty][tx] = (tin && ra < mc) ? av.W0[(size_t)ra * (T + 2) + tt] : NEG_INF_F;
         sw1[ty][tx] = (tin && ra < mc) ? av.W1[(size_t)ra * (T + 2) + tt] : NEG_INF_F;
-        ss[ty][tx] = (tin && rc < mc) ? av.SR[(size_t)rc * (T + 2) + tt] : NEG_INF_F;
+        ss[ty][tx] = (tin && rc < mc) ? av.SR[(size_t)rc * (T + 2) + tt] + (use_corr ? corr[tt] : 0.f) : NEG_INF_F;
         __syncthreads();
 #pragma unroll 8
         for (int u = 0; u < 32; u++) {
@@ -2375,7 +2703,7 @@ __global__ __launch_bounds__(256) void match_grad_ml1_stream_kernel(const float 
                                                                    const float *__restrict__ aux_c, const float *__restrict__ match_all,
                                                                    const int64_t *__restrict__ out_len,
                                                                    const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad, int L,
-                                                                   int T, int Mc, int B) {
+                                                                   int T, int Mc, int B, int use_corr) {
     const int b = blockIdx.y;
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= L * T) return;
@@ -2392,20 +2720,25 @@ __global__ __launch_bounds__(256) void match_grad_ml1_stream_kernel(const float 
     AuxViewStream av(const_cast<float *>(aux_c), b, Mc, T);
     const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)B);
     const int x = i / T, s = i - x * T;
+    // corrections of the columns (see pipeline_finish_outside_kernel): on the forward's offsets they are 0 and -D_t
+    const float *corr = ExchangeView(const_cast<float *>(aux_c), b, Mc, T).corr;
+    const int CLEN = corr_len(T);
     float out = 0.f;
     if (x >= 1 && x < m && s < n) {
         const int a_id = x >> 1;
         const size_t row = (size_t)a_id * (T + 2);
+        const float c0 = use_corr ? corr[s] : 0.f;
         if (x & 1) {
             const float bs = av.BETA[row + s];
             const float mas = to_b2(mt[(size_t)x * T + s]);
-            if (s + 1 <= n - 1) out += ex2(bs + mas + av.F0[row + s + 1]);
+            if (s + 1 <= n - 1) out += ex2((bs + mas + av.F0[row + s + 1]) + c0);
             if (s >= 1 && s + 1 <= n - 1 && a_id >= 1)
-                out += ex2(av.BETA[row + s - 1] + to_b2(mt[(size_t)(x - 1) * T + s - 1]) + mas + (av.F1[row + s + 1] - av.D[s]));
-            if (a_id == mc - 1 && s == n - 1) out += ex2(bs + mas);
+                out += ex2(av.BETA[row + s - 1] + to_b2(mt[(size_t)(x - 1) * T + s - 1]) + mas +
+                           (av.F1[row + s + 1] + (use_corr ? corr[CLEN + s] : -av.D[s])));
+            if (a_id == mc - 1 && s == n - 1) out += ex2((bs + mas) + c0);
         } else if (a_id >= 1 && a_id < mc && s + 2 <= n - 1) {
             out += ex2(av.BETA[row + s] + to_b2(mt[(size_t)x * T + s]) + to_b2(mt[(size_t)(x + 1) * T + s + 1]) +
-                       (av.F1[row + s + 2] - av.D[s + 1]));
+                       (av.F1[row + s + 2] + (use_corr ? corr[CLEN + s + 1] : -av.D[s + 1])));
         }
         if (!(out == out)) out = 0.f;
     }
@@ -2437,10 +2770,20 @@ int pipeline_chunks(int B, int T, int Mc) {  // NQ, or 0 where the pipelined swe
 
 template <int NQ>
 int launch_fwd_pipe(const float *match_all, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B, int L, int T, int Mc,
-                    hipStream_t stream) {
+                    hipStream_t stream, bool both) {
     constexpr int CL = 64 * NQ / NLP;
     const size_t match_bytes = (size_t)2 * NLP * T * sizeof(float);
-    if (match_bytes <= LDS_BUDGET - 8192) {
+    if (both) {  // the outside pipeline in the same launch, behind the forward one in dispatch order
+        if (match_bytes <= LDS_BUDGET - 8192) {
+            auto k = inside_both_ml1_pipe_kernel<NQ, true>;
+            PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)match_bytes));
+            hipLaunchKernelGGL(k, dim3(2 * B * CL), dim3(NTP), match_bytes, stream, match_all, ol, tl, S, aux, L, T, Mc,
+                               g_pipeline_spin_limit.load(), B * CL);
+        } else {
+            hipLaunchKernelGGL((inside_both_ml1_pipe_kernel<NQ, false>), dim3(2 * B * CL), dim3(NTP), 0, stream, match_all, ol, tl, S, aux,
+                               L, T, Mc, g_pipeline_spin_limit.load(), B * CL);
+        }
+    } else if (match_bytes <= LDS_BUDGET - 8192) {
         auto k = inside_fwd_ml1_pipe_kernel<NQ, true>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)match_bytes));
         hipLaunchKernelGGL(k, dim3(B * CL), dim3(NTP), match_bytes, stream, match_all, ol, tl, S, aux, L, T, Mc,
@@ -2473,8 +2816,14 @@ int launch_bwd_pipe(const float *S, float *aux, const float *match_all, const in
     return PCFGNAT_OK;
 }
 
+// The sweeps run side by side while the batch needs no more than the configured number of workgroups for both pipelines.
+bool side_by_side_applies(int B, int T, int Mc) {
+    const int NQ = pipeline_chunks(B, T, Mc);
+    return NQ != 0 && (int64_t)2 * B * (64 * NQ / NLP) <= g_pipeline_max_wg.load();
+}
+
 int launch_fwd_stream(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B,
-                      int L, int T, int Mc, hipStream_t stream) {
+                      int L, int T, int Mc, hipStream_t stream, bool side_by_side = false) {
     const int MP = stream_mp(Mc);
     PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss: aux must be 16-byte aligned");
     hipLaunchKernelGGL(compact_links_ml1_kernel, dim3(MP / 32, MP / 32, B), dim3(256), 0, stream, links, ol, aux, L, T, Mc, MP);
@@ -2483,13 +2832,13 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
     const int NQ = pipeline_chunks(B, T, Mc);
     int rc = PCFGNAT_OK;
     switch (NQ) {
-        case 2: rc = launch_fwd_pipe<2>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
-        case 3: rc = launch_fwd_pipe<3>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
-        case 4: rc = launch_fwd_pipe<4>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
-        case 5: rc = launch_fwd_pipe<5>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
-        case 6: rc = launch_fwd_pipe<6>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
-        case 7: rc = launch_fwd_pipe<7>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
-        case 8: rc = launch_fwd_pipe<8>(match_all, ol, tl, S, aux, B, L, T, Mc, stream); break;
+        case 2: rc = launch_fwd_pipe<2>(match_all, ol, tl, S, aux, B, L, T, Mc, stream, side_by_side); break;
+        case 3: rc = launch_fwd_pipe<3>(match_all, ol, tl, S, aux, B, L, T, Mc, stream, side_by_side); break;
+        case 4: rc = launch_fwd_pipe<4>(match_all, ol, tl, S, aux, B, L, T, Mc, stream, side_by_side); break;
+        case 5: rc = launch_fwd_pipe<5>(match_all, ol, tl, S, aux, B, L, T, Mc, stream, side_by_side); break;
+        case 6: rc = launch_fwd_pipe<6>(match_all, ol, tl, S, aux, B, L, T, Mc, stream, side_by_side); break;
+        case 7: rc = launch_fwd_pipe<7>(match_all, ol, tl, S, aux, B, L, T, Mc, stream, side_by_side); break;
+        case 8: rc = launch_fwd_pipe<8>(match_all, ol, tl, S, aux, B, L, T, Mc, stream, side_by_side); break;
         default: break;
     }
     if (rc != PCFGNAT_OK) return rc;
@@ -2505,11 +2854,19 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
                            T, Mc, MP, only_flagged);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
+    if (side_by_side) {  // the outside tables to common offsets, and the corrections of the posteriors
+        hipLaunchKernelGGL(pipeline_finish_outside_kernel, dim3(64 * NQ / NLP, B), dim3(256), (size_t)2 * (T + 4) * sizeof(double), stream,
+                           aux, ol, tl, L, T, Mc);
+        PCFGNAT_HIP_CHECK(hipGetLastError());
+    }
     return PCFGNAT_OK;
 }
 
+// side_by_side: the outside pipeline has already run, beside the forward one (launch_both_stream): only the redo of the
+// sentences it gave up and the posteriors (with their per-column corrections) are left to do.
 int launch_bwd_stream(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
-                      const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream) {
+                      const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream,
+                      bool side_by_side = false) {
     const int MP = stream_mp(Mc);
     const int tiles = (Mc + 31) / 32;
     PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss_backward: aux must be 16-byte aligned");
@@ -2517,7 +2874,7 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
     const int NQ = pipeline_chunks(B, T, Mc);
     int rc = PCFGNAT_OK;
-    switch (NQ) {
+    switch (side_by_side ? 0 : NQ) {
         case 2: rc = launch_bwd_pipe<2>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
         case 3: rc = launch_bwd_pipe<3>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
         case 4: rc = launch_bwd_pipe<4>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
@@ -2542,10 +2899,12 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
     const size_t nlg = (size_t)B * L * 2 * L;
     hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, stream, lg, nlg);
     PCFGNAT_HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL(links_grad_ml1_stream_kernel, dim3(tiles, tiles, B), dim3(1024), 0, stream, go, S, aux, links, ol, tl, lg, L, T, Mc, norm_B);
+    const int use_corr = side_by_side ? 1 : 0;
+    hipLaunchKernelGGL(links_grad_ml1_stream_kernel, dim3(tiles, tiles, B), dim3(1024), 0, stream, go, S, aux, links, ol, tl, lg, L, T, Mc,
+                       norm_B, use_corr);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL(match_grad_ml1_stream_kernel, dim3((L * T + 255) / 256, B), dim3(256), 0, stream, go, S, aux, match_all, ol, tl, mg, L,
-                       T, Mc, norm_B);
+                       T, Mc, norm_B, use_corr);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -2724,6 +3083,12 @@ int pcfgnat::inside_forward_backward_impl(const float *grad_output, const float 
         rc = launch_fused<1>(grad_output, match_all, links, output_length, target_length, S, aux, match_all_grad, links_grad, (int)B, (int)L,
                              (int)T, Mc, (int)norm_B, s, &done, pad, pad_done);
     if (rc != PCFGNAT_OK || done) return rc;
+    if (ml == 1 && Mc > 64 && side_by_side_applies((int)B, (int)T, Mc)) {  // the two pipelined sweeps in one launch
+        rc = launch_fwd_stream(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s, true);
+        if (rc != PCFGNAT_OK) return rc;
+        return launch_bwd_stream(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
+                                 (int)L, (int)T, Mc, (int)norm_B, s, true);
+    }
     rc = pcfgnat_pcfg_loss(match_all, links, output_length, target_length, S, aux, B, L, T, ml, stream);
     if (rc != PCFGNAT_OK) return rc;
     return inside_backward_impl(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, B, L, T,

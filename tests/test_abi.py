@@ -31,8 +31,8 @@ def test_library_exports_every_declared_symbol():
     assert lib.pcfgnat_abi_version() == 1
     assert lib.pcfgnat_pcfg_aux_floats(40, 128, 32, 1) == 40 * (6 * 64 * 34 + 6 * 36)
     # more than 128 main-chain nodes: six tables, the shifts (padded to 16 bytes), two link copies with rows of 64*ceil(Mc/64)
-    assert lib.pcfgnat_pcfg_aux_floats(8, 512, 140, 1) == 8 * (6 * 256 * 142 + 144 + 4 * 256 * 256 + 4 * 256 * 142 + 16 * 144 + 4)
-    assert lib.pcfgnat_pcfg_aux_floats(1, 282, 9, 1) == (6 * 141 * 11 + 13 + 3) // 4 * 4 + 4 * 141 * 192 + 4 * 192 * 11 + 12 * 13 + 4
+    assert lib.pcfgnat_pcfg_aux_floats(8, 512, 140, 1) == 8 * (6 * 256 * 142 + 144 + 4 * 256 * 256 + 4 * 256 * 142 + 16 * 144 + 4 + 4 * 256 * 142 + 16 * 144 + 2 * 144)
+    assert lib.pcfgnat_pcfg_aux_floats(1, 282, 9, 1) == (6 * 141 * 11 + 13 + 3) // 4 * 4 + 4 * 141 * 192 + 4 * 192 * 11 + 12 * 13 + 4 + 4 * 192 * 11 + 12 * 13 + 2 * 14
 
 
 def test_argument_errors_without_gpu():
