@@ -2108,7 +2108,7 @@ __global__ __launch_bounds__(NTP) void inside_fwd_ml1_pipe_kernel(const float *_
 // outside sweep chooses its own shifts (e_{t+1} = maximum of the part of the weight columns W0_{t-1}, W1_{t-1} it saw) and
 // keeps offsets P_t = e_1 + .. + e_t of its own (true value = relative value + P_t); what it publishes are absolute
 // weights (as doubles) which the readers bring to their own offsets, exactly as the forward sweep does with its
-// columns.  pipeline_finish_outside_kernel then moves the blocks' tables (Bh, W0, W1) to the offsets of the last block
+// columns.  pipeline_finish_kernel then moves the blocks' tables (Bh, W0, W1) to the offsets of the last block
 // that holds nodes of the sentence - it saw every column whole - and writes one correction per column for the
 // posterior kernels,
 //   corr_t  = P_t     + O_t - ll      (rule a -> c at column t; emission with the null left child; base cell)
@@ -2330,11 +2330,38 @@ __global__ __launch_bounds__(NTP) void inside_both_ml1_pipe_kernel(const float *
 // Bh[c][t], W0[c][t], W1[c][t] += delta_t.  Block K writes the corrections corr_t, corr1_t (see above).  A sentence
 // whose outside sweep gave up is redone afterwards on the forward's offsets: corr = 0, corr1_t = -D_t.
 // Dynamic LDS: two rows of T+4 doubles.
-__global__ __launch_bounds__(256) void pipeline_finish_outside_kernel(float *__restrict__ aux, const int64_t *__restrict__ out_len,
-                                                                     const int64_t *__restrict__ tgt_len, int L, int T, int Mc) {
-    extern __shared__ double sm_row[];  // [2][T+4]
+// Inclusive prefix sums of v[0..len) in place (LDS, doubles) by the 256 threads of a workgroup: every thread sums a run of
+// consecutive entries, the runs are chained by shuffles inside the waves and through `part` (LDS, four doubles) across
+// them.  All threads must call it; barriers inside.
+__device__ __forceinline__ void block_prefix_sum(double *v, int len, double *part, int tid) {
+    const int run = (len + 255) / 256, lo = tid * run;
+    double acc = 0.0;
+    for (int i = 0; i < run; i++)
+        if (lo + i < len) acc += v[lo + i];
+    double incl = acc;
+    for (int o = 1; o < 64; o <<= 1) {
+        const double y = __shfl_up(incl, o);
+        if ((tid & 63) >= o) incl += y;
+    }
+    if ((tid & 63) == 63) part[tid >> 6] = incl;
+    __syncthreads();
+    double run_sum = incl - acc;  // the entries before this thread's run
+    for (int w = 0; w < (tid >> 6); w++) run_sum += part[w];
+    for (int i = 0; i < run; i++) {
+        if (lo + i < len) {
+            run_sum += v[lo + i];
+            v[lo + i] = run_sum;
+        }
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ void pipeline_finish_outside_block(const int k, const int b, float *__restrict__ aux,
+                                                              const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
+                                                              int L, int T, int Mc, double *sm_row) {
+    __shared__ double sm_part[4];
     double *sm_a = sm_row, *sm_b = sm_row + (T + 4);
-    const int k = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const int tid = threadIdx.x;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     if (!lengths_ok(m, n, L, T)) return;
     const int mc = m / 2, K = (mc - 1) / NLP, CLEN = corr_len(T);
@@ -2345,72 +2372,69 @@ __global__ __launch_bounds__(256) void pipeline_finish_outside_kernel(float *__r
     const float *EK = xv.shiftsE + (size_t)K * (T + 4);
     if (k == K) {
         if (redo) {
-            for (int t = tid; t < T + 4 && t < CLEN; t += 256) {
+            for (int t = tid; t < CLEN; t += 256) {
                 xv.corr[t] = 0.f;
-                xv.corr[CLEN + t] = -av.D[t];
+                xv.corr[CLEN + t] = (t < T + 4) ? -av.D[t] : 0.f;
             }
             return;
         }
-        // P_t = e_1 + .. + e_t (sm_a), O_t = D_{t+1} + .. + D_{n-1} (sm_b); short serial scans by one thread
-        for (int t = tid; t < T + 4; t += 256) {
-            sm_a[t] = (t >= 1 && t <= n - 1) ? (double)EK[t] : 0.0;
-            sm_b[t] = (t >= 1 && t <= n - 1) ? (double)av.D[t] : 0.0;
+        // sm_a[t] = P_t = e_1 + .. + e_t; sm_b[u] = D_{n-1} + .. + D_{n-1-u}, so that O_t = sm_b[n-2-t] (O_{n-1} = 0)
+        for (int t = tid; t < n; t += 256) {
+            sm_a[t] = (t >= 1) ? (double)EK[t] : 0.0;
+            sm_b[t] = (n - 1 - t >= 1) ? (double)av.D[n - 1 - t] : 0.0;
         }
         __syncthreads();
-        if (tid == 0) {
-            double acc = 0.0;
-            for (int t = 0; t <= n - 1; t++) {
-                acc += sm_a[t];
-                sm_a[t] = acc;
-            }
-            acc = 0.0;
-            for (int t = n - 1; t >= 0; t--) {
-                const double d = sm_b[t];
-                sm_b[t] = acc;
-                acc += d;
-            }
-        }
-        __syncthreads();
-        const double ll_abs = (double)av.SR[0] + sm_b[0];
+        block_prefix_sum(sm_a, n, sm_part, tid);
+        block_prefix_sum(sm_b, n, sm_part, tid);
+        const double O0 = (n >= 2) ? sm_b[n - 2] : 0.0;
+        const double ll_abs = (double)av.SR[0] + O0;
         for (int t = tid; t < CLEN; t += 256) {
             const bool in = t <= n - 1;
-            xv.corr[t] = in ? (float)(sm_a[t] + sm_b[t] - ll_abs) : 0.f;
-            xv.corr[CLEN + t] = (in && t >= 1) ? (float)(sm_a[t - 1] + sm_b[t] - ll_abs) : 0.f;
+            const double Ot = (in && t <= n - 2) ? sm_b[n - 2 - t] : 0.0;
+            xv.corr[t] = in ? (float)(sm_a[t] + Ot - ll_abs) : 0.f;
+            xv.corr[CLEN + t] = (in && t >= 1) ? (float)(sm_a[t - 1] + Ot - ll_abs) : 0.f;
         }
         return;
     }
     if (redo) return;
     const float *Ek = xv.shiftsE + (size_t)k * (T + 4);
-    for (int t = tid; t < T + 4; t += 256) sm_a[t] = (t >= 1 && t <= n - 1) ? (double)Ek[t] - (double)EK[t] : 0.0;
+    for (int t = tid; t < n; t += 256) sm_a[t] = (t >= 1) ? (double)Ek[t] - (double)EK[t] : 0.0;
     __syncthreads();
-    if (tid == 0) {
-        double acc = 0.0;
-        for (int t = 0; t <= n - 1; t++) {
-            acc += sm_a[t];
-            sm_a[t] = acc;  // delta_t
-        }
-    }
-    __syncthreads();
+    block_prefix_sum(sm_a, n, sm_part, tid);  // delta_t
     const int TS = T + 2, cells = NLP * TS;
-    for (int i = tid; i < cells; i += 256) {
-        const int g = i / TS, t = i - g * TS, c_id = NLP * k + g;
-        if (c_id >= mc || t > n - 1) continue;
-        const size_t o = (size_t)c_id * TS + t;
-        av.BETA[o] = (float)((double)av.BETA[o] + sm_a[t]);
-        if (t >= 1) {
-            av.W0[o] = (float)((double)av.W0[o] + sm_a[t]);
-            av.W1[o] = (float)((double)av.W1[o] + sm_a[t]);
+    for (int base = tid; base < cells; base += 4 * 256) {  // four cells per thread in flight
+        float bv[4], v0[4], v1[4];
+        size_t o[4];
+        int tc[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int i = base + u * 256, g = i / TS, t = i - g * TS, c_id = NLP * k + g;
+            const bool ok = i < cells && c_id < mc && t <= n - 1;
+            tc[u] = ok ? t : -1;
+            o[u] = (size_t)(ok ? c_id : NLP * k) * TS + (ok ? t : 0);
+            bv[u] = av.BETA[o[u]];
+            v0[u] = av.W0[o[u]];
+            v1[u] = av.W1[o[u]];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int t = tc[u];
+            if (t >= 0) av.BETA[o[u]] = (float)((double)bv[u] + sm_a[t]);
+            if (t >= 1) {
+                av.W0[o[u]] = (float)((double)v0[u] + sm_a[t]);
+                av.W1[o[u]] = (float)((double)v1[u] + sm_a[t]);
+            }
         }
     }
 }
 
 // Moves the tables of blocks 1 .. CL-1 from their own column offsets to those of block 0 (see above): with
 // O_s = sum_{t > s} D_t, R[a][s] is relative to O_s and F0h[a][t], F1h[a][t] to O_{t-1}.  Grid (CL-1, B).
-__global__ __launch_bounds__(256) void pipeline_rebase_kernel(float *__restrict__ aux, const int64_t *__restrict__ out_len,
-                                                             const int64_t *__restrict__ tgt_len, int L, int T, int Mc) {
-    extern __shared__ double sm_delta[];  // [T+2]: own offset minus block 0's, per column
+__device__ __forceinline__ void pipeline_rebase_block(const int k, const int b, float *__restrict__ aux,
+                                                      const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len, int L,
+                                                      int T, int Mc, double *sm_delta) {
     __shared__ double sm_part[4];
-    const int k = blockIdx.x + 1, b = blockIdx.y, tid = threadIdx.x;
+    const int tid = threadIdx.x;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     if (!lengths_ok(m, n, L, T)) return;
     const int mc = m / 2;
@@ -2468,6 +2492,24 @@ __global__ __launch_bounds__(256) void pipeline_rebase_kernel(float *__restrict_
             }
         }
     }
+}
+
+// Grid (CL-1, B).  Dynamic LDS: T+2 doubles.
+__global__ __launch_bounds__(256) void pipeline_rebase_kernel(float *__restrict__ aux, const int64_t *__restrict__ out_len,
+                                                             const int64_t *__restrict__ tgt_len, int L, int T, int Mc) {
+    extern __shared__ double sm_dyn[];
+    pipeline_rebase_block((int)blockIdx.x + 1, (int)blockIdx.y, aux, out_len, tgt_len, L, T, Mc, sm_dyn);
+}
+
+// After the sweeps side by side and the forward's redo: grid (2 CL - 1, B); the first CL-1 blocks of a sentence rebase the
+// forward tables, the other CL finish the outside sweep's.  Dynamic LDS: 2 (T+4) doubles.
+__global__ __launch_bounds__(256) void pipeline_finish_kernel(float *__restrict__ aux, const int64_t *__restrict__ out_len,
+                                                             const int64_t *__restrict__ tgt_len, int L, int T, int Mc, int CL) {
+    extern __shared__ double sm_dyn[];
+    if ((int)blockIdx.x < CL - 1)  // workgroup-uniform
+        pipeline_rebase_block((int)blockIdx.x + 1, (int)blockIdx.y, aux, out_len, tgt_len, L, T, Mc, sm_dyn);
+    else
+        pipeline_finish_outside_block((int)blockIdx.x - (CL - 1), (int)blockIdx.y, aux, out_len, tgt_len, L, T, Mc, sm_dyn);
 }
 
 // Outside sweep of one block.  Same tables as inside_bwd_ml1_stream_kernel.  Dynamic LDS: D [T+4], then (MATCH_LDS) the
@@ -2720,7 +2762,7 @@ __global__ __launch_bounds__(256) void match_grad_ml1_stream_kernel(const float 
     AuxViewStream av(const_cast<float *>(aux_c), b, Mc, T);
     const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)B);
     const int x = i / T, s = i - x * T;
-    // corrections of the columns (see pipeline_finish_outside_kernel): on the forward's offsets they are 0 and -D_t
+    // corrections of the columns (see pipeline_finish_kernel): on the forward's offsets they are 0 and -D_t
     const float *corr = ExchangeView(const_cast<float *>(aux_c), b, Mc, T).corr;
     const int CLEN = corr_len(T);
     float out = 0.f;
@@ -2776,8 +2818,11 @@ int launch_fwd_pipe(const float *match_all, const int64_t *ol, const int64_t *tl
     if (both) {  // the outside pipeline in the same launch, behind the forward one in dispatch order
         if (match_bytes <= LDS_BUDGET - 8192) {
             auto k = inside_both_ml1_pipe_kernel<NQ, true>;
-            PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)match_bytes));
-            hipLaunchKernelGGL(k, dim3(2 * B * CL), dim3(NTP), match_bytes, stream, match_all, ol, tl, S, aux, L, T, Mc,
+            // while every block of both pipelines can have a compute unit of its own, claim more than half of a unit's LDS
+            // so that no two blocks share one (and its instruction issue)
+            const size_t lds = (2 * B * CL <= 256 && match_bytes < PAD_EXCLUSIVE_LDS) ? PAD_EXCLUSIVE_LDS : match_bytes;
+            PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            hipLaunchKernelGGL(k, dim3(2 * B * CL), dim3(NTP), lds, stream, match_all, ol, tl, S, aux, L, T, Mc,
                                g_pipeline_spin_limit.load(), B * CL);
         } else {
             hipLaunchKernelGGL((inside_both_ml1_pipe_kernel<NQ, false>), dim3(2 * B * CL), dim3(NTP), 0, stream, match_all, ol, tl, S, aux,
@@ -2793,6 +2838,7 @@ int launch_fwd_pipe(const float *match_all, const int64_t *ol, const int64_t *tl
                            Mc, g_pipeline_spin_limit.load());
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
+    if (both) return PCFGNAT_OK;  // rebased together with the outside tables, once the redo of the forward has run
     hipLaunchKernelGGL(pipeline_rebase_kernel, dim3(CL - 1, B), dim3(256), (size_t)(T + 2) * sizeof(double), stream, aux, ol, tl, L, T,
                        Mc);
     PCFGNAT_HIP_CHECK(hipGetLastError());
@@ -2854,9 +2900,10 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
                            T, Mc, MP, only_flagged);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
-    if (side_by_side) {  // the outside tables to common offsets, and the corrections of the posteriors
-        hipLaunchKernelGGL(pipeline_finish_outside_kernel, dim3(64 * NQ / NLP, B), dim3(256), (size_t)2 * (T + 4) * sizeof(double), stream,
-                           aux, ol, tl, L, T, Mc);
+    if (side_by_side) {  // both sweeps' tables to common offsets, and the corrections of the posteriors
+        const int CL = 64 * NQ / NLP;
+        hipLaunchKernelGGL(pipeline_finish_kernel, dim3(2 * CL - 1, B), dim3(256), (size_t)2 * (T + 4) * sizeof(double), stream, aux, ol, tl,
+                           L, T, Mc, CL);
         PCFGNAT_HIP_CHECK(hipGetLastError());
     }
     return PCFGNAT_OK;
