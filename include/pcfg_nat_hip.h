@@ -132,8 +132,9 @@ int pcfgnat_pcfg_loss_backward(const float *grad_output, const float *S, float *
  * in one call.  For max_left = 1 and graphs of up to 128 nodes whose tables fit in LDS (every shipped training shape) the
  * inside and the outside sweep of a sentence run side by side as two workgroups of one launch - the outside recurrence
  * depends on links, emissions and its own earlier columns only, not on the inside table - and a second launch multiplies
- * their tables into the gradients; otherwise the sweeps follow each other as in the two calls.  aux (8-byte aligned,
- * pcfgnat_pcfg_aux_floats floats) carries the tables between the launches.
+ * their tables into the gradients; graphs of 130..1026 nodes are swept by two pipelines of workgroups per sentence,
+ * forward and outside, side by side in one launch (see pcfgnat_pipeline_config); otherwise the sweeps follow each other as
+ * in the two calls.  aux (pcfgnat_pcfg_aux_floats floats) carries the tables between the launches.
  */
 int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *match_all, const float *links,
                                        const int64_t *output_length, const int64_t *target_length, float *S, float *aux,
@@ -145,7 +146,8 @@ int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *ma
  * Viterbi sweep of pcfgnat_viterbi_decode for 194 <= L <= 514).  There a sentence is
  * swept by one workgroup per block of 16 main-chain nodes, the blocks following each other as a pipeline, as long as the
  * batch needs no more than max_workgroups of them (B * 4 * ceil((L/2)/64) <= max_workgroups, default 2^20), and by one
- * workgroup per sentence otherwise.  A block that waits for the one ahead of it for more than spin_limit rounds of polling
+ * workgroup per sentence otherwise.  pcfgnat_pcfg_loss_forward_backward runs the forward and the outside pipeline of a
+ * sentence side by side in one launch while twice that number fits, one after the other otherwise.  A block that waits for the one ahead of it for more than spin_limit rounds of polling
  * (default 2^20, about a second) gives the sentence up, and the one-workgroup sweep redoes it in the same call; results
  * are the same either way up to fp32 rounding.  max_workgroups = 0 switches the pipeline off; a negative argument leaves
  * that setting unchanged.  Process-wide, takes effect with the next call.
