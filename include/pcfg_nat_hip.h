@@ -155,6 +155,13 @@ int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *ma
 void pcfgnat_pipeline_config(int max_workgroups, int spin_limit);
 
 /*
+ * No counterpart in the reference: a wait limit of its own for the outside pipeline where the two pipelines of a sentence
+ * run side by side (pcfgnat_pcfg_loss_forward_backward); negative (the default) = the common limit of
+ * pcfgnat_pipeline_config.  It lets a test make one of the two sweeps give up and be redone while the other completes.
+ */
+void pcfgnat_pipeline_outside_spin_limit(int spin_limit);
+
+/*
  * The float64 instantiation the reference also dispatches (AT_DISPATCH_FLOATING_TYPES in pcfg_loss.cu:395,
  * pcfg_loss_backward.cu:693, pcfg_best_tree.cu:349, pcfg_viterbi.cu:291; no shipped script uses it).  Same arguments,
  * layouts and results as the float32 entry points above and below with double tables; every max_left, 1 included,

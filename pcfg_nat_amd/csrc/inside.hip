@@ -2318,11 +2318,12 @@ __global__ __launch_bounds__(NTP) void inside_both_ml1_pipe_kernel(const float *
                                                                   const int64_t *__restrict__ out_len,
                                                                   const int64_t *__restrict__ tgt_len, float *__restrict__ S,
                                                                   float *__restrict__ aux, int L, int T, int Mc, int spin_limit,
-                                                                  int fwd_blocks) {
+                                                                  int spin_limit_outside, int fwd_blocks) {
     if ((int)blockIdx.x < fwd_blocks)  // workgroup-uniform
         inside_fwd_ml1_pipe_body<NQ, MATCH_LDS>((int)blockIdx.x, match_all, out_len, tgt_len, S, aux, L, T, Mc, spin_limit);
     else
-        outside_free_ml1_pipe_body<NQ, MATCH_LDS>((int)blockIdx.x - fwd_blocks, match_all, out_len, tgt_len, aux, L, T, Mc, spin_limit);
+        outside_free_ml1_pipe_body<NQ, MATCH_LDS>((int)blockIdx.x - fwd_blocks, match_all, out_len, tgt_len, aux, L, T, Mc,
+                                                  spin_limit_outside);
 }
 
 // After the sweeps side by side (and the forward's redo, if any): grid (CL, B), 256 threads.  Block k < K (K = the last
@@ -2805,6 +2806,7 @@ __global__ __launch_bounds__(256) void criterion_loss_kernel(const float *__rest
 // block first, so a block never waits for one that has not been started).  Both numbers can be changed through
 // pcfgnat_pipeline_config.
 std::atomic<int> g_pipeline_max_wg{1 << 20}, g_pipeline_spin_limit{1 << 20};
+std::atomic<int> g_pipeline_spin_limit_outside{-1};  // side-by-side launch only; negative: the common limit
 int pipeline_chunks(int B, int T, int Mc) {  // NQ, or 0 where the pipelined sweeps do not apply
     const int NQ = stream_mp(Mc) / 64, CL = 64 * NQ / NLP;
     return (NQ >= 2 && NQ <= 8 && T + 2 < 4096 && (int64_t)B * CL <= g_pipeline_max_wg.load()) ? NQ : 0;
@@ -2816,6 +2818,7 @@ int launch_fwd_pipe(const float *match_all, const int64_t *ol, const int64_t *tl
     constexpr int CL = 64 * NQ / NLP;
     const size_t match_bytes = (size_t)2 * NLP * T * sizeof(float);
     if (both) {  // the outside pipeline in the same launch, behind the forward one in dispatch order
+        const int spin_out = g_pipeline_spin_limit_outside.load() >= 0 ? g_pipeline_spin_limit_outside.load() : g_pipeline_spin_limit.load();
         if (match_bytes <= LDS_BUDGET - 8192) {
             auto k = inside_both_ml1_pipe_kernel<NQ, true>;
             // while every block of both pipelines can have a compute unit of its own, claim more than half of a unit's LDS
@@ -2823,10 +2826,10 @@ int launch_fwd_pipe(const float *match_all, const int64_t *ol, const int64_t *tl
             const size_t lds = (2 * B * CL <= 256 && match_bytes < PAD_EXCLUSIVE_LDS) ? PAD_EXCLUSIVE_LDS : match_bytes;
             PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             hipLaunchKernelGGL(k, dim3(2 * B * CL), dim3(NTP), lds, stream, match_all, ol, tl, S, aux, L, T, Mc,
-                               g_pipeline_spin_limit.load(), B * CL);
+                               g_pipeline_spin_limit.load(), spin_out, B * CL);
         } else {
             hipLaunchKernelGGL((inside_both_ml1_pipe_kernel<NQ, false>), dim3(2 * B * CL), dim3(NTP), 0, stream, match_all, ol, tl, S, aux,
-                               L, T, Mc, g_pipeline_spin_limit.load(), B * CL);
+                               L, T, Mc, g_pipeline_spin_limit.load(), spin_out, B * CL);
         }
     } else if (match_bytes <= LDS_BUDGET - 8192) {
         auto k = inside_fwd_ml1_pipe_kernel<NQ, true>;
@@ -3060,6 +3063,8 @@ extern "C" void pcfgnat_pipeline_config(int max_workgroups, int spin_limit) {
     if (max_workgroups >= 0) g_pipeline_max_wg.store(max_workgroups);
     if (spin_limit >= 0) g_pipeline_spin_limit.store(spin_limit);
 }
+
+extern "C" void pcfgnat_pipeline_outside_spin_limit(int spin_limit) { g_pipeline_spin_limit_outside.store(spin_limit); }
 
 extern "C" size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml) {
     if (B <= 0 || L < 2 || T < 0 || ml < 0) return 0;

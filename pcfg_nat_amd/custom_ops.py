@@ -23,14 +23,17 @@ def get_pcfg_kernel():
     return _lib.load()
 
 
-def pipeline_config(max_workgroups=None, spin_limit=None):
+def pipeline_config(max_workgroups=None, spin_limit=None, outside_spin_limit=None):
     """Tuning of the long-graph inside sweeps (no counterpart in the reference): graphs of 130..1026 nodes are swept by
     one workgroup per block of 16 main-chain nodes, pipelined, while the batch needs no more than ``max_workgroups`` of
     them (default 2**20; 0 = always one workgroup per sentence).  ``spin_limit`` bounds the wait of a block for the one
     ahead of it (default 2**20 rounds of polling); a sentence whose blocks give up is redone by the one-workgroup sweep
-    in the same call.  ``None`` leaves a setting as it is."""
-    _lib.load().pcfgnat_pipeline_config(-1 if max_workgroups is None else int(max_workgroups),
-                                       -1 if spin_limit is None else int(spin_limit))
+    in the same call.  ``outside_spin_limit``: a limit of its own for the outside pipeline where the two run side by
+    side (negative = the common one).  ``None`` leaves a setting as it is."""
+    lib = _lib.load()
+    lib.pcfgnat_pipeline_config(-1 if max_workgroups is None else int(max_workgroups), -1 if spin_limit is None else int(spin_limit))
+    if outside_spin_limit is not None:
+        lib.pcfgnat_pipeline_outside_spin_limit(int(outside_spin_limit))
 
 
 def _stream(t):

@@ -256,25 +256,32 @@ def _inside_all(batch, match):
     return ll.detach().cpu(), md.grad.cpu(), ld.grad.cpu()
 
 
-@pytest.mark.parametrize("mode", ["one_workgroup", "blocks_give_up"])
+@pytest.mark.parametrize("mode", ["one_workgroup", "blocks_give_up", "pipelines_in_turn", "forward_gives_up", "outside_gives_up"])
 @pytest.mark.parametrize("L,T,ms,ns", [(200, 50, [200, 132, 164], [50, 30, 44]), (320, 40, [320, 262, 4], [40, 31, 2]),
                                        (512, 140, [512, 444], [140, 120]),
                                        (600, 24, [600, 520], [24, 24]), (1024, 30, [1024, 770, 900], [30, 22, 30])])
 def test_long_graph_sweeps_agree(mode, L, T, ms, ns):
-    """Graphs of 130..1026 nodes: the pipelined sweeps (default), the one-workgroup streaming sweeps
-    (pipeline switched off) and the redo path (blocks that give up at once: spin limit 0) compute the same tables; the
-    default path is compared with the oracle in test_inside_forward_backward_vs_oracle."""
+    """Graphs of 130..1026 nodes: the two pipelined sweeps side by side (default), one after the other (a workgroup budget
+    that holds one pipeline but not two), the one-workgroup streaming sweeps (pipeline switched off) and the redo path
+    (blocks that give up at once: spin limit 0; both sweeps, or only one of the two that run side by side) compute the
+    same tables; the default path is compared with the oracle in test_inside_forward_backward_vs_oracle."""
     batch = synth.training_batch(len(ms), L, T, 60, ms, ns, seed=L + T)
     match = _match_for(batch)
     ll0, mg0, lg0 = _inside_all(batch, match)
     try:
         if mode == "one_workgroup":
             ops.pipeline_config(max_workgroups=0)
+        elif mode == "pipelines_in_turn":
+            ops.pipeline_config(max_workgroups=len(ms) * 4 * ((L // 2 + 63) // 64))
+        elif mode == "forward_gives_up":  # ... and is redone, while the outside pipeline beside it completes
+            ops.pipeline_config(spin_limit=0, outside_spin_limit=1 << 20)
+        elif mode == "outside_gives_up":
+            ops.pipeline_config(outside_spin_limit=0)
         else:
             ops.pipeline_config(spin_limit=0)
         ll1, mg1, lg1 = _inside_all(batch, match)
     finally:
-        ops.pipeline_config(max_workgroups=1 << 20, spin_limit=1 << 20)
+        ops.pipeline_config(max_workgroups=1 << 20, spin_limit=1 << 20, outside_spin_limit=-1)
     fin = torch.isfinite(ll0)
     assert fin.any() and torch.equal(fin, torch.isfinite(ll1))
     assert torch.allclose(ll0[fin], ll1[fin], rtol=1e-5)
