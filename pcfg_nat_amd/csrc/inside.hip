@@ -2717,15 +2717,24 @@ __global__ __launch_bounds__(1024) void links_grad_ml1_stream_kernel(const float
     const float A0 = ok ? to_b2(lk[((size_t)a * 2 + 0) * L + c]) : NEG_INF_F;
     const float A1 = (ok && a_id >= 1) ? to_b2(lk[((size_t)a * 2 + 1) * L + c]) : NEG_INF_F;
     float acc0 = 0.f, acc1 = 0.f;
-    for (int t0 = 1; t0 <= n - 1; t0 += 32) {
-        // rows = nodes of the tile, columns = 32 consecutive target positions
+    // rows = nodes of the tile, columns = 32 consecutive target positions; the next chunk of the tables is requested before
+    // the current one is worked on (the tables come from other compute units' stores: microseconds away)
+    const int ra = at * 32 + ty, rc = ct * 32 + ty;
+    auto fetch = [&](int t0, float &f0, float &f1, float &fs) {
         const int tt = t0 + tx;
-        const int ra = at * 32 + ty, rc = ct * 32 + ty;
         const bool tin = tt <= n - 1;
-        sw0[ty][tx] = (tin && ra < mc) ? av.W0[(size_t)ra * (T + 2) + tt] : NEG_INF_F;
-        sw1[ty][tx] = (tin && ra < mc) ? av.W1[(size_t)ra * (T + 2) + tt] : NEG_INF_F;
-        ss[ty][tx] = (tin && rc < mc) ? av.SR[(size_t)rc * (T + 2) + tt] + (use_corr ? corr[tt] : 0.f) : NEG_INF_F;
+        f0 = (tin && ra < mc) ? av.W0[(size_t)ra * (T + 2) + tt] : NEG_INF_F;
+        f1 = (tin && ra < mc) ? av.W1[(size_t)ra * (T + 2) + tt] : NEG_INF_F;
+        fs = (tin && rc < mc) ? av.SR[(size_t)rc * (T + 2) + tt] + (use_corr ? corr[tt] : 0.f) : NEG_INF_F;
+    };
+    float f0, f1, fs;
+    fetch(1, f0, f1, fs);
+    for (int t0 = 1; t0 <= n - 1; t0 += 32) {
+        sw0[ty][tx] = f0;
+        sw1[ty][tx] = f1;
+        ss[ty][tx] = fs;
         __syncthreads();
+        if (t0 + 32 <= n - 1) fetch(t0 + 32, f0, f1, fs);  // uniform
 #pragma unroll 8
         for (int u = 0; u < 32; u++) {
             const float sc = ss[tx][u];
