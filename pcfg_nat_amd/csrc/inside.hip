@@ -1664,11 +1664,18 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
 // Compact copies of the main-chain links for the streaming sweeps: Ac[k][a_id][c_id] = At[k][c_id][a_id] =
 // log2(e) * links[2*a_id+1][k][2*c_id+1] where a_id <= c_id < mc (k = 1 needs a_id >= 1), -inf everywhere else including the
 // padding columns up to MP.  One block per 32 x 32 tile of (parent, child) pairs, grid (MP/32, MP/32, B).  The blocks of a
-// sentence also share the filling of its exchange tables.
+// sentence also share the filling of its exchange tables and, when the caller hands one over (single call), the zero fill of
+// the sentence's slab of links_grad (2 L^2 floats), which the posterior kernel only writes at its posterior cells.
 __global__ __launch_bounds__(256) void compact_links_ml1_kernel(const float *__restrict__ links, const int64_t *__restrict__ out_len,
-                                                               float *__restrict__ aux, int L, int T, int Mc, int MP) {
+                                                               float *__restrict__ aux, int L, int T, int Mc, int MP,
+                                                               float *__restrict__ zero_slabs) {
     __shared__ float tile[2][32][33];
     const int b = blockIdx.z;
+    if (zero_slabs != nullptr) {
+        float *z = zero_slabs + (size_t)b * L * 2 * L;
+        const size_t nthreads = (size_t)gridDim.x * gridDim.y * 256, me = ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
+        for (size_t i = me; i < (size_t)L * 2 * L; i += nthreads) z[i] = 0.f;
+    }
     const int m = (int)out_len[b];
     const int mc = (m >= 2 && m <= L) ? m / 2 : 0;
     AuxViewStream av(aux, b, Mc, T);
@@ -2880,11 +2887,12 @@ bool side_by_side_applies(int B, int T, int Mc) {
     return NQ != 0 && (int64_t)2 * B * (64 * NQ / NLP) <= g_pipeline_max_wg.load();
 }
 
+// zero_slabs: links_grad, where the call also has the backward to do (its slab is then zeroed here, beside the compact copies)
 int launch_fwd_stream(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B,
-                      int L, int T, int Mc, hipStream_t stream, bool side_by_side = false) {
+                      int L, int T, int Mc, hipStream_t stream, bool side_by_side = false, float *zero_slabs = nullptr) {
     const int MP = stream_mp(Mc);
     PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss: aux must be 16-byte aligned");
-    hipLaunchKernelGGL(compact_links_ml1_kernel, dim3(MP / 32, MP / 32, B), dim3(256), 0, stream, links, ol, aux, L, T, Mc, MP);
+    hipLaunchKernelGGL(compact_links_ml1_kernel, dim3(MP / 32, MP / 32, B), dim3(256), 0, stream, links, ol, aux, L, T, Mc, MP, zero_slabs);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     // pipelined sweep first where it applies; the one-workgroup sweep then only redoes sentences whose blocks gave up
     const int NQ = pipeline_chunks(B, T, Mc);
@@ -2925,7 +2933,7 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
 // sentences it gave up and the posteriors (with their per-column corrections) are left to do.
 int launch_bwd_stream(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
                       const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream,
-                      bool side_by_side = false) {
+                      bool side_by_side = false, bool slabs_zeroed = false) {
     const int MP = stream_mp(Mc);
     const int tiles = (Mc + 31) / 32;
     PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss_backward: aux must be 16-byte aligned");
@@ -2955,9 +2963,11 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
         hipLaunchKernelGGL(k, dim3(B), dim3(NT), base, stream, S, aux, match_all, ol, tl, L, T, Mc, MP, only_flagged);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
-    const size_t nlg = (size_t)B * L * 2 * L;
-    hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, stream, lg, nlg);
-    PCFGNAT_HIP_CHECK(hipGetLastError());
+    if (!slabs_zeroed) {
+        const size_t nlg = (size_t)B * L * 2 * L;
+        hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, stream, lg, nlg);
+        PCFGNAT_HIP_CHECK(hipGetLastError());
+    }
     const int use_corr = side_by_side ? 1 : 0;
     hipLaunchKernelGGL(links_grad_ml1_stream_kernel, dim3(tiles, tiles, B), dim3(1024), 0, stream, go, S, aux, links, ol, tl, lg, L, T, Mc,
                        norm_B, use_corr);
@@ -3145,10 +3155,10 @@ int pcfgnat::inside_forward_backward_impl(const float *grad_output, const float 
                              (int)T, Mc, (int)norm_B, s, &done, pad, pad_done);
     if (rc != PCFGNAT_OK || done) return rc;
     if (ml == 1 && Mc > 64 && side_by_side_applies((int)B, (int)T, Mc)) {  // the two pipelined sweeps in one launch
-        rc = launch_fwd_stream(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s, true);
+        rc = launch_fwd_stream(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s, true, links_grad);
         if (rc != PCFGNAT_OK) return rc;
         return launch_bwd_stream(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
-                                 (int)L, (int)T, Mc, (int)norm_B, s, true);
+                                 (int)L, (int)T, Mc, (int)norm_B, s, true, true);
     }
     rc = pcfgnat_pcfg_loss(match_all, links, output_length, target_length, S, aux, B, L, T, ml, stream);
     if (rc != PCFGNAT_OK) return rc;
