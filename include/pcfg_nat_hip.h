@@ -147,7 +147,8 @@ int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *ma
  * swept by one workgroup per block of 16 main-chain nodes, the blocks following each other as a pipeline, as long as the
  * batch needs no more than max_workgroups of them (B * 4 * ceil((L/2)/64) <= max_workgroups, default 2^20), and by one
  * workgroup per sentence otherwise.  pcfgnat_pcfg_loss_forward_backward runs the forward and the outside pipeline of a
- * sentence side by side in one launch while twice that number fits, one after the other otherwise.  A block that waits for the one ahead of it for more than spin_limit rounds of polling
+ * sentence side by side in one launch while twice that number fits, one after the other otherwise.  A block that waits
+ * for the one ahead of it for more than spin_limit rounds of polling
  * (default 2^20, about a second) gives the sentence up, and the one-workgroup sweep redoes it in the same call; results
  * are the same either way up to fp32 rounding.  max_workgroups = 0 switches the pipeline off; a negative argument leaves
  * that setting unchanged.  Process-wide, takes effect with the next call.
