@@ -1930,7 +1930,8 @@ __device__ __forceinline__ void inside_fwd_ml1_pipe_body(const int bid, const fl
     float *sm_main = sm_match, *sm_leaf = sm_match + NLP * T;
     const int b = bid / CL, k = CL - 1 - bid % CL;  // the leading (highest) block first
     const int tid = threadIdx.x, gidx = (tid >> 4) & (NLP - 1), j = tid & 15, lane = tid & 63;
-    const bool collector = tid >= 16 * NLP;
+    const bool collector = tid >= 16 * NLP && tid < NTP;  // (waves beyond NTP, in the side-by-side launch, only share the barriers)
+    const bool compute = tid < 16 * NLP;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const float *mt = match_all + (size_t)b * L * T;
     float *Sb = S + (size_t)b * Mc * (T + 2);
@@ -1971,7 +1972,7 @@ __device__ __forceinline__ void inside_fwd_ml1_pipe_body(const int bid, const fl
     const int ar = row_ok ? a_id : NLP * k;
     const int q0 = (NLP * k) / 64;  // the chunk that holds the block's diagonal
     float4 A0[NQ], A1[NQ];
-    if (!collector) {
+    if (compute) {
         const float4 *r0 = reinterpret_cast<const float4 *>(av.Ac + ((size_t)0 * Mc + ar) * MP) + j;
         const float4 *r1 = reinterpret_cast<const float4 *>(av.Ac + ((size_t)1 * Mc + ar) * MP) + j;
 #pragma unroll
@@ -2056,7 +2057,7 @@ __device__ __forceinline__ void inside_fwd_ml1_pipe_body(const int bid, const fl
             }
             vm = wave_max(vm);
             if (lane == 0) sm_Dv[(t - 1) & 1] = vm;
-        } else {
+        } else if (compute) {
             // the next column's emissions: from LDS, or requested now so that they travel during the column's work
             float ma_raw = 0.f, ml_raw = 0.f;
             if (t > 1) {
@@ -2123,20 +2124,25 @@ __global__ __launch_bounds__(NTP) void inside_fwd_ml1_pipe_kernel(const float *_
 // with O_t the forward's offsets; for a sentence whose outside sweep was redone on the forward's offsets by the
 // one-workgroup kernel they are 0 and -D_t.
 // ------------------------------------------------------------------------------------------------------------
-template <int NQ, bool MATCH_LDS>
+template <int NQ, bool MATCH_LDS, int CW>
 __device__ __forceinline__ void outside_free_ml1_pipe_body(const int bid, const float *__restrict__ match_all,
                                                           const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
                                                           float *__restrict__ aux, int L, int T, int Mc, int spin_limit) {
     constexpr int MP = 64 * NQ, CL = MP / NLP;
     __shared__ __attribute__((aligned(16))) float w0[2][MP];
     __shared__ __attribute__((aligned(16))) float w1[2][MP];
-    __shared__ float sm_Ev[2];  // shift chosen at the step that reads the columns t: maximum of the visible part of the columns t-1
+    __shared__ float sm_Ev[2][4];  // shift chosen at the step that reads the columns t: maximum of the visible part of the
+                                   // columns t-1, one partial maximum per collector wave
     __shared__ int sm_dead;
     extern __shared__ float sm_em[];
     float *sm_main = sm_em, *sm_leaf = sm_em + NLP * T;
     const int b = bid / CL, k = bid % CL;  // the leading (lowest) block first
     const int tid = threadIdx.x, gidx = (tid >> 4) & (NLP - 1), j = tid & 15, lane = tid & 63;
+    // CW collector waves behind the compute waves (four: one per SIMD, for launches in which a block has a compute unit to
+    // itself; one otherwise): wave cw takes the chunks cw, cw+CW, .. of both planes
     const bool collector = tid >= 16 * NLP;
+    const int cw = (CW == 1) ? 0 : ((tid >> 6) & 3);
+    constexpr int NR = (NQ + CW - 1) / CW;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const float *mt = match_all + (size_t)b * L * T;
     AuxViewStream av(aux, b, Mc, T);
@@ -2148,11 +2154,8 @@ __device__ __forceinline__ void outside_free_ml1_pipe_body(const int bid, const 
         (&w0[0][0])[i] = NEG_INF_F;
         (&w1[0][0])[i] = NEG_INF_F;
     }
-    if (tid == 0) {
-        sm_dead = 0;
-        sm_Ev[0] = 0.f;
-        sm_Ev[1] = 0.f;
-    }
+    if (tid == 0) sm_dead = 0;
+    if (tid < 8) (&sm_Ev[0][0])[tid] = (tid & 3) ? NEG_INF_F : 0.f;  // slots of absent collector waves stay at -inf
     if (MATCH_LDS) {
         for (int i = tid; i < NLP * T; i += NTP) {
             const int g = i / T, s = i - g * T, node = NLP * k + g;
@@ -2208,12 +2211,13 @@ __device__ __forceinline__ void outside_free_ml1_pipe_body(const int bid, const 
         Ek[1] = 0.f;
     }
     const unsigned long long MINUS_INF64 = (unsigned long long)__double_as_longlong(-__builtin_huge_val());
-    unsigned long long x0[NQ], x1[NQ];  // collector: the entries of the blocks below, requested one step before they are handed on
+    unsigned long long x0[NR], x1[NR];  // collectors: the entries of the blocks below, requested one step before they are handed on
 #pragma unroll
-    for (int r = 0; r < NQ; r++) {
-        const bool need = collector && k > 0 && n >= 3;
-        x0[r] = need ? entry_load(Xo + (size_t)2 * 2 * MP + 64 * r + lane) : MINUS_INF64;
-        x1[r] = need ? entry_load(Xo + (size_t)2 * 2 * MP + MP + 64 * r + lane) : MINUS_INF64;
+    for (int ri = 0; ri < NR; ri++) {
+        const int r = cw + CW * ri;
+        const bool need = collector && k > 0 && n >= 3 && r < NQ;
+        x0[ri] = need ? entry_load(Xo + (size_t)2 * 2 * MP + 64 * r + lane) : MINUS_INF64;
+        x1[ri] = need ? entry_load(Xo + (size_t)2 * 2 * MP + MP + 64 * r + lane) : MINUS_INF64;
     }
     double P = 0.0;      // P_t, the offset of the columns being read
     float e_cur = 0.f;   // e_t
@@ -2221,7 +2225,7 @@ __device__ __forceinline__ void outside_free_ml1_pipe_body(const int bid, const 
         const float *c0 = w0[t & 1], *c1 = w1[t & 1];
         float *n0 = w0[(t + 1) & 1], *n1 = w1[(t + 1) & 1];
         const bool more = t < n - 1;
-        const float E = sm_Ev[t & 1];
+        const float E = fmaxf(fmaxf(sm_Ev[t & 1][0], sm_Ev[t & 1][1]), fmaxf(sm_Ev[t & 1][2], sm_Ev[t & 1][3]));
         const float e_next = is_finite(E) ? E : 0.f;  // e_{t+1}
         const double P_next = P + (double)e_next;     // P_{t+1}
         if (collector) {
@@ -2230,16 +2234,16 @@ __device__ __forceinline__ void outside_free_ml1_pipe_body(const int bid, const 
                 // the requests went out for every lane (a branch around a load ends in a wait for it); entries of other
                 // blocks' nodes beyond the sentence are never written and read as -inf
 #pragma unroll
-                for (int r = 0; r < NQ; r++) {
-                    if (64 * r + lane >= min(NLP * k, mc)) {
-                        x0[r] = MINUS_INF64;
-                        x1[r] = MINUS_INF64;
+                for (int ri = 0; ri < NR; ri++) {
+                    if (64 * (cw + CW * ri) + lane >= min(NLP * k, mc)) {
+                        x0[ri] = MINUS_INF64;
+                        x1[ri] = MINUS_INF64;
                     }
                 }
                 for (int spins = 0;; spins++) {
                     bool pending = false;
 #pragma unroll
-                    for (int r = 0; r < NQ; r++) pending |= (x0[r] == EMPTY64) | (x1[r] == EMPTY64);
+                    for (int ri = 0; ri < NR; ri++) pending |= (x0[ri] == EMPTY64) | (x1[ri] == EMPTY64);
                     if (!__any(pending)) break;
                     if (spins >= spin_limit || ((spins & 63) == 63 && gave_up(xv.flags + FLAG_BWD))) {
                         sm_dead = 1;
@@ -2247,37 +2251,39 @@ __device__ __forceinline__ void outside_free_ml1_pipe_body(const int bid, const 
                     }
                     __builtin_amdgcn_s_sleep(2);  // leave the issue slots of this SIMD to its compute wave
 #pragma unroll
-                    for (int r = 0; r < NQ; r++) {
-                        if (x0[r] == EMPTY64) x0[r] = entry_load(src + 64 * r);
-                        if (x1[r] == EMPTY64) x1[r] = entry_load(src + MP + 64 * r);
+                    for (int ri = 0; ri < NR; ri++) {
+                        const int r = min(cw + CW * ri, NQ - 1);
+                        if (x0[ri] == EMPTY64) x0[ri] = entry_load(src + 64 * r);
+                        if (x1[ri] == EMPTY64) x1[ri] = entry_load(src + MP + 64 * r);
                     }
                 }
 #pragma unroll
-                for (int r = 0; r < NQ; r++) {
-                    const int i = 64 * r + lane;
-                    if (i < NLP * k) {
-                        n0[i] = (x0[r] == EMPTY64) ? NEG_INF_F : (float)(__longlong_as_double((long long)x0[r]) - P_next);
-                        n1[i] = (x1[r] == EMPTY64) ? NEG_INF_F : (float)(__longlong_as_double((long long)x1[r]) - P_next);
+                for (int ri = 0; ri < NR; ri++) {
+                    const int r = cw + CW * ri, i = 64 * r + lane;
+                    if (r < NQ && i < NLP * k) {
+                        n0[i] = (x0[ri] == EMPTY64) ? NEG_INF_F : (float)(__longlong_as_double((long long)x0[ri]) - P_next);
+                        n1[i] = (x1[ri] == EMPTY64) ? NEG_INF_F : (float)(__longlong_as_double((long long)x1[ri]) - P_next);
                     }
                 }
             }
             if (t + 2 <= n - 1 && k > 0) {  // request column t+2 now: it has the whole next step to arrive
                 const unsigned long long *src = Xo + (size_t)(t + 2) * 2 * MP + lane;
 #pragma unroll
-                for (int r = 0; r < NQ; r++) {
-                    x0[r] = entry_load(src + 64 * r);
-                    x1[r] = entry_load(src + MP + 64 * r);
+                for (int ri = 0; ri < NR; ri++) {
+                    const int r = min(cw + CW * ri, NQ - 1);  // (a wave without a chunk of its own re-reads the last one and drops it)
+                    x0[ri] = entry_load(src + 64 * r);
+                    x1[ri] = entry_load(src + MP + 64 * r);
                 }
             }
             // the shift of the next step from the visible part of the columns t, which is complete
             float vm = NEG_INF_F;
 #pragma unroll
-            for (int r = 0; r < NQ; r++) {
-                const int i = 64 * r + lane;
-                if (i < NLP * (k + 1)) vm = fmaxf(vm, fmaxf(c0[i], c1[i]));
+            for (int ri = 0; ri < NR; ri++) {
+                const int r = cw + CW * ri, i = 64 * r + lane;
+                if (r < NQ && i < NLP * (k + 1)) vm = fmaxf(vm, fmaxf(c0[i], c1[i]));
             }
             vm = wave_max(vm);
-            if (lane == 0) sm_Ev[(t + 1) & 1] = vm;
+            if (lane == 0) sm_Ev[(t + 1) & 1][cw] = vm;
         } else {
             float mc_raw = 0.f, ml_raw = 0.f;
             if (more) {
@@ -2320,8 +2326,8 @@ __device__ __forceinline__ void outside_free_ml1_pipe_body(const int bid, const 
 
 // Both sweeps in one launch: the first `fwd_blocks` workgroups are the forward pipeline's, the others the outside one's
 // (leading blocks first within either).
-template <int NQ, bool MATCH_LDS>
-__global__ __launch_bounds__(NTP) void inside_both_ml1_pipe_kernel(const float *__restrict__ match_all,
+template <int NQ, bool MATCH_LDS, int CW>
+__global__ __launch_bounds__(16 * NLP + 64 * CW) void inside_both_ml1_pipe_kernel(const float *__restrict__ match_all,
                                                                   const int64_t *__restrict__ out_len,
                                                                   const int64_t *__restrict__ tgt_len, float *__restrict__ S,
                                                                   float *__restrict__ aux, int L, int T, int Mc, int spin_limit,
@@ -2329,7 +2335,7 @@ __global__ __launch_bounds__(NTP) void inside_both_ml1_pipe_kernel(const float *
     if ((int)blockIdx.x < fwd_blocks)  // workgroup-uniform
         inside_fwd_ml1_pipe_body<NQ, MATCH_LDS>((int)blockIdx.x, match_all, out_len, tgt_len, S, aux, L, T, Mc, spin_limit);
     else
-        outside_free_ml1_pipe_body<NQ, MATCH_LDS>((int)blockIdx.x - fwd_blocks, match_all, out_len, tgt_len, aux, L, T, Mc,
+        outside_free_ml1_pipe_body<NQ, MATCH_LDS, CW>((int)blockIdx.x - fwd_blocks, match_all, out_len, tgt_len, aux, L, T, Mc,
                                                   spin_limit_outside);
 }
 
@@ -2835,16 +2841,24 @@ int launch_fwd_pipe(const float *match_all, const int64_t *ol, const int64_t *tl
     const size_t match_bytes = (size_t)2 * NLP * T * sizeof(float);
     if (both) {  // the outside pipeline in the same launch, behind the forward one in dispatch order
         const int spin_out = g_pipeline_spin_limit_outside.load() >= 0 ? g_pipeline_spin_limit_outside.load() : g_pipeline_spin_limit.load();
+        // while every block of both pipelines can have a compute unit of its own: claim more than half of a unit's LDS so
+        // that no two blocks share one (and its instruction issue), and spread the outside sweep's collecting over four waves
+        const bool roomy = 2 * B * CL <= 256;
         if (match_bytes <= LDS_BUDGET - 8192) {
-            auto k = inside_both_ml1_pipe_kernel<NQ, true>;
-            // while every block of both pipelines can have a compute unit of its own, claim more than half of a unit's LDS
-            // so that no two blocks share one (and its instruction issue)
-            const size_t lds = (2 * B * CL <= 256 && match_bytes < PAD_EXCLUSIVE_LDS) ? PAD_EXCLUSIVE_LDS : match_bytes;
-            PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            hipLaunchKernelGGL(k, dim3(2 * B * CL), dim3(NTP), lds, stream, match_all, ol, tl, S, aux, L, T, Mc,
-                               g_pipeline_spin_limit.load(), spin_out, B * CL);
+            const size_t lds = (roomy && match_bytes < PAD_EXCLUSIVE_LDS) ? PAD_EXCLUSIVE_LDS : match_bytes;
+            if (roomy) {
+                auto k = inside_both_ml1_pipe_kernel<NQ, true, 4>;
+                PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                hipLaunchKernelGGL(k, dim3(2 * B * CL), dim3(16 * NLP + 256), lds, stream, match_all, ol, tl, S, aux, L, T, Mc,
+                                   g_pipeline_spin_limit.load(), spin_out, B * CL);
+            } else {
+                auto k = inside_both_ml1_pipe_kernel<NQ, true, 1>;
+                PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                hipLaunchKernelGGL(k, dim3(2 * B * CL), dim3(NTP), lds, stream, match_all, ol, tl, S, aux, L, T, Mc,
+                                   g_pipeline_spin_limit.load(), spin_out, B * CL);
+            }
         } else {
-            hipLaunchKernelGGL((inside_both_ml1_pipe_kernel<NQ, false>), dim3(2 * B * CL), dim3(NTP), 0, stream, match_all, ol, tl, S, aux,
+            hipLaunchKernelGGL((inside_both_ml1_pipe_kernel<NQ, false, 1>), dim3(2 * B * CL), dim3(NTP), 0, stream, match_all, ol, tl, S, aux,
                                L, T, Mc, g_pipeline_spin_limit.load(), spin_out, B * CL);
         }
     } else if (match_bytes <= LDS_BUDGET - 8192) {
