@@ -1917,21 +1917,24 @@ __device__ __forceinline__ void slab_row_lse(const float4 (&A0)[NQ], const float
 // Forward sweep of one block.  Same tables as inside_fwd_ml1_stream_kernel, relative to the block's own offsets (see
 // above).  Dynamic LDS (MATCH_LDS): the emissions of the block's nodes, main [NLP][T] and leaf [NLP][T]; without it they
 // are requested one column ahead.
-template <int NQ, bool MATCH_LDS>
+template <int NQ, bool MATCH_LDS, int CW>
 __device__ __forceinline__ void inside_fwd_ml1_pipe_body(const int bid, const float *__restrict__ match_all,
                                                         const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
                                                         float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc,
                                                         int spin_limit) {
     constexpr int MP = 64 * NQ, CL = MP / NLP;
     __shared__ __attribute__((aligned(16))) float col[2][MP];
-    __shared__ float sm_Dv[2];  // shift of the step that reads column t: maximum of the visible part of column t+1
+    __shared__ float sm_Dv[2][4];  // shift of the step that reads column t: maximum of the visible part of column t+1, one
+                                   // partial maximum per collector wave
     __shared__ int sm_dead;
     extern __shared__ float sm_match[];
     float *sm_main = sm_match, *sm_leaf = sm_match + NLP * T;
     const int b = bid / CL, k = CL - 1 - bid % CL;  // the leading (highest) block first
     const int tid = threadIdx.x, gidx = (tid >> 4) & (NLP - 1), j = tid & 15, lane = tid & 63;
-    const bool collector = tid >= 16 * NLP && tid < NTP;  // (waves beyond NTP, in the side-by-side launch, only share the barriers)
-    const bool compute = tid < 16 * NLP;
+    // CW collector waves behind the compute waves (see outside_free_ml1_pipe_body): wave cw takes the chunks cw, cw+CW, ..
+    const bool collector = tid >= 16 * NLP, compute = !collector;
+    const int cw = (CW == 1) ? 0 : ((tid >> 6) & 3);
+    constexpr int NR = (NQ + CW - 1) / CW;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const float *mt = match_all + (size_t)b * L * T;
     float *Sb = S + (size_t)b * Mc * (T + 2);
@@ -1961,10 +1964,9 @@ __device__ __forceinline__ void inside_fwd_ml1_pipe_body(const int bid, const fl
     __syncthreads();
     if (tid == 0) {
         col[(n - 1) & 1][mc - 1] = base_cell;
-        sm_Dv[0] = 0.f;
-        sm_Dv[1] = 0.f;
         sm_dead = 0;
     }
+    if (tid < 8) (&sm_Dv[0][0])[tid] = (tid & 3) ? NEG_INF_F : 0.f;  // slots of absent collector waves stay at -inf
 
     // this lane's node and its link rows (rows beyond the sentence: any valid row, the result is discarded)
     const int a_id = NLP * k + gidx;
@@ -2003,17 +2005,17 @@ __device__ __forceinline__ void inside_fwd_ml1_pipe_body(const int bid, const fl
     unsigned long long *Xf = xv.fcol;
     float *Dk = xv.shifts + (size_t)k * (T + 4);
     const unsigned long long MINUS_INF64 = (unsigned long long)__double_as_longlong(-__builtin_huge_val());
-    unsigned long long x[NQ];  // collector: the entries of the blocks above, requested one step before they are handed on
+    unsigned long long x[NR];  // collectors: the entries of the blocks above, requested one step before they are handed on
 #pragma unroll
-    for (int r = 0; r < NQ; r++) {
-        const int i = NLP * (k + 1) + 64 * r + lane;
-        x[r] = (collector && n >= 3) ? entry_load(Xf + (size_t)(n - 2) * MP + i) : MINUS_INF64;
+    for (int ri = 0; ri < NR; ri++) {
+        const int r = cw + CW * ri, i = NLP * (k + 1) + 64 * min(r, NQ - 1) + lane;
+        x[ri] = (collector && n >= 3 && r < NQ) ? entry_load(Xf + (size_t)(n - 2) * MP + i) : MINUS_INF64;
     }
     double O = 0.0;  // offset of the column being read
     for (int t = n - 1; t >= 1; t--) {
         const float *cur = col[t & 1];
         float *nxt = col[(t - 1) & 1];
-        const float D = sm_Dv[t & 1];
+        const float D = fmaxf(fmaxf(sm_Dv[t & 1][0], sm_Dv[t & 1][1]), fmaxf(sm_Dv[t & 1][2], sm_Dv[t & 1][3]));
         const float Ds = (D == NEG_INF_F) ? 0.f : D;
         const double O_new = O + (double)Ds;  // offset of column t-1
         if (collector) {
@@ -2022,12 +2024,12 @@ __device__ __forceinline__ void inside_fwd_ml1_pipe_body(const int bid, const fl
                 // the requests went out for every lane (a branch around a load ends in a wait for it); entries beyond the
                 // sentence are never written and read as -inf
 #pragma unroll
-                for (int r = 0; r < NQ; r++)
-                    if (NLP * (k + 1) + 64 * r + lane >= mc) x[r] = MINUS_INF64;
+                for (int ri = 0; ri < NR; ri++)
+                    if (cw + CW * ri >= NQ || NLP * (k + 1) + 64 * (cw + CW * ri) + lane >= mc) x[ri] = MINUS_INF64;
                 for (int spins = 0;; spins++) {
                     bool pending = false;
 #pragma unroll
-                    for (int r = 0; r < NQ; r++) pending |= (x[r] == EMPTY64);
+                    for (int ri = 0; ri < NR; ri++) pending |= (x[ri] == EMPTY64);
                     if (!__any(pending)) break;
                     if (spins >= spin_limit || ((spins & 63) == 63 && gave_up(xv.flags + FLAG_FWD))) {
                         sm_dead = 1;
@@ -2035,28 +2037,29 @@ __device__ __forceinline__ void inside_fwd_ml1_pipe_body(const int bid, const fl
                     }
                     __builtin_amdgcn_s_sleep(2);  // leave the issue slots of this SIMD to its compute wave
 #pragma unroll
-                    for (int r = 0; r < NQ; r++)
-                        if (x[r] == EMPTY64) x[r] = entry_load(src + 64 * r);
+                    for (int ri = 0; ri < NR; ri++)
+                        if (x[ri] == EMPTY64) x[ri] = entry_load(src + 64 * min(cw + CW * ri, NQ - 1));
                 }
 #pragma unroll
-                for (int r = 0; r < NQ; r++) {
-                    const int i = NLP * (k + 1) + 64 * r + lane;
-                    if (i < MP) nxt[i] = (x[r] == EMPTY64) ? NEG_INF_F : (float)(__longlong_as_double((long long)x[r]) - O_new);
+                for (int ri = 0; ri < NR; ri++) {
+                    const int r = cw + CW * ri, i = NLP * (k + 1) + 64 * r + lane;
+                    if (r < NQ && i < MP) nxt[i] = (x[ri] == EMPTY64) ? NEG_INF_F : (float)(__longlong_as_double((long long)x[ri]) - O_new);
                 }
             }
             if (t > 2) {  // request column t-2 now: it has the whole next step to arrive
 #pragma unroll
-                for (int r = 0; r < NQ; r++) x[r] = entry_load(Xf + (size_t)(t - 2) * MP + NLP * (k + 1) + 64 * r + lane);
+                for (int ri = 0; ri < NR; ri++)
+                    x[ri] = entry_load(Xf + (size_t)(t - 2) * MP + NLP * (k + 1) + 64 * min(cw + CW * ri, NQ - 1) + lane);
             }
             // the shift of the next step from the visible part of column t, which is complete
             float vm = NEG_INF_F;
 #pragma unroll
-            for (int r = 0; r < NQ; r++) {
-                const int i = NLP * k + 64 * r + lane;
-                if (i < MP) vm = fmaxf(vm, cur[i]);
+            for (int ri = 0; ri < NR; ri++) {
+                const int r = cw + CW * ri, i = NLP * k + 64 * r + lane;
+                if (r < NQ && i < MP) vm = fmaxf(vm, cur[i]);
             }
             vm = wave_max(vm);
-            if (lane == 0) sm_Dv[(t - 1) & 1] = vm;
+            if (lane == 0) sm_Dv[(t - 1) & 1][cw] = vm;
         } else if (compute) {
             // the next column's emissions: from LDS, or requested now so that they travel during the column's work
             float ma_raw = 0.f, ml_raw = 0.f;
@@ -2101,12 +2104,13 @@ __device__ __forceinline__ void inside_fwd_ml1_pipe_body(const int bid, const fl
     }
 }
 
-template <int NQ, bool MATCH_LDS>
-__global__ __launch_bounds__(NTP) void inside_fwd_ml1_pipe_kernel(const float *__restrict__ match_all,
-                                                                 const int64_t *__restrict__ out_len,
-                                                                 const int64_t *__restrict__ tgt_len, float *__restrict__ S,
-                                                                 float *__restrict__ aux, int L, int T, int Mc, int spin_limit) {
-    inside_fwd_ml1_pipe_body<NQ, MATCH_LDS>((int)blockIdx.x, match_all, out_len, tgt_len, S, aux, L, T, Mc, spin_limit);
+template <int NQ, bool MATCH_LDS, int CW = 1>
+__global__ __launch_bounds__(16 * NLP + 64 * CW) void inside_fwd_ml1_pipe_kernel(const float *__restrict__ match_all,
+                                                                                const int64_t *__restrict__ out_len,
+                                                                                const int64_t *__restrict__ tgt_len, float *__restrict__ S,
+                                                                                float *__restrict__ aux, int L, int T, int Mc,
+                                                                                int spin_limit) {
+    inside_fwd_ml1_pipe_body<NQ, MATCH_LDS, CW>((int)blockIdx.x, match_all, out_len, tgt_len, S, aux, L, T, Mc, spin_limit);
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -2333,7 +2337,7 @@ __global__ __launch_bounds__(16 * NLP + 64 * CW) void inside_both_ml1_pipe_kerne
                                                                   float *__restrict__ aux, int L, int T, int Mc, int spin_limit,
                                                                   int spin_limit_outside, int fwd_blocks) {
     if ((int)blockIdx.x < fwd_blocks)  // workgroup-uniform
-        inside_fwd_ml1_pipe_body<NQ, MATCH_LDS>((int)blockIdx.x, match_all, out_len, tgt_len, S, aux, L, T, Mc, spin_limit);
+        inside_fwd_ml1_pipe_body<NQ, MATCH_LDS, CW>((int)blockIdx.x, match_all, out_len, tgt_len, S, aux, L, T, Mc, spin_limit);
     else
         outside_free_ml1_pipe_body<NQ, MATCH_LDS, CW>((int)blockIdx.x - fwd_blocks, match_all, out_len, tgt_len, aux, L, T, Mc,
                                                   spin_limit_outside);
@@ -2861,6 +2865,12 @@ int launch_fwd_pipe(const float *match_all, const int64_t *ol, const int64_t *tl
             hipLaunchKernelGGL((inside_both_ml1_pipe_kernel<NQ, false, 1>), dim3(2 * B * CL), dim3(NTP), 0, stream, match_all, ol, tl, S, aux,
                                L, T, Mc, g_pipeline_spin_limit.load(), spin_out, B * CL);
         }
+    } else if (match_bytes <= LDS_BUDGET - 8192 && B * CL <= 256) {  // a compute unit per block: four collector waves
+        auto k = inside_fwd_ml1_pipe_kernel<NQ, true, 4>;
+        const size_t lds = match_bytes < PAD_EXCLUSIVE_LDS ? PAD_EXCLUSIVE_LDS : match_bytes;
+        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(k, dim3(B * CL), dim3(16 * NLP + 256), lds, stream, match_all, ol, tl, S, aux, L, T, Mc,
+                           g_pipeline_spin_limit.load());
     } else if (match_bytes <= LDS_BUDGET - 8192) {
         auto k = inside_fwd_ml1_pipe_kernel<NQ, true>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)match_bytes));
