@@ -259,7 +259,9 @@ def _inside_all(batch, match):
 @pytest.mark.parametrize("mode", ["one_workgroup", "blocks_give_up", "pipelines_in_turn", "forward_gives_up", "outside_gives_up"])
 @pytest.mark.parametrize("L,T,ms,ns", [(200, 50, [200, 132, 164], [50, 30, 44]), (320, 40, [320, 262, 4], [40, 31, 2]),
                                        (512, 140, [512, 444], [140, 120]),
-                                       (600, 24, [600, 520], [24, 24]), (1024, 30, [1024, 770, 900], [30, 22, 30])])
+                                       (600, 24, [600, 520], [24, 24]), (1024, 30, [1024, 770, 900], [30, 22, 30]),
+                                       # more blocks than compute units: the blocks share them (one collector wave each)
+                                       (200, 20, [200, 132, 164, 96] * 10, [20, 13, 17, 9] * 10)])
 def test_long_graph_sweeps_agree(mode, L, T, ms, ns):
     """Graphs of 130..1026 nodes: the two pipelined sweeps side by side (default), one after the other (a workgroup budget
     that holds one pipeline but not two), the one-workgroup streaming sweeps (pipeline switched off) and the redo path
