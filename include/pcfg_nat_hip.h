@@ -142,6 +142,23 @@ int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *ma
                                        void *stream);
 
 /*
+ * No counterpart in the reference: pcfgnat_pcfg_loss_forward_backward for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  Same arguments and results
+ * without `aux`: the auxiliary table lives in a device array of PCFGNAT_STATIC_AUX_FLOATS floats (32 MiB) that the library
+ * holds on every GPU it is loaded on until the process ends.  The call allocates nothing.  Shapes with
+ * pcfgnat_pcfg_aux_floats(B, L, T, ml) > PCFGNAT_STATIC_AUX_FLOATS are rejected with PCFGNAT_EINVAL before anything is
+ * enqueued (BASELINE-sized batches fit: 40 sentences of 128 nodes take 2 MiB, 8 of 512 nodes with 140 target tokens
+ * 24 MiB).  All calls on one GPU share that GPU's array: calls that overlap there (two streams, two threads) race, and
+ * the kernels of one call must have finished before the next call on another stream is enqueued.
+ */
+#define PCFGNAT_STATIC_AUX_FLOATS (8u * 1024u * 1024u)
+size_t pcfgnat_static_aux_floats(void);
+int pcfgnat_pcfg_loss_forward_backward_static(const float *grad_output, const float *match_all, const float *links,
+                                              const int64_t *output_length, const int64_t *target_length, float *S,
+                                              float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T,
+                                              int64_t ml, void *stream);
+
+/*
  * No counterpart in the reference: tuning of the long-graph paths (max_left = 1; inside sweeps for 130 <= L <= 1026, the
  * Viterbi sweep of pcfgnat_viterbi_decode for 194 <= L <= 514).  There a sentence is
  * swept by one workgroup per block of 16 main-chain nodes, the blocks following each other as a pipeline, as long as the

@@ -23,6 +23,7 @@
 #include "common.hip.h"
 
 #include <atomic>
+#include <mutex>
 
 namespace pcfgnat {
 namespace {
@@ -3194,6 +3195,57 @@ extern "C" int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, cons
                                                  const int64_t *output_length, const int64_t *target_length, float *S, float *aux,
                                                  float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T,
                                                  int64_t ml, void *stream) {
+    return inside_forward_backward_impl(grad_output, match_all, links, output_length, target_length, S, aux, match_all_grad, links_grad,
+                                        B, L, T, ml, B, stream);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// pcfgnat_pcfg_loss_forward_backward for callers that cannot allocate device memory (code under HIP graph capture,
+// serving loops, harnesses that forbid hipMalloc): the auxiliary table lives in a device array of fixed size that
+// belongs to the library.  Every device the code object is loaded on holds its own copy of the array at its own
+// address, looked up once per device; in host code the array's name is only a handle for that lookup, never an address.
+// ---------------------------------------------------------------------------------------------------------------
+namespace {
+static __device__ __align__(256) float static_aux[PCFGNAT_STATIC_AUX_FLOATS];
+constexpr int STATIC_AUX_MAX_DEVICES = 64;
+float *g_static_aux_ptr[STATIC_AUX_MAX_DEVICES];
+std::mutex g_static_aux_mutex;
+
+// The address of the current device's copy of static_aux (looked up with that device current, kept for later calls).
+int static_aux_address(float **out) {
+    int dev = -1;
+    PCFGNAT_HIP_CHECK(hipGetDevice(&dev));
+    PCFGNAT_REQUIRE(dev >= 0 && dev < STATIC_AUX_MAX_DEVICES, "pcfg_loss_forward_backward_static: device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_static_aux_mutex);
+    if (g_static_aux_ptr[dev] == nullptr) {
+        float *ptr = nullptr;
+        PCFGNAT_HIP_CHECK(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(static_aux)));
+        if (ptr == nullptr) return pcfgnat::fail(PCFGNAT_EHIP, "pcfg_loss_forward_backward_static: no device address for the static table");
+        g_static_aux_ptr[dev] = ptr;
+    }
+    *out = g_static_aux_ptr[dev];
+    return PCFGNAT_OK;
+}
+}  // namespace
+
+extern "C" size_t pcfgnat_static_aux_floats(void) { return (size_t)PCFGNAT_STATIC_AUX_FLOATS; }
+
+extern "C" int pcfgnat_pcfg_loss_forward_backward_static(const float *grad_output, const float *match_all, const float *links,
+                                                        const int64_t *output_length, const int64_t *target_length, float *S,
+                                                        float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T,
+                                                        int64_t ml, void *stream) {
+    int rc = check_dims("pcfg_loss_forward_backward_static", B, L, T, ml);
+    if (rc != PCFGNAT_OK) return rc;
+    const size_t need = pcfgnat_pcfg_aux_floats(B, L, T, ml);
+    PCFGNAT_REQUIRE(need <= (size_t)PCFGNAT_STATIC_AUX_FLOATS,
+                    "pcfg_loss_forward_backward_static: B=%lld L=%lld T=%lld max_left=%lld needs %zu floats of auxiliary table, the "
+                    "library's static table holds %zu (use pcfgnat_pcfg_loss_forward_backward with a buffer of the caller's)",
+                    (long long)B, (long long)L, (long long)T, (long long)ml, need, (size_t)PCFGNAT_STATIC_AUX_FLOATS);
+    float *aux = nullptr;
+    rc = static_aux_address(&aux);
+    if (rc != PCFGNAT_OK) return rc;
+    // every table the kernels read from aux is written earlier in the same call (arrival marks of the pipelined sweeps
+    // included), so what an earlier call left in the array does not matter
     return inside_forward_backward_impl(grad_output, match_all, links, output_length, target_length, S, aux, match_all_grad, links_grad,
                                         B, L, T, ml, B, stream);
 }
