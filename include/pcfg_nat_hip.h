@@ -226,6 +226,11 @@ int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *
  * alternate between `stream` and one helper stream the library keeps per device (created on first use, default
  * priority), so that the latency-bound inside kernels of one slice run beside the bandwidth-bound gather kernels of the
  * next; the helper stream forks from and joins back into `stream`, so the call stays ordered on `stream`.
+ * loss_scale, loss_scale_dev: the factor the caller's loss carries downstream of this criterion (nat_pcfg_loss.py:139-140
+ * `loss * factor`, times the fp16 loss scale of every shipped training script): a host value times an optional float32
+ * scalar in device memory (NULL = 1).  Both gradients come out multiplied by it; it enters the weights -1/(target_length*B)
+ * in float32, i.e. ahead of the single rounding of d loss / d logits to the logits' dtype, as in pcfg_loss.py:77-83, 176-177.
+ * loss_out[0] stays the unscaled loss.
  * events: NULL, or eight hipEvent_t (entries may be NULL) recorded before/after the gather forward, (unused pair), the
  * inside forward+backward and the gather backward of slice 0 (for timing).
  */
@@ -233,7 +238,31 @@ int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, cons
                            const int64_t *output_length, const int64_t *target_length, const unsigned char *matchmask,
                            const unsigned char *keep_word_mask, float *match_all, float *S,
                            float *aux, float *match_all_grad, float *links_grad, float *row_lse, float *loss_out, int64_t B,
-                           int64_t L, int64_t V, int64_t T, int64_t ml, int64_t slices, void *stream, void *const *events);
+                           int64_t L, int64_t V, int64_t T, int64_t ml, int64_t slices, float loss_scale,
+                           const float *loss_scale_dev, void *stream, void *const *events);
+
+/*
+ * The same pass cut where autograd cuts it (no counterpart in the reference, which leaves the cut to torch:
+ * pcfg_loss.py:67-83 saves the inside gradients in the forward and scales them by grad_output in the backward,
+ * :176-177 scale the probabilities by the upstream gradient before they are cast to the logits' dtype).
+ *   forward:  gather with eos mask (read only) -> inside forward + backward with weights -1/(target_length*B) -> loss.
+ *             Leaves match_all_grad, links_grad (both at an upstream gradient of 1), row_lse, loss_out[0..1]; the logits are
+ *             untouched except that the rows of pad nodes may already be zeroed (*pad_rows_zeroed tells, pass it on).
+ *   backward: logits_inout becomes upstream * d loss / d logits in one read + write pass, links_grad_inout is multiplied by
+ *             upstream.  upstream_dev: one float32 in device memory (the gradient flowing into the loss, e.g. the fp16 loss
+ *             scale times the criterion's factor; NULL = 1).  It multiplies the emission posteriors in float32 ahead of the
+ *             single rounding to the logits' dtype, so gradients below the fp16 range at scale 1 survive, and no value ever
+ *             passes through the host.
+ */
+int pcfgnat_criterion_forward(void *logits, int dtype, const int64_t *targets, const float *links, const int64_t *output_length,
+                              const int64_t *target_length, const unsigned char *matchmask, const unsigned char *keep_word_mask,
+                              float *match_all, float *S, float *aux, float *match_all_grad, float *links_grad, float *row_lse,
+                              float *loss_out, int *pad_rows_zeroed, int64_t B, int64_t L, int64_t V, int64_t T, int64_t ml,
+                              void *stream);
+int pcfgnat_criterion_backward(void *logits_inout, int dtype, const int64_t *targets, const float *match_all_grad,
+                               const float *row_lse, const unsigned char *keep_word_mask, const int64_t *output_length,
+                               int pad_rows_zeroed, const float *upstream_dev, float *links_grad_inout, int64_t B, int64_t L,
+                               int64_t V, int64_t T, int64_t ml, void *stream);
 
 /*
  * The link scorer of the model (glat_decomposed_with_link_two_hands_tri_pcfg.py:140-201, `extract_links`) after its four

@@ -45,7 +45,10 @@ SIGNATURES = {
     "pcfgnat_pcfg_viterbi_f64": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "pcfgnat_criterion_loss": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_criterion_step": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
-                                      _i64, _i64, _vp, _vp]),
+                                      _i64, _i64, ctypes.c_float, _vp, _vp, _vp]),
+    "pcfgnat_criterion_forward": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
+                                         _i64, _i64, _vp]),
+    "pcfgnat_criterion_backward": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_extract_links_pack": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_extract_links_forward": (_int, [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_extract_links_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,

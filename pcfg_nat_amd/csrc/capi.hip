@@ -10,7 +10,7 @@ char *error_buffer() {
 }
 }  // namespace pcfgnat
 
-extern "C" int pcfgnat_abi_version(void) { return 1; }
+extern "C" int pcfgnat_abi_version(void) { return 2; }
 
 extern "C" const char *pcfgnat_last_error(void) { return pcfgnat::error_buffer(); }
 
@@ -57,8 +57,8 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
                                       const int64_t *output_length, const int64_t *target_length, const unsigned char *matchmask,
                                       const unsigned char *keep_word_mask, float *match_all, float *S,
                                       float *aux, float *match_all_grad, float *links_grad, float *row_lse, float *loss_out, int64_t B,
-                                      int64_t L, int64_t V, int64_t T, int64_t ml, int64_t slices, void *stream,
-                                      void *const *events) {
+                                      int64_t L, int64_t V, int64_t T, int64_t ml, int64_t slices, float loss_scale,
+                                      const float *loss_scale_dev, void *stream, void *const *events) {
     if (dtype != PCFGNAT_F16 && dtype != PCFGNAT_F32)
         return pcfgnat::fail(PCFGNAT_EUNSUPPORTED, "criterion_step: logits must be float16 or float32 (the PCFG kernels are float32)");
     PCFGNAT_REQUIRE(B >= 1 && L >= 4 && T >= 2 && V >= 1 && ml >= 0, "criterion_step: bad dimensions");
@@ -110,17 +110,18 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
         PCFGNAT_MARK(4);
         // the rows of pad nodes of the logits gradient are zeroed beside the sweeps where the inside launch can host that
         bool pad_done = false;
-        rc = pcfgnat::inside_forward_backward_impl(nullptr, ma_i, lk_i, ol_i, tl_i, S_i, aux_i, mg_i, lkg_i, nb, L, T, ml, B, s,
+        rc = pcfgnat::inside_forward_backward_impl(nullptr, ma_i, lk_i, ol_i, tl_i, S_i, aux_i, mg_i, lkg_i, nb, L, T, ml,
+                                                   pcfgnat::seed_of(B, loss_scale, loss_scale_dev), s,
                                                    pcfgnat::PadFill{(unsigned char *)lg_i, (int64_t)V * (int64_t)esz}, &pad_done);
         if (rc != PCFGNAT_OK) return rc;
         PCFGNAT_MARK(5);
         PCFGNAT_MARK(6);
         if (slices == 1)  // the loss is reduced by the first workgroup of the same launch (S is complete by now)
             rc = pcfgnat::lsg_backward_lse_with_loss(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, S, Mc * (T + 2), target_length,
-                                                     loss_out, keep_i, ol_i, pad_done ? 1 : 0, s);
+                                                     loss_out, keep_i, ol_i, pad_done ? 1 : 0, nullptr, s);
         else
             rc = pcfgnat::lsg_backward_lse_with_loss(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, nullptr, 0, nullptr, nullptr,
-                                                     keep_i, ol_i, pad_done ? 1 : 0, s);
+                                                     keep_i, ol_i, pad_done ? 1 : 0, nullptr, s);
         if (rc != PCFGNAT_OK) return rc;
         PCFGNAT_MARK(7);
 #undef PCFGNAT_MARK
@@ -131,4 +132,67 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
     }
     if (slices == 1) return PCFGNAT_OK;
     return pcfgnat_criterion_loss(S, target_length, loss_out, B, L, T, ml, stream);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The same pass cut at the point where autograd cuts it: everything that does not depend on the loss's upstream gradient
+// in the forward (gather, both sweeps, the emission and rule posteriors with the criterion's weights, the loss), the one
+// pass that turns the logits into their gradient in the backward, where the upstream gradient - a scalar in device
+// memory - multiplies the emission posteriors in float32 ahead of the single rounding to the logits' dtype (the
+// reference scales its saved gradients before the cast as well: pcfg_loss.py:77-83, 176-177).  No host read anywhere.
+// ---------------------------------------------------------------------------------------------------------------
+namespace {
+__global__ __launch_bounds__(256) void scale_by_device_scalar_kernel(float *__restrict__ p, size_t n, const float *__restrict__ scale_dev) {
+    const float sc = *scale_dev;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] *= sc;
+}
+}  // namespace
+
+extern "C" int pcfgnat_criterion_forward(void *logits, int dtype, const int64_t *targets, const float *links,
+                                         const int64_t *output_length, const int64_t *target_length, const unsigned char *matchmask,
+                                         const unsigned char *keep_word_mask, float *match_all, float *S, float *aux,
+                                         float *match_all_grad, float *links_grad, float *row_lse, float *loss_out,
+                                         int *pad_rows_zeroed, int64_t B, int64_t L, int64_t V, int64_t T, int64_t ml, void *stream) {
+    if (dtype != PCFGNAT_F16 && dtype != PCFGNAT_F32)
+        return pcfgnat::fail(PCFGNAT_EUNSUPPORTED, "criterion_forward: logits must be float16 or float32 (the PCFG kernels are float32)");
+    PCFGNAT_REQUIRE(B >= 1 && L >= 4 && T >= 2 && V >= 1 && ml >= 0, "criterion_forward: bad dimensions");
+    PCFGNAT_REQUIRE(logits && targets && links && output_length && target_length && match_all && S && aux && match_all_grad &&
+                        links_grad && row_lse && loss_out && pad_rows_zeroed,
+                    "criterion_forward: null pointer");
+    PCFGNAT_REQUIRE((matchmask == nullptr) == (keep_word_mask == nullptr),
+                    "criterion_forward: matchmask and keep_word_mask must be given together (or both be null)");
+    const size_t esz = (dtype == PCFGNAT_F16) ? 2 : 4;
+    *pad_rows_zeroed = 0;
+    int rc = pcfgnat::lsg_forward_lse_force(logits, dtype, targets, match_all, row_lse, output_length, target_length, matchmask,
+                                            keep_word_mask, B, L, V, T, stream);
+    if (rc != PCFGNAT_OK) return rc;
+    bool pad_done = false;
+    rc = pcfgnat::inside_forward_backward_impl(nullptr, match_all, links, output_length, target_length, S, aux, match_all_grad, links_grad,
+                                               B, L, T, ml, pcfgnat::seed_of(B), stream,
+                                               pcfgnat::PadFill{(unsigned char *)logits, (int64_t)V * (int64_t)esz}, &pad_done);
+    if (rc != PCFGNAT_OK) return rc;
+    *pad_rows_zeroed = pad_done ? 1 : 0;
+    return pcfgnat_criterion_loss(S, target_length, loss_out, B, L, T, ml, stream);
+}
+
+extern "C" int pcfgnat_criterion_backward(void *logits_inout, int dtype, const int64_t *targets, const float *match_all_grad,
+                                          const float *row_lse, const unsigned char *keep_word_mask, const int64_t *output_length,
+                                          int pad_rows_zeroed, const float *upstream_dev, float *links_grad_inout, int64_t B, int64_t L,
+                                          int64_t V, int64_t T, int64_t ml, void *stream) {
+    if (dtype != PCFGNAT_F16 && dtype != PCFGNAT_F32)
+        return pcfgnat::fail(PCFGNAT_EUNSUPPORTED, "criterion_backward: logits must be float16 or float32");
+    PCFGNAT_REQUIRE(B >= 1 && L >= 4 && T >= 2 && V >= 1 && ml >= 0, "criterion_backward: bad dimensions");
+    PCFGNAT_REQUIRE(logits_inout && targets && match_all_grad && row_lse && output_length, "criterion_backward: null pointer");
+    int rc = pcfgnat::lsg_backward_lse_with_loss(logits_inout, dtype, targets, T, 0, 1, match_all_grad, row_lse, B, L, V, T, nullptr, 0,
+                                                 nullptr, nullptr, keep_word_mask, output_length, pad_rows_zeroed ? 1 : 0, upstream_dev,
+                                                 stream);
+    if (rc != PCFGNAT_OK) return rc;
+    if (links_grad_inout != nullptr && upstream_dev != nullptr) {
+        const size_t n = (size_t)B * L * (ml + 1) * L;
+        const unsigned grid = (unsigned)((n + 256 * 8 - 1) / (256 * 8));
+        hipLaunchKernelGGL(scale_by_device_scalar_kernel, dim3(grid < 1 ? 1 : grid), dim3(256), 0, (hipStream_t)stream, links_grad_inout,
+                           n, upstream_dev);
+        PCFGNAT_HIP_CHECK(hipGetLastError());
+    }
+    return PCFGNAT_OK;
 }

@@ -34,11 +34,34 @@ inline int fail(int code, const char *fmt, ...) {
     } while (0)
 
 // ---- internal entry points shared between translation units ---------------------------------------------------
-// Like the public functions of the same name, with the batch size that normalises the criterion's weights
-// (-1/(n_b * norm_B) when grad_output is null) passed separately, so that a batch can be processed in slices.
+// The criterion's own weights, used when grad_output is null: d(-(ll/n).mean() * factor)/d ll_b = -factor/(n_b * norm_B)
+// (nat_pcfg_loss.py:135, 139-140; pcfg_loss.py:77-83 for the upstream factor).  norm_B is passed apart from the batch size
+// so that a batch can be processed in slices; the factor is a host value times an optional scalar in device memory (an
+// fp16 loss scale that only the device knows), both 1 by default.
+struct Seed {
+    int norm_B;
+    float scale;
+    const float *scale_dev;
+};
+inline Seed seed_of(int64_t norm_B, float scale = 1.0f, const float *scale_dev = nullptr) {
+    return Seed{(int)norm_B, scale, scale_dev};
+}
+__device__ __forceinline__ float seed_weight(const float *grad_out, int b, int n, const Seed &sd) {
+    if (grad_out) return grad_out[b];
+    float g = -1.0f / ((float)n * (float)sd.norm_B);
+    if (sd.scale_dev) g *= *sd.scale_dev;
+    return g * sd.scale;
+}
+__device__ __forceinline__ double seed_weight(const double *grad_out, int b, int n, const Seed &sd) {
+    if (grad_out) return grad_out[b];
+    double g = -1.0 / ((double)n * (double)sd.norm_B);
+    if (sd.scale_dev) g *= (double)*sd.scale_dev;
+    return g * (double)sd.scale;
+}
+// Like the public functions of the same name, with the weights above in place of the batch size.
 int inside_backward_impl(const float *grad_output, const float *S, float *aux, const float *match_all, const float *links,
                          const int64_t *output_length, const int64_t *target_length, float *match_all_grad, float *links_grad, int64_t B,
-                         int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream);
+                         int64_t L, int64_t T, int64_t ml, Seed seed, void *stream);
 // A side task for the launch that holds the sweeps of short graphs, which leaves most of the chip and all of the memory
 // bandwidth idle: zero the rows of the pad nodes (at or beyond a sentence's output length) of a [B,L,row_bytes] buffer -
 // the criterion step's logits, whose gradient rows they are.  base null: nothing to do.  *pad_done (if given) tells
@@ -49,7 +72,7 @@ struct PadFill {
 };
 int inside_forward_backward_impl(const float *grad_output, const float *match_all, const float *links, const int64_t *output_length,
                                  const int64_t *target_length, float *S, float *aux, float *match_all_grad, float *links_grad,
-                                 int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream,
+                                 int64_t B, int64_t L, int64_t T, int64_t ml, Seed seed, void *stream,
                                  PadFill pad = PadFill{nullptr, 0}, bool *pad_done = nullptr);
 
 // Read-only logsoftmax_gather over the [B,T] targets with the eos mask, which also returns the first arg max of every row;
@@ -61,11 +84,13 @@ int lsg_forward_eos_argmax(const void *logits, int dtype, const int64_t *targets
 // pcfgnat_logsoftmax_gather_backward_lse whose first workgroup also reduces the criterion's loss when loss_out is given
 // (lsg.hip); rows with keep[row] != 0 get a zero gradient; with pad_output_length, the rows of nodes at or beyond a
 // sentence's output length (whose grad_selected rows the caller guarantees to be all zero) are zeroed without being read,
-// or left alone when the caller has zeroed them already (pad_rows_zeroed)
+// or left alone when the caller has zeroed them already (pad_rows_zeroed); gscale_dev (may be null): one float in device
+// memory that multiplies grad_selected on the fly
 int lsg_backward_lse_with_loss(void *logits_inout, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T,
                                const float *S, int64_t ll_stride, const int64_t *target_length, float *loss_out,
-                               const unsigned char *keep, const int64_t *pad_output_length, int pad_rows_zeroed, void *stream);
+                               const unsigned char *keep, const int64_t *pad_output_length, int pad_rows_zeroed, const float *gscale_dev,
+                               void *stream);
 // pcfgnat_logsoftmax_gather_lse over the [B,T] targets with the eos mask and the force-emit masks; the rows of nodes at
 // or beyond a sentence's output length are left unread (zeros in selected and lse)
 int lsg_forward_lse_force(const void *logits, int dtype, const int64_t *targets, void *selected, void *lse,
@@ -82,7 +107,7 @@ size_t generic_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml);
 int generic_forward(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int64_t B,
                     int64_t L, int64_t T, int64_t ml, void *stream);
 int generic_backward(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
-                     const int64_t *tl, float *mg, float *lg, int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream);
+                     const int64_t *tl, float *mg, float *lg, int64_t B, int64_t L, int64_t T, int64_t ml, Seed seed, void *stream);
 int generic_best_tree(const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl,
                       int64_t *tree, int64_t B, int64_t L, int64_t T, int64_t ml, void *stream);
 int generic_viterbi(const float *ob, const float *links, const int64_t *ol, float *S, int64_t *R, int64_t *Lt, int64_t *M, int64_t B,

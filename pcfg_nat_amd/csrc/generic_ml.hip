@@ -158,7 +158,7 @@ __global__ __launch_bounds__(NTG) void generic_bwd_kernel(const RT *__restrict__
                                                          RT *__restrict__ aux_all, const RT *__restrict__ match_all,
                                                          const RT *__restrict__ links_all, const int64_t *__restrict__ out_len,
                                                          const int64_t *__restrict__ tgt_len, RT *__restrict__ mg_all,
-                                                         RT *__restrict__ lg_all, int L, int T, int ml, int norm_B) {
+                                                         RT *__restrict__ lg_all, int L, int T, int ml, Seed seed) {
     const Dims d(L, T, ml);
     const int b = blockIdx.x, tid = threadIdx.x;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(NTG) void generic_bwd_kernel(const RT *__restrict__
     for (size_t i = tid; i < d.s_size(); i += NTG) Sg[i] = 0.f;
     for (size_t i = tid; i < d.c_size(); i += NTG) Cg[i] = 0.f;
     __syncthreads();
-    const RT g = grad_out ? grad_out[b] : -1.0f / ((RT)n * (RT)norm_B);
+    const RT g = seed_weight(grad_out, b, n, seed);
     if (tid == 0) Sg[0] = g;  // :76-80
     __syncthreads();
     // main chain, start ascending (:83-112, 175-205, 348-376, 512-531)
@@ -438,9 +438,9 @@ int forward_t(const RT *match_all, const RT *links, const int64_t *ol, const int
 }
 template <typename RT>
 int backward_t(const RT *go, const RT *S, RT *aux, const RT *match_all, const RT *links, const int64_t *ol, const int64_t *tl, RT *mg, RT *lg,
-               int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream) {
+               int64_t B, int64_t L, int64_t T, int64_t ml, Seed seed, void *stream) {
     hipLaunchKernelGGL(generic_bwd_kernel<RT>, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, go, S, aux, match_all, links, ol, tl, mg,
-                       lg, (int)L, (int)T, (int)ml, (int)norm_B);
+                       lg, (int)L, (int)T, (int)ml, seed);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -477,8 +477,8 @@ int generic_forward(const float *match_all, const float *links, const int64_t *o
 }
 
 int generic_backward(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
-                     const int64_t *tl, float *mg, float *lg, int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream) {
-    return backward_t<float>(go, S, aux, match_all, links, ol, tl, mg, lg, B, L, T, ml, norm_B, stream);
+                     const int64_t *tl, float *mg, float *lg, int64_t B, int64_t L, int64_t T, int64_t ml, Seed seed, void *stream) {
+    return backward_t<float>(go, S, aux, match_all, links, ol, tl, mg, lg, B, L, T, ml, seed, stream);
 }
 
 int generic_best_tree(const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl,
@@ -521,7 +521,7 @@ extern "C" int pcfgnat_pcfg_loss_backward_f64(const double *grad_output, const d
     PCFGNAT_REQUIRE(grad_output && S && aux && match_all && links && output_length && target_length && match_all_grad && links_grad,
                     "pcfg_loss_backward_f64: null pointer");
     return backward_t<double>(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, B, L, T, ml,
-                              B, stream);
+                              seed_of(B), stream);
 }
 
 extern "C" int pcfgnat_pcfg_best_tree_f64(const double *S, double *aux, const double *match_all, const double *links,

@@ -523,7 +523,7 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
                                                             float *__restrict__ aux, const float *__restrict__ match_all,
                                                             const float *__restrict__ links, const int64_t *__restrict__ out_len,
                                                             const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad,
-                                                            float *__restrict__ lgrad, int L, int T, int Mc, int norm_B) {
+                                                            float *__restrict__ lgrad, int L, int T, int Mc, Seed seed) {
     constexpr int NQ = 8 * R;
     constexpr int MP = 64 * R;
     const int TS = T + 2;
@@ -556,8 +556,8 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
         return;
     }
     const int mc = m / 2;
-    // a null grad_output selects the criterion's own weights: d(-(ll/n).mean())/d ll_b = -1/(n_b * norm_B)
-    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)norm_B);
+    // a null grad_output selects the criterion's own weights: -factor/(n_b * norm_B), see Seed
+    const float g = seed_weight(grad_out, b, n, seed);
 
     PCFGNAT_PHASE(8);
     // links_grad is zero outside the cells the register accumulators own (written at the very end, after the barriers of
@@ -701,7 +701,7 @@ __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__re
                                                               const float *__restrict__ links, const int64_t *__restrict__ out_len,
                                                               const int64_t *__restrict__ tgt_len, float *__restrict__ S,
                                                               float *__restrict__ mgrad, float *__restrict__ lgrad, int L, int T,
-                                                              int Mc, int norm_B) {
+                                                              int Mc, Seed seed) {
     constexpr int NQ = 8 * R;
     constexpr int MP = 64 * R;
     const int TS = T + 2;
@@ -740,7 +740,7 @@ __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__re
         return;
     }
     const int mc = m / 2;
-    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)norm_B);
+    const float g = seed_weight(grad_out, b, n, seed);
 
     // ---- forward
     float A0[R][NQ], A1[R][NQ];
@@ -1150,7 +1150,7 @@ __global__ __launch_bounds__(256) void inside_combine_ml1_kernel(const float *__
                                                                 float *__restrict__ aux, const float *__restrict__ match_all,
                                                                 const float *__restrict__ links, const int64_t *__restrict__ out_len,
                                                                 const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad,
-                                                                float *__restrict__ lgrad, int L, int T, int Mc, int norm_B) {
+                                                                float *__restrict__ lgrad, int L, int T, int Mc, Seed seed) {
     const int TS = T + 2, TP = T + 4;
     extern __shared__ float smem[];
     float *corr = smem;               // [TP]
@@ -1174,8 +1174,8 @@ __global__ __launch_bounds__(256) void inside_combine_ml1_kernel(const float *__
         return;
     }
     const int mc = m / 2;
-    // a null grad_output selects the criterion's own weights: d(-(ll/n).mean())/d ll_b = -1/(n_b * norm_B)
-    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)norm_B);
+    // a null grad_output selects the criterion's own weights: -factor/(n_b * norm_B), see Seed
+    const float g = seed_weight(grad_out, b, n, seed);
     // this thread's pair: parent 4*part + tid/64, child tid%64; its two link values travel during the staging
     const int a_id = 4 * part + (tid >> 6), c_id = tid & 63;
     const bool pair_ok = a_id < mc && c_id < mc && a_id <= c_id;
@@ -2714,7 +2714,7 @@ __global__ __launch_bounds__(1024) void links_grad_ml1_stream_kernel(const float
                                                                     const float *__restrict__ aux_c, const float *__restrict__ links,
                                                                     const int64_t *__restrict__ out_len,
                                                                     const int64_t *__restrict__ tgt_len, float *__restrict__ lgrad,
-                                                                    int L, int T, int Mc, int B, int use_corr) {
+                                                                    int L, int T, int Mc, Seed seed, int use_corr) {
     __shared__ float sw0[32][33], sw1[32][33], ss[32][33];
     const int b = blockIdx.z, at = blockIdx.y, ct = blockIdx.x;
     if (ct < at) return;
@@ -2726,7 +2726,7 @@ __global__ __launch_bounds__(1024) void links_grad_ml1_stream_kernel(const float
     if (at * 32 >= mc || ct * 32 >= mc) return;
     AuxViewStream av(const_cast<float *>(aux_c), b, Mc, T);
     const float *corr = ExchangeView(const_cast<float *>(aux_c), b, Mc, T).corr;  // per column, when the sweeps ran side by side
-    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)B);
+    const float g = seed_weight(grad_out, b, n, seed);
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     const int a_id = at * 32 + ty, c_id = ct * 32 + tx;
     const int a = 2 * a_id + 1, c = 2 * c_id + 1;
@@ -2773,7 +2773,7 @@ __global__ __launch_bounds__(256) void match_grad_ml1_stream_kernel(const float 
                                                                    const float *__restrict__ aux_c, const float *__restrict__ match_all,
                                                                    const int64_t *__restrict__ out_len,
                                                                    const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad, int L,
-                                                                   int T, int Mc, int B, int use_corr) {
+                                                                   int T, int Mc, Seed seed, int use_corr) {
     const int b = blockIdx.y;
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= L * T) return;
@@ -2788,7 +2788,7 @@ __global__ __launch_bounds__(256) void match_grad_ml1_stream_kernel(const float 
     }
     const int mc = m / 2;
     AuxViewStream av(const_cast<float *>(aux_c), b, Mc, T);
-    const float g = grad_out ? grad_out[b] : -1.0f / ((float)n * (float)B);
+    const float g = seed_weight(grad_out, b, n, seed);
     const int x = i / T, s = i - x * T;
     // corrections of the columns (see pipeline_finish_kernel): on the forward's offsets they are 0 and -D_t
     const float *corr = ExchangeView(const_cast<float *>(aux_c), b, Mc, T).corr;
@@ -2957,7 +2957,7 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
 // side_by_side: the outside pipeline has already run, beside the forward one (launch_both_stream): only the redo of the
 // sentences it gave up and the posteriors (with their per-column corrections) are left to do.
 int launch_bwd_stream(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
-                      const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream,
+                      const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, Seed seed, hipStream_t stream,
                       bool side_by_side = false, bool slabs_zeroed = false) {
     const int MP = stream_mp(Mc);
     const int tiles = (Mc + 31) / 32;
@@ -2995,10 +2995,10 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
     }
     const int use_corr = side_by_side ? 1 : 0;
     hipLaunchKernelGGL(links_grad_ml1_stream_kernel, dim3(tiles, tiles, B), dim3(1024), 0, stream, go, S, aux, links, ol, tl, lg, L, T, Mc,
-                       norm_B, use_corr);
+                       seed, use_corr);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL(match_grad_ml1_stream_kernel, dim3((L * T + 255) / 256, B), dim3(256), 0, stream, go, S, aux, match_all, ol, tl, mg, L,
-                       T, Mc, norm_B, use_corr);
+                       T, Mc, seed, use_corr);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -3024,18 +3024,18 @@ int launch_fwd(const float *match_all, const float *links, const int64_t *ol, co
 
 template <int R>
 int launch_bwd(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
-               const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream) {
+               const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, Seed seed, hipStream_t stream) {
     const size_t base = ((size_t)head_floats(T) + 4 * 64 * R) * sizeof(float);
     const size_t with_tab = base + ((size_t)2 * Mc * T + (size_t)4 * Mc * (T + 2)) * sizeof(float);
     if (with_tab <= LDS_BUDGET) {
         auto k = inside_bwd_ml1_kernel<R, true>;
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_tab));
-        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), with_tab, stream, go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc, norm_B);
+        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), with_tab, stream, go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc, seed);
     } else {
         auto k = inside_bwd_ml1_kernel<R, false>;
         PCFGNAT_REQUIRE(base <= LDS_BUDGET, "pcfg_loss_backward: target length %d too large for the column offsets in LDS", T);
         PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)base));
-        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), base, stream, go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc, norm_B);
+        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), base, stream, go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc, seed);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
@@ -3044,7 +3044,7 @@ int launch_bwd(const float *go, const float *S, float *aux, const float *match_a
 // Returns PCFGNAT_EUNSUPPORTED (without a message being an error for the caller) when the fused kernel does not apply.
 template <int R>
 int launch_fused(const float *go, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux,
-                 float *mg, float *lg, int B, int L, int T, int Mc, int norm_B, hipStream_t stream, bool *done,
+                 float *mg, float *lg, int B, int L, int T, int Mc, Seed seed, hipStream_t stream, bool *done,
                  PadFill pad = PadFill{nullptr, 0}, bool *pad_done = nullptr) {
     const size_t need = ((size_t)head_floats(T) + 4 * 64 * R + (size_t)4 * Mc * (T + 2) + (size_t)2 * Mc * T) * sizeof(float);
     *done = false;
@@ -3070,7 +3070,7 @@ int launch_fused(const float *go, const float *match_all, const float *links, co
             PCFGNAT_HIP_CHECK(hipGetLastError());
             if (fill && pad_done) *pad_done = true;
             hipLaunchKernelGGL(inside_combine_ml1_kernel, dim3(16, B), dim3(256), comb_bytes, stream, go, S, aux, match_all, links, ol, tl,
-                               mg, lg, L, T, Mc, norm_B);
+                               mg, lg, L, T, Mc, seed);
             PCFGNAT_HIP_CHECK(hipGetLastError());
             *done = true;
             return PCFGNAT_OK;
@@ -3079,7 +3079,7 @@ int launch_fused(const float *go, const float *match_all, const float *links, co
     if (need > LDS_BUDGET) return PCFGNAT_OK;
     auto k = inside_fused_ml1_kernel<R>;
     PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)need));
-    hipLaunchKernelGGL(k, dim3(B), dim3(NTR), need, stream, go, match_all, links, ol, tl, S, mg, lg, L, T, Mc, norm_B);
+    hipLaunchKernelGGL(k, dim3(B), dim3(NTR), need, stream, go, match_all, links, ol, tl, S, mg, lg, L, T, Mc, seed);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     *done = true;
     return PCFGNAT_OK;
@@ -3134,7 +3134,7 @@ extern "C" int pcfgnat_pcfg_loss(const float *match_all, const float *links, con
 
 int pcfgnat::inside_backward_impl(const float *grad_output, const float *S, float *aux, const float *match_all, const float *links,
                                   const int64_t *output_length, const int64_t *target_length, float *match_all_grad, float *links_grad,
-                                  int64_t B, int64_t L, int64_t T, int64_t ml, int64_t norm_B, void *stream) {
+                                  int64_t B, int64_t L, int64_t T, int64_t ml, Seed seed, void *stream) {
     int rc = check_dims("pcfg_loss_backward", B, L, T, ml);
     if (rc != PCFGNAT_OK) return rc;
     if (B == 0) return PCFGNAT_OK;
@@ -3142,14 +3142,14 @@ int pcfgnat::inside_backward_impl(const float *grad_output, const float *S, floa
                     "pcfg_loss_backward: null pointer");
     if (ml != 1)
         return generic_backward(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, B, L, T,
-                                ml, norm_B, stream);
+                                ml, seed, stream);
     const int Mc = (int)((L - 2) / 2 + 1);
     hipStream_t s = (hipStream_t)stream;
     if (Mc <= 64)
         return launch_bwd<1>(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
-                             (int)L, (int)T, Mc, (int)norm_B, s);
+                             (int)L, (int)T, Mc, seed, s);
     return launch_bwd_stream(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
-                             (int)L, (int)T, Mc, (int)norm_B, s);
+                             (int)L, (int)T, Mc, seed, s);
 }
 
 extern "C" int pcfgnat_pcfg_loss_backward(const float *grad_output, const float *S, float *aux, const float *match_all,
@@ -3157,13 +3157,13 @@ extern "C" int pcfgnat_pcfg_loss_backward(const float *grad_output, const float 
                                           float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T, int64_t ml,
                                           void *stream) {
     return inside_backward_impl(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, B, L, T,
-                                ml, B, stream);
+                                ml, seed_of(B), stream);
 }
 
 int pcfgnat::inside_forward_backward_impl(const float *grad_output, const float *match_all, const float *links,
                                           const int64_t *output_length, const int64_t *target_length, float *S, float *aux,
                                           float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T, int64_t ml,
-                                          int64_t norm_B, void *stream, PadFill pad, bool *pad_done) {
+                                          Seed seed, void *stream, PadFill pad, bool *pad_done) {
     if (pad_done) *pad_done = false;
     int rc = check_dims("pcfg_loss_forward_backward", B, L, T, ml);
     if (rc != PCFGNAT_OK) return rc;
@@ -3177,18 +3177,18 @@ int pcfgnat::inside_forward_backward_impl(const float *grad_output, const float 
         // general max_left: the two plain kernels
     } else if (Mc <= 64)
         rc = launch_fused<1>(grad_output, match_all, links, output_length, target_length, S, aux, match_all_grad, links_grad, (int)B, (int)L,
-                             (int)T, Mc, (int)norm_B, s, &done, pad, pad_done);
+                             (int)T, Mc, seed, s, &done, pad, pad_done);
     if (rc != PCFGNAT_OK || done) return rc;
     if (ml == 1 && Mc > 64 && side_by_side_applies((int)B, (int)T, Mc)) {  // the two pipelined sweeps in one launch
         rc = launch_fwd_stream(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s, true, links_grad);
         if (rc != PCFGNAT_OK) return rc;
         return launch_bwd_stream(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
-                                 (int)L, (int)T, Mc, (int)norm_B, s, true, true);
+                                 (int)L, (int)T, Mc, seed, s, true, true);
     }
     rc = pcfgnat_pcfg_loss(match_all, links, output_length, target_length, S, aux, B, L, T, ml, stream);
     if (rc != PCFGNAT_OK) return rc;
     return inside_backward_impl(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, B, L, T,
-                                ml, norm_B, stream);
+                                ml, seed, stream);
 }
 
 extern "C" int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *match_all, const float *links,
@@ -3196,7 +3196,7 @@ extern "C" int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, cons
                                                  float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T,
                                                  int64_t ml, void *stream) {
     return inside_forward_backward_impl(grad_output, match_all, links, output_length, target_length, S, aux, match_all_grad, links_grad,
-                                        B, L, T, ml, B, stream);
+                                        B, L, T, ml, seed_of(B), stream);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -3247,7 +3247,7 @@ extern "C" int pcfgnat_pcfg_loss_forward_backward_static(const float *grad_outpu
     // every table the kernels read from aux is written earlier in the same call (arrival marks of the pipelined sweeps
     // included), so what an earlier call left in the array does not matter
     return inside_forward_backward_impl(grad_output, match_all, links, output_length, target_length, S, aux, match_all_grad, links_grad,
-                                        B, L, T, ml, B, stream);
+                                        B, L, T, ml, seed_of(B), stream);
 }
 
 extern "C" int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *out, int64_t B, int64_t L, int64_t T,

@@ -461,10 +461,15 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
                                                      int L, int V, int Tn,
                                                      const typename Elem<T>::compute *__restrict__ lse, LossTask loss,
                                                      const unsigned char *__restrict__ detach_rows,
-                                                     const int64_t *__restrict__ pad_out_len, int pad_rows_zeroed) {
+                                                     const int64_t *__restrict__ pad_out_len, int pad_rows_zeroed,
+                                                     const float *__restrict__ gscale_dev) {
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
     constexpr int FIX = (TCAP + NT - 1) / NT;
+    // an upstream factor of the whole gradient that only the device knows (the loss's own upstream gradient under fp16 loss
+    // scaling): folded into g in the compute type, ahead of the single rounding to the buffer's dtype (pcfg_loss.py:77-83,
+    // 176-177 scale g before the cast as well)
+    const CT gs = (FROM_LOGITS && gscale_dev != nullptr) ? (CT)*gscale_dev : (CT)1;
     if (loss.out != nullptr && blockIdx.x == 0) criterion_loss_block<NT>(loss);  // workgroup-uniform
     __shared__ __attribute__((aligned(16))) int s_idx[TCAP + 4];  // padded to a multiple of four with -2 (matches nothing)
     __shared__ CT s_g[TCAP];   // cast(g[s]) in the buffer's dtype, widened again
@@ -507,7 +512,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
         const bool live = detach_rows == nullptr || detach_rows[row] == 0;
         CT part = 0;
         for (int s = lane; s < Tn && live; s += 64) part += gr[s];
-        const CT ns = FROM_LOGITS ? -wave_sum(part) : Elem<T>::widen(Elem<T>::narrow(-wave_sum(part)));
+        const CT ns = FROM_LOGITS ? -wave_sum(part) * gs : Elem<T>::widen(Elem<T>::narrow(-wave_sum(part)));
         const RowNorm<CT> rn = RowNorm<CT>::from_lse(FROM_LOGITS ? lse[row] : (CT)0);
 
         for (int s = tid; s < ((Tn + 3) & ~3); s += NT) {
@@ -519,7 +524,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
             bool ok = (uint64_t)t < (uint64_t)V;
             s_idx[s] = ok ? (int)t : -1;
             if (FROM_LOGITS) {
-                s_g[s] = live ? gr[s] : (CT)0;
+                s_g[s] = live ? gr[s] * gs : (CT)0;
                 s_p[s] = ok ? rn.e(Elem<T>::widen(pr[t])) : (CT)0;
             } else {
                 s_g[s] = live ? Elem<T>::widen(Elem<T>::narrow(gr[s])) : (CT)0;
@@ -618,7 +623,7 @@ int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
 template <typename T>
 int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, const void *g, int64_t rows, int L, int V,
                int Tn, const void *lse, const LossTask &loss, hipStream_t stream, const unsigned char *detach_rows = nullptr,
-               const int64_t *pad_out_len = nullptr, int pad_rows_zeroed = 0) {
+               const int64_t *pad_out_len = nullptr, int pad_rows_zeroed = 0, const float *gscale_dev = nullptr) {
     using CT = typename Elem<T>::compute;
     constexpr int NT = 512;
     constexpr int MAXC = 10;
@@ -627,10 +632,10 @@ int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
     int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
     if (lse != nullptr)
         hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, true>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,
-                           (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss, detach_rows, pad_out_len, pad_rows_zeroed);
+                           (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev);
     else
         hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, false>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl,
-                           st, (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss, detach_rows, pad_out_len, pad_rows_zeroed);
+                           st, (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss, detach_rows, pad_out_len, pad_rows_zeroed, nullptr);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -727,18 +732,18 @@ static int lsg_backward_dispatch(void *buf, int dtype, const int64_t *select_idx
                                  const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T, void *stream,
                                  const LossTask &loss = LossTask{nullptr, nullptr, nullptr, 0, 0},
                                  const unsigned char *detach_rows = nullptr, const int64_t *pad_out_len = nullptr,
-                                 int pad_rows_zeroed = 0) {
+                                 int pad_rows_zeroed = 0, const float *gscale_dev = nullptr) {
     int rc = check_common(buf, select_idx, grad_selected, B, L, V, T);
     if (rc != PCFGNAT_OK) return rc;
     if (B * L == 0) return PCFGNAT_OK;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case PCFGNAT_F16:
-            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed);
+            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev);
         case PCFGNAT_F32:
-            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed);
+            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev);
         case PCFGNAT_F64:
-            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed);
+            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev);
         default:
             return fail(PCFGNAT_EINVAL, "logsoftmax_gather_backward: unknown dtype code %d", dtype);
     }
@@ -761,11 +766,11 @@ int pcfgnat::lsg_backward_lse_with_loss(void *logits_inout, int dtype, const int
                                         const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T,
                                         const float *S, int64_t ll_stride, const int64_t *target_length, float *loss_out,
                                         const unsigned char *keep, const int64_t *pad_output_length, int pad_rows_zeroed,
-                                        void *stream) {
+                                        const float *gscale_dev, void *stream) {
     PCFGNAT_REQUIRE(B >= 1 && L >= 1 && lse && (loss_out == nullptr || (S && target_length)),
                     "logsoftmax_gather_backward: null pointer or empty batch");
     return lsg_backward_dispatch(logits_inout, dtype, select_idx, sb, sl, st, grad_selected, lse, B, L, V, T, stream,
-                                 LossTask{S, target_length, loss_out, (int)B, ll_stride}, keep, pad_output_length, pad_rows_zeroed);
+                                 LossTask{S, target_length, loss_out, (int)B, ll_stride}, keep, pad_output_length, pad_rows_zeroed, gscale_dev);
 }
 
 int pcfgnat::lsg_forward_lse_force(const void *logits, int dtype, const int64_t *targets, void *selected, void *lse,

@@ -742,8 +742,39 @@ def pcfg_lookahead_decode(links, unreduced_logits, unreduced_tokens, output_leng
     return (tokens, idx) if return_pointers else tokens
 
 
+def _criterion_args(name, logits, targets, links, output_length, target_length, matchmask, keep_word_mask):
+    """Checks shared by the criterion entry points; returns (code, B, L, V, T, ml, Mc, targets, links, ol, tl, mask tensors)."""
+    _need_cuda(name, logits, targets, links, output_length, target_length)
+    if logits.dim() != 3 or not logits.is_contiguous():
+        raise RuntimeError("%s: logits must be a contiguous [bsz, prelen, vocab] tensor" % name)
+    B, L, V = logits.shape
+    if targets.dim() != 2 or targets.size(0) != B or targets.dtype != torch.int64:
+        raise RuntimeError("%s: targets must be an int64 [bsz, tarlen] tensor" % name)
+    T = targets.size(1)
+    code = _DTYPE_CODE.get(logits.dtype)
+    if code is None or code == _lib.F64:
+        raise RuntimeError("%s: logits must be float16 or float32" % name)
+    if links.dim() != 4 or links.size(0) != B or links.size(1) != L or links.size(3) != L or links.dtype != torch.float32:
+        raise RuntimeError("%s: links must be float32 [bsz, prelen, max_left+1, prelen]" % name)
+    ml = links.size(2) - 1
+    targets, links = targets.contiguous(), links.contiguous()
+    ol = _lengths(name, output_length, B)
+    tl = _lengths(name, target_length, B)
+    Mc = (L - 2) // (ml + 1) + 1
+    if (matchmask is None) != (keep_word_mask is None):
+        raise RuntimeError("%s: matchmask and keep_word_mask go together" % name)
+    mm8 = keep8 = None
+    if matchmask is not None:
+        _need_cuda(name, logits, matchmask, keep_word_mask)
+        if tuple(matchmask.shape) != (B, T, L) or tuple(keep_word_mask.shape) != (B, L):
+            raise RuntimeError("%s: matchmask must be [bsz, tarlen, prelen] and keep_word_mask [bsz, prelen]" % name)
+        mm8 = matchmask.to(torch.uint8).contiguous()
+        keep8 = keep_word_mask.to(torch.uint8).contiguous()
+    return code, B, L, V, T, ml, Mc, targets, links, ol, tl, mm8, keep8
+
+
 def pcfg_criterion_step(logits, targets, links, output_length, target_length, events=None, slices=None, matchmask=None,
-                        keep_word_mask=None):
+                        keep_word_mask=None, loss_scale=1.0):
     """The criterion's whole training pass in one native call (``pcfgnat_criterion_step``): ``logits`` [B,L,V] (fp16 or
     fp32, contiguous) is consumed in place and holds d loss / d logits afterwards.  ``events``: optional list of eight
     ``torch.cuda.Event(enable_timing=True)`` (each recorded at least once before; entries may be None) that the library records before/after
@@ -753,39 +784,28 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
     ``matchmask`` [B,T,L] / ``keep_word_mask`` [B,L] (bool, as the glancing step returns them): the criterion's
     force-emit masking (nat_pcfg_loss.py:116-121); both None = off (``--no-force-emit``).  The rows of the pad nodes at
     or beyond a sentence's ``output_length`` feed nothing (neither sweep reads them, their gradient is zero): the gather
-    forward leaves them unread (zeros in the returned ``match_all``) and the backward zeroes them without reading.  Returns
+    forward leaves them unread (zeros in the returned ``match_all``) and the backward zeroes them without reading.
+    ``loss_scale``: the factor the caller's loss carries downstream of the criterion (``loss * factor``,
+    nat_pcfg_loss.py:139-140, times the fp16 loss scale) - a Python number, or a one-element float32 tensor on the device
+    (no host read); both gradients come out multiplied by it, the factor entering in float32 ahead of the single rounding
+    of d loss / d logits to the logits' dtype (pcfg_loss.py:77-83, 176-177).  The returned loss stays unscaled.  Returns
     (loss_and_invalid [2] float32, links_grad, ll [B], match_all_eos_masked, match_all_grad)."""
     lib = get_pcfg_kernel()
-    _need_cuda("pcfg_criterion_step", logits, targets, links, output_length, target_length)
-    if logits.dim() != 3 or not logits.is_contiguous():
-        raise RuntimeError("pcfg_criterion_step: logits must be a contiguous [bsz, prelen, vocab] tensor")
-    B, L, V = logits.shape
-    if targets.dim() != 2 or targets.size(0) != B or targets.dtype != torch.int64:
-        raise RuntimeError("pcfg_criterion_step: targets must be an int64 [bsz, tarlen] tensor")
-    T = targets.size(1)
-    code = _DTYPE_CODE.get(logits.dtype)
-    if code is None or code == _lib.F64:
-        raise RuntimeError("pcfg_criterion_step: logits must be float16 or float32")
-    if links.dim() != 4 or links.size(0) != B or links.size(1) != L or links.size(3) != L or links.dtype != torch.float32:
-        raise RuntimeError("pcfg_criterion_step: links must be float32 [bsz, prelen, max_left+1, prelen]")
-    ml = links.size(2) - 1
-    targets, links = targets.contiguous(), links.contiguous()
-    ol = _lengths("pcfg_criterion_step", output_length, B)
-    tl = _lengths("pcfg_criterion_step", target_length, B)
-    Mc = (L - 2) // (ml + 1) + 1
+    code, B, L, V, T, ml, Mc, targets, links, ol, tl, mm8, keep8 = _criterion_args(
+        "pcfg_criterion_step", logits, targets, links, output_length, target_length, matchmask, keep_word_mask)
     dev = logits.device
     if slices is None:
         slices = 1
-    if (matchmask is None) != (keep_word_mask is None):
-        raise RuntimeError("pcfg_criterion_step: matchmask and keep_word_mask go together")
-    mm_ptr = keep_ptr = None
-    if matchmask is not None:
-        _need_cuda("pcfg_criterion_step", logits, matchmask, keep_word_mask)
-        if tuple(matchmask.shape) != (B, T, L) or tuple(keep_word_mask.shape) != (B, L):
-            raise RuntimeError("pcfg_criterion_step: matchmask must be [bsz, tarlen, prelen] and keep_word_mask [bsz, prelen]")
-        mm8 = matchmask.to(torch.uint8).contiguous()
-        keep8 = keep_word_mask.to(torch.uint8).contiguous()
-        mm_ptr, keep_ptr = mm8.data_ptr(), keep8.data_ptr()
+    mm_ptr = mm8.data_ptr() if mm8 is not None else None
+    keep_ptr = keep8.data_ptr() if keep8 is not None else None
+    scale_host, scale_dev = 1.0, None
+    if torch.is_tensor(loss_scale):
+        _need_cuda("pcfg_criterion_step", logits, loss_scale)
+        if loss_scale.numel() != 1:
+            raise RuntimeError("pcfg_criterion_step: loss_scale must be a number or a one-element tensor")
+        scale_dev = loss_scale.detach().reshape(1).to(torch.float32)
+    else:
+        scale_host = float(loss_scale)
     ev_arr = None
     if events is not None:
         import ctypes
@@ -803,28 +823,77 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
         _lib.check(lib.pcfgnat_criterion_step(logits.data_ptr(), code, targets.data_ptr(), links.data_ptr(), ol.data_ptr(),
                                               tl.data_ptr(), mm_ptr, keep_ptr, match.data_ptr(), S.data_ptr(), aux.data_ptr(), mg.data_ptr(),
                                               lg.data_ptr(), row_lse.data_ptr(), out.data_ptr(), B, L, V, T, ml, slices,
+                                              scale_host, scale_dev.data_ptr() if scale_dev is not None else None,
                                               _stream(logits), ev_arr), lib)
     return out, lg, S[:, 0, 0], match, mg
 
 
+def _criterion_forward(logits, targets, links, output_length, target_length, matchmask=None, keep_word_mask=None):
+    """Forward half of the criterion pass (``pcfgnat_criterion_forward``): everything that does not depend on the loss's
+    upstream gradient.  Returns (loss_and_invalid [2], ll [B], state) where ``state`` carries what
+    ``_criterion_backward`` needs; ``logits`` must stay untouched until then (rows of pad nodes may already be zeroed)."""
+    import ctypes
+    lib = get_pcfg_kernel()
+    code, B, L, V, T, ml, Mc, targets, links, ol, tl, mm8, keep8 = _criterion_args(
+        "pcfg_criterion", logits, targets, links, output_length, target_length, matchmask, keep_word_mask)
+    dev = logits.device
+    pad_zeroed = ctypes.c_int(0)
+    with torch.cuda.device(dev):
+        match = torch.empty((B, L, T), dtype=torch.float32, device=dev)
+        S = torch.empty((B, Mc, T + 2), dtype=torch.float32, device=dev)
+        aux = torch.empty((max(1, lib.pcfgnat_pcfg_aux_floats(B, L, T, ml)),), dtype=torch.float32, device=dev)
+        mg = torch.empty_like(match)
+        lg = torch.empty_like(links)
+        row_lse = torch.empty((B, L), dtype=torch.float32, device=dev)
+        out = torch.empty((2,), dtype=torch.float32, device=dev)
+        _lib.check(lib.pcfgnat_criterion_forward(logits.data_ptr(), code, targets.data_ptr(), links.data_ptr(), ol.data_ptr(),
+                                                 tl.data_ptr(), mm8.data_ptr() if mm8 is not None else None,
+                                                 keep8.data_ptr() if keep8 is not None else None, match.data_ptr(), S.data_ptr(),
+                                                 aux.data_ptr(), mg.data_ptr(), lg.data_ptr(), row_lse.data_ptr(), out.data_ptr(),
+                                                 ctypes.byref(pad_zeroed), B, L, V, T, ml, _stream(logits)), lib)
+    state = {"targets": targets, "match_all_grad": mg, "links_grad": lg, "row_lse": row_lse, "keep": keep8, "output_length": ol,
+             "pad_rows_zeroed": int(pad_zeroed.value), "dims": (code, B, L, V, T, ml)}
+    return out, S[:, 0, 0], state
+
+
+def _criterion_backward(logits, state, upstream):
+    """Backward half (``pcfgnat_criterion_backward``): ``logits`` becomes ``upstream`` * d loss / d logits in place and the
+    saved rule gradients are multiplied by ``upstream`` (a one-element tensor on the device; it is never read by the
+    host).  Returns (logits, links_grad)."""
+    lib = get_pcfg_kernel()
+    code, B, L, V, T, ml = state["dims"]
+    up = upstream.detach().reshape(1).to(device=logits.device, dtype=torch.float32)
+    keep8 = state["keep"]
+    with torch.cuda.device(logits.device):
+        _lib.check(lib.pcfgnat_criterion_backward(logits.data_ptr(), code, state["targets"].data_ptr(), state["match_all_grad"].data_ptr(),
+                                                  state["row_lse"].data_ptr(), keep8.data_ptr() if keep8 is not None else None,
+                                                  state["output_length"].data_ptr(), state["pad_rows_zeroed"], up.data_ptr(),
+                                                  state["links_grad"].data_ptr(), B, L, V, T, ml, _stream(logits)), lib)
+    return logits, state["links_grad"]
+
+
 class PCFGCriterionFunc(Function):
-    """The criterion's loss (nat_pcfg_loss.py:98-145) as one differentiable op over ``pcfg_criterion_step``.  Like the
-    reference's own ops (pcfg_loss.py:67-73 runs the inside backward eagerly inside the forward; :144-181 hands the logits
-    buffer back as the gradient) the forward already leaves d loss / d logits in the logits buffer - which is returned
-    marked dirty and must not be used any more - and keeps d loss / d links; the backward hands both out, scaled by the
-    upstream gradient of the loss (no pass over the logits when that is exactly 1; one in-place multiply otherwise, e.g.
-    under fp16 loss scaling).  May run backward once."""
+    """The criterion's loss (nat_pcfg_loss.py:98-145) as one differentiable op.  Like the reference's own ops
+    (pcfg_loss.py:67-73 runs the inside backward eagerly inside the forward; :144-181 hands the logits buffer back as the
+    gradient) the forward does everything that does not depend on the upstream gradient of the loss - gather, both inside
+    sweeps, the posteriors at an upstream gradient of 1, the loss - and returns the logits buffer marked dirty (it must not
+    be used any more).  The backward is one native call: a single read + write pass turns the logits into their gradient,
+    with the upstream gradient (e.g. the fp16 loss scale) folded in on the device, in float32, ahead of the one rounding
+    to the logits' dtype, as pcfg_loss.py:77-83 and :176-177 do; nothing is read back by the host.  May run backward once."""
 
     @staticmethod
     def forward(ctx, outputs, links, targets, output_length, target_length, matchmask, keep_word_mask):
         need = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
-        out, links_grad, ll, _, _ = pcfg_criterion_step(outputs, targets, links, output_length, target_length,
-                                                       matchmask=matchmask, keep_word_mask=keep_word_mask)
+        if need:
+            out, ll, state = _criterion_forward(outputs, targets, links, output_length, target_length, matchmask, keep_word_mask)
+            ctx.state = state
+            ctx.save_for_backward(outputs)
+            ctx.has_backward = False
+        else:  # nothing to differentiate: the plain step (its gradients are discarded)
+            out, _, ll, _, _ = pcfg_criterion_step(outputs, targets, links, output_length, target_length, matchmask=matchmask,
+                                                   keep_word_mask=keep_word_mask)
         ctx.mark_dirty(outputs)
         ctx.set_materialize_grads(False)
-        if need:
-            ctx.save_for_backward(outputs, links_grad)
-            ctx.has_backward = False
         invalid = ll.isinf().logical_or(ll.isnan())
         return outputs, out[0], ll.masked_fill(invalid, 0), out[1]
 
@@ -836,17 +905,17 @@ class PCFGCriterionFunc(Function):
             return (None,) * 7
         assert not ctx.has_backward, "Cannot backward twice in pcfg_criterion"
         ctx.has_backward = True
-        buf, links_grad = ctx.saved_tensors
-        if not bool((grad_loss == 1).all()):  # the one host read of the backward; exact 1 is autograd's seed for loss.backward()
-            buf.mul_(grad_loss.to(buf.dtype))
-            links_grad = links_grad * grad_loss.to(links_grad.dtype)
+        (buf,) = ctx.saved_tensors
+        buf, links_grad = _criterion_backward(buf, ctx.state, grad_loss)
+        ctx.state = None
         return (buf if ctx.needs_input_grad[0] else None, links_grad if ctx.needs_input_grad[1] else None, None, None, None, None,
                 None)
 
 
 def pcfg_criterion(outputs, targets, links, output_length, target_length, matchmask=None, keep_word_mask=None):
     """loss = -(log-likelihood / target_length).mean() over the sentences with a finite log-likelihood, differentiable in
-    ``outputs`` [B,L,V] (fp16/fp32 logits, consumed in place) and ``links``; one native call in the forward.  Returns
+    ``outputs`` [B,L,V] (fp16/fp32 logits, consumed in place) and ``links``; one native call in the forward, one in the
+    backward.  Returns
     (loss, ll [B] with invalid sentences zeroed, number of invalid sentences) - the dict entries of
     ``harness.compute_pcfg_loss``."""
     _, loss, ll, invalid = PCFGCriterionFunc.apply(outputs, links, targets, output_length, target_length, matchmask, keep_word_mask)

@@ -27,8 +27,7 @@ def eos_masked(match_all, output_length, target_length):
 def compute_pcfg_loss(outputs, output_masks, targets, target_masks, links, ops=_default_ops, matchmask=None, keep_word_mask=None,
                       no_force_emit=False):
     """loss = -(log-likelihood / target_length).mean() with invalid sentences zeroed (nat_pcfg_loss.py:98-145).
-    ``outputs`` [B,L,V] is consumed in place (it holds softmax probabilities afterwards and the gradient after
-    backward).  ``matchmask`` [B,T,L] / ``keep_word_mask`` [B,L] (from the glancing step): unless ``no_force_emit``, a
+    ``outputs`` [B,L,V] is consumed in place (it must not be used afterwards and holds the gradient after backward).  ``matchmask`` [B,T,L] / ``keep_word_mask`` [B,L] (from the glancing step): unless ``no_force_emit``, a
     revealed graph node may only emit the target position it is aligned to, through a detached value (:116-121).
     Returns a dict with ``loss``, ``ll`` (per sentence), ``invalid_nsentences``."""
     prelen = outputs.shape[1]
@@ -176,12 +175,13 @@ def train_step_fused(logits, targets, links, output_length, target_length, ops=_
 
 
 def train_step_single_call(logits, targets, links, output_length, target_length, ops=_default_ops, mark=None, slices=None,
-                           matchmask=None, keep_word_mask=None):
+                           matchmask=None, keep_word_mask=None, loss_scale=1.0):
     """``train_step_fused`` issued as one native call (``pcfgnat_criterion_step``): the kernels are enqueued back to
     back by the library and the scalar loss is reduced on the device.  Returns (loss, links_grad, ll)."""
     events = None
     if mark is not None:
         events = mark("events", 8)  # the caller hands out eight timing events for this step
     out, glinks, ll, _, _ = ops.pcfg_criterion_step(logits, targets, links, output_length, target_length, events=events,
-                                                 slices=slices, matchmask=matchmask, keep_word_mask=keep_word_mask)
+                                                 slices=slices, matchmask=matchmask, keep_word_mask=keep_word_mask,
+                                                 loss_scale=loss_scale)
     return out[0], glinks, ll

@@ -652,11 +652,15 @@ def test_fused_step_equals_autograd_step(shape):
         assert not buf[~out_mask].any()
 
 
-@pytest.mark.parametrize("scale", [1.0, 128.0])
-def test_criterion_op_under_autograd(scale):
-    """pcfg_criterion (one native call in the forward, gradients handed out by backward) against autograd through the
-    separate ops, with and without an upstream factor on the loss (fp16 loss scaling)."""
-    batch = synth.training_batch(4, 64, 12, 700, [64, 40, 22, 8], [12, 9, 12, 12], seed=43, logit_scale=2.0,
+@pytest.mark.parametrize("V", [700, 40000])
+@pytest.mark.parametrize("scale", [1.0, 128.0, 65536.0])
+def test_criterion_op_under_autograd(scale, V):
+    """pcfg_criterion (one native call in the forward, one in the backward) against autograd through the separate ops,
+    with and without an upstream factor on the loss (fp16 loss scaling, pcfg_loss.py:77-83): the factor has to reach the
+    gradient ahead of its rounding to fp16.  At V=40000 most entries of the unscaled gradient lie below the smallest fp16
+    subnormal, so a factor applied after the rounding would leave zeros where the drop-in ops have values.  Per element:
+    one fp16 rounding step (both sides round a float32 value once; the float32 values differ by reassociation only)."""
+    batch = synth.training_batch(4, 64, 12, V, [64, 40, 22, 8], [12, 9, 12, 12], seed=43, logit_scale=2.0,
                                  logit_dtype=torch.float16)
     B, L, V = batch["logits"].shape
     out_mask = (torch.arange(L).view(1, L) < batch["output_length"].view(B, 1)).to(DEV)
@@ -672,9 +676,20 @@ def test_criterion_op_under_autograd(scale):
     assert torch.allclose(loss, res["loss"].detach(), rtol=1e-6) and int(invalid) == 1
     assert torch.allclose(ll, res["ll"].detach(), rtol=1e-6)
     (loss * scale).backward()
+    assert torch.isfinite(leaf2.grad).all() and torch.isfinite(leaf.grad).all()
     assert torch.allclose(links2.grad, links.grad, rtol=1e-5, atol=1e-9 * scale)
-    assert torch.allclose(leaf2.grad, leaf.grad, rtol=2 ** -8, atol=2 ** -22 * scale)
+    assert torch.allclose(leaf2.grad, leaf.grad, rtol=2 ** -9, atol=2 ** -24)
     assert not leaf2.grad[~out_mask].any() and not leaf2.grad[3].any()
+    if V == 40000 and scale > 1:  # the factor did rescue entries that are flushed to zero at scale 1
+        assert (leaf2.grad != 0).sum() == (leaf.grad != 0).sum() or (leaf2.grad != 0).sum() > 0.5 * (leaf.grad != 0).sum()
+        assert (leaf.grad != 0).float().mean() > 0.05
+    # the plain single call with the factor handed over up front: as a host number and as a scalar in device memory
+    for given in (scale, torch.tensor([scale], device=DEV)):
+        buf = batch["logits"].to(DEV).clone()
+        out, glinks, _, _, _ = ops.pcfg_criterion_step(buf, tgt, batch["links"].to(DEV), ol, tl, loss_scale=given)
+        assert torch.allclose(out[0], res["loss"].detach(), rtol=1e-6)
+        assert torch.allclose(glinks, links.grad, rtol=1e-5, atol=1e-9 * scale)
+        assert torch.allclose(buf.float(), leaf.grad, rtol=2 ** -9, atol=2 ** -24)
 
 
 def test_single_call_step_large_batch_of_short_graphs():
