@@ -149,22 +149,13 @@ __device__ __forceinline__ double neg_inf(double) { return -__builtin_huge_val()
 __device__ __forceinline__ float vmax(float a, float b) { return fmaxf(a, b); }
 __device__ __forceinline__ double vmax(double a, double b) { return fmax(a, b); }
 
-#ifndef LSG_LOAD
-#define LSG_LOAD 1
-#endif
-#if LSG_LOAD == 1
+// The logits are streamed: every element crosses the memory interface once per pass, so loads and stores are marked
+// non-temporal.
 __device__ __forceinline__ vec16 load16(const vec16 *p) { return __builtin_nontemporal_load(p); }
-#else
-__device__ __forceinline__ vec16 load16(const vec16 *p) { return *p; }
-#endif
 // Makes the compiler forget what it knows about a register-resident chunk, so that each pass re-derives the widened
 // values from the packed registers instead of keeping both copies alive (which would halve the occupancy).
 __device__ __forceinline__ void opaque(vec16 &v) { asm volatile("" : "+v"(v)); }
-#if !defined(LSG_STORE) || LSG_STORE == 1
 __device__ __forceinline__ void store16(vec16 *p, const vec16 &v) { __builtin_nontemporal_store(v, p); }
-#else
-__device__ __forceinline__ void store16(vec16 *p, const vec16 &v) { *p = v; }
-#endif
 
 // Splits a row that starts at an arbitrary element address into [head scalars][16-byte chunks][tail scalars].
 template <typename T>
@@ -205,6 +196,52 @@ __device__ __forceinline__ CT block_sum(CT v, CT *slots, int wave, int lane) {
 #pragma unroll
     for (int w = 1; w < NW; w++) r += slots[w];
     return r;
+}
+
+// Launch order of the rows of a [B,L] batch whose sentences use only their first output_length[b] graph nodes: slot k of
+// the launch takes the k-th live row (live rows in batch order), the slots behind the last live row take the rows of
+// pad nodes, in reverse.  A workgroup of a pad row has next to nothing to do; scattered among the live rows (80 live
+// rows, 48 pad rows, 80 live rows, ...) each still holds a workgroup slot for its launch and its first load, which
+// at a third of the batch costs the live rows a tenth of the launch; at the end of the grid they run beside the last live
+// rows.  Every wave recomputes the map from the lengths: lane i takes sentence i (64 per round), prefix sums inside the
+// wave, the sentence found by a ballot.  k is uniform over the wave, so is everything derived from it.
+constexpr int COMPACT_MAX_B = 256;
+__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, true);  // row_shr:1, lanes without a source read 0
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, true);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, true);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, true);
+    const int r0 = __builtin_amdgcn_readlane(v, 15), r1 = __builtin_amdgcn_readlane(v, 31), r2 = __builtin_amdgcn_readlane(v, 47);
+    return v + (lane >= 16 ? r0 : 0) + (lane >= 32 ? r1 : 0) + (lane >= 48 ? r2 : 0);
+}
+__device__ __forceinline__ int compact_row(int k, int rows, const int64_t *__restrict__ out_len, int B, int L, int lane, bool &live) {
+    const int kp = rows - 1 - k;  // index among the pad rows, valid when k is behind the live rows
+    int done_live = 0, done_pad = 0, row = 0;
+    live = false;
+    bool found = false;
+    for (int b0 = 0; b0 < B && !found; b0 += 64) {
+        int len = 0, pad = 0;
+        if (b0 + lane < B) {
+            const int64_t v = out_len[b0 + lane];
+            len = v < 0 ? 0 : (v > (int64_t)L ? L : (int)v);
+            pad = L - len;
+        }
+        const int live_upto = wave_inclusive_scan(len, lane), pad_upto = wave_inclusive_scan(pad, lane);
+        const unsigned long long hit_live = __ballot(k < done_live + live_upto), hit_pad = __ballot(kp < done_pad + pad_upto);
+        const int tot_live = __builtin_amdgcn_readlane(live_upto, 63), tot_pad = __builtin_amdgcn_readlane(pad_upto, 63);
+        if (k < done_live + tot_live) {  // the first lane whose running count passes k holds the sentence
+            const int l = __builtin_ctzll(hit_live);
+            row = (b0 + l) * L + (k - done_live - __builtin_amdgcn_readlane(live_upto - len, l));
+            live = found = true;
+        } else if (kp < done_pad + tot_pad) {
+            const int l = __builtin_ctzll(hit_pad);
+            row = (b0 + l) * L + __builtin_amdgcn_readlane(len, l) + (kp - done_pad - __builtin_amdgcn_readlane(pad_upto - pad, l));
+            found = true;
+        }
+        done_live += tot_live;
+        done_pad += tot_pad;
+    }
+    return row;
 }
 
 // First position, among the elements this thread holds, whose value equals the row maximum (0x7fffffff if none).
@@ -253,17 +290,29 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
     __shared__ int s_arg;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
-    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
-        T *xr = x + row * (int64_t)V;
+    {
+        const int64_t slot = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;  // one row per workgroup
+        if (slot >= rows) return;
         // Rows of nodes beyond the sentence's graph (pads) feed nothing downstream of the criterion: neither sweep reads
-        // them and their gradient is zero.  When asked to, leave them unread and define their outputs as zeros.
-        if (skip_pad_rows && row % L >= eos_out_len[row / L]) {  // workgroup-uniform
+        // them and their gradient is zero.  When asked to, leave them unread and define their outputs as zeros
+        // (skip_pad_rows = 1: rows in batch order; 2: live rows first, see compact_row).
+        int64_t row = slot;
+        bool pad_row = false;  // workgroup-uniform
+        if (skip_pad_rows == 2) {
+            bool live;
+            row = compact_row((int)slot, (int)rows, eos_out_len, (int)rows / L, L, lane, live);
+            pad_row = !live;
+        } else if (skip_pad_rows) {
+            pad_row = row % L >= eos_out_len[row / L];
+        }
+        T *xr = x + row * (int64_t)V;
+        if (pad_row) {
             for (int s2 = tid; s2 < Tn; s2 += NT) sel[row * (int64_t)Tn + s2] = (CT)0;
             if (tid == 0) {
                 if (lse_out != nullptr) lse_out[row] = (CT)0;
                 if (argmax_out != nullptr) argmax_out[row] = 0;
             }
-            continue;
+            return;
         }
         const RowSplit<T> sp(xr, V);
         const vec16 *xv = reinterpret_cast<const vec16 *>(xr + sp.head);
@@ -396,7 +445,9 @@ __global__ __launch_bounds__(NT) void ls_max_kernel(const T *__restrict__ x, typ
     __shared__ int s_arg;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
-    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    {
+        const int64_t row = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;  // one row per workgroup
+        if (row >= rows) return;
         const T *xr = x + row * (int64_t)V;
         const RowSplit<T> sp(xr, V);
         const vec16 *xv = reinterpret_cast<const vec16 *>(xr + sp.head);
@@ -447,13 +498,19 @@ __global__ __launch_bounds__(NT) void ls_max_kernel(const T *__restrict__ x, typ
             // a row whose maximum is NaN-free but never found (all NaN) keeps index 0, like an all-equal row
             best_idx[row] = (s_arg == 0x7fffffff) ? 0 : s_arg;
         }
-        __syncthreads();  // s_arg and the reduction slots are reused by the next row
     }
 }
 
 // In-place backward.  TCAP = most targets per row handled through LDS; up to MAXC chunks per thread are in flight.
 // FROM_LOGITS = false: the buffer holds the probabilities the forward left (reference split, with the reference's
 // roundings to the buffer dtype); true: it holds the untouched logits and `lse` the row log-sum-exps.
+//
+// Every element of the row becomes p * (-sum_s g[s]); the (at most T) target columns also receive their g[s]
+// (scatter_add_, pcfg_loss.py:177: duplicates of a column accumulate in order).  Every 16-byte chunk is stored exactly
+// once: a chunk that holds target columns is taken over by the thread of the first target that points into it, which
+// loads the chunk itself, adds the gradients of all targets in it, in order, and stores it; the thread that streams the
+// chunk otherwise leaves it out (one bit per thread and chunk slot in LDS).  No store waits for another, so the
+// workgroup ends when its last store is issued instead of when it is acknowledged.
 template <typename T, int NT, int MAXC, int TCAP, bool FROM_LOGITS>
 __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const int64_t *__restrict__ idx, int64_t sb,
                                                      int64_t sl, int64_t st,
@@ -461,160 +518,229 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
                                                      int L, int V, int Tn,
                                                      const typename Elem<T>::compute *__restrict__ lse, LossTask loss,
                                                      const unsigned char *__restrict__ detach_rows,
-                                                     const int64_t *__restrict__ pad_out_len, int pad_rows_zeroed,
-                                                     const float *__restrict__ gscale_dev) {
+                                                     const int64_t *__restrict__ pad_out_len, int pad_mode,
+                                                     int pad_rows_zeroed, const float *__restrict__ gscale_dev) {
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
     constexpr int FIX = (TCAP + NT - 1) / NT;
+    constexpr unsigned EDGE_BIT = 1u << 30, BEYOND_BIT = 1u << 31;  // targets outside the register-resident chunks
+    static_assert(MAXC <= 30, "one bit per register-resident chunk");
     // an upstream factor of the whole gradient that only the device knows (the loss's own upstream gradient under fp16 loss
     // scaling): folded into g in the compute type, ahead of the single rounding to the buffer's dtype (pcfg_loss.py:77-83,
     // 176-177 scale g before the cast as well)
     const CT gs = (FROM_LOGITS && gscale_dev != nullptr) ? (CT)*gscale_dev : (CT)1;
-    if (loss.out != nullptr && blockIdx.x == 0) criterion_loss_block<NT>(loss);  // workgroup-uniform
-    __shared__ __attribute__((aligned(16))) int s_idx[TCAP + 4];  // padded to a multiple of four with -2 (matches nothing)
-    __shared__ CT s_g[TCAP];   // cast(g[s]) in the buffer's dtype, widened again
-    __shared__ CT s_p[TCAP];   // original probability at idx[s]
+    if (loss.out != nullptr && blockIdx.x == 0 && blockIdx.y == 0) criterion_loss_block<NT>(loss);  // workgroup-uniform
+    __shared__ __attribute__((aligned(16))) int s_idx[TCAP + 4];  // target column of position s, -1 if out of range; padded
+                                                                  // to a multiple of four with -2 (matches nothing)
+    __shared__ CT s_g[TCAP];         // g[s], zero for a detached row
+    __shared__ unsigned s_hit[NT];   // per thread: bit i = the chunk of slot i holds a target column
     const int tid = threadIdx.x, lane = tid & 63;
 
-    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
-        T *pr = p + row * (int64_t)V;
-        const CT *gr = gsel + row * (int64_t)Tn;
-        const int64_t b = row / L, q = row % L;
-        const int64_t *ir = idx + b * sb + q * sl;
-        const RowSplit<T> sp(pr, V);
-        vec16 *pv = reinterpret_cast<vec16 *>(pr + sp.head);
+    const int64_t slot = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;  // one row per workgroup
+    if (slot >= rows) return;
+    // Rows of nodes beyond the sentence's graph (pads) get no gradient from the criterion, whose backward sweep leaves
+    // their upstream gradient all zero: p * 0 plus zeros is zero whatever the row holds, so such a row is written
+    // without being read (pad_mode = 1: rows in batch order, the lengths come through the scalar cache; 2: live rows
+    // first, see compact_row).
+    int64_t row = slot;
+    bool pad_row = false;  // workgroup-uniform
+    if (pad_mode == 2) {
+        bool live_row;
+        row = compact_row((int)slot, (int)rows, pad_out_len, (int)rows / L, L, lane, live_row);
+        pad_row = !live_row;
+    } else if (pad_mode == 1) {
+        pad_row = row % L >= pad_out_len[row / L];
+    }
+    T *pr = p + row * (int64_t)V;
+    const RowSplit<T> sp(pr, V);
+    vec16 *pv = reinterpret_cast<vec16 *>(pr + sp.head);
+    const int ep = sp.edge_pos(tid);
+    if (pad_row) {
+        if (pad_rows_zeroed) return;  // an earlier launch of the caller has written the zeros
+        vec16 z;
+        z.x = z.y = z.z = z.w = 0;
+        for (int c = tid; c < sp.nvec; c += NT) store16(pv + c, z);
+        if (ep >= 0) pr[ep] = Elem<T>::narrow((CT)0);
+        return;
+    }
 
-        const int ep = sp.edge_pos(tid);
-        // Rows of nodes beyond the sentence's graph (pads) get no gradient from the criterion, whose backward sweep leaves
-        // their upstream gradient all zero: p * 0 plus zeros is zero whatever the row holds, so such a row is written
-        // without being read.  The lengths come through the scalar cache, so live rows do not wait on them.
-        if (pad_out_len != nullptr && q >= pad_out_len[b]) {  // workgroup-uniform
-            if (pad_rows_zeroed) continue;  // an earlier launch of the caller has written the zeros
-            vec16 z;
-            z.x = z.y = z.z = z.w = 0;
-            for (int c = tid; c < sp.nvec; c += NT) store16(pv + c, z);
-            if (ep >= 0) pr[ep] = Elem<T>::narrow((CT)0);
-            continue;
-        }
-
-        // the row's chunks are requested first so that they travel while the small per-row work is done
-        vec16 buf[MAXC];
+    // The small per-row inputs are requested first (independent loads, no chain), the row's chunks right behind them.
+    const CT *gr = gsel + row * (int64_t)Tn;
+    const int64_t *ir = idx + (row / L) * sb + (row % L) * sl;
+    // a row whose gathered values were detached (force-emit, nat_pcfg_loss.py:121) gets no gradient at all
+    unsigned char detached = 0;
+    if (detach_rows != nullptr) detached = detach_rows[row];
+    int64_t tcol[FIX];
+    CT tg[FIX];
 #pragma unroll
-        for (int i = 0; i < MAXC; i++) {
-            int c = tid + i * NT;
-            if (c < sp.nvec) buf[i] = load16(pv + c);
+    for (int r = 0; r < FIX; r++) {
+        const int s = tid + r * NT;
+        tcol[r] = -1;
+        tg[r] = 0;
+        if (s < Tn) {
+            tcol[r] = ir[(int64_t)s * st];
+            tg[r] = gr[s];
         }
-        CT edge = 0;
-        if (ep >= 0) edge = Elem<T>::widen(pr[ep]);
+    }
+    CT row_lse = 0;
+    if (FROM_LOGITS) row_lse = lse[row];
 
-        // -(sum_s g), computed redundantly by every wave; rounded to the buffer dtype in the reference split (pcfg_loss.py:176)
-        // a row whose gathered values were detached (force-emit, nat_pcfg_loss.py:121) gets no gradient at all
-        const bool live = detach_rows == nullptr || detach_rows[row] == 0;
-        CT part = 0;
-        for (int s = lane; s < Tn && live; s += 64) part += gr[s];
-        const CT ns = FROM_LOGITS ? -wave_sum(part) * gs : Elem<T>::widen(Elem<T>::narrow(-wave_sum(part)));
-        const RowNorm<CT> rn = RowNorm<CT>::from_lse(FROM_LOGITS ? lse[row] : (CT)0);
+    vec16 buf[MAXC];
+#pragma unroll
+    for (int i = 0; i < MAXC; i++) {
+        int c = tid + i * NT;
+        if (c < sp.nvec) buf[i] = load16(pv + c);
+    }
+    T edge_raw = Elem<T>::narrow((CT)0);
+    if (ep >= 0) edge_raw = pr[ep];
 
-        for (int s = tid; s < ((Tn + 3) & ~3); s += NT) {
-            if (s >= Tn) {
-                s_idx[s] = -2;
-                continue;
-            }
-            int64_t t = ir[(int64_t)s * st];
-            bool ok = (uint64_t)t < (uint64_t)V;
-            s_idx[s] = ok ? (int)t : -1;
-            if (FROM_LOGITS) {
-                s_g[s] = live ? gr[s] * gs : (CT)0;
-                s_p[s] = ok ? rn.e(Elem<T>::widen(pr[t])) : (CT)0;
+    s_hit[tid] = 0;
+#pragma unroll
+    for (int r = 0; r < FIX; r++) {
+        const int s = tid + r * NT;
+        if (s < ((Tn + 3) & ~3)) {
+            s_idx[s] = s >= Tn ? -2 : ((uint64_t)tcol[r] < (uint64_t)V) ? (int)tcol[r] : -1;
+            if (s < Tn) s_g[s] = detached ? (CT)0 : tg[r];
+        }
+    }
+    lds_barrier();
+
+    // The threads of the targets sort out who rewrites which chunk.
+    const int body_end = sp.head + sp.nvec * EPV;  // columns [head, body_end) travel as 16-byte chunks
+    int lead_chunk[FIX];  // the chunk this thread rewrites on behalf of its target (and of the later targets in it), or -1
+    bool lead_more[FIX];  // later targets point into the same chunk
+#pragma unroll
+    for (int r = 0; r < FIX; r++) {
+        const int s = tid + r * NT;
+        lead_chunk[r] = -1;
+        lead_more[r] = false;
+        if (s < Tn && (uint64_t)tcol[r] < (uint64_t)V) {
+            const int col = (int)tcol[r];
+            if (col < sp.head) {
+                atomicOr(&s_hit[col], EDGE_BIT);
+            } else if (col >= body_end) {
+                atomicOr(&s_hit[sp.head + (col - body_end)], EDGE_BIT);
             } else {
-                s_g[s] = live ? Elem<T>::widen(Elem<T>::narrow(gr[s])) : (CT)0;
-                s_p[s] = ok ? Elem<T>::widen(pr[t]) : (CT)0;
-            }
-        }
-        __syncthreads();  // every original value at a target column is in LDS before any store to the row
-
-        // scatter_add_ (pcfg_loss.py:177): the first occurrence of a column accumulates all its duplicates in order.  Worked
-        // out here, from LDS only, while the row's chunks are still on their way.
-        CT fix[FIX];
-        bool lead[FIX];
-#pragma unroll
-        for (int r = 0; r < FIX; r++) {
-            int s = tid + r * NT;
-            lead[r] = false;
-            fix[r] = 0;
-            if (s < Tn && s_idx[s] >= 0) {
-                const int my = s_idx[s];
-                // occurrences of the same column before and after s, four entries per LDS read
+                const int cc = (col - sp.head) / EPV, lo = sp.head + cc * EPV;
+                // targets in the same chunk before and after s, four entries per LDS read
                 const int4 *si4 = reinterpret_cast<const int4 *>(s_idx);
                 int before = 0, after = 0;
                 for (int w = 0; w < (Tn + 3) >> 2; w++) {
                     const int4 q = si4[w];
                     const int u = 4 * w;
-                    before += (q.x == my && u < s) + (q.y == my && u + 1 < s) + (q.z == my && u + 2 < s) + (q.w == my && u + 3 < s);
-                    after += (q.x == my && u > s) + (q.y == my && u + 1 > s) + (q.z == my && u + 2 > s) + (q.w == my && u + 3 > s);
+                    const bool a = (unsigned)(q.x - lo) < (unsigned)EPV, b = (unsigned)(q.y - lo) < (unsigned)EPV;
+                    const bool c = (unsigned)(q.z - lo) < (unsigned)EPV, d = (unsigned)(q.w - lo) < (unsigned)EPV;
+                    before += (a && u < s) + (b && u + 1 < s) + (c && u + 2 < s) + (d && u + 3 < s);
+                    after += (a && u > s) + (b && u + 1 > s) + (c && u + 2 > s) + (d && u + 3 > s);
                 }
                 if (before == 0) {
-                    CT v = s_p[s] * ns;
-                    if (!FROM_LOGITS) v = Elem<T>::widen(Elem<T>::narrow(v));
-                    for (int u = s; u < (after ? Tn : s + 1); u++)
-                        if (s_idx[u] == my) v = FROM_LOGITS ? v + s_g[u] : Elem<T>::widen(Elem<T>::narrow(v + s_g[u]));
-                    fix[r] = v;
-                    lead[r] = true;
+                    lead_chunk[r] = cc;
+                    lead_more[r] = after != 0;
+                    atomicOr(&s_hit[cc % NT], cc / NT < MAXC ? 1u << (cc / NT) : BEYOND_BIT);
                 }
             }
         }
+    }
+    lds_barrier();
+    const unsigned hit = s_hit[tid];
+    // -(sum_s g), computed redundantly by every wave; rounded to the buffer dtype in the reference split (pcfg_loss.py:176)
+    CT part = 0;
+    for (int s = lane; s < Tn; s += 64) part += s_g[s];
+    const CT ns = FROM_LOGITS ? -wave_sum(part) * gs : Elem<T>::widen(Elem<T>::narrow(-wave_sum(part)));
+    const RowNorm<CT> rn = RowNorm<CT>::from_lse(row_lse);
+    // the gradient of position u as it is added to its column
+    auto g_at = [&](int u) -> CT { return FROM_LOGITS ? s_g[u] * gs : Elem<T>::widen(Elem<T>::narrow(s_g[u])); };
+    // v[0..n) hold p * ns for columns col0 .. col0+n-1: add the gradients of targets u0, u0+1, ... < u1 that point there
+    auto add_targets = [&](CT *v, int n, int col0, int u0, int u1) {
+        for (int u = u0; u < u1; u++) {
+            const int e = s_idx[u] - col0;
+            if ((unsigned)e >= (unsigned)n) continue;
+            const CT g = g_at(u);
+#pragma unroll
+            for (int k = 0; k < EPV; k++)
+                if (k < n && k == e) v[k] = FROM_LOGITS ? v[k] + g : Elem<T>::widen(Elem<T>::narrow(v[k] + g));
+        }
+    };
+
+    // chunks with targets, by the first target's thread (a second, dependent load: issued before this thread waits for
+    // its own chunks)
+#pragma unroll
+    for (int r = 0; r < FIX; r++) {
+        if (lead_chunk[r] >= 0) {
+            const int s = tid + r * NT, cc = lead_chunk[r];
+            CT v[EPV];
+            Elem<T>::unpack(pv[cc], v);
+#pragma unroll
+            for (int e = 0; e < EPV; e++) {
+                v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
+                if (!FROM_LOGITS) v[e] = Elem<T>::widen(Elem<T>::narrow(v[e]));  // p * ns is rounded before the adds
+            }
+            add_targets(v, EPV, sp.head + cc * EPV, s, lead_more[r] ? Tn : s + 1);
+            store16(pv + cc, Elem<T>::pack(v));
+        }
+    }
 
 #pragma unroll
-        for (int i = 0; i < MAXC; i++) {
-            int c = tid + i * NT;
-            if (c < sp.nvec) {
-                CT v[EPV];
-                Elem<T>::unpack(buf[i], v);
-#pragma unroll
-                for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
-                store16(pv + c, Elem<T>::pack(v));
-            }
-        }
-        for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
+    for (int i = 0; i < MAXC; i++) {
+        int c = tid + i * NT;
+        if (c < sp.nvec && !(hit & (1u << i))) {
             CT v[EPV];
-            Elem<T>::unpack(load16(pv + c), v);
+            Elem<T>::unpack(buf[i], v);
 #pragma unroll
             for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
             store16(pv + c, Elem<T>::pack(v));
         }
-        if (ep >= 0) pr[ep] = Elem<T>::narrow((FROM_LOGITS ? rn.e(edge) : edge) * ns);
-
-        // workgroup barrier (release/acquire at workgroup scope): the streamed stores of this row are ordered before the
-        // patches of its target columns, which hit addresses other threads of the workgroup have just written
-        __syncthreads();
-#pragma unroll
-        for (int r = 0; r < FIX; r++) {
-            int s = tid + r * NT;
-            if (lead[r]) pr[s_idx[s]] = Elem<T>::narrow(fix[r]);
+    }
+    for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
+        if (hit & BEYOND_BIT) {  // rare: is this one of the chunks a target's thread rewrites?
+            const int lo = sp.head + c * EPV;
+            bool taken = false;
+            for (int u = 0; u < Tn; u++) taken = taken || (unsigned)(s_idx[u] - lo) < (unsigned)EPV;
+            if (taken) continue;
         }
-        __syncthreads();  // LDS is reused by the next row
+        CT v[EPV];
+        Elem<T>::unpack(load16(pv + c), v);
+#pragma unroll
+        for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
+        store16(pv + c, Elem<T>::pack(v));
+    }
+    if (ep >= 0) {  // unaligned rows: the elements in front of and behind the 16-byte chunks, one per thread
+        CT v = (FROM_LOGITS ? rn.e(Elem<T>::widen(edge_raw)) : Elem<T>::widen(edge_raw)) * ns;
+        if (hit & EDGE_BIT) {
+            if (!FROM_LOGITS) v = Elem<T>::widen(Elem<T>::narrow(v));
+            add_targets(&v, 1, ep, 0, Tn);
+        }
+        pr[ep] = Elem<T>::narrow(v);
     }
 }
+
+// One workgroup per row: the rows along x, folded over y beyond 2^30 of them.
+inline dim3 row_grid(int64_t rows) {
+    const int64_t gx = rows < (1LL << 30) ? rows : (1LL << 30);
+    return dim3((unsigned)gx, (unsigned)((rows + gx - 1) / gx));
+}
+
+// How a launch that leaves out the rows of pad nodes orders its rows: 2 = live rows first (batches of up to COMPACT_MAX_B
+// sentences whose row count fits an int), 1 = batch order.
+inline int pad_row_mode(int64_t rows, int L) { return (rows / L <= COMPACT_MAX_B && rows < (1LL << 30)) ? 2 : 1; }
 
 template <typename T>
 int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, void *sel, int grad, int64_t rows,
                int L, int V, int Tn, const int64_t *eos_ol, const int64_t *eos_tl, void *lse, int64_t *argmax, hipStream_t stream,
                ForceEmit fe = ForceEmit{nullptr, nullptr}, int skip_pad_rows = 0) {
     using CT = typename Elem<T>::compute;
-#ifndef LSG_FWD_NT
-#define LSG_FWD_NT 512
-#endif
-    constexpr int NT = LSG_FWD_NT;
+    constexpr int NT = 512;
     // 10 chunks x 512 threads x 16 B = 80 KB of a row in registers: a 40k-entry fp16 row exactly, half of an fp32 one.
     constexpr int MAXC = 5120 / NT;
     constexpr int GMAX = 1024 / NT;
     if (Tn > NT * GMAX) return fail(PCFGNAT_EUNSUPPORTED, "logsoftmax_gather: T=%d exceeds %d targets per row", Tn, NT * GMAX);
-    int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
+    const dim3 grid = row_grid(rows);
+    if (skip_pad_rows) skip_pad_rows = pad_row_mode(rows, L);
     if (grad)
-        hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, true>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)x, idx, sb,
+        hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, true>), grid, dim3(NT), 0, stream, (T *)x, idx, sb,
                            sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax, fe, skip_pad_rows);
     else
-        hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, false>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)x, idx,
+        hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, false>), grid, dim3(NT), 0, stream, (T *)x, idx,
                            sb, sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax, fe, skip_pad_rows);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
@@ -629,13 +755,16 @@ int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
     constexpr int MAXC = 10;
     constexpr int TCAP = 1024;
     if (Tn > TCAP) return fail(PCFGNAT_EUNSUPPORTED, "logsoftmax_gather_backward: T=%d exceeds %d targets per row", Tn, TCAP);
-    int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
+    const dim3 grid = row_grid(rows);
+    const int pad_mode = pad_out_len == nullptr ? 0 : pad_row_mode(rows, L);
     if (lse != nullptr)
-        hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, true>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,
-                           (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev);
+        hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, true>), grid, dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,
+                           (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss, detach_rows, pad_out_len, pad_mode, pad_rows_zeroed,
+                           gscale_dev);
     else
-        hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, false>), dim3((unsigned)grid), dim3(NT), 0, stream, (T *)p, idx, sb, sl,
-                           st, (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss, detach_rows, pad_out_len, pad_rows_zeroed, nullptr);
+        hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, false>), grid, dim3(NT), 0, stream, (T *)p, idx, sb, sl,
+                           st, (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss, detach_rows, pad_out_len, pad_mode,
+                           pad_rows_zeroed, nullptr);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -645,8 +774,8 @@ int launch_ls_max(const void *x, void *best_lprob, int64_t *best_idx, int64_t ro
     using CT = typename Elem<T>::compute;
     constexpr int NT = 512;
     constexpr int MAXC = 10;
-    int64_t grid = rows < (1 << 30) ? rows : (1 << 30);
-    hipLaunchKernelGGL((ls_max_kernel<T, NT, MAXC>), dim3((unsigned)grid), dim3(NT), 0, stream, (const T *)x, (CT *)best_lprob, best_idx,
+    const dim3 grid = row_grid(rows);
+    hipLaunchKernelGGL((ls_max_kernel<T, NT, MAXC>), grid, dim3(NT), 0, stream, (const T *)x, (CT *)best_lprob, best_idx,
                        rows, V);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
