@@ -23,6 +23,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the roofline kernel at this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled against a
 # plain device copy of known size; summary in profiles/lsg_cfg2_hbm_traffic_pmc.md.  None = not measured for this build.
 # (lsg_bwd: the single-call step at this batch's lengths - 3408 of 5120 rows read and written.)
+EVENT_EVERY = 4  # steps between two bracketed launches of the roofline kernel inside the timed region
 ROOFLINE_KERNEL = {"single": "lsg_bwd", "fused": "lsg_bwd", "unfused": "lsg_fwd"}
 ROOFLINE_KERNEL_NAME = {"lsg_bwd": "lsg_bwd_kernel<half, from logits>", "lsg_fwd": "lsg_fwd_kernel<half, grad>"}
 MEASURED_TRAFFIC_BYTES = {"lsg_bwd": 553.47e6, "lsg_fwd": None}
@@ -173,7 +174,7 @@ def glat_timing(logits, targets, links, out_len):
     return {"ms_per_call": start.elapsed_time(end) / reps}
 
 
-def operator_api_timing(bufs, targets, links, ol, tl, args, timed_windows):
+def operator_api_timing(bufs, targets, links, ol, tl, args, timed_windows, host_enqueue_ms):
     """One training pass through the five drop-in names, driven by the criterion's own code under autograd
     (``harness.compute_pcfg_loss`` restates nat_pcfg_loss.py:98-145 call for call) and ``loss.backward()``; with a loss
     scale of 128 on top, as under ``--fp16``.  The logits reach the criterion as the non-leaf output of an upstream layer,
@@ -209,6 +210,9 @@ def operator_api_timing(bufs, targets, links, ol, tl, args, timed_windows):
     res["sentences_per_s_median"] = B / (res["ms_per_step_median"] * 1e-3)
     scaled = timed_windows(lambda i: step(i, 128.0), windows=3)
     res["loss_scale_128_ms_per_step_median"] = scaled["ms_per_step_median"]
+    # These figures are bound by the host: the criterion's glue is some forty small torch kernels per step, and the host
+    # takes as long to enqueue a step as the step takes on the wall clock.
+    res["host_enqueue_ms_per_step"] = host_enqueue_ms(lambda i: step(i, 128.0))
     return res
 
 
@@ -343,8 +347,15 @@ def main():
     mode = "unfused" if args.unfused else args.step
     roof = ROOFLINE_KERNEL[mode]
 
+    sampled = {"step": 0}
+
     def mark(name, phase):
         if name == "events":  # single-call step: the library records the events we hand out around its kernels
+            # Inside the timed region the roofline kernel is bracketed in every fourth step only: a pair of timing events
+            # holds up the queue by about 20 us, a tenth of the step.
+            sampled["step"] += 1
+            if not detail["on"] and (sampled["step"] - 1) % EVENT_EVERY != 0:
+                return None
             evs = []
             for kernel in ("lsg_fwd", "inside_fwd", "inside_bwd", "lsg_bwd"):
                 for _ in range(2):
@@ -373,6 +384,7 @@ def main():
     for i in range(args.warmup):
         losses.append(step_fn(bufs[i], targets, links, ol, tl)[0])
     torch.cuda.synchronize()
+    sampled["step"] = 0
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for i in range(args.warmup, total):
@@ -389,12 +401,26 @@ def main():
             out[name] = sum(d) / len(d)
         return out
 
+    def fresh_logits():
+        for i in range(args.warmup, total):  # the path has overwritten the buffers with gradients
+            bufs[i].copy_(torch.randn(B, L, V, device=dev, dtype=torch.float32, generator=ggen).mul_(2))
+
+    def host_enqueue_ms(fn):
+        """Host time to enqueue one step of ``fn`` (no wait for the GPU inside the window)."""
+        fresh_logits()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.warmup, total):
+            fn(i)
+        t1 = time.perf_counter()
+        torch.cuda.synchronize()
+        return (t1 - t0) * 1e3 / args.steps
+
     def timed_windows(fn, windows=5):
         """ms per step of ``fn(i)`` over several windows of args.steps steps each; every window gets fresh logits."""
         per = []
         for _ in range(windows):
-            for i in range(args.warmup, total):  # fresh logits: the path has overwritten the buffers with gradients
-                bufs[i].copy_(torch.randn(B, L, V, device=dev, dtype=torch.float32, generator=ggen).mul_(2))
+            fresh_logits()
             s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
             s0.record()
@@ -408,6 +434,7 @@ def main():
                 "ms_per_step_min": per[0], "ms_per_step_max": per[-1]}
 
     kern_ms = averages()  # the roofline kernel only: measured inside the timed region
+    roof_launches = len(pairs[roof]) // 2
     # per-kernel detail from a separate instrumented pass over buffers that have already been consumed (same work:
     # every value is finite, the kernels do not branch on data)
     roof_in_region = kern_ms[roof]
@@ -457,7 +484,8 @@ def main():
         "roofline": {"bound": "hbm", "kernel": ROOFLINE_KERNEL_NAME[roof], "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": (traffic * B_timed / B) if traffic else None,
-                     "algorithmic_bytes": roof_bytes, "avg_ms": kern_ms[roof], "sentences_per_launch": B_timed,
+                     "algorithmic_bytes": roof_bytes, "avg_ms": kern_ms[roof], "launches_timed": roof_launches,
+                     "sentences_per_launch": B_timed,
                      "rows_per_launch": B_timed * L, "rows_read": live_rows if live_rows is not None else B_timed * L},
         "kernels_ms": kern_ms,
         "lsg_fwd_gbs": fwd_bytes / (kern_ms["lsg_fwd"] * 1e-3) / 1e9,
@@ -474,7 +502,7 @@ def main():
         result["single_call_scaled"] = sc
     # the drop-in path: the unchanged criterion code over the operator API under autograd (dag_logsoftmax_gather_inplace ->
     # eos mask -> cuda_pcfg_loss -> loss -> backward), which reads and rewrites every row (it is not told the lengths)
-    result["operator_api"] = operator_api_timing(bufs, targets, links, ol, tl, args, timed_windows)
+    result["operator_api"] = operator_api_timing(bufs, targets, links, ol, tl, args, timed_windows, host_enqueue_ms)
     if not args.no_decode:
         result["viterbi"] = decode_timing(dev)
         result["glat_alignment"] = glat_timing(torch.randn(B, L, V, device=dev, generator=ggen).mul_(2).half(), targets, links, ol)

@@ -12,7 +12,11 @@
  *     (thread-local).  Numerical failure (a sentence whose log-likelihood is -inf) is not an error.
  *   - B = batch, L = graph size (decoder positions), T = padded target length, V = vocabulary,
  *     ml = links.size(2) - 1 ("max_left"), Mc = (L-2)/(ml+1)+1 main-chain nodes, Lq = L/4.
- *   - all PCFG tables are float32, lengths are int64, like every caller in the reference.
+ *   - PCFG tables are float32 (the `_f64` entry points take float64 tables, which the reference also dispatches,
+ *     pcfg_loss.cu:395), lengths are int64, like every caller in the reference.
+ *   - state: the entry points keep nothing between calls except the two process-wide tuning settings of
+ *     pcfgnat_pipeline_config, a per-device cache of kernel attributes and, only for pcfgnat_criterion_step with
+ *     slices > 1, one helper stream per device (calls with slices > 1 must not overlap on one device).
  */
 #ifndef PCFG_NAT_HIP_H
 #define PCFG_NAT_HIP_H
@@ -166,11 +170,26 @@ int pcfgnat_pcfg_loss_forward_backward_static(const float *grad_output, const fl
  * workgroup per sentence otherwise.  pcfgnat_pcfg_loss_forward_backward runs the forward and the outside pipeline of a
  * sentence side by side in one launch while twice that number fits, one after the other otherwise.  A block that waits
  * for the one ahead of it for more than spin_limit rounds of polling
- * (default 2^20, about a second) gives the sentence up, and the one-workgroup sweep redoes it in the same call; results
+ * (default 2^15, some tens of milliseconds; the blocks of a sentence normally follow each other at about 2 us) gives the
+ * sentence up, and the one-workgroup sweep redoes it in the same call; results
  * are the same either way up to fp32 rounding.  max_workgroups = 0 switches the pipeline off; a negative argument leaves
- * that setting unchanged.  Process-wide, takes effect with the next call.
+ * that setting unchanged.  The two settings are process-wide (all threads, streams and devices), meant for tests and
+ * tuning, and take effect with the next call.
+ *
+ * Progress: the waits rely on the leading blocks of a sentence having the lower workgroup indices and on workgroups being
+ * started in index order, so that a block never waits for one that has not been started while it occupies the slot
+ * that block needs.  HIP does not promise that order; where it does not hold (or where another tenant keeps the leading
+ * block from running) the bounded wait expires and the sentence is redone, which costs time, never correctness.
  */
 void pcfgnat_pipeline_config(int max_workgroups, int spin_limit);
+
+/*
+ * No counterpart in the reference: diagnostic counters of that fallback since the library was loaded - inside sweeps
+ * (forward and outside counted apart) and single-call Viterbi decodes that the one-workgroup kernels redid because a
+ * pipelined sweep gave up.  Reads two device counters of the current device (synchronises with the device); reset != 0
+ * clears them.  A caller that sees them grow outside tests is paying the bounded wait on those calls.
+ */
+int pcfgnat_pipeline_redo_counts(unsigned long long *inside_sweeps, unsigned long long *viterbi_sentences, int reset);
 
 /*
  * No counterpart in the reference: a wait limit of its own for the outside pipeline where the two pipelines of a sentence

@@ -141,22 +141,27 @@ def inside_bwd(grad_out, S, C, match, links, out_len, tgt_len, dtype=np.float64)
     return mg, lg
 
 
-def best_tree(S, C, match, links, out_len, tgt_len, dtype=np.float64):
-    """pcfg_best_tree (pcfg_best_tree.cu:333-360) on given inside tables.  Returns tree [B,L] int64."""
+def best_tree(S, C, match, links, out_len, tgt_len, dtype=np.float64, return_margin=False):
+    """pcfg_best_tree (pcfg_best_tree.cu:333-360) on given inside tables.  Returns tree [B,L] int64; with
+    ``return_margin`` also a [B,3] array about the arg-max decisions of the trace: the smallest gap between the best and
+    the second-best candidate (0 = an exact tie, inf = no decision had two finite candidates), the number of exact ties,
+    the smallest gap that is not a tie."""
     sfx, _ = _sfx(dtype)
     B, L, T = match.shape
     ml = links.shape[2] - 1
     match, links, S, C = _c(match, dtype), _c(links, dtype), _c(S, dtype), _c(C, dtype)
     out_len, tgt_len = _c(out_len, np.int64), _c(tgt_len, np.int64)
     tree = np.empty((B, L), dtype=np.int64)
+    margin = np.empty((B, 3), dtype=dtype) if return_margin else None
     getattr(_lib(), "oracle_best_tree" + sfx)(_p(S), _p(C), _p(match), _p(links), _p(out_len), _p(tgt_len), _p(tree),
-                                               B, L, T, ml)
-    return tree
+                                               _p(margin) if return_margin else None, B, L, T, ml)
+    return (tree, margin) if return_margin else tree
 
 
-def viterbi(ob, links, out_len, dtype=np.float32):
+def viterbi(ob, links, out_len, dtype=np.float32, return_margin=False):
     """pcfg_viterbi (pcfg_viterbi.cu:272-301).  Returns (S [B,L,L//4], R, Lt, M [B,L,L//4] int64); the autograd
-    wrapper exposes scores = S[:,1,:] (pcfg_loss.py:136)."""
+    wrapper exposes scores = S[:,1,:] (pcfg_loss.py:136).  With ``return_margin`` a fifth value: the [B,3] margin
+    array of ``best_tree``, over all table entries."""
     sfx, _ = _sfx(dtype)
     B, L = ob.shape
     ml = links.shape[2] - 1
@@ -168,8 +173,10 @@ def viterbi(ob, links, out_len, dtype=np.float32):
     R = np.empty((B, L, Lq), dtype=np.int64)
     Lt = np.empty((B, L, Lq), dtype=np.int64)
     M = np.empty((B, L, Lq), dtype=np.int64)
-    getattr(_lib(), "oracle_viterbi" + sfx)(_p(ob), _p(links), _p(out_len), _p(S), _p(Cv), _p(R), _p(Lt), _p(M), B, L, ml)
-    return S, R, Lt, M
+    margin = np.empty((B, 3), dtype=dtype) if return_margin else None
+    getattr(_lib(), "oracle_viterbi" + sfx)(_p(ob), _p(links), _p(out_len), _p(S), _p(Cv), _p(R), _p(Lt), _p(M),
+                                             _p(margin) if return_margin else None, B, L, ml)
+    return (S, R, Lt, M, margin) if return_margin else (S, R, Lt, M)
 
 
 def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unreduced_tokens, left_tree_mask, pad_index):

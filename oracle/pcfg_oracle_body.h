@@ -314,15 +314,34 @@ void FN(oracle_inside_bwd)(const REAL *grad_out, const REAL *S, const REAL *C, c
  * calculate_C_kernel_trace (:239-301).  The 4-lane scan and the strict-'>' lane merge
  * (lane priority 0 > 2 > 1 > 3, :140-174) are reproduced so that exact ties resolve identically.
  * St/Ct: zero-filled mark tables shaped like S/C.  tree: [L] int64, filled with -1 (:220).
+ * min_margin (may be NULL; not part of the reference): three values about the arg-max decisions of the trace that had
+ * two finite candidates - [0] the smallest gap between the best and the second-best candidate (0 = exact tie, +inf = no
+ * such decision), [1] the number of exact ties, [2] the smallest gap that is not a tie: how far the chosen indices are
+ * from flipping under rounding, and how often only the scan order decides.
  * ------------------------------------------------------------------------------------------- */
+#define TRACK_MARGIN(t)                                \
+    do {                                               \
+        if ((t) > g1) { g2 = g1; g1 = (t); }           \
+        else if ((t) > g2) g2 = (t);                   \
+    } while (0)
+#define CLOSE_MARGIN()                                                                                   \
+    do {                                                                                                 \
+        if (min_margin && g2 > NEG_INF) {                                                                \
+            REAL gap_ = g1 - g2;                                                                         \
+            if (gap_ < min_margin[0]) min_margin[0] = gap_;                                              \
+            if (gap_ == 0) min_margin[1] += 1;                                                           \
+            else if (gap_ < min_margin[2]) min_margin[2] = gap_;                                         \
+        }                                                                                                \
+    } while (0)
 static void FN(best_tree_one)(const REAL *S, const REAL *C, const REAL *match, const REAL *links, int m, int n,
-                              unsigned char *St, unsigned char *Ct, int64_t *tree, int L, int T, int ml)
+                              unsigned char *St, unsigned char *Ct, int64_t *tree, int L, int T, int ml, REAL *min_margin)
 {
     const int Mc = (L - 2) / (ml + 1) + 1;
     const int Lc = L - Mc;
     memset(St, 0, (size_t)Mc * (T + 2));
     memset(Ct, 0, (size_t)Lc * (T + 2) * (ml + 2));
     for (int a = 0; a < L; a++) tree[a] = -1;
+    if (min_margin) { min_margin[0] = min_margin[2] = -NEG_INF; min_margin[1] = 0; }
     S_AT(St, 0, 0) = 1; /* :112-116 */
     for (int s = 0; s <= n; s++) { /* task index start-1, :94-119 */
         for (int a_id = 0; a_id < Mc; a_id++) {
@@ -331,6 +350,7 @@ static void FN(best_tree_one)(const REAL *S, const REAL *C, const REAL *match, c
             int b_start = a - ml < 1 ? 1 : a - ml;
             REAL lane_val[4];
             int lane_c[4], lane_j[4], lane_b[4];
+            REAL g1 = NEG_INF, g2 = NEG_INF;
             for (int x = 0; x < 4; x++) {
                 REAL maxval = NEG_INF;
                 int max_c = -1, max_j = 0, max_b = -1;
@@ -342,6 +362,7 @@ static void FN(best_tree_one)(const REAL *S, const REAL *C, const REAL *match, c
                             int b_id = LT_E2I(_b);
                             REAL t = LK(a, a - b, c) + S_AT(S, c_id, s + j + 1) + C_AT(C, b_id, s, j) + MA(a, s + j);
                             if (isnan(t)) t = NEG_INF;
+                            TRACK_MARGIN(t);
                             if (t > maxval) { maxval = t; max_c = c_id; max_j = j; max_b = b_id; }
                         }
                 }
@@ -356,6 +377,7 @@ static void FN(best_tree_one)(const REAL *S, const REAL *C, const REAL *match, c
                 C_AT(Ct, lane_b[0], s, lane_j[0]) = 1;
             }
             tree[a] = s + lane_j[0]; /* :182 */
+            CLOSE_MARGIN();
         }
     }
     if (ml == 0) return; /* :308 */
@@ -368,7 +390,7 @@ static void FN(best_tree_one)(const REAL *S, const REAL *C, const REAL *match, c
             for (int i = 0; i < n - gap - 1; i++) {
                 if (C_AT(Ct, a_id, i, gap) == 0) continue;
                 int max_j = 0, max_b = -1, max_c = -1;
-                REAL maxval = NEG_INF;
+                REAL maxval = NEG_INF, g1 = NEG_INF, g2 = NEG_INF;
                 for (int j = 0; j < gap; j++)
                     for (int b = b_start; b < a + 1; b++) {
                         int _b = b == a ? 0 : b;
@@ -377,9 +399,11 @@ static void FN(best_tree_one)(const REAL *S, const REAL *C, const REAL *match, c
                             int c_id = LT_E2I(c);
                             REAL t = LK(a, a - b, c) + C_AT(C, b_id, i, j) + C_AT(C, c_id, i + j + 1, gap - j - 1) + MA(a, i + j);
                             if (isnan(t)) t = NEG_INF;
+                            TRACK_MARGIN(t);
                             if (t > maxval) { maxval = t; max_j = j; max_b = b_id; max_c = c_id; }
                         }
                     }
+                CLOSE_MARGIN();
                 if (max_b != -1 && max_c != -1) {
                     C_AT(Ct, max_b, i, max_j) = 1;
                     C_AT(Ct, max_c, i + max_j + 1, gap - max_j - 1) = 1;
@@ -392,7 +416,7 @@ static void FN(best_tree_one)(const REAL *S, const REAL *C, const REAL *match, c
 
 /* pcfg_best_tree (pcfg_best_tree.cu:333-360). */
 void FN(oracle_best_tree)(const REAL *S, const REAL *C, const REAL *match, const REAL *links, const int64_t *out_len,
-                          const int64_t *tgt_len, int64_t *tree, int B, int L, int T, int ml)
+                          const int64_t *tgt_len, int64_t *tree, REAL *min_margin, int B, int L, int T, int ml)
 {
     const int Mc = (L - 2) / (ml + 1) + 1;
     const int Lc = L - Mc;
@@ -402,7 +426,7 @@ void FN(oracle_best_tree)(const REAL *S, const REAL *C, const REAL *match, const
         unsigned char *Ct = (unsigned char *)malloc((size_t)Lc * (T + 2) * (ml + 2));
         FN(best_tree_one)(S + (size_t)bt * Mc * (T + 2), C + (size_t)bt * Lc * (T + 2) * (ml + 2), match + (size_t)bt * L * T,
                           links + (size_t)bt * L * (ml + 1) * L, (int)out_len[bt], (int)tgt_len[bt], St, Ct,
-                          tree + (size_t)bt * L, L, T, ml);
+                          tree + (size_t)bt * L, L, T, ml, min_margin ? min_margin + 3 * bt : NULL);
         free(St);
         free(Ct);
     }
@@ -416,9 +440,10 @@ void FN(oracle_best_tree)(const REAL *S, const REAL *C, const REAL *match, const
  * reproducible bit for bit.
  * ------------------------------------------------------------------------------------------- */
 static void FN(viterbi_one)(const REAL *ob, const REAL *links, int m, REAL *S, REAL *Cv, int64_t *R, int64_t *Lt,
-                            int64_t *M, int L, int ml)
+                            int64_t *M, int L, int ml, REAL *min_margin)
 {
     const int Lq = L / 4;
+    if (min_margin) { min_margin[0] = min_margin[2] = -NEG_INF; min_margin[1] = 0; } /* as in best_tree_one, over every table entry */
 #define V_AT(t, a, l) (t)[(size_t)(a) * Lq + (l)]
     for (size_t i = 0; i < (size_t)L * Lq; i++) { S[i] = NEG_INF; Cv[i] = NEG_INF; R[i] = 0; Lt[i] = 0; M[i] = 0; }
     for (int a = 1; a < L; a++) { /* :196-205 */
@@ -431,7 +456,7 @@ static void FN(viterbi_one)(const REAL *ob, const REAL *links, int m, REAL *S, R
             if (!(a > 0 && a < m && (a % (ml + 1) != 1))) continue;
             int hi = ((a - 1) / (ml + 1) + 1) * (ml + 1) + 1;
             int b_start = a - ml < 1 ? 1 : a - ml;
-            REAL maxval = NEG_INF;
+            REAL maxval = NEG_INF, g1 = NEG_INF, g2 = NEG_INF;
             int max_b = 0, max_c = 0, max_j = 0;
             for (int j = 0; j < gap; j++)
                 for (int b = b_start; b < a + 1; b++) {
@@ -439,9 +464,11 @@ static void FN(viterbi_one)(const REAL *ob, const REAL *links, int m, REAL *S, R
                     for (int c = a + 1; c < hi && c < m; c++) {
                         REAL t = LK(a, a - b, c) + V_AT(Cv, _b, j) + V_AT(Cv, c, gap - j - 1) + ob[a];
                         if (isnan(t)) t = NEG_INF;
+                        TRACK_MARGIN(t);
                         if (t > maxval) { maxval = t; max_b = _b; max_c = c; max_j = j; }
                     }
                 }
+            CLOSE_MARGIN();
             if (!isinf(maxval)) {
                 V_AT(Cv, a, gap) = maxval; V_AT(R, a, gap) = max_c; V_AT(Lt, a, gap) = max_b; V_AT(M, a, gap) = max_j;
             }
@@ -454,6 +481,7 @@ static void FN(viterbi_one)(const REAL *ob, const REAL *links, int m, REAL *S, R
             int b_start = a - ml < 1 ? 1 : a - ml;
             REAL lane_val[4];
             int lane_c[4], lane_j[4], lane_b[4];
+            REAL g1 = NEG_INF, g2 = NEG_INF;
             for (int x = 0; x < 4; x++) {
                 REAL maxval = NEG_INF;
                 int max_b = 0, max_c = 0, max_j = 0;
@@ -465,6 +493,7 @@ static void FN(viterbi_one)(const REAL *ob, const REAL *links, int m, REAL *S, R
                             REAL sc = (len - j - 1 >= 0) ? V_AT(S, c, len - j - 1) : NEG_INF;
                             REAL t = LK(a, a - b, c) + V_AT(Cv, _b, j) + sc + ob[a]; /* :83 */
                             if (isnan(t)) t = NEG_INF;
+                            TRACK_MARGIN(t);
                             if (t > maxval) { maxval = t; max_b = _b; max_c = c; max_j = j; }
                         }
                 }
@@ -476,6 +505,7 @@ static void FN(viterbi_one)(const REAL *ob, const REAL *links, int m, REAL *S, R
             if (!isinf(lane_val[0])) { /* :125-131 */
                 V_AT(S, a, len) = lane_val[0]; V_AT(Lt, a, len) = lane_b[0]; V_AT(R, a, len) = lane_c[0]; V_AT(M, a, len) = lane_j[0];
             }
+            CLOSE_MARGIN();
         }
     }
 #undef V_AT
@@ -484,17 +514,19 @@ static void FN(viterbi_one)(const REAL *ob, const REAL *links, int m, REAL *S, R
 /* pcfg_viterbi (pcfg_viterbi.cu:272-301).  S: [B,L,Lq] (the wrapper returns row 1), Cv: scratch of the
  * same shape, R/Lt/M: [B,L,Lq] int64. */
 void FN(oracle_viterbi)(const REAL *ob, const REAL *links, const int64_t *out_len, REAL *S, REAL *Cv, int64_t *R, int64_t *Lt,
-                        int64_t *M, int B, int L, int ml)
+                        int64_t *M, REAL *min_margin, int B, int L, int ml)
 {
     const int Lq = L / 4;
 #pragma omp parallel for schedule(dynamic, 1)
     for (int bt = 0; bt < B; bt++) {
         size_t o = (size_t)bt * L * Lq;
         FN(viterbi_one)(ob + (size_t)bt * L, links + (size_t)bt * L * (ml + 1) * L, (int)out_len[bt], S + o, Cv + o, R + o, Lt + o,
-                        M + o, L, ml);
+                        M + o, L, ml, min_margin ? min_margin + 3 * bt : NULL);
     }
 }
 
+#undef TRACK_MARGIN
+#undef CLOSE_MARGIN
 #undef MC_I2E
 #undef MC_E2I
 #undef LT_I2E

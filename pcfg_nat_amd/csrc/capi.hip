@@ -2,11 +2,49 @@
 #include "common.hip.h"
 
 #include <mutex>
+#include <unordered_map>
 
 namespace pcfgnat {
 char *error_buffer() {
     static thread_local char buf[512] = {0};
     return buf;
+}
+}  // namespace pcfgnat
+
+namespace pcfgnat {
+namespace {
+constexpr int MAX_DEVICES_SEEN = 64;
+std::mutex g_device_facts_mutex;
+int g_compute_units[MAX_DEVICES_SEEN] = {0};
+std::unordered_map<const void *, size_t> g_dynamic_lds[MAX_DEVICES_SEEN];
+}  // namespace
+
+int device_compute_units() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES_SEEN) return 256;
+    std::lock_guard<std::mutex> lock(g_device_facts_mutex);
+    if (g_compute_units[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        g_compute_units[dev] = n;
+    }
+    return g_compute_units[dev];
+}
+
+int ensure_dynamic_lds(const void *kernel, size_t bytes) {
+    int dev = 0;
+    PCFGNAT_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES_SEEN) {  // beyond the table: set it every time
+        PCFGNAT_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+        return PCFGNAT_OK;
+    }
+    std::lock_guard<std::mutex> lock(g_device_facts_mutex);
+    size_t &have = g_dynamic_lds[dev][kernel];
+    if (bytes > have) {
+        PCFGNAT_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+        have = bytes;
+    }
+    return PCFGNAT_OK;
 }
 }  // namespace pcfgnat
 

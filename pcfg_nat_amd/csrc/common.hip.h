@@ -33,6 +33,18 @@ inline int fail(int code, const char *fmt, ...) {
         if (!(cond)) return ::pcfgnat::fail(PCFGNAT_EINVAL, __VA_ARGS__); \
     } while (0)
 
+// ---- per-device facts and settings, looked up once (capi.hip) ---------------------------------------------------
+// Compute units of the current device (hipDeviceAttributeMultiprocessorCount; 256 on MI355X, fewer on a partition).
+int device_compute_units();
+// Allows `kernel` to be launched with `bytes` of dynamic LDS on the current device.  The attribute is set once per
+// (device, kernel) and raised only when a larger size comes along, not on every launch.
+int ensure_dynamic_lds(const void *kernel, size_t bytes);
+#define PCFGNAT_DYNAMIC_LDS(kernel, bytes)                                                   \
+    do {                                                                                     \
+        int _rc = ::pcfgnat::ensure_dynamic_lds((const void *)(kernel), (size_t)(bytes));     \
+        if (_rc != PCFGNAT_OK) return _rc;                                                   \
+    } while (0)
+
 // ---- internal entry points shared between translation units ---------------------------------------------------
 // The criterion's own weights, used when grad_output is null: d(-(ll/n).mean() * factor)/d ll_b = -factor/(n_b * norm_B)
 // (nat_pcfg_loss.py:135, 139-140; pcfg_loss.py:77-83 for the upstream factor).  norm_B is passed apart from the batch size
@@ -101,6 +113,12 @@ int lsg_forward_lse_force(const void *logits, int dtype, const int64_t *targets,
 // bound on a block's wait for the one ahead of it, in rounds of polling
 int pipeline_max_workgroups();
 int pipeline_spin_limit();
+// Default bound of a block's wait: 2^15 rounds of a short sleep and one device-scope load, some tens of milliseconds -
+// a hundred times the lag of the last block of a sentence behind the first (the blocks of a sentence follow each other
+// at about 2 us per block), short enough for a sweep that cannot make progress to fall back without being noticed as a stall.
+#define PCFGNAT_DEFAULT_SPIN_LIMIT (1 << 15)
+// sentences redone by the one-workgroup Viterbi kernel after their pipelined sweep gave up (viterbi.hip)
+int viterbi_redo_count(unsigned long long *count, int reset);
 
 // General max_left (generic_ml.hip)
 size_t generic_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml);
@@ -128,6 +146,23 @@ constexpr int DPP_QUAD_XOR1 = 0xB1;  // quad_perm:[1,0,3,2]
 constexpr int DPP_QUAD_XOR2 = 0x4E;  // quad_perm:[2,3,0,1]
 constexpr int DPP_ROW_HALF_MIRROR = 0x141;
 constexpr int DPP_ROW_MIRROR = 0x140;
+
+// max(v, v of the partner lane) as one DPP instruction.  Written in assembly because fmaxf() on a value that comes out
+// of a DPP move (or an LDS load) is compiled to move + canonicalise + max, four instructions in loops that are bound by
+// instruction issue; the hardware max already quiets NaNs in the IEEE mode kernels run in.  The leading s_nop covers
+// the two wait states a DPP read needs after a VALU write of the same register, which the compiler does not track
+// through inline assembly; inputs must not come straight from a transcendental instruction (v_exp/v_log), same reason.
+#define PCFGNAT_DPP_MAX(name, ctrl)                                                                          \
+    __device__ __forceinline__ float name(float v) {                                                          \
+        float r;                                                                                              \
+        asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v)); \
+        return r;                                                                                             \
+    }
+PCFGNAT_DPP_MAX(dpp_max_xor1, "quad_perm:[1,0,3,2]")
+PCFGNAT_DPP_MAX(dpp_max_xor2, "quad_perm:[2,3,0,1]")
+PCFGNAT_DPP_MAX(dpp_max_half_mirror, "row_half_mirror")
+PCFGNAT_DPP_MAX(dpp_max_mirror, "row_mirror")
+#undef PCFGNAT_DPP_MAX
 
 // All 16 lanes of a DPP row end up with the row's maximum / sum.
 __device__ __forceinline__ float row16_max(float v) {
@@ -255,18 +290,5 @@ __device__ __forceinline__ void entry_store(unsigned *p, float v) {
     __hip_atomic_store(p, __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ bool gave_up(const int *flag) { return __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0; }
-
-// Phase timestamps for tuning builds only (-DPCFGNAT_PHASE_TIMING): thread 0 of workgroup 0 stores the 100 MHz wall clock.
-#ifdef PCFGNAT_PHASE_TIMING
-__device__ unsigned long long pcfgnat_phase_ts[32];
-#define PCFGNAT_PHASE(i)                                                                     \
-    do {                                                                                     \
-        if (blockIdx.x == 0 && threadIdx.x == 0) pcfgnat::pcfgnat_phase_ts[i] = wall_clock64(); \
-    } while (0)
-#else
-#define PCFGNAT_PHASE(i) \
-    do {                 \
-    } while (0)
-#endif
 
 }  // namespace pcfgnat

@@ -109,26 +109,14 @@ constexpr size_t LDS_BUDGET = 128 * 1024;  // of the 160 KB a gfx950 workgroup m
 constexpr float LOG2E_F = 1.4426950408889634f;
 constexpr double LN2_D = 0.6931471805599453094;
 
+// Diagnostic: sweeps (forward or outside, counted apart) that the one-workgroup kernels redid because the pipelined
+// sweep of the sentence gave up, since the library was loaded (pcfgnat_pipeline_redo_counts).
+__device__ unsigned long long g_inside_redone;
+
 __device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float lg2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float to_b2(float natural) { return sanitize(natural) * LOG2E_F; }
 
-// max(v, v of the partner lane) as one DPP instruction.  Written in assembly because fmaxf() on a value that comes out
-// of a DPP move (or an LDS load) is compiled to move + canonicalise + max, four instructions in loops that are bound by
-// instruction issue; the hardware max already quiets NaNs in the IEEE mode kernels run in.  The leading s_nop covers
-// the two wait states a DPP read needs after a VALU write of the same register, which the compiler does not track
-// through inline assembly; inputs must not come straight from a transcendental instruction (v_exp/v_log), same reason.
-#define PCFGNAT_DPP_MAX(name, ctrl)                                                                          \
-    __device__ __forceinline__ float name(float v) {                                                          \
-        float r;                                                                                              \
-        asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v)); \
-        return r;                                                                                             \
-    }
-PCFGNAT_DPP_MAX(dpp_max_xor1, "quad_perm:[1,0,3,2]")
-PCFGNAT_DPP_MAX(dpp_max_xor2, "quad_perm:[2,3,0,1]")
-PCFGNAT_DPP_MAX(dpp_max_half_mirror, "row_half_mirror")
-PCFGNAT_DPP_MAX(dpp_max_mirror, "row_mirror")
-#undef PCFGNAT_DPP_MAX
 
 __device__ __forceinline__ float row8_max(float v) {
     v = dpp_max_xor1(v);
@@ -324,7 +312,6 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
         return;
     }
     const int mc = m / 2;  // active main-chain nodes: a_id < mc
-    PCFGNAT_PHASE(0);
 
     // link slabs -> registers; the loads are unconditional (clamped addresses) so that they are all in flight together
     float A0[R][NQ], A1[R][NQ];
@@ -382,7 +369,6 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
         }
     }
     __syncthreads();
-    PCFGNAT_PHASE(1);
     FwdSweepArgs sa{col, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, av.F0, av.F1, av.SR, hd.slots, hd.D, hd.O, base_cell * LOG2E_F, n, mc, Mc, T, j, g8};
     switch (p) {  // wave-uniform: every wave runs the sweep specialised for its node block
         case 0: fwd_sweep<R, TAB_LDS, 0>(A0, A1, sa); break;
@@ -394,7 +380,6 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
         case 6: fwd_sweep<R, TAB_LDS, 6>(A0, A1, sa); break;
         default: fwd_sweep<R, TAB_LDS, 7>(A0, A1, sa); break;
     }
-    PCFGNAT_PHASE(2);
     if (TAB_LDS) {
         for (int i = tid; i < Mc * TS; i += NTR) {
             const int t = i - (i / TS) * TS;
@@ -409,7 +394,6 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
         av.D[i] = hd.D[i];
         if (i < TS) av.O[i] = hd.O[i];
     }
-    PCFGNAT_PHASE(3);
 }
 
 template <int R, bool TAB_LDS>
@@ -559,7 +543,6 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
     // a null grad_output selects the criterion's own weights: -factor/(n_b * norm_B), see Seed
     const float g = seed_weight(grad_out, b, n, seed);
 
-    PCFGNAT_PHASE(8);
     // links_grad is zero outside the cells the register accumulators own (written at the very end, after the barriers of
     // the sweep have ordered them behind this fill): clear the whole slab now, while the loads below are in flight
     {
@@ -638,7 +621,6 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
         if (TAB_LDS) sm_B[0] = beta00;
     }
     __syncthreads();
-    PCFGNAT_PHASE(9);
     BwdSweepArgs sa{w0, w1, sm_S, sm_B, sm_main, sm_leaf, mt, av.SR, av.BETA, hd.D, beta00, n, mc, Mc, T, j, g8};
     switch (p) {  // wave-uniform
         case 0: bwd_sweep<R, TAB_LDS, 0>(A0, A1, G0, G1, sa); break;
@@ -651,7 +633,6 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
         default: bwd_sweep<R, TAB_LDS, 7>(A0, A1, G0, G1, sa); break;
     }
     __syncthreads();  // BETA written by the group leaders is read by every thread below
-    PCFGNAT_PHASE(10);
 
     // rule posteriors -> links_grad (pcfg_loss_backward.cu:512-531); everything else in the slab is zero
 #pragma unroll
@@ -666,8 +647,6 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
             }
         }
     }
-    PCFGNAT_PHASE(11);
-    PCFGNAT_PHASE(12);
     // emission posteriors -> match_all_grad (pcfg_loss_backward.cu:348-382, 429-433)
     for (int i = tid; i < L * T; i += NTR) {
         const int x = i / T, s = i - x * T;
@@ -688,7 +667,6 @@ __global__ __launch_bounds__(NTR) void inside_bwd_ml1_kernel(const float *__rest
         }
         mg[i] = g * out;
     }
-    PCFGNAT_PHASE(13);
 }
 
 // Forward and backward in one launch, one workgroup per sentence (the single call's path where the paired sweeps further
@@ -1095,7 +1073,8 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
 
 // Workgroups per sentence that zero the rows of its pad nodes beside the sweeps (see PadFill).
 constexpr int PAD_WGS = 32;
-constexpr int PAD_MAX_SWEEP_WGS = 192;  // of the 256 compute units
+// The fill rides along while the sweeps take up no more than three quarters of the compute units (192 of 256 on MI355X).
+inline int pad_max_sweep_wgs() { return device_compute_units() * 3 / 4; }
 constexpr size_t PAD_EXCLUSIVE_LDS = 84 * 1024;  // more than half of the 160 KB of a gfx950 compute unit
 
 // Zeroes the bytes of rows [m_b, L) of sentence b - one contiguous span - as one of PAD_WGS workgroups: 16-byte
@@ -1535,7 +1514,10 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
                                                                   float *__restrict__ aux, int L, int T, int Mc, int MP,
                                                                   int only_flagged) {
     // only_flagged: run only for sentences whose pipelined sweep gave up (the flag was written by an earlier launch)
-    if (only_flagged && ExchangeView(aux, blockIdx.x, Mc, T).flags[FLAG_FWD] == 0) return;
+    if (only_flagged) {
+        if (ExchangeView(aux, blockIdx.x, Mc, T).flags[FLAG_FWD] == 0) return;
+        if (threadIdx.x == 0) atomicAdd(&g_inside_redone, 1ull);
+    }
     extern __shared__ float smem[];
     float *col = smem;               // [2][MP]
     float *f1prev = smem + 2 * MP;    // [MP]
@@ -1725,7 +1707,10 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
                                                                   const int64_t *__restrict__ out_len,
                                                                   const int64_t *__restrict__ tgt_len, int L, int T, int Mc, int MP,
                                                                   int only_flagged) {
-    if (only_flagged && ExchangeView(aux, blockIdx.x, Mc, T).flags[FLAG_BWD] == 0) return;
+    if (only_flagged) {
+        if (ExchangeView(aux, blockIdx.x, Mc, T).flags[FLAG_BWD] == 0) return;
+        if (threadIdx.x == 0) atomicAdd(&g_inside_redone, 1ull);
+    }
     extern __shared__ float smem[];
     float *w0 = smem;             // [2][MP]
     float *w1 = smem + 2 * MP;     // [2][MP]
@@ -2832,7 +2817,7 @@ __global__ __launch_bounds__(256) void criterion_loss_kernel(const float *__rest
 // and still 1.8x at 512 sentences (8192 workgroups: the blocks of a sentence are adjacent in dispatch order, leading
 // block first, so a block never waits for one that has not been started).  Both numbers can be changed through
 // pcfgnat_pipeline_config.
-std::atomic<int> g_pipeline_max_wg{1 << 20}, g_pipeline_spin_limit{1 << 20};
+std::atomic<int> g_pipeline_max_wg{1 << 20}, g_pipeline_spin_limit{PCFGNAT_DEFAULT_SPIN_LIMIT};
 std::atomic<int> g_pipeline_spin_limit_outside{-1};  // side-by-side launch only; negative: the common limit
 int pipeline_chunks(int B, int T, int Mc) {  // NQ, or 0 where the pipelined sweeps do not apply
     const int NQ = stream_mp(Mc) / 64, CL = 64 * NQ / NLP;
@@ -2848,17 +2833,17 @@ int launch_fwd_pipe(const float *match_all, const int64_t *ol, const int64_t *tl
         const int spin_out = g_pipeline_spin_limit_outside.load() >= 0 ? g_pipeline_spin_limit_outside.load() : g_pipeline_spin_limit.load();
         // while every block of both pipelines can have a compute unit of its own: claim more than half of a unit's LDS so
         // that no two blocks share one (and its instruction issue), and spread the outside sweep's collecting over four waves
-        const bool roomy = 2 * B * CL <= 256;
+        const bool roomy = 2 * B * CL <= device_compute_units();
         if (match_bytes <= LDS_BUDGET - 8192) {
             const size_t lds = (roomy && match_bytes < PAD_EXCLUSIVE_LDS) ? PAD_EXCLUSIVE_LDS : match_bytes;
             if (roomy) {
                 auto k = inside_both_ml1_pipe_kernel<NQ, true, 4>;
-                PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                PCFGNAT_DYNAMIC_LDS(k, lds);
                 hipLaunchKernelGGL(k, dim3(2 * B * CL), dim3(16 * NLP + 256), lds, stream, match_all, ol, tl, S, aux, L, T, Mc,
                                    g_pipeline_spin_limit.load(), spin_out, B * CL);
             } else {
                 auto k = inside_both_ml1_pipe_kernel<NQ, true, 1>;
-                PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                PCFGNAT_DYNAMIC_LDS(k, lds);
                 hipLaunchKernelGGL(k, dim3(2 * B * CL), dim3(NTP), lds, stream, match_all, ol, tl, S, aux, L, T, Mc,
                                    g_pipeline_spin_limit.load(), spin_out, B * CL);
             }
@@ -2866,15 +2851,15 @@ int launch_fwd_pipe(const float *match_all, const int64_t *ol, const int64_t *tl
             hipLaunchKernelGGL((inside_both_ml1_pipe_kernel<NQ, false, 1>), dim3(2 * B * CL), dim3(NTP), 0, stream, match_all, ol, tl, S, aux,
                                L, T, Mc, g_pipeline_spin_limit.load(), spin_out, B * CL);
         }
-    } else if (match_bytes <= LDS_BUDGET - 8192 && B * CL <= 256) {  // a compute unit per block: four collector waves
+    } else if (match_bytes <= LDS_BUDGET - 8192 && B * CL <= device_compute_units()) {  // a compute unit per block: four collector waves
         auto k = inside_fwd_ml1_pipe_kernel<NQ, true, 4>;
         const size_t lds = match_bytes < PAD_EXCLUSIVE_LDS ? PAD_EXCLUSIVE_LDS : match_bytes;
-        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        PCFGNAT_DYNAMIC_LDS(k, lds);
         hipLaunchKernelGGL(k, dim3(B * CL), dim3(16 * NLP + 256), lds, stream, match_all, ol, tl, S, aux, L, T, Mc,
                            g_pipeline_spin_limit.load());
     } else if (match_bytes <= LDS_BUDGET - 8192) {
         auto k = inside_fwd_ml1_pipe_kernel<NQ, true>;
-        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)match_bytes));
+        PCFGNAT_DYNAMIC_LDS(k, match_bytes);
         hipLaunchKernelGGL(k, dim3(B * CL), dim3(NTP), match_bytes, stream, match_all, ol, tl, S, aux, L, T, Mc,
                            g_pipeline_spin_limit.load());
     } else {
@@ -2895,7 +2880,7 @@ int launch_bwd_pipe(const float *S, float *aux, const float *match_all, const in
     const size_t base = (size_t)(T + 4) * sizeof(float), with_match = base + (size_t)2 * NLP * T * sizeof(float);
     if (with_match <= LDS_BUDGET - 8192) {
         auto k = inside_bwd_ml1_pipe_kernel<NQ, true>;
-        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_match));
+        PCFGNAT_DYNAMIC_LDS(k, with_match);
         hipLaunchKernelGGL(k, dim3(B * CL), dim3(NTP), with_match, stream, S, aux, match_all, ol, tl, L, T, Mc,
                            g_pipeline_spin_limit.load());
     } else {
@@ -2938,7 +2923,7 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
     if (with_match <= LDS_BUDGET) {
         auto k = inside_fwd_ml1_stream_kernel<true, 4>;
-        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_match));
+        PCFGNAT_DYNAMIC_LDS(k, with_match);
         hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_match, stream, match_all, links, ol, tl, S, aux, L, T, Mc, MP, only_flagged);
     } else {
         hipLaunchKernelGGL((inside_fwd_ml1_stream_kernel<false, 4>), dim3(B), dim3(NT), base, stream, match_all, links, ol, tl, S, aux, L,
@@ -2981,7 +2966,7 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
     // lanes per node: four while one pass covers all nodes; beyond that the outside sweep measured faster with eight
     if (with_match <= LDS_BUDGET) {
         auto k = Mc <= NT / 4 ? inside_bwd_ml1_stream_kernel<true, 4> : inside_bwd_ml1_stream_kernel<true, 8>;
-        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_match));
+        PCFGNAT_DYNAMIC_LDS(k, with_match);
         hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_match, stream, S, aux, match_all, ol, tl, L, T, Mc, MP, only_flagged);
     } else {
         auto k = Mc <= NT / 4 ? inside_bwd_ml1_stream_kernel<false, 4> : inside_bwd_ml1_stream_kernel<false, 8>;
@@ -3010,12 +2995,12 @@ int launch_fwd(const float *match_all, const float *links, const int64_t *ol, co
     const size_t with_tab = base + ((size_t)2 * Mc * T + (size_t)3 * Mc * (T + 2)) * sizeof(float);
     if (with_tab <= LDS_BUDGET) {
         auto k = inside_fwd_ml1_kernel<R, true>;
-        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_tab));
+        PCFGNAT_DYNAMIC_LDS(k, with_tab);
         hipLaunchKernelGGL(k, dim3(B), dim3(NTR), with_tab, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
     } else {
         auto k = inside_fwd_ml1_kernel<R, false>;
         PCFGNAT_REQUIRE(base <= LDS_BUDGET, "pcfg_loss: target length %d too large for the column offsets in LDS", T);
-        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)base));
+        PCFGNAT_DYNAMIC_LDS(k, base);
         hipLaunchKernelGGL(k, dim3(B), dim3(NTR), base, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
@@ -3029,12 +3014,12 @@ int launch_bwd(const float *go, const float *S, float *aux, const float *match_a
     const size_t with_tab = base + ((size_t)2 * Mc * T + (size_t)4 * Mc * (T + 2)) * sizeof(float);
     if (with_tab <= LDS_BUDGET) {
         auto k = inside_bwd_ml1_kernel<R, true>;
-        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_tab));
+        PCFGNAT_DYNAMIC_LDS(k, with_tab);
         hipLaunchKernelGGL(k, dim3(B), dim3(NTR), with_tab, stream, go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc, seed);
     } else {
         auto k = inside_bwd_ml1_kernel<R, false>;
         PCFGNAT_REQUIRE(base <= LDS_BUDGET, "pcfg_loss_backward: target length %d too large for the column offsets in LDS", T);
-        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)base));
+        PCFGNAT_DYNAMIC_LDS(k, base);
         hipLaunchKernelGGL(k, dim3(B), dim3(NTR), base, stream, go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc, seed);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
@@ -3054,17 +3039,15 @@ int launch_fused(const float *go, const float *match_all, const float *links, co
         const size_t comb_bytes = ((size_t)(T + 4) + (size_t)Mc * (T + 2) + (size_t)8 * (T + 2)) * sizeof(float);
         if (pair_bytes <= LDS_BUDGET && comb_bytes <= 64 * 1024 && L <= 128) {
             PCFGNAT_REQUIRE(((uintptr_t)aux & 7) == 0, "pcfg_loss_forward_backward: aux must be 8-byte aligned");
-            PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)inside_pair_ml1_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                  (int)pair_bytes));
+            PCFGNAT_DYNAMIC_LDS(inside_pair_ml1_kernel, pair_bytes);
             // the fill rides along only while the sweeps leave compute units free for it (the gather backward writes the
             // zeros itself otherwise)
-            const bool fill = pad.base != nullptr && pad.row_bytes > 0 && 2 * B <= PAD_MAX_SWEEP_WGS;
+            const bool fill = pad.base != nullptr && pad.row_bytes > 0 && 2 * B <= pad_max_sweep_wgs();
             // With the fill, every workgroup of the launch claims more than half of a compute unit's LDS, so that no fill
             // workgroup shares a compute unit (and its instruction issue) with a sweep.
             const size_t launch_bytes = (fill && pair_bytes < PAD_EXCLUSIVE_LDS) ? PAD_EXCLUSIVE_LDS : pair_bytes;
             if (launch_bytes != pair_bytes)
-                PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)inside_pair_ml1_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                      (int)launch_bytes));
+                PCFGNAT_DYNAMIC_LDS(inside_pair_ml1_kernel, launch_bytes);
             hipLaunchKernelGGL(inside_pair_ml1_kernel, dim3((2 + (fill ? PAD_WGS : 0)) * B), dim3(NTR), launch_bytes, stream, match_all,
                                links, ol, tl, S, aux, L, T, Mc, B, pad);
             PCFGNAT_HIP_CHECK(hipGetLastError());
@@ -3078,7 +3061,7 @@ int launch_fused(const float *go, const float *match_all, const float *links, co
     }
     if (need > LDS_BUDGET) return PCFGNAT_OK;
     auto k = inside_fused_ml1_kernel<R>;
-    PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)need));
+    PCFGNAT_DYNAMIC_LDS(k, need);
     hipLaunchKernelGGL(k, dim3(B), dim3(NTR), need, stream, go, match_all, links, ol, tl, S, mg, lg, L, T, Mc, seed);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     *done = true;
@@ -3109,6 +3092,16 @@ extern "C" void pcfgnat_pipeline_config(int max_workgroups, int spin_limit) {
 }
 
 extern "C" void pcfgnat_pipeline_outside_spin_limit(int spin_limit) { g_pipeline_spin_limit_outside.store(spin_limit); }
+
+extern "C" int pcfgnat_pipeline_redo_counts(unsigned long long *inside_sweeps, unsigned long long *viterbi_sentences, int reset) {
+    PCFGNAT_REQUIRE(inside_sweeps && viterbi_sentences, "pipeline_redo_counts: null pointer");
+    PCFGNAT_HIP_CHECK(hipMemcpyFromSymbol(inside_sweeps, HIP_SYMBOL(g_inside_redone), sizeof(*inside_sweeps)));
+    if (reset) {
+        const unsigned long long zero = 0;
+        PCFGNAT_HIP_CHECK(hipMemcpyToSymbol(HIP_SYMBOL(g_inside_redone), &zero, sizeof(zero)));
+    }
+    return viterbi_redo_count(viterbi_sentences, reset);
+}
 
 extern "C" size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml) {
     if (B <= 0 || L < 2 || T < 0 || ml < 0) return 0;
@@ -3277,12 +3270,12 @@ extern "C" int pcfgnat_pcfg_best_tree(const float *S, float *aux, const float *m
     const size_t with_links = tables + (size_t)2 * Mc * Mc * sizeof(float);
     if (with_links <= LDS_BUDGET) {
         auto k = best_tree_ml1_kernel<2>;
-        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)with_links));
+        PCFGNAT_DYNAMIC_LDS(k, with_links);
         hipLaunchKernelGGL(k, dim3((unsigned)B), dim3(BT_NT), with_links, (hipStream_t)stream, S, match_all, links, output_length,
                            target_length, tree, (int)L, (int)T, Mc);
     } else if (tables <= LDS_BUDGET) {
         auto k = best_tree_ml1_kernel<1>;
-        PCFGNAT_HIP_CHECK(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)tables));
+        PCFGNAT_DYNAMIC_LDS(k, tables);
         hipLaunchKernelGGL(k, dim3((unsigned)B), dim3(BT_NT), tables, (hipStream_t)stream, S, match_all, links, output_length,
                            target_length, tree, (int)L, (int)T, Mc);
     } else {

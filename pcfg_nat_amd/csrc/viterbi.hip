@@ -39,22 +39,13 @@ __device__ __forceinline__ void row16_argmax_step(float &best, int &key) {
 
 __device__ __forceinline__ float nan_to_ninf(float v) { return (v != v) ? NEG_INF_F : v; }
 
-// Row maximum with one DPP instruction per step (fmaxf() on a DPP result costs move + canonicalise + max).  The leading
-// s_nop covers the wait states a DPP read needs after a VALU write of its source, which the compiler does not track
-// through inline assembly.  Inputs are never NaN here.
-#define PCFGNAT_DPP_MAX(name, ctrl)                                                                          \
-    __device__ __forceinline__ float name(float v) {                                                          \
-        float r;                                                                                              \
-        asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v)); \
-        return r;                                                                                             \
-    }
-PCFGNAT_DPP_MAX(vit_max_xor1, "quad_perm:[1,0,3,2]")
-PCFGNAT_DPP_MAX(vit_max_xor2, "quad_perm:[2,3,0,1]")
-PCFGNAT_DPP_MAX(vit_max_half_mirror, "row_half_mirror")
-PCFGNAT_DPP_MAX(vit_max_mirror, "row_mirror")
-#undef PCFGNAT_DPP_MAX
+// Diagnostic: sentences whose pipelined sweep gave up and which the one-workgroup kernel therefore redid, since the library
+// was loaded (pcfgnat_pipeline_redo_counts).
+__device__ unsigned long long g_viterbi_redone;
+
+// Row maximum with one DPP instruction per step; inputs are never NaN here.
 __device__ __forceinline__ float row16_max_raw(float v) {
-    return vit_max_mirror(vit_max_half_mirror(vit_max_xor2(vit_max_xor1(v))));
+    return dpp_max_mirror(dpp_max_half_mirror(dpp_max_xor2(dpp_max_xor1(v))));
 }
 
 // Back-pointer accessors of the readout walk.  FullTraces: the reference's three int64 tables [L][Lq].
@@ -194,6 +185,7 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
     int *Wb = COMPACT ? dec.W + (size_t)b * rowsW * Lq : nullptr;
     const bool in_contract = !(m < 2 || m > L || (m % 2) != 0);
     const bool from_pipe = COMPACT && dec.pipe_flags != nullptr && dec.pipe_flags[b] == 0;  // workgroup-uniform
+    if (COMPACT && dec.pipe_flags != nullptr && !from_pipe && tid == 0) atomicAdd(&g_viterbi_redone, 1ull);
 
     if (COMPACT) {
         if (!from_pipe)
@@ -865,5 +857,14 @@ extern "C" int pcfgnat_viterbi_decoding_host(const int64_t *pred_length, const i
                                    stack, stack + L, (int)L, (int)Lq);
     }
     free(stack);
+    return PCFGNAT_OK;
+}
+
+int pcfgnat::viterbi_redo_count(unsigned long long *count, int reset) {
+    PCFGNAT_HIP_CHECK(hipMemcpyFromSymbol(count, HIP_SYMBOL(g_viterbi_redone), sizeof(*count)));
+    if (reset) {
+        const unsigned long long zero = 0;
+        PCFGNAT_HIP_CHECK(hipMemcpyToSymbol(HIP_SYMBOL(g_viterbi_redone), &zero, sizeof(zero)));
+    }
     return PCFGNAT_OK;
 }

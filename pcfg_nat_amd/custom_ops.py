@@ -8,6 +8,8 @@ contract; the arithmetic runs in hand-written HIP kernels for gfx950 reached thr
 ``libpcfg_nat_hip.so`` on the current HIP stream.  There is no CPU path: calling with CPU tensors (other than
 ``viterbi_decoding``, whose reference version is itself a host loop) raises.
 """
+import threading
+
 import torch
 from torch.autograd import Function
 
@@ -23,17 +25,31 @@ def get_pcfg_kernel():
     return _lib.load()
 
 
+DEFAULT_SPIN_LIMIT = 1 << 15  # PCFGNAT_DEFAULT_SPIN_LIMIT of the library
+
+
 def pipeline_config(max_workgroups=None, spin_limit=None, outside_spin_limit=None):
     """Tuning of the long-graph inside sweeps (no counterpart in the reference): graphs of 130..1026 nodes are swept by
     one workgroup per block of 16 main-chain nodes, pipelined, while the batch needs no more than ``max_workgroups`` of
     them (default 2**20; 0 = always one workgroup per sentence).  ``spin_limit`` bounds the wait of a block for the one
-    ahead of it (default 2**20 rounds of polling); a sentence whose blocks give up is redone by the one-workgroup sweep
-    in the same call.  ``outside_spin_limit``: a limit of its own for the outside pipeline where the two run side by
-    side (negative = the common one).  ``None`` leaves a setting as it is."""
+    ahead of it (default 2**15 rounds of polling, tens of milliseconds); a sentence whose blocks give up is redone by the
+    one-workgroup sweep in the same call.  ``outside_spin_limit``: a limit of its own for the outside pipeline where the
+    two run side by side (negative = the common one).  ``None`` leaves a setting as it is.  The settings are process-wide
+    (every thread, stream and device): for tests and tuning, not for per-call use."""
     lib = _lib.load()
     lib.pcfgnat_pipeline_config(-1 if max_workgroups is None else int(max_workgroups), -1 if spin_limit is None else int(spin_limit))
     if outside_spin_limit is not None:
         lib.pcfgnat_pipeline_outside_spin_limit(int(outside_spin_limit))
+
+
+def pipeline_redo_counts(reset=False):
+    """(inside sweeps, single-call Viterbi decodes) that the one-workgroup kernels had to redo on the current device
+    because a pipelined sweep gave up, since the library was loaded or the last reset.  Synchronises with the device."""
+    import ctypes
+    lib = _lib.load()
+    a, b = ctypes.c_ulonglong(0), ctypes.c_ulonglong(0)
+    _lib.check(lib.pcfgnat_pipeline_redo_counts(ctypes.byref(a), ctypes.byref(b), int(bool(reset))), lib)
+    return a.value, b.value
 
 
 def _stream(t):
@@ -478,18 +494,22 @@ def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unre
     if dev.type == "cuda":
         with torch.cuda.device(dev):
             scratch = torch.empty((B, 2 * L), dtype=torch.int64, device=dev)
-            cnt = _pinned_counts(dev, B)  # written by the kernel, read after the one stream wait
-            _lib.check(lib.pcfgnat_viterbi_decoding(pl.data_ptr(), ol.data_ptr(), Lt.data_ptr(), Rt.data_ptr(), Mt.data_ptr(),
-                                                    tok.data_ptr(), mask.data_ptr(), mask.size(0), int(pad_index),
-                                                    out.data_ptr(), cnt.data_ptr(), scratch.data_ptr(), B, L, Lq,
-                                                    _stream(out)), lib)
-            torch.cuda.current_stream(dev).synchronize()
+            cnt = _pinned_counts.take(B)  # written by the kernel, read after the one stream wait
+            try:
+                _lib.check(lib.pcfgnat_viterbi_decoding(pl.data_ptr(), ol.data_ptr(), Lt.data_ptr(), Rt.data_ptr(), Mt.data_ptr(),
+                                                        tok.data_ptr(), mask.data_ptr(), mask.size(0), int(pad_index),
+                                                        out.data_ptr(), cnt.data_ptr(), scratch.data_ptr(), B, L, Lq,
+                                                        _stream(out)), lib)
+                torch.cuda.current_stream(dev).synchronize()
+                counts = cnt[:B].tolist()
+            finally:
+                _pinned_counts.give_back(cnt)
     else:
         cnt = torch.empty((B,), dtype=torch.int64)
         _lib.check(lib.pcfgnat_viterbi_decoding_host(pl.data_ptr(), ol.data_ptr(), Lt.data_ptr(), Rt.data_ptr(),
                                                      Mt.data_ptr(), tok.data_ptr(), mask.data_ptr(), mask.size(0),
                                                      int(pad_index), out.data_ptr(), cnt.data_ptr(), B, L, Lq), lib)
-    counts = cnt.tolist()
+        counts = cnt.tolist()
     if B and min(counts) < 0:
         raise RuntimeError("viterbi_decoding: malformed traces")
     maxlen = max(counts) if B else 0
@@ -640,19 +660,30 @@ def _length_penalty(Lq, beta, device):
     return pen
 
 
-_PINNED_COUNTS = {}
+class _PinnedCounts:
+    """Pinned int64 host buffers for the per-sentence token counts of the decode calls.  Pinned host memory is addressable
+    from the device, so the kernels write the counts straight into it and the caller reads them after waiting for its
+    stream.  A call takes a buffer out of the pool for its own use and puts it back when it has read the counts: calls
+    that overlap (several host threads, several streams of one device) never share one.  Allocating pinned memory takes
+    about a hundred microseconds, hence the pool; it holds as many buffers as calls have ever overlapped."""
+
+    def __init__(self):
+        self._lock = threading.Lock()
+        self._free = []
+
+    def take(self, n):
+        with self._lock:
+            for i, buf in enumerate(self._free):
+                if buf.numel() >= n:
+                    return self._free.pop(i)
+        return torch.empty((max(n, 64),), dtype=torch.int64, pin_memory=True)
+
+    def give_back(self, buf):
+        with self._lock:
+            self._free.append(buf)
 
 
-def _pinned_counts(device, n):
-    """A pinned int64 host buffer of n entries per device, reused between calls (grown when a larger batch comes).  Pinned
-    host memory is addressable from the device, so the decode kernels write their per-sentence token counts straight
-    into it; the caller reads them after waiting for the stream (calls that overlap on one device would share it)."""
-    key = str(device)
-    buf = _PINNED_COUNTS.get(key)
-    if buf is None or buf.numel() < n:
-        buf = torch.empty((max(n, 64),), dtype=torch.int64, pin_memory=True)
-        _PINNED_COUNTS[key] = buf
-    return buf[:n]
+_pinned_counts = _PinnedCounts()
 
 
 def pcfg_viterbi_decode(unreduced_logits, links, output_length, unreduced_tokens, left_tree_mask, pad_index, beta=1.0):
@@ -688,12 +719,15 @@ def pcfg_viterbi_decode(unreduced_logits, links, output_length, unreduced_tokens
         base = block.data_ptr()
         # the emitted counts go straight into pinned host memory, which the device addresses like its own: the one
         # synchronisation of the decode is a stream wait, with no copy in front of it
-        host = _pinned_counts(dev, B)
-        _lib.check(lib.pcfgnat_viterbi_decode(ob.data_ptr(), links.data_ptr(), ol.data_ptr(), tok.data_ptr(), mask.data_ptr(),
-                                              mask.size(0), int(pad_index), pen.data_ptr(), base, base + 8 * nwork,
-                                              host.data_ptr(), base + 8 * (nwork + B * L), B, L, ml, _stream(ob)), lib)
-        torch.cuda.current_stream(dev).synchronize()
-    counts = host.tolist()
+        host = _pinned_counts.take(B)  # written by the kernel, read after the one stream wait
+        try:
+            _lib.check(lib.pcfgnat_viterbi_decode(ob.data_ptr(), links.data_ptr(), ol.data_ptr(), tok.data_ptr(), mask.data_ptr(),
+                                                  mask.size(0), int(pad_index), pen.data_ptr(), base, base + 8 * nwork,
+                                                  host.data_ptr(), base + 8 * (nwork + B * L), B, L, ml, _stream(ob)), lib)
+            torch.cuda.current_stream(dev).synchronize()
+            counts = host[:B].tolist()
+        finally:
+            _pinned_counts.give_back(host)
     if B and min(counts) < 0:
         raise RuntimeError("viterbi_decoding: malformed traces")
     maxlen = max(counts) if B else 0
@@ -729,12 +763,15 @@ def pcfg_lookahead_decode(links, unreduced_logits, unreduced_tokens, output_leng
     with torch.cuda.device(dev):
         idx = torch.empty((B, L), dtype=torch.int64, device=dev)
         out = torch.empty((B, L), dtype=torch.int64, device=dev)
-        cnt = _pinned_counts(dev, B)  # written by the kernel, read after the one stream wait
-        _lib.check(lib.pcfgnat_lookahead_decode(links.data_ptr(), ob_ptr, float(beta), ol.data_ptr(), tok.data_ptr(), mask.data_ptr(),
-                                                mask.size(0), int(pad_index), idx.data_ptr(), out.data_ptr(), cnt.data_ptr(), B, L,
-                                                K - 1, _stream(links)), lib)
-        torch.cuda.current_stream(dev).synchronize()
-    counts = cnt.tolist()
+        cnt = _pinned_counts.take(B)  # written by the kernel, read after the one stream wait
+        try:
+            _lib.check(lib.pcfgnat_lookahead_decode(links.data_ptr(), ob_ptr, float(beta), ol.data_ptr(), tok.data_ptr(),
+                                                    mask.data_ptr(), mask.size(0), int(pad_index), idx.data_ptr(), out.data_ptr(),
+                                                    cnt.data_ptr(), B, L, K - 1, _stream(links)), lib)
+            torch.cuda.current_stream(dev).synchronize()
+            counts = cnt[:B].tolist()
+        finally:
+            _pinned_counts.give_back(cnt)
     if B and min(counts) < 0:
         raise RuntimeError("pcfg_lookahead_decode: the walk does not terminate")
     maxlen = max(counts) if B else 0

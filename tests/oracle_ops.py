@@ -6,6 +6,33 @@ from torch.autograd import Function
 
 from oracle import oracle
 
+# What the oracle has met in its arg-max decisions since the last reset_margins(), per operator: [smallest gap between the
+# best and the second-best candidate (0 = an exact tie), number of exact ties, smallest gap that is not a tie] - how far
+# the bit-exact index comparisons sit from a rounding flip, and how often only the scan order decides.
+margins = {}
+
+
+def reset_margins():
+    margins["best_tree"] = [float("inf"), 0, float("inf")]
+    margins["viterbi"] = [float("inf"), 0, float("inf")]
+
+
+def _note(op, margin):
+    if len(margin):
+        m = margins[op]
+        m[0] = min(m[0], float(margin[:, 0].min()))
+        m[1] += int(margin[:, 1].sum())
+        m[2] = min(m[2], float(margin[:, 2].min()))
+
+
+def margin_text(op):
+    m = margins[op]
+    return "smallest arg-max margin %.3e, %d exact ties (decided by the scan order), smallest margin that is not a tie %.3e" % (
+        m[0], m[1], m[2])
+
+
+reset_margins()
+
 
 class _Loss(Function):
     @staticmethod
@@ -30,12 +57,15 @@ def cuda_pcfg_best_tree(match_all, links, output_length, target_length):
     m, lk = match_all.detach().double().numpy(), links.detach().double().numpy()
     ol, tl = output_length.numpy(), target_length.numpy()
     S, C = oracle.inside_fwd(m, lk, ol, tl)
-    tree = oracle.best_tree(S, C, m, lk, ol, tl)
+    tree, margin = oracle.best_tree(S, C, m, lk, ol, tl, return_margin=True)
+    _note("best_tree", margin)
     return torch.from_numpy(tree), torch.from_numpy(S[:, 0, 0].copy()).float()
 
 
 def cuda_pcfg_viterbi(ob_lprob, links, output_length):
-    S, R, Lt, M = oracle.viterbi(ob_lprob.numpy(), links.numpy(), output_length.numpy(), dtype=np.float32)
+    S, R, Lt, M, margin = oracle.viterbi(ob_lprob.numpy(), links.numpy(), output_length.numpy(), dtype=np.float32,
+                                         return_margin=True)
+    _note("viterbi", margin)
     return torch.from_numpy(S[:, 1, :].copy()), torch.from_numpy(R), torch.from_numpy(Lt), torch.from_numpy(M)
 
 

@@ -196,6 +196,12 @@ def _train_case(name):
         return synth.training_batch(3, 126, 96, 60, [126, 126, 70], [96, 2, 51], seed=19)
     if name == "L128_T104":  # just beyond: forward and outside sweeps as separate launches
         return synth.training_batch(2, 128, 104, 60, [128, 96], [104, 80], seed=20)
+    if name == "L130":  # 65 main-chain nodes: the first shape of the pipelined sweeps
+        return synth.training_batch(3, 130, 30, 100, [130, 128, 66], [30, 30, 17], seed=21)
+    if name == "L132":
+        return synth.training_batch(2, 132, 34, 100, [132, 130], [34, 29], seed=22)
+    if name == "L1028":  # 514 main-chain nodes: the first shape beyond the pipelined sweeps
+        return synth.training_batch(2, 1028, 16, 50, [1028, 1026], [16, 13], seed=23)
     if name == "L256":
         return synth.training_batch(3, 256, 40, 200, [256, 200, 130], [40, 33, 38], seed=12)
     if name == "L512":  # streaming kernels, emissions staged in LDS
@@ -217,7 +223,8 @@ def _match_for(batch):
     return harness.eos_masked(sel.float(), batch["output_length"], batch["target_length"])
 
 
-@pytest.mark.parametrize("case", ["cfg1", "wmt_small", "ragged_short", "L128_T100", "L126_T96", "L128_T104", "L256", "L320_mixed", "L512", "L512_long", "L1026", "L2050"])
+@pytest.mark.parametrize("case", ["cfg1", "wmt_small", "ragged_short", "L128_T100", "L126_T96", "L128_T104", "L130", "L132", "L256",
+                                  "L320_mixed", "L512", "L512_long", "L1026", "L1028", "L2050"])
 def test_inside_forward_backward_vs_oracle(case):
     batch = _train_case(case)
     match = _match_for(batch)
@@ -260,8 +267,11 @@ def _inside_all(batch, match):
 @pytest.mark.parametrize("L,T,ms,ns", [(200, 50, [200, 132, 164], [50, 30, 44]), (320, 40, [320, 262, 4], [40, 31, 2]),
                                        (512, 140, [512, 444], [140, 120]),
                                        (600, 24, [600, 520], [24, 24]), (1024, 30, [1024, 770, 900], [30, 22, 30]),
+                                       (130, 30, [130, 128, 66], [30, 30, 17]),
                                        # more blocks than compute units: the blocks share them (one collector wave each)
-                                       (200, 20, [200, 132, 164, 96] * 10, [20, 13, 17, 9] * 10)])
+                                       (200, 20, [200, 132, 164, 96] * 10, [20, 13, 17, 9] * 10),
+                                       # a large batch: 4096 blocks per pipeline, sixteen times the compute units
+                                       (512, 24, [512, 444, 386, 512] * 64, [24, 21, 24, 18] * 64)])
 def test_long_graph_sweeps_agree(mode, L, T, ms, ns):
     """Graphs of 130..1026 nodes: the two pipelined sweeps side by side (default), one after the other (a workgroup budget
     that holds one pipeline but not two), the one-workgroup streaming sweeps (pipeline switched off) and the redo path
@@ -269,21 +279,31 @@ def test_long_graph_sweeps_agree(mode, L, T, ms, ns):
     same tables; the default path is compared with the oracle in test_inside_forward_backward_vs_oracle."""
     batch = synth.training_batch(len(ms), L, T, 60, ms, ns, seed=L + T)
     match = _match_for(batch)
+    ops.pipeline_redo_counts(reset=True)
     ll0, mg0, lg0 = _inside_all(batch, match)
+    assert ops.pipeline_redo_counts()[0] == 0, "the pipelined sweeps of the default path gave up"
     try:
         if mode == "one_workgroup":
             ops.pipeline_config(max_workgroups=0)
         elif mode == "pipelines_in_turn":
             ops.pipeline_config(max_workgroups=len(ms) * 4 * ((L // 2 + 63) // 64))
         elif mode == "forward_gives_up":  # ... and is redone, while the outside pipeline beside it completes
-            ops.pipeline_config(spin_limit=0, outside_spin_limit=1 << 20)
+            ops.pipeline_config(spin_limit=0, outside_spin_limit=ops.DEFAULT_SPIN_LIMIT)
         elif mode == "outside_gives_up":
             ops.pipeline_config(outside_spin_limit=0)
         else:
             ops.pipeline_config(spin_limit=0)
         ll1, mg1, lg1 = _inside_all(batch, match)
     finally:
-        ops.pipeline_config(max_workgroups=1 << 20, spin_limit=1 << 20, outside_spin_limit=-1)
+        ops.pipeline_config(max_workgroups=1 << 20, spin_limit=ops.DEFAULT_SPIN_LIMIT, outside_spin_limit=-1)
+    # the fallback is visible in the diagnostic counter: every sweep of every sentence that ran as a pipeline and gave up
+    # (a block gives up only if it has to wait at all, so how many sentences are redone varies from run to run)
+    redone = ops.pipeline_redo_counts(reset=True)[0]
+    if mode in ("one_workgroup", "pipelines_in_turn"):
+        assert redone == 0, (mode, redone)
+    else:
+        most = len(ms) * (2 if mode == "blocks_give_up" else 1)
+        assert 0 < redone <= most, (mode, redone, most)
     fin = torch.isfinite(ll0)
     assert fin.any() and torch.equal(fin, torch.isfinite(ll1))
     assert torch.allclose(ll0[fin], ll1[fin], rtol=1e-5)
@@ -516,8 +536,47 @@ def test_single_call_decode_sweeps_agree(mode, case):
         got_tok, got_len = harness.viterbi_decode(ob.to(DEV), tok.to(DEV), links.to(DEV), ol.to(DEV), left_mask.to(DEV),
                                                   single_call=True)
     finally:
-        ops.pipeline_config(max_workgroups=1 << 20, spin_limit=1 << 20)
+        ops.pipeline_config(max_workgroups=1 << 20, spin_limit=ops.DEFAULT_SPIN_LIMIT)
     assert torch.equal(got_len.cpu(), want_len) and torch.equal(got_tok.cpu(), want_tok)
+
+
+def test_decodes_overlapping_on_one_device():
+    """Two host threads decode different batches on two streams of one device at the same time, many times over: every call
+    gets the token counts of its own batch (each call owns the pinned host buffer the kernel writes them to)."""
+    import threading
+    import oracle_ops
+    cases = []
+    for name in ("L96", "L160"):
+        batch = _decode_case(name)
+        ob, tok = synth.ob_and_tokens(batch["logits"])
+        links, ol = batch["links"], batch["output_length"]
+        mask = synth.support_masks(links.shape[1], 1)[0]
+        want = harness.viterbi_decode(ob, tok, links, ol, mask, ops=oracle_ops)
+        cases.append(([t.to(DEV) for t in (ob, tok, links, ol, mask)], want))
+    errors = []
+    start = threading.Barrier(2)
+
+    def worker(k):
+        try:
+            args, (want_tok, want_len) = cases[k]
+            stream = torch.cuda.Stream()
+            stream.wait_stream(torch.cuda.default_stream())
+            start.wait()
+            with torch.cuda.stream(stream):
+                for i in range(60):
+                    got_tok, got_len = harness.viterbi_decode(*args, single_call=(i % 2 == 0))
+                    if not (torch.equal(got_len.cpu(), want_len) and torch.equal(got_tok.cpu(), want_tok)):
+                        errors.append((k, i))
+        except Exception as e:  # noqa: BLE001 - reported below, in the main thread
+            errors.append((k, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
 
 
 @pytest.mark.parametrize("ml,L,ms", [(1, 32, [32, 20, 8]), (3, 34, [34, 26]), (1, 400, [400, 284, 20, 400]), (1, 18, [18])])

@@ -189,6 +189,46 @@ def test_viterbi_tie_order_is_lane_structured():
     assert right_child_of_root((4, 8, 12, 2, 6, 10, 14, 1, 5, 9, 13)) == 3
 
 
+def test_argmax_margins_hand_cases():
+    """The margins the oracle reports beside its traces: 0 where candidates tie exactly, the hand-derived gap where one
+    link is lifted above the others, inf where no decision has two finite candidates."""
+    L = m = 14
+    match, links = _uniform_case(L, m, 3)
+    ol, tl = np.array([m]), np.array([3])
+    S, C = oracle.inside_fwd(match, links, ol, tl)
+    _, margin = oracle.best_tree(S, C, match, links, ol, tl, return_margin=True)
+    assert margin[0, 0] == 0.0 and margin[0, 1] >= 1   # every child of the root ties
+    lk = links.copy()
+    lk[0, 1, 0, 7] = -0.25                       # root -> c_id 3 is now 0.75 better than its siblings
+    S, C = oracle.inside_fwd(match, lk, ol, tl)
+    tree, margin = oracle.best_tree(S, C, match, lk, ol, tl, return_margin=True)
+    assert tree[0, 7] == 1 and margin[0, 0] == 0.75 and margin[0, 1] == 0 and margin[0, 2] == 0.75   # node 7 -> last node: one candidate
+    # a chain with a single derivation: no decision has a runner-up
+    chain = np.full((1, L, 2, L), NINF)
+    for a in range(1, m - 1, 2):
+        chain[0, a, 0, a + 2] = -1.0
+    mt = np.full((1, L, 7), -1.0)
+    S, C = oracle.inside_fwd(mt, chain, ol, np.array([7]))
+    _, margin = oracle.best_tree(S, C, mt, chain, ol, np.array([7]), return_margin=True)
+    assert np.isposinf(margin[0, 0]) and margin[0, 1] == 0
+    # viterbi: the uniform graph ties everywhere
+    ob = np.full((1, 32), -1.0)
+    _, lk32 = _uniform_case(32, 32, 3)
+    *_, vm = oracle.viterbi(ob, lk32, np.array([32]), dtype=np.float32, return_margin=True)
+    assert vm[0, 0] == 0.0 and vm[0, 1] > 0
+    ch32 = np.full((1, 32, 2, 32), NINF)
+    for a in range(1, 31, 2):
+        ch32[0, a, 0, a + 2] = -1.0
+    *_, vm = oracle.viterbi(ob, ch32, np.array([32]), dtype=np.float64, return_margin=True)
+    assert np.isposinf(vm[0, 0])                 # a chain: one candidate per entry
+    # two ways from node 23 to the end in four tokens: 23 -> 25 -> 29 -> 31 (links -1, -1.5, -1) and 23 -> 27 -> 29 -> 31
+    # (-1.25, -1, -1): the second wins by 0.25, and no other entry has two candidates
+    ch32[0, 25, 0, 29] = -1.5
+    ch32[0, 23, 0, 27] = -1.25
+    S32, R32, _, _, vm = oracle.viterbi(ob, ch32, np.array([32]), dtype=np.float64, return_margin=True)
+    assert R32[0, 23, 4] == 27 and vm[0, 0] == 0.25 and vm[0, 1] == 0 and vm[0, 2] == 0.25
+
+
 # ---- lookahead / greedy decode (glat_decomposed_with_link_two_hands_tri_pcfg.py:419-481) -------------------------------
 
 def _inorder(node, length, idx, L, mask, tokens, pad, out):
