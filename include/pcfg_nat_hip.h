@@ -184,6 +184,14 @@ int pcfgnat_pcfg_loss_forward_backward_static(const float *grad_output, const fl
 void pcfgnat_pipeline_config(int max_workgroups, int spin_limit);
 
 /*
+ * No counterpart in the reference: the rule posteriors of graphs beyond 130 nodes are summed over the target positions on
+ * the matrix cores, as products of two factors per term; a 32x32 tile of (parent, child) pairs in which the product of
+ * the largest factors would exceed 2^log2_limit (default 120) is recomputed with one exponential per term instead,
+ * which has no range limit.  Process-wide, for tests: a limit of -inf sends every tile down the second path.
+ */
+void pcfgnat_links_grad_range_limit(float log2_limit);
+
+/*
  * No counterpart in the reference: diagnostic counters of that fallback since the library was loaded - inside sweeps
  * (forward and outside counted apart) and single-call Viterbi decodes that the one-workgroup kernels redid because a
  * pipelined sweep gave up.  Reads two device counters of the current device (synchronises with the device); reset != 0

@@ -2692,15 +2692,44 @@ __global__ __launch_bounds__(NTP) void inside_bwd_ml1_pipe_kernel(const float *_
     }
 }
 
-// Rule posteriors from the outside weights: lg[a][k][c] = g * sum_{t=1}^{n-1} exp(links[a][k][c] + Wk[a][t] + R[c][t]).
-// One block per 32x32 tile of (parent, child) pairs; the slab has been zero-filled beforehand.  use_corr: the outside
-// tables are relative to offsets of their own (sweeps side by side) and every column takes its correction corr_t.
-__global__ __launch_bounds__(1024) void links_grad_ml1_stream_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
-                                                                    const float *__restrict__ aux_c, const float *__restrict__ links,
-                                                                    const int64_t *__restrict__ out_len,
-                                                                    const int64_t *__restrict__ tgt_len, float *__restrict__ lgrad,
-                                                                    int L, int T, int Mc, Seed seed, int use_corr) {
-    __shared__ float sw0[32][33], sw1[32][33], ss[32][33];
+// Rule posteriors from the outside weights: lg[a][k][c] = g * sum_{t=1}^{n-1} exp(links[a][k][c] + Wk[a][t] + R[c][t]),
+// the one step of the path with operand reuse: per sentence and left option a [Mc,T] x [T,Mc] contraction, which as one
+// exponential per term is 9 M exponentials per sentence of 256 main-chain nodes and 140 target tokens.  Here the terms are
+// factored, 2^(A) * sum_t 2^(W_t[a] - u_t) * 2^(R_t[c] + corr_t + u_t), and the sum over t runs on the matrix cores in
+// fp32 (v_mfma_f32_32x32x2_f32): 0.6 M exponentials per sentence and 36 MFLOP.
+//
+// One workgroup of four waves per 32x32 tile of (parent, child) pairs with child tile >= parent tile.  The tile's rows
+// of the three tables (outside weights of both left options, inside scores) are brought into LDS as base-2 logarithms,
+// up to LG_SPAN target positions at a time and all loads of a span in flight together (the tables come from other
+// compute units' stores, microseconds away); each wave then takes a quarter of the positions: it exponentiates its
+// operands on the way from LDS to the matrix instruction and keeps a partial sum of the whole tile, the four partial
+// sums being added through LDS at the end.  Range: the tables vary by hundreds of units along t and along the nodes,
+// and only their sums are bounded (a posterior is at most 1).  Per position t the tile's largest outside weight wmax_t
+// and largest inside score rmax_t give E_t = wmax_t + rmax_t, and the shift u_t = (wmax_t - rmax_t) / 2 makes both
+// factors at most 2^(E_t / 2).  Where every pair of the tile is a rule (child tile behind the parent tile)
+// E_t + A <= 0, so nothing overflows and a term that underflows is worth less than 2^(-126 + E_t / 2 - A) of a
+// posterior.  In the tiles on the diagonal the two maxima may belong to a pair that is no rule and E_t grows with the
+// tile (which is why the tiles are 32 wide); a tile with E_t above range_limit (120 by default: factors below 2^60,
+// terms lost only below 2^-40 of a posterior for rules down to 2^-26) is recomputed by its workgroup as one exponential
+// per term, which is exact over the whole range (the log-domain form the sweeps use).
+// The slab has been zero-filled beforehand.  use_corr: the outside tables are relative to offsets of their own (sweeps
+// side by side) and every column takes its correction corr_t.  Dynamic LDS: 3 * 32 * (span + 1) + span floats, span = the
+// number of positions staged at a time (a multiple of 8, at most LG_SPAN).
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+constexpr int LG_TILE = 32, LG_SPAN = 256;
+inline int links_grad_span(int T) { return T - 1 >= LG_SPAN ? LG_SPAN : ((T - 1 + 7) / 8) * 8; }
+inline size_t links_grad_lds_bytes(int T) { return ((size_t)3 * LG_TILE * (links_grad_span(T) + 1) + links_grad_span(T)) * sizeof(float); }
+__global__ __launch_bounds__(256) void links_grad_ml1_stream_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
+                                                                   const float *__restrict__ aux_c, const float *__restrict__ links,
+                                                                   const int64_t *__restrict__ out_len,
+                                                                   const int64_t *__restrict__ tgt_len, float *__restrict__ lgrad,
+                                                                   int L, int T, int Mc, Seed seed, int use_corr, float range_limit,
+                                                                   int span) {
+    extern __shared__ float lg_lds[];
+    const int ld = span + 1;                 // row pitch: odd, so that a column of 32 rows falls into 32 banks
+    float *sw0 = lg_lds, *sw1 = sw0 + LG_TILE * ld, *ss = sw1 + LG_TILE * ld, *s_u = ss + LG_TILE * ld;  // [32][ld] x 3, [span]
+    __shared__ float s_part[3][64][17];  // partial sums of waves 1..3, one accumulator set at a time
+    __shared__ int s_bad;
     const int b = blockIdx.z, at = blockIdx.y, ct = blockIdx.x;
     if (ct < at) return;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
@@ -2708,48 +2737,160 @@ __global__ __launch_bounds__(1024) void links_grad_ml1_stream_kernel(const float
     const float ll = Sb[0];
     if (!(lengths_ok(m, n, L, T) && (ll == ll) && (fabsf(ll) != __builtin_huge_valf()))) return;
     const int mc = m / 2;
-    if (at * 32 >= mc || ct * 32 >= mc) return;
+    if (at * LG_TILE >= mc || ct * LG_TILE >= mc) return;
     AuxViewStream av(const_cast<float *>(aux_c), b, Mc, T);
     const float *corr = ExchangeView(const_cast<float *>(aux_c), b, Mc, T).corr;  // per column, when the sweeps ran side by side
     const float g = seed_weight(grad_out, b, n, seed);
-    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-    const int a_id = at * 32 + ty, c_id = ct * 32 + tx;
-    const int a = 2 * a_id + 1, c = 2 * c_id + 1;
-    const bool ok = a_id < mc && c_id < mc && a_id <= c_id;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const float *lk = links + (size_t)b * L * 2 * L;
-    const float A0 = ok ? to_b2(lk[((size_t)a * 2 + 0) * L + c]) : NEG_INF_F;
-    const float A1 = (ok && a_id >= 1) ? to_b2(lk[((size_t)a * 2 + 1) * L + c]) : NEG_INF_F;
-    float acc0 = 0.f, acc1 = 0.f;
-    // rows = nodes of the tile, columns = 32 consecutive target positions; the next chunk of the tables is requested before
-    // the current one is worked on (the tables come from other compute units' stores: microseconds away)
-    const int ra = at * 32 + ty, rc = ct * 32 + ty;
-    auto fetch = [&](int t0, float &f0, float &f1, float &fs) {
-        const int tt = t0 + tx;
-        const bool tin = tt <= n - 1;
-        f0 = (tin && ra < mc) ? av.W0[(size_t)ra * (T + 2) + tt] : NEG_INF_F;
-        f1 = (tin && ra < mc) ? av.W1[(size_t)ra * (T + 2) + tt] : NEG_INF_F;
-        fs = (tin && rc < mc) ? av.SR[(size_t)rc * (T + 2) + tt] + (use_corr ? corr[tt] : 0.f) : NEG_INF_F;
+    float *lg = lgrad + (size_t)b * L * 2 * L;
+    if (tid == 0) s_bad = 0;
+
+    // positions t1 .. t1 + span - 1 of the tile's rows into LDS (-inf beyond the sentence): thread (tx, ty) takes the positions
+    // tx, tx + 32, ... of the rows ty, ty + 8, ty + 16, ty + 24 of the three tables; every load of the span is issued before
+    // the first value is stored, so the span costs one trip to memory
+    const int tx = tid & 31, ty = tid >> 5;
+    auto stage = [&](int t1) {
+        float v0[LG_SPAN / 32][4], v1[LG_SPAN / 32][4], vs[LG_SPAN / 32][4];
+#pragma unroll
+        for (int q = 0; q < LG_SPAN / 32; q++) {
+            if (32 * q < span) {  // uniform
+                const int tt = t1 + 32 * q + tx;
+                const bool tin = tt <= n - 1;
+                const float cr = (tin && use_corr) ? corr[tt] : 0.f;
+#pragma unroll
+                for (int p = 0; p < 4; p++) {
+                    const int ra = at * LG_TILE + ty + 8 * p, rc = ct * LG_TILE + ty + 8 * p;
+                    v0[q][p] = (tin && ra < mc) ? av.W0[(size_t)ra * (T + 2) + tt] : NEG_INF_F;
+                    v1[q][p] = (tin && ra < mc) ? av.W1[(size_t)ra * (T + 2) + tt] : NEG_INF_F;
+                    vs[q][p] = (tin && rc < mc) ? av.SR[(size_t)rc * (T + 2) + tt] + cr : NEG_INF_F;
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < LG_SPAN / 32; q++) {
+            if (32 * q + tx < span) {
+#pragma unroll
+                for (int p = 0; p < 4; p++) {
+                    sw0[(ty + 8 * p) * ld + 32 * q + tx] = v0[q][p];
+                    sw1[(ty + 8 * p) * ld + 32 * q + tx] = v1[q][p];
+                    ss[(ty + 8 * p) * ld + 32 * q + tx] = vs[q][p];
+                }
+            }
+        }
     };
-    float f0, f1, fs;
-    fetch(1, f0, f1, fs);
-    for (int t0 = 1; t0 <= n - 1; t0 += 32) {
-        sw0[ty][tx] = f0;
-        sw1[ty][tx] = f1;
-        ss[ty][tx] = fs;
+
+    // ---- the contraction on the matrix cores
+    const int row = lane & 31, kk = lane >> 5;
+    floatx16 acc0, acc1;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc0[r] = acc1[r] = 0.f;
+    for (int t1 = 1; t1 <= n - 1; t1 += span) {
+        stage(t1);
         __syncthreads();
-        if (t0 + 32 <= n - 1) fetch(t0 + 32, f0, f1, fs);  // uniform
+        // per position: the largest outside weight of the tile's parents, the largest inside score of its children, the shift
+        for (int k = tid; k < span; k += 256) {
+            float wmax = NEG_INF_F, rmax = NEG_INF_F;
 #pragma unroll 8
-        for (int u = 0; u < 32; u++) {
-            const float sc = ss[tx][u];
-            acc0 += ex2((A0 + sw0[ty][u]) + sc);
-            acc1 += ex2((A1 + sw1[ty][u]) + sc);
+            for (int r = 0; r < LG_TILE; r++) {
+                wmax = fmaxf(wmax, fmaxf(sw0[r * ld + k], sw1[r * ld + k]));
+                rmax = fmaxf(rmax, ss[r * ld + k]);
+            }
+            const bool empty = wmax == NEG_INF_F || rmax == NEG_INF_F;  // no term at this position
+            if (!empty && !(wmax + rmax <= range_limit)) s_bad = 1;
+            s_u[k] = empty ? __builtin_nanf("") : 0.5f * (wmax - rmax);
+        }
+        __syncthreads();
+        const int live = min(span, n - t1);  // positions of this span inside the sentence (the rest holds -inf)
+        for (int k0 = 8 * wave; k0 < live; k0 += 32) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int k = k0 + 2 * j + kk;
+                // a position without a finite factor on one side contributes nothing, whatever the other side holds (it is
+                // not bounded there: 0 * inf must not reach the accumulators)
+                const float u = s_u[k];
+                const bool none = !(u == u);
+                const float y = none ? 0.f : ex2(ss[row * ld + k] + u);
+                const float x0 = none ? 0.f : ex2(sw0[row * ld + k] - u), x1 = none ? 0.f : ex2(sw1[row * ld + k] - u);
+                acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x0, y, acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(x1, y, acc1, 0, 0, 0);
+            }
         }
         __syncthreads();
     }
-    if (ok) {
-        float *lg = lgrad + (size_t)b * L * 2 * L;
-        lg[((size_t)a * 2 + 0) * L + c] = (acc0 == acc0) ? g * acc0 : 0.f;
-        lg[((size_t)a * 2 + 1) * L + c] = (acc1 == acc1) ? g * acc1 : 0.f;
+    if (!s_bad) {  // uniform: last written before the barrier that ends the loop (or never)
+        // the four partial sums, one accumulator set at a time: waves 1..3 hand theirs to wave 0
+#pragma unroll
+        for (int set = 0; set < 2; set++) {
+            if (wave > 0) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) s_part[wave - 1][lane][r] = set == 0 ? acc0[r] : acc1[r];
+            }
+            __syncthreads();
+            if (wave == 0) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const float add = (s_part[0][lane][r] + s_part[1][lane][r]) + s_part[2][lane][r];
+                    if (set == 0) acc0[r] += add;
+                    else acc1[r] += add;
+                }
+            }
+            __syncthreads();
+        }
+        if (wave != 0) return;
+        // accumulator r of lane l: row (r % 4) + 4 * (l / 32) + 8 * (r / 4), column l % 32 of the tile
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int a_id = at * LG_TILE + (r & 3) + 4 * kk + 8 * (r >> 2), c_id = ct * LG_TILE + row;
+            if (a_id < mc && c_id < mc && a_id <= c_id) {
+                const int a = 2 * a_id + 1, c = 2 * c_id + 1;
+                const float A0 = to_b2(lk[((size_t)a * 2 + 0) * L + c]);
+                const float A1 = a_id >= 1 ? to_b2(lk[((size_t)a * 2 + 1) * L + c]) : NEG_INF_F;
+                const float v0 = ex2(A0) * acc0[r], v1 = ex2(A1) * acc1[r];
+                lg[((size_t)a * 2 + 0) * L + c] = (v0 == v0) ? g * v0 : 0.f;
+                lg[((size_t)a * 2 + 1) * L + c] = (v1 == v1) ? g * v1 : 0.f;
+            }
+        }
+        return;
+    }
+
+    // ---- a factor left the range: the tile again, one exponential per term (four pairs per thread)
+    float A0[4], A1[4], e0[4], e1[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int a_id = at * LG_TILE + ty + 8 * q, c_id = ct * LG_TILE + tx;
+        const bool ok = a_id < mc && c_id < mc && a_id <= c_id;
+        const int a = 2 * a_id + 1, c = 2 * c_id + 1;
+        A0[q] = ok ? to_b2(lk[((size_t)a * 2 + 0) * L + c]) : NEG_INF_F;
+        A1[q] = (ok && a_id >= 1) ? to_b2(lk[((size_t)a * 2 + 1) * L + c]) : NEG_INF_F;
+        e0[q] = e1[q] = 0.f;
+    }
+    for (int t1 = 1; t1 <= n - 1; t1 += span) {
+        if (t1 + span <= n - 1 || t1 > 1) {  // (a single span is still in LDS)
+            __syncthreads();
+            stage(t1);
+            __syncthreads();
+        }
+        const int live = min(span, n - t1);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const int i = ty + 8 * q;
+#pragma unroll 4
+            for (int u = 0; u < live; u++) {
+                const float sc = ss[tx * ld + u];
+                e0[q] += ex2((A0[q] + sw0[i * ld + u]) + sc);
+                e1[q] += ex2((A1[q] + sw1[i * ld + u]) + sc);
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int a_id = at * LG_TILE + ty + 8 * q, c_id = ct * LG_TILE + tx;
+        if (a_id < mc && c_id < mc && a_id <= c_id) {
+            const int a = 2 * a_id + 1, c = 2 * c_id + 1;
+            lg[((size_t)a * 2 + 0) * L + c] = (e0[q] == e0[q]) ? g * e0[q] : 0.f;
+            lg[((size_t)a * 2 + 1) * L + c] = (e1[q] == e1[q]) ? g * e1[q] : 0.f;
+        }
     }
 }
 
@@ -2819,6 +2960,9 @@ __global__ __launch_bounds__(256) void criterion_loss_kernel(const float *__rest
 // pcfgnat_pipeline_config.
 std::atomic<int> g_pipeline_max_wg{1 << 20}, g_pipeline_spin_limit{PCFGNAT_DEFAULT_SPIN_LIMIT};
 std::atomic<int> g_pipeline_spin_limit_outside{-1};  // side-by-side launch only; negative: the common limit
+// Largest base-2 exponent a factor of the rule posteriors of long graphs may have on the matrix cores (see
+// links_grad_ml1_stream_kernel); a tile beyond it is recomputed term by term.  pcfgnat_links_grad_range_limit.
+std::atomic<float> g_links_grad_range_limit{120.f};
 int pipeline_chunks(int B, int T, int Mc) {  // NQ, or 0 where the pipelined sweeps do not apply
     const int NQ = stream_mp(Mc) / 64, CL = 64 * NQ / NLP;
     return (NQ >= 2 && NQ <= 8 && T + 2 < 4096 && (int64_t)B * CL <= g_pipeline_max_wg.load()) ? NQ : 0;
@@ -2945,7 +3089,7 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
                       const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, Seed seed, hipStream_t stream,
                       bool side_by_side = false, bool slabs_zeroed = false) {
     const int MP = stream_mp(Mc);
-    const int tiles = (Mc + 31) / 32;
+    const int tiles = (Mc + LG_TILE - 1) / LG_TILE;
     PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss_backward: aux must be 16-byte aligned");
     const size_t base = ((size_t)5 * MP + T + 4) * sizeof(float);
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
@@ -2979,8 +3123,9 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
         PCFGNAT_HIP_CHECK(hipGetLastError());
     }
     const int use_corr = side_by_side ? 1 : 0;
-    hipLaunchKernelGGL(links_grad_ml1_stream_kernel, dim3(tiles, tiles, B), dim3(1024), 0, stream, go, S, aux, links, ol, tl, lg, L, T, Mc,
-                       seed, use_corr);
+    PCFGNAT_DYNAMIC_LDS(links_grad_ml1_stream_kernel, links_grad_lds_bytes(T));
+    hipLaunchKernelGGL(links_grad_ml1_stream_kernel, dim3(tiles, tiles, B), dim3(256), links_grad_lds_bytes(T), stream, go, S, aux, links,
+                       ol, tl, lg, L, T, Mc, seed, use_corr, g_links_grad_range_limit.load(), links_grad_span(T));
     PCFGNAT_HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL(match_grad_ml1_stream_kernel, dim3((L * T + 255) / 256, B), dim3(256), 0, stream, go, S, aux, match_all, ol, tl, mg, L,
                        T, Mc, seed, use_corr);
@@ -3092,6 +3237,8 @@ extern "C" void pcfgnat_pipeline_config(int max_workgroups, int spin_limit) {
 }
 
 extern "C" void pcfgnat_pipeline_outside_spin_limit(int spin_limit) { g_pipeline_spin_limit_outside.store(spin_limit); }
+
+extern "C" void pcfgnat_links_grad_range_limit(float log2_limit) { g_links_grad_range_limit.store(log2_limit); }
 
 extern "C" int pcfgnat_pipeline_redo_counts(unsigned long long *inside_sweeps, unsigned long long *viterbi_sentences, int reset) {
     PCFGNAT_REQUIRE(inside_sweeps && viterbi_sentences, "pipeline_redo_counts: null pointer");

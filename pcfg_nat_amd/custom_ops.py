@@ -42,6 +42,12 @@ def pipeline_config(max_workgroups=None, spin_limit=None, outside_spin_limit=Non
         lib.pcfgnat_pipeline_outside_spin_limit(int(outside_spin_limit))
 
 
+def links_grad_range_limit(log2_limit=120.0):
+    """Test hook (process-wide): the largest base-2 exponent a factor of the rule posteriors of long graphs may have on the
+    matrix cores before its tile is recomputed term by term; ``float('-inf')`` forces the second path everywhere."""
+    _lib.load().pcfgnat_links_grad_range_limit(float(log2_limit))
+
+
 def pipeline_redo_counts(reset=False):
     """(inside sweeps, single-call Viterbi decodes) that the one-workgroup kernels had to redo on the current device
     because a pipelined sweep gave up, since the library was loaded or the last reset.  Synchronises with the device."""

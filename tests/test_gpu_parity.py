@@ -312,6 +312,17 @@ def test_long_graph_sweeps_agree(mode, L, T, ms, ns):
             assert (g0 - g1).abs().max() <= 1e-4 * max(g0.abs().max().item(), 1e-30)
 
 
+@pytest.mark.parametrize("case", ["L130", "L256", "L320_mixed", "L512_long", "L1028"])
+def test_rule_posteriors_term_by_term_path(case):
+    """The rule posteriors of long graphs with every tile sent down the path without a range limit (one exponential per
+    term instead of the factored sum on the matrix cores): same gradients, against the float64 oracle."""
+    try:
+        ops.links_grad_range_limit(float("-inf"))
+        test_inside_forward_backward_vs_oracle(case)
+    finally:
+        ops.links_grad_range_limit()
+
+
 @pytest.mark.parametrize("L,T,ms,ns", [(128, 30, [128, 90], [30, 22]), (320, 40, [320, 262], [40, 31]), (600, 24, [600, 520], [24, 24])])
 def test_inside_spiky_inputs_vs_oracle(L, T, ms, ns):
     """Emissions and links with jumps of hundreds of units and scattered -inf entries: neighbouring columns of the tables
