@@ -20,13 +20,15 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
-# HBM bytes per launch of the roofline kernel at this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled against a
-# plain device copy of known size; summary in profiles/lsg_cfg2_hbm_traffic_pmc.md.  None = not measured for this build.
-# (lsg_bwd: the single-call step at this batch's lengths - 3408 of 5120 rows read and written.)
+# Bytes per launch of the roofline kernel at this workload as the L2 caches request them from the memory side, from
+# rocprofv3 FETCH_SIZE / WRITE_SIZE scaled against a plain device copy of known size; summary in
+# profiles/lsg_cfg2_hbm_traffic_pmc.md.  None = not measured for this build.  (lsg_bwd: the single-call step at this
+# batch's lengths - 3408 of 5120 rows read and written.  Part of its reads are served by the 256 MB memory-side cache, where
+# the forward pass leaves the rows, which is how the kernel exceeds the rate of a device copy.)
 EVENT_EVERY = 4  # steps between two bracketed launches of the roofline kernel inside the timed region
 ROOFLINE_KERNEL = {"single": "lsg_bwd", "fused": "lsg_bwd", "unfused": "lsg_fwd"}
 ROOFLINE_KERNEL_NAME = {"lsg_bwd": "lsg_bwd_kernel<half, from logits>", "lsg_fwd": "lsg_fwd_kernel<half, grad>"}
-MEASURED_TRAFFIC_BYTES = {"lsg_bwd": 553.47e6, "lsg_fwd": None}
+MEASURED_TRAFFIC_BYTES = {"lsg_bwd": 555.04e6, "lsg_fwd": 273.77e6}
 
 
 def parse():
