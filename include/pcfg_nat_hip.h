@@ -324,21 +324,30 @@ int pcfgnat_extract_links_unpack(const float *dA, const float *dKr, const float 
                                  void *dkl, void *dkr, int64_t B, int64_t L, int64_t H, int64_t F, void *stream);
 
 /*
- * GLAT glancing with the `number-random` strategy (nat_pcfg_loss.py:193-269) in one call: lengths from the pad counts
+ * GLAT glancing (nat_pcfg_loss.py:193-269) in one call: lengths from the pad counts
  * (:195-196), arg max of the logits (:199), logsoftmax_gather without gradient + eos mask (:200-207), best-tree alignment
- * (:210), and everything the criterion derives from the alignment (:212-255).
+ * (:210), and everything the criterion derives from the alignment (:212-255), for each of its glance strategies:
+ * PCFGNAT_GLANCE_NUMBER_RANDOM (`number-random`, :235-242, every shipped script), PCFGNAT_GLANCE_CMLM (`cmlm`, :244-251),
+ * PCFGNAT_GLANCE_DEFAULT (no strategy named, :231-233).
  *   logits [B,L,V] (F16/F32/F64, read only); targets [B,T], prev_output_tokens [B,L] int64; links [B,L,ml+1,L] float32;
- *   noise [B,L] float32: the caller's randn draw of :235 (the uniform draw of :253 cannot change the result, because
- *   keep_prob is 0 or 1; the caller still makes it to keep its random stream in step); context_p: glancing ratio.
+ *   the caller's random draws, float32, made in the reference's order: noise [B,L] = randn (:235 / :245; number-random and
+ *   cmlm, else may be null), length_rand [B] = rand (:247; cmlm only, else may be null), keep_rand [B,L] = rand (:253; read
+ *   by the default strategy only - with the other two keep_prob is 0 or 1 and the draw cannot change the result, the
+ *   caller still makes it to keep its random stream in step - may be null for them); context_p: glancing ratio.
  * Workspaces: match_all [B,L,T], S [B,Mc,T+2], aux [pcfgnat_pcfg_aux_floats] float32; pred_tokens [B,L], lengths [2,B] int64
  * (the logits of pad nodes at or beyond a sentence's output length are not read: zeros in match_all and pred_tokens).
  * Outputs: path [B,L] int64 (target position of every node, -1 off the tree); matchmask [B,T,L], keep_word_mask [B,L]
- * (one byte per flag, 0/1); glat_prev_output_tokens [B,L], same_num [B], glance_nums [B] int64; loss_out[0] =
+ * (one byte per flag, 0/1); glat_prev_output_tokens [B,L], same_num [B], glance_nums [B] int64 (zeros for the default
+ * strategy, which has none); loss_out[0] =
  * -(ll/target_length).mean() over sentences with a finite best-tree likelihood ll = S[b,0,0], loss_out[1] = number of
  * the others.  On return lengths[0,:] = output_length and lengths[1,:] = target_length.
  */
+#define PCFGNAT_GLANCE_NUMBER_RANDOM 0
+#define PCFGNAT_GLANCE_CMLM 1
+#define PCFGNAT_GLANCE_DEFAULT 2
 int pcfgnat_glat_step(const void *logits, int dtype, const int64_t *targets, const int64_t *prev_output_tokens,
-                      const float *links, const float *noise, float context_p, int64_t pad_index, float *match_all, float *S,
+                      const float *links, int glance_strategy, const float *noise, const float *length_rand,
+                      const float *keep_rand, float context_p, int64_t pad_index, float *match_all, float *S,
                       float *aux, int64_t *pred_tokens, int64_t *lengths, int64_t *path, unsigned char *matchmask,
                       unsigned char *keep_word_mask, int64_t *glat_prev_output_tokens, int64_t *same_num,
                       int64_t *glance_nums, float *loss_out, int64_t B, int64_t L, int64_t V, int64_t T, int64_t ml,

@@ -56,7 +56,7 @@ SIGNATURES = {
     "pcfgnat_extract_links_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
                                               _i64, _i64, _vp]),
     "pcfgnat_extract_links_unpack": (_int, [_vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
-    "pcfgnat_glat_step": (_int, [_vp, _int, _vp, _vp, _vp, _vp, ctypes.c_float, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+    "pcfgnat_glat_step": (_int, [_vp, _int, _vp, _vp, _vp, _int, _vp, _vp, _vp, ctypes.c_float, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                  _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_pcfg_best_tree": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_pcfg_viterbi": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),

@@ -48,7 +48,7 @@ int ensure_dynamic_lds(const void *kernel, size_t bytes) {
 }
 }  // namespace pcfgnat
 
-extern "C" int pcfgnat_abi_version(void) { return 2; }
+extern "C" int pcfgnat_abi_version(void) { return 3; }
 
 extern "C" const char *pcfgnat_last_error(void) { return pcfgnat::error_buffer(); }
 

@@ -604,12 +604,18 @@ def pcfg_extract_links(query_chunks, key_chunks_left, key_chunks_right, gate_log
                                       left_tree_mask, right_tree_mask, main_chain)
 
 
+GLANCE_STRATEGIES = {"number-random": 0, "cmlm": 1, None: 2}  # PCFGNAT_GLANCE_* of the library
+
+
 def pcfg_glat_step(word_ins_out, tgt_tokens, prev_output_tokens, links, context_p, pad_index, generator=None,
-                   noise_device=None):
-    """GLAT glancing, ``number-random`` strategy (nat_pcfg_loss.py:193-269), as one native call.  Same results as the
-    torch glue over the separate ops; ``word_ins_out`` is only read.  The two random draws of the reference (``randn``
-    for the glance scores, then ``rand``) are made here, in that order, on the tokens' device or on ``noise_device``.
-    Returns the dict of ``harness.glat_alignment``."""
+                   noise_device=None, glance_strategy="number-random"):
+    """GLAT glancing (nat_pcfg_loss.py:193-269) as one native call, for each glance strategy of the reference
+    (``"number-random"``, ``"cmlm"``, ``None``).  Same results as the torch glue over the separate ops; ``word_ins_out``
+    is only read.  The random draws of the reference (``randn`` for the glance scores, ``rand`` for cmlm's lengths, then
+    ``rand`` for the revealed nodes, as far as the strategy makes them) are made here, in that order, on the tokens' device
+    or on ``noise_device``.  Returns the dict of ``harness.glat_alignment``."""
+    if glance_strategy not in GLANCE_STRATEGIES:
+        raise RuntimeError("pcfg_glat_step: unknown glance strategy %r" % (glance_strategy,))
     lib = get_pcfg_kernel()
     _need_cuda("pcfg_glat_step", word_ins_out, tgt_tokens, prev_output_tokens, links)
     if word_ins_out.dim() != 3 or not word_ins_out.is_contiguous():
@@ -630,8 +636,14 @@ def pcfg_glat_step(word_ins_out, tgt_tokens, prev_output_tokens, links, context_
     dev = word_ins_out.device
     tgt, prev, links = tgt_tokens.contiguous(), prev_output_tokens.contiguous(), links.contiguous()
     ndev = dev if noise_device is None else torch.device(noise_device)
-    noise = torch.randn((B, L), device=ndev, dtype=torch.float, generator=generator).to(dev)
-    torch.rand((B, L), device=ndev, generator=generator)  # the reference's second draw: cannot change the result
+    noise = len_rand = keep_rand = None
+    if glance_strategy is not None:
+        noise = torch.randn((B, L), device=ndev, dtype=torch.float, generator=generator).to(dev)
+    if glance_strategy == "cmlm":
+        len_rand = torch.rand((B,), device=ndev, dtype=torch.float, generator=generator).to(dev)
+    keep_rand = torch.rand((B, L), device=ndev, generator=generator)  # the reference's last draw
+    # (number-random, cmlm: it cannot change the result and is made only to keep the stream in step)
+    keep_rand = keep_rand.to(dev) if glance_strategy is None else None
     with torch.cuda.device(dev):
         f32 = dict(dtype=torch.float32, device=dev)
         i64 = dict(dtype=torch.int64, device=dev)
@@ -643,8 +655,10 @@ def pcfg_glat_step(word_ins_out, tgt_tokens, prev_output_tokens, links, context_
         matchmask = torch.empty((B, T, L), dtype=torch.bool, device=dev)
         keep = torch.empty((B, L), dtype=torch.bool, device=dev)
         out = torch.empty((2,), **f32)
+        ptr = lambda t: None if t is None else t.data_ptr()  # noqa: E731
         _lib.check(lib.pcfgnat_glat_step(word_ins_out.data_ptr(), code, tgt.data_ptr(), prev.data_ptr(), links.data_ptr(),
-                                         noise.data_ptr(), float(context_p), int(pad_index), match.data_ptr(), S.data_ptr(),
+                                         GLANCE_STRATEGIES[glance_strategy], ptr(noise), ptr(len_rand), ptr(keep_rand),
+                                         float(context_p), int(pad_index), match.data_ptr(), S.data_ptr(),
                                          aux.data_ptr(), ints[0].data_ptr(), small[0].data_ptr(), ints[1].data_ptr(),
                                          matchmask.data_ptr(), keep.data_ptr(), ints[2].data_ptr(), small[2].data_ptr(),
                                          small[3].data_ptr(), out.data_ptr(), B, L, V, T, ml, _stream(word_ins_out)), lib)

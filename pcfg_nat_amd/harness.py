@@ -49,15 +49,18 @@ def compute_pcfg_loss(outputs, output_masks, targets, target_masks, links, ops=_
 
 
 def glat_alignment(word_ins_out, tgt_tokens, prev_output_tokens, links, context_p, pad=PAD, ops=_default_ops,
-                   generator=None, noise_device=None, single_call=False):
-    """GLAT glancing with the ``number-random`` strategy (nat_pcfg_loss.py:193-269): best-tree alignment of target
-    tokens to graph nodes, then a random subset of the aligned nodes is revealed.  RNG order: ``randn`` then ``rand``.
-    The reference draws both on the tokens' device; ``noise_device`` (e.g. "cpu") draws them elsewhere and moves them,
-    which makes a run reproducible across devices.  ``single_call``: the same pass as one native call
-    (``ops.pcfg_glat_step``)."""
+                   generator=None, noise_device=None, single_call=False, glance_strategy="number-random"):
+    """GLAT glancing (nat_pcfg_loss.py:193-269): best-tree alignment of target tokens to graph nodes, then a random
+    subset of the aligned nodes is revealed, chosen by the criterion's ``glance_strategy``: ``"number-random"`` (every
+    shipped script; :235-242), ``"cmlm"`` (:244-251) or ``None`` (:231-233).  RNG order as in the reference: ``randn``
+    (not for ``None``), ``rand`` over the batch (``cmlm`` only), ``rand`` over the nodes.  The reference draws on the
+    tokens' device; ``noise_device`` (e.g. "cpu") draws elsewhere and moves the numbers, which makes a run reproducible
+    across devices.  ``single_call``: the same pass as one native call (``ops.pcfg_glat_step``)."""
+    if glance_strategy not in ("number-random", "cmlm", None):
+        raise RuntimeError("glat_alignment: unknown glance strategy %r" % (glance_strategy,))
     if single_call:
         return ops.pcfg_glat_step(word_ins_out, tgt_tokens, prev_output_tokens, links, context_p, pad, generator=generator,
-                                  noise_device=noise_device)
+                                  noise_device=noise_device, glance_strategy=glance_strategy)
     batch_size, prelen = links.shape[0], links.shape[1]
     tarlen = tgt_tokens.shape[1]
     target_length = (~tgt_tokens.eq(pad)).sum(1)
@@ -78,12 +81,20 @@ def glat_alignment(word_ins_out, tgt_tokens, prev_output_tokens, links, context_
     same_num = ((pred_tokens == oracle) & predict_align_mask).sum(1)
     dev = tgt_tokens.device
     ndev = dev if noise_device is None else torch.device(noise_device)
-    prob = torch.randn(oracle.shape, device=ndev, dtype=torch.float, generator=generator).to(dev)
-    prob.masked_fill_(~predict_align_mask, -100)
-    glance_nums = ((target_length - same_num) * context_p + 0.5).to(torch.long)
-    prob_thresh = prob.sort(descending=True)[0].gather(-1, (glance_nums - 1).clip(min=0).unsqueeze(-1)).squeeze(-1)
-    prob_thresh.masked_fill_(glance_nums == 0, 100)
-    keep_prob = (prob >= prob_thresh.unsqueeze(-1)).to(prob.dtype)
+    if glance_strategy is None:
+        glance_nums = torch.zeros_like(target_length)
+        keep_prob = ((target_length - same_num) / target_length * context_p).unsqueeze(-1) * predict_align_mask.float()
+    else:
+        prob = torch.randn(oracle.shape, device=ndev, dtype=torch.float, generator=generator).to(dev)
+        prob.masked_fill_(~predict_align_mask, -100)
+        if glance_strategy == "cmlm":
+            fraction = torch.rand(target_length.shape, device=ndev, dtype=torch.float, generator=generator).to(dev)
+            glance_nums = (target_length * fraction + 0.5).to(torch.long)
+        else:
+            glance_nums = ((target_length - same_num) * context_p + 0.5).to(torch.long)
+        prob_thresh = prob.sort(descending=True)[0].gather(-1, (glance_nums - 1).clip(min=0).unsqueeze(-1)).squeeze(-1)
+        prob_thresh.masked_fill_(glance_nums == 0, 100)
+        keep_prob = (prob >= prob_thresh.unsqueeze(-1)).to(prob.dtype)
     keep_word_mask = (torch.rand(prev_output_tokens.shape, device=ndev, generator=generator).to(dev) < keep_prob).bool()
     glat_prev_output_tokens = prev_output_tokens.masked_fill(keep_word_mask, 0) + oracle.masked_fill(~keep_word_mask, 0)
     return {"path": path, "matchmask": matchmask, "keep_word_mask": keep_word_mask,

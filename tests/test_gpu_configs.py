@@ -140,19 +140,24 @@ def test_config5_glat_alignment():
     assert torch.equal(got["keep_word_mask"].cpu(), want["keep_word_mask"])
     assert torch.equal(got["glat_prev_output_tokens"].cpu(), want["glat_prev_output_tokens"])
     assert torch.equal(got["matchmask"].cpu(), want["matchmask"])
-    # the same pass as one native call: identical decisions, same random stream consumed
-    for p in (0.5, 0.0, 1.0):
+    # the same pass as one native call, and the torch glue over the device operators, for every glance strategy of the
+    # criterion: identical decisions, same random stream consumed
+    for strategy, p in (("number-random", 0.5), ("number-random", 0.0), ("number-random", 1.0), ("cmlm", 0.5), (None, 0.5),
+                        (None, 1.0)):
         g2 = torch.Generator().manual_seed(7)
         want = harness.glat_alignment(batch["logits"].float(), batch["targets"], prev, batch["links"], p, ops=oracle_ops,
-                                      generator=g2)
-        g3 = torch.Generator().manual_seed(7)
-        one = harness.glat_alignment(logits, batch["targets"].to(DEV), prev.to(DEV), batch["links"].to(DEV), p, generator=g3,
-                                     noise_device="cpu", single_call=True)
-        assert torch.equal(logits, batch["logits"].to(DEV))
-        assert torch.equal(g2.get_state(), g3.get_state())
-        for key in ("path", "keep_word_mask", "glat_prev_output_tokens", "matchmask", "same_num", "glance_nums"):
-            assert one[key].dtype == want[key].dtype and torch.equal(one[key].cpu(), want[key]), key
-        assert torch.allclose(one["max_tree_lprob"].cpu(), want["max_tree_lprob"], rtol=2e-5)
+                                      generator=g2, glance_strategy=strategy)
+        if strategy is None:  # a real coin per node: some aligned nodes revealed, some not
+            assert 0 < int(want["keep_word_mask"].sum()) < int((want["path"] >= 0).sum())
+        for single_call in (True, False):
+            g3 = torch.Generator().manual_seed(7)
+            one = harness.glat_alignment(logits, batch["targets"].to(DEV), prev.to(DEV), batch["links"].to(DEV), p, generator=g3,
+                                         noise_device="cpu", single_call=single_call, glance_strategy=strategy)
+            assert torch.equal(logits, batch["logits"].to(DEV))
+            assert torch.equal(g2.get_state(), g3.get_state())
+            for key in ("path", "keep_word_mask", "glat_prev_output_tokens", "matchmask", "same_num", "glance_nums"):
+                assert one[key].dtype == want[key].dtype and torch.equal(one[key].cpu(), want[key]), (strategy, p, single_call, key)
+            assert torch.allclose(one["max_tree_lprob"].cpu(), want["max_tree_lprob"], rtol=2e-5)
 
 
 def test_config4_viterbi_decode():

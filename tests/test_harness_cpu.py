@@ -1,6 +1,7 @@
 """The criterion / decoder glue (pcfg_nat_amd/harness.py) run over the CPU oracle: checks the glue itself (eos masking,
 loss reduction, GLAT sampling, length selection) on the tiny plumbing configuration."""
 import numpy as np
+import pytest
 import torch
 
 import oracle_ops
@@ -74,6 +75,48 @@ def test_glat_alignment_is_deterministic_and_consistent():
     assert (keep.sum(1) <= a["glance_nums"]).all()
     assert a["matchmask"].shape == (B, batch["targets"].shape[1], L)
     assert torch.equal(a["matchmask"].sum(-1).sum(-1), n)
+
+
+def test_glance_strategies_consume_the_reference_random_stream():
+    """The three glance strategies of the criterion (nat_pcfg_loss.py:231-251) over the oracle: `number-random` reveals
+    round((n - same) * p) nodes chosen by a randn ranking, `cmlm` a uniform share of the target length, the default flips a
+    coin per aligned node with probability (n - same) / n * p; each consumes exactly the draws the reference makes, in its
+    order (randn [B,L]; rand [B] for cmlm; rand [B,L])."""
+    batch = synth.config1()
+    B, L, V = batch["logits"].shape
+    prev = torch.full((B, L), 3, dtype=torch.int64)
+    n = batch["target_length"]
+
+    def run(strategy, p):
+        gen = torch.Generator().manual_seed(11)
+        out = harness.glat_alignment(batch["logits"].clone(), batch["targets"], prev, batch["links"], p, ops=oracle_ops,
+                                     generator=gen, glance_strategy=strategy)
+        return out, gen
+
+    def stream_after(draws):
+        gen = torch.Generator().manual_seed(11)
+        for kind, shape in draws:
+            (torch.randn if kind == "n" else torch.rand)(shape, generator=gen)
+        return gen.get_state()
+
+    out, gen = run("number-random", 0.5)
+    assert torch.equal(gen.get_state(), stream_after([("n", (B, L)), ("u", (B, L))]))
+    assert torch.equal(out["keep_word_mask"].sum(1), ((n - out["same_num"]) * 0.5 + 0.5).long())
+    out, gen = run("cmlm", 0.5)
+    assert torch.equal(gen.get_state(), stream_after([("n", (B, L)), ("u", (B,)), ("u", (B, L))]))
+    g = torch.Generator().manual_seed(11)
+    torch.randn((B, L), generator=g)
+    want_nums = (n * torch.rand((B,), generator=g) + 0.5).long()
+    assert torch.equal(out["glance_nums"], want_nums) and torch.equal(out["keep_word_mask"].sum(1), want_nums.clamp(max=n))
+    out, gen = run(None, 1.0)
+    assert torch.equal(gen.get_state(), stream_after([("u", (B, L))]))
+    aligned = out["path"] >= 0
+    assert not (out["keep_word_mask"] & ~aligned).any()
+    u = torch.rand((B, L), generator=torch.Generator().manual_seed(11))
+    share = ((n - out["same_num"]) / n * 1.0).unsqueeze(-1)
+    assert torch.equal(out["keep_word_mask"], (u < share * aligned.float()))
+    with pytest.raises(RuntimeError):
+        run("random", 0.5)
 
 
 def test_force_emit_semantics():
