@@ -2713,13 +2713,29 @@ __global__ __launch_bounds__(NTP) void inside_bwd_ml1_pipe_kernel(const float *_
 // terms lost only below 2^-40 of a posterior for rules down to 2^-26) is recomputed by its workgroup as one exponential
 // per term, which is exact over the whole range (the log-domain form the sweeps use).
 // The slab has been zero-filled beforehand.  use_corr: the outside tables are relative to offsets of their own (sweeps
-// side by side) and every column takes its correction corr_t.  Dynamic LDS: 3 * 32 * (span + 1) + span floats, span = the
-// number of positions staged at a time (a multiple of 8, at most LG_SPAN).
+// side by side) and every column takes its correction corr_t.  Dynamic LDS: 3 * 32 * (span + 1) + span floats (and at
+// least the 3 * 64 * 17 of the partial sums), span = the number of positions staged at a time (a multiple of 8, at most
+// LG_SPAN).
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 constexpr int LG_TILE = 32, LG_SPAN = 256;
-inline int links_grad_span(int T) { return T - 1 >= LG_SPAN ? LG_SPAN : ((T - 1 + 7) / 8) * 8; }
-inline size_t links_grad_lds_bytes(int T) { return ((size_t)3 * LG_TILE * (links_grad_span(T) + 1) + links_grad_span(T)) * sizeof(float); }
-__global__ __launch_bounds__(256) void links_grad_ml1_stream_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
+constexpr size_t LG_PART_BYTES = (size_t)3 * 64 * 17 * sizeof(float);  // the partial sums of three waves, one accumulator set
+inline size_t links_grad_lds_bytes(int span) {
+    const size_t tables = ((size_t)3 * LG_TILE * (span + 1) + span) * sizeof(float);
+    return tables > LG_PART_BYTES ? tables : LG_PART_BYTES;
+}
+// Positions staged at a time, as (span, variant): all of them (up to LG_SPAN, two workgroups to a compute unit: the
+// registers that hold a span in flight) while the live tiles fit the device in one round; beyond that equal spans of at
+// most LG_SPAN_SMALL with the variant that keeps fewer loads in flight and lets three workgroups share a compute unit.
+constexpr int LG_SPAN_SMALL = 96;
+inline int links_grad_span(int T, long tiles_live, bool &small) {
+    const int all = T - 1 >= LG_SPAN ? LG_SPAN : ((T - 1 + 7) / 8) * 8;
+    small = all > LG_SPAN_SMALL && tiles_live > 2L * device_compute_units();
+    if (!small) return all;
+    const int stages = (T - 1 + LG_SPAN_SMALL - 1) / LG_SPAN_SMALL;
+    return (((T - 1 + stages - 1) / stages) + 7) / 8 * 8;
+}
+template <int QMAX>  // the span is at most 32 * QMAX positions
+__global__ __launch_bounds__(256, QMAX < 8 ? 3 : 2) void links_grad_ml1_stream_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
                                                                    const float *__restrict__ aux_c, const float *__restrict__ links,
                                                                    const int64_t *__restrict__ out_len,
                                                                    const int64_t *__restrict__ tgt_len, float *__restrict__ lgrad,
@@ -2728,7 +2744,8 @@ __global__ __launch_bounds__(256) void links_grad_ml1_stream_kernel(const float 
     extern __shared__ float lg_lds[];
     const int ld = span + 1;                 // row pitch: odd, so that a column of 32 rows falls into 32 banks
     float *sw0 = lg_lds, *sw1 = sw0 + LG_TILE * ld, *ss = sw1 + LG_TILE * ld, *s_u = ss + LG_TILE * ld;  // [32][ld] x 3, [span]
-    __shared__ float s_part[3][64][17];  // partial sums of waves 1..3, one accumulator set at a time
+    float (*s_part)[64][17] = reinterpret_cast<float (*)[64][17]>(lg_lds);  // partial sums of waves 1..3, one accumulator set
+                                                                            // at a time, over the tables once they are used up
     __shared__ int s_bad;
     const int b = blockIdx.z, at = blockIdx.y, ct = blockIdx.x;
     if (ct < at) return;
@@ -2751,9 +2768,9 @@ __global__ __launch_bounds__(256) void links_grad_ml1_stream_kernel(const float 
     // the first value is stored, so the span costs one trip to memory
     const int tx = tid & 31, ty = tid >> 5;
     auto stage = [&](int t1) {
-        float v0[LG_SPAN / 32][4], v1[LG_SPAN / 32][4], vs[LG_SPAN / 32][4];
+        float v0[QMAX][4], v1[QMAX][4], vs[QMAX][4];
 #pragma unroll
-        for (int q = 0; q < LG_SPAN / 32; q++) {
+        for (int q = 0; q < QMAX; q++) {
             if (32 * q < span) {  // uniform
                 const int tt = t1 + 32 * q + tx;
                 const bool tin = tt <= n - 1;
@@ -2768,7 +2785,7 @@ __global__ __launch_bounds__(256) void links_grad_ml1_stream_kernel(const float 
             }
         }
 #pragma unroll
-        for (int q = 0; q < LG_SPAN / 32; q++) {
+        for (int q = 0; q < QMAX; q++) {
             if (32 * q + tx < span) {
 #pragma unroll
                 for (int p = 0; p < 4; p++) {
@@ -3123,9 +3140,12 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
         PCFGNAT_HIP_CHECK(hipGetLastError());
     }
     const int use_corr = side_by_side ? 1 : 0;
-    PCFGNAT_DYNAMIC_LDS(links_grad_ml1_stream_kernel, links_grad_lds_bytes(T));
-    hipLaunchKernelGGL(links_grad_ml1_stream_kernel, dim3(tiles, tiles, B), dim3(256), links_grad_lds_bytes(T), stream, go, S, aux, links,
-                       ol, tl, lg, L, T, Mc, seed, use_corr, g_links_grad_range_limit.load(), links_grad_span(T));
+    bool small;
+    const int span = links_grad_span(T, (long)B * tiles * (tiles + 1) / 2, small);
+    auto lgk = small ? links_grad_ml1_stream_kernel<LG_SPAN_SMALL / 32> : links_grad_ml1_stream_kernel<LG_SPAN / 32>;
+    PCFGNAT_DYNAMIC_LDS(lgk, links_grad_lds_bytes(span));
+    hipLaunchKernelGGL(lgk, dim3(tiles, tiles, B), dim3(256), links_grad_lds_bytes(span), stream, go, S, aux, links, ol, tl, lg, L, T,
+                       Mc, seed, use_corr, g_links_grad_range_limit.load(), span);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL(match_grad_ml1_stream_kernel, dim3((L * T + 255) / 256, B), dim3(256), 0, stream, go, S, aux, match_all, ol, tl, mg, L,
                        T, Mc, seed, use_corr);
