@@ -324,6 +324,21 @@ int pcfgnat_extract_links_unpack(const float *dA, const float *dKr, const float 
                                  void *dkl, void *dkr, int64_t B, int64_t L, int64_t H, int64_t F, void *stream);
 
 /*
+ * The same scorer (same reference lines) with the three products inside the kernels, on the matrix cores: one call
+ * forward, nothing for the caller to multiply.  Built for float16 chunks with F a multiple of 16 up to 128 and float32
+ * chunks with F a multiple of 8 up to 64, as long as the rows of a 32-parent tile fit the local memory
+ * (pcfgnat_extract_links_fused_supported returns 1; otherwise the calls return PCFGNAT_EUNSUPPORTED and the five-call
+ * form above applies).  Chunks [B,L,H,F] contiguous and 16-byte aligned, the other arguments as above.
+ *   fused_forward: -> links [B,L,2,L], head_lse [B,L,H].
+ */
+int pcfgnat_extract_links_fused_supported(int dtype, int64_t L, int64_t H, int64_t F);
+int pcfgnat_extract_links_fused_forward(const void *query_chunks, const void *key_chunks_left, const void *key_chunks_right, int dtype,
+                                        const float *gate_logits, const int64_t *prev_output_tokens, int64_t pad_index,
+                                        const unsigned char *left_tree_mask, const unsigned char *right_tree_mask,
+                                        const unsigned char *main_chain, float *links, float *head_lse, int64_t B, int64_t L,
+                                        int64_t H, int64_t F, void *stream);
+
+/*
  * GLAT glancing (nat_pcfg_loss.py:193-269) in one call: lengths from the pad counts
  * (:195-196), arg max of the logits (:199), logsoftmax_gather without gradient + eos mask (:200-207), best-tree alignment
  * (:210), and everything the criterion derives from the alignment (:212-255), for each of its glance strategies:

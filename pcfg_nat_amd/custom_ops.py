@@ -545,9 +545,23 @@ class PCFGExtractLinksFunc(Function):
             raise RuntimeError("pcfg_extract_links: tree masks must be [prelen, prelen] and main_chain [prelen]")
         dev = query_chunks.device
         code = _DTYPE_CODE[query_chunks.dtype]
+        fused = bool(lib.pcfgnat_extract_links_fused_supported(code, L, H, F))
         with torch.cuda.device(dev):
             st = _stream(query_chunks)
             q, kl, kr = query_chunks.contiguous(), key_chunks_left.contiguous(), key_chunks_right.contiguous()
+            if fused and not any(ctx.needs_input_grad[:4]):
+                # the products on the matrix cores inside the one kernel; nothing is kept for a backward
+                gate = gate_logits.float().contiguous()
+                prev = prev_output_tokens.to(torch.int64).contiguous()
+                masks = [t.contiguous() if t.dtype in (torch.bool, torch.uint8) else t.ne(0).contiguous()
+                         for t in (left_tree_mask, right_tree_mask, main_chain)]
+                links = torch.empty((B, L, 2, L), dtype=torch.float32, device=dev)
+                lse = torch.empty((B, L, H), dtype=torch.float32, device=dev)
+                _lib.check(lib.pcfgnat_extract_links_fused_forward(q.data_ptr(), kl.data_ptr(), kr.data_ptr(), code, gate.data_ptr(),
+                                                                   prev.data_ptr(), int(pad_index), masks[0].data_ptr(),
+                                                                   masks[1].data_ptr(), masks[2].data_ptr(), links.data_ptr(),
+                                                                   lse.data_ptr(), B, L, H, F, st), lib)
+                return links
             A = torch.empty((B, H, 2 * L, F), dtype=torch.float32, device=dev)
             Kr = torch.empty((B, H, L, F), dtype=torch.float32, device=dev)
             _lib.check(lib.pcfgnat_extract_links_pack(q.data_ptr(), kl.data_ptr(), kr.data_ptr(), code, A.data_ptr(), Kr.data_ptr(),

@@ -480,6 +480,49 @@ def test_extract_links_forward_backward_vs_torch_restatement(B, L, H, F, dtype):
         assert err <= tol * scale, (name, err, scale)
 
 
+@pytest.mark.parametrize("B,L,H,F,dtype", [(2, 34, 8, 16, torch.float32), (4, 128, 8, 64, torch.float16), (2, 514, 4, 8, torch.float32),
+                                            (2, 22, 16, 8, torch.float32), (2, 12, 1, 8, torch.float32), (2, 200, 4, 16, torch.float16),
+                                            (3, 130, 8, 64, torch.float32), (2, 66, 16, 32, torch.float16), (2, 40, 2, 128, torch.float16)])
+def test_extract_links_products_inside_the_kernel(B, L, H, F, dtype):
+    """The scorer with its three products on the matrix cores inside the kernel (what `pcfg_extract_links` runs when no
+    gradient is asked for): links against the float64 restatement, the per-head normalisers against the five-call form,
+    graphs that are no multiple of the 32-wide tiles, padded sentences, 1 to 16 heads."""
+    from oracle import extract_links_ref as ref
+    lib = ops.get_pcfg_kernel()
+    assert lib.pcfgnat_extract_links_fused_supported(ops._DTYPE_CODE[dtype], L, H, F) == 1
+    g = torch.Generator().manual_seed(L + H)
+    q, kl, kr = ((torch.randn(B, L, H, F, generator=g) * 0.7).to(dtype) for _ in range(3))
+    gate = torch.randn(B, L, H, generator=g).to(dtype)
+    ms = [L, max(4, (L // 2) // 2 * 2), 4, L][:B]
+    prev = torch.full((B, L), 3).masked_fill(torch.arange(L).view(1, L) >= torch.tensor(ms).view(B, 1), synth.PAD)
+    lm, rm, mc = synth.support_masks(L, 1)
+    want = ref.extract_links(*(t.double() for t in (q, kl, kr, gate)), prev, synth.PAD, lm, rm, mc).double()
+    fin = torch.isfinite(want)
+    dev = [t.to(DEV) for t in (q, kl, kr, gate)]
+    with torch.no_grad():
+        got = ops.pcfg_extract_links(*dev, prev.to(DEV), synth.PAD, lm.to(DEV), rm.to(DEV), mc.to(DEV))
+    assert got.dtype == torch.float32 and torch.equal(torch.isfinite(got).cpu(), fin)
+    assert torch.allclose(got.cpu().double()[fin], want[fin], rtol=2e-5, atol=2e-5)
+    # the five-call form (taken when a gradient is needed) gives the same links
+    leaves = [t.clone().requires_grad_(True) for t in dev]
+    other = ops.pcfg_extract_links(*leaves, prev.to(DEV), synth.PAD, lm.to(DEV), rm.to(DEV), mc.to(DEV)).detach()
+    assert torch.equal(torch.isfinite(other), torch.isfinite(got))
+    assert torch.allclose(got[fin.to(DEV)], other[fin.to(DEV)], rtol=2e-5, atol=2e-5)
+
+
+def test_extract_links_fused_form_rejects_what_it_does_not_cover():
+    lib = ops.get_pcfg_kernel()
+    assert lib.pcfgnat_extract_links_fused_supported(ops._DTYPE_CODE[torch.float32], 256, 2, 24) == 0   # head dimension
+    assert lib.pcfgnat_extract_links_fused_supported(ops._DTYPE_CODE[torch.float64], 64, 2, 16) == 0    # dtype
+    assert lib.pcfgnat_extract_links_fused_supported(ops._DTYPE_CODE[torch.float16], 64, 3, 16) == 0    # heads
+    assert lib.pcfgnat_extract_links_fused_supported(ops._DTYPE_CODE[torch.float32], 64, 16, 64) == 0   # tile rows beyond the LDS
+    x = torch.zeros(1, 64, 3, 16, device=DEV, dtype=torch.float16)
+    rc = lib.pcfgnat_extract_links_fused_forward(x.data_ptr(), x.data_ptr(), x.data_ptr(), ops._DTYPE_CODE[torch.float16], x.data_ptr(),
+                                                 x.data_ptr(), 1, x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(),
+                                                 1, 64, 3, 16, None)
+    assert rc != 0 and b"heads" in lib.pcfgnat_last_error()
+
+
 def _decode_case(name):
     if name == "short":
         return synth.decode_batch([5, 9, 16, 3, 12], seed=3, V=500)
