@@ -329,14 +329,27 @@ int pcfgnat_extract_links_unpack(const float *dA, const float *dKr, const float 
  * chunks with F a multiple of 8 up to 64, as long as the rows of a 32-parent tile fit the local memory
  * (pcfgnat_extract_links_fused_supported returns 1; otherwise the calls return PCFGNAT_EUNSUPPORTED and the five-call
  * form above applies).  Chunks [B,L,H,F] contiguous and 16-byte aligned, the other arguments as above.
- *   fused_forward: -> links [B,L,2,L], head_lse [B,L,H].
+ *   fused_forward:  -> links [B,L,2,L], head_lse [B,L,H] and, where tile_masks is not null, tile_masks [B,L,1+ceil(L/32)]
+ *                   (per parent a word of flags and its allowed right children as bits; what the backward reads).
+ *   fused_backward: grad_links, links, head_lse, tile_masks as the forward left them, and the chunks and gate logits
+ *                   of the forward -> gradients of the three chunk tensors [B,L,H,F] in `dtype` and of the gate logits
+ *                   [B,L,H] float32, in three launches; built for head dimensions up to 64 (fused_backward_supported
+ *                   returns 1).  workspace: device memory of fused_backward_workspace_bytes(B, L, H, F) bytes, 16-byte
+ *                   aligned, contents irrelevant on entry.
  */
 int pcfgnat_extract_links_fused_supported(int dtype, int64_t L, int64_t H, int64_t F);
 int pcfgnat_extract_links_fused_forward(const void *query_chunks, const void *key_chunks_left, const void *key_chunks_right, int dtype,
                                         const float *gate_logits, const int64_t *prev_output_tokens, int64_t pad_index,
                                         const unsigned char *left_tree_mask, const unsigned char *right_tree_mask,
-                                        const unsigned char *main_chain, float *links, float *head_lse, int64_t B, int64_t L,
-                                        int64_t H, int64_t F, void *stream);
+                                        const unsigned char *main_chain, float *links, float *head_lse, unsigned *tile_masks,
+                                        int64_t B, int64_t L, int64_t H, int64_t F, void *stream);
+int pcfgnat_extract_links_fused_backward_supported(int dtype, int64_t L, int64_t H, int64_t F);
+size_t pcfgnat_extract_links_fused_backward_workspace_bytes(int64_t B, int64_t L, int64_t H, int64_t F);
+int pcfgnat_extract_links_fused_backward(const float *grad_links, const float *links, const float *head_lse,
+                                         const unsigned *tile_masks, const void *query_chunks, const void *key_chunks_left,
+                                         const void *key_chunks_right, int dtype, const float *gate_logits, void *dq, void *dkl,
+                                         void *dkr, float *dgate, float *workspace, int64_t B, int64_t L, int64_t H, int64_t F,
+                                         void *stream);
 
 /*
  * GLAT glancing (nat_pcfg_loss.py:193-269) in one call: lengths from the pad counts

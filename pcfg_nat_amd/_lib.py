@@ -57,8 +57,12 @@ SIGNATURES = {
                                               _i64, _i64, _vp]),
     "pcfgnat_extract_links_unpack": (_int, [_vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_extract_links_fused_supported": (_int, [_int, _i64, _i64, _i64]),
-    "pcfgnat_extract_links_fused_forward": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
-                                                    _i64, _vp]),
+    "pcfgnat_extract_links_fused_forward": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
+                                                    _i64, _i64, _vp]),
+    "pcfgnat_extract_links_fused_backward_supported": (_int, [_int, _i64, _i64, _i64]),
+    "pcfgnat_extract_links_fused_backward_workspace_bytes": (ctypes.c_size_t, [_i64, _i64, _i64, _i64]),
+    "pcfgnat_extract_links_fused_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
+                                                     _i64, _i64, _vp]),
     "pcfgnat_glat_step": (_int, [_vp, _int, _vp, _vp, _vp, _int, _vp, _vp, _vp, ctypes.c_float, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                  _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_pcfg_best_tree": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),

@@ -15,60 +15,10 @@
 // instruction sequence is the same permutation for both operands, which a contraction does not see.
 // fp16 chunks: v_mfma_f32_32x32x16_f16 (products of fp16 values are exact in fp32, accumulation in fp32: what the
 // reference's `.to(float)` + einsum computes up to the order of the sum).  fp32 chunks: v_mfma_f32_32x32x2_f32.
-#include "common.hip.h"
+#include "links_fused.hip.h"
 
 namespace pcfgnat {
 namespace {
-
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-
-constexpr int PT = 32;        // parents per tile
-constexpr int LF_NT = 256;    // threads per workgroup: four waves
-
-typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-
-constexpr float LF_LOG2E = 1.4426950408889634f, LF_LN2 = 0.6931471805599453f;
-constexpr float LF_FLOOR = -1e30f;  // stands for "no term yet" where -inf would give inf - inf
-__device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ __forceinline__ float lg2(float x) { return __builtin_amdgcn_logf(x); }
-
-template <typename T>
-struct Chunk;
-template <>
-struct Chunk<__half> {
-    static constexpr int EPC = 8;  // elements per 16-byte chunk
-    // acc += a (rows) x b (columns) over the 16 elements the two halves of the wave hold
-    static __device__ __forceinline__ void mma(const uint4 &a, const uint4 &b, floatx16 &acc) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), acc, 0, 0, 0);
-    }
-    static __device__ __forceinline__ float dot(const uint4 &a, const uint4 &b, float acc) {
-        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a.x), __builtin_bit_cast(half2_t, b.x), acc, false);
-        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a.y), __builtin_bit_cast(half2_t, b.y), acc, false);
-        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a.z), __builtin_bit_cast(half2_t, b.z), acc, false);
-        return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a.w), __builtin_bit_cast(half2_t, b.w), acc, false);
-    }
-};
-template <>
-struct Chunk<float> {
-    static constexpr int EPC = 4;
-    static __device__ __forceinline__ void mma(const uint4 &a, const uint4 &b, floatx16 &acc) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), acc, 0, 0, 0);
-    }
-    static __device__ __forceinline__ float dot(const uint4 &a, const uint4 &b, float acc) {
-        acc = __builtin_fmaf(__uint_as_float(a.x), __uint_as_float(b.x), acc);
-        acc = __builtin_fmaf(__uint_as_float(a.y), __uint_as_float(b.y), acc);
-        acc = __builtin_fmaf(__uint_as_float(a.z), __uint_as_float(b.z), acc);
-        return __builtin_fmaf(__uint_as_float(a.w), __uint_as_float(b.w), acc);
-    }
-};
-
-// right child of accumulator r in lane half kb, relative to the tile: rows (r % 4) + 4 * kb + 8 * (r / 4)
-__device__ __forceinline__ int acc_row(int r, int kb) { return (r & 3) + 4 * kb + 8 * (r >> 2); }
 
 // LDS of the forward kernel, in bytes: the query and left-key rows of the parent tile for all heads (row pitch: the row
 // plus one chunk, which spreads the 32 rows of a column of chunks over the banks), the left-key row of node 0, and the
@@ -92,8 +42,8 @@ __global__ __launch_bounds__(LF_NT) void links_fused_fwd_kernel(const T *__restr
                                                                const unsigned char *__restrict__ ltm,
                                                                const unsigned char *__restrict__ rtm,
                                                                const unsigned char *__restrict__ main_chain,
-                                                               float *__restrict__ links, float *__restrict__ lse_out, int L, int H,
-                                                               float scale2) {
+                                                               float *__restrict__ links, float *__restrict__ lse_out,
+                                                               unsigned *__restrict__ masks_out, int L, int H, float scale2) {
     constexpr int EPC = Chunk<T>::EPC, F = 2 * NCH * EPC;
     extern __shared__ uint4 lf_lds[];
     const int HF = H * F, cpr = HF / EPC, pitch = cpr + 1;  // chunks per row of all heads, row pitch in chunks
@@ -242,6 +192,12 @@ __global__ __launch_bounds__(LF_NT) void links_fused_fwd_kernel(const T *__restr
     if (tid < cpr) sK0[tid] = vk0_first;
     for (int j = tid + LF_NT; j < cpr; j += LF_NT) sK0[j] = reinterpret_cast<const uint4 *>(kl + (size_t)b * L * HF)[j];
     __syncthreads();
+    if (masks_out != nullptr) {  // [B,L,1+nw]: the flags of every parent, then its allowed right children (for the backward)
+        for (int i = tid; i < PT * (1 + nw); i += LF_NT) {
+            const int pp = i / (1 + nw), w = i - pp * (1 + nw);
+            if (a0 + pp < L) masks_out[((size_t)b * L + a0 + pp) * (1 + nw) + w] = (w == 0) ? s_flags[pp] : s_allow[pp * nw + w - 1];
+        }
+    }
     // ---- per (parent, head): the two q.kl terms and the log-softmax of the gates, in base 2
     {
         const int pp = tid & 31, a = a0 + pp;
@@ -477,12 +433,6 @@ __global__ __launch_bounds__(LF_NT) void links_fused_fwd_kernel(const T *__restr
     }
 }
 
-// chunks per lane of one head's row: 1, 2, 4 or 8
-bool fused_head_dim_built(int dtype, int64_t F) {
-    const int64_t unit = dtype == PCFGNAT_F16 ? 16 : 8;
-    return F == unit || F == 2 * unit || F == 4 * unit || F == 8 * unit;
-}
-
 int check_fused_args(const char *who, int dtype, int64_t B, int64_t L, int64_t H, int64_t F) {
     PCFGNAT_REQUIRE(B >= 0 && L >= 2 && F >= 1, "%s: bad dimensions (B=%lld L=%lld F=%lld)", who, (long long)B, (long long)L, (long long)F);
     if (!(H == 1 || H == 2 || H == 4 || H == 8 || H == 16))
@@ -498,8 +448,8 @@ int check_fused_args(const char *who, int dtype, int64_t B, int64_t L, int64_t H
 
 template <typename T>
 int launch_fused_fwd(const void *q, const void *kl, const void *kr, const float *gate, const int64_t *prev, int64_t pad,
-                     const unsigned char *ltm, const unsigned char *rtm, const unsigned char *mc, float *links, float *lse, int64_t B,
-                     int64_t L, int64_t H, int64_t F, hipStream_t s) {
+                     const unsigned char *ltm, const unsigned char *rtm, const unsigned char *mc, float *links, float *lse,
+                     unsigned *masks_out, int64_t B, int64_t L, int64_t H, int64_t F, hipStream_t s) {
     const size_t lds = fused_fwd_lds_bytes((int)L, (int)H, (int)F, (int)sizeof(T));
     if (lds > (size_t)160 * 1024)
         return fail(PCFGNAT_EUNSUPPORTED, "extract_links_fused_forward: %zu bytes of LDS needed (H*F = %lld, L = %lld)", lds,
@@ -511,7 +461,7 @@ int launch_fused_fwd(const void *q, const void *kl, const void *kr, const float 
         auto k = links_fused_fwd_kernel<T, nch>;                                                                                      \
         PCFGNAT_DYNAMIC_LDS(k, lds);                                                                                                  \
         hipLaunchKernelGGL(k, grid, dim3(LF_NT), lds, s, (const T *)q, (const T *)kl, (const T *)kr, gate, prev, pad, ltm, rtm, mc, links, \
-                           lse, (int)L, (int)H, scale);                                                                               \
+                           lse, masks_out, (int)L, (int)H, scale);                                                                               \
         break;                                                                                                                        \
     }
     switch (F / (2 * Chunk<T>::EPC)) {
@@ -542,7 +492,8 @@ extern "C" int pcfgnat_extract_links_fused_forward(const void *query_chunks, con
                                                    int dtype, const float *gate_logits, const int64_t *prev_output_tokens,
                                                    int64_t pad_index, const unsigned char *left_tree_mask,
                                                    const unsigned char *right_tree_mask, const unsigned char *main_chain, float *links,
-                                                   float *head_lse, int64_t B, int64_t L, int64_t H, int64_t F, void *stream) {
+                                                   float *head_lse, unsigned *tile_masks, int64_t B, int64_t L, int64_t H, int64_t F,
+                                                   void *stream) {
     int rc = check_fused_args("extract_links_fused_forward", dtype, B, L, H, F);
     if (rc != PCFGNAT_OK) return rc;
     if (B == 0) return PCFGNAT_OK;
@@ -554,7 +505,7 @@ extern "C" int pcfgnat_extract_links_fused_forward(const void *query_chunks, con
     hipStream_t s = (hipStream_t)stream;
     if (dtype == PCFGNAT_F16)
         return launch_fused_fwd<__half>(query_chunks, key_chunks_left, key_chunks_right, gate_logits, prev_output_tokens, pad_index,
-                                        left_tree_mask, right_tree_mask, main_chain, links, head_lse, B, L, H, F, s);
+                                        left_tree_mask, right_tree_mask, main_chain, links, head_lse, tile_masks, B, L, H, F, s);
     return launch_fused_fwd<float>(query_chunks, key_chunks_left, key_chunks_right, gate_logits, prev_output_tokens, pad_index,
-                                   left_tree_mask, right_tree_mask, main_chain, links, head_lse, B, L, H, F, s);
+                                   left_tree_mask, right_tree_mask, main_chain, links, head_lse, tile_masks, B, L, H, F, s);
 }

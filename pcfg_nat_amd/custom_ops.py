@@ -523,14 +523,16 @@ def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unre
 
 
 class PCFGExtractLinksFunc(Function):
-    """The model's link scorer after its projections (glat_decomposed_with_link_two_hands_tri_pcfg.py:153-199): the
-    batched products go through torch's GEMM library (one product forward, two backward), everything else (packing,
-    masking, the gather of the left terms, the joint log-softmax over (left option, right child) per head, the gate
-    mixture and the whole backward of these) runs in five small kernels that never materialise a [B,L,2L,H] tensor."""
+    """The model's link scorer after its projections (glat_decomposed_with_link_two_hands_tri_pcfg.py:153-199).  For fp16
+    and fp32 chunks with head dimensions the library covers, the batched products run on the matrix cores inside the
+    kernels (one launch forward, three backward).  Otherwise (float64, other head dimensions) the products go through
+    torch's GEMM library (one product forward, two backward) and everything else (packing, masking, the gather of the
+    left terms, the joint log-softmax over (left option, right child) per head, the gate mixture and the whole backward of
+    these) runs in five small kernels.  Neither form materialises a [B,L,2L,H] tensor."""
 
     @staticmethod
     def forward(ctx, query_chunks, key_chunks_left, key_chunks_right, gate_logits, prev_output_tokens, pad_index,
-                left_tree_mask, right_tree_mask, main_chain):
+                left_tree_mask, right_tree_mask, main_chain, products_inside=True):
         lib = get_pcfg_kernel()
         _need_cuda("pcfg_extract_links", query_chunks, key_chunks_left, key_chunks_right, gate_logits, prev_output_tokens,
                    left_tree_mask, right_tree_mask, main_chain)
@@ -545,22 +547,30 @@ class PCFGExtractLinksFunc(Function):
             raise RuntimeError("pcfg_extract_links: tree masks must be [prelen, prelen] and main_chain [prelen]")
         dev = query_chunks.device
         code = _DTYPE_CODE[query_chunks.dtype]
-        fused = bool(lib.pcfgnat_extract_links_fused_supported(code, L, H, F))
+        fused = products_inside and bool(lib.pcfgnat_extract_links_fused_supported(code, L, H, F))
         with torch.cuda.device(dev):
             st = _stream(query_chunks)
             q, kl, kr = query_chunks.contiguous(), key_chunks_left.contiguous(), key_chunks_right.contiguous()
-            if fused and not any(ctx.needs_input_grad[:4]):
-                # the products on the matrix cores inside the one kernel; nothing is kept for a backward
+            fused_bwd = bool(lib.pcfgnat_extract_links_fused_backward_supported(code, L, H, F))
+            need_grad = any(ctx.needs_input_grad[:4])
+            ctx.fused = fused and (fused_bwd or not need_grad)
+            if ctx.fused:
+                # the products on the matrix cores inside the kernels: one launch forward, three backward
                 gate = gate_logits.float().contiguous()
                 prev = prev_output_tokens.to(torch.int64).contiguous()
                 masks = [t.contiguous() if t.dtype in (torch.bool, torch.uint8) else t.ne(0).contiguous()
                          for t in (left_tree_mask, right_tree_mask, main_chain)]
                 links = torch.empty((B, L, 2, L), dtype=torch.float32, device=dev)
                 lse = torch.empty((B, L, H), dtype=torch.float32, device=dev)
+                tile_masks = torch.empty((B, L, 1 + (L + 31) // 32), dtype=torch.int32, device=dev) if need_grad else None
                 _lib.check(lib.pcfgnat_extract_links_fused_forward(q.data_ptr(), kl.data_ptr(), kr.data_ptr(), code, gate.data_ptr(),
                                                                    prev.data_ptr(), int(pad_index), masks[0].data_ptr(),
                                                                    masks[1].data_ptr(), masks[2].data_ptr(), links.data_ptr(),
-                                                                   lse.data_ptr(), B, L, H, F, st), lib)
+                                                                   lse.data_ptr(), tile_masks.data_ptr() if need_grad else None,
+                                                                   B, L, H, F, st), lib)
+                if need_grad:
+                    ctx.save_for_backward(links, lse, tile_masks, q, kl, kr, gate)
+                    ctx.chunk_dtype, ctx.gate_dtype = query_chunks.dtype, gate_logits.dtype
                 return links
             A = torch.empty((B, H, 2 * L, F), dtype=torch.float32, device=dev)
             Kr = torch.empty((B, H, L, F), dtype=torch.float32, device=dev)
@@ -578,6 +588,7 @@ class PCFGExtractLinksFunc(Function):
                                                          masks[0].data_ptr(), masks[1].data_ptr(), masks[2].data_ptr(),
                                                          links.data_ptr(), lse.data_ptr(), B, L, H, F, st), lib)
         ctx.save_for_backward(links, lse, Z, A, Kr, gate, prev, *masks)
+        ctx.fused = False
         ctx.pad_index = int(pad_index)
         ctx.chunk_dtype, ctx.gate_dtype = query_chunks.dtype, gate_logits.dtype
         return links
@@ -585,6 +596,23 @@ class PCFGExtractLinksFunc(Function):
     @staticmethod
     def backward(ctx, grad_links):
         lib = get_pcfg_kernel()
+        if ctx.fused:
+            links, lse, tile_masks, q, kl, kr, gate = ctx.saved_tensors
+            B, L, H, F = q.shape
+            dev = q.device
+            code = _DTYPE_CODE[ctx.chunk_dtype]
+            with torch.cuda.device(dev):
+                st = _stream(q)
+                G = grad_links.float().contiguous()
+                dq, dkl, dkr = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+                dgate = torch.empty((B, L, H), dtype=torch.float32, device=dev)
+                ws = torch.empty((lib.pcfgnat_extract_links_fused_backward_workspace_bytes(B, L, H, F) + 3) // 4, dtype=torch.float32,
+                                 device=dev)
+                _lib.check(lib.pcfgnat_extract_links_fused_backward(G.data_ptr(), links.data_ptr(), lse.data_ptr(), tile_masks.data_ptr(),
+                                                                    q.data_ptr(), kl.data_ptr(), kr.data_ptr(), code, gate.data_ptr(),
+                                                                    dq.data_ptr(), dkl.data_ptr(), dkr.data_ptr(), dgate.data_ptr(),
+                                                                    ws.data_ptr(), B, L, H, F, st), lib)
+            return dq, dkl, dkr, dgate.to(ctx.gate_dtype), None, None, None, None, None, None
         links, lse, Z, A, Kr, gate, prev, ltm, rtm, mc = ctx.saved_tensors
         B, H, L2, F = A.shape
         L = L2 // 2
@@ -607,15 +635,16 @@ class PCFGExtractLinksFunc(Function):
             _lib.check(lib.pcfgnat_extract_links_unpack(dA.data_ptr(), dKr.data_ptr(), dsab.data_ptr(), A.data_ptr(),
                                                         _DTYPE_CODE[ctx.chunk_dtype], dq.data_ptr(), dkl.data_ptr(), dkr.data_ptr(),
                                                         B, L, H, F, st), lib)
-        return dq, dkl, dkr, dgate.to(ctx.gate_dtype), None, None, None, None, None
+        return dq, dkl, dkr, dgate.to(ctx.gate_dtype), None, None, None, None, None, None
 
 
 def pcfg_extract_links(query_chunks, key_chunks_left, key_chunks_right, gate_logits, prev_output_tokens, pad_index, left_tree_mask,
-                       right_tree_mask, main_chain):
+                       right_tree_mask, main_chain, products_inside=True):
     """links [bsz, prelen, 2, prelen] float32 from the projected chunks [bsz, prelen, heads, head_dim] and the gate logits
-    [bsz, prelen, heads]; differentiable in the first four arguments.  max_left = 1."""
+    [bsz, prelen, heads]; differentiable in the first four arguments.  max_left = 1.  products_inside=False takes the form
+    whose products go through torch's GEMM library also where the library's own kernels would cover the shape."""
     return PCFGExtractLinksFunc.apply(query_chunks, key_chunks_left, key_chunks_right, gate_logits, prev_output_tokens, pad_index,
-                                      left_tree_mask, right_tree_mask, main_chain)
+                                      left_tree_mask, right_tree_mask, main_chain, products_inside)
 
 
 GLANCE_STRATEGIES = {"number-random": 0, "cmlm": 1, None: 2}  # PCFGNAT_GLANCE_* of the library

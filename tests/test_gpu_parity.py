@@ -519,7 +519,7 @@ def test_extract_links_fused_form_rejects_what_it_does_not_cover():
     x = torch.zeros(1, 64, 3, 16, device=DEV, dtype=torch.float16)
     rc = lib.pcfgnat_extract_links_fused_forward(x.data_ptr(), x.data_ptr(), x.data_ptr(), ops._DTYPE_CODE[torch.float16], x.data_ptr(),
                                                  x.data_ptr(), 1, x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(),
-                                                 1, 64, 3, 16, None)
+                                                 None, 1, 64, 3, 16, None)
     assert rc != 0 and b"heads" in lib.pcfgnat_last_error()
 
 
