@@ -268,12 +268,13 @@ def link_scorer_timing(dev):
 
     G = G.masked_fill(~torch.isfinite(fwd()), 0)  # the upstream gradient of masked links is zero
 
-    def fwd_bwd():
+    def fwd_bwd(products_inside=True):
         ts = [t.detach().requires_grad_(True) for t in (q, kl, kr, gate)]
-        ops.pcfg_extract_links(*ts, prev, synth.PAD, lm, rm, mc).backward(G)
+        ops.pcfg_extract_links(*ts, prev, synth.PAD, lm, rm, mc, products_inside).backward(G)
 
     res = {}
-    for name, fn in (("forward_ms", fwd), ("forward_backward_ms", fwd_bwd)):
+    for name, fn in (("forward_ms", fwd), ("forward_backward_ms", fwd_bwd),
+                     ("forward_backward_products_through_torch_ms", lambda: fwd_bwd(False))):
         for _ in range(3):
             fn()
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -13,11 +13,12 @@
 //   d kr[c,h]     = sum_a ( (dz[a,0,c] + dz[a,1,c]) q[a,h] + dz[a,0,c] kl[0,h] + dz[a,1,c] kl[src(a,1),h] )
 // Three launches; the masks of every parent come from the forward.  The four waves of a workgroup work on four heads of
 // the same tiles and share nothing but the reading of links and G:
-//   parents:  one wave per (sentence, head, tile of 32 parents) runs over the tiles of right children twice (dg, then
-//             dz) and leaves d q, d kl (all rows but row 0), d gate and, for the other two launches, dg and ds;
-//   children: one wave per (sentence, head, tile of 32 right children) runs over the tiles of parents and leaves d kr
-//             and the column sums of dz[.,0,.];
-//   row 0:    d kl[0,h] from what the other two left.
+//   dg:       one wave per (sentence, head, tile of 32 parents) runs over the tiles of right children and leaves dg, d gate;
+//   main:     the same waves run over them again for dz and leave d q, d kl (all rows but row 0) and ds, while, in the
+//             same launch, one wave per (sentence, head, tile of 32 right children) runs over the tiles of parents and
+//             leaves d kr and the column sums of dz[.,0,.] (the two kinds of workgroups do not depend on each other and
+//             fill the device together);
+//   row 0:    d kl[0,h] from what the main launch left.
 // The products with dz run in fp32 (v_mfma_f32_32x32x2_f32, dz as one operand straight from the accumulator layout or
 // transposed through LDS); the scores use the same chunks and instructions as the forward.
 #include "links_fused.hip.h"
@@ -131,29 +132,75 @@ __device__ __forceinline__ void entries_read(const float *buf, int arr, int p, i
     }
 }
 
+// ---- fp16 chunks: the products with dz on the fp16 matrix instruction.  A value x S (S a power of two that brings the
+// largest |x| of the tile just below 2^14) is handed over as the sum of two fp16 numbers, hi = x S rounded toward zero
+// and lo = the rest, exact up to 2^-20 |x S| (2^-25 absolutely); the keys are fp16 already, so each product is two
+// instructions of 16 contraction steps instead of sixteen fp32 instructions of two.
+__device__ __forceinline__ void split_pair(float x0, float x1, float S, unsigned &hi, unsigned &lo) {
+    const float y0 = x0 * S, y1 = x1 * S;
+    const auto h = __builtin_amdgcn_cvt_pkrtz(y0, y1);
+    hi = __builtin_bit_cast(unsigned, h);
+    lo = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pkrtz(y0 - (float)h[0], y1 - (float)h[1]));
+}
+// the lane's entries r = 8m .. 8m+7 as the operand of step m
+__device__ __forceinline__ void split_operands(const float (&x)[16], float S, uint4 (&hi)[2], uint4 (&lo)[2]) {
+#pragma unroll
+    for (int m = 0; m < 2; m++) {
+        split_pair(x[8 * m + 0], x[8 * m + 1], S, hi[m].x, lo[m].x);
+        split_pair(x[8 * m + 2], x[8 * m + 3], S, hi[m].y, lo[m].y);
+        split_pair(x[8 * m + 4], x[8 * m + 5], S, hi[m].z, lo[m].z);
+        split_pair(x[8 * m + 6], x[8 * m + 7], S, hi[m].w, lo[m].w);
+    }
+}
+// S and 1 / S for a tile whose largest magnitude over the wave is mx; false: nothing to add (all zero, or too small to matter)
+__device__ __forceinline__ bool tile_scale(float mx, float &S, float &inv) {
+    const int e = ((__float_as_int(mx) >> 23) & 255) - 127;  // floor(log2(mx)) for normal numbers
+    if (!(mx > 0.f) || e < -100) return false;
+    const int es = e > 100 ? 100 : e;  // (beyond that the values are not finite in any useful sense)
+    S = __int_as_float((127 + 13 - es) << 23);
+    inv = __int_as_float((127 - 13 + es) << 23);
+    return true;
+}
+__device__ __forceinline__ floatx16 mma16(const uint4 &a, const uint4 &b, floatx16 acc) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), acc, 0, 0, 0);
+}
+__device__ __forceinline__ unsigned short half_bits(const uint4 &c, int i) {
+    const unsigned w = (i < 2) ? c.x : (i < 4) ? c.y : (i < 6) ? c.z : c.w;
+    return (unsigned short)(w >> (16 * (i & 1)));
+}
+// The tables in LDS are written and read through pointers of different types by the same wave (whose LDS operations
+// execute in order): this keeps the compiler from moving the reads above the writes.
+__device__ __forceinline__ void lds_order() { __asm__ volatile("" ::: "memory"); }
+constexpr int KT_PITCH = 36;  // halves per row of a transposed tile [element][32 rows]: 8-byte reads of 32 lanes fall into 64 banks
+
 // LDS per wave, in chunks: TILES tiles of 32 rows of one head (row pitch: the row plus one chunk) and one more row.
 template <int NCH, int TILES>
 constexpr int bwd_wave_chunks() {
     return TILES * PT * (2 * NCH + 1) + (2 * NCH + 1);
 }
 constexpr int BWD_TD_PITCH = 33;  // floats per row of a transposed 32 x 32 tile
+constexpr int DH_PITCH = 40;      // halves per row of a [right child][parent] plane: 16-byte reads of 16 lanes fall into 64 banks
+constexpr int BWD_TD_FLOATS = 4 * PT * DH_PITCH / 2;  // per wave: four fp16 planes, or two fp32 tiles and a row (fewer)
+static_assert(BWD_TD_FLOATS >= 2 * PT * BWD_TD_PITCH + PT, "transposed tiles of the children's launch");
 
-// ---- parents' launch.  grid (tiles of 32 parents, groups of four heads, B); wave w of the workgroup takes head
-// 4 * group + w (a wave without a head still helps to move the entries).  masks: [B,L,1+nw] words as the forward left
-// them (flags, then the allowed right children).
-template <typename T, int NCH>
-__global__ __launch_bounds__(LF_NT) void links_fused_bwd_parents_kernel(
-    const T *__restrict__ q, const T *__restrict__ kl, const T *__restrict__ kr, const float *__restrict__ gate,
-    const float *__restrict__ head_lse, const float *__restrict__ links, const float *__restrict__ G, const unsigned *__restrict__ masks,
-    T *__restrict__ dq, T *__restrict__ dkl, float *__restrict__ dgate, BwdWorkspace ws, int L, int H, float scale2, float scale) {
+// ---- the parents' part of a workgroup: blockIdx.x = tile of 32 parents, blockIdx.y = group of four heads, sentence b;
+// wave w takes head 4 * group + w (a wave without a head still helps to move the entries).  masks: [B,L,1+nw] words as
+// the forward left them (flags, then the allowed right children).  MODE 0: the run that gives dg (and d gate); MODE 1:
+// the run that gives dz and its products, with dg read back.
+template <typename T, int NCH, int MODE>
+__device__ __forceinline__ void bwd_parents(uint4 *lb_lds, int b, const T *__restrict__ q, const T *__restrict__ kl, const T *__restrict__ kr,
+                                            const float *__restrict__ gate, const float *__restrict__ head_lse,
+                                            const float *__restrict__ links, const float *__restrict__ G, const unsigned *__restrict__ masks,
+                                            T *__restrict__ dq, T *__restrict__ dkl, float *__restrict__ dgate, BwdWorkspace ws, int L, int H,
+                                            float scale2, float scale) {
     constexpr int EPC = Chunk<T>::EPC, F = 2 * NCH * EPC, FT = (F + 31) / 32, RPC = 2 * NCH + 1;
-    extern __shared__ uint4 lb_lds[];
     const int nw = (L + 31) / 32;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int b = blockIdx.z, a0 = blockIdx.x * PT, h = blockIdx.y * 4 + wave;
+    const int a0 = blockIdx.x * PT, h = blockIdx.y * 4 + wave;
     const bool active = h < H;
-    uint4 *tQ = lb_lds + wave * bwd_wave_chunks<NCH, 3>(), *tK1 = tQ + PT * RPC, *tKr = tK1 + PT * RPC, *tK0 = tKr + PT * RPC;
-    float *s_ent = reinterpret_cast<float *>(lb_lds + 4 * bwd_wave_chunks<NCH, 3>());  // two buffers of entries
+    constexpr int TILES = MODE == 0 ? 2 : 3;  // the run for dg keeps no table of the right keys
+    uint4 *tQ = lb_lds + wave * bwd_wave_chunks<NCH, TILES>(), *tK1 = tQ + PT * RPC, *tKr = tK1 + PT * RPC, *tK0 = tQ + TILES * PT * RPC;
+    float *s_ent = reinterpret_cast<float *>(lb_lds + 4 * bwd_wave_chunks<NCH, TILES>());  // two buffers of entries
     float *s_ds = s_ent + 2 * ENT_FLOATS + wave * 64;                                 // [2][32] per wave
     const int p = lane & 31, kb = lane >> 5, a = a0 + p;
     const bool in = a < L;
@@ -235,17 +282,17 @@ __global__ __launch_bounds__(LF_NT) void links_fused_bwd_parents_kernel(
     for (int t = 0; t < FT; t++)
 #pragma unroll
         for (int r = 0; r < 16; r++) accQ[t][r] = accK[t][r] = 0.f;
-    float dg = 0.f, gsum = 0.f, ds0 = 0.f, ds1 = 0.f;
+    float dg = (MODE == 1 && in) ? ws.dg[((size_t)b * L + a) * H + hh] : 0.f, gsum = 0.f, ds0 = 0.f, ds1 = 0.f;
     uint4 cur[NCH], nxt[NCH];
     unsigned allow_cur, allow_nxt;
     right_keys(0, cur, allow_cur);
     entries_store(s_ent, tid, ent);
     __syncthreads();
-    // ---- two runs over the tiles of right children as one sequence of steps: the first run gives dg = sum G w (and the sum
-    // of G over the finite links), the second dz and its products with the right keys
+    // ---- one run over the tiles of right children: dg = sum G w (and the sum of G over the finite links), or dz and its
+    // products with the right keys
 #pragma unroll 1
-    for (int s = 0; s < 2 * nw; s++) {
-        const int sn = min(s + 1, 2 * nw - 1), ctn = sn < nw ? sn : sn - nw;  // the tile of step s is s mod nw
+    for (int s = 0; s < nw; s++) {
+        const int ctn = min(s + 1, nw - 1);
         entries_request(links, G, b, a0, 32 * ctn, L, vec4, tid, ent);
         right_keys(ctn, nxt, allow_nxt);
         const float *buf = s_ent + (s & 1) * ENT_FLOATS;
@@ -256,22 +303,30 @@ __global__ __launch_bounds__(LF_NT) void links_fused_bwd_parents_kernel(
             entries_read(buf, 1, p, 0, kb, g0);
             entries_read(buf, 1, p, 1, kb, g1);
             scores(cur, allow_cur, z0, z1);
-            if (s < nw) {
+            if (MODE == 0) {
                 entry_gradients<true>(z0, z1, g0, g1, l0, l1, pt, 0.f, scale, dg, gsum, dz0, dz1);
                 if (s == nw - 1) {
                     dg += __shfl_xor(dg, 32);
                     gsum += __shfl_xor(gsum, 32);
                     if (in && kb == 0) {
-                        // (the sum over the heads of dg is the sum of G over the finite links)
-                        dgate[((size_t)b * L + a) * H + h] = dg - ex2(pt.lg2v) * gsum;
+                        // (the sum over the heads of dg is the sum of G over the finite links; a single head has a constant gate)
+                        dgate[((size_t)b * L + a) * H + h] = H == 1 ? 0.f : dg - ex2(pt.lg2v) * gsum;
                         ws.dg[((size_t)b * L + a) * H + h] = dg;
                         ws.lg[((size_t)b * L + a) * H + h] = pt.lg2v;
                     }
                 }
             } else {
-                // the right keys of the tile as a table [row][element] for the products below
+                // the right keys of the tile as a table for the products below: [row][element], for fp16 [element][row]
+                if constexpr (sizeof(T) == 2) {
+                    unsigned short *krt = reinterpret_cast<unsigned short *>(tKr);
 #pragma unroll
-                for (int j = 0; j < NCH; j++) tKr[p * RPC + 2 * j + kb] = cur[j];
+                    for (int j = 0; j < NCH; j++)
+#pragma unroll
+                        for (int i = 0; i < 8; i++) krt[((2 * j + kb) * 8 + i) * KT_PITCH + p] = half_bits(cur[j], i);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < NCH; j++) tKr[p * RPC + 2 * j + kb] = cur[j];
+                }
                 float unused_dg = 0.f, unused_gs = 0.f;
                 entry_gradients<false>(z0, z1, g0, g1, l0, l1, pt, dg, scale, unused_dg, unused_gs, dz0, dz1);
 #pragma unroll
@@ -280,19 +335,61 @@ __global__ __launch_bounds__(LF_NT) void links_fused_bwd_parents_kernel(
                     ds1 += dz1[r];
                 }
                 // d q[p][f] += sum_c (dz0 + dz1)[p][c] kr[c][f],  d kl[src(p)][f] += sum_c dz1[p][c] kr[c][f]: dz is already
-                // laid out as the row operand (lane: parent p, step r: right child acc_row(r, kb)); lane (f, kb) supplies
-                // kr[acc_row(r, kb)][f]
-                float kv[FT][16];
+                // laid out as the row operand (lane: parent p, right children acc_row(r, kb)); lane (f, kb) supplies the keys
+                // of the same right children
+                lds_order();
+                if constexpr (sizeof(T) == 2) {
+                    float dzs[16], mx = 0.f;
 #pragma unroll
-                for (int r = 0; r < 16; r++)
+                    for (int r = 0; r < 16; r++) {
+                        dzs[r] = dz0[r] + dz1[r];
+                        mx = fmaxf(mx, fmaxf(fabsf(dzs[r]), fabsf(dz1[r])));
+                    }
+                    float S, inv;
+                    if (tile_scale(wave_max(mx), S, inv)) {  // uniform
+                        uint4 hs[2], ls[2], h1[2], l1[2];
+                        split_operands(dzs, S, hs, ls);
+                        split_operands(dz1, S, h1, l1);
+                        const unsigned short *krt = reinterpret_cast<const unsigned short *>(tKr);
 #pragma unroll
-                    for (int t = 0; t < FT; t++) kv[t][r] = (32 * t + p < F) ? Chunk<T>::elem(tKr + acc_row(r, kb) * RPC, 32 * t + p) : 0.f;
+                        for (int t = 0; t < FT; t++) {
+                            const int f = 32 * t + p;
+                            floatx16 tq, tk;
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
+                            for (int r = 0; r < 16; r++) tq[r] = tk[r] = 0.f;
 #pragma unroll
-                    for (int t = 0; t < FT; t++) {
-                        accQ[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(dz0[r] + dz1[r], kv[t][r], accQ[t], 0, 0, 0);
-                        accK[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(dz1[r], kv[t][r], accK[t], 0, 0, 0);
+                            for (int m = 0; m < 2; m++) {  // the right children acc_row(8m .. 8m+7, kb): 16m + 4kb + {0..3, 8..11}
+                                uint4 bop = make_uint4(0, 0, 0, 0);
+                                if (f < F) {
+                                    const uint2 lo8 = *reinterpret_cast<const uint2 *>(krt + f * KT_PITCH + 16 * m + 4 * kb);
+                                    const uint2 hi8 = *reinterpret_cast<const uint2 *>(krt + f * KT_PITCH + 16 * m + 8 + 4 * kb);
+                                    bop = make_uint4(lo8.x, lo8.y, hi8.x, hi8.y);
+                                }
+                                tq = mma16(hs[m], bop, tq);
+                                tk = mma16(h1[m], bop, tk);
+                                tq = mma16(ls[m], bop, tq);
+                                tk = mma16(l1[m], bop, tk);
+                            }
+#pragma unroll
+                            for (int r = 0; r < 16; r++) {
+                                accQ[t][r] = __builtin_fmaf(tq[r], inv, accQ[t][r]);
+                                accK[t][r] = __builtin_fmaf(tk[r], inv, accK[t][r]);
+                            }
+                        }
+                    }
+                } else {
+                    float kv[FT][16];
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+#pragma unroll
+                        for (int t = 0; t < FT; t++) kv[t][r] = (32 * t + p < F) ? Chunk<T>::elem(tKr + acc_row(r, kb) * RPC, 32 * t + p) : 0.f;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+#pragma unroll
+                        for (int t = 0; t < FT; t++) {
+                            accQ[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(dz0[r] + dz1[r], kv[t][r], accQ[t], 0, 0, 0);
+                            accK[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(dz1[r], kv[t][r], accK[t], 0, 0, 0);
+                        }
                     }
                 }
             }
@@ -303,7 +400,7 @@ __global__ __launch_bounds__(LF_NT) void links_fused_bwd_parents_kernel(
         entries_store(s_ent + ((s + 1) & 1) * ENT_FLOATS, tid, ent);
         __syncthreads();
     }
-    if (!active) return;
+    if (!active || MODE == 0) return;
     ds0 += __shfl_xor(ds0, 32);
     ds1 += __shfl_xor(ds1, 32);
     if (kb == 0) {
@@ -314,6 +411,7 @@ __global__ __launch_bounds__(LF_NT) void links_fused_bwd_parents_kernel(
             ws.ds[(((size_t)b * H + h) * L + a) * 2 + 1] = ds1;
         }
     }
+    lds_order();
     // ---- the q.kl terms and the stores: lane (f, kb) holds the parents acc_row(r, kb) of column f
 #pragma unroll
     for (int t = 0; t < FT; t++) {
@@ -332,32 +430,33 @@ __global__ __launch_bounds__(LF_NT) void links_fused_bwd_parents_kernel(
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int ar = a0 + acc_row(r, kb);
-            if (ar >= L) continue;
-            dq[((size_t)b * L + ar) * HF + (size_t)h * F + f] = Chunk<T>::cast(accQ[t][r] + d0[r] * k0f + d1[r] * (ar == 0 ? k0f : k1f[r]));
             const float dk = accK[t][r] + (ar >= 1 ? d1[r] * qf[r] : 0.f);
             const int src = (ar - 1 < 0) ? L - 1 : ar - 1;
-            if (src == 0) ws.row0[((size_t)b * H + h) * F + f] = dk;  // completed by the last launch
-            else dkl[((size_t)b * L + src) * HF + (size_t)h * F + f] = Chunk<T>::cast(dk);
+            if (ar < L) {
+                dq[((size_t)b * L + ar) * HF + (size_t)h * F + f] = Chunk<T>::cast(accQ[t][r] + d0[r] * k0f + d1[r] * (ar == 0 ? k0f : k1f[r]));
+                dkl[((size_t)b * L + src) * HF + (size_t)h * F + f] = Chunk<T>::cast(dk);  // (row 0 is written again by the last launch)
+            }
+            if (a0 == 0 && acc_row(r, kb) == 1) ws.row0[((size_t)b * H + h) * F + f] = dk;  // parent 1: row 0 as far as it gets here
         }
     }
 }
 
-// ---- children's launch.  grid (tiles of 32 right children, groups of four heads, B); wave w takes head 4 * group + w.
+// ---- the children's part of a workgroup: blockIdx.x = tile of 32 right children, blockIdx.y = group of four heads,
+// sentence b; wave w takes head 4 * group + w.
 template <typename T, int NCH>
-__global__ __launch_bounds__(LF_NT) void links_fused_bwd_children_kernel(
-    const T *__restrict__ q, const T *__restrict__ kl, const T *__restrict__ kr, const float *__restrict__ head_lse,
-    const float *__restrict__ links, const float *__restrict__ G, const unsigned *__restrict__ masks, T *__restrict__ dkr, BwdWorkspace ws,
-    int L, int H, float scale2, float scale) {
+__device__ __forceinline__ void bwd_children(uint4 *lb_lds, int b, const T *__restrict__ q, const T *__restrict__ kl, const T *__restrict__ kr,
+                                             const float *__restrict__ head_lse, const float *__restrict__ links,
+                                             const float *__restrict__ G, const unsigned *__restrict__ masks, T *__restrict__ dkr,
+                                             BwdWorkspace ws, int L, int H, float scale2, float scale) {
     constexpr int EPC = Chunk<T>::EPC, F = 2 * NCH * EPC, FT = (F + 31) / 32, RPC = 2 * NCH + 1;
-    extern __shared__ uint4 lb_lds[];
     const int nw = (L + 31) / 32;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int b = blockIdx.z, ct = blockIdx.x, c0 = ct * PT, h = blockIdx.y * 4 + wave;
+    const int ct = blockIdx.x, c0 = ct * PT, h = blockIdx.y * 4 + wave;
     const bool active = h < H;
     const int hh = active ? h : 0;
     uint4 *tQ = lb_lds + wave * bwd_wave_chunks<NCH, 2>(), *tK1 = tQ + PT * RPC, *tK0 = tK1 + PT * RPC;
     float *s_ent = reinterpret_cast<float *>(lb_lds + 4 * bwd_wave_chunks<NCH, 2>());
-    float *tD = s_ent + 2 * ENT_FLOATS + wave * (2 * PT * BWD_TD_PITCH + PT);  // [2][32][33], [32]
+    float *tD = s_ent + 2 * ENT_FLOATS + wave * BWD_TD_FLOATS;  // fp32: [2][32][33], [32]; fp16: four planes
     float *s_cs = tD + 2 * PT * BWD_TD_PITCH;
     const int p = lane & 31, kb = lane >> 5;
     const int HF = H * F;
@@ -405,7 +504,9 @@ __global__ __launch_bounds__(LF_NT) void links_fused_bwd_children_kernel(
     for (int t = 0; t < FT; t++)
 #pragma unroll
         for (int r = 0; r < 16; r++) accR[t][r] = 0.f;
-    float cs0 = 0.f;
+    float cs0 = 0.f, csum[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) csum[r] = 0.f;
     ParentLoad cur, nxt;
     parent_request(0, cur);
     entries_store(s_ent, tid, ent);
@@ -426,8 +527,17 @@ __global__ __launch_bounds__(LF_NT) void links_fused_bwd_children_kernel(
             float sab0 = 0.f, sab1 = 0.f;
 #pragma unroll
             for (int j = 0; j < NCH; j++) {
-                tQ[p * RPC + 2 * j + kb] = cur.vq[j];
-                tK1[p * RPC + 2 * j + kb] = cur.vk[j];
+                if constexpr (sizeof(T) == 2) {  // [element][parent]
+                    unsigned short *qt = reinterpret_cast<unsigned short *>(tQ), *k1t = reinterpret_cast<unsigned short *>(tK1);
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        qt[((2 * j + kb) * 8 + i) * KT_PITCH + p] = half_bits(cur.vq[j], i);
+                        k1t[((2 * j + kb) * 8 + i) * KT_PITCH + p] = half_bits(cur.vk[j], i);
+                    }
+                } else {  // [parent][element]
+                    tQ[p * RPC + 2 * j + kb] = cur.vq[j];
+                    tK1[p * RPC + 2 * j + kb] = cur.vk[j];
+                }
                 const uint4 v0 = tK0[2 * j + kb];
                 sab0 = Chunk<T>::dot(cur.vq[j], v0, sab0);
                 sab1 = Chunk<T>::dot(cur.vq[j], a == 0 ? v0 : cur.vk[j], sab1);
@@ -463,34 +573,116 @@ __global__ __launch_bounds__(LF_NT) void links_fused_bwd_children_kernel(
             entries_read(buf, 1, p, 1, kb, g1);
             float unused_dg = 0.f, unused_gs = 0.f;
             entry_gradients<false>(z0, z1, g0, g1, l0, l1, ptm, cur.dgv, scale, unused_dg, unused_gs, dz0, dz1);
-            // transposed through LDS: tD[k][parent][right child], read back with the right child as the row of the operand
+            // d kr[c][f] += sum_p (dz0 + dz1)[p][c] q[p][f] + sum_p dz1[p][c] kl[src(p)][f], and the column sums of dz0: dz goes
+            // through LDS to the lanes of its right child (the row of the operand), lane (f, kb) supplies the parents' rows
+            if constexpr (sizeof(T) == 2) {
+                float dzs[16], mx = 0.f;
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                tD[p * BWD_TD_PITCH + acc_row(r, kb)] = dz0[r];
-                tD[(PT + p) * BWD_TD_PITCH + acc_row(r, kb)] = dz1[r];
-            }
-            // d kr[c][f] += sum_p (dz0 + dz1)[p][c] q[p][f] + sum_p dz1[p][c] kl[src(p)][f]: lane (c, kb) supplies the gradients
-            // of parent 2 s + kb in step s, lane (f, kb) the elements of that parent's rows
-            float d0v[16], d1v[16], qv[FT][16], kv[FT][16];
-#pragma unroll
-            for (int s = 0; s < 16; s++) {  // every read before the first product
-                const int pp = 2 * s + kb;
-                d0v[s] = tD[pp * BWD_TD_PITCH + p];
-                d1v[s] = tD[(PT + pp) * BWD_TD_PITCH + p];
-#pragma unroll
-                for (int t = 0; t < FT; t++) {
-                    const int f = 32 * t + p;
-                    qv[t][s] = (f < F) ? Chunk<T>::elem(tQ + pp * RPC, f) : 0.f;
-                    kv[t][s] = (f < F) ? Chunk<T>::elem(tK1 + pp * RPC, f) : 0.f;
+                for (int r = 0; r < 16; r++) {
+                    dzs[r] = dz0[r] + dz1[r];
+                    mx = fmaxf(mx, fmaxf(fabsf(dzs[r]), fabsf(dz1[r])));
                 }
-            }
+                float S, inv;
+                if (tile_scale(wave_max(mx), S, inv)) {  // uniform
+                    // four planes [right child][parent] of fp16: dz0 + dz1 as hi and lo, dz1 as hi and lo
+                    unsigned short *dh = reinterpret_cast<unsigned short *>(tD);
 #pragma unroll
-            for (int s = 0; s < 16; s++) {
-                cs0 += d0v[s];
+                    for (int r = 0; r < 16; r += 2) {
+                        unsigned hs, ls, h1, l1;
+                        split_pair(dzs[r], dzs[r + 1], S, hs, ls);
+                        split_pair(dz1[r], dz1[r + 1], S, h1, l1);
+                        const int c_a = acc_row(r, kb) * DH_PITCH + p, c_b = acc_row(r + 1, kb) * DH_PITCH + p;
+                        dh[0 * PT * DH_PITCH + c_a] = (unsigned short)hs;
+                        dh[0 * PT * DH_PITCH + c_b] = (unsigned short)(hs >> 16);
+                        dh[1 * PT * DH_PITCH + c_a] = (unsigned short)ls;
+                        dh[1 * PT * DH_PITCH + c_b] = (unsigned short)(ls >> 16);
+                        dh[2 * PT * DH_PITCH + c_a] = (unsigned short)h1;
+                        dh[2 * PT * DH_PITCH + c_b] = (unsigned short)(h1 >> 16);
+                        dh[3 * PT * DH_PITCH + c_a] = (unsigned short)l1;
+                        dh[3 * PT * DH_PITCH + c_b] = (unsigned short)(l1 >> 16);
+                    }
+                    lds_order();
+                    // step m: the parents 16m + 8kb .. + 7
+                    uint4 aop[4][2];
 #pragma unroll
-                for (int t = 0; t < FT; t++) {
-                    accR[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(d0v[s] + d1v[s], qv[t][s], accR[t], 0, 0, 0);
-                    accR[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(d1v[s], kv[t][s], accR[t], 0, 0, 0);
+                    for (int pl = 0; pl < 4; pl++)
+#pragma unroll
+                        for (int m = 0; m < 2; m++)
+                            aop[pl][m] = *reinterpret_cast<const uint4 *>(dh + pl * PT * DH_PITCH + p * DH_PITCH + 16 * m + 8 * kb);
+                    const unsigned short *qt = reinterpret_cast<const unsigned short *>(tQ), *k1t = reinterpret_cast<const unsigned short *>(tK1);
+#pragma unroll
+                    for (int t = 0; t < FT; t++) {
+                        const int f = 32 * t + p;
+                        floatx16 tr;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) tr[r] = 0.f;
+#pragma unroll
+                        for (int m = 0; m < 2; m++) {
+                            uint4 bq = make_uint4(0, 0, 0, 0), bk = bq;
+                            if (f < F) {
+                                const uint2 q0 = *reinterpret_cast<const uint2 *>(qt + f * KT_PITCH + 16 * m + 8 * kb);
+                                const uint2 q1 = *reinterpret_cast<const uint2 *>(qt + f * KT_PITCH + 16 * m + 8 * kb + 4);
+                                const uint2 k0 = *reinterpret_cast<const uint2 *>(k1t + f * KT_PITCH + 16 * m + 8 * kb);
+                                const uint2 k1 = *reinterpret_cast<const uint2 *>(k1t + f * KT_PITCH + 16 * m + 8 * kb + 4);
+                                bq = make_uint4(q0.x, q0.y, q1.x, q1.y);
+                                bk = make_uint4(k0.x, k0.y, k1.x, k1.y);
+                            }
+                            tr = mma16(aop[0][m], bq, tr);
+                            tr = mma16(aop[2][m], bk, tr);
+                            tr = mma16(aop[1][m], bq, tr);
+                            tr = mma16(aop[3][m], bk, tr);
+                        }
+#pragma unroll
+                        for (int r = 0; r < 16; r++) accR[t][r] = __builtin_fmaf(tr[r], inv, accR[t][r]);
+                    }
+                    // the column sums of dz0 = (dz0 + dz1) - dz1: a product with a column of ones (every column of the result)
+                    floatx16 tc;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) tc[r] = 0.f;
+                    const uint4 ones = make_uint4(0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u);
+#pragma unroll
+                    for (int m = 0; m < 2; m++) {
+                        const uint4 n1 = make_uint4(aop[2][m].x ^ 0x80008000u, aop[2][m].y ^ 0x80008000u, aop[2][m].z ^ 0x80008000u,
+                                                    aop[2][m].w ^ 0x80008000u);
+                        const uint4 n3 = make_uint4(aop[3][m].x ^ 0x80008000u, aop[3][m].y ^ 0x80008000u, aop[3][m].z ^ 0x80008000u,
+                                                    aop[3][m].w ^ 0x80008000u);
+                        tc = mma16(aop[0][m], ones, tc);
+                        tc = mma16(n1, ones, tc);
+                        tc = mma16(aop[1][m], ones, tc);
+                        tc = mma16(n3, ones, tc);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 16; r++) csum[r] = __builtin_fmaf(tc[r], inv, csum[r]);
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    tD[p * BWD_TD_PITCH + acc_row(r, kb)] = dz0[r];
+                    tD[(PT + p) * BWD_TD_PITCH + acc_row(r, kb)] = dz1[r];
+                }
+                lds_order();
+                // lane (c, kb) supplies the gradients of parent 2 s + kb in step s, lane (f, kb) the elements of that parent's rows
+                float d0v[16], d1v[16], qv[FT][16], kv[FT][16];
+#pragma unroll
+                for (int s = 0; s < 16; s++) {  // every read before the first product
+                    const int pp = 2 * s + kb;
+                    d0v[s] = tD[pp * BWD_TD_PITCH + p];
+                    d1v[s] = tD[(PT + pp) * BWD_TD_PITCH + p];
+#pragma unroll
+                    for (int t = 0; t < FT; t++) {
+                        const int f = 32 * t + p;
+                        qv[t][s] = (f < F) ? Chunk<T>::elem(tQ + pp * RPC, f) : 0.f;
+                        kv[t][s] = (f < F) ? Chunk<T>::elem(tK1 + pp * RPC, f) : 0.f;
+                    }
+                }
+#pragma unroll
+                for (int s = 0; s < 16; s++) {
+                    cs0 += d0v[s];
+#pragma unroll
+                    for (int t = 0; t < FT; t++) {
+                        accR[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(d0v[s] + d1v[s], qv[t][s], accR[t], 0, 0, 0);
+                        accR[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(d1v[s], kv[t][s], accR[t], 0, 0, 0);
+                    }
                 }
             }
         }
@@ -499,26 +691,62 @@ __global__ __launch_bounds__(LF_NT) void links_fused_bwd_children_kernel(
         __syncthreads();
     }
     if (!active) return;
-    cs0 += __shfl_xor(cs0, 32);  // lane (c, kb) summed the parents of its half
-    if (kb == 0) {
-        s_cs[p] = cs0;
-        if (c0 + p < L) ws.cs[((size_t)b * H + h) * L + c0 + p] = cs0;
+    // ---- the column sums: per lane for the right children acc_row(r, kb) it stores below
+    if constexpr (sizeof(T) == 2) {
+        if (p == 0) {
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                if (c0 + acc_row(r, kb) < L) ws.cs[((size_t)b * H + h) * L + c0 + acc_row(r, kb)] = csum[r];
+        }
+    } else {
+        cs0 += __shfl_xor(cs0, 32);  // lane (c, kb) summed the parents of its half
+        if (kb == 0) {
+            s_cs[p] = cs0;
+            if (c0 + p < L) ws.cs[((size_t)b * H + h) * L + c0 + p] = cs0;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) csum[r] = s_cs[acc_row(r, kb)];
     }
+    lds_order();
     // ---- the null option's left key and the stores: lane (f, kb) holds the right children acc_row(r, kb) of column f
 #pragma unroll
     for (int t = 0; t < FT; t++) {
         const int f = 32 * t + p;
         if (f >= F) continue;
         const float k0f = Chunk<T>::elem(tK0, f);
-        float csr[16];
-#pragma unroll
-        for (int r = 0; r < 16; r++) csr[r] = s_cs[acc_row(r, kb)];
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int c = c0 + acc_row(r, kb);
-            if (c < L) dkr[((size_t)b * L + c) * HF + (size_t)h * F + f] = Chunk<T>::cast(accR[t][r] + csr[r] * k0f);
+            if (c < L) dkr[((size_t)b * L + c) * HF + (size_t)h * F + f] = Chunk<T>::cast(accR[t][r] + csum[r] * k0f);
         }
     }
+}
+
+// ---- first launch: dg, d gate.  grid (tiles of 32 parents, groups of four heads, B)
+template <typename T, int NCH>
+__global__ __launch_bounds__(LF_NT) void links_fused_bwd_dg_kernel(const T *__restrict__ q, const T *__restrict__ kl, const T *__restrict__ kr,
+                                                                  const float *__restrict__ gate, const float *__restrict__ head_lse,
+                                                                  const float *__restrict__ links, const float *__restrict__ G,
+                                                                  const unsigned *__restrict__ masks, float *__restrict__ dgate,
+                                                                  BwdWorkspace ws, int L, int H, float scale2, float scale) {
+    extern __shared__ uint4 lb_lds[];
+    bwd_parents<T, NCH, 0>(lb_lds, blockIdx.z, q, kl, kr, gate, head_lse, links, G, masks, nullptr, nullptr, dgate, ws, L, H, scale2, scale);
+}
+
+// ---- second launch: the parents' and the children's parts side by side, so that the device is filled by both.
+// grid (tiles of 32, groups of four heads, 2 B): sentence blockIdx.z as parents for blockIdx.z < B, else blockIdx.z - B as children.
+template <typename T, int NCH>
+__global__ __launch_bounds__(LF_NT) void links_fused_bwd_main_kernel(const T *__restrict__ q, const T *__restrict__ kl, const T *__restrict__ kr,
+                                                                    const float *__restrict__ gate, const float *__restrict__ head_lse,
+                                                                    const float *__restrict__ links, const float *__restrict__ G,
+                                                                    const unsigned *__restrict__ masks, T *__restrict__ dq, T *__restrict__ dkl,
+                                                                    T *__restrict__ dkr, BwdWorkspace ws, int B, int L, int H, float scale2,
+                                                                    float scale) {
+    extern __shared__ uint4 lb_lds[];
+    if ((int)blockIdx.z < B)
+        bwd_parents<T, NCH, 1>(lb_lds, blockIdx.z, q, kl, kr, gate, head_lse, links, G, masks, dq, dkl, nullptr, ws, L, H, scale2, scale);
+    else
+        bwd_children<T, NCH>(lb_lds, blockIdx.z - B, q, kl, kr, head_lse, links, G, masks, dkr, ws, L, H, scale2, scale);
 }
 
 // ---- d kl[0,h]: what the parents' launch left, the null option of every parent and parent 0's clamped left option.
@@ -553,8 +781,12 @@ constexpr size_t bwd_parents_lds_bytes() {
     return (size_t)4 * bwd_wave_chunks<NCH, 3>() * 16 + sizeof(float) * (2 * ENT_FLOATS + 4 * 64);
 }
 template <int NCH>
+constexpr size_t bwd_dg_lds_bytes() {
+    return (size_t)4 * bwd_wave_chunks<NCH, 2>() * 16 + sizeof(float) * (2 * ENT_FLOATS + 4 * 64);
+}
+template <int NCH>
 constexpr size_t bwd_children_lds_bytes() {
-    return (size_t)4 * bwd_wave_chunks<NCH, 2>() * 16 + sizeof(float) * (2 * ENT_FLOATS + 4 * (2 * PT * BWD_TD_PITCH + PT));
+    return (size_t)4 * bwd_wave_chunks<NCH, 2>() * 16 + sizeof(float) * (2 * ENT_FLOATS + 4 * BWD_TD_FLOATS);
 }
 static_assert(bwd_parents_lds_bytes<8>() <= 160 * 1024 && bwd_children_lds_bytes<8>() <= 160 * 1024, "LDS of the backward kernels");
 
@@ -563,19 +795,19 @@ int launch_fused_bwd(const void *q, const void *kl, const void *kr, const float 
                      const unsigned *masks, void *dq, void *dkl, void *dkr, float *dgate, float *wsp, int64_t B, int64_t L, int64_t H,
                      hipStream_t s) {
     constexpr int F = 2 * NCH * Chunk<T>::EPC;
-    const size_t lds_p = bwd_parents_lds_bytes<NCH>(), lds_c = bwd_children_lds_bytes<NCH>();
+    const size_t lds_p = bwd_parents_lds_bytes<NCH>(), lds_c = bwd_children_lds_bytes<NCH>(), lds_m = lds_p > lds_c ? lds_p : lds_c;
     const BwdWorkspace ws = bwd_workspace(wsp, B, L, H, F);
     const unsigned tiles = (unsigned)((L + PT - 1) / PT), groups = (unsigned)((H + 3) / 4);
     const float scale = 1.0f / sqrtf((float)F);
-    auto kp = links_fused_bwd_parents_kernel<T, NCH>;
-    PCFGNAT_DYNAMIC_LDS(kp, lds_p);
-    hipLaunchKernelGGL(kp, dim3(tiles, groups, (unsigned)B), dim3(LF_NT), lds_p, s, (const T *)q, (const T *)kl, (const T *)kr, gate, lse, links, G,
-                       masks, (T *)dq, (T *)dkl, dgate, ws, (int)L, (int)H, scale * LF_LOG2E, scale);
+    auto kd = links_fused_bwd_dg_kernel<T, NCH>;
+    PCFGNAT_DYNAMIC_LDS(kd, bwd_dg_lds_bytes<NCH>());
+    hipLaunchKernelGGL(kd, dim3(tiles, groups, (unsigned)B), dim3(LF_NT), bwd_dg_lds_bytes<NCH>(), s, (const T *)q, (const T *)kl, (const T *)kr, gate, lse, links, G,
+                       masks, dgate, ws, (int)L, (int)H, scale * LF_LOG2E, scale);
     PCFGNAT_HIP_CHECK(hipGetLastError());
-    auto kc = links_fused_bwd_children_kernel<T, NCH>;
-    PCFGNAT_DYNAMIC_LDS(kc, lds_c);
-    hipLaunchKernelGGL(kc, dim3(tiles, groups, (unsigned)B), dim3(LF_NT), lds_c, s, (const T *)q, (const T *)kl, (const T *)kr, lse, links, G, masks,
-                       (T *)dkr, ws, (int)L, (int)H, scale * LF_LOG2E, scale);
+    auto km = links_fused_bwd_main_kernel<T, NCH>;
+    PCFGNAT_DYNAMIC_LDS(km, lds_m);
+    hipLaunchKernelGGL(km, dim3(tiles, groups, (unsigned)(2 * B)), dim3(LF_NT), lds_m, s, (const T *)q, (const T *)kl, (const T *)kr, gate, lse, links,
+                       G, masks, (T *)dq, (T *)dkl, (T *)dkr, ws, (int)B, (int)L, (int)H, scale * LF_LOG2E, scale);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL((links_fused_bwd_row0_kernel<T>), dim3((unsigned)(B * H)), dim3(256), 0, s, (const T *)q, (const T *)kr, (T *)dkl, ws,
                        (int)L, (int)H, F);
@@ -606,8 +838,8 @@ extern "C" int pcfgnat_extract_links_fused_backward(const float *grad_links, con
                                                     const void *key_chunks_right, int dtype, const float *gate_logits, void *dq, void *dkl,
                                                     void *dkr, float *dgate, float *workspace, int64_t B, int64_t L, int64_t H, int64_t F,
                                                     void *stream) {
-    PCFGNAT_REQUIRE(B >= 0 && L >= 2 && F >= 1, "extract_links_fused_backward: bad dimensions (B=%lld L=%lld F=%lld)", (long long)B,
-                    (long long)L, (long long)F);
+    PCFGNAT_REQUIRE(B >= 0 && B <= 32767 && L >= 2 && F >= 1, "extract_links_fused_backward: bad dimensions (B=%lld L=%lld F=%lld)",
+                    (long long)B, (long long)L, (long long)F);
     if (!pcfgnat_extract_links_fused_backward_supported(dtype, L, H, F))
         return fail(PCFGNAT_EUNSUPPORTED, "extract_links_fused_backward: dtype code %d, L = %lld, %lld heads of %lld is not built", dtype,
                     (long long)L, (long long)H, (long long)F);

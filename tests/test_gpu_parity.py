@@ -452,8 +452,12 @@ def test_glat_single_call_small_ragged(ml):
 
 @pytest.mark.parametrize("B,L,H,F,dtype", [(3, 18, 2, 4, torch.float32), (2, 34, 8, 16, torch.float32), (4, 128, 8, 64, torch.float16),
                                             (2, 514, 4, 8, torch.float32), (2, 22, 16, 8, torch.float32), (2, 12, 1, 8, torch.float32),
-                                            (2, 200, 4, 16, torch.float16), (2, 256, 2, 24, torch.float32)])
-def test_extract_links_forward_backward_vs_torch_restatement(B, L, H, F, dtype):
+                                            (2, 200, 4, 16, torch.float16), (2, 256, 2, 24, torch.float32), (3, 130, 8, 64, torch.float32),
+                                            (2, 66, 16, 32, torch.float16), (2, 96, 2, 64, torch.float16)])
+@pytest.mark.parametrize("products_inside", [True, False])
+def test_extract_links_forward_backward_vs_torch_restatement(B, L, H, F, dtype, products_inside):
+    """Both forms of the scorer (products on the matrix cores inside the kernels where the shape is covered; products
+    through torch's GEMM library) against the float64 restatement: links and all four gradients."""
     from oracle import extract_links_ref as ref
     g = torch.Generator().manual_seed(L + H)
     q, kl, kr = ((torch.randn(B, L, H, F, generator=g) * 0.7).to(dtype) for _ in range(3))
@@ -468,7 +472,7 @@ def test_extract_links_forward_backward_vs_torch_restatement(B, L, H, F, dtype):
     G = torch.randn(want.shape, generator=g, dtype=torch.float64).masked_fill(~fin, 0)
     want.masked_fill(~fin, 0).mul(G).sum().backward()
     dleaves = [t.to(DEV).requires_grad_(True) for t in (q, kl, kr, gate)]
-    got = ops.pcfg_extract_links(*dleaves, prev.to(DEV), synth.PAD, lm.to(DEV), rm.to(DEV), mc.to(DEV))
+    got = ops.pcfg_extract_links(*dleaves, prev.to(DEV), synth.PAD, lm.to(DEV), rm.to(DEV), mc.to(DEV), products_inside)
     assert got.dtype == torch.float32 and torch.equal(torch.isfinite(got).cpu(), fin)
     assert torch.allclose(got.cpu().double()[fin], want.detach()[fin], rtol=2e-5, atol=2e-5)
     got.masked_fill(~fin.to(DEV), 0).mul(G.float().to(DEV)).sum().backward()
@@ -484,9 +488,9 @@ def test_extract_links_forward_backward_vs_torch_restatement(B, L, H, F, dtype):
                                             (2, 22, 16, 8, torch.float32), (2, 12, 1, 8, torch.float32), (2, 200, 4, 16, torch.float16),
                                             (3, 130, 8, 64, torch.float32), (2, 66, 16, 32, torch.float16), (2, 40, 2, 128, torch.float16)])
 def test_extract_links_products_inside_the_kernel(B, L, H, F, dtype):
-    """The scorer with its three products on the matrix cores inside the kernel (what `pcfg_extract_links` runs when no
-    gradient is asked for): links against the float64 restatement, the per-head normalisers against the five-call form,
-    graphs that are no multiple of the 32-wide tiles, padded sentences, 1 to 16 heads."""
+    """The scorer's forward with its three products on the matrix cores inside the kernel, also at head dimension 128
+    (where only the forward is built): links against the float64 restatement and against the five-call form, graphs that
+    are no multiple of the 32-wide tiles, padded sentences, 1 to 16 heads."""
     from oracle import extract_links_ref as ref
     lib = ops.get_pcfg_kernel()
     assert lib.pcfgnat_extract_links_fused_supported(ops._DTYPE_CODE[dtype], L, H, F) == 1
@@ -503,9 +507,9 @@ def test_extract_links_products_inside_the_kernel(B, L, H, F, dtype):
         got = ops.pcfg_extract_links(*dev, prev.to(DEV), synth.PAD, lm.to(DEV), rm.to(DEV), mc.to(DEV))
     assert got.dtype == torch.float32 and torch.equal(torch.isfinite(got).cpu(), fin)
     assert torch.allclose(got.cpu().double()[fin], want[fin], rtol=2e-5, atol=2e-5)
-    # the five-call form (taken when a gradient is needed) gives the same links
-    leaves = [t.clone().requires_grad_(True) for t in dev]
-    other = ops.pcfg_extract_links(*leaves, prev.to(DEV), synth.PAD, lm.to(DEV), rm.to(DEV), mc.to(DEV)).detach()
+    # the five-call form gives the same links
+    with torch.no_grad():
+        other = ops.pcfg_extract_links(*dev, prev.to(DEV), synth.PAD, lm.to(DEV), rm.to(DEV), mc.to(DEV), False)
     assert torch.equal(torch.isfinite(other), torch.isfinite(got))
     assert torch.allclose(got[fin.to(DEV)], other[fin.to(DEV)], rtol=2e-5, atol=2e-5)
 
@@ -516,6 +520,8 @@ def test_extract_links_fused_form_rejects_what_it_does_not_cover():
     assert lib.pcfgnat_extract_links_fused_supported(ops._DTYPE_CODE[torch.float64], 64, 2, 16) == 0    # dtype
     assert lib.pcfgnat_extract_links_fused_supported(ops._DTYPE_CODE[torch.float16], 64, 3, 16) == 0    # heads
     assert lib.pcfgnat_extract_links_fused_supported(ops._DTYPE_CODE[torch.float32], 64, 16, 64) == 0   # tile rows beyond the LDS
+    assert lib.pcfgnat_extract_links_fused_backward_supported(ops._DTYPE_CODE[torch.float16], 64, 2, 128) == 0  # backward: up to 64
+    assert lib.pcfgnat_extract_links_fused_backward_supported(ops._DTYPE_CODE[torch.float16], 64, 2, 64) == 1
     x = torch.zeros(1, 64, 3, 16, device=DEV, dtype=torch.float16)
     rc = lib.pcfgnat_extract_links_fused_forward(x.data_ptr(), x.data_ptr(), x.data_ptr(), ops._DTYPE_CODE[torch.float16], x.data_ptr(),
                                                  x.data_ptr(), 1, x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(),
