@@ -54,12 +54,22 @@ struct ParentTerms {
     float lse2;        // lse (0 likewise)
     float lg2v;        // log gate
 };
-__device__ __forceinline__ void gate_terms(const float *__restrict__ grow, int H, int h, float lse, ParentTerms &pt) {
-    float mx = NEG_INF_F;
-    for (int j = 0; j < H; j++) mx = fmaxf(mx, grow[j]);
+// log2 of the gate of head h from the row of gate logits (H <= 16; every load of the row in flight together)
+__device__ __forceinline__ float log2_gate(const float *__restrict__ grow, int H, int h) {
+    float gv[16], mx = NEG_INF_F, mine = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; j++) gv[j] = (j < H) ? grow[j] : NEG_INF_F;
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        mx = fmaxf(mx, gv[j]);
+        mine = (j == h) ? gv[j] : mine;
+    }
     float sum = 0.f;
-    for (int j = 0; j < H; j++) sum += ex2((grow[j] - mx) * LF_LOG2E);
-    pt.lg2v = (grow[h] - mx) * LF_LOG2E - lg2(sum);
+#pragma unroll
+    for (int j = 0; j < 16; j++) sum += ex2((gv[j] - mx) * LF_LOG2E);
+    return (mine - mx) * LF_LOG2E - lg2(sum);
+}
+__device__ __forceinline__ void lse_terms(float lse, ParentTerms &pt) {
     pt.lse2 = (lse == NEG_INF_F) ? 0.f : lse * LF_LOG2E;
     pt.off = (lse == NEG_INF_F) ? 0.f : pt.lg2v - pt.lse2;
 }
@@ -227,7 +237,8 @@ __device__ __forceinline__ void bwd_parents(uint4 *lb_lds, int b, const T *__res
             v0[j] = k0row[2 * j + kb];
         }
         const float lse = head_lse[((size_t)b * L + ai) * H + hh];
-        gate_terms(gate + ((size_t)b * L + ai) * H, H, hh, lse, pt);
+        pt.lg2v = MODE == 0 ? log2_gate(gate + ((size_t)b * L + ai) * H, H, hh) : ws.lg[((size_t)b * L + ai) * H + hh];
+        lse_terms(lse, pt);
 #pragma unroll
         for (int j = 0; j < NCH; j++) {
             tQ[p * RPC + 2 * j + kb] = vq[j];
@@ -521,8 +532,7 @@ __device__ __forceinline__ void bwd_children(uint4 *lb_lds, int b, const T *__re
             const int a = 32 * pt + p;
             ParentTerms ptm;
             ptm.lg2v = cur.lgv;
-            ptm.lse2 = (cur.lse == NEG_INF_F) ? 0.f : cur.lse * LF_LOG2E;
-            ptm.off = (cur.lse == NEG_INF_F) ? 0.f : ptm.lg2v - ptm.lse2;
+            lse_terms(cur.lse, ptm);
             // the parents' rows as chunks (column operand of the scores) and as tables for the products
             float sab0 = 0.f, sab1 = 0.f;
 #pragma unroll
