@@ -45,6 +45,34 @@ def test_argument_errors_without_gpu():
         _lib.check(rc)
 
 
+def test_link_scorer_form_selection_without_gpu():
+    """Which shapes the scorer with its products inside the kernels covers, what its backward needs as workspace, and its
+    argument errors: host logic of the library, no GPU call."""
+    lib = _lib.load()
+    f16, f32, f64 = (custom_ops._DTYPE_CODE[t] for t in (torch.float16, torch.float32, torch.float64))
+    for F in (16, 32, 64, 128):
+        assert lib.pcfgnat_extract_links_fused_supported(f16, 128, 8, F) == 1
+        assert lib.pcfgnat_extract_links_fused_backward_supported(f16, 128, 8, F) == (1 if F <= 64 else 0)
+    for F in (8, 16, 32, 64):
+        assert lib.pcfgnat_extract_links_fused_supported(f32, 128, 8, F) == 1
+        assert lib.pcfgnat_extract_links_fused_backward_supported(f32, 128, 8, F) == 1
+    for dtype, Lg, H, F in ((f16, 128, 8, 8), (f16, 128, 8, 48), (f32, 128, 8, 24), (f32, 128, 8, 128), (f64, 128, 8, 64),
+                           (f16, 128, 3, 64), (f16, 1, 8, 64), (f16, 8193, 8, 64), (f32, 128, 16, 64)):
+        assert lib.pcfgnat_extract_links_fused_supported(dtype, Lg, H, F) == 0, (dtype, Lg, H, F)
+    assert lib.pcfgnat_extract_links_fused_backward_supported(f32, 128, 16, 64) == 1  # per-head tiles: no limit on heads x dimension
+    B, Lg, H, F = 40, 128, 8, 64
+    assert lib.pcfgnat_extract_links_fused_backward_workspace_bytes(B, Lg, H, F) == 4 * (2 * B * Lg * H + 3 * B * H * Lg + B * H * F)
+    assert lib.pcfgnat_extract_links_fused_backward_workspace_bytes(B, 1, H, F) == 0
+    rc = lib.pcfgnat_extract_links_fused_backward(None, None, None, None, None, None, None, f16, None, None, None, None, None, None,
+                                                  2, 64, 8, 48, None)
+    assert rc == _lib.EUNSUPPORTED and b"not built" in lib.pcfgnat_last_error()
+    rc = lib.pcfgnat_extract_links_fused_backward(None, None, None, None, None, None, None, f16, None, None, None, None, None, None,
+                                                  2, 64, 8, 64, None)
+    assert rc == _lib.EINVAL and b"null pointer" in lib.pcfgnat_last_error()
+    rc = lib.pcfgnat_extract_links_fused_forward(None, None, None, f32, None, None, 1, None, None, None, None, None, None, 0, 64, 8, 64, None)
+    assert rc == _lib.OK  # an empty batch is no work
+
+
 def test_ops_refuse_to_run_without_gpu():
     if torch.cuda.is_available():
         pytest.skip("GPU present")
