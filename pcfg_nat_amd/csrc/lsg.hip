@@ -519,7 +519,9 @@ __global__ __launch_bounds__(NT) void ls_max_kernel(const T *__restrict__ x, typ
 // once: a chunk that holds target columns is taken over by the thread of the first target that points into it, which
 // loads the chunk itself, adds the gradients of all targets in it, in order, and stores it; the thread that streams the
 // chunk otherwise leaves it out (one bit per thread and chunk slot in LDS).  No store waits for another, so the
-// workgroup ends when its last store is issued instead of when it is acknowledged.
+// workgroup ends when its last store is issued instead of when it is acknowledged.  The second load of such a chunk is
+// non-temporal like the row's: as an ordinary load it left up to 140 lines per row in the L2, which the next kernel
+// paid for (the gather forward behind it ran 2 us slower at 32 targets per row and 11 us at 140).
 template <typename T, int NT, int MAXC, int TCAP, bool FROM_LOGITS>
 __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const int64_t *__restrict__ idx, int64_t sb,
                                                      int64_t sl, int64_t st,
@@ -678,7 +680,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
         if (lead_chunk[r] >= 0) {
             const int s = tid + r * NT, cc = lead_chunk[r];
             CT v[EPV];
-            Elem<T>::unpack(pv[cc], v);
+            Elem<T>::unpack(load16(pv + cc), v);  // streamed like the row: an ordinary load would leave its line in the L2
 #pragma unroll
             for (int e = 0; e < EPV; e++) {
                 v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
