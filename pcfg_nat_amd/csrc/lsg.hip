@@ -619,12 +619,14 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
     // The threads of the targets sort out who rewrites which chunk.
     const int body_end = sp.head + sp.nvec * EPV;  // columns [head, body_end) travel as 16-byte chunks
     int lead_chunk[FIX];  // the chunk this thread rewrites on behalf of its target (and of the later targets in it), or -1
-    bool lead_more[FIX];  // later targets point into the same chunk
+    int lead_more[FIX];   // how many later targets point into the same chunk,
+    int lead_next[FIX];   // and the first of them
 #pragma unroll
     for (int r = 0; r < FIX; r++) {
         const int s = tid + r * NT;
         lead_chunk[r] = -1;
-        lead_more[r] = false;
+        lead_more[r] = 0;
+        lead_next[r] = 0;
         if (s < Tn && (uint64_t)tcol[r] < (uint64_t)V) {
             const int col = (int)tcol[r];
             if (col < sp.head) {
@@ -635,18 +637,21 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
                 const int cc = (col - sp.head) / EPV, lo = sp.head + cc * EPV;
                 // targets in the same chunk before and after s, four entries per LDS read
                 const int4 *si4 = reinterpret_cast<const int4 *>(s_idx);
-                int before = 0, after = 0;
+                int before = 0, after = 0, next = 0x7fffffff;
                 for (int w = 0; w < (Tn + 3) >> 2; w++) {
                     const int4 q = si4[w];
                     const int u = 4 * w;
                     const bool a = (unsigned)(q.x - lo) < (unsigned)EPV, b = (unsigned)(q.y - lo) < (unsigned)EPV;
                     const bool c = (unsigned)(q.z - lo) < (unsigned)EPV, d = (unsigned)(q.w - lo) < (unsigned)EPV;
                     before += (a && u < s) + (b && u + 1 < s) + (c && u + 2 < s) + (d && u + 3 < s);
-                    after += (a && u > s) + (b && u + 1 > s) + (c && u + 2 > s) + (d && u + 3 > s);
+                    const int later = (a && u > s) + (b && u + 1 > s) + (c && u + 2 > s) + (d && u + 3 > s);
+                    if (later != 0 && after == 0) next = (a && u > s) ? u : (b && u + 1 > s) ? u + 1 : (c && u + 2 > s) ? u + 2 : u + 3;
+                    after += later;
                 }
                 if (before == 0) {
                     lead_chunk[r] = cc;
-                    lead_more[r] = after != 0;
+                    lead_more[r] = after;
+                    lead_next[r] = next;
                     atomicOr(&s_hit[cc % NT], cc / NT < MAXC ? 1u << (cc / NT) : BEYOND_BIT);
                 }
             }
@@ -686,7 +691,15 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
                 v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
                 if (!FROM_LOGITS) v[e] = Elem<T>::widen(Elem<T>::narrow(v[e]));  // p * ns is rounded before the adds
             }
-            add_targets(v, EPV, sp.head + cc * EPV, s, lead_more[r] ? Tn : s + 1);
+            // its own target, then the later ones of the chunk in order: from the first of them until all are found (a walk
+            // over every later target would hold up the whole wave for the one lane that shares its chunk)
+            add_targets(v, EPV, sp.head + cc * EPV, s, s + 1);
+            for (int u = lead_next[r], left = lead_more[r]; left > 0; u++) {
+                if ((unsigned)(s_idx[u] - (sp.head + cc * EPV)) < (unsigned)EPV) {
+                    add_targets(v, EPV, sp.head + cc * EPV, u, u + 1);
+                    left--;
+                }
+            }
             store16(pv + cc, Elem<T>::pack(v));
         }
     }
@@ -767,18 +780,24 @@ int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
     using CT = typename Elem<T>::compute;
     constexpr int NT = 512;
     constexpr int MAXC = 10;
-    constexpr int TCAP = 1024;
+    constexpr int TCAP = 1024;  // most targets per row; up to NT of them the kernel with one target per thread (fewer registers)
     if (Tn > TCAP) return fail(PCFGNAT_EUNSUPPORTED, "logsoftmax_gather_backward: T=%d exceeds %d targets per row", Tn, TCAP);
     const dim3 grid = row_grid(rows);
     const int pad_mode = pad_out_len == nullptr ? 0 : pad_row_mode(rows, L);
-    if (lse != nullptr)
-        hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, true>), grid, dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,
-                           (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss, detach_rows, pad_out_len, pad_mode, pad_rows_zeroed,
-                           gscale_dev);
-    else
-        hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, TCAP, false>), grid, dim3(NT), 0, stream, (T *)p, idx, sb, sl,
-                           st, (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss, detach_rows, pad_out_len, pad_mode,
-                           pad_rows_zeroed, nullptr);
+#define PCFGNAT_LSG_BWD(tcap)                                                                                                              \
+    do {                                                                                                                                   \
+        if (lse != nullptr)                                                                                                                \
+            hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, tcap, true>), grid, dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,              \
+                               (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss, detach_rows, pad_out_len, pad_mode, pad_rows_zeroed,  \
+                               gscale_dev);                                                                                                \
+        else                                                                                                                               \
+            hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, tcap, false>), grid, dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,             \
+                               (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss, detach_rows, pad_out_len, pad_mode,               \
+                               pad_rows_zeroed, nullptr);                                                                                  \
+    } while (0)
+    if (Tn <= NT) PCFGNAT_LSG_BWD(NT);
+    else PCFGNAT_LSG_BWD(TCAP);
+#undef PCFGNAT_LSG_BWD
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
