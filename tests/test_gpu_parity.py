@@ -514,6 +514,36 @@ def test_extract_links_products_inside_the_kernel(B, L, H, F, dtype):
     assert torch.allclose(got[fin.to(DEV)], other[fin.to(DEV)], rtol=2e-5, atol=2e-5)
 
 
+@pytest.mark.parametrize("B,L,H,F,dtype,ms", [(1, 2, 2, 16, torch.float16, [2]), (2, 3, 4, 8, torch.float32, [3, 2]),
+                                               (3, 6, 8, 16, torch.float16, [6, 0, 4]), (1, 70, 16, 64, torch.float16, [66]),
+                                               (2, 33, 1, 64, torch.float32, [33, 32])])
+def test_extract_links_products_inside_edge_shapes(B, L, H, F, dtype, ms):
+    """The smallest graphs, a single sentence, a sentence that is all pad, sixteen heads of 64, a tile boundary at 32 + 1
+    nodes: links and gradients of the form with the products inside against the form with the products through torch."""
+    g = torch.Generator().manual_seed(7 * L + H)
+    q, kl, kr = ((torch.randn(B, L, H, F, generator=g) * 0.7).to(dtype).to(DEV) for _ in range(3))
+    gate = torch.randn(B, L, H, generator=g).to(dtype).to(DEV)
+    prev = torch.full((B, L), 3).masked_fill(torch.arange(L).view(1, L) >= torch.tensor(ms).view(B, 1), synth.PAD).to(DEV)
+    lm, rm, mc = (t.to(DEV) for t in synth.support_masks(L, 1))
+    G = torch.randn(B, L, 2, L, generator=g).to(DEV)
+    res = []
+    for inside in (True, False):
+        leaves = [t.clone().requires_grad_(True) for t in (q, kl, kr, gate)]
+        out = ops.pcfg_extract_links(*leaves, prev, synth.PAD, lm, rm, mc, inside)
+        fin = torch.isfinite(out)
+        out.masked_fill(~fin, 0).mul(G).sum().backward()
+        res.append((out.detach(), [t.grad for t in leaves]))
+    (a, ga), (b, gb) = res
+    assert torch.equal(torch.isfinite(a), torch.isfinite(b))
+    fin = torch.isfinite(a)
+    assert torch.allclose(a[fin], b[fin], rtol=2e-5, atol=2e-5)
+    for name, x, y in zip(("q", "kl", "kr", "gate"), ga, gb):
+        assert torch.isfinite(x).all(), name
+        scale = max(y.float().abs().max().item(), 1e-6)
+        tol = 4e-3 if dtype == torch.float16 else 1e-4  # fp16: both results are rounded to the chunks' dtype
+        assert (x.float() - y.float()).abs().max().item() <= tol * scale, name
+
+
 def test_extract_links_fused_form_rejects_what_it_does_not_cover():
     lib = ops.get_pcfg_kernel()
     assert lib.pcfgnat_extract_links_fused_supported(ops._DTYPE_CODE[torch.float32], 256, 2, 24) == 0   # head dimension
