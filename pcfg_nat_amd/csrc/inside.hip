@@ -1657,7 +1657,14 @@ __global__ __launch_bounds__(256) void compact_links_ml1_kernel(const float *__r
     if (zero_slabs != nullptr) {
         float *z = zero_slabs + (size_t)b * L * 2 * L;
         const size_t nthreads = (size_t)gridDim.x * gridDim.y * 256, me = ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
-        for (size_t i = me; i < (size_t)L * 2 * L; i += nthreads) z[i] = 0.f;
+        const size_t nz = (size_t)L * 2 * L;
+        if ((reinterpret_cast<uintptr_t>(z) & 15) == 0) {  // 16 bytes per store where the slab allows it
+            float4 *z4 = reinterpret_cast<float4 *>(z);
+            for (size_t i = me; i < nz / 4; i += nthreads) z4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (me < (nz & 3)) z[(nz & ~(size_t)3) + me] = 0.f;
+        } else {
+            for (size_t i = me; i < nz; i += nthreads) z[i] = 0.f;
+        }
     }
     const int m = (int)out_len[b];
     const int mc = (m >= 2 && m <= L) ? m / 2 : 0;
@@ -1667,13 +1674,14 @@ __global__ __launch_bounds__(256) void compact_links_ml1_kernel(const float *__r
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
     {   // the exchange tables of the pipelined sweeps start out empty (all ones), their flags lowered
         ExchangeView xv(aux, b, Mc, T);
-        unsigned *x = reinterpret_cast<unsigned *>(xv.fcol);
-        const size_t words = (size_t)4 * MP * (T + 2);
+        // both tables start 16-byte aligned and hold a multiple of four words (MP is a multiple of 64)
+        uint4 *x = reinterpret_cast<uint4 *>(xv.fcol), *y = reinterpret_cast<uint4 *>(xv.obw);
+        const size_t quads = (size_t)MP * (T + 2);
         const size_t nthreads = (size_t)gridDim.x * gridDim.y * 256, me = ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
-        unsigned *y = reinterpret_cast<unsigned *>(xv.obw);
-        for (size_t i = me; i < words; i += nthreads) {
-            x[i] = 0xFFFFFFFFu;
-            y[i] = 0xFFFFFFFFu;
+        const uint4 ones = make_uint4(0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu);
+        for (size_t i = me; i < quads; i += nthreads) {
+            x[i] = ones;
+            y[i] = ones;
         }
         if (me < 4) xv.flags[me] = 0;
     }
@@ -2692,6 +2700,78 @@ __global__ __launch_bounds__(NTP) void inside_bwd_ml1_pipe_kernel(const float *_
     }
 }
 
+// Emission posteriors (element-wise) from BETA, F0, F1: the epilogue of the register-resident backward, for the long
+// graphs a kernel of its own or the work of the rule posterior launch's spare workgroups.
+struct MatchGradArgs {
+    const float *match_all;
+    float *mgrad;  // null: the caller has a launch of its own for them
+};
+
+// The cells first, first + stride, ... of sentence b (cell i = node i / T, position i % T), NB of them at a time with
+// every load of the batch issued ahead of its arithmetic: addresses of terms a cell does not have fall back to offset 0.
+template <int NB>
+__device__ __forceinline__ void match_grad_cells(const int b, const int first, const int stride, const float *__restrict__ grad_out,
+                                                 const float *__restrict__ S, const float *__restrict__ aux_c,
+                                                 const float *__restrict__ match_all, const int64_t *__restrict__ out_len,
+                                                 const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad, int L, int T, int Mc,
+                                                 Seed seed, int use_corr) {
+    const int m = (int)out_len[b], n = (int)tgt_len[b];
+    const float *Sb = S + (size_t)b * Mc * (T + 2);
+    const float *mt = match_all + (size_t)b * L * T;
+    float *mg = mgrad + (size_t)b * L * T;
+    const float ll = Sb[0];
+    const int cells = L * T;
+    if (!(lengths_ok(m, n, L, T) && (ll == ll) && (fabsf(ll) != __builtin_huge_valf()))) {
+        for (int i = first; i < cells; i += stride) mg[i] = 0.f;
+        return;
+    }
+    const int mc = m / 2;
+    AuxViewStream av(const_cast<float *>(aux_c), b, Mc, T);
+    const float g = seed_weight(grad_out, b, n, seed);
+    // corrections of the columns (see pipeline_finish_kernel): on the forward's offsets they are 0 and -D_t
+    const float *corr = ExchangeView(const_cast<float *>(aux_c), b, Mc, T).corr;
+    const float *shift1 = use_corr ? corr + corr_len(T) : av.D;  // the second correction, or (negated) the forward's shift
+    for (int i0 = first; i0 < cells; i0 += NB * stride) {
+        float bs[NB], bp[NB], mx[NB], mo[NB], f0[NB], f1[NB], c0[NB], c1[NB];
+        bool t_main[NB], t_prev[NB], t_last[NB], t_leaf[NB];
+#pragma unroll
+        for (int u = 0; u < NB; u++) {
+            const int i = i0 + u * stride;
+            const bool in = i < cells;
+            const int x = in ? i / T : 0, s = in ? i - x * T : 0, a_id = x >> 1;
+            const bool cell = in && x >= 1 && x < m && s < n, odd = (x & 1) != 0;
+            t_main[u] = cell && odd && s + 1 <= n - 1;
+            t_prev[u] = cell && odd && s >= 1 && s + 1 <= n - 1 && a_id >= 1;
+            t_last[u] = cell && odd && a_id == mc - 1 && s == n - 1;
+            t_leaf[u] = cell && !odd && a_id >= 1 && a_id < mc && s + 2 <= n - 1;
+            const bool any = t_main[u] || t_prev[u] || t_last[u] || t_leaf[u];
+            const size_t row = any ? (size_t)a_id * (T + 2) : 0;
+            const int sa = any ? s : 0;
+            bs[u] = av.BETA[row + sa];
+            bp[u] = av.BETA[t_prev[u] ? row + sa - 1 : 0];
+            mx[u] = mt[any ? (size_t)x * T + sa : 0];
+            mo[u] = mt[t_prev[u] ? (size_t)(x - 1) * T + sa - 1 : (t_leaf[u] ? (size_t)(x + 1) * T + sa + 1 : 0)];
+            f0[u] = av.F0[t_main[u] ? row + sa + 1 : 0];
+            f1[u] = av.F1[t_prev[u] ? row + sa + 1 : (t_leaf[u] ? row + sa + 2 : 0)];
+            c0[u] = use_corr ? corr[sa] : 0.f;
+            c1[u] = shift1[t_leaf[u] ? sa + 1 : sa];
+        }
+#pragma unroll
+        for (int u = 0; u < NB; u++) {
+            const int i = i0 + u * stride;
+            if (i >= cells) break;
+            const float mas = to_b2(mx[u]), mos = to_b2(mo[u]), sh = use_corr ? c1[u] : -c1[u];
+            float out = 0.f;
+            if (t_main[u]) out += ex2((bs[u] + mas + f0[u]) + c0[u]);
+            if (t_prev[u]) out += ex2(bp[u] + mos + mas + (f1[u] + sh));
+            if (t_last[u]) out += ex2((bs[u] + mas) + c0[u]);
+            if (t_leaf[u]) out += ex2(bs[u] + mas + mos + (f1[u] + sh));
+            if (!(out == out)) out = 0.f;
+            mg[i] = g * out;
+        }
+    }
+}
+
 // Rule posteriors from the outside weights: lg[a][k][c] = g * sum_{t=1}^{n-1} exp(links[a][k][c] + Wk[a][t] + R[c][t]),
 // the one step of the path with operand reuse: per sentence and left option a [Mc,T] x [T,Mc] contraction, which as one
 // exponential per term is 9 M exponentials per sentence of 256 main-chain nodes and 140 target tokens.  Here the terms are
@@ -2740,7 +2820,7 @@ __global__ __launch_bounds__(256, QMAX < 8 ? 3 : 2) void links_grad_ml1_stream_k
                                                                    const int64_t *__restrict__ out_len,
                                                                    const int64_t *__restrict__ tgt_len, float *__restrict__ lgrad,
                                                                    int L, int T, int Mc, Seed seed, int use_corr, float range_limit,
-                                                                   int span) {
+                                                                   int span, MatchGradArgs emis) {
     extern __shared__ float lg_lds[];
     const int ld = span + 1;                 // row pitch: odd, so that a column of 32 rows falls into 32 banks
     float *sw0 = lg_lds, *sw1 = sw0 + LG_TILE * ld, *ss = sw1 + LG_TILE * ld, *s_u = ss + LG_TILE * ld;  // [32][ld] x 3, [span]
@@ -2748,7 +2828,14 @@ __global__ __launch_bounds__(256, QMAX < 8 ? 3 : 2) void links_grad_ml1_stream_k
                                                                             // at a time, over the tables once they are used up
     __shared__ int s_bad;
     const int b = blockIdx.z, at = blockIdx.y, ct = blockIdx.x;
-    if (ct < at) return;
+    if (ct < at) {  // no tile of rules here: the sentence's emission posteriors, shared among these workgroups
+        if (emis.mgrad != nullptr) {
+            const int spare = (int)(gridDim.y * (gridDim.y - 1) / 2);
+            match_grad_cells<4>(b, (at * (at - 1) / 2 + ct) * 256 + (int)threadIdx.x, spare * 256, grad_out, S, aux_c, emis.match_all,
+                                out_len, tgt_len, emis.mgrad, L, T, Mc, seed, use_corr);
+        }
+        return;
+    }
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const float *Sb = S + (size_t)b * Mc * (T + 2);
     const float ll = Sb[0];
@@ -2911,51 +2998,14 @@ __global__ __launch_bounds__(256, QMAX < 8 ? 3 : 2) void links_grad_ml1_stream_k
     }
 }
 
-// Emission posteriors (element-wise) from BETA, F0, F1: the epilogue of the register-resident backward as a kernel.
+// The emission posteriors as a launch of their own: one cell per thread.
 __global__ __launch_bounds__(256) void match_grad_ml1_stream_kernel(const float *__restrict__ grad_out, const float *__restrict__ S,
                                                                    const float *__restrict__ aux_c, const float *__restrict__ match_all,
                                                                    const int64_t *__restrict__ out_len,
                                                                    const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad, int L,
                                                                    int T, int Mc, Seed seed, int use_corr) {
-    const int b = blockIdx.y;
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= L * T) return;
-    const int m = (int)out_len[b], n = (int)tgt_len[b];
-    const float *Sb = S + (size_t)b * Mc * (T + 2);
-    const float *mt = match_all + (size_t)b * L * T;
-    float *mg = mgrad + (size_t)b * L * T;
-    const float ll = Sb[0];
-    if (!(lengths_ok(m, n, L, T) && (ll == ll) && (fabsf(ll) != __builtin_huge_valf()))) {
-        mg[i] = 0.f;
-        return;
-    }
-    const int mc = m / 2;
-    AuxViewStream av(const_cast<float *>(aux_c), b, Mc, T);
-    const float g = seed_weight(grad_out, b, n, seed);
-    const int x = i / T, s = i - x * T;
-    // corrections of the columns (see pipeline_finish_kernel): on the forward's offsets they are 0 and -D_t
-    const float *corr = ExchangeView(const_cast<float *>(aux_c), b, Mc, T).corr;
-    const int CLEN = corr_len(T);
-    float out = 0.f;
-    if (x >= 1 && x < m && s < n) {
-        const int a_id = x >> 1;
-        const size_t row = (size_t)a_id * (T + 2);
-        const float c0 = use_corr ? corr[s] : 0.f;
-        if (x & 1) {
-            const float bs = av.BETA[row + s];
-            const float mas = to_b2(mt[(size_t)x * T + s]);
-            if (s + 1 <= n - 1) out += ex2((bs + mas + av.F0[row + s + 1]) + c0);
-            if (s >= 1 && s + 1 <= n - 1 && a_id >= 1)
-                out += ex2(av.BETA[row + s - 1] + to_b2(mt[(size_t)(x - 1) * T + s - 1]) + mas +
-                           (av.F1[row + s + 1] + (use_corr ? corr[CLEN + s] : -av.D[s])));
-            if (a_id == mc - 1 && s == n - 1) out += ex2((bs + mas) + c0);
-        } else if (a_id >= 1 && a_id < mc && s + 2 <= n - 1) {
-            out += ex2(av.BETA[row + s] + to_b2(mt[(size_t)x * T + s]) + to_b2(mt[(size_t)(x + 1) * T + s + 1]) +
-                       (av.F1[row + s + 2] + (use_corr ? corr[CLEN + s + 1] : -av.D[s + 1])));
-        }
-        if (!(out == out)) out = 0.f;
-    }
-    mg[i] = g * out;
+    match_grad_cells<1>((int)blockIdx.y, (int)(blockIdx.x * blockDim.x + threadIdx.x), (int)(gridDim.x * blockDim.x), grad_out, S, aux_c,
+                        match_all, out_len, tgt_len, mgrad, L, T, Mc, seed, use_corr);
 }
 
 __global__ void fill_zero_kernel(float *p, size_t n) {
@@ -3144,12 +3194,19 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
     const int span = links_grad_span(T, (long)B * tiles * (tiles + 1) / 2, small);
     auto lgk = small ? links_grad_ml1_stream_kernel<LG_SPAN_SMALL / 32> : links_grad_ml1_stream_kernel<LG_SPAN / 32>;
     PCFGNAT_DYNAMIC_LDS(lgk, links_grad_lds_bytes(span));
+    // The workgroups below the diagonal of the tile grid have no rules to do: they take the emission posteriors while that
+    // leaves each of their threads a handful of cells; otherwise those get a launch of their own.
+    const long spare_threads = (long)tiles * (tiles - 1) / 2 * 256;
+    const bool emis_inside = spare_threads > 0 && (long)L * T <= 16 * spare_threads;
     hipLaunchKernelGGL(lgk, dim3(tiles, tiles, B), dim3(256), links_grad_lds_bytes(span), stream, go, S, aux, links, ol, tl, lg, L, T,
-                       Mc, seed, use_corr, g_links_grad_range_limit.load(), span);
+                       Mc, seed, use_corr, g_links_grad_range_limit.load(), span,
+                       MatchGradArgs{match_all, emis_inside ? mg : nullptr});
     PCFGNAT_HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL(match_grad_ml1_stream_kernel, dim3((L * T + 255) / 256, B), dim3(256), 0, stream, go, S, aux, match_all, ol, tl, mg, L,
-                       T, Mc, seed, use_corr);
-    PCFGNAT_HIP_CHECK(hipGetLastError());
+    if (!emis_inside) {
+        hipLaunchKernelGGL(match_grad_ml1_stream_kernel, dim3((L * T + 255) / 256, B), dim3(256), 0, stream, go, S, aux, match_all, ol, tl,
+                           mg, L, T, Mc, seed, use_corr);
+        PCFGNAT_HIP_CHECK(hipGetLastError());
+    }
     return PCFGNAT_OK;
 }
 
