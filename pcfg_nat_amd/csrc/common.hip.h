@@ -238,19 +238,25 @@ struct LossTask {
     int B;
     int64_t stride;
 };
-template <int NT>
+// NT threads form the sum (the order of the additions, and with it the rounding, is a function of NT alone); the
+// workgroup may be larger (BLOCK threads), its other threads only keep the barriers company.
+template <int NT, int BLOCK = NT>
 __device__ __forceinline__ void criterion_loss_block(const LossTask &t) {
+    static_assert(BLOCK >= NT, "the workgroup holds at least the threads that sum");
     __shared__ float s_sum[NT];
     __shared__ float s_bad[NT];
+    const bool member = BLOCK == NT || (int)threadIdx.x < NT;
     float acc = 0.f, bad = 0.f;
-    for (int b = threadIdx.x; b < t.B; b += NT) {
-        const float ll = t.S[(size_t)b * t.stride];
-        const bool ok = (ll == ll) && (fabsf(ll) != __builtin_huge_valf());
-        if (ok) acc += ll / (float)t.tgt_len[b];
-        else bad += 1.f;
+    if (member) {
+        for (int b = threadIdx.x; b < t.B; b += NT) {
+            const float ll = t.S[(size_t)b * t.stride];
+            const bool ok = (ll == ll) && (fabsf(ll) != __builtin_huge_valf());
+            if (ok) acc += ll / (float)t.tgt_len[b];
+            else bad += 1.f;
+        }
+        s_sum[threadIdx.x] = acc;
+        s_bad[threadIdx.x] = bad;
     }
-    s_sum[threadIdx.x] = acc;
-    s_bad[threadIdx.x] = bad;
     __syncthreads();
     for (int o = NT / 2; o > 0; o >>= 1) {
         if ((int)threadIdx.x < o) {
