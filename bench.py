@@ -89,8 +89,8 @@ def _percentile(sorted_vals, q):
 def decode_timing(dev, n_b1=256):
     """Viterbi decode of the inference configuration (BASELINE config 4: src ~U[5,100], L = 4*src, V=40000, fp16 logits
     ~N(0,3)) as the model runs it: front-end (log-softmax + max over the vocabulary, one read of the logits) followed by
-    tables + length selection + readout as one native call; the emitted token counts are read back by the host, which
-    is the decode's one synchronisation.  Batch 1: wall-clock latency per sentence over the first ``n_b1`` sentences
+    tables + length selection + readout, all enqueued by one native call; the emitted token counts are read back by the
+    host, which is the decode's one synchronisation.  Batch 1: wall-clock latency per sentence over the first ``n_b1`` sentences
     of the configuration (median, 95th percentile, mean; front-end and decode also timed apart).  Batch 64: throughput
     over ten chunks of length-sorted sentences."""
     import torch
@@ -112,8 +112,7 @@ def decode_timing(dev, n_b1=256):
 
     def run(case):
         logits, links, m, mask = case
-        ob, tok = ops.logsoftmax_max(logits)
-        return harness.viterbi_decode(ob, tok, links, m, mask, single_call=True)
+        return harness.decode_from_logits(logits, links, m, mask, single_call=True)
 
     def wall(fn):
         torch.cuda.synchronize()

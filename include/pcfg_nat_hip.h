@@ -432,6 +432,18 @@ int pcfgnat_viterbi_decode(const float *ob_lprob, const float *links, const int6
                            int64_t L, int64_t ml, void *stream);
 
 /*
+ * The decode as the model runs it (glat_decomposed_with_link_two_hands_tri_pcfg.py:414-416 followed by :483-502) enqueued
+ * by one call: pcfgnat_logsoftmax_max over logits [B,L,V] (float16 or float32) into best_lprob [B,L] float32 and best_idx
+ * [B,L] int64 (both out: the node scores and node tokens of the decode), then pcfgnat_viterbi_decode on them.  The other
+ * arguments and the results are those of pcfgnat_viterbi_decode.
+ */
+int pcfgnat_viterbi_decode_logits(const void *logits, int dtype, int64_t V, float *best_lprob, int64_t *best_idx,
+                                  const float *links, const int64_t *output_length, const int64_t *left_tree_mask,
+                                  int64_t mask_dim, int64_t pad_index, const float *length_penalty, void *workspace,
+                                  int64_t *out_tokens, int64_t *out_count, int64_t *pred_length, int64_t B, int64_t L,
+                                  int64_t ml, void *stream);
+
+/*
  * The `lookahead` and `greedy` decode strategies of glat_decomposed_with_link_two_hands_tri_pcfg.py:419-481 in one launch:
  * per node the first arg max over (k, c) of (links[b,a,k,c] + ob[b,c]*beta) + ob[b,left(a,k)]*beta (lookahead; ob_lprob
  * NULL selects greedy: links alone), then the in-order walk from node 1 over these pointers.  The reference builds the

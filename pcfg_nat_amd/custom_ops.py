@@ -749,44 +749,21 @@ class _PinnedCounts:
 _pinned_counts = _PinnedCounts()
 
 
-def pcfg_viterbi_decode(unreduced_logits, links, output_length, unreduced_tokens, left_tree_mask, pad_index, beta=1.0):
-    """The model's whole Viterbi decode (glat_decomposed_with_link_two_hands_tri_pcfg.py:483-502) in one native call:
-    ``cuda_pcfg_viterbi`` -> length penalty ``arange ** beta`` -> NaN masking -> arg max over lengths >= 1 ->
-    ``viterbi_decoding``.  Returns (tokens float32 [B, maxlen] right-padded with ``pad_index``, pred_length int64 [B]),
-    the values the separate calls give."""
+def _viterbi_decode_call(name, B, L, ml, dev, extra_words, call):
+    """Shared tail of the Viterbi decode calls: one allocation (workspace | tokens [B,L] | predicted lengths [B] |
+    ``extra_words`` more int64 words for the caller), the native call, the one stream wait, the emitted counts.  ``call``
+    receives (lib, base address of the block, workspace words, address of the pinned counts) and returns the status."""
     lib = get_pcfg_kernel()
-    _need_cuda("pcfg_viterbi_decode", unreduced_logits, links, output_length, unreduced_tokens, left_tree_mask)
-    if unreduced_logits.dim() != 2 or links.dim() != 4:
-        raise RuntimeError("pcfg_viterbi_decode: unreduced_logits must be [bsz, prelen] and links [bsz, prelen, max_left+1, prelen]")
-    if unreduced_logits.dtype != torch.float32 or links.dtype != torch.float32:
-        raise RuntimeError("pcfg_viterbi_decode: unreduced_logits and links must be float32")
-    B, L = unreduced_logits.shape
-    if links.size(0) != B or links.size(1) != L or links.size(3) != L:
-        raise RuntimeError("pcfg_viterbi_decode: links shape %s does not match unreduced_logits %s"
-                           % (tuple(links.shape), tuple(unreduced_logits.shape)))
-    if left_tree_mask.dim() != 2 or left_tree_mask.size(0) != left_tree_mask.size(1):
-        raise RuntimeError("pcfg_viterbi_decode: left_tree_mask must be square")
-    ml = links.size(2) - 1
-    dev = unreduced_logits.device
-    ob, links = unreduced_logits.contiguous(), links.contiguous()
-    ol = _lengths("pcfg_viterbi_decode", output_length, B)
-    tok = unreduced_tokens.to(dtype=torch.int64).contiguous()
-    mask = left_tree_mask.to(dtype=torch.int64).contiguous()
-    pen = _length_penalty(L // 4, beta, dev)
     with torch.cuda.device(dev):
         nwork = (lib.pcfgnat_viterbi_decode_workspace_bytes(B, L, ml) + 7) // 8
-        # one allocation: workspace | tokens [B,L] | emitted counts [B] | predicted lengths [B]
-        block = torch.empty((nwork + B * L + B,), dtype=torch.int64, device=dev)
+        block = torch.empty((nwork + B * L + B + extra_words,), dtype=torch.int64, device=dev)
         out = block[nwork:nwork + B * L].view(B, L)
-        pred = block[nwork + B * L:]
-        base = block.data_ptr()
+        pred = block[nwork + B * L:nwork + B * L + B]
         # the emitted counts go straight into pinned host memory, which the device addresses like its own: the one
         # synchronisation of the decode is a stream wait, with no copy in front of it
         host = _pinned_counts.take(B)  # written by the kernel, read after the one stream wait
         try:
-            _lib.check(lib.pcfgnat_viterbi_decode(ob.data_ptr(), links.data_ptr(), ol.data_ptr(), tok.data_ptr(), mask.data_ptr(),
-                                                  mask.size(0), int(pad_index), pen.data_ptr(), base, base + 8 * nwork,
-                                                  host.data_ptr(), base + 8 * (nwork + B * L), B, L, ml, _stream(ob)), lib)
+            _lib.check(call(lib, block.data_ptr(), nwork, host.data_ptr()), lib)
             torch.cuda.current_stream(dev).synchronize()
             counts = host[:B].tolist()
         finally:
@@ -794,7 +771,82 @@ def pcfg_viterbi_decode(unreduced_logits, links, output_length, unreduced_tokens
     if B and min(counts) < 0:
         raise RuntimeError("viterbi_decoding: malformed traces")
     maxlen = max(counts) if B else 0
-    return out[:, :maxlen].to(torch.float32), pred
+    return out[:, :maxlen].to(torch.float32), pred, block
+
+
+def _check_decode_graph(name, B, L, links, left_tree_mask):
+    if links.dim() != 4 or links.dtype != torch.float32:
+        raise RuntimeError("%s: links must be float32 [bsz, prelen, max_left+1, prelen]" % name)
+    if links.size(0) != B or links.size(1) != L or links.size(3) != L:
+        raise RuntimeError("%s: links shape %s does not match [bsz, prelen] = %s" % (name, tuple(links.shape), (B, L)))
+    if left_tree_mask.dim() != 2 or left_tree_mask.size(0) != left_tree_mask.size(1):
+        raise RuntimeError("%s: left_tree_mask must be square" % name)
+
+
+def pcfg_viterbi_decode(unreduced_logits, links, output_length, unreduced_tokens, left_tree_mask, pad_index, beta=1.0):
+    """The model's whole Viterbi decode (glat_decomposed_with_link_two_hands_tri_pcfg.py:483-502) in one native call:
+    ``cuda_pcfg_viterbi`` -> length penalty ``arange ** beta`` -> NaN masking -> arg max over lengths >= 1 ->
+    ``viterbi_decoding``.  Returns (tokens float32 [B, maxlen] right-padded with ``pad_index``, pred_length int64 [B]),
+    the values the separate calls give."""
+    _need_cuda("pcfg_viterbi_decode", unreduced_logits, links, output_length, unreduced_tokens, left_tree_mask)
+    if unreduced_logits.dim() != 2 or links.dim() != 4:
+        raise RuntimeError("pcfg_viterbi_decode: unreduced_logits must be [bsz, prelen] and links [bsz, prelen, max_left+1, prelen]")
+    if unreduced_logits.dtype != torch.float32 or links.dtype != torch.float32:
+        raise RuntimeError("pcfg_viterbi_decode: unreduced_logits and links must be float32")
+    B, L = unreduced_logits.shape
+    _check_decode_graph("pcfg_viterbi_decode", B, L, links, left_tree_mask)
+    ml = links.size(2) - 1
+    dev = unreduced_logits.device
+    ob, links = unreduced_logits.contiguous(), links.contiguous()
+    ol = _lengths("pcfg_viterbi_decode", output_length, B)
+    tok = unreduced_tokens.to(dtype=torch.int64).contiguous()
+    mask = left_tree_mask.to(dtype=torch.int64).contiguous()
+    pen = _length_penalty(L // 4, beta, dev)
+    stream = _stream(ob)
+
+    def call(lib, base, nwork, counts):
+        return lib.pcfgnat_viterbi_decode(ob.data_ptr(), links.data_ptr(), ol.data_ptr(), tok.data_ptr(), mask.data_ptr(), mask.size(0),
+                                          int(pad_index), pen.data_ptr(), base, base + 8 * nwork, counts,
+                                          base + 8 * (nwork + B * L), B, L, ml, stream)
+
+    tokens, pred, _ = _viterbi_decode_call("pcfg_viterbi_decode", B, L, ml, dev, 0, call)
+    return tokens, pred
+
+
+def pcfg_viterbi_decode_logits(logits, links, output_length, left_tree_mask, pad_index, beta=1.0, return_nodes=False):
+    """The decode as the model runs it, from the vocabulary logits [bsz, prelen, vocab] (float16 or float32):
+    ``logits.log_softmax(-1).max(-1)`` (glat_decomposed_with_link_two_hands_tri_pcfg.py:414-416) and the Viterbi decode
+    (:483-502) enqueued by one native call.  Returns what ``pcfg_viterbi_decode(*logsoftmax_max(logits), ...)`` returns:
+    (tokens float32 [B, maxlen], pred_length int64 [B]); with ``return_nodes`` also the node scores [B,L] float32 and node
+    tokens [B,L] int64 of the front-end."""
+    _need_cuda("pcfg_viterbi_decode_logits", logits, links, output_length, left_tree_mask)
+    if logits.dim() != 3 or not logits.is_contiguous():
+        raise RuntimeError("pcfg_viterbi_decode_logits: logits must be a contiguous [bsz, prelen, vocab] tensor")
+    if logits.dtype not in (torch.float16, torch.float32):
+        raise RuntimeError("pcfg_viterbi_decode_logits: logits must be float16 or float32 (got %s)" % logits.dtype)
+    B, L, V = logits.shape
+    _check_decode_graph("pcfg_viterbi_decode_logits", B, L, links, left_tree_mask)
+    ml = links.size(2) - 1
+    dev = logits.device
+    links = links.contiguous()
+    ol = _lengths("pcfg_viterbi_decode_logits", output_length, B)
+    mask = left_tree_mask.to(dtype=torch.int64).contiguous()
+    pen = _length_penalty(L // 4, beta, dev)
+    code = _DTYPE_CODE[logits.dtype]
+    stream = _stream(logits)
+    nodes = B * L
+
+    def call(lib, base, nwork, counts):
+        idx = base + 8 * (nwork + nodes + B)  # node tokens [B,L] int64, then node scores [B,L] float32
+        return lib.pcfgnat_viterbi_decode_logits(logits.data_ptr(), code, V, idx + 8 * nodes, idx, links.data_ptr(), ol.data_ptr(),
+                                                 mask.data_ptr(), mask.size(0), int(pad_index), pen.data_ptr(), base, base + 8 * nwork,
+                                                 counts, base + 8 * (nwork + nodes), B, L, ml, stream)
+
+    tokens, pred, block = _viterbi_decode_call("pcfg_viterbi_decode_logits", B, L, ml, dev, nodes + (nodes + 1) // 2, call)
+    if not return_nodes:
+        return tokens, pred
+    tail = block[block.numel() - (nodes + (nodes + 1) // 2):]
+    return tokens, pred, tail[nodes:].view(torch.float32)[:nodes].view(B, L), tail[:nodes].view(B, L)
 
 
 def pcfg_lookahead_decode(links, unreduced_logits, unreduced_tokens, output_length, left_tree_mask, pad_index, beta=1.0,

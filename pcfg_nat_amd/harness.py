@@ -124,6 +124,16 @@ def viterbi_decode(unreduced_logits, unreduced_tokens, links, output_length, lef
     return tokens.to(device=pred_length.device), pred_length
 
 
+def decode_from_logits(logits, links, output_length, left_tree_mask, pad=PAD, beta=1.0, ops=_default_ops, single_call=False):
+    """The decode from the vocabulary logits, as the model runs it (glat_decomposed_with_link_two_hands_tri_pcfg.py:414-416,
+    483-502): ``log_softmax`` and ``max`` over the vocabulary, then ``viterbi_decode``.  ``single_call``: both enqueued by
+    one native call (``ops.pcfg_viterbi_decode_logits``).  Returns (tokens float32 [B,maxlen], pred_length [B])."""
+    if single_call:
+        return ops.pcfg_viterbi_decode_logits(logits, links, output_length.long(), left_tree_mask, pad, beta)
+    ob, tok = ops.logsoftmax_max(logits)
+    return viterbi_decode(ob, tok, links, output_length, left_tree_mask, pad, beta, ops=ops, single_call=True)
+
+
 def train_step_direct(logits, targets, links, output_length, target_length, ops=_default_ops, mark=None):
     """One training pass of the structured loss issued as the bare sequence of native calls that autograd performs for
     ``compute_pcfg_loss(...)['loss'].backward()`` (nat_pcfg_loss.py:98-145 and pcfg_loss.py:55-83, 147-179), without

@@ -607,6 +607,31 @@ def test_viterbi_tables_bit_exact_and_decode(case):
         assert got_tok.dtype == torch.float32 and torch.equal(got_tok.cpu(), want_tok)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("case", ["short", "L96", "L224", "L400", "L600"])
+def test_decode_from_logits_is_front_end_plus_decode(case, dtype):
+    """The call that takes the vocabulary logits returns, bit for bit, what the front-end followed by the decode returns
+    (the same kernels enqueued by one call), node scores and node tokens included; the decode itself is held against the
+    oracle by the tests above."""
+    batch = _decode_case(case)
+    logits = batch["logits"].to(dtype).to(DEV).contiguous()
+    links, ol = batch["links"].to(DEV), batch["output_length"].to(DEV)
+    left_mask = synth.support_masks(links.shape[1], 1)[0].to(DEV)
+    for beta in (1.0, 0.7):
+        ob, tok = ops.logsoftmax_max(logits)
+        want_tok, want_len = ops.pcfg_viterbi_decode(ob, links, ol, tok, left_mask, synth.PAD, beta)
+        got_tok, got_len, got_ob, got_nodes = ops.pcfg_viterbi_decode_logits(logits, links, ol, left_mask, synth.PAD, beta,
+                                                                             return_nodes=True)
+        assert torch.equal(got_ob, ob) and torch.equal(got_nodes, tok)
+        assert got_len.dtype == torch.int64 and torch.equal(got_len, want_len)
+        assert got_tok.dtype == torch.float32 and torch.equal(got_tok, want_tok)
+    got_tok, got_len = harness.decode_from_logits(logits, links, ol, left_mask, single_call=True)
+    two_tok, two_len = harness.decode_from_logits(logits, links, ol, left_mask)
+    assert torch.equal(got_tok, two_tok) and torch.equal(got_len, two_len)
+    with pytest.raises(RuntimeError, match="float16 or float32"):
+        ops.pcfg_viterbi_decode_logits(logits.double(), links, ol, left_mask, synth.PAD)
+
+
 @pytest.mark.parametrize("mode", ["one_workgroup", "blocks_give_up"])
 @pytest.mark.parametrize("case", ["L224", "L288", "L400", "L512"])
 def test_single_call_decode_sweeps_agree(mode, case):
