@@ -515,15 +515,17 @@ __global__ __launch_bounds__(NT) void ls_max_kernel(const T *__restrict__ x, typ
 // roundings to the buffer dtype); true: it holds the untouched logits and `lse` the row log-sum-exps.
 //
 // Every element of the row becomes p * (-sum_s g[s]); the (at most T) target columns also receive their g[s]
-// (scatter_add_, pcfg_loss.py:177: duplicates of a column accumulate in order).  Every 16-byte chunk is stored exactly
-// once: a chunk that holds target columns is taken over by the thread of the first target that points into it, which
-// loads the chunk itself, adds the gradients of all targets in it, in order, and stores it; the thread that streams the
-// chunk otherwise leaves it out (one bit per thread and chunk slot in LDS).  No store waits for another, so the
-// workgroup ends when its last store is issued instead of when it is acknowledged.  The second load of such a chunk is
-// non-temporal like the row's: as an ordinary load it left up to 140 lines per row in the L2, which the next kernel
-// paid for (the gather forward behind it ran 2 us slower at 32 targets per row and 11 us at 140).
+// (scatter_add_, pcfg_loss.py:177: duplicates of a column accumulate in order).  Every 16-byte chunk is loaded once and
+// stored once, by the thread that streams it: the thread of a target posts (target, chunk slot, element) into the
+// streaming thread's mailbox in LDS (BOX entries per thread, taken in the order of arrival and sorted by target before
+// use, so that duplicates of a column are added in the order of the targets whatever the arrival order was); a thread
+// whose mailbox overflowed goes through all targets for each of its chunks instead.  No second load, no store beside
+// the row's own stream: as a take-over of such chunks by the targets' threads (a second, dependent load per target,
+// a 16-byte store of its own and a hole in the stream's stores) the same work took 123 instead of 95-100 us at 140
+// targets per row, of which the scattered stores were 8 us, the holes 7 us and the second loads 5 us (each switched
+// off in turn).
 template <typename T, int NT, int MAXC, int TCAP, bool FROM_LOGITS>
-__global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const int64_t *__restrict__ idx, int64_t sb,
+__global__ __launch_bounds__(NT, FROM_LOGITS ? 1 : 6) void lsg_bwd_kernel(T *__restrict__ p, const int64_t *__restrict__ idx, int64_t sb,
                                                      int64_t sl, int64_t st,
                                                      const typename Elem<T>::compute *__restrict__ gsel, int64_t rows,
                                                      int L, int V, int Tn,
@@ -534,8 +536,15 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
     constexpr int FIX = (TCAP + NT - 1) / NT;
-    constexpr unsigned EDGE_BIT = 1u << 30, BEYOND_BIT = 1u << 31;  // targets outside the register-resident chunks
+    constexpr int BOX = 4;                      // mailbox entries per streaming thread
+    constexpr unsigned EDGE_BIT = 1u << 30;     // in the mailbox count: a target points at this thread's element outside the chunks
+    constexpr unsigned COUNT_MASK = 0xFFFFu;
+    constexpr int SLOT_SHIFT = 16;              // above the count: one bit per chunk slot (bit MAXC: any chunk beyond them) that holds
+                                                // a target which found the mailbox full
+    static_assert(SLOT_SHIFT + MAXC < 30, "the slot bits end below EDGE_BIT");
+    constexpr unsigned NO_ENTRY = 0xFFFFFFFFu;  // sorts behind every entry; its slot field matches no slot
     static_assert(MAXC <= 30, "one bit per register-resident chunk");
+    static_assert(TCAP <= 1024, "a target index takes ten bits of a mailbox entry");
     // an upstream factor of the whole gradient that only the device knows (the loss's own upstream gradient under fp16 loss
     // scaling): folded into g in the compute type, ahead of the single rounding to the buffer's dtype (pcfg_loss.py:77-83,
     // 176-177 scale g before the cast as well)
@@ -544,7 +553,8 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
     __shared__ __attribute__((aligned(16))) int s_idx[TCAP + 4];  // target column of position s, -1 if out of range; padded
                                                                   // to a multiple of four with -2 (matches nothing)
     __shared__ CT s_g[TCAP];         // g[s], zero for a detached row
-    __shared__ unsigned s_hit[NT];   // per thread: bit i = the chunk of slot i holds a target column
+    __shared__ unsigned s_cnt[NT];   // per thread: how many targets point into its chunks (and EDGE_BIT)
+    __shared__ __attribute__((aligned(16))) unsigned s_box[NT * BOX];  // (target << 16) | (chunk slot << 4) | element
     const int tid = threadIdx.x, lane = tid & 63;
 
     const int64_t slot = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;  // one row per workgroup
@@ -605,7 +615,7 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
     T edge_raw = Elem<T>::narrow((CT)0);
     if (ep >= 0) edge_raw = pr[ep];
 
-    s_hit[tid] = 0;
+    s_cnt[tid] = 0;
 #pragma unroll
     for (int r = 0; r < FIX; r++) {
         const int s = tid + r * NT;
@@ -616,49 +626,57 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
     }
     lds_barrier();
 
-    // The threads of the targets sort out who rewrites which chunk.
+    // The threads of the targets post them to the threads that stream their chunks.
     const int body_end = sp.head + sp.nvec * EPV;  // columns [head, body_end) travel as 16-byte chunks
-    int lead_chunk[FIX];  // the chunk this thread rewrites on behalf of its target (and of the later targets in it), or -1
-    int lead_more[FIX];   // how many later targets point into the same chunk,
-    int lead_next[FIX];   // and the first of them
 #pragma unroll
     for (int r = 0; r < FIX; r++) {
         const int s = tid + r * NT;
-        lead_chunk[r] = -1;
-        lead_more[r] = 0;
-        lead_next[r] = 0;
         if (s < Tn && (uint64_t)tcol[r] < (uint64_t)V) {
             const int col = (int)tcol[r];
             if (col < sp.head) {
-                atomicOr(&s_hit[col], EDGE_BIT);
+                atomicOr(&s_cnt[col], EDGE_BIT);
             } else if (col >= body_end) {
-                atomicOr(&s_hit[sp.head + (col - body_end)], EDGE_BIT);
+                atomicOr(&s_cnt[sp.head + (col - body_end)], EDGE_BIT);
             } else {
-                const int cc = (col - sp.head) / EPV, lo = sp.head + cc * EPV;
-                // targets in the same chunk before and after s, four entries per LDS read
-                const int4 *si4 = reinterpret_cast<const int4 *>(s_idx);
-                int before = 0, after = 0, next = 0x7fffffff;
-                for (int w = 0; w < (Tn + 3) >> 2; w++) {
-                    const int4 q = si4[w];
-                    const int u = 4 * w;
-                    const bool a = (unsigned)(q.x - lo) < (unsigned)EPV, b = (unsigned)(q.y - lo) < (unsigned)EPV;
-                    const bool c = (unsigned)(q.z - lo) < (unsigned)EPV, d = (unsigned)(q.w - lo) < (unsigned)EPV;
-                    before += (a && u < s) + (b && u + 1 < s) + (c && u + 2 < s) + (d && u + 3 < s);
-                    const int later = (a && u > s) + (b && u + 1 > s) + (c && u + 2 > s) + (d && u + 3 > s);
-                    if (later != 0 && after == 0) next = (a && u > s) ? u : (b && u + 1 > s) ? u + 1 : (c && u + 2 > s) ? u + 2 : u + 3;
-                    after += later;
-                }
-                if (before == 0) {
-                    lead_chunk[r] = cc;
-                    lead_more[r] = after;
-                    lead_next[r] = next;
-                    atomicOr(&s_hit[cc % NT], cc / NT < MAXC ? 1u << (cc / NT) : BEYOND_BIT);
-                }
+                const int cc = (col - sp.head) / EPV, e = (col - sp.head) - cc * EPV, owner = cc % NT;
+                const unsigned at = atomicAdd(&s_cnt[owner], 1u) & COUNT_MASK;
+                if (at < (unsigned)BOX) s_box[owner * BOX + at] = ((unsigned)s << 16) | ((unsigned)(cc / NT) << 4) | (unsigned)e;
+                else atomicOr(&s_cnt[owner], 1u << (SLOT_SHIFT + min(cc / NT, MAXC)));  // no room: at least which chunk it is
             }
         }
     }
     lds_barrier();
-    const unsigned hit = s_hit[tid];
+    const unsigned posted = s_cnt[tid];
+    const int count = (int)(posted & COUNT_MASK);
+    const bool overflow = count > BOX;  // (then every target is looked at for every chunk that holds one)
+    // bit i: an entry for the chunk of slot i; bit 31: one for a chunk beyond the register-resident ones.  The entries
+    // themselves stay in LDS (sorted by target, the high bits, where there are several) and are read again by the few
+    // threads that have any, chunk by chunk: held in registers they cost the kernel its third workgroup per compute unit.
+    unsigned mine = 0;
+    uint4 *my_box = reinterpret_cast<uint4 *>(s_box) + tid;
+    if (count > 0) {
+        uint4 q = *my_box;
+        q.y = count > 1 ? q.y : NO_ENTRY;
+        q.z = count > 2 ? q.z : NO_ENTRY;
+        q.w = count > 3 ? q.w : NO_ENTRY;
+        auto order = [](unsigned &x, unsigned &y) {
+            const unsigned lo = min(x, y), hi = max(x, y);
+            x = lo;
+            y = hi;
+        };
+        order(q.x, q.y);  // a sorting network of five exchanges
+        order(q.z, q.w);
+        order(q.x, q.z);
+        order(q.y, q.w);
+        order(q.y, q.z);
+        *my_box = q;
+        const unsigned e[BOX] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int k = 0; k < BOX; k++)
+            if (e[k] != NO_ENTRY) mine |= ((e[k] >> 4) & 0xFFFu) < (unsigned)MAXC ? 1u << ((e[k] >> 4) & 0xFFFu) : 1u << 31;
+        const unsigned late = (posted >> SLOT_SHIFT) & ((2u << MAXC) - 1u);
+        mine |= (late & ((1u << MAXC) - 1u)) | ((late >> MAXC) << 31);
+    }
     // -(sum_s g), computed redundantly by every wave; rounded to the buffer dtype in the reference split (pcfg_loss.py:176)
     CT part = 0;
     for (int s = lane; s < Tn; s += 64) part += s_g[s];
@@ -677,60 +695,59 @@ __global__ __launch_bounds__(NT) void lsg_bwd_kernel(T *__restrict__ p, const in
                 if (k < n && k == e) v[k] = FROM_LOGITS ? v[k] + g : Elem<T>::widen(Elem<T>::narrow(v[k] + g));
         }
     };
-
-    // chunks with targets, by the first target's thread (a second, dependent load: issued before this thread waits for
-    // its own chunks)
+    // v[] holds p * ns of the chunk in slot `slot`: the posted targets of that chunk, in their order
+    auto add_posted = [&](CT *v, int slot) {
+        const uint4 q = *my_box;
+        const unsigned box[BOX] = {q.x, q.y, q.z, q.w};
 #pragma unroll
-    for (int r = 0; r < FIX; r++) {
-        if (lead_chunk[r] >= 0) {
-            const int s = tid + r * NT, cc = lead_chunk[r];
-            CT v[EPV];
-            Elem<T>::unpack(load16(pv + cc), v);  // streamed like the row: an ordinary load would leave its line in the L2
+        for (int k = 0; k < BOX; k++) {
+            if (((box[k] >> 4) & 0xFFFu) == (unsigned)slot) {
+                const int e = (int)(box[k] & 15u);
+                const CT g = g_at((int)(box[k] >> 16));
 #pragma unroll
-            for (int e = 0; e < EPV; e++) {
-                v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
-                if (!FROM_LOGITS) v[e] = Elem<T>::widen(Elem<T>::narrow(v[e]));  // p * ns is rounded before the adds
+                for (int j = 0; j < EPV; j++)
+                    if (j == e) v[j] = FROM_LOGITS ? v[j] + g : Elem<T>::widen(Elem<T>::narrow(v[j] + g));
             }
-            // its own target, then the later ones of the chunk in order: from the first of them until all are found (a walk
-            // over every later target would hold up the whole wave for the one lane that shares its chunk)
-            add_targets(v, EPV, sp.head + cc * EPV, s, s + 1);
-            for (int u = lead_next[r], left = lead_more[r]; left > 0; u++) {
-                if ((unsigned)(s_idx[u] - (sp.head + cc * EPV)) < (unsigned)EPV) {
-                    add_targets(v, EPV, sp.head + cc * EPV, u, u + 1);
-                    left--;
-                }
-            }
-            store16(pv + cc, Elem<T>::pack(v));
         }
-    }
+    };
 
 #pragma unroll
     for (int i = 0; i < MAXC; i++) {
         int c = tid + i * NT;
-        if (c < sp.nvec && !(hit & (1u << i))) {
+        if (c < sp.nvec) {
             CT v[EPV];
             Elem<T>::unpack(buf[i], v);
 #pragma unroll
             for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
+            if (mine & (1u << i)) {
+                if (!FROM_LOGITS) {  // p * ns is rounded before the adds
+#pragma unroll
+                    for (int e = 0; e < EPV; e++) v[e] = Elem<T>::widen(Elem<T>::narrow(v[e]));
+                }
+                if (overflow) add_targets(v, EPV, sp.head + c * EPV, 0, Tn);
+                else add_posted(v, i);
+            }
             store16(pv + c, Elem<T>::pack(v));
         }
     }
     for (int c = tid + MAXC * NT; c < sp.nvec; c += NT) {
-        if (hit & BEYOND_BIT) {  // rare: is this one of the chunks a target's thread rewrites?
-            const int lo = sp.head + c * EPV;
-            bool taken = false;
-            for (int u = 0; u < Tn; u++) taken = taken || (unsigned)(s_idx[u] - lo) < (unsigned)EPV;
-            if (taken) continue;
-        }
         CT v[EPV];
         Elem<T>::unpack(load16(pv + c), v);
 #pragma unroll
         for (int e = 0; e < EPV; e++) v[e] = (FROM_LOGITS ? rn.e(v[e]) : v[e]) * ns;
+        if (mine & (1u << 31)) {
+            if (!FROM_LOGITS) {
+#pragma unroll
+                for (int e = 0; e < EPV; e++) v[e] = Elem<T>::widen(Elem<T>::narrow(v[e]));
+            }
+            if (overflow) add_targets(v, EPV, sp.head + c * EPV, 0, Tn);
+            else add_posted(v, c / NT);
+        }
         store16(pv + c, Elem<T>::pack(v));
     }
     if (ep >= 0) {  // unaligned rows: the elements in front of and behind the 16-byte chunks, one per thread
         CT v = (FROM_LOGITS ? rn.e(Elem<T>::widen(edge_raw)) : Elem<T>::widen(edge_raw)) * ns;
-        if (hit & EDGE_BIT) {
+        if (posted & EDGE_BIT) {
             if (!FROM_LOGITS) v = Elem<T>::widen(Elem<T>::narrow(v));
             add_targets(&v, 1, ep, 0, Tn);
         }

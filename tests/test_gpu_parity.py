@@ -96,6 +96,58 @@ def test_lsg_backward_matches_torch_ops(dtype):
         assert torch.allclose(got, ref, rtol=1e-5, atol=1e-9)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_lsg_backward_adds_duplicate_targets_in_target_order(dtype):
+    """Targets that share a column are added one after the other in the order of the target positions (scatter_add_ along
+    the last dimension, pcfg_loss.py:177), however they reach the thread that owns the column: three of one column (sorted
+    on arrival), six of another (more than the thread keeps: it goes through all targets), columns of one thread's
+    different chunks, two elements of one chunk.  The upstream gradients are multiples of 2^-5, so that their sum is exact
+    in any order and every bit of the result is fixed: compared for equality with the same operations one at a time."""
+    g = torch.Generator().manual_seed(21)
+    B, L, V, T = 2, 5, 16384, 24
+    epv = 8 if dtype == torch.float16 else 4
+    probs = torch.softmax(torch.randn(B, L, V, generator=g) * 2, -1).to(dtype)
+    tgt = torch.randint(0, V, (B, T), generator=g)
+    a, b, c = 1000, 3001, 77
+    tgt[:, [2, 9, 15]] = a
+    tgt[:, [0, 4, 5, 11, 20, 23]] = b
+    tgt[:, 6] = c
+    tgt[:, 7] = c + 1                # the same 16-byte chunk
+    tgt[:, 8] = c + 512 * epv        # the same thread's next chunk
+    tgt[:, 10] = c + 2 * 512 * epv
+    idx = tgt.unsqueeze(1).expand(-1, L, -1).contiguous()
+    gout = torch.randint(-40, 41, (B, L, T), generator=g).float() / 32
+    # one rounding to the buffer's dtype per operation, the targets one after the other
+    ref = probs.clone()
+    ref.mul_(gout.sum(-1, keepdim=True).neg_().to(ref.dtype))
+    for t in range(T):
+        for b_ in range(B):
+            col = int(tgt[b_, t])
+            ref[b_, :, col] = (ref[b_, :, col].float() + gout[b_, :, t].to(dtype).float()).to(dtype)
+    if dtype == torch.float32:  # which is what torch's own call does on the CPU
+        ref2 = probs.clone()
+        ref2.mul_(gout.sum(-1, keepdim=True).neg_())
+        ref2.scatter_add_(-1, idx, gout)
+        assert torch.equal(ref, ref2)
+    got = probs.clone().to(DEV)
+    ops._logsoftmax_gather_backward(got, idx.to(DEV), gout.to(DEV))
+    assert torch.equal(got.cpu(), ref)
+    # the recomputing backward (row log-sum-exps instead of probabilities in the buffer) adds in float32 and rounds once
+    x = (torch.randn(B, L, V, generator=g) * 2).to(dtype)
+    xd = x.to(DEV)
+    sel, lse = ops._logsoftmax_gather_lse(xd, idx.to(DEV))
+    ops._logsoftmax_gather_backward_lse(xd, idx.to(DEV), gout.to(DEV), lse)
+    want = torch.exp(x.float() - lse.cpu().unsqueeze(-1)) * gout.sum(-1, keepdim=True).neg_()
+    for t in range(T):
+        for b_ in range(B):
+            want[b_, :, int(tgt[b_, t])] += gout[b_, :, t]
+    assert torch.allclose(xd.cpu().float(), want.to(dtype).float(), rtol=2 ** -9 if dtype == torch.float16 else 1e-5, atol=1e-7)
+    at = torch.zeros(B, V, dtype=torch.bool)
+    at.scatter_(1, tgt, True)
+    cols = at.unsqueeze(1).expand(-1, L, -1)
+    assert torch.allclose(xd.cpu().float()[cols], want[cols], rtol=2 ** -10 if dtype == torch.float16 else 2e-6, atol=1e-7)
+
+
 @pytest.mark.parametrize("dtype,V", [(torch.float16, 2048), (torch.float16, 333), (torch.float32, 1001), (torch.float64, 257)])
 def test_lsg_lse_split_matches_autograd(dtype, V):
     """Read-only forward + recomputing backward against torch's own log_softmax/gather gradient in float64."""
