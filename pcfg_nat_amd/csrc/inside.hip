@@ -1558,18 +1558,12 @@ __device__ __forceinline__ void stream_row_lse(const float4 *__restrict__ r0, co
 
 // Dynamic LDS: col[2][MP], f1prev[MP], f0prev[MP], per-wave column maxima slots[2][16], then (if MATCH_LDS) match main
 // [Mc][T], match leaf [Mc][T].
+// (sentence b by one workgroup of NT threads; the kernels below run it)
 template <bool MATCH_LDS, int SL>
-__global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
-                                                                  const int64_t *__restrict__ out_len,
-                                                                  const int64_t *__restrict__ tgt_len, float *__restrict__ S,
-                                                                  float *__restrict__ aux, int L, int T, int Mc, int MP,
-                                                                  int only_flagged) {
-    // only_flagged: run only for sentences whose pipelined sweep gave up (the flag was written by an earlier launch)
-    if (only_flagged) {
-        if (ExchangeView(aux, blockIdx.x, Mc, T).flags[FLAG_FWD] == 0) return;
-        if (threadIdx.x == 0) atomicAdd(&g_inside_redone, 1ull);
-    }
-    extern __shared__ float smem[];
+__device__ __forceinline__ void inside_fwd_ml1_stream_block(const int b, const float *__restrict__ match_all,
+                                                            const float *__restrict__ links, const int64_t *__restrict__ out_len,
+                                                            const int64_t *__restrict__ tgt_len, float *__restrict__ S,
+                                                            float *__restrict__ aux, int L, int T, int Mc, int MP, float *smem) {
     float *col = smem;               // [2][MP]
     float *f1prev = smem + 2 * MP;    // [MP]
     float *f0prev = smem + 3 * MP;    // [MP]  (only a guess for the next column)
@@ -1578,7 +1572,7 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
     float *sm_leaf = sm_main + (MATCH_LDS ? Mc * T : 0);
 
     constexpr int SCH = 4 * SL, SROWS = NT / SL;
-    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid / SL, j = tid % SL;
+    const int tid = threadIdx.x, gidx = tid / SL, j = tid % SL;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const float *mt = match_all + (size_t)b * L * T;
     float *Sb = S + (size_t)b * Mc * (T + 2);
@@ -1695,6 +1689,21 @@ __global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *
     }
 }
 
+template <bool MATCH_LDS, int SL>
+__global__ __launch_bounds__(NT) void inside_fwd_ml1_stream_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
+                                                                  const int64_t *__restrict__ out_len,
+                                                                  const int64_t *__restrict__ tgt_len, float *__restrict__ S,
+                                                                  float *__restrict__ aux, int L, int T, int Mc, int MP,
+                                                                  int only_flagged) {
+    // only_flagged: run only for sentences whose pipelined sweep gave up (the flag was written by an earlier launch)
+    if (only_flagged) {
+        if (ExchangeView(aux, blockIdx.x, Mc, T).flags[FLAG_FWD] == 0) return;
+        if (threadIdx.x == 0) atomicAdd(&g_inside_redone, 1ull);
+    }
+    extern __shared__ float smem[];
+    inside_fwd_ml1_stream_block<MATCH_LDS, SL>((int)blockIdx.x, match_all, links, out_len, tgt_len, S, aux, L, T, Mc, MP, smem);
+}
+
 // Compact copies of the main-chain links for the streaming sweeps: Ac[k][a_id][c_id] = At[k][c_id][a_id] =
 // log2(e) * links[2*a_id+1][k][2*c_id+1] where a_id <= c_id < mc (k = 1 needs a_id >= 1), -inf everywhere else including the
 // padding columns up to MP.  One block per 32 x 32 tile of (parent, child) pairs, grid (MP/32, MP/32, B).  The blocks of a
@@ -1760,17 +1769,12 @@ __global__ __launch_bounds__(256) void compact_links_ml1_kernel(const float *__r
 }
 
 // Outside sweep.  Dynamic LDS: w0[2][MP], w1[2][MP], bprev[MP], D[T+4], then (if MATCH_LDS) match main/leaf [Mc][T] each.
+// (sentence b by one workgroup of NT threads; the kernels below run it)
 template <bool MATCH_LDS, int SL>
-__global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *__restrict__ S, float *__restrict__ aux,
-                                                                  const float *__restrict__ match_all,
-                                                                  const int64_t *__restrict__ out_len,
-                                                                  const int64_t *__restrict__ tgt_len, int L, int T, int Mc, int MP,
-                                                                  int only_flagged) {
-    if (only_flagged) {
-        if (ExchangeView(aux, blockIdx.x, Mc, T).flags[FLAG_BWD] == 0) return;
-        if (threadIdx.x == 0) atomicAdd(&g_inside_redone, 1ull);
-    }
-    extern __shared__ float smem[];
+__device__ __forceinline__ void inside_bwd_ml1_stream_block(const int b, const float *__restrict__ S, float *__restrict__ aux,
+                                                            const float *__restrict__ match_all, const int64_t *__restrict__ out_len,
+                                                            const int64_t *__restrict__ tgt_len, int L, int T, int Mc, int MP,
+                                                            float *smem) {
     float *w0 = smem;             // [2][MP]
     float *w1 = smem + 2 * MP;     // [2][MP]
     float *bprev = smem + 4 * MP;  // [MP]
@@ -1779,7 +1783,7 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
     float *sm_leaf = sm_main + (MATCH_LDS ? Mc * T : 0);
 
     constexpr int SCH = 4 * SL, SROWS = NT / SL;
-    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid / SL, j = tid % SL;
+    const int tid = threadIdx.x, gidx = tid / SL, j = tid % SL;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const float *mt = match_all + (size_t)b * L * T;
     const float *Sb = S + (size_t)b * Mc * (T + 2);
@@ -1957,6 +1961,67 @@ __device__ __forceinline__ void slab_row_lse(const float4 (&A0)[NQ], const float
             out1 = a1.finish();
         }
     }
+}
+
+template <bool MATCH_LDS, int SL>
+__global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *__restrict__ S, float *__restrict__ aux,
+                                                                  const float *__restrict__ match_all,
+                                                                  const int64_t *__restrict__ out_len,
+                                                                  const int64_t *__restrict__ tgt_len, int L, int T, int Mc, int MP,
+                                                                  int only_flagged) {
+    if (only_flagged) {
+        if (ExchangeView(aux, blockIdx.x, Mc, T).flags[FLAG_BWD] == 0) return;
+        if (threadIdx.x == 0) atomicAdd(&g_inside_redone, 1ull);
+    }
+    extern __shared__ float smem[];
+    inside_bwd_ml1_stream_block<MATCH_LDS, SL>((int)blockIdx.x, S, aux, match_all, out_len, tgt_len, L, T, Mc, MP, smem);
+}
+
+// Both sweeps' second chance in one launch, after the pipelines that ran side by side: grid (B, 2), workgroup (b, 0)
+// sweeps sentence b forward again if its forward pipeline gave up, workgroup (b, 1) its outside sweep if that pipeline
+// gave up.  The outside sweep reads the forward's column shifts and log-likelihood: where both are redone, its workgroup
+// waits for the forward's, which was dispatched before it (x runs fastest) and waits for nobody; the forward's tables
+// reach it through a device-scope release / acquire pair around the flag FLAG_FWD_REDONE (the two workgroups may sit on
+// different L2s).  In the normal case neither flag is set and the launch ends at once - one launch where two stood.
+// Dynamic LDS: the larger of the two sweeps' needs without the emissions.
+constexpr int FLAG_FWD_REDONE = 2;
+template <int SLB>
+__global__ __launch_bounds__(NT) void inside_redo_ml1_stream_kernel(const float *match_all, const float *links, const int64_t *out_len,
+                                                                   const int64_t *tgt_len, float *S, float *aux, int L, int T, int Mc,
+                                                                   int MP, int wait_limit) {
+    extern __shared__ float smem[];
+    const int b = blockIdx.x;
+    int *flags = ExchangeView(aux, b, Mc, T).flags;
+    if (blockIdx.y == 0) {
+        if (flags[FLAG_FWD] == 0) return;
+        if (threadIdx.x == 0) atomicAdd(&g_inside_redone, 1ull);
+        inside_fwd_ml1_stream_block<false, 4>(b, match_all, links, out_len, tgt_len, S, aux, L, T, Mc, MP, smem);
+        __threadfence();  // every thread's table entries are out before the flag
+        __syncthreads();
+        if (threadIdx.x == 0) __hip_atomic_store(flags + FLAG_FWD_REDONE, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
+    if (flags[FLAG_BWD] == 0) return;
+    if (threadIdx.x == 0) atomicAdd(&g_inside_redone, 1ull);
+    if (flags[FLAG_FWD] != 0) {
+        __shared__ int s_arrived;
+        if (threadIdx.x == 0) {
+            // The forward's workgroup is running or done and waits for nobody, so this wait ends; it is bounded all the
+            // same (seconds), like every wait between workgroups here.  Past the bound the sentence is given up: its
+            // log-likelihood becomes NaN, which the posterior kernels and the loss treat as an invalid sentence.
+            int arrived = 0;
+            for (int spins = 0; spins < wait_limit && !arrived; spins++) {
+                arrived = __hip_atomic_load(flags + FLAG_FWD_REDONE, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) != 0;
+                if (!arrived) __builtin_amdgcn_s_sleep(16);
+            }
+            s_arrived = arrived;
+            if (!arrived) S[(size_t)b * Mc * (T + 2)] = __builtin_nanf("");
+        }
+        __syncthreads();
+        if (!s_arrived) return;
+        __threadfence();
+    }
+    inside_bwd_ml1_stream_block<false, SLB>(b, S, aux, match_all, out_len, tgt_len, L, T, Mc, MP, smem);
 }
 
 // Forward sweep of one block.  Same tables as inside_fwd_ml1_stream_kernel, relative to the block's own offsets (see
@@ -3183,6 +3248,25 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
     const int only_flagged = NQ != 0;
     const size_t base = ((size_t)4 * MP + 32) * sizeof(float);
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
+    if (side_by_side) {
+        // both pipelines have run: one launch for the second chance of either sweep (in the normal case it finds no flag
+        // set and ends at once), then both sweeps' tables to common offsets and the corrections of the posteriors
+        const size_t base_bwd = ((size_t)5 * MP + T + 4) * sizeof(float);
+        const size_t lds = base > base_bwd ? base : base_bwd;
+        constexpr int WAIT_LIMIT = 1 << 23;  // polls of about a microsecond
+        if (Mc <= NT / 4)
+            hipLaunchKernelGGL(inside_redo_ml1_stream_kernel<4>, dim3(B, 2), dim3(NT), lds, stream, match_all, links, ol, tl, S, aux, L, T,
+                               Mc, MP, WAIT_LIMIT);
+        else
+            hipLaunchKernelGGL(inside_redo_ml1_stream_kernel<8>, dim3(B, 2), dim3(NT), lds, stream, match_all, links, ol, tl, S, aux, L, T,
+                               Mc, MP, WAIT_LIMIT);
+        PCFGNAT_HIP_CHECK(hipGetLastError());
+        const int CL = 64 * NQ / NLP;
+        hipLaunchKernelGGL(pipeline_finish_kernel, dim3(2 * CL - 1, B), dim3(256), (size_t)2 * (T + 4) * sizeof(double), stream, aux, ol, tl,
+                           L, T, Mc, CL);
+        PCFGNAT_HIP_CHECK(hipGetLastError());
+        return PCFGNAT_OK;
+    }
     if (with_match <= LDS_BUDGET) {
         auto k = inside_fwd_ml1_stream_kernel<true, 4>;
         PCFGNAT_DYNAMIC_LDS(k, with_match);
@@ -3192,12 +3276,6 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
                            T, Mc, MP, only_flagged);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
-    if (side_by_side) {  // both sweeps' tables to common offsets, and the corrections of the posteriors
-        const int CL = 64 * NQ / NLP;
-        hipLaunchKernelGGL(pipeline_finish_kernel, dim3(2 * CL - 1, B), dim3(256), (size_t)2 * (T + 4) * sizeof(double), stream, aux, ol, tl,
-                           L, T, Mc, CL);
-        PCFGNAT_HIP_CHECK(hipGetLastError());
-    }
     return PCFGNAT_OK;
 }
 
@@ -3226,7 +3304,9 @@ int launch_bwd_stream(const float *go, const float *S, float *aux, const float *
     if (rc != PCFGNAT_OK) return rc;
     const int only_flagged = NQ != 0;
     // lanes per node: four while one pass covers all nodes; beyond that the outside sweep measured faster with eight
-    if (with_match <= LDS_BUDGET) {
+    if (side_by_side) {
+        // (the outside sweep's second chance has run in the launch it shares with the forward's: launch_fwd_stream)
+    } else if (with_match <= LDS_BUDGET) {
         auto k = Mc <= NT / 4 ? inside_bwd_ml1_stream_kernel<true, 4> : inside_bwd_ml1_stream_kernel<true, 8>;
         PCFGNAT_DYNAMIC_LDS(k, with_match);
         hipLaunchKernelGGL(k, dim3(B), dim3(NT), with_match, stream, S, aux, match_all, ol, tl, L, T, Mc, MP, only_flagged);
