@@ -193,12 +193,13 @@ constexpr int DH_PITCH = 40;      // halves per row of a [right child][parent] p
 constexpr int BWD_TD_FLOATS = 4 * PT * DH_PITCH / 2;  // per wave: four fp16 planes, or two fp32 tiles and a row (fewer)
 static_assert(BWD_TD_FLOATS >= 2 * PT * BWD_TD_PITCH + PT, "transposed tiles of the children's launch");
 
-// ---- the parents' part of a workgroup: blockIdx.x = tile of 32 parents, blockIdx.y = group of four heads, sentence b;
+// ---- the parents' part of a workgroup: a tile of 32 parents, a group of four heads, sentence b;
 // wave w takes head 4 * group + w (a wave without a head still helps to move the entries).  masks: [B,L,1+nw] words as
 // the forward left them (flags, then the allowed right children).  MODE 0: the run that gives dg (and d gate); MODE 1:
 // the run that gives dz and its products, with dg read back.
 template <typename T, int NCH, int MODE>
-__device__ __forceinline__ void bwd_parents(uint4 *lb_lds, int b, const T *__restrict__ q, const T *__restrict__ kl, const T *__restrict__ kr,
+__device__ __forceinline__ void bwd_parents(uint4 *lb_lds, int tile, int group, int b, const T *__restrict__ q, const T *__restrict__ kl,
+                                            const T *__restrict__ kr,
                                             const float *__restrict__ gate, const float *__restrict__ head_lse,
                                             const float *__restrict__ links, const float *__restrict__ G, const unsigned *__restrict__ masks,
                                             T *__restrict__ dq, T *__restrict__ dkl, float *__restrict__ dgate, BwdWorkspace ws, int L, int H,
@@ -206,7 +207,7 @@ __device__ __forceinline__ void bwd_parents(uint4 *lb_lds, int b, const T *__res
     constexpr int EPC = Chunk<T>::EPC, F = 2 * NCH * EPC, FT = (F + 31) / 32, RPC = 2 * NCH + 1;
     const int nw = (L + 31) / 32;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int a0 = blockIdx.x * PT, h = blockIdx.y * 4 + wave;
+    const int a0 = tile * PT, h = group * 4 + wave;
     const bool active = h < H;
     constexpr int TILES = MODE == 0 ? 2 : 3;  // the run for dg keeps no table of the right keys
     uint4 *tQ = lb_lds + wave * bwd_wave_chunks<NCH, TILES>(), *tK1 = tQ + PT * RPC, *tKr = tK1 + PT * RPC, *tK0 = tQ + TILES * PT * RPC;
@@ -217,10 +218,26 @@ __device__ __forceinline__ void bwd_parents(uint4 *lb_lds, int b, const T *__res
     const int ai = in ? a : 0, hh = active ? h : 0;
     const int HF = H * F;
     const bool vec4 = (L & 3) == 0;
-    EntryLoad ent;
-    entries_request(links, G, b, a0, 0, L, vec4, tid, ent);
     const unsigned *mrow = masks + ((size_t)b * L + ai) * (1 + nw);
     const unsigned flags = in ? mrow[0] : 1u;
+    // The tiles of right children that hold an allowed (parent, right child) pair: [s_lo, s_hi).  The tiles in front of
+    // the parents' own and those of the pad nodes behind the sentence hold none, contribute nothing and are not even
+    // loaded (a step costs a trip to memory whatever it computes).  Masks do not depend on the head: every wave of the
+    // workgroup finds the same range.
+    // The first of them is requested on a guess, beside the masks: the parents' own tile, which is where the rules of a
+    // parent begin (right children come behind their parent); a wrong guess costs the request a second time.
+    const int guess = min(tile, nw - 1);
+    EntryLoad ent;
+    entries_request(links, G, b, a0, 32 * guess, L, vec4, tid, ent);
+    int s_lo = nw, s_hi = 0;
+    for (int ct = 0; ct < nw; ct++) {
+        if (__ballot(in && (flags & 1u) == 0 && mrow[1 + ct] != 0u) != 0ull) {
+            s_lo = min(s_lo, ct);
+            s_hi = ct + 1;
+        }
+    }
+    if (s_hi == 0) s_lo = guess;
+    if (s_lo != guess) entries_request(links, G, b, a0, 32 * s_lo, L, vec4, tid, ent);  // (uniform over the workgroup)
     // ---- the wave's rows of head h: query, left key src(a,1), left key of node 0; chunks 2j + kb of row p per lane
     ParentTerms pt;
     {
@@ -296,18 +313,21 @@ __device__ __forceinline__ void bwd_parents(uint4 *lb_lds, int b, const T *__res
     float dg = (MODE == 1 && in) ? ws.dg[((size_t)b * L + a) * H + hh] : 0.f, gsum = 0.f, ds0 = 0.f, ds1 = 0.f;
     uint4 cur[NCH], nxt[NCH];
     unsigned allow_cur, allow_nxt;
-    right_keys(0, cur, allow_cur);
+    right_keys(s_lo, cur, allow_cur);
     entries_store(s_ent, tid, ent);
     __syncthreads();
     // ---- one run over the tiles of right children: dg = sum G w (and the sum of G over the finite links), or dz and its
     // products with the right keys
 #pragma unroll 1
-    for (int s = 0; s < nw; s++) {
-        const int ctn = min(s + 1, nw - 1);
+    for (int s = s_lo; s < s_hi; s++) {
+        const int ctn = min(s + 1, s_hi - 1);
         entries_request(links, G, b, a0, 32 * ctn, L, vec4, tid, ent);
         right_keys(ctn, nxt, allow_nxt);
-        const float *buf = s_ent + (s & 1) * ENT_FLOATS;
-        if (active) {
+        const float *buf = s_ent + ((s - s_lo) & 1) * ENT_FLOATS;
+        // a tile without a single allowed (parent, right child) pair - the children in front of the parents, the pad nodes
+        // behind the sentence - holds no finite link and contributes nothing: left out (the decision is the wave's)
+        const bool live = __ballot(usable && allow_cur != 0u) != 0ull;
+        if (active && live) {
             float g0[16], g1[16], l0[16], l1[16], z0[16], z1[16], dz0[16], dz1[16];
             entries_read(buf, 0, p, 0, kb, l0);
             entries_read(buf, 0, p, 1, kb, l1);
@@ -316,16 +336,6 @@ __device__ __forceinline__ void bwd_parents(uint4 *lb_lds, int b, const T *__res
             scores(cur, allow_cur, z0, z1);
             if (MODE == 0) {
                 entry_gradients<true>(z0, z1, g0, g1, l0, l1, pt, 0.f, scale, dg, gsum, dz0, dz1);
-                if (s == nw - 1) {
-                    dg += __shfl_xor(dg, 32);
-                    gsum += __shfl_xor(gsum, 32);
-                    if (in && kb == 0) {
-                        // (the sum over the heads of dg is the sum of G over the finite links; a single head has a constant gate)
-                        dgate[((size_t)b * L + a) * H + h] = H == 1 ? 0.f : dg - ex2(pt.lg2v) * gsum;
-                        ws.dg[((size_t)b * L + a) * H + h] = dg;
-                        ws.lg[((size_t)b * L + a) * H + h] = pt.lg2v;
-                    }
-                }
             } else {
                 // the right keys of the tile as a table for the products below: [row][element], for fp16 [element][row]
                 if constexpr (sizeof(T) == 2) {
@@ -408,8 +418,18 @@ __device__ __forceinline__ void bwd_parents(uint4 *lb_lds, int b, const T *__res
 #pragma unroll
         for (int j = 0; j < NCH; j++) cur[j] = nxt[j];
         allow_cur = allow_nxt;
-        entries_store(s_ent + ((s + 1) & 1) * ENT_FLOATS, tid, ent);
+        entries_store(s_ent + ((s - s_lo + 1) & 1) * ENT_FLOATS, tid, ent);
         __syncthreads();
+    }
+    if (MODE == 0 && active) {
+        dg += __shfl_xor(dg, 32);
+        gsum += __shfl_xor(gsum, 32);
+        if (in && kb == 0) {
+            // (the sum over the heads of dg is the sum of G over the finite links; a single head has a constant gate)
+            dgate[((size_t)b * L + a) * H + h] = H == 1 ? 0.f : dg - ex2(pt.lg2v) * gsum;
+            ws.dg[((size_t)b * L + a) * H + h] = dg;
+            ws.lg[((size_t)b * L + a) * H + h] = pt.lg2v;
+        }
     }
     if (!active || MODE == 0) return;
     ds0 += __shfl_xor(ds0, 32);
@@ -455,14 +475,15 @@ __device__ __forceinline__ void bwd_parents(uint4 *lb_lds, int b, const T *__res
 // ---- the children's part of a workgroup: blockIdx.x = tile of 32 right children, blockIdx.y = group of four heads,
 // sentence b; wave w takes head 4 * group + w.
 template <typename T, int NCH>
-__device__ __forceinline__ void bwd_children(uint4 *lb_lds, int b, const T *__restrict__ q, const T *__restrict__ kl, const T *__restrict__ kr,
+__device__ __forceinline__ void bwd_children(uint4 *lb_lds, int tile, int group, int b, const T *__restrict__ q, const T *__restrict__ kl,
+                                             const T *__restrict__ kr,
                                              const float *__restrict__ head_lse, const float *__restrict__ links,
                                              const float *__restrict__ G, const unsigned *__restrict__ masks, T *__restrict__ dkr,
                                              BwdWorkspace ws, int L, int H, float scale2, float scale) {
     constexpr int EPC = Chunk<T>::EPC, F = 2 * NCH * EPC, FT = (F + 31) / 32, RPC = 2 * NCH + 1;
     const int nw = (L + 31) / 32;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int ct = blockIdx.x, c0 = ct * PT, h = blockIdx.y * 4 + wave;
+    const int ct = tile, c0 = ct * PT, h = group * 4 + wave;
     const bool active = h < H;
     const int hh = active ? h : 0;
     uint4 *tQ = lb_lds + wave * bwd_wave_chunks<NCH, 2>(), *tK1 = tQ + PT * RPC, *tK0 = tK1 + PT * RPC;
@@ -472,8 +493,21 @@ __device__ __forceinline__ void bwd_children(uint4 *lb_lds, int b, const T *__re
     const int p = lane & 31, kb = lane >> 5;
     const int HF = H * F;
     const bool vec4 = (L & 3) == 0;
+    // the tiles of parents that hold an allowed pair with this tile of right children: [p_lo, p_hi), as in the parents' part
+    // (the first tile requested on a guess, tile 0: parents come in front of their right children)
     EntryLoad ent;
     entries_request(links, G, b, 0, c0, L, vec4, tid, ent);
+    int p_lo = nw, p_hi = 0;
+    for (int t = 0; t < nw; t++) {
+        const int a = 32 * t + p;
+        const unsigned *mrow = masks + ((size_t)b * L + min(a, L - 1)) * (1 + nw);
+        if (__ballot(a < L && (mrow[0] & 1u) == 0 && mrow[1 + ct] != 0u) != 0ull) {
+            p_lo = min(p_lo, t);
+            p_hi = t + 1;
+        }
+    }
+    if (p_hi == 0) p_lo = 0;
+    if (p_lo != 0) entries_request(links, G, b, 32 * p_lo, c0, L, vec4, tid, ent);  // (the guess was tile 0; uniform over the workgroup)
     // the right keys of the wave's tile (the row operand of the scores) stay in registers; the left key of node 0 in LDS
     uint4 akr[NCH];
     {
@@ -519,16 +553,18 @@ __device__ __forceinline__ void bwd_children(uint4 *lb_lds, int b, const T *__re
 #pragma unroll
     for (int r = 0; r < 16; r++) csum[r] = 0.f;
     ParentLoad cur, nxt;
-    parent_request(0, cur);
+    parent_request(p_lo, cur);
     entries_store(s_ent, tid, ent);
     __syncthreads();
 #pragma unroll 1
-    for (int pt = 0; pt < nw; pt++) {
-        const int ptn = min(pt + 1, nw - 1);
+    for (int pt = p_lo; pt < p_hi; pt++) {
+        const int ptn = min(pt + 1, p_hi - 1);
         entries_request(links, G, b, 32 * ptn, c0, L, vec4, tid, ent);
         parent_request(ptn, nxt);
-        const float *buf = s_ent + (pt & 1) * ENT_FLOATS;
-        if (active) {
+        const float *buf = s_ent + ((pt - p_lo) & 1) * ENT_FLOATS;
+        // (a tile without an allowed pair contributes nothing, as in the parents' part)
+        const bool live = __ballot((cur.flags & 1u) == 0 && cur.allow != 0u) != 0ull;
+        if (active && live) {
             const int a = 32 * pt + p;
             ParentTerms ptm;
             ptm.lg2v = cur.lgv;
@@ -697,7 +733,7 @@ __device__ __forceinline__ void bwd_children(uint4 *lb_lds, int b, const T *__re
             }
         }
         cur = nxt;
-        entries_store(s_ent + ((pt + 1) & 1) * ENT_FLOATS, tid, ent);
+        entries_store(s_ent + ((pt - p_lo + 1) & 1) * ENT_FLOATS, tid, ent);
         __syncthreads();
     }
     if (!active) return;
@@ -740,11 +776,12 @@ __global__ __launch_bounds__(LF_NT) void links_fused_bwd_dg_kernel(const T *__re
                                                                   const unsigned *__restrict__ masks, float *__restrict__ dgate,
                                                                   BwdWorkspace ws, int L, int H, float scale2, float scale) {
     extern __shared__ uint4 lb_lds[];
-    bwd_parents<T, NCH, 0>(lb_lds, blockIdx.z, q, kl, kr, gate, head_lse, links, G, masks, nullptr, nullptr, dgate, ws, L, H, scale2, scale);
+    bwd_parents<T, NCH, 0>(lb_lds, blockIdx.x, blockIdx.y, blockIdx.z, q, kl, kr, gate, head_lse, links, G, masks, nullptr, nullptr, dgate, ws, L, H,
+                           scale2, scale);
 }
 
 // ---- second launch: the parents' and the children's parts side by side, so that the device is filled by both.
-// grid (tiles of 32, groups of four heads, 2 B): sentence blockIdx.z as parents for blockIdx.z < B, else blockIdx.z - B as children.
+// grid (tiles of 32, groups of four heads, 2 B): tiles x groups x B workgroups for the parents and as many for the children.
 template <typename T, int NCH>
 __global__ __launch_bounds__(LF_NT) void links_fused_bwd_main_kernel(const T *__restrict__ q, const T *__restrict__ kl, const T *__restrict__ kr,
                                                                     const float *__restrict__ gate, const float *__restrict__ head_lse,
@@ -753,10 +790,17 @@ __global__ __launch_bounds__(LF_NT) void links_fused_bwd_main_kernel(const T *__
                                                                     T *__restrict__ dkr, BwdWorkspace ws, int B, int L, int H, float scale2,
                                                                     float scale) {
     extern __shared__ uint4 lb_lds[];
-    if ((int)blockIdx.z < B)
-        bwd_parents<T, NCH, 1>(lb_lds, blockIdx.z, q, kl, kr, gate, head_lse, links, G, masks, dq, dkl, nullptr, ws, L, H, scale2, scale);
+    // Which (role, tile, group of heads, sentence) a workgroup takes follows from its place in the launch order (x runs
+    // fastest), heaviest first: a tile of parents has the tiles of right children from its own on to do, a tile of right
+    // children the tiles of parents up to its own, so the first tile of parents and the last of children lead, and the
+    // workgroups that find most of their tiles masked come when the others are running out.
+    const int tiles = gridDim.x, groups = gridDim.y;
+    const int n = blockIdx.x + tiles * (blockIdx.y + groups * blockIdx.z), per_class = groups * 2 * B;
+    const int k = n / per_class, j = n - k * per_class, role = j & 1, r = j >> 1, group = r % groups, b = r / groups;
+    if (role == 0)
+        bwd_parents<T, NCH, 1>(lb_lds, k, group, b, q, kl, kr, gate, head_lse, links, G, masks, dq, dkl, nullptr, ws, L, H, scale2, scale);
     else
-        bwd_children<T, NCH>(lb_lds, blockIdx.z - B, q, kl, kr, head_lse, links, G, masks, dkr, ws, L, H, scale2, scale);
+        bwd_children<T, NCH>(lb_lds, tiles - 1 - k, group, b, q, kl, kr, head_lse, links, G, masks, dkr, ws, L, H, scale2, scale);
 }
 
 // ---- d kl[0,h]: what the parents' launch left, the null option of every parent and parent 0's clamped left option.
