@@ -9,6 +9,7 @@ contract; the arithmetic runs in hand-written HIP kernels for gfx950 reached thr
 ``viterbi_decoding``, whose reference version is itself a host loop) raises.
 """
 import threading
+import weakref
 
 import torch
 from torch.autograd import Function
@@ -522,6 +523,26 @@ def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unre
     return out[:, :maxlen].to(torch.float32)
 
 
+_MASK_CACHE = {}
+
+
+def _as_flag_mask(t):
+    """A support mask as the kernels read it (one byte per entry, non-zero = set).  The masks of a model are built once per
+    graph length and handed to every call: the converted copy of an integer mask is kept while the tensor it was made
+    from is alive and unchanged (same storage, same version counter), so that a call does not pay a launch per mask."""
+    if t.dtype in (torch.bool, torch.uint8):
+        return t.contiguous()
+    key = (t.data_ptr(), t._version, t.dtype, tuple(t.shape), tuple(t.stride()), str(t.device))
+    hit = _MASK_CACHE.get(key)
+    if hit is not None and hit[0]() is t:
+        return hit[1]
+    flags = t.ne(0).contiguous()
+    if len(_MASK_CACHE) >= 64:
+        _MASK_CACHE.clear()
+    _MASK_CACHE[key] = (weakref.ref(t), flags)
+    return flags
+
+
 class PCFGExtractLinksFunc(Function):
     """The model's link scorer after its projections (glat_decomposed_with_link_two_hands_tri_pcfg.py:153-199).  For fp16
     and fp32 chunks with head dimensions the library covers, the batched products run on the matrix cores inside the
@@ -558,8 +579,7 @@ class PCFGExtractLinksFunc(Function):
                 # the products on the matrix cores inside the kernels: one launch forward, three backward
                 gate = gate_logits.float().contiguous()
                 prev = prev_output_tokens.to(torch.int64).contiguous()
-                masks = [t.contiguous() if t.dtype in (torch.bool, torch.uint8) else t.ne(0).contiguous()
-                         for t in (left_tree_mask, right_tree_mask, main_chain)]
+                masks = [_as_flag_mask(t) for t in (left_tree_mask, right_tree_mask, main_chain)]
                 links = torch.empty((B, L, 2, L), dtype=torch.float32, device=dev)
                 lse = torch.empty((B, L, H), dtype=torch.float32, device=dev)
                 tile_masks = torch.empty((B, L, 1 + (L + 31) // 32), dtype=torch.int32, device=dev) if need_grad else None
@@ -579,9 +599,7 @@ class PCFGExtractLinksFunc(Function):
             Z = torch.matmul(A, Kr.transpose(-1, -2))
             gate = gate_logits.float().contiguous()
             prev = prev_output_tokens.to(torch.int64).contiguous()
-            masks = []
-            for t in (left_tree_mask, right_tree_mask, main_chain):
-                masks.append(t.contiguous() if t.dtype in (torch.bool, torch.uint8) else t.ne(0).contiguous())
+            masks = [_as_flag_mask(t) for t in (left_tree_mask, right_tree_mask, main_chain)]
             links = torch.empty((B, L, 2, L), dtype=torch.float32, device=dev)
             lse = torch.empty((B, L, H), dtype=torch.float32, device=dev)
             _lib.check(lib.pcfgnat_extract_links_forward(Z.data_ptr(), A.data_ptr(), gate.data_ptr(), prev.data_ptr(), int(pad_index),

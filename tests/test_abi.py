@@ -98,3 +98,21 @@ def test_host_readout_matches_oracle():
                                           tokens, left_mask, 1)
         assert got.dtype == torch.float32
         assert np.array_equal(got.numpy(), want)
+
+
+def test_support_mask_conversion_is_kept_per_tensor_and_version():
+    """The link scorer converts integer support masks to flag bytes once per tensor: the same tensor gives the kept copy,
+    an in-place change or another tensor (also one with equal contents) gives a fresh one."""
+    import torch
+    from pcfg_nat_amd import custom_ops as ops
+    m = torch.tensor([[0, 1], [2, 0]])
+    a = ops._as_flag_mask(m)
+    assert a.dtype == torch.bool and a.tolist() == [[False, True], [True, False]]
+    assert ops._as_flag_mask(m) is a
+    m[0, 0] = 5
+    b = ops._as_flag_mask(m)
+    assert b is not a and b.tolist() == [[True, True], [True, False]]
+    other = m.clone()
+    assert ops._as_flag_mask(other) is not b and ops._as_flag_mask(other).tolist() == b.tolist()
+    flags = torch.tensor([True, False])
+    assert ops._as_flag_mask(flags) is flags
