@@ -664,12 +664,14 @@ __global__ __launch_bounds__(NT, FROM_LOGITS ? 1 : 6) void lsg_bwd_kernel(T *__r
             x = lo;
             y = hi;
         };
-        order(q.x, q.y);  // a sorting network of five exchanges
-        order(q.z, q.w);
-        order(q.x, q.z);
-        order(q.y, q.w);
-        order(q.y, q.z);
-        *my_box = q;
+        if (count > 1) {  // a sorting network of five exchanges
+            order(q.x, q.y);
+            order(q.z, q.w);
+            order(q.x, q.z);
+            order(q.y, q.w);
+            order(q.y, q.z);
+        }
+        *my_box = q;  // (sorted, the unused entries marked)
         const unsigned e[BOX] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int k = 0; k < BOX; k++)
