@@ -8,6 +8,8 @@ contract; the arithmetic runs in hand-written HIP kernels for gfx950 reached thr
 ``libpcfg_nat_hip.so`` on the current HIP stream.  There is no CPU path: calling with CPU tensors (other than
 ``viterbi_decoding``, whose reference version is itself a host loop) raises.
 """
+import ctypes
+import os
 import threading
 import weakref
 
@@ -503,11 +505,12 @@ def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unre
             scratch = torch.empty((B, 2 * L), dtype=torch.int64, device=dev)
             cnt = _pinned_counts.take(B)  # written by the kernel, read after the one stream wait
             try:
+                _pinned_counts.arm(cnt, B)
                 _lib.check(lib.pcfgnat_viterbi_decoding(pl.data_ptr(), ol.data_ptr(), Lt.data_ptr(), Rt.data_ptr(), Mt.data_ptr(),
                                                         tok.data_ptr(), mask.data_ptr(), mask.size(0), int(pad_index),
                                                         out.data_ptr(), cnt.data_ptr(), scratch.data_ptr(), B, L, Lq,
                                                         _stream(out)), lib)
-                torch.cuda.current_stream(dev).synchronize()
+                _pinned_counts.wait(cnt, B, torch.cuda.current_stream(dev))
                 counts = cnt[:B].tolist()
             finally:
                 _pinned_counts.give_back(cnt)
@@ -743,8 +746,8 @@ def _length_penalty(Lq, beta, device):
 
 class _PinnedCounts:
     """Pinned int64 host buffers for the per-sentence token counts of the decode calls.  Pinned host memory is addressable
-    from the device, so the kernels write the counts straight into it and the caller reads them after waiting for its
-    stream.  A call takes a buffer out of the pool for its own use and puts it back when it has read the counts: calls
+    from the device, so the kernels write the counts straight into it and the caller reads them as they arrive (``arm`` /
+    ``wait`` below), at the latest after waiting for its stream.  A call takes a buffer out of the pool for its own use and puts it back when it has read the counts: calls
     that overlap (several host threads, several streams of one device) never share one.  Allocating pinned memory takes
     about a hundred microseconds, hence the pool; it holds as many buffers as calls have ever overlapped."""
 
@@ -762,6 +765,33 @@ class _PinnedCounts:
     def give_back(self, buf):
         with self._lock:
             self._free.append(buf)
+
+    # The kernels write a sentence's count (>= -1) as the last thing they do for it.  Instead of waiting for the stream,
+    # whose wake-up costs the host some microseconds after the kernel has ended, the caller marks the entries before the
+    # launch and watches them turn: device stores to pinned host memory reach the host while the kernel is still running.
+    # Where they do not (a host-memory mode in which they only arrive with the end of the kernel), the watch runs into
+    # its bound once, the stream wait takes over and the watching is switched off for the rest of the process.
+    NOT_YET = -2
+    SPIN_LIMIT = 200000  # reads of an entry that has not turned: some tens of milliseconds
+    polling = os.environ.get("PCFGNAT_DECODE_POLL", "1") != "0"
+
+    def arm(self, buf, n):
+        if self.polling:
+            buf[:n].fill_(self.NOT_YET)
+
+    def wait(self, buf, n, stream):
+        if self.polling:
+            entries = (ctypes.c_int64 * n).from_address(buf.data_ptr())
+            i = spins = 0
+            while i < n and spins < self.SPIN_LIMIT:
+                if entries[i] != self.NOT_YET:
+                    i += 1
+                else:
+                    spins += 1
+            if i == n:
+                return
+            _PinnedCounts.polling = False
+        stream.synchronize()
 
 
 _pinned_counts = _PinnedCounts()
@@ -781,8 +811,9 @@ def _viterbi_decode_call(name, B, L, ml, dev, extra_words, call):
         # synchronisation of the decode is a stream wait, with no copy in front of it
         host = _pinned_counts.take(B)  # written by the kernel, read after the one stream wait
         try:
+            _pinned_counts.arm(host, B)
             _lib.check(call(lib, block.data_ptr(), nwork, host.data_ptr()), lib)
-            torch.cuda.current_stream(dev).synchronize()
+            _pinned_counts.wait(host, B, torch.cuda.current_stream(dev))
             counts = host[:B].tolist()
         finally:
             _pinned_counts.give_back(host)
@@ -898,10 +929,11 @@ def pcfg_lookahead_decode(links, unreduced_logits, unreduced_tokens, output_leng
         out = torch.empty((B, L), dtype=torch.int64, device=dev)
         cnt = _pinned_counts.take(B)  # written by the kernel, read after the one stream wait
         try:
+            _pinned_counts.arm(cnt, B)
             _lib.check(lib.pcfgnat_lookahead_decode(links.data_ptr(), ob_ptr, float(beta), ol.data_ptr(), tok.data_ptr(),
                                                     mask.data_ptr(), mask.size(0), int(pad_index), idx.data_ptr(), out.data_ptr(),
                                                     cnt.data_ptr(), B, L, K - 1, _stream(links)), lib)
-            torch.cuda.current_stream(dev).synchronize()
+            _pinned_counts.wait(cnt, B, torch.cuda.current_stream(dev))
             counts = cnt[:B].tolist()
         finally:
             _pinned_counts.give_back(cnt)

@@ -684,6 +684,29 @@ def test_decode_from_logits_is_front_end_plus_decode(case, dtype):
         ops.pcfg_viterbi_decode_logits(logits.double(), links, ol, left_mask, synth.PAD)
 
 
+def test_decode_waits_for_the_stream_where_the_counts_do_not_turn():
+    """The decode calls watch the token counts turn in pinned host memory; a watch that runs into its bound (forced here by
+    a bound of zero reads) hands over to the stream wait and switches the watching off, with the same results."""
+    import oracle_ops
+    batch = _decode_case("L96")
+    ob, tok = synth.ob_and_tokens(batch["logits"])
+    links, ol = batch["links"], batch["output_length"]
+    left_mask, _, _ = synth.support_masks(links.shape[1], 1)
+    want_tok, want_len = harness.viterbi_decode(ob, tok, links, ol, left_mask, ops=oracle_ops)
+    pool = type(ops._pinned_counts)
+    limit, polling = pool.SPIN_LIMIT, pool.polling
+    try:
+        pool.polling, pool.SPIN_LIMIT = True, 0
+        for expect_polling_before in (True, False):
+            assert pool.polling == expect_polling_before
+            got_tok, got_len = harness.viterbi_decode(ob.to(DEV), tok.to(DEV), links.to(DEV), ol.to(DEV), left_mask.to(DEV),
+                                                      single_call=True)
+            assert torch.equal(got_len.cpu(), want_len) and torch.equal(got_tok.cpu(), want_tok)
+        assert pool.polling is False
+    finally:
+        pool.SPIN_LIMIT, pool.polling = limit, polling
+
+
 @pytest.mark.parametrize("mode", ["one_workgroup", "blocks_give_up"])
 @pytest.mark.parametrize("case", ["L224", "L288", "L400", "L512"])
 def test_single_call_decode_sweeps_agree(mode, case):
