@@ -96,15 +96,18 @@ def test_lsg_backward_matches_torch_ops(dtype):
         assert torch.allclose(got, ref, rtol=1e-5, atol=1e-9)
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
-def test_lsg_backward_adds_duplicate_targets_in_target_order(dtype):
+@pytest.mark.parametrize("dtype,V,T", [(torch.float16, 16384, 24), (torch.float32, 16384, 24), (torch.float32, 30001, 40),
+                                       (torch.float16, 50000, 600)])
+def test_lsg_backward_adds_duplicate_targets_in_target_order(dtype, V, T):
     """Targets that share a column are added one after the other in the order of the target positions (scatter_add_ along
     the last dimension, pcfg_loss.py:177), however they reach the thread that owns the column: three of one column (sorted
     on arrival), six of another (more than the thread keeps: it goes through all targets), columns of one thread's
     different chunks, two elements of one chunk.  The upstream gradients are multiples of 2^-5, so that their sum is exact
-    in any order and every bit of the result is fixed: compared for equality with the same operations one at a time."""
+    in any order and every bit of the result is fixed: compared for equality with the same operations one at a time.
+    The larger vocabularies have rows with more 16-byte chunks than a thread keeps in registers (targets in those chunks
+    too, the odd one with rows that start off the 16-byte grid), the last case more than 512 targets per row."""
     g = torch.Generator().manual_seed(21)
-    B, L, V, T = 2, 5, 16384, 24
+    B, L = 2, 5
     epv = 8 if dtype == torch.float16 else 4
     probs = torch.softmax(torch.randn(B, L, V, generator=g) * 2, -1).to(dtype)
     tgt = torch.randint(0, V, (B, T), generator=g)
@@ -115,6 +118,11 @@ def test_lsg_backward_adds_duplicate_targets_in_target_order(dtype):
     tgt[:, 7] = c + 1                # the same 16-byte chunk
     tgt[:, 8] = c + 512 * epv        # the same thread's next chunk
     tgt[:, 10] = c + 2 * 512 * epv
+    if V > 10 * 512 * epv + 100:     # chunks beyond the ten a thread keeps in registers: one target, a pair, a triple
+        far = 10 * 512 * epv + 40
+        tgt[:, 12] = far
+        tgt[:, [13, 16]] = far + 3 * epv + 1
+        tgt[:, [14, 17, 19]] = V - 2
     idx = tgt.unsqueeze(1).expand(-1, L, -1).contiguous()
     gout = torch.randint(-40, 41, (B, L, T), generator=g).float() / 32
     # one rounding to the buffer's dtype per operation, the targets one after the other
