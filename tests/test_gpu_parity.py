@@ -510,6 +510,28 @@ def test_glat_single_call_small_ragged(ml):
     assert torch.allclose(got["max_tree_lprob"].cpu(), want["max_tree_lprob"], rtol=2e-5)
 
 
+@pytest.mark.parametrize("case", ["wmt_small", "L130", "L256", "L512_long"])
+@pytest.mark.parametrize("strategy", ["number-random", None])
+def test_glat_single_call_on_longer_graphs(case, strategy):
+    """The one-call GLAT pass (best tree and glue by one workgroup per sentence) against the torch glue over the separate
+    device operators with the same random numbers, on graphs whose link matrices or whose tables no longer fit the
+    workgroup's LDS beside each other (the walk then reads them from memory); the separate operators are held against the
+    oracle by the tests above."""
+    batch = _train_case(case)
+    logits, tgt, links = batch["logits"].to(DEV), batch["targets"].to(DEV), batch["links"].to(DEV)
+    B, L, _ = logits.shape
+    prev = torch.full((B, L), 3, dtype=torch.int64)
+    prev = prev.masked_fill(torch.arange(L).view(1, L) >= batch["output_length"].view(B, 1), synth.PAD).to(DEV)
+    g1, g2 = torch.Generator().manual_seed(11), torch.Generator().manual_seed(11)
+    want = harness.glat_alignment(logits, tgt, prev, links, 0.5, generator=g1, noise_device="cpu", glance_strategy=strategy)
+    got = harness.glat_alignment(logits, tgt, prev, links, 0.5, generator=g2, noise_device="cpu", glance_strategy=strategy,
+                                 single_call=True)
+    for key in ("path", "keep_word_mask", "glat_prev_output_tokens", "matchmask", "same_num", "glance_nums"):
+        assert got[key].dtype == want[key].dtype and torch.equal(got[key], want[key]), key
+    assert torch.allclose(got["max_tree_lprob"], want["max_tree_lprob"], rtol=2e-5)
+    assert int((got["path"] >= 0).sum()) > 0
+
+
 @pytest.mark.parametrize("B,L,H,F,dtype", [(3, 18, 2, 4, torch.float32), (2, 34, 8, 16, torch.float32), (4, 128, 8, 64, torch.float16),
                                             (2, 514, 4, 8, torch.float32), (2, 22, 16, 8, torch.float32), (2, 12, 1, 8, torch.float32),
                                             (2, 200, 4, 16, torch.float16), (2, 256, 2, 24, torch.float32), (3, 130, 8, 64, torch.float32),
