@@ -626,6 +626,47 @@ def test_extract_links_products_inside_edge_shapes(B, L, H, F, dtype, ms):
         assert (x.float() - y.float()).abs().max().item() <= tol * scale, name
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_extract_links_products_inside_arbitrary_masks(dtype):
+    """The backward leaves out the tiles of 32 x 32 (parent, right child) pairs in which the masks allow nothing and runs
+    over the range of tiles that hold pairs, which it finds from the masks alone: tree masks that are no triangle (allowed
+    right children in front of their parents), a band of right children that no parent may take (a hole in the middle of
+    the range), parents without any allowed right child, pad nodes behind the sentences - against the form with the
+    products through torch, which knows no tiles."""
+    g = torch.Generator().manual_seed(99)
+    B, L, H, F = 3, 162, 4, 16  # six tiles, the last one partial
+    q, kl, kr = ((torch.randn(B, L, H, F, generator=g) * 0.7).to(dtype).to(DEV) for _ in range(3))
+    gate = torch.randn(B, L, H, generator=g).to(dtype).to(DEV)
+    ms = [L, 100, 40]
+    prev = torch.full((B, L), 3).masked_fill(torch.arange(L).view(1, L) >= torch.tensor(ms).view(B, 1), synth.PAD).to(DEV)
+    rm = (torch.rand(L, L, generator=g) > 0.15).long()   # 1 = forbidden: about 15 % of the pairs allowed, anywhere
+    rm[:, 64:96] = 1                                     # no parent may take a right child of the third tile
+    rm[32:64, :32] = 0                                   # the second tile of parents: every child of the first tile
+    rm[96:100, :] = 1                                    # a few parents without a right child
+    lm = (torch.rand(L, L, generator=g) > 0.5).long()
+    lm[:, 0] = 0                                         # node 0 may be everybody's left child
+    mc = torch.ones(L, dtype=torch.bool)
+    lm, rm, mc = lm.to(DEV), rm.to(DEV), mc.to(DEV)
+    G = torch.randn(B, L, 2, L, generator=g).to(DEV)
+    res = []
+    for inside in (True, False):
+        leaves = [t.clone().requires_grad_(True) for t in (q, kl, kr, gate)]
+        out = ops.pcfg_extract_links(*leaves, prev, synth.PAD, lm, rm, mc, inside)
+        fin = torch.isfinite(out)
+        out.masked_fill(~fin, 0).mul(G).sum().backward()
+        res.append((out.detach(), [t.grad for t in leaves]))
+    (a, ga), (b, gb) = res
+    fin = torch.isfinite(a)
+    assert torch.equal(fin, torch.isfinite(b)) and fin.any() and not fin[:, :, :, 64:96].any()
+    assert fin[0, 32:64, :, :32].any()                   # links to right children in front of the parents
+    assert torch.allclose(a[fin], b[fin], rtol=2e-5, atol=2e-5)
+    for name, x, y in zip(("q", "kl", "kr", "gate"), ga, gb):
+        assert torch.isfinite(x).all(), name
+        scale = max(y.float().abs().max().item(), 1e-6)
+        tol = 4e-3 if dtype == torch.float16 else 1e-4
+        assert (x.float() - y.float()).abs().max().item() <= tol * scale, name
+
+
 def test_extract_links_fused_form_rejects_what_it_does_not_cover():
     lib = ops.get_pcfg_kernel()
     assert lib.pcfgnat_extract_links_fused_supported(ops._DTYPE_CODE[torch.float32], 256, 2, 24) == 0   # head dimension
