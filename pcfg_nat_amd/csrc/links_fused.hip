@@ -349,21 +349,77 @@ __global__ __launch_bounds__(LF_NT) void links_fused_fwd_kernel(const T *__restr
     }
     __syncthreads();
 
-    // ---- pass 2: mix the heads, online over h per entry; tiles outside, heads inside.  The running shift of an entry is
-    // kept integral, so that moving the sum to a new shift is an exact change of exponent and each term costs one
-    // exponential.
+    // ---- pass 2: mix the heads per entry; tiles outside, heads inside.  What a head adds to an entry is a probability
+    // (its gate's share times its softmax: 2^t with t <= 0), so the sum over the heads can neither overflow nor lose its
+    // largest term, and it is formed as it stands: one exponential and one addition per term.  Only where an allowed
+    // entry's sum comes out below 2^-100 may terms have been lost to underflow; the wave then takes the tile again with a
+    // running integral shift per entry (moving the sum to a new shift is an exact change of exponent), which covers the
+    // whole range of the logarithmic form at nine more instructions per term.
     if (ntw > 0) {
         const int a = a0 + p;
         const bool unusable = (flags & 1u) != 0;
         const bool vec4 = (L & 3) == 0;
+        // the links of tile ct from the sums and shifts of its entries: links = (shift + log2 sum) ln 2
+        auto store_tile = [&](int ct, const float (&mx0)[16], const float (&sm0)[16], const float (&mx1)[16], const float (&sm1)[16]) {
+            if (a >= L) return;
+            float *out0 = links + ((size_t)b * L + a) * 2 * L, *out1 = out0 + L;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                float v0[4], v1[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int r = 4 * g + u;
+                    v0[u] = (unusable || sm0[r] == 0.f) ? NEG_INF_F : (mx0[r] + lg2(sm0[r])) * LF_LN2;
+                    v1[u] = (unusable || sm1[r] == 0.f) ? NEG_INF_F : (mx1[r] + lg2(sm1[r])) * LF_LN2;
+                }
+                const int c = 32 * ct + 8 * g + 4 * kb;  // the four rows of the group are consecutive right children
+                if (vec4 && c < L) {
+                    *reinterpret_cast<float4 *>(out0 + c) = make_float4(v0[0], v0[1], v0[2], v0[3]);
+                    *reinterpret_cast<float4 *>(out1 + c) = make_float4(v1[0], v1[1], v1[2], v1[3]);
+                } else {
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        if (c + u < L) {
+                            out0[c + u] = v0[u];
+                            out1[c + u] = v1[u];
+                        }
+                    }
+                }
+            }
+        };
+        // tile ct over all heads with the running shift (the rare second go; its keys are not requested ahead)
+        auto shifted_tile = [&](int ct) {
+            float mx0[16], sm0[16], mx1[16], sm1[16];
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                mx0[r] = mx1[r] = LF_FLOOR;
+                sm0[r] = sm1[r] = 0.f;
+            }
+            penalties(ct);
+#pragma unroll 1
+            for (int h = 0; h < H; h++) {
+                uint4 keys[NCH];
+                right_keys(ct, h, keys);
+                float z0[16], z1[16];
+                scores(keys, h, z0, z1);
+                const float off = s_lse[p * H + h];
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const float t0 = z0[r] + off, t1 = z1[r] + off;
+                    const float n0 = fmaxf(mx0[r], __builtin_ceilf(t0)), n1 = fmaxf(mx1[r], __builtin_ceilf(t1));
+                    sm0[r] = __builtin_ldexpf(sm0[r], (int)fmaxf(mx0[r] - n0, -256.f)) + ex2(t0 - n0);  // 2^-256 of a sum of H terms is 0
+                    sm1[r] = __builtin_ldexpf(sm1[r], (int)fmaxf(mx1[r] - n1, -256.f)) + ex2(t1 - n1);
+                    mx0[r] = n0;
+                    mx1[r] = n1;
+                }
+            }
+            store_tile(ct, mx0, sm0, mx1, sm1);
+        };
         uint4 cur[NCH], nxt[NCH];
         right_keys(wave, 0, cur);
-        float mx0[16], sm0[16], mx1[16], sm1[16];
+        float sm0[16], sm1[16];
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            mx0[r] = mx1[r] = LF_FLOOR;
-            sm0[r] = sm1[r] = 0.f;
-        }
+        for (int r = 0; r < 16; r++) sm0[r] = sm1[r] = 0.f;
         const int steps = H * ntw;
         int h = 0, i = 0;  // step it = i * H + h
 #pragma unroll 1
@@ -387,45 +443,24 @@ __global__ __launch_bounds__(LF_NT) void links_fused_fwd_kernel(const T *__restr
             const float off = s_lse[p * H + h];
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const float t0 = z0[r] + off, t1 = z1[r] + off;
-                const float n0 = fmaxf(mx0[r], __builtin_ceilf(t0)), n1 = fmaxf(mx1[r], __builtin_ceilf(t1));
-                sm0[r] = __builtin_ldexpf(sm0[r], (int)fmaxf(mx0[r] - n0, -256.f)) + ex2(t0 - n0);  // 2^-256 of a sum of H terms is 0
-                sm1[r] = __builtin_ldexpf(sm1[r], (int)fmaxf(mx1[r] - n1, -256.f)) + ex2(t1 - n1);
-                mx0[r] = n0;
-                mx1[r] = n1;
+                sm0[r] += ex2(z0[r] + off);
+                sm1[r] += ex2(z1[r] + off);
             }
             if (h == H - 1) {  // the tile is complete
-                if (a < L) {
-                    float *out0 = links + ((size_t)b * L + a) * 2 * L, *out1 = out0 + L;
+                bool thin = false;  // an allowed entry (penalty 0) with a sum so small that terms may have underflowed
 #pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        float v0[4], v1[4];
+                for (int r = 0; r < 16; r++)
+                    thin = thin || (pen0[r] == 0.f && sm0[r] < LF_THIN_SUM) || (pen1[r] == 0.f && sm1[r] < LF_THIN_SUM);
+                if (__ballot(thin && !unusable) != 0ull) {
+                    shifted_tile(ct);
+                } else {
+                    float zero[16];
 #pragma unroll
-                        for (int u = 0; u < 4; u++) {
-                            const int r = 4 * g + u;
-                            v0[u] = (unusable || sm0[r] == 0.f) ? NEG_INF_F : (mx0[r] + lg2(sm0[r])) * LF_LN2;
-                            v1[u] = (unusable || sm1[r] == 0.f) ? NEG_INF_F : (mx1[r] + lg2(sm1[r])) * LF_LN2;
-                        }
-                        const int c = 32 * ct + 8 * g + 4 * kb;  // the four rows of the group are consecutive right children
-                        if (vec4 && c < L) {
-                            *reinterpret_cast<float4 *>(out0 + c) = make_float4(v0[0], v0[1], v0[2], v0[3]);
-                            *reinterpret_cast<float4 *>(out1 + c) = make_float4(v1[0], v1[1], v1[2], v1[3]);
-                        } else {
-#pragma unroll
-                            for (int u = 0; u < 4; u++) {
-                                if (c + u < L) {
-                                    out0[c + u] = v0[u];
-                                    out1[c + u] = v1[u];
-                                }
-                            }
-                        }
-                    }
+                    for (int r = 0; r < 16; r++) zero[r] = 0.f;
+                    store_tile(ct, zero, sm0, zero, sm1);
                 }
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    mx0[r] = mx1[r] = LF_FLOOR;
-                    sm0[r] = sm1[r] = 0.f;
-                }
+                for (int r = 0; r < 16; r++) sm0[r] = sm1[r] = 0.f;
             }
             h = hn;
             i = in;

@@ -10,6 +10,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int PT = 32;        // parents per tile
 constexpr int LF_NT = 256;    // threads per workgroup: four waves
+constexpr float LF_THIN_SUM = 7.888609e-31f;  // 2^-100: below it a sum of probabilities may have lost terms to underflow
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));

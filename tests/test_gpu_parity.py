@@ -627,6 +627,27 @@ def test_extract_links_products_inside_edge_shapes(B, L, H, F, dtype, ms):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_extract_links_products_inside_keeps_links_far_below_float_range(dtype):
+    """Sharp heads: many links come out hundreds of nats below zero, where every head's share of the entry is below the
+    smallest float.  The mixture over the heads, formed as a plain sum of probabilities where that is safe, must take such
+    entries through the shifted form and return the logarithm the float64 restatement has - finite, not -inf."""
+    from oracle import extract_links_ref as ref
+    g = torch.Generator().manual_seed(123)
+    B, L, H, F = 2, 96, 2, 64
+    q, kl, kr = ((torch.randn(B, L, H, F, generator=g) * 8).to(dtype) for _ in range(3))
+    gate = torch.randn(B, L, H, generator=g).to(dtype)
+    prev = torch.full((B, L), 3).masked_fill(torch.arange(L).view(1, L) >= torch.tensor([L, 70]).view(B, 1), synth.PAD)
+    lm, rm, mc = synth.support_masks(L, 1)
+    want = ref.extract_links(q.double(), kl.double(), kr.double(), gate.double(), prev, synth.PAD, lm, rm, mc).double()
+    fin = torch.isfinite(want)
+    assert (want[fin] < -100).sum() > 100 and (want[fin] < -200).any()   # far below log(2^-126) = -87.3
+    got = ops.pcfg_extract_links(q.to(DEV), kl.to(DEV), kr.to(DEV), gate.to(DEV), prev.to(DEV), synth.PAD, lm.to(DEV), rm.to(DEV),
+                                 mc.to(DEV))
+    assert torch.equal(torch.isfinite(got).cpu(), fin)
+    assert torch.allclose(got.cpu().double()[fin], want[fin], rtol=2e-5, atol=2e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_extract_links_products_inside_arbitrary_masks(dtype):
     """The backward leaves out the tiles of 32 x 32 (parent, right child) pairs in which the masks allow nothing and runs
     over the range of tiles that hold pairs, which it finds from the masks alone: tree masks that are no triangle (allowed
