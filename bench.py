@@ -274,7 +274,7 @@ def link_scorer_timing(dev):
     res = {}
     for name, fn in (("forward_ms", fwd), ("forward_backward_ms", fwd_bwd),
                      ("forward_backward_products_through_torch_ms", lambda: fwd_bwd(False))):
-        for _ in range(40):  # autograd's backward thread takes some tens of calls to reach its steady pace
+        for _ in range(10):
             fn()
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
