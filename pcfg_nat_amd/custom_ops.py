@@ -584,8 +584,11 @@ class PCFGExtractLinksFunc(Function):
                 prev = prev_output_tokens.to(torch.int64).contiguous()
                 masks = [_as_flag_mask(t) for t in (left_tree_mask, right_tree_mask, main_chain)]
                 links = torch.empty((B, L, 2, L), dtype=torch.float32, device=dev)
-                lse = torch.empty((B, L, H), dtype=torch.float32, device=dev)
-                tile_masks = torch.empty((B, L, 1 + (L + 31) // 32), dtype=torch.int32, device=dev) if need_grad else None
+                # the per-head normalisers and, for the backward, the masks per parent as bits: one allocation
+                nw = 1 + (L + 31) // 32
+                side = torch.empty((B * L * (H + (nw if need_grad else 0)),), dtype=torch.float32, device=dev)
+                lse = side[:B * L * H].view(B, L, H)
+                tile_masks = side[B * L * H:].view(torch.int32).view(B, L, nw) if need_grad else None
                 _lib.check(lib.pcfgnat_extract_links_fused_forward(q.data_ptr(), kl.data_ptr(), kr.data_ptr(), code, gate.data_ptr(),
                                                                    prev.data_ptr(), int(pad_index), masks[0].data_ptr(),
                                                                    masks[1].data_ptr(), masks[2].data_ptr(), links.data_ptr(),
@@ -625,10 +628,10 @@ class PCFGExtractLinksFunc(Function):
             with torch.cuda.device(dev):
                 st = _stream(q)
                 G = grad_links.float().contiguous()
-                dq, dkl, dkr = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
-                dgate = torch.empty((B, L, H), dtype=torch.float32, device=dev)
-                ws = torch.empty((lib.pcfgnat_extract_links_fused_backward_workspace_bytes(B, L, H, F) + 3) // 4, dtype=torch.float32,
-                                 device=dev)
+                dq, dkl, dkr = torch.empty((3, B, L, H, F), dtype=q.dtype, device=dev).unbind(0)  # one allocation each way
+                nws = (lib.pcfgnat_extract_links_fused_backward_workspace_bytes(B, L, H, F) + 3) // 4
+                block = torch.empty((nws + B * L * H,), dtype=torch.float32, device=dev)  # the workspace first: it wants 16-byte alignment
+                ws, dgate = block[:nws], block[nws:].view(B, L, H)
                 _lib.check(lib.pcfgnat_extract_links_fused_backward(G.data_ptr(), links.data_ptr(), lse.data_ptr(), tile_masks.data_ptr(),
                                                                     q.data_ptr(), kl.data_ptr(), kr.data_ptr(), code, gate.data_ptr(),
                                                                     dq.data_ptr(), dkl.data_ptr(), dkr.data_ptr(), dgate.data_ptr(),
