@@ -192,6 +192,22 @@ void pcfgnat_pipeline_config(int max_workgroups, int spin_limit);
 void pcfgnat_links_grad_range_limit(float log2_limit);
 
 /*
+ * No counterpart in the reference: graphs of up to 130 nodes are swept in the linear domain (probabilities in double,
+ * one multiply-add per term) where the numbers allow it - links and emissions between 2^-150 and 2^8 or zero, every
+ * intermediate at least 2^-bits or exactly zero - and in the log domain, which has no range limit, otherwise; the choice
+ * is made per sentence and per sweep by the kernel.  bits: default and maximum 500; 0 switches the linear sweeps off.
+ * Process-wide, for tests.
+ */
+void pcfgnat_inside_linear_bits(int bits);
+
+/*
+ * No counterpart in the reference: diagnostic counters since the library was loaded (or the last reset) on the current
+ * device - sweeps (forward and outside sweeps count apart) completed in the linear domain, and sweeps the linear
+ * domain handed over to the log domain.  Synchronises with the device.
+ */
+int pcfgnat_inside_linear_counts(unsigned long long *swept, unsigned long long *handed_over, int reset);
+
+/*
  * No counterpart in the reference: diagnostic counters of that fallback since the library was loaded - inside sweeps
  * (forward and outside counted apart) and single-call Viterbi decodes that the one-workgroup kernels redid because a
  * pipelined sweep gave up.  Reads two device counters of the current device (synchronises with the device); reset != 0

@@ -80,6 +80,11 @@ struct AuxView {
 // Head of the dynamic LDS of the register-resident kernels: per-wave column maxima slots[2][8] (16-byte aligned), the
 // column offsets O [T+2] (double) and the shifts D [T+4].
 __host__ __device__ inline int head_floats(int T) { return 16 + 2 * (T + 2) + (T + 4); }
+// Floats of dynamic LDS of the forward role with its tables in LDS and one tile of 64 nodes (rounded to 16 bytes): head,
+// col [2][64], emissions of main nodes and leaves [Mc][T], R, F0h, F1h [Mc][T+2].
+__host__ __device__ inline size_t fwd_role_floats(int Mc, int T) {
+    return ((size_t)head_floats(T) + 2 * 64 + (size_t)2 * Mc * T + (size_t)3 * Mc * (T + 2) + 3) & ~(size_t)3;
+}
 struct LdsHead {
     float *slots, *D;
     double *O;
@@ -113,6 +118,10 @@ constexpr double LN2_D = 0.6931471805599453094;
 // Diagnostic: sweeps (forward or outside, counted apart) that the one-workgroup kernels redid because the pipelined
 // sweep of the sentence gave up, since the library was loaded (pcfgnat_pipeline_redo_counts).
 __device__ unsigned long long g_inside_redone;
+// Diagnostic: sweeps (forward or outside, counted apart) that ran in the linear domain, and those of them that were
+// handed to the log-domain sweep because a number left the range, since the library was loaded
+// (pcfgnat_inside_linear_counts).
+__device__ unsigned long long g_linear_swept, g_linear_handed_over;
 
 __device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float lg2(float x) { return __builtin_amdgcn_logf(x); }
@@ -281,13 +290,334 @@ __device__ __forceinline__ void fwd_sweep(const float (&A0)[R][8 * R], const flo
     }
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// The same two sweeps in the linear domain.  A step of the log-domain sweeps above is bound by instruction issue: some
+// 180 instructions of bookkeeping per wave and step (shifts, reductions over the node's lanes, the table entries) plus
+// add, max, subtract, exp2, add per term in two passes, on two waves per SIMD.  With the probabilities themselves in
+// double a term is one fused multiply-add, and the work is split so that the chain from one column to the next is
+// short: waves 0-3 (one per SIMD) own 16 nodes each, a quad of lanes per node, and do nothing but load the column,
+// multiply, add up the quad, and store the node's three results as doubles into rotating columns; waves 4-6 follow one
+// step behind and turn those columns into the table entries (base-2 logarithms, as the log-domain sweep leaves them),
+// find the exponent of the column maximum, keep the offsets, and watch the range.  The offset of a column is set to the
+// absolute exponent of the latest column maximum known when it is chosen (one or two columns back), so the entries
+// stay within a few steps' worth of decay of one; following the relative exponent alone, with that delay, would
+// oscillate.
+// Doubles are there for their exponent range, not their precision: columns are still rescaled every step, by a power
+// of two (exact), and the tables are relative to the same kind of offsets (D, O / E, P hold integers here).
+// What the range cannot hold must not be lost silently - a node whose inside value is 2^-600 of its column's largest
+// may still carry the whole posterior.  So a sweep only accepts numbers it can follow: links and emissions between
+// 2^-LIN_INPUT_BITS and 2^LIN_INPUT_TOP (or zero), every shifted row sum and every column entry at least 2^-lin_bits
+// (lin_bits <= 500; or exactly zero, which then is a sum of exact zeros: with these bounds a column grows by less than
+// 2^25 a step, shifts stay below 2^80, and no product of nonzero factors gets below 2^-900; all terms are positive, so
+// nothing cancels).  Anything else raises the workgroup's flag and the sentence is swept again in the log domain by the
+// code above.  lin_bits <= 0 switches the linear sweeps off.
+// ------------------------------------------------------------------------------------------------------------
+constexpr float LIN_INPUT_BITS = 150.f, LIN_INPUT_TOP = 8.f;
+constexpr int LIN_BITS_MAX = 500;
+
+// the partner lane's double inside a quad (every lane has a source, so there is no old value to keep)
+template <int CTRL>
+__device__ __forceinline__ double dpp_d(double v) {
+    return __hiloint2double(__builtin_amdgcn_mov_dpp(__double2hiint(v), CTRL, 0xF, 0xF, true),
+                            __builtin_amdgcn_mov_dpp(__double2loint(v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ double quad_sum_d(double v) {
+    v += dpp_d<DPP_QUAD_XOR1>(v);
+    v += dpp_d<DPP_QUAD_XOR2>(v);
+    return v;
+}
+// Wave64 maximum of an int: DPP inside the rows, the four row results through scalar registers.
+__device__ __forceinline__ int wave_max_i(int v) {
+    v = max(v, dpp_i<DPP_QUAD_XOR1>(v));
+    v = max(v, dpp_i<DPP_QUAD_XOR2>(v));
+    v = max(v, dpp_i<DPP_ROW_HALF_MIRROR>(v));
+    v = max(v, dpp_i<DPP_ROW_MIRROR>(v));
+    const int a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+    const int c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+    return max(max(a, b), max(c, d));
+}
+__device__ __forceinline__ int clamp_shift(int k) { return max(-1000, min(1000, k)); }
+// 2^k for -1022 <= k <= 1023
+__device__ __forceinline__ double pow2_int(int k) { return __hiloint2double((1023 + k) << 20, 0); }
+// 2^v for a base-2 logarithm that passes lin_input_ok (-inf: 0; anything else: some number, the sweep is not used then):
+// the fraction through the hardware exp2, the integer part added to the exponent field
+__device__ __forceinline__ double pow2_of(float v) {
+    const float fl = floorf(v);
+    const double r = (double)ex2(v - fl);
+    const int hi = __double2hiint(r) + ((int)fl << 20);
+    const bool zero = v == NEG_INF_F;
+    return __hiloint2double(zero ? 0 : hi, zero ? 0 : __double2loint(r));
+}
+// 1 if the sweep can take the base-2 logarithm v (as an int, to be combined without branches)
+__device__ __forceinline__ int lin_input_ok(float v) { return (v == NEG_INF_F) | ((v >= -LIN_INPUT_BITS) & (v <= LIN_INPUT_TOP)); }
+// binary exponent e of a positive normal double, d = f * 2^e with f in [0.5, 1)
+__device__ __forceinline__ int exponent_of(double d) { return ((__double2hiint(d) >> 20) & 0x7ff) - 1022; }
+constexpr int NO_EXPONENT = -(1 << 20);  // stands for the exponent of zero
+__device__ __forceinline__ int exponent_or_none(double d) { return d > 0.0 ? exponent_of(d) : NO_EXPONENT; }
+// log2 of a double that is zero or a positive normal number, as a float
+__device__ __forceinline__ float log2_of(double d) {
+    const int hi = __double2hiint(d);
+    const double f = __hiloint2double((hi & 0x800fffff) | 0x3fe00000, __double2loint(d));
+    const float r = (float)exponent_of(d) + lg2((float)f);
+    return d > 0.0 ? r : NEG_INF_F;
+}
+// Order-preserving key of a nonnegative double for running minima over what must stay above the range bound: the high
+// word minus one, unsigned, which sends an exact zero to the top.
+__device__ __forceinline__ unsigned range_key(double d) { return (unsigned)__double2hiint(d) - 1u; }
+__device__ __forceinline__ unsigned range_key_of_bits(int bits) { return ((unsigned)(1023 - bits) << 20) - 1u; }
+
+// Extra dynamic LDS of a linear sweep, behind the role's own (16-byte aligned): three rotating columns [2][64] of
+// doubles, the emission probabilities of main nodes and leaves [Mc][T] each, the shifts [T+4] and the flag (ints).
+__host__ __device__ inline size_t align16(size_t bytes) { return (bytes + 15) & ~(size_t)15; }
+__host__ __device__ inline size_t lin_extra_bytes(int Mc, int T) {
+    return ((size_t)3 * 128 + (size_t)2 * Mc * T) * sizeof(double) + align16((size_t)(T + 6) * sizeof(int));
+}
+struct LinLds {
+    double *col0, *col1, *col2, *em, *el;
+    int *kbuf, *flag;
+    __device__ LinLds(double *base, int Mc, int T) {
+        col0 = base;
+        col1 = col0 + 128;
+        col2 = col1 + 128;
+        em = col2 + 128;
+        el = em + Mc * T;
+        kbuf = reinterpret_cast<int *>(el + Mc * T);
+        flag = kbuf + T + 4;
+    }
+};
+
+// Emission probabilities of the main-chain nodes and of their leaves, [Mc][T] each, filled by the 256 threads of the
+// table waves; false if one is out of range.
+__device__ __forceinline__ bool lin_fill_emissions(double *em, double *el, const float *__restrict__ mt, int mc, int n, int Mc, int T) {
+    int ok_all = 1;
+    const int cells = Mc * T;
+    for (int i0 = threadIdx.x - 256; i0 < cells; i0 += 8 * 256) {  // eight cells' loads in flight per thread
+        float vm[8], vl[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int i = min(i0 + k * 256, cells - 1), a_id = i / T, s = i - a_id * T;
+            vm[k] = mt[(size_t)(2 * a_id + 1) * T + s];
+            vl[k] = mt[(size_t)(2 * a_id) * T + s];
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int i = i0 + k * 256, a_id = i / T, s = i - a_id * T;
+            if (i < cells) {
+                const bool ok = a_id < mc && s < n;
+                const float bm = ok ? to_b2(vm[k]) : NEG_INF_F, bl = (ok && a_id >= 1) ? to_b2(vl[k]) : NEG_INF_F;
+                ok_all &= lin_input_ok(bm) & lin_input_ok(bl);
+                em[i] = pow2_of(bm);
+                el[i] = pow2_of(bl);
+            }
+        }
+    }
+    return ok_all != 0;
+}
+
+// Keeps loaded values (and their loads) in front of the arithmetic that follows, so that all LDS reads of a step are
+// issued back to back instead of two at a time between the multiply-adds.
+__device__ __forceinline__ void pin(double2 &v) { asm volatile("" : "+v"(v.x), "+v"(v.y)); }
+__device__ __forceinline__ void pin(double &v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void pin(int &v) { asm volatile("" : "+v"(v)); }
+
+struct FwdLinArgs {
+    const float *mt, *lk;
+    float *sm_S, *sm_F0, *sm_F1, *sm_D;
+    double *sm_O;
+    int m, n, mc, Mc, L, T;
+};
+
+// Forward sweep, linear domain, of the wave that owns the nodes 16W .. 16W+15: lane = 4 * node + j, and lane j of a quad
+// takes the children 16q + 4j .. 16q + 4j + 3 of every block of 16, q >= W (the blocks below hold only children left of
+// every node of the wave).  col0: inside probabilities of the column read / written; col1, col2: the row sums of the
+// step, for the table waves.  Returns false if a link is out of range.
+template <int W>
+__device__ __forceinline__ bool fwd_sweep_lin(const LinLds &x, const FwdLinArgs &g) {
+    constexpr int MP = 64;
+    const int n = g.n, mc = g.mc, Mc = g.Mc, L = g.L, T = g.T;
+    const int lane = threadIdx.x & 63, j = lane & 3, a_id = 16 * W + (lane >> 2);
+    const bool live = a_id < mc;
+    const int ai = live ? a_id : 0;
+    int ok = 1;
+    double EA0[4][4], EA1[4][4];
+    {
+        float A0[4][4], A1[4][4];
+        const size_t row = (size_t)(2 * min(a_id, Mc - 1) + 1) * 2;
+#pragma unroll
+        for (int q = W; q < 4; q++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int c = 2 * min(16 * q + 4 * j + i, Mc - 1) + 1;
+                A0[q][i] = g.lk[(row + 0) * L + c];
+                A1[q][i] = g.lk[(row + 1) * L + c];
+            }
+        }
+#pragma unroll
+        for (int q = W; q < 4; q++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int c_id = 16 * q + 4 * j + i;
+                const bool in = live && c_id < mc && c_id >= a_id;
+                const float b0 = in ? to_b2(A0[q][i]) : NEG_INF_F, b1 = (in && a_id >= 1) ? to_b2(A1[q][i]) : NEG_INF_F;
+                ok &= lin_input_ok(b0) & lin_input_ok(b1);
+                EA0[q][i] = pow2_of(b0);
+                EA1[q][i] = pow2_of(b1);
+            }
+        }
+    }
+    {  // the table cells the sweep never writes (the table waves are busy with the emissions)
+        const int TS = T + 2;
+        const float base_b2 = sanitize(g.mt[(size_t)(g.m - 1) * T + (n - 1)]) * LOG2E_F;  // pcfg_loss.cu:142-147
+        for (int i = threadIdx.x; i < Mc * TS; i += 256) {
+            g.sm_S[i] = (i == (mc - 1) * TS + (n - 1)) ? base_b2 : NEG_INF_F;
+            g.sm_F0[i] = NEG_INF_F;
+            g.sm_F1[i] = NEG_INF_F;
+        }
+    }
+    __syncthreads();  // the table waves have staged the emissions, the first column and the first shift
+    double F1prev = 0.0;
+    double em_p = x.em[ai * T + n - 2], el_p = x.el[ai * T + n - 2], em_t = x.em[ai * T + n - 1];
+    for (int t = n - 1; t >= 1; t--) {
+        const double2 *cur = reinterpret_cast<const double2 *>(x.col0 + (t & 1) * MP);
+        double2 xv[4][2];
+#pragma unroll
+        for (int q = W; q < 4; q++) {
+            xv[q][0] = cur[8 * q + 2 * j];
+            xv[q][1] = cur[8 * q + 2 * j + 1];
+        }
+        int k = x.kbuf[t];
+#pragma unroll
+        for (int q = W; q < 4; q++) {
+            pin(xv[q][0]);
+            pin(xv[q][1]);
+        }
+        pin(k);
+        const double down = pow2_int(-k);
+        double emd = em_p * down, rest = ((F1prev * down) * el_p) * em_t;
+        pin(emd);
+        pin(rest);
+        double a0 = 0.0, b0 = 0.0, a1 = 0.0, b1 = 0.0;
+#pragma unroll
+        for (int q = W; q < 4; q++) {
+            a0 = __builtin_fma(EA0[q][0], xv[q][0].x, a0);
+            b0 = __builtin_fma(EA0[q][1], xv[q][0].y, b0);
+            a1 = __builtin_fma(EA1[q][0], xv[q][0].x, a1);
+            b1 = __builtin_fma(EA1[q][1], xv[q][0].y, b1);
+            a0 = __builtin_fma(EA0[q][2], xv[q][1].x, a0);
+            b0 = __builtin_fma(EA0[q][3], xv[q][1].y, b0);
+            a1 = __builtin_fma(EA1[q][2], xv[q][1].x, a1);
+            b1 = __builtin_fma(EA1[q][3], xv[q][1].y, b1);
+        }
+        const double s0 = quad_sum_d(a0 + b0), s1 = quad_sum_d(a1 + b1);
+        double x_new = __builtin_fma(emd, s0, rest);
+        if (!live) x_new = 0.0;
+        const double F0 = s0 * down, F1 = s1 * down;
+        F1prev = F1;
+        if (j == 0) {
+            x.col0[((t - 1) & 1) * MP + a_id] = x_new;
+            x.col1[(t & 1) * MP + a_id] = F0;
+            x.col2[(t & 1) * MP + a_id] = F1;
+        }
+        if (t >= 2) {  // the emissions of the next step: they do not wait for the barrier
+            em_t = em_p;
+            em_p = x.em[ai * T + t - 2];
+            el_p = x.el[ai * T + t - 2];
+        }
+        lds_barrier();
+    }
+    return ok != 0;
+}
+
+// The table waves of the forward sweep (role 0: column entries, shifts and offsets; 1, 2: the two row sums; 3: idle).
+// They stage the emissions and the first column, then follow one step behind the sweep: iteration t turns column t and
+// the row sums of step t+1 into table entries; pass t = 0 after the last barrier finishes the job.  Returns the smallest
+// range key seen; ok: false if an emission is out of range.
+__device__ __forceinline__ unsigned fwd_tables_lin(const LinLds &x, const FwdLinArgs &g, int role, bool &ok) {
+    constexpr int MP = 64;
+    const int n = g.n, mc = g.mc, Mc = g.Mc, T = g.T, TS = g.T + 2, ht = threadIdx.x - 256, node = threadIdx.x & 63;
+    const bool live = node < mc;
+    const float base_b2 = sanitize(g.mt[(size_t)(g.m - 1) * T + (n - 1)]) * LOG2E_F;  // pcfg_loss.cu:142-147
+    ok = lin_fill_emissions(x.em, x.el, g.mt, mc, n, Mc, T) && lin_input_ok(base_b2) != 0;
+    const double x_base = pow2_of(base_b2);
+    const int e_base = exponent_or_none(x_base);
+    const int k_base = e_base == NO_EXPONENT ? 0 : clamp_shift(e_base);  // the first step's shift: from the base cell
+    for (int i = ht; i < 2 * MP; i += 256) {
+        x.col0[i] = (i == ((n - 1) & 1) * MP + mc - 1) ? x_base : 0.0;
+        x.col1[i] = 0.0;
+        x.col2[i] = 0.0;
+    }
+    for (int i = ht; i < TS + 2; i += 256) {
+        g.sm_D[i] = (i == n - 1) ? (float)k_base : 0.f;
+        if (i < TS) g.sm_O[i] = (i == n - 2) ? (double)k_base : 0.0;
+        x.kbuf[i] = (i == n - 1) ? k_base : 0;
+    }
+    if (ht == 0) *x.flag = 0;
+    __syncthreads();
+    unsigned lowest = ~0u;
+    int k_last = k_base;       // k_t at iteration t
+    double O_run = k_base;     // O[t-1] at iteration t
+    for (int t = n - 1; t >= 0; t--) {
+        if (role == 0) {
+            const double v = x.col0[(t & 1) * MP + node];
+            if (t >= 2) {
+                // O[t-2] becomes the absolute exponent of the largest entry of column t: the shift of step t-1 is what is
+                // left of that exponent (relative to O[t]) after the shift of step t
+                const int e = wave_max_i(exponent_or_none(v));
+                const int k = e == NO_EXPONENT ? 0 : clamp_shift(e - k_last);
+                if (node == 0) {
+                    x.kbuf[t - 1] = k;
+                    g.sm_D[t - 1] = (float)k;
+                    O_run += (double)k;
+                    g.sm_O[t - 2] = O_run;
+                }
+                k_last = k;
+            }
+            if (t < n - 1 && live) g.sm_S[node * TS + t] = log2_of(v);
+            lowest = min(lowest, range_key(v));
+        } else if (role <= 2 && t < n - 1) {
+            const double v = (role == 1 ? x.col1 : x.col2)[((t + 1) & 1) * MP + node];
+            if (live) (role == 1 ? g.sm_F0 : g.sm_F1)[node * TS + t + 1] = log2_of(v);
+            lowest = min(lowest, range_key(v));
+        }
+        if (t >= 1) lds_barrier();
+    }
+    return lowest;
+}
+
+// The forward sweep of a sentence in the linear domain (R = 1, tables in LDS): fills sm_S, sm_F0, sm_F1, hd.D, hd.O like
+// the log-domain code of inside_fwd_ml1_body and returns true, or returns false (workgroup-uniform) with the tables in an
+// undefined state.  `lin` is the extra LDS (lin_extra_bytes(Mc, T)).
+__device__ __forceinline__ bool inside_fwd_lin_attempt(const float *__restrict__ mt, const float *__restrict__ lk, const LdsHead &hd,
+                                                      float *sm_S, float *sm_F0, float *sm_F1, double *lin, int m, int n, int L,
+                                                      int T, int Mc, int lin_bits) {
+    const LinLds x(lin, Mc, T);
+    const FwdLinArgs g{mt, lk, sm_S, sm_F0, sm_F1, hd.D, hd.O, m, n, m / 2, Mc, L, T};
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    unsigned lowest = ~0u;
+    bool ok;
+    switch (wave) {  // wave-uniform; every branch meets the same barriers
+        case 0: ok = fwd_sweep_lin<0>(x, g); break;
+        case 1: ok = fwd_sweep_lin<1>(x, g); break;
+        case 2: ok = fwd_sweep_lin<2>(x, g); break;
+        case 3: ok = fwd_sweep_lin<3>(x, g); break;
+        default: lowest = fwd_tables_lin(x, g, 7 - wave, ok); break;  // role 0 beside the sweep wave with the fewest children
+    }
+    if (!ok || lowest < range_key_of_bits(lin_bits)) *x.flag = 1;
+    __syncthreads();
+    const bool good = *x.flag == 0;
+    if (threadIdx.x == 0) atomicAdd(good ? &g_linear_swept : &g_linear_handed_over, 1ull);
+    __syncthreads();  // the flag's cell may be written again by the log-domain sweep's staging
+    return good;
+}
+
 // Forward.  Dynamic LDS: head (see LdsHead), col[2][64R]; with TAB_LDS also the emissions of main nodes and of their
 // leaves [Mc][T] and the R, F0h, F1h tables [Mc][T+2] (all base 2), which are copied out in bulk when the sweep is over -
 // the sweep itself then touches no global memory.
 template <int R, bool TAB_LDS>
 __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__restrict__ match_all, const float *__restrict__ links,
                                                    const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
-                                                   float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc) {
+                                                   float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc,
+                                                   int lin_bits = 0) {
     constexpr int NQ = 8 * R;
     constexpr int MP = 64 * R;
     const int TS = T + 2;
@@ -314,6 +644,12 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
     }
     const int mc = m / 2;  // active main-chain nodes: a_id < mc
 
+    // the linear-domain sweep first, where the launch brought the LDS for it; what it cannot follow is swept below
+    bool swept = false;
+    if (R == 1 && TAB_LDS && lin_bits > 0)
+        swept = inside_fwd_lin_attempt(mt, lk, hd, sm_S, sm_F0, sm_F1, reinterpret_cast<double *>(smem + fwd_role_floats(Mc, T)), m, n,
+                                       L, T, Mc, lin_bits);
+    if (!swept) {
     // link slabs -> registers; the loads are unconditional (clamped addresses) so that they are all in flight together
     float A0[R][NQ], A1[R][NQ];
 #pragma unroll
@@ -381,6 +717,7 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
         case 6: fwd_sweep<R, TAB_LDS, 6>(A0, A1, sa); break;
         default: fwd_sweep<R, TAB_LDS, 7>(A0, A1, sa); break;
     }
+    }
     if (TAB_LDS) {
         for (int i = tid; i < Mc * TS; i += NTR) {
             const int t = i - (i / TS) * TS;
@@ -400,8 +737,9 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
 template <int R, bool TAB_LDS>
 __global__ __launch_bounds__(NTR) void inside_fwd_ml1_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
                                                             const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
-                                                            float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc) {
-    inside_fwd_ml1_body<R, TAB_LDS>(blockIdx.x, match_all, links, out_len, tgt_len, S, aux, L, T, Mc);
+                                                            float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc,
+                                                            int lin_bits) {
+    inside_fwd_ml1_body<R, TAB_LDS>(blockIdx.x, match_all, links, out_len, tgt_len, S, aux, L, T, Mc, lin_bits);
 }
 
 struct BwdSweepArgs {
@@ -967,6 +1305,198 @@ __device__ __forceinline__ void outside_sweep_free(const float (&A0)[1][8], cons
     }
 }
 
+struct OutsideLinArgs {
+    const float *mt, *lk;
+    float *sm_B, *sm_W0, *sm_W1, *sm_E;
+    double *sm_P;
+    int n, mc, Mc, L, T;
+};
+
+// Outside sweep, linear domain, of the wave that owns the children 16W .. 16W+15: lane = 4 * node + j, and lane j of a
+// quad takes the parents 16q + 4j .. 16q + 4j + 3 of every block of 16, q <= W (the blocks beyond hold only parents
+// right of every node of the wave).  col0, col1: the weights W0_t, W1_t the parents offer (read at step t, written
+// for t+1); col2: the betas, for the table waves.  Returns false if a link is out of range.
+template <int W>
+__device__ __forceinline__ bool outside_sweep_lin(const LinLds &x, const OutsideLinArgs &g) {
+    constexpr int NB = W + 1, MP = 64;
+    const int n = g.n, mc = g.mc, Mc = g.Mc, L = g.L, T = g.T;
+    const int lane = threadIdx.x & 63, j = lane & 3, c_id = 16 * W + (lane >> 2);
+    const bool live = c_id < mc;
+    const int ci = live ? c_id : 0;
+    int ok = 1;
+    double EA0[NB][4], EA1[NB][4];
+    {
+        float A0[NB][4], A1[NB][4];
+        const int c = 2 * min(c_id, Mc - 1) + 1;
+#pragma unroll
+        for (int q = 0; q < NB; q++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const size_t row = (size_t)(2 * min(16 * q + 4 * j + i, Mc - 1) + 1) * 2;
+                A0[q][i] = g.lk[(row + 0) * L + c];
+                A1[q][i] = g.lk[(row + 1) * L + c];
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < NB; q++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int a_id = 16 * q + 4 * j + i;
+                const bool in = live && a_id < mc && a_id <= c_id;
+                const float b0 = in ? to_b2(A0[q][i]) : NEG_INF_F, b1 = (in && a_id >= 1) ? to_b2(A1[q][i]) : NEG_INF_F;
+                ok &= lin_input_ok(b0) & lin_input_ok(b1);
+                EA0[q][i] = pow2_of(b0);
+                EA1[q][i] = pow2_of(b1);
+            }
+        }
+    }
+    {  // the table cells the sweep never writes (the table waves are busy with the emissions)
+        const int TS = T + 2;
+        for (int i = threadIdx.x; i < Mc * TS; i += 256) {
+            g.sm_B[i] = NEG_INF_F;
+            g.sm_W0[i] = NEG_INF_F;
+            g.sm_W1[i] = NEG_INF_F;
+        }
+    }
+    __syncthreads();  // the table waves have staged the emissions and the first columns
+    double bprev = (c_id == 0) ? 1.0 : 0.0;  // beta[root][0] = 0
+    int e_cur = 0;
+    double em_t = live ? x.em[ci * T + 1] : 0.0, el_p = live ? x.el[ci * T + 0] : 0.0;
+    for (int t = 1; t <= n - 1; t++) {
+        const double2 *c0 = reinterpret_cast<const double2 *>(x.col0 + (t & 1) * MP);
+        const double2 *c1 = reinterpret_cast<const double2 *>(x.col1 + (t & 1) * MP);
+        double2 u0[NB][2], u1[NB][2];
+#pragma unroll
+        for (int q = 0; q < NB; q++) {
+            u0[q][0] = c0[8 * q + 2 * j];
+            u0[q][1] = c0[8 * q + 2 * j + 1];
+            u1[q][0] = c1[8 * q + 2 * j];
+            u1[q][1] = c1[8 * q + 2 * j + 1];
+        }
+        int e_next = x.kbuf[t];
+#pragma unroll
+        for (int q = 0; q < NB; q++) {
+            pin(u0[q][0]);
+            pin(u0[q][1]);
+            pin(u1[q][0]);
+            pin(u1[q][1]);
+        }
+        pin(e_next);
+        // what of the weights offered at the next two positions does not wait for this step's sum
+        double emd = pow2_int(-e_next) * em_t;
+        double nw1 = ((bprev * pow2_int(-(e_next + e_cur))) * el_p) * em_t;
+        pin(emd);
+        pin(nw1);
+        double a0 = 0.0, b0 = 0.0, a1 = 0.0, b1 = 0.0;
+#pragma unroll
+        for (int q = 0; q < NB; q++) {
+            a0 = __builtin_fma(EA0[q][0], u0[q][0].x, a0);
+            b0 = __builtin_fma(EA0[q][1], u0[q][0].y, b0);
+            a1 = __builtin_fma(EA1[q][0], u1[q][0].x, a1);
+            b1 = __builtin_fma(EA1[q][1], u1[q][0].y, b1);
+            a0 = __builtin_fma(EA0[q][2], u0[q][1].x, a0);
+            b0 = __builtin_fma(EA0[q][3], u0[q][1].y, b0);
+            a1 = __builtin_fma(EA1[q][2], u1[q][1].x, a1);
+            b1 = __builtin_fma(EA1[q][3], u1[q][1].y, b1);
+        }
+        const double beta = quad_sum_d((a0 + b0) + (a1 + b1));  // (zero for children beyond the sentence: their link columns are)
+        const double nw0 = beta * emd;
+        bprev = beta;
+        if (j == 0) {
+            x.col0[((t + 1) & 1) * MP + c_id] = nw0;
+            x.col1[((t + 1) & 1) * MP + c_id] = nw1;
+            x.col2[(t & 1) * MP + c_id] = beta;
+        }
+        e_cur = e_next;
+        if (t + 1 <= n - 1) {  // the emissions of the next step: they do not wait for the barrier
+            em_t = live ? x.em[ci * T + t + 1] : 0.0;
+            el_p = live ? x.el[ci * T + t] : 0.0;
+        }
+        lds_barrier();
+    }
+    return ok != 0;
+}
+
+// The table waves of the outside sweep (role 0: betas, shifts and offsets; 1, 2: the two weights; 3: idle).  They stage the
+// emissions and the first columns, then follow one step behind the sweep: iteration t turns the betas of step t-1 and the
+// weight columns W0_t, W1_t into table entries; pass t = n after the last barrier finishes the job.  Returns the smallest
+// range key seen; ok: false if an emission is out of range.
+__device__ __forceinline__ unsigned outside_tables_lin(const LinLds &x, const OutsideLinArgs &g, int role, bool &ok) {
+    constexpr int MP = 64;
+    const int n = g.n, mc = g.mc, Mc = g.Mc, T = g.T, TS = g.T + 2, TP = g.T + 4, ht = threadIdx.x - 256, node = threadIdx.x & 63;
+    const bool live = node < mc;
+    const float w00_b2 = to_b2(g.mt[(size_t)1 * T + 0]);  // W0_1: the root offers match[root][0] to its null-left children
+    ok = lin_fill_emissions(x.em, x.el, g.mt, mc, n, Mc, T);
+    for (int i = ht; i < 2 * MP; i += 256) {
+        x.col0[i] = (i == 1 * MP + 0) ? pow2_of(w00_b2) : 0.0;
+        x.col1[i] = 0.0;
+        x.col2[i] = (i == 0) ? 1.0 : 0.0;  // beta column 0
+    }
+    for (int i = ht; i < TP; i += 256) {
+        g.sm_E[i] = 0.f;
+        g.sm_P[i] = 0.0;
+        x.kbuf[i] = 0;
+    }
+    if (ht == 0) *x.flag = 0;
+    __syncthreads();
+    unsigned lowest = ~0u;
+    int k_last = 0, k_before = 0;  // E_{t+1}, E_t at iteration t
+    double P_run = 0.0;            // P[t+1] at iteration t
+    for (int t = 1; t <= n; t++) {
+        if (role == 0) {
+            const double v = x.col2[((t - 1) & 1) * MP + node];
+            if (t + 1 <= n - 1) {
+                // P[t+2] becomes the absolute exponent of the largest beta of column t-1: the shift of step t+1 is what is
+                // left of that exponent (relative to P[t-1]) after the shifts of the steps t-1 and t
+                const int e = wave_max_i(exponent_or_none(v));
+                const int k = e == NO_EXPONENT ? 0 : clamp_shift(e - k_last - k_before);
+                if (node == 0) {
+                    x.kbuf[t + 1] = k;
+                    g.sm_E[t + 2] = (float)k;
+                    P_run += (double)k;
+                    g.sm_P[t + 2] = P_run;
+                }
+                k_before = k_last;
+                k_last = k;
+            }
+            if (live) g.sm_B[node * TS + t - 1] = log2_of(v);
+            lowest = min(lowest, range_key(v));
+        } else if (role <= 2) {
+            const double v = (role == 1 ? x.col0 : x.col1)[(t & 1) * MP + node];
+            if (live) (role == 1 ? g.sm_W0 : g.sm_W1)[node * TS + t] = log2_of(v);
+            lowest = min(lowest, range_key(v));
+        }
+        if (t <= n - 1) lds_barrier();
+    }
+    return lowest;
+}
+
+// The outside sweep of a sentence in the linear domain: fills sm_B, sm_W0, sm_W1, sm_E, sm_P like the log-domain code of
+// inside_outside_ml1_body and returns true, or returns false (workgroup-uniform) with them in an undefined state.
+// `lin` is the extra LDS (lin_extra_bytes(Mc, T)).
+__device__ __forceinline__ bool inside_outside_lin_attempt(const float *__restrict__ mt, const float *__restrict__ lk, double *sm_P,
+                                                          float *sm_E, float *sm_B, float *sm_W0, float *sm_W1, double *lin, int m,
+                                                          int n, int L, int T, int Mc, int lin_bits) {
+    const LinLds x(lin, Mc, T);
+    const OutsideLinArgs g{mt, lk, sm_B, sm_W0, sm_W1, sm_E, sm_P, n, m / 2, Mc, L, T};
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    unsigned lowest = ~0u;
+    bool ok;
+    switch (wave) {  // wave-uniform; every branch meets the same barriers
+        case 0: ok = outside_sweep_lin<0>(x, g); break;
+        case 1: ok = outside_sweep_lin<1>(x, g); break;
+        case 2: ok = outside_sweep_lin<2>(x, g); break;
+        case 3: ok = outside_sweep_lin<3>(x, g); break;
+        default: lowest = outside_tables_lin(x, g, wave - 4, ok); break;
+    }
+    if (!ok || lowest < range_key_of_bits(lin_bits)) *x.flag = 1;
+    __syncthreads();
+    const bool good = *x.flag == 0;
+    if (threadIdx.x == 0) atomicAdd(good ? &g_linear_swept : &g_linear_handed_over, 1ull);
+    __syncthreads();
+    return good;
+}
+
 // Dynamic LDS of the outside role: P [T+4] (double), slots [16], E [T+4], w0 [2][64], w1 [2][64], Bh, W0h, W1h [Mc][T+2],
 // emissions of main nodes and leaves [Mc][T].
 __host__ __device__ inline size_t outside_role_bytes(int Mc, int T) {
@@ -976,7 +1506,7 @@ __host__ __device__ inline size_t outside_role_bytes(int Mc, int T) {
 __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float *__restrict__ match_all,
                                                        const float *__restrict__ links, const int64_t *__restrict__ out_len,
                                                        const int64_t *__restrict__ tgt_len, float *__restrict__ aux, int L, int T,
-                                                       int Mc) {
+                                                       int Mc, int lin_bits) {
     constexpr int NQ = 8, MP = 64;
     const int TS = T + 2, TP = T + 4;
     extern __shared__ double smem_d[];
@@ -1000,6 +1530,13 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
     const float *lk = links + (size_t)b * L * 2 * L;
     AuxView av(aux, b, Mc, T);
 
+    // the linear-domain sweep first, where the launch brought the LDS for it; what it cannot follow is swept below
+    bool swept = false;
+    if (lin_bits > 0)
+        swept = inside_outside_lin_attempt(mt, lk, sm_P, sm_E, sm_B, sm_W0, sm_W1,
+                                           reinterpret_cast<double *>(reinterpret_cast<char *>(smem_d) + align16(outside_role_bytes(Mc, T))),
+                                           m, n, L, T, Mc, lin_bits);
+    if (!swept) {
     // transposed link slabs: this thread's group owns child c, its lanes the parents a <= c; unconditional loads
     const int own = 8 * p + g8;
     float A0[1][NQ], A1[1][NQ];
@@ -1060,6 +1597,7 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
             default: outside_sweep_free<7>(A0, A1, sa); break;
         }
     }
+    }
     __syncthreads();
     for (int i = tid; i < Mc * TS; i += NTR) {
         av.BETA[i] = sm_B[i];
@@ -1112,14 +1650,14 @@ __device__ __forceinline__ void pad_fill_block(const PadFill pad, const int64_t 
 __global__ __launch_bounds__(NTR) void inside_pair_ml1_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
                                                              const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
                                                              float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc,
-                                                             int nsent, PadFill pad) {
+                                                             int nsent, PadFill pad, int lin_bits) {
     if ((int)blockIdx.x >= 2 * nsent) {  // workgroup-uniform
         pad_fill_block(pad, out_len, (int)blockIdx.x - 2 * nsent, L);
         return;
     }
     const int b = blockIdx.x >> 1;
-    if ((blockIdx.x & 1) == 0) inside_fwd_ml1_body<1, true>(b, match_all, links, out_len, tgt_len, S, aux, L, T, Mc);
-    else inside_outside_ml1_body(b, match_all, links, out_len, tgt_len, aux, L, T, Mc);
+    if ((blockIdx.x & 1) == 0) inside_fwd_ml1_body<1, true>(b, match_all, links, out_len, tgt_len, S, aux, L, T, Mc, lin_bits);
+    else inside_outside_ml1_body(b, match_all, links, out_len, tgt_len, aux, L, T, Mc, lin_bits);
 }
 
 // Posteriors from the tables of the two sweeps: grid (16, B), 256 threads.  Workgroup (q, b) owns the parents 4q .. 4q+3 of
@@ -3146,6 +3684,10 @@ std::atomic<int> g_pipeline_spin_limit_outside{-1};  // side-by-side launch only
 // Largest base-2 exponent a factor of the rule posteriors of long graphs may have on the matrix cores (see
 // links_grad_ml1_stream_kernel); a tile beyond it is recomputed term by term.  pcfgnat_links_grad_range_limit.
 std::atomic<float> g_links_grad_range_limit{120.f};
+// Smallest nonzero number, as a power of two, that the linear-domain sweeps of graphs of up to 130 nodes accept before
+// they hand the sentence to the log-domain sweep (see LIN_INPUT_BITS); 0 switches them off.  pcfgnat_inside_linear_bits.
+std::atomic<int> g_inside_linear_bits{LIN_BITS_MAX};
+inline int inside_linear_bits() { return g_inside_linear_bits.load(); }
 int pipeline_chunks(int B, int T, int Mc) {  // NQ, or 0 where the pipelined sweeps do not apply
     const int NQ = stream_mp(Mc) / 64, CL = 64 * NQ / NLP;
     return (NQ >= 2 && NQ <= 8 && T + 2 < 4096 && (int64_t)B * CL <= g_pipeline_max_wg.load()) ? NQ : 0;
@@ -3348,13 +3890,17 @@ int launch_fwd(const float *match_all, const float *links, const int64_t *ol, co
     const size_t with_tab = base + ((size_t)2 * Mc * T + (size_t)3 * Mc * (T + 2)) * sizeof(float);
     if (with_tab <= LDS_BUDGET) {
         auto k = inside_fwd_ml1_kernel<R, true>;
-        PCFGNAT_DYNAMIC_LDS(k, with_tab);
-        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), with_tab, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
+        // with room for its columns and emission probabilities behind the tables, the sweep runs in the linear domain
+        const size_t with_lin = fwd_role_floats(Mc, T) * sizeof(float) + lin_extra_bytes(Mc, T);
+        const int lin_bits = (R == 1 && with_lin <= LDS_BUDGET) ? inside_linear_bits() : 0;
+        const size_t lds = lin_bits > 0 ? with_lin : with_tab;
+        PCFGNAT_DYNAMIC_LDS(k, lds);
+        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), lds, stream, match_all, links, ol, tl, S, aux, L, T, Mc, lin_bits);
     } else {
         auto k = inside_fwd_ml1_kernel<R, false>;
         PCFGNAT_REQUIRE(base <= LDS_BUDGET, "pcfg_loss: target length %d too large for the column offsets in LDS", T);
         PCFGNAT_DYNAMIC_LDS(k, base);
-        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), base, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
+        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), base, stream, match_all, links, ol, tl, S, aux, L, T, Mc, 0);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
@@ -3388,7 +3934,13 @@ int launch_fused(const float *go, const float *match_all, const float *links, co
     *done = false;
     if (R == 1) {  // the two sweeps side by side as two workgroups per sentence, then the posteriors
         const size_t fwd_bytes = ((size_t)head_floats(T) + 2 * 64 + (size_t)2 * Mc * T + (size_t)3 * Mc * (T + 2)) * sizeof(float);
-        const size_t pair_bytes = fwd_bytes > outside_role_bytes(Mc, T) ? fwd_bytes : outside_role_bytes(Mc, T);
+        size_t pair_bytes = fwd_bytes > outside_role_bytes(Mc, T) ? fwd_bytes : outside_role_bytes(Mc, T);
+        // with room for their columns and emission probabilities behind the tables, the sweeps run in the linear domain
+        const size_t fwd_lin = fwd_role_floats(Mc, T) * sizeof(float) + lin_extra_bytes(Mc, T);
+        const size_t out_lin = align16(outside_role_bytes(Mc, T)) + lin_extra_bytes(Mc, T);
+        const size_t pair_lin = fwd_lin > out_lin ? fwd_lin : out_lin;
+        const int lin_bits = pair_lin <= LDS_BUDGET ? inside_linear_bits() : 0;
+        if (lin_bits > 0) pair_bytes = pair_lin;
         const size_t comb_bytes = ((size_t)(T + 4) + (size_t)Mc * (T + 2) + (size_t)8 * (T + 2)) * sizeof(float);
         if (pair_bytes <= LDS_BUDGET && comb_bytes <= 64 * 1024 && L <= 128) {
             PCFGNAT_REQUIRE(((uintptr_t)aux & 7) == 0, "pcfg_loss_forward_backward: aux must be 8-byte aligned");
@@ -3402,7 +3954,7 @@ int launch_fused(const float *go, const float *match_all, const float *links, co
             if (launch_bytes != pair_bytes)
                 PCFGNAT_DYNAMIC_LDS(inside_pair_ml1_kernel, launch_bytes);
             hipLaunchKernelGGL(inside_pair_ml1_kernel, dim3((2 + (fill ? PAD_WGS : 0)) * B), dim3(NTR), launch_bytes, stream, match_all,
-                               links, ol, tl, S, aux, L, T, Mc, B, pad);
+                               links, ol, tl, S, aux, L, T, Mc, B, pad, lin_bits);
             PCFGNAT_HIP_CHECK(hipGetLastError());
             if (fill && pad_done) *pad_done = true;
             hipLaunchKernelGGL(inside_combine_ml1_kernel, dim3(16, B), dim3(256), comb_bytes, stream, go, S, aux, match_all, links, ol, tl,
@@ -3447,6 +3999,7 @@ extern "C" void pcfgnat_pipeline_config(int max_workgroups, int spin_limit) {
 extern "C" void pcfgnat_pipeline_outside_spin_limit(int spin_limit) { g_pipeline_spin_limit_outside.store(spin_limit); }
 
 extern "C" void pcfgnat_links_grad_range_limit(float log2_limit) { g_links_grad_range_limit.store(log2_limit); }
+extern "C" void pcfgnat_inside_linear_bits(int bits) { g_inside_linear_bits.store(bits < 0 ? 0 : (bits > LIN_BITS_MAX ? LIN_BITS_MAX : bits)); }
 
 extern "C" int pcfgnat_pipeline_redo_counts(unsigned long long *inside_sweeps, unsigned long long *viterbi_sentences, int reset) {
     PCFGNAT_REQUIRE(inside_sweeps && viterbi_sentences, "pipeline_redo_counts: null pointer");
@@ -3456,6 +4009,18 @@ extern "C" int pcfgnat_pipeline_redo_counts(unsigned long long *inside_sweeps, u
         PCFGNAT_HIP_CHECK(hipMemcpyToSymbol(HIP_SYMBOL(g_inside_redone), &zero, sizeof(zero)));
     }
     return viterbi_redo_count(viterbi_sentences, reset);
+}
+
+extern "C" int pcfgnat_inside_linear_counts(unsigned long long *swept, unsigned long long *handed_over, int reset) {
+    PCFGNAT_REQUIRE(swept && handed_over, "inside_linear_counts: null pointer");
+    PCFGNAT_HIP_CHECK(hipMemcpyFromSymbol(swept, HIP_SYMBOL(g_linear_swept), sizeof(*swept)));
+    PCFGNAT_HIP_CHECK(hipMemcpyFromSymbol(handed_over, HIP_SYMBOL(g_linear_handed_over), sizeof(*handed_over)));
+    if (reset) {
+        const unsigned long long zero = 0;
+        PCFGNAT_HIP_CHECK(hipMemcpyToSymbol(HIP_SYMBOL(g_linear_swept), &zero, sizeof(zero)));
+        PCFGNAT_HIP_CHECK(hipMemcpyToSymbol(HIP_SYMBOL(g_linear_handed_over), &zero, sizeof(zero)));
+    }
+    return PCFGNAT_OK;
 }
 
 extern "C" size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml) {

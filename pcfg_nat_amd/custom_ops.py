@@ -61,6 +61,22 @@ def pipeline_redo_counts(reset=False):
     return a.value, b.value
 
 
+def inside_linear_bits(bits=500):
+    """Test hook (process-wide): the smallest nonzero number, as a power of two, that the linear-domain sweeps of graphs of
+    up to 130 nodes accept before they hand a sentence to the log-domain sweep; 0 switches them off."""
+    _lib.load().pcfgnat_inside_linear_bits(int(bits))
+
+
+def inside_linear_counts(reset=False):
+    """(sweeps completed in the linear domain, sweeps handed over to the log domain) on the current device since the
+    library was loaded or the last reset; forward and outside sweeps count apart.  Synchronises with the device."""
+    import ctypes
+    lib = _lib.load()
+    a, b = ctypes.c_ulonglong(0), ctypes.c_ulonglong(0)
+    _lib.check(lib.pcfgnat_inside_linear_counts(ctypes.byref(a), ctypes.byref(b), int(bool(reset))), lib)
+    return a.value, b.value
+
+
 def _stream(t):
     return torch.cuda.current_stream(t.device).cuda_stream
 

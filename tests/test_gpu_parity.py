@@ -383,6 +383,67 @@ def test_rule_posteriors_term_by_term_path(case):
         ops.links_grad_range_limit()
 
 
+@pytest.mark.parametrize("L,T,ms,ns", [(128, 32, [128, 96, 40, 4], [32, 25, 11, 2]), (64, 48, [64, 30], [48, 9]),
+                                       (130, 20, [130, 66], [20, 12]), (36, 54, [36, 36], [54, 40])])
+def test_inside_linear_and_log_domain_sweeps_agree(L, T, ms, ns):
+    """Graphs of up to 130 nodes are swept in the linear domain (doubles, one multiply-add per term) where the numbers
+    allow it and in the log domain otherwise.  Here the same batches go through both - loss and gradients through the
+    two-workgroup pass, the table of the forward kernel alone - and must agree far inside the tolerance either is held
+    to against the oracle; the counters tell that each run took the sweep it was meant to take."""
+    batch = synth.training_batch(len(ms), L, T, 80, ms, ns, seed=3 * L + T)
+    match = _match_for(batch)
+    ol, tl = batch["output_length"].to(DEV), batch["target_length"].to(DEV)
+    runs = {}
+    try:
+        for name, bits in (("linear", 500), ("log", 0)):
+            ops.inside_linear_bits(bits)
+            ops.inside_linear_counts(reset=True)
+            ll, mg, lg = _inside_all(batch, match)
+            S = ops._pcfg_loss_tables(match.to(DEV), batch["links"].to(DEV), ol, tl, 1, "test")[0].cpu()
+            runs[name] = (ll, mg, lg, S, ops.inside_linear_counts())
+    finally:
+        ops.inside_linear_bits()
+    Mc = (L - 2) // 2 + 1
+    if Mc <= 64:
+        assert runs["linear"][4] == (3 * len(ms), 0)  # forward and outside sweep of the pass, forward sweep of the tables
+    else:
+        assert runs["linear"][4] == (0, 0)  # more than one tile of 64 nodes: no linear sweep for these
+    assert runs["log"][4] == (0, 0)
+    (ll_a, mg_a, lg_a, S_a, _), (ll_b, mg_b, lg_b, S_b, _) = runs["linear"], runs["log"]
+    assert torch.equal(torch.isfinite(S_a), torch.isfinite(S_b))
+    fin = torch.isfinite(S_b)
+    assert torch.allclose(S_a[fin], S_b[fin], rtol=2e-6, atol=2e-4)
+    assert torch.allclose(ll_a, ll_b, rtol=2e-6)
+    for got, want in ((mg_a, mg_b), (lg_a, lg_b)):
+        for bi in range(len(ms)):
+            assert (got[bi] - want[bi]).abs().max() <= 2e-5 * max(float(want[bi].abs().max()), 1e-30)
+
+
+def test_inside_linear_sweep_hands_over_what_it_cannot_follow():
+    """Of four sentences one has an emission 400 nats down, one a link 300 nats down, one a node whose inside value falls
+    2^-600 below its column's largest, one nothing special: the linear sweeps keep the last (both of its sweeps) and hand
+    the others to the log domain, and every sentence comes out right against the float64 oracle."""
+    L, T, ms, ns = 64, 20, [64, 64, 64, 64], [20, 20, 20, 20]
+    batch = synth.training_batch(4, L, T, 80, ms, ns, seed=77)
+    match = _match_for(batch).clone()
+    links = batch["links"].clone()
+    match[0, 9, 5] = -400.0
+    fin = torch.isfinite(links[1, 5, 0])
+    links[1, 5, 0, int(fin.nonzero()[0])] = -300.0
+    match[2, 41:, :] = match[2, 41:, :] - 90.0  # every emission of the right part of the graph: 5 tokens are 2^-650
+    batch = dict(batch, links=links)
+    S64, C64, mg64, lg64 = _oracle_inside(batch, match.numpy())
+    ops.inside_linear_counts(reset=True)
+    ll, mg, lg = _inside_all(batch, match)
+    swept, handed = ops.inside_linear_counts()
+    assert handed >= 3 and swept >= 2 and swept + handed == 8, (swept, handed)
+    w = torch.linspace(0.5, 1.5, 4).double().numpy()
+    assert np.allclose(ll.double().numpy(), S64[:, 0, 0], rtol=1e-5)
+    for bi in range(4):
+        for got, want in ((mg[bi].double().numpy(), mg64[bi] * w[bi]), (lg[bi].double().numpy(), lg64[bi] * w[bi])):
+            assert np.abs(got - want).max() <= 1e-4 * max(np.abs(want).max(), 1e-30), bi
+
+
 @pytest.mark.parametrize("L,T,ms,ns", [(128, 30, [128, 90], [30, 22]), (320, 40, [320, 262], [40, 31]), (600, 24, [600, 520], [24, 24])])
 def test_inside_spiky_inputs_vs_oracle(L, T, ms, ns):
     """Emissions and links with jumps of hundreds of units and scattered -inf entries: neighbouring columns of the tables
