@@ -1610,16 +1610,17 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
     }
 }
 
-// Workgroups per sentence that zero the rows of its pad nodes beside the sweeps (see PadFill).
-constexpr int PAD_WGS = 32;
+// Workgroups per sentence that zero the rows of its pad nodes (see PadFill): PAD_WGS_SWEEPS of them beside the sweeps, the
+// others beside the posteriors, in proportion to how long the two launches take without them.
+constexpr int PAD_WGS = 32, PAD_WGS_SWEEPS = 22;
 // The fill rides along while the sweeps take up no more than three quarters of the compute units (192 of 256 on MI355X).
 inline int pad_max_sweep_wgs() { return device_compute_units() * 3 / 4; }
 constexpr size_t PAD_EXCLUSIVE_LDS = 84 * 1024;  // more than half of the 160 KB of a gfx950 compute unit
 
 // Zeroes the bytes of rows [m_b, L) of sentence b - one contiguous span - as one of PAD_WGS workgroups: 16-byte
 // streaming stores over the aligned body, byte stores over what is left at either end.
-__device__ __forceinline__ void pad_fill_block(const PadFill pad, const int64_t *__restrict__ out_len, int z, int L) {
-    const int b = z / PAD_WGS, part = z % PAD_WGS, tid = threadIdx.x;
+__device__ __forceinline__ void pad_fill_block(const PadFill pad, const int64_t *__restrict__ out_len, int b, int part, int L) {
+    const int tid = threadIdx.x, NTF = blockDim.x;
     int64_t m = out_len[b];
     m = m < 0 ? 0 : (m > L ? L : m);
     unsigned char *begin = pad.base + ((int64_t)b * L + m) * pad.row_bytes;
@@ -1629,7 +1630,7 @@ __device__ __forceinline__ void pad_fill_block(const PadFill pad, const int64_t 
     unsigned char *body_end = reinterpret_cast<unsigned char *>(reinterpret_cast<uintptr_t>(end) & ~(uintptr_t)15);
     if (body >= body_end) {  // shorter than one aligned chunk
         if (part == 0)
-            for (unsigned char *q = begin + tid; q < end; q += NTR) *q = 0;
+            for (unsigned char *q = begin + tid; q < end; q += NTF) *q = 0;
         return;
     }
     if (part == 0) {
@@ -1642,17 +1643,18 @@ __device__ __forceinline__ void pad_fill_block(const PadFill pad, const int64_t 
     const int64_t lo = per * part, hi = (lo + per < nv) ? lo + per : nv;
     u32x4 zero;
     zero.x = zero.y = zero.z = zero.w = 0;
-    for (int64_t i = lo + tid; i < hi; i += NTR) __builtin_nontemporal_store(zero, v + i);
+    for (int64_t i = lo + tid; i < hi; i += NTF) __builtin_nontemporal_store(zero, v + i);
 }
 
-// 2*nsent workgroups: 2b runs the forward sweep of sentence b, 2b+1 its outside sweep; PAD_WGS*nsent more when there is
-// a pad-fill task, which land on the compute units the sweeps leave free.
+// 2*nsent workgroups: 2b runs the forward sweep of sentence b, 2b+1 its outside sweep; PAD_WGS_SWEEPS*nsent more when
+// there is a pad-fill task, which land on the compute units the sweeps leave free.
 __global__ __launch_bounds__(NTR) void inside_pair_ml1_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
                                                              const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
                                                              float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc,
                                                              int nsent, PadFill pad, int lin_bits) {
     if ((int)blockIdx.x >= 2 * nsent) {  // workgroup-uniform
-        pad_fill_block(pad, out_len, (int)blockIdx.x - 2 * nsent, L);
+        const int z = (int)blockIdx.x - 2 * nsent;
+        pad_fill_block(pad, out_len, z / PAD_WGS_SWEEPS, z % PAD_WGS_SWEEPS, L);
         return;
     }
     const int b = blockIdx.x >> 1;
@@ -1660,7 +1662,8 @@ __global__ __launch_bounds__(NTR) void inside_pair_ml1_kernel(const float *__res
     else inside_outside_ml1_body(b, match_all, links, out_len, tgt_len, aux, L, T, Mc, lin_bits);
 }
 
-// Posteriors from the tables of the two sweeps: grid (16, B), 256 threads.  Workgroup (q, b) owns the parents 4q .. 4q+3 of
+// Posteriors from the tables of the two sweeps: grid (16, B), 256 threads (PAD_WGS - PAD_WGS_SWEEPS more workgroups per
+// sentence when there is a pad-fill task).  Workgroup (q, b) owns the parents 4q .. 4q+3 of
 // sentence b: it writes the rows 8q .. 8q+7 of the links_grad slab (zeros included) and a sixteenth of the match_all_grad
 // cells.  One thread per (parent, child) pair sums both planes over the columns.
 // Dynamic LDS: corr [T+4], R [Mc][T+2], W0h, W1h of the workgroup's parents [4][T+2].
@@ -1668,7 +1671,12 @@ __global__ __launch_bounds__(256) void inside_combine_ml1_kernel(const float *__
                                                                 float *__restrict__ aux, const float *__restrict__ match_all,
                                                                 const float *__restrict__ links, const int64_t *__restrict__ out_len,
                                                                 const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad,
-                                                                float *__restrict__ lgrad, int L, int T, int Mc, Seed seed) {
+                                                                float *__restrict__ lgrad, int L, int T, int Mc, Seed seed,
+                                                                PadFill pad) {
+    if (blockIdx.x >= 16) {  // workgroup-uniform: the part of the pad fill that rides along with this launch
+        pad_fill_block(pad, out_len, blockIdx.y, PAD_WGS_SWEEPS + (int)blockIdx.x - 16, L);
+        return;
+    }
     const int TS = T + 2, TP = T + 4;
     extern __shared__ float smem[];
     float *corr = smem;               // [TP]
@@ -1685,7 +1693,51 @@ __global__ __launch_bounds__(256) void inside_combine_ml1_kernel(const float *__
     const int cells = L * T, cell0 = (int)((int64_t)cells * part / 16), cell1 = (int)((int64_t)cells * (part + 1) / 16);
     const int row0 = min(8 * part, L), row1 = min(8 * part + 8, L);
     for (int i = row0 * 2 * L + tid; i < row1 * 2 * L; i += 256) lg[i] = 0.f;
+
+    // Everything this thread will read is requested here, before anything is used: no address depends on a loaded value
+    // (indices are clamped, the lengths only decide later which values count), so the launch pays one trip to memory
+    // instead of one per stage - which matters most while the pad fill beside it keeps the memory system busy.
     const float ll = S[(size_t)b * Mc * TS];
+    // this thread's pair: parent 4*part + tid/64, child tid%64
+    const int a_id = 4 * part + (tid >> 6), c_id = tid & 63;
+    const size_t cell = ((size_t)(2 * min(a_id, Mc - 1) + 1) * 2) * L + 2 * min(c_id, Mc - 1) + 1;
+    const float l0 = lk[cell], l1 = lk[cell + L];
+    const double sr0 = (double)av.SR[0], o0 = av.O[0];
+    const int tc = min(tid, TP - 1);
+    const double p_t = av.P[tc], o_t = av.O[tc];
+    constexpr int RV = 16;  // R table: up to 16 * 256 entries (64 nodes, T + 2 <= 64)
+    float rv[RV];
+#pragma unroll
+    for (int k = 0; k < RV; k++) rv[k] = av.SR[min(k * 256 + tid, Mc * TS - 1)];
+    const int wi = min(tid, 4 * TS - 1);
+    const bool w_in = 4 * part + wi / TS < Mc;
+    const size_t w_at = w_in ? (size_t)4 * part * TS + wi : 0;
+    const float w0v = av.W0[w_at], w1v = av.W1[w_at];
+    // the operands of this thread's first emission cell (clamped addresses; the cell's case picks the terms later)
+    struct CellIn {
+        double ps, os, ps1, os1;
+        float bs, bs1, f0n, f1n, f1nn, mas, mprev, mnext;
+    };
+    auto load_cell = [&](int i) {
+        CellIn c;
+        const int x = i / T, s = i - x * T, e_id = x >> 1;
+        const size_t o = (size_t)min(e_id, Mc - 1) * TS + s;
+        c.ps = av.P[s];
+        c.os = av.O[s];
+        c.ps1 = av.P[max(s, 1) - 1];
+        c.os1 = av.O[s + 1];
+        c.bs = av.BETA[o];
+        c.bs1 = av.BETA[max(o, (size_t)1) - 1];
+        c.f0n = av.F0[o + 1];
+        c.f1n = av.F1[o + 1];
+        c.f1nn = av.F1[o + 2];
+        c.mas = mt[i];
+        c.mprev = mt[max(i - T - 1, 0)];            // (x-1, s-1): the leaf's emission before parent x
+        c.mnext = mt[min(i + T + 1, L * T - 1)];    // (x+1, s+1): the parent's emission after leaf x
+        return c;
+    };
+    const CellIn first = load_cell(min(cell0 + tid, cells - 1));
+
     const bool valid = lengths_ok(m, n, L, T) && (ll == ll) && (fabsf(ll) != __builtin_huge_valf());
     if (!valid) {  // invalid sentence: all-zero gradients (nat_pcfg_loss.py:123-133 zeroes its loss as well)
         for (int i = cell0 + tid; i < cell1; i += 256) mg[i] = 0.f;
@@ -1694,48 +1746,39 @@ __global__ __launch_bounds__(256) void inside_combine_ml1_kernel(const float *__
     const int mc = m / 2;
     // a null grad_output selects the criterion's own weights: -factor/(n_b * norm_B), see Seed
     const float g = seed_weight(grad_out, b, n, seed);
-    // this thread's pair: parent 4*part + tid/64, child tid%64; its two link values travel during the staging
-    const int a_id = 4 * part + (tid >> 6), c_id = tid & 63;
     const bool pair_ok = a_id < mc && c_id < mc && a_id <= c_id;
-    const size_t cell = ((size_t)(2 * min(a_id, Mc - 1) + 1) * 2) * L + 2 * min(c_id, Mc - 1) + 1;
-    const float l0 = lk[cell], l1 = lk[cell + L];
-    const double ll_abs = (double)av.SR[0] + av.O[0];
-    for (int t = tid; t <= n - 1; t += 256) corr[t] = (float)(av.P[t] + av.O[t] - ll_abs);
-    for (int i0 = 0; i0 < Mc * TS; i0 += 8 * 256) {  // eight loads in flight per thread
-        float v[8];
+    const double ll_abs = sr0 + o0;
+    if (tid <= n - 1) corr[tid] = (float)(p_t + o_t - ll_abs);
+    for (int t = tid + 256; t <= n - 1; t += 256) corr[t] = (float)(av.P[t] + av.O[t] - ll_abs);
 #pragma unroll
-        for (int k = 0; k < 8; k++) v[k] = av.SR[min(i0 + k * 256 + tid, Mc * TS - 1)];
-#pragma unroll
-        for (int k = 0; k < 8; k++)
-            if (i0 + k * 256 + tid < Mc * TS) sm_R[i0 + k * 256 + tid] = v[k];
+    for (int k = 0; k < RV; k++)
+        if (k * 256 + tid < Mc * TS) sm_R[k * 256 + tid] = rv[k];
+    for (int i = RV * 256 + tid; i < Mc * TS; i += 256) sm_R[i] = av.SR[i];
+    if (tid < 4 * TS) {
+        sm_W0[tid] = w_in ? w0v : NEG_INF_F;
+        sm_W1[tid] = w_in ? w1v : NEG_INF_F;
     }
-    for (int i = tid; i < 4 * TS; i += 256) {
+    for (int i = tid + 256; i < 4 * TS; i += 256) {
         const bool in = 4 * part + i / TS < Mc;
         sm_W0[i] = in ? av.W0[(size_t)4 * part * TS + i] : NEG_INF_F;
         sm_W1[i] = in ? av.W1[(size_t)4 * part * TS + i] : NEG_INF_F;
     }
     // emission posteriors -> match_all_grad (pcfg_loss_backward.cu:348-382, 429-433)
-    // every operand is loaded whatever the cell's case (clamped addresses), so the loads travel together; the case picks the terms
     for (int i = cell0 + tid; i < cell1; i += 256) {
+        const CellIn c = (i == cell0 + tid) ? first : load_cell(i);
         const int x = i / T, s = i - x * T, e_id = x >> 1;
-        const size_t o = (size_t)e_id * TS + s;
-        const double ps = av.P[s], os = av.O[s], ps1 = av.P[max(s, 1) - 1], os1 = av.O[s + 1];
-        const float bs = av.BETA[o], bs1 = av.BETA[max(o, (size_t)1) - 1];
-        const float f0n = av.F0[o + 1], f1n = av.F1[o + 1], f1nn = av.F1[o + 2];
-        const float mas = to_b2(mt[i]);
-        const float mprev = to_b2(mt[max(i - T - 1, 0)]);            // (x-1, s-1): the leaf's emission before parent x
-        const float mnext = to_b2(mt[min(i + T + 1, L * T - 1)]);    // (x+1, s+1): the parent's emission after leaf x
-        const float cs = (float)(ps + os - ll_abs), cs1 = (float)(ps1 + os - ll_abs), cs2 = (float)(ps + os1 - ll_abs);
+        const float mas = to_b2(c.mas), mprev = to_b2(c.mprev), mnext = to_b2(c.mnext);
+        const float cs = (float)(c.ps + c.os - ll_abs), cs1 = (float)(c.ps1 + c.os - ll_abs), cs2 = (float)(c.ps + c.os1 - ll_abs);
         const bool in = x >= 1 && x < m && s < n, odd = x & 1;
         float out = 0.f;
         // a emits s with the null left child
-        out += (in && odd && s + 1 <= n - 1) ? ex2((bs + mas + f0n) + cs) : 0.f;
+        out += (in && odd && s + 1 <= n - 1) ? ex2((c.bs + mas + c.f0n) + cs) : 0.f;
         // a emits s after its leaf emitted s-1
-        out += (in && odd && s >= 1 && s + 1 <= n - 1 && e_id >= 1) ? ex2((bs1 + mprev + mas + f1n) + cs1) : 0.f;
+        out += (in && odd && s >= 1 && s + 1 <= n - 1 && e_id >= 1) ? ex2((c.bs1 + mprev + mas + c.f1n) + cs1) : 0.f;
         // base cell
-        out += (in && odd && e_id == mc - 1 && s == n - 1) ? ex2((bs + mas) + cs) : 0.f;
+        out += (in && odd && e_id == mc - 1 && s == n - 1) ? ex2((c.bs + mas) + cs) : 0.f;
         // leaf of parent a = x+1
-        out += (in && !odd && e_id >= 1 && e_id < mc && s + 2 <= n - 1) ? ex2((bs + mas + mnext + f1nn) + cs2) : 0.f;
+        out += (in && !odd && e_id >= 1 && e_id < mc && s + 2 <= n - 1) ? ex2((c.bs + mas + mnext + c.f1nn) + cs2) : 0.f;
         if (!(out == out)) out = 0.f;
         mg[i] = g * out;
     }
@@ -3953,12 +3996,12 @@ int launch_fused(const float *go, const float *match_all, const float *links, co
             const size_t launch_bytes = (fill && pair_bytes < PAD_EXCLUSIVE_LDS) ? PAD_EXCLUSIVE_LDS : pair_bytes;
             if (launch_bytes != pair_bytes)
                 PCFGNAT_DYNAMIC_LDS(inside_pair_ml1_kernel, launch_bytes);
-            hipLaunchKernelGGL(inside_pair_ml1_kernel, dim3((2 + (fill ? PAD_WGS : 0)) * B), dim3(NTR), launch_bytes, stream, match_all,
+            hipLaunchKernelGGL(inside_pair_ml1_kernel, dim3((2 + (fill ? PAD_WGS_SWEEPS : 0)) * B), dim3(NTR), launch_bytes, stream, match_all,
                                links, ol, tl, S, aux, L, T, Mc, B, pad, lin_bits);
             PCFGNAT_HIP_CHECK(hipGetLastError());
             if (fill && pad_done) *pad_done = true;
-            hipLaunchKernelGGL(inside_combine_ml1_kernel, dim3(16, B), dim3(256), comb_bytes, stream, go, S, aux, match_all, links, ol, tl,
-                               mg, lg, L, T, Mc, seed);
+            hipLaunchKernelGGL(inside_combine_ml1_kernel, dim3(16 + (fill ? PAD_WGS - PAD_WGS_SWEEPS : 0), B), dim3(256), comb_bytes, stream,
+                               go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc, seed, fill ? pad : PadFill{nullptr, 0});
             PCFGNAT_HIP_CHECK(hipGetLastError());
             *done = true;
             return PCFGNAT_OK;
