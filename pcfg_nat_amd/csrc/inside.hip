@@ -18,8 +18,11 @@
 // reads links, emissions and its own earlier columns only, so in the single call the two run side by side as two
 // workgroups (inside_pair_ml1_kernel) and a parallel kernel multiplies their tables into the posteriors
 // (inside_combine_ml1_kernel); in the two-call API the outside sweep accumulates rule posteriors in registers and
-// emission posteriors come from an element-wise epilogue.  Graphs of more than 130 nodes use the streaming or the
-// pipelined sweeps further down (link rows from L2, or spread over several workgroups per sentence).
+// emission posteriors come from an element-wise epilogue.  Where the tables leave room in LDS (the shipped shapes do),
+// these sweeps run in the linear domain - probabilities as doubles, one multiply-add per term, the table entries made
+// by waves of their own - and fall back to the log domain per sentence when a number leaves the range (further down).
+// Graphs of more than 130 nodes use the streaming or the pipelined sweeps (link rows from L2, or spread over several
+// workgroups per sentence).
 #include "common.hip.h"
 #include "glat_glue.hip.h"
 
