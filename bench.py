@@ -502,6 +502,16 @@ def main():
         sc["sentences_per_s_median"] = B / (sc["ms_per_step_median"] * 1e-3)
         sc["loss_scale"] = 128.0
         result["single_call_scaled"] = sc
+        # the same single call with the inside and outside sweeps in the linear domain, an option that is off by default: it
+        # pays on emissions as flat as these synthetic ones and costs on a model that is sure of itself
+        from pcfg_nat_amd import custom_ops
+        try:
+            custom_ops.inside_linear_bits(500)
+            lin = timed_windows(lambda i: step_fn(bufs[i], targets, links, ol, tl))
+        finally:
+            custom_ops.inside_linear_bits(0)
+        lin["sentences_per_s_median"] = B / (lin["ms_per_step_median"] * 1e-3)
+        result["single_call_linear_sweeps"] = lin
     # the drop-in path: the unchanged criterion code over the operator API under autograd (dag_logsoftmax_gather_inplace ->
     # eos mask -> cuda_pcfg_loss -> loss -> backward), which reads and rewrites every row (it is not told the lengths)
     result["operator_api"] = operator_api_timing(bufs, targets, links, ol, tl, args, timed_windows, host_enqueue_ms)

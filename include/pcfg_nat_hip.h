@@ -192,11 +192,12 @@ void pcfgnat_pipeline_config(int max_workgroups, int spin_limit);
 void pcfgnat_links_grad_range_limit(float log2_limit);
 
 /*
- * No counterpart in the reference: graphs of up to 130 nodes are swept in the linear domain (probabilities in double,
- * one multiply-add per term) where the numbers allow it - links and emissions between 2^-150 and 2^8 or zero, every
- * intermediate at least 2^-bits or exactly zero - and in the log domain, which has no range limit, otherwise; the choice
- * is made per sentence and per sweep by the kernel.  bits: default and maximum 500; 0 switches the linear sweeps off.
- * Process-wide, for tests.
+ * No counterpart in the reference: with bits > 0, graphs of up to 130 nodes are swept in the linear domain (probabilities
+ * in double, one multiply-add per term) where the numbers allow it - links and emissions between 2^-150 and 2^8 or zero,
+ * every intermediate at least 2^-bits or exactly zero - and in the log domain, which has no range limit, otherwise; the
+ * choice is made per sentence and per sweep by the kernel, at the end of the linear sweep.  Pays where emissions are not
+ * peaked (a third off the sweeps' time), costs where a model is sure of itself (a sentence handed over is swept twice).
+ * bits: at most 500; 0, the default, switches the linear sweeps off.  Process-wide.
  */
 void pcfgnat_inside_linear_bits(int bits);
 

@@ -19,8 +19,9 @@
 // workgroups (inside_pair_ml1_kernel) and a parallel kernel multiplies their tables into the posteriors
 // (inside_combine_ml1_kernel); in the two-call API the outside sweep accumulates rule posteriors in registers and
 // emission posteriors come from an element-wise epilogue.  Where the tables leave room in LDS (the shipped shapes do),
-// these sweeps run in the linear domain - probabilities as doubles, one multiply-add per term, the table entries made
-// by waves of their own - and fall back to the log domain per sentence when a number leaves the range (further down).
+// these sweeps can run in the linear domain instead - probabilities as doubles, one multiply-add per term, the table
+// entries made by waves of their own - falling back to the log domain per sentence when a number leaves the range
+// (further down; off unless pcfgnat_inside_linear_bits switches it on).
 // Graphs of more than 130 nodes use the streaming or the pipelined sweeps (link rows from L2, or spread over several
 // workgroups per sentence).
 #include "common.hip.h"
@@ -1613,9 +1614,11 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
     }
 }
 
-// Workgroups per sentence that zero the rows of its pad nodes (see PadFill): PAD_WGS_SWEEPS of them beside the sweeps, the
-// others beside the posteriors, in proportion to how long the two launches take without them.
-constexpr int PAD_WGS = 32, PAD_WGS_SWEEPS = 22;
+// Workgroups per sentence that zero the rows of its pad nodes (see PadFill): PadFill::with_sweeps of them beside the
+// sweeps, the others beside the posteriors.  One fill workgroup per compute unit on the units the sweeps leave free
+// writes about 4.3 TB/s: beside the log-domain sweeps (29 us) the whole fill fits, beside the shorter linear-domain
+// ones (20 us) two thirds of it.
+constexpr int PAD_WGS = 32, PAD_WGS_BESIDE_LINEAR_SWEEPS = 22;
 // The fill rides along while the sweeps take up no more than three quarters of the compute units (192 of 256 on MI355X).
 inline int pad_max_sweep_wgs() { return device_compute_units() * 3 / 4; }
 constexpr size_t PAD_EXCLUSIVE_LDS = 84 * 1024;  // more than half of the 160 KB of a gfx950 compute unit
@@ -1649,15 +1652,15 @@ __device__ __forceinline__ void pad_fill_block(const PadFill pad, const int64_t 
     for (int64_t i = lo + tid; i < hi; i += NTF) __builtin_nontemporal_store(zero, v + i);
 }
 
-// 2*nsent workgroups: 2b runs the forward sweep of sentence b, 2b+1 its outside sweep; PAD_WGS_SWEEPS*nsent more when
+// 2*nsent workgroups: 2b runs the forward sweep of sentence b, 2b+1 its outside sweep; pad_parts*nsent more when
 // there is a pad-fill task, which land on the compute units the sweeps leave free.
 __global__ __launch_bounds__(NTR) void inside_pair_ml1_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
                                                              const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
                                                              float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc,
-                                                             int nsent, PadFill pad, int lin_bits) {
+                                                             int nsent, PadFill pad, int pad_parts, int lin_bits) {
     if ((int)blockIdx.x >= 2 * nsent) {  // workgroup-uniform
         const int z = (int)blockIdx.x - 2 * nsent;
-        pad_fill_block(pad, out_len, z / PAD_WGS_SWEEPS, z % PAD_WGS_SWEEPS, L);
+        pad_fill_block(pad, out_len, z / pad_parts, z % pad_parts, L);
         return;
     }
     const int b = blockIdx.x >> 1;
@@ -1665,7 +1668,7 @@ __global__ __launch_bounds__(NTR) void inside_pair_ml1_kernel(const float *__res
     else inside_outside_ml1_body(b, match_all, links, out_len, tgt_len, aux, L, T, Mc, lin_bits);
 }
 
-// Posteriors from the tables of the two sweeps: grid (16, B), 256 threads (PAD_WGS - PAD_WGS_SWEEPS more workgroups per
+// Posteriors from the tables of the two sweeps: grid (16, B), 256 threads (PAD_WGS - pad_parts more workgroups per
 // sentence when there is a pad-fill task).  Workgroup (q, b) owns the parents 4q .. 4q+3 of
 // sentence b: it writes the rows 8q .. 8q+7 of the links_grad slab (zeros included) and a sixteenth of the match_all_grad
 // cells.  One thread per (parent, child) pair sums both planes over the columns.
@@ -1675,9 +1678,9 @@ __global__ __launch_bounds__(256) void inside_combine_ml1_kernel(const float *__
                                                                 const float *__restrict__ links, const int64_t *__restrict__ out_len,
                                                                 const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad,
                                                                 float *__restrict__ lgrad, int L, int T, int Mc, Seed seed,
-                                                                PadFill pad) {
+                                                                PadFill pad, int pad_parts) {
     if (blockIdx.x >= 16) {  // workgroup-uniform: the part of the pad fill that rides along with this launch
-        pad_fill_block(pad, out_len, blockIdx.y, PAD_WGS_SWEEPS + (int)blockIdx.x - 16, L);
+        pad_fill_block(pad, out_len, blockIdx.y, pad_parts + (int)blockIdx.x - 16, L);
         return;
     }
     const int TS = T + 2, TP = T + 4;
@@ -3731,8 +3734,9 @@ std::atomic<int> g_pipeline_spin_limit_outside{-1};  // side-by-side launch only
 // links_grad_ml1_stream_kernel); a tile beyond it is recomputed term by term.  pcfgnat_links_grad_range_limit.
 std::atomic<float> g_links_grad_range_limit{120.f};
 // Smallest nonzero number, as a power of two, that the linear-domain sweeps of graphs of up to 130 nodes accept before
-// they hand the sentence to the log-domain sweep (see LIN_INPUT_BITS); 0 switches them off.  pcfgnat_inside_linear_bits.
-std::atomic<int> g_inside_linear_bits{LIN_BITS_MAX};
+// they hand the sentence to the log-domain sweep (see LIN_INPUT_BITS); 0, the default, switches them off: they pay on
+// emissions that are not peaked and cost on a model that is sure of itself.  pcfgnat_inside_linear_bits.
+std::atomic<int> g_inside_linear_bits{0};
 inline int inside_linear_bits() { return g_inside_linear_bits.load(); }
 int pipeline_chunks(int B, int T, int Mc) {  // NQ, or 0 where the pipelined sweeps do not apply
     const int NQ = stream_mp(Mc) / 64, CL = 64 * NQ / NLP;
@@ -3999,12 +4003,13 @@ int launch_fused(const float *go, const float *match_all, const float *links, co
             const size_t launch_bytes = (fill && pair_bytes < PAD_EXCLUSIVE_LDS) ? PAD_EXCLUSIVE_LDS : pair_bytes;
             if (launch_bytes != pair_bytes)
                 PCFGNAT_DYNAMIC_LDS(inside_pair_ml1_kernel, launch_bytes);
-            hipLaunchKernelGGL(inside_pair_ml1_kernel, dim3((2 + (fill ? PAD_WGS_SWEEPS : 0)) * B), dim3(NTR), launch_bytes, stream, match_all,
-                               links, ol, tl, S, aux, L, T, Mc, B, pad, lin_bits);
+            const int pad_parts = lin_bits > 0 ? PAD_WGS_BESIDE_LINEAR_SWEEPS : PAD_WGS;
+            hipLaunchKernelGGL(inside_pair_ml1_kernel, dim3((2 + (fill ? pad_parts : 0)) * B), dim3(NTR), launch_bytes, stream, match_all,
+                               links, ol, tl, S, aux, L, T, Mc, B, pad, pad_parts, lin_bits);
             PCFGNAT_HIP_CHECK(hipGetLastError());
             if (fill && pad_done) *pad_done = true;
-            hipLaunchKernelGGL(inside_combine_ml1_kernel, dim3(16 + (fill ? PAD_WGS - PAD_WGS_SWEEPS : 0), B), dim3(256), comb_bytes, stream,
-                               go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc, seed, fill ? pad : PadFill{nullptr, 0});
+            hipLaunchKernelGGL(inside_combine_ml1_kernel, dim3(16 + (fill ? PAD_WGS - pad_parts : 0), B), dim3(256), comb_bytes, stream,
+                               go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc, seed, fill ? pad : PadFill{nullptr, 0}, pad_parts);
             PCFGNAT_HIP_CHECK(hipGetLastError());
             *done = true;
             return PCFGNAT_OK;

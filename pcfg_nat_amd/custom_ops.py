@@ -61,9 +61,9 @@ def pipeline_redo_counts(reset=False):
     return a.value, b.value
 
 
-def inside_linear_bits(bits=500):
-    """Test hook (process-wide): the smallest nonzero number, as a power of two, that the linear-domain sweeps of graphs of
-    up to 130 nodes accept before they hand a sentence to the log-domain sweep; 0 switches them off."""
+def inside_linear_bits(bits=0):
+    """Process-wide setting: the smallest nonzero number, as a power of two, that the linear-domain sweeps of graphs of up to
+    130 nodes accept before they hand a sentence to the log-domain sweep (at most 500); 0, the default, switches them off."""
     _lib.load().pcfgnat_inside_linear_bits(int(bits))
 
 
