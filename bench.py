@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # profiles/lsg_cfg2_hbm_traffic_pmc.md.  None = not measured for this build.  (lsg_bwd: the single-call step at this
 # batch's lengths - 3408 of 5120 rows read and written.  Part of its reads are served by the 256 MB memory-side cache, where
 # the forward pass leaves the rows, which is how the kernel exceeds the rate of a device copy.)
-EVENT_EVERY = 4  # steps between two bracketed launches of the roofline kernel inside the timed region
+EVENT_EVERY = 5  # steps between two bracketed launches of the roofline kernel inside the timed region
 ROOFLINE_KERNEL = {"single": "lsg_bwd", "fused": "lsg_bwd", "unfused": "lsg_fwd"}
 ROOFLINE_KERNEL_NAME = {"lsg_bwd": "lsg_bwd_kernel<half, from logits>", "lsg_fwd": "lsg_fwd_kernel<half, grad>"}
 MEASURED_TRAFFIC_BYTES = {"lsg_bwd": 546.55e6, "lsg_fwd": 273.76e6}

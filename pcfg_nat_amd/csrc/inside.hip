@@ -164,6 +164,10 @@ struct FwdSweepArgs {
     double *sm_O;
     float base_b2;  // the base cell S[last][n-1], base 2
     int n, mc, Mc, T, j, g8;
+    // where the sweep starts: column n-1 with offset 0 or, taking over from a linear-domain sweep that ran out of range,
+    // an earlier column t_start, found in col with its offset O_start, the row sums F1 of the step before it in sm_F1
+    int t_start;
+    double O_start;
 };
 
 // max of three values that need no canonicalisation (loaded from tables this kernel wrote)
@@ -195,12 +199,20 @@ __device__ __forceinline__ void fwd_sweep(const float (&A0)[R][8 * R], const flo
     constexpr int MP = 64 * R;
     const int T = x.T, TS = x.T + 2, j = x.j;
     float F1prev[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) F1prev[r] = NEG_INF_F;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    double O = 0.0;           // offset of the column being read
     float wprev = x.base_b2;  // this wave's maximum of the column written by the previous step
-    for (int t = x.n - 1; t >= 1; t--) {
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        F1prev[r] = NEG_INF_F;
+        if (TAB_LDS && x.t_start < x.n - 1) {
+            const int a_id = 64 * r + 8 * P + x.g8;
+            const float c_own = x.col[(x.t_start & 1) * MP + a_id];
+            F1prev[r] = (a_id < x.mc) ? x.sm_F1[a_id * TS + x.t_start + 1] : NEG_INF_F;
+            wprev = (r == 0) ? c_own : fmaxf(wprev, c_own);
+        }
+    }
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    double O = x.O_start;  // offset of the column being read
+    for (int t = x.t_start; t >= 1; t--) {
         const float *cur = x.col + (t & 1) * MP;
         float *nxt = x.col + ((t - 1) & 1) * MP;
         float wmax = NEG_INF_F;
@@ -310,13 +322,21 @@ __device__ __forceinline__ void fwd_sweep(const float (&A0)[R][8 * R], const flo
 // of two (exact), and the tables are relative to the same kind of offsets (D, O / E, P hold integers here).
 // What the range cannot hold must not be lost silently - a node whose inside value is 2^-600 of its column's largest
 // may still carry the whole posterior.  So a sweep only accepts numbers it can follow: links and emissions between
-// 2^-LIN_INPUT_BITS and 2^LIN_INPUT_TOP (or zero), every shifted row sum and every column entry at least 2^-lin_bits
-// (lin_bits <= 500; or exactly zero, which then is a sum of exact zeros: with these bounds a column grows by less than
-// 2^25 a step, shifts stay below 2^80, and no product of nonzero factors gets below 2^-900; all terms are positive, so
-// nothing cancels).  Anything else raises the workgroup's flag and the sentence is swept again in the log domain by the
-// code above.  lin_bits <= 0 switches the linear sweeps off.
+// 2^-LIN_INPUT_BITS and 2^LIN_INPUT_TOP (or zero), and every number a later step multiplies - column entries, the row
+// sums F1, betas, offered weights - at least 2^-lin_bits (lin_bits <= 500; or exactly zero, which then is a sum of exact
+// zeros: with these bounds a column grows by less than 2^25 a step, shifts stay below 2^80, and no product of nonzero
+// factors gets below 2^-900; all terms are positive, so nothing cancels).  An input out of range raises the workgroup's
+// flag and the sentence is swept in the log domain by the code above.  A number below 2^-lin_bits on the way (peaked
+// emissions: a node far from the alignment loses tens of bits per token against the column's largest) stops the sweep
+// instead: the table wave that watches the range - one step behind the sweep, so the number itself is still a product
+// of accepted ones and exact - sets a mark beside the shift the sweep reads at the top of its next step; every wave
+// leaves its loop behind that step (whose results nobody reads), and the log-domain sweep goes on from the last column that holds only such numbers, reading
+// its state (column, row sums, shift, offset) from the tables, which both kinds of sweep keep in the same form.  What
+// the interrupted steps wrote beyond that column is overwritten.  lin_bits <= 0 switches the linear sweeps off.
 // ------------------------------------------------------------------------------------------------------------
 constexpr float LIN_INPUT_BITS = 150.f, LIN_INPUT_TOP = 8.f;
+// Nothing a sweep accepts can get below 2^-900; a number this small means the bounds above do not hold.
+constexpr int LIN_FLOOR_BITS = 1000;
 constexpr int LIN_BITS_MAX = 500;
 
 // the partner lane's double inside a quad (every lane has a source, so there is no old value to keep)
@@ -371,10 +391,11 @@ __device__ __forceinline__ unsigned range_key(double d) { return (unsigned)__dou
 __device__ __forceinline__ unsigned range_key_of_bits(int bits) { return ((unsigned)(1023 - bits) << 20) - 1u; }
 
 // Extra dynamic LDS of a linear sweep, behind the role's own (16-byte aligned): three rotating columns [2][64] of
-// doubles, the emission probabilities of main nodes and leaves [Mc][T] each, the shifts [T+4] and the flag (ints).
+// doubles, the emission probabilities of main nodes and leaves [Mc][T] each, per step its shift and its stop mark
+// [T+4][2] and the flag (ints).
 __host__ __device__ inline size_t align16(size_t bytes) { return (bytes + 15) & ~(size_t)15; }
 __host__ __device__ inline size_t lin_extra_bytes(int Mc, int T) {
-    return ((size_t)3 * 128 + (size_t)2 * Mc * T) * sizeof(double) + align16((size_t)(T + 6) * sizeof(int));
+    return ((size_t)3 * 128 + (size_t)2 * Mc * T) * sizeof(double) + align16((size_t)(2 * (T + 4) + 2) * sizeof(int));
 }
 struct LinLds {
     double *col0, *col1, *col2, *em, *el;
@@ -386,7 +407,7 @@ struct LinLds {
         em = col2 + 128;
         el = em + Mc * T;
         kbuf = reinterpret_cast<int *>(el + Mc * T);
-        flag = kbuf + T + 4;
+        flag = kbuf + 2 * (T + 4);
     }
 };
 
@@ -418,6 +439,15 @@ __device__ __forceinline__ bool lin_fill_emissions(double *em, double *el, const
     return ok_all != 0;
 }
 
+// The emissions a linear-domain sweep staged, as the base-2 logarithms the log-domain sweep works on (all threads of the
+// workgroup; the linear-domain sweep used these numbers, so the sweep that takes over does too).
+__device__ __forceinline__ void lin_emissions_to_logs(const LinLds &x, float *fm, float *fl, int Mc, int T) {
+    for (int i = threadIdx.x; i < Mc * T; i += blockDim.x) {
+        fm[i] = log2_of(x.em[i]);
+        fl[i] = log2_of(x.el[i]);
+    }
+}
+
 // Keeps loaded values (and their loads) in front of the arithmetic that follows, so that all LDS reads of a step are
 // issued back to back instead of two at a time between the multiply-adds.
 __device__ __forceinline__ void pin(double2 &v) { asm volatile("" : "+v"(v.x), "+v"(v.y)); }
@@ -436,7 +466,7 @@ struct FwdLinArgs {
 // every node of the wave).  col0: inside probabilities of the column read / written; col1, col2: the row sums of the
 // step, for the table waves.  Returns false if a link is out of range.
 template <int W>
-__device__ __forceinline__ bool fwd_sweep_lin(const LinLds &x, const FwdLinArgs &g) {
+__device__ __forceinline__ bool fwd_sweep_lin(const LinLds &x, const FwdLinArgs &g, int &stopped_at) {
     constexpr int MP = 64;
     const int n = g.n, mc = g.mc, Mc = g.Mc, L = g.L, T = g.T;
     const int lane = threadIdx.x & 63, j = lane & 3, a_id = 16 * W + (lane >> 2);
@@ -481,7 +511,10 @@ __device__ __forceinline__ bool fwd_sweep_lin(const LinLds &x, const FwdLinArgs 
     __syncthreads();  // the table waves have staged the emissions, the first column and the first shift
     double F1prev = 0.0;
     double em_p = x.em[ai * T + n - 2], el_p = x.el[ai * T + n - 2], em_t = x.em[ai * T + n - 1];
-    for (int t = n - 1; t >= 1; t--) {
+    // A stop mark (column t+1 holds a number below the range) ends the loop behind the step that read it, not inside it
+    // - a branch in the middle of the step costs more than the step whose results nobody reads.
+    int stop = 0;
+    for (int t = n - 1; t >= 1 && !stop; t--) {
         const double2 *cur = reinterpret_cast<const double2 *>(x.col0 + (t & 1) * MP);
         double2 xv[4][2];
 #pragma unroll
@@ -489,13 +522,16 @@ __device__ __forceinline__ bool fwd_sweep_lin(const LinLds &x, const FwdLinArgs 
             xv[q][0] = cur[8 * q + 2 * j];
             xv[q][1] = cur[8 * q + 2 * j + 1];
         }
-        int k = x.kbuf[t];
+        const int2 ks = *reinterpret_cast<const int2 *>(x.kbuf + 2 * t);  // the step's shift and its stop mark
+        int k = ks.x;
 #pragma unroll
         for (int q = W; q < 4; q++) {
             pin(xv[q][0]);
             pin(xv[q][1]);
         }
         pin(k);
+        stop = __builtin_amdgcn_readfirstlane(ks.y);
+        stopped_at = stop ? t : stopped_at;
         const double down = pow2_int(-k);
         double emd = em_p * down, rest = ((F1prev * down) * el_p) * em_t;
         pin(emd);
@@ -532,11 +568,14 @@ __device__ __forceinline__ bool fwd_sweep_lin(const LinLds &x, const FwdLinArgs 
     return ok != 0;
 }
 
-// The table waves of the forward sweep (role 0: column entries, shifts and offsets; 1, 2: the two row sums; 3: idle).
-// They stage the emissions and the first column, then follow one step behind the sweep: iteration t turns column t and
-// the row sums of step t+1 into table entries; pass t = 0 after the last barrier finishes the job.  Returns the smallest
-// range key seen; ok: false if an emission is out of range.
-__device__ __forceinline__ unsigned fwd_tables_lin(const LinLds &x, const FwdLinArgs &g, int role, bool &ok) {
+// The table waves of the forward sweep (role 0: column entries, shifts and offsets; 1, 2: the two row sums; 3: the range
+// watch).  They stage the emissions and the first column, then follow one step behind the sweep: iteration t turns
+// column t and the row sums of step t+1 into table entries; pass t = 0 after the last barrier finishes the job.  The
+// watch looks at what step t-1 will multiply - column t, the row sums F1 of step t+1 (F0 is used up in the step that
+// makes it) - and marks step t-1 if one of them is below the range: the sweep reads the mark with the shift at the top
+// of that step and every wave leaves its loop behind it.  Returns the smallest range key seen in what the sweep stands
+// for; ok: false if an emission is out of range.
+__device__ __forceinline__ unsigned fwd_tables_lin(const LinLds &x, const FwdLinArgs &g, int role, bool &ok, int lin_bits, int &stopped_at) {
     constexpr int MP = 64;
     const int n = g.n, mc = g.mc, Mc = g.Mc, T = g.T, TS = g.T + 2, ht = threadIdx.x - 256, node = threadIdx.x & 63;
     const bool live = node < mc;
@@ -553,14 +592,20 @@ __device__ __forceinline__ unsigned fwd_tables_lin(const LinLds &x, const FwdLin
     for (int i = ht; i < TS + 2; i += 256) {
         g.sm_D[i] = (i == n - 1) ? (float)k_base : 0.f;
         if (i < TS) g.sm_O[i] = (i == n - 2) ? (double)k_base : 0.0;
-        x.kbuf[i] = (i == n - 1) ? k_base : 0;
+        x.kbuf[2 * i] = (i == n - 1) ? k_base : 0;
+        x.kbuf[2 * i + 1] = 0;
     }
     if (ht == 0) *x.flag = 0;
     __syncthreads();
     unsigned lowest = ~0u;
     int k_last = k_base;       // k_t at iteration t
     double O_run = k_base;     // O[t-1] at iteration t
+    const unsigned too_small = range_key_of_bits(lin_bits);
     for (int t = n - 1; t >= 0; t--) {
+        // the sweep stops behind step t if that step is marked; what this pass then makes of column t (which step t+1
+        // computed from the numbers that stopped it) is overwritten by the sweep that takes over, and is not vouched for
+        const int mark = x.kbuf[2 * t + 1];
+        unsigned seen = lowest;
         if (role == 0) {
             const double v = x.col0[(t & 1) * MP + node];
             if (t >= 2) {
@@ -569,7 +614,7 @@ __device__ __forceinline__ unsigned fwd_tables_lin(const LinLds &x, const FwdLin
                 const int e = wave_max_i(exponent_or_none(v));
                 const int k = e == NO_EXPONENT ? 0 : clamp_shift(e - k_last);
                 if (node == 0) {
-                    x.kbuf[t - 1] = k;
+                    x.kbuf[2 * (t - 1)] = k;
                     g.sm_D[t - 1] = (float)k;
                     O_run += (double)k;
                     g.sm_O[t - 2] = O_run;
@@ -577,41 +622,55 @@ __device__ __forceinline__ unsigned fwd_tables_lin(const LinLds &x, const FwdLin
                 k_last = k;
             }
             if (t < n - 1 && live) g.sm_S[node * TS + t] = log2_of(v);
-            lowest = min(lowest, range_key(v));
+            seen = min(lowest, range_key(v));
         } else if (role <= 2 && t < n - 1) {
             const double v = (role == 1 ? x.col1 : x.col2)[((t + 1) & 1) * MP + node];
             if (live) (role == 1 ? g.sm_F0 : g.sm_F1)[node * TS + t + 1] = log2_of(v);
-            lowest = min(lowest, range_key(v));
+            seen = min(lowest, range_key(v));
+        } else if (role == 3 && t >= 1) {
+            const double v = x.col0[(t & 1) * MP + node], f1 = x.col2[((t + 1) & 1) * MP + node];
+            const bool below = min(range_key(v), range_key(f1)) < too_small;
+            if (__builtin_amdgcn_ballot_w64(below) != 0 && node == 0) x.kbuf[2 * (t - 1) + 1] = 1;
         }
         if (t >= 1) lds_barrier();
+        if (mark != 0) {
+            stopped_at = t;  // (0: marked while the last step ran - the caller finds that in the mark itself)
+            break;
+        }
+        lowest = seen;
     }
     return lowest;
 }
 
 // The forward sweep of a sentence in the linear domain (R = 1, tables in LDS): fills sm_S, sm_F0, sm_F1, hd.D, hd.O like
-// the log-domain code of inside_fwd_ml1_body and returns true, or returns false (workgroup-uniform) with the tables in an
-// undefined state.  `lin` is the extra LDS (lin_extra_bytes(Mc, T)).
-__device__ __forceinline__ bool inside_fwd_lin_attempt(const float *__restrict__ mt, const float *__restrict__ lk, const LdsHead &hd,
-                                                      float *sm_S, float *sm_F0, float *sm_F1, double *lin, int m, int n, int L,
-                                                      int T, int Mc, int lin_bits) {
+// the log-domain code of inside_fwd_ml1_body.  Returns (workgroup-uniform) 0 if the sweep is complete; t >= 1 if it stopped
+// with column t as the last one it can vouch for - sm_S[.][t..], sm_F0/sm_F1[.][t+1..], hd.D[t+1..], hd.O[t..] are in
+// place and the log-domain sweep takes over from there; -1 if nothing of it can be used (an input out of range).
+// `lin` is the extra LDS (lin_extra_bytes(Mc, T)).
+__device__ __forceinline__ int inside_fwd_lin_attempt(const float *__restrict__ mt, const float *__restrict__ lk, const LdsHead &hd,
+                                                     float *sm_S, float *sm_F0, float *sm_F1, double *lin, int m, int n, int L, int T,
+                                                     int Mc, int lin_bits) {
     const LinLds x(lin, Mc, T);
     const FwdLinArgs g{mt, lk, sm_S, sm_F0, sm_F1, hd.D, hd.O, m, n, m / 2, Mc, L, T};
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     unsigned lowest = ~0u;
     bool ok;
+    int stopped_at = 0;  // the step in front of which the sweep stopped (every wave leaves its loop at the same one)
     switch (wave) {  // wave-uniform; every branch meets the same barriers
-        case 0: ok = fwd_sweep_lin<0>(x, g); break;
-        case 1: ok = fwd_sweep_lin<1>(x, g); break;
-        case 2: ok = fwd_sweep_lin<2>(x, g); break;
-        case 3: ok = fwd_sweep_lin<3>(x, g); break;
-        default: lowest = fwd_tables_lin(x, g, 7 - wave, ok); break;  // role 0 beside the sweep wave with the fewest children
+        case 0: ok = fwd_sweep_lin<0>(x, g, stopped_at); break;
+        case 1: ok = fwd_sweep_lin<1>(x, g, stopped_at); break;
+        case 2: ok = fwd_sweep_lin<2>(x, g, stopped_at); break;
+        case 3: ok = fwd_sweep_lin<3>(x, g, stopped_at); break;
+        default: lowest = fwd_tables_lin(x, g, 7 - wave, ok, lin_bits, stopped_at); break;  // role 0 beside the sweep wave with the fewest children
     }
-    if (!ok || lowest < range_key_of_bits(lin_bits)) *x.flag = 1;
+    if (!ok || lowest < range_key_of_bits(LIN_FLOOR_BITS)) *x.flag = 1;
     __syncthreads();
     const bool good = *x.flag == 0;
-    if (threadIdx.x == 0) atomicAdd(good ? &g_linear_swept : &g_linear_handed_over, 1ull);
+    // a number below the range in column 1 (or in the F1 of step 2) is met while the last step runs: that step is redone
+    const int resume_at = stopped_at > 0 ? stopped_at + 1 : (x.kbuf[1] != 0 ? 1 : 0);
+    if (threadIdx.x == 0) atomicAdd(good && resume_at == 0 ? &g_linear_swept : &g_linear_handed_over, 1ull);
     __syncthreads();  // the flag's cell may be written again by the log-domain sweep's staging
-    return good;
+    return good ? resume_at : -1;
 }
 
 // Forward.  Dynamic LDS: head (see LdsHead), col[2][64R]; with TAB_LDS also the emissions of main nodes and of their
@@ -649,11 +708,12 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
     const int mc = m / 2;  // active main-chain nodes: a_id < mc
 
     // the linear-domain sweep first, where the launch brought the LDS for it; what it cannot follow is swept below
-    bool swept = false;
+    int resume_at = -1;  // 0: swept; t >= 1: the sweep below takes over at column t; -1: it starts from the base cell
     if (R == 1 && TAB_LDS && lin_bits > 0)
-        swept = inside_fwd_lin_attempt(mt, lk, hd, sm_S, sm_F0, sm_F1, reinterpret_cast<double *>(smem + fwd_role_floats(Mc, T)), m, n,
-                                       L, T, Mc, lin_bits);
-    if (!swept) {
+        resume_at = inside_fwd_lin_attempt(mt, lk, hd, sm_S, sm_F0, sm_F1,
+                                           reinterpret_cast<double *>(smem + fwd_role_floats(Mc, T)), m, n, L, T, Mc, lin_bits);
+    if (resume_at != 0) {
+    const int t_start = resume_at > 0 ? resume_at : n - 1;
     // link slabs -> registers; the loads are unconditional (clamped addresses) so that they are all in flight together
     float A0[R][NQ], A1[R][NQ];
 #pragma unroll
@@ -669,17 +729,21 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
     }
     const float base_cell = sanitize(mt[(size_t)(m - 1) * T + (n - 1)]);  // pcfg_loss.cu:142-147
     if (TAB_LDS) {
-        for (int i = tid; i < Mc * T; i += NTR) {
-            const int a_id = i / T, s = i - a_id * T;
-            const float vm = mt[(size_t)(2 * a_id + 1) * T + s], vl = mt[(size_t)(2 * a_id) * T + s];
-            const bool ok = a_id < mc && s < n;
-            sm_main[i] = ok ? to_b2(vm) : NEG_INF_F;
-            sm_leaf[i] = (ok && a_id >= 1) ? to_b2(vl) : NEG_INF_F;
-        }
-        for (int i = tid; i < Mc * TS; i += NTR) {
-            sm_S[i] = (i == (mc - 1) * TS + (n - 1)) ? base_cell * LOG2E_F : NEG_INF_F;
-            sm_F0[i] = NEG_INF_F;
-            sm_F1[i] = NEG_INF_F;
+        if (resume_at > 0) {
+            lin_emissions_to_logs(LinLds(reinterpret_cast<double *>(smem + fwd_role_floats(Mc, T)), Mc, T), sm_main, sm_leaf, Mc, T);
+        } else {
+            for (int i = tid; i < Mc * T; i += NTR) {
+                const int a_id = i / T, s = i - a_id * T;
+                const float vm = mt[(size_t)(2 * a_id + 1) * T + s], vl = mt[(size_t)(2 * a_id) * T + s];
+                const bool ok = a_id < mc && s < n;
+                sm_main[i] = ok ? to_b2(vm) : NEG_INF_F;
+                sm_leaf[i] = (ok && a_id >= 1) ? to_b2(vl) : NEG_INF_F;
+            }
+            for (int i = tid; i < Mc * TS; i += NTR) {
+                sm_S[i] = (i == (mc - 1) * TS + (n - 1)) ? base_cell * LOG2E_F : NEG_INF_F;
+                sm_F0[i] = NEG_INF_F;
+                sm_F1[i] = NEG_INF_F;
+            }
         }
     } else {
         // cells of S and R the sweep never writes: rows beyond the sentence, columns from n-1 on (except the base cell)
@@ -692,12 +756,23 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
             }
         }
     }
-    for (int i = tid; i < MP; i += NTR) col[((n - 1) & 1) * MP + i] = (i == mc - 1) ? base_cell * LOG2E_F : NEG_INF_F;
-    for (int i = tid; i < TS + 2; i += NTR) {
-        hd.D[i] = 0.f;
-        if (i < TS) hd.O[i] = 0.0;
+    double O_start = 0.0;
+    if (TAB_LDS && resume_at > 0) {
+        // column t_start as the linear-domain sweep left it in the table, its maximum as the shift of the first step
+        const int node = tid & 63;
+        const float own = node < mc ? sm_S[node * TS + t_start] : NEG_INF_F;
+        const float col_max = wave_max(own);
+        if (tid < MP) col[(t_start & 1) * MP + tid] = own;
+        if (tid < 16) hd.slots[tid] = col_max;
+        O_start = hd.O[t_start];
+    } else {
+        for (int i = tid; i < MP; i += NTR) col[((n - 1) & 1) * MP + i] = (i == mc - 1) ? base_cell * LOG2E_F : NEG_INF_F;
+        for (int i = tid; i < TS + 2; i += NTR) {
+            hd.D[i] = 0.f;
+            if (i < TS) hd.O[i] = 0.0;
+        }
+        if (tid < 16) hd.slots[tid] = base_cell * LOG2E_F;  // maximum of column n-1
     }
-    if (tid < 16) hd.slots[tid] = base_cell * LOG2E_F;  // maximum of column n-1
 #pragma unroll
     for (int r = 0; r < R; r++) {
         const int a_id = 64 * r + 8 * p + g8;
@@ -710,7 +785,7 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
         }
     }
     __syncthreads();
-    FwdSweepArgs sa{col, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, av.F0, av.F1, av.SR, hd.slots, hd.D, hd.O, base_cell * LOG2E_F, n, mc, Mc, T, j, g8};
+    FwdSweepArgs sa{col, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, av.F0, av.F1, av.SR, hd.slots, hd.D, hd.O, base_cell * LOG2E_F, n, mc, Mc, T, j, g8, t_start, O_start};
     switch (p) {  // wave-uniform: every wave runs the sweep specialised for its node block
         case 0: fwd_sweep<R, TAB_LDS, 0>(A0, A1, sa); break;
         case 1: fwd_sweep<R, TAB_LDS, 1>(A0, A1, sa); break;
@@ -1108,7 +1183,7 @@ __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__re
     }
     __syncthreads();
     {
-        FwdSweepArgs sa{w0, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, nullptr, nullptr, nullptr, hd.slots, hd.D, hd.O, base_cell * LOG2E_F, n, mc, Mc, T, j, g8};
+        FwdSweepArgs sa{w0, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, nullptr, nullptr, nullptr, hd.slots, hd.D, hd.O, base_cell * LOG2E_F, n, mc, Mc, T, j, g8, n - 1, 0.0};
         switch (p) {
             case 0: fwd_sweep<R, true, 0>(A0, A1, sa); break;
             case 1: fwd_sweep<R, true, 1>(A0, A1, sa); break;
@@ -1233,6 +1308,9 @@ struct OutsideFreeArgs {
     float *sm_E;                   // [T+4] shifts
     double *sm_P;                  // [T+4] offsets
     int n, mc, T, j, g8, wave;
+    // first step: 1 or, taking over from a linear-domain sweep that ran out of range, a later one, whose weight columns
+    // are in w0, w1, with the betas of the column before it in sm_B and its shift and offset in sm_E, sm_P
+    int t_start;
 };
 
 template <int P>
@@ -1243,10 +1321,10 @@ __device__ __forceinline__ void outside_sweep_free(const float (&A0)[1][8], cons
     const int q_end = P + 1;  // chunks beyond hold only parents a > c
     const bool live = c_id < x.mc;
     const int ci = live ? c_id : 0;
-    float bprev = (c_id == 0) ? 0.f : NEG_INF_F;  // relative beta of column t-1 (beta[root][0] = 0)
-    float e_cur = 0.f;                             // E_t
-    double Pt = 0.0;                               // P_t
-    for (int t = 1; t <= x.n - 1; t++) {
+    float bprev = live ? x.sm_B[ci * TS + x.t_start - 1] : NEG_INF_F;  // relative beta of column t-1 (beta[root][0] = 0)
+    float e_cur = x.sm_E[x.t_start];                                   // E_t
+    double Pt = x.sm_P[x.t_start];                                     // P_t
+    for (int t = x.t_start; t <= x.n - 1; t++) {
         const float *c0 = x.w0 + (t & 1) * MP, *c1 = x.w1 + (t & 1) * MP;
         float *n0 = x.w0 + ((t + 1) & 1) * MP, *n1 = x.w1 + ((t + 1) & 1) * MP;
         float u0[NQ], u1[NQ];
@@ -1321,7 +1399,7 @@ struct OutsideLinArgs {
 // right of every node of the wave).  col0, col1: the weights W0_t, W1_t the parents offer (read at step t, written
 // for t+1); col2: the betas, for the table waves.  Returns false if a link is out of range.
 template <int W>
-__device__ __forceinline__ bool outside_sweep_lin(const LinLds &x, const OutsideLinArgs &g) {
+__device__ __forceinline__ bool outside_sweep_lin(const LinLds &x, const OutsideLinArgs &g, int &stopped_at) {
     constexpr int NB = W + 1, MP = 64;
     const int n = g.n, mc = g.mc, Mc = g.Mc, L = g.L, T = g.T;
     const int lane = threadIdx.x & 63, j = lane & 3, c_id = 16 * W + (lane >> 2);
@@ -1366,7 +1444,8 @@ __device__ __forceinline__ bool outside_sweep_lin(const LinLds &x, const Outside
     double bprev = (c_id == 0) ? 1.0 : 0.0;  // beta[root][0] = 0
     int e_cur = 0;
     double em_t = live ? x.em[ci * T + 1] : 0.0, el_p = live ? x.el[ci * T + 0] : 0.0;
-    for (int t = 1; t <= n - 1; t++) {
+    int stop = 0;  // as in the forward sweep: the loop ends behind the step that read a stop mark
+    for (int t = 1; t <= n - 1 && !stop; t++) {
         const double2 *c0 = reinterpret_cast<const double2 *>(x.col0 + (t & 1) * MP);
         const double2 *c1 = reinterpret_cast<const double2 *>(x.col1 + (t & 1) * MP);
         double2 u0[NB][2], u1[NB][2];
@@ -1377,7 +1456,8 @@ __device__ __forceinline__ bool outside_sweep_lin(const LinLds &x, const Outside
             u1[q][0] = c1[8 * q + 2 * j];
             u1[q][1] = c1[8 * q + 2 * j + 1];
         }
-        int e_next = x.kbuf[t];
+        const int2 ks = *reinterpret_cast<const int2 *>(x.kbuf + 2 * t);  // the step's shift and its stop mark
+        int e_next = ks.x;
 #pragma unroll
         for (int q = 0; q < NB; q++) {
             pin(u0[q][0]);
@@ -1386,6 +1466,8 @@ __device__ __forceinline__ bool outside_sweep_lin(const LinLds &x, const Outside
             pin(u1[q][1]);
         }
         pin(e_next);
+        stop = __builtin_amdgcn_readfirstlane(ks.y);
+        stopped_at = stop ? t : stopped_at;
         // what of the weights offered at the next two positions does not wait for this step's sum
         double emd = pow2_int(-e_next) * em_t;
         double nw1 = ((bprev * pow2_int(-(e_next + e_cur))) * el_p) * em_t;
@@ -1421,11 +1503,15 @@ __device__ __forceinline__ bool outside_sweep_lin(const LinLds &x, const Outside
     return ok != 0;
 }
 
-// The table waves of the outside sweep (role 0: betas, shifts and offsets; 1, 2: the two weights; 3: idle).  They stage the
-// emissions and the first columns, then follow one step behind the sweep: iteration t turns the betas of step t-1 and the
-// weight columns W0_t, W1_t into table entries; pass t = n after the last barrier finishes the job.  Returns the smallest
-// range key seen; ok: false if an emission is out of range.
-__device__ __forceinline__ unsigned outside_tables_lin(const LinLds &x, const OutsideLinArgs &g, int role, bool &ok) {
+// The table waves of the outside sweep (role 0: betas, shifts and offsets; 1, 2: the two weights; 3: the range watch).
+// They stage the emissions and the first columns, then follow one step behind the sweep: iteration t turns the betas of
+// step t-1 and the weight columns W0_t, W1_t into table entries; pass t = n after the last barrier finishes the job.
+// The watch looks at the same numbers - what step t reads - and marks step t+1 if one of them is below the range (the
+// results of step t then cannot be trusted): the sweep reads the mark with the shift at the top of that step and every
+// wave leaves its loop behind it.  Returns the smallest range key seen in what the sweep stands for; ok: false if an
+// emission is out of range.
+__device__ __forceinline__ unsigned outside_tables_lin(const LinLds &x, const OutsideLinArgs &g, int role, bool &ok, int lin_bits,
+                                                       int &stopped_at) {
     constexpr int MP = 64;
     const int n = g.n, mc = g.mc, Mc = g.Mc, T = g.T, TS = g.T + 2, TP = g.T + 4, ht = threadIdx.x - 256, node = threadIdx.x & 63;
     const bool live = node < mc;
@@ -1439,14 +1525,20 @@ __device__ __forceinline__ unsigned outside_tables_lin(const LinLds &x, const Ou
     for (int i = ht; i < TP; i += 256) {
         g.sm_E[i] = 0.f;
         g.sm_P[i] = 0.0;
-        x.kbuf[i] = 0;
+        x.kbuf[2 * i] = 0;
+        x.kbuf[2 * i + 1] = 0;
     }
     if (ht == 0) *x.flag = 0;
     __syncthreads();
     unsigned lowest = ~0u;
     int k_last = 0, k_before = 0;  // E_{t+1}, E_t at iteration t
     double P_run = 0.0;            // P[t+1] at iteration t
+    const unsigned too_small = range_key_of_bits(lin_bits);
     for (int t = 1; t <= n; t++) {
+        // the sweep stops behind step t if that step is marked; what this pass then makes of the columns of step t-1
+        // (computed from the numbers that stopped it) is overwritten by the sweep that takes over, and is not vouched for
+        const int mark = x.kbuf[2 * t + 1];
+        unsigned seen = lowest;
         if (role == 0) {
             const double v = x.col2[((t - 1) & 1) * MP + node];
             if (t + 1 <= n - 1) {
@@ -1455,7 +1547,7 @@ __device__ __forceinline__ unsigned outside_tables_lin(const LinLds &x, const Ou
                 const int e = wave_max_i(exponent_or_none(v));
                 const int k = e == NO_EXPONENT ? 0 : clamp_shift(e - k_last - k_before);
                 if (node == 0) {
-                    x.kbuf[t + 1] = k;
+                    x.kbuf[2 * (t + 1)] = k;
                     g.sm_E[t + 2] = (float)k;
                     P_run += (double)k;
                     g.sm_P[t + 2] = P_run;
@@ -1464,41 +1556,55 @@ __device__ __forceinline__ unsigned outside_tables_lin(const LinLds &x, const Ou
                 k_last = k;
             }
             if (live) g.sm_B[node * TS + t - 1] = log2_of(v);
-            lowest = min(lowest, range_key(v));
+            seen = min(lowest, range_key(v));
         } else if (role <= 2) {
             const double v = (role == 1 ? x.col0 : x.col1)[(t & 1) * MP + node];
             if (live) (role == 1 ? g.sm_W0 : g.sm_W1)[node * TS + t] = log2_of(v);
-            lowest = min(lowest, range_key(v));
+            seen = min(lowest, range_key(v));
+        } else if (t <= n - 1) {
+            const double bt = x.col2[((t - 1) & 1) * MP + node], u0 = x.col0[(t & 1) * MP + node], u1 = x.col1[(t & 1) * MP + node];
+            const bool below = min(range_key(bt), min(range_key(u0), range_key(u1))) < too_small;
+            if (__builtin_amdgcn_ballot_w64(below) != 0 && node == 0) x.kbuf[2 * (t + 1) + 1] = 1;
         }
         if (t <= n - 1) lds_barrier();
+        if (mark != 0) {
+            stopped_at = t;  // (n: marked while the last step ran; the sweep waves find that in the mark itself)
+            break;
+        }
+        lowest = seen;
     }
     return lowest;
 }
 
 // The outside sweep of a sentence in the linear domain: fills sm_B, sm_W0, sm_W1, sm_E, sm_P like the log-domain code of
-// inside_outside_ml1_body and returns true, or returns false (workgroup-uniform) with them in an undefined state.
+// inside_outside_ml1_body.  Returns (workgroup-uniform) 0 if the sweep is complete; t >= 1 if step t is the first it
+// cannot vouch for - sm_W0/sm_W1[.][..t], sm_B[.][..t-1], sm_E[..t], sm_P[..t] are in place and the log-domain sweep
+// takes over from there; -1 if nothing of it can be used (an input out of range).
 // `lin` is the extra LDS (lin_extra_bytes(Mc, T)).
-__device__ __forceinline__ bool inside_outside_lin_attempt(const float *__restrict__ mt, const float *__restrict__ lk, double *sm_P,
-                                                          float *sm_E, float *sm_B, float *sm_W0, float *sm_W1, double *lin, int m,
-                                                          int n, int L, int T, int Mc, int lin_bits) {
+__device__ __forceinline__ int inside_outside_lin_attempt(const float *__restrict__ mt, const float *__restrict__ lk, double *sm_P,
+                                                         float *sm_E, float *sm_B, float *sm_W0, float *sm_W1, double *lin, int m, int n,
+                                                         int L, int T, int Mc, int lin_bits) {
     const LinLds x(lin, Mc, T);
     const OutsideLinArgs g{mt, lk, sm_B, sm_W0, sm_W1, sm_E, sm_P, n, m / 2, Mc, L, T};
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     unsigned lowest = ~0u;
     bool ok;
+    int stopped_at = 0;  // the step in front of which the sweep stopped (every wave leaves its loop at the same one)
     switch (wave) {  // wave-uniform; every branch meets the same barriers
-        case 0: ok = outside_sweep_lin<0>(x, g); break;
-        case 1: ok = outside_sweep_lin<1>(x, g); break;
-        case 2: ok = outside_sweep_lin<2>(x, g); break;
-        case 3: ok = outside_sweep_lin<3>(x, g); break;
-        default: lowest = outside_tables_lin(x, g, wave - 4, ok); break;
+        case 0: ok = outside_sweep_lin<0>(x, g, stopped_at); break;
+        case 1: ok = outside_sweep_lin<1>(x, g, stopped_at); break;
+        case 2: ok = outside_sweep_lin<2>(x, g, stopped_at); break;
+        case 3: ok = outside_sweep_lin<3>(x, g, stopped_at); break;
+        default: lowest = outside_tables_lin(x, g, wave - 4, ok, lin_bits, stopped_at); break;
     }
-    if (!ok || lowest < range_key_of_bits(lin_bits)) *x.flag = 1;
+    if (!ok || lowest < range_key_of_bits(LIN_FLOOR_BITS)) *x.flag = 1;
     __syncthreads();
     const bool good = *x.flag == 0;
-    if (threadIdx.x == 0) atomicAdd(good ? &g_linear_swept : &g_linear_handed_over, 1ull);
+    // a number below the range among what the last step reads is met while that step runs: it is redone
+    const int resume_at = (stopped_at > 0 && stopped_at < n) ? stopped_at - 1 : (x.kbuf[2 * n + 1] != 0 ? n - 1 : 0);
+    if (threadIdx.x == 0) atomicAdd(good && resume_at == 0 ? &g_linear_swept : &g_linear_handed_over, 1ull);
     __syncthreads();
-    return good;
+    return good ? resume_at : -1;
 }
 
 // Dynamic LDS of the outside role: P [T+4] (double), slots [16], E [T+4], w0 [2][64], w1 [2][64], Bh, W0h, W1h [Mc][T+2],
@@ -1535,12 +1641,11 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
     AuxView av(aux, b, Mc, T);
 
     // the linear-domain sweep first, where the launch brought the LDS for it; what it cannot follow is swept below
-    bool swept = false;
-    if (lin_bits > 0)
-        swept = inside_outside_lin_attempt(mt, lk, sm_P, sm_E, sm_B, sm_W0, sm_W1,
-                                           reinterpret_cast<double *>(reinterpret_cast<char *>(smem_d) + align16(outside_role_bytes(Mc, T))),
-                                           m, n, L, T, Mc, lin_bits);
-    if (!swept) {
+    int resume_at = -1;  // 0: swept; t >= 1: the sweep below takes over at step t; -1: it starts from the root
+    double *lin = reinterpret_cast<double *>(reinterpret_cast<char *>(smem_d) + align16(outside_role_bytes(Mc, T)));
+    if (lin_bits > 0) resume_at = inside_outside_lin_attempt(mt, lk, sm_P, sm_E, sm_B, sm_W0, sm_W1, lin, m, n, L, T, Mc, lin_bits);
+    if (resume_at != 0) {
+    const int t_start = resume_at > 0 ? resume_at : 1;
     // transposed link slabs: this thread's group owns child c, its lanes the parents a <= c; unconditional loads
     const int own = 8 * p + g8;
     float A0[1][NQ], A1[1][NQ];
@@ -1553,6 +1658,18 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
             A1[0][q] = lk[(row + 1) * L + c];
         }
     }
+    if (resume_at > 0) {
+        // the weight columns of step t_start as the linear-domain sweep left them in the tables, the maximum of the beta
+        // column before them as the shift of the first step
+        lin_emissions_to_logs(LinLds(lin, Mc, T), sm_main, sm_leaf, Mc, T);
+        const int node = tid & 63;
+        const float col_max = wave_max(node < mc ? sm_B[node * TS + t_start - 1] : NEG_INF_F);
+        if (tid < MP) {
+            w0[(t_start & 1) * MP + tid] = tid < mc ? sm_W0[tid * TS + t_start] : NEG_INF_F;
+            w1[(t_start & 1) * MP + tid] = tid < mc ? sm_W1[tid * TS + t_start] : NEG_INF_F;
+        }
+        if (tid < 16) slots[tid] = col_max;
+    } else {
     for (int i = tid; i < Mc * T; i += NTR) {
         const int a_id = i / T, s = i - a_id * T;
         const float vm = mt[(size_t)(2 * a_id + 1) * T + s], vl = mt[(size_t)(2 * a_id) * T + s];
@@ -1574,6 +1691,7 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
         sm_P[i] = 0.0;
     }
     if (tid < 16) slots[tid] = (tid < 8) ? 0.f : NEG_INF_F;  // maximum of the relative beta column 0
+    }
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
         const int a_id = j + 8 * q;
@@ -1582,14 +1700,14 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
         A1[0][q] = (ok && a_id >= 1) ? to_b2(A1[0][q]) : NEG_INF_F;
     }
     __syncthreads();
-    if (tid == 0) {  // W_1 columns: the root offers match[root][0] to its null-left children
+    if (tid == 0 && resume_at < 0) {  // W_1 columns: the root offers match[root][0] to its null-left children
         const float w00 = sm_main[0];
         w0[1 * MP + 0] = w00;
         sm_W0[0 * TS + 1] = w00;
     }
     __syncthreads();
     {
-        OutsideFreeArgs sa{w0, w1, sm_B, sm_W0, sm_W1, sm_main, sm_leaf, slots, sm_E, sm_P, n, mc, T, j, g8, (tid >> 6)};
+        OutsideFreeArgs sa{w0, w1, sm_B, sm_W0, sm_W1, sm_main, sm_leaf, slots, sm_E, sm_P, n, mc, T, j, g8, (tid >> 6), t_start};
         switch (p) {  // wave-uniform
             case 0: outside_sweep_free<0>(A0, A1, sa); break;
             case 1: outside_sweep_free<1>(A0, A1, sa); break;

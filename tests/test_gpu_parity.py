@@ -448,6 +448,47 @@ def test_inside_linear_sweep_hands_over_what_it_cannot_follow():
             assert np.abs(got - want).max() <= 1e-4 * max(np.abs(want).max(), 1e-30), bi
 
 
+@pytest.mark.parametrize("wrong", [-16.0, -24.0, -32.0])
+def test_inside_linear_sweep_stops_and_log_domain_takes_over(wrong):
+    """Peaked emissions, as a trained model gives them: every token has one node that emits it with probability 0.8, all
+    other nodes are `wrong` nats down (every input inside the range the linear sweeps accept).  A node far from the
+    alignment then falls more than 2^-500 below its column's largest after some tokens: the linear-domain sweeps stop
+    there and the log-domain sweeps go on from that column with what is in the tables.  Loss, table and gradients against
+    the float64 oracle; the counters tell that sweeps were handed over, and since no input is out of range every one of
+    them was handed over on the way, not from the start."""
+    L, T = 128, 32
+    ms, ns = [128, 128, 96, 64, 40, 128], [32, 30, 25, 17, 11, 9]
+    batch = synth.training_batch(len(ms), L, T, 80, ms, ns, seed=41)
+    g = torch.Generator().manual_seed(int(-wrong))
+    match = wrong + 2.0 * torch.randn(len(ms), L, T, generator=g)
+    for b, (m, n) in enumerate(zip(ms, ns)):
+        for t in range(n):
+            a = 2 * int(round(t * (m // 2 - 1) / max(n - 1, 1))) + 1
+            match[b, min(a, m - 1), t] = -0.2
+    match = harness.eos_masked(match, batch["output_length"], batch["target_length"])
+    assert float(match[torch.isfinite(match)].min()) > -100.0
+    S64, C64, mg64, lg64 = _oracle_inside(batch, match.numpy())
+    ol, tl = batch["output_length"].to(DEV), batch["target_length"].to(DEV)
+    try:
+        ops.inside_linear_bits(500)
+        ops.inside_linear_counts(reset=True)
+        ll, mg, lg = _inside_all(batch, match)
+        S = ops._pcfg_loss_tables(match.to(DEV), batch["links"].to(DEV), ol, tl, 1, "test")[0].cpu().double().numpy()
+        swept, handed = ops.inside_linear_counts()
+    finally:
+        ops.inside_linear_bits()
+    assert swept + handed == 3 * len(ms) and handed >= 1, (swept, handed)
+    print("emissions %.0f nats down: %d sweeps complete in the linear domain, %d taken over" % (wrong, swept, handed))
+    assert np.array_equal(np.isneginf(S), np.isneginf(S64))
+    fin = np.isfinite(S64)
+    assert np.allclose(S[fin], S64[fin], rtol=2e-6, atol=1e-4)
+    assert np.allclose(ll.double().numpy(), S64[:, 0, 0], rtol=1e-5)
+    w = torch.linspace(0.5, 1.5, len(ms)).double().numpy()
+    for bi in range(len(ms)):
+        for got, want in ((mg[bi].double().numpy(), mg64[bi] * w[bi]), (lg[bi].double().numpy(), lg64[bi] * w[bi])):
+            assert np.abs(got - want).max() <= 1e-4 * max(np.abs(want).max(), 1e-30), bi
+
+
 @pytest.mark.parametrize("L,T,ms,ns", [(128, 30, [128, 90], [30, 22]), (320, 40, [320, 262], [40, 31]), (600, 24, [600, 520], [24, 24])])
 def test_inside_spiky_inputs_vs_oracle(L, T, ms, ns):
     """Emissions and links with jumps of hundreds of units and scattered -inf entries: neighbouring columns of the tables
