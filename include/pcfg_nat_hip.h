@@ -195,8 +195,10 @@ void pcfgnat_links_grad_range_limit(float log2_limit);
  * No counterpart in the reference: with bits > 0, graphs of up to 130 nodes are swept in the linear domain (probabilities
  * in double, one multiply-add per term) where the numbers allow it - links and emissions between 2^-150 and 2^8 or zero,
  * every intermediate at least 2^-bits or exactly zero - and in the log domain, which has no range limit, otherwise; the
- * choice is made per sentence and per sweep by the kernel, at the end of the linear sweep.  Pays where emissions are not
- * peaked (a third off the sweeps' time), costs where a model is sure of itself (a sentence handed over is swept twice).
+ * choice is made per sentence and per sweep by the kernel: an input out of range sends the whole sweep to the log domain,
+ * a number below the range on the way stops the linear sweep there and the log-domain sweep goes on from that column.
+ * Pays where emissions are not peaked (a fifth off the sweeps' time), costs where a model is sure of itself (up to a
+ * tenth more when a sentence leaves the range in its first columns).
  * bits: at most 500; 0, the default, switches the linear sweeps off.  Process-wide.
  */
 void pcfgnat_inside_linear_bits(int bits);
@@ -204,7 +206,7 @@ void pcfgnat_inside_linear_bits(int bits);
 /*
  * No counterpart in the reference: diagnostic counters since the library was loaded (or the last reset) on the current
  * device - sweeps (forward and outside sweeps count apart) completed in the linear domain, and sweeps the linear
- * domain handed over to the log domain.  Synchronises with the device.
+ * domain handed over to the log domain, from the start or on the way.  Synchronises with the device.
  */
 int pcfgnat_inside_linear_counts(unsigned long long *swept, unsigned long long *handed_over, int reset);
 

@@ -63,12 +63,13 @@ def pipeline_redo_counts(reset=False):
 
 def inside_linear_bits(bits=0):
     """Process-wide setting: the smallest nonzero number, as a power of two, that the linear-domain sweeps of graphs of up to
-    130 nodes accept before they hand a sentence to the log-domain sweep (at most 500); 0, the default, switches them off."""
+    130 nodes accept before the log-domain sweep takes the sentence over at that column (at most 500); 0, the default, switches
+    them off."""
     _lib.load().pcfgnat_inside_linear_bits(int(bits))
 
 
 def inside_linear_counts(reset=False):
-    """(sweeps completed in the linear domain, sweeps handed over to the log domain) on the current device since the
+    """(sweeps completed in the linear domain, sweeps handed over to the log domain from the start or on the way) on the current device since the
     library was loaded or the last reset; forward and outside sweeps count apart.  Synchronises with the device."""
     import ctypes
     lib = _lib.load()
