@@ -350,11 +350,13 @@ def main():
     roof = ROOFLINE_KERNEL[mode]
 
     sampled = {"step": 0}
+    pool = []
 
     def mark(name, phase):
         if name == "events":  # single-call step: the library records the events we hand out around its kernels
-            # Inside the timed region the roofline kernel is bracketed in every fourth step only: a pair of timing events
-            # holds up the queue by about 20 us, a tenth of the step.
+            # Inside the timed region the roofline kernel is bracketed in every fifth step only: a pair of timing events
+            # holds up the queue by about 20 us, a tenth of the step.  The events of the region are created and
+            # materialised ahead of it (the pool), so that the region holds only the two records around the kernel.
             sampled["step"] += 1
             if not detail["on"] and (sampled["step"] - 1) % EVENT_EVERY != 0:
                 return None
@@ -364,8 +366,11 @@ def main():
                     if kernel != roof and not detail["on"]:
                         evs.append(None)
                         continue
-                    ev = torch.cuda.Event(enable_timing=True)
-                    ev.record()  # materialises the HIP event; the library records it again at the right place
+                    if pool:
+                        ev = pool.pop()
+                    else:
+                        ev = torch.cuda.Event(enable_timing=True)
+                        ev.record()  # materialises the HIP event; the library records it again at the right place
                     pairs.setdefault(kernel, []).append(ev)
                     evs.append(ev)
             return evs
@@ -385,6 +390,11 @@ def main():
     losses = []
     for i in range(args.warmup):
         losses.append(step_fn(bufs[i], targets, links, ol, tl)[0])
+    if mode == "single":
+        for _ in range(2 * ((args.steps + EVENT_EVERY - 1) // EVENT_EVERY)):
+            ev = torch.cuda.Event(enable_timing=True)
+            ev.record()
+            pool.append(ev)
     torch.cuda.synchronize()
     sampled["step"] = 0
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
