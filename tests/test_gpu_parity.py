@@ -489,6 +489,50 @@ def test_inside_linear_sweep_stops_and_log_domain_takes_over(wrong):
             assert np.abs(got - want).max() <= 1e-4 * max(np.abs(want).max(), 1e-30), bi
 
 
+@pytest.mark.parametrize("n,width,bits", [(16, 4, 500), (16, 6, 500), (16, 1, 100), (5, 1, 100), (4, 1, 100), (3, 1, 100), (2, 1, 100)])
+def test_inside_linear_sweep_stops_at_every_column(n, width, bits):
+    """One sentence per column p: `width` consecutive tokens from p on are emitted with probability e^-95 by every node but
+    one (inputs still inside the range the linear sweeps accept), so the spread of the columns grows by 137 bits a token
+    there and passes 2^bits at a column that moves with p - from the first step of either sweep to its last, where the
+    number below the range is only met while the last step runs; sentences of two to five tokens with a range of 100 bits
+    put every such case next to the ends of the sweeps.  Everything against the float64 oracle."""
+    L, T = 64, 16
+    cases = list(range(0, max(n - width, 0) + 1))
+    ms, ns = [64 - 2 * (p % 3) for p in cases], [n] * len(cases)
+    batch = synth.training_batch(len(cases), L, T, 80, ms, ns, seed=5 * n + width)
+    g = torch.Generator().manual_seed(n + width)
+    match = -3.0 + torch.randn(len(cases), L, T, generator=g)
+    for b, (p0, m) in enumerate(zip(cases, ms)):
+        for t in range(p0, min(p0 + width, n)):
+            a = 2 * int(round(t * (m // 2 - 1) / max(n - 1, 1))) + 1
+            keep = match[b, min(a, m - 1), t].clone()
+            match[b, :, t] -= 95.0
+            match[b, min(a, m - 1), t] = keep
+    match = harness.eos_masked(match, batch["output_length"], batch["target_length"])
+    assert float(match[torch.isfinite(match)].min()) > -103.0
+    S64, C64, mg64, lg64 = _oracle_inside(batch, match.numpy())
+    ol, tl = batch["output_length"].to(DEV), batch["target_length"].to(DEV)
+    try:
+        ops.inside_linear_bits(bits)
+        ops.inside_linear_counts(reset=True)
+        ll, mg, lg = _inside_all(batch, match)
+        S = ops._pcfg_loss_tables(match.to(DEV), batch["links"].to(DEV), ol, tl, 1, "test")[0].cpu().double().numpy()
+        swept, handed = ops.inside_linear_counts()
+    finally:
+        ops.inside_linear_bits()
+    assert swept + handed == 3 * len(cases), (swept, handed)
+    print("n %d, range 2^-%d, %d tokens 95 nats down from column p, p = 0..%d: %d sweeps complete in the linear domain, %d taken over"
+          % (n, bits, width, cases[-1], swept, handed))
+    assert np.array_equal(np.isneginf(S), np.isneginf(S64))
+    fin = np.isfinite(S64)
+    assert np.allclose(S[fin], S64[fin], rtol=2e-6, atol=1e-4)
+    assert np.allclose(ll.double().numpy(), S64[:, 0, 0], rtol=1e-5)
+    w = torch.linspace(0.5, 1.5, len(cases)).double().numpy() if len(cases) > 1 else np.array([0.5])
+    for bi in range(len(cases)):
+        for got, want in ((mg[bi].double().numpy(), mg64[bi] * w[bi]), (lg[bi].double().numpy(), lg64[bi] * w[bi])):
+            assert np.abs(got - want).max() <= 1e-4 * max(np.abs(want).max(), 1e-30), bi
+
+
 @pytest.mark.parametrize("L,T,ms,ns", [(128, 30, [128, 90], [30, 22]), (320, 40, [320, 262], [40, 31]), (600, 24, [600, 520], [24, 24])])
 def test_inside_spiky_inputs_vs_oracle(L, T, ms, ns):
     """Emissions and links with jumps of hundreds of units and scattered -inf entries: neighbouring columns of the tables
