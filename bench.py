@@ -86,76 +86,156 @@ def _percentile(sorted_vals, q):
     return sorted_vals[min(len(sorted_vals) - 1, int(q * len(sorted_vals)))]
 
 
-def decode_timing(dev, n_b1=256):
-    """Viterbi decode of the inference configuration (BASELINE config 4: src ~U[5,100], L = 4*src, V=40000, fp16 logits
-    ~N(0,3)) as the model runs it: front-end (log-softmax + max over the vocabulary, one read of the logits) followed by
-    tables + length selection + readout, all enqueued by one native call; the emitted token counts are read back by the
-    host, which is the decode's one synchronisation.  Batch 1: wall-clock latency per sentence over the first ``n_b1`` sentences
-    of the configuration (median, 95th percentile, mean; front-end and decode also timed apart).  Batch 64: throughput
-    over ten chunks of length-sorted sentences."""
+def cpu_model_string():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _cpu_viterbi_decode(ob, tok, links, m, mask):
+    """The oracle's Viterbi decode of one batch on the host (pcfg_viterbi.cu:22-140 and pcfg_loss.cpp:12-73 restated in C,
+    OpenMP over the sentences; the length selection of glat_decomposed_with_link_two_hands_tri_pcfg.py:489-497 in numpy).
+    Returns (seconds, tokens float32 [B,maxlen], pred_length [B])."""
+    import numpy as np
+    from oracle import oracle
+    from pcfg_nat_amd import synth
+
+    t0 = time.perf_counter()
+    S, R, Lt, M = oracle.viterbi(ob, links, m, dtype=np.float32)
+    Lq = S.shape[2]
+    with np.errstate(divide="ignore", invalid="ignore"):
+        sc = S[:, 1, :] / np.arange(Lq, dtype=np.float32)[None, :]
+    sc = np.where(np.isnan(sc), -np.inf, sc)
+    pred = sc[:, 1:].argmax(-1) + 1
+    out = oracle.viterbi_decoding(pred, m, Lt, R, M, tok, mask, synth.PAD)
+    return time.perf_counter() - t0, out, pred
+
+
+def decode_timing(dev, cpu=True, front_end_sample=16):
+    """Viterbi decode of the inference configuration (BASELINE config 4: 1000 sentences, src ~U[5,100], L = 4*src, V=40000,
+    fp16 logits ~N(0,3)) as the model runs it: front-end (log-softmax + max over the vocabulary, one read of the logits)
+    followed by tables + length selection + readout, all enqueued by one native call; the emitted token counts are read back
+    by the host, which is the decode's one synchronisation.  Batch 1: wall-clock latency of every one of the 1000 sentences
+    (median, 95th percentile, mean; front-end and decode also timed apart).  Batch 64: throughput over all 16 length-sorted
+    batches of the same 1000 sentences (15 of 64 and one of 40).  With ``cpu`` the same sentences are decoded by the oracle
+    on the host cores from the node scores the GPU front-end produced (batch 1: one sentence, hence one core, at a time;
+    batch 64: OpenMP over the sentences), the front-end by torch's CPU ``log_softmax`` + ``max`` on a strided sample of
+    ``front_end_sample`` sentences; the tokens of both paths are compared."""
+    import numpy as np
     import torch
     from pcfg_nat_amd import custom_ops as ops, harness, synth
 
     V = 40000
     lens = synth.config4_lengths()
-    out = {}
+    n_sent = len(lens)
+    out = {"sentences": n_sent,
+           "src_length_histogram": {"%d-%d" % (lo, lo + 19): int(((lens >= lo) & (lens < lo + 20)).sum()) for lo in range(5, 101, 20)}}
     gen = torch.Generator().manual_seed(3)
     ggen = torch.Generator(device=dev).manual_seed(4)
 
     def make(src):
         m = 4 * src
         L = int(m.max())
-        links = synth.make_links(len(src), L, m, 1, gen).to(dev)
+        links = synth.make_links(len(src), L, m, 1, gen)
         logits = (torch.randn(len(src), L, V, device=dev, dtype=torch.float32, generator=ggen) * 3).half()
-        mask = synth.support_masks(L, 1)[0].to(dev)
-        return logits, links, m.to(dev), mask
+        mask = synth.support_masks(L, 1)[0]
+        return {"logits": logits, "links": links.to(dev), "m": m.to(dev), "mask": mask.to(dev),
+                "links_cpu": links.numpy() if cpu else None, "m_cpu": m.numpy(), "mask_cpu": mask.numpy()}
 
-    def run(case):
-        logits, links, m, mask = case
-        return harness.decode_from_logits(logits, links, m, mask, single_call=True)
+    def run(c):
+        return harness.decode_from_logits(c["logits"], c["links"], c["m"], c["mask"], single_call=True)
 
     def wall(fn):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        fn()
+        res = fn()
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3
+        return (time.perf_counter() - t0) * 1e3, res
+
+    def cpu_front_end(cases):
+        """torch on the host cores: log_softmax over the vocabulary and max, per sampled sentence; ms per graph node."""
+        ms = nodes = 0
+        for c in cases:
+            x = c["logits"].cpu()
+            t0 = time.perf_counter()
+            torch.log_softmax(x.float(), dim=-1).max(dim=-1)
+            ms += (time.perf_counter() - t0) * 1e3
+            nodes += x.shape[0] * x.shape[1]
+        return ms / nodes
 
     try:
-        sample = lens[:n_b1]
-        cases = [make(sample[i:i + 1]) for i in range(len(sample))]
+        cases = [make(lens[i:i + 1]) for i in range(n_sent)]
         for c in cases:  # one untimed pass: every kernel variant the lengths select has been loaded once
             run(c)
-        total = sorted(wall(lambda c=c: run(c)) for c in cases)
-        front = sorted(wall(lambda c=c: ops.logsoftmax_max(c[0])) for c in cases)
-        pre = [ops.logsoftmax_max(c[0]) for c in cases]
-        dec = sorted(wall(lambda c=c, o=o: harness.viterbi_decode(o[0], o[1], c[1], c[2], c[3], single_call=True))
+        timed = [wall(lambda c=c: run(c)) for c in cases]
+        total = sorted(t for t, _ in timed)
+        front = sorted(wall(lambda c=c: ops.logsoftmax_max(c["logits"]))[0] for c in cases)
+        pre = [ops.logsoftmax_max(c["logits"]) for c in cases]
+        dec = sorted(wall(lambda c=c, o=o: harness.viterbi_decode(o[0], o[1], c["links"], c["m"], c["mask"], single_call=True))[0]
                      for c, o in zip(cases, pre))
         out["b1"] = {"sentences": len(cases),
                      "ms_per_sentence_p50": _percentile(total, 0.5), "ms_per_sentence_p95": _percentile(total, 0.95),
                      "ms_per_sentence_mean": sum(total) / len(total),
                      "front_end_ms_p50": _percentile(front, 0.5), "front_end_ms_p95": _percentile(front, 0.95),
-                     "decode_ms_p50": _percentile(dec, 0.5), "decode_ms_p95": _percentile(dec, 0.95)}
+                     "decode_ms_p50": _percentile(dec, 0.5), "decode_ms_p95": _percentile(dec, 0.95),
+                     "decode_ms_mean": sum(dec) / len(dec)}
         out["b1_ms_per_sentence"] = out["b1"]["ms_per_sentence_p50"]
-        del cases, pre
-        # batch 64: sorted by length
+        out["host_polling_still_on"] = bool(ops._pinned_counts.polling_on())
+        if cpu:
+            from oracle import oracle
+            per, same = [], True
+            for c, o, (_, got) in zip(cases, pre, timed):
+                sec, want, want_len = _cpu_viterbi_decode(o[0].cpu().numpy(), o[1].cpu().numpy(), c["links_cpu"], c["m_cpu"], c["mask_cpu"])
+                per.append(sec * 1e3)
+                same = same and np.array_equal(got[0].cpu().numpy(), want) and np.array_equal(got[1].cpu().numpy(), want_len)
+            per.sort()
+            fe = cpu_front_end(cases[::max(1, n_sent // front_end_sample)][:front_end_sample])
+            mean_nodes = float(4 * lens.double().mean())
+            out["cpu_b1"] = {"kind": "port", "cores": 1, "threads_available": oracle.num_threads(), "sentences": len(per),
+                             "decode_ms_p50": _percentile(per, 0.5), "decode_ms_p95": _percentile(per, 0.95),
+                             "decode_ms_mean": sum(per) / len(per),
+                             "front_end_ms_per_node": fe, "front_end_ms_mean_sentence": fe * mean_nodes,
+                             "front_end_sample": "%d sentences, every %d-th of the 1000, torch CPU log_softmax(float32) + max on %d threads"
+                                                 % (front_end_sample, max(1, n_sent // front_end_sample), torch.get_num_threads()),
+                             "ms_per_sentence_mean": sum(per) / len(per) + fe * mean_nodes,
+                             "tokens_equal_gpu": bool(same)}
+        del cases, pre, timed
+        # batch 64: all sentences, sorted by length
         srt = torch.sort(lens)[0]
-        chunks = [make(srt[i:i + 64]) for i in range(0, 640, 64)]
+        chunks = [make(srt[i:i + 64]) for i in range(0, n_sent, 64)]
         for c in chunks:  # untimed pass, as above
             run(c)
-        t_all = wall(lambda: [run(c) for c in chunks])
-        pre = [ops.logsoftmax_max(c[0]) for c in chunks]
-        t_dec = wall(lambda: [harness.viterbi_decode(o[0], o[1], c[1], c[2], c[3], single_call=True) for c, o in zip(chunks, pre)])
-        out["b64_sentences_per_s"] = 640 / (t_all * 1e-3)
-        out["b64_decode_only_sentences_per_s"] = 640 / (t_dec * 1e-3)
+        t_all, got = wall(lambda: [run(c) for c in chunks])
+        pre = [ops.logsoftmax_max(c["logits"]) for c in chunks]
+        t_dec, _ = wall(lambda: [harness.viterbi_decode(o[0], o[1], c["links"], c["m"], c["mask"], single_call=True) for c, o in zip(chunks, pre)])
+        out["b64_batches"] = len(chunks)
+        out["b64_sentences_per_s"] = n_sent / (t_all * 1e-3)
+        out["b64_decode_only_sentences_per_s"] = n_sent / (t_dec * 1e-3)
+        if cpu:
+            sec, same = 0.0, True
+            for c, o, g in zip(chunks, pre, got):
+                s1, want, want_len = _cpu_viterbi_decode(o[0].cpu().numpy(), o[1].cpu().numpy(), c["links_cpu"], c["m_cpu"], c["mask_cpu"])
+                sec += s1
+                same = same and np.array_equal(g[0].cpu().numpy(), want) and np.array_equal(g[1].cpu().numpy(), want_len)
+            nodes = float(sum(c["logits"].shape[0] * c["logits"].shape[1] for c in chunks))
+            out["cpu_b64"] = {"kind": "port", "cores": oracle.num_threads(), "decode_only_sentences_per_s": n_sent / sec,
+                              "sentences_per_s_with_front_end": n_sent / (sec + out["cpu_b1"]["front_end_ms_per_node"] * nodes * 1e-3),
+                              "tokens_equal_gpu": bool(same)}
     except RuntimeError as e:  # a shape the library does not build yet
         out["error"] = str(e)[:200]
     return out
 
 
-def glat_timing(logits, targets, links, out_len):
+def glat_timing(logits, targets, links, out_len, cpu=None):
     """The GLAT alignment pass that precedes the loss in every training step (nat_pcfg_loss.py:193-269) on the same
-    batch, as one native call: gather + eos mask + arg max, inside forward, best tree, glancing glue."""
+    batch, as one native call: gather + eos mask + arg max, inside forward, best tree, glancing glue.  ``cpu``: the CPU
+    copies of (targets, links, output_length, target_length); the same pass is then also timed over the oracle on the host
+    cores (torch CPU arg max, the oracle's gather, inside forward and best tree, the criterion's glue as torch CPU ops)."""
     import torch
     from pcfg_nat_amd import harness, synth
 
@@ -172,16 +252,51 @@ def glat_timing(logits, targets, links, out_len):
         harness.glat_alignment(logits, targets, prev, links, 0.5, single_call=True)
     end.record()
     torch.cuda.synchronize()
-    return {"ms_per_call": start.elapsed_time(end) / reps}
+    res = {"ms_per_call": start.elapsed_time(end) / reps}
+    if cpu is not None:
+        import numpy as np
+        from oracle import oracle
+
+        tg, lk, ol, tl = cpu
+        x = logits.cpu()
+        prev_c = prev.cpu()
+
+        class OracleOps:  # the two operators of the pass over the oracle, float32
+            @staticmethod
+            def dag_logsoftmax_gather_inplace(word_ins_out, select_idx):
+                sel, _ = oracle.lsg_fwd(word_ins_out.numpy(), select_idx.numpy(), want_probs=False, dtype=np.float32)
+                return word_ins_out, torch.from_numpy(sel)
+
+            @staticmethod
+            def cuda_pcfg_best_tree(match_all, links, output_length, target_length):
+                m, k, o, t = match_all.numpy(), links.numpy(), output_length.numpy(), target_length.numpy()
+                S, C = oracle.inside_fwd(m, k, o, t, dtype=np.float32)
+                tree = oracle.best_tree(S, C, m, k, o, t, dtype=np.float32)
+                return torch.from_numpy(tree), torch.from_numpy(S[:, 0, 0].copy())
+
+        times = []
+        for _ in range(4):
+            t0 = time.perf_counter()
+            harness.glat_alignment(x.float(), tg, prev_c, lk, 0.5, ops=OracleOps)
+            times.append(time.perf_counter() - t0)
+        best = sorted(times[1:])[1]
+        res["cpu"] = {"kind": "port", "cores": oracle.num_threads(), "ms_per_call": best * 1e3,
+                      "sample": "the same batch of %d sentences, float32 oracle + torch CPU glue, median of 3 runs after one warm-up" % B}
+        res["speedup_vs_cpu"] = best * 1e3 / res["ms_per_call"]
+    return res
 
 
 def operator_api_timing(bufs, targets, links, ol, tl, args, timed_windows, host_enqueue_ms):
     """One training pass through the five drop-in names, driven by the criterion's own code under autograd
     (``harness.compute_pcfg_loss`` restates nat_pcfg_loss.py:98-145 call for call) and ``loss.backward()``; with a loss
     scale of 128 on top, as under ``--fp16``.  The logits reach the criterion as the non-leaf output of an upstream layer,
-    which is played by a Function that hands out its buffer and swallows the gradient (no extra pass over the logits)."""
+    which is played by a Function that hands out its buffer and swallows the gradient (no extra pass over the logits).
+
+    The host's share is split three ways: the whole step; the two operators alone under autograd, fed with precomputed
+    tensors in place of the criterion's glue (their wrappers, the autograd bookkeeping and the kernels); the four native
+    calls behind them issued from Python without autograd."""
     import torch
-    from pcfg_nat_amd import harness, synth
+    from pcfg_nat_amd import custom_ops as ops, harness, synth
 
     class UpstreamLayer(torch.autograd.Function):
         @staticmethod
@@ -214,6 +329,69 @@ def operator_api_timing(bufs, targets, links, ol, tl, args, timed_windows, host_
     # These figures are bound by the host: the criterion's glue is some forty small torch kernels per step, and the host
     # takes as long to enqueue a step as the step takes on the wall clock.
     res["host_enqueue_ms_per_step"] = host_enqueue_ms(lambda i: step(i, 128.0))
+
+    # the two operators alone, under autograd, the glue replaced by tensors computed once
+    idx = targets.unsqueeze(1).expand(-1, L, -1)
+    with torch.no_grad():
+        _, m0 = ops.dag_logsoftmax_gather_inplace(bufs[0].clone(), idx)
+        match_pre = harness.eos_masked(m0, ol, tl)
+        w_pre = (-1.0 / (tl * B)).float() * 128.0
+        g_pre = torch.zeros_like(match_pre)
+
+    def operators_only(i):
+        lk = links.detach().requires_grad_(True)
+        ma = match_pre.detach().requires_grad_(True)
+        _, sel = ops.dag_logsoftmax_gather_inplace(UpstreamLayer.apply(weight, bufs[i]), idx)
+        ll = ops.cuda_pcfg_loss(ma, lk, ol, tl)
+        ll.backward(w_pre)
+        sel.backward(g_pre)
+
+    for i in range(args.warmup):
+        operators_only(i)
+    res["operators_only_host_enqueue_ms_per_step"] = host_enqueue_ms(operators_only)
+    res["operators_only_ms_per_step_median"] = timed_windows(operators_only, windows=3)["ms_per_step_median"]
+
+    def native_calls_only(i):
+        harness.train_step_fused(bufs[i], targets, links, ol, tl)
+
+    for i in range(args.warmup):
+        native_calls_only(i)
+    res["four_native_calls_host_enqueue_ms_per_step"] = host_enqueue_ms(native_calls_only)
+    res["glue_host_enqueue_ms_per_step"] = res["host_enqueue_ms_per_step"] - res["operators_only_host_enqueue_ms_per_step"]
+    return res
+
+
+def criterion_autograd_timing(bufs, targets, links, ol, tl, args, timed_windows, host_enqueue_ms):
+    """The single call as a trainer adopts it: ``custom_ops.pcfg_criterion`` under autograd (one native call in the forward,
+    one in the backward) followed by ``(loss * 128).backward()``, the logits arriving as the output of an upstream layer."""
+    import torch
+    from pcfg_nat_amd import custom_ops as ops
+
+    class UpstreamLayer(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, weight, buf):
+            out = buf.new_empty(0)
+            out.set_(buf.untyped_storage(), buf.storage_offset(), buf.shape, buf.stride())
+            return out
+
+        @staticmethod
+        def backward(ctx, grad):
+            return None, None
+
+    B = bufs[0].shape[0]
+    weight = torch.ones(1, device=bufs[0].device, requires_grad=True)
+
+    def step(i):
+        lk = links.detach().requires_grad_(True)
+        loss, _, _ = ops.pcfg_criterion(UpstreamLayer.apply(weight, bufs[i]), targets, lk, ol, tl)
+        (loss * 128.0).backward()
+
+    for i in range(args.warmup):
+        step(i)
+    res = timed_windows(step)
+    res["sentences_per_s_median"] = B / (res["ms_per_step_median"] * 1e-3)
+    res["host_enqueue_ms_per_step"] = host_enqueue_ms(step)
+    res["loss_scale"] = 128.0
     return res
 
 
@@ -524,17 +702,32 @@ def main():
         result["single_call_linear_sweeps"] = lin
     # the drop-in path: the unchanged criterion code over the operator API under autograd (dag_logsoftmax_gather_inplace ->
     # eos mask -> cuda_pcfg_loss -> loss -> backward), which reads and rewrites every row (it is not told the lengths)
+    result["criterion_autograd"] = criterion_autograd_timing(bufs, targets, links, ol, tl, args, timed_windows, host_enqueue_ms)
     result["operator_api"] = operator_api_timing(bufs, targets, links, ol, tl, args, timed_windows, host_enqueue_ms)
+    cpu = not args.no_cpu_baseline
     if not args.no_decode:
-        result["viterbi"] = decode_timing(dev)
-        result["glat_alignment"] = glat_timing(torch.randn(B, L, V, device=dev, generator=ggen).mul_(2).half(), targets, links, ol)
+        result["viterbi"] = decode_timing(dev, cpu=cpu)
+        result["glat_alignment"] = glat_timing(torch.randn(B, L, V, device=dev, generator=ggen).mul_(2).half(), targets, links, ol,
+                                               cpu=(targets_cpu, links_cpu, m, n) if cpu else None)
         result["long_sentences"] = long_sentence_timing(dev)
         result["link_scorer"] = link_scorer_timing(dev)
         result["decode_front_end"] = decode_front_end_timing(dev)
     if not args.no_cpu_baseline:
         batch_cpu = {"output_length": m, "target_length": n, "links": links_cpu, "targets": targets_cpu}
         result["cpu_baseline"] = cpu_baseline(batch_cpu, sample_logits, args.cpu_sentences)
+        result["cpu_baseline"]["cpu_model"] = cpu_model_string()
+        result["cpu_baseline"]["host_cpus"] = os.cpu_count()
         result["speedup_vs_cpu"] = result["value"] / result["cpu_baseline"]["value"]
+        if "viterbi" in result and "cpu_b1" in result["viterbi"]:  # the second half of the metric, beside its CPU figures
+            vit = result["viterbi"]
+            result["cpu_baseline"]["viterbi"] = {
+                "b1_ms_per_sentence": vit["cpu_b1"]["ms_per_sentence_mean"], "b1_decode_only_ms_per_sentence": vit["cpu_b1"]["decode_ms_mean"],
+                "b1_cores": vit["cpu_b1"]["cores"], "b64_sentences_per_s": vit["cpu_b64"]["sentences_per_s_with_front_end"],
+                "b64_decode_only_sentences_per_s": vit["cpu_b64"]["decode_only_sentences_per_s"], "b64_cores": vit["cpu_b64"]["cores"],
+                "kind": "port", "sample": "all 1000 sentences of the inference configuration (the front-end on a strided sample of 16)",
+                "gpu_b1_ms_per_sentence_mean": vit["b1"]["ms_per_sentence_mean"], "gpu_b64_sentences_per_s": vit["b64_sentences_per_s"]}
+        if "glat_alignment" in result and "cpu" in result["glat_alignment"]:
+            result["cpu_baseline"]["glat_alignment_ms_per_call"] = result["glat_alignment"]["cpu"]["ms_per_call"]
     print(json.dumps(result))
 
 

@@ -9,8 +9,8 @@ contract; the arithmetic runs in hand-written HIP kernels for gfx950 reached thr
 ``viterbi_decoding``, whose reference version is itself a host loop) raises.
 """
 import ctypes
-import os
 import threading
+import time
 import weakref
 
 import torch
@@ -522,12 +522,12 @@ def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unre
             scratch = torch.empty((B, 2 * L), dtype=torch.int64, device=dev)
             cnt = _pinned_counts.take(B)  # written by the kernel, read after the one stream wait
             try:
-                _pinned_counts.arm(cnt, B)
+                armed = _pinned_counts.arm(cnt, B, torch.cuda.current_stream(dev))
                 _lib.check(lib.pcfgnat_viterbi_decoding(pl.data_ptr(), ol.data_ptr(), Lt.data_ptr(), Rt.data_ptr(), Mt.data_ptr(),
                                                         tok.data_ptr(), mask.data_ptr(), mask.size(0), int(pad_index),
                                                         out.data_ptr(), cnt.data_ptr(), scratch.data_ptr(), B, L, Lq,
                                                         _stream(out)), lib)
-                _pinned_counts.wait(cnt, B, torch.cuda.current_stream(dev))
+                _pinned_counts.wait(cnt, B, torch.cuda.current_stream(dev), armed)
                 counts = cnt[:B].tolist()
             finally:
                 _pinned_counts.give_back(cnt)
@@ -774,6 +774,8 @@ class _PinnedCounts:
     def __init__(self):
         self._lock = threading.Lock()
         self._free = []
+        self._polling = True
+        self._misses = 0
 
     def take(self, n):
         with self._lock:
@@ -789,28 +791,43 @@ class _PinnedCounts:
     # The kernels write a sentence's count (>= -1) as the last thing they do for it.  Instead of waiting for the stream,
     # whose wake-up costs the host some microseconds after the kernel has ended, the caller marks the entries before the
     # launch and watches them turn: device stores to pinned host memory reach the host while the kernel is still running.
-    # Where they do not (a host-memory mode in which they only arrive with the end of the kernel), the watch runs into
-    # its bound once, the stream wait takes over and the watching is switched off for the rest of the process.
+    # The watch is for the latency-bound case only - a decode enqueued on an idle stream: with work already pending on the
+    # stream (``stream.query()`` false before the launch) the call goes straight to the stream wait.  A watch is bounded by
+    # time; one that runs into its bound hands over to the stream wait for that call, and only after several such misses
+    # in a row (a host-memory mode in which the stores only arrive with the end of the kernel) is the watching switched off.
     NOT_YET = -2
-    SPIN_LIMIT = 200000  # reads of an entry that has not turned: some tens of milliseconds
-    polling = os.environ.get("PCFGNAT_DECODE_POLL", "1") != "0"
+    WATCH_SECONDS = 0.005       # longest a call watches before it waits for the stream instead
+    MISSES_TO_SWITCH_OFF = 8    # consecutive watches that ran into the bound
 
-    def arm(self, buf, n):
-        if self.polling:
-            buf[:n].fill_(self.NOT_YET)
+    def polling_on(self):
+        return self._polling
 
-    def wait(self, buf, n, stream):
-        if self.polling:
+    def arm(self, buf, n, stream):
+        """Marks the entries and returns True if this call is going to watch them."""
+        if not self._polling or not stream.query():
+            return False
+        buf[:n].fill_(self.NOT_YET)
+        return True
+
+    def wait(self, buf, n, stream, armed):
+        if armed:
             entries = (ctypes.c_int64 * n).from_address(buf.data_ptr())
+            deadline = time.perf_counter() + self.WATCH_SECONDS
             i = spins = 0
-            while i < n and spins < self.SPIN_LIMIT:
+            while i < n:
                 if entries[i] != self.NOT_YET:
                     i += 1
-                else:
-                    spins += 1
-            if i == n:
-                return
-            _PinnedCounts.polling = False
+                    continue
+                spins += 1
+                if (spins & 255) == 0 and time.perf_counter() > deadline:
+                    break
+            with self._lock:
+                if i == n:
+                    self._misses = 0
+                    return
+                self._misses += 1
+                if self._misses >= self.MISSES_TO_SWITCH_OFF:
+                    self._polling = False
         stream.synchronize()
 
 
@@ -831,9 +848,9 @@ def _viterbi_decode_call(name, B, L, ml, dev, extra_words, call):
         # synchronisation of the decode is a stream wait, with no copy in front of it
         host = _pinned_counts.take(B)  # written by the kernel, read after the one stream wait
         try:
-            _pinned_counts.arm(host, B)
+            armed = _pinned_counts.arm(host, B, torch.cuda.current_stream(dev))
             _lib.check(call(lib, block.data_ptr(), nwork, host.data_ptr()), lib)
-            _pinned_counts.wait(host, B, torch.cuda.current_stream(dev))
+            _pinned_counts.wait(host, B, torch.cuda.current_stream(dev), armed)
             counts = host[:B].tolist()
         finally:
             _pinned_counts.give_back(host)
@@ -949,11 +966,11 @@ def pcfg_lookahead_decode(links, unreduced_logits, unreduced_tokens, output_leng
         out = torch.empty((B, L), dtype=torch.int64, device=dev)
         cnt = _pinned_counts.take(B)  # written by the kernel, read after the one stream wait
         try:
-            _pinned_counts.arm(cnt, B)
+            armed = _pinned_counts.arm(cnt, B, torch.cuda.current_stream(dev))
             _lib.check(lib.pcfgnat_lookahead_decode(links.data_ptr(), ob_ptr, float(beta), ol.data_ptr(), tok.data_ptr(),
                                                     mask.data_ptr(), mask.size(0), int(pad_index), idx.data_ptr(), out.data_ptr(),
                                                     cnt.data_ptr(), B, L, K - 1, _stream(links)), lib)
-            _pinned_counts.wait(cnt, B, torch.cuda.current_stream(dev))
+            _pinned_counts.wait(cnt, B, torch.cuda.current_stream(dev), armed)
             counts = cnt[:B].tolist()
         finally:
             _pinned_counts.give_back(cnt)

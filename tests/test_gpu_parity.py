@@ -927,26 +927,55 @@ def test_decode_from_logits_is_front_end_plus_decode(case, dtype):
 
 
 def test_decode_waits_for_the_stream_where_the_counts_do_not_turn():
-    """The decode calls watch the token counts turn in pinned host memory; a watch that runs into its bound (forced here by
-    a bound of zero reads) hands over to the stream wait and switches the watching off, with the same results."""
+    """The decode calls watch the token counts turn in pinned host memory.  A watch that runs into its time bound (forced
+    here by a bound of zero seconds) hands over to the stream wait for that call with the same results; the watching is
+    switched off only after several such misses in a row, and one watch that succeeds resets the count.  A call that finds
+    work pending on its stream does not watch at all."""
     import oracle_ops
     batch = _decode_case("L96")
     ob, tok = synth.ob_and_tokens(batch["logits"])
     links, ol = batch["links"], batch["output_length"]
     left_mask, _, _ = synth.support_masks(links.shape[1], 1)
     want_tok, want_len = harness.viterbi_decode(ob, tok, links, ol, left_mask, ops=oracle_ops)
-    pool = type(ops._pinned_counts)
-    limit, polling = pool.SPIN_LIMIT, pool.polling
+    args = (ob.to(DEV), tok.to(DEV), links.to(DEV), ol.to(DEV), left_mask.to(DEV))
+
+    def decode():
+        torch.cuda.synchronize()
+        got_tok, got_len = harness.viterbi_decode(*args, single_call=True)
+        assert torch.equal(got_len.cpu(), want_len) and torch.equal(got_tok.cpu(), want_tok)
+
+    pool = ops._pinned_counts
+    saved = (pool.WATCH_SECONDS, pool._polling, pool._misses)
     try:
-        pool.polling, pool.SPIN_LIMIT = True, 0
-        for expect_polling_before in (True, False):
-            assert pool.polling == expect_polling_before
-            got_tok, got_len = harness.viterbi_decode(ob.to(DEV), tok.to(DEV), links.to(DEV), ol.to(DEV), left_mask.to(DEV),
-                                                      single_call=True)
-            assert torch.equal(got_len.cpu(), want_len) and torch.equal(got_tok.cpu(), want_tok)
-        assert pool.polling is False
+        pool._polling, pool._misses = True, 0
+        decode()
+        assert pool.polling_on() and pool._misses == 0  # the counts turned inside the bound
+        pool.WATCH_SECONDS = -1.0  # every watch misses (the bound is looked at every 256 reads: the kernel has not ended by then)
+        for k in range(1, pool.MISSES_TO_SWITCH_OFF):
+            decode()
+            assert pool.polling_on()
+        misses_before = pool._misses
+        pool.WATCH_SECONDS = saved[0]
+        decode()
+        assert pool._misses == 0 or misses_before == 0  # a watch that succeeds resets the count
+        pool.WATCH_SECONDS = -1.0
+        pool._misses = pool.MISSES_TO_SWITCH_OFF - 1
+        decode()
+        if pool._misses:  # (a kernel that ended within the first 256 reads is no miss)
+            assert not pool.polling_on()
+        decode()  # without watching: the stream wait alone
+        # work pending on the stream: no watch, whatever the setting
+        pool._polling, pool._misses, pool.WATCH_SECONDS = True, 0, saved[0]
+        big = torch.empty(64 << 20, device=DEV)
+        for _ in range(8):
+            big.normal_()
+        buf = pool.take(4)
+        armed = pool.arm(buf, 4, torch.cuda.current_stream(DEV))
+        pool.give_back(buf)
+        assert armed is False
+        decode()
     finally:
-        pool.SPIN_LIMIT, pool.polling = limit, polling
+        pool.WATCH_SECONDS, pool._polling, pool._misses = saved
 
 
 @pytest.mark.parametrize("mode", ["one_workgroup", "blocks_give_up"])
