@@ -44,8 +44,6 @@ def parse():
                          "the reference point for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--step", choices=["single", "fused"], default="single",
                     help="single: one native call per step (default); fused: four native calls from Python")
-    ap.add_argument("--slices", type=int, default=1,
-                    help="batch slices of the single-call step that alternate between two streams (1 = no pipelining)")
     ap.add_argument("--unfused", action="store_true",
                     help="issue the criterion's glue (eos mask, gradient scaling) as separate torch ops, like the reference")
     return ap.parse_args()
@@ -539,7 +537,7 @@ def main():
             if not detail["on"] and (sampled["step"] - 1) % EVENT_EVERY != 0:
                 return None
             evs = []
-            for kernel in ("lsg_fwd", "inside_fwd", "inside_bwd", "lsg_bwd"):
+            for kernel in ("lsg_fwd", "inside_fwd_bwd", "lsg_bwd"):
                 for _ in range(2):
                     if kernel != roof and not detail["on"]:
                         evs.append(None)
@@ -558,13 +556,8 @@ def main():
         ev.record()
         pairs.setdefault(name, []).append(ev)
 
-    if mode == "single":
-        def step_fn(*a, **kw):
-            return harness.train_step_single_call(*a, slices=args.slices, **kw)
-    else:
-        step_fn = {"unfused": harness.train_step_direct, "fused": harness.train_step_fused}[mode]
-    # sentences whose logsoftmax_gather launch the timing events bracket
-    B_timed = (B // args.slices) if mode == "single" and args.slices > 1 else B
+    step_fn = {"unfused": harness.train_step_direct, "fused": harness.train_step_fused, "single": harness.train_step_single_call}[mode]
+    B_timed = B  # sentences whose logsoftmax_gather launch the timing events bracket
     losses = []
     for i in range(args.warmup):
         losses.append(step_fn(bufs[i], targets, links, ol, tl)[0])
@@ -635,9 +628,6 @@ def main():
     torch.cuda.synchronize()
     kern_ms = averages()
     kern_ms[roof] = roof_in_region
-    if mode == "single":  # the library issues the inside forward and backward together, bracketed by the third pair
-        kern_ms.pop("inside_fwd", None)
-        kern_ms["inside_fwd_bwd"] = kern_ms.pop("inside_bwd")
     # the single-call step neither reads the logits of the pad nodes behind a sentence's graph nor re-reads them in the
     # backward (their gradient rows are written as zeros); the other modes go through the operator API, which cannot know
     live_rows = int(m[:B_timed].sum()) if mode == "single" else None
@@ -668,8 +658,7 @@ def main():
                                   else "forward read-only, backward recomputes softmax from row log-sum-exps, three passes "
                                        "over the logits")
                                + ("as separate torch ops" if args.unfused else "folded into the kernels, %s" %
-                                  ("one native call per step, %d batch slice(s) on two streams" % args.slices if args.step == "single"
-                                   else "four native calls per step")),
+                                  ("one native call per step" if args.step == "single" else "four native calls per step")),
                    "global_batch": B, "graph_nodes": L, "target_len": T, "vocab": V},
         "roofline": {"bound": "hbm", "kernel": ROOFLINE_KERNEL_NAME[roof], "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
@@ -686,20 +675,10 @@ def main():
     result["headline_windows"]["sentences_per_s_median"] = B / (result["headline_windows"]["ms_per_step_median"] * 1e-3)
     if mode == "single":
         # the same single call with an upstream factor of 128 on the loss (fp16 loss scaling), folded into the weights
-        sc = timed_windows(lambda i: harness.train_step_single_call(bufs[i], targets, links, ol, tl, slices=args.slices, loss_scale=128.0))
+        sc = timed_windows(lambda i: harness.train_step_single_call(bufs[i], targets, links, ol, tl, loss_scale=128.0))
         sc["sentences_per_s_median"] = B / (sc["ms_per_step_median"] * 1e-3)
         sc["loss_scale"] = 128.0
         result["single_call_scaled"] = sc
-        # the same single call with the inside and outside sweeps in the linear domain, an option that is off by default: it
-        # pays on emissions as flat as these synthetic ones and costs on a model that is sure of itself
-        from pcfg_nat_amd import custom_ops
-        try:
-            custom_ops.inside_linear_bits(500)
-            lin = timed_windows(lambda i: step_fn(bufs[i], targets, links, ol, tl))
-        finally:
-            custom_ops.inside_linear_bits(0)
-        lin["sentences_per_s_median"] = B / (lin["ms_per_step_median"] * 1e-3)
-        result["single_call_linear_sweeps"] = lin
     # the drop-in path: the unchanged criterion code over the operator API under autograd (dag_logsoftmax_gather_inplace ->
     # eos mask -> cuda_pcfg_loss -> loss -> backward), which reads and rewrites every row (it is not told the lengths)
     result["criterion_autograd"] = criterion_autograd_timing(bufs, targets, links, ol, tl, args, timed_windows, host_enqueue_ms)

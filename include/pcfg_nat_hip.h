@@ -14,9 +14,8 @@
  *     ml = links.size(2) - 1 ("max_left"), Mc = (L-2)/(ml+1)+1 main-chain nodes, Lq = L/4.
  *   - PCFG tables are float32 (the `_f64` entry points take float64 tables, which the reference also dispatches,
  *     pcfg_loss.cu:395), lengths are int64, like every caller in the reference.
- *   - state: the entry points keep nothing between calls except the two process-wide tuning settings of
- *     pcfgnat_pipeline_config, a per-device cache of kernel attributes and, only for pcfgnat_criterion_step with
- *     slices > 1, one helper stream per device (calls with slices > 1 must not overlap on one device).
+ *   - state: the entry points keep nothing between calls except a per-device cache of kernel attributes (and the
+ *     process-wide test and tuning settings of pcfg_nat_hip_testing.h, which no call needs).
  */
 #ifndef PCFG_NAT_HIP_H
 #define PCFG_NAT_HIP_H
@@ -192,25 +191,6 @@ void pcfgnat_pipeline_config(int max_workgroups, int spin_limit);
 void pcfgnat_links_grad_range_limit(float log2_limit);
 
 /*
- * No counterpart in the reference: with bits > 0, graphs of up to 130 nodes are swept in the linear domain (probabilities
- * in double, one multiply-add per term) where the numbers allow it - links and emissions between 2^-150 and 2^8 or zero,
- * every intermediate at least 2^-bits or exactly zero - and in the log domain, which has no range limit, otherwise; the
- * choice is made per sentence and per sweep by the kernel: an input out of range sends the whole sweep to the log domain,
- * a number below the range on the way stops the linear sweep there and the log-domain sweep goes on from that column.
- * Pays where emissions are not peaked (a fifth off the sweeps' time), costs where a model is sure of itself (up to a
- * tenth more when a sentence leaves the range in its first columns).
- * bits: at most 500; 0, the default, switches the linear sweeps off.  Process-wide.
- */
-void pcfgnat_inside_linear_bits(int bits);
-
-/*
- * No counterpart in the reference: diagnostic counters since the library was loaded (or the last reset) on the current
- * device - sweeps (forward and outside sweeps count apart) completed in the linear domain, and sweeps the linear
- * domain handed over to the log domain, from the start or on the way.  Synchronises with the device.
- */
-int pcfgnat_inside_linear_counts(unsigned long long *swept, unsigned long long *handed_over, int reset);
-
-/*
  * No counterpart in the reference: diagnostic counters of that fallback since the library was loaded - inside sweeps
  * (forward and outside counted apart) and single-call Viterbi decodes that the one-workgroup kernels redid because a
  * pipelined sweep gave up.  Reads two device counters of the current device (synchronises with the device); reset != 0
@@ -268,23 +248,19 @@ int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *
  * (nat_pcfg_loss.py:116-121) with the outputs of the glancing step - a graph node whose input was revealed
  * (keep_word_mask) may only emit the target position it is aligned to (matchmask), through a detached value, i.e. the
  * logits row of such a node gets a zero gradient.
- * slices: 1 = the whole batch at once; k > 1 = the batch is processed as k slices (sentences [i*B/k, (i+1)*B/k)) that
- * alternate between `stream` and one helper stream the library keeps per device (created on first use, default
- * priority), so that the latency-bound inside kernels of one slice run beside the bandwidth-bound gather kernels of the
- * next; the helper stream forks from and joins back into `stream`, so the call stays ordered on `stream`.
  * loss_scale, loss_scale_dev: the factor the caller's loss carries downstream of this criterion (nat_pcfg_loss.py:139-140
  * `loss * factor`, times the fp16 loss scale of every shipped training script): a host value times an optional float32
  * scalar in device memory (NULL = 1).  Both gradients come out multiplied by it; it enters the weights -1/(target_length*B)
  * in float32, i.e. ahead of the single rounding of d loss / d logits to the logits' dtype, as in pcfg_loss.py:77-83, 176-177.
  * loss_out[0] stays the unscaled loss.
- * events: NULL, or eight hipEvent_t (entries may be NULL) recorded before/after the gather forward, (unused pair), the
- * inside forward+backward and the gather backward of slice 0 (for timing).
+ * events: NULL, or six hipEvent_t (entries may be NULL) recorded before/after the gather forward, the inside
+ * forward+backward and the gather backward (for timing).
  */
 int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, const float *links,
                            const int64_t *output_length, const int64_t *target_length, const unsigned char *matchmask,
                            const unsigned char *keep_word_mask, float *match_all, float *S,
                            float *aux, float *match_all_grad, float *links_grad, float *row_lse, float *loss_out, int64_t B,
-                           int64_t L, int64_t V, int64_t T, int64_t ml, int64_t slices, float loss_scale,
+                           int64_t L, int64_t V, int64_t T, int64_t ml, float loss_scale,
                            const float *loss_scale_dev, void *stream, void *const *events);
 
 /*

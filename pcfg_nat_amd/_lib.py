@@ -35,8 +35,6 @@ SIGNATURES = {
     "pcfgnat_pipeline_outside_spin_limit": (None, [_int]),
     "pcfgnat_pipeline_redo_counts": (_int, [_vp, _vp, _int]),
     "pcfgnat_links_grad_range_limit": (None, [ctypes.c_float]),
-    "pcfgnat_inside_linear_bits": (None, [_int]),
-    "pcfgnat_inside_linear_counts": (_int, [_vp, _vp, _int]),
     "pcfgnat_pcfg_loss": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_pcfg_loss_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_pcfg_loss_forward_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
@@ -49,7 +47,7 @@ SIGNATURES = {
     "pcfgnat_pcfg_viterbi_f64": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "pcfgnat_criterion_loss": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_criterion_step": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
-                                      _i64, _i64, ctypes.c_float, _vp, _vp, _vp]),
+                                      _i64, ctypes.c_float, _vp, _vp, _vp]),
     "pcfgnat_criterion_forward": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                                          _i64, _i64, _vp]),
     "pcfgnat_criterion_backward": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),

@@ -48,54 +48,20 @@ int ensure_dynamic_lds(const void *kernel, size_t bytes) {
 }
 }  // namespace pcfgnat
 
-extern "C" int pcfgnat_abi_version(void) { return 3; }
+extern "C" int pcfgnat_abi_version(void) { return 4; }
 
 extern "C" const char *pcfgnat_last_error(void) { return pcfgnat::error_buffer(); }
 
 // ---------------------------------------------------------------------------------------------------------------
 // One call for the whole training pass of the criterion (fs_plugins/criterions/nat_pcfg_loss.py:98-145 and the backward
 // autograd derives from it): gather with eos mask -> inside forward+backward seeded with -1/(n_b*B) -> in-place gather
-// backward -> loss.  Nothing is allocated.
-//
-// With slices > 1 the batch is cut into slices that alternate between the caller's stream and one helper stream per
-// device: the inside kernels of a slice are latency-bound on a few dozen CUs, the gather kernels of its neighbour are
-// HBM-bound on all of them, so running them side by side hides the former.  The helper stream forks from and joins
-// back into the caller's stream through events, i.e. for the caller everything is ordered on `stream` as usual.
+// backward -> loss.  Nothing is allocated, everything is enqueued on the caller's stream.
 // ---------------------------------------------------------------------------------------------------------------
-namespace {
-struct DeviceHelper {
-    hipStream_t stream = nullptr;
-    hipEvent_t fork = nullptr, join = nullptr, gathered[2] = {nullptr, nullptr};
-    bool ready = false;
-};
-constexpr int MAX_DEVICES = 64;
-DeviceHelper g_helpers[MAX_DEVICES];
-std::mutex g_helpers_mutex;
-
-int get_helper(DeviceHelper **out) {
-    int dev = 0;
-    PCFGNAT_HIP_CHECK(hipGetDevice(&dev));
-    if (dev < 0 || dev >= MAX_DEVICES) return pcfgnat::fail(PCFGNAT_EINVAL, "criterion_step: device index %d out of range", dev);
-    std::lock_guard<std::mutex> lock(g_helpers_mutex);
-    DeviceHelper &h = g_helpers[dev];
-    if (!h.ready) {
-        PCFGNAT_HIP_CHECK(hipStreamCreateWithFlags(&h.stream, hipStreamNonBlocking));  // default priority
-        PCFGNAT_HIP_CHECK(hipEventCreateWithFlags(&h.fork, hipEventDisableTiming));
-        PCFGNAT_HIP_CHECK(hipEventCreateWithFlags(&h.join, hipEventDisableTiming));
-        PCFGNAT_HIP_CHECK(hipEventCreateWithFlags(&h.gathered[0], hipEventDisableTiming));
-        PCFGNAT_HIP_CHECK(hipEventCreateWithFlags(&h.gathered[1], hipEventDisableTiming));
-        h.ready = true;
-    }
-    *out = &h;
-    return PCFGNAT_OK;
-}
-}  // namespace
-
 extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, const float *links,
                                       const int64_t *output_length, const int64_t *target_length, const unsigned char *matchmask,
                                       const unsigned char *keep_word_mask, float *match_all, float *S,
                                       float *aux, float *match_all_grad, float *links_grad, float *row_lse, float *loss_out, int64_t B,
-                                      int64_t L, int64_t V, int64_t T, int64_t ml, int64_t slices, float loss_scale,
+                                      int64_t L, int64_t V, int64_t T, int64_t ml, float loss_scale,
                                       const float *loss_scale_dev, void *stream, void *const *events) {
     if (dtype != PCFGNAT_F16 && dtype != PCFGNAT_F32)
         return pcfgnat::fail(PCFGNAT_EUNSUPPORTED, "criterion_step: logits must be float16 or float32 (the PCFG kernels are float32)");
@@ -105,71 +71,34 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
                     "criterion_step: null pointer");
     PCFGNAT_REQUIRE((matchmask == nullptr) == (keep_word_mask == nullptr),
                     "criterion_step: matchmask and keep_word_mask must be given together (or both be null)");
-    if (slices < 1) slices = 1;
-    if (slices > B) slices = B;
-    hipStream_t main_stream = (hipStream_t)stream;
-    DeviceHelper *h = nullptr;
-    if (slices > 1) {
-        int rc = get_helper(&h);
-        if (rc != PCFGNAT_OK) return rc;
-        PCFGNAT_HIP_CHECK(hipEventRecord(h->fork, main_stream));
-        PCFGNAT_HIP_CHECK(hipStreamWaitEvent(h->stream, h->fork, 0));
-    }
+    hipStream_t s = (hipStream_t)stream;
     const size_t esz = (dtype == PCFGNAT_F16) ? 2 : 4;
     const int64_t Mc = (L - 2) / (ml + 1) + 1;
-    const size_t aux_per_sentence = pcfgnat_pcfg_aux_floats(1, L, T, ml);
-    for (int64_t i = 0; i < slices; i++) {
-        const int64_t b0 = i * B / slices, b1 = (i + 1) * B / slices, nb = b1 - b0;
-        if (nb == 0) continue;
-        hipStream_t s = (i & 1) ? h->stream : main_stream;
-        char *lg_i = (char *)logits + (size_t)b0 * L * V * esz;
-        const int64_t *tg_i = targets + (size_t)b0 * T, *ol_i = output_length + b0, *tl_i = target_length + b0;
-        const float *lk_i = links + (size_t)b0 * L * (ml + 1) * L;
-        float *ma_i = match_all + (size_t)b0 * L * T, *S_i = S + (size_t)b0 * Mc * (T + 2), *aux_i = aux + (size_t)b0 * aux_per_sentence;
-        float *mg_i = match_all_grad + (size_t)b0 * L * T, *lkg_i = links_grad + (size_t)b0 * L * (ml + 1) * L;
-        float *lse_i = row_lse + (size_t)b0 * L;
-        const unsigned char *mm_i = matchmask ? matchmask + (size_t)b0 * T * L : nullptr;
-        const unsigned char *keep_i = keep_word_mask ? keep_word_mask + (size_t)b0 * L : nullptr;
-        const bool mark = events && i == 0;  // timing events bracket the kernels of slice 0
-#define PCFGNAT_MARK(k)                                                                   \
-    do {                                                                                  \
-        if (mark && events[k]) PCFGNAT_HIP_CHECK(hipEventRecord((hipEvent_t)events[k], s)); \
+#define PCFGNAT_MARK(k)                                                                     \
+    do {                                                                                    \
+        if (events && events[k]) PCFGNAT_HIP_CHECK(hipEventRecord((hipEvent_t)events[k], s)); \
     } while (0)
-        // stagger: the gather of slice i starts when the gather of slice i-1 is done, so that it runs beside the inside
-        // kernels of slice i-1 rather than beside its gather
-        if (i > 0) PCFGNAT_HIP_CHECK(hipStreamWaitEvent(s, h->gathered[(i - 1) & 1], 0));
-        PCFGNAT_MARK(0);
-        int rc = pcfgnat::lsg_forward_lse_force(lg_i, dtype, tg_i, ma_i, lse_i, ol_i, tl_i, mm_i, keep_i, nb, L, V, T, s);
-        if (rc != PCFGNAT_OK) return rc;
-        PCFGNAT_MARK(1);
-        if (slices > 1) PCFGNAT_HIP_CHECK(hipEventRecord(h->gathered[i & 1], s));
-        PCFGNAT_MARK(2);
-        PCFGNAT_MARK(3);  // forward and backward are issued by one internal call: bracketed together by 4..5
-        PCFGNAT_MARK(4);
-        // the rows of pad nodes of the logits gradient are zeroed beside the sweeps where the inside launch can host that
-        bool pad_done = false;
-        rc = pcfgnat::inside_forward_backward_impl(nullptr, ma_i, lk_i, ol_i, tl_i, S_i, aux_i, mg_i, lkg_i, nb, L, T, ml,
-                                                   pcfgnat::seed_of(B, loss_scale, loss_scale_dev), s,
-                                                   pcfgnat::PadFill{(unsigned char *)lg_i, (int64_t)V * (int64_t)esz}, &pad_done);
-        if (rc != PCFGNAT_OK) return rc;
-        PCFGNAT_MARK(5);
-        PCFGNAT_MARK(6);
-        if (slices == 1)  // the loss is reduced by the first workgroup of the same launch (S is complete by now)
-            rc = pcfgnat::lsg_backward_lse_with_loss(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, S, Mc * (T + 2), target_length,
-                                                     loss_out, keep_i, ol_i, pad_done ? 1 : 0, nullptr, s);
-        else
-            rc = pcfgnat::lsg_backward_lse_with_loss(lg_i, dtype, tg_i, T, 0, 1, mg_i, lse_i, nb, L, V, T, nullptr, 0, nullptr, nullptr,
-                                                     keep_i, ol_i, pad_done ? 1 : 0, nullptr, s);
-        if (rc != PCFGNAT_OK) return rc;
-        PCFGNAT_MARK(7);
+    PCFGNAT_MARK(0);
+    int rc = pcfgnat::lsg_forward_lse_force(logits, dtype, targets, match_all, row_lse, output_length, target_length, matchmask,
+                                            keep_word_mask, B, L, V, T, s);
+    if (rc != PCFGNAT_OK) return rc;
+    PCFGNAT_MARK(1);
+    PCFGNAT_MARK(2);
+    // the rows of pad nodes of the logits gradient are zeroed beside the sweeps where the inside launch can host that
+    bool pad_done = false;
+    rc = pcfgnat::inside_forward_backward_impl(nullptr, match_all, links, output_length, target_length, S, aux, match_all_grad, links_grad,
+                                               B, L, T, ml, pcfgnat::seed_of(B, loss_scale, loss_scale_dev), s,
+                                               pcfgnat::PadFill{(unsigned char *)logits, (int64_t)V * (int64_t)esz}, &pad_done);
+    if (rc != PCFGNAT_OK) return rc;
+    PCFGNAT_MARK(3);
+    PCFGNAT_MARK(4);
+    // the loss is reduced by the first workgroup of the same launch (S is complete by now)
+    rc = pcfgnat::lsg_backward_lse_with_loss(logits, dtype, targets, T, 0, 1, match_all_grad, row_lse, B, L, V, T, S, Mc * (T + 2),
+                                             target_length, loss_out, keep_word_mask, output_length, pad_done ? 1 : 0, nullptr, s);
+    if (rc != PCFGNAT_OK) return rc;
+    PCFGNAT_MARK(5);
 #undef PCFGNAT_MARK
-    }
-    if (slices > 1) {
-        PCFGNAT_HIP_CHECK(hipEventRecord(h->join, h->stream));
-        PCFGNAT_HIP_CHECK(hipStreamWaitEvent(main_stream, h->join, 0));
-    }
-    if (slices == 1) return PCFGNAT_OK;
-    return pcfgnat_criterion_loss(S, target_length, loss_out, B, L, T, ml, stream);
+    return PCFGNAT_OK;
 }
 
 // ---------------------------------------------------------------------------------------------------------------

@@ -18,10 +18,7 @@
 // reads links, emissions and its own earlier columns only, so in the single call the two run side by side as two
 // workgroups (inside_pair_ml1_kernel) and a parallel kernel multiplies their tables into the posteriors
 // (inside_combine_ml1_kernel); in the two-call API the outside sweep accumulates rule posteriors in registers and
-// emission posteriors come from an element-wise epilogue.  Where the tables leave room in LDS (the shipped shapes do),
-// these sweeps can run in the linear domain instead - probabilities as doubles, one multiply-add per term, the table
-// entries made by waves of their own - falling back to the log domain per sentence when a number leaves the range
-// (further down; off unless pcfgnat_inside_linear_bits switches it on).
+// emission posteriors come from an element-wise epilogue.
 // Graphs of more than 130 nodes use the streaming or the pipelined sweeps (link rows from L2, or spread over several
 // workgroups per sentence).
 #include "common.hip.h"
@@ -36,12 +33,6 @@ namespace {
 constexpr int NT = 1024;       // threads per sentence
 
 __device__ __forceinline__ float sanitize(float v) { return (v != v) ? NEG_INF_F : v; }
-
-__device__ __forceinline__ float lse2(float a, float b) {
-    float m = fmaxf(a, b);
-    if (m == NEG_INF_F) return NEG_INF_F;
-    return m + __logf(__expf(a - m) + __expf(b - m));
-}
 
 // Column offsets.  Entries of S grow like (tokens left) x (log-probability per token), thousands for long sentences,
 // where fp32 resolves only ~1e-4 - and posteriors are exponentials of sums of such entries.  Every sweep therefore
@@ -84,11 +75,6 @@ struct AuxView {
 // Head of the dynamic LDS of the register-resident kernels: per-wave column maxima slots[2][8] (16-byte aligned), the
 // column offsets O [T+2] (double) and the shifts D [T+4].
 __host__ __device__ inline int head_floats(int T) { return 16 + 2 * (T + 2) + (T + 4); }
-// Floats of dynamic LDS of the forward role with its tables in LDS and one tile of 64 nodes (rounded to 16 bytes): head,
-// col [2][64], emissions of main nodes and leaves [Mc][T], R, F0h, F1h [Mc][T+2].
-__host__ __device__ inline size_t fwd_role_floats(int Mc, int T) {
-    return ((size_t)head_floats(T) + 2 * 64 + (size_t)2 * Mc * T + (size_t)3 * Mc * (T + 2) + 3) & ~(size_t)3;
-}
 struct LdsHead {
     float *slots, *D;
     double *O;
@@ -122,10 +108,6 @@ constexpr double LN2_D = 0.6931471805599453094;
 // Diagnostic: sweeps (forward or outside, counted apart) that the one-workgroup kernels redid because the pipelined
 // sweep of the sentence gave up, since the library was loaded (pcfgnat_pipeline_redo_counts).
 __device__ unsigned long long g_inside_redone;
-// Diagnostic: sweeps (forward or outside, counted apart) that ran in the linear domain, and those of them that were
-// handed to the log-domain sweep because a number left the range, since the library was loaded
-// (pcfgnat_inside_linear_counts).
-__device__ unsigned long long g_linear_swept, g_linear_handed_over;
 
 __device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float lg2(float x) { return __builtin_amdgcn_logf(x); }
@@ -152,10 +134,6 @@ __device__ __forceinline__ float lse2_b2(float a, float b) {
 // node block of wave w inside a 64-node tile (wave-uniform scalar)
 __device__ __forceinline__ int wave_block(int wave) { return __builtin_amdgcn_readfirstlane(wave < 4 ? wave : 11 - wave); }
 
-// Keeps a value (and the load that produced it) out of the conditionally executed blocks that consume it, so that all
-// LDS reads of a step are issued back to back instead of one per branch, each followed by its own wait.
-__device__ __forceinline__ void pin(float &v) { asm volatile("" : "+v"(v)); }
-
 struct FwdSweepArgs {
     float *col, *sm_main, *sm_leaf, *sm_S, *sm_F0, *sm_F1;
     const float *mt;
@@ -164,10 +142,6 @@ struct FwdSweepArgs {
     double *sm_O;
     float base_b2;  // the base cell S[last][n-1], base 2
     int n, mc, Mc, T, j, g8;
-    // where the sweep starts: column n-1 with offset 0 or, taking over from a linear-domain sweep that ran out of range,
-    // an earlier column t_start, found in col with its offset O_start, the row sums F1 of the step before it in sm_F1
-    int t_start;
-    double O_start;
 };
 
 // max of three values that need no canonicalisation (loaded from tables this kernel wrote)
@@ -201,18 +175,10 @@ __device__ __forceinline__ void fwd_sweep(const float (&A0)[R][8 * R], const flo
     float F1prev[R];
     float wprev = x.base_b2;  // this wave's maximum of the column written by the previous step
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-        F1prev[r] = NEG_INF_F;
-        if (TAB_LDS && x.t_start < x.n - 1) {
-            const int a_id = 64 * r + 8 * P + x.g8;
-            const float c_own = x.col[(x.t_start & 1) * MP + a_id];
-            F1prev[r] = (a_id < x.mc) ? x.sm_F1[a_id * TS + x.t_start + 1] : NEG_INF_F;
-            wprev = (r == 0) ? c_own : fmaxf(wprev, c_own);
-        }
-    }
+    for (int r = 0; r < R; r++) F1prev[r] = NEG_INF_F;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    double O = x.O_start;  // offset of the column being read
-    for (int t = x.t_start; t >= 1; t--) {
+    double O = 0.0;  // offset of the column being read
+    for (int t = x.n - 1; t >= 1; t--) {
         const float *cur = x.col + (t & 1) * MP;
         float *nxt = x.col + ((t - 1) & 1) * MP;
         float wmax = NEG_INF_F;
@@ -306,381 +272,13 @@ __device__ __forceinline__ void fwd_sweep(const float (&A0)[R][8 * R], const flo
     }
 }
 
-// ------------------------------------------------------------------------------------------------------------
-// The same two sweeps in the linear domain.  A step of the log-domain sweeps above is bound by instruction issue: some
-// 180 instructions of bookkeeping per wave and step (shifts, reductions over the node's lanes, the table entries) plus
-// add, max, subtract, exp2, add per term in two passes, on two waves per SIMD.  With the probabilities themselves in
-// double a term is one fused multiply-add, and the work is split so that the chain from one column to the next is
-// short: waves 0-3 (one per SIMD) own 16 nodes each, a quad of lanes per node, and do nothing but load the column,
-// multiply, add up the quad, and store the node's three results as doubles into rotating columns; waves 4-6 follow one
-// step behind and turn those columns into the table entries (base-2 logarithms, as the log-domain sweep leaves them),
-// find the exponent of the column maximum, keep the offsets, and watch the range.  The offset of a column is set to the
-// absolute exponent of the latest column maximum known when it is chosen (one or two columns back), so the entries
-// stay within a few steps' worth of decay of one; following the relative exponent alone, with that delay, would
-// oscillate.
-// Doubles are there for their exponent range, not their precision: columns are still rescaled every step, by a power
-// of two (exact), and the tables are relative to the same kind of offsets (D, O / E, P hold integers here).
-// What the range cannot hold must not be lost silently - a node whose inside value is 2^-600 of its column's largest
-// may still carry the whole posterior.  So a sweep only accepts numbers it can follow: links and emissions between
-// 2^-LIN_INPUT_BITS and 2^LIN_INPUT_TOP (or zero), and every number a later step multiplies - column entries, the row
-// sums F1, betas, offered weights - at least 2^-lin_bits (lin_bits <= 500; or exactly zero, which then is a sum of exact
-// zeros: with these bounds a column grows by less than 2^25 a step, shifts stay below 2^80, and no product of nonzero
-// factors gets below 2^-900; all terms are positive, so nothing cancels).  An input out of range raises the workgroup's
-// flag and the sentence is swept in the log domain by the code above.  A number below 2^-lin_bits on the way (peaked
-// emissions: a node far from the alignment loses tens of bits per token against the column's largest) stops the sweep
-// instead: the table wave that watches the range - one step behind the sweep, so the number itself is still a product
-// of accepted ones and exact - sets a mark beside the shift the sweep reads at the top of its next step; every wave
-// leaves its loop behind that step (whose results nobody reads), and the log-domain sweep goes on from the last column that holds only such numbers, reading
-// its state (column, row sums, shift, offset) from the tables, which both kinds of sweep keep in the same form.  What
-// the interrupted steps wrote beyond that column is overwritten.  lin_bits <= 0 switches the linear sweeps off.
-// ------------------------------------------------------------------------------------------------------------
-constexpr float LIN_INPUT_BITS = 150.f, LIN_INPUT_TOP = 8.f;
-// Nothing a sweep accepts can get below 2^-900; a number this small means the bounds above do not hold.
-constexpr int LIN_FLOOR_BITS = 1000;
-constexpr int LIN_BITS_MAX = 500;
-
-// the partner lane's double inside a quad (every lane has a source, so there is no old value to keep)
-template <int CTRL>
-__device__ __forceinline__ double dpp_d(double v) {
-    return __hiloint2double(__builtin_amdgcn_mov_dpp(__double2hiint(v), CTRL, 0xF, 0xF, true),
-                            __builtin_amdgcn_mov_dpp(__double2loint(v), CTRL, 0xF, 0xF, true));
-}
-__device__ __forceinline__ double quad_sum_d(double v) {
-    v += dpp_d<DPP_QUAD_XOR1>(v);
-    v += dpp_d<DPP_QUAD_XOR2>(v);
-    return v;
-}
-// Wave64 maximum of an int: DPP inside the rows, the four row results through scalar registers.
-__device__ __forceinline__ int wave_max_i(int v) {
-    v = max(v, dpp_i<DPP_QUAD_XOR1>(v));
-    v = max(v, dpp_i<DPP_QUAD_XOR2>(v));
-    v = max(v, dpp_i<DPP_ROW_HALF_MIRROR>(v));
-    v = max(v, dpp_i<DPP_ROW_MIRROR>(v));
-    const int a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
-    const int c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
-    return max(max(a, b), max(c, d));
-}
-__device__ __forceinline__ int clamp_shift(int k) { return max(-1000, min(1000, k)); }
-// 2^k for -1022 <= k <= 1023
-__device__ __forceinline__ double pow2_int(int k) { return __hiloint2double((1023 + k) << 20, 0); }
-// 2^v for a base-2 logarithm that passes lin_input_ok (-inf: 0; anything else: some number, the sweep is not used then):
-// the fraction through the hardware exp2, the integer part added to the exponent field
-__device__ __forceinline__ double pow2_of(float v) {
-    const float fl = floorf(v);
-    const double r = (double)ex2(v - fl);
-    const int hi = __double2hiint(r) + ((int)fl << 20);
-    const bool zero = v == NEG_INF_F;
-    return __hiloint2double(zero ? 0 : hi, zero ? 0 : __double2loint(r));
-}
-// 1 if the sweep can take the base-2 logarithm v (as an int, to be combined without branches)
-__device__ __forceinline__ int lin_input_ok(float v) { return (v == NEG_INF_F) | ((v >= -LIN_INPUT_BITS) & (v <= LIN_INPUT_TOP)); }
-// binary exponent e of a positive normal double, d = f * 2^e with f in [0.5, 1)
-__device__ __forceinline__ int exponent_of(double d) { return ((__double2hiint(d) >> 20) & 0x7ff) - 1022; }
-constexpr int NO_EXPONENT = -(1 << 20);  // stands for the exponent of zero
-__device__ __forceinline__ int exponent_or_none(double d) { return d > 0.0 ? exponent_of(d) : NO_EXPONENT; }
-// log2 of a double that is zero or a positive normal number, as a float
-__device__ __forceinline__ float log2_of(double d) {
-    const int hi = __double2hiint(d);
-    const double f = __hiloint2double((hi & 0x800fffff) | 0x3fe00000, __double2loint(d));
-    const float r = (float)exponent_of(d) + lg2((float)f);
-    return d > 0.0 ? r : NEG_INF_F;
-}
-// Order-preserving key of a nonnegative double for running minima over what must stay above the range bound: the high
-// word minus one, unsigned, which sends an exact zero to the top.
-__device__ __forceinline__ unsigned range_key(double d) { return (unsigned)__double2hiint(d) - 1u; }
-__device__ __forceinline__ unsigned range_key_of_bits(int bits) { return ((unsigned)(1023 - bits) << 20) - 1u; }
-
-// Extra dynamic LDS of a linear sweep, behind the role's own (16-byte aligned): three rotating columns [2][64] of
-// doubles, the emission probabilities of main nodes and leaves [Mc][T] each, per step its shift and its stop mark
-// [T+4][2] and the flag (ints).
-__host__ __device__ inline size_t align16(size_t bytes) { return (bytes + 15) & ~(size_t)15; }
-__host__ __device__ inline size_t lin_extra_bytes(int Mc, int T) {
-    return ((size_t)3 * 128 + (size_t)2 * Mc * T) * sizeof(double) + align16((size_t)(2 * (T + 4) + 2) * sizeof(int));
-}
-struct LinLds {
-    double *col0, *col1, *col2, *em, *el;
-    int *kbuf, *flag;
-    __device__ LinLds(double *base, int Mc, int T) {
-        col0 = base;
-        col1 = col0 + 128;
-        col2 = col1 + 128;
-        em = col2 + 128;
-        el = em + Mc * T;
-        kbuf = reinterpret_cast<int *>(el + Mc * T);
-        flag = kbuf + 2 * (T + 4);
-    }
-};
-
-// Emission probabilities of the main-chain nodes and of their leaves, [Mc][T] each, filled by the 256 threads of the
-// table waves; false if one is out of range.
-__device__ __forceinline__ bool lin_fill_emissions(double *em, double *el, const float *__restrict__ mt, int mc, int n, int Mc, int T) {
-    int ok_all = 1;
-    const int cells = Mc * T;
-    for (int i0 = threadIdx.x - 256; i0 < cells; i0 += 8 * 256) {  // eight cells' loads in flight per thread
-        float vm[8], vl[8];
-#pragma unroll
-        for (int k = 0; k < 8; k++) {
-            const int i = min(i0 + k * 256, cells - 1), a_id = i / T, s = i - a_id * T;
-            vm[k] = mt[(size_t)(2 * a_id + 1) * T + s];
-            vl[k] = mt[(size_t)(2 * a_id) * T + s];
-        }
-#pragma unroll
-        for (int k = 0; k < 8; k++) {
-            const int i = i0 + k * 256, a_id = i / T, s = i - a_id * T;
-            if (i < cells) {
-                const bool ok = a_id < mc && s < n;
-                const float bm = ok ? to_b2(vm[k]) : NEG_INF_F, bl = (ok && a_id >= 1) ? to_b2(vl[k]) : NEG_INF_F;
-                ok_all &= lin_input_ok(bm) & lin_input_ok(bl);
-                em[i] = pow2_of(bm);
-                el[i] = pow2_of(bl);
-            }
-        }
-    }
-    return ok_all != 0;
-}
-
-// The emissions a linear-domain sweep staged, as the base-2 logarithms the log-domain sweep works on (all threads of the
-// workgroup; the linear-domain sweep used these numbers, so the sweep that takes over does too).
-__device__ __forceinline__ void lin_emissions_to_logs(const LinLds &x, float *fm, float *fl, int Mc, int T) {
-    for (int i = threadIdx.x; i < Mc * T; i += blockDim.x) {
-        fm[i] = log2_of(x.em[i]);
-        fl[i] = log2_of(x.el[i]);
-    }
-}
-
-// Keeps loaded values (and their loads) in front of the arithmetic that follows, so that all LDS reads of a step are
-// issued back to back instead of two at a time between the multiply-adds.
-__device__ __forceinline__ void pin(double2 &v) { asm volatile("" : "+v"(v.x), "+v"(v.y)); }
-__device__ __forceinline__ void pin(double &v) { asm volatile("" : "+v"(v)); }
-__device__ __forceinline__ void pin(int &v) { asm volatile("" : "+v"(v)); }
-
-struct FwdLinArgs {
-    const float *mt, *lk;
-    float *sm_S, *sm_F0, *sm_F1, *sm_D;
-    double *sm_O;
-    int m, n, mc, Mc, L, T;
-};
-
-// Forward sweep, linear domain, of the wave that owns the nodes 16W .. 16W+15: lane = 4 * node + j, and lane j of a quad
-// takes the children 16q + 4j .. 16q + 4j + 3 of every block of 16, q >= W (the blocks below hold only children left of
-// every node of the wave).  col0: inside probabilities of the column read / written; col1, col2: the row sums of the
-// step, for the table waves.  Returns false if a link is out of range.
-template <int W>
-__device__ __forceinline__ bool fwd_sweep_lin(const LinLds &x, const FwdLinArgs &g, int &stopped_at) {
-    constexpr int MP = 64;
-    const int n = g.n, mc = g.mc, Mc = g.Mc, L = g.L, T = g.T;
-    const int lane = threadIdx.x & 63, j = lane & 3, a_id = 16 * W + (lane >> 2);
-    const bool live = a_id < mc;
-    const int ai = live ? a_id : 0;
-    int ok = 1;
-    double EA0[4][4], EA1[4][4];
-    {
-        float A0[4][4], A1[4][4];
-        const size_t row = (size_t)(2 * min(a_id, Mc - 1) + 1) * 2;
-#pragma unroll
-        for (int q = W; q < 4; q++) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int c = 2 * min(16 * q + 4 * j + i, Mc - 1) + 1;
-                A0[q][i] = g.lk[(row + 0) * L + c];
-                A1[q][i] = g.lk[(row + 1) * L + c];
-            }
-        }
-#pragma unroll
-        for (int q = W; q < 4; q++) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int c_id = 16 * q + 4 * j + i;
-                const bool in = live && c_id < mc && c_id >= a_id;
-                const float b0 = in ? to_b2(A0[q][i]) : NEG_INF_F, b1 = (in && a_id >= 1) ? to_b2(A1[q][i]) : NEG_INF_F;
-                ok &= lin_input_ok(b0) & lin_input_ok(b1);
-                EA0[q][i] = pow2_of(b0);
-                EA1[q][i] = pow2_of(b1);
-            }
-        }
-    }
-    {  // the table cells the sweep never writes (the table waves are busy with the emissions)
-        const int TS = T + 2;
-        const float base_b2 = sanitize(g.mt[(size_t)(g.m - 1) * T + (n - 1)]) * LOG2E_F;  // pcfg_loss.cu:142-147
-        for (int i = threadIdx.x; i < Mc * TS; i += 256) {
-            g.sm_S[i] = (i == (mc - 1) * TS + (n - 1)) ? base_b2 : NEG_INF_F;
-            g.sm_F0[i] = NEG_INF_F;
-            g.sm_F1[i] = NEG_INF_F;
-        }
-    }
-    __syncthreads();  // the table waves have staged the emissions, the first column and the first shift
-    double F1prev = 0.0;
-    double em_p = x.em[ai * T + n - 2], el_p = x.el[ai * T + n - 2], em_t = x.em[ai * T + n - 1];
-    // A stop mark (column t+1 holds a number below the range) ends the loop behind the step that read it, not inside it
-    // - a branch in the middle of the step costs more than the step whose results nobody reads.
-    int stop = 0;
-    for (int t = n - 1; t >= 1 && !stop; t--) {
-        const double2 *cur = reinterpret_cast<const double2 *>(x.col0 + (t & 1) * MP);
-        double2 xv[4][2];
-#pragma unroll
-        for (int q = W; q < 4; q++) {
-            xv[q][0] = cur[8 * q + 2 * j];
-            xv[q][1] = cur[8 * q + 2 * j + 1];
-        }
-        const int2 ks = *reinterpret_cast<const int2 *>(x.kbuf + 2 * t);  // the step's shift and its stop mark
-        int k = ks.x;
-#pragma unroll
-        for (int q = W; q < 4; q++) {
-            pin(xv[q][0]);
-            pin(xv[q][1]);
-        }
-        pin(k);
-        stop = __builtin_amdgcn_readfirstlane(ks.y);
-        stopped_at = stop ? t : stopped_at;
-        const double down = pow2_int(-k);
-        double emd = em_p * down, rest = ((F1prev * down) * el_p) * em_t;
-        pin(emd);
-        pin(rest);
-        double a0 = 0.0, b0 = 0.0, a1 = 0.0, b1 = 0.0;
-#pragma unroll
-        for (int q = W; q < 4; q++) {
-            a0 = __builtin_fma(EA0[q][0], xv[q][0].x, a0);
-            b0 = __builtin_fma(EA0[q][1], xv[q][0].y, b0);
-            a1 = __builtin_fma(EA1[q][0], xv[q][0].x, a1);
-            b1 = __builtin_fma(EA1[q][1], xv[q][0].y, b1);
-            a0 = __builtin_fma(EA0[q][2], xv[q][1].x, a0);
-            b0 = __builtin_fma(EA0[q][3], xv[q][1].y, b0);
-            a1 = __builtin_fma(EA1[q][2], xv[q][1].x, a1);
-            b1 = __builtin_fma(EA1[q][3], xv[q][1].y, b1);
-        }
-        const double s0 = quad_sum_d(a0 + b0), s1 = quad_sum_d(a1 + b1);
-        double x_new = __builtin_fma(emd, s0, rest);
-        if (!live) x_new = 0.0;
-        const double F0 = s0 * down, F1 = s1 * down;
-        F1prev = F1;
-        if (j == 0) {
-            x.col0[((t - 1) & 1) * MP + a_id] = x_new;
-            x.col1[(t & 1) * MP + a_id] = F0;
-            x.col2[(t & 1) * MP + a_id] = F1;
-        }
-        if (t >= 2) {  // the emissions of the next step: they do not wait for the barrier
-            em_t = em_p;
-            em_p = x.em[ai * T + t - 2];
-            el_p = x.el[ai * T + t - 2];
-        }
-        lds_barrier();
-    }
-    return ok != 0;
-}
-
-// The table waves of the forward sweep (role 0: column entries, shifts and offsets; 1, 2: the two row sums; 3: the range
-// watch).  They stage the emissions and the first column, then follow one step behind the sweep: iteration t turns
-// column t and the row sums of step t+1 into table entries; pass t = 0 after the last barrier finishes the job.  The
-// watch looks at what step t-1 will multiply - column t, the row sums F1 of step t+1 (F0 is used up in the step that
-// makes it) - and marks step t-1 if one of them is below the range: the sweep reads the mark with the shift at the top
-// of that step and every wave leaves its loop behind it.  Returns the smallest range key seen in what the sweep stands
-// for; ok: false if an emission is out of range.
-__device__ __forceinline__ unsigned fwd_tables_lin(const LinLds &x, const FwdLinArgs &g, int role, bool &ok, int lin_bits, int &stopped_at) {
-    constexpr int MP = 64;
-    const int n = g.n, mc = g.mc, Mc = g.Mc, T = g.T, TS = g.T + 2, ht = threadIdx.x - 256, node = threadIdx.x & 63;
-    const bool live = node < mc;
-    const float base_b2 = sanitize(g.mt[(size_t)(g.m - 1) * T + (n - 1)]) * LOG2E_F;  // pcfg_loss.cu:142-147
-    ok = lin_fill_emissions(x.em, x.el, g.mt, mc, n, Mc, T) && lin_input_ok(base_b2) != 0;
-    const double x_base = pow2_of(base_b2);
-    const int e_base = exponent_or_none(x_base);
-    const int k_base = e_base == NO_EXPONENT ? 0 : clamp_shift(e_base);  // the first step's shift: from the base cell
-    for (int i = ht; i < 2 * MP; i += 256) {
-        x.col0[i] = (i == ((n - 1) & 1) * MP + mc - 1) ? x_base : 0.0;
-        x.col1[i] = 0.0;
-        x.col2[i] = 0.0;
-    }
-    for (int i = ht; i < TS + 2; i += 256) {
-        g.sm_D[i] = (i == n - 1) ? (float)k_base : 0.f;
-        if (i < TS) g.sm_O[i] = (i == n - 2) ? (double)k_base : 0.0;
-        x.kbuf[2 * i] = (i == n - 1) ? k_base : 0;
-        x.kbuf[2 * i + 1] = 0;
-    }
-    if (ht == 0) *x.flag = 0;
-    __syncthreads();
-    unsigned lowest = ~0u;
-    int k_last = k_base;       // k_t at iteration t
-    double O_run = k_base;     // O[t-1] at iteration t
-    const unsigned too_small = range_key_of_bits(lin_bits);
-    for (int t = n - 1; t >= 0; t--) {
-        // the sweep stops behind step t if that step is marked; what this pass then makes of column t (which step t+1
-        // computed from the numbers that stopped it) is overwritten by the sweep that takes over, and is not vouched for
-        const int mark = x.kbuf[2 * t + 1];
-        unsigned seen = lowest;
-        if (role == 0) {
-            const double v = x.col0[(t & 1) * MP + node];
-            if (t >= 2) {
-                // O[t-2] becomes the absolute exponent of the largest entry of column t: the shift of step t-1 is what is
-                // left of that exponent (relative to O[t]) after the shift of step t
-                const int e = wave_max_i(exponent_or_none(v));
-                const int k = e == NO_EXPONENT ? 0 : clamp_shift(e - k_last);
-                if (node == 0) {
-                    x.kbuf[2 * (t - 1)] = k;
-                    g.sm_D[t - 1] = (float)k;
-                    O_run += (double)k;
-                    g.sm_O[t - 2] = O_run;
-                }
-                k_last = k;
-            }
-            if (t < n - 1 && live) g.sm_S[node * TS + t] = log2_of(v);
-            seen = min(lowest, range_key(v));
-        } else if (role <= 2 && t < n - 1) {
-            const double v = (role == 1 ? x.col1 : x.col2)[((t + 1) & 1) * MP + node];
-            if (live) (role == 1 ? g.sm_F0 : g.sm_F1)[node * TS + t + 1] = log2_of(v);
-            seen = min(lowest, range_key(v));
-        } else if (role == 3 && t >= 1) {
-            const double v = x.col0[(t & 1) * MP + node], f1 = x.col2[((t + 1) & 1) * MP + node];
-            const bool below = min(range_key(v), range_key(f1)) < too_small;
-            if (__builtin_amdgcn_ballot_w64(below) != 0 && node == 0) x.kbuf[2 * (t - 1) + 1] = 1;
-        }
-        if (t >= 1) lds_barrier();
-        if (mark != 0) {
-            stopped_at = t;  // (0: marked while the last step ran - the caller finds that in the mark itself)
-            break;
-        }
-        lowest = seen;
-    }
-    return lowest;
-}
-
-// The forward sweep of a sentence in the linear domain (R = 1, tables in LDS): fills sm_S, sm_F0, sm_F1, hd.D, hd.O like
-// the log-domain code of inside_fwd_ml1_body.  Returns (workgroup-uniform) 0 if the sweep is complete; t >= 1 if it stopped
-// with column t as the last one it can vouch for - sm_S[.][t..], sm_F0/sm_F1[.][t+1..], hd.D[t+1..], hd.O[t..] are in
-// place and the log-domain sweep takes over from there; -1 if nothing of it can be used (an input out of range).
-// `lin` is the extra LDS (lin_extra_bytes(Mc, T)).
-__device__ __forceinline__ int inside_fwd_lin_attempt(const float *__restrict__ mt, const float *__restrict__ lk, const LdsHead &hd,
-                                                     float *sm_S, float *sm_F0, float *sm_F1, double *lin, int m, int n, int L, int T,
-                                                     int Mc, int lin_bits) {
-    const LinLds x(lin, Mc, T);
-    const FwdLinArgs g{mt, lk, sm_S, sm_F0, sm_F1, hd.D, hd.O, m, n, m / 2, Mc, L, T};
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    unsigned lowest = ~0u;
-    bool ok;
-    int stopped_at = 0;  // the step in front of which the sweep stopped (every wave leaves its loop at the same one)
-    switch (wave) {  // wave-uniform; every branch meets the same barriers
-        case 0: ok = fwd_sweep_lin<0>(x, g, stopped_at); break;
-        case 1: ok = fwd_sweep_lin<1>(x, g, stopped_at); break;
-        case 2: ok = fwd_sweep_lin<2>(x, g, stopped_at); break;
-        case 3: ok = fwd_sweep_lin<3>(x, g, stopped_at); break;
-        default: lowest = fwd_tables_lin(x, g, 7 - wave, ok, lin_bits, stopped_at); break;  // role 0 beside the sweep wave with the fewest children
-    }
-    if (!ok || lowest < range_key_of_bits(LIN_FLOOR_BITS)) *x.flag = 1;
-    __syncthreads();
-    const bool good = *x.flag == 0;
-    // a number below the range in column 1 (or in the F1 of step 2) is met while the last step runs: that step is redone
-    const int resume_at = stopped_at > 0 ? stopped_at + 1 : (x.kbuf[1] != 0 ? 1 : 0);
-    if (threadIdx.x == 0) atomicAdd(good && resume_at == 0 ? &g_linear_swept : &g_linear_handed_over, 1ull);
-    __syncthreads();  // the flag's cell may be written again by the log-domain sweep's staging
-    return good ? resume_at : -1;
-}
-
 // Forward.  Dynamic LDS: head (see LdsHead), col[2][64R]; with TAB_LDS also the emissions of main nodes and of their
 // leaves [Mc][T] and the R, F0h, F1h tables [Mc][T+2] (all base 2), which are copied out in bulk when the sweep is over -
 // the sweep itself then touches no global memory.
 template <int R, bool TAB_LDS>
 __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__restrict__ match_all, const float *__restrict__ links,
                                                    const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
-                                                   float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc,
-                                                   int lin_bits = 0) {
+                                                   float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc) {
     constexpr int NQ = 8 * R;
     constexpr int MP = 64 * R;
     const int TS = T + 2;
@@ -707,13 +305,6 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
     }
     const int mc = m / 2;  // active main-chain nodes: a_id < mc
 
-    // the linear-domain sweep first, where the launch brought the LDS for it; what it cannot follow is swept below
-    int resume_at = -1;  // 0: swept; t >= 1: the sweep below takes over at column t; -1: it starts from the base cell
-    if (R == 1 && TAB_LDS && lin_bits > 0)
-        resume_at = inside_fwd_lin_attempt(mt, lk, hd, sm_S, sm_F0, sm_F1,
-                                           reinterpret_cast<double *>(smem + fwd_role_floats(Mc, T)), m, n, L, T, Mc, lin_bits);
-    if (resume_at != 0) {
-    const int t_start = resume_at > 0 ? resume_at : n - 1;
     // link slabs -> registers; the loads are unconditional (clamped addresses) so that they are all in flight together
     float A0[R][NQ], A1[R][NQ];
 #pragma unroll
@@ -729,21 +320,17 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
     }
     const float base_cell = sanitize(mt[(size_t)(m - 1) * T + (n - 1)]);  // pcfg_loss.cu:142-147
     if (TAB_LDS) {
-        if (resume_at > 0) {
-            lin_emissions_to_logs(LinLds(reinterpret_cast<double *>(smem + fwd_role_floats(Mc, T)), Mc, T), sm_main, sm_leaf, Mc, T);
-        } else {
-            for (int i = tid; i < Mc * T; i += NTR) {
-                const int a_id = i / T, s = i - a_id * T;
-                const float vm = mt[(size_t)(2 * a_id + 1) * T + s], vl = mt[(size_t)(2 * a_id) * T + s];
-                const bool ok = a_id < mc && s < n;
-                sm_main[i] = ok ? to_b2(vm) : NEG_INF_F;
-                sm_leaf[i] = (ok && a_id >= 1) ? to_b2(vl) : NEG_INF_F;
-            }
-            for (int i = tid; i < Mc * TS; i += NTR) {
-                sm_S[i] = (i == (mc - 1) * TS + (n - 1)) ? base_cell * LOG2E_F : NEG_INF_F;
-                sm_F0[i] = NEG_INF_F;
-                sm_F1[i] = NEG_INF_F;
-            }
+        for (int i = tid; i < Mc * T; i += NTR) {
+            const int a_id = i / T, s = i - a_id * T;
+            const float vm = mt[(size_t)(2 * a_id + 1) * T + s], vl = mt[(size_t)(2 * a_id) * T + s];
+            const bool ok = a_id < mc && s < n;
+            sm_main[i] = ok ? to_b2(vm) : NEG_INF_F;
+            sm_leaf[i] = (ok && a_id >= 1) ? to_b2(vl) : NEG_INF_F;
+        }
+        for (int i = tid; i < Mc * TS; i += NTR) {
+            sm_S[i] = (i == (mc - 1) * TS + (n - 1)) ? base_cell * LOG2E_F : NEG_INF_F;
+            sm_F0[i] = NEG_INF_F;
+            sm_F1[i] = NEG_INF_F;
         }
     } else {
         // cells of S and R the sweep never writes: rows beyond the sentence, columns from n-1 on (except the base cell)
@@ -756,23 +343,12 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
             }
         }
     }
-    double O_start = 0.0;
-    if (TAB_LDS && resume_at > 0) {
-        // column t_start as the linear-domain sweep left it in the table, its maximum as the shift of the first step
-        const int node = tid & 63;
-        const float own = node < mc ? sm_S[node * TS + t_start] : NEG_INF_F;
-        const float col_max = wave_max(own);
-        if (tid < MP) col[(t_start & 1) * MP + tid] = own;
-        if (tid < 16) hd.slots[tid] = col_max;
-        O_start = hd.O[t_start];
-    } else {
-        for (int i = tid; i < MP; i += NTR) col[((n - 1) & 1) * MP + i] = (i == mc - 1) ? base_cell * LOG2E_F : NEG_INF_F;
-        for (int i = tid; i < TS + 2; i += NTR) {
-            hd.D[i] = 0.f;
-            if (i < TS) hd.O[i] = 0.0;
-        }
-        if (tid < 16) hd.slots[tid] = base_cell * LOG2E_F;  // maximum of column n-1
+    for (int i = tid; i < MP; i += NTR) col[((n - 1) & 1) * MP + i] = (i == mc - 1) ? base_cell * LOG2E_F : NEG_INF_F;
+    for (int i = tid; i < TS + 2; i += NTR) {
+        hd.D[i] = 0.f;
+        if (i < TS) hd.O[i] = 0.0;
     }
+    if (tid < 16) hd.slots[tid] = base_cell * LOG2E_F;  // maximum of column n-1
 #pragma unroll
     for (int r = 0; r < R; r++) {
         const int a_id = 64 * r + 8 * p + g8;
@@ -785,7 +361,7 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
         }
     }
     __syncthreads();
-    FwdSweepArgs sa{col, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, av.F0, av.F1, av.SR, hd.slots, hd.D, hd.O, base_cell * LOG2E_F, n, mc, Mc, T, j, g8, t_start, O_start};
+    FwdSweepArgs sa{col, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, av.F0, av.F1, av.SR, hd.slots, hd.D, hd.O, base_cell * LOG2E_F, n, mc, Mc, T, j, g8};
     switch (p) {  // wave-uniform: every wave runs the sweep specialised for its node block
         case 0: fwd_sweep<R, TAB_LDS, 0>(A0, A1, sa); break;
         case 1: fwd_sweep<R, TAB_LDS, 1>(A0, A1, sa); break;
@@ -795,7 +371,6 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
         case 5: fwd_sweep<R, TAB_LDS, 5>(A0, A1, sa); break;
         case 6: fwd_sweep<R, TAB_LDS, 6>(A0, A1, sa); break;
         default: fwd_sweep<R, TAB_LDS, 7>(A0, A1, sa); break;
-    }
     }
     if (TAB_LDS) {
         for (int i = tid; i < Mc * TS; i += NTR) {
@@ -816,9 +391,8 @@ __device__ __forceinline__ void inside_fwd_ml1_body(const int b, const float *__
 template <int R, bool TAB_LDS>
 __global__ __launch_bounds__(NTR) void inside_fwd_ml1_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
                                                             const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
-                                                            float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc,
-                                                            int lin_bits) {
-    inside_fwd_ml1_body<R, TAB_LDS>(blockIdx.x, match_all, links, out_len, tgt_len, S, aux, L, T, Mc, lin_bits);
+                                                            float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc) {
+    inside_fwd_ml1_body<R, TAB_LDS>(blockIdx.x, match_all, links, out_len, tgt_len, S, aux, L, T, Mc);
 }
 
 struct BwdSweepArgs {
@@ -1183,7 +757,7 @@ __global__ __launch_bounds__(NTR) void inside_fused_ml1_kernel(const float *__re
     }
     __syncthreads();
     {
-        FwdSweepArgs sa{w0, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, nullptr, nullptr, nullptr, hd.slots, hd.D, hd.O, base_cell * LOG2E_F, n, mc, Mc, T, j, g8, n - 1, 0.0};
+        FwdSweepArgs sa{w0, sm_main, sm_leaf, sm_S, sm_F0, sm_F1, mt, Sb, nullptr, nullptr, nullptr, hd.slots, hd.D, hd.O, base_cell * LOG2E_F, n, mc, Mc, T, j, g8};
         switch (p) {
             case 0: fwd_sweep<R, true, 0>(A0, A1, sa); break;
             case 1: fwd_sweep<R, true, 1>(A0, A1, sa); break;
@@ -1308,9 +882,6 @@ struct OutsideFreeArgs {
     float *sm_E;                   // [T+4] shifts
     double *sm_P;                  // [T+4] offsets
     int n, mc, T, j, g8, wave;
-    // first step: 1 or, taking over from a linear-domain sweep that ran out of range, a later one, whose weight columns
-    // are in w0, w1, with the betas of the column before it in sm_B and its shift and offset in sm_E, sm_P
-    int t_start;
 };
 
 template <int P>
@@ -1321,10 +892,10 @@ __device__ __forceinline__ void outside_sweep_free(const float (&A0)[1][8], cons
     const int q_end = P + 1;  // chunks beyond hold only parents a > c
     const bool live = c_id < x.mc;
     const int ci = live ? c_id : 0;
-    float bprev = live ? x.sm_B[ci * TS + x.t_start - 1] : NEG_INF_F;  // relative beta of column t-1 (beta[root][0] = 0)
-    float e_cur = x.sm_E[x.t_start];                                   // E_t
-    double Pt = x.sm_P[x.t_start];                                     // P_t
-    for (int t = x.t_start; t <= x.n - 1; t++) {
+    float bprev = live ? x.sm_B[ci * TS] : NEG_INF_F;  // relative beta of column t-1 (beta[root][0] = 0)
+    float e_cur = x.sm_E[1];                           // E_t
+    double Pt = x.sm_P[1];                             // P_t
+    for (int t = 1; t <= x.n - 1; t++) {
         const float *c0 = x.w0 + (t & 1) * MP, *c1 = x.w1 + (t & 1) * MP;
         float *n0 = x.w0 + ((t + 1) & 1) * MP, *n1 = x.w1 + ((t + 1) & 1) * MP;
         float u0[NQ], u1[NQ];
@@ -1387,226 +958,6 @@ __device__ __forceinline__ void outside_sweep_free(const float (&A0)[1][8], cons
     }
 }
 
-struct OutsideLinArgs {
-    const float *mt, *lk;
-    float *sm_B, *sm_W0, *sm_W1, *sm_E;
-    double *sm_P;
-    int n, mc, Mc, L, T;
-};
-
-// Outside sweep, linear domain, of the wave that owns the children 16W .. 16W+15: lane = 4 * node + j, and lane j of a
-// quad takes the parents 16q + 4j .. 16q + 4j + 3 of every block of 16, q <= W (the blocks beyond hold only parents
-// right of every node of the wave).  col0, col1: the weights W0_t, W1_t the parents offer (read at step t, written
-// for t+1); col2: the betas, for the table waves.  Returns false if a link is out of range.
-template <int W>
-__device__ __forceinline__ bool outside_sweep_lin(const LinLds &x, const OutsideLinArgs &g, int &stopped_at) {
-    constexpr int NB = W + 1, MP = 64;
-    const int n = g.n, mc = g.mc, Mc = g.Mc, L = g.L, T = g.T;
-    const int lane = threadIdx.x & 63, j = lane & 3, c_id = 16 * W + (lane >> 2);
-    const bool live = c_id < mc;
-    const int ci = live ? c_id : 0;
-    int ok = 1;
-    double EA0[NB][4], EA1[NB][4];
-    {
-        float A0[NB][4], A1[NB][4];
-        const int c = 2 * min(c_id, Mc - 1) + 1;
-#pragma unroll
-        for (int q = 0; q < NB; q++) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const size_t row = (size_t)(2 * min(16 * q + 4 * j + i, Mc - 1) + 1) * 2;
-                A0[q][i] = g.lk[(row + 0) * L + c];
-                A1[q][i] = g.lk[(row + 1) * L + c];
-            }
-        }
-#pragma unroll
-        for (int q = 0; q < NB; q++) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int a_id = 16 * q + 4 * j + i;
-                const bool in = live && a_id < mc && a_id <= c_id;
-                const float b0 = in ? to_b2(A0[q][i]) : NEG_INF_F, b1 = (in && a_id >= 1) ? to_b2(A1[q][i]) : NEG_INF_F;
-                ok &= lin_input_ok(b0) & lin_input_ok(b1);
-                EA0[q][i] = pow2_of(b0);
-                EA1[q][i] = pow2_of(b1);
-            }
-        }
-    }
-    {  // the table cells the sweep never writes (the table waves are busy with the emissions)
-        const int TS = T + 2;
-        for (int i = threadIdx.x; i < Mc * TS; i += 256) {
-            g.sm_B[i] = NEG_INF_F;
-            g.sm_W0[i] = NEG_INF_F;
-            g.sm_W1[i] = NEG_INF_F;
-        }
-    }
-    __syncthreads();  // the table waves have staged the emissions and the first columns
-    double bprev = (c_id == 0) ? 1.0 : 0.0;  // beta[root][0] = 0
-    int e_cur = 0;
-    double em_t = live ? x.em[ci * T + 1] : 0.0, el_p = live ? x.el[ci * T + 0] : 0.0;
-    int stop = 0;  // as in the forward sweep: the loop ends behind the step that read a stop mark
-    for (int t = 1; t <= n - 1 && !stop; t++) {
-        const double2 *c0 = reinterpret_cast<const double2 *>(x.col0 + (t & 1) * MP);
-        const double2 *c1 = reinterpret_cast<const double2 *>(x.col1 + (t & 1) * MP);
-        double2 u0[NB][2], u1[NB][2];
-#pragma unroll
-        for (int q = 0; q < NB; q++) {
-            u0[q][0] = c0[8 * q + 2 * j];
-            u0[q][1] = c0[8 * q + 2 * j + 1];
-            u1[q][0] = c1[8 * q + 2 * j];
-            u1[q][1] = c1[8 * q + 2 * j + 1];
-        }
-        const int2 ks = *reinterpret_cast<const int2 *>(x.kbuf + 2 * t);  // the step's shift and its stop mark
-        int e_next = ks.x;
-#pragma unroll
-        for (int q = 0; q < NB; q++) {
-            pin(u0[q][0]);
-            pin(u0[q][1]);
-            pin(u1[q][0]);
-            pin(u1[q][1]);
-        }
-        pin(e_next);
-        stop = __builtin_amdgcn_readfirstlane(ks.y);
-        stopped_at = stop ? t : stopped_at;
-        // what of the weights offered at the next two positions does not wait for this step's sum
-        double emd = pow2_int(-e_next) * em_t;
-        double nw1 = ((bprev * pow2_int(-(e_next + e_cur))) * el_p) * em_t;
-        pin(emd);
-        pin(nw1);
-        double a0 = 0.0, b0 = 0.0, a1 = 0.0, b1 = 0.0;
-#pragma unroll
-        for (int q = 0; q < NB; q++) {
-            a0 = __builtin_fma(EA0[q][0], u0[q][0].x, a0);
-            b0 = __builtin_fma(EA0[q][1], u0[q][0].y, b0);
-            a1 = __builtin_fma(EA1[q][0], u1[q][0].x, a1);
-            b1 = __builtin_fma(EA1[q][1], u1[q][0].y, b1);
-            a0 = __builtin_fma(EA0[q][2], u0[q][1].x, a0);
-            b0 = __builtin_fma(EA0[q][3], u0[q][1].y, b0);
-            a1 = __builtin_fma(EA1[q][2], u1[q][1].x, a1);
-            b1 = __builtin_fma(EA1[q][3], u1[q][1].y, b1);
-        }
-        const double beta = quad_sum_d((a0 + b0) + (a1 + b1));  // (zero for children beyond the sentence: their link columns are)
-        const double nw0 = beta * emd;
-        bprev = beta;
-        if (j == 0) {
-            x.col0[((t + 1) & 1) * MP + c_id] = nw0;
-            x.col1[((t + 1) & 1) * MP + c_id] = nw1;
-            x.col2[(t & 1) * MP + c_id] = beta;
-        }
-        e_cur = e_next;
-        if (t + 1 <= n - 1) {  // the emissions of the next step: they do not wait for the barrier
-            em_t = live ? x.em[ci * T + t + 1] : 0.0;
-            el_p = live ? x.el[ci * T + t] : 0.0;
-        }
-        lds_barrier();
-    }
-    return ok != 0;
-}
-
-// The table waves of the outside sweep (role 0: betas, shifts and offsets; 1, 2: the two weights; 3: the range watch).
-// They stage the emissions and the first columns, then follow one step behind the sweep: iteration t turns the betas of
-// step t-1 and the weight columns W0_t, W1_t into table entries; pass t = n after the last barrier finishes the job.
-// The watch looks at the same numbers - what step t reads - and marks step t+1 if one of them is below the range (the
-// results of step t then cannot be trusted): the sweep reads the mark with the shift at the top of that step and every
-// wave leaves its loop behind it.  Returns the smallest range key seen in what the sweep stands for; ok: false if an
-// emission is out of range.
-__device__ __forceinline__ unsigned outside_tables_lin(const LinLds &x, const OutsideLinArgs &g, int role, bool &ok, int lin_bits,
-                                                       int &stopped_at) {
-    constexpr int MP = 64;
-    const int n = g.n, mc = g.mc, Mc = g.Mc, T = g.T, TS = g.T + 2, TP = g.T + 4, ht = threadIdx.x - 256, node = threadIdx.x & 63;
-    const bool live = node < mc;
-    const float w00_b2 = to_b2(g.mt[(size_t)1 * T + 0]);  // W0_1: the root offers match[root][0] to its null-left children
-    ok = lin_fill_emissions(x.em, x.el, g.mt, mc, n, Mc, T);
-    for (int i = ht; i < 2 * MP; i += 256) {
-        x.col0[i] = (i == 1 * MP + 0) ? pow2_of(w00_b2) : 0.0;
-        x.col1[i] = 0.0;
-        x.col2[i] = (i == 0) ? 1.0 : 0.0;  // beta column 0
-    }
-    for (int i = ht; i < TP; i += 256) {
-        g.sm_E[i] = 0.f;
-        g.sm_P[i] = 0.0;
-        x.kbuf[2 * i] = 0;
-        x.kbuf[2 * i + 1] = 0;
-    }
-    if (ht == 0) *x.flag = 0;
-    __syncthreads();
-    unsigned lowest = ~0u;
-    int k_last = 0, k_before = 0;  // E_{t+1}, E_t at iteration t
-    double P_run = 0.0;            // P[t+1] at iteration t
-    const unsigned too_small = range_key_of_bits(lin_bits);
-    for (int t = 1; t <= n; t++) {
-        // the sweep stops behind step t if that step is marked; what this pass then makes of the columns of step t-1
-        // (computed from the numbers that stopped it) is overwritten by the sweep that takes over, and is not vouched for
-        const int mark = x.kbuf[2 * t + 1];
-        unsigned seen = lowest;
-        if (role == 0) {
-            const double v = x.col2[((t - 1) & 1) * MP + node];
-            if (t + 1 <= n - 1) {
-                // P[t+2] becomes the absolute exponent of the largest beta of column t-1: the shift of step t+1 is what is
-                // left of that exponent (relative to P[t-1]) after the shifts of the steps t-1 and t
-                const int e = wave_max_i(exponent_or_none(v));
-                const int k = e == NO_EXPONENT ? 0 : clamp_shift(e - k_last - k_before);
-                if (node == 0) {
-                    x.kbuf[2 * (t + 1)] = k;
-                    g.sm_E[t + 2] = (float)k;
-                    P_run += (double)k;
-                    g.sm_P[t + 2] = P_run;
-                }
-                k_before = k_last;
-                k_last = k;
-            }
-            if (live) g.sm_B[node * TS + t - 1] = log2_of(v);
-            seen = min(lowest, range_key(v));
-        } else if (role <= 2) {
-            const double v = (role == 1 ? x.col0 : x.col1)[(t & 1) * MP + node];
-            if (live) (role == 1 ? g.sm_W0 : g.sm_W1)[node * TS + t] = log2_of(v);
-            seen = min(lowest, range_key(v));
-        } else if (t <= n - 1) {
-            const double bt = x.col2[((t - 1) & 1) * MP + node], u0 = x.col0[(t & 1) * MP + node], u1 = x.col1[(t & 1) * MP + node];
-            const bool below = min(range_key(bt), min(range_key(u0), range_key(u1))) < too_small;
-            if (__builtin_amdgcn_ballot_w64(below) != 0 && node == 0) x.kbuf[2 * (t + 1) + 1] = 1;
-        }
-        if (t <= n - 1) lds_barrier();
-        if (mark != 0) {
-            stopped_at = t;  // (n: marked while the last step ran; the sweep waves find that in the mark itself)
-            break;
-        }
-        lowest = seen;
-    }
-    return lowest;
-}
-
-// The outside sweep of a sentence in the linear domain: fills sm_B, sm_W0, sm_W1, sm_E, sm_P like the log-domain code of
-// inside_outside_ml1_body.  Returns (workgroup-uniform) 0 if the sweep is complete; t >= 1 if step t is the first it
-// cannot vouch for - sm_W0/sm_W1[.][..t], sm_B[.][..t-1], sm_E[..t], sm_P[..t] are in place and the log-domain sweep
-// takes over from there; -1 if nothing of it can be used (an input out of range).
-// `lin` is the extra LDS (lin_extra_bytes(Mc, T)).
-__device__ __forceinline__ int inside_outside_lin_attempt(const float *__restrict__ mt, const float *__restrict__ lk, double *sm_P,
-                                                         float *sm_E, float *sm_B, float *sm_W0, float *sm_W1, double *lin, int m, int n,
-                                                         int L, int T, int Mc, int lin_bits) {
-    const LinLds x(lin, Mc, T);
-    const OutsideLinArgs g{mt, lk, sm_B, sm_W0, sm_W1, sm_E, sm_P, n, m / 2, Mc, L, T};
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    unsigned lowest = ~0u;
-    bool ok;
-    int stopped_at = 0;  // the step in front of which the sweep stopped (every wave leaves its loop at the same one)
-    switch (wave) {  // wave-uniform; every branch meets the same barriers
-        case 0: ok = outside_sweep_lin<0>(x, g, stopped_at); break;
-        case 1: ok = outside_sweep_lin<1>(x, g, stopped_at); break;
-        case 2: ok = outside_sweep_lin<2>(x, g, stopped_at); break;
-        case 3: ok = outside_sweep_lin<3>(x, g, stopped_at); break;
-        default: lowest = outside_tables_lin(x, g, wave - 4, ok, lin_bits, stopped_at); break;
-    }
-    if (!ok || lowest < range_key_of_bits(LIN_FLOOR_BITS)) *x.flag = 1;
-    __syncthreads();
-    const bool good = *x.flag == 0;
-    // a number below the range among what the last step reads is met while that step runs: it is redone
-    const int resume_at = (stopped_at > 0 && stopped_at < n) ? stopped_at - 1 : (x.kbuf[2 * n + 1] != 0 ? n - 1 : 0);
-    if (threadIdx.x == 0) atomicAdd(good && resume_at == 0 ? &g_linear_swept : &g_linear_handed_over, 1ull);
-    __syncthreads();
-    return good ? resume_at : -1;
-}
-
 // Dynamic LDS of the outside role: P [T+4] (double), slots [16], E [T+4], w0 [2][64], w1 [2][64], Bh, W0h, W1h [Mc][T+2],
 // emissions of main nodes and leaves [Mc][T].
 __host__ __device__ inline size_t outside_role_bytes(int Mc, int T) {
@@ -1616,7 +967,7 @@ __host__ __device__ inline size_t outside_role_bytes(int Mc, int T) {
 __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float *__restrict__ match_all,
                                                        const float *__restrict__ links, const int64_t *__restrict__ out_len,
                                                        const int64_t *__restrict__ tgt_len, float *__restrict__ aux, int L, int T,
-                                                       int Mc, int lin_bits) {
+                                                       int Mc) {
     constexpr int NQ = 8, MP = 64;
     const int TS = T + 2, TP = T + 4;
     extern __shared__ double smem_d[];
@@ -1640,12 +991,6 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
     const float *lk = links + (size_t)b * L * 2 * L;
     AuxView av(aux, b, Mc, T);
 
-    // the linear-domain sweep first, where the launch brought the LDS for it; what it cannot follow is swept below
-    int resume_at = -1;  // 0: swept; t >= 1: the sweep below takes over at step t; -1: it starts from the root
-    double *lin = reinterpret_cast<double *>(reinterpret_cast<char *>(smem_d) + align16(outside_role_bytes(Mc, T)));
-    if (lin_bits > 0) resume_at = inside_outside_lin_attempt(mt, lk, sm_P, sm_E, sm_B, sm_W0, sm_W1, lin, m, n, L, T, Mc, lin_bits);
-    if (resume_at != 0) {
-    const int t_start = resume_at > 0 ? resume_at : 1;
     // transposed link slabs: this thread's group owns child c, its lanes the parents a <= c; unconditional loads
     const int own = 8 * p + g8;
     float A0[1][NQ], A1[1][NQ];
@@ -1658,18 +1003,6 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
             A1[0][q] = lk[(row + 1) * L + c];
         }
     }
-    if (resume_at > 0) {
-        // the weight columns of step t_start as the linear-domain sweep left them in the tables, the maximum of the beta
-        // column before them as the shift of the first step
-        lin_emissions_to_logs(LinLds(lin, Mc, T), sm_main, sm_leaf, Mc, T);
-        const int node = tid & 63;
-        const float col_max = wave_max(node < mc ? sm_B[node * TS + t_start - 1] : NEG_INF_F);
-        if (tid < MP) {
-            w0[(t_start & 1) * MP + tid] = tid < mc ? sm_W0[tid * TS + t_start] : NEG_INF_F;
-            w1[(t_start & 1) * MP + tid] = tid < mc ? sm_W1[tid * TS + t_start] : NEG_INF_F;
-        }
-        if (tid < 16) slots[tid] = col_max;
-    } else {
     for (int i = tid; i < Mc * T; i += NTR) {
         const int a_id = i / T, s = i - a_id * T;
         const float vm = mt[(size_t)(2 * a_id + 1) * T + s], vl = mt[(size_t)(2 * a_id) * T + s];
@@ -1691,7 +1024,6 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
         sm_P[i] = 0.0;
     }
     if (tid < 16) slots[tid] = (tid < 8) ? 0.f : NEG_INF_F;  // maximum of the relative beta column 0
-    }
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
         const int a_id = j + 8 * q;
@@ -1700,14 +1032,14 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
         A1[0][q] = (ok && a_id >= 1) ? to_b2(A1[0][q]) : NEG_INF_F;
     }
     __syncthreads();
-    if (tid == 0 && resume_at < 0) {  // W_1 columns: the root offers match[root][0] to its null-left children
+    if (tid == 0) {  // W_1 columns: the root offers match[root][0] to its null-left children
         const float w00 = sm_main[0];
         w0[1 * MP + 0] = w00;
         sm_W0[0 * TS + 1] = w00;
     }
     __syncthreads();
     {
-        OutsideFreeArgs sa{w0, w1, sm_B, sm_W0, sm_W1, sm_main, sm_leaf, slots, sm_E, sm_P, n, mc, T, j, g8, (tid >> 6), t_start};
+        OutsideFreeArgs sa{w0, w1, sm_B, sm_W0, sm_W1, sm_main, sm_leaf, slots, sm_E, sm_P, n, mc, T, j, g8, (tid >> 6)};
         switch (p) {  // wave-uniform
             case 0: outside_sweep_free<0>(A0, A1, sa); break;
             case 1: outside_sweep_free<1>(A0, A1, sa); break;
@@ -1718,7 +1050,6 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
             case 6: outside_sweep_free<6>(A0, A1, sa); break;
             default: outside_sweep_free<7>(A0, A1, sa); break;
         }
-    }
     }
     __syncthreads();
     for (int i = tid; i < Mc * TS; i += NTR) {
@@ -1732,11 +1063,9 @@ __device__ __forceinline__ void inside_outside_ml1_body(const int b, const float
     }
 }
 
-// Workgroups per sentence that zero the rows of its pad nodes (see PadFill): PadFill::with_sweeps of them beside the
-// sweeps, the others beside the posteriors.  One fill workgroup per compute unit on the units the sweeps leave free
-// writes about 4.3 TB/s: beside the log-domain sweeps (29 us) the whole fill fits, beside the shorter linear-domain
-// ones (20 us) two thirds of it.
-constexpr int PAD_WGS = 32, PAD_WGS_BESIDE_LINEAR_SWEEPS = 22;
+// Workgroups per sentence that zero the rows of its pad nodes (see PadFill) beside the sweeps.  One fill workgroup per
+// compute unit on the units the sweeps leave free writes about 4.3 TB/s: beside the sweeps (29 us) the whole fill fits.
+constexpr int PAD_WGS = 32;
 // The fill rides along while the sweeps take up no more than three quarters of the compute units (192 of 256 on MI355X).
 inline int pad_max_sweep_wgs() { return device_compute_units() * 3 / 4; }
 constexpr size_t PAD_EXCLUSIVE_LDS = 84 * 1024;  // more than half of the 160 KB of a gfx950 compute unit
@@ -1770,24 +1099,23 @@ __device__ __forceinline__ void pad_fill_block(const PadFill pad, const int64_t 
     for (int64_t i = lo + tid; i < hi; i += NTF) __builtin_nontemporal_store(zero, v + i);
 }
 
-// 2*nsent workgroups: 2b runs the forward sweep of sentence b, 2b+1 its outside sweep; pad_parts*nsent more when
+// 2*nsent workgroups: 2b runs the forward sweep of sentence b, 2b+1 its outside sweep; PAD_WGS*nsent more when
 // there is a pad-fill task, which land on the compute units the sweeps leave free.
 __global__ __launch_bounds__(NTR) void inside_pair_ml1_kernel(const float *__restrict__ match_all, const float *__restrict__ links,
                                                              const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
                                                              float *__restrict__ S, float *__restrict__ aux, int L, int T, int Mc,
-                                                             int nsent, PadFill pad, int pad_parts, int lin_bits) {
+                                                             int nsent, PadFill pad) {
     if ((int)blockIdx.x >= 2 * nsent) {  // workgroup-uniform
         const int z = (int)blockIdx.x - 2 * nsent;
-        pad_fill_block(pad, out_len, z / pad_parts, z % pad_parts, L);
+        pad_fill_block(pad, out_len, z / PAD_WGS, z % PAD_WGS, L);
         return;
     }
     const int b = blockIdx.x >> 1;
-    if ((blockIdx.x & 1) == 0) inside_fwd_ml1_body<1, true>(b, match_all, links, out_len, tgt_len, S, aux, L, T, Mc, lin_bits);
-    else inside_outside_ml1_body(b, match_all, links, out_len, tgt_len, aux, L, T, Mc, lin_bits);
+    if ((blockIdx.x & 1) == 0) inside_fwd_ml1_body<1, true>(b, match_all, links, out_len, tgt_len, S, aux, L, T, Mc);
+    else inside_outside_ml1_body(b, match_all, links, out_len, tgt_len, aux, L, T, Mc);
 }
 
-// Posteriors from the tables of the two sweeps: grid (16, B), 256 threads (PAD_WGS - pad_parts more workgroups per
-// sentence when there is a pad-fill task).  Workgroup (q, b) owns the parents 4q .. 4q+3 of
+// Posteriors from the tables of the two sweeps: grid (16, B), 256 threads.  Workgroup (q, b) owns the parents 4q .. 4q+3 of
 // sentence b: it writes the rows 8q .. 8q+7 of the links_grad slab (zeros included) and a sixteenth of the match_all_grad
 // cells.  One thread per (parent, child) pair sums both planes over the columns.
 // Dynamic LDS: corr [T+4], R [Mc][T+2], W0h, W1h of the workgroup's parents [4][T+2].
@@ -1795,12 +1123,7 @@ __global__ __launch_bounds__(256) void inside_combine_ml1_kernel(const float *__
                                                                 float *__restrict__ aux, const float *__restrict__ match_all,
                                                                 const float *__restrict__ links, const int64_t *__restrict__ out_len,
                                                                 const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad,
-                                                                float *__restrict__ lgrad, int L, int T, int Mc, Seed seed,
-                                                                PadFill pad, int pad_parts) {
-    if (blockIdx.x >= 16) {  // workgroup-uniform: the part of the pad fill that rides along with this launch
-        pad_fill_block(pad, out_len, blockIdx.y, pad_parts + (int)blockIdx.x - 16, L);
-        return;
-    }
+                                                                float *__restrict__ lgrad, int L, int T, int Mc, Seed seed) {
     const int TS = T + 2, TP = T + 4;
     extern __shared__ float smem[];
     float *corr = smem;               // [TP]
@@ -3851,11 +3174,6 @@ std::atomic<int> g_pipeline_spin_limit_outside{-1};  // side-by-side launch only
 // Largest base-2 exponent a factor of the rule posteriors of long graphs may have on the matrix cores (see
 // links_grad_ml1_stream_kernel); a tile beyond it is recomputed term by term.  pcfgnat_links_grad_range_limit.
 std::atomic<float> g_links_grad_range_limit{120.f};
-// Smallest nonzero number, as a power of two, that the linear-domain sweeps of graphs of up to 130 nodes accept before
-// they hand the sentence to the log-domain sweep (see LIN_INPUT_BITS); 0, the default, switches them off: they pay on
-// emissions that are not peaked and cost on a model that is sure of itself.  pcfgnat_inside_linear_bits.
-std::atomic<int> g_inside_linear_bits{0};
-inline int inside_linear_bits() { return g_inside_linear_bits.load(); }
 int pipeline_chunks(int B, int T, int Mc) {  // NQ, or 0 where the pipelined sweeps do not apply
     const int NQ = stream_mp(Mc) / 64, CL = 64 * NQ / NLP;
     return (NQ >= 2 && NQ <= 8 && T + 2 < 4096 && (int64_t)B * CL <= g_pipeline_max_wg.load()) ? NQ : 0;
@@ -4058,17 +3376,13 @@ int launch_fwd(const float *match_all, const float *links, const int64_t *ol, co
     const size_t with_tab = base + ((size_t)2 * Mc * T + (size_t)3 * Mc * (T + 2)) * sizeof(float);
     if (with_tab <= LDS_BUDGET) {
         auto k = inside_fwd_ml1_kernel<R, true>;
-        // with room for its columns and emission probabilities behind the tables, the sweep runs in the linear domain
-        const size_t with_lin = fwd_role_floats(Mc, T) * sizeof(float) + lin_extra_bytes(Mc, T);
-        const int lin_bits = (R == 1 && with_lin <= LDS_BUDGET) ? inside_linear_bits() : 0;
-        const size_t lds = lin_bits > 0 ? with_lin : with_tab;
-        PCFGNAT_DYNAMIC_LDS(k, lds);
-        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), lds, stream, match_all, links, ol, tl, S, aux, L, T, Mc, lin_bits);
+        PCFGNAT_DYNAMIC_LDS(k, with_tab);
+        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), with_tab, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
     } else {
         auto k = inside_fwd_ml1_kernel<R, false>;
         PCFGNAT_REQUIRE(base <= LDS_BUDGET, "pcfg_loss: target length %d too large for the column offsets in LDS", T);
         PCFGNAT_DYNAMIC_LDS(k, base);
-        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), base, stream, match_all, links, ol, tl, S, aux, L, T, Mc, 0);
+        hipLaunchKernelGGL(k, dim3(B), dim3(NTR), base, stream, match_all, links, ol, tl, S, aux, L, T, Mc);
     }
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
@@ -4102,13 +3416,7 @@ int launch_fused(const float *go, const float *match_all, const float *links, co
     *done = false;
     if (R == 1) {  // the two sweeps side by side as two workgroups per sentence, then the posteriors
         const size_t fwd_bytes = ((size_t)head_floats(T) + 2 * 64 + (size_t)2 * Mc * T + (size_t)3 * Mc * (T + 2)) * sizeof(float);
-        size_t pair_bytes = fwd_bytes > outside_role_bytes(Mc, T) ? fwd_bytes : outside_role_bytes(Mc, T);
-        // with room for their columns and emission probabilities behind the tables, the sweeps run in the linear domain
-        const size_t fwd_lin = fwd_role_floats(Mc, T) * sizeof(float) + lin_extra_bytes(Mc, T);
-        const size_t out_lin = align16(outside_role_bytes(Mc, T)) + lin_extra_bytes(Mc, T);
-        const size_t pair_lin = fwd_lin > out_lin ? fwd_lin : out_lin;
-        const int lin_bits = pair_lin <= LDS_BUDGET ? inside_linear_bits() : 0;
-        if (lin_bits > 0) pair_bytes = pair_lin;
+        const size_t pair_bytes = fwd_bytes > outside_role_bytes(Mc, T) ? fwd_bytes : outside_role_bytes(Mc, T);
         const size_t comb_bytes = ((size_t)(T + 4) + (size_t)Mc * (T + 2) + (size_t)8 * (T + 2)) * sizeof(float);
         if (pair_bytes <= LDS_BUDGET && comb_bytes <= 64 * 1024 && L <= 128) {
             PCFGNAT_REQUIRE(((uintptr_t)aux & 7) == 0, "pcfg_loss_forward_backward: aux must be 8-byte aligned");
@@ -4121,13 +3429,12 @@ int launch_fused(const float *go, const float *match_all, const float *links, co
             const size_t launch_bytes = (fill && pair_bytes < PAD_EXCLUSIVE_LDS) ? PAD_EXCLUSIVE_LDS : pair_bytes;
             if (launch_bytes != pair_bytes)
                 PCFGNAT_DYNAMIC_LDS(inside_pair_ml1_kernel, launch_bytes);
-            const int pad_parts = lin_bits > 0 ? PAD_WGS_BESIDE_LINEAR_SWEEPS : PAD_WGS;
-            hipLaunchKernelGGL(inside_pair_ml1_kernel, dim3((2 + (fill ? pad_parts : 0)) * B), dim3(NTR), launch_bytes, stream, match_all,
-                               links, ol, tl, S, aux, L, T, Mc, B, pad, pad_parts, lin_bits);
+            hipLaunchKernelGGL(inside_pair_ml1_kernel, dim3((2 + (fill ? PAD_WGS : 0)) * B), dim3(NTR), launch_bytes, stream, match_all,
+                               links, ol, tl, S, aux, L, T, Mc, B, pad);
             PCFGNAT_HIP_CHECK(hipGetLastError());
             if (fill && pad_done) *pad_done = true;
-            hipLaunchKernelGGL(inside_combine_ml1_kernel, dim3(16 + (fill ? PAD_WGS - pad_parts : 0), B), dim3(256), comb_bytes, stream,
-                               go, S, aux, match_all, links, ol, tl, mg, lg, L, T, Mc, seed, fill ? pad : PadFill{nullptr, 0}, pad_parts);
+            hipLaunchKernelGGL(inside_combine_ml1_kernel, dim3(16, B), dim3(256), comb_bytes, stream, go, S, aux, match_all, links, ol, tl,
+                               mg, lg, L, T, Mc, seed);
             PCFGNAT_HIP_CHECK(hipGetLastError());
             *done = true;
             return PCFGNAT_OK;
@@ -4168,7 +3475,6 @@ extern "C" void pcfgnat_pipeline_config(int max_workgroups, int spin_limit) {
 extern "C" void pcfgnat_pipeline_outside_spin_limit(int spin_limit) { g_pipeline_spin_limit_outside.store(spin_limit); }
 
 extern "C" void pcfgnat_links_grad_range_limit(float log2_limit) { g_links_grad_range_limit.store(log2_limit); }
-extern "C" void pcfgnat_inside_linear_bits(int bits) { g_inside_linear_bits.store(bits < 0 ? 0 : (bits > LIN_BITS_MAX ? LIN_BITS_MAX : bits)); }
 
 extern "C" int pcfgnat_pipeline_redo_counts(unsigned long long *inside_sweeps, unsigned long long *viterbi_sentences, int reset) {
     PCFGNAT_REQUIRE(inside_sweeps && viterbi_sentences, "pipeline_redo_counts: null pointer");
@@ -4178,18 +3484,6 @@ extern "C" int pcfgnat_pipeline_redo_counts(unsigned long long *inside_sweeps, u
         PCFGNAT_HIP_CHECK(hipMemcpyToSymbol(HIP_SYMBOL(g_inside_redone), &zero, sizeof(zero)));
     }
     return viterbi_redo_count(viterbi_sentences, reset);
-}
-
-extern "C" int pcfgnat_inside_linear_counts(unsigned long long *swept, unsigned long long *handed_over, int reset) {
-    PCFGNAT_REQUIRE(swept && handed_over, "inside_linear_counts: null pointer");
-    PCFGNAT_HIP_CHECK(hipMemcpyFromSymbol(swept, HIP_SYMBOL(g_linear_swept), sizeof(*swept)));
-    PCFGNAT_HIP_CHECK(hipMemcpyFromSymbol(handed_over, HIP_SYMBOL(g_linear_handed_over), sizeof(*handed_over)));
-    if (reset) {
-        const unsigned long long zero = 0;
-        PCFGNAT_HIP_CHECK(hipMemcpyToSymbol(HIP_SYMBOL(g_linear_swept), &zero, sizeof(zero)));
-        PCFGNAT_HIP_CHECK(hipMemcpyToSymbol(HIP_SYMBOL(g_linear_handed_over), &zero, sizeof(zero)));
-    }
-    return PCFGNAT_OK;
 }
 
 extern "C" size_t pcfgnat_pcfg_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml) {

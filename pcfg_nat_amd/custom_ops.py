@@ -61,23 +61,6 @@ def pipeline_redo_counts(reset=False):
     return a.value, b.value
 
 
-def inside_linear_bits(bits=0):
-    """Process-wide setting: the smallest nonzero number, as a power of two, that the linear-domain sweeps of graphs of up to
-    130 nodes accept before the log-domain sweep takes the sentence over at that column (at most 500); 0, the default, switches
-    them off."""
-    _lib.load().pcfgnat_inside_linear_bits(int(bits))
-
-
-def inside_linear_counts(reset=False):
-    """(sweeps completed in the linear domain, sweeps handed over to the log domain from the start or on the way) on the current device since the
-    library was loaded or the last reset; forward and outside sweeps count apart.  Synchronises with the device."""
-    import ctypes
-    lib = _lib.load()
-    a, b = ctypes.c_ulonglong(0), ctypes.c_ulonglong(0)
-    _lib.check(lib.pcfgnat_inside_linear_counts(ctypes.byref(a), ctypes.byref(b), int(bool(reset))), lib)
-    return a.value, b.value
-
-
 def _stream(t):
     return torch.cuda.current_stream(t.device).cuda_stream
 
@@ -1012,14 +995,12 @@ def _criterion_args(name, logits, targets, links, output_length, target_length, 
     return code, B, L, V, T, ml, Mc, targets, links, ol, tl, mm8, keep8
 
 
-def pcfg_criterion_step(logits, targets, links, output_length, target_length, events=None, slices=None, matchmask=None,
+def pcfg_criterion_step(logits, targets, links, output_length, target_length, events=None, matchmask=None,
                         keep_word_mask=None, loss_scale=1.0):
     """The criterion's whole training pass in one native call (``pcfgnat_criterion_step``): ``logits`` [B,L,V] (fp16 or
-    fp32, contiguous) is consumed in place and holds d loss / d logits afterwards.  ``events``: optional list of eight
+    fp32, contiguous) is consumed in place and holds d loss / d logits afterwards.  ``events``: optional list of six
     ``torch.cuda.Event(enable_timing=True)`` (each recorded at least once before; entries may be None) that the library records before/after
-    the gather forward, inside forward, inside backward and gather backward of the first slice.  ``slices``: how many
-    batch slices alternate between the current stream and the library's helper stream (default 1: measured on MI355X the
-    bandwidth-bound gather kernels leave no room for a second kernel on the CUs, so slicing does not pay).
+    the gather forward, the inside forward + backward and the gather backward.
     ``matchmask`` [B,T,L] / ``keep_word_mask`` [B,L] (bool, as the glancing step returns them): the criterion's
     force-emit masking (nat_pcfg_loss.py:116-121); both None = off (``--no-force-emit``).  The rows of the pad nodes at
     or beyond a sentence's ``output_length`` feed nothing (neither sweep reads them, their gradient is zero): the gather
@@ -1033,8 +1014,6 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
     code, B, L, V, T, ml, Mc, targets, links, ol, tl, mm8, keep8 = _criterion_args(
         "pcfg_criterion_step", logits, targets, links, output_length, target_length, matchmask, keep_word_mask)
     dev = logits.device
-    if slices is None:
-        slices = 1
     mm_ptr = mm8.data_ptr() if mm8 is not None else None
     keep_ptr = keep8.data_ptr() if keep8 is not None else None
     scale_host, scale_dev = 1.0, None
@@ -1048,9 +1027,9 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
     ev_arr = None
     if events is not None:
         import ctypes
-        if len(events) != 8:
-            raise RuntimeError("pcfg_criterion_step: events must hold eight torch.cuda.Event objects")
-        ev_arr = (ctypes.c_void_p * 8)(*[(e.cuda_event if e is not None else None) for e in events])
+        if len(events) != 6:
+            raise RuntimeError("pcfg_criterion_step: events must hold six torch.cuda.Event objects")
+        ev_arr = (ctypes.c_void_p * 6)(*[(e.cuda_event if e is not None else None) for e in events])
     with torch.cuda.device(dev):
         match = torch.empty((B, L, T), dtype=torch.float32, device=dev)
         S = torch.empty((B, Mc, T + 2), dtype=torch.float32, device=dev)
@@ -1061,7 +1040,7 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
         out = torch.empty((2,), dtype=torch.float32, device=dev)
         _lib.check(lib.pcfgnat_criterion_step(logits.data_ptr(), code, targets.data_ptr(), links.data_ptr(), ol.data_ptr(),
                                               tl.data_ptr(), mm_ptr, keep_ptr, match.data_ptr(), S.data_ptr(), aux.data_ptr(), mg.data_ptr(),
-                                              lg.data_ptr(), row_lse.data_ptr(), out.data_ptr(), B, L, V, T, ml, slices,
+                                              lg.data_ptr(), row_lse.data_ptr(), out.data_ptr(), B, L, V, T, ml,
                                               scale_host, scale_dev.data_ptr() if scale_dev is not None else None,
                                               _stream(logits), ev_arr), lib)
     return out, lg, S[:, 0, 0], match, mg

@@ -195,14 +195,14 @@ def train_step_fused(logits, targets, links, output_length, target_length, ops=_
     return loss, glinks, ll
 
 
-def train_step_single_call(logits, targets, links, output_length, target_length, ops=_default_ops, mark=None, slices=None,
+def train_step_single_call(logits, targets, links, output_length, target_length, ops=_default_ops, mark=None,
                            matchmask=None, keep_word_mask=None, loss_scale=1.0):
     """``train_step_fused`` issued as one native call (``pcfgnat_criterion_step``): the kernels are enqueued back to
     back by the library and the scalar loss is reduced on the device.  Returns (loss, links_grad, ll)."""
     events = None
     if mark is not None:
-        events = mark("events", 8)  # the caller hands out eight timing events for this step
+        events = mark("events", 6)  # the caller hands out six timing events for this step
     out, glinks, ll, _, _ = ops.pcfg_criterion_step(logits, targets, links, output_length, target_length, events=events,
-                                                 slices=slices, matchmask=matchmask, keep_word_mask=keep_word_mask,
+                                                 matchmask=matchmask, keep_word_mask=keep_word_mask,
                                                  loss_scale=loss_scale)
     return out[0], glinks, ll

@@ -383,46 +383,10 @@ def test_rule_posteriors_term_by_term_path(case):
         ops.links_grad_range_limit()
 
 
-@pytest.mark.parametrize("L,T,ms,ns", [(128, 32, [128, 96, 40, 4], [32, 25, 11, 2]), (64, 48, [64, 30], [48, 9]),
-                                       (130, 20, [130, 66], [20, 12]), (36, 54, [36, 36], [54, 40])])
-def test_inside_linear_and_log_domain_sweeps_agree(L, T, ms, ns):
-    """Graphs of up to 130 nodes can be swept in the linear domain (doubles, one multiply-add per term; an option) where
-    the numbers allow it, and are swept in the log domain otherwise.  Here the same batches go through both - loss and gradients through the
-    two-workgroup pass, the table of the forward kernel alone - and must agree far inside the tolerance either is held
-    to against the oracle; the counters tell that each run took the sweep it was meant to take."""
-    batch = synth.training_batch(len(ms), L, T, 80, ms, ns, seed=3 * L + T)
-    match = _match_for(batch)
-    ol, tl = batch["output_length"].to(DEV), batch["target_length"].to(DEV)
-    runs = {}
-    try:
-        for name, bits in (("linear", 500), ("log", 0)):
-            ops.inside_linear_bits(bits)
-            ops.inside_linear_counts(reset=True)
-            ll, mg, lg = _inside_all(batch, match)
-            S = ops._pcfg_loss_tables(match.to(DEV), batch["links"].to(DEV), ol, tl, 1, "test")[0].cpu()
-            runs[name] = (ll, mg, lg, S, ops.inside_linear_counts())
-    finally:
-        ops.inside_linear_bits()
-    Mc = (L - 2) // 2 + 1
-    if Mc <= 64:
-        assert runs["linear"][4] == (3 * len(ms), 0)  # forward and outside sweep of the pass, forward sweep of the tables
-    else:
-        assert runs["linear"][4] == (0, 0)  # more than one tile of 64 nodes: no linear sweep for these
-    assert runs["log"][4] == (0, 0)
-    (ll_a, mg_a, lg_a, S_a, _), (ll_b, mg_b, lg_b, S_b, _) = runs["linear"], runs["log"]
-    assert torch.equal(torch.isfinite(S_a), torch.isfinite(S_b))
-    fin = torch.isfinite(S_b)
-    assert torch.allclose(S_a[fin], S_b[fin], rtol=2e-6, atol=2e-4)
-    assert torch.allclose(ll_a, ll_b, rtol=2e-6)
-    for got, want in ((mg_a, mg_b), (lg_a, lg_b)):
-        for bi in range(len(ms)):
-            assert (got[bi] - want[bi]).abs().max() <= 2e-5 * max(float(want[bi].abs().max()), 1e-30)
-
-
-def test_inside_linear_sweep_hands_over_what_it_cannot_follow():
+def test_inside_extreme_inputs_vs_oracle():
     """Of four sentences one has an emission 400 nats down, one a link 300 nats down, one a node whose inside value falls
-    2^-600 below its column's largest, one nothing special: the linear sweeps keep the last (both of its sweeps) and hand
-    the others to the log domain, and every sentence comes out right against the float64 oracle."""
+    2^-600 below its column's largest, one nothing special: every sentence comes out right against the float64 oracle (the
+    sweeps work in the log domain relative to per-column offsets, so none of this leaves their range)."""
     L, T, ms, ns = 64, 20, [64, 64, 64, 64], [20, 20, 20, 20]
     batch = synth.training_batch(4, L, T, 80, ms, ns, seed=77)
     match = _match_for(batch).clone()
@@ -433,14 +397,7 @@ def test_inside_linear_sweep_hands_over_what_it_cannot_follow():
     match[2, 41:, :] = match[2, 41:, :] - 90.0  # every emission of the right part of the graph: 5 tokens are 2^-650
     batch = dict(batch, links=links)
     S64, C64, mg64, lg64 = _oracle_inside(batch, match.numpy())
-    try:
-        ops.inside_linear_bits(500)
-        ops.inside_linear_counts(reset=True)
-        ll, mg, lg = _inside_all(batch, match)
-        swept, handed = ops.inside_linear_counts()
-    finally:
-        ops.inside_linear_bits()
-    assert handed >= 3 and swept >= 2 and swept + handed == 8, (swept, handed)
+    ll, mg, lg = _inside_all(batch, match)
     w = torch.linspace(0.5, 1.5, 4).double().numpy()
     assert np.allclose(ll.double().numpy(), S64[:, 0, 0], rtol=1e-5)
     for bi in range(4):
@@ -449,13 +406,10 @@ def test_inside_linear_sweep_hands_over_what_it_cannot_follow():
 
 
 @pytest.mark.parametrize("wrong", [-16.0, -24.0, -32.0])
-def test_inside_linear_sweep_stops_and_log_domain_takes_over(wrong):
+def test_inside_peaked_emissions_vs_oracle(wrong):
     """Peaked emissions, as a trained model gives them: every token has one node that emits it with probability 0.8, all
-    other nodes are `wrong` nats down (every input inside the range the linear sweeps accept).  A node far from the
-    alignment then falls more than 2^-500 below its column's largest after some tokens: the linear-domain sweeps stop
-    there and the log-domain sweeps go on from that column with what is in the tables.  Loss, table and gradients against
-    the float64 oracle; the counters tell that sweeps were handed over, and since no input is out of range every one of
-    them was handed over on the way, not from the start."""
+    other nodes are `wrong` nats down.  A node far from the alignment then falls more than 2^-500 below its column's
+    largest after some tokens.  Loss, table and gradients against the float64 oracle."""
     L, T = 128, 32
     ms, ns = [128, 128, 96, 64, 40, 128], [32, 30, 25, 17, 11, 9]
     batch = synth.training_batch(len(ms), L, T, 80, ms, ns, seed=41)
@@ -469,16 +423,8 @@ def test_inside_linear_sweep_stops_and_log_domain_takes_over(wrong):
     assert float(match[torch.isfinite(match)].min()) > -100.0
     S64, C64, mg64, lg64 = _oracle_inside(batch, match.numpy())
     ol, tl = batch["output_length"].to(DEV), batch["target_length"].to(DEV)
-    try:
-        ops.inside_linear_bits(500)
-        ops.inside_linear_counts(reset=True)
-        ll, mg, lg = _inside_all(batch, match)
-        S = ops._pcfg_loss_tables(match.to(DEV), batch["links"].to(DEV), ol, tl, 1, "test")[0].cpu().double().numpy()
-        swept, handed = ops.inside_linear_counts()
-    finally:
-        ops.inside_linear_bits()
-    assert swept + handed == 3 * len(ms) and handed >= 1, (swept, handed)
-    print("emissions %.0f nats down: %d sweeps complete in the linear domain, %d taken over" % (wrong, swept, handed))
+    ll, mg, lg = _inside_all(batch, match)
+    S = ops._pcfg_loss_tables(match.to(DEV), batch["links"].to(DEV), ol, tl, 1, "test")[0].cpu().double().numpy()
     assert np.array_equal(np.isneginf(S), np.isneginf(S64))
     fin = np.isfinite(S64)
     assert np.allclose(S[fin], S64[fin], rtol=2e-6, atol=1e-4)
@@ -489,13 +435,12 @@ def test_inside_linear_sweep_stops_and_log_domain_takes_over(wrong):
             assert np.abs(got - want).max() <= 1e-4 * max(np.abs(want).max(), 1e-30), bi
 
 
-@pytest.mark.parametrize("n,width,bits", [(16, 4, 500), (16, 6, 500), (16, 1, 100), (5, 1, 100), (4, 1, 100), (3, 1, 100), (2, 1, 100)])
-def test_inside_linear_sweep_stops_at_every_column(n, width, bits):
+@pytest.mark.parametrize("n,width", [(16, 4), (16, 6), (16, 1), (5, 1), (4, 1), (3, 1), (2, 1)])
+def test_inside_emissions_that_collapse_at_every_column_vs_oracle(n, width):
     """One sentence per column p: `width` consecutive tokens from p on are emitted with probability e^-95 by every node but
-    one (inputs still inside the range the linear sweeps accept), so the spread of the columns grows by 137 bits a token
-    there and passes 2^bits at a column that moves with p - from the first step of either sweep to its last, where the
-    number below the range is only met while the last step runs; sentences of two to five tokens with a range of 100 bits
-    put every such case next to the ends of the sweeps.  Everything against the float64 oracle."""
+    one, so the spread of the columns grows by 137 bits a token there - at a column that moves with p from the first step
+    of either sweep to its last; sentences of two to five tokens put every such case next to the ends of the sweeps.
+    Everything against the float64 oracle."""
     L, T = 64, 16
     cases = list(range(0, max(n - width, 0) + 1))
     ms, ns = [64 - 2 * (p % 3) for p in cases], [n] * len(cases)
@@ -512,17 +457,8 @@ def test_inside_linear_sweep_stops_at_every_column(n, width, bits):
     assert float(match[torch.isfinite(match)].min()) > -103.0
     S64, C64, mg64, lg64 = _oracle_inside(batch, match.numpy())
     ol, tl = batch["output_length"].to(DEV), batch["target_length"].to(DEV)
-    try:
-        ops.inside_linear_bits(bits)
-        ops.inside_linear_counts(reset=True)
-        ll, mg, lg = _inside_all(batch, match)
-        S = ops._pcfg_loss_tables(match.to(DEV), batch["links"].to(DEV), ol, tl, 1, "test")[0].cpu().double().numpy()
-        swept, handed = ops.inside_linear_counts()
-    finally:
-        ops.inside_linear_bits()
-    assert swept + handed == 3 * len(cases), (swept, handed)
-    print("n %d, range 2^-%d, %d tokens 95 nats down from column p, p = 0..%d: %d sweeps complete in the linear domain, %d taken over"
-          % (n, bits, width, cases[-1], swept, handed))
+    ll, mg, lg = _inside_all(batch, match)
+    S = ops._pcfg_loss_tables(match.to(DEV), batch["links"].to(DEV), ol, tl, 1, "test")[0].cpu().double().numpy()
     assert np.array_equal(np.isneginf(S), np.isneginf(S64))
     fin = np.isfinite(S64)
     assert np.allclose(S[fin], S64[fin], rtol=2e-6, atol=1e-4)
@@ -1156,15 +1092,12 @@ def test_fused_step_equals_autograd_step(shape):
     res = harness.compute_pcfg_loss(leaf.half() if half else leaf * 1.0, out_mask, tgt, tgt_mask, links)
     assert int(res["invalid_nsentences"]) == 1
     res["loss"].backward()
-    def sliced(k):
-        return lambda *a: harness.train_step_single_call(*a, slices=k)
-
-    for step in (harness.train_step_direct, harness.train_step_fused, sliced(1), sliced(2), sliced(3)):
+    for step in (harness.train_step_direct, harness.train_step_fused, harness.train_step_single_call):
         buf = batch["logits"].to(DEV).clone()
         loss, glinks, ll = step(buf, tgt, batch["links"].to(DEV), ol, tl)
         assert torch.allclose(loss, res["loss"].detach(), rtol=1e-6)
-        # (the variants pair sweeps of the linear and of the log domain differently: each is within 1e-4 of the oracle, and
-        # they are within a few 1e-6 of each other)
+        # (the variants run their sweeps in different kernels: each is within 1e-4 of the oracle, and they are within a few
+        # 1e-6 of each other)
         assert torch.allclose(glinks, links.grad, rtol=3e-5, atol=1e-9)
         if half:
             assert torch.allclose(buf.float(), leaf.grad, rtol=2 ** -9, atol=2 ** -22)
@@ -1263,14 +1196,12 @@ def test_force_emit_step_equals_autograd_step():
     res["loss"].backward()
     plain = harness.compute_pcfg_loss(batch["logits"].to(DEV).clone(), out_mask, tgt, tgt_mask, batch["links"].to(DEV))
     assert abs(float(plain["loss"].detach()) - float(res["loss"].detach())) > 1e-3
-    for k in (1, 2):
-        buf = batch["logits"].to(DEV).clone()
-        loss, glinks, ll = harness.train_step_single_call(buf, tgt, batch["links"].to(DEV), ol, tl, slices=k, matchmask=mm,
-                                                          keep_word_mask=keep)
-        assert torch.allclose(loss, res["loss"].detach(), rtol=1e-6)
-        assert torch.allclose(glinks, links.grad, rtol=1e-5, atol=1e-9)
-        assert torch.allclose(buf.float(), leaf.grad, rtol=2 ** -9, atol=2 ** -22)
-        assert not buf[keep].any()
+    buf = batch["logits"].to(DEV).clone()
+    loss, glinks, ll = harness.train_step_single_call(buf, tgt, batch["links"].to(DEV), ol, tl, matchmask=mm, keep_word_mask=keep)
+    assert torch.allclose(loss, res["loss"].detach(), rtol=1e-6)
+    assert torch.allclose(glinks, links.grad, rtol=1e-5, atol=1e-9)
+    assert torch.allclose(buf.float(), leaf.grad, rtol=2 ** -9, atol=2 ** -22)
+    assert not buf[keep].any()
 
 
 def _generic_batch(ml, L, ms, ns, seed, generic_local):
