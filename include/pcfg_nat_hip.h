@@ -268,10 +268,12 @@ int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, cons
  * pcfg_loss.py:67-83 saves the inside gradients in the forward and scales them by grad_output in the backward,
  * :176-177 scale the probabilities by the upstream gradient before they are cast to the logits' dtype).
  *   forward:  gather with eos mask (read only) -> inside forward + backward with weights -1/(target_length*B) -> loss.
- *             Leaves match_all_grad, links_grad (both at an upstream gradient of 1), row_lse, loss_out[0..1]; the logits are
- *             untouched except that the rows of pad nodes may already be zeroed (*pad_rows_zeroed tells, pass it on).
+ *             Leaves match_all_grad, links_grad (both at an upstream gradient of 1), row_lse, loss_out[0..1] and, where ll_out
+ *             is not null, ll_out [B] = the log-likelihoods with those of invalid sentences zeroed (nat_pcfg_loss.py:123-133);
+ *             the logits are untouched except that the rows of pad nodes may already be zeroed (*pad_rows_zeroed tells, pass
+ *             it on).
  *   backward: logits_inout becomes upstream * d loss / d logits in one read + write pass, links_grad_inout is multiplied by
- *             upstream.  upstream_dev: one float32 in device memory (the gradient flowing into the loss, e.g. the fp16 loss
+ *             upstream by the threads of the same launch.  upstream_dev: one float32 in device memory (the gradient flowing into the loss, e.g. the fp16 loss
  *             scale times the criterion's factor; NULL = 1).  It multiplies the emission posteriors in float32 ahead of the
  *             single rounding to the logits' dtype, so gradients below the fp16 range at scale 1 survive, and no value ever
  *             passes through the host.
@@ -279,8 +281,8 @@ int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *targets, cons
 int pcfgnat_criterion_forward(void *logits, int dtype, const int64_t *targets, const float *links, const int64_t *output_length,
                               const int64_t *target_length, const unsigned char *matchmask, const unsigned char *keep_word_mask,
                               float *match_all, float *S, float *aux, float *match_all_grad, float *links_grad, float *row_lse,
-                              float *loss_out, int *pad_rows_zeroed, int64_t B, int64_t L, int64_t V, int64_t T, int64_t ml,
-                              void *stream);
+                              float *loss_out, float *ll_out, int *pad_rows_zeroed, int64_t B, int64_t L, int64_t V, int64_t T,
+                              int64_t ml, void *stream);
 int pcfgnat_criterion_backward(void *logits_inout, int dtype, const int64_t *targets, const float *match_all_grad,
                                const float *row_lse, const unsigned char *keep_word_mask, const int64_t *output_length,
                                int pad_rows_zeroed, const float *upstream_dev, float *links_grad_inout, int64_t B, int64_t L,

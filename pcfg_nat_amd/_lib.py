@@ -10,11 +10,13 @@ import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libpcfg_nat_hip.so")
+EXT_PATH = os.path.join(_HERE, "lib", "_pcfg_nat_torch.so")
 
 OK, EINVAL, EUNSUPPORTED, EHIP = 0, 1, 2, 3
 F16, F32, F64 = 0, 1, 2
 
 _lib = None
+_ext = None
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -48,7 +50,7 @@ SIGNATURES = {
     "pcfgnat_criterion_loss": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_criterion_step": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                                       _i64, ctypes.c_float, _vp, _vp, _vp]),
-    "pcfgnat_criterion_forward": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
+    "pcfgnat_criterion_forward": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                                          _i64, _i64, _vp]),
     "pcfgnat_criterion_backward": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_extract_links_pack": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
@@ -104,6 +106,26 @@ def load():
         fn.argtypes = args
     _lib = lib
     return lib
+
+
+def load_ext():
+    """The host side of the training operators as a torch extension (``csrc/torch_ext.cpp``: checks, allocation, autograd
+    nodes and the C-ABI call in C++), built beside the library by the same Makefile.  Loaded once, after the library itself
+    (the extension links to it).  Raises if it has not been built."""
+    global _ext
+    if _ext is not None:
+        return _ext
+    load()
+    if not os.path.exists(EXT_PATH):
+        raise RuntimeError("_pcfg_nat_torch.so is missing (%s): build it with `make -C pcfg_nat_amd/csrc`" % EXT_PATH)
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("_pcfg_nat_torch", EXT_PATH)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    if mod.abi_version() != _lib.pcfgnat_abi_version():
+        raise RuntimeError("_pcfg_nat_torch.so was built against another version of libpcfg_nat_hip.so: rebuild both")
+    _ext = mod
+    return mod
 
 
 def check(rc, lib=None):

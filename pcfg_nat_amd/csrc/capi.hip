@@ -108,17 +108,10 @@ extern "C" int pcfgnat_criterion_step(void *logits, int dtype, const int64_t *ta
 // memory - multiplies the emission posteriors in float32 ahead of the single rounding to the logits' dtype (the
 // reference scales its saved gradients before the cast as well: pcfg_loss.py:77-83, 176-177).  No host read anywhere.
 // ---------------------------------------------------------------------------------------------------------------
-namespace {
-__global__ __launch_bounds__(256) void scale_by_device_scalar_kernel(float *__restrict__ p, size_t n, const float *__restrict__ scale_dev) {
-    const float sc = *scale_dev;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] *= sc;
-}
-}  // namespace
-
 extern "C" int pcfgnat_criterion_forward(void *logits, int dtype, const int64_t *targets, const float *links,
                                          const int64_t *output_length, const int64_t *target_length, const unsigned char *matchmask,
                                          const unsigned char *keep_word_mask, float *match_all, float *S, float *aux,
-                                         float *match_all_grad, float *links_grad, float *row_lse, float *loss_out,
+                                         float *match_all_grad, float *links_grad, float *row_lse, float *loss_out, float *ll_out,
                                          int *pad_rows_zeroed, int64_t B, int64_t L, int64_t V, int64_t T, int64_t ml, void *stream) {
     if (dtype != PCFGNAT_F16 && dtype != PCFGNAT_F32)
         return pcfgnat::fail(PCFGNAT_EUNSUPPORTED, "criterion_forward: logits must be float16 or float32 (the PCFG kernels are float32)");
@@ -139,7 +132,7 @@ extern "C" int pcfgnat_criterion_forward(void *logits, int dtype, const int64_t 
                                                pcfgnat::PadFill{(unsigned char *)logits, (int64_t)V * (int64_t)esz}, &pad_done);
     if (rc != PCFGNAT_OK) return rc;
     *pad_rows_zeroed = pad_done ? 1 : 0;
-    return pcfgnat_criterion_loss(S, target_length, loss_out, B, L, T, ml, stream);
+    return pcfgnat::criterion_loss_impl(S, target_length, loss_out, ll_out, B, L, T, ml, stream);
 }
 
 extern "C" int pcfgnat_criterion_backward(void *logits_inout, int dtype, const int64_t *targets, const float *match_all_grad,
@@ -150,18 +143,12 @@ extern "C" int pcfgnat_criterion_backward(void *logits_inout, int dtype, const i
         return pcfgnat::fail(PCFGNAT_EUNSUPPORTED, "criterion_backward: logits must be float16 or float32");
     PCFGNAT_REQUIRE(B >= 1 && L >= 4 && T >= 2 && V >= 1 && ml >= 0, "criterion_backward: bad dimensions");
     PCFGNAT_REQUIRE(logits_inout && targets && match_all_grad && row_lse && output_length, "criterion_backward: null pointer");
-    int rc = pcfgnat::lsg_backward_lse_with_loss(logits_inout, dtype, targets, T, 0, 1, match_all_grad, row_lse, B, L, V, T, nullptr, 0,
-                                                 nullptr, nullptr, keep_word_mask, output_length, pad_rows_zeroed ? 1 : 0, upstream_dev,
-                                                 stream);
-    if (rc != PCFGNAT_OK) return rc;
-    if (links_grad_inout != nullptr && upstream_dev != nullptr) {
-        const size_t n = (size_t)B * L * (ml + 1) * L;
-        const unsigned grid = (unsigned)((n + 256 * 8 - 1) / (256 * 8));
-        hipLaunchKernelGGL(scale_by_device_scalar_kernel, dim3(grid < 1 ? 1 : grid), dim3(256), 0, (hipStream_t)stream, links_grad_inout,
-                           n, upstream_dev);
-        PCFGNAT_HIP_CHECK(hipGetLastError());
-    }
-    return PCFGNAT_OK;
+    // the rule gradients take the same factor: one float per thread of the same launch
+    const pcfgnat::ScaleTask rules{(links_grad_inout != nullptr && upstream_dev != nullptr) ? links_grad_inout : nullptr,
+                                   (size_t)B * L * (ml + 1) * L};
+    return pcfgnat::lsg_backward_lse_with_loss(logits_inout, dtype, targets, T, 0, 1, match_all_grad, row_lse, B, L, V, T, nullptr, 0,
+                                               nullptr, nullptr, keep_word_mask, output_length, pad_rows_zeroed ? 1 : 0, upstream_dev,
+                                               stream, rules);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

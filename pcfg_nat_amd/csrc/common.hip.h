@@ -70,6 +70,12 @@ __device__ __forceinline__ double seed_weight(const double *grad_out, int b, int
     if (sd.scale_dev) g *= (double)*sd.scale_dev;
     return g * (double)sd.scale;
 }
+// A buffer that the gather backward multiplies by its device-side upstream factor on the way (the rule gradients of the
+// criterion's backward: one float per thread of the launch, instead of a launch of their own).  p null: nothing to do.
+struct ScaleTask {
+    float *p;
+    size_t n;
+};
 // Like the public functions of the same name, with the weights above in place of the batch size.
 int inside_backward_impl(const float *grad_output, const float *S, float *aux, const float *match_all, const float *links,
                          const int64_t *output_length, const int64_t *target_length, float *match_all_grad, float *links_grad, int64_t B,
@@ -102,12 +108,16 @@ int lsg_backward_lse_with_loss(void *logits_inout, int dtype, const int64_t *sel
                                const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T,
                                const float *S, int64_t ll_stride, const int64_t *target_length, float *loss_out,
                                const unsigned char *keep, const int64_t *pad_output_length, int pad_rows_zeroed, const float *gscale_dev,
-                               void *stream);
+                               void *stream, ScaleTask also_scale = ScaleTask{nullptr, 0});
 // pcfgnat_logsoftmax_gather_lse over the [B,T] targets with the eos mask and the force-emit masks; the rows of nodes at
 // or beyond a sentence's output length are left unread (zeros in selected and lse)
 int lsg_forward_lse_force(const void *logits, int dtype, const int64_t *targets, void *selected, void *lse,
                           const int64_t *output_length, const int64_t *target_length, const unsigned char *matchmask,
                           const unsigned char *keep, int64_t B, int64_t L, int64_t V, int64_t T, void *stream);
+
+// pcfgnat_criterion_loss that also writes the log-likelihoods with the invalid ones zeroed (ll_out [B], may be null)
+int criterion_loss_impl(const float *S, const int64_t *target_length, float *out, float *ll_out, int64_t B, int64_t L, int64_t T,
+                        int64_t ml, void *stream);
 
 // Settings of pcfgnat_pipeline_config (inside.hip): the most workgroups a pipelined sweep may use (0 = pipelines off) and the
 // bound on a block's wait for the one ahead of it, in rounds of polling
@@ -237,7 +247,9 @@ struct LossTask {
     float *out;  // null: nothing to do
     int B;
     int64_t stride;
+    float *ll_out = nullptr;  // [B] or null: the log-likelihoods with the invalid ones (non-finite) zeroed
 };
+
 // NT threads form the sum (the order of the additions, and with it the rounding, is a function of NT alone); the
 // workgroup may be larger (BLOCK threads), its other threads only keep the barriers company.
 template <int NT, int BLOCK = NT>
@@ -253,6 +265,7 @@ __device__ __forceinline__ void criterion_loss_block(const LossTask &t) {
             const bool ok = (ll == ll) && (fabsf(ll) != __builtin_huge_valf());
             if (ok) acc += ll / (float)t.tgt_len[b];
             else bad += 1.f;
+            if (t.ll_out != nullptr) t.ll_out[b] = ok ? ll : 0.f;
         }
         s_sum[threadIdx.x] = acc;
         s_bad[threadIdx.x] = bad;

@@ -3160,8 +3160,8 @@ __global__ void fill_zero_kernel(float *p, size_t n) {
 // loss = -(1/B) * sum_b [ll_b finite] ll_b / n_b and the number of invalid sentences (nat_pcfg_loss.py:123-135), reduced
 // in a fixed order by one workgroup.  out[0] = loss, out[1] = invalid count.
 __global__ __launch_bounds__(256) void criterion_loss_kernel(const float *__restrict__ S, const int64_t *__restrict__ tgt_len,
-                                                            float *__restrict__ out, int B, int Mc, int T) {
-    criterion_loss_block<256>(LossTask{S, tgt_len, out, B, (int64_t)Mc * (T + 2)});
+                                                            float *__restrict__ out, int B, int Mc, int T, float *__restrict__ ll_out) {
+    criterion_loss_block<256>(LossTask{S, tgt_len, out, B, (int64_t)Mc * (T + 2), ll_out});
 }
 
 // The pipelined sweeps are used while a batch needs no more than g_pipeline_max_wg workgroups.  The default is no limit in
@@ -3626,15 +3626,20 @@ extern "C" int pcfgnat_pcfg_loss_forward_backward_static(const float *grad_outpu
                                         B, L, T, ml, seed_of(B), stream);
 }
 
-extern "C" int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *out, int64_t B, int64_t L, int64_t T,
-                                      int64_t ml, void *stream) {
+int pcfgnat::criterion_loss_impl(const float *S, const int64_t *target_length, float *out, float *ll_out, int64_t B, int64_t L, int64_t T,
+                                 int64_t ml, void *stream) {
     int rc = check_dims("criterion_loss", B, L, T, ml);
     if (rc != PCFGNAT_OK) return rc;
     PCFGNAT_REQUIRE(B >= 1 && S && target_length && out, "criterion_loss: null pointer or empty batch");
     const int Mc = (int)((L - 2) / (ml + 1) + 1);
-    hipLaunchKernelGGL(criterion_loss_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, S, target_length, out, (int)B, Mc, (int)T);
+    hipLaunchKernelGGL(criterion_loss_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, S, target_length, out, (int)B, Mc, (int)T, ll_out);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
+}
+
+extern "C" int pcfgnat_criterion_loss(const float *S, const int64_t *target_length, float *out, int64_t B, int64_t L, int64_t T,
+                                      int64_t ml, void *stream) {
+    return criterion_loss_impl(S, target_length, out, nullptr, B, L, T, ml, stream);
 }
 
 namespace pcfgnat {

@@ -532,7 +532,7 @@ __global__ __launch_bounds__(NT, FROM_LOGITS ? 1 : 6) void lsg_bwd_kernel(T *__r
                                                      const typename Elem<T>::compute *__restrict__ lse, LossTask loss,
                                                      const unsigned char *__restrict__ detach_rows,
                                                      const int64_t *__restrict__ pad_out_len, int pad_mode,
-                                                     int pad_rows_zeroed, const float *__restrict__ gscale_dev) {
+                                                     int pad_rows_zeroed, const float *__restrict__ gscale_dev, ScaleTask also_scale) {
     using CT = typename Elem<T>::compute;
     constexpr int EPV = Elem<T>::EPV;
     constexpr int FIX = (TCAP + NT - 1) / NT;
@@ -558,6 +558,11 @@ __global__ __launch_bounds__(NT, FROM_LOGITS ? 1 : 6) void lsg_bwd_kernel(T *__r
     const int tid = threadIdx.x, lane = tid & 63;
 
     const int64_t slot = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;  // one row per workgroup
+    if (also_scale.p != nullptr && gscale_dev != nullptr) {  // a side task spread over every thread of the launch
+        const size_t total = (size_t)gridDim.x * gridDim.y * NT;
+        const float sc = *gscale_dev;
+        for (size_t i = (size_t)slot * NT + tid; i < also_scale.n; i += total) also_scale.p[i] *= sc;
+    }
     if (slot >= rows) return;
     // Rows of nodes beyond the sentence's graph (pads) get no gradient from the criterion, whose backward sweep leaves
     // their upstream gradient all zero: p * 0 plus zeros is zero whatever the row holds, so such a row is written
@@ -795,7 +800,8 @@ int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
 template <typename T>
 int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, const void *g, int64_t rows, int L, int V,
                int Tn, const void *lse, const LossTask &loss, hipStream_t stream, const unsigned char *detach_rows = nullptr,
-               const int64_t *pad_out_len = nullptr, int pad_rows_zeroed = 0, const float *gscale_dev = nullptr) {
+               const int64_t *pad_out_len = nullptr, int pad_rows_zeroed = 0, const float *gscale_dev = nullptr,
+               ScaleTask also_scale = ScaleTask{nullptr, 0}) {
     using CT = typename Elem<T>::compute;
     constexpr int NT = 512;
     constexpr int MAXC = 10;
@@ -808,11 +814,11 @@ int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
         if (lse != nullptr)                                                                                                                \
             hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, tcap, true>), grid, dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,              \
                                (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss, detach_rows, pad_out_len, pad_mode, pad_rows_zeroed,  \
-                               gscale_dev);                                                                                                \
+                               gscale_dev, also_scale);                                                                                    \
         else                                                                                                                               \
             hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, tcap, false>), grid, dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,             \
                                (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss, detach_rows, pad_out_len, pad_mode,               \
-                               pad_rows_zeroed, nullptr);                                                                                  \
+                               pad_rows_zeroed, nullptr, ScaleTask{nullptr, 0});                                                           \
     } while (0)
     if (Tn <= NT) PCFGNAT_LSG_BWD(NT);
     else PCFGNAT_LSG_BWD(TCAP);
@@ -911,20 +917,21 @@ extern "C" int pcfgnat_logsoftmax_max(const void *logits, int dtype, void *best_
 
 static int lsg_backward_dispatch(void *buf, int dtype, const int64_t *select_idx, int64_t sb, int64_t sl, int64_t st,
                                  const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T, void *stream,
-                                 const LossTask &loss = LossTask{nullptr, nullptr, nullptr, 0, 0},
+                                 const LossTask &loss = LossTask{nullptr, nullptr, nullptr, 0, 0, nullptr},
                                  const unsigned char *detach_rows = nullptr, const int64_t *pad_out_len = nullptr,
-                                 int pad_rows_zeroed = 0, const float *gscale_dev = nullptr) {
+                                 int pad_rows_zeroed = 0, const float *gscale_dev = nullptr,
+                                 ScaleTask also_scale = ScaleTask{nullptr, 0}) {
     int rc = check_common(buf, select_idx, grad_selected, B, L, V, T);
     if (rc != PCFGNAT_OK) return rc;
     if (B * L == 0) return PCFGNAT_OK;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case PCFGNAT_F16:
-            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev);
+            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev, also_scale);
         case PCFGNAT_F32:
-            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev);
+            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev, also_scale);
         case PCFGNAT_F64:
-            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev);
+            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev, also_scale);
         default:
             return fail(PCFGNAT_EINVAL, "logsoftmax_gather_backward: unknown dtype code %d", dtype);
     }
@@ -947,11 +954,12 @@ int pcfgnat::lsg_backward_lse_with_loss(void *logits_inout, int dtype, const int
                                         const void *grad_selected, const void *lse, int64_t B, int64_t L, int64_t V, int64_t T,
                                         const float *S, int64_t ll_stride, const int64_t *target_length, float *loss_out,
                                         const unsigned char *keep, const int64_t *pad_output_length, int pad_rows_zeroed,
-                                        const float *gscale_dev, void *stream) {
+                                        const float *gscale_dev, void *stream, ScaleTask also_scale) {
     PCFGNAT_REQUIRE(B >= 1 && L >= 1 && lse && (loss_out == nullptr || (S && target_length)),
                     "logsoftmax_gather_backward: null pointer or empty batch");
     return lsg_backward_dispatch(logits_inout, dtype, select_idx, sb, sl, st, grad_selected, lse, B, L, V, T, stream,
-                                 LossTask{S, target_length, loss_out, (int)B, ll_stride}, keep, pad_output_length, pad_rows_zeroed, gscale_dev);
+                                 LossTask{S, target_length, loss_out, (int)B, ll_stride}, keep, pad_output_length, pad_rows_zeroed, gscale_dev,
+                                 also_scale);
 }
 
 int pcfgnat::lsg_forward_lse_force(const void *logits, int dtype, const int64_t *targets, void *selected, void *lse,

@@ -28,6 +28,26 @@ def get_pcfg_kernel():
     return _lib.load()
 
 
+# Host side of the three training operators (cuda_pcfg_loss, dag_logsoftmax_gather_inplace, pcfg_criterion): the torch
+# extension (C++ checks, allocation and autograd nodes; what a training run uses) or the Python Functions of this module
+# over ctypes (same kernels, same results; kept for float64 tables and as the readable statement of the contract).
+_HOST_BACKEND = "extension"
+
+
+def host_backend(name=None):
+    """Selects ("extension" / "python") or reports which host-side implementation the training operators use."""
+    global _HOST_BACKEND
+    if name is not None:
+        if name not in ("extension", "python"):
+            raise RuntimeError("host_backend: 'extension' or 'python'")
+        _HOST_BACKEND = name
+    return _HOST_BACKEND
+
+
+def _ext():
+    return _lib.load_ext() if _HOST_BACKEND == "extension" else None
+
+
 DEFAULT_SPIN_LIMIT = 1 << 15  # PCFGNAT_DEFAULT_SPIN_LIMIT of the library
 
 
@@ -216,7 +236,14 @@ class CUDAPCFGLossFunc(Function):
         return None, None, None, None
 
 
-cuda_pcfg_loss = CUDAPCFGLossFunc.apply
+def cuda_pcfg_loss(match_all, links, output_length, target_length):
+    """``CUDAPCFGLossFunc.apply`` (pcfg_loss.py:85); float32 tables go through the C++ autograd node of the torch extension."""
+    ext = _ext()
+    if ext is None or match_all.dtype != torch.float32 or links.dtype != torch.float32 or not match_all.is_cuda:
+        return CUDAPCFGLossFunc.apply(match_all, links, output_length, target_length)
+    if not (1 <= CUDAPCFGLossFunc.config <= 4):
+        raise RuntimeError("config should be 1~4")
+    return ext.cuda_pcfg_loss(match_all, links, output_length, target_length)
 
 
 class CUDAPCFGBestTreeFunc(Function):
@@ -346,7 +373,12 @@ class DagLogsoftmaxGatherFunc(Function):
         return grad_input, None
 
 
-dag_logsoftmax_gather_inplace = DagLogsoftmaxGatherFunc.apply
+def dag_logsoftmax_gather_inplace(word_ins_out, select_idx):
+    """``DagLogsoftmaxGatherFunc.apply`` (pcfg_loss.py:181), through the C++ autograd node of the torch extension."""
+    ext = _ext()
+    if ext is None or not word_ins_out.is_cuda:
+        return DagLogsoftmaxGatherFunc.apply(word_ins_out, select_idx)
+    return ext.dag_logsoftmax_gather_inplace(word_ins_out, select_idx)
 
 
 def _logsoftmax_gather(word_ins_out, select_idx, require_gradient, eos_lengths=None):
@@ -1048,7 +1080,7 @@ def pcfg_criterion_step(logits, targets, links, output_length, target_length, ev
 
 def _criterion_forward(logits, targets, links, output_length, target_length, matchmask=None, keep_word_mask=None):
     """Forward half of the criterion pass (``pcfgnat_criterion_forward``): everything that does not depend on the loss's
-    upstream gradient.  Returns (loss_and_invalid [2], ll [B], state) where ``state`` carries what
+    upstream gradient.  Returns (loss_and_invalid [2 + B], ll [B] with the invalid sentences zeroed, state) where ``state`` carries what
     ``_criterion_backward`` needs; ``logits`` must stay untouched until then (rows of pad nodes may already be zeroed)."""
     import ctypes
     lib = get_pcfg_kernel()
@@ -1063,15 +1095,15 @@ def _criterion_forward(logits, targets, links, output_length, target_length, mat
         mg = torch.empty_like(match)
         lg = torch.empty_like(links)
         row_lse = torch.empty((B, L), dtype=torch.float32, device=dev)
-        out = torch.empty((2,), dtype=torch.float32, device=dev)
+        out = torch.empty((2 + B,), dtype=torch.float32, device=dev)  # loss, invalid count, ll with the invalid ones zeroed
         _lib.check(lib.pcfgnat_criterion_forward(logits.data_ptr(), code, targets.data_ptr(), links.data_ptr(), ol.data_ptr(),
                                                  tl.data_ptr(), mm8.data_ptr() if mm8 is not None else None,
                                                  keep8.data_ptr() if keep8 is not None else None, match.data_ptr(), S.data_ptr(),
                                                  aux.data_ptr(), mg.data_ptr(), lg.data_ptr(), row_lse.data_ptr(), out.data_ptr(),
-                                                 ctypes.byref(pad_zeroed), B, L, V, T, ml, _stream(logits)), lib)
+                                                 out.data_ptr() + 8, ctypes.byref(pad_zeroed), B, L, V, T, ml, _stream(logits)), lib)
     state = {"targets": targets, "match_all_grad": mg, "links_grad": lg, "row_lse": row_lse, "keep": keep8, "output_length": ol,
              "pad_rows_zeroed": int(pad_zeroed.value), "dims": (code, B, L, V, T, ml)}
-    return out, S[:, 0, 0], state
+    return out, out[2:], state
 
 
 def _criterion_backward(logits, state, upstream):
@@ -1110,10 +1142,10 @@ class PCFGCriterionFunc(Function):
         else:  # nothing to differentiate: the plain step (its gradients are discarded)
             out, _, ll, _, _ = pcfg_criterion_step(outputs, targets, links, output_length, target_length, matchmask=matchmask,
                                                    keep_word_mask=keep_word_mask)
+            ll = ll.masked_fill(ll.isinf().logical_or(ll.isnan()), 0)
         ctx.mark_dirty(outputs)
         ctx.set_materialize_grads(False)
-        invalid = ll.isinf().logical_or(ll.isnan())
-        return outputs, out[0], ll.masked_fill(invalid, 0), out[1]
+        return outputs, out[0], ll, out[1]
 
     @staticmethod
     def backward(ctx, grad_outputs, grad_loss, grad_ll, grad_invalid):
@@ -1136,6 +1168,9 @@ def pcfg_criterion(outputs, targets, links, output_length, target_length, matchm
     backward.  Returns
     (loss, ll [B] with invalid sentences zeroed, number of invalid sentences) - the dict entries of
     ``harness.compute_pcfg_loss``."""
+    ext = _ext()
+    if ext is not None and outputs.is_cuda:
+        return ext.pcfg_criterion(outputs, targets, links, output_length, target_length, matchmask, keep_word_mask)
     _, loss, ll, invalid = PCFGCriterionFunc.apply(outputs, links, targets, output_length, target_length, matchmask, keep_word_mask)
     return loss, ll, invalid
 

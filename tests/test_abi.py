@@ -35,6 +35,19 @@ def test_library_exports_every_declared_symbol():
     assert lib.pcfgnat_pcfg_aux_floats(1, 282, 9, 1) == (6 * 141 * 11 + 13 + 3) // 4 * 4 + 4 * 141 * 192 + 4 * 192 * 11 + 12 * 13 + 4 + 4 * 192 * 11 + 12 * 13 + 2 * 14
 
 
+def test_torch_extension_loads_without_gpu():
+    """The host side of the training operators (a torch extension linked to the library) imports on a machine without a
+    GPU, reports the library's ABI version and raises loud errors for CPU tensors before anything is enqueued."""
+    ext = _lib.load_ext()
+    assert ext.abi_version() == _lib.load().pcfgnat_abi_version()
+    for name in ("cuda_pcfg_loss", "dag_logsoftmax_gather_inplace", "pcfg_criterion"):
+        assert hasattr(ext, name)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ext.cuda_pcfg_loss(torch.zeros(1, 8, 4), torch.zeros(1, 8, 2, 8), torch.tensor([8]), torch.tensor([4]))
+    with pytest.raises(RuntimeError, match="GPU"):
+        ext.dag_logsoftmax_gather_inplace(torch.zeros(1, 8, 16), torch.zeros(1, 8, 4, dtype=torch.int64))
+
+
 def test_argument_errors_without_gpu():
     lib = _lib.load()
     rc = lib.pcfgnat_pcfg_loss(None, None, None, None, None, None, 2, 16, 4, 30, None)
