@@ -38,7 +38,12 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--cpu-sentences", type=int, default=40, help="sentences of the batch timed on the CPU oracle")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-decode", action="store_true", help="skip the viterbi decode timing")
+    ap.add_argument("--no-decode", action="store_true", help="skip the legs beyond the training step (same as --legs autograd,operator)")
+    ap.add_argument("--legs", default="all",
+                    help="comma-separated legs to run beside the headline step: autograd, operator, decode, glat, long, links, "
+                         "frontend (default: all; 'none' for the headline alone) - for profiling runs that want few kernels")
+    ap.add_argument("--decode-sentences", type=int, default=1000,
+                    help="sentences of the inference configuration the decode leg uses (default: all 1000)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of a logits-sized fp16 buffer (409.6 MB read, 409.6 MB written): "
                          "the reference point for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters")
@@ -114,7 +119,7 @@ def _cpu_viterbi_decode(ob, tok, links, m, mask):
     return time.perf_counter() - t0, out, pred
 
 
-def decode_timing(dev, cpu=True, front_end_sample=16):
+def decode_timing(dev, cpu=True, front_end_sample=16, n_sent=1000):
     """Viterbi decode of the inference configuration (BASELINE config 4: 1000 sentences, src ~U[5,100], L = 4*src, V=40000,
     fp16 logits ~N(0,3)) as the model runs it: front-end (log-softmax + max over the vocabulary, one read of the logits)
     followed by tables + length selection + readout, all enqueued by one native call; the emitted token counts are read back
@@ -129,7 +134,7 @@ def decode_timing(dev, cpu=True, front_end_sample=16):
     from pcfg_nat_amd import custom_ops as ops, harness, synth
 
     V = 40000
-    lens = synth.config4_lengths()
+    lens = synth.config4_lengths()[:n_sent]
     n_sent = len(lens)
     out = {"sentences": n_sent,
            "src_length_histogram": {"%d-%d" % (lo, lo + 19): int(((lens >= lo) & (lens < lo + 20)).sum()) for lo in range(5, 101, 20)}}
@@ -681,15 +686,28 @@ def main():
         result["single_call_scaled"] = sc
     # the drop-in path: the unchanged criterion code over the operator API under autograd (dag_logsoftmax_gather_inplace ->
     # eos mask -> cuda_pcfg_loss -> loss -> backward), which reads and rewrites every row (it is not told the lengths)
-    result["criterion_autograd"] = criterion_autograd_timing(bufs, targets, links, ol, tl, args, timed_windows, host_enqueue_ms)
-    result["operator_api"] = operator_api_timing(bufs, targets, links, ol, tl, args, timed_windows, host_enqueue_ms)
+    legs = {"autograd", "operator", "decode", "glat", "long", "links", "frontend"}
+    if args.legs != "all":
+        legs = {x for x in args.legs.split(",") if x and x != "none"}
+    if args.no_decode:
+        legs &= {"autograd", "operator"}
+    from pcfg_nat_amd import custom_ops
+    result["host_backend"] = custom_ops.host_backend()
+    if "autograd" in legs:
+        result["criterion_autograd"] = criterion_autograd_timing(bufs, targets, links, ol, tl, args, timed_windows, host_enqueue_ms)
+    if "operator" in legs:
+        result["operator_api"] = operator_api_timing(bufs, targets, links, ol, tl, args, timed_windows, host_enqueue_ms)
     cpu = not args.no_cpu_baseline
-    if not args.no_decode:
-        result["viterbi"] = decode_timing(dev, cpu=cpu)
+    if "decode" in legs:
+        result["viterbi"] = decode_timing(dev, cpu=cpu, n_sent=args.decode_sentences)
+    if "glat" in legs:
         result["glat_alignment"] = glat_timing(torch.randn(B, L, V, device=dev, generator=ggen).mul_(2).half(), targets, links, ol,
                                                cpu=(targets_cpu, links_cpu, m, n) if cpu else None)
+    if "long" in legs:
         result["long_sentences"] = long_sentence_timing(dev)
+    if "links" in legs:
         result["link_scorer"] = link_scorer_timing(dev)
+    if "frontend" in legs:
         result["decode_front_end"] = decode_front_end_timing(dev)
     if not args.no_cpu_baseline:
         batch_cpu = {"output_length": m, "target_length": n, "links": links_cpu, "targets": targets_cpu}

@@ -222,34 +222,68 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
     const int r0 = __builtin_amdgcn_readlane(v, 15), r1 = __builtin_amdgcn_readlane(v, 31), r2 = __builtin_amdgcn_readlane(v, 47);
     return v + (lane >= 16 ? r0 : 0) + (lane >= 32 ? r1 : 0) + (lane >= 48 ? r2 : 0);
 }
-__device__ __forceinline__ int compact_row(int k, int rows, const int64_t *__restrict__ out_len, int B, int L, int lane, bool &live) {
-    const int kp = rows - 1 - k;  // index among the pad rows, valid when k is behind the live rows
-    int done_live = 0, done_pad = 0, row = 0;
-    live = false;
-    bool found = false;
-    for (int b0 = 0; b0 < B && !found; b0 += 64) {
+struct RowOf {
+    int b, p;   // sentence and node
+    bool live;  // false: the row of a pad node
+};
+__device__ __forceinline__ RowOf compact_row(int k, const int64_t *__restrict__ out_len, int B, int L, int lane) {
+    RowOf r{0, 0, false};
+    // the live rows: sentence by sentence in rounds of 64 (one round for batches of up to 64 sentences)
+    int done_live = 0;
+    for (int b0 = 0; b0 < B; b0 += 64) {
+        int len = 0;
+        if (b0 + lane < B) {
+            const int64_t v = out_len[b0 + lane];
+            len = v < 0 ? 0 : (v > (int64_t)L ? L : (int)v);
+        }
+        const int live_upto = wave_inclusive_scan(len, lane);
+        const int tot_live = __builtin_amdgcn_readlane(live_upto, 63);
+        if (k < done_live + tot_live) {  // the first lane whose running count passes k holds the sentence
+            const int l = __builtin_ctzll(__ballot(k < done_live + live_upto));
+            r.b = b0 + l;
+            r.p = k - done_live - __builtin_amdgcn_readlane(live_upto - len, l);
+            r.live = true;
+            return r;
+        }
+        done_live += tot_live;
+    }
+    // behind the live rows: the rows of pad nodes, in reverse (these workgroups have next to nothing to do)
+    const int kp = B * L - 1 - k;
+    int done_pad = 0;
+    for (int b0 = 0; b0 < B; b0 += 64) {
         int len = 0, pad = 0;
         if (b0 + lane < B) {
             const int64_t v = out_len[b0 + lane];
             len = v < 0 ? 0 : (v > (int64_t)L ? L : (int)v);
             pad = L - len;
         }
-        const int live_upto = wave_inclusive_scan(len, lane), pad_upto = wave_inclusive_scan(pad, lane);
-        const unsigned long long hit_live = __ballot(k < done_live + live_upto), hit_pad = __ballot(kp < done_pad + pad_upto);
-        const int tot_live = __builtin_amdgcn_readlane(live_upto, 63), tot_pad = __builtin_amdgcn_readlane(pad_upto, 63);
-        if (k < done_live + tot_live) {  // the first lane whose running count passes k holds the sentence
-            const int l = __builtin_ctzll(hit_live);
-            row = (b0 + l) * L + (k - done_live - __builtin_amdgcn_readlane(live_upto - len, l));
-            live = found = true;
-        } else if (kp < done_pad + tot_pad) {
-            const int l = __builtin_ctzll(hit_pad);
-            row = (b0 + l) * L + __builtin_amdgcn_readlane(len, l) + (kp - done_pad - __builtin_amdgcn_readlane(pad_upto - pad, l));
-            found = true;
+        const int pad_upto = wave_inclusive_scan(pad, lane);
+        const int tot_pad = __builtin_amdgcn_readlane(pad_upto, 63);
+        if (kp < done_pad + tot_pad) {
+            const int l = __builtin_ctzll(__ballot(kp < done_pad + pad_upto));
+            r.b = b0 + l;
+            r.p = __builtin_amdgcn_readlane(len, l) + (kp - done_pad - __builtin_amdgcn_readlane(pad_upto - pad, l));
+            return r;
         }
-        done_live += tot_live;
         done_pad += tot_pad;
     }
-    return row;
+    return r;
+}
+
+// The row of a workgroup.  The launch is a grid of (L, min(B, 65535), ceil(B / 65535)) workgroups, so sentence and node
+// come out of the workgroup index without a division (a 64-bit division by a run-time L is some hundred scalar
+// instructions in front of the row's first load).  mode 2: the workgroup's running number selects the k-th live row.
+__device__ __forceinline__ bool row_of_workgroup(int mode, const int64_t *__restrict__ out_len, int B, int L, int lane, RowOf &r) {
+    const int b = (int)blockIdx.z * 65535 + (int)blockIdx.y;
+    if (b >= B) return false;
+    if (mode == 2) {
+        r = compact_row(b * L + (int)blockIdx.x, out_len, B, L, lane);
+    } else {
+        r.b = b;
+        r.p = (int)blockIdx.x;
+        r.live = mode == 0 || (int64_t)r.p < out_len[b];
+    }
+    return true;
 }
 
 // First position, among the elements this thread holds, whose value equals the row maximum (0x7fffffff if none).
@@ -286,7 +320,7 @@ __device__ __forceinline__ int first_pos_of_max(const vec16 (&buf)[MAXC], const 
 template <typename T, int NT, int MAXC, int GMAX, bool GRAD, bool KEEP>
 __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const int64_t *__restrict__ idx, int64_t sb,
                                                      int64_t sl, int64_t st,
-                                                     typename Elem<T>::compute *__restrict__ sel, int64_t rows, int L,
+                                                     typename Elem<T>::compute *__restrict__ sel, int B, int L,
                                                      int V, int Tn, const int64_t *__restrict__ eos_out_len,
                                                      const int64_t *__restrict__ eos_tgt_len,
                                                      typename Elem<T>::compute *__restrict__ lse_out,
@@ -300,20 +334,13 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
     {
-        const int64_t slot = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;  // one row per workgroup
-        if (slot >= rows) return;
-        // Rows of nodes beyond the sentence's graph (pads) feed nothing downstream of the criterion: neither sweep reads
-        // them and their gradient is zero.  When asked to, leave them unread and define their outputs as zeros
-        // (skip_pad_rows = 1: rows in batch order; 2: live rows first, see compact_row).
-        int64_t row = slot;
-        bool pad_row = false;  // workgroup-uniform
-        if (skip_pad_rows == 2) {
-            bool live;
-            row = compact_row((int)slot, (int)rows, eos_out_len, (int)rows / L, L, lane, live);
-            pad_row = !live;
-        } else if (skip_pad_rows) {
-            pad_row = row % L >= eos_out_len[row / L];
-        }
+        // One row per workgroup.  Rows of nodes beyond the sentence's graph (pads) feed nothing downstream of the
+        // criterion: neither sweep reads them and their gradient is zero.  When asked to, leave them unread and define
+        // their outputs as zeros (skip_pad_rows = 1: rows in batch order; 2: live rows first, see compact_row).
+        RowOf at;
+        if (!row_of_workgroup(skip_pad_rows, eos_out_len, B, L, lane, at)) return;
+        const int64_t row = (int64_t)at.b * L + at.p;
+        const bool pad_row = !at.live;  // workgroup-uniform
         T *xr = x + row * (int64_t)V;
         if (pad_row) {
             for (int s2 = tid; s2 < Tn; s2 += NT) sel[row * (int64_t)Tn + s2] = (CT)0;
@@ -331,8 +358,7 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
         // before anything is stored to the row (the stores come after two workgroup reductions over the loaded data).
         int64_t tg[GMAX];
         {
-            const int64_t b = row / L, p = row % L;
-            const int64_t *ir = idx + b * sb + p * sl;
+            const int64_t *ir = idx + at.b * sb + at.p * sl;
 #pragma unroll
             for (int g = 0; g < GMAX; g++) {
                 const int s = tid + g * NT;
@@ -399,8 +425,7 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
         // optional fused eos mask (nat_pcfg_loss.py:111-115): only the last graph node may emit the last target token
         int eos_col = -1;
         if (eos_out_len != nullptr) {
-            const int64_t b = row / L, pnode = row % L;
-            if (pnode != eos_out_len[b] - 1) eos_col = (int)(eos_tgt_len[b] - 1);
+            if (at.p != eos_out_len[at.b] - 1) eos_col = (int)(eos_tgt_len[at.b] - 1);
         }
         const bool forced = fe.keep != nullptr && fe.keep[row] != 0;  // (nat_pcfg_loss.py:116-121)
 #pragma unroll
@@ -408,7 +433,7 @@ __global__ __launch_bounds__(NT) void lsg_fwd_kernel(T *__restrict__ x, const in
             int s = tid + g * NT;
             if (s < Tn) {
                 CT val = (s == eos_col) ? neg_inf(CT()) : rn.logprob(gv[g], sum);
-                if (forced && fe.matchmask[((row / L) * (int64_t)Tn + s) * L + row % L] == 0) val = neg_inf(CT());
+                if (forced && fe.matchmask[((int64_t)at.b * Tn + s) * L + at.p] == 0) val = neg_inf(CT());
                 sel[row * (int64_t)Tn + s] = val;
             }
         }
@@ -527,7 +552,7 @@ __global__ __launch_bounds__(NT) void ls_max_kernel(const T *__restrict__ x, typ
 template <typename T, int NT, int MAXC, int TCAP, bool FROM_LOGITS>
 __global__ __launch_bounds__(NT, FROM_LOGITS ? 1 : 6) void lsg_bwd_kernel(T *__restrict__ p, const int64_t *__restrict__ idx, int64_t sb,
                                                      int64_t sl, int64_t st,
-                                                     const typename Elem<T>::compute *__restrict__ gsel, int64_t rows,
+                                                     const typename Elem<T>::compute *__restrict__ gsel, int B,
                                                      int L, int V, int Tn,
                                                      const typename Elem<T>::compute *__restrict__ lse, LossTask loss,
                                                      const unsigned char *__restrict__ detach_rows,
@@ -549,7 +574,7 @@ __global__ __launch_bounds__(NT, FROM_LOGITS ? 1 : 6) void lsg_bwd_kernel(T *__r
     // scaling): folded into g in the compute type, ahead of the single rounding to the buffer's dtype (pcfg_loss.py:77-83,
     // 176-177 scale g before the cast as well)
     const CT gs = (FROM_LOGITS && gscale_dev != nullptr) ? (CT)*gscale_dev : (CT)1;
-    if (loss.out != nullptr && blockIdx.x == 0 && blockIdx.y == 0) criterion_loss_block<NT>(loss);  // workgroup-uniform
+    if (loss.out != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0) criterion_loss_block<NT>(loss);  // workgroup-uniform
     __shared__ __attribute__((aligned(16))) int s_idx[TCAP + 4];  // target column of position s, -1 if out of range; padded
                                                                   // to a multiple of four with -2 (matches nothing)
     __shared__ CT s_g[TCAP];         // g[s], zero for a detached row
@@ -557,26 +582,20 @@ __global__ __launch_bounds__(NT, FROM_LOGITS ? 1 : 6) void lsg_bwd_kernel(T *__r
     __shared__ __attribute__((aligned(16))) unsigned s_box[NT * BOX];  // (target << 16) | (chunk slot << 4) | element
     const int tid = threadIdx.x, lane = tid & 63;
 
-    const int64_t slot = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;  // one row per workgroup
     if (also_scale.p != nullptr && gscale_dev != nullptr) {  // a side task spread over every thread of the launch
-        const size_t total = (size_t)gridDim.x * gridDim.y * NT;
+        const size_t slot = ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+        const size_t total = (size_t)gridDim.x * gridDim.y * gridDim.z * NT;
         const float sc = *gscale_dev;
-        for (size_t i = (size_t)slot * NT + tid; i < also_scale.n; i += total) also_scale.p[i] *= sc;
+        for (size_t i = slot * NT + tid; i < also_scale.n; i += total) also_scale.p[i] *= sc;
     }
-    if (slot >= rows) return;
-    // Rows of nodes beyond the sentence's graph (pads) get no gradient from the criterion, whose backward sweep leaves
-    // their upstream gradient all zero: p * 0 plus zeros is zero whatever the row holds, so such a row is written
-    // without being read (pad_mode = 1: rows in batch order, the lengths come through the scalar cache; 2: live rows
-    // first, see compact_row).
-    int64_t row = slot;
-    bool pad_row = false;  // workgroup-uniform
-    if (pad_mode == 2) {
-        bool live_row;
-        row = compact_row((int)slot, (int)rows, pad_out_len, (int)rows / L, L, lane, live_row);
-        pad_row = !live_row;
-    } else if (pad_mode == 1) {
-        pad_row = row % L >= pad_out_len[row / L];
-    }
+    // One row per workgroup.  Rows of nodes beyond the sentence's graph (pads) get no gradient from the criterion, whose
+    // backward sweep leaves their upstream gradient all zero: p * 0 plus zeros is zero whatever the row holds, so such a
+    // row is written without being read (pad_mode = 1: rows in batch order, the lengths come through the scalar cache; 2:
+    // live rows first, see compact_row).
+    RowOf at;
+    if (!row_of_workgroup(pad_mode, pad_out_len, B, L, lane, at)) return;
+    const int64_t row = (int64_t)at.b * L + at.p;
+    const bool pad_row = !at.live;  // workgroup-uniform
     T *pr = p + row * (int64_t)V;
     const RowSplit<T> sp(pr, V);
     vec16 *pv = reinterpret_cast<vec16 *>(pr + sp.head);
@@ -592,7 +611,7 @@ __global__ __launch_bounds__(NT, FROM_LOGITS ? 1 : 6) void lsg_bwd_kernel(T *__r
 
     // The small per-row inputs are requested first (independent loads, no chain), the row's chunks right behind them.
     const CT *gr = gsel + row * (int64_t)Tn;
-    const int64_t *ir = idx + (row / L) * sb + (row % L) * sl;
+    const int64_t *ir = idx + at.b * sb + at.p * sl;
     // a row whose gathered values were detached (force-emit, nat_pcfg_loss.py:121) gets no gradient at all
     unsigned char detached = 0;
     if (detach_rows != nullptr) detached = detach_rows[row];
@@ -767,13 +786,18 @@ inline dim3 row_grid(int64_t rows) {
     const int64_t gx = rows < (1LL << 30) ? rows : (1LL << 30);
     return dim3((unsigned)gx, (unsigned)((rows + gx - 1) / gx));
 }
+// One workgroup per (node, sentence): see row_of_workgroup.
+inline dim3 node_sentence_grid(int64_t B, int L) {
+    const int64_t gy = B < 65535 ? B : 65535;
+    return dim3((unsigned)L, (unsigned)gy, (unsigned)((B + gy - 1) / gy));
+}
 
 // How a launch that leaves out the rows of pad nodes orders its rows: 2 = live rows first (batches of up to COMPACT_MAX_B
 // sentences whose row count fits an int), 1 = batch order.
 inline int pad_row_mode(int64_t rows, int L) { return (rows / L <= COMPACT_MAX_B && rows < (1LL << 30)) ? 2 : 1; }
 
 template <typename T>
-int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, void *sel, int grad, int64_t rows,
+int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, void *sel, int grad, int64_t B,
                int L, int V, int Tn, const int64_t *eos_ol, const int64_t *eos_tl, void *lse, int64_t *argmax, hipStream_t stream,
                ForceEmit fe = ForceEmit{nullptr, nullptr}, int skip_pad_rows = 0) {
     using CT = typename Elem<T>::compute;
@@ -782,23 +806,25 @@ int launch_fwd(void *x, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
     constexpr int MAXC = 5120 / NT;
     constexpr int GMAX = 1024 / NT;
     if (Tn > NT * GMAX) return fail(PCFGNAT_EUNSUPPORTED, "logsoftmax_gather: T=%d exceeds %d targets per row", Tn, NT * GMAX);
-    const dim3 grid = row_grid(rows);
-    if (skip_pad_rows) skip_pad_rows = pad_row_mode(rows, L);
+    PCFGNAT_REQUIRE(B * L < (1LL << 31) && B < 65535LL * 65535LL, "logsoftmax_gather: %lld rows exceed what one launch indexes",
+                    (long long)(B * L));
+    const dim3 grid = node_sentence_grid(B, L);
+    if (skip_pad_rows) skip_pad_rows = pad_row_mode(B * L, L);
     if (grad)
         hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, true, false>), grid, dim3(NT), 0, stream, (T *)x, idx, sb,
-                           sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax, fe, skip_pad_rows);
+                           sl, st, (CT *)sel, (int)B, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax, fe, skip_pad_rows);
     else if (lse != nullptr)  // log-sum-exp split: the backward pass over the same rows follows
         hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, false, true>), grid, dim3(NT), 0, stream, (T *)x, idx,
-                           sb, sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax, fe, skip_pad_rows);
+                           sb, sl, st, (CT *)sel, (int)B, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax, fe, skip_pad_rows);
     else
         hipLaunchKernelGGL((lsg_fwd_kernel<T, NT, MAXC, GMAX, false, false>), grid, dim3(NT), 0, stream, (T *)x, idx,
-                           sb, sl, st, (CT *)sel, rows, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax, fe, skip_pad_rows);
+                           sb, sl, st, (CT *)sel, (int)B, L, V, Tn, eos_ol, eos_tl, (CT *)lse, argmax, fe, skip_pad_rows);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
 
 template <typename T>
-int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, const void *g, int64_t rows, int L, int V,
+int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, const void *g, int64_t B, int L, int V,
                int Tn, const void *lse, const LossTask &loss, hipStream_t stream, const unsigned char *detach_rows = nullptr,
                const int64_t *pad_out_len = nullptr, int pad_rows_zeroed = 0, const float *gscale_dev = nullptr,
                ScaleTask also_scale = ScaleTask{nullptr, 0}) {
@@ -807,17 +833,19 @@ int launch_bwd(void *p, const int64_t *idx, int64_t sb, int64_t sl, int64_t st, 
     constexpr int MAXC = 10;
     constexpr int TCAP = 1024;  // most targets per row; up to NT of them the kernel with one target per thread (fewer registers)
     if (Tn > TCAP) return fail(PCFGNAT_EUNSUPPORTED, "logsoftmax_gather_backward: T=%d exceeds %d targets per row", Tn, TCAP);
-    const dim3 grid = row_grid(rows);
-    const int pad_mode = pad_out_len == nullptr ? 0 : pad_row_mode(rows, L);
+    PCFGNAT_REQUIRE(B * L < (1LL << 31) && B < 65535LL * 65535LL, "logsoftmax_gather_backward: %lld rows exceed what one launch indexes",
+                    (long long)(B * L));
+    const dim3 grid = node_sentence_grid(B, L);
+    const int pad_mode = pad_out_len == nullptr ? 0 : pad_row_mode(B * L, L);
 #define PCFGNAT_LSG_BWD(tcap)                                                                                                              \
     do {                                                                                                                                   \
         if (lse != nullptr)                                                                                                                \
             hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, tcap, true>), grid, dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,              \
-                               (const CT *)g, rows, L, V, Tn, (const CT *)lse, loss, detach_rows, pad_out_len, pad_mode, pad_rows_zeroed,  \
+                               (const CT *)g, (int)B, L, V, Tn, (const CT *)lse, loss, detach_rows, pad_out_len, pad_mode, pad_rows_zeroed, \
                                gscale_dev, also_scale);                                                                                    \
         else                                                                                                                               \
             hipLaunchKernelGGL((lsg_bwd_kernel<T, NT, MAXC, tcap, false>), grid, dim3(NT), 0, stream, (T *)p, idx, sb, sl, st,             \
-                               (const CT *)g, rows, L, V, Tn, (const CT *)nullptr, loss, detach_rows, pad_out_len, pad_mode,               \
+                               (const CT *)g, (int)B, L, V, Tn, (const CT *)nullptr, loss, detach_rows, pad_out_len, pad_mode,             \
                                pad_rows_zeroed, nullptr, ScaleTask{nullptr, 0});                                                           \
     } while (0)
     if (Tn <= NT) PCFGNAT_LSG_BWD(NT);
@@ -863,11 +891,11 @@ static int lsg_forward_dispatch(void *word_ins_out, int dtype, const int64_t *se
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case PCFGNAT_F16:
-            return launch_fwd<__half>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe, skip_pad_rows);
+            return launch_fwd<__half>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe, skip_pad_rows);
         case PCFGNAT_F32:
-            return launch_fwd<float>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe, skip_pad_rows);
+            return launch_fwd<float>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe, skip_pad_rows);
         case PCFGNAT_F64:
-            return launch_fwd<double>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B * L, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe, skip_pad_rows);
+            return launch_fwd<double>(word_ins_out, select_idx, sb, sl, st, selected, require_grad, B, (int)L, (int)V, (int)T, eos_ol, eos_tl, lse, argmax, s, fe, skip_pad_rows);
         default:
             return fail(PCFGNAT_EINVAL, "logsoftmax_gather: unknown dtype code %d (float16, float32, float64 are dispatched)", dtype);
     }
@@ -927,11 +955,11 @@ static int lsg_backward_dispatch(void *buf, int dtype, const int64_t *select_idx
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case PCFGNAT_F16:
-            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev, also_scale);
+            return launch_bwd<__half>(buf, select_idx, sb, sl, st, grad_selected, B, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev, also_scale);
         case PCFGNAT_F32:
-            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev, also_scale);
+            return launch_bwd<float>(buf, select_idx, sb, sl, st, grad_selected, B, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev, also_scale);
         case PCFGNAT_F64:
-            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B * L, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev, also_scale);
+            return launch_bwd<double>(buf, select_idx, sb, sl, st, grad_selected, B, (int)L, (int)V, (int)T, lse, loss, s, detach_rows, pad_out_len, pad_rows_zeroed, gscale_dev, also_scale);
         default:
             return fail(PCFGNAT_EINVAL, "logsoftmax_gather_backward: unknown dtype code %d", dtype);
     }
