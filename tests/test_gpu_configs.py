@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 import torch
 
+import gradcheck
 import oracle_ops
 from oracle import oracle
 from pcfg_nat_amd import custom_ops as ops
@@ -60,6 +61,7 @@ def _check_training_batch(batch, chunk, grad_tol=1e-4):
     # the oracle (float64 tables) on every sentence, end to end through the same glue, a few sentences at a time to bound
     # the host memory of the [*, L, V] float tensors
     worst = {"ll": 0.0, "match_all_grad": 0.0, "links_grad": 0.0, "logits_grad": 0.0}
+    worst_bands = np.zeros((2, len(gradcheck.BANDS)))
     for s0 in range(0, B, chunk):
         sample = list(range(s0, min(B, s0 + chunk)))
         sub = {k: (v[sample] if torch.is_tensor(v) else v) for k, v in batch.items()}
@@ -81,6 +83,9 @@ def _check_training_batch(batch, chunk, grad_tol=1e-4):
             err = ((mgd[b] - mg_o[i]).abs().max() / mg_o[i].abs().max()).item()
             worst["match_all_grad"] = max(worst["match_all_grad"], err)
             assert err <= grad_tol, "match_all_grad of sentence %d: normwise error %.2e" % (b, err)
+            # every entry, relative to its own size
+            worst_bands[0] = np.maximum(worst_bands[0], gradcheck.assert_elementwise(mgd[b].numpy(), mg_o[i].numpy(), "match_all_grad of sentence %d" % b))
+            worst_bands[1] = np.maximum(worst_bands[1], gradcheck.assert_elementwise(lg[b].numpy(), lg_o[i].numpy(), "links_grad of sentence %d" % b))
             want_g = leaf.grad[i]
             got_g = g[b].cpu()
             # fp16 buffer: each element within fp16 rounding of the fp32 gradient (plus the rounding of the row factor)
@@ -91,6 +96,9 @@ def _check_training_batch(batch, chunk, grad_tol=1e-4):
     print("all %d sentences against the float64 oracle, worst errors: ll %.2e relative, match_all_grad %.2e, links_grad %.2e "
           "normwise, logits gradient %.2e of the row maximum (fp16 storage)"
           % (B, worst["ll"], worst["match_all_grad"], worst["links_grad"], worst["logits_grad"]))
+    print("worst relative error of an entry, by its share of the sentence maximum (%s): match_all_grad %s, links_grad %s"
+          % (", ".join(">= %.0e" % f for f, _ in gradcheck.BANDS), " ".join("%.1e" % e for e in worst_bands[0]),
+             " ".join("%.1e" % e for e in worst_bands[1])))
 
 
 def test_config2_full_size():

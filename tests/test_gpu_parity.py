@@ -9,6 +9,8 @@ import math
 
 import numpy as np
 import pytest
+
+import gradcheck
 import torch
 
 from oracle import oracle
@@ -305,6 +307,7 @@ def test_inside_forward_backward_vs_oracle(case):
     lg_want = lg64 * wn[:, None, None, None]
     mg_got, lg_got = md.grad.cpu().double().numpy(), ld.grad.cpu().double().numpy()
     assert np.isfinite(mg_got).all() and np.isfinite(lg_got).all()
+    worst = np.zeros((2, len(gradcheck.BANDS)))
     for bi in range(len(wn)):
         scale = max(np.abs(mg_want[bi]).max(), 1e-30)
         assert np.abs(mg_got[bi] - mg_want[bi]).max() <= 1e-4 * scale, (case, bi)
@@ -312,6 +315,12 @@ def test_inside_forward_backward_vs_oracle(case):
         assert np.abs(lg_got[bi] - lg_want[bi]).max() <= 1e-4 * scale, (case, bi)
         if not fin[bi]:
             assert not mg_got[bi].any() and not lg_got[bi].any()
+        # every entry, relative to its own size
+        worst[0] = np.maximum(worst[0], gradcheck.assert_elementwise(mg_got[bi], mg_want[bi], "%s: match_all_grad of sentence %d" % (case, bi)))
+        worst[1] = np.maximum(worst[1], gradcheck.assert_elementwise(lg_got[bi], lg_want[bi], "%s: links_grad of sentence %d" % (case, bi)))
+    print("%s: worst relative error of an entry, by its share of the sentence maximum (%s): match_all_grad %s, links_grad %s"
+          % (case, ", ".join(">= %.0e" % f for f, _ in gradcheck.BANDS), " ".join("%.1e" % e for e in worst[0]),
+             " ".join("%.1e" % e for e in worst[1])))
 
 
 def _inside_all(batch, match):
