@@ -153,6 +153,8 @@ int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *ma
  * enqueued (BASELINE-sized batches fit: 40 sentences of 128 nodes take 2 MiB, 8 of 512 nodes with 140 target tokens
  * 24 MiB).  All calls on one GPU share that GPU's array: calls that overlap there (two streams, two threads) race, and
  * the kernels of one call must have finished before the next call on another stream is enqueued.
+ * The first call on a device looks up the array's address and sets kernel attributes (hipGetSymbolAddress,
+ * hipFuncSetAttribute), which a stream capture may refuse: make one call per device and shape outside a capture first.
  */
 #define PCFGNAT_STATIC_AUX_FLOATS (8u * 1024u * 1024u)
 size_t pcfgnat_static_aux_floats(void);
@@ -160,50 +162,6 @@ int pcfgnat_pcfg_loss_forward_backward_static(const float *grad_output, const fl
                                               const int64_t *output_length, const int64_t *target_length, float *S,
                                               float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T,
                                               int64_t ml, void *stream);
-
-/*
- * No counterpart in the reference: tuning of the long-graph paths (max_left = 1; inside sweeps for 130 <= L <= 1026, the
- * Viterbi sweep of pcfgnat_viterbi_decode for 194 <= L <= 514).  There a sentence is
- * swept by one workgroup per block of 16 main-chain nodes, the blocks following each other as a pipeline, as long as the
- * batch needs no more than max_workgroups of them (B * 4 * ceil((L/2)/64) <= max_workgroups, default 2^20), and by one
- * workgroup per sentence otherwise.  pcfgnat_pcfg_loss_forward_backward runs the forward and the outside pipeline of a
- * sentence side by side in one launch while twice that number fits, one after the other otherwise.  A block that waits
- * for the one ahead of it for more than spin_limit rounds of polling
- * (default 2^15, some tens of milliseconds; the blocks of a sentence normally follow each other at about 2 us) gives the
- * sentence up, and the one-workgroup sweep redoes it in the same call; results
- * are the same either way up to fp32 rounding.  max_workgroups = 0 switches the pipeline off; a negative argument leaves
- * that setting unchanged.  The two settings are process-wide (all threads, streams and devices), meant for tests and
- * tuning, and take effect with the next call.
- *
- * Progress: the waits rely on the leading blocks of a sentence having the lower workgroup indices and on workgroups being
- * started in index order, so that a block never waits for one that has not been started while it occupies the slot
- * that block needs.  HIP does not promise that order; where it does not hold (or where another tenant keeps the leading
- * block from running) the bounded wait expires and the sentence is redone, which costs time, never correctness.
- */
-void pcfgnat_pipeline_config(int max_workgroups, int spin_limit);
-
-/*
- * No counterpart in the reference: the rule posteriors of graphs beyond 130 nodes are summed over the target positions on
- * the matrix cores, as products of two factors per term; a 32x32 tile of (parent, child) pairs in which the product of
- * the largest factors would exceed 2^log2_limit (default 120) is recomputed with one exponential per term instead,
- * which has no range limit.  Process-wide, for tests: a limit of -inf sends every tile down the second path.
- */
-void pcfgnat_links_grad_range_limit(float log2_limit);
-
-/*
- * No counterpart in the reference: diagnostic counters of that fallback since the library was loaded - inside sweeps
- * (forward and outside counted apart) and single-call Viterbi decodes that the one-workgroup kernels redid because a
- * pipelined sweep gave up.  Reads two device counters of the current device (synchronises with the device); reset != 0
- * clears them.  A caller that sees them grow outside tests is paying the bounded wait on those calls.
- */
-int pcfgnat_pipeline_redo_counts(unsigned long long *inside_sweeps, unsigned long long *viterbi_sentences, int reset);
-
-/*
- * No counterpart in the reference: a wait limit of its own for the outside pipeline where the two pipelines of a sentence
- * run side by side (pcfgnat_pcfg_loss_forward_backward); negative (the default) = the common limit of
- * pcfgnat_pipeline_config.  It lets a test make one of the two sweeps give up and be redone while the other completes.
- */
-void pcfgnat_pipeline_outside_spin_limit(int spin_limit);
 
 /*
  * The float64 instantiation the reference also dispatches (AT_DISPATCH_FLOATING_TYPES in pcfg_loss.cu:395,

@@ -22,7 +22,7 @@ _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
 _int = ctypes.c_int
 
-# name -> (restype, argtypes); mirrors include/pcfg_nat_hip.h one to one
+# name -> (restype, argtypes); mirrors include/pcfg_nat_hip.h and include/pcfg_nat_hip_testing.h one to one
 SIGNATURES = {
     "pcfgnat_abi_version": (_int, []),
     "pcfgnat_last_error": (ctypes.c_char_p, []),
@@ -35,7 +35,8 @@ SIGNATURES = {
     "pcfgnat_pcfg_aux_floats": (ctypes.c_size_t, [_i64, _i64, _i64, _i64]),
     "pcfgnat_pipeline_config": (None, [_int, _int]),
     "pcfgnat_pipeline_outside_spin_limit": (None, [_int]),
-    "pcfgnat_pipeline_redo_counts": (_int, [_vp, _vp, _int]),
+    "pcfgnat_pipeline_redo_wait_limit": (None, [_int]),
+    "pcfgnat_pipeline_redo_counts": (_int, [_vp, _vp, _vp, _int]),
     "pcfgnat_links_grad_range_limit": (None, [ctypes.c_float]),
     "pcfgnat_pcfg_loss": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_pcfg_loss_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),

@@ -8,6 +8,7 @@
 #include <stdarg.h>
 
 #include "../../include/pcfg_nat_hip.h"
+#include "../../include/pcfg_nat_hip_testing.h"
 
 namespace pcfgnat {
 

@@ -108,6 +108,10 @@ constexpr double LN2_D = 0.6931471805599453094;
 // Diagnostic: sweeps (forward or outside, counted apart) that the one-workgroup kernels redid because the pipelined
 // sweep of the sentence gave up, since the library was loaded (pcfgnat_pipeline_redo_counts).
 __device__ unsigned long long g_inside_redone;
+// Diagnostic: sentences given up for good - both pipelined sweeps gave up AND the outside sweep's second chance outwaited
+// its bound for the forward's (seconds; pcfgnat_pipeline_redo_wait_limit).  Their log-likelihood is NaN, which the
+// criterion counts as an invalid sentence: never a wrong gradient, and never unnoticed, thanks to this counter.
+__device__ unsigned long long g_inside_given_up;
 
 __device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float lg2(float x) { return __builtin_amdgcn_logf(x); }
@@ -2013,6 +2017,9 @@ __global__ __launch_bounds__(NT) void inside_bwd_ml1_stream_kernel(const float *
 // different L2s).  In the normal case neither flag is set and the launch ends at once - one launch where two stood.
 // Dynamic LDS: the larger of the two sweeps' needs without the emissions.
 constexpr int FLAG_FWD_REDONE = 2;
+// set where the second chance of a sentence was given up: pipeline_finish_kernel, the next launch, then turns the
+// sentence's log-likelihood into NaN (not this launch: the forward's workgroup may still be writing it)
+constexpr int FLAG_GIVEN_UP = 3;
 template <int SLB>
 __global__ __launch_bounds__(NT) void inside_redo_ml1_stream_kernel(const float *match_all, const float *links, const int64_t *out_len,
                                                                    const int64_t *tgt_len, float *S, float *aux, int L, int T, int Mc,
@@ -2035,15 +2042,18 @@ __global__ __launch_bounds__(NT) void inside_redo_ml1_stream_kernel(const float 
         __shared__ int s_arrived;
         if (threadIdx.x == 0) {
             // The forward's workgroup is running or done and waits for nobody, so this wait ends; it is bounded all the
-            // same (seconds), like every wait between workgroups here.  Past the bound the sentence is given up: its
-            // log-likelihood becomes NaN, which the posterior kernels and the loss treat as an invalid sentence.
+            // same (seconds), like every wait between workgroups here.  Past the bound the sentence is given up: the next
+            // launch turns its log-likelihood into NaN, which the posterior kernels and the loss treat as an invalid sentence.
             int arrived = 0;
             for (int spins = 0; spins < wait_limit && !arrived; spins++) {
                 arrived = __hip_atomic_load(flags + FLAG_FWD_REDONE, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) != 0;
                 if (!arrived) __builtin_amdgcn_s_sleep(16);
             }
             s_arrived = arrived;
-            if (!arrived) S[(size_t)b * Mc * (T + 2)] = __builtin_nanf("");
+            if (!arrived) {
+                flags[FLAG_GIVEN_UP] = 1;
+                atomicAdd(&g_inside_given_up, 1ull);
+            }
         }
         __syncthreads();
         if (!s_arrived) return;
@@ -2660,8 +2670,12 @@ __global__ __launch_bounds__(256) void pipeline_rebase_kernel(float *__restrict_
 // After the sweeps side by side and the forward's redo: grid (2 CL - 1, B); the first CL-1 blocks of a sentence rebase the
 // forward tables, the other CL finish the outside sweep's.  Dynamic LDS: 2 (T+4) doubles.
 __global__ __launch_bounds__(256) void pipeline_finish_kernel(float *__restrict__ aux, const int64_t *__restrict__ out_len,
-                                                             const int64_t *__restrict__ tgt_len, int L, int T, int Mc, int CL) {
+                                                             const int64_t *__restrict__ tgt_len, int L, int T, int Mc, int CL,
+                                                             float *__restrict__ S) {
     extern __shared__ double sm_dyn[];
+    // a sentence whose second chance was given up (see inside_redo_ml1_stream_kernel) becomes an invalid one
+    if (blockIdx.x == 0 && threadIdx.x == 0 && ExchangeView(aux, blockIdx.y, Mc, T).flags[FLAG_GIVEN_UP] != 0)
+        S[(size_t)blockIdx.y * Mc * (T + 2)] = __builtin_nanf("");
     if ((int)blockIdx.x < CL - 1)  // workgroup-uniform
         pipeline_rebase_block((int)blockIdx.x + 1, (int)blockIdx.y, aux, out_len, tgt_len, L, T, Mc, sm_dyn);
     else
@@ -3171,12 +3185,28 @@ __global__ __launch_bounds__(256) void criterion_loss_kernel(const float *__rest
 // pcfgnat_pipeline_config.
 std::atomic<int> g_pipeline_max_wg{1 << 20}, g_pipeline_spin_limit{PCFGNAT_DEFAULT_SPIN_LIMIT};
 std::atomic<int> g_pipeline_spin_limit_outside{-1};  // side-by-side launch only; negative: the common limit
+// Bound of the one wait of the second-chance launch (the outside sweep's workgroup for the forward's, where both are
+// redone), in polls of about a microsecond.  pcfgnat_pipeline_redo_wait_limit.
+constexpr int DEFAULT_REDO_WAIT_LIMIT = 1 << 23;
+std::atomic<int> g_redo_wait_limit{DEFAULT_REDO_WAIT_LIMIT};
 // Largest base-2 exponent a factor of the rule posteriors of long graphs may have on the matrix cores (see
 // links_grad_ml1_stream_kernel); a tile beyond it is recomputed term by term.  pcfgnat_links_grad_range_limit.
 std::atomic<float> g_links_grad_range_limit{120.f};
-int pipeline_chunks(int B, int T, int Mc) {  // NQ, or 0 where the pipelined sweeps do not apply
+// How a call sweeps its long graphs, decided once per call from one reading of the process-wide setting (a setting that
+// changes while a call is being enqueued must not reach half of its launches).
+struct PipelinePlan {
+    int NQ;             // chunks of 64 nodes per sentence; 0: the pipelined sweeps do not apply
+    bool side_by_side;  // forward and outside pipeline in one launch
+};
+PipelinePlan pipeline_plan(int B, int T, int Mc) {
+    const int max_wg = g_pipeline_max_wg.load();
     const int NQ = stream_mp(Mc) / 64, CL = 64 * NQ / NLP;
-    return (NQ >= 2 && NQ <= 8 && T + 2 < 4096 && (int64_t)B * CL <= g_pipeline_max_wg.load()) ? NQ : 0;
+    PipelinePlan plan{0, false};
+    if (NQ >= 2 && NQ <= 8 && T + 2 < 4096 && (int64_t)B * CL <= max_wg) {
+        plan.NQ = NQ;
+        plan.side_by_side = (int64_t)2 * B * CL <= max_wg;
+    }
+    return plan;
 }
 
 template <int NQ>
@@ -3246,21 +3276,14 @@ int launch_bwd_pipe(const float *S, float *aux, const float *match_all, const in
     return PCFGNAT_OK;
 }
 
-// The sweeps run side by side while the batch needs no more than the configured number of workgroups for both pipelines.
-bool side_by_side_applies(int B, int T, int Mc) {
-    const int NQ = pipeline_chunks(B, T, Mc);
-    return NQ != 0 && (int64_t)2 * B * (64 * NQ / NLP) <= g_pipeline_max_wg.load();
-}
-
 // zero_slabs: links_grad, where the call also has the backward to do (its slab is then zeroed here, beside the compact copies)
 int launch_fwd_stream(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int B,
-                      int L, int T, int Mc, hipStream_t stream, bool side_by_side = false, float *zero_slabs = nullptr) {
+                      int L, int T, int Mc, hipStream_t stream, int NQ, bool side_by_side = false, float *zero_slabs = nullptr) {
     const int MP = stream_mp(Mc);
     PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss: aux must be 16-byte aligned");
     hipLaunchKernelGGL(compact_links_ml1_kernel, dim3(MP / 32, MP / 32, B), dim3(256), 0, stream, links, ol, aux, L, T, Mc, MP, zero_slabs);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     // pipelined sweep first where it applies; the one-workgroup sweep then only redoes sentences whose blocks gave up
-    const int NQ = pipeline_chunks(B, T, Mc);
     int rc = PCFGNAT_OK;
     switch (NQ) {
         case 2: rc = launch_fwd_pipe<2>(match_all, ol, tl, S, aux, B, L, T, Mc, stream, side_by_side); break;
@@ -3281,7 +3304,7 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
         // set and ends at once), then both sweeps' tables to common offsets and the corrections of the posteriors
         const size_t base_bwd = ((size_t)5 * MP + T + 4) * sizeof(float);
         const size_t lds = base > base_bwd ? base : base_bwd;
-        constexpr int WAIT_LIMIT = 1 << 23;  // polls of about a microsecond
+        const int WAIT_LIMIT = g_redo_wait_limit.load();  // polls of about a microsecond
         if (Mc <= NT / 4)
             hipLaunchKernelGGL(inside_redo_ml1_stream_kernel<4>, dim3(B, 2), dim3(NT), lds, stream, match_all, links, ol, tl, S, aux, L, T,
                                Mc, MP, WAIT_LIMIT);
@@ -3291,7 +3314,7 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
         PCFGNAT_HIP_CHECK(hipGetLastError());
         const int CL = 64 * NQ / NLP;
         hipLaunchKernelGGL(pipeline_finish_kernel, dim3(2 * CL - 1, B), dim3(256), (size_t)2 * (T + 4) * sizeof(double), stream, aux, ol, tl,
-                           L, T, Mc, CL);
+                           L, T, Mc, CL, S);
         PCFGNAT_HIP_CHECK(hipGetLastError());
         return PCFGNAT_OK;
     }
@@ -3310,14 +3333,13 @@ int launch_fwd_stream(const float *match_all, const float *links, const int64_t 
 // side_by_side: the outside pipeline has already run, beside the forward one (launch_both_stream): only the redo of the
 // sentences it gave up and the posteriors (with their per-column corrections) are left to do.
 int launch_bwd_stream(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
-                      const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, Seed seed, hipStream_t stream,
+                      const int64_t *tl, float *mg, float *lg, int B, int L, int T, int Mc, Seed seed, hipStream_t stream, int NQ,
                       bool side_by_side = false, bool slabs_zeroed = false) {
     const int MP = stream_mp(Mc);
     const int tiles = (Mc + LG_TILE - 1) / LG_TILE;
     PCFGNAT_REQUIRE(((uintptr_t)aux & 15) == 0, "pcfg_loss_backward: aux must be 16-byte aligned");
     const size_t base = ((size_t)5 * MP + T + 4) * sizeof(float);
     const size_t with_match = base + (size_t)2 * Mc * T * sizeof(float);
-    const int NQ = pipeline_chunks(B, T, Mc);
     int rc = PCFGNAT_OK;
     switch (side_by_side ? 0 : NQ) {
         case 2: rc = launch_bwd_pipe<2>(S, aux, match_all, ol, tl, B, L, T, Mc, stream); break;
@@ -3476,12 +3498,17 @@ extern "C" void pcfgnat_pipeline_outside_spin_limit(int spin_limit) { g_pipeline
 
 extern "C" void pcfgnat_links_grad_range_limit(float log2_limit) { g_links_grad_range_limit.store(log2_limit); }
 
-extern "C" int pcfgnat_pipeline_redo_counts(unsigned long long *inside_sweeps, unsigned long long *viterbi_sentences, int reset) {
-    PCFGNAT_REQUIRE(inside_sweeps && viterbi_sentences, "pipeline_redo_counts: null pointer");
+extern "C" void pcfgnat_pipeline_redo_wait_limit(int polls) { g_redo_wait_limit.store(polls < 0 ? DEFAULT_REDO_WAIT_LIMIT : polls); }
+
+extern "C" int pcfgnat_pipeline_redo_counts(unsigned long long *inside_sweeps, unsigned long long *viterbi_sentences,
+                                            unsigned long long *inside_given_up, int reset) {
+    PCFGNAT_REQUIRE(inside_sweeps && viterbi_sentences && inside_given_up, "pipeline_redo_counts: null pointer");
     PCFGNAT_HIP_CHECK(hipMemcpyFromSymbol(inside_sweeps, HIP_SYMBOL(g_inside_redone), sizeof(*inside_sweeps)));
+    PCFGNAT_HIP_CHECK(hipMemcpyFromSymbol(inside_given_up, HIP_SYMBOL(g_inside_given_up), sizeof(*inside_given_up)));
     if (reset) {
         const unsigned long long zero = 0;
         PCFGNAT_HIP_CHECK(hipMemcpyToSymbol(HIP_SYMBOL(g_inside_redone), &zero, sizeof(zero)));
+        PCFGNAT_HIP_CHECK(hipMemcpyToSymbol(HIP_SYMBOL(g_inside_given_up), &zero, sizeof(zero)));
     }
     return viterbi_redo_count(viterbi_sentences, reset);
 }
@@ -3505,7 +3532,8 @@ extern "C" int pcfgnat_pcfg_loss(const float *match_all, const float *links, con
     const int Mc = (int)((L - 2) / 2 + 1);
     hipStream_t s = (hipStream_t)stream;
     if (Mc <= 64) return launch_fwd<1>(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s);
-    return launch_fwd_stream(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s);
+    return launch_fwd_stream(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s,
+                             pipeline_plan((int)B, (int)T, Mc).NQ);
 }
 
 int pcfgnat::inside_backward_impl(const float *grad_output, const float *S, float *aux, const float *match_all, const float *links,
@@ -3525,7 +3553,7 @@ int pcfgnat::inside_backward_impl(const float *grad_output, const float *S, floa
         return launch_bwd<1>(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
                              (int)L, (int)T, Mc, seed, s);
     return launch_bwd_stream(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
-                             (int)L, (int)T, Mc, seed, s);
+                             (int)L, (int)T, Mc, seed, s, pipeline_plan((int)B, (int)T, Mc).NQ);
 }
 
 extern "C" int pcfgnat_pcfg_loss_backward(const float *grad_output, const float *S, float *aux, const float *match_all,
@@ -3555,11 +3583,13 @@ int pcfgnat::inside_forward_backward_impl(const float *grad_output, const float 
         rc = launch_fused<1>(grad_output, match_all, links, output_length, target_length, S, aux, match_all_grad, links_grad, (int)B, (int)L,
                              (int)T, Mc, seed, s, &done, pad, pad_done);
     if (rc != PCFGNAT_OK || done) return rc;
-    if (ml == 1 && Mc > 64 && side_by_side_applies((int)B, (int)T, Mc)) {  // the two pipelined sweeps in one launch
-        rc = launch_fwd_stream(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s, true, links_grad);
+    const PipelinePlan plan = (ml == 1 && Mc > 64) ? pipeline_plan((int)B, (int)T, Mc) : PipelinePlan{0, false};
+    if (plan.side_by_side) {  // the two pipelined sweeps in one launch
+        rc = launch_fwd_stream(match_all, links, output_length, target_length, S, aux, (int)B, (int)L, (int)T, Mc, s, plan.NQ, true,
+                               links_grad);
         if (rc != PCFGNAT_OK) return rc;
         return launch_bwd_stream(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, (int)B,
-                                 (int)L, (int)T, Mc, seed, s, true, true);
+                                 (int)L, (int)T, Mc, seed, s, plan.NQ, true, true);
     }
     rc = pcfgnat_pcfg_loss(match_all, links, output_length, target_length, S, aux, B, L, T, ml, stream);
     if (rc != PCFGNAT_OK) return rc;

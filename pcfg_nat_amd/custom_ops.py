@@ -11,7 +11,6 @@ contract; the arithmetic runs in hand-written HIP kernels for gfx950 reached thr
 import ctypes
 import threading
 import time
-import weakref
 
 import torch
 from torch.autograd import Function
@@ -72,13 +71,20 @@ def links_grad_range_limit(log2_limit=120.0):
 
 
 def pipeline_redo_counts(reset=False):
-    """(inside sweeps, single-call Viterbi decodes) that the one-workgroup kernels had to redo on the current device
-    because a pipelined sweep gave up, since the library was loaded or the last reset.  Synchronises with the device."""
-    import ctypes
+    """(inside sweeps, single-call Viterbi decodes, sentences given up) on the current device since the library was loaded
+    or the last reset: sweeps and decodes that the one-workgroup kernels had to redo because a pipelined sweep gave up, and
+    sentences whose second chance also ran out of its (seconds long) bound and came back with a NaN log-likelihood - an
+    invalid sentence for the criterion; must stay zero.  Synchronises with the device."""
     lib = _lib.load()
-    a, b = ctypes.c_ulonglong(0), ctypes.c_ulonglong(0)
-    _lib.check(lib.pcfgnat_pipeline_redo_counts(ctypes.byref(a), ctypes.byref(b), int(bool(reset))), lib)
-    return a.value, b.value
+    a, b, c = ctypes.c_ulonglong(0), ctypes.c_ulonglong(0), ctypes.c_ulonglong(0)
+    _lib.check(lib.pcfgnat_pipeline_redo_counts(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c), int(bool(reset))), lib)
+    return a.value, b.value, c.value
+
+
+def pipeline_redo_wait_limit(polls=-1):
+    """Test hook (process-wide): bound of the outside sweep's wait for the forward sweep where both are redone, in polls of
+    about a microsecond (negative: the default, 2**23); 0 makes the wait expire at once, which gives the sentence up."""
+    _lib.load().pcfgnat_pipeline_redo_wait_limit(int(polls))
 
 
 def _stream(t):
@@ -563,18 +569,25 @@ _MASK_CACHE = {}
 
 def _as_flag_mask(t):
     """A support mask as the kernels read it (one byte per entry, non-zero = set).  The masks of a model are built once per
-    graph length and handed to every call: the converted copy of an integer mask is kept while the tensor it was made
-    from is alive and unchanged (same storage, same version counter), so that a call does not pay a launch per mask."""
+    graph length and handed to every call, often as fresh views of one tensor (``mask[:L, :L]``): the converted copy of an
+    integer mask is kept under the view's storage address, offset, shape, strides and version counter, together with the
+    tensor it was made from (which keeps that storage, and with it the address, from being reused), so that a call does not
+    pay a launch per mask.  Tensors without a version counter (created under ``torch.inference_mode``) are converted on
+    every call."""
     if t.dtype in (torch.bool, torch.uint8):
         return t.contiguous()
-    key = (t.data_ptr(), t._version, t.dtype, tuple(t.shape), tuple(t.stride()), str(t.device))
+    try:
+        version = t._version
+    except RuntimeError:  # inference tensors do not track versions
+        return t.ne(0).contiguous()
+    key = (t.untyped_storage().data_ptr(), t.storage_offset(), version, t.dtype, tuple(t.shape), tuple(t.stride()), str(t.device))
     hit = _MASK_CACHE.get(key)
-    if hit is not None and hit[0]() is t:
+    if hit is not None:
         return hit[1]
     flags = t.ne(0).contiguous()
     if len(_MASK_CACHE) >= 64:
         _MASK_CACHE.clear()
-    _MASK_CACHE[key] = (weakref.ref(t), flags)
+    _MASK_CACHE[key] = (t, flags)
     return flags
 
 
@@ -607,6 +620,10 @@ class PCFGExtractLinksFunc(Function):
         with torch.cuda.device(dev):
             st = _stream(query_chunks)
             q, kl, kr = query_chunks.contiguous(), key_chunks_left.contiguous(), key_chunks_right.contiguous()
+            # what the kernels with the products inside also ask for: chunks on 16-byte boundaries (a contiguous view at
+            # an odd storage offset is not) and, in the backward, a batch that fits its grid; otherwise the five-call
+            # form, which takes any layout
+            fused = fused and all(x.data_ptr() % 16 == 0 for x in (q, kl, kr)) and B <= 32767
             fused_bwd = bool(lib.pcfgnat_extract_links_fused_backward_supported(code, L, H, F))
             need_grad = any(ctx.needs_input_grad[:4])
             ctx.fused = fused and (fused_bwd or not need_grad)
@@ -660,6 +677,8 @@ class PCFGExtractLinksFunc(Function):
             with torch.cuda.device(dev):
                 st = _stream(q)
                 G = grad_links.float().contiguous()
+                if G.data_ptr() % 16:  # (a view at an odd offset: the kernels read it in 16-byte pieces)
+                    G = G.clone()
                 dq, dkl, dkr = torch.empty((3, B, L, H, F), dtype=q.dtype, device=dev).unbind(0)  # one allocation each way
                 nws = (lib.pcfgnat_extract_links_fused_backward_workspace_bytes(B, L, H, F) + 3) // 4
                 block = torch.empty((nws + B * L * H,), dtype=torch.float32, device=dev)  # the workspace first: it wants 16-byte alignment

@@ -332,6 +332,36 @@ def _inside_all(batch, match):
     return ll.detach().cpu(), md.grad.cpu(), ld.grad.cpu()
 
 
+def test_sentence_given_up_is_counted_and_invalid():
+    """Where both pipelined sweeps of a sentence give up (spin limit 0) and the second chance of the outside sweep also
+    runs out of its bound for the forward's (forced: a bound of zero polls, so the wait expires without waiting), the
+    sentence is given up: NaN log-likelihood, zero gradients, and the third diagnostic counter says how many - a valid
+    sentence never turns invalid unnoticed.  The default path leaves that counter at zero (test_long_graph_sweeps_agree)."""
+    L, T, ms, ns = 320, 40, [320, 262, 200], [40, 31, 25]
+    batch = synth.training_batch(len(ms), L, T, 60, ms, ns, seed=L + T)
+    match = _match_for(batch)
+    ll0, mg0, lg0 = _inside_all(batch, match)
+    assert torch.isfinite(ll0).all()
+    ops.pipeline_redo_counts(reset=True)
+    try:
+        ops.pipeline_config(spin_limit=0)
+        ops.pipeline_redo_wait_limit(0)
+        ll1, mg1, lg1 = _inside_all(batch, match)
+    finally:
+        ops.pipeline_config(max_workgroups=1 << 20, spin_limit=ops.DEFAULT_SPIN_LIMIT, outside_spin_limit=-1)
+        ops.pipeline_redo_wait_limit()
+    redone, _, given_up = ops.pipeline_redo_counts(reset=True)
+    bad = torch.isnan(ll1)
+    assert given_up == int(bad.sum()), (given_up, ll1)
+    assert given_up >= 1, "no sentence had both of its sweeps give up: the case was not exercised"
+    for b in range(len(ms)):
+        if bad[b]:
+            assert not mg1[b].any() and not lg1[b].any()
+        else:
+            assert torch.allclose(ll1[b], ll0[b], rtol=1e-5)
+            assert (mg1[b] - mg0[b]).abs().max() <= 2e-5 * mg0[b].abs().max()
+
+
 @pytest.mark.parametrize("mode", ["one_workgroup", "blocks_give_up", "pipelines_in_turn", "forward_gives_up", "outside_gives_up"])
 @pytest.mark.parametrize("L,T,ms,ns", [(200, 50, [200, 132, 164], [50, 30, 44]), (320, 40, [320, 262, 4], [40, 31, 2]),
                                        (512, 140, [512, 444], [140, 120]),
@@ -350,7 +380,8 @@ def test_long_graph_sweeps_agree(mode, L, T, ms, ns):
     match = _match_for(batch)
     ops.pipeline_redo_counts(reset=True)
     ll0, mg0, lg0 = _inside_all(batch, match)
-    assert ops.pipeline_redo_counts()[0] == 0, "the pipelined sweeps of the default path gave up"
+    counts = ops.pipeline_redo_counts()
+    assert counts[0] == 0 and counts[2] == 0, "the pipelined sweeps of the default path gave up: %s" % (counts,)
     try:
         if mode == "one_workgroup":
             ops.pipeline_config(max_workgroups=0)
@@ -367,7 +398,8 @@ def test_long_graph_sweeps_agree(mode, L, T, ms, ns):
         ops.pipeline_config(max_workgroups=1 << 20, spin_limit=ops.DEFAULT_SPIN_LIMIT, outside_spin_limit=-1)
     # the fallback is visible in the diagnostic counter: every sweep of every sentence that ran as a pipeline and gave up
     # (a block gives up only if it has to wait at all, so how many sentences are redone varies from run to run)
-    redone = ops.pipeline_redo_counts(reset=True)[0]
+    redone, _, given_up = ops.pipeline_redo_counts(reset=True)
+    assert given_up == 0, "a second chance ran out of its bound"
     if mode in ("one_workgroup", "pipelines_in_turn"):
         assert redone == 0, (mode, redone)
     else:

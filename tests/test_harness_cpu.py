@@ -179,3 +179,26 @@ def test_support_masks_closed_form():
     left3, right3, main3 = synth.support_masks(14, 3)
     assert main3.nonzero().flatten().tolist() == [1, 5, 9, 13]
     assert left3[5, 2:5].eq(0).all() and left3[3, 2] == 0 and right3[3, 4] == 0 and left3[3, 4] == 1
+
+
+def test_flag_mask_cache_handles_views_and_inference_tensors():
+    """Integer support masks are converted to byte flags once and found again under fresh views of the same tensor; a
+    mask changed in place is converted again; tensors created under inference mode (no version counter) are converted on
+    every call instead of raising."""
+    from pcfg_nat_amd import custom_ops
+    custom_ops._MASK_CACHE.clear()
+    mask = torch.zeros(8, 8, dtype=torch.int64)
+    mask[2, 3] = 1
+    a = custom_ops._as_flag_mask(mask[:6, :6])
+    b = custom_ops._as_flag_mask(mask[:6, :6])  # a fresh view object of the same storage
+    assert a is b and a.dtype == torch.bool and bool(a[2, 3]) and int(a.sum()) == 1
+    assert len(custom_ops._MASK_CACHE) == 1
+    mask[4, 4] = 1  # in place: the version counter moves on
+    c = custom_ops._as_flag_mask(mask[:6, :6])
+    assert c is not a and int(c.sum()) == 2
+    with torch.inference_mode():
+        inf = torch.ones(4, 4, dtype=torch.int64)
+    d = custom_ops._as_flag_mask(inf)
+    assert d.dtype == torch.bool and bool(d.all())
+    flags = torch.ones(4, 4, dtype=torch.bool)
+    assert custom_ops._as_flag_mask(flags) is flags or torch.equal(custom_ops._as_flag_mask(flags), flags)

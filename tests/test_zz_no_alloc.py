@@ -80,6 +80,24 @@ def test_static_table_matches_caller_buffer_twice_in_a_row():
     _compare(_run(lib, True, *big), _run(lib, False, *big), exact=False)
 
 
+def test_static_table_with_general_max_left():
+    """The entry point also dispatches to the kernels for max_left != 1 (tables in the same static array): max_left = 2,
+    two calls in a row, the second smaller; same kernels as the caller-buffer call, one workgroup per sentence: bit-equal."""
+    lib = _lib.load()
+    for B, L, T, ms, ns, seed in ((3, 32, 12, [32, 20, 8], [12, 9, 4], 21), (2, 20, 8, [20, 11], [8, 5], 22)):
+        batch = synth.training_batch(B, L, T, 64, ms, ns, seed=seed, ml=2)
+        idx = batch["targets"].unsqueeze(1).expand(-1, L, -1)
+        match = harness.eos_masked(torch.log_softmax(batch["logits"], -1).gather(-1, idx), batch["output_length"],
+                                   batch["target_length"])
+        go = torch.linspace(0.5, 1.5, B)
+        args = [t.to(DEV).contiguous() for t in (go, match, batch["links"], batch["output_length"], batch["target_length"])]
+        assert args[2].size(2) == 3
+        print("static inside forward+backward, max_left = 2: B=%d L=%d T=%d" % (B, L, T), flush=True)
+        static, plain = _run(lib, True, *args), _run(lib, False, *args)
+        assert torch.isfinite(plain[0]).all()
+        _compare(static, plain, exact=True)
+
+
 def test_static_table_rejects_what_does_not_fit():
     lib = _lib.load()
     B, L, T = 256, 512, 24
