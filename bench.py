@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 EVENT_EVERY = 5  # steps between two bracketed launches of the roofline kernel inside the timed region
 ROOFLINE_KERNEL = {"single": "lsg_bwd", "fused": "lsg_bwd", "unfused": "lsg_fwd"}
 ROOFLINE_KERNEL_NAME = {"lsg_bwd": "lsg_bwd_kernel<half, from logits>", "lsg_fwd": "lsg_fwd_kernel<half, grad>"}
-MEASURED_TRAFFIC_BYTES = {"lsg_bwd": 546.55e6, "lsg_fwd": 273.76e6}
+MEASURED_TRAFFIC_BYTES = {"lsg_bwd": 546.65e6, "lsg_fwd": 273.84e6}
 
 
 def parse():
