@@ -40,7 +40,7 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the legs beyond the training step (same as --legs autograd,operator)")
     ap.add_argument("--legs", default="all",
-                    help="comma-separated legs to run beside the headline step: autograd, operator, decode, glat, long, links, "
+                    help="comma-separated legs to run beside the headline step: autograd, operator, decode, glat, long, links, maxleft3, "
                          "frontend (default: all; 'none' for the headline alone) - for profiling runs that want few kernels")
     ap.add_argument("--decode-sentences", type=int, default=1000,
                     help="sentences of the inference configuration the decode leg uses (default: all 1000)")
@@ -468,6 +468,41 @@ def link_scorer_timing(dev):
     return res
 
 
+def max_left3_timing(dev):
+    """The inside loss forward + backward for ``--left-tree-layer 2`` (max_left = 3: a left subtree of up to three nodes
+    under every main-chain node) at the training shape: B=40, L=130 (32 groups of four nodes), T=32, through
+    ``cuda_pcfg_loss`` (forward with the eager backward inside, pcfg_loss.py:67-73)."""
+    import torch
+    from pcfg_nat_amd import custom_ops as ops, synth
+
+    B, L, T, ml = 40, 130, 32, 3
+    gen = torch.Generator().manual_seed(1003)
+    src, n = synth._wmt_lengths(B, gen, 10, 32, T)  # src here = 4 * source length
+    m = src + 2                                      # full groups: (m - 2) % (ml + 1) == 0
+    links = synth.make_links(B, L, m, ml, gen).to(dev)
+    match_all = torch.log_softmax(torch.randn(B, L, T, generator=gen) * 2, dim=-1).to(dev)
+    ol, tl = m.to(dev), n.to(dev)
+
+    def step():
+        ma = match_all.detach().requires_grad_(True)
+        lk = links.detach().requires_grad_(True)
+        return ops.cuda_pcfg_loss(ma, lk, ol, tl)
+
+    for _ in range(3):
+        step()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    reps = 10
+    start.record()
+    for _ in range(reps):
+        ll = step()
+    end.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(end) / reps
+    return {"ms_per_call": ms, "sentences_per_s": B / (ms * 1e-3), "valid_sentences": int(torch.isfinite(ll).sum()),
+            "path": ops.max_left_path(ml), "workload": "B=40, L=130, T=32, max_left=3, inside forward + backward"}
+
+
 def decode_front_end_timing(dev):
     """max_v log_softmax and arg max over the vocabulary in one read of the logits (the model's decode front-end) at
     B=64, L=400, V=40000 fp16 (2.05 GB)."""
@@ -686,7 +721,7 @@ def main():
         result["single_call_scaled"] = sc
     # the drop-in path: the unchanged criterion code over the operator API under autograd (dag_logsoftmax_gather_inplace ->
     # eos mask -> cuda_pcfg_loss -> loss -> backward), which reads and rewrites every row (it is not told the lengths)
-    legs = {"autograd", "operator", "decode", "glat", "long", "links", "frontend"}
+    legs = {"autograd", "operator", "decode", "glat", "long", "links", "frontend", "maxleft3"}
     if args.legs != "all":
         legs = {x for x in args.legs.split(",") if x and x != "none"}
     if args.no_decode:
@@ -709,6 +744,8 @@ def main():
         result["link_scorer"] = link_scorer_timing(dev)
     if "frontend" in legs:
         result["decode_front_end"] = decode_front_end_timing(dev)
+    if "maxleft3" in legs:
+        result["max_left_3"] = max_left3_timing(dev)
     if not args.no_cpu_baseline:
         batch_cpu = {"output_length": m, "target_length": n, "links": links_cpu, "targets": targets_cpu}
         result["cpu_baseline"] = cpu_baseline(batch_cpu, sample_logits, args.cpu_sentences)

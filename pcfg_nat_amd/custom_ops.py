@@ -242,6 +242,12 @@ class CUDAPCFGLossFunc(Function):
         return None, None, None, None
 
 
+def max_left_path(max_left):
+    """Which kernel family serves the PCFG operators for this ``max_left`` (= ``links.size(2) - 1``): "tuned" for the
+    value of the shipped scripts, "generic" for the plain one-workgroup-per-sentence restatement."""
+    return "tuned" if int(max_left) == 1 else "generic"
+
+
 def cuda_pcfg_loss(match_all, links, output_length, target_length):
     """``CUDAPCFGLossFunc.apply`` (pcfg_loss.py:85); float32 tables go through the C++ autograd node of the torch extension."""
     ext = _ext()
