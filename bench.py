@@ -488,19 +488,30 @@ def max_left3_timing(dev):
         lk = links.detach().requires_grad_(True)
         return ops.cuda_pcfg_loss(ma, lk, ol, tl)
 
-    for _ in range(3):
-        step()
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    reps = 10
-    start.record()
-    for _ in range(reps):
-        ll = step()
-    end.record()
-    torch.cuda.synchronize()
-    ms = start.elapsed_time(end) / reps
-    return {"ms_per_call": ms, "sentences_per_s": B / (ms * 1e-3), "valid_sentences": int(torch.isfinite(ll).sum()),
-            "path": ops.max_left_path(ml), "workload": "B=40, L=130, T=32, max_left=3, inside forward + backward"}
+    def timed(reps):
+        for _ in range(3):
+            step()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(reps):
+            ll = step()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / reps, ll
+
+    ms, ll = timed(20)
+    res = {"ms_per_call": ms, "sentences_per_s": B / (ms * 1e-3), "valid_sentences": int(torch.isfinite(ll).sum()),
+           "path": ops.max_left_path(ml, L, T), "workload": "B=40, L=130, T=32, max_left=3, inside forward + backward"}
+    was = ops.max_left3_tuned(0)  # the same call through the plain one-workgroup-per-sentence kernels
+    try:
+        ms_plain, ll_plain = timed(5)
+    finally:
+        ops.max_left3_tuned(was)
+    res["plain_kernels_ms_per_call"] = ms_plain
+    res["speedup_vs_plain_kernels"] = ms_plain / ms
+    res["log_likelihoods_agree"] = bool(torch.allclose(ll, ll_plain, rtol=1e-5))
+    return res
 
 
 def decode_front_end_timing(dev):

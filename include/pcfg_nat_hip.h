@@ -138,11 +138,20 @@ int pcfgnat_pcfg_loss_backward(const float *grad_output, const float *S, float *
  * their tables into the gradients; graphs of 130..1026 nodes are swept by two pipelines of workgroups per sentence,
  * forward and outside, side by side in one launch (see pcfgnat_pipeline_config); otherwise the sweeps follow each other as
  * in the two calls.  aux (pcfgnat_pcfg_aux_floats floats) carries the tables between the launches.
+ * For max_left = 3 (--left-tree-layer 2; general loops pcfg_loss.cu:148-214, 262-349) and shapes for which
+ * pcfgnat_max_left3_supported answers 1, the sentences whose links hold no rule of a composite local tree - every sentence
+ * the model's link scorer can produce: it allows main-chain nodes only as right children
+ * (glat_decomposed_with_link_two_hands_tri_pcfg.py:175) - are served by one launch with all tables in LDS; any other
+ * sentence of the batch, and every other max_left, by the plain kernels of the two calls.
  */
 int pcfgnat_pcfg_loss_forward_backward(const float *grad_output, const float *match_all, const float *links,
                                        const int64_t *output_length, const int64_t *target_length, float *S, float *aux,
                                        float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T, int64_t ml,
                                        void *stream);
+
+/* 1 when pcfgnat_pcfg_loss_forward_backward serves max_left = 3 at this graph size and target length with its one-launch
+ * kernel (graphs of up to 254 nodes, targets of up to 64 tokens), 0 when the plain kernels run. */
+int pcfgnat_max_left3_supported(int64_t L, int64_t T);
 
 /*
  * No counterpart in the reference: pcfgnat_pcfg_loss_forward_backward for callers that cannot allocate device memory

@@ -47,6 +47,14 @@ void pcfgnat_pipeline_redo_wait_limit(int polls);
  * -inf sends every tile down the second path. */
 void pcfgnat_links_grad_range_limit(float log2_limit);
 
+/* Switches the one-launch kernel for max_left = 3 on (1, the default) or off (0: the plain kernels serve every sentence),
+ * so that tests can hold the two against each other; a negative value changes nothing.  Returns the previous setting. */
+int pcfgnat_max_left3_tuned(int on);
+
+/* Diagnostic counters of that kernel on the current device since the library was loaded (or the last reset): sentences it
+ * served, and sentences it left to the plain kernels because their links hold a rule of a composite local tree. */
+int pcfgnat_max_left3_counts(unsigned long long *served, unsigned long long *left_to_plain, int reset);
+
 /* Diagnostic counters since the library was loaded (or the last reset) on the current device: inside sweeps (forward and
  * outside counted apart) and single-call Viterbi decodes that the one-workgroup kernels redid because a pipelined sweep
  * gave up, and sentences given up for good (see pcfgnat_pipeline_redo_wait_limit).  reset != 0 clears them.  A caller that

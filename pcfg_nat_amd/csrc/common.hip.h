@@ -134,9 +134,15 @@ int viterbi_redo_count(unsigned long long *count, int reset);
 // General max_left (generic_ml.hip)
 size_t generic_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml);
 int generic_forward(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int64_t B,
-                    int64_t L, int64_t T, int64_t ml, void *stream);
+                    int64_t L, int64_t T, int64_t ml, void *stream, int skip_ml3_taken = 0);
 int generic_backward(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
-                     const int64_t *tl, float *mg, float *lg, int64_t B, int64_t L, int64_t T, int64_t ml, Seed seed, void *stream);
+                     const int64_t *tl, float *mg, float *lg, int64_t B, int64_t L, int64_t T, int64_t ml, Seed seed, void *stream, int skip_ml3_taken = 0);
+// max_left = 3 with the rules the model can produce (inside_ml3.hip): forward and backward in one launch for the sentences
+// that qualify; the others are left to generic_forward / generic_backward with skip_ml3_taken = 1, which skip the rest.
+bool inside_ml3_supported(int64_t L, int64_t T);
+int inside_ml3_forward_backward(const float *grad_output, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl,
+                                float *S, float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T, Seed seed,
+                                void *stream);
 int generic_best_tree(const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl,
                       int64_t *tree, int64_t B, int64_t L, int64_t T, int64_t ml, void *stream);
 int generic_viterbi(const float *ob, const float *links, const int64_t *ol, float *S, int64_t *R, int64_t *Lt, int64_t *M, int64_t B,
@@ -230,6 +236,24 @@ __device__ __forceinline__ double wave_sum(double v) {
 }
 
 constexpr float NEG_INF_F = -__builtin_huge_valf();
+
+// max_left = 3: does this sentence hold a rule through which the loops of pcfg_loss.cu:301-348 could build a composite
+// local tree?  Those are links[x, k, c] for the local nodes x = a-3, a-2 in front of every main-chain node a = 5, 9, ...,
+// m-1, right children x < c < a, every left option k - twelve per group; the model's link scorer leaves them all -inf
+// (a local node has no allowed right child).  Workgroup-uniform result; m must be a valid graph size ((m - 2) % 4 == 0).
+template <int NT>
+__device__ __forceinline__ bool ml3_composite_rules(const float *__restrict__ links, int L, int m, int tid) {
+    const int groups = (m - 2) / 4;
+    int found = 0;
+    for (int i = tid; i < groups * 12; i += NT) {
+        const int gi = i / 12, e = i - gi * 12, a = 4 * gi + 5;
+        const int x = e < 8 ? a - 3 : a - 2;
+        const int c = e < 8 ? a - 2 + (e >> 2) : a - 1;
+        const float v = links[((size_t)x * 4 + (e & 3)) * L + c];
+        found |= (v > NEG_INF_F) ? 1 : 0;  // (NaN counts as -inf, as in pcfg_loss.cu:162)
+    }
+    return __syncthreads_or(found) != 0;
+}
 
 // The criterion's reduction (nat_pcfg_loss.py:123-135) by one workgroup of NT threads, in a fixed order:
 // out[0] = -(1/B) * sum_b [ll_b finite] ll_b / n_b, out[1] = number of sentences with a non-finite ll_b, where

@@ -64,16 +64,27 @@ __device__ __forceinline__ bool len_ok(const Dims &d, int m, int n) {
     return m >= d.ml + 3 && m <= d.L && ((m - 2) % (d.ml + 1)) == 0 && n >= 2 && n <= d.T;
 }
 
+// Sentences that the one-launch kernel for max_left = 3 (inside_ml3.hip) has served: everything except valid sentences
+// that hold a rule of a composite local tree.  Only asked when that kernel ran in front (skip_ml3_taken).
+__device__ __forceinline__ bool taken_by_ml3(int skip_ml3_taken, const float *links, const Dims &d, int m, int n, int tid) {
+    if (!skip_ml3_taken) return false;  // (uniform)
+    if (!len_ok(d, m, n)) return true;
+    return !ml3_composite_rules<NTG>(links, d.L, m, tid);
+}
+__device__ __forceinline__ bool taken_by_ml3(int, const double *, const Dims &, int, int, int) { return false; }
+
 // ---- inside forward (pcfg_loss.cu:262-349 then :84-224) -----------------------------------------------------
 template <typename RT>
 __global__ __launch_bounds__(NTG) void generic_fwd_kernel(const RT *__restrict__ match_all, const RT *__restrict__ links_all,
                                                          const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
-                                                         RT *__restrict__ S_all, RT *__restrict__ aux_all, int L, int T, int ml) {
+                                                         RT *__restrict__ S_all, RT *__restrict__ aux_all, int L, int T, int ml,
+                                                         int skip_ml3_taken) {
     const Dims d(L, T, ml);
     const int b = blockIdx.x, tid = threadIdx.x;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const RT *match = match_all + (size_t)b * L * T;
     const RT *links = links_all + (size_t)b * L * (ml + 1) * L;
+    if (taken_by_ml3(skip_ml3_taken, links, d, m, n, tid)) return;
     RT *S = S_all + (size_t)b * d.s_size();
     RT *C = aux_all + (size_t)b * d.aux_floats();
     for (size_t i = tid; i < d.s_size(); i += NTG) S[i] = neg_inf<RT>();
@@ -158,12 +169,13 @@ __global__ __launch_bounds__(NTG) void generic_bwd_kernel(const RT *__restrict__
                                                          RT *__restrict__ aux_all, const RT *__restrict__ match_all,
                                                          const RT *__restrict__ links_all, const int64_t *__restrict__ out_len,
                                                          const int64_t *__restrict__ tgt_len, RT *__restrict__ mg_all,
-                                                         RT *__restrict__ lg_all, int L, int T, int ml, Seed seed) {
+                                                         RT *__restrict__ lg_all, int L, int T, int ml, Seed seed, int skip_ml3_taken) {
     const Dims d(L, T, ml);
     const int b = blockIdx.x, tid = threadIdx.x;
     const int m = (int)out_len[b], n = (int)tgt_len[b];
     const RT *match = match_all + (size_t)b * L * T;
     const RT *links = links_all + (size_t)b * L * (ml + 1) * L;
+    if (taken_by_ml3(skip_ml3_taken, links, d, m, n, tid)) return;
     const RT *S = S_all + (size_t)b * d.s_size();
     RT *aux = aux_all + (size_t)b * d.aux_floats();
     const RT *C = aux;
@@ -430,17 +442,17 @@ size_t generic_aux_floats(int64_t B, int64_t L, int64_t T, int64_t ml) { return 
 namespace {
 template <typename RT>
 int forward_t(const RT *match_all, const RT *links, const int64_t *ol, const int64_t *tl, RT *S, RT *aux, int64_t B, int64_t L, int64_t T,
-              int64_t ml, void *stream) {
+              int64_t ml, void *stream, int skip_ml3_taken = 0) {
     hipLaunchKernelGGL(generic_fwd_kernel<RT>, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, match_all, links, ol, tl, S, aux, (int)L,
-                       (int)T, (int)ml);
+                       (int)T, (int)ml, skip_ml3_taken);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
 template <typename RT>
 int backward_t(const RT *go, const RT *S, RT *aux, const RT *match_all, const RT *links, const int64_t *ol, const int64_t *tl, RT *mg, RT *lg,
-               int64_t B, int64_t L, int64_t T, int64_t ml, Seed seed, void *stream) {
+               int64_t B, int64_t L, int64_t T, int64_t ml, Seed seed, void *stream, int skip_ml3_taken = 0) {
     hipLaunchKernelGGL(generic_bwd_kernel<RT>, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, go, S, aux, match_all, links, ol, tl, mg,
-                       lg, (int)L, (int)T, (int)ml, seed);
+                       lg, (int)L, (int)T, (int)ml, seed, skip_ml3_taken);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -472,13 +484,14 @@ int check_f64(const char *who, int64_t B, int64_t L, int64_t T, int64_t ml) {
 }  // namespace
 
 int generic_forward(const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux, int64_t B,
-                    int64_t L, int64_t T, int64_t ml, void *stream) {
-    return forward_t<float>(match_all, links, ol, tl, S, aux, B, L, T, ml, stream);
+                    int64_t L, int64_t T, int64_t ml, void *stream, int skip_ml3_taken) {
+    return forward_t<float>(match_all, links, ol, tl, S, aux, B, L, T, ml, stream, skip_ml3_taken);
 }
 
 int generic_backward(const float *go, const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol,
-                     const int64_t *tl, float *mg, float *lg, int64_t B, int64_t L, int64_t T, int64_t ml, Seed seed, void *stream) {
-    return backward_t<float>(go, S, aux, match_all, links, ol, tl, mg, lg, B, L, T, ml, seed, stream);
+                     const int64_t *tl, float *mg, float *lg, int64_t B, int64_t L, int64_t T, int64_t ml, Seed seed, void *stream,
+                     int skip_ml3_taken) {
+    return backward_t<float>(go, S, aux, match_all, links, ol, tl, mg, lg, B, L, T, ml, seed, stream, skip_ml3_taken);
 }
 
 int generic_best_tree(const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl,

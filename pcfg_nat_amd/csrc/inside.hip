@@ -452,6 +452,16 @@ int pcfgnat::inside_forward_backward_impl(const float *grad_output, const float 
     const int Mc = (int)((L - 2) / 2 + 1);
     hipStream_t s = (hipStream_t)stream;
     bool done = false;
+    if (ml == 3 && inside_ml3_supported(L, T) && ((uintptr_t)links_grad % 16) == 0) {
+        // max_left = 3: the sentences whose rules the model can produce in one launch, the others by the plain kernels
+        rc = inside_ml3_forward_backward(grad_output, match_all, links, output_length, target_length, S, match_all_grad, links_grad, B, L,
+                                         T, seed, stream);
+        if (rc != PCFGNAT_OK) return rc;
+        rc = generic_forward(match_all, links, output_length, target_length, S, aux, B, L, T, ml, stream, 1);
+        if (rc != PCFGNAT_OK) return rc;
+        return generic_backward(grad_output, S, aux, match_all, links, output_length, target_length, match_all_grad, links_grad, B, L, T, ml,
+                                seed, stream, 1);
+    }
     if (ml != 1) {
         // general max_left: the two plain kernels
     } else if (Mc <= 64)

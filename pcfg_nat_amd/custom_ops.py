@@ -242,10 +242,31 @@ class CUDAPCFGLossFunc(Function):
         return None, None, None, None
 
 
-def max_left_path(max_left):
-    """Which kernel family serves the PCFG operators for this ``max_left`` (= ``links.size(2) - 1``): "tuned" for the
-    value of the shipped scripts, "generic" for the plain one-workgroup-per-sentence restatement."""
-    return "tuned" if int(max_left) == 1 else "generic"
+def max_left_path(max_left, L=None, T=None):
+    """Which kernel family serves ``cuda_pcfg_loss`` for this ``max_left`` (= ``links.size(2) - 1``): "tuned" for the value
+    of the shipped scripts and, at graph sizes and target lengths the library says it covers, for ``max_left = 3``;
+    "generic" for the plain one-workgroup-per-sentence restatement."""
+    ml = int(max_left)
+    if ml == 1:
+        return "tuned"
+    if ml == 3 and L is not None and T is not None and get_pcfg_kernel().pcfgnat_max_left3_supported(int(L), int(T)):
+        return "tuned"
+    return "generic"
+
+
+def max_left3_counts(reset=False):
+    """Diagnostic: (sentences served by the one-launch kernel for ``max_left = 3``, sentences it left to the plain kernels)
+    on the current device since the last reset."""
+    import ctypes
+    a, b = ctypes.c_ulonglong(0), ctypes.c_ulonglong(0)
+    lib = get_pcfg_kernel()
+    _lib.check(lib.pcfgnat_max_left3_counts(ctypes.byref(a), ctypes.byref(b), 1 if reset else 0), lib)
+    return int(a.value), int(b.value)
+
+
+def max_left3_tuned(on=-1):
+    """Test hook: switches the one-launch kernel for ``max_left = 3`` off (0) or on (1); returns the previous setting."""
+    return int(get_pcfg_kernel().pcfgnat_max_left3_tuned(int(on)))
 
 
 def cuda_pcfg_loss(match_all, links, output_length, target_length):

@@ -1290,6 +1290,99 @@ def test_general_max_left_vs_oracle(ml, L, ms, ns, generic_local):
     assert torch.allclose(ll2, ll.detach(), rtol=1e-6, equal_nan=True)
 
 
+def _max_left3_against_oracle(match, links, ol, tl, valid):
+    """cuda_pcfg_loss at max_left = 3 against the float64 oracle: log-likelihoods, both gradients entry by entry."""
+    B = match.size(0)
+    S64, C64 = oracle.inside_fwd(match.numpy(), links.numpy(), ol.numpy(), tl.numpy(), dtype=np.float64)
+    mg64, lg64 = oracle.inside_bwd(np.ones(B), S64, C64, match.numpy(), links.numpy(), ol.numpy(), tl.numpy())
+    md = match.to(DEV).requires_grad_(True)
+    ld = links.to(DEV).requires_grad_(True)
+    ll = ops.cuda_pcfg_loss(md, ld, ol.to(DEV), tl.to(DEV))
+    got = ll.detach().cpu().double().numpy()
+    want = S64[:, 0, 0]
+    fin = np.isfinite(want) & np.asarray(valid)
+    assert fin.any() and np.array_equal(np.isfinite(got), fin)
+    assert np.allclose(got[fin], want[fin], rtol=1e-5)
+    ll.masked_fill(~torch.isfinite(ll), 0).sum().backward()
+    worst = 0.0
+    for bi in range(B):
+        for name, g_got, g_want in (("match_all_grad", md.grad[bi], mg64[bi]), ("links_grad", ld.grad[bi], lg64[bi])):
+            g_got = g_got.cpu().double().numpy()
+            assert np.isfinite(g_got).all()
+            if not fin[bi]:
+                assert not g_got.any()
+                continue
+            worst = max([worst] + gradcheck.assert_elementwise(g_got, g_want, "%s of sentence %d" % (name, bi)))
+    return ll.detach(), md.grad, ld.grad, worst
+
+
+@pytest.mark.parametrize("L,ms,ns", [
+    (66, [66, 50, 34, 6], [14, 20, 9, 2]),
+    (130, [130, 98, 42, 130], [32, 20, 12, 2]),
+    (254, [254, 130], [64, 33]),
+])
+def test_max_left3_one_launch_kernel_vs_oracle(L, ms, ns):
+    """Links as the model's scorer produces them for --left-tree-layer 2 (no local node has a rule: right children are
+    main-chain nodes only), every left option of the main-chain nodes finite: the one-launch kernel serves every sentence
+    and agrees with the float64 oracle and with the plain kernels."""
+    match, links, ol, tl = _generic_batch(3, L, ms, ns, seed=300 + L, generic_local=False)
+    assert ops.max_left_path(3, L, max(ns)) == "tuned"
+    ops.max_left3_counts(reset=True)
+    ll, mg, lg, worst = _max_left3_against_oracle(match, links, ol, tl, [True] * len(ms))
+    assert ops.max_left3_counts() == (len(ms), 0)
+    print("max_left = 3, L=%d: worst relative error of a gradient entry %.2e" % (L, worst))
+    was = ops.max_left3_tuned(0)
+    try:
+        assert ops.max_left_path(3, L, max(ns)) == "generic"
+        ll_p, mg_p, lg_p, _ = _max_left3_against_oracle(match, links, ol, tl, [True] * len(ms))
+        assert ops.max_left3_counts() == (len(ms), 0)  # (the plain kernels ran alone: the counters did not move)
+    finally:
+        ops.max_left3_tuned(was)
+    assert torch.allclose(ll, ll_p, rtol=2e-6)
+    assert torch.allclose(mg, mg_p, rtol=2e-4, atol=1e-7) and torch.allclose(lg, lg_p, rtol=2e-4, atol=1e-7)
+
+
+def test_max_left3_mixed_batch_and_invalid_lengths():
+    """Sentences with and without rules of composite local trees in one batch, and graph sizes outside the contract: the
+    one-launch kernel takes what it covers, the plain kernels the rest, neither touches the other's sentences."""
+    from test_oracle_inside import random_links
+    L, T = 46, 12
+    ms, ns = [46, 30, 46, 22, 38, 46], [12, 9, 7, 6, 10, 5]
+    composite = [False, True, False, True, False, True]
+    rng = np.random.default_rng(77)
+    links = np.stack([random_links(rng, L, m, 3, p_drop=0.1, generic_local=c) for m, c in zip(ms, composite)]).astype(np.float32)
+    match = (rng.normal(size=(len(ms), L, T)) - 2.0).astype(np.float32)
+    ol, tl = torch.tensor(ms), torch.tensor(ns)
+    match = harness.eos_masked(torch.from_numpy(match), ol, tl)
+    ops.max_left3_counts(reset=True)
+    _max_left3_against_oracle(match, torch.from_numpy(links), ol, tl, [True] * len(ms))
+    assert ops.max_left3_counts() == (3, 3)
+    # graph sizes that are no whole number of groups, or too small: NaN log-likelihood, zero gradients, no fault
+    bad_ol = torch.tensor([45, 30, 4, 22, 38, 47])
+    md = match.to(DEV).requires_grad_(True)
+    ld = torch.from_numpy(links).to(DEV).requires_grad_(True)
+    ll = ops.cuda_pcfg_loss(md, ld, bad_ol.to(DEV), tl.to(DEV))
+    ok = torch.tensor([False, True, False, True, True, False])
+    assert torch.equal(torch.isfinite(ll).cpu(), ok) and torch.isnan(ll[~ok.to(DEV)]).all()
+    ll.masked_fill(~torch.isfinite(ll), 0).sum().backward()
+    assert not md.grad[~ok.to(DEV)].any() and not ld.grad[~ok.to(DEV)].any()
+    assert torch.isfinite(md.grad).all() and torch.isfinite(ld.grad).all()
+
+
+def test_max_left3_model_shaped_batch_vs_oracle():
+    """The bench's shape (B=40, L=130, T=32) with jointly normalised links on the model's support."""
+    B, L, T, ml = 40, 130, 32, 3
+    gen = torch.Generator().manual_seed(1003)
+    src, n = synth._wmt_lengths(B, gen, 10, 32, T)
+    m = src + 2
+    links = synth.make_links(B, L, m, ml, gen)
+    match = harness.eos_masked(torch.log_softmax(torch.randn(B, L, T, generator=gen) * 2, dim=-1), m, n)
+    ops.max_left3_counts(reset=True)
+    _, _, _, worst = _max_left3_against_oracle(match, links, m, n, [True] * B)
+    assert ops.max_left3_counts() == (B, 0)
+    print("max_left = 3 at B=40, L=130, T=32: worst relative error of a gradient entry %.2e" % worst)
+
+
 @pytest.mark.parametrize("ml,L,ms", [(3, 66, [66, 50, 34]), (7, 74, [74, 42]), (0, 24, [24, 13]), (2, 50, [50, 32])])
 def test_general_max_left_viterbi_bit_exact(ml, L, ms):
     from test_oracle_inside import random_links
