@@ -290,6 +290,95 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> pcfg_criterion(const at::Tensor &
     return std::make_tuple(out[1], out[2], out[3]);
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// pcfg_extract_links with the products inside the kernels (glat_decomposed_with_link_two_hands_tri_pcfg.py:153-199 after
+// the projections): one native call forward, one backward.  The caller (custom_ops.pcfg_extract_links) has made sure
+// that the shape is one the library covers and passes the three tree masks as one byte per flag.
+// ---------------------------------------------------------------------------------------------------------------
+struct LinksFn : public torch::autograd::Function<LinksFn> {
+    static at::Tensor forward(AutogradContext *ctx, at::Tensor query_chunks, at::Tensor key_chunks_left, at::Tensor key_chunks_right,
+                              at::Tensor gate_logits, at::Tensor prev_output_tokens, int64_t pad_index, at::Tensor left_tree_mask,
+                              at::Tensor right_tree_mask, at::Tensor main_chain) {
+        const char *who = "pcfg_extract_links";
+        need_gpu(who, {&query_chunks, &key_chunks_left, &key_chunks_right, &gate_logits, &prev_output_tokens, &left_tree_mask,
+                       &right_tree_mask, &main_chain});
+        TORCH_CHECK(query_chunks.dim() == 4 && key_chunks_left.sizes() == query_chunks.sizes() &&
+                        key_chunks_right.sizes() == query_chunks.sizes(),
+                    who, ": query and key chunks must share the shape [bsz, prelen, heads, head_dim]");
+        TORCH_CHECK(query_chunks.scalar_type() == key_chunks_left.scalar_type() && query_chunks.scalar_type() == key_chunks_right.scalar_type(),
+                    who, ": query and key chunks must share one of float16, float32");
+        const int64_t B = query_chunks.size(0), L = query_chunks.size(1), H = query_chunks.size(2), F = query_chunks.size(3);
+        TORCH_CHECK(gate_logits.dim() == 3 && gate_logits.size(0) == B && gate_logits.size(1) == L && gate_logits.size(2) == H &&
+                        prev_output_tokens.dim() == 2 && prev_output_tokens.size(0) == B && prev_output_tokens.size(1) == L,
+                    who, ": gate_logits must be [bsz, prelen, heads] and prev_output_tokens [bsz, prelen]");
+        for (const at::Tensor *t : {&left_tree_mask, &right_tree_mask})
+            TORCH_CHECK(t->scalar_type() == at::kByte && t->dim() == 2 && t->size(0) == L && t->size(1) == L && t->is_contiguous(), who,
+                        ": tree masks must be contiguous uint8 [prelen, prelen]");
+        TORCH_CHECK(main_chain.scalar_type() == at::kByte && main_chain.dim() == 1 && main_chain.size(0) == L && main_chain.is_contiguous(),
+                    who, ": main_chain must be contiguous uint8 [prelen]");
+        const int code = dtype_code(query_chunks, who);
+        // (gradient mode is switched off inside a forward: whether a backward may follow is read off the inputs alone)
+        const bool need = query_chunks.requires_grad() || key_chunks_left.requires_grad() || key_chunks_right.requires_grad() ||
+                          gate_logits.requires_grad();
+        TORCH_CHECK(pcfgnat_extract_links_fused_supported(code, L, H, F) &&
+                        (!need || pcfgnat_extract_links_fused_backward_supported(code, L, H, F)),
+                    who, ": shape not covered by the kernels with the products inside");
+        const c10::DeviceGuard guard(query_chunks.device());
+        const at::Tensor q = query_chunks.contiguous(), kl = key_chunks_left.contiguous(), kr = key_chunks_right.contiguous();
+        const at::Tensor gate = gate_logits.to(at::kFloat).contiguous(), prev = prev_output_tokens.to(at::kLong).contiguous();
+        const auto f32 = q.options().dtype(at::kFloat);
+        at::Tensor links = at::empty({B, L, 2, L}, f32);
+        const int64_t nw = 1 + (L + 31) / 32;
+        at::Tensor side = at::empty({B * L * (H + (need ? nw : 0))}, f32);  // per-head normalisers, then the masks per parent as bits
+        float *lse = side.data_ptr<float>();
+        unsigned *tile_masks = need ? reinterpret_cast<unsigned *>(lse + B * L * H) : nullptr;
+        check_rc(pcfgnat_extract_links_fused_forward(q.data_ptr(), kl.data_ptr(), kr.data_ptr(), code, gate.data_ptr<float>(),
+                                                     prev.data_ptr<int64_t>(), pad_index, left_tree_mask.data_ptr<unsigned char>(),
+                                                     right_tree_mask.data_ptr<unsigned char>(), main_chain.data_ptr<unsigned char>(),
+                                                     links.data_ptr<float>(), lse, tile_masks, B, L, H, F, stream_of(q)));
+        if (need) {
+            ctx->save_for_backward({links, side, q, kl, kr, gate});
+            ctx->saved_data["gate_dtype"] = (int64_t)gate_logits.scalar_type();
+        }
+        return links;
+    }
+
+    static variable_list backward(AutogradContext *ctx, variable_list grads) {
+        const auto saved = ctx->get_saved_variables();
+        TORCH_CHECK(saved.size() == 6, "pcfg_extract_links: nothing was kept for a backward pass");
+        const at::Tensor &links = saved[0], &side = saved[1], &q = saved[2], &kl = saved[3], &kr = saved[4], &gate = saved[5];
+        const int64_t B = q.size(0), L = q.size(1), H = q.size(2), F = q.size(3);
+        const c10::DeviceGuard guard(q.device());
+        at::Tensor G = grads[0].to(at::kFloat).contiguous();
+        if (reinterpret_cast<uintptr_t>(G.data_ptr()) % 16) G = G.clone();  // (a view at an odd offset: read in 16-byte pieces)
+        at::Tensor d = at::empty({3, B, L, H, F}, q.options().requires_grad(false));
+        const int64_t nws = (int64_t)((pcfgnat_extract_links_fused_backward_workspace_bytes(B, L, H, F) + 3) / 4);
+        at::Tensor block = at::empty({nws + B * L * H}, q.options().dtype(at::kFloat).requires_grad(false));  // the workspace first: it wants 16-byte alignment
+        float *ws = block.data_ptr<float>();
+        const float *lse = side.data_ptr<float>();
+        check_rc(pcfgnat_extract_links_fused_backward(G.data_ptr<float>(), links.data_ptr<float>(), lse,
+                                                      reinterpret_cast<const unsigned *>(lse + B * L * H), q.data_ptr(), kl.data_ptr(),
+                                                      kr.data_ptr(), dtype_code(q, "pcfg_extract_links"), gate.data_ptr<float>(),
+                                                      d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), ws + nws, ws, B, L, H, F,
+                                                      stream_of(q)));
+        const at::Tensor dgate = block.narrow(0, nws, B * L * H).view({B, L, H});
+        const auto gate_dtype = (at::ScalarType)ctx->saved_data["gate_dtype"].toInt();
+        variable_list out(9);
+        out[0] = d[0];
+        out[1] = d[1];
+        out[2] = d[2];
+        out[3] = dgate.to(gate_dtype);
+        return out;
+    }
+};
+
+at::Tensor pcfg_extract_links_fused(const at::Tensor &query_chunks, const at::Tensor &key_chunks_left, const at::Tensor &key_chunks_right,
+                                    const at::Tensor &gate_logits, const at::Tensor &prev_output_tokens, int64_t pad_index,
+                                    const at::Tensor &left_tree_mask, const at::Tensor &right_tree_mask, const at::Tensor &main_chain) {
+    return LinksFn::apply(query_chunks, key_chunks_left, key_chunks_right, gate_logits, prev_output_tokens, pad_index, left_tree_mask,
+                          right_tree_mask, main_chain);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -300,4 +389,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("pcfg_criterion", &pcfg_criterion, "the criterion's loss as one differentiable op (nat_pcfg_loss.py:98-145)", py::arg("outputs"),
           py::arg("targets"), py::arg("links"), py::arg("output_length"), py::arg("target_length"), py::arg("matchmask") = py::none(),
           py::arg("keep_word_mask") = py::none());
+    m.def("pcfg_extract_links_fused", &pcfg_extract_links_fused,
+          "the link scorer after its projections, products inside the kernels (glat_decomposed_with_link_two_hands_tri_pcfg.py:153-199)");
 }

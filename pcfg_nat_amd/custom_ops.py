@@ -745,6 +745,21 @@ def pcfg_extract_links(query_chunks, key_chunks_left, key_chunks_right, gate_log
     """links [bsz, prelen, 2, prelen] float32 from the projected chunks [bsz, prelen, heads, head_dim] and the gate logits
     [bsz, prelen, heads]; differentiable in the first four arguments.  max_left = 1.  products_inside=False takes the form
     whose products go through torch's GEMM library also where the library's own kernels would cover the shape."""
+    ext = _ext()
+    if (ext is not None and products_inside and query_chunks.is_cuda and query_chunks.dim() == 4
+            and query_chunks.dtype in (torch.float16, torch.float32) and query_chunks.size(0) <= 32767):
+        # the C++ autograd node, where the kernels with the products inside cover the shape and the layout
+        lib = get_pcfg_kernel()
+        code = _DTYPE_CODE[query_chunks.dtype]
+        _, L, H, F = query_chunks.shape
+        need_grad = any(t.requires_grad for t in (query_chunks, key_chunks_left, key_chunks_right, gate_logits))
+        if (lib.pcfgnat_extract_links_fused_supported(code, L, H, F)
+                and (not need_grad or lib.pcfgnat_extract_links_fused_backward_supported(code, L, H, F))
+                and all(t.is_contiguous() and t.data_ptr() % 16 == 0 for t in (query_chunks, key_chunks_left, key_chunks_right))):
+            masks = [_as_flag_mask(t) for t in (left_tree_mask, right_tree_mask, main_chain)]
+            masks = [m.view(torch.uint8) if m.dtype == torch.bool else m for m in masks]  # (same bytes)
+            return ext.pcfg_extract_links_fused(query_chunks, key_chunks_left, key_chunks_right, gate_logits, prev_output_tokens,
+                                                int(pad_index), *masks)
     return PCFGExtractLinksFunc.apply(query_chunks, key_chunks_left, key_chunks_right, gate_logits, prev_output_tokens, pad_index,
                                       left_tree_mask, right_tree_mask, main_chain, products_inside)
 

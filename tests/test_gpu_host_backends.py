@@ -1,4 +1,4 @@
-"""The host side of the three training operators exists twice - as C++ autograd nodes in the torch extension (what runs by
+"""The host side of the training operators (and of the link scorer with its products inside the kernels) exists twice - as C++ autograd nodes in the torch extension (what runs by
 default) and as the Python Functions of ``custom_ops`` over ctypes.  Both enqueue the same kernels with the same arguments,
 so every result must be bit-identical; the contract checks (in-place buffer, single backward, loud errors) hold in both."""
 import pytest
@@ -143,3 +143,30 @@ def test_contract_of_the_in_place_operators(backend):
                              batch["target_length"].to(DEV))
     assert torch.equal(ll1, ll.detach())
     assert match.grad is not None and torch.isfinite(match.grad).all()
+
+
+def test_link_scorer_backends_give_identical_results():
+    """pcfg_extract_links through the C++ node and through the Python Function: same kernels, same arguments."""
+    B, L, H, F = 3, 64, 4, 32
+    g = torch.Generator().manual_seed(5)
+    chunks = [(torch.randn(B, L, H, F, generator=g) * 0.5).half().to(DEV) for _ in range(3)]
+    gate = torch.randn(B, L, H, generator=g).half().to(DEV)
+    m = torch.tensor([64, 40, 24])
+    prev = torch.full((B, L), 3).masked_fill(torch.arange(L).view(1, L) >= m.view(B, 1), synth.PAD).to(DEV)
+    lm, rm, mc = (x.to(DEV) for x in synth.support_masks(L, 1))
+    G = torch.randn(B, L, 2, L, generator=g).to(DEV)
+    results = {}
+    before = ops.host_backend()
+    try:
+        for name in ("extension", "python"):
+            ops.host_backend(name)
+            ts = [t.detach().requires_grad_(True) for t in chunks + [gate]]
+            links = ops.pcfg_extract_links(*ts, prev, synth.PAD, lm, rm, mc)
+            links.backward(G.masked_fill(~torch.isfinite(links.detach()), 0))
+            results[name] = [links.detach()] + [t.grad for t in ts]
+            with torch.no_grad():  # (no backward to prepare: the masks per parent are not written)
+                assert torch.equal(ops.pcfg_extract_links(*chunks, gate, prev, synth.PAD, lm, rm, mc), links.detach())
+    finally:
+        ops.host_backend(before)
+    for a, b in zip(results["extension"], results["python"]):
+        assert a.dtype == b.dtype and torch.equal(a, b)
