@@ -34,8 +34,8 @@ MEASURED_TRAFFIC_BYTES = {"lsg_bwd": 546.65e6, "lsg_fwd": 273.84e6}
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-sentences", type=int, default=40, help="sentences of the batch timed on the CPU oracle")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the legs beyond the training step (same as --legs autograd,operator)")
