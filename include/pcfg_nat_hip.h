@@ -388,12 +388,15 @@ int pcfgnat_viterbi_decoding(const int64_t *pred_length, const int64_t *output_l
  * back to back on full tables in `workspace`.  workspace: pcfgnat_viterbi_decode_workspace_bytes(B, L, max_left) bytes,
  * 8-byte aligned.
  *   out_tokens [B,L] int64, out_count [B] int64 (as pcfgnat_viterbi_decoding), pred_length [B] int64.
+ *   out_tokens_f32 [B,L] float32 or NULL: the same rows once more as float32, the type the model hands on (:501 ends in
+ *   `.float()`), written by the kernel that walks the tree so that the caller launches no conversion of its own.  A
+ *   sentence's out_count is the last thing stored for it.
  */
 size_t pcfgnat_viterbi_decode_workspace_bytes(int64_t B, int64_t L, int64_t ml);
 int pcfgnat_viterbi_decode(const float *ob_lprob, const float *links, const int64_t *output_length, const int64_t *tokens,
                            const int64_t *left_tree_mask, int64_t mask_dim, int64_t pad_index, const float *length_penalty,
-                           void *workspace, int64_t *out_tokens, int64_t *out_count, int64_t *pred_length, int64_t B,
-                           int64_t L, int64_t ml, void *stream);
+                           void *workspace, int64_t *out_tokens, float *out_tokens_f32, int64_t *out_count,
+                           int64_t *pred_length, int64_t B, int64_t L, int64_t ml, void *stream);
 
 /*
  * The decode as the model runs it (glat_decomposed_with_link_two_hands_tri_pcfg.py:414-416 followed by :483-502) enqueued
@@ -404,8 +407,8 @@ int pcfgnat_viterbi_decode(const float *ob_lprob, const float *links, const int6
 int pcfgnat_viterbi_decode_logits(const void *logits, int dtype, int64_t V, float *best_lprob, int64_t *best_idx,
                                   const float *links, const int64_t *output_length, const int64_t *left_tree_mask,
                                   int64_t mask_dim, int64_t pad_index, const float *length_penalty, void *workspace,
-                                  int64_t *out_tokens, int64_t *out_count, int64_t *pred_length, int64_t B, int64_t L,
-                                  int64_t ml, void *stream);
+                                  int64_t *out_tokens, float *out_tokens_f32, int64_t *out_count, int64_t *pred_length,
+                                  int64_t B, int64_t L, int64_t ml, void *stream);
 
 /*
  * The `lookahead` and `greedy` decode strategies of glat_decomposed_with_link_two_hands_tri_pcfg.py:419-481 in one launch:

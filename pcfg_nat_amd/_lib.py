@@ -75,8 +75,8 @@ SIGNATURES = {
     "pcfgnat_pcfg_viterbi": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "pcfgnat_viterbi_decoding": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "pcfgnat_viterbi_decode_workspace_bytes": (ctypes.c_size_t, [_i64, _i64, _i64]),
-    "pcfgnat_viterbi_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
-    "pcfgnat_viterbi_decode_logits": (_int, [_vp, _int, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "pcfgnat_viterbi_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "pcfgnat_viterbi_decode_logits": (_int, [_vp, _int, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "pcfgnat_lookahead_decode": (_int, [_vp, _vp, ctypes.c_float, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "pcfgnat_viterbi_decoding_host": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64]),
 }

@@ -48,7 +48,7 @@ int ensure_dynamic_lds(const void *kernel, size_t bytes) {
 }
 }  // namespace pcfgnat
 
-extern "C" int pcfgnat_abi_version(void) { return 4; }
+extern "C" int pcfgnat_abi_version(void) { return 5; }
 
 extern "C" const char *pcfgnat_last_error(void) { return pcfgnat::error_buffer(); }
 
@@ -158,12 +158,12 @@ extern "C" int pcfgnat_criterion_backward(void *logits_inout, int dtype, const i
 extern "C" int pcfgnat_viterbi_decode_logits(const void *logits, int dtype, int64_t V, float *best_lprob, int64_t *best_idx,
                                              const float *links, const int64_t *output_length, const int64_t *left_tree_mask,
                                              int64_t mask_dim, int64_t pad_index, const float *length_penalty, void *workspace,
-                                             int64_t *out_tokens, int64_t *out_count, int64_t *pred_length, int64_t B, int64_t L,
-                                             int64_t ml, void *stream) {
+                                             int64_t *out_tokens, float *out_tokens_f32, int64_t *out_count, int64_t *pred_length,
+                                             int64_t B, int64_t L, int64_t ml, void *stream) {
     if (dtype != PCFGNAT_F16 && dtype != PCFGNAT_F32)
         return pcfgnat::fail(PCFGNAT_EUNSUPPORTED, "viterbi_decode_logits: logits must be float16 or float32 (the Viterbi tables are float32)");
     int rc = pcfgnat_logsoftmax_max(logits, dtype, best_lprob, best_idx, B, L, V, stream);
     if (rc != PCFGNAT_OK) return rc;
     return pcfgnat_viterbi_decode(best_lprob, links, output_length, best_idx, left_tree_mask, mask_dim, pad_index, length_penalty,
-                                  workspace, out_tokens, out_count, pred_length, B, L, ml, stream);
+                                  workspace, out_tokens, out_tokens_f32, out_count, pred_length, B, L, ml, stream);
 }

@@ -157,6 +157,7 @@ struct DecodeArgs {
     const float *penalty;          // [Lq]
     int *W;                        // [B][L/2][Lq] workspace
     int64_t *out_tokens, *out_count, *pred_length;
+    float *out_tokens_f32;         // [B][L] or null: the emitted tokens once more as float32, the type the model hands on
     int64_t mask_dim, pad;
     // set when the pipelined sweep has run before this kernel: sentences whose flag is down only need the length
     // selection (root scores [B][Lq]) and the walk, the others are redone from scratch
@@ -327,16 +328,23 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
     }  // in_contract
     if (COMPACT) {
         __syncthreads();  // the workspace records and the padded output row are visible to the walking thread
+        int64_t count = 0;
         if (tid < 64) {
             const int pl = select_length(sm_scores, dec.penalty, Lq, tid);
             if (tid == 0) {
                 int *stack_node = dyn + Lq, *stack_len = stack_node + L;
                 const CompactTraces tr{Wb, Lq, rowsW};
                 dec.pred_length[b] = pl;
-                dec.out_count[b] = readout_one(pl, out_len[b], tr, dec.tokens + (size_t)b * L, dec.mask, dec.mask_dim, dec.pad,
-                                               dec.out_tokens + (size_t)b * L, stack_node, stack_len, L, Lq);
+                count = readout_one(pl, out_len[b], tr, dec.tokens + (size_t)b * L, dec.mask, dec.mask_dim, dec.pad,
+                                    dec.out_tokens + (size_t)b * L, stack_node, stack_len, L, Lq);
             }
         }
+        if (dec.out_tokens_f32 != nullptr) {  // workgroup-uniform
+            __syncthreads();                  // the walked row is visible to the whole workgroup
+            for (int i = tid; i < L; i += NT) dec.out_tokens_f32[(size_t)b * L + i] = (float)dec.out_tokens[(size_t)b * L + i];
+        }
+        // the count goes out last: a host that watches it in pinned memory finds the sentence's kernel as good as through
+        if (tid == 0) dec.out_count[b] = count;
     }
 }
 
@@ -596,6 +604,12 @@ __global__ __launch_bounds__(64) void select_length_kernel(const float *__restri
     if (threadIdx.x == 0) pred_length[b] = pl;
 }
 
+// The emitted tokens as float32 (the general path of the single-call decode; the one-workgroup decode converts its own row).
+__global__ __launch_bounds__(256) void tokens_to_float_kernel(const int64_t *__restrict__ tokens, float *__restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = (float)tokens[i];
+}
+
 // `lookahead` / `greedy` decode (glat_decomposed_with_link_two_hands_tri_pcfg.py:419-481), one workgroup per sentence:
 // every wave takes rows of the sentence's link tensor and finds the first arg max over the flattened (k, c) of
 //   (links[a][k][c] + ob[c] * beta) + ob[left(a,k)] * beta     (lookahead, :421-427; left(a,0) = 0, left(a,k) = max(a-k, 0))
@@ -784,8 +798,8 @@ extern "C" size_t pcfgnat_viterbi_decode_workspace_bytes(int64_t B, int64_t L, i
 
 extern "C" int pcfgnat_viterbi_decode(const float *ob_lprob, const float *links, const int64_t *output_length, const int64_t *tokens,
                                       const int64_t *left_tree_mask, int64_t mask_dim, int64_t pad_index, const float *length_penalty,
-                                      void *workspace, int64_t *out_tokens, int64_t *out_count, int64_t *pred_length, int64_t B,
-                                      int64_t L, int64_t ml, void *stream) {
+                                      void *workspace, int64_t *out_tokens, float *out_tokens_f32, int64_t *out_count,
+                                      int64_t *pred_length, int64_t B, int64_t L, int64_t ml, void *stream) {
     PCFGNAT_REQUIRE(B >= 0 && L >= 4, "viterbi_decode: need B >= 0 and L >= 4 (got B=%lld L=%lld)", (long long)B, (long long)L);
     PCFGNAT_REQUIRE(ml >= 0 && ml <= 63 && L / 4 > ml, "viterbi_decode: max_left out of range for this graph size");
     PCFGNAT_REQUIRE(mask_dim >= 1, "viterbi_decode: bad mask dimension");
@@ -797,8 +811,8 @@ extern "C" int pcfgnat_viterbi_decode(const float *ob_lprob, const float *links,
     hipStream_t s = (hipStream_t)stream;
     const int Lq = (int)(L / 4);
     if (decode_is_fused(L, ml)) {
-        DecodeArgs dec{tokens,     left_tree_mask, length_penalty, (int *)workspace, out_tokens, out_count,
-                       pred_length, mask_dim,       pad_index,      nullptr,          nullptr};
+        DecodeArgs dec{tokens,      left_tree_mask, length_penalty, (int *)workspace, out_tokens, out_count,
+                       pred_length, out_tokens_f32, mask_dim,       pad_index,        nullptr,    nullptr};
         switch (decode_chunks(L)) {
             case 2: return launch_decode<2>(ob_lprob, links, output_length, dec, workspace, B, L, s);
             case 4: return launch_decode<4>(ob_lprob, links, output_length, dec, workspace, B, L, s);
@@ -818,8 +832,14 @@ extern "C" int pcfgnat_viterbi_decode(const float *ob_lprob, const float *links,
     if (rc != PCFGNAT_OK) return rc;
     hipLaunchKernelGGL(select_length_kernel, dim3((unsigned)B), dim3(64), 0, s, Sw, length_penalty, pred_length, (int)L, Lq);
     PCFGNAT_HIP_CHECK(hipGetLastError());
-    return pcfgnat_viterbi_decoding(pred_length, output_length, Lw, Rw, Mw, tokens, left_tree_mask, mask_dim, pad_index, out_tokens,
-                                    out_count, stacks, B, L, Lq, stream);
+    rc = pcfgnat_viterbi_decoding(pred_length, output_length, Lw, Rw, Mw, tokens, left_tree_mask, mask_dim, pad_index, out_tokens,
+                                  out_count, stacks, B, L, Lq, stream);
+    if (rc != PCFGNAT_OK || out_tokens_f32 == nullptr) return rc;
+    const size_t cells_out = (size_t)B * L;
+    hipLaunchKernelGGL(tokens_to_float_kernel, dim3((unsigned)((cells_out + 255) / 256)), dim3(256), 0, s, out_tokens, out_tokens_f32,
+                       cells_out);
+    PCFGNAT_HIP_CHECK(hipGetLastError());
+    return PCFGNAT_OK;
 }
 
 extern "C" int pcfgnat_viterbi_decoding(const int64_t *pred_length, const int64_t *output_length, const int64_t *Lt, const int64_t *R,

@@ -8,6 +8,7 @@ contract; the arithmetic runs in hand-written HIP kernels for gfx950 reached thr
 ``libpcfg_nat_hip.so`` on the current HIP stream.  There is no CPU path: calling with CPU tensors (other than
 ``viterbi_decoding``, whose reference version is itself a host loop) raises.
 """
+import contextlib
 import ctypes
 import threading
 import time
@@ -575,8 +576,7 @@ def viterbi_decoding(pred_length, output_length, L_trace, R_trace, M_trace, unre
                                                         tok.data_ptr(), mask.data_ptr(), mask.size(0), int(pad_index),
                                                         out.data_ptr(), cnt.data_ptr(), scratch.data_ptr(), B, L, Lq,
                                                         _stream(out)), lib)
-                _pinned_counts.wait(cnt, B, torch.cuda.current_stream(dev), armed)
-                counts = cnt[:B].tolist()
+                counts = _pinned_counts.wait(cnt, B, torch.cuda.current_stream(dev), armed)
             finally:
                 _pinned_counts.give_back(cnt)
     else:
@@ -832,7 +832,7 @@ _PENALTY_CACHE = {}
 def _length_penalty(Lq, beta, device):
     """``arange(Lq) ** beta`` as the reference computes it (glat_decomposed_with_link_two_hands_tri_pcfg.py:489-492),
     cached per (Lq, beta, device)."""
-    key = (int(Lq), float(beta), str(device))
+    key = (int(Lq), float(beta), device.type, device.index)
     pen = _PENALTY_CACHE.get(key)
     if pen is None:
         pen = (torch.arange(Lq).unsqueeze(0) ** beta).to(device=device, dtype=torch.float32).contiguous().view(-1)
@@ -840,12 +840,28 @@ def _length_penalty(Lq, beta, device):
     return pen
 
 
+class _CountBuffer:
+    """One pinned int64 host buffer: the tensor that owns the memory, its address, and the same words as a ctypes array
+    (the host marks and reads a handful of entries per call; going through the array costs a fraction of a tensor op)."""
+    __slots__ = ("tensor", "ptr", "words", "capacity")
+
+    def __init__(self, n):
+        self.capacity = max(n, 64)
+        self.tensor = torch.empty((self.capacity,), dtype=torch.int64, pin_memory=True)
+        self.ptr = self.tensor.data_ptr()
+        self.words = (ctypes.c_int64 * self.capacity).from_address(self.ptr)
+
+    def data_ptr(self):
+        return self.ptr
+
+
 class _PinnedCounts:
     """Pinned int64 host buffers for the per-sentence token counts of the decode calls.  Pinned host memory is addressable
     from the device, so the kernels write the counts straight into it and the caller reads them as they arrive (``arm`` /
-    ``wait`` below), at the latest after waiting for its stream.  A call takes a buffer out of the pool for its own use and puts it back when it has read the counts: calls
-    that overlap (several host threads, several streams of one device) never share one.  Allocating pinned memory takes
-    about a hundred microseconds, hence the pool; it holds as many buffers as calls have ever overlapped."""
+    ``wait`` below), at the latest after waiting for its stream.  A call takes a buffer out of the pool for its own use and
+    puts it back when it has read the counts: calls that overlap (several host threads, several streams of one device)
+    never share one.  Allocating pinned memory takes about a hundred microseconds, hence the pool; it holds as many buffers
+    as calls have ever overlapped."""
 
     def __init__(self):
         self._lock = threading.Lock()
@@ -856,9 +872,9 @@ class _PinnedCounts:
     def take(self, n):
         with self._lock:
             for i, buf in enumerate(self._free):
-                if buf.numel() >= n:
+                if buf.capacity >= n:
                     return self._free.pop(i)
-        return torch.empty((max(n, 64),), dtype=torch.int64, pin_memory=True)
+        return _CountBuffer(n)
 
     def give_back(self, buf):
         with self._lock:
@@ -882,58 +898,88 @@ class _PinnedCounts:
         """Marks the entries and returns True if this call is going to watch them."""
         if not self._polling or not stream.query():
             return False
-        buf[:n].fill_(self.NOT_YET)
+        words = buf.words
+        for i in range(n):
+            words[i] = self.NOT_YET
         return True
 
     def wait(self, buf, n, stream, armed):
+        """Returns the n counts once the kernels have written them."""
+        words = buf.words
         if armed:
-            entries = (ctypes.c_int64 * n).from_address(buf.data_ptr())
+            not_yet = self.NOT_YET
             deadline = time.perf_counter() + self.WATCH_SECONDS
             i = spins = 0
             while i < n:
-                if entries[i] != self.NOT_YET:
+                if words[i] != not_yet:
                     i += 1
                     continue
                 spins += 1
                 if (spins & 255) == 0 and time.perf_counter() > deadline:
                     break
+            if i == n:
+                if self._misses:
+                    with self._lock:
+                        self._misses = 0
+                return words[:n]
             with self._lock:
-                if i == n:
-                    self._misses = 0
-                    return
                 self._misses += 1
                 if self._misses >= self.MISSES_TO_SWITCH_OFF:
                     self._polling = False
         stream.synchronize()
+        return words[:n]
 
 
 _pinned_counts = _PinnedCounts()
 
+# a float32 token row handed back as a view keeps its whole block alive; beyond this size the row is copied out instead
+_DECODE_VIEW_MAX_WORDS = 1 << 17
+_DECODE_WORKSPACE_WORDS = {}
+
+
+def _on_device(dev):
+    """Context that makes ``dev`` the current device; free when it already is."""
+    return contextlib.nullcontext() if torch.cuda.current_device() == dev.index else torch.cuda.device(dev)
+
 
 def _viterbi_decode_call(name, B, L, ml, dev, extra_words, call):
-    """Shared tail of the Viterbi decode calls: one allocation (workspace | tokens [B,L] | predicted lengths [B] |
-    ``extra_words`` more int64 words for the caller), the native call, the one stream wait, the emitted counts.  ``call``
-    receives (lib, base address of the block, workspace words, address of the pinned counts) and returns the status."""
-    lib = get_pcfg_kernel()
-    with torch.cuda.device(dev):
-        nwork = (lib.pcfgnat_viterbi_decode_workspace_bytes(B, L, ml) + 7) // 8
-        block = torch.empty((nwork + B * L + B + extra_words,), dtype=torch.int64, device=dev)
-        out = block[nwork:nwork + B * L].view(B, L)
-        pred = block[nwork + B * L:nwork + B * L + B]
+    """Shared tail of the Viterbi decode calls: one allocation (workspace | tokens [B,L] int64 | predicted lengths [B] |
+    tokens [B,L] float32 | ``extra_words`` more int64 words for the caller), the native call, the one wait, the emitted
+    counts.  ``call`` receives (lib, stream handle, base address of the block, workspace words, address of the float32
+    tokens, address of the pinned counts, address of the caller's words) and returns the status.  The kernels write the
+    float32 tokens themselves, so nothing is enqueued behind the native call, and everything the host can do without the
+    counts (the views of the results) it does while the kernels run."""
+    lib = _lib.load()
+    nodes = B * L
+    fwords = (nodes + 1) // 2
+    nwork = _DECODE_WORKSPACE_WORDS.get((B, L, ml))
+    if nwork is None:
+        nwork = _DECODE_WORKSPACE_WORDS[(B, L, ml)] = (lib.pcfgnat_viterbi_decode_workspace_bytes(B, L, ml) + 7) // 8
+    with _on_device(dev):
+        stream = torch.cuda.current_stream(dev)
+        block = torch.empty((nwork + nodes + B + fwords + extra_words,), dtype=torch.int64, device=dev)
+        base = block.data_ptr()
         # the emitted counts go straight into pinned host memory, which the device addresses like its own: the one
-        # synchronisation of the decode is a stream wait, with no copy in front of it
-        host = _pinned_counts.take(B)  # written by the kernel, read after the one stream wait
+        # synchronisation of the decode is a wait for them (or for the stream), with no copy in front of it
+        host = _pinned_counts.take(B)
         try:
-            armed = _pinned_counts.arm(host, B, torch.cuda.current_stream(dev))
-            _lib.check(call(lib, block.data_ptr(), nwork, host.data_ptr()), lib)
-            _pinned_counts.wait(host, B, torch.cuda.current_stream(dev), armed)
-            counts = host[:B].tolist()
+            armed = _pinned_counts.arm(host, B, stream)
+            rc = call(lib, stream.cuda_stream, base, nwork, base + 8 * (nwork + nodes + B), host.ptr,
+                      base + 8 * (nwork + nodes + B + fwords))
+            if rc != _lib.OK:
+                _lib.check(rc, lib)
+            pred = block[nwork + nodes:nwork + nodes + B]
+            tokf = block[nwork + nodes + B:nwork + nodes + B + fwords].view(torch.float32)[:nodes].view(B, L)
+            counts = _pinned_counts.wait(host, B, stream, armed)
         finally:
             _pinned_counts.give_back(host)
     if B and min(counts) < 0:
         raise RuntimeError("viterbi_decoding: malformed traces")
     maxlen = max(counts) if B else 0
-    return out[:, :maxlen].to(torch.float32), pred, block
+    tokens = tokf[:, :maxlen]  # one sentence: a contiguous view; a batch: its rows are copied together
+    if B != 1 or block.numel() > _DECODE_VIEW_MAX_WORDS:
+        tokens = tokens.clone(memory_format=torch.contiguous_format)
+    return tokens, pred, block
 
 
 def _check_decode_graph(name, B, L, links, left_tree_mask):
@@ -964,11 +1010,10 @@ def pcfg_viterbi_decode(unreduced_logits, links, output_length, unreduced_tokens
     tok = unreduced_tokens.to(dtype=torch.int64).contiguous()
     mask = left_tree_mask.to(dtype=torch.int64).contiguous()
     pen = _length_penalty(L // 4, beta, dev)
-    stream = _stream(ob)
 
-    def call(lib, base, nwork, counts):
+    def call(lib, stream, base, nwork, tokens_f32, counts, extra):
         return lib.pcfgnat_viterbi_decode(ob.data_ptr(), links.data_ptr(), ol.data_ptr(), tok.data_ptr(), mask.data_ptr(), mask.size(0),
-                                          int(pad_index), pen.data_ptr(), base, base + 8 * nwork, counts,
+                                          int(pad_index), pen.data_ptr(), base, base + 8 * nwork, tokens_f32, counts,
                                           base + 8 * (nwork + B * L), B, L, ml, stream)
 
     tokens, pred, _ = _viterbi_decode_call("pcfg_viterbi_decode", B, L, ml, dev, 0, call)
@@ -995,14 +1040,13 @@ def pcfg_viterbi_decode_logits(logits, links, output_length, left_tree_mask, pad
     mask = left_tree_mask.to(dtype=torch.int64).contiguous()
     pen = _length_penalty(L // 4, beta, dev)
     code = _DTYPE_CODE[logits.dtype]
-    stream = _stream(logits)
     nodes = B * L
 
-    def call(lib, base, nwork, counts):
-        idx = base + 8 * (nwork + nodes + B)  # node tokens [B,L] int64, then node scores [B,L] float32
+    def call(lib, stream, base, nwork, tokens_f32, counts, idx):
+        # the caller's words: node tokens [B,L] int64, then node scores [B,L] float32
         return lib.pcfgnat_viterbi_decode_logits(logits.data_ptr(), code, V, idx + 8 * nodes, idx, links.data_ptr(), ol.data_ptr(),
                                                  mask.data_ptr(), mask.size(0), int(pad_index), pen.data_ptr(), base, base + 8 * nwork,
-                                                 counts, base + 8 * (nwork + nodes), B, L, ml, stream)
+                                                 tokens_f32, counts, base + 8 * (nwork + nodes), B, L, ml, stream)
 
     tokens, pred, block = _viterbi_decode_call("pcfg_viterbi_decode_logits", B, L, ml, dev, nodes + (nodes + 1) // 2, call)
     if not return_nodes:
@@ -1046,8 +1090,7 @@ def pcfg_lookahead_decode(links, unreduced_logits, unreduced_tokens, output_leng
             _lib.check(lib.pcfgnat_lookahead_decode(links.data_ptr(), ob_ptr, float(beta), ol.data_ptr(), tok.data_ptr(),
                                                     mask.data_ptr(), mask.size(0), int(pad_index), idx.data_ptr(), out.data_ptr(),
                                                     cnt.data_ptr(), B, L, K - 1, _stream(links)), lib)
-            _pinned_counts.wait(cnt, B, torch.cuda.current_stream(dev), armed)
-            counts = cnt[:B].tolist()
+            counts = _pinned_counts.wait(cnt, B, torch.cuda.current_stream(dev), armed)
         finally:
             _pinned_counts.give_back(cnt)
     if B and min(counts) < 0:

@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), name
         assert name in _lib.SIGNATURES, "binding table lacks %s" % name
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.pcfgnat_abi_version() == 4
+    assert lib.pcfgnat_abi_version() == 5
     assert lib.pcfgnat_pcfg_aux_floats(40, 128, 32, 1) == 40 * (6 * 64 * 34 + 6 * 36)
     # more than 128 main-chain nodes: six tables, the shifts (padded to 16 bytes), two link copies with rows of 64*ceil(Mc/64)
     assert lib.pcfgnat_pcfg_aux_floats(8, 512, 140, 1) == 8 * (6 * 256 * 142 + 144 + 4 * 256 * 256 + 4 * 256 * 142 + 16 * 144 + 4 + 4 * 256 * 142 + 16 * 144 + 2 * 144)
