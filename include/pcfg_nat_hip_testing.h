@@ -55,6 +55,10 @@ int pcfgnat_max_left3_tuned(int on);
  * served, and sentences it left to the plain kernels because their links hold a rule of a composite local tree. */
 int pcfgnat_max_left3_counts(unsigned long long *served, unsigned long long *left_to_plain, int reset);
 
+/* The same two counters for the Viterbi tables at max_left = 3 (pcfgnat_pcfg_viterbi and the decode calls built on it),
+ * whose one-launch kernel the same switch turns on and off. */
+int pcfgnat_max_left3_viterbi_counts(unsigned long long *served, unsigned long long *left_to_plain, int reset);
+
 /* Diagnostic counters since the library was loaded (or the last reset) on the current device: inside sweeps (forward and
  * outside counted apart) and single-call Viterbi decodes that the one-workgroup kernels redid because a pipelined sweep
  * gave up, and sentences given up for good (see pcfgnat_pipeline_redo_wait_limit).  reset != 0 clears them.  A caller that

@@ -40,6 +40,7 @@ SIGNATURES = {
     "pcfgnat_links_grad_range_limit": (None, [ctypes.c_float]),
     "pcfgnat_max_left3_tuned": (_int, [_int]),
     "pcfgnat_max_left3_counts": (_int, [_vp, _vp, _int]),
+    "pcfgnat_max_left3_viterbi_counts": (_int, [_vp, _vp, _int]),
     "pcfgnat_max_left3_supported": (_int, [_i64, _i64]),
     "pcfgnat_pcfg_loss": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "pcfgnat_pcfg_loss_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),

@@ -146,7 +146,11 @@ int inside_ml3_forward_backward(const float *grad_output, const float *match_all
 int generic_best_tree(const float *S, float *aux, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl,
                       int64_t *tree, int64_t B, int64_t L, int64_t T, int64_t ml, void *stream);
 int generic_viterbi(const float *ob, const float *links, const int64_t *ol, float *S, int64_t *R, int64_t *Lt, int64_t *M, int64_t B,
-                    int64_t L, int64_t ml, void *stream);
+                    int64_t L, int64_t ml, void *stream, int skip_ml3_taken = 0);
+// max_left = 3: whether the tuned kernels are switched on (pcfgnat_max_left3_tuned) and, for the Viterbi tables, whether a
+// graph of L nodes fits the one-launch kernel (viterbi.hip); generic_viterbi with skip_ml3_taken = 1 then does the rest.
+bool ml3_tuned_on();
+bool viterbi_ml3_supported(int64_t L);
 
 // ---- DPP helpers: reductions inside a row of 16 lanes and across a wave64 -------------------------------------
 // dpp_ctrl encodings (GFX9): quad_perm = perm bits, row_half_mirror = 0x141, row_mirror = 0x140.

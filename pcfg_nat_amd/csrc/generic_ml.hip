@@ -72,6 +72,13 @@ __device__ __forceinline__ bool taken_by_ml3(int skip_ml3_taken, const float *li
     return !ml3_composite_rules<NTG>(links, d.L, m, tid);
 }
 __device__ __forceinline__ bool taken_by_ml3(int, const double *, const Dims &, int, int, int) { return false; }
+// The same for the Viterbi tables (viterbi_ml3_kernel): a sentence of valid size is left over only if it holds such a rule.
+__device__ __forceinline__ bool viterbi_taken_by_ml3(int skip_ml3_taken, const float *links, int L, int m, int tid) {
+    if (!skip_ml3_taken) return false;  // (uniform)
+    if (m < 2 || m > L || ((m - 2) % 4) != 0) return true;
+    return !ml3_composite_rules<NTG>(links, L, m, tid);
+}
+__device__ __forceinline__ bool viterbi_taken_by_ml3(int, const double *, int, int, int) { return false; }
 
 // ---- inside forward (pcfg_loss.cu:262-349 then :84-224) -----------------------------------------------------
 template <typename RT>
@@ -353,12 +360,14 @@ template <typename RT>
 __global__ __launch_bounds__(NTG) void generic_viterbi_kernel(const RT *__restrict__ ob_all, const RT *__restrict__ links_all,
                                                              const int64_t *__restrict__ out_len, RT *__restrict__ S_all,
                                                              int64_t *__restrict__ R_all,
-                                                             int64_t *__restrict__ Lt_all, int64_t *__restrict__ M_all, int L, int ml) {
+                                                             int64_t *__restrict__ Lt_all, int64_t *__restrict__ M_all, int L, int ml,
+                                                             int skip_ml3_taken) {
     const int Lq = L / 4;
     const int b = blockIdx.x, tid = threadIdx.x;
     const int m = (int)out_len[b];
     const RT *ob = ob_all + (size_t)b * L;
     const RT *links = links_all + (size_t)b * L * (ml + 1) * L;
+    if (viterbi_taken_by_ml3(skip_ml3_taken, links, L, m, tid)) return;
     const size_t tab = (size_t)b * L * Lq;
     // the local-tree table lives in the rows of S that belong to local nodes and node 0 (the S sweep only touches
     // main-chain rows); those cells are put back to -inf at the end, as the reference returns them
@@ -466,9 +475,9 @@ int best_tree_t(const RT *S, RT *aux, const RT *match_all, const RT *links, cons
 }
 template <typename RT>
 int viterbi_t(const RT *ob, const RT *links, const int64_t *ol, RT *S, int64_t *R, int64_t *Lt, int64_t *M, int64_t B, int64_t L, int64_t ml,
-              void *stream) {
+              void *stream, int skip_ml3_taken = 0) {
     hipLaunchKernelGGL(generic_viterbi_kernel<RT>, dim3((unsigned)B), dim3(NTG), 0, (hipStream_t)stream, ob, links, ol, S, R, Lt, M, (int)L,
-                       (int)ml);
+                       (int)ml, skip_ml3_taken);
     PCFGNAT_HIP_CHECK(hipGetLastError());
     return PCFGNAT_OK;
 }
@@ -500,8 +509,8 @@ int generic_best_tree(const float *S, float *aux, const float *match_all, const 
 }
 
 int generic_viterbi(const float *ob, const float *links, const int64_t *ol, float *S, int64_t *R, int64_t *Lt, int64_t *M, int64_t B,
-                    int64_t L, int64_t ml, void *stream) {
-    return viterbi_t<float>(ob, links, ol, S, R, Lt, M, B, L, ml, stream);
+                    int64_t L, int64_t ml, void *stream, int skip_ml3_taken) {
+    return viterbi_t<float>(ob, links, ol, S, R, Lt, M, B, L, ml, stream, skip_ml3_taken);
 }
 
 }  // namespace pcfgnat

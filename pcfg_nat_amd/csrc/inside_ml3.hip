@@ -340,6 +340,8 @@ bool g_ml3_tuned = true;
 
 }  // namespace
 
+bool ml3_tuned_on() { return g_ml3_tuned; }
+
 bool inside_ml3_supported(int64_t L, int64_t T) {
     if (!g_ml3_tuned || L < 6) return false;
     const int64_t Mc = (L - 2) / 4 + 1;

@@ -349,6 +349,156 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
 }
 
 // ------------------------------------------------------------------------------------------------------------
+// max_left = 3 (two layers of local tree in front of every main-chain node; pcfg_viterbi.cu:22-140 with ml = 3) for
+// sentences whose links hold no rule of a composite local tree (ml3_composite_rules: every sentence the model's scorer can
+// produce, where a local node has no allowed right child).  Then calculate_C_kernel (:177-241) leaves only the two leaves
+// a-1 and a-3 with yield 1 and the null child with yield 0, and the main-chain recursion is the one above with a stride of
+// four nodes and three left options per (parent, child) instead of two:
+//   S[a][len] = ob[a] + max over c of  links[a][0][c] + 0 + S[c][len-1],  links[a][3][c] + ob[a-3] + S[c][len-2],
+//                                      links[a][1][c] + ob[a-1] + S[c][len-2]
+// visited in that order per child, which is the reference's (yield j ascending, then left node b ascending), with the
+// same association order and the same tie order across its 4-lane strided scan.  Outputs are the reference's full tables.
+// A sentence that does hold such a rule is left untouched for the general kernel launched behind (skip_ml3_taken).
+__device__ unsigned long long g_viterbi_ml3_counts[2];  // diagnostic: sentences served here, sentences left to the general kernel
+
+__device__ __forceinline__ int tie_key3(int rel_c, int option) {
+    const int lane = rel_c & 3;
+    const int rank = (lane == 0) ? 0 : (lane == 2) ? 1 : (lane == 1) ? 2 : 3;
+    return (rank << 24) | (rel_c << 2) | option;
+}
+
+template <int NQ>
+__global__ __launch_bounds__(NT) void viterbi_ml3_kernel(const float *__restrict__ ob_lprob, const float *__restrict__ links,
+                                                        const int64_t *__restrict__ out_len, float *__restrict__ S,
+                                                        int64_t *__restrict__ Rt, int64_t *__restrict__ Lt, int64_t *__restrict__ Mt,
+                                                        int L, int Lq) {
+    constexpr int R = (NQ + 3) / 4;
+    constexpr int MP = 64 * R;
+    __shared__ float col[3 * MP];
+    const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j16 = tid & 15;
+    const int m = (int)out_len[b];
+    const float *ob = ob_lprob + (size_t)b * L;
+    const float *lk = links + (size_t)b * L * 4 * L;
+    const size_t tab = (size_t)b * L * Lq;
+    float *Sb = S + tab;
+    int64_t *Rb = Rt + tab, *Lb = Lt + tab, *Mb = Mt + tab;
+    const bool in_contract = !(m < 2 || m > L || ((m - 2) % 4) != 0);
+    const bool composite = in_contract && ml3_composite_rules<NT>(lk, L, m, tid);  // workgroup-uniform
+    if (tid == 0) atomicAdd(&g_viterbi_ml3_counts[composite ? 1 : 0], 1ull);
+    if (composite) return;
+    for (size_t i = tid; i < (size_t)L * Lq; i += NT) {  // pcfg_viterbi.cu:159, 287-289
+        Sb[i] = NEG_INF_F;
+        Rb[i] = 0;
+        Lb[i] = 0;
+        Mb[i] = 0;
+    }
+    if (!in_contract) return;  // out of contract: the empty tables
+    const int mc = (m - 2) / 4 + 1;
+
+    // slabs: unconditional loads from clamped addresses (all in flight together), masked afterwards; what does not change
+    // from length to length (links + 0, links + ob[leaf]) is added once, in the reference's association order
+    float A0[R][NQ], A3[R][NQ], A1[R][NQ], ob_a[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int a = 4 * min(gidx + 64 * r, mc - 1) + 1;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            if (q >= 4 * r) {
+                const int c = 4 * min(j16 + 16 * q, mc - 1) + 1;
+                A0[r][q] = lk[((size_t)a * 4 + 0) * L + c];
+                A3[r][q] = lk[((size_t)a * 4 + 3) * L + c];
+                A1[r][q] = lk[((size_t)a * 4 + 1) * L + c];
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int a_id = gidx + 64 * r, a = 4 * min(a_id, mc - 1) + 1;
+        const float oa = ob[a], leaf1 = ob[a - 1], leaf3 = ob[max(a - 3, 0)];
+        ob_a[r] = (a_id < mc) ? oa : NEG_INF_F;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            if (q >= 4 * r) {
+                const int c_id = j16 + 16 * q;
+                const bool ok = a_id < mc && c_id < mc && c_id >= a_id;
+                const bool with_leaf = ok && a_id >= 1;  // the root's only left child is the null node (:70, b_start = 1)
+                A0[r][q] = ok ? A0[r][q] + 0.f : NEG_INF_F;
+                A3[r][q] = with_leaf ? A3[r][q] + leaf3 : NEG_INF_F;
+                A1[r][q] = with_leaf ? A1[r][q] + leaf1 : NEG_INF_F;
+            }
+        }
+    }
+    // length 0: nothing; length 1: only the last node (pcfg_viterbi.cu:57-59)
+    for (int i = tid; i < 3 * MP; i += NT) col[i] = (i == 1 * MP + mc - 1) ? ob[m - 1] : NEG_INF_F;
+    __syncthreads();  // also orders the table fill above before the cells written below
+    if (tid == 0 && Lq > 1) Sb[(size_t)(m - 1) * Lq + 1] = ob[m - 1];
+
+    const int len_end = m / 4;  // pcfg_viterbi.cu:67
+    int i1 = 1, i2 = 0, i0 = 2;  // column slots of len-1, len-2, len
+    for (int len = 2; len < len_end; len++) {
+        const float *cur1 = col + i1 * MP, *cur2 = col + i2 * MP;
+        float *nxt = col + i0 * MP;
+        float sc1[NQ], sc2[NQ];
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            sc1[q] = cur1[j16 + 16 * q];
+            sc2[q] = cur2[j16 + 16 * q];
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int a_id = gidx + 64 * r;
+            float best = NEG_INF_F;
+            int sel = -1;
+#pragma unroll
+            for (int q = 0; q < NQ; q++) {
+                if (q >= 4 * r) {
+                    const float c0 = (A0[r][q] + sc1[q]) + ob_a[r];
+                    const float c3 = (A3[r][q] + sc2[q]) + ob_a[r];
+                    const float c1 = (A1[r][q] + sc2[q]) + ob_a[r];
+                    if (c0 > best) {  // false for NaN and for -inf against the initial -inf
+                        best = c0;
+                        sel = 4 * q;
+                    }
+                    if (c3 > best) {
+                        best = c3;
+                        sel = 4 * q + 1;
+                    }
+                    if (c1 > best) {
+                        best = c1;
+                        sel = 4 * q + 2;
+                    }
+                }
+            }
+            // row maximum first, then the smallest tie key among the lanes that hold it
+            const float mine = best;
+            best = row16_max_raw(best);
+            int key = (sel < 0 || mine != best) ? 0x7fffffff : tie_key3(j16 + 16 * (sel >> 2) - a_id, sel & 3);
+            key = min(key, dpp_i<DPP_QUAD_XOR1>(key));
+            key = min(key, dpp_i<DPP_QUAD_XOR2>(key));
+            key = min(key, dpp_i<DPP_ROW_HALF_MIRROR>(key));
+            key = min(key, dpp_i<DPP_ROW_MIRROR>(key));
+            if (j16 == 0) {
+                nxt[a_id] = best;
+                if (best != NEG_INF_F && a_id < mc) {  // pcfg_viterbi.cu:125-131
+                    const int a = 4 * a_id + 1;
+                    const int option = key & 3, rel = (key >> 2) & 0x3fffff;
+                    const unsigned o = (unsigned)(a * Lq + len);  // 32-bit offset from the uniform table bases
+                    Sb[o] = best;
+                    Lb[o] = option == 0 ? 0 : option == 1 ? a - 3 : a - 1;
+                    Rb[o] = 4 * (a_id + rel) + 1;
+                    Mb[o] = option ? 1 : 0;
+                }
+            }
+        }
+        const int t = i2;
+        i2 = i1;
+        i1 = i0;
+        i0 = t;
+        lds_barrier();
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
 // Pipelined sweep for the single-call decode of long graphs (same idea as the pipelined inside sweeps): the main chain is
 // cut into blocks of 16 parents, one workgroup per block - four compute waves (one 16-lane row per parent, its
 // triangular link slabs in registers) and one collector wave.  A parent combines children c >= a only, so the top
@@ -715,10 +865,27 @@ extern "C" int pcfgnat_pcfg_viterbi(const float *ob_lprob, const float *links, c
     PCFGNAT_REQUIRE(L / 4 > ml, "pcfg_viterbi: L/4 must exceed max_left");
     if (B == 0) return PCFGNAT_OK;
     PCFGNAT_REQUIRE(ob_lprob && links && output_length && S && R && Lt && M, "pcfg_viterbi: null pointer");
-    if (ml != 1) return generic_viterbi(ob_lprob, links, output_length, S, R, Lt, M, B, L, ml, stream);
-    const int Mc = (int)((L - 2) / 2 + 1);
     const int Lq = (int)(L / 4);
     hipStream_t s = (hipStream_t)stream;
+    if (ml == 3 && viterbi_ml3_supported(L)) {
+        // the sentences without a rule of a composite local tree in one launch, the others by the general kernel behind
+        const int Mc3 = (int)((L - 2) / 4 + 1);
+#define PCFGNAT_VITERBI3_CASE(nq)                                                                                             \
+    else if (Mc3 <= 16 * (nq))                                                                                               \
+        hipLaunchKernelGGL((viterbi_ml3_kernel<nq>), dim3((unsigned)B), dim3(NT), 0, s, ob_lprob, links, output_length, S, R, Lt, M, \
+                           (int)L, Lq)
+        if (false) {
+        }
+        PCFGNAT_VITERBI3_CASE(2);
+        PCFGNAT_VITERBI3_CASE(4);
+        PCFGNAT_VITERBI3_CASE(6);
+        PCFGNAT_VITERBI3_CASE(8);
+#undef PCFGNAT_VITERBI3_CASE
+        PCFGNAT_HIP_CHECK(hipGetLastError());
+        return generic_viterbi(ob_lprob, links, output_length, S, R, Lt, M, B, L, ml, stream, 1);
+    }
+    if (ml != 1) return generic_viterbi(ob_lprob, links, output_length, S, R, Lt, M, B, L, ml, stream);
+    const int Mc = (int)((L - 2) / 2 + 1);
 #define PCFGNAT_VITERBI_CASE(nq)                                                                                              \
     else if (Mc <= 16 * (nq))                                                                                                \
         hipLaunchKernelGGL((viterbi_ml1_kernel<nq, false>), dim3((unsigned)B), dim3(NT), 0, s, ob_lprob, links, output_length, S, R, Lt, \
@@ -877,6 +1044,20 @@ extern "C" int pcfgnat_viterbi_decoding_host(const int64_t *pred_length, const i
                                    stack, stack + L, (int)L, (int)Lq);
     }
     free(stack);
+    return PCFGNAT_OK;
+}
+
+bool pcfgnat::viterbi_ml3_supported(int64_t L) { return ml3_tuned_on() && L >= 6 && (L - 2) / 4 + 1 <= 128; }
+
+extern "C" int pcfgnat_max_left3_viterbi_counts(unsigned long long *served, unsigned long long *left_to_plain, int reset) {
+    unsigned long long h[2] = {0, 0};
+    PCFGNAT_HIP_CHECK(hipMemcpyFromSymbol(h, HIP_SYMBOL(pcfgnat::g_viterbi_ml3_counts), sizeof(h)));
+    if (served) *served = h[0];
+    if (left_to_plain) *left_to_plain = h[1];
+    if (reset) {
+        const unsigned long long z[2] = {0, 0};
+        PCFGNAT_HIP_CHECK(hipMemcpyToSymbol(HIP_SYMBOL(pcfgnat::g_viterbi_ml3_counts), z, sizeof(z)));
+    }
     return PCFGNAT_OK;
 }
 

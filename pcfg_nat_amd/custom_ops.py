@@ -255,13 +255,13 @@ def max_left_path(max_left, L=None, T=None):
     return "generic"
 
 
-def max_left3_counts(reset=False):
+def max_left3_counts(reset=False, viterbi=False):
     """Diagnostic: (sentences served by the one-launch kernel for ``max_left = 3``, sentences it left to the plain kernels)
-    on the current device since the last reset."""
-    import ctypes
+    on the current device since the last reset; ``viterbi``: the counters of the Viterbi tables instead of the loss."""
     a, b = ctypes.c_ulonglong(0), ctypes.c_ulonglong(0)
     lib = get_pcfg_kernel()
-    _lib.check(lib.pcfgnat_max_left3_counts(ctypes.byref(a), ctypes.byref(b), 1 if reset else 0), lib)
+    fn = lib.pcfgnat_max_left3_viterbi_counts if viterbi else lib.pcfgnat_max_left3_counts
+    _lib.check(fn(ctypes.byref(a), ctypes.byref(b), 1 if reset else 0), lib)
     return int(a.value), int(b.value)
 
 

@@ -1397,6 +1397,79 @@ def test_general_max_left_viterbi_bit_exact(ml, L, ms):
     assert np.array_equal(R.cpu().numpy(), R_o) and np.array_equal(Lt.cpu().numpy(), L_o) and np.array_equal(M.cpu().numpy(), M_o)
 
 
+def _viterbi_tables_equal_oracle(ob, links, ol):
+    scores, R, Lt, M = ops.cuda_pcfg_viterbi(torch.from_numpy(ob).to(DEV), torch.from_numpy(links).to(DEV), ol.to(DEV))
+    S_o, R_o, L_o, M_o = oracle.viterbi(ob, links, ol.numpy(), dtype=np.float32)
+    assert np.array_equal(scores.cpu().numpy(), S_o[:, 1, :])
+    assert np.array_equal(R.cpu().numpy(), R_o) and np.array_equal(Lt.cpu().numpy(), L_o) and np.array_equal(M.cpu().numpy(), M_o)
+    return S_o, (scores, R, Lt, M)
+
+
+@pytest.mark.parametrize("quantised", [False, True])
+@pytest.mark.parametrize("L,ms", [(18, [18, 14, 6, 2]), (66, [66, 50, 34, 6]), (130, [130, 98, 42]), (258, [258, 254, 130]),
+                                  (402, [402, 202]), (510, [510, 398])])
+def test_max_left3_viterbi_one_launch_kernel_bit_exact(L, ms, quantised):
+    """Viterbi tables at max_left = 3 with links as the model's scorer produces them (no local node has a rule): the
+    one-launch kernel serves every sentence and returns the oracle's scores and back-pointers bit for bit, as do the plain
+    kernels.  ``quantised``: values on a grid of quarters, so that exact ties between candidates are the rule and the
+    winner is decided by the reference's scan order (lane of its strided scan, child, yield, left node)."""
+    from test_oracle_inside import random_links
+    rng = np.random.default_rng(900 + L + (1 if quantised else 0))
+    links = np.stack([random_links(rng, L, m, 3, p_drop=0.1) for m in ms]).astype(np.float32)
+    ob = (rng.normal(size=(len(ms), L)) - 1.0).astype(np.float32)
+    if quantised:
+        links = (np.round(links * 2) / 2).astype(np.float32)  # (-inf stays -inf)
+        ob = (np.round(ob * 2) / 2).astype(np.float32)
+    ol = torch.tensor(ms)
+    ops.max_left3_counts(reset=True, viterbi=True)
+    S_o, tuned = _viterbi_tables_equal_oracle(ob, links, ol)
+    assert ops.max_left3_counts(viterbi=True) == (len(ms), 0)
+    assert np.isfinite(S_o[0, 1, 2:]).any()
+    was = ops.max_left3_tuned(0)
+    try:
+        _, plain = _viterbi_tables_equal_oracle(ob, links, ol)
+        assert ops.max_left3_counts(viterbi=True) == (len(ms), 0)  # (the plain kernel ran alone: the counters did not move)
+    finally:
+        ops.max_left3_tuned(was)
+    for t, p in zip(tuned, plain):
+        assert torch.equal(t, p)
+
+
+def test_max_left3_viterbi_mixed_batch_and_invalid_lengths():
+    """Sentences with and without rules of composite local trees in one batch, and graph sizes outside the contract (empty
+    tables): the one-launch kernel takes what it covers, the plain kernel the rest."""
+    from test_oracle_inside import random_links
+    L = 46
+    ms = [46, 30, 45, 22, 4, 46, 47, 38]
+    composite = [False, True, False, True, False, True, False, False]
+    rng = np.random.default_rng(78)
+    links = np.stack([random_links(rng, L, min(m, L), 3, p_drop=0.1, generic_local=c) for m, c in zip(ms, composite)]).astype(np.float32)
+    ob = (rng.normal(size=(len(ms), L)) - 1.0).astype(np.float32)
+    ops.max_left3_counts(reset=True, viterbi=True)
+    S_o, _ = _viterbi_tables_equal_oracle(ob, links, torch.tensor(ms))
+    assert ops.max_left3_counts(viterbi=True) == (5, 3)
+    assert np.isfinite(S_o[[0, 1, 3, 5, 7], 1, :]).any(axis=1).all() and not np.isfinite(S_o[[2, 4, 6], 1, :]).any()
+
+
+@pytest.mark.parametrize("ml,L,ms", [(3, 66, [66, 50, 34, 6]), (3, 258, [258, 130]), (2, 50, [50, 32]), (0, 24, [24, 13])])
+def test_general_max_left_decode_vs_oracle(ml, L, ms):
+    """The Viterbi decode at max_left != 1 (full tables, selection and walk as separate launches): the single native call and
+    the three operators one by one emit the oracle's tokens and lengths, with the left-tree mask of that tree shape."""
+    import oracle_ops
+    gen = torch.Generator().manual_seed(100 * ml + L)
+    m = torch.tensor(ms)
+    links = synth.make_links(len(ms), L, m, ml, gen)
+    ob, tok = synth.ob_and_tokens(torch.randn(len(ms), L, 48, generator=gen) * 3)
+    left_mask = synth.support_masks(L, ml)[0]
+    want_tok, want_len = harness.viterbi_decode(ob, tok, links, m, left_mask, ops=oracle_ops)
+    assert want_tok.shape[1] >= 3 and (want_len > 1).any()  # a real tree, not the one-token fallback of a dead graph
+    for single in (False, True):
+        got_tok, got_len = harness.viterbi_decode(ob.to(DEV), tok.to(DEV), links.to(DEV), m.to(DEV), left_mask.to(DEV),
+                                                  single_call=single)
+        assert torch.equal(got_len.cpu(), want_len)
+        assert got_tok.dtype == torch.float32 and torch.equal(got_tok.cpu(), want_tok)
+
+
 @pytest.mark.parametrize("ml,L,ms,ns,generic_local", [
     (1, 32, [32, 20, 8], [10, 8, 3], False),
     (1, 130, [130, 96], [22, 30], False),
