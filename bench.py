@@ -513,7 +513,47 @@ def max_left3_timing(dev):
     res["plain_kernels_ms_per_call"] = ms_plain
     res["speedup_vs_plain_kernels"] = ms_plain / ms
     res["log_likelihoods_agree"] = bool(torch.allclose(ll, ll_plain, rtol=1e-5))
+    res["viterbi_decode"] = max_left3_decode_timing(dev)
     return res
+
+
+def max_left3_decode_timing(dev):
+    """The single-call Viterbi decode (tables, length selection, walk) for ``--left-tree-layer 2`` on graphs of 130, 258 and
+    402 nodes (source lengths 32, 64, 100) at batch 1 and of 258 nodes at batch 64, wall clock per call, with the
+    one-launch table kernel and with the plain kernel."""
+    import time
+    import torch
+    from pcfg_nat_amd import custom_ops as ops, synth
+
+    ml, out = 3, []
+    gen = torch.Generator().manual_seed(1004)
+    for B, L in ((1, 130), (1, 258), (1, 402), (64, 258)):
+        m = torch.full((B,), L, dtype=torch.int64)
+        links = synth.make_links(B, L, m, ml, gen).to(dev)
+        ob, tok = synth.ob_and_tokens(torch.randn(B, L, 48, generator=gen) * 3)
+        mask = synth.support_masks(L, ml)[0].to(dev)
+        args = (ob.to(dev), links, m.to(dev), tok.to(dev), mask, synth.PAD)
+
+        def timed(reps):
+            for _ in range(2):
+                ops.pcfg_viterbi_decode(*args)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                got = ops.pcfg_viterbi_decode(*args)
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / reps * 1e3, got
+
+        ms, got = timed(20)
+        was = ops.max_left3_tuned(0)
+        try:
+            ms_plain, got_plain = timed(3)
+        finally:
+            ops.max_left3_tuned(was)
+        out.append({"batch": B, "graph_nodes": L, "ms_per_call": ms, "plain_kernel_ms_per_call": ms_plain,
+                    "speedup_vs_plain_kernel": ms_plain / ms, "emitted_tokens_max": int(got[0].size(1)),
+                    "same_tokens": bool(torch.equal(got[0], got_plain[0]) and torch.equal(got[1], got_plain[1]))})
+    return out
 
 
 def decode_front_end_timing(dev):
