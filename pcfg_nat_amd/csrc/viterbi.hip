@@ -56,35 +56,20 @@ struct FullTraces {
     __host__ __device__ int64_t right(int64_t node, int64_t len) const { return Ri[node * Lq + len]; }
     __host__ __device__ int64_t mid(int64_t node, int64_t len) const { return Mi[node * Lq + len]; }
 };
-// CompactTraces: one int32 per (main-chain node, length), 0 = empty cell, else 1 + ((c_id - a_id) << 1 | j); the rows of
-// the local leaves are never written by the sweep and read as zeros, as they do in the full tables.
-struct CompactTraces {
-    const int *W;
-    int Lq, rows;
-    __device__ int rec(int64_t node, int64_t len) const {
-        const int64_t a_id = node >> 1;
-        return ((node & 1) && a_id < rows) ? W[a_id * Lq + len] : 0;
-    }
-    __device__ int64_t left(int64_t node, int64_t len) const {
-        const int r = rec(node, len);
-        return (r != 0 && ((r - 1) & 1)) ? node - 1 : 0;
-    }
-    __device__ int64_t right(int64_t node, int64_t len) const {
-        const int r = rec(node, len);
-        return r == 0 ? 0 : 2 * ((node >> 1) + ((r - 1) >> 1)) + 1;
-    }
-    __device__ int64_t mid(int64_t node, int64_t len) const {
-        const int r = rec(node, len);
-        return r == 0 ? 0 : ((r - 1) & 1);
-    }
+// What the walk reads besides the traces: the nodes' tokens and the left-tree mask, from memory.
+struct WalkInputs {
+    const int64_t *tok, *mask;
+    int64_t mask_dim;
+    __host__ __device__ bool in_range(int64_t node, int64_t l) const { return !(l < 0 || l >= mask_dim || node >= mask_dim); }
+    __host__ __device__ bool forbidden(int64_t node, int64_t l) const { return mask[node * mask_dim + l] != 0; }
+    __host__ __device__ int64_t token(int64_t node) const { return tok[node]; }
 };
 
 // One walk per sentence (pcfg_loss.cpp:22-59).  Shared by the device kernels and the host entry point.  SI = integer
 // type of the explicit stacks.
-template <typename Traces, typename SI>
-__host__ __device__ inline int64_t readout_one(int64_t pred_len, int64_t max_h, const Traces &tr, const int64_t *tok,
-                                               const int64_t *mask, int64_t mask_dim, int64_t pad, int64_t *out, SI *stack_node,
-                                               SI *stack_len, int L, int Lq) {
+template <typename Traces, typename Inputs, typename SI>
+__host__ __device__ inline int64_t readout_one(int64_t pred_len, int64_t max_h, const Traces &tr, const Inputs &in, int64_t pad,
+                                               int64_t *out, SI *stack_node, SI *stack_len, int L, int Lq) {
     const int cap = L;
     int sp = 0;
     int64_t cnt = 0, node = 1, len = pred_len, last = -1;
@@ -99,8 +84,8 @@ __host__ __device__ inline int64_t readout_one(int64_t pred_len, int64_t max_h, 
             sp++;
             int64_t l = tr.left(node, len);
             l = (l == node) ? 0 : l;
-            if (l < 0 || l >= mask_dim || node >= mask_dim) return -1;
-            if (mask[node * mask_dim + l]) break;
+            if (!in.in_range(node, l)) return -1;
+            if (in.forbidden(node, l)) break;
             const int64_t nl = tr.mid(node, len);
             node = l;
             len = nl;
@@ -108,7 +93,7 @@ __host__ __device__ inline int64_t readout_one(int64_t pred_len, int64_t max_h, 
         sp--;
         node = stack_node[sp];
         len = stack_len[sp];
-        const int64_t t = tok[node];
+        const int64_t t = in.token(node);
         if (t != pad && t != last) {
             last = t;
             if (cnt >= cap) return -1;
@@ -118,6 +103,45 @@ __host__ __device__ inline int64_t readout_one(int64_t pred_len, int64_t max_h, 
         const int64_t nl = len - tr.mid(node, len) - 1;
         node = r;
         len = nl;
+    }
+    return cnt;
+}
+
+// The same walk over the compact records of the single-call decode (max_left = 1): one int32 per (main-chain node,
+// length), 0 = empty cell, else 1 + ((c_id - a_id) << 1 | j); the rows of the local leaves are never written and read as
+// zeros, as they do in the full tables.  With such traces the walk needs no stack: it runs down the main chain, and a
+// node's left child is the null node or the leaf in front of it, whose own children are null - so per main-chain node
+// the walk above emits the leaf (if the record names it, it is not node 0 and the mask allows the descent), then the
+// node, and goes on to the right child with what is left of the length.  Inputs staged in LDS by the workgroup: the
+// tokens, and of the mask the one entry per node that can matter, (node, node - 1).  W holds [rows][stride] records.
+// Returns the number of tokens emitted, -1 for malformed traces (as readout_one).
+__device__ inline int64_t walk_compact_ml1(int pred_len, int64_t max_h, const int *W, int stride, int rows, const int64_t *tok,
+                                           const unsigned char *leaf_forbidden, int64_t mask_dim, int64_t pad, int64_t *out, int L,
+                                           int Lq) {
+    int64_t cnt = 0, last = -1;
+    int node = 1, len = pred_len;
+    if (len < 0 || len >= Lq) return -1;
+    while (node < max_h && node != 0) {
+        if (node >= L || len < 0 || len >= Lq || node >= mask_dim) return -1;
+        const int a_id = node >> 1;
+        const int r = ((node & 1) && a_id < rows) ? W[a_id * stride + len] : 0;
+        const int j = (r != 0) ? ((r - 1) & 1) : 0;
+        if (j && node > 1 && !leaf_forbidden[node]) {
+            const int64_t t = tok[node - 1];
+            if (t != pad && t != last) {
+                last = t;
+                if (cnt >= L) return -1;
+                out[cnt++] = t;
+            }
+        }
+        const int64_t t = tok[node];
+        if (t != pad && t != last) {
+            last = t;
+            if (cnt >= L) return -1;
+            out[cnt++] = t;
+        }
+        node = (r != 0) ? 2 * (a_id + ((r - 1) >> 1)) + 1 : 0;
+        len = len - j - 1;
     }
     return cnt;
 }
@@ -173,8 +197,11 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
     constexpr int R = (NQ + 3) / 4;
     constexpr int MP = 64 * R;
     __shared__ float col[3 * MP];
-    extern __shared__ int dyn[];  // COMPACT: scores [Lq] (float), stacks [2][L] (int)
-    float *sm_scores = reinterpret_cast<float *>(dyn);
+    // COMPACT: tokens [L] (int64), scores [Lq] (float), mask entries [L] (bytes)
+    extern __shared__ __align__(8) int64_t dyn64[];
+    int64_t *sm_tok = dyn64;
+    float *sm_scores = reinterpret_cast<float *>(dyn64 + L);
+    unsigned char *sm_leaf = reinterpret_cast<unsigned char *>(sm_scores + Lq);
     const int b = blockIdx.x, tid = threadIdx.x, gidx = tid >> 4, j16 = tid & 15;
     const int m = (int)out_len[b];
     const float *ob = ob_lprob + (size_t)b * L;
@@ -192,7 +219,12 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
         if (!from_pipe)
             for (int i = tid; i < rowsW * Lq; i += NT) Wb[i] = 0;
         for (int i = tid; i < Lq; i += NT) sm_scores[i] = from_pipe ? dec.pipe_scores[(size_t)b * Lq + i] : NEG_INF_F;
-        for (int i = tid; i < L; i += NT) dec.out_tokens[(size_t)b * L + i] = dec.pad;
+        for (int i = tid; i < L; i += NT) {
+            dec.out_tokens[(size_t)b * L + i] = dec.pad;
+            // what the walk will read, staged while the sweep runs
+            sm_tok[i] = dec.tokens[(size_t)b * L + i];
+            sm_leaf[i] = (i < dec.mask_dim && i >= 1 && dec.mask[(size_t)i * dec.mask_dim + (i - 1)] != 0) ? 1 : 0;
+        }
     } else {
         // tables start as -inf / 0 (pcfg_viterbi.cu:159, 287-289)
         for (size_t i = tid; i < (size_t)L * Lq; i += NT) {
@@ -332,11 +364,9 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
         if (tid < 64) {
             const int pl = select_length(sm_scores, dec.penalty, Lq, tid);
             if (tid == 0) {
-                int *stack_node = dyn + Lq, *stack_len = stack_node + L;
-                const CompactTraces tr{Wb, Lq, rowsW};
                 dec.pred_length[b] = pl;
-                count = readout_one(pl, out_len[b], tr, dec.tokens + (size_t)b * L, dec.mask, dec.mask_dim, dec.pad,
-                                    dec.out_tokens + (size_t)b * L, stack_node, stack_len, L, Lq);
+                count = walk_compact_ml1(pl, out_len[b], Wb, Lq, rowsW, sm_tok, sm_leaf, dec.mask_dim, dec.pad,
+                                         dec.out_tokens + (size_t)b * L, L, Lq);
             }
         }
         if (dec.out_tokens_f32 != nullptr) {  // workgroup-uniform
@@ -742,8 +772,8 @@ __global__ void readout_kernel(const int64_t *pred_length, const int64_t *output
     const size_t tab = (size_t)i * L * Lq;
     int64_t *stack_node = scratch + (size_t)i * 2 * L, *stack_len = stack_node + L;
     const FullTraces tr{Lt + tab, Rt + tab, Mt + tab, Lq};
-    out_count[i] = readout_one(pred_length[i], output_length[i], tr, tokens + (size_t)i * L, mask, mask_dim, pad, out, stack_node,
-                               stack_len, L, Lq);
+    const WalkInputs in{tokens + (size_t)i * L, mask, mask_dim};
+    out_count[i] = readout_one(pred_length[i], output_length[i], tr, in, pad, out, stack_node, stack_len, L, Lq);
 }
 
 // Length selection on full tables (one wave per sentence): scores[len] = S[b][1][len].
@@ -928,7 +958,7 @@ template <int NQ>
 int launch_decode(const float *ob_lprob, const float *links, const int64_t *output_length, DecodeArgs dec, void *workspace, int64_t B,
                   int64_t L, hipStream_t s) {
     const int Lq = (int)(L / 4);
-    const size_t dyn = ((size_t)Lq + 2 * (size_t)L) * sizeof(int);
+    const size_t dyn = (size_t)L * sizeof(int64_t) + (size_t)Lq * sizeof(int) + (size_t)L;
     const size_t nw = (size_t)B * (size_t)(L / 2) * Lq, nx = (size_t)B * Lq * 16 * NQ, ns = (size_t)B * Lq;
     if (decode_pipelined(NQ, B)) {
         int *W = (int *)workspace;
@@ -1040,8 +1070,8 @@ extern "C" int pcfgnat_viterbi_decoding_host(const int64_t *pred_length, const i
         for (int64_t k = 0; k < L; k++) out[k] = pad_index;
         const size_t tab = (size_t)i * L * Lq;
         const FullTraces tr{Lt + tab, R + tab, M + tab, (int)Lq};
-        out_count[i] = readout_one(pred_length[i], output_length[i], tr, tokens + (size_t)i * L, left_tree_mask, mask_dim, pad_index, out,
-                                   stack, stack + L, (int)L, (int)Lq);
+        const WalkInputs in{tokens + (size_t)i * L, left_tree_mask, mask_dim};
+        out_count[i] = readout_one(pred_length[i], output_length[i], tr, in, pad_index, out, stack, stack + L, (int)L, (int)Lq);
     }
     free(stack);
     return PCFGNAT_OK;
