@@ -280,6 +280,7 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
     }
 
     const int len_end = m / 4;  // pcfg_viterbi.cu:67
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int i1 = 1, i2 = 0, i0 = 2;  // column slots of len-1, len-2, len
     for (int len = 2; len < len_end; len++) {
         const float *cur1 = col + i1 * MP, *cur2 = col + i2 * MP;
@@ -298,6 +299,12 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const int a_id = gidx + 64 * r;
+            // The link matrices are triangular and the sentence may be shorter than the slabs: a wave whose four parents
+            // all lie behind the last node has nothing to do in this pass, and a chunk of children that lies in front of
+            // all four parents, or behind the last node, holds no candidate for it.  (Wave-uniform tests; the columns
+            // keep their initial -inf in the rows nobody writes.)
+            const int row_lo = 64 * r + 4 * wave;
+            if (row_lo >= mc) continue;
             float best = NEG_INF_F;
             int sel = -1;
             if (RELOAD) {
@@ -312,7 +319,7 @@ __global__ __launch_bounds__(NT) void viterbi_ml1_kernel(const float *__restrict
             }
 #pragma unroll
             for (int q = 0; q < NQ; q++) {
-                if (q >= 4 * r) {
+                if (q >= 4 * r && 16 * q + 15 >= row_lo && 16 * q < mc) {
                     const float c0 = (A0[r][q] + sc1[q]) + ob_a[r];
                     const float c1 = (A1[r][q] + sc2[q]) + ob_a[r];
                     if (c0 > best) {  // false for NaN and for -inf against the initial -inf
@@ -464,6 +471,7 @@ __global__ __launch_bounds__(NT) void viterbi_ml3_kernel(const float *__restrict
     if (tid == 0 && Lq > 1) Sb[(size_t)(m - 1) * Lq + 1] = ob[m - 1];
 
     const int len_end = m / 4;  // pcfg_viterbi.cu:67
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int i1 = 1, i2 = 0, i0 = 2;  // column slots of len-1, len-2, len
     for (int len = 2; len < len_end; len++) {
         const float *cur1 = col + i1 * MP, *cur2 = col + i2 * MP;
@@ -477,11 +485,13 @@ __global__ __launch_bounds__(NT) void viterbi_ml3_kernel(const float *__restrict
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const int a_id = gidx + 64 * r;
+            const int row_lo = 64 * r + 4 * wave;  // (as in viterbi_ml1_kernel: passes and chunks without a candidate)
+            if (row_lo >= mc) continue;
             float best = NEG_INF_F;
             int sel = -1;
 #pragma unroll
             for (int q = 0; q < NQ; q++) {
-                if (q >= 4 * r) {
+                if (q >= 4 * r && 16 * q + 15 >= row_lo && 16 * q < mc) {
                     const float c0 = (A0[r][q] + sc1[q]) + ob_a[r];
                     const float c3 = (A3[r][q] + sc2[q]) + ob_a[r];
                     const float c1 = (A1[r][q] + sc2[q]) + ob_a[r];
