@@ -379,6 +379,88 @@ at::Tensor pcfg_extract_links_fused(const at::Tensor &query_chunks, const at::Te
                           right_tree_mask, main_chain);
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The Viterbi decode as one native call (glat_decomposed_with_link_two_hands_tri_pcfg.py:414-416, 483-502): checks, the one
+// allocation and the enqueue.  A decode of one short sentence is a few tens of microseconds of kernels; the same steps in
+// Python (a dozen tensor-attribute calls, the device context, ctypes marshalling of twenty arguments) cost the host about
+// ten more in front of the first launch.
+//
+// From the vocabulary logits [B,L,V] (float16 / float32; `node_scores`, `node_tokens` undefined) or from the node scores
+// [B,L] float32 and node tokens [B,L] (`logits` undefined).  One block holds workspace | tokens [B,L] int64 | predicted
+// lengths [B] | tokens [B,L] float32 | (from logits) node tokens [B,L] int64, node scores [B,L] float32.  The kernels write
+// the per-sentence token counts to `counts_address` (pinned host memory owned by the caller, B int64); if `may_watch` and
+// the stream is idle the entries are marked "not yet" (-2) first and the caller may watch them turn instead of waiting
+// for the stream.  Returns (tokens float32 [B,L], predicted lengths [B], the block, whether the entries were marked).
+// ---------------------------------------------------------------------------------------------------------------
+std::tuple<at::Tensor, at::Tensor, at::Tensor, bool> viterbi_decode_enqueue(const c10::optional<at::Tensor> &logits,
+                                                                            const c10::optional<at::Tensor> &node_scores,
+                                                                            const c10::optional<at::Tensor> &node_tokens,
+                                                                            const at::Tensor &links_in, const at::Tensor &output_length,
+                                                                            const at::Tensor &left_tree_mask, int64_t pad_index,
+                                                                            const at::Tensor &length_penalty, int64_t counts_address,
+                                                                            bool may_watch) {
+    const bool from_logits = logits.has_value() && logits->defined();
+    const char *who = from_logits ? "pcfg_viterbi_decode_logits" : "pcfg_viterbi_decode";
+    at::Tensor ob, tok;
+    int64_t B, L, V = 0;
+    if (from_logits) {
+        need_gpu(who, {&*logits, &links_in, &output_length, &left_tree_mask, &length_penalty});
+        TORCH_CHECK(logits->dim() == 3 && logits->is_contiguous(), who, ": logits must be a contiguous [bsz, prelen, vocab] tensor");
+        TORCH_CHECK(logits->scalar_type() == at::kHalf || logits->scalar_type() == at::kFloat, who,
+                    ": logits must be float16 or float32 (got ", logits->scalar_type(), ")");
+        B = logits->size(0), L = logits->size(1), V = logits->size(2);
+    } else {
+        TORCH_CHECK(node_scores.has_value() && node_tokens.has_value(), who, ": node scores and node tokens are needed");
+        need_gpu(who, {&*node_scores, &links_in, &output_length, &*node_tokens, &left_tree_mask, &length_penalty});
+        TORCH_CHECK(node_scores->dim() == 2 && links_in.dim() == 4, who,
+                    ": unreduced_logits must be [bsz, prelen] and links [bsz, prelen, max_left+1, prelen]");
+        TORCH_CHECK(node_scores->scalar_type() == at::kFloat && links_in.scalar_type() == at::kFloat, who,
+                    ": unreduced_logits and links must be float32");
+        B = node_scores->size(0), L = node_scores->size(1);
+        ob = node_scores->contiguous();
+        tok = node_tokens->scalar_type() == at::kLong ? node_tokens->contiguous() : node_tokens->to(at::kLong).contiguous();
+        TORCH_CHECK(tok.dim() == 2 && tok.size(0) == B && tok.size(1) == L, who, ": unreduced_tokens must be [bsz, prelen]");
+    }
+    TORCH_CHECK(links_in.dim() == 4 && links_in.scalar_type() == at::kFloat, who, ": links must be float32 [bsz, prelen, max_left+1, prelen]");
+    TORCH_CHECK(links_in.size(0) == B && links_in.size(1) == L && links_in.size(3) == L, who, ": links shape ", links_in.sizes(),
+                " does not match [bsz, prelen] = (", B, ", ", L, ")");
+    TORCH_CHECK(left_tree_mask.dim() == 2 && left_tree_mask.size(0) == left_tree_mask.size(1), who, ": left_tree_mask must be square");
+    const int64_t ml = links_in.size(2) - 1;
+    TORCH_CHECK(length_penalty.scalar_type() == at::kFloat && length_penalty.is_contiguous() && length_penalty.numel() >= L / 4, who,
+                ": length penalty must be float32 [prelen / 4]");
+    const at::Tensor links = links_in.contiguous();
+    const at::Tensor ol = lengths(who, output_length, B);
+    const at::Tensor mask = left_tree_mask.scalar_type() == at::kLong ? left_tree_mask.contiguous() : left_tree_mask.to(at::kLong).contiguous();
+    const c10::DeviceGuard guard(links.device());
+    const int64_t nodes = B * L, fwords = (nodes + 1) / 2;
+    const int64_t nwork = (int64_t)((pcfgnat_viterbi_decode_workspace_bytes(B, L, ml) + 7) / 8);
+    const int64_t extra = from_logits ? nodes + fwords : 0;
+    at::Tensor block = at::empty({nwork + nodes + B + fwords + extra}, links.options().dtype(at::kLong).requires_grad(false));
+    int64_t *base = block.data_ptr<int64_t>();
+    int64_t *out_tokens = base + nwork, *pred = out_tokens + nodes;
+    float *tokens_f32 = reinterpret_cast<float *>(pred + B);
+    const auto stream = c10::hip::getCurrentHIPStream(links.device().index());
+    int64_t *counts = reinterpret_cast<int64_t *>(static_cast<intptr_t>(counts_address));
+    TORCH_CHECK(counts != nullptr || B == 0, who, ": no buffer for the token counts");
+    const bool marked = may_watch && B > 0 && stream.query();
+    if (marked)
+        for (int64_t i = 0; i < B; i++) counts[i] = -2;
+    if (from_logits) {
+        int64_t *best_idx = pred + B + fwords;
+        float *best_lprob = reinterpret_cast<float *>(best_idx + nodes);
+        check_rc(pcfgnat_viterbi_decode_logits(logits->data_ptr(), dtype_code(*logits, who), V, best_lprob, best_idx, links.data_ptr<float>(),
+                                               ol.data_ptr<int64_t>(), mask.data_ptr<int64_t>(), mask.size(0), pad_index,
+                                               length_penalty.data_ptr<float>(), base, out_tokens, tokens_f32, counts, pred, B, L, ml,
+                                               (void *)stream.stream()));
+    } else {
+        check_rc(pcfgnat_viterbi_decode(ob.data_ptr<float>(), links.data_ptr<float>(), ol.data_ptr<int64_t>(), tok.data_ptr<int64_t>(),
+                                        mask.data_ptr<int64_t>(), mask.size(0), pad_index, length_penalty.data_ptr<float>(), base, out_tokens,
+                                        tokens_f32, counts, pred, B, L, ml, (void *)stream.stream()));
+    }
+    at::Tensor tokf = block.slice(0, nwork + nodes + B, nwork + nodes + B + fwords).view(at::kFloat).slice(0, 0, nodes).view({B, L});
+    return std::make_tuple(tokf, block.slice(0, nwork + nodes, nwork + nodes + B), block, marked);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -389,6 +471,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("pcfg_criterion", &pcfg_criterion, "the criterion's loss as one differentiable op (nat_pcfg_loss.py:98-145)", py::arg("outputs"),
           py::arg("targets"), py::arg("links"), py::arg("output_length"), py::arg("target_length"), py::arg("matchmask") = py::none(),
           py::arg("keep_word_mask") = py::none());
+    m.def("viterbi_decode_enqueue", &viterbi_decode_enqueue,
+          "checks, allocation and enqueue of the single-call Viterbi decode (glat_decomposed_with_link_two_hands_tri_pcfg.py:414-416, 483-502)");
     m.def("pcfg_extract_links_fused", &pcfg_extract_links_fused,
           "the link scorer after its projections, products inside the kernels (glat_decomposed_with_link_two_hands_tri_pcfg.py:153-199)");
 }

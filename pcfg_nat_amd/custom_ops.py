@@ -904,7 +904,8 @@ class _PinnedCounts:
         return True
 
     def wait(self, buf, n, stream, armed):
-        """Returns the n counts once the kernels have written them."""
+        """Returns the n counts once the kernels have written them.  ``stream``: the stream of the call, or a device (its
+        current stream is looked up only if the call has to wait for it)."""
         words = buf.words
         if armed:
             not_yet = self.NOT_YET
@@ -926,6 +927,8 @@ class _PinnedCounts:
                 self._misses += 1
                 if self._misses >= self.MISSES_TO_SWITCH_OFF:
                     self._polling = False
+        if isinstance(stream, torch.device):
+            stream = torch.cuda.current_stream(stream)
         stream.synchronize()
         return words[:n]
 
@@ -973,13 +976,37 @@ def _viterbi_decode_call(name, B, L, ml, dev, extra_words, call):
             counts = _pinned_counts.wait(host, B, stream, armed)
         finally:
             _pinned_counts.give_back(host)
+    return _emitted(tokf, counts, B, block), pred, block
+
+
+def _emitted(tokf, counts, B, block):
+    """The emitted part of the float32 token rows [B,L]: one sentence is a contiguous view of its row, the rows of a batch
+    are copied together."""
     if B and min(counts) < 0:
         raise RuntimeError("viterbi_decoding: malformed traces")
     maxlen = max(counts) if B else 0
-    tokens = tokf[:, :maxlen]  # one sentence: a contiguous view; a batch: its rows are copied together
+    tokens = tokf[:, :maxlen]
     if B != 1 or block.numel() > _DECODE_VIEW_MAX_WORDS:
         tokens = tokens.clone(memory_format=torch.contiguous_format)
-    return tokens, pred, block
+    return tokens
+
+
+def _viterbi_decode_ext(ext, logits, node_scores, node_tokens, links, output_length, left_tree_mask, pad_index, beta):
+    """The decode calls through the torch extension: checks, allocation and enqueue in C++ (``viterbi_decode_enqueue``),
+    the watch for the counts here.  Returns (tokens, pred_length, block, nodes)."""
+    if links.dim() != 4:
+        raise RuntimeError("pcfg_viterbi_decode: links must be float32 [bsz, prelen, max_left+1, prelen]")
+    B, L = links.size(0), links.size(1)
+    dev = links.device
+    pen = _length_penalty(L // 4, beta, dev)
+    host = _pinned_counts.take(B)
+    try:
+        tokf, pred, block, marked = ext.viterbi_decode_enqueue(logits, node_scores, node_tokens, links, output_length, left_tree_mask,
+                                                               int(pad_index), pen, host.ptr, _pinned_counts.polling_on())
+        counts = _pinned_counts.wait(host, B, dev, marked)
+    finally:
+        _pinned_counts.give_back(host)
+    return _emitted(tokf, counts, B, block), pred, block, B * L
 
 
 def _check_decode_graph(name, B, L, links, left_tree_mask):
@@ -996,6 +1023,11 @@ def pcfg_viterbi_decode(unreduced_logits, links, output_length, unreduced_tokens
     ``cuda_pcfg_viterbi`` -> length penalty ``arange ** beta`` -> NaN masking -> arg max over lengths >= 1 ->
     ``viterbi_decoding``.  Returns (tokens float32 [B, maxlen] right-padded with ``pad_index``, pred_length int64 [B]),
     the values the separate calls give."""
+    ext = _ext()
+    if ext is not None:
+        tokens, pred, _, _ = _viterbi_decode_ext(ext, None, unreduced_logits, unreduced_tokens, links, output_length, left_tree_mask,
+                                                 pad_index, beta)
+        return tokens, pred
     _need_cuda("pcfg_viterbi_decode", unreduced_logits, links, output_length, unreduced_tokens, left_tree_mask)
     if unreduced_logits.dim() != 2 or links.dim() != 4:
         raise RuntimeError("pcfg_viterbi_decode: unreduced_logits must be [bsz, prelen] and links [bsz, prelen, max_left+1, prelen]")
@@ -1026,6 +1058,14 @@ def pcfg_viterbi_decode_logits(logits, links, output_length, left_tree_mask, pad
     (:483-502) enqueued by one native call.  Returns what ``pcfg_viterbi_decode(*logsoftmax_max(logits), ...)`` returns:
     (tokens float32 [B, maxlen], pred_length int64 [B]); with ``return_nodes`` also the node scores [B,L] float32 and node
     tokens [B,L] int64 of the front-end."""
+    ext = _ext()
+    if ext is not None:
+        tokens, pred, block, nodes = _viterbi_decode_ext(ext, logits, None, None, links, output_length, left_tree_mask, pad_index, beta)
+        if not return_nodes:
+            return tokens, pred
+        tail = block[block.numel() - (nodes + (nodes + 1) // 2):]
+        return tokens, pred, tail[nodes:].view(torch.float32)[:nodes].view(links.size(0), links.size(1)), \
+            tail[:nodes].view(links.size(0), links.size(1))
     _need_cuda("pcfg_viterbi_decode_logits", logits, links, output_length, left_tree_mask)
     if logits.dim() != 3 or not logits.is_contiguous():
         raise RuntimeError("pcfg_viterbi_decode_logits: logits must be a contiguous [bsz, prelen, vocab] tensor")

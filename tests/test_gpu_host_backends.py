@@ -170,3 +170,44 @@ def test_link_scorer_backends_give_identical_results():
         ops.host_backend(before)
     for a, b in zip(results["extension"], results["python"]):
         assert a.dtype == b.dtype and torch.equal(a, b)
+
+
+def test_decode_backends_give_identical_results(backend):
+    """The single-call Viterbi decode through the C++ enqueue function and through the Python wrapper over ctypes: the
+    oracle's tokens and lengths from both, from the logits (with the front-end's node scores and tokens) and from the node
+    scores; a batch, one sentence, an empty batch; the same loud errors."""
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    import oracle_ops
+    from pcfg_nat_amd import harness
+    batch = synth.decode_batch([30, 8, 51, 3], seed=11, V=300)
+    L = batch["links"].shape[1]
+    lm = synth.support_masks(L, 1)[0]
+    ob, tok = synth.ob_and_tokens(batch["logits"])
+    want_tok, want_len = harness.viterbi_decode(ob, tok, batch["links"], batch["output_length"], lm, ops=oracle_ops, beta=0.8)
+    logits, links, ol, lmd = batch["logits"].to(DEV), batch["links"].to(DEV), batch["output_length"].to(DEV), lm.to(DEV)
+    got_tok, got_len, scores, toks = ops.pcfg_viterbi_decode_logits(logits, links, ol, lmd, synth.PAD, 0.8, return_nodes=True)
+    assert got_tok.dtype == torch.float32 and torch.equal(got_tok.cpu(), want_tok) and torch.equal(got_len.cpu(), want_len)
+    assert torch.equal(toks.cpu(), tok) and torch.allclose(scores.cpu(), ob, atol=2e-6)
+    got_tok, got_len = ops.pcfg_viterbi_decode(scores, links, ol, toks.int(), lmd.bool(), synth.PAD, 0.8)  # (dtypes are converted)
+    assert torch.equal(got_tok.cpu(), want_tok) and torch.equal(got_len.cpu(), want_len)
+    # one sentence: the row comes back as a view, still the oracle's tokens
+    one = synth.decode_batch([19], seed=12, V=300)
+    L1 = one["links"].shape[1]
+    lm1 = synth.support_masks(L1, 1)[0]
+    ob1, tok1 = synth.ob_and_tokens(one["logits"])
+    w_tok, w_len = harness.viterbi_decode(ob1, tok1, one["links"], one["output_length"], lm1, ops=oracle_ops)
+    g_tok, g_len = ops.pcfg_viterbi_decode_logits(one["logits"].to(DEV), one["links"].to(DEV), one["output_length"].to(DEV), lm1.to(DEV),
+                                                  synth.PAD)
+    assert g_tok.is_contiguous() and torch.equal(g_tok.cpu(), w_tok) and torch.equal(g_len.cpu(), w_len)
+    # nothing to decode
+    e_tok, e_len = ops.pcfg_viterbi_decode_logits(logits[:0], links[:0], ol[:0], lmd, synth.PAD)
+    assert e_tok.shape == (0, 0) and e_len.shape == (0,)
+    with pytest.raises(RuntimeError, match="float16 or float32"):
+        ops.pcfg_viterbi_decode_logits(logits.double(), links, ol, lmd, synth.PAD)
+    with pytest.raises(RuntimeError, match="lengths should be long"):
+        ops.pcfg_viterbi_decode_logits(logits, links, ol.int(), lmd, synth.PAD)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ops.pcfg_viterbi_decode_logits(logits, links.cpu(), ol, lmd, synth.PAD)
+    with pytest.raises(RuntimeError, match="does not match"):
+        ops.pcfg_viterbi_decode_logits(logits, links[:, :-2], ol, lmd, synth.PAD)
