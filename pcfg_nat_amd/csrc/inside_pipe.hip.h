@@ -46,12 +46,25 @@ template <int NQ, bool JOINT>
 __device__ __forceinline__ void slab_row_lse(const float4 (&A0)[NQ], const float4 (&A1)[NQ], const float4 *u0, const float4 *u1, int qa,
                                              int qb, bool live, bool has1, float g, float &out0, float &out1) {
     g = is_finite(g) ? g : 0.f;
+    // the column(s) first, all LDS reads in flight together: a read inside each chunk's branch (qa, qb are run-time values)
+    // costs the block one LDS round trip per chunk and step
+    float4 v0[NQ], v1[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+        v0[q] = u0[16 * q];
+        if (JOINT) v1[q] = u1[16 * q];
+    }
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {  // (keeps the reads up here)
+        asm volatile("" : "+v"(v0[q].x), "+v"(v0[q].y), "+v"(v0[q].z), "+v"(v0[q].w));
+        if (JOINT) asm volatile("" : "+v"(v1[q].x), "+v"(v1[q].y), "+v"(v1[q].z), "+v"(v1[q].w));
+    }
     float s0 = 0.f, s1 = 0.f;
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
         if (q >= qa && q < qb) {
-            const float4 c0 = minus(u0[16 * q], g);
-            const float4 c1 = JOINT ? minus(u1[16 * q], g) : c0;
+            const float4 c0 = minus(v0[q], g);
+            const float4 c1 = JOINT ? minus(v1[q], g) : c0;
             s0 += sum4_ex2(A0[q], c0);
             s1 += sum4_ex2(A1[q], c1);
         }
@@ -73,8 +86,8 @@ __device__ __forceinline__ void slab_row_lse(const float4 (&A0)[NQ], const float
 #pragma unroll
         for (int q = 0; q < NQ; q++) {
             if (q >= qa && q < qb) {
-                const float4 c0 = u0[16 * q];
-                const float4 c1 = JOINT ? u1[16 * q] : c0;
+                const float4 c0 = v0[q];
+                const float4 c1 = JOINT ? v1[q] : c0;
                 a0.add4(A0[q], c0);
                 a1.add4(A1[q], c1);
             }

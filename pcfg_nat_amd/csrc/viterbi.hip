@@ -650,13 +650,23 @@ __global__ __launch_bounds__(VP_NT) void viterbi_ml1_pipe_kernel(const float *__
                 for (int r = 0; r < RQ; r++) x[r] = entry_load(Xb + (size_t)(len + 1) * MP + 16 * (k + 1) + 64 * r + lane);
             }
         } else {
+            // the two columns first, all reads in flight together (a read inside each chunk's branch costs the block one
+            // LDS round trip per chunk: 106 -> 89 us at 12 blocks), then the chunks that hold children of this block
+            float sc1[NQ], sc2[NQ];
+#pragma unroll
+            for (int q = 0; q < NQ; q++) {
+                sc1[q] = cur1[j16 + 16 * q];
+                sc2[q] = cur2[j16 + 16 * q];
+            }
+#pragma unroll
+            for (int q = 0; q < NQ; q++) asm volatile("" : "+v"(sc1[q]), "+v"(sc2[q]));  // (keeps the reads up here)
             float best = NEG_INF_F;
             int sel = -1;
 #pragma unroll
             for (int q = 0; q < NQ; q++) {
                 if (q >= k) {
-                    const float c0 = (A0[q] + cur1[j16 + 16 * q]) + ob_a;
-                    const float c1 = (A1[q] + cur2[j16 + 16 * q]) + ob_a;
+                    const float c0 = (A0[q] + sc1[q]) + ob_a;
+                    const float c1 = (A1[q] + sc2[q]) + ob_a;
                     if (c0 > best) {  // false for NaN and for -inf against the initial -inf
                         best = c0;
                         sel = 2 * q;
