@@ -584,6 +584,7 @@ __global__ __launch_bounds__(VP_NT) void viterbi_ml1_pipe_kernel(const float *__
     float A0[NQ], A1[NQ];
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
+        A0[q] = A1[q] = NEG_INF_F;
         if (q >= k) {
             const int c = 2 * min(j16 + 16 * q, mc - 1) + 1;
             A0[q] = lk[((size_t)a * 2 + 0) * L + c];
@@ -662,18 +663,23 @@ __global__ __launch_bounds__(VP_NT) void viterbi_ml1_pipe_kernel(const float *__
             for (int q = 0; q < NQ; q++) asm volatile("" : "+v"(sc1[q]), "+v"(sc2[q]));  // (keeps the reads up here)
             float best = NEG_INF_F;
             int sel = -1;
+            // chunks in groups of four under one branch each (the chunks in front of the block hold -inf in the slabs): a
+            // branch per chunk scattered the loop over the kernel's code, and the jumps cost more than the chunks
 #pragma unroll
-            for (int q = 0; q < NQ; q++) {
-                if (q >= k) {
-                    const float c0 = (A0[q] + sc1[q]) + ob_a;
-                    const float c1 = (A1[q] + sc2[q]) + ob_a;
-                    if (c0 > best) {  // false for NaN and for -inf against the initial -inf
-                        best = c0;
-                        sel = 2 * q;
-                    }
-                    if (c1 > best) {
-                        best = c1;
-                        sel = 2 * q + 1;
+            for (int q4 = 0; q4 < NQ; q4 += 4) {
+                if (q4 + 3 >= k) {
+#pragma unroll
+                    for (int q = q4; q < q4 + 4 && q < NQ; q++) {
+                        const float c0 = (A0[q] + sc1[q]) + ob_a;
+                        const float c1 = (A1[q] + sc2[q]) + ob_a;
+                        if (c0 > best) {  // false for NaN and for -inf against the initial -inf
+                            best = c0;
+                            sel = 2 * q;
+                        }
+                        if (c1 > best) {
+                            best = c1;
+                            sel = 2 * q + 1;
+                        }
                     }
                 }
             }
