@@ -903,6 +903,35 @@ def test_decode_from_logits_is_front_end_plus_decode(case, dtype):
         ops.pcfg_viterbi_decode_logits(logits.double(), links, ol, left_mask, synth.PAD)
 
 
+@pytest.mark.parametrize("case", ["L96", "L288", "L600"])
+def test_single_call_decode_c_abi_without_float_tokens(case):
+    """pcfgnat_viterbi_decode through ctypes with out_tokens_f32 = NULL (a caller that only wants the int64 rows): the
+    one-workgroup decode, the pipelined one and the general path leave the rows and counts the wrapper's float32 tokens
+    come from."""
+    from pcfg_nat_amd import _lib
+    lib = ops.get_pcfg_kernel()
+    batch = _decode_case(case)
+    ob, tok = synth.ob_and_tokens(batch["logits"])
+    links, ol = batch["links"].to(DEV), batch["output_length"].to(DEV)
+    B, L = ob.shape
+    left_mask = synth.support_masks(L, 1)[0].to(DEV)
+    ob, tok = ob.to(DEV), tok.to(DEV)
+    want_tok, want_len = ops.pcfg_viterbi_decode(ob, links, ol, tok, left_mask, synth.PAD)
+    pen = ops._length_penalty(L // 4, 1.0, ob.device)
+    work = torch.empty((lib.pcfgnat_viterbi_decode_workspace_bytes(B, L, 1) + 7) // 8, dtype=torch.int64, device=DEV)
+    rows = torch.full((B, L), -7, dtype=torch.int64, device=DEV)
+    counts = torch.full((B,), -7, dtype=torch.int64, device=DEV)
+    pred = torch.full((B,), -7, dtype=torch.int64, device=DEV)
+    _lib.check(lib.pcfgnat_viterbi_decode(ob.data_ptr(), links.data_ptr(), ol.data_ptr(), tok.data_ptr(), left_mask.data_ptr(), L,
+                                          synth.PAD, pen.data_ptr(), work.data_ptr(), rows.data_ptr(), None, counts.data_ptr(),
+                                          pred.data_ptr(), B, L, 1, torch.cuda.current_stream().cuda_stream), lib)
+    torch.cuda.synchronize()
+    assert torch.equal(pred, want_len)
+    n = int(counts.max())
+    assert n == want_tok.shape[1] and torch.equal(rows[:, :n].float(), want_tok)
+    assert (rows[:, n:] == synth.PAD).all()
+
+
 def test_decode_waits_for_the_stream_where_the_counts_do_not_turn():
     """The decode calls watch the token counts turn in pinned host memory.  A watch that runs into its time bound (forced
     here by a bound of zero seconds) hands over to the stream wait for that call with the same results; the watching is
