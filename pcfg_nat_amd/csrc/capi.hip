@@ -126,12 +126,16 @@ extern "C" int pcfgnat_criterion_forward(void *logits, int dtype, const int64_t 
     int rc = pcfgnat::lsg_forward_lse_force(logits, dtype, targets, match_all, row_lse, output_length, target_length, matchmask,
                                             keep_word_mask, B, L, V, T, stream);
     if (rc != PCFGNAT_OK) return rc;
-    bool pad_done = false;
+    bool pad_done = false, loss_done = false;
+    // the loss is formed beside the posteriors where the kernels of this shape offer that, by a launch of its own otherwise
+    const pcfgnat::LossTask loss{S, target_length, loss_out, (int)B, (int64_t)((L - 2) / (ml + 1) + 1) * (T + 2), ll_out};
     rc = pcfgnat::inside_forward_backward_impl(nullptr, match_all, links, output_length, target_length, S, aux, match_all_grad, links_grad,
                                                B, L, T, ml, pcfgnat::seed_of(B), stream,
-                                               pcfgnat::PadFill{(unsigned char *)logits, (int64_t)V * (int64_t)esz}, &pad_done);
+                                               pcfgnat::PadFill{(unsigned char *)logits, (int64_t)V * (int64_t)esz}, &pad_done, &loss,
+                                               &loss_done);
     if (rc != PCFGNAT_OK) return rc;
     *pad_rows_zeroed = pad_done ? 1 : 0;
+    if (loss_done) return PCFGNAT_OK;
     return pcfgnat::criterion_loss_impl(S, target_length, loss_out, ll_out, B, L, T, ml, stream);
 }
 

@@ -92,7 +92,8 @@ struct PadFill {
 int inside_forward_backward_impl(const float *grad_output, const float *match_all, const float *links, const int64_t *output_length,
                                  const int64_t *target_length, float *S, float *aux, float *match_all_grad, float *links_grad,
                                  int64_t B, int64_t L, int64_t T, int64_t ml, Seed seed, void *stream,
-                                 PadFill pad = PadFill{nullptr, 0}, bool *pad_done = nullptr);
+                                 PadFill pad = PadFill{nullptr, 0}, bool *pad_done = nullptr, const struct LossTask *loss = nullptr,
+                                 bool *loss_done = nullptr);
 
 // Read-only logsoftmax_gather over the [B,T] targets with the eos mask, which also returns the first arg max of every row;
 // the rows of nodes at or beyond a sentence's output length are left unread (zeros in selected and argmax)

@@ -308,7 +308,7 @@ int launch_bwd(const float *go, const float *S, float *aux, const float *match_a
 template <int R>
 int launch_fused(const float *go, const float *match_all, const float *links, const int64_t *ol, const int64_t *tl, float *S, float *aux,
                  float *mg, float *lg, int B, int L, int T, int Mc, Seed seed, hipStream_t stream, bool *done,
-                 PadFill pad = PadFill{nullptr, 0}, bool *pad_done = nullptr) {
+                 PadFill pad = PadFill{nullptr, 0}, bool *pad_done = nullptr, const LossTask *loss = nullptr, bool *loss_done = nullptr) {
     const size_t need = ((size_t)head_floats(T) + 4 * 64 * R + (size_t)4 * Mc * (T + 2) + (size_t)2 * Mc * T) * sizeof(float);
     *done = false;
     if (R == 1) {  // the two sweeps side by side as two workgroups per sentence, then the posteriors
@@ -330,9 +330,12 @@ int launch_fused(const float *go, const float *match_all, const float *links, co
                                links, ol, tl, S, aux, L, T, Mc, B, pad);
             PCFGNAT_HIP_CHECK(hipGetLastError());
             if (fill && pad_done) *pad_done = true;
-            hipLaunchKernelGGL(inside_combine_ml1_kernel, dim3(16, B), dim3(256), comb_bytes, stream, go, S, aux, match_all, links, ol, tl,
-                               mg, lg, L, T, Mc, seed);
+            const bool with_loss = loss != nullptr && loss->out != nullptr;
+            hipLaunchKernelGGL(inside_combine_ml1_kernel, dim3(16, B + (with_loss ? 1 : 0)), dim3(256), comb_bytes, stream, go, S, aux,
+                               match_all, links, ol, tl, mg, lg, L, T, Mc, seed,
+                               with_loss ? *loss : LossTask{nullptr, nullptr, nullptr, 0, 0, nullptr});
             PCFGNAT_HIP_CHECK(hipGetLastError());
+            if (with_loss && loss_done) *loss_done = true;
             *done = true;
             return PCFGNAT_OK;
         }
@@ -442,8 +445,10 @@ extern "C" int pcfgnat_pcfg_loss_backward(const float *grad_output, const float 
 int pcfgnat::inside_forward_backward_impl(const float *grad_output, const float *match_all, const float *links,
                                           const int64_t *output_length, const int64_t *target_length, float *S, float *aux,
                                           float *match_all_grad, float *links_grad, int64_t B, int64_t L, int64_t T, int64_t ml,
-                                          Seed seed, void *stream, PadFill pad, bool *pad_done) {
+                                          Seed seed, void *stream, PadFill pad, bool *pad_done, const LossTask *loss,
+                                          bool *loss_done) {
     if (pad_done) *pad_done = false;
+    if (loss_done) *loss_done = false;
     int rc = check_dims("pcfg_loss_forward_backward", B, L, T, ml);
     if (rc != PCFGNAT_OK) return rc;
     if (B == 0) return PCFGNAT_OK;
@@ -466,7 +471,7 @@ int pcfgnat::inside_forward_backward_impl(const float *grad_output, const float 
         // general max_left: the two plain kernels
     } else if (Mc <= 64)
         rc = launch_fused<1>(grad_output, match_all, links, output_length, target_length, S, aux, match_all_grad, links_grad, (int)B, (int)L,
-                             (int)T, Mc, seed, s, &done, pad, pad_done);
+                             (int)T, Mc, seed, s, &done, pad, pad_done, loss, loss_done);
     if (rc != PCFGNAT_OK || done) return rc;
     const PipelinePlan plan = (ml == 1 && Mc > 64) ? pipeline_plan((int)B, (int)T, Mc) : PipelinePlan{0, false};
     if (plan.side_by_side) {  // the two pipelined sweeps in one launch

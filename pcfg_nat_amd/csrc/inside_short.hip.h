@@ -1044,7 +1044,14 @@ __global__ __launch_bounds__(256) void inside_combine_ml1_kernel(const float *__
                                                                 float *__restrict__ aux, const float *__restrict__ match_all,
                                                                 const float *__restrict__ links, const int64_t *__restrict__ out_len,
                                                                 const int64_t *__restrict__ tgt_len, float *__restrict__ mgrad,
-                                                                float *__restrict__ lgrad, int L, int T, int Mc, Seed seed) {
+                                                                float *__restrict__ lgrad, int L, int T, int Mc, Seed seed,
+                                                                LossTask loss) {
+    // With a loss to form (the criterion's forward under autograd), the launch has one more row of workgroups, whose first
+    // one reduces the log-likelihoods the sweeps left - beside the posteriors instead of in a launch of its own behind them.
+    if (loss.out != nullptr && blockIdx.y == gridDim.y - 1) {  // workgroup-uniform
+        if (blockIdx.x == 0) criterion_loss_block<256>(loss);
+        return;
+    }
     const int TS = T + 2, TP = T + 4;
     extern __shared__ float smem[];
     float *corr = smem;               // [TP]
