@@ -1,6 +1,7 @@
 // General max_left ("ml" = links.size(2) - 1 = 2^left_tree_layer - 1): the inside loss, its exact backward, the best-tree
 // trace and the viterbi tables for any ml other than 1 (ml = 1, the setting of every shipped script, has its own tuned
-// kernels in inside.hip / viterbi.hip).
+// kernels in inside.hip / viterbi.hip; at ml = 3 the loss and the viterbi tables of sentences without composite local
+// trees are taken by inside_ml3.hip / viterbi.hip, and the kernels here skip them).
 //
 // Replaces the general-ml paths of the reference's pcfg_loss.cu (:84-349), pcfg_loss_backward.cu (:28-603),
 // pcfg_best_tree.cu (:64-301) and pcfg_viterbi.cu (:22-241).

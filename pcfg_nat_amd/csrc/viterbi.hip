@@ -1,7 +1,8 @@
 // Viterbi (max-product) tables per output length with back-pointers, and the tree-to-sequence readout.
 //
 // Replaces the reference's pcfg_viterbi.cu (calculate_C_kernel :177-241, calculate_S_kernel :22-140) and the
-// host loop viterbi_decoding (pcfg_loss.cpp:12-73), for max_left = 1.
+// host loop viterbi_decoding (pcfg_loss.cpp:12-73), for max_left = 1 - and for max_left = 3 where a sentence's links hold
+// no rule of a composite local tree (viterbi_ml3_kernel; any other case: generic_ml.hip).
 //
 // S[a][len] = ob[a] + max over (c >= a, j in {0,1}) of links[a][j][c] + C[j] + S[c][len-j-1], with C[0] = 0 (null left
 // child) and C[1] = ob[a-1] (the local leaf).  Every candidate is evaluated as ((links + C) + S) + ob in fp32, the
